@@ -1,0 +1,527 @@
+/*
+ * CPU oracle (test infrastructure; see itex_oracle.h for the full header comment, the list of
+ * parity pins and of the parts whose parity is unpinned).
+ *
+ * Build with contraction off: every fp32 operation below must round on its own
+ * (gcc -O2 -ffp-contract=off -fno-fast-math).
+ */
+#include "itex_oracle.h"
+
+#include <float.h>
+#include <math.h>
+#include <stdlib.h>
+#include <string.h>
+
+/* Eigen::NumTraits<T>::highest() / lowest() for the quantized types
+ * (used at itex/core/utils/quantization_util.h:58-59). */
+static int64_t q_highest(int T) {
+  switch (T) {
+    case ORC_QINT8: return 127;
+    case ORC_QUINT8: return 255;
+    case ORC_QINT32: return 2147483647LL;
+    default: return 0;
+  }
+}
+static int64_t q_lowest(int T) {
+  switch (T) {
+    case ORC_QINT8: return -128;
+    case ORC_QUINT8: return 0;
+    case ORC_QINT32: return -2147483648LL;
+    default: return 0;
+  }
+}
+
+/* oneDNN destination conversion: clamp in fp32 to the destination range, then convert with
+ * round-to-nearest-even.  NaN maps to the lower bound here (parity unpinned). */
+static inline float sat_rne(float y, float lo, float hi) {
+  y = fmaxf(y, lo);
+  y = fminf(y, hi);
+  return rintf(y);
+}
+static inline void sat_bounds(int T, float* lo, float* hi) {
+  if (T == ORC_QINT8) { *lo = -128.0f; *hi = 127.0f; }
+  else if (T == ORC_QUINT8) { *lo = 0.0f; *hi = 255.0f; }
+  else { *lo = -2147483648.0f; *hi = 2147483520.0f; } /* largest fp32 below 2^31 */
+}
+static inline void store_q(void* q, int64_t i, int T, float r) {
+  if (T == ORC_QINT8) ((int8_t*)q)[i] = (int8_t)(int32_t)r;
+  else if (T == ORC_QUINT8) ((uint8_t*)q)[i] = (uint8_t)(int32_t)r;
+  else ((int32_t*)q)[i] = (int32_t)r;
+}
+
+/* QuantizeV2Op::AdjustInputMinMaxRange, itex/core/kernels/common/quantize_op.h:130-152 */
+int orc_adjust_input_range(float in_min, float in_max, float ensure_minimum_range, float* adj_min,
+                           float* adj_max) {
+  if (!(in_max >= in_min)) return ORC_INVALID_ARGUMENT; /* :133-135 */
+  *adj_min = fminf(0.0f, in_min);                        /* :137 */
+  const float epsilon = fmaxf(1.0f, fmaxf(fabsf(in_min), fabsf(in_max))) * ensure_minimum_range;
+  *adj_max = fmaxf(0.0f, fmaxf(in_max, *adj_min + epsilon)); /* :150-151 */
+  return ORC_OK;
+}
+
+/* GetScaleAndZeropointAndAlignMinMax<T>, itex/core/utils/quantization_util.h:54-84.
+ * int64 operands are converted to float before the fp32 division / subtraction, exactly as the
+ * usual arithmetic conversions do in the reference expression. */
+int orc_scale_zeropoint_align(int T, int mode, int dequantize, float* min_data, float* max_data,
+                              int length, float* scales, int32_t* zero_points) {
+  const float max_int = (float)q_highest(T);
+  const float span = (float)(q_highest(T) - q_lowest(T));
+  if (mode == ORC_SCALED) {
+    for (int i = 0; i < length; ++i) {
+      float abs_range = fmaxf(fabsf(min_data[i]), fabsf(max_data[i]));
+      max_data[i] = abs_range;
+      min_data[i] = -abs_range;
+      scales[i] = dequantize ? (abs_range / max_int) : (max_int / abs_range);
+      zero_points[i] = 0;
+    }
+  } else if (mode == ORC_MIN_FIRST) {
+    for (int i = 0; i < length; ++i) {
+      scales[i] = dequantize ? ((max_data[i] - min_data[i]) / span)
+                             : (span / (max_data[i] - min_data[i]));
+      /* std::round: half away from zero */
+      zero_points[i] = dequantize ? (int32_t)roundf(max_int - max_data[i] / scales[i])
+                                  : (int32_t)roundf(max_int - max_data[i] * scales[i]);
+    }
+  } else {
+    return ORC_INVALID_ARGUMENT;
+  }
+  return ORC_OK;
+}
+
+/* Legacy MIN_FIRST scale, quantize_op.h:204-214: (number_of_steps - 1.0) is a double, so the
+ * division is carried out in double and rounded once to float on assignment. */
+float orc_legacy_min_first_scale(int T, float adj_min, float adj_max) {
+  const int number_of_bits = (T == ORC_QINT32) ? 32 : 8;
+  const int64_t number_of_steps = (int64_t)1 << number_of_bits;
+  return (float)(((double)number_of_steps - 1.0) / (double)(adj_max - adj_min));
+}
+
+/* QuantizeV2Op::Compute, quantize_op.h:154-408.  The tensor is viewed as [outer, slices, inner]
+ * with `slices` the size of `axis` (1 for per-tensor). */
+int orc_quantize_v2(const float* x, int64_t outer, int64_t slices, int64_t inner, int T, int mode,
+                    int classic_asymmetric, float ensure_minimum_range, const float* in_min,
+                    const float* in_max, void* q, float* out_min, float* out_max) {
+  if (T != ORC_QINT8 && T != ORC_QUINT8) return ORC_INVALID_ARGUMENT;
+  if (mode != ORC_SCALED && mode != ORC_MIN_FIRST) return ORC_INVALID_ARGUMENT; /* :94-97 */
+  float* mn = (float*)malloc(sizeof(float) * (size_t)slices);
+  float* mx = (float*)malloc(sizeof(float) * (size_t)slices);
+  float* scale = (float*)malloc(sizeof(float) * (size_t)slices);
+  int32_t* zp = (int32_t*)malloc(sizeof(int32_t) * (size_t)slices);
+  int st = ORC_OK;
+  for (int64_t s = 0; s < slices && st == ORC_OK; ++s)
+    st = orc_adjust_input_range(in_min[s], in_max[s], ensure_minimum_range, &mn[s], &mx[s]);
+  if (st != ORC_OK) goto done;
+
+  const int legacy = (mode == ORC_MIN_FIRST && !classic_asymmetric);
+  if (!legacy) {
+    orc_scale_zeropoint_align(T, mode, 0, mn, mx, (int)slices, scale, zp); /* :198-202 */
+  } else {
+    for (int64_t s = 0; s < slices; ++s) {
+      scale[s] = orc_legacy_min_first_scale(T, mn[s], mx[s]);
+      zp[s] = 0;
+    }
+  }
+  float lo, hi;
+  sat_bounds(T, &lo, &hi);
+#pragma omp parallel for collapse(2) schedule(static)
+  for (int64_t o = 0; o < outer; ++o) {
+    for (int64_t s = 0; s < slices; ++s) {
+      const float sc = scale[s];
+      const int64_t base = (o * slices + s) * inner;
+      if (mode == ORC_SCALED) {
+        /* reorder with a source scale (:256-275): q = sat(rne(x * scale)) */
+        for (int64_t i = 0; i < inner; ++i) store_q(q, base + i, T, sat_rne(x[base + i] * sc, lo, hi));
+      } else if (!legacy) {
+        /* reorder with source scale and destination zero point (:276-291):
+         * q = sat(rne(x * scale + zp)), the zero point is added in fp32 before the conversion */
+        const float zpf = (float)zp[s];
+        for (int64_t i = 0; i < inner; ++i)
+          store_q(q, base + i, T, sat_rne(x[base + i] * sc + zpf, lo, hi));
+      } else {
+        /* binary_add of x and shift=-min', both sources scaled by `scale` (:292-314, 383-391):
+         * three separately rounded fp32 operations */
+        const float shift = -mn[s]; /* :244-245 */
+        const float t1 = shift * sc;
+        for (int64_t i = 0; i < inner; ++i) {
+          const float t0 = x[base + i] * sc;
+          store_q(q, base + i, T, sat_rne(t0 + t1, lo, hi));
+        }
+      }
+    }
+  }
+  /* output ranges, :397-408 */
+  for (int64_t s = 0; s < slices; ++s) {
+    if (T == ORC_QUINT8 && mode == ORC_SCALED) { out_min[s] = 0.0f; out_max[s] = mx[s]; }
+    else { out_min[s] = mn[s]; out_max[s] = mx[s]; }
+  }
+done:
+  free(mn); free(mx); free(scale); free(zp);
+  return st;
+}
+
+/* DequantizeOp::Compute, itex/core/kernels/common/dequantize_op.h:67-178: reorder with a source
+ * scale and (MIN_FIRST) a source zero point: y = ((float)q - zp) * scale. */
+int orc_dequantize(const void* q, int64_t outer, int64_t slices, int64_t inner, int T, int mode,
+                   const float* in_min, const float* in_max, float* y) {
+  if (T != ORC_QINT8 && T != ORC_QUINT8) return ORC_INVALID_ARGUMENT;
+  if (mode != ORC_SCALED && mode != ORC_MIN_FIRST) return ORC_INVALID_ARGUMENT;
+  float* mn = (float*)malloc(sizeof(float) * (size_t)slices);
+  float* mx = (float*)malloc(sizeof(float) * (size_t)slices);
+  float* scale = (float*)malloc(sizeof(float) * (size_t)slices);
+  int32_t* zp = (int32_t*)malloc(sizeof(int32_t) * (size_t)slices);
+  memcpy(mn, in_min, sizeof(float) * (size_t)slices);
+  memcpy(mx, in_max, sizeof(float) * (size_t)slices);
+  orc_scale_zeropoint_align(T, mode, 1, mn, mx, (int)slices, scale, zp); /* :101-103 */
+#pragma omp parallel for collapse(2) schedule(static)
+  for (int64_t o = 0; o < outer; ++o) {
+    for (int64_t s = 0; s < slices; ++s) {
+      const float sc = scale[s];
+      const float zpf = (mode == ORC_MIN_FIRST) ? (float)zp[s] : 0.0f;
+      const int64_t base = (o * slices + s) * inner;
+      for (int64_t i = 0; i < inner; ++i) {
+        const float v = (T == ORC_QINT8) ? (float)((const int8_t*)q)[base + i]
+                                         : (float)((const uint8_t*)q)[base + i];
+        y[base + i] = (v - zpf) * sc;
+      }
+    }
+  }
+  free(mn); free(mx); free(scale); free(zp);
+  return ORC_OK;
+}
+
+/* OneDnnRequantizePerChannelOp::Compute,
+ * itex/core/kernels/onednn/block/requantize_per_channel_op.cc:44-159.  Channel = last dimension. */
+int orc_requantize_per_channel(const int32_t* x, int64_t rows, int64_t depth, const float* in_min,
+                               const float* in_max, float req_min, float req_max, int out_type,
+                               void* q, float* out_min, float* out_max) {
+  if (out_type != ORC_QINT8 && out_type != ORC_QUINT8) return ORC_INVALID_ARGUMENT; /* :40-42 */
+  const float factor = (out_type == ORC_QINT8) ? 127.0f : 255.0f;                     /* :82 */
+  const float requested_min_max = fmaxf(fabsf(req_min), fabsf(req_max));              /* :83-85 */
+  float* scales = (float*)malloc(sizeof(float) * (size_t)depth);
+  for (int64_t i = 0; i < depth; ++i) {
+    const float mm = fmaxf(fabsf(in_min[i]), fabsf(in_max[i]));
+    scales[i] = factor * (mm / requested_min_max / 2147483648.0f); /* :91-95 */
+  }
+  float lo, hi;
+  sat_bounds(out_type, &lo, &hi);
+#pragma omp parallel for schedule(static)
+  for (int64_t r = 0; r < rows; ++r)
+    for (int64_t c = 0; c < depth; ++c)
+      store_q(q, r * depth + c, out_type, sat_rne((float)x[r * depth + c] * scales[c], lo, hi));
+  *out_min = req_min; /* :149-150 */
+  *out_max = req_max;
+  free(scales);
+  return ORC_OK;
+}
+
+/* OneDnnRequantizationRangePerChannelOp::Compute,
+ * itex/core/kernels/onednn/block/requantization_range_per_channel_op.cc:41-159. */
+int orc_requantization_range_per_channel(const int32_t* x, int64_t rows, int64_t depth,
+                                         const float* in_min, const float* in_max,
+                                         float clip_value_max, float* out_min, float* out_max) {
+  float out_min_max = FLT_MIN; /* std::numeric_limits<float>::min(), :78 */
+  int is_non_negative = 1;
+  for (int64_t c = 0; c < depth; ++c) {
+    int32_t mn = INT32_MAX, mx = INT32_MIN;
+    for (int64_t r = 0; r < rows; ++r) {
+      const int32_t v = x[r * depth + c];
+      if (v < mn) mn = v;
+      if (v > mx) mx = v;
+    }
+    /* std::abs(int32) wraps for INT32_MIN upstream (undefined behaviour; parity unpinned) */
+    const int32_t amn = (mn == INT32_MIN) ? INT32_MIN : (mn < 0 ? -mn : mn);
+    const int32_t amx = (mx == INT32_MIN) ? INT32_MIN : (mx < 0 ? -mx : mx);
+    const int32_t abs_max = amn > amx ? amn : amx;                       /* :133-134 */
+    const float scale = fmaxf(fabsf(in_min[c]), fabsf(in_max[c]));       /* :135-136 */
+    const float range = scale * (float)abs_max / 2147483648.0f;          /* :137-138 */
+    if (mn < 0) is_non_negative = 0;                                     /* :139 */
+    out_min_max = fmaxf(out_min_max, range);                             /* :142 */
+  }
+  if (out_min_max > clip_value_max) out_min_max = clip_value_max;        /* :150 */
+  *out_min = is_non_negative ? 0.0f : -out_min_max;                      /* :158-159 */
+  *out_max = out_min_max;
+  return ORC_OK;
+}
+
+/* Exact int32 accumulation of a[M,K] (u8 or s8, row-major) times w (s8; TF layout [K,N] row-major,
+ * or [N,K] when transpose_b), quantized_matmul_common.h:183-226 (inner_product_forward). */
+void orc_int_gemm(const void* a, int a_type, const int8_t* w, int transpose_b, int64_t M, int64_t K,
+                  int64_t N, int32_t* acc) {
+#pragma omp parallel for schedule(static)
+  for (int64_t m = 0; m < M; ++m) {
+    int32_t* row = acc + m * N;
+    for (int64_t n = 0; n < N; ++n) row[n] = 0;
+    if (!transpose_b) {
+      for (int64_t k = 0; k < K; ++k) {
+        const int32_t av = (a_type == ORC_QUINT8) ? (int32_t)((const uint8_t*)a)[m * K + k]
+                                                  : (int32_t)((const int8_t*)a)[m * K + k];
+        const int8_t* wr = w + k * N;
+        for (int64_t n = 0; n < N; ++n) row[n] += av * (int32_t)wr[n];
+      }
+    } else {
+      for (int64_t n = 0; n < N; ++n) {
+        const int8_t* wr = w + n * K;
+        int32_t s = 0;
+        if (a_type == ORC_QUINT8) {
+          const uint8_t* ar = (const uint8_t*)a + m * K;
+          for (int64_t k = 0; k < K; ++k) s += (int32_t)ar[k] * (int32_t)wr[k];
+        } else {
+          const int8_t* ar = (const int8_t*)a + m * K;
+          for (int64_t k = 0; k < K; ++k) s += (int32_t)ar[k] * (int32_t)wr[k];
+        }
+        row[n] = s;
+      }
+    }
+  }
+}
+
+/* Column sums of the [K,N] weight, quantized_matmul_common.h:569-573. */
+void orc_weight_colsum(const int8_t* w, int64_t K, int64_t N, int32_t* colsum) {
+  for (int64_t j = 0; j < N; ++j) colsum[j] = 0;
+  for (int64_t i = 0; i < K; ++i)
+    for (int64_t j = 0; j < N; ++j) colsum[j] += (int32_t)w[i * N + j];
+}
+
+static int eltwise_from_activation(int act, orc_eltwise* e) {
+  /* table at itex/core/utils/onednn/onednn_post_op_util.cc:34-68 */
+  switch (act) {
+    case ORC_ACT_RELU: e->alg = ORC_ELT_RELU; e->alpha = 0.0f; e->beta = 0.0f; return 1;
+    case ORC_ACT_RELU6: e->alg = ORC_ELT_CLIP; e->alpha = 0.0f; e->beta = 6.0f; return 1;
+    case ORC_ACT_LEAKYRELU: e->alg = ORC_ELT_RELU; e->alpha = 0.0f; e->beta = 0.0f; return 1;
+    default: return 0;
+  }
+}
+
+/*
+ * Host-side parameter preparation of the quantized MatMul kernels:
+ *   output scales  - ExtendInt8PostOps: V2 quantized_matmul_common.h:1809-1908,
+ *                    V1 :1610-1702, legacy :1472-1508 (+ :1526-1530 for the ReLU variant)
+ *   scaled bias    - GetScaledBias (fp32 bias), :466-660
+ *   post-op chain  - PostOpUtil::AddOps / SetPostOp, onednn_post_op_util.cc:73-128, 237-273
+ * `scales` must hold max(nb,1) floats, `bias_out` N floats.  `colsum` (N int32, column sums of the
+ * [K,N] weight) is only read for input_mode == MIN_FIRST.
+ */
+int orc_qmatmul_prepare(const orc_matmul_attrs* at, int64_t N, const int32_t* colsum, float min_a,
+                        float max_a, const float* min_b, const float* max_b, int64_t nb,
+                        float min_out, float max_out, const float* bias, float* scales,
+                        float* bias_out, orc_epilogue_desc* ep) {
+  const int out_q8 = (at->t_out == ORC_QINT8 || at->t_out == ORC_QUINT8);
+  const int out_f32 = (at->t_out == ORC_FLOAT);
+  const int out_s32 = (at->t_out == ORC_QINT32);
+  if (!out_q8 && !out_f32 && !out_s32) return ORC_INVALID_ARGUMENT;
+  if (at->input_mode != ORC_MIN_FIRST && at->input_mode != ORC_SCALED) return ORC_INVALID_ARGUMENT;
+  if (nb != 1 && nb != N) return ORC_INVALID_ARGUMENT;
+
+  const float max_int8_input = (at->t_in == ORC_QUINT8) ? 255.0f : 127.0f;  /* :503-506 */
+  const float max_int8_weight = 127.0f;
+  const float range_input = (at->input_mode == ORC_MIN_FIRST)
+                                ? max_a - min_a
+                                : fmaxf(fabsf(min_a), fabsf(max_a));          /* :507-510 */
+  const float max_int8_output = (at->t_out == ORC_QUINT8) ? 255.0f : 127.0f;
+
+  memset(ep, 0, sizeof(*ep));
+
+  /* ---- post-op chain -------------------------------------------------------------------- */
+  int has_linear = 0, has_leaky = 0;
+  float linear_alpha = 0.0f, linear_beta = 0.0f;
+  if (eltwise_from_activation(at->activation, &ep->elt[ep->n_eltwise])) ep->n_eltwise++;
+  if (at->activation == ORC_ACT_LEAKYRELU) has_leaky = 1;
+  if (at->api == ORC_API_V2 && at->has_requantize && at->out_min_first) {
+    /* :1753-1757: "Linear" is appended to fused_ops */
+    ep->elt[ep->n_eltwise].alg = ORC_ELT_LINEAR;
+    ep->elt[ep->n_eltwise].alpha = 1.0f;
+    ep->elt[ep->n_eltwise].beta = 0.0f;
+    ep->n_eltwise++;
+    has_linear = 1;
+  }
+  const int has_activation = ep->n_eltwise > 0; /* has_activation_ is set by every eltwise */
+
+  /* ---- output scales ---------------------------------------------------------------------- */
+  if (at->api == ORC_API_V2) {
+    const int has_output_scales = at->has_requantize || at->has_dequantize;
+    if (has_output_scales) { /* :1815-1865 */
+      for (int64_t i = 0; i < nb; ++i) {
+        const float range_weight = fmaxf(fabsf(min_b[i]), fabsf(max_b[i]));
+        scales[i] = (range_input * range_weight) / (max_int8_input * max_int8_weight);
+      }
+      if (at->has_requantize && !has_activation && !has_linear) {
+        const float range_output = fmaxf(fabsf(min_out), fabsf(max_out));
+        for (int64_t i = 0; i < nb; ++i) scales[i] = scales[i] * (max_int8_output / range_output);
+      }
+      ep->n_scales = (int)nb;
+    }
+    /* :1867-1885: the activation's post-op scale is stored but never reaches oneDNN
+     * (onednn_post_op_util.cc:248-263 appends eltwise(alg, alpha, beta) only) */
+    if (has_linear) { /* :1887-1900 */
+      const float range_output = max_out - min_out;
+      linear_alpha = max_int8_output / range_output;
+      linear_beta = -min_out * max_int8_output / range_output;
+    }
+  } else if (at->api == ORC_API_V1) {
+    if (out_s32) { /* :1611-1614 */
+      scales[0] = 1.0f;
+      ep->n_scales = 1;
+    } else { /* :1615-1701 */
+      for (int64_t i = 0; i < nb; ++i) {
+        const float range_weight = fmaxf(fabsf(min_b[i]), fabsf(max_b[i]));
+        scales[i] = (range_input * range_weight) / (max_int8_input * max_int8_weight);
+      }
+      if (out_q8) {
+        const float range_output = fmaxf(fabsf(min_out), fabsf(max_out));
+        if (at->n_fused_ops == 1) {
+          const float f = (at->t_out == ORC_QINT8) ? 127.0f : 255.0f;
+          for (int64_t i = 0; i < nb; ++i) scales[i] = scales[i] * (f / range_output);
+        } /* else: folded into the activation's post-op scale, which is dropped */
+      }
+      ep->n_scales = (int)nb;
+    }
+  } else if (at->api == ORC_API_LEGACY) { /* :1472-1508, per-tensor weights only */
+    if (!out_s32) {
+      /* ComputeOutputRangeForInt32 (:409-421) with <quint8, qint8, qint32> */
+      const float a_level = (max_a - min_a) / 255.0f;
+      const float b_level = (max_b[0] - min_b[0]) / 254.0f;
+      const float c_level = a_level * b_level;
+      const float min_o = c_level * -2147483648.0f;
+      const float max_o = c_level * 2147483648.0f; /* (float)INT32_MAX */
+      const float scale_int32 = fmaxf(fabsf(min_o), fabsf(max_o));
+      const float scale_eightbit = fmaxf(fabsf(min_out), fabsf(max_out));
+      float scale;
+      if (at->t_out == ORC_QUINT8) scale = scale_int32 / scale_eightbit / 8388608.0f;
+      else if (at->t_out == ORC_QINT8) scale = scale_int32 / scale_eightbit / 16777216.0f;
+      else scale = scale_int32 / 2147483648.0f;
+      scales[0] = scale;
+      ep->n_scales = 1;
+    }
+  } else {
+    return ORC_INVALID_ARGUMENT;
+  }
+
+  /* alpha / beta overrides applied to EVERY eltwise of the chain, onednn_post_op_util.cc:251-262 */
+  for (int e = 0; e < ep->n_eltwise; ++e) {
+    if (has_leaky) ep->elt[e].alpha = at->leakyrelu_alpha;
+    if (has_linear) { ep->elt[e].alpha = linear_alpha; ep->elt[e].beta = linear_beta; }
+  }
+
+  /* ---- scaled bias, GetScaledBias :466-660 ------------------------------------------------ */
+  /* bias_scales, :511-519 */
+  float* bias_scales = (float*)malloc(sizeof(float) * (size_t)nb);
+  for (int64_t i = 0; i < nb; ++i) {
+    const float range_weight = fmaxf(fabsf(min_b[i]), fabsf(max_b[i]));
+    bias_scales[i] = (max_int8_input * max_int8_weight) / (range_input * range_weight);
+  }
+  int st = ORC_OK;
+  if (at->input_mode == ORC_MIN_FIRST) { /* :520-601 */
+    const float q_min_input = max_int8_input * min_a / range_input; /* :557 */
+    for (int64_t j = 0; j < N; ++j) {
+      const float sj = (nb != N) ? bias_scales[0] : bias_scales[j]; /* :561-565 */
+      const float sum = (float)colsum[j];                            /* int * float */
+      if (out_f32) {
+        bias_out[j] = bias[j] + (sum * q_min_input / sj);            /* :578-580 */
+      } else if (out_q8) {
+        if (ep->n_scales == 0) { st = ORC_INVALID_ARGUMENT; break; } /* out-of-bounds upstream */
+        const float os = (ep->n_scales == 1) ? scales[0] : scales[j];
+        bias_out[j] = bias[j] * sj * os + (sum * q_min_input * os);  /* :583-595 */
+      } else {
+        bias_out[j] = bias[j] * sj + (sum * q_min_input);            /* :597-599 */
+      }
+    }
+  } else { /* :602-634: reorder of a {1,N} bias with source scales */
+    /* mask 0 for one weight scale; mask 1 otherwise, which selects dimension 0 of extent 1, so a
+     * single scale (the first) applies to all N entries.  Parity unpinned for nb > 1. */
+    for (int64_t j = 0; j < N; ++j) bias_out[j] = bias[j] * bias_scales[0];
+  }
+  free(bias_scales);
+  return st;
+}
+
+static inline float apply_eltwise(const orc_eltwise* e, float x) {
+  switch (e->alg) {
+    case ORC_ELT_RELU:  /* eltwise_relu: x > 0 ? x : x * alpha; alpha == 0 is max(x, 0) */
+      if (e->alpha == 0.0f) return fmaxf(x, 0.0f);
+      return x > 0.0f ? x : x * e->alpha;
+    case ORC_ELT_CLIP:  /* eltwise_clip_v2(alpha = low, beta = high) */
+      return fminf(fmaxf(x, e->alpha), e->beta);
+    case ORC_ELT_LINEAR: /* alpha * x + beta */
+      return e->alpha * x + e->beta;
+    default: return x;
+  }
+}
+
+/* oneDNN int8 inner-product epilogue (execute at quantized_matmul_common.h:92):
+ * y = fl(fl((float)acc * scale[n]) + bias[n]) -> eltwise chain -> destination conversion. */
+void orc_qmatmul_epilogue(const int32_t* acc, int64_t M, int64_t N, const orc_epilogue_desc* ep,
+                          const float* scales, const float* bias, int t_out, void* out) {
+  float lo = 0, hi = 0;
+  if (t_out != ORC_FLOAT) sat_bounds(t_out, &lo, &hi);
+#pragma omp parallel for schedule(static)
+  for (int64_t m = 0; m < M; ++m) {
+    for (int64_t n = 0; n < N; ++n) {
+      float y = (float)acc[m * N + n];
+      if (ep->n_scales == 1) y = y * scales[0];
+      else if (ep->n_scales > 1) y = y * scales[n];
+      y = y + bias[n];
+      for (int e = 0; e < ep->n_eltwise; ++e) y = apply_eltwise(&ep->elt[e], y);
+      if (t_out == ORC_FLOAT) ((float*)out)[m * N + n] = y;
+      else store_q(out, m * N + n, t_out, sat_rne(y, lo, hi));
+    }
+  }
+}
+
+/* OneDnnFloatForOneQuantizedLevel<T>, itex/core/kernels/onednn/block/quantized_ops.h:24-38 */
+static float float_for_one_level(int T, float range_min, float range_max) {
+  int64_t highest = q_highest(T), lowest = q_lowest(T);
+  if (lowest < -highest) ++lowest;
+  return (range_max - range_min) / (float)(highest - lowest);
+}
+
+/* AllocateNativeOutputMinMax, quantized_ops.h:142-203 (+ :40-83 for the qint32 ranges).
+ * n_out receives the number of entries written (0 for fp32 output, which has no min/max). */
+int orc_qmatmul_output_minmax(const orc_matmul_attrs* at, float min_a, float max_a,
+                              const float* min_b, const float* max_b, int64_t nb, int b_rank,
+                              float min_out, float max_out, float* out_min, float* out_max,
+                              int64_t* n_out) {
+  if (at->t_out == ORC_QINT8 || at->t_out == ORC_QUINT8) {
+    out_min[0] = min_out;
+    out_max[0] = max_out;
+    *n_out = 1;
+  } else if (at->t_out == ORC_QINT32) {
+    const int64_t cnt = (b_rank == 0) ? 1 : nb;
+    for (int64_t n = 0; n < cnt; ++n) {
+      const float a_level = float_for_one_level(at->t_in, min_a, max_a);
+      const float b_level = float_for_one_level(ORC_QINT8, min_b[n], max_b[n]);
+      const float c_level = a_level * b_level;
+      out_min[n] = c_level * (float)q_lowest(ORC_QINT32);
+      out_max[n] = c_level * (float)q_highest(ORC_QINT32);
+    }
+    *n_out = cnt;
+  } else if (at->t_out == ORC_FLOAT) {
+    *n_out = 0;
+  } else {
+    return ORC_INVALID_ARGUMENT;
+  }
+  return ORC_OK;
+}
+
+/* LegacyQuantizedMatMulOpBase::Compute, quantized_matmul_common.h:61-102 — whole op. */
+int orc_qmatmul(const orc_matmul_attrs* at, const void* a, const int8_t* w, int transpose_b,
+                int64_t M, int64_t K, int64_t N, const float* bias, float min_a, float max_a,
+                const float* min_b, const float* max_b, int64_t nb, float min_out, float max_out,
+                void* out) {
+  /* the compensation loop indexes the weight as [K,N] regardless of transpose_b (:569-573) */
+  if (transpose_b && at->input_mode == ORC_MIN_FIRST) return ORC_UNIMPLEMENTED;
+  int32_t* acc = (int32_t*)malloc(sizeof(int32_t) * (size_t)(M * N));
+  int32_t* colsum = (int32_t*)malloc(sizeof(int32_t) * (size_t)N);
+  float* scales = (float*)malloc(sizeof(float) * (size_t)(nb > 0 ? nb : 1));
+  float* sb = (float*)malloc(sizeof(float) * (size_t)N);
+  orc_epilogue_desc ep;
+  if (!transpose_b) orc_weight_colsum(w, K, N, colsum);
+  else memset(colsum, 0, sizeof(int32_t) * (size_t)N);
+  int st = orc_qmatmul_prepare(at, N, colsum, min_a, max_a, min_b, max_b, nb, min_out, max_out,
+                               bias, scales, sb, &ep);
+  if (st == ORC_OK) {
+    orc_int_gemm(a, at->t_in, w, transpose_b, M, K, N, acc);
+    orc_qmatmul_epilogue(acc, M, N, &ep, scales, sb, at->t_out, out);
+  }
+  free(acc); free(colsum); free(scales); free(sb);
+  return st;
+}

@@ -1,0 +1,122 @@
+/*
+ * CPU oracle for the INT8 quantized-inference path of intel-extension-for-tensorflow (ITEX).
+ *
+ * TEST INFRASTRUCTURE ONLY.  This library is a plain-C restatement of what the reference
+ * computes on its CPU (oneDNN) path.  It is the checker for the HIP kernels and the timed
+ * "cpu_baseline" of the benchmark; nothing in the shipped library links, loads or calls it.
+ *
+ * Every function cites the reference file:line it follows (paths relative to the reference
+ * tree).  The arithmetic that the reference delegates to oneDNN (reorder, binary,
+ * inner_product_forward; oneDNN is not vendored in the reference tree, pinned at commit
+ * 242d4d9 by itex/workspace.bzl:64-75) is restated from oneDNN's documented int8 semantics:
+ *   exact int32 accumulation;  y = fl(fl((float)acc * scale[oc]) + bias[oc]);
+ *   eltwise post-ops in order;  saturate to the destination type;  round to nearest even.
+ *
+ * Parity pins (see tests/test_oracle_*.py):
+ *   - QuantizeV2 / Dequantize: the reference's own golden vectors
+ *     (test/tensorflow/python/kernel_tests/block_layout/quantized_ops_test.py:49-268,
+ *      dequantize_op_test.py:102-170).
+ *   - integer GEMM: brute force against numpy int64.
+ *   - parameter math: closed forms evaluated independently in numpy float32/float64.
+ *   - epilogue order (multiply, then add, separately rounded; saturate; RNE) is cross-checked
+ *     against the oneDNN build bundled with PyTorch where that is importable.
+ * Parity unpinned (no reference-held vector and no way to execute oneDNN@242d4d9 here):
+ *   NaN / Inf inputs to the quantizers; the result of the size-mismatched bias reorder in
+ *   orc_qmatmul_prepare (SCALED input, per-channel weights; see the comment there);
+ *   abs(INT32_MIN) in orc_requantization_range_per_channel (undefined behaviour upstream).
+ */
+#ifndef ITEX_ORACLE_H_
+#define ITEX_ORACLE_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* TF_DataType values used at the op boundary (tensorflow/c/tf_datatype.h). */
+enum { ORC_FLOAT = 1, ORC_INT32 = 3, ORC_QINT8 = 11, ORC_QUINT8 = 12, ORC_QINT32 = 13 };
+/* QuantizeMode, same order as itex/core/utils/quantization_util.h:29-33. */
+enum { ORC_MIN_COMBINED = 0, ORC_MIN_FIRST = 1, ORC_SCALED = 2 };
+/* status */
+enum { ORC_OK = 0, ORC_INVALID_ARGUMENT = 3, ORC_UNIMPLEMENTED = 12 };
+
+/* Which kernel class of quantized_matmul_common.h prepares the epilogue. */
+enum {
+  ORC_API_V2 = 0,     /* QuantizedFusedMatMulV2Op: _QuantizedMatMul, _ITEXQuantizedMatMul */
+  ORC_API_V1 = 1,     /* QuantizedFusedMatMulOp: _QuantizedFusedMatMul{,AndRequantize,AndDequantize} */
+  ORC_API_LEGACY = 2  /* QuantizedMatMulOp / QuantizedMatMulReluOp: QuantizedMatMulWithBias* */
+};
+
+/* eltwise post-op algorithms (subset of onednn_post_op_util.cc:34-68) */
+enum { ORC_ELT_RELU = 1, ORC_ELT_CLIP = 2, ORC_ELT_LINEAR = 3 };
+/* activation names accepted in fused_ops */
+enum { ORC_ACT_NONE = 0, ORC_ACT_RELU = 1, ORC_ACT_RELU6 = 2, ORC_ACT_LEAKYRELU = 3 };
+
+typedef struct {
+  int alg;
+  float alpha;
+  float beta;
+} orc_eltwise;
+
+typedef struct {
+  int api;               /* ORC_API_* */
+  int t_in;              /* ORC_QUINT8 | ORC_QINT8 (T1) */
+  int t_out;             /* ORC_QINT32 | ORC_QINT8 | ORC_QUINT8 | ORC_FLOAT */
+  int input_mode;        /* ORC_MIN_FIRST | ORC_SCALED */
+  int out_min_first;     /* V2 only: output_quant_mode == "MIN_FIRST" */
+  int activation;        /* ORC_ACT_* fused after BiasAdd */
+  int has_requantize;    /* V2: "Requantize" in fused_ops */
+  int has_dequantize;    /* V2: "Dequantize" in fused_ops */
+  int n_fused_ops;       /* V1: fused_ops.size() (1 = BiasAdd only, 2 = BiasAdd + activation) */
+  float leakyrelu_alpha;
+} orc_matmul_attrs;
+
+typedef struct {
+  int n_scales;          /* 0 (no output scale), 1 (per tensor) or N (per output channel) */
+  int n_eltwise;         /* 0..2 */
+  orc_eltwise elt[2];
+} orc_epilogue_desc;
+
+int orc_adjust_input_range(float in_min, float in_max, float ensure_minimum_range,
+                           float* adj_min, float* adj_max);
+int orc_scale_zeropoint_align(int T, int mode, int dequantize, float* min_data, float* max_data,
+                              int length, float* scales, int32_t* zero_points);
+float orc_legacy_min_first_scale(int T, float adj_min, float adj_max);
+
+int orc_quantize_v2(const float* x, int64_t outer, int64_t slices, int64_t inner, int T, int mode,
+                    int classic_asymmetric, float ensure_minimum_range, const float* in_min,
+                    const float* in_max, void* q, float* out_min, float* out_max);
+int orc_dequantize(const void* q, int64_t outer, int64_t slices, int64_t inner, int T, int mode,
+                   const float* in_min, const float* in_max, float* y);
+
+int orc_requantize_per_channel(const int32_t* x, int64_t rows, int64_t depth, const float* in_min,
+                               const float* in_max, float req_min, float req_max, int out_type,
+                               void* q, float* out_min, float* out_max);
+int orc_requantization_range_per_channel(const int32_t* x, int64_t rows, int64_t depth,
+                                         const float* in_min, const float* in_max,
+                                         float clip_value_max, float* out_min, float* out_max);
+
+void orc_int_gemm(const void* a, int a_type, const int8_t* w, int transpose_b, int64_t M, int64_t K,
+                  int64_t N, int32_t* acc);
+void orc_weight_colsum(const int8_t* w, int64_t K, int64_t N, int32_t* colsum);
+
+int orc_qmatmul_prepare(const orc_matmul_attrs* at, int64_t N, const int32_t* colsum, float min_a,
+                        float max_a, const float* min_b, const float* max_b, int64_t nb,
+                        float min_out, float max_out, const float* bias, float* scales,
+                        float* bias_out, orc_epilogue_desc* ep);
+void orc_qmatmul_epilogue(const int32_t* acc, int64_t M, int64_t N, const orc_epilogue_desc* ep,
+                          const float* scales, const float* bias, int t_out, void* out);
+int orc_qmatmul_output_minmax(const orc_matmul_attrs* at, float min_a, float max_a,
+                              const float* min_b, const float* max_b, int64_t nb, int b_rank,
+                              float min_out, float max_out, float* out_min, float* out_max,
+                              int64_t* n_out);
+int orc_qmatmul(const orc_matmul_attrs* at, const void* a, const int8_t* w, int transpose_b,
+                int64_t M, int64_t K, int64_t N, const float* bias, float min_a, float max_a,
+                const float* min_b, const float* max_b, int64_t nb, float min_out, float max_out,
+                void* out);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ITEX_ORACLE_H_ */

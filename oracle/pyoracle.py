@@ -1,0 +1,227 @@
+"""ctypes binding of the CPU oracle (oracle/libitex_oracle.so).
+
+Test infrastructure only: imported by tests/, by __graft_entry__.smoke() and by the cpu_baseline leg
+of bench.py, always as the checker or the timed CPU baseline, never by the shipped library.
+"""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "libitex_oracle.so")
+
+FLOAT, INT32, QINT8, QUINT8, QINT32 = 1, 3, 11, 12, 13
+MIN_COMBINED, MIN_FIRST, SCALED = 0, 1, 2
+API_V2, API_V1, API_LEGACY = 0, 1, 2
+ACT_NONE, ACT_RELU, ACT_RELU6, ACT_LEAKYRELU = 0, 1, 2, 3
+OK, INVALID_ARGUMENT, UNIMPLEMENTED = 0, 3, 12
+
+NP_OF = {QINT8: np.int8, QUINT8: np.uint8, QINT32: np.int32, FLOAT: np.float32}
+
+
+def build():
+    """Compile the oracle with its Makefile (gcc, contraction off)."""
+    subprocess.run(["make", "-C", _HERE, "-B", "libitex_oracle.so"], check=True,
+                   stdout=subprocess.DEVNULL)
+
+
+class Eltwise(C.Structure):
+    _fields_ = [("alg", C.c_int), ("alpha", C.c_float), ("beta", C.c_float)]
+
+
+class MatmulAttrs(C.Structure):
+    _fields_ = [("api", C.c_int), ("t_in", C.c_int), ("t_out", C.c_int), ("input_mode", C.c_int),
+                ("out_min_first", C.c_int), ("activation", C.c_int), ("has_requantize", C.c_int),
+                ("has_dequantize", C.c_int), ("n_fused_ops", C.c_int),
+                ("leakyrelu_alpha", C.c_float)]
+
+
+class EpilogueDesc(C.Structure):
+    _fields_ = [("n_scales", C.c_int), ("n_eltwise", C.c_int), ("elt", Eltwise * 2)]
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB_PATH):
+            build()
+        _lib = C.CDLL(_LIB_PATH)
+        _lib.orc_legacy_min_first_scale.restype = C.c_float
+        _lib.orc_legacy_min_first_scale.argtypes = [C.c_int, C.c_float, C.c_float]
+    return _lib
+
+
+def _p(a):
+    return a.ctypes.data_as(C.c_void_p)
+
+
+def _f32(v):
+    return np.ascontiguousarray(np.atleast_1d(np.asarray(v, dtype=np.float32)))
+
+
+def adjust_input_range(mn, mx, ensure_minimum_range=0.01):
+    a, b = C.c_float(), C.c_float()
+    st = lib().orc_adjust_input_range(C.c_float(mn), C.c_float(mx), C.c_float(ensure_minimum_range),
+                                      C.byref(a), C.byref(b))
+    return st, np.float32(a.value), np.float32(b.value)
+
+
+def scale_zeropoint_align(T, mode, dequantize, mn, mx):
+    mn, mx = _f32(mn).copy(), _f32(mx).copy()
+    n = mn.size
+    sc = np.zeros(n, np.float32)
+    zp = np.zeros(n, np.int32)
+    st = lib().orc_scale_zeropoint_align(T, mode, int(dequantize), _p(mn), _p(mx), n, _p(sc), _p(zp))
+    return st, mn, mx, sc, zp
+
+
+def legacy_min_first_scale(T, mn, mx):
+    return np.float32(lib().orc_legacy_min_first_scale(T, C.c_float(mn), C.c_float(mx)))
+
+
+def _split(shape, axis):
+    shape = tuple(int(s) for s in shape)
+    if axis is None or axis < 0:
+        return 1, 1, int(np.prod(shape, dtype=np.int64))
+    outer = int(np.prod(shape[:axis], dtype=np.int64))
+    inner = int(np.prod(shape[axis + 1:], dtype=np.int64))
+    return outer, shape[axis], inner
+
+
+def quantize_v2(x, mn, mx, T, mode, axis=None, classic=False, ensure_minimum_range=0.01):
+    """Returns (status, q, out_min, out_max)."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    outer, slices, inner = _split(x.shape, axis)
+    mn, mx = _f32(mn), _f32(mx)
+    assert mn.size == slices and mx.size == slices
+    q = np.zeros(x.shape, NP_OF[T])
+    omn, omx = np.zeros(slices, np.float32), np.zeros(slices, np.float32)
+    st = lib().orc_quantize_v2(_p(x), C.c_int64(outer), C.c_int64(slices), C.c_int64(inner), T, mode,
+                               int(classic), C.c_float(ensure_minimum_range), _p(mn), _p(mx), _p(q),
+                               _p(omn), _p(omx))
+    return st, q, omn, omx
+
+
+def dequantize(q, mn, mx, T, mode, axis=None):
+    q = np.ascontiguousarray(q, dtype=NP_OF[T])
+    outer, slices, inner = _split(q.shape, axis)
+    mn, mx = _f32(mn), _f32(mx)
+    assert mn.size == slices and mx.size == slices
+    y = np.zeros(q.shape, np.float32)
+    st = lib().orc_dequantize(_p(q), C.c_int64(outer), C.c_int64(slices), C.c_int64(inner), T, mode,
+                              _p(mn), _p(mx), _p(y))
+    return st, y
+
+
+def requantize_per_channel(x, in_min, in_max, req_min, req_max, out_type):
+    x = np.ascontiguousarray(x, dtype=np.int32)
+    depth = x.shape[-1]
+    rows = x.size // depth
+    in_min, in_max = _f32(in_min), _f32(in_max)
+    assert in_min.size == depth and in_max.size == depth
+    q = np.zeros(x.shape, NP_OF[out_type])
+    omn, omx = C.c_float(), C.c_float()
+    st = lib().orc_requantize_per_channel(_p(x), C.c_int64(rows), C.c_int64(depth), _p(in_min),
+                                          _p(in_max), C.c_float(req_min), C.c_float(req_max),
+                                          out_type, _p(q), C.byref(omn), C.byref(omx))
+    return st, q, np.float32(omn.value), np.float32(omx.value)
+
+
+def requantization_range_per_channel(x, in_min, in_max, clip_value_max):
+    x = np.ascontiguousarray(x, dtype=np.int32)
+    depth = x.shape[-1]
+    rows = x.size // depth
+    in_min, in_max = _f32(in_min), _f32(in_max)
+    omn, omx = C.c_float(), C.c_float()
+    st = lib().orc_requantization_range_per_channel(_p(x), C.c_int64(rows), C.c_int64(depth),
+                                                    _p(in_min), _p(in_max),
+                                                    C.c_float(clip_value_max), C.byref(omn),
+                                                    C.byref(omx))
+    return st, np.float32(omn.value), np.float32(omx.value)
+
+
+def int_gemm(a, w, transpose_b=False):
+    a = np.ascontiguousarray(a)
+    w = np.ascontiguousarray(w, dtype=np.int8)
+    a_type = QUINT8 if a.dtype == np.uint8 else QINT8
+    M, K = a.shape
+    N = w.shape[0] if transpose_b else w.shape[1]
+    acc = np.zeros((M, N), np.int32)
+    lib().orc_int_gemm(_p(a), a_type, _p(w), int(transpose_b), C.c_int64(M), C.c_int64(K),
+                       C.c_int64(N), _p(acc))
+    return acc
+
+
+def weight_colsum(w):
+    w = np.ascontiguousarray(w, dtype=np.int8)
+    K, N = w.shape
+    cs = np.zeros(N, np.int32)
+    lib().orc_weight_colsum(_p(w), C.c_int64(K), C.c_int64(N), _p(cs))
+    return cs
+
+
+def matmul_attrs(api=API_V2, t_in=QUINT8, t_out=FLOAT, input_mode=MIN_FIRST, out_min_first=False,
+                 activation=ACT_NONE, has_requantize=False, has_dequantize=False, n_fused_ops=1,
+                 leakyrelu_alpha=0.2):
+    return MatmulAttrs(api, t_in, t_out, input_mode, int(out_min_first), activation,
+                       int(has_requantize), int(has_dequantize), n_fused_ops, leakyrelu_alpha)
+
+
+def qmatmul_prepare(at, N, colsum, min_a, max_a, min_b, max_b, min_out, max_out, bias):
+    """Returns (status, scales[n_scales], scaled_bias[N], EpilogueDesc)."""
+    min_b, max_b = _f32(min_b), _f32(max_b)
+    nb = min_b.size
+    bias = _f32(bias)
+    colsum = np.ascontiguousarray(colsum, dtype=np.int32)
+    scales = np.zeros(max(nb, 1), np.float32)
+    sb = np.zeros(N, np.float32)
+    ep = EpilogueDesc()
+    st = lib().orc_qmatmul_prepare(C.byref(at), C.c_int64(N), _p(colsum), C.c_float(min_a),
+                                   C.c_float(max_a), _p(min_b), _p(max_b), C.c_int64(nb),
+                                   C.c_float(min_out), C.c_float(max_out), _p(bias), _p(scales),
+                                   _p(sb), C.byref(ep))
+    return st, scales[:ep.n_scales].copy(), sb, ep
+
+
+def qmatmul_epilogue(acc, ep, scales, bias, t_out):
+    acc = np.ascontiguousarray(acc, dtype=np.int32)
+    M, N = acc.shape
+    scales = _f32(scales) if ep.n_scales else np.zeros(1, np.float32)
+    bias = _f32(bias)
+    out = np.zeros((M, N), NP_OF[t_out])
+    lib().orc_qmatmul_epilogue(_p(acc), C.c_int64(M), C.c_int64(N), C.byref(ep), _p(scales),
+                               _p(bias), t_out, _p(out))
+    return out
+
+
+def qmatmul_output_minmax(at, min_a, max_a, min_b, max_b, b_rank, min_out, max_out):
+    min_b, max_b = _f32(min_b), _f32(max_b)
+    nb = min_b.size
+    omn, omx = np.zeros(max(nb, 1), np.float32), np.zeros(max(nb, 1), np.float32)
+    n_out = C.c_int64()
+    st = lib().orc_qmatmul_output_minmax(C.byref(at), C.c_float(min_a), C.c_float(max_a), _p(min_b),
+                                         _p(max_b), C.c_int64(nb), b_rank, C.c_float(min_out),
+                                         C.c_float(max_out), _p(omn), _p(omx), C.byref(n_out))
+    return st, omn[:n_out.value].copy(), omx[:n_out.value].copy()
+
+
+def qmatmul(at, a, w, bias, min_a, max_a, min_b, max_b, min_out=0.0, max_out=0.0,
+            transpose_b=False):
+    """Whole op.  Returns (status, out[M,N])."""
+    a = np.ascontiguousarray(a)
+    w = np.ascontiguousarray(w, dtype=np.int8)
+    M, K = a.shape
+    N = w.shape[0] if transpose_b else w.shape[1]
+    min_b, max_b = _f32(min_b), _f32(max_b)
+    bias = _f32(bias)
+    out = np.zeros((M, N), NP_OF[at.t_out])
+    st = lib().orc_qmatmul(C.byref(at), _p(a), _p(w), int(transpose_b), C.c_int64(M), C.c_int64(K),
+                           C.c_int64(N), _p(bias), C.c_float(min_a), C.c_float(max_a), _p(min_b),
+                           _p(max_b), C.c_int64(min_b.size), C.c_float(min_out), C.c_float(max_out),
+                           _p(out))
+    return st, out

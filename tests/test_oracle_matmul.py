@@ -1,0 +1,251 @@
+"""Pins the CPU oracle's quantized MatMul restatement.
+
+  * integer GEMM: brute force against numpy int64 (exact);
+  * MIN_FIRST zero-point compensation and the output scale: the reference-held 2x3 . 3x4 case of
+    native_quantized_fused_matmul_test.py must reproduce the fp32 product within the reference's own
+    tolerance (0.2) and, tighter, within the bound the quantization steps allow -- a dropped or
+    sign-flipped compensation term misses by > 1;
+  * requantize scaling: dequantizing the int8 output with the frozen range must reproduce the fp32
+    product to half an output step (+ input quantization noise);
+  * the documented quirks (bias inflation for SCALED input, lost requantize factor behind an
+    activation) are asserted through their observable consequence, not by retyping the formula;
+  * epilogue order against the oneDNN bundled in PyTorch (skipped if that op is unavailable).
+"""
+import numpy as np
+import pytest
+
+from oracle import pyoracle as orc
+
+
+def quant_weights_per_channel(w):
+    r = np.max(np.abs(w), axis=0).astype(np.float32)
+    _, q, mn, mx = orc.quantize_v2(w, -r, r, orc.QINT8, orc.SCALED, axis=1)
+    return q, mn, mx
+
+
+def quant_weights_per_tensor(w):
+    _, q, mn, mx = orc.quantize_v2(w, w.min(), w.max(), orc.QINT8, orc.SCALED)
+    return q, mn, mx
+
+
+@pytest.mark.parametrize("a_dtype", [np.uint8, np.int8])
+@pytest.mark.parametrize("transpose_b", [False, True])
+def test_int_gemm_brute_force(a_dtype, transpose_b):
+    rng = np.random.default_rng(0)
+    for (M, K, N) in [(1, 1, 1), (3, 17, 5), (16, 64, 48), (7, 129, 33)]:
+        info = np.iinfo(a_dtype)
+        a = rng.integers(info.min, info.max + 1, size=(M, K)).astype(a_dtype)
+        w = rng.integers(-128, 128, size=(K, N)).astype(np.int8)
+        ref = a.astype(np.int64) @ w.astype(np.int64)
+        got = orc.int_gemm(a, np.ascontiguousarray(w.T) if transpose_b else w, transpose_b)
+        np.testing.assert_array_equal(got.astype(np.int64), ref)
+    # extreme values: no overflow at the largest K of the configs
+    K = 14336
+    a = np.full((1, K), 255, np.uint8)
+    w = np.full((K, 2), -128, np.int8)
+    w[:, 1] = 127
+    got = orc.int_gemm(a, w)
+    assert got.tolist() == [[255 * -128 * K, 255 * 127 * K]]
+
+
+def test_colsum():
+    rng = np.random.default_rng(1)
+    w = rng.integers(-128, 128, size=(300, 37)).astype(np.int8)
+    np.testing.assert_array_equal(orc.weight_colsum(w), w.astype(np.int64).sum(0))
+
+
+@pytest.mark.parametrize("per_channel", [False, True])
+@pytest.mark.parametrize("api", [orc.API_V1, orc.API_V2])
+def test_reference_fused_matmul_case(golden, per_channel, api):
+    g = golden["fused_matmul"]
+    x = np.array(g["x"], np.float32)
+    w = np.array(g["w"], np.float32)
+    b = np.array(g["bias"], np.float32)
+    st, xq, xmn, xmx = orc.quantize_v2(x, x.min(), x.max(), orc.QUINT8, orc.MIN_FIRST)
+    assert xq.tolist() == [[218, 180, 0], [146, 165, 255]]
+    if per_channel:
+        # the reference test quantizes with (min, max) per column, axis=1
+        _, wq, wmn, wmx = orc.quantize_v2(w, w.min(0), w.max(0), orc.QINT8, orc.SCALED, axis=1)
+    else:
+        wq, wmn, wmx = quant_weights_per_tensor(w)
+    at = orc.matmul_attrs(api=api, t_in=orc.QUINT8, t_out=orc.FLOAT, input_mode=orc.MIN_FIRST,
+                          has_dequantize=True, n_fused_ops=1)
+    st, y = orc.qmatmul(at, xq, wq, b, xmn[0], xmx[0], wmn, wmx)
+    assert st == orc.OK
+    ref = x @ w + b
+    err = np.max(np.abs(y - ref))
+    assert err < g["tolerance"]
+    # quantization-noise bound: K * (step_x/2 * |w|max + step_w/2 * |x|max) is ~0.1 here
+    assert err < 0.06
+    # a missing compensation term would be off by about |min_a| * colsum(w) ~ 1
+    assert np.max(np.abs(y - ref)) < 0.1 * np.max(np.abs(0.66 * w.sum(0)))
+
+
+def test_requantize_output_scale_round_trip():
+    rng = np.random.default_rng(4)
+    M, K, N = 32, 256, 48
+    x = rng.standard_normal((M, K)).astype(np.float32)
+    w = (rng.standard_normal((K, N)) * 0.05).astype(np.float32)
+    b = (rng.standard_normal(N) * 0.1).astype(np.float32)
+    _, xq, xmn, xmx = orc.quantize_v2(x, x.min(), x.max(), orc.QUINT8, orc.MIN_FIRST)
+    wq, wmn, wmx = quant_weights_per_channel(w)
+    ref = x @ w + b
+    r_out = float(np.max(np.abs(ref)))
+    for api in (orc.API_V1, orc.API_V2):
+        at = orc.matmul_attrs(api=api, t_in=orc.QUINT8, t_out=orc.QINT8, input_mode=orc.MIN_FIRST,
+                              has_requantize=True, n_fused_ops=1)
+        st, q = orc.qmatmul(at, xq, wq, b, xmn[0], xmx[0], wmn, wmx, -r_out, r_out)
+        assert st == orc.OK
+        st, y = orc.dequantize(q, -r_out, r_out, orc.QINT8, orc.SCALED)
+        assert np.max(np.abs(y - ref)) < 0.5 * r_out / 127 + 0.08
+        st, omn, omx = orc.qmatmul_output_minmax(at, xmn[0], xmx[0], wmn, wmx, 1, -r_out, r_out)
+        assert (omn[0], omx[0]) == (np.float32(-r_out), np.float32(r_out))
+
+
+def test_s32_output_range_and_values():
+    rng = np.random.default_rng(9)
+    M, K, N = 4, 64, 8
+    xq = rng.integers(0, 256, size=(M, K)).astype(np.uint8)
+    wq = rng.integers(-127, 128, size=(K, N)).astype(np.int8)
+    zero_bias = np.zeros(N, np.float32)
+    # SCALED input + zero bias: the s32 output is the accumulator (|acc| < 2^24 here -> exact)
+    at = orc.matmul_attrs(api=orc.API_V1, t_in=orc.QUINT8, t_out=orc.QINT32, input_mode=orc.SCALED,
+                          n_fused_ops=1)
+    st, y = orc.qmatmul(at, xq, wq, zero_bias, 0.0, 2.0, [-1.0], [1.0])
+    np.testing.assert_array_equal(y, xq.astype(np.int64) @ wq.astype(np.int64))
+    st, omn, omx = orc.qmatmul_output_minmax(at, 0.0, 2.0, [-1.0], [1.0], 0, 0, 0)
+    lvl = np.float32(np.float32(2.0) / np.float32(255)) * np.float32(np.float32(2.0) / np.float32(254))
+    assert omn[0] == np.float32(lvl * np.float32(-2**31)) and omx[0] == np.float32(lvl * np.float32(2**31))
+    st, omn, omx = orc.qmatmul_output_minmax(at, 0.0, 2.0, [-1.0] * N, [1.0] * N, 1, 0, 0)
+    assert omn.size == N
+
+
+def test_quirk_scaled_input_inflates_bias():
+    # SCALED input + fp32 bias: bias is multiplied by A*127/(r_in*r_w) (oneDNN-2.x-era scaling) while
+    # the primitive adds it after scaling.  Observable: doubling the bias moves the fp32 output by
+    # bias * bs, not by bias.
+    rng = np.random.default_rng(6)
+    M, K, N = 4, 32, 8
+    xq = rng.integers(-127, 128, size=(M, K)).astype(np.int8)
+    wq = rng.integers(-127, 128, size=(K, N)).astype(np.int8)
+    b = rng.standard_normal(N).astype(np.float32)
+    at = orc.matmul_attrs(api=orc.API_V2, t_in=orc.QINT8, t_out=orc.FLOAT, input_mode=orc.SCALED,
+                          has_dequantize=True)
+    _, y0 = orc.qmatmul(at, xq, wq, np.zeros(N, np.float32), -2.0, 2.0, [-0.5], [0.5])
+    _, y1 = orc.qmatmul(at, xq, wq, b, -2.0, 2.0, [-0.5], [0.5])
+    bs = 127.0 * 127.0 / (2.0 * 0.5)
+    np.testing.assert_allclose(y1 - y0, np.broadcast_to(b * bs, (M, N)), rtol=1e-4, atol=1e-2)
+    # per-channel weights: the single scale bs[0] applies to every channel
+    mb = np.linspace(0.25, 1.0, N).astype(np.float32)
+    _, z0 = orc.qmatmul(at, xq, wq, np.zeros(N, np.float32), -2.0, 2.0, -mb, mb)
+    _, z1 = orc.qmatmul(at, xq, wq, b, -2.0, 2.0, -mb, mb)
+    bs0 = 127.0 * 127.0 / (2.0 * 0.25)
+    np.testing.assert_allclose(z1 - z0, np.broadcast_to(b * bs0, (M, N)), rtol=1e-4, atol=1e-2)
+
+
+def test_quirk_activation_drops_requantize_factor():
+    # [BiasAdd, Relu, Requantize]: the 255/r_out factor is lost, the u8 output is relu(y) in real
+    # units (saturated), while [BiasAdd, Requantize] applies it.
+    rng = np.random.default_rng(8)
+    M, K, N = 8, 64, 16
+    x = rng.standard_normal((M, K)).astype(np.float32)
+    w = (rng.standard_normal((K, N)) * 0.3).astype(np.float32)
+    _, xq, xmn, xmx = orc.quantize_v2(x, x.min(), x.max(), orc.QUINT8, orc.MIN_FIRST)
+    wq, wmn, wmx = quant_weights_per_channel(w)
+    zero = np.zeros(N, np.float32)
+    ref = np.maximum(x @ w, 0)
+    r_out = float(ref.max())
+    at = orc.matmul_attrs(api=orc.API_V2, t_in=orc.QUINT8, t_out=orc.QUINT8, input_mode=orc.MIN_FIRST,
+                          activation=orc.ACT_RELU, has_requantize=True, n_fused_ops=2)
+    _, q = orc.qmatmul(at, xq, wq, zero, xmn[0], xmx[0], wmn, wmx, 0.0, r_out)
+    assert np.max(np.abs(q.astype(np.float32) - np.clip(np.rint(ref), 0, 255))) <= 1
+    at1 = orc.matmul_attrs(api=orc.API_V1, t_in=orc.QUINT8, t_out=orc.QUINT8, input_mode=orc.MIN_FIRST,
+                           activation=orc.ACT_RELU, has_requantize=True, n_fused_ops=2)
+    _, q1 = orc.qmatmul(at1, xq, wq, zero, xmn[0], xmx[0], wmn, wmx, 0.0, r_out)
+    np.testing.assert_array_equal(q, q1)
+    # legacy QuantizedMatMulWithBiasAndReluAndRequantize is not affected (factor lives in the output scale)
+    wq1, wmn1, wmx1 = quant_weights_per_tensor(w)
+    atl = orc.matmul_attrs(api=orc.API_LEGACY, t_in=orc.QUINT8, t_out=orc.QUINT8, input_mode=orc.MIN_FIRST,
+                           activation=orc.ACT_RELU)
+    _, ql = orc.qmatmul(atl, xq, wq1, zero, xmn[0], xmx[0], wmn1, wmx1, 0.0, r_out)
+    _, yl = orc.dequantize(ql, 0.0, r_out, orc.QUINT8, orc.SCALED)
+    # legacy scale uses (max_b-min_b)/254 and (max_a-min_a)/255 levels: a close, not identical, grid
+    assert np.max(np.abs(yl - ref)) < 0.03 * r_out + 0.1
+
+
+def test_min_first_output_linear_overrides_relu_alpha():
+    # output_quant_mode=MIN_FIRST + Requantize appends Linear and its alpha/beta overwrite EVERY
+    # eltwise in the chain (onednn_post_op_util.cc:251-262)
+    at = orc.matmul_attrs(api=orc.API_V2, t_in=orc.QUINT8, t_out=orc.QUINT8, input_mode=orc.MIN_FIRST,
+                          out_min_first=True, activation=orc.ACT_RELU, has_requantize=True)
+    st, sc, sb, ep = orc.qmatmul_prepare(at, 2, [0, 0], 0.0, 1.0, [-1.0], [1.0], -1.0, 3.0, [0.0, 0.0])
+    assert ep.n_eltwise == 2
+    alpha = np.float32(255.0) / np.float32(4.0)
+    beta = np.float32(np.float32(1.0) * np.float32(255.0)) / np.float32(4.0)
+    for e in range(2):
+        assert ep.elt[e].alpha == alpha and ep.elt[e].beta == beta
+    # the output scale carries no requantize factor in that case
+    assert sc[0] == np.float32(np.float32(1.0) * np.float32(1.0)) / np.float32(255.0 * 127.0)
+
+
+def test_epilogue_rounding_and_saturation():
+    ep = orc.EpilogueDesc()
+    ep.n_scales = 1
+    acc = np.array([[1, 3, 5, 7, -1, -3, 600, -600, 2**31 - 1, -2**31]], np.int32)
+    out = orc.qmatmul_epilogue(acc, ep, [0.5], np.zeros(10, np.float32), orc.QINT8)
+    assert out.tolist() == [[0, 2, 2, 4, 0, -2, 127, -128, 127, -128]]
+    out = orc.qmatmul_epilogue(acc, ep, [0.5], np.zeros(10, np.float32), orc.QUINT8)
+    assert out.tolist() == [[0, 2, 2, 4, 0, 0, 255, 0, 255, 0]]
+    # s32 destination goes through fp32: 2^31-1 -> 2^31 in fp32 -> saturates to 2147483520
+    out = orc.qmatmul_epilogue(acc, ep, [1.0], np.zeros(10, np.float32), orc.QINT32)
+    assert out[0, 8] == 2147483520 and out[0, 9] == -2**31 and out[0, 6] == 600
+
+
+def test_epilogue_mul_then_add_not_fused():
+    # pick acc, s, b so that fl(fl(acc*s)+b) != fl(acc*s+b)
+    rng = np.random.default_rng(12)
+    acc = rng.integers(-2**23, 2**23, size=(1, 4096)).astype(np.int32)
+    s = np.float32(0.00123457)
+    b = rng.standard_normal(4096).astype(np.float32)
+    ep = orc.EpilogueDesc()
+    ep.n_scales = 1
+    out = orc.qmatmul_epilogue(acc, ep, [s], b, orc.FLOAT)
+    two_step = ((acc.astype(np.float64) * np.float64(s)).astype(np.float32).astype(np.float64) + b).astype(np.float32)
+    fused = (acc.astype(np.float64) * np.float64(s) + b).astype(np.float32)
+    assert np.any(two_step != fused)
+    np.testing.assert_array_equal(out, two_step)
+
+
+def test_epilogue_against_torch_onednn():
+    """oneDNN 3.x as bundled with PyTorch (a different build than the reference pins; a cross-check
+    of operation order, rounding and saturation, not the definition)."""
+    torch = pytest.importorskip("torch")
+    if not hasattr(torch.ops, "onednn") or not hasattr(torch.ops.onednn, "qlinear_pointwise"):
+        pytest.skip("torch.ops.onednn.qlinear_pointwise unavailable")
+    rng = np.random.default_rng(13)
+    M, K, N = 16, 64, 32
+    xq = rng.integers(0, 256, size=(M, K)).astype(np.uint8)
+    wq = rng.integers(-127, 128, size=(K, N)).astype(np.int8)
+    sw = (rng.random(N).astype(np.float32) * 0.01 + 0.001)
+    b = rng.standard_normal(N).astype(np.float32)
+    try:
+        w_t = torch.from_numpy(np.ascontiguousarray(wq.T))  # [N, K]
+        packed = torch.ops.onednn.qlinear_prepack(w_t, [M, K])
+        outs = {}
+        for post, out_dtype in (("none", torch.float32), ("relu", torch.float32), ("none", torch.uint8)):
+            outs[(post, out_dtype)] = torch.ops.onednn.qlinear_pointwise(
+                torch.from_numpy(xq), 1.0, 0, packed, torch.from_numpy(sw),
+                torch.zeros(N, dtype=torch.int64), torch.from_numpy(b), 1.0, 0, out_dtype, post, [], "")
+    except Exception as e:  # signature differs between torch builds
+        pytest.skip("qlinear_pointwise not callable here: %r" % (e,))
+    acc = orc.int_gemm(xq, wq)
+    ep = orc.EpilogueDesc()
+    ep.n_scales = N
+    np.testing.assert_array_equal(outs[("none", torch.float32)].numpy(),
+                                  orc.qmatmul_epilogue(acc, ep, sw, b, orc.FLOAT))
+    np.testing.assert_array_equal(outs[("none", torch.uint8)].numpy(),
+                                  orc.qmatmul_epilogue(acc, ep, sw, b, orc.QUINT8))
+    ep.n_eltwise = 1
+    ep.elt[0].alg, ep.elt[0].alpha, ep.elt[0].beta = 1, 0.0, 0.0
+    np.testing.assert_array_equal(outs[("relu", torch.float32)].numpy(),
+                                  orc.qmatmul_epilogue(acc, ep, sw, b, orc.FLOAT))
