@@ -1,0 +1,193 @@
+/*
+ * itexhip.h - C ABI of the MI355X (gfx950) kernels behind ITEX's INT8 quantized-inference ops.
+ *
+ * Every entry point takes plain device pointers, sizes, POD parameter structs and a HIP stream
+ * (passed as void*, i.e. a hipStream_t; NULL = the default stream), enqueues its work on that
+ * stream and returns without synchronising.  Return value: 0 on success, otherwise one of the
+ * ITEXHIP_* codes below (the values are TF_Code values so that the op kernels can forward them);
+ * itexhip_last_error() returns a thread-local message for the last failure.
+ *
+ * These functions sit where the reference calls oneDNN primitives; each declaration cites the
+ * reference call site it replaces (paths relative to the reference tree).  The host-side parameter
+ * math (ranges -> scale / zero point / shift) stays in the op kernels, as in the reference.
+ */
+#ifndef ITEXHIP_H_
+#define ITEXHIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* status codes (subset of TF_Code) */
+enum {
+  ITEXHIP_OK = 0,
+  ITEXHIP_INVALID_ARGUMENT = 3,
+  ITEXHIP_UNIMPLEMENTED = 12,
+  ITEXHIP_INTERNAL = 13
+};
+
+/* element types, numbered like TF_DataType */
+enum {
+  ITEXHIP_FLOAT = 1,
+  ITEXHIP_INT32 = 3,
+  ITEXHIP_QINT8 = 11,
+  ITEXHIP_QUINT8 = 12,
+  ITEXHIP_QINT32 = 13
+};
+
+/* QuantizeMode, numbered like itex/core/utils/quantization_util.h:29-33 */
+enum { ITEXHIP_MIN_COMBINED = 0, ITEXHIP_MIN_FIRST = 1, ITEXHIP_SCALED = 2 };
+
+const char* itexhip_last_error(void);
+/* "gfx950" and the library version; no GPU call. */
+const char* itexhip_build_info(void);
+
+/* ------------------------------------------------------------------------------------------
+ * QuantizeV2.  q[i] = sat_T(rne(fl(x[i] * scale) + addend))
+ *   SCALED            : addend = 0            (oneDNN reorder, src scale;
+ *                                              itex/core/kernels/common/quantize_op.h:256-275,394)
+ *   classic MIN_FIRST : addend = (float)zp    (reorder, src scale + dst zero point; :276-291)
+ *   legacy MIN_FIRST  : addend = fl(shift * scale), shift = -min'  (binary_add with both sources
+ *                                              scaled; :292-314, 383-391)
+ * dst_type is ITEXHIP_QINT8 or ITEXHIP_QUINT8.  The per-axis form views the tensor as
+ * [outer, slices, inner] and reads scale[s] / addend[s] from device vectors (addend may be NULL).
+ * ---------------------------------------------------------------------------------------- */
+int itexhip_quantize(const float* x, void* q, int64_t n, int dst_type, float scale, float addend,
+                     void* stream);
+int itexhip_quantize_axis(const float* x, void* q, int64_t outer, int64_t slices, int64_t inner,
+                          int dst_type, const float* scales, const float* addends, void* stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Dequantize.  y[i] = ((float)q[i] - zero_point) * scale
+ * (oneDNN reorder with src scale and src zero point;
+ *  itex/core/kernels/common/dequantize_op.h:129-145,169).  src_type QINT8 or QUINT8.
+ * ---------------------------------------------------------------------------------------- */
+int itexhip_dequantize(const void* q, float* y, int64_t n, int src_type, float scale,
+                       int32_t zero_point, void* stream);
+int itexhip_dequantize_axis(const void* q, float* y, int64_t outer, int64_t slices, int64_t inner,
+                            int src_type, const float* scales, const int32_t* zero_points,
+                            void* stream);
+
+/* ------------------------------------------------------------------------------------------
+ * RequantizePerChannel.  q[r, c] = sat_T(rne((float)x[r, c] * scale[c])), channel = last dim
+ * (oneDNN reorder s32 -> s8/u8 with per-channel src scale;
+ *  itex/core/kernels/onednn/block/requantize_per_channel_op.cc:97-140).
+ * `scales` is a device vector of `depth` floats; depth == 1 is the per-tensor case.
+ * ---------------------------------------------------------------------------------------- */
+int itexhip_requantize_per_channel(const int32_t* x, void* q, int64_t rows, int64_t depth,
+                                   int dst_type, const float* scales, void* stream);
+/* per-tensor form with the scale passed by value */
+int itexhip_requantize(const int32_t* x, void* q, int64_t n, int dst_type, float scale,
+                       void* stream);
+
+/* ------------------------------------------------------------------------------------------
+ * RequantizationRangePerChannel reduction: per channel c (last dim) the minimum and maximum of
+ * x[:, c] (Eigen reductions at
+ * itex/core/kernels/onednn/block/requantization_range_per_channel_op.cc:110-127).
+ * min_out / max_out are device vectors of `depth` int32.  The float range itself is scalar host
+ * math on these 2*depth integers and stays in the op kernel.
+ * itexhip_minmax_f32 is the fp32 counterpart (2 floats: min, max) for computing QuantizeV2 ranges
+ * on the device; NaNs are ignored.
+ * ---------------------------------------------------------------------------------------- */
+int itexhip_minmax_i32_per_channel(const int32_t* x, int64_t rows, int64_t depth, int32_t* min_out,
+                                   int32_t* max_out, void* stream);
+int itexhip_minmax_f32(const float* x, int64_t n, float* minmax_out, void* stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Quantized MatMul (oneDNN inner_product_forward u8/s8 x s8 -> s32 with fused epilogue;
+ * itex/core/kernels/common/quantized_matmul_common.h:223-226 (primitive), :92 (execute)).
+ * ---------------------------------------------------------------------------------------- */
+
+/* Which kernel class prepares the epilogue (quantized_matmul_common.h). */
+enum {
+  ITEXHIP_API_V2 = 0,     /* QuantizedFusedMatMulV2Op (:1711-1909) */
+  ITEXHIP_API_V1 = 1,     /* QuantizedFusedMatMulOp   (:1539-1708) */
+  ITEXHIP_API_LEGACY = 2  /* QuantizedMatMulOp / QuantizedMatMulReluOp (:1412-1531) */
+};
+enum { ITEXHIP_ACT_NONE = 0, ITEXHIP_ACT_RELU = 1, ITEXHIP_ACT_RELU6 = 2, ITEXHIP_ACT_LEAKYRELU = 3 };
+enum { ITEXHIP_ELT_RELU = 1, ITEXHIP_ELT_CLIP = 2, ITEXHIP_ELT_LINEAR = 3 };
+
+typedef struct {
+  int alg;      /* ITEXHIP_ELT_* */
+  float alpha;
+  float beta;
+} itexhip_eltwise;
+
+/* What the fused epilogue applies after the integer accumulation:
+ *   y = fl(fl((float)acc * scale[n]) + bias[n]); eltwise chain; convert to the output type. */
+typedef struct {
+  int n_scales;   /* 0: no scale, 1: scales[0] for all channels, N: per output channel */
+  int n_eltwise;  /* 0..2 */
+  itexhip_eltwise elt[2];
+} itexhip_epilogue;
+
+/* Attributes and host-memory scalars of one quantized MatMul node. */
+typedef struct {
+  int api;             /* ITEXHIP_API_* */
+  int t_in;            /* T1: QUINT8 | QINT8 */
+  int t_out;           /* QINT32 | QINT8 | QUINT8 | FLOAT */
+  int input_mode;      /* input_quant_mode: MIN_FIRST | SCALED */
+  int out_min_first;   /* V2: output_quant_mode == "MIN_FIRST" */
+  int activation;      /* ITEXHIP_ACT_* */
+  int has_requantize;  /* V2: "Requantize" in fused_ops */
+  int has_dequantize;  /* V2: "Dequantize" in fused_ops */
+  int n_fused_ops;     /* V1: fused_ops.size() */
+  float leakyrelu_alpha;
+  float min_a, max_a;      /* host scalars */
+  float min_out, max_out;  /* min/max_freezed_output (requantize) */
+} itexhip_matmul_params;
+
+/* Host-only: the epilogue descriptor (scale count, eltwise chain with the reference's alpha/beta
+ * overrides) for a node; follows ExtendInt8PostOps (quantized_matmul_common.h:1472-1508,
+ * 1610-1702, 1809-1908) and PostOpUtil::SetPostOp
+ * (itex/core/utils/onednn/onednn_post_op_util.cc:237-273).  nb = number of weight ranges. */
+int itexhip_qmatmul_epilogue_desc(const itexhip_matmul_params* p, int64_t nb, itexhip_epilogue* ep);
+
+/* Device: per-channel output scales and the scaled / zero-point-compensated bias
+ * (ExtendInt8PostOps as above; GetScaledBias, quantized_matmul_common.h:466-660), computed by one
+ * small kernel from device copies of min_b / max_b (nb floats each), the fp32 bias (N floats) and
+ * the weight column sums (N int32, from itexhip_qgemm_prepack_b).  Writes `scales_out`
+ * (max(ep.n_scales,1) floats) and `bias_out` (N floats).  No host synchronisation. */
+int itexhip_qmatmul_prepare(const itexhip_matmul_params* p, const float* min_b, const float* max_b,
+                            int64_t nb, const float* bias, const int32_t* colsum, int64_t N,
+                            float* scales_out, float* bias_out, void* stream);
+
+/* Weight prepack: the s8 weight (TF layout [K,N] row-major, or [N,K] when transpose_b) is
+ * rearranged into MFMA operand tiles (16 output channels x 64 k per 1 KiB tile, k zero-padded) and
+ * its column sums over k are written to colsum[N].  This replaces the reference's cached weight
+ * reorder (quantized_matmul_common.h:238-275) and its host-side column-sum loop (:569-573).
+ * `packed` must hold itexhip_qgemm_packed_bytes(K, N) bytes. */
+int64_t itexhip_qgemm_packed_bytes(int64_t K, int64_t N);
+int itexhip_qgemm_prepack_b(const int8_t* w, int transpose_b, int64_t K, int64_t N, int8_t* packed,
+                            int32_t* colsum, void* stream);
+
+/* out[M,N] = epilogue( a[M,K] (u8 or s8, row-major) x packed weight ), exact int32 accumulation.
+ * a_type QUINT8 | QINT8; out_type QINT32 | QINT8 | QUINT8 | FLOAT.  `colsum` is needed for QUINT8
+ * activations (they are fed to the signed MFMA as a-128 and corrected by 128*colsum[n]).
+ * `scales` has ep->n_scales floats (may be NULL when 0), `bias` N floats (NULL = no bias add).
+ * Dispatches to the bandwidth-bound small-M kernel for M <= 16 and to the MFMA tile kernel
+ * otherwise; the two explicit entry points below force one path. */
+int itexhip_qgemm(const void* a, int a_type, const int8_t* packed_b, const int32_t* colsum,
+                  int64_t M, int64_t K, int64_t N, const float* scales, const float* bias,
+                  const itexhip_epilogue* ep, int out_type, void* out, void* stream);
+int itexhip_qgemm_tile(const void* a, int a_type, const int8_t* packed_b, const int32_t* colsum,
+                       int64_t M, int64_t K, int64_t N, const float* scales, const float* bias,
+                       const itexhip_epilogue* ep, int out_type, void* out, void* stream);
+int itexhip_qgemv(const void* a, int a_type, const int8_t* packed_b, const int32_t* colsum,
+                  int64_t M, int64_t K, int64_t N, const float* scales, const float* bias,
+                  const itexhip_epilogue* ep, int out_type, void* out, void* stream);
+
+/* Same contract on the unpacked TF-layout weight, any shape (no alignment requirements): one
+ * thread per output element.  Used for shapes the tile kernels do not cover (K not a multiple of
+ * 16) and as an on-device cross-check. */
+int itexhip_qgemm_naive(const void* a, int a_type, const int8_t* w, int transpose_b, int64_t M,
+                        int64_t K, int64_t N, const float* scales, const float* bias,
+                        const itexhip_epilogue* ep, int out_type, void* out, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ITEXHIP_H_ */

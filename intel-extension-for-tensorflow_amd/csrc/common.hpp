@@ -1,0 +1,80 @@
+// Shared host/device helpers of the itexhip kernels (gfx950 only).
+#ifndef ITEXHIP_COMMON_HPP_
+#define ITEXHIP_COMMON_HPP_
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#include "itexhip.h"
+
+// Every fp32 operation in the quantization arithmetic must round on its own: no fused multiply-add.
+#pragma clang fp contract(off)
+
+namespace itexhip {
+
+// native vector types (usable with the nontemporal load/store builtins)
+typedef float f4 __attribute__((ext_vector_type(4)));
+typedef int i4 __attribute__((ext_vector_type(4)));
+
+void set_error(const char* fmt, ...);
+
+inline int hip_fail(hipError_t e, const char* what) {
+  set_error("%s: %s", what, hipGetErrorString(e));
+  return ITEXHIP_INTERNAL;
+}
+
+#define ITEXHIP_CHECK_LAUNCH(what)                                   \
+  do {                                                               \
+    hipError_t e__ = hipGetLastError();                              \
+    if (e__ != hipSuccess) return ::itexhip::hip_fail(e__, what);    \
+  } while (0)
+
+#define ITEXHIP_REQUIRE(cond, ...)            \
+  do {                                        \
+    if (!(cond)) {                            \
+      ::itexhip::set_error(__VA_ARGS__);      \
+      return ITEXHIP_INVALID_ARGUMENT;        \
+    }                                         \
+  } while (0)
+
+inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s); }
+
+inline bool aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
+
+// Saturation bounds of the destination type, in fp32 (the s32 upper bound is the largest float
+// below 2^31).
+template <int T> struct Sat;
+template <> struct Sat<ITEXHIP_QINT8> { static constexpr float lo = -128.0f, hi = 127.0f; };
+template <> struct Sat<ITEXHIP_QUINT8> { static constexpr float lo = 0.0f, hi = 255.0f; };
+template <> struct Sat<ITEXHIP_QINT32> { static constexpr float lo = -2147483648.0f, hi = 2147483520.0f; };
+
+// clamp in fp32, then round to nearest even (v_rndne_f32), then convert.
+template <int T>
+__device__ __forceinline__ int sat_rne(float y) {
+  y = fmaxf(y, Sat<T>::lo);
+  y = fminf(y, Sat<T>::hi);
+  return static_cast<int>(__builtin_rintf(y));
+}
+
+__device__ __forceinline__ uint32_t pack4(int a, int b, int c, int d) {
+  return (static_cast<uint32_t>(a) & 0xffu) | ((static_cast<uint32_t>(b) & 0xffu) << 8) |
+         ((static_cast<uint32_t>(c) & 0xffu) << 16) | ((static_cast<uint32_t>(d) & 0xffu) << 24);
+}
+
+__device__ __forceinline__ float apply_eltwise(const itexhip_eltwise& e, float x) {
+  switch (e.alg) {
+    case ITEXHIP_ELT_RELU:
+      if (e.alpha == 0.0f) return fmaxf(x, 0.0f);
+      return x > 0.0f ? x : x * e.alpha;
+    case ITEXHIP_ELT_CLIP:
+      return fminf(fmaxf(x, e.alpha), e.beta);
+    case ITEXHIP_ELT_LINEAR:
+      return e.alpha * x + e.beta;
+    default:
+      return x;
+  }
+}
+
+}  // namespace itexhip
+#endif  // ITEXHIP_COMMON_HPP_

@@ -1,0 +1,532 @@
+// HBM-bound elementwise kernels: QuantizeV2, Dequantize, RequantizePerChannel and the min/max
+// reductions.  One wavefront instruction moves 1 KiB (16 B per lane, lanes contiguous); each thread
+// keeps several such loads in flight before it converts and stores.
+#include "common.hpp"
+
+namespace itexhip {
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kUnroll = 4;  // 16-byte loads in flight per thread
+
+// ------------------------------------------------------------------------------------------------
+// Quantize: q = sat(rne(fl(x * scale) + addend))
+// ------------------------------------------------------------------------------------------------
+template <int T>
+__device__ __forceinline__ uint32_t quantize4(f4 v, float scale, float addend) {
+  const float a = v.x * scale, b = v.y * scale, c = v.z * scale, d = v.w * scale;
+  return pack4(sat_rne<T>(a + addend), sat_rne<T>(b + addend), sat_rne<T>(c + addend),
+               sat_rne<T>(d + addend));
+}
+
+// n4 = number of complete groups of 4 elements; the caller handles the tail.
+template <int T>
+__global__ __launch_bounds__(kThreads) void quantize_vec_kernel(const f4* __restrict__ x,
+                                                                uint32_t* __restrict__ q, int64_t n4,
+                                                                float scale, float addend) {
+  const int64_t base = static_cast<int64_t>(blockIdx.x) * (kThreads * kUnroll) + threadIdx.x;
+  f4 v[kUnroll];
+#pragma unroll
+  for (int j = 0; j < kUnroll; ++j) {
+    const int64_t i = base + j * kThreads;
+    if (i < n4) v[j] = __builtin_nontemporal_load(&x[i]);
+  }
+#pragma unroll
+  for (int j = 0; j < kUnroll; ++j) {
+    const int64_t i = base + j * kThreads;
+    if (i < n4) __builtin_nontemporal_store(quantize4<T>(v[j], scale, addend), &q[i]);
+  }
+}
+
+template <int T>
+__global__ __launch_bounds__(kThreads) void quantize_scalar_kernel(const float* __restrict__ x,
+                                                                   uint8_t* __restrict__ q,
+                                                                   int64_t begin, int64_t n,
+                                                                   float scale, float addend) {
+  const int64_t i = begin + static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+  if (i < n) {
+    const float t = x[i] * scale;
+    q[i] = static_cast<uint8_t>(sat_rne<T>(t + addend));
+  }
+}
+
+// [outer, slices, inner] with per-slice scale / addend
+template <int T>
+__global__ __launch_bounds__(kThreads) void quantize_axis_kernel(const float* __restrict__ x,
+                                                                 uint8_t* __restrict__ q, int64_t n,
+                                                                 int64_t slices, int64_t inner,
+                                                                 const float* __restrict__ scales,
+                                                                 const float* __restrict__ addends) {
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+  if (i < n) {
+    const int64_t s = (i / inner) % slices;
+    const float t = x[i] * scales[s];
+    const float a = addends ? addends[s] : 0.0f;
+    q[i] = static_cast<uint8_t>(sat_rne<T>(t + a));
+  }
+}
+
+// ------------------------------------------------------------------------------------------------
+// Dequantize: y = ((float)q - zp) * scale
+// ------------------------------------------------------------------------------------------------
+template <int T>
+__device__ __forceinline__ float widen(uint32_t w, int byte) {
+  const uint32_t b = (w >> (8 * byte)) & 0xffu;
+  if (T == ITEXHIP_QINT8) return static_cast<float>(static_cast<int>(static_cast<int8_t>(b)));
+  return static_cast<float>(b);
+}
+
+template <int T>
+__global__ __launch_bounds__(kThreads) void dequantize_vec_kernel(const uint32_t* __restrict__ q,
+                                                                  f4* __restrict__ y, int64_t n4,
+                                                                  float scale, float zp) {
+  const int64_t base = static_cast<int64_t>(blockIdx.x) * (kThreads * kUnroll) + threadIdx.x;
+  uint32_t w[kUnroll];
+#pragma unroll
+  for (int j = 0; j < kUnroll; ++j) {
+    const int64_t i = base + j * kThreads;
+    if (i < n4) w[j] = __builtin_nontemporal_load(&q[i]);
+  }
+#pragma unroll
+  for (int j = 0; j < kUnroll; ++j) {
+    const int64_t i = base + j * kThreads;
+    if (i < n4) {
+      f4 o;
+      o.x = (widen<T>(w[j], 0) - zp) * scale;
+      o.y = (widen<T>(w[j], 1) - zp) * scale;
+      o.z = (widen<T>(w[j], 2) - zp) * scale;
+      o.w = (widen<T>(w[j], 3) - zp) * scale;
+      __builtin_nontemporal_store(o, &y[i]);
+    }
+  }
+}
+
+template <int T>
+__global__ __launch_bounds__(kThreads) void dequantize_axis_kernel(const uint8_t* __restrict__ q,
+                                                                   float* __restrict__ y, int64_t begin,
+                                                                   int64_t n, int64_t slices,
+                                                                   int64_t inner,
+                                                                   const float* __restrict__ scales,
+                                                                   const int32_t* __restrict__ zps,
+                                                                   float scale0, float zp0) {
+  const int64_t i = begin + static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+  if (i < n) {
+    float sc = scale0, zp = zp0;
+    if (scales) {
+      const int64_t s = (i / inner) % slices;
+      sc = scales[s];
+      zp = zps ? static_cast<float>(zps[s]) : 0.0f;
+    }
+    const float v = (T == ITEXHIP_QINT8) ? static_cast<float>(static_cast<int8_t>(q[i]))
+                                         : static_cast<float>(q[i]);
+    y[i] = (v - zp) * sc;
+  }
+}
+
+// ------------------------------------------------------------------------------------------------
+// Requantize: q = sat(rne((float)x * scale[c]))
+// ------------------------------------------------------------------------------------------------
+// kMode 0: one scale passed by value; 1: depth % 4 == 0, scales read as f4; n4 = groups of 4
+template <int T, int kMode>
+__global__ __launch_bounds__(kThreads) void requantize_vec_kernel(const i4* __restrict__ x,
+                                                                  uint32_t* __restrict__ q, int64_t n4,
+                                                                  float scale,
+                                                                  const float* __restrict__ scales,
+                                                                  int64_t depth4) {
+  const int64_t base = static_cast<int64_t>(blockIdx.x) * (kThreads * kUnroll) + threadIdx.x;
+  i4 v[kUnroll];
+#pragma unroll
+  for (int j = 0; j < kUnroll; ++j) {
+    const int64_t i = base + j * kThreads;
+    if (i < n4) v[j] = __builtin_nontemporal_load(&x[i]);
+  }
+#pragma unroll
+  for (int j = 0; j < kUnroll; ++j) {
+    const int64_t i = base + j * kThreads;
+    if (i < n4) {
+      f4 s = f4{scale, scale, scale, scale};
+      if (kMode == 1) s = reinterpret_cast<const f4*>(scales)[i % depth4];
+      const float a = static_cast<float>(v[j].x) * s.x, b = static_cast<float>(v[j].y) * s.y;
+      const float c = static_cast<float>(v[j].z) * s.z, d = static_cast<float>(v[j].w) * s.w;
+      __builtin_nontemporal_store(pack4(sat_rne<T>(a), sat_rne<T>(b), sat_rne<T>(c), sat_rne<T>(d)),
+                                  &q[i]);
+    }
+  }
+}
+
+template <int T>
+__global__ __launch_bounds__(kThreads) void requantize_scalar_kernel(const int32_t* __restrict__ x,
+                                                                     uint8_t* __restrict__ q,
+                                                                     int64_t begin, int64_t n,
+                                                                     int64_t depth, float scale,
+                                                                     const float* __restrict__ scales) {
+  const int64_t i = begin + static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+  if (i < n) {
+    const float s = scales ? scales[i % depth] : scale;
+    q[i] = static_cast<uint8_t>(sat_rne<T>(static_cast<float>(x[i]) * s));
+  }
+}
+
+// ------------------------------------------------------------------------------------------------
+// min / max reductions
+// ------------------------------------------------------------------------------------------------
+__global__ void fill_minmax_i32_kernel(int32_t* mn, int32_t* mx, int64_t depth) {
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i < depth) {
+    mn[i] = INT32_MAX;
+    mx[i] = INT32_MIN;
+  }
+}
+
+__device__ __forceinline__ int wave_min(int v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = min(v, __shfl_xor(v, o, 64));
+  return v;
+}
+__device__ __forceinline__ int wave_max(int v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = max(v, __shfl_xor(v, o, 64));
+  return v;
+}
+
+// Whole-tensor (depth == 1) reduction: grid-stride over i4, wavefront reduction, one atomic pair
+// per wavefront.
+__global__ __launch_bounds__(kThreads) void minmax_i32_flat_kernel(const i4* __restrict__ x, int64_t n4,
+                                                                   const int32_t* __restrict__ tail,
+                                                                   int ntail, int32_t* mn_out,
+                                                                   int32_t* mx_out) {
+  int mn = INT32_MAX, mx = INT32_MIN;
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * kThreads;
+  int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+  for (; i + 3 * stride < n4; i += 4 * stride) {
+    i4 v[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) v[j] = __builtin_nontemporal_load(&x[i + j * stride]);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      mn = min(min(mn, v[j].x), min(v[j].y, min(v[j].z, v[j].w)));
+      mx = max(max(mx, v[j].x), max(v[j].y, max(v[j].z, v[j].w)));
+    }
+  }
+  for (; i < n4; i += stride) {
+    const i4 v = x[i];
+    mn = min(min(mn, v.x), min(v.y, min(v.z, v.w)));
+    mx = max(max(mx, v.x), max(v.y, max(v.z, v.w)));
+  }
+  if (blockIdx.x == 0 && static_cast<int>(threadIdx.x) < ntail) {
+    mn = min(mn, tail[threadIdx.x]);
+    mx = max(mx, tail[threadIdx.x]);
+  }
+  mn = wave_min(mn);
+  mx = wave_max(mx);
+  if ((threadIdx.x & 63) == 0) {
+    atomicMin(mn_out, mn);
+    atomicMax(mx_out, mx);
+  }
+}
+
+// Per-channel reduction, channel = last dim: thread owns one channel of its block's column group
+// and walks a chunk of rows (loads are contiguous across the threads of a wavefront).
+__global__ __launch_bounds__(kThreads) void minmax_i32_channel_kernel(const int32_t* __restrict__ x,
+                                                                      int64_t rows, int64_t depth,
+                                                                      int64_t rows_per_block,
+                                                                      int32_t* mn_out, int32_t* mx_out) {
+  const int64_t c = static_cast<int64_t>(blockIdx.y) * kThreads + threadIdx.x;
+  if (c >= depth) return;
+  const int64_t r0 = static_cast<int64_t>(blockIdx.x) * rows_per_block;
+  const int64_t r1 = min(rows, r0 + rows_per_block);
+  int mn = INT32_MAX, mx = INT32_MIN;
+  for (int64_t r = r0; r < r1; ++r) {
+    const int v = x[r * depth + c];
+    mn = min(mn, v);
+    mx = max(mx, v);
+  }
+  if (r0 < r1) {
+    atomicMin(&mn_out[c], mn);
+    atomicMax(&mx_out[c], mx);
+  }
+}
+
+// order-preserving map fp32 -> int32 (and back)
+__device__ __forceinline__ int f2key(float f) {
+  const int b = __float_as_int(f);
+  return b >= 0 ? b : b ^ 0x7fffffff;
+}
+__device__ __forceinline__ float key2f(int k) { return __int_as_float(k >= 0 ? k : k ^ 0x7fffffff); }
+
+__global__ void fill_minmax_f32_kernel(int* keys) {
+  keys[0] = f2key(__builtin_inff());
+  keys[1] = f2key(-__builtin_inff());
+}
+__global__ void finish_minmax_f32_kernel(int* keys) {
+  const float mn = key2f(keys[0]), mx = key2f(keys[1]);
+  reinterpret_cast<float*>(keys)[0] = mn;
+  reinterpret_cast<float*>(keys)[1] = mx;
+}
+
+__global__ __launch_bounds__(kThreads) void minmax_f32_kernel(const f4* __restrict__ x, int64_t n4,
+                                                              const float* __restrict__ tail, int ntail,
+                                                              int* keys) {
+  float mn = __builtin_inff(), mx = -__builtin_inff();
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * kThreads;
+  int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+  for (; i + 3 * stride < n4; i += 4 * stride) {
+    f4 v[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) v[j] = __builtin_nontemporal_load(&x[i + j * stride]);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      mn = fminf(fminf(mn, v[j].x), fminf(v[j].y, fminf(v[j].z, v[j].w)));
+      mx = fmaxf(fmaxf(mx, v[j].x), fmaxf(v[j].y, fmaxf(v[j].z, v[j].w)));
+    }
+  }
+  for (; i < n4; i += stride) {
+    const f4 v = x[i];
+    mn = fminf(fminf(mn, v.x), fminf(v.y, fminf(v.z, v.w)));
+    mx = fmaxf(fmaxf(mx, v.x), fmaxf(v.y, fmaxf(v.z, v.w)));
+  }
+  if (blockIdx.x == 0 && static_cast<int>(threadIdx.x) < ntail) {
+    mn = fminf(mn, tail[threadIdx.x]);
+    mx = fmaxf(mx, tail[threadIdx.x]);
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    mn = fminf(mn, __shfl_xor(mn, o, 64));
+    mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+  }
+  if ((threadIdx.x & 63) == 0) {
+    atomicMin(&keys[0], f2key(mn));
+    atomicMax(&keys[1], f2key(mx));
+  }
+}
+
+inline unsigned blocks_for(int64_t n, int64_t per_block) {
+  return static_cast<unsigned>((n + per_block - 1) / per_block);
+}
+
+}  // namespace
+}  // namespace itexhip
+
+using namespace itexhip;
+
+extern "C" int itexhip_quantize(const float* x, void* q, int64_t n, int dst_type, float scale,
+                                float addend, void* stream) {
+  ITEXHIP_REQUIRE(dst_type == ITEXHIP_QINT8 || dst_type == ITEXHIP_QUINT8,
+                  "itexhip_quantize: dst_type must be qint8 or quint8, got %d", dst_type);
+  ITEXHIP_REQUIRE(n >= 0, "itexhip_quantize: negative size");
+  if (n == 0) return ITEXHIP_OK;
+  ITEXHIP_REQUIRE(x && q, "itexhip_quantize: null buffer");
+  hipStream_t st = as_stream(stream);
+  int64_t done = 0;
+  if (aligned(x, 16) && aligned(q, 4) && n >= 4) {
+    const int64_t n4 = n / 4;
+    const unsigned grid = blocks_for(n4, kThreads * kUnroll);
+    if (dst_type == ITEXHIP_QINT8)
+      quantize_vec_kernel<ITEXHIP_QINT8><<<grid, kThreads, 0, st>>>(
+          reinterpret_cast<const f4*>(x), reinterpret_cast<uint32_t*>(q), n4, scale, addend);
+    else
+      quantize_vec_kernel<ITEXHIP_QUINT8><<<grid, kThreads, 0, st>>>(
+          reinterpret_cast<const f4*>(x), reinterpret_cast<uint32_t*>(q), n4, scale, addend);
+    done = n4 * 4;
+  }
+  if (done < n) {
+    const unsigned grid = blocks_for(n - done, kThreads);
+    if (dst_type == ITEXHIP_QINT8)
+      quantize_scalar_kernel<ITEXHIP_QINT8><<<grid, kThreads, 0, st>>>(
+          x, reinterpret_cast<uint8_t*>(q), done, n, scale, addend);
+    else
+      quantize_scalar_kernel<ITEXHIP_QUINT8><<<grid, kThreads, 0, st>>>(
+          x, reinterpret_cast<uint8_t*>(q), done, n, scale, addend);
+  }
+  ITEXHIP_CHECK_LAUNCH("itexhip_quantize");
+  return ITEXHIP_OK;
+}
+
+extern "C" int itexhip_quantize_axis(const float* x, void* q, int64_t outer, int64_t slices,
+                                     int64_t inner, int dst_type, const float* scales,
+                                     const float* addends, void* stream) {
+  ITEXHIP_REQUIRE(dst_type == ITEXHIP_QINT8 || dst_type == ITEXHIP_QUINT8,
+                  "itexhip_quantize_axis: dst_type must be qint8 or quint8, got %d", dst_type);
+  ITEXHIP_REQUIRE(outer >= 0 && slices >= 0 && inner >= 0, "itexhip_quantize_axis: negative size");
+  const int64_t n = outer * slices * inner;
+  if (n == 0) return ITEXHIP_OK;
+  ITEXHIP_REQUIRE(x && q && scales, "itexhip_quantize_axis: null buffer");
+  const unsigned grid = blocks_for(n, kThreads);
+  if (dst_type == ITEXHIP_QINT8)
+    quantize_axis_kernel<ITEXHIP_QINT8><<<grid, kThreads, 0, as_stream(stream)>>>(
+        x, reinterpret_cast<uint8_t*>(q), n, slices, inner, scales, addends);
+  else
+    quantize_axis_kernel<ITEXHIP_QUINT8><<<grid, kThreads, 0, as_stream(stream)>>>(
+        x, reinterpret_cast<uint8_t*>(q), n, slices, inner, scales, addends);
+  ITEXHIP_CHECK_LAUNCH("itexhip_quantize_axis");
+  return ITEXHIP_OK;
+}
+
+extern "C" int itexhip_dequantize(const void* q, float* y, int64_t n, int src_type, float scale,
+                                  int32_t zero_point, void* stream) {
+  ITEXHIP_REQUIRE(src_type == ITEXHIP_QINT8 || src_type == ITEXHIP_QUINT8,
+                  "itexhip_dequantize: src_type must be qint8 or quint8, got %d", src_type);
+  ITEXHIP_REQUIRE(n >= 0, "itexhip_dequantize: negative size");
+  if (n == 0) return ITEXHIP_OK;
+  ITEXHIP_REQUIRE(q && y, "itexhip_dequantize: null buffer");
+  hipStream_t st = as_stream(stream);
+  const float zp = static_cast<float>(zero_point);
+  int64_t done = 0;
+  if (aligned(q, 4) && aligned(y, 16) && n >= 4) {
+    const int64_t n4 = n / 4;
+    const unsigned grid = blocks_for(n4, kThreads * kUnroll);
+    if (src_type == ITEXHIP_QINT8)
+      dequantize_vec_kernel<ITEXHIP_QINT8><<<grid, kThreads, 0, st>>>(
+          reinterpret_cast<const uint32_t*>(q), reinterpret_cast<f4*>(y), n4, scale, zp);
+    else
+      dequantize_vec_kernel<ITEXHIP_QUINT8><<<grid, kThreads, 0, st>>>(
+          reinterpret_cast<const uint32_t*>(q), reinterpret_cast<f4*>(y), n4, scale, zp);
+    done = n4 * 4;
+  }
+  if (done < n) {
+    const unsigned grid = blocks_for(n - done, kThreads);
+    if (src_type == ITEXHIP_QINT8)
+      dequantize_axis_kernel<ITEXHIP_QINT8><<<grid, kThreads, 0, st>>>(
+          reinterpret_cast<const uint8_t*>(q), y, done, n, 1, 1, nullptr, nullptr, scale, zp);
+    else
+      dequantize_axis_kernel<ITEXHIP_QUINT8><<<grid, kThreads, 0, st>>>(
+          reinterpret_cast<const uint8_t*>(q), y, done, n, 1, 1, nullptr, nullptr, scale, zp);
+  }
+  ITEXHIP_CHECK_LAUNCH("itexhip_dequantize");
+  return ITEXHIP_OK;
+}
+
+extern "C" int itexhip_dequantize_axis(const void* q, float* y, int64_t outer, int64_t slices,
+                                       int64_t inner, int src_type, const float* scales,
+                                       const int32_t* zero_points, void* stream) {
+  ITEXHIP_REQUIRE(src_type == ITEXHIP_QINT8 || src_type == ITEXHIP_QUINT8,
+                  "itexhip_dequantize_axis: src_type must be qint8 or quint8, got %d", src_type);
+  ITEXHIP_REQUIRE(outer >= 0 && slices >= 0 && inner >= 0, "itexhip_dequantize_axis: negative size");
+  const int64_t n = outer * slices * inner;
+  if (n == 0) return ITEXHIP_OK;
+  ITEXHIP_REQUIRE(q && y && scales, "itexhip_dequantize_axis: null buffer");
+  const unsigned grid = blocks_for(n, kThreads);
+  if (src_type == ITEXHIP_QINT8)
+    dequantize_axis_kernel<ITEXHIP_QINT8><<<grid, kThreads, 0, as_stream(stream)>>>(
+        reinterpret_cast<const uint8_t*>(q), y, 0, n, slices, inner, scales, zero_points, 0.f, 0.f);
+  else
+    dequantize_axis_kernel<ITEXHIP_QUINT8><<<grid, kThreads, 0, as_stream(stream)>>>(
+        reinterpret_cast<const uint8_t*>(q), y, 0, n, slices, inner, scales, zero_points, 0.f, 0.f);
+  ITEXHIP_CHECK_LAUNCH("itexhip_dequantize_axis");
+  return ITEXHIP_OK;
+}
+
+namespace {
+template <int T>
+int requantize_impl(const int32_t* x, void* q, int64_t n, int64_t depth, float scale,
+                    const float* scales, hipStream_t st) {
+  int64_t done = 0;
+  const bool vec_ok = aligned(x, 16) && aligned(q, 4) && n >= 4;
+  if (vec_ok && scales == nullptr) {
+    const int64_t n4 = n / 4;
+    requantize_vec_kernel<T, 0><<<blocks_for(n4, kThreads * kUnroll), kThreads, 0, st>>>(
+        reinterpret_cast<const i4*>(x), reinterpret_cast<uint32_t*>(q), n4, scale, nullptr, 1);
+    done = n4 * 4;
+  } else if (vec_ok && depth % 4 == 0 && aligned(scales, 16)) {
+    const int64_t n4 = n / 4;  // n is a multiple of depth, hence of 4
+    requantize_vec_kernel<T, 1><<<blocks_for(n4, kThreads * kUnroll), kThreads, 0, st>>>(
+        reinterpret_cast<const i4*>(x), reinterpret_cast<uint32_t*>(q), n4, 0.f, scales, depth / 4);
+    done = n4 * 4;
+  }
+  if (done < n) {
+    requantize_scalar_kernel<T><<<blocks_for(n - done, kThreads), kThreads, 0, st>>>(
+        x, reinterpret_cast<uint8_t*>(q), done, n, depth, scale, scales);
+  }
+  ITEXHIP_CHECK_LAUNCH("itexhip_requantize");
+  return ITEXHIP_OK;
+}
+}  // namespace
+
+extern "C" int itexhip_requantize_per_channel(const int32_t* x, void* q, int64_t rows, int64_t depth,
+                                              int dst_type, const float* scales, void* stream) {
+  ITEXHIP_REQUIRE(dst_type == ITEXHIP_QINT8 || dst_type == ITEXHIP_QUINT8,
+                  "itexhip_requantize_per_channel: dst_type must be qint8 or quint8, got %d", dst_type);
+  ITEXHIP_REQUIRE(rows >= 0 && depth >= 0, "itexhip_requantize_per_channel: negative size");
+  const int64_t n = rows * depth;
+  if (n == 0) return ITEXHIP_OK;
+  ITEXHIP_REQUIRE(x && q && scales, "itexhip_requantize_per_channel: null buffer");
+  if (dst_type == ITEXHIP_QINT8)
+    return requantize_impl<ITEXHIP_QINT8>(x, q, n, depth, 0.f, scales, as_stream(stream));
+  return requantize_impl<ITEXHIP_QUINT8>(x, q, n, depth, 0.f, scales, as_stream(stream));
+}
+
+extern "C" int itexhip_requantize(const int32_t* x, void* q, int64_t n, int dst_type, float scale,
+                                  void* stream) {
+  ITEXHIP_REQUIRE(dst_type == ITEXHIP_QINT8 || dst_type == ITEXHIP_QUINT8,
+                  "itexhip_requantize: dst_type must be qint8 or quint8, got %d", dst_type);
+  ITEXHIP_REQUIRE(n >= 0, "itexhip_requantize: negative size");
+  if (n == 0) return ITEXHIP_OK;
+  ITEXHIP_REQUIRE(x && q, "itexhip_requantize: null buffer");
+  if (dst_type == ITEXHIP_QINT8)
+    return requantize_impl<ITEXHIP_QINT8>(x, q, n, 1, scale, nullptr, as_stream(stream));
+  return requantize_impl<ITEXHIP_QUINT8>(x, q, n, 1, scale, nullptr, as_stream(stream));
+}
+
+extern "C" int itexhip_minmax_i32_per_channel(const int32_t* x, int64_t rows, int64_t depth,
+                                              int32_t* min_out, int32_t* max_out, void* stream) {
+  ITEXHIP_REQUIRE(rows >= 0 && depth >= 0, "itexhip_minmax_i32_per_channel: negative size");
+  if (depth == 0) return ITEXHIP_OK;
+  ITEXHIP_REQUIRE(min_out && max_out, "itexhip_minmax_i32_per_channel: null output");
+  hipStream_t st = as_stream(stream);
+  fill_minmax_i32_kernel<<<blocks_for(depth, 256), 256, 0, st>>>(min_out, max_out, depth);
+  if (rows > 0) {
+    ITEXHIP_REQUIRE(x, "itexhip_minmax_i32_per_channel: null input");
+    if (depth == 1) {
+      const bool vec = aligned(x, 16);
+      const int64_t n4 = vec ? rows / 4 : 0;
+      const int ntail = static_cast<int>(rows - n4 * 4);
+      if (vec) {
+        const unsigned grid = static_cast<unsigned>(
+            std::min<int64_t>(2048, std::max<int64_t>(1, (n4 + kThreads - 1) / kThreads)));
+        minmax_i32_flat_kernel<<<grid, kThreads, 0, st>>>(reinterpret_cast<const i4*>(x), n4,
+                                                          x + n4 * 4, ntail, min_out, max_out);
+      } else {
+        const int64_t rpb = 4096;
+        dim3 grid(blocks_for(rows, rpb), 1);
+        minmax_i32_channel_kernel<<<grid, kThreads, 0, st>>>(x, rows, 1, rpb, min_out, max_out);
+      }
+    } else {
+      // enough row chunks to occupy the device, at least 64 rows each
+      const int64_t col_blocks = (depth + kThreads - 1) / kThreads;
+      int64_t row_blocks = std::max<int64_t>(1, 4096 / col_blocks);
+      int64_t rpb = std::max<int64_t>(64, (rows + row_blocks - 1) / row_blocks);
+      row_blocks = (rows + rpb - 1) / rpb;
+      ITEXHIP_REQUIRE(col_blocks <= 65535, "itexhip_minmax_i32_per_channel: depth too large");
+      dim3 grid(static_cast<unsigned>(row_blocks), static_cast<unsigned>(col_blocks));
+      minmax_i32_channel_kernel<<<grid, kThreads, 0, st>>>(x, rows, depth, rpb, min_out, max_out);
+    }
+  }
+  ITEXHIP_CHECK_LAUNCH("itexhip_minmax_i32_per_channel");
+  return ITEXHIP_OK;
+}
+
+extern "C" int itexhip_minmax_f32(const float* x, int64_t n, float* minmax_out, void* stream) {
+  ITEXHIP_REQUIRE(n >= 0, "itexhip_minmax_f32: negative size");
+  ITEXHIP_REQUIRE(minmax_out, "itexhip_minmax_f32: null output");
+  hipStream_t st = as_stream(stream);
+  int* keys = reinterpret_cast<int*>(minmax_out);
+  fill_minmax_f32_kernel<<<1, 1, 0, st>>>(keys);
+  if (n > 0) {
+    ITEXHIP_REQUIRE(x, "itexhip_minmax_f32: null input");
+    // the vector body starts at the first 16-byte boundary; head and tail go through `tail` slots
+    const uintptr_t addr = reinterpret_cast<uintptr_t>(x);
+    int64_t head = static_cast<int64_t>(((16 - (addr & 15)) & 15) / 4);
+    if (head > n) head = n;
+    const int64_t n4 = (n - head) / 4;
+    const int64_t ntail = n - head - n4 * 4;
+    const unsigned grid = static_cast<unsigned>(
+        std::min<int64_t>(2048, std::max<int64_t>(1, (n4 + kThreads - 1) / kThreads)));
+    minmax_f32_kernel<<<grid, kThreads, 0, st>>>(reinterpret_cast<const f4*>(x + head), n4,
+                                                 x + head + n4 * 4, static_cast<int>(ntail), keys);
+    if (head > 0)
+      minmax_f32_kernel<<<1, kThreads, 0, st>>>(nullptr, 0, x, static_cast<int>(head), keys);
+  }
+  finish_minmax_f32_kernel<<<1, 1, 0, st>>>(keys);
+  ITEXHIP_CHECK_LAUNCH("itexhip_minmax_f32");
+  return ITEXHIP_OK;
+}

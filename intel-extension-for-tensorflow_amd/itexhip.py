@@ -1,0 +1,188 @@
+"""ctypes binding of lib/libitexhip.so (the C ABI declared in include/itexhip.h).
+
+All buffers are raw device addresses (ints) or objects with a `data_ptr()` method (torch tensors);
+streams are raw hipStream_t handles (ints, 0 = default stream).  Every call checks the status and
+raises ItexHipError with the library's message.
+"""
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libitexhip.so")
+
+OK, INVALID_ARGUMENT, UNIMPLEMENTED, INTERNAL = 0, 3, 12, 13
+FLOAT, INT32, QINT8, QUINT8, QINT32 = 1, 3, 11, 12, 13
+MIN_COMBINED, MIN_FIRST, SCALED = 0, 1, 2
+API_V2, API_V1, API_LEGACY = 0, 1, 2
+ACT_NONE, ACT_RELU, ACT_RELU6, ACT_LEAKYRELU = 0, 1, 2, 3
+ELT_RELU, ELT_CLIP, ELT_LINEAR = 1, 2, 3
+
+EXPORTS = [
+    "itexhip_last_error", "itexhip_build_info", "itexhip_quantize", "itexhip_quantize_axis",
+    "itexhip_dequantize", "itexhip_dequantize_axis", "itexhip_requantize_per_channel",
+    "itexhip_requantize", "itexhip_minmax_i32_per_channel", "itexhip_minmax_f32",
+    "itexhip_qmatmul_epilogue_desc", "itexhip_qmatmul_prepare", "itexhip_qgemm_packed_bytes",
+    "itexhip_qgemm_prepack_b", "itexhip_qgemm", "itexhip_qgemm_tile", "itexhip_qgemv",
+    "itexhip_qgemm_naive",
+]
+
+
+class ItexHipError(RuntimeError):
+    def __init__(self, code, msg):
+        super().__init__("itexhip status %d: %s" % (code, msg))
+        self.code = code
+
+
+class Eltwise(C.Structure):
+    _fields_ = [("alg", C.c_int), ("alpha", C.c_float), ("beta", C.c_float)]
+
+
+class Epilogue(C.Structure):
+    _fields_ = [("n_scales", C.c_int), ("n_eltwise", C.c_int), ("elt", Eltwise * 2)]
+
+
+class MatmulParams(C.Structure):
+    _fields_ = [("api", C.c_int), ("t_in", C.c_int), ("t_out", C.c_int), ("input_mode", C.c_int),
+                ("out_min_first", C.c_int), ("activation", C.c_int), ("has_requantize", C.c_int),
+                ("has_dequantize", C.c_int), ("n_fused_ops", C.c_int), ("leakyrelu_alpha", C.c_float),
+                ("min_a", C.c_float), ("max_a", C.c_float), ("min_out", C.c_float),
+                ("max_out", C.c_float)]
+
+
+# One HIP runtime per process: PyTorch ships its own libamdhip64.so.7 and loads it by path.  If this
+# library were loaded first, the system runtime would be mapped as well and the second one to
+# initialise finds no device.  Importing torch first lets the dynamic loader satisfy this library's
+# libamdhip64.so.7 dependency with the copy that is already mapped.
+try:
+    import torch  # noqa: F401
+except ImportError:  # a process without PyTorch uses the system runtime
+    pass
+
+if not os.path.exists(LIB_PATH):
+    raise ImportError("native library missing: %s (run intel-extension-for-tensorflow_amd/build.py)"
+                      % LIB_PATH)
+_lib = C.CDLL(LIB_PATH)
+_lib.itexhip_last_error.restype = C.c_char_p
+_lib.itexhip_build_info.restype = C.c_char_p
+_lib.itexhip_qgemm_packed_bytes.restype = C.c_int64
+_lib.itexhip_qgemm_packed_bytes.argtypes = [C.c_int64, C.c_int64]
+
+
+def raw():
+    """The ctypes.CDLL handle."""
+    return _lib
+
+
+def _ptr(x):
+    if x is None:
+        return C.c_void_p(0)
+    if hasattr(x, "data_ptr"):
+        return C.c_void_p(x.data_ptr())
+    return C.c_void_p(int(x))
+
+
+def _check(st):
+    if st != OK:
+        raise ItexHipError(st, _lib.itexhip_last_error().decode())
+
+
+def _i64(v):
+    return C.c_int64(int(v))
+
+
+def build_info():
+    return _lib.itexhip_build_info().decode()
+
+
+def quantize(x, q, n, dst_type, scale, addend=0.0, stream=0):
+    _check(_lib.itexhip_quantize(_ptr(x), _ptr(q), _i64(n), dst_type, C.c_float(scale),
+                                 C.c_float(addend), _ptr(stream)))
+
+
+def quantize_axis(x, q, outer, slices, inner, dst_type, scales, addends=None, stream=0):
+    _check(_lib.itexhip_quantize_axis(_ptr(x), _ptr(q), _i64(outer), _i64(slices), _i64(inner),
+                                      dst_type, _ptr(scales), _ptr(addends), _ptr(stream)))
+
+
+def dequantize(q, y, n, src_type, scale, zero_point=0, stream=0):
+    _check(_lib.itexhip_dequantize(_ptr(q), _ptr(y), _i64(n), src_type, C.c_float(scale),
+                                   C.c_int32(int(zero_point)), _ptr(stream)))
+
+
+def dequantize_axis(q, y, outer, slices, inner, src_type, scales, zero_points=None, stream=0):
+    _check(_lib.itexhip_dequantize_axis(_ptr(q), _ptr(y), _i64(outer), _i64(slices), _i64(inner),
+                                        src_type, _ptr(scales), _ptr(zero_points), _ptr(stream)))
+
+
+def requantize_per_channel(x, q, rows, depth, dst_type, scales, stream=0):
+    _check(_lib.itexhip_requantize_per_channel(_ptr(x), _ptr(q), _i64(rows), _i64(depth), dst_type,
+                                               _ptr(scales), _ptr(stream)))
+
+
+def requantize(x, q, n, dst_type, scale, stream=0):
+    _check(_lib.itexhip_requantize(_ptr(x), _ptr(q), _i64(n), dst_type, C.c_float(scale),
+                                   _ptr(stream)))
+
+
+def minmax_i32_per_channel(x, rows, depth, min_out, max_out, stream=0):
+    _check(_lib.itexhip_minmax_i32_per_channel(_ptr(x), _i64(rows), _i64(depth), _ptr(min_out),
+                                               _ptr(max_out), _ptr(stream)))
+
+
+def minmax_f32(x, n, minmax_out, stream=0):
+    _check(_lib.itexhip_minmax_f32(_ptr(x), _i64(n), _ptr(minmax_out), _ptr(stream)))
+
+
+def matmul_params(api=API_V2, t_in=QUINT8, t_out=FLOAT, input_mode=MIN_FIRST, out_min_first=False,
+                  activation=ACT_NONE, has_requantize=False, has_dequantize=False, n_fused_ops=1,
+                  leakyrelu_alpha=0.2, min_a=0.0, max_a=0.0, min_out=0.0, max_out=0.0):
+    return MatmulParams(api, t_in, t_out, input_mode, int(out_min_first), activation,
+                        int(has_requantize), int(has_dequantize), n_fused_ops, leakyrelu_alpha,
+                        min_a, max_a, min_out, max_out)
+
+
+def qmatmul_epilogue_desc(params, nb):
+    ep = Epilogue()
+    _check(_lib.itexhip_qmatmul_epilogue_desc(C.byref(params), _i64(nb), C.byref(ep)))
+    return ep
+
+
+def qmatmul_prepare(params, min_b, max_b, nb, bias, colsum, N, scales_out, bias_out, stream=0):
+    _check(_lib.itexhip_qmatmul_prepare(C.byref(params), _ptr(min_b), _ptr(max_b), _i64(nb),
+                                        _ptr(bias), _ptr(colsum), _i64(N), _ptr(scales_out),
+                                        _ptr(bias_out), _ptr(stream)))
+
+
+def qgemm_packed_bytes(K, N):
+    return int(_lib.itexhip_qgemm_packed_bytes(int(K), int(N)))
+
+
+def qgemm_prepack_b(w, transpose_b, K, N, packed, colsum, stream=0):
+    _check(_lib.itexhip_qgemm_prepack_b(_ptr(w), int(bool(transpose_b)), _i64(K), _i64(N),
+                                        _ptr(packed), _ptr(colsum), _ptr(stream)))
+
+
+def _gemm_call(fn, a, a_type, b, colsum, M, K, N, scales, bias, ep, out_type, out, stream):
+    _check(fn(_ptr(a), a_type, _ptr(b), _ptr(colsum), _i64(M), _i64(K), _i64(N), _ptr(scales),
+              _ptr(bias), C.byref(ep), out_type, _ptr(out), _ptr(stream)))
+
+
+def qgemm(a, a_type, packed_b, colsum, M, K, N, scales, bias, ep, out_type, out, stream=0):
+    _gemm_call(_lib.itexhip_qgemm, a, a_type, packed_b, colsum, M, K, N, scales, bias, ep, out_type,
+               out, stream)
+
+
+def qgemm_tile(a, a_type, packed_b, colsum, M, K, N, scales, bias, ep, out_type, out, stream=0):
+    _gemm_call(_lib.itexhip_qgemm_tile, a, a_type, packed_b, colsum, M, K, N, scales, bias, ep,
+               out_type, out, stream)
+
+
+def qgemv(a, a_type, packed_b, colsum, M, K, N, scales, bias, ep, out_type, out, stream=0):
+    _gemm_call(_lib.itexhip_qgemv, a, a_type, packed_b, colsum, M, K, N, scales, bias, ep, out_type,
+               out, stream)
+
+
+def qgemm_naive(a, a_type, w, transpose_b, M, K, N, scales, bias, ep, out_type, out, stream=0):
+    _check(_lib.itexhip_qgemm_naive(_ptr(a), a_type, _ptr(w), int(bool(transpose_b)), _i64(M),
+                                    _i64(K), _i64(N), _ptr(scales), _ptr(bias), C.byref(ep),
+                                    out_type, _ptr(out), _ptr(stream)))

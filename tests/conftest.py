@@ -17,3 +17,17 @@ def golden():
     import json
     with open(os.path.join(ROOT, "tests", "golden", "reference_vectors.json")) as f:
         return json.load(f)
+
+
+@pytest.fixture(scope="session")
+def hip():
+    """The ctypes binding of the native library; importing it fails if the library is not built."""
+    import __graft_entry__ as entry
+    return entry.load_package().itexhip
+
+
+@pytest.fixture(scope="session")
+def dev():
+    import torch
+    assert torch.cuda.is_available(), "GPU tests need a GPU"
+    return torch.device("cuda:0")

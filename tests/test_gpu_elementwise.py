@@ -1,0 +1,302 @@
+"""GPU parity: QuantizeV2 / Dequantize / RequantizePerChannel / range reductions through the C ABI
+versus the CPU oracle.  Integer outputs and min/max bit-exact; fp32 outputs bit-exact (the bar is
+1 ULP of the int->fp32 scale product; the kernels perform the same single fp32 multiply)."""
+import numpy as np
+import pytest
+
+from oracle import pyoracle as orc
+
+pytestmark = pytest.mark.gpu
+
+TORCH_OF = None
+
+
+def tdtype(T):
+    import torch
+    return {orc.QINT8: torch.int8, orc.QUINT8: torch.uint8}[T]
+
+
+def scale_per_slice(shape, axis, values):
+    out = np.take(values, np.remainder(np.arange(np.prod(shape)), len(values))).reshape(shape)
+    if axis is not None:
+        scale_shape = [1] * len(shape)
+        scale_shape[axis] = shape[axis]
+        out = out * np.arange(1, shape[axis] + 1).reshape(scale_shape)
+    return out
+
+
+def host_quant_params(T, mode, classic, mn, mx, ensure=0.01):
+    """Host-side parameter math (the op kernel's job) done with the oracle's scalar helpers, returning
+    what the C ABI takes: per-slice scale and addend, and the reported output range."""
+    mn = np.atleast_1d(np.float32(mn))
+    mx = np.atleast_1d(np.float32(mx))
+    amn, amx = np.zeros_like(mn), np.zeros_like(mx)
+    for i in range(mn.size):
+        st, amn[i], amx[i] = orc.adjust_input_range(float(mn[i]), float(mx[i]), ensure)
+        assert st == orc.OK
+    if mode == orc.SCALED or classic:
+        st, omn, omx, sc, zp = orc.scale_zeropoint_align(T, mode, False, amn, amx)
+        add = zp.astype(np.float32) if mode == orc.MIN_FIRST else np.zeros_like(sc)
+        if mode == orc.SCALED and T == orc.QUINT8:
+            omn = np.zeros_like(omn)
+    else:
+        sc = np.array([orc.legacy_min_first_scale(T, float(a), float(b)) for a, b in zip(amn, amx)], np.float32)
+        add = (-amn).astype(np.float32) * sc
+        omn, omx = amn, amx
+    return sc, add, omn, omx
+
+
+def gpu_quantize(hip, dev, x, T, mode, mn, mx, axis=None, classic=False):
+    import torch
+    sc, add, omn, omx = host_quant_params(T, mode, classic, mn, mx)
+    x_d = torch.from_numpy(np.ascontiguousarray(x)).to(dev)
+    q_d = torch.empty(x.shape, dtype=tdtype(T), device=dev)
+    if axis is None:
+        hip.quantize(x_d, q_d, x.size, T, float(sc[0]), float(add[0]))
+    else:
+        outer = int(np.prod(x.shape[:axis], dtype=np.int64))
+        inner = int(np.prod(x.shape[axis + 1:], dtype=np.int64))
+        sc_d = torch.from_numpy(sc).to(dev)
+        add_d = torch.from_numpy(add).to(dev)
+        hip.quantize_axis(x_d, q_d, outer, x.shape[axis], inner, T, sc_d, add_d)
+    torch.cuda.synchronize()
+    return q_d.cpu().numpy(), omn, omx
+
+
+def test_quantize_golden_vectors(hip, dev, golden):
+    T = {"quint8": orc.QUINT8, "qint8": orc.QINT8}
+    Mo = {"MIN_FIRST": orc.MIN_FIRST, "SCALED": orc.SCALED}
+    for case in golden["quantize_v2"]:
+        x = np.array(case["x"], np.float32).reshape(case["shape"])
+        q, omn, omx = gpu_quantize(hip, dev, x, T[case["T"]], Mo[case["mode"]], case["min_range"],
+                                   case["max_range"], classic=case["classic_asymmetric_algorithm"])
+        assert q.ravel().tolist() == case["expected"], case["source"]
+
+
+def test_quantize_axis_golden(hip, dev, golden):
+    g = golden["quantize_v2_axis"]
+    shape = np.array(g["shape"])
+    values = np.array(g["values"], np.float32)
+    expected = scale_per_slice(shape, None, np.array(g["quant_values"], np.int32))
+    for axis in g["axes"]:
+        x = scale_per_slice(shape, axis, values).astype(np.float32)
+        if axis is None:
+            mn, mx = g["min_unit"], g["max_unit"]
+        else:
+            mn = [g["min_unit"] * (s + 1) for s in range(shape[axis])]
+            mx = [g["max_unit"] * (s + 1) for s in range(shape[axis])]
+        q, omn, omx = gpu_quantize(hip, dev, x, orc.QINT8, orc.SCALED, mn, mx, axis=axis)
+        np.testing.assert_array_equal(q.astype(np.int32), expected)
+
+
+def outlier_normal(rng, n, frac, mult):
+    x = rng.standard_normal(n).astype(np.float32)
+    k = max(1, int(n * frac))
+    idx = rng.integers(0, n, k)
+    x[idx] *= mult
+    return x
+
+
+@pytest.mark.parametrize("T,mode,classic", [
+    (orc.QINT8, orc.SCALED, False), (orc.QUINT8, orc.SCALED, False),
+    (orc.QUINT8, orc.MIN_FIRST, False), (orc.QINT8, orc.MIN_FIRST, False),
+    (orc.QUINT8, orc.MIN_FIRST, True)])
+@pytest.mark.parametrize("n", [1, 3, 4, 5, 1023, 4096, (1 << 20) + 7])
+def test_quantize_random_vs_oracle(hip, dev, T, mode, classic, n):
+    rng = np.random.default_rng(30 + n % 97)
+    x = outlier_normal(rng, n, 1e-4, 50.0)
+    # ties and saturation: exact half-steps for scale 1 when the range is +-127
+    mn, mx = float(x.min()), float(x.max())
+    st, q_ref, omn_ref, omx_ref = orc.quantize_v2(x, mn, mx, T, mode, None, classic)
+    q, omn, omx = gpu_quantize(hip, dev, x, T, mode, mn, mx, classic=classic)
+    np.testing.assert_array_equal(q, q_ref)
+    np.testing.assert_array_equal(omn, omn_ref)
+    np.testing.assert_array_equal(omx, omx_ref)
+
+
+def test_quantize_ties_and_saturation(hip, dev):
+    x = np.concatenate([np.arange(-130, 131, dtype=np.float32) + 0.5,
+                        np.array([300.0, -300.0, 1e30, -1e30, 0.0, -0.0], np.float32)])
+    for T in (orc.QINT8, orc.QUINT8):
+        st, q_ref, _, _ = orc.quantize_v2(x, -127.0, 127.0, T, orc.SCALED)
+        q, _, _ = gpu_quantize(hip, dev, x, T, orc.SCALED, -127.0, 127.0)
+        if T == orc.QINT8:
+            np.testing.assert_array_equal(q, q_ref)
+            assert q[0] == -128 and q[130 + 0] % 2 == 0
+        else:
+            # quint8 SCALED scale is 255/127: not all ties, still must equal the oracle
+            np.testing.assert_array_equal(q, q_ref)
+
+
+def test_quantize_unaligned_pointers(hip, dev):
+    import torch
+    rng = np.random.default_rng(1)
+    x = rng.standard_normal(1000 + 3).astype(np.float32)
+    x_d = torch.from_numpy(x).to(dev)
+    q_d = torch.zeros(1003 + 8, dtype=torch.int8, device=dev)
+    # input offset by one float (not 16-byte aligned), output offset by 1 byte
+    hip.quantize(x_d.data_ptr() + 4, q_d.data_ptr() + 1, 1002, hip.QINT8, 20.0, 0.0)
+    torch.cuda.synchronize()
+    st, q_ref, _, _ = orc.quantize_v2(x[1:], -6.35, 6.35, orc.QINT8, orc.SCALED)
+    got = q_d.cpu().numpy()
+    np.testing.assert_array_equal(got[1:1003], q_ref)
+    assert got[0] == 0 and np.all(got[1003:] == 0)
+
+
+def test_narrow_range_flag_is_inert(hip, dev):
+    # the reference reads narrow_range and ignores it: there is no such argument at this level;
+    # saturation is full-range (-128) in both cases
+    q, _, _ = gpu_quantize(hip, dev, np.array([-10.0, 10.0], np.float32), orc.QINT8, orc.SCALED, -1.0, 1.0)
+    assert q.tolist() == [-128, 127]
+
+
+@pytest.mark.parametrize("T,mode", [(orc.QINT8, orc.SCALED), (orc.QUINT8, orc.SCALED),
+                                    (orc.QUINT8, orc.MIN_FIRST), (orc.QINT8, orc.MIN_FIRST)])
+@pytest.mark.parametrize("n", [1, 5, 4099, 1 << 20])
+def test_dequantize_vs_oracle(hip, dev, T, mode, n):
+    import torch
+    rng = np.random.default_rng(n)
+    info = np.iinfo(orc.NP_OF[T])
+    q = rng.integers(info.min, info.max + 1, n).astype(orc.NP_OF[T])
+    mn, mx = np.float32(-3.7), np.float32(5.2)
+    st, y_ref = orc.dequantize(q, mn, mx, T, mode)
+    st, _, _, sc, zp = orc.scale_zeropoint_align(T, mode, True, mn, mx)
+    q_d = torch.from_numpy(q).to(dev)
+    y_d = torch.empty(n, dtype=torch.float32, device=dev)
+    hip.dequantize(q_d, y_d, n, T, float(sc[0]), int(zp[0]) if mode == orc.MIN_FIRST else 0)
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(y_d.cpu().numpy(), y_ref)
+
+
+def test_dequantize_golden(hip, dev, golden):
+    import torch
+    g = golden["dequantize_axis"]
+    shape = np.array(g["shape"])
+    q = scale_per_slice(shape, None, np.array(g["values"], np.int32)).astype(np.int8)
+    deq = np.array(g["dequant_values"], np.float32)
+    for axis in g["axes"]:
+        expected = scale_per_slice(shape, axis, deq)
+        if axis is None:
+            mn, mx = [g["min_unit"]], [g["max_unit"]]
+        else:
+            mn = [g["min_unit"] * (s + 1) for s in range(shape[axis])]
+            mx = [g["max_unit"] * (s + 1) for s in range(shape[axis])]
+        st, _, _, sc, zp = orc.scale_zeropoint_align(orc.QINT8, orc.SCALED, True, mn, mx)
+        q_d = torch.from_numpy(q).to(dev)
+        y_d = torch.empty(q.shape, dtype=torch.float32, device=dev)
+        if axis is None:
+            hip.dequantize(q_d, y_d, q.size, orc.QINT8, float(sc[0]), 0)
+        else:
+            outer = int(np.prod(shape[:axis], dtype=np.int64))
+            inner = int(np.prod(shape[axis + 1:], dtype=np.int64))
+            hip.dequantize_axis(q_d, y_d, outer, int(shape[axis]), inner, orc.QINT8,
+                                torch.from_numpy(sc).to(dev), torch.from_numpy(zp).to(dev))
+        torch.cuda.synchronize()
+        y = y_d.cpu().numpy()
+        np.testing.assert_allclose(y, expected, rtol=g["tolerance"], atol=g["tolerance"])
+        st, y_ref = orc.dequantize(q, mn, mx, orc.QINT8, orc.SCALED, axis)
+        np.testing.assert_array_equal(y, y_ref)
+
+
+@pytest.mark.parametrize("out_type", [orc.QINT8, orc.QUINT8])
+@pytest.mark.parametrize("shape", [(1, 1, 1, 1), (2, 3, 5, 7), (2, 4, 8, 64), (1, 1, 4096, 1), (1, 1, 1000, 3), (4, 8, 16, 256)])
+def test_requantize_per_channel_vs_oracle(hip, dev, out_type, shape):
+    import torch
+    rng = np.random.default_rng(sum(shape))
+    x = np.rint(rng.standard_normal(shape) * (1 << 20)).astype(np.int32)
+    x.flat[0] = np.iinfo(np.int32).max
+    x.flat[-1] = np.iinfo(np.int32).min
+    depth = shape[-1]
+    in_min = -(rng.random(depth).astype(np.float32) * 8 + 0.1)
+    in_max = rng.random(depth).astype(np.float32) * 8 + 0.1
+    req_min, req_max = -0.004, 0.0035
+    st, q_ref, omn, omx = orc.requantize_per_channel(x, in_min, in_max, req_min, req_max, out_type)
+    factor = np.float32(127.0 if out_type == orc.QINT8 else 255.0)
+    mm = np.maximum(np.abs(in_min), np.abs(in_max))
+    scales = factor * (mm / np.maximum(np.abs(np.float32(req_min)), np.abs(np.float32(req_max))) / np.float32(2 ** 31))
+    x_d = torch.from_numpy(x).to(dev)
+    q_d = torch.empty(shape, dtype=tdtype(out_type), device=dev)
+    hip.requantize_per_channel(x_d, q_d, x.size // depth, depth, out_type, torch.from_numpy(scales).to(dev))
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(q_d.cpu().numpy(), q_ref)
+    if depth == 1:
+        hip.requantize(x_d, q_d.zero_(), x.size, out_type, float(scales[0]))
+        torch.cuda.synchronize()
+        np.testing.assert_array_equal(q_d.cpu().numpy(), q_ref)
+
+
+@pytest.mark.parametrize("shape", [(1, 1), (7, 1), (100003, 1), (1 << 20, 1), (33, 3), (1000, 64), (257, 300), (5, 1000)])
+def test_minmax_i32_per_channel(hip, dev, shape):
+    import torch
+    rng = np.random.default_rng(shape[0])
+    x = rng.integers(-2 ** 31, 2 ** 31, size=shape, dtype=np.int64).astype(np.int32)
+    x_d = torch.from_numpy(x).to(dev)
+    mn_d = torch.zeros(shape[1], dtype=torch.int32, device=dev)
+    mx_d = torch.zeros(shape[1], dtype=torch.int32, device=dev)
+    for _ in range(2):  # second call must not see the first call's result
+        hip.minmax_i32_per_channel(x_d, shape[0], shape[1], mn_d, mx_d)
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(mn_d.cpu().numpy(), x.min(0))
+    np.testing.assert_array_equal(mx_d.cpu().numpy(), x.max(0))
+    # the op's float range is host math on these integers: compare with the oracle end to end
+    in_min = -(rng.random(shape[1]).astype(np.float32) + 0.5)
+    in_max = rng.random(shape[1]).astype(np.float32) + 0.5
+    st, omn_ref, omx_ref = orc.requantization_range_per_channel(x, in_min, in_max, 6.0)
+    mn, mx = mn_d.cpu().numpy(), mx_d.cpu().numpy()
+    out = np.float32(np.finfo(np.float32).tiny)
+    nonneg = True
+    for c in range(shape[1]):
+        amax = np.int32(max(abs(int(mn[c])) if mn[c] != -2 ** 31 else -2 ** 31, abs(int(mx[c]))))
+        r = np.float32(max(abs(in_min[c]), abs(in_max[c]))) * np.float32(amax) / np.float32(2 ** 31)
+        out = max(out, np.float32(r))
+        nonneg = nonneg and mn[c] >= 0
+    out = min(out, np.float32(6.0))
+    assert np.float32(out) == omx_ref and (np.float32(0.0) if nonneg else -np.float32(out)) == omn_ref
+
+
+@pytest.mark.parametrize("n,offset", [(1, 0), (5, 0), (1027, 1), (1 << 20, 0), ((1 << 20) + 3, 3)])
+def test_minmax_f32(hip, dev, n, offset):
+    import torch
+    rng = np.random.default_rng(n)
+    x = outlier_normal(rng, n + offset, 1e-3, 50.0)
+    if n > 100:
+        x[offset + 17] = np.nan  # ignored
+    x_d = torch.from_numpy(x).to(dev)
+    out = torch.zeros(2, dtype=torch.float32, device=dev)
+    hip.minmax_f32(x_d.data_ptr() + 4 * offset, n, out)
+    torch.cuda.synchronize()
+    got = out.cpu().numpy()
+    assert got[0] == np.nanmin(x[offset:]) and got[1] == np.nanmax(x[offset:])
+
+
+def test_full_size_quantize_properties(hip, dev):
+    """2^28 elements (the benchmark size): oracle on a strided sample + structural properties."""
+    import torch
+    n = 1 << 28
+    g = torch.Generator(device=dev)
+    g.manual_seed(30)
+    x_d = torch.randn(n, device=dev, generator=g)
+    x_d[::9973] *= 50.0
+    mm = torch.zeros(2, dtype=torch.float32, device=dev)
+    hip.minmax_f32(x_d, n, mm)
+    mn, mx = [float(v) for v in mm.cpu().numpy()]
+    assert mn == float(x_d.min()) and mx == float(x_d.max())
+    for T, mode in ((orc.QINT8, orc.SCALED), (orc.QUINT8, orc.MIN_FIRST)):
+        sc, add, omn, omx = host_quant_params(T, mode, False, mn, mx)
+        q_d = torch.empty(n, dtype=tdtype(T), device=dev)
+        hip.quantize(x_d, q_d, n, T, float(sc[0]), float(add[0]))
+        torch.cuda.synchronize()
+        # sample: three windows (start, middle, end) checked exactly against the oracle
+        for lo in (0, n // 2 - 12345, n - (1 << 20)):
+            xs = x_d[lo:lo + (1 << 20)].cpu().numpy()
+            st, q_ref, _, _ = orc.quantize_v2(xs, mn, mx, T, mode)
+            np.testing.assert_array_equal(q_d[lo:lo + (1 << 20)].cpu().numpy(), q_ref)
+        # size-independent property: dequantize(quantize(x)) is within half a step of clip(x)
+        st, _, _, dsc, dzp = orc.scale_zeropoint_align(T, mode, True, omn, omx)
+        y_d = torch.empty(n, dtype=torch.float32, device=dev)
+        hip.dequantize(q_d, y_d, n, T, float(dsc[0]), int(dzp[0]))
+        torch.cuda.synchronize()
+        step = float(dsc[0])
+        err = float((y_d - x_d.clamp(float(omn[0]), float(omx[0]))).abs().max())
+        assert err <= step * (0.5 if mode == orc.SCALED else 1.0) * 1.001 + 1e-6
+        del q_d, y_d

@@ -1,0 +1,284 @@
+"""GPU parity of the quantized MatMul path through the C ABI versus the CPU oracle:
+prepack + column sums, device-side parameter preparation, MFMA tile kernel, small-M kernel and the
+shape-agnostic kernel.  int32 accumulators / int8 outputs / prepared vectors bit-exact; fp32 outputs
+bit-exact as well (bar: 1 ULP of the int32->fp32 scale product)."""
+import numpy as np
+import pytest
+
+from oracle import pyoracle as orc
+
+pytestmark = pytest.mark.gpu
+
+
+def tdt(T):
+    import torch
+    return {orc.QINT8: torch.int8, orc.QUINT8: torch.uint8, orc.QINT32: torch.int32, orc.FLOAT: torch.float32}[T]
+
+
+class Linear:
+    """A quantized linear layer resident on the GPU (weights prepacked once)."""
+
+    def __init__(self, hip, dev, wq, min_b, max_b, bias):
+        import torch
+        self.hip, self.dev = hip, dev
+        self.K, self.N = wq.shape
+        self.wq, self.min_b, self.max_b, self.bias = wq, np.atleast_1d(min_b), np.atleast_1d(max_b), bias
+        self.w_d = torch.from_numpy(wq).to(dev)
+        self.packed = torch.empty(hip.qgemm_packed_bytes(self.K, self.N), dtype=torch.int8, device=dev)
+        self.colsum = torch.empty(self.N, dtype=torch.int32, device=dev)
+        hip.qgemm_prepack_b(self.w_d, False, self.K, self.N, self.packed, self.colsum)
+        self.min_b_d = torch.from_numpy(self.min_b.astype(np.float32)).to(dev)
+        self.max_b_d = torch.from_numpy(self.max_b.astype(np.float32)).to(dev)
+        self.bias_d = torch.from_numpy(bias).to(dev)
+        self.scales_d = torch.empty(max(self.N, 1), dtype=torch.float32, device=dev)
+        self.sbias_d = torch.empty(self.N, dtype=torch.float32, device=dev)
+
+    def run(self, xq, kw, min_a, max_a, min_out=0.0, max_out=0.0, path="auto"):
+        import torch
+        hip = self.hip
+        M = xq.shape[0]
+        t_in = orc.QUINT8 if xq.dtype == np.uint8 else orc.QINT8
+        p = hip.matmul_params(t_in=t_in, min_a=float(min_a), max_a=float(max_a), min_out=float(min_out),
+                              max_out=float(max_out), **kw)
+        nb = self.min_b.size
+        ep = hip.qmatmul_epilogue_desc(p, nb)
+        hip.qmatmul_prepare(p, self.min_b_d, self.max_b_d, nb, self.bias_d, self.colsum, self.N,
+                            self.scales_d, self.sbias_d)
+        x_d = torch.from_numpy(xq).to(self.dev)
+        out = torch.empty((M, self.N), dtype=tdt(kw["t_out"]), device=self.dev)
+        fn = {"auto": hip.qgemm, "tile": hip.qgemm_tile, "gemv": hip.qgemv}.get(path)
+        if path == "naive":
+            hip.qgemm_naive(x_d, t_in, self.w_d, False, M, self.K, self.N, self.scales_d, self.sbias_d, ep,
+                            kw["t_out"], out)
+        else:
+            fn(x_d, t_in, self.packed, self.colsum, M, self.K, self.N, self.scales_d, self.sbias_d, ep,
+               kw["t_out"], out)
+        torch.cuda.synchronize()
+        return out.cpu().numpy()
+
+    def oracle(self, xq, kw, min_a, max_a, min_out=0.0, max_out=0.0):
+        t_in = orc.QUINT8 if xq.dtype == np.uint8 else orc.QINT8
+        at = orc.matmul_attrs(t_in=t_in, **kw)
+        st, y = orc.qmatmul(at, xq, self.wq, self.bias, min_a, max_a, self.min_b, self.max_b, min_out, max_out)
+        assert st == orc.OK
+        return y
+
+
+def make_layer(hip, dev, K, N, seed, per_channel=True, wstd=0.02):
+    rng = np.random.default_rng(seed)
+    w = (rng.standard_normal((K, N)) * wstd).astype(np.float32)
+    bias = (rng.standard_normal(N) * 0.01).astype(np.float32)
+    if per_channel:
+        r = np.abs(w).max(0).astype(np.float32)
+        _, wq, mn, mx = orc.quantize_v2(w, -r, r, orc.QINT8, orc.SCALED, axis=1)
+    else:
+        _, wq, mn, mx = orc.quantize_v2(w, w.min(), w.max(), orc.QINT8, orc.SCALED)
+    return Linear(hip, dev, wq, mn, mx, bias), w, bias
+
+
+def make_acts(M, K, seed, mode=orc.MIN_FIRST, outlier=0.0):
+    rng = np.random.default_rng(seed)
+    x = rng.standard_normal((M, K)).astype(np.float32)
+    if outlier:
+        idx = rng.integers(0, x.size, max(1, int(x.size * outlier)))
+        x.flat[idx] *= 20.0
+    T = orc.QUINT8 if mode == orc.MIN_FIRST else orc.QINT8
+    _, xq, mn, mx = orc.quantize_v2(x, x.min(), x.max(), T, mode)
+    return x, xq, float(mn[0]), float(mx[0])
+
+
+V2_DEQ = dict(api=orc.API_V2, t_out=orc.FLOAT, input_mode=orc.MIN_FIRST, has_dequantize=True)
+V2_DEQ_RELU = dict(V2_DEQ, activation=orc.ACT_RELU)
+V2_REQ_S8 = dict(api=orc.API_V2, t_out=orc.QINT8, input_mode=orc.MIN_FIRST, has_requantize=True)
+V2_REQ_U8_RELU = dict(api=orc.API_V2, t_out=orc.QUINT8, input_mode=orc.MIN_FIRST, has_requantize=True,
+                      activation=orc.ACT_RELU, n_fused_ops=2)
+V1_S32 = dict(api=orc.API_V1, t_out=orc.QINT32, input_mode=orc.MIN_FIRST, n_fused_ops=1)
+
+
+def test_prepack_colsum(hip, dev):
+    import torch
+    rng = np.random.default_rng(0)
+    for (K, N) in [(64, 16), (3, 4), (100, 37), (4096, 1024), (130, 48)]:
+        w = rng.integers(-128, 128, size=(K, N)).astype(np.int8)
+        w_d = torch.from_numpy(w).to(dev)
+        nbytes = hip.qgemm_packed_bytes(K, N)
+        packed = torch.full((nbytes,), 77, dtype=torch.int8, device=dev)
+        colsum = torch.full((N,), 123, dtype=torch.int32, device=dev)
+        hip.qgemm_prepack_b(w_d, False, K, N, packed, colsum)
+        torch.cuda.synchronize()
+        np.testing.assert_array_equal(colsum.cpu().numpy(), orc.weight_colsum(w))
+        # layout: chunk [n/16][k/64], lane (n%16) + 16*((k%64)/16), 16 consecutive k per lane
+        KT, NT = (K + 63) // 64, (N + 15) // 16
+        wp = np.zeros((NT * 16, KT * 64), np.int8)
+        wp[:N, :K] = w.T
+        ref = wp.reshape(NT, 16, KT, 4, 16).transpose(0, 2, 3, 1, 4).reshape(-1)
+        np.testing.assert_array_equal(packed.cpu().numpy(), ref)
+        # transposed source gives the same packing
+        wt_d = torch.from_numpy(np.ascontiguousarray(w.T)).to(dev)
+        packed2 = torch.empty_like(packed)
+        hip.qgemm_prepack_b(wt_d, True, K, N, packed2, colsum)
+        torch.cuda.synchronize()
+        np.testing.assert_array_equal(packed2.cpu().numpy(), ref)
+
+
+@pytest.mark.parametrize("kw", [V2_DEQ, V2_REQ_S8, V2_REQ_U8_RELU, V1_S32,
+                                dict(api=orc.API_V1, t_out=orc.QINT8, input_mode=orc.MIN_FIRST, n_fused_ops=1),
+                                dict(api=orc.API_V2, t_out=orc.QUINT8, input_mode=orc.MIN_FIRST, has_requantize=True,
+                                     out_min_first=True, activation=orc.ACT_RELU),
+                                dict(api=orc.API_V2, t_out=orc.FLOAT, input_mode=orc.SCALED, has_dequantize=True),
+                                dict(api=orc.API_V2, t_out=orc.QINT32, input_mode=orc.SCALED)])
+@pytest.mark.parametrize("per_channel", [True, False])
+def test_prepare_vs_oracle(hip, dev, kw, per_channel):
+    import torch
+    N, K = 200, 64
+    layer, w, bias = make_layer(hip, dev, K, N, 3, per_channel)
+    t_in = orc.QUINT8 if kw["input_mode"] == orc.MIN_FIRST else orc.QINT8
+    min_a, max_a, min_out, max_out = -2.3, 3.1, -1.7, 2.9
+    at = orc.matmul_attrs(t_in=t_in, **kw)
+    cs = orc.weight_colsum(layer.wq)
+    st, sc_ref, sb_ref, ep_ref = orc.qmatmul_prepare(at, N, cs, min_a, max_a, layer.min_b, layer.max_b,
+                                                     min_out, max_out, bias)
+    assert st == orc.OK
+    p = hip.matmul_params(t_in=t_in, min_a=min_a, max_a=max_a, min_out=min_out, max_out=max_out, **kw)
+    nb = layer.min_b.size
+    layer.scales_d.fill_(-7.0)
+    hip.qmatmul_prepare(p, layer.min_b_d, layer.max_b_d, nb, layer.bias_d, layer.colsum, N, layer.scales_d,
+                        layer.sbias_d)
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(layer.sbias_d.cpu().numpy(), sb_ref)
+    np.testing.assert_array_equal(layer.scales_d.cpu().numpy()[:ep_ref.n_scales], sc_ref)
+
+
+def test_reference_fused_matmul_case(hip, dev, golden):
+    """The 2x3 . 3x4 case of the reference's own test (K = 3 goes through the shape-agnostic kernel)."""
+    g = golden["fused_matmul"]
+    x = np.array(g["x"], np.float32)
+    w = np.array(g["w"], np.float32)
+    b = np.array(g["bias"], np.float32)
+    _, xq, xmn, xmx = orc.quantize_v2(x, x.min(), x.max(), orc.QUINT8, orc.MIN_FIRST)
+    for per_channel in (False, True):
+        if per_channel:
+            _, wq, wmn, wmx = orc.quantize_v2(w, w.min(0), w.max(0), orc.QINT8, orc.SCALED, axis=1)
+        else:
+            _, wq, wmn, wmx = orc.quantize_v2(w, w.min(), w.max(), orc.QINT8, orc.SCALED)
+        layer = Linear(hip, dev, wq, wmn, wmx, b)
+        for api in (orc.API_V1, orc.API_V2):
+            kw = dict(V2_DEQ, api=api)
+            y = layer.run(xq, kw, xmn[0], xmx[0], path="naive")
+            np.testing.assert_allclose(y, x @ w + b, rtol=g["tolerance"], atol=g["tolerance"])
+            np.testing.assert_array_equal(y, layer.oracle(xq, kw, xmn[0], xmx[0]))
+
+
+SHAPES = [(17, 64, 16), (32, 128, 48), (100, 256, 200), (256, 512, 256), (300, 1024, 520), (128, 1024, 1024),
+          (513, 192, 1000), (64, 4096, 64)]
+
+
+@pytest.mark.parametrize("M,K,N", SHAPES)
+@pytest.mark.parametrize("kw", [V2_DEQ_RELU, V2_REQ_S8, V1_S32])
+def test_tile_kernel_vs_oracle(hip, dev, M, K, N, kw):
+    layer, w, bias = make_layer(hip, dev, K, N, seed=K + N)
+    x, xq, mn, mx = make_acts(M, K, seed=M)
+    r_out = float(np.abs(x @ w + bias).max())
+    ref = layer.oracle(xq, kw, mn, mx, -r_out, r_out)
+    got = layer.run(xq, kw, mn, mx, -r_out, r_out, path="tile")
+    np.testing.assert_array_equal(got, ref)
+
+
+@pytest.mark.parametrize("M", [1, 2, 4, 7, 16])
+@pytest.mark.parametrize("K,N", [(64, 16), (256, 100), (4096, 512), (1024, 4096), (8192, 48)])
+@pytest.mark.parametrize("kw", [V2_DEQ, V2_REQ_S8])
+def test_gemv_kernel_vs_oracle(hip, dev, M, K, N, kw):
+    layer, w, bias = make_layer(hip, dev, K, N, seed=K + N + 1)
+    x, xq, mn, mx = make_acts(M, K, seed=M + 100)
+    r_out = float(np.abs(x @ w + bias).max())
+    ref = layer.oracle(xq, kw, mn, mx, -r_out, r_out)
+    np.testing.assert_array_equal(layer.run(xq, kw, mn, mx, -r_out, r_out, path="gemv"), ref)
+    np.testing.assert_array_equal(layer.run(xq, kw, mn, mx, -r_out, r_out, path="auto"), ref)
+    np.testing.assert_array_equal(layer.run(xq, kw, mn, mx, -r_out, r_out, path="tile"), ref)
+
+
+def test_signed_activations_and_extremes(hip, dev):
+    rng = np.random.default_rng(5)
+    K, N, M = 512, 64, 48
+    wq = rng.integers(-128, 128, size=(K, N)).astype(np.int8)
+    wq[:, 0] = -128
+    wq[:, 1] = 127
+    bias = np.zeros(N, np.float32)
+    layer = Linear(hip, dev, wq, np.float32([-1.0]), np.float32([1.0]), bias)
+    kw = dict(api=orc.API_V1, t_out=orc.QINT32, input_mode=orc.SCALED, n_fused_ops=1)
+    for dtype in (np.int8, np.uint8):
+        info = np.iinfo(dtype)
+        xq = rng.integers(info.min, info.max + 1, size=(M, K)).astype(dtype)
+        xq[0, :] = info.max
+        xq[1, :] = info.min
+        ref = layer.oracle(xq, kw, -1.0, 1.0)
+        exact = xq.astype(np.int64) @ wq.astype(np.int64)
+        # |acc| < 2^24 here so the fp32 round trip of the s32 output is exact
+        np.testing.assert_array_equal(ref, exact)
+        for path in ("tile", "naive"):
+            np.testing.assert_array_equal(layer.run(xq, kw, -1.0, 1.0, path=path), exact)
+        np.testing.assert_array_equal(layer.run(xq[:16], kw, -1.0, 1.0, path="gemv"), exact[:16])
+
+
+def test_config1_literal(hip, dev):
+    """BASELINE config 1: SCALED qint8 activations, per-channel weights, fp32 bias,
+    [BiasAdd, Relu, Requantize] -> quint8, V1 and V2 spellings agree with the oracle (including the
+    reference's as-written bias scaling and dropped requantize factor)."""
+    M, K, N = 128, 1024, 1024
+    layer, w, bias = make_layer(hip, dev, K, N, seed=0)
+    x, xq, mn, mx = make_acts(M, K, seed=0, mode=orc.SCALED)
+    r_out = float(np.maximum(x @ w + bias, 0).max())
+    for kw in (dict(api=orc.API_V1, t_out=orc.QUINT8, input_mode=orc.SCALED, activation=orc.ACT_RELU, n_fused_ops=2),
+               dict(api=orc.API_V2, t_out=orc.QUINT8, input_mode=orc.SCALED, activation=orc.ACT_RELU,
+                    has_requantize=True, n_fused_ops=3)):
+        ref = layer.oracle(xq, kw, mn, mx, 0.0, r_out)
+        np.testing.assert_array_equal(layer.run(xq, kw, mn, mx, 0.0, r_out), ref)
+
+
+@pytest.mark.parametrize("K,N,relu", [(768, 2304, False), (768, 768, False), (768, 3072, True), (3072, 768, False)])
+def test_bert_linears_rows_sampled(hip, dev, K, N, relu):
+    """BASELINE config 2 at full size (M = 4096); the oracle checks 96 sampled rows exactly."""
+    M = 4096
+    layer, w, bias = make_layer(hip, dev, K, N, seed=K * 3 + N)
+    x, xq, mn, mx = make_acts(M, K, seed=1)
+    kw = V2_DEQ_RELU if relu else V2_DEQ
+    got = layer.run(xq, kw, mn, mx)
+    rows = np.random.default_rng(2).choice(M, 96, replace=False)
+    ref = layer.oracle(xq[rows], kw, mn, mx)
+    np.testing.assert_array_equal(got[rows], ref)
+    full = np.maximum(x @ w + bias, 0) if relu else x @ w + bias
+    assert np.abs(got - full).max() < 0.2
+
+
+@pytest.mark.parametrize("K,N", [(4096, 4096), (4096, 6144), (4096, 14336), (14336, 4096)])
+def test_llama_prefill_rows_sampled(hip, dev, K, N):
+    """BASELINE config 4 at full size (M = 2048): int8 output bit-exact on 64 sampled rows, and the
+    size-independent property sum_n acc[m, n] = a[m, :] . rowsum(w) on the s32 output of all rows."""
+    import torch
+    M = 2048
+    layer, w, bias = make_layer(hip, dev, K, N, seed=20 + K % 7 + N % 11)
+    x, xq, mn, mx = make_acts(M, K, seed=21, outlier=1e-3)
+    r_out = float(np.abs(x[:64] @ w + bias).max()) * 1.5
+    got = layer.run(xq, V2_REQ_S8, mn, mx, -r_out, r_out)
+    rows = np.random.default_rng(3).choice(M, 64, replace=False)
+    ref = layer.oracle(xq[rows], V2_REQ_S8, mn, mx, -r_out, r_out)
+    np.testing.assert_array_equal(got[rows], ref)
+    # checksum of the raw accumulators over every row (zero bias, SCALED-mode bias path keeps it zero)
+    layer0 = Linear(hip, dev, layer.wq, layer.min_b, layer.max_b, np.zeros(N, np.float32))
+    kw = dict(api=orc.API_V1, t_out=orc.QINT32, input_mode=orc.SCALED, n_fused_ops=1)
+    acc = layer0.run(xq, kw, mn, mx).astype(np.int64)
+    if np.abs(acc).max() < 2 ** 24:  # exact through the fp32 epilogue only below 2^24
+        rowsum_w = layer.wq.astype(np.int64).sum(1)
+        np.testing.assert_array_equal(acc.sum(1), xq.astype(np.int64) @ rowsum_w)
+
+
+@pytest.mark.parametrize("M", [1, 4, 16])
+@pytest.mark.parametrize("K,N", [(4096, 14336), (14336, 4096)])
+def test_llama_decode_gemv(hip, dev, M, K, N):
+    """BASELINE config 3 at full size, every output checked against the oracle."""
+    layer, w, bias = make_layer(hip, dev, K, N, seed=10 + M)
+    layer_zero_bias = Linear(hip, dev, layer.wq, layer.min_b, layer.max_b, np.zeros(N, np.float32))
+    x, xq, mn, mx = make_acts(M, K, seed=11 + M)
+    ref = layer_zero_bias.oracle(xq, V2_DEQ, mn, mx)
+    np.testing.assert_array_equal(layer_zero_bias.run(xq, V2_DEQ, mn, mx), ref)
+    assert np.abs(ref - x @ w).max() < 0.2
