@@ -1,0 +1,315 @@
+#!/usr/bin/env python3
+"""Benchmark of the INT8 quantized-inference hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only NAME[,NAME...]] [--no-cpu]
+
+Headline ("value"): the Llama-3-8B-shaped INT8 prefill linear, M=2048 K=4096 N=14336, quint8
+activations x per-channel qint8 weights, fused bias + requantize to qint8 (`_QuantizedMatMul`
+fused_ops=[BiasAdd, Requantize]).  One step = the device-side parameter preparation kernel plus the
+MFMA GEMM kernel, inputs resident in HBM.  The same JSON line carries, under "others", the other
+benchmark workloads (standalone quantization ops at 2^28 elements, decode GEMV, BERT linears, the
+remaining prefill shapes), each with its own roofline fraction.
+
+Timing uses HIP events on the stream the kernels are launched on (PyTorch's current stream, whose
+raw handle is passed through the C ABI).
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_HBM_GBS = 8000.0      # MI355X HBM3E, published
+PEAK_INT8_TOPS = 5000.0    # MI355X dense int8 MFMA, published (tera-ops/s)
+
+
+def _setup():
+    import torch
+    import __graft_entry__ as entry
+    hip = entry.load_package().itexhip
+    if not torch.cuda.is_available():
+        raise SystemExit("bench.py needs a GPU (torch.cuda.is_available() is False)")
+    return torch, hip
+
+
+class Timer:
+    """HIP-event timing of `fn` launched `steps` times back to back on the current stream."""
+
+    def __init__(self, torch):
+        self.torch = torch
+
+    def run(self, fn, steps, warmup):
+        torch = self.torch
+        for i in range(warmup):
+            fn(i)
+        torch.cuda.synchronize()
+        start = torch.cuda.Event(enable_timing=True)
+        stop = torch.cuda.Event(enable_timing=True)
+        start.record()
+        for i in range(steps):
+            fn(warmup + i)
+        stop.record()
+        torch.cuda.synchronize()
+        return start.elapsed_time(stop) / steps  # ms per step
+
+
+def _stream(torch):
+    return torch.cuda.current_stream().cuda_stream
+
+
+# ------------------------------------------------------------------------------------------------
+# synthetic data
+# ------------------------------------------------------------------------------------------------
+def make_weights(torch, hip, K, N, seed, dev):
+    """qint8 symmetric per-output-channel weights from N(0, 0.02), prepacked; returns a dict."""
+    g = torch.Generator(device=dev)
+    g.manual_seed(seed)
+    w = torch.randn(K, N, device=dev, generator=g) * 0.02
+    r = w.abs().amax(0)
+    wq = torch.round(w * (127.0 / r)).clamp_(-127, 127).to(torch.int8)
+    del w
+    packed = torch.empty(hip.qgemm_packed_bytes(K, N), dtype=torch.int8, device=dev)
+    colsum = torch.empty(N, dtype=torch.int32, device=dev)
+    hip.qgemm_prepack_b(wq, False, K, N, packed, colsum, _stream(torch))
+    bias = torch.randn(N, device=dev, generator=g) * 0.01
+    return dict(K=K, N=N, wq=wq, packed=packed, colsum=colsum, min_b=(-r).contiguous(), max_b=r.contiguous(),
+                bias=bias, scales=torch.empty(N, dtype=torch.float32, device=dev),
+                sbias=torch.empty(N, dtype=torch.float32, device=dev))
+
+
+def make_acts(torch, hip, M, K, seed, dev, outlier_frac=0.0, outlier_mult=1.0):
+    """fp32 N(0,1) activations (+ outliers) quantized to quint8 with MIN_FIRST by the HIP kernel."""
+    from oracle import pyoracle as orc
+    g = torch.Generator(device=dev)
+    g.manual_seed(seed)
+    x = torch.randn(M, K, device=dev, generator=g)
+    if outlier_frac:
+        n_out = max(1, int(M * K * outlier_frac))
+        idx = torch.randint(0, M * K, (n_out,), device=dev, generator=g)
+        x.view(-1)[idx] *= outlier_mult
+    mn, mx = float(x.min()), float(x.max())
+    _, amn, amx = orc.adjust_input_range(mn, mx)
+    scale = orc.legacy_min_first_scale(orc.QUINT8, amn, amx)
+    xq = torch.empty(M, K, dtype=torch.uint8, device=dev)
+    import numpy as np
+    hip.quantize(x, xq, M * K, hip.QUINT8, float(scale), float(np.float32(-amn) * scale), _stream(torch))
+    return x, xq, float(amn), float(amx)
+
+
+# ------------------------------------------------------------------------------------------------
+# workloads
+# ------------------------------------------------------------------------------------------------
+def bench_linear(torch, hip, timer, M, K, N, kind, steps, warmup, dev, seed, rotate=1):
+    """kind: 'requant_s8' ([BiasAdd, Requantize] -> qint8), 'deq' / 'deq_relu' ([.., Dequantize] -> fp32).
+    rotate > 1 cycles through that many distinct weight copies so that the weight stream comes from
+    HBM, not from the 256 MiB last-level cache."""
+    layers = [make_weights(torch, hip, K, N, seed + i, dev) for i in range(rotate)]
+    x, xq, min_a, max_a = make_acts(torch, hip, M, K, seed + 100, dev,
+                                    outlier_frac=1e-3 if kind == "requant_s8" else 0.0, outlier_mult=20.0)
+    if kind == "requant_s8":
+        t_out, out_dtype = hip.QINT8, torch.int8
+        r_out = float((x[:64] @ (layers[0]["wq"].float() * (layers[0]["max_b"] / 127.0))).abs().max()) * 1.5
+        p = hip.matmul_params(api=hip.API_V2, t_in=hip.QUINT8, t_out=t_out, input_mode=hip.MIN_FIRST,
+                              has_requantize=True, min_a=min_a, max_a=max_a, min_out=-r_out, max_out=r_out)
+        out_bytes = 1
+    else:
+        t_out, out_dtype = hip.FLOAT, torch.float32
+        p = hip.matmul_params(api=hip.API_V2, t_in=hip.QUINT8, t_out=t_out, input_mode=hip.MIN_FIRST,
+                              has_dequantize=True,
+                              activation=hip.ACT_RELU if kind == "deq_relu" else hip.ACT_NONE,
+                              min_a=min_a, max_a=max_a)
+        out_bytes = 4
+    del x
+    ep = hip.qmatmul_epilogue_desc(p, N)
+    out = torch.empty(M, N, dtype=out_dtype, device=dev)
+    st = _stream(torch)
+
+    def step(i):
+        L = layers[i % rotate]
+        hip.qmatmul_prepare(p, L["min_b"], L["max_b"], N, L["bias"], L["colsum"], N, L["scales"], L["sbias"], st)
+        hip.qgemm(xq, hip.QUINT8, L["packed"], L["colsum"], M, K, N, L["scales"], L["sbias"], ep, t_out, out, st)
+
+    def gemm_only(i):
+        L = layers[i % rotate]
+        hip.qgemm(xq, hip.QUINT8, L["packed"], L["colsum"], M, K, N, L["scales"], L["sbias"], ep, t_out, out, st)
+
+    ms_step = timer.run(step, steps, warmup)
+    ms_kernel = timer.run(gemm_only, steps, warmup)
+    ops = 2.0 * M * N * K
+    nbytes = M * K + K * N + out_bytes * M * N + 8 * N
+    res = dict(M=M, K=K, N=N, kind=kind, ms_per_step=ms_step, us_kernel=ms_kernel * 1e3,
+               tops=ops / (ms_step * 1e-3) / 1e12, tops_kernel=ops / (ms_kernel * 1e-3) / 1e12,
+               gbs_kernel=nbytes / (ms_kernel * 1e-3) / 1e9, ops=ops, bytes=nbytes)
+    res["_ctx"] = dict(layers=layers, xq=xq, p=p, min_a=min_a, max_a=max_a)
+    return res
+
+
+def bench_elementwise(torch, hip, timer, n, steps, warmup, dev):
+    import numpy as np
+    from oracle import pyoracle as orc
+    g = torch.Generator(device=dev)
+    g.manual_seed(30)
+    x = torch.randn(n, device=dev, generator=g)
+    x[::10007] *= 50.0
+    st = _stream(torch)
+    mm = torch.zeros(2, dtype=torch.float32, device=dev)
+    hip.minmax_f32(x, n, mm, st)
+    mn, mx = [float(v) for v in mm.cpu().numpy()]
+    out = []
+
+    def add(name, fn, nbytes):
+        ms = timer.run(fn, steps, warmup)
+        out.append(dict(name=name, n=n, us_kernel=ms * 1e3, gbs=nbytes / (ms * 1e-3) / 1e9, bytes=nbytes,
+                        frac=nbytes / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS))
+
+    q8 = torch.empty(n, dtype=torch.int8, device=dev)
+    qu8 = torch.empty(n, dtype=torch.uint8, device=dev)
+    _, amn, amx = orc.adjust_input_range(mn, mx)
+    _, _, _, sc, _ = orc.scale_zeropoint_align(orc.QINT8, orc.SCALED, False, amn, amx)
+    add("quantize_v2_scaled_qint8", lambda i: hip.quantize(x, q8, n, hip.QINT8, float(sc[0]), 0.0, st), 5 * n)
+    scale = orc.legacy_min_first_scale(orc.QUINT8, amn, amx)
+    addend = float(np.float32(-amn) * scale)
+    add("quantize_v2_min_first_quint8", lambda i: hip.quantize(x, qu8, n, hip.QUINT8, float(scale), addend, st), 5 * n)
+    add("minmax_f32_range_pass", lambda i: hip.minmax_f32(x, n, mm, st), 4 * n)
+    y = x  # reuse the fp32 buffer as the dequantize output
+    _, _, _, dsc, dzp = orc.scale_zeropoint_align(orc.QUINT8, orc.MIN_FIRST, True, amn, amx)
+    add("dequantize_min_first_quint8", lambda i: hip.dequantize(qu8, y, n, hip.QUINT8, float(dsc[0]), int(dzp[0]), st), 5 * n)
+    _, _, _, dsc, _ = orc.scale_zeropoint_align(orc.QINT8, orc.SCALED, True, amn, amx)
+    add("dequantize_scaled_qint8", lambda i: hip.dequantize(q8, y, n, hip.QINT8, float(dsc[0]), 0, st), 5 * n)
+    # Requantize: int32 accumulators ~ N(0, 2^20), range pass then per-tensor requantize to qint8
+    acc = (torch.randn(n, device=dev, generator=g) * float(1 << 20)).round_().to(torch.int32)
+    imn = torch.zeros(1, dtype=torch.int32, device=dev)
+    imx = torch.zeros(1, dtype=torch.int32, device=dev)
+    add("requantization_range_int32", lambda i: hip.minmax_i32_per_channel(acc, n, 1, imn, imx, st), 4 * n)
+    amax = max(abs(int(imn.cpu())), abs(int(imx.cpu())))
+    # input range (-1, 1); requested range = the range the range-op reports: 1.0 * amax / 2^31
+    req = np.float32(1.0) * np.float32(amax) / np.float32(2.0 ** 31)
+    rscale = float(np.float32(127.0) * (np.float32(1.0) / req / np.float32(2.0 ** 31)))
+    add("requantize_int32_to_qint8", lambda i: hip.requantize(acc, q8, n, hip.QINT8, rscale, st), 5 * n)
+    return out
+
+
+def cpu_baseline_gemm(ctx, M_sample, K, N):
+    """The oracle (a scalar-C restatement of the reference's CPU path, OpenMP over rows) on the first
+    M_sample rows of the headline workload."""
+    import numpy as np
+    from oracle import pyoracle as orc
+    L = ctx["layers"][0]
+    xq = ctx["xq"][:M_sample].cpu().numpy()
+    wq = L["wq"].cpu().numpy()
+    bias = L["bias"].cpu().numpy()
+    min_b, max_b = L["min_b"].cpu().numpy(), L["max_b"].cpu().numpy()
+    p = ctx["p"]
+    at = orc.matmul_attrs(api=orc.API_V2, t_in=orc.QUINT8, t_out=orc.QINT8, input_mode=orc.MIN_FIRST,
+                          has_requantize=True)
+    t0 = time.perf_counter()
+    st, y = orc.qmatmul(at, xq, wq, bias, p.min_a, p.max_a, min_b, max_b, p.min_out, p.max_out)
+    dt = time.perf_counter() - t0
+    assert st == orc.OK
+    return 2.0 * M_sample * K * N / dt / 1e12, dt, y
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--only", type=str, default="", help="comma list of: headline, prefill, bert, gemv, elementwise")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--cpu-rows", type=int, default=2048, help="rows of the headline workload the CPU oracle runs")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU only: this build has no multi-GPU path (--gpus must be 1)", file=sys.stderr)
+        sys.exit(2)
+    only = set(s for s in args.only.split(",") if s) or {"headline", "prefill", "bert", "gemv", "elementwise"}
+
+    torch, hip = _setup()
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    timer = Timer(torch)
+    K_steps, W = args.steps, args.warmup
+    others = []
+
+    M, K, N = 2048, 4096, 14336
+    head = bench_linear(torch, hip, timer, M, K, N, "requant_s8", K_steps, W, dev, seed=22)
+    ctx = head.pop("_ctx")
+
+    cpu = None
+    if not args.no_cpu:
+        rows = min(args.cpu_rows, M)
+        tops_cpu, dt, y_cpu = cpu_baseline_gemm(ctx, rows, K, N)
+        # the same rows from the GPU must be identical
+        L = ctx["layers"][0]
+        ep = hip.qmatmul_epilogue_desc(ctx["p"], N)
+        out = torch.empty(M, N, dtype=torch.int8, device=dev)
+        hip.qmatmul_prepare(ctx["p"], L["min_b"], L["max_b"], N, L["bias"], L["colsum"], N, L["scales"], L["sbias"],
+                            _stream(torch))
+        hip.qgemm(ctx["xq"], hip.QUINT8, L["packed"], L["colsum"], M, K, N, L["scales"], L["sbias"], ep, hip.QINT8,
+                  out, _stream(torch))
+        torch.cuda.synchronize()
+        same = bool((out[:rows].cpu().numpy() == y_cpu).all())
+        cores = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
+        cpu = dict(value=tops_cpu, unit="TOP/s", cores=cores, kind="port",
+                   sample="first %d of %d rows of the headline workload (same weights), %.1f s; GPU rows identical: %s"
+                          % (rows, M, dt, same))
+    del ctx
+
+    if "prefill" in only:
+        for (k, n, seed) in ((4096, 4096, 20), (4096, 6144, 21), (14336, 4096, 23)):
+            r = bench_linear(torch, hip, timer, 2048, k, n, "requant_s8", K_steps, W, dev, seed)
+            r.pop("_ctx")
+            r.update(name="prefill_gemm", bound="mfma", frac=r["tops_kernel"] / PEAK_INT8_TOPS)
+            others.append(r)
+    if "bert" in only:
+        for (k, n, kind, seed) in ((768, 2304, "deq", 1), (768, 768, "deq", 2), (768, 3072, "deq_relu", 3),
+                                   (3072, 768, "deq", 4)):
+            r = bench_linear(torch, hip, timer, 4096, k, n, kind, K_steps, W, dev, seed)
+            r.pop("_ctx")
+            t_roof = max(r["ops"] / (PEAK_INT8_TOPS * 1e12), r["bytes"] / (PEAK_HBM_GBS * 1e9))
+            r.update(name="bert_linear", bound="max(mfma,hbm)", frac=t_roof / (r["us_kernel"] * 1e-6),
+                     frac_mfma=r["tops_kernel"] / PEAK_INT8_TOPS, frac_hbm=r["gbs_kernel"] / PEAK_HBM_GBS)
+            others.append(r)
+    if "gemv" in only:
+        for (k, n) in ((4096, 14336), (14336, 4096)):
+            for m in (1, 4, 16):
+                r = bench_linear(torch, hip, timer, m, k, n, "deq", K_steps, W, dev, seed=10, rotate=8)
+                r.pop("_ctx")
+                r.update(name="decode_gemv", bound="hbm", frac=r["gbs_kernel"] / PEAK_HBM_GBS,
+                         note="8 weight copies cycled (470 MB > last-level cache)")
+                others.append(r)
+    if "elementwise" in only:
+        for r in bench_elementwise(torch, hip, timer, 1 << 28, max(10, K_steps // 2), max(3, W // 2), dev):
+            r.update(bound="hbm")
+            others.append(r)
+
+    traffic = None
+    tpath = os.path.join(ROOT, "profiles", "traffic.json")
+    if os.path.exists(tpath):
+        try:
+            traffic = json.load(open(tpath)).get("qgemm_tile_prefill_2048x4096x14336")
+        except Exception:
+            traffic = None
+
+    line = {
+        "metric": "int8 GEMM TOPS (% MFMA peak); quantize/GEMV GB/s (% HBM peak), 1 MI355X",
+        "value": head["tops"], "unit": "TOP/s", "n_gpus": 1, "steps": K_steps, "warmup": W,
+        "ms_per_step": head["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "s8/u8 x s8 -> s32 (fp32 epilogue)", "data": "synthetic",
+        "config": {"workload": "Llama-3-8B prefill linear M=2048 K=4096 N=14336: quint8 act (MIN_FIRST, N(0,1) + 0.1% x20 "
+                               "outliers) x qint8 per-channel weights, _QuantizedMatMul [BiasAdd, Requantize] -> qint8; "
+                               "step = param-prep kernel + MFMA GEMM kernel"},
+        "roofline": {"bound": "mfma", "achieved": head["tops_kernel"], "peak": PEAK_INT8_TOPS, "unit": "TFLOP/s",
+                     "frac": head["tops_kernel"] / PEAK_INT8_TOPS, "traffic": traffic,
+                     "kernel": "qgemm_tile_kernel", "us_per_launch": head["us_kernel"],
+                     "note": "ops are int8 multiply-accumulates (2*M*N*K per launch); achieved and peak are tera-ops/s"},
+        "cpu_baseline": cpu,
+        "others": others,
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,92 +1,31 @@
 // Quantized MatMul on gfx950: u8/s8 activations x s8 weights -> exact int32 accumulation on the i8
-// MFMA (v_mfma_i32_16x16x64_i8), fused fp32 epilogue in registers.
+// MFMA (v_mfma_i32_32x32x32_i8: one wavefront alone keeps the matrix pipe ~94% busy with it, against
+// ~60% with the 16x16x64 form), fused fp32 epilogue in registers.
 //
-// Operand roles.  The weight is the MFMA "A" operand (its 16 rows are 16 output channels n), the
-// activation is the "B" operand (its 16 columns are 16 rows m of the activation matrix).  A lane then
-// ends up with 4 consecutive output channels of one output row, which is what a row-major [M,N]
-// output wants (4 int8 = one dword store, 4 fp32 = one 16-byte store).
+// Operand roles.  The weight is the MFMA "A" operand (its 32 rows are 32 output channels n), the
+// activation is the "B" operand (its 32 columns are 32 rows m of the activation matrix).  A lane then
+// ends up with groups of 4 consecutive output channels of one output row, which is what a row-major
+// [M,N] output wants (4 int8 = one dword store, 4 fp32 = one 16-byte store).
 //
-// Operand tile ("chunk") = 16 rows x 64 k = 1 KiB, stored in lane order: lane l holds 16 consecutive
-// k of row (l % 16), k-group (l / 16).  The prepacked weight is the sequence of such chunks
-// [n/16][k/64]; activation chunks are formed on the fly.  Both operands use the same (lane, byte) -> k
-// mapping, so the order in which the instruction consumes k inside a chunk cannot affect the integer
-// sum.
+// Operand tile ("chunk") = 32 rows x 32 k = 1 KiB, stored in lane order: lane l holds 16 consecutive
+// k of row (l % 32), k-group (l / 32).  The prepacked weight is the sequence of such chunks
+// [n/32][k/32] with k padded to a multiple of 64; activation chunks are formed on the fly.  Both
+// operands use the same (lane, byte) -> k mapping, so the order in which the instruction consumes k
+// inside a chunk cannot affect the integer sum.
 //
 // Unsigned activations: the MFMA is signed x signed, so u8 values are fed as (a ^ 0x80) = a - 128 and
 // the epilogue adds 128 * colsum[n] back (exact: |acc| <= 255 * 127 * K stays far below 2^31 for the
 // K this library accepts).
-#include <algorithm>
-
-#include "common.hpp"
+#include "qgemm_common.hpp"
 
 namespace itexhip {
-namespace {
 
-typedef int v4i __attribute__((ext_vector_type(4)));
-
-constexpr int kChunkBytes = 1024;  // 16 rows x 64 k
-constexpr int64_t kMaxK = 1 << 16; // 255 * 128 * 65536 < 2^31
-
-struct EpilogueArgs {
-  const float* scales;
-  const float* bias;
-  const int32_t* colsum;
-  int n_scales;
-  int comp_mul;  // 128 for u8 activations, 0 for s8
-  int n_eltwise;
-  itexhip_eltwise elt[2];
-};
-
-// ------------------------------------------------------------------------------------------------
-// Epilogue for one 16x16 accumulator tile held in MFMA layout: lane l, register r ->
-//   m = m0 + (l % 16), n = n0 + (l / 16) * 4 + r.
-// ------------------------------------------------------------------------------------------------
+// MFMA tile kernels, one translation unit per output type (qgemm_tile_*.hip)
 template <int OUT_T>
-__device__ __forceinline__ void epilogue_tile(const v4i& acc, int m, int n, int M, int N,
-                                              const EpilogueArgs& e, void* __restrict__ out,
-                                              bool vec_ok) {
-  if (m >= M || n >= N) return;
-  float y[4];
-  const bool full = (n + 3 < N);
-#pragma unroll
-  for (int r = 0; r < 4; ++r) {
-    const int nn = n + r;
-    if (!full && nn >= N) { y[r] = 0.0f; continue; }
-    int a = acc[r];
-    if (e.comp_mul) a += e.comp_mul * e.colsum[nn];
-    float v = static_cast<float>(a);
-    if (e.n_scales == 1) v = v * e.scales[0];
-    else if (e.n_scales > 1) v = v * e.scales[nn];
-    if (e.bias) v = v + e.bias[nn];
-    for (int k = 0; k < e.n_eltwise; ++k) v = apply_eltwise(e.elt[k], v);
-    y[r] = v;
-  }
-  const int64_t o = static_cast<int64_t>(m) * N + n;
-  if constexpr (OUT_T == ITEXHIP_FLOAT) {
-    float* p = reinterpret_cast<float*>(out) + o;
-    if (full && vec_ok) {
-      *reinterpret_cast<float4*>(p) = make_float4(y[0], y[1], y[2], y[3]);
-    } else {
-      for (int r = 0; r < 4 && n + r < N; ++r) p[r] = y[r];
-    }
-  } else if constexpr (OUT_T == ITEXHIP_QINT32) {
-    int32_t* p = reinterpret_cast<int32_t*>(out) + o;
-    if (full && vec_ok) {
-      *reinterpret_cast<int4*>(p) = make_int4(sat_rne<ITEXHIP_QINT32>(y[0]), sat_rne<ITEXHIP_QINT32>(y[1]),
-                                              sat_rne<ITEXHIP_QINT32>(y[2]), sat_rne<ITEXHIP_QINT32>(y[3]));
-    } else {
-      for (int r = 0; r < 4 && n + r < N; ++r) p[r] = sat_rne<ITEXHIP_QINT32>(y[r]);
-    }
-  } else {
-    uint8_t* p = reinterpret_cast<uint8_t*>(out) + o;
-    if (full && vec_ok) {
-      *reinterpret_cast<uint32_t*>(p) =
-          pack4(sat_rne<OUT_T>(y[0]), sat_rne<OUT_T>(y[1]), sat_rne<OUT_T>(y[2]), sat_rne<OUT_T>(y[3]));
-    } else {
-      for (int r = 0; r < 4 && n + r < N; ++r) p[r] = static_cast<uint8_t>(sat_rne<OUT_T>(y[r]));
-    }
-  }
-}
+int dispatch_tile(const uint8_t* a, uint32_t a_xor, const uint8_t* bp, int M, int K, int N,
+                  const EpilogueArgs& e, void* out, hipStream_t st);
+
+namespace {
 
 // ------------------------------------------------------------------------------------------------
 // Weight prepack + column sums.  One thread produces one 16-byte piece (row n, 16 consecutive k).
@@ -104,8 +43,8 @@ __global__ __launch_bounds__(256) void prepack_b_kernel(const int8_t* __restrict
   if (chunk >= static_cast<int64_t>(NT) * KT) return;  // whole wavefront leaves together
   const int lane = threadIdx.x & 63;
   const int nt = static_cast<int>(chunk / KT), kt = static_cast<int>(chunk % KT);
-  const int n = nt * 16 + (lane & 15);
-  const int k0 = kt * 64 + (lane >> 4) * 16;
+  const int n = nt * kChunkRows + (lane & 31);
+  const int k0 = kt * kChunkK + (lane >> 5) * 16;
   union { int8_t b[16]; v4i v; } piece;
   int sum = 0;
 #pragma unroll
@@ -118,185 +57,84 @@ __global__ __launch_bounds__(256) void prepack_b_kernel(const int8_t* __restrict
     sum += v;
   }
   *reinterpret_cast<v4i*>(packed + chunk * kChunkBytes + lane * 16) = piece.v;
-  // add up the four k-groups of this row, then one atomic per row and chunk
-  sum += __shfl_xor(sum, 16, 64);
+  // add up the two k-groups of this row, then one atomic per row and chunk
   sum += __shfl_xor(sum, 32, 64);
-  if (lane < 16 && n < N && sum != 0) atomicAdd(&colsum[n], sum);
+  if (lane < 32 && n < N && sum != 0) atomicAdd(&colsum[n], sum);
 }
 
 // ------------------------------------------------------------------------------------------------
-// Tile kernel (compute bound, M > 16).
-//   block tile BM (activation rows) x BN (output channels), K step 64 (one chunk deep),
-//   WAVES_M x WAVES_N wavefronts, each owning a (BM/WAVES_M) x (BN/WAVES_N) sub-tile,
-//   double-buffered LDS staging in chunk order, global -> register -> LDS prefetch of the next step
-//   while the MFMAs of the current one run.
-// ------------------------------------------------------------------------------------------------
-template <int BM, int BN, int WAVES_M, int WAVES_N, int OUT_T>
-__global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void qgemm_tile_kernel(
-    const uint8_t* __restrict__ a, uint32_t a_xor, const uint8_t* __restrict__ bp, int M, int K, int N,
-    int KT, int NT, int num_m, int num_n, EpilogueArgs e, void* __restrict__ out) {
-  constexpr int NW = WAVES_M * WAVES_N;
-  constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
-  constexpr int TM = WM / 16, TN = WN / 16;
-  constexpr int A_CHUNKS = BM / 16, B_CHUNKS = BN / 16;
-  constexpr int A_PER_WAVE = A_CHUNKS / NW, B_PER_WAVE = B_CHUNKS / NW;
-  static_assert(A_CHUNKS % NW == 0 && B_CHUNKS % NW == 0, "chunks must divide among wavefronts");
-  constexpr int STAGE_BYTES = (A_CHUNKS + B_CHUNKS) * kChunkBytes;
-
-  extern __shared__ __align__(16) uint8_t lds[];
-
-  // ---- block -> tile mapping: consecutive workgroup ids go round-robin to the 8 XCDs; give every
-  // XCD a contiguous range of tiles (m fastest) so that the tiles sharing a weight panel share an L2.
-  int pid = blockIdx.x;
-  const int total = num_m * num_n;
-  if ((total & 7) == 0) pid = (pid & 7) * (total >> 3) + (pid >> 3);
-  const int tile_m = pid % num_m, tile_n = pid / num_m;
-  const int m_base = tile_m * BM, n_base = tile_n * BN;
-
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const int wm = wave % WAVES_M, wn = wave / WAVES_M;
-  const int lrow = lane & 15, lgrp = lane >> 4;
-
-  v4i acc[TN][TM];
-#pragma unroll
-  for (int j = 0; j < TN; ++j)
-#pragma unroll
-    for (int i = 0; i < TM; ++i) acc[j][i] = v4i{0, 0, 0, 0};
-
-  v4i stage_a[A_PER_WAVE], stage_b[B_PER_WAVE];
-
-  auto load_global = [&](int kt) {
-#pragma unroll
-    for (int c = 0; c < A_PER_WAVE; ++c) {
-      const int chunk = wave * A_PER_WAVE + c;
-      const int m = m_base + chunk * 16 + lrow;
-      const int k = kt * 64 + lgrp * 16;
-      v4i v = v4i{0, 0, 0, 0};
-      if (m < M && k < K) v = *reinterpret_cast<const v4i*>(a + static_cast<int64_t>(m) * K + k);
-      stage_a[c] = v;
-    }
-#pragma unroll
-    for (int c = 0; c < B_PER_WAVE; ++c) {
-      const int nt = (n_base >> 4) + wave * B_PER_WAVE + c;
-      v4i v = v4i{0, 0, 0, 0};
-      if (nt < NT)
-        v = *reinterpret_cast<const v4i*>(bp + (static_cast<int64_t>(nt) * KT + kt) * kChunkBytes + lane * 16);
-      stage_b[c] = v;
-    }
-  };
-  auto store_lds = [&](int buf) {
-    uint8_t* base = lds + buf * STAGE_BYTES;
-#pragma unroll
-    for (int c = 0; c < A_PER_WAVE; ++c) {
-      v4i v = stage_a[c];
-      v.x ^= a_xor; v.y ^= a_xor; v.z ^= a_xor; v.w ^= a_xor;
-      *reinterpret_cast<v4i*>(base + (wave * A_PER_WAVE + c) * kChunkBytes + lane * 16) = v;
-    }
-#pragma unroll
-    for (int c = 0; c < B_PER_WAVE; ++c)
-      *reinterpret_cast<v4i*>(base + (A_CHUNKS + wave * B_PER_WAVE + c) * kChunkBytes + lane * 16) = stage_b[c];
-  };
-  auto compute = [&](int buf) {
-    const uint8_t* base = lds + buf * STAGE_BYTES;
-    v4i fa[TM], fb[TN];
-#pragma unroll
-    for (int i = 0; i < TM; ++i)
-      fa[i] = *reinterpret_cast<const v4i*>(base + (wm * TM + i) * kChunkBytes + lane * 16);
-#pragma unroll
-    for (int j = 0; j < TN; ++j)
-      fb[j] = *reinterpret_cast<const v4i*>(base + (A_CHUNKS + wn * TN + j) * kChunkBytes + lane * 16);
-#pragma unroll
-    for (int j = 0; j < TN; ++j)
-#pragma unroll
-      for (int i = 0; i < TM; ++i)
-        acc[j][i] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fb[j], fa[i], acc[j][i], 0, 0, 0);
-  };
-
-  load_global(0);
-  store_lds(0);
-  __syncthreads();
-  for (int kt = 0; kt < KT; ++kt) {
-    const int buf = kt & 1;
-    if (kt + 1 < KT) load_global(kt + 1);
-    compute(buf);
-    if (kt + 1 < KT) store_lds(buf ^ 1);
-    __syncthreads();
-  }
-
-  const bool vec_ok = (N & 3) == 0;
-#pragma unroll
-  for (int j = 0; j < TN; ++j)
-#pragma unroll
-    for (int i = 0; i < TM; ++i) {
-      const int m = m_base + (wm * TM + i) * 16 + lrow;
-      const int n = n_base + (wn * TN + j) * 16 + lgrp * 4;
-      epilogue_tile<OUT_T>(acc[j][i], m, n, M, N, e, out, vec_ok);
-    }
-}
-
-// ------------------------------------------------------------------------------------------------
-// Small-M kernel (M <= 16, bandwidth bound on the weight).  One workgroup owns one 16-channel strip
-// of the weight, a contiguous stream of KT chunks; its WAVES wavefronts take chunks round-robin
-// (all of a wavefront's loads are issued before the first MFMA), multiply them with the matching
-// activation chunk, and the partial 16x16 tiles are added up through LDS.
+// Small-M kernel (M <= 16, bandwidth bound on the weight).  One workgroup owns one 32-channel strip
+// of the weight, a contiguous stream of KC chunks (1 KiB each, one fully coalesced wavefront load);
+// its WAVES wavefronts take chunks round-robin (all loads of a batch are issued before the first
+// MFMA), multiply them with the matching activation chunk (rows >= M are zero), and the partial
+// 32x32 tiles are added up in LDS with integer atomics (exact, order free).
 // ------------------------------------------------------------------------------------------------
 template <int WAVES, int OUT_T>
 __global__ __launch_bounds__(64 * WAVES) void qgemv_kernel(const uint8_t* __restrict__ a, uint32_t a_xor,
                                                            const uint8_t* __restrict__ bp, int M, int K,
-                                                           int N, int KT, EpilogueArgs e,
+                                                           int N, int KC, EpilogueArgs e,
                                                            void* __restrict__ out) {
   constexpr int UNROLL = 4;
-  __shared__ int red[WAVES][64 * 4];
+  __shared__ int red[16 * 64];
   const int nt = blockIdx.x;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const int lrow = lane & 15, lgrp = lane >> 4;
-  const uint8_t* strip = bp + static_cast<int64_t>(nt) * KT * kChunkBytes + lane * 16;
+  const int lrow = lane & 31, lgrp = lane >> 5;
+  const uint8_t* strip = bp + static_cast<int64_t>(nt) * KC * kChunkBytes + lane * 16;
   const uint8_t* arow = a + static_cast<int64_t>(lrow) * K + lgrp * 16;
   const bool row_ok = lrow < M;
 
-  v4i acc = v4i{0, 0, 0, 0};
-  int kt = wave;
-  for (; kt + (UNROLL - 1) * WAVES < KT; kt += UNROLL * WAVES) {
+  v16i acc;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) acc[r] = 0;
+  auto act_chunk = [&](int kc) {
+    v4i v = v4i{0, 0, 0, 0};
+    if (row_ok && kc * kChunkK + lgrp * 16 < K) {
+      v = *reinterpret_cast<const v4i*>(arow + static_cast<int64_t>(kc) * kChunkK);
+      v.x ^= a_xor; v.y ^= a_xor; v.z ^= a_xor; v.w ^= a_xor;
+    }
+    return v;
+  };
+  int kc = wave;
+  for (; kc + (UNROLL - 1) * WAVES < KC; kc += UNROLL * WAVES) {
     v4i w[UNROLL], x[UNROLL];
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u)
       w[u] = __builtin_nontemporal_load(
-          reinterpret_cast<const v4i*>(strip + static_cast<int64_t>(kt + u * WAVES) * kChunkBytes));
+          reinterpret_cast<const v4i*>(strip + static_cast<int64_t>(kc + u * WAVES) * kChunkBytes));
 #pragma unroll
-    for (int u = 0; u < UNROLL; ++u) {
-      const int k = (kt + u * WAVES) * 64 + lgrp * 16;
-      v4i v = v4i{0, 0, 0, 0};
-      if (row_ok && k < K) {
-        v = *reinterpret_cast<const v4i*>(arow + static_cast<int64_t>(kt + u * WAVES) * 64);
-        v.x ^= a_xor; v.y ^= a_xor; v.z ^= a_xor; v.w ^= a_xor;
-      }
-      x[u] = v;
-    }
+    for (int u = 0; u < UNROLL; ++u) x[u] = act_chunk(kc + u * WAVES);
 #pragma unroll
-    for (int u = 0; u < UNROLL; ++u) acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(w[u], x[u], acc, 0, 0, 0);
+    for (int u = 0; u < UNROLL; ++u) acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(w[u], x[u], acc, 0, 0, 0);
   }
-  for (; kt < KT; kt += WAVES) {
+  for (; kc < KC; kc += WAVES) {
     const v4i w = __builtin_nontemporal_load(
-        reinterpret_cast<const v4i*>(strip + static_cast<int64_t>(kt) * kChunkBytes));
-    const int k = kt * 64 + lgrp * 16;
-    v4i v = v4i{0, 0, 0, 0};
-    if (row_ok && k < K) {
-      v = *reinterpret_cast<const v4i*>(arow + static_cast<int64_t>(kt) * 64);
-      v.x ^= a_xor; v.y ^= a_xor; v.z ^= a_xor; v.w ^= a_xor;
-    }
-    acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(w, v, acc, 0, 0, 0);
+        reinterpret_cast<const v4i*>(strip + static_cast<int64_t>(kc) * kChunkBytes));
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(w, act_chunk(kc), acc, 0, 0, 0);
   }
 
-#pragma unroll
-  for (int r = 0; r < 4; ++r) red[wave][r * 64 + lane] = acc[r];
-  __syncthreads();
+  // cross-wavefront reduction: wavefront 0 stores, the others add
   if (wave == 0) {
-    v4i s = v4i{0, 0, 0, 0};
 #pragma unroll
-    for (int w = 0; w < WAVES; ++w)
+    for (int r = 0; r < 16; ++r) red[r * 64 + lane] = acc[r];
+  }
+  __syncthreads();
+  if (wave != 0) {
 #pragma unroll
-      for (int r = 0; r < 4; ++r) s[r] += red[w][r * 64 + lane];
-    epilogue_tile<OUT_T>(s, lrow, nt * 16 + lgrp * 4, M, N, e, out, (N & 3) == 0);
+    for (int r = 0; r < 16; ++r) atomicAdd(&red[r * 64 + lane], acc[r]);
+  }
+  __syncthreads();
+  if (wave == 0 && row_ok) {
+    const bool vec_ok = (N & 3) == 0 && aligned16(e.scales) && aligned16(e.bias) && aligned16(e.colsum) && aligned16(out);
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const int n = nt * kChunkRows + g * 8 + lgrp * 4;
+      if (n < N) {
+        const v4i part = v4i{red[(4 * g + 0) * 64 + lane], red[(4 * g + 1) * 64 + lane], red[(4 * g + 2) * 64 + lane],
+                             red[(4 * g + 3) * 64 + lane]};
+        const ChannelParams p = load_channel_params(e, n, N, vec_ok);
+        epilogue_store<OUT_T, 2>(part, p, lrow, n, M, N, e, out, vec_ok);
+      }
+    }
   }
 }
 
@@ -365,46 +203,16 @@ EpilogueArgs make_args(int a_type, const int32_t* colsum, const float* scales, c
   return e;
 }
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, int OUT_T>
-int launch_tile(const uint8_t* a, uint32_t a_xor, const uint8_t* bp, int M, int K, int N,
-                const EpilogueArgs& e, void* out, hipStream_t st) {
-  const int KT = (K + 63) / 64, NT = (N + 15) / 16;
-  const int num_m = (M + BM - 1) / BM, num_n = (N + BN - 1) / BN;
-  constexpr size_t lds_bytes = 2 * (BM / 16 + BN / 16) * kChunkBytes;
-  auto kern = qgemm_tile_kernel<BM, BN, WAVES_M, WAVES_N, OUT_T>;
-  static bool attr_set = false;  // benign race: the call is idempotent
-  if (!attr_set) {
-    hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes));
-    if (err != hipSuccess) return hip_fail(err, "hipFuncSetAttribute(qgemm_tile_kernel)");
-    attr_set = true;
-  }
-  kern<<<dim3(static_cast<unsigned>(num_m * num_n)), dim3(64 * WAVES_M * WAVES_N), lds_bytes, st>>>(
-      a, a_xor, bp, M, K, N, KT, NT, num_m, num_n, e, out);
-  return ITEXHIP_OK;
-}
-
-template <int OUT_T>
-int dispatch_tile(const uint8_t* a, uint32_t a_xor, const uint8_t* bp, int M, int K, int N,
-                  const EpilogueArgs& e, void* out, hipStream_t st) {
-  // pick the largest tile that still gives every CU work
-  const int64_t tiles_256 = static_cast<int64_t>((M + 255) / 256) * ((N + 255) / 256);
-  const int64_t tiles_128 = static_cast<int64_t>((M + 127) / 128) * ((N + 127) / 128);
-  if (tiles_256 >= 256) return launch_tile<256, 256, 2, 2, OUT_T>(a, a_xor, bp, M, K, N, e, out, st);
-  if (tiles_128 >= 256) return launch_tile<128, 128, 2, 2, OUT_T>(a, a_xor, bp, M, K, N, e, out, st);
-  return launch_tile<64, 64, 2, 2, OUT_T>(a, a_xor, bp, M, K, N, e, out, st);
-}
-
 template <int OUT_T>
 int dispatch_gemv(const uint8_t* a, uint32_t a_xor, const uint8_t* bp, int M, int K, int N,
                   const EpilogueArgs& e, void* out, hipStream_t st) {
-  const int KT = (K + 63) / 64, NT = (N + 15) / 16;
-  if (KT >= 128)
-    qgemv_kernel<16, OUT_T><<<NT, 64 * 16, 0, st>>>(a, a_xor, bp, M, K, N, KT, e, out);
-  else if (KT >= 32)
-    qgemv_kernel<8, OUT_T><<<NT, 64 * 8, 0, st>>>(a, a_xor, bp, M, K, N, KT, e, out);
+  const int KC = 2 * ((K + 63) / 64), NT = (N + kChunkRows - 1) / kChunkRows;
+  if (KC >= 256)
+    qgemv_kernel<16, OUT_T><<<NT, 64 * 16, 0, st>>>(a, a_xor, bp, M, K, N, KC, e, out);
+  else if (KC >= 64)
+    qgemv_kernel<8, OUT_T><<<NT, 64 * 8, 0, st>>>(a, a_xor, bp, M, K, N, KC, e, out);
   else
-    qgemv_kernel<2, OUT_T><<<NT, 64 * 2, 0, st>>>(a, a_xor, bp, M, K, N, KT, e, out);
+    qgemv_kernel<2, OUT_T><<<NT, 64 * 2, 0, st>>>(a, a_xor, bp, M, K, N, KC, e, out);
   return ITEXHIP_OK;
 }
 
@@ -426,6 +234,7 @@ int packed_path(bool gemv, const void* a, int a_type, const int8_t* packed_b, co
   ITEXHIP_REQUIRE(aligned(a, 16) && aligned(packed_b, 16), "%s: operands must be 16-byte aligned", who);
   ITEXHIP_REQUIRE(a_type != ITEXHIP_QUINT8 || colsum, "%s: quint8 activations need colsum", who);
   ITEXHIP_REQUIRE(!gemv || M <= 16, "%s: M must be <= 16", who);
+  ITEXHIP_REQUIRE(M * K < (1LL << 31), "%s: activation matrix too large (M * K must be < 2^31)", who);
   const uint32_t a_xor = (a_type == ITEXHIP_QUINT8) ? 0x80808080u : 0u;
   const EpilogueArgs e = make_args(a_type, colsum, scales, bias, ep);
   const uint8_t* ap = reinterpret_cast<const uint8_t*>(a);
@@ -454,7 +263,7 @@ using namespace itexhip;
 
 extern "C" int64_t itexhip_qgemm_packed_bytes(int64_t K, int64_t N) {
   if (K < 0 || N < 0) return -1;
-  return ((N + 15) / 16) * ((K + 63) / 64) * kChunkBytes;
+  return ((N + kChunkRows - 1) / kChunkRows) * (2 * ((K + 63) / 64)) * kChunkBytes;
 }
 
 extern "C" int itexhip_qgemm_prepack_b(const int8_t* w, int transpose_b, int64_t K, int64_t N,
@@ -467,7 +276,7 @@ extern "C" int itexhip_qgemm_prepack_b(const int8_t* w, int transpose_b, int64_t
   if (K > 0) {
     ITEXHIP_REQUIRE(w && packed, "itexhip_qgemm_prepack_b: null buffer");
     ITEXHIP_REQUIRE(aligned(packed, 16), "itexhip_qgemm_prepack_b: packed buffer must be 16-byte aligned");
-    const int KT = static_cast<int>((K + 63) / 64), NT = static_cast<int>((N + 15) / 16);
+    const int KT = 2 * static_cast<int>((K + 63) / 64), NT = static_cast<int>((N + kChunkRows - 1) / kChunkRows);
     const int64_t chunks = static_cast<int64_t>(KT) * NT;
     prepack_b_kernel<<<static_cast<unsigned>((chunks + 3) / 4), 256, 0, st>>>(
         w, transpose_b, static_cast<int>(K), static_cast<int>(N), KT, NT, packed, colsum);

@@ -107,11 +107,12 @@ def test_prepack_colsum(hip, dev):
         hip.qgemm_prepack_b(w_d, False, K, N, packed, colsum)
         torch.cuda.synchronize()
         np.testing.assert_array_equal(colsum.cpu().numpy(), orc.weight_colsum(w))
-        # layout: chunk [n/16][k/64], lane (n%16) + 16*((k%64)/16), 16 consecutive k per lane
-        KT, NT = (K + 63) // 64, (N + 15) // 16
-        wp = np.zeros((NT * 16, KT * 64), np.int8)
+        # layout: chunk [n/32][k/32] (k padded to a multiple of 64), lane (n%32) + 32*((k%32)/16),
+        # 16 consecutive k per lane
+        KC, NT = 2 * ((K + 63) // 64), (N + 31) // 32
+        wp = np.zeros((NT * 32, KC * 32), np.int8)
         wp[:N, :K] = w.T
-        ref = wp.reshape(NT, 16, KT, 4, 16).transpose(0, 2, 3, 1, 4).reshape(-1)
+        ref = wp.reshape(NT, 32, KC, 2, 16).transpose(0, 2, 3, 1, 4).reshape(-1)
         np.testing.assert_array_equal(packed.cpu().numpy(), ref)
         # transposed source gives the same packing
         wt_d = torch.from_numpy(np.ascontiguousarray(w.T)).to(dev)
