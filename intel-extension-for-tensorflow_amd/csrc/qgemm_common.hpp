@@ -84,6 +84,34 @@ __device__ __forceinline__ ChannelParams load_channel_params(const EpilogueArgs&
   return p;
 }
 
+// The 4 outputs of one channel group in registers: epilogue arithmetic + conversion, no store.
+// 8-bit outputs come back packed in .x; 32-bit outputs as 4 lanes of raw bits.
+template <int OUT_T, int ACT>
+__device__ __forceinline__ v4i epilogue_convert(const v4i acc, const ChannelParams& p, const EpilogueArgs& e) {
+  float y[4];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    float v = static_cast<float>(acc[r] + p.comp[r]);
+    v = v * p.scale[r];
+    if (e.bias) v = v + p.bias[r];
+    if (ACT == 1) {
+      v = fmaxf(v, 0.0f);
+    } else if (ACT == 2) {
+      for (int k = 0; k < e.n_eltwise; ++k) v = apply_eltwise(e.elt[k], v);
+    }
+    y[r] = v;
+  }
+  if constexpr (OUT_T == ITEXHIP_FLOAT) {
+    return v4i{__float_as_int(y[0]), __float_as_int(y[1]), __float_as_int(y[2]), __float_as_int(y[3])};
+  } else if constexpr (OUT_T == ITEXHIP_QINT32) {
+    return v4i{sat_rne<ITEXHIP_QINT32>(y[0]), sat_rne<ITEXHIP_QINT32>(y[1]), sat_rne<ITEXHIP_QINT32>(y[2]),
+               sat_rne<ITEXHIP_QINT32>(y[3])};
+  } else {
+    return v4i{static_cast<int>(pack4(sat_rne<OUT_T>(y[0]), sat_rne<OUT_T>(y[1]), sat_rne<OUT_T>(y[2]),
+                                      sat_rne<OUT_T>(y[3]))), 0, 0, 0};
+  }
+}
+
 template <int OUT_T, int ACT>
 __device__ __forceinline__ void epilogue_store(const v4i acc, const ChannelParams& p, int m, int n, int M, int N,
                                                const EpilogueArgs& e, void* __restrict__ out, bool vec_ok) {

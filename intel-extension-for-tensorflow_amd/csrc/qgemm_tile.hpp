@@ -9,29 +9,45 @@ namespace itexhip {
 
 // ------------------------------------------------------------------------------------------------
 // Tile kernel (compute bound, M > 16).
-//   Block tile BM (activation rows) x BN (output channels), K step 64 (two chunks deep),
+//   Block tile BM (activation rows) x BN (output channels), K step 64 (two 32-deep MFMA chunks),
 //   WAVES_M x WAVES_N wavefronts, each owning a (BM/WAVES_M) x (BN/WAVES_N) sub-tile of accumulators
 //   (TM x TN tiles of 32x32, 16 registers each, kept in AGPRs).
 //
-//   Software pipeline over K steps, one barrier per step, ring of 3 LDS stages:
-//     step k computes from stage k%3; it reads the fragments of step k+1 from stage (k+1)%3 (published
-//     by the previous barrier), writes the chunks of step k+2 (loaded from global memory during step
-//     k-1) into stage (k+2)%3 and issues the global loads of step k+3.
+//   Operands reach LDS by direct global->LDS loads (global_load_lds_dwordx4: each lane's 16 bytes land
+//   at LDS base + 16 * lane, no VGPRs and no ds_write on the way).  LDS is the busiest unit of this
+//   kernel (128 B/clk shared by fragment reads and staging), so staging must not cost store slots.
+//
+//   Software pipeline over K steps, one barrier per step, ring of 4 LDS stages:
+//     step k computes from stage k%4 and reads the fragments of step k+1 from stage (k+1)%4; the loads
+//     of step k+3 are issued into stage (k+3)%4; before the barrier that ends step k each wavefront
+//     waits for its loads of step k+2 (issued during step k-1, a full step earlier).
 //   Inside a step the work is cut into 2*TN slices (k-chunk kc, channel tile j) of TM MFMAs: the weight
 //   fragment of the next slice is read while the MFMAs of the current one run, so only two weight
 //   fragments are live; the activation fragments of the next step are read one slice at a time into a
-//   second register set; staging stores and global loads are spread over the slices the same way.
+//   second register set; the loads are spread over the slices the same way.
 //
-//   Activation staging.  One wavefront load covers 16 rows x 64 B (4 lanes per row: the texture
-//   addresser serves a quad of lanes per cycle only when the quad is contiguous).  In LDS the piece
-//   (row r, k-chunk kc, k-group g) lives in chunk kc of its 32-row tile at 16-byte slot
-//   (g*32 + r) ^ (4*kc + 2*g); the XOR spreads the 8 lanes an LDS cycle serves over the 8 bank groups
-//   for the staging stores and keeps the fragment reads (lane l reads slot l ^ (4*kc + 2*(l/32)))
-//   conflict free.  Weight chunks are already in lane order in memory and are copied linearly.
+//   Activation staging.  One wavefront load covers 16 rows x 64 B, 4 consecutive lanes per row (the
+//   texture addresser serves a quad of lanes per cycle only when the quad is contiguous).  Quad q of a
+//   load holds row q; inside the quad, piece p (= 2*kc + g, 16 bytes of k) sits at lane
+//   p ^ ((q >> 1) & 3).  That rotation makes the fragment reads conflict free: the 8 lanes an LDS cycle
+//   serves read 8 consecutive rows, whose 16-byte slots then fall into 8 different bank groups.
+//   Weight chunks are already in fragment lane order in memory and are copied linearly.
+//   Unsigned activations are turned into signed ones (x ^ 0x80) after the fragment read.
 //
 //   Rows >= M and channel tiles >= NT are loaded from clamped (valid) addresses: whatever they
 //   contribute lands in outputs that are never stored.  Columns k >= K multiply zero-padded weights.
 // ------------------------------------------------------------------------------------------------
+__device__ __forceinline__ void lds_dma16(const void* gptr, uint32_t lds_addr) {
+  // m0 = LDS byte address of lane 0's destination; the instruction adds 16 * lane
+  asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(gptr), "s"(lds_addr) : "memory", "m0");
+}
+
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+  // s_waitcnt with only vmcnt active (gfx9 encoding: vmcnt[3:0] | expcnt 7 << 4 | lgkmcnt 15 << 8 | vmcnt[5:4] << 14)
+  __builtin_amdgcn_s_waitcnt((N & 15) | (7 << 4) | (15 << 8) | ((N >> 4) << 14));
+}
+
 template <int BM, int BN, int WAVES_M, int WAVES_N, int OUT_T, int ACT>
 __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void qgemm_tile_kernel(
     const uint8_t* __restrict__ a, uint32_t a_xor, const uint8_t* __restrict__ bp, int M, int K, int N,
@@ -39,16 +55,21 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void qgemm_tile_kernel(
   constexpr int NW = WAVES_M * WAVES_N;
   constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
   constexpr int TM = WM / 32, TN = WN / 32;
-  constexpr int A_TILES = BM / 32, B_TILES = BN / 32;      // 32-row tiles per block
+  constexpr int A_TILES = BM / 32, B_TILES = BN / 32;          // 32-row tiles per block
   constexpr int A_LOADS = A_TILES * 2, B_LOADS = B_TILES * 2;  // wavefront loads (1 KiB each) per step
   constexpr int A_PER_WAVE = A_LOADS / NW, B_PER_WAVE = B_LOADS / NW;
-  constexpr int NSTG = A_PER_WAVE + B_PER_WAVE;
+  constexpr int NLD = A_PER_WAVE + B_PER_WAVE;                 // loads per wavefront per step
   constexpr int NSLICE = 2 * TN;
+  constexpr int NSTAGE = 4;
   static_assert(A_LOADS % NW == 0 && B_LOADS % NW == 0, "loads must divide among wavefronts");
+  static_assert(NLD < 32, "vmcnt budget");
+  static_assert(NSLICE % 2 == 0, "slices come in two halves");
   constexpr int STAGE_BYTES = (A_LOADS + B_LOADS) * kChunkBytes;
   constexpr int B_REGION = A_LOADS * kChunkBytes;
 
   extern __shared__ __align__(16) uint8_t lds[];
+  const uint32_t lds_base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(
+      (__attribute__((address_space(3))) void*)lds));
 
   // ---- block -> tile mapping: consecutive workgroup ids go round-robin to the 8 XCDs; give every
   // XCD a contiguous range of tiles (m fastest) so that the tiles sharing a weight panel share an L2.
@@ -58,7 +79,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void qgemm_tile_kernel(
   const int tile_m = pid % num_m, tile_n = pid / num_m;
   const int m_base = tile_m * BM, n_base = tile_n * BN;
 
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const int wm = wave % WAVES_M, wn = wave / WAVES_M;
   const int lrow = lane & 31, lgrp = lane >> 5;
 
@@ -68,127 +89,187 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void qgemm_tile_kernel(
     for (int r = 0; r < 16; ++r) acc[t][r] = 0;
   });
 
-  // ---- staging sources / destinations of this wavefront
-  // activation load c covers rows [16*h, 16*h+16) of 32-row tile rt, both k-chunks: lane -> (row, piece)
-  const int q_row = lane >> 2, q_piece = lane & 3;  // piece = kc*2 + g
-  uint32_t off_a[A_PER_WAVE];   // byte offset of (row, piece 0.., k = 0) in the activation matrix
-  uint32_t dst_a[A_PER_WAVE];   // byte offset inside a stage
+  // ---- staging sources of this wavefront
+  // activation load `ld` covers rows [16*h, 16*h+16) of 32-row tile rt: lane -> (row q, piece p)
+  const int q_row = lane >> 2;
+  const int q_piece = (lane & 3) ^ ((q_row >> 1) & 3);  // piece = 2*kc + g
+  uint32_t off_a[A_PER_WAVE];  // byte offset of the lane's row in the activation matrix
   const uint8_t* src_b[B_PER_WAVE];
-  uint32_t dst_b[B_PER_WAVE];
   static_for<A_PER_WAVE>([&](auto c) {
-    const int ld = wave * A_PER_WAVE + c;  // 0 .. A_LOADS-1
-    const int rt = ld >> 1, h = ld & 1;
-    const int r = h * 16 + q_row;
-    const int m = min(m_base + rt * 32 + r, M - 1);
+    const int ld = wave * A_PER_WAVE + c;  // 0 .. A_LOADS-1 = (rt, h)
+    const int m = min(m_base + ld * 16 + q_row, M - 1);
     off_a[c] = static_cast<uint32_t>(m) * static_cast<uint32_t>(K);  // M * K < 2^31 checked by the host
-    const int kc = q_piece >> 1, g = q_piece & 1;
-    dst_a[c] = static_cast<uint32_t>((rt * 2 + kc) * kChunkBytes + (((g * 32 + r) ^ (4 * kc + 2 * g)) << 4));
   });
   static_for<B_PER_WAVE>([&](auto c) {
-    const int ld = wave * B_PER_WAVE + c;  // 0 .. B_LOADS-1: (channel tile, k-chunk)
+    const int ld = wave * B_PER_WAVE + c;  // 0 .. B_LOADS-1 = (channel tile, k-chunk)
     const int nt = min((n_base >> 5) + (ld >> 1), NT - 1);
     src_b[c] = bp + (static_cast<int64_t>(nt) * (2 * KT) + (ld & 1)) * kChunkBytes + lane * 16;
-    dst_b[c] = static_cast<uint32_t>(B_REGION + ld * kChunkBytes + lane * 16);
   });
-
-  v4i stg[NSTG];
-  auto load_chunk = [&](auto c, int kt) {
+  auto issue_load = [&](auto c, int kt, int stage) {
     constexpr int ci = decltype(c)::value;
+    const uint32_t stage_addr = lds_base + stage * STAGE_BYTES;
     if constexpr (ci < A_PER_WAVE) {
       const uint32_t kofs = static_cast<uint32_t>(min(kt * 64 + q_piece * 16, K - 16));
-      stg[ci] = *reinterpret_cast<const v4i*>(a + off_a[ci] + kofs);
+      lds_dma16(a + off_a[ci] + kofs, stage_addr + (wave * A_PER_WAVE + ci) * kChunkBytes);
     } else {
-      stg[ci] = *reinterpret_cast<const v4i*>(src_b[ci - A_PER_WAVE] + static_cast<int64_t>(kt) * (2 * kChunkBytes));
-    }
-  };
-  auto store_chunk = [&](auto c, int stage) {
-    constexpr int ci = decltype(c)::value;
-    uint8_t* base = lds + stage * STAGE_BYTES;
-    if constexpr (ci < A_PER_WAVE) {
-      v4i v = stg[ci];
-      v.x ^= a_xor; v.y ^= a_xor; v.z ^= a_xor; v.w ^= a_xor;
-      *reinterpret_cast<v4i*>(base + dst_a[ci]) = v;
-    } else {
-      *reinterpret_cast<v4i*>(base + dst_b[ci - A_PER_WAVE]) = stg[ci];
+      lds_dma16(src_b[ci - A_PER_WAVE] + static_cast<int64_t>(kt) * (2 * kChunkBytes),
+                stage_addr + B_REGION + (wave * B_PER_WAVE + (ci - A_PER_WAVE)) * kChunkBytes);
     }
   };
   // fragment reads: activation fragment (k-chunk kc, row tile i of this wavefront), weight fragment (kc, j)
-  const uint32_t frag_a_lane[2] = {static_cast<uint32_t>((lane ^ (2 * lgrp)) << 4),
-                                   static_cast<uint32_t>((lane ^ (4 + 2 * lgrp)) << 4)};
-  auto lds_a = [&](int stage, int kc, int i) {
-    return *reinterpret_cast<const v4i*>(lds + stage * STAGE_BYTES + ((wm * TM + i) * 2 + kc) * kChunkBytes + frag_a_lane[kc]);
+  const int fq = lrow & 15, fh = lrow >> 4;
+  const uint32_t frag_a_lane[2] = {
+      static_cast<uint32_t>(fh * kChunkBytes + ((4 * fq + ((0 + lgrp) ^ ((fq >> 1) & 3))) << 4)),
+      static_cast<uint32_t>(fh * kChunkBytes + ((4 * fq + ((2 + lgrp) ^ ((fq >> 1) & 3))) << 4))};
+  auto lds_a_raw = [&](int stage, int kc, int i) {
+    return *reinterpret_cast<const v4i*>(lds + stage * STAGE_BYTES + (wm * TM + i) * (2 * kChunkBytes) + frag_a_lane[kc]);
+  };
+  auto flip = [&](v4i v) {  // u8 -> s8 (x - 128) for unsigned activations, identity for signed ones
+    v.x ^= a_xor; v.y ^= a_xor; v.z ^= a_xor; v.w ^= a_xor;
+    return v;
   };
   auto lds_b = [&](int stage, int kc, int j) {
     return *reinterpret_cast<const v4i*>(lds + stage * STAGE_BYTES + B_REGION + ((wn * TN + j) * 2 + kc) * kChunkBytes + lane * 16);
   };
 
-  // ---- prologue: stages 0 and 1 filled, chunks of step 2 in flight
-  static_for<NSTG>([&](auto c) { load_chunk(c, 0); });
-  static_for<NSTG>([&](auto c) { store_chunk(c, 0); });
-  static_for<NSTG>([&](auto c) { load_chunk(c, min(1, KT - 1)); });
-  static_for<NSTG>([&](auto c) { store_chunk(c, 1); });
-  static_for<NSTG>([&](auto c) { load_chunk(c, min(2, KT - 1)); });
+  // ---- prologue: loads of steps 0, 1, 2 in flight; wait for steps 0 and 1
+  static_for<NLD>([&](auto c) { issue_load(c, 0, 0); });
+  static_for<NLD>([&](auto c) { issue_load(c, min(1, KT - 1), 1); });
+  static_for<NLD>([&](auto c) { issue_load(c, min(2, KT - 1), 2); });
+  wait_vmcnt<NLD>();
   __syncthreads();
 
-  v4i fa_cur[2 * TM], fa_nxt[2 * TM], fb[2], fb_first;
-  static_for<2 * TM>([&](auto x) { fa_cur[x] = lds_a(0, decltype(x)::value / TM, decltype(x)::value % TM); });
+  v4i fa0[2 * TM], fa1[2 * TM], fb[2];
+  static_for<2 * TM>([&](auto x) { fa0[x] = lds_a_raw(0, decltype(x)::value / TM, decltype(x)::value % TM); });
+  static_for<2 * TM>([&](auto x) { fa0[x] = flip(fa0[x]); });
   fb[0] = lds_b(0, 0, 0);
 
-  // K loop, branch free: past the end of K the prefetches read stale stages / clamped addresses and
-  // the staging stores go to a stage nobody reads any more.  All LDS reads of a step are issued in
-  // slices 0 .. NSLICE-2, so the MFMAs of the last slice cover their latency before the barrier.
-  int st_cur = 0, st_nxt = 1, st_fill = 2;
-  for (int kt = 0; kt < KT; ++kt) {
+  // One K step, branch free: past the end of K the loads re-fetch the last step into stages nobody
+  // reads and the prefetches read stale stages.
+  //
+  // A wavefront that runs alone on its SIMD only hides other instructions in the shadow of an MFMA
+  // (32 cycles for 32x32x32) if they are issued between two MFMAs, so the step is laid out as
+  // NSLICE * TM slots of "one MFMA + a little other work" and the compiler is kept from regrouping
+  // them.  Per slice (k-chunk kc, channel tile j): slot 0 reads the weight fragment of the next
+  // slice, the following slots read (first half of the step) or sign-flip (second half) the
+  // activation fragments of the next step, the last slot issues one global->LDS load.
+  // The two activation fragment sets swap roles from step to step (loop unrolled by two).
+  constexpr int FA = 2 * TM;                       // activation fragments per step
+  constexpr int FA_PER_SLICE = (FA + NSLICE / 2 - 1) / (NSLICE / 2);
+  static_assert(FA_PER_SLICE + 2 <= TM || TM < 4, "slots per slice");
+  auto step = [&](int kt, const v4i (&fa_cur)[FA], v4i (&fa_nxt)[FA]) {
+    const int st_cur = kt & 3, st_nxt = (kt + 1) & 3, st_fill = (kt + 3) & 3;
     const int kt_load = min(kt + 3, KT - 1);
     static_for<NSLICE>([&](auto sl) {
       constexpr int s = decltype(sl)::value;
       constexpr int kc = s / TN, j = s % TN;
-      // staging traffic of this slice
-      static_for<NSTG>([&](auto c) {
-        if constexpr (decltype(c)::value * NSLICE / NSTG == s) {
-          store_chunk(c, st_fill);
-          load_chunk(c, kt_load);
-        }
-      });
-      // fragment prefetch of this slice
-      if constexpr (s + 1 < NSLICE) fb[(s + 1) & 1] = lds_b(st_cur, (s + 1) / TN, (s + 1) % TN);
-      if constexpr (s == NSLICE - 2) fb_first = lds_b(st_nxt, 0, 0);
-      static_for<2 * TM>([&](auto x) {
-        if constexpr (decltype(x)::value * (NSLICE - 1) / (2 * TM) == s)
-          fa_nxt[x] = lds_a(st_nxt, decltype(x)::value / TM, decltype(x)::value % TM);
-      });
       static_for<TM>([&](auto i) {
-        constexpr int t = j * TM + decltype(i)::value;
-        acc[t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fb[s & 1], fa_cur[kc * TM + decltype(i)::value], acc[t], 0, 0, 0);
+        constexpr int ii = decltype(i)::value;
+        constexpr int t = j * TM + ii;
+        acc[t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fb[s & 1], fa_cur[kc * TM + ii], acc[t], 0, 0, 0);
+        // ---- the slot behind this MFMA
+        if constexpr (ii == 0) {
+          if constexpr (s + 1 < NSLICE) fb[(s + 1) & 1] = lds_b(st_cur, (s + 1) / TN, (s + 1) % TN);
+          else fb[0] = lds_b(st_nxt, 0, 0);  // NSLICE is even: fb[0] was last used by slice NSLICE-2
+        }
+        if constexpr (ii == TM - 1) {
+          static_for<NLD>([&](auto c) {
+            if constexpr (decltype(c)::value * NSLICE / NLD == s) issue_load(c, kt_load, st_fill);
+          });
+        }
+        if constexpr ((TM < 3) ? (ii == 0) : (ii >= 1 && ii <= FA_PER_SLICE)) {
+          constexpr int slot = (TM < 3) ? 0 : ii - 1;
+          constexpr int per = (TM < 3) ? FA_PER_SLICE : 1;
+          static_for<per>([&](auto u) {
+            constexpr int x = (s % (NSLICE / 2)) * FA_PER_SLICE + slot * per + decltype(u)::value;
+            if constexpr (x < FA) {
+              if constexpr (s < NSLICE / 2) fa_nxt[x] = lds_a_raw(st_nxt, x / TM, x % TM);
+              else fa_nxt[x] = flip(fa_nxt[x]);
+            }
+          });
+        }
+        __builtin_amdgcn_sched_barrier(0);
       });
-      __builtin_amdgcn_sched_barrier(0);
     });
-    static_for<2 * TM>([&](auto x) { fa_cur[x] = fa_nxt[x]; });
-    fb[0] = fb_first;
+    wait_vmcnt<NLD>();  // the loads of step kt+2 (issued during step kt-1) have landed
     __syncthreads();
-    const int t = st_cur;
-    st_cur = st_nxt;
-    st_nxt = st_fill;
-    st_fill = t;
+  };
+  int kt = 0;
+  if (KT & 1) {  // odd step count: one step first, then hand its prefetched fragments to set 0
+    step(0, fa0, fa1);
+    static_for<2 * TM>([&](auto x) { fa0[x] = fa1[x]; });
+    kt = 1;
   }
+  for (; kt < KT; kt += 2) {
+    step(kt, fa0, fa1);
+    step(kt + 1, fa1, fa0);
+  }
+  wait_vmcnt<0>();  // no load may still be writing LDS when the epilogue reuses it
+  __syncthreads();
 
-  // ---- epilogue straight from the accumulator registers
+  // ---- epilogue.  Fast path: convert in registers, transpose through a private LDS buffer (the ring
+  // is free after the last barrier) and store rows of 128 contiguous bytes, 16 B per lane.  A lane of
+  // the MFMA layout owns one row and scattered 4-channel groups, which would make every store a
+  // 64-address scatter.  The buffer holds [WM rows][ROWB bytes] with a 16-byte pad per row: for 8-bit
+  // outputs all TN channel tiles at once, for 32-bit outputs one channel tile per pass.
+  constexpr int ESZ = (OUT_T == ITEXHIP_QINT8 || OUT_T == ITEXHIP_QUINT8) ? 1 : 4;
+  constexpr int JB = (ESZ == 1) ? TN : 1;    // channel tiles per pass
+  constexpr int ROWB = JB * 32 * ESZ;        // row bytes in the buffer
+  constexpr int PITCH = ROWB + 16;
+  constexpr int LPR = ROWB / 16;             // lanes per row when flushing
+  constexpr int RPP = 64 / LPR;              // rows per flush instruction
+  static_assert(NW * WM * PITCH <= NSTAGE * STAGE_BYTES, "epilogue buffer must fit in the ring");
   const bool vec_ok = (N & 3) == 0 && aligned16(e.scales) && aligned16(e.bias) && aligned16(e.colsum) && aligned16(out);
-  static_for<TN>([&](auto j) {
-    static_for<4>([&](auto g) {
-      const int n = n_base + (wn * TN + j) * 32 + decltype(g)::value * 8 + lgrp * 4;
-      if (n < N) {
-        const ChannelParams p = load_channel_params(e, n, N, vec_ok);
-        static_for<TM>([&](auto i) {
-          constexpr int t = decltype(j)::value * TM + decltype(i)::value;
-          constexpr int r0 = decltype(g)::value * 4;
-          const int m = m_base + (wm * TM + i) * 32 + lrow;
-          const v4i part = v4i{acc[t][r0], acc[t][r0 + 1], acc[t][r0 + 2], acc[t][r0 + 3]};
-          epilogue_store<OUT_T, ACT>(part, p, m, n, M, N, e, out, vec_ok);
+  const bool fast = vec_ok && ((static_cast<int64_t>(N) * ESZ) & 15) == 0;
+  if (fast) {
+    uint8_t* ebuf = lds + wave * (WM * PITCH);
+    const int f_row = lane / LPR, f_piece = lane % LPR;
+    static_for<TN / JB>([&](auto jb) {
+      static_for<JB>([&](auto jj) {
+        constexpr int j = decltype(jb)::value * JB + decltype(jj)::value;
+        static_for<4>([&](auto g) {
+          const int n = n_base + (wn * TN + j) * 32 + decltype(g)::value * 8 + lgrp * 4;
+          const ChannelParams p = load_channel_params(e, min(n, N - 4), N, true);
+          static_for<TM>([&](auto i) {
+            constexpr int t = j * TM + decltype(i)::value;
+            constexpr int r0 = decltype(g)::value * 4;
+            const v4i part = v4i{acc[t][r0], acc[t][r0 + 1], acc[t][r0 + 2], acc[t][r0 + 3]};
+            const v4i o = epilogue_convert<OUT_T, ACT>(part, p, e);
+            uint8_t* dst = ebuf + (decltype(i)::value * 32 + lrow) * PITCH +
+                           (decltype(jj)::value * 32 + decltype(g)::value * 8 + lgrp * 4) * ESZ;
+            if constexpr (ESZ == 1) *reinterpret_cast<int*>(dst) = o.x;
+            else *reinterpret_cast<v4i*>(dst) = o;
+          });
         });
+      });
+      // flush: lane -> (row, 16-byte piece); LDS operations of one wavefront complete in order
+      const int n_col = n_base + (wn * TN + decltype(jb)::value * JB) * 32 + f_piece * (16 / ESZ);
+#pragma unroll
+      for (int pass = 0; pass < WM / RPP; ++pass) {
+        const int row = pass * RPP + f_row;
+        const v4i v = *reinterpret_cast<const v4i*>(ebuf + row * PITCH + f_piece * 16);
+        const int m = m_base + wm * WM + row;
+        if (m < M && n_col < N)  // N * ESZ is a multiple of 16, so a piece is entirely inside or outside
+          *reinterpret_cast<v4i*>(reinterpret_cast<uint8_t*>(out) + (static_cast<int64_t>(m) * N + n_col) * ESZ) = v;
       }
     });
-  });
+  } else {
+    static_for<TN>([&](auto j) {
+      static_for<4>([&](auto g) {
+        const int n = n_base + (wn * TN + j) * 32 + decltype(g)::value * 8 + lgrp * 4;
+        if (n < N) {
+          const ChannelParams p = load_channel_params(e, n, N, vec_ok);
+          static_for<TM>([&](auto i) {
+            constexpr int t = decltype(j)::value * TM + decltype(i)::value;
+            constexpr int r0 = decltype(g)::value * 4;
+            const int m = m_base + (wm * TM + i) * 32 + lrow;
+            const v4i part = v4i{acc[t][r0], acc[t][r0 + 1], acc[t][r0 + 2], acc[t][r0 + 3]};
+            epilogue_store<OUT_T, ACT>(part, p, m, n, M, N, e, out, vec_ok);
+          });
+        }
+      });
+    });
+  }
 }
 
 template <int BM, int BN, int WAVES_M, int WAVES_N, int OUT_T, int ACT>
@@ -196,7 +277,7 @@ int launch_tile(const uint8_t* a, uint32_t a_xor, const uint8_t* bp, int M, int 
                 const EpilogueArgs& e, void* out, hipStream_t st) {
   const int KT = (K + 63) / 64, NT = (N + kChunkRows - 1) / kChunkRows;
   const int num_m = (M + BM - 1) / BM, num_n = (N + BN - 1) / BN;
-  constexpr size_t lds_bytes = 3 * (BM / 16 + BN / 16) * kChunkBytes;
+  constexpr size_t lds_bytes = 4 * (BM / 16 + BN / 16) * kChunkBytes;
   auto kern = qgemm_tile_kernel<BM, BN, WAVES_M, WAVES_N, OUT_T, ACT>;
   static bool attr_set = false;  // benign race: the call is idempotent
   if (!attr_set) {
