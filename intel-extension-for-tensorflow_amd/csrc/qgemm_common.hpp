@@ -86,6 +86,9 @@ __device__ __forceinline__ ChannelParams load_channel_params(const EpilogueArgs&
 
 // The 4 outputs of one channel group in registers: epilogue arithmetic + conversion, no store.
 // 8-bit outputs come back packed in .x; 32-bit outputs as 4 lanes of raw bits.
+// 8-bit conversion: after the clamp to [lo, hi] (integers, |.| <= 255) adding 1.5 * 2^23 in fp32
+// rounds to nearest even and leaves the integer in the low mantissa bits (two's complement for
+// negatives), so the low byte of the sum is the result: one add instead of round + convert.
 template <int OUT_T, int ACT>
 __device__ __forceinline__ v4i epilogue_convert(const v4i acc, const ChannelParams& p, const EpilogueArgs& e) {
   float y[4];
@@ -107,8 +110,16 @@ __device__ __forceinline__ v4i epilogue_convert(const v4i acc, const ChannelPara
     return v4i{sat_rne<ITEXHIP_QINT32>(y[0]), sat_rne<ITEXHIP_QINT32>(y[1]), sat_rne<ITEXHIP_QINT32>(y[2]),
                sat_rne<ITEXHIP_QINT32>(y[3])};
   } else {
-    return v4i{static_cast<int>(pack4(sat_rne<OUT_T>(y[0]), sat_rne<OUT_T>(y[1]), sat_rne<OUT_T>(y[2]),
-                                      sat_rne<OUT_T>(y[3]))), 0, 0, 0};
+    uint32_t b[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      float v = fminf(fmaxf(y[r], Sat<OUT_T>::lo), Sat<OUT_T>::hi);
+      b[r] = static_cast<uint32_t>(__float_as_int(v + 12582912.0f));
+    }
+    // bytes: result = {b0.byte0, b1.byte0, b2.byte0, b3.byte0}; v_perm selects from {hi operand bytes 4..7, lo 0..3}
+    const uint32_t lo01 = __builtin_amdgcn_perm(b[1], b[0], 0x0c0c0400u);  // [b0.0, b1.0, 0, 0]
+    const uint32_t hi23 = __builtin_amdgcn_perm(b[3], b[2], 0x04000c0cu);  // [0, 0, b2.0, b3.0]
+    return v4i{static_cast<int>(lo01 | hi23), 0, 0, 0};
   }
 }
 

@@ -41,6 +41,11 @@ __device__ __forceinline__ void lds_dma16(const void* gptr, uint32_t lds_addr) {
   // m0 = LDS byte address of lane 0's destination; the instruction adds 16 * lane
   asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(gptr), "s"(lds_addr) : "memory", "m0");
 }
+// same with a wavefront-uniform 64-bit base (SGPR pair) and a 32-bit per-lane byte offset: no vector
+// address arithmetic per load
+__device__ __forceinline__ void lds_dma16(const void* sbase, uint32_t lane_off, uint32_t lds_addr) {
+  asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(lane_off), "s"(sbase), "s"(lds_addr) : "memory", "m0");
+}
 
 template <int N>
 __device__ __forceinline__ void wait_vmcnt() {
@@ -48,9 +53,11 @@ __device__ __forceinline__ void wait_vmcnt() {
   __builtin_amdgcn_s_waitcnt((N & 15) | (7 << 4) | (15 << 8) | ((N >> 4) << 14));
 }
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, int OUT_T, int ACT>
+// FLIP: activations are unsigned (fed as x ^ 0x80).  KALIGNED: K is a multiple of 64, so activation
+// loads never need a per-lane clamp and use a uniform base that advances by 64 bytes per step.
+template <int BM, int BN, int WAVES_M, int WAVES_N, int OUT_T, int ACT, bool FLIP, bool KALIGNED>
 __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void qgemm_tile_kernel(
-    const uint8_t* __restrict__ a, uint32_t a_xor, const uint8_t* __restrict__ bp, int M, int K, int N,
+    const uint8_t* __restrict__ a, const uint8_t* __restrict__ bp, int M, int K, int N,
     int KT, int NT, int num_m, int num_n, EpilogueArgs e, void* __restrict__ out) {
   constexpr int NW = WAVES_M * WAVES_N;
   constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
@@ -93,26 +100,32 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void qgemm_tile_kernel(
   // activation load `ld` covers rows [16*h, 16*h+16) of 32-row tile rt: lane -> (row q, piece p)
   const int q_row = lane >> 2;
   const int q_piece = (lane & 3) ^ ((q_row >> 1) & 3);  // piece = 2*kc + g
-  uint32_t off_a[A_PER_WAVE];  // byte offset of the lane's row in the activation matrix
-  const uint8_t* src_b[B_PER_WAVE];
+  uint32_t off_a[A_PER_WAVE];       // byte offset of the lane's row (+ piece when KALIGNED) in the activation matrix
+  const uint8_t* src_b[B_PER_WAVE];  // wavefront-uniform chunk pointers of step 0
   static_for<A_PER_WAVE>([&](auto c) {
     const int ld = wave * A_PER_WAVE + c;  // 0 .. A_LOADS-1 = (rt, h)
     const int m = min(m_base + ld * 16 + q_row, M - 1);
-    off_a[c] = static_cast<uint32_t>(m) * static_cast<uint32_t>(K);  // M * K < 2^31 checked by the host
+    off_a[c] = static_cast<uint32_t>(m) * static_cast<uint32_t>(K) +  // M * K < 2^31 checked by the host
+               (KALIGNED ? q_piece * 16 : 0);
   });
   static_for<B_PER_WAVE>([&](auto c) {
     const int ld = wave * B_PER_WAVE + c;  // 0 .. B_LOADS-1 = (channel tile, k-chunk)
     const int nt = min((n_base >> 5) + (ld >> 1), NT - 1);
-    src_b[c] = bp + (static_cast<int64_t>(nt) * (2 * KT) + (ld & 1)) * kChunkBytes + lane * 16;
+    src_b[c] = bp + (static_cast<int64_t>(nt) * (2 * KT) + (ld & 1)) * kChunkBytes;
   });
+  const uint32_t lane16 = lane * 16;
   auto issue_load = [&](auto c, int kt, int stage) {
     constexpr int ci = decltype(c)::value;
     const uint32_t stage_addr = lds_base + stage * STAGE_BYTES;
     if constexpr (ci < A_PER_WAVE) {
-      const uint32_t kofs = static_cast<uint32_t>(min(kt * 64 + q_piece * 16, K - 16));
-      lds_dma16(a + off_a[ci] + kofs, stage_addr + (wave * A_PER_WAVE + ci) * kChunkBytes);
+      if constexpr (KALIGNED) {
+        lds_dma16(a + static_cast<int64_t>(kt) * 64, off_a[ci], stage_addr + (wave * A_PER_WAVE + ci) * kChunkBytes);
+      } else {
+        const uint32_t kofs = static_cast<uint32_t>(min(kt * 64 + q_piece * 16, K - 16));
+        lds_dma16(a + off_a[ci] + kofs, stage_addr + (wave * A_PER_WAVE + ci) * kChunkBytes);
+      }
     } else {
-      lds_dma16(src_b[ci - A_PER_WAVE] + static_cast<int64_t>(kt) * (2 * kChunkBytes),
+      lds_dma16(src_b[ci - A_PER_WAVE] + static_cast<int64_t>(kt) * (2 * kChunkBytes), lane16,
                 stage_addr + B_REGION + (wave * B_PER_WAVE + (ci - A_PER_WAVE)) * kChunkBytes);
     }
   };
@@ -125,7 +138,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void qgemm_tile_kernel(
     return *reinterpret_cast<const v4i*>(lds + stage * STAGE_BYTES + (wm * TM + i) * (2 * kChunkBytes) + frag_a_lane[kc]);
   };
   auto flip = [&](v4i v) {  // u8 -> s8 (x - 128) for unsigned activations, identity for signed ones
-    v.x ^= a_xor; v.y ^= a_xor; v.z ^= a_xor; v.w ^= a_xor;
+    if constexpr (FLIP) { v.x ^= 0x80808080; v.y ^= 0x80808080; v.z ^= 0x80808080; v.w ^= 0x80808080; }
     return v;
   };
   auto lds_b = [&](int stage, int kc, int j) {
@@ -139,10 +152,14 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void qgemm_tile_kernel(
   wait_vmcnt<NLD>();
   __syncthreads();
 
-  v4i fa0[2 * TM], fa1[2 * TM], fb[2];
+  // weight fragments rotate through FBN registers sets and are read FBD slices ahead of their use
+  constexpr int FBD = (NSLICE >= 4) ? 2 : 1;
+  constexpr int FBN = (NSLICE >= 4) ? 4 : 2;
+  static_assert(NSLICE % FBN == 0, "the weight fragment rotation must close over a step");
+  v4i fa0[2 * TM], fa1[2 * TM], fb[FBN];
   static_for<2 * TM>([&](auto x) { fa0[x] = lds_a_raw(0, decltype(x)::value / TM, decltype(x)::value % TM); });
   static_for<2 * TM>([&](auto x) { fa0[x] = flip(fa0[x]); });
-  fb[0] = lds_b(0, 0, 0);
+  static_for<FBD>([&](auto d) { fb[d] = lds_b(0, decltype(d)::value / TN, decltype(d)::value % TN); });
 
   // One K step, branch free: past the end of K the loads re-fetch the last step into stages nobody
   // reads and the prefetches read stale stages.
@@ -166,11 +183,12 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void qgemm_tile_kernel(
       static_for<TM>([&](auto i) {
         constexpr int ii = decltype(i)::value;
         constexpr int t = j * TM + ii;
-        acc[t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fb[s & 1], fa_cur[kc * TM + ii], acc[t], 0, 0, 0);
+        acc[t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fb[s % FBN], fa_cur[kc * TM + ii], acc[t], 0, 0, 0);
         // ---- the slot behind this MFMA
         if constexpr (ii == 0) {
-          if constexpr (s + 1 < NSLICE) fb[(s + 1) & 1] = lds_b(st_cur, (s + 1) / TN, (s + 1) % TN);
-          else fb[0] = lds_b(st_nxt, 0, 0);  // NSLICE is even: fb[0] was last used by slice NSLICE-2
+          constexpr int sn = s + FBD;  // the slice whose weight fragment is read now
+          if constexpr (sn < NSLICE) fb[sn % FBN] = lds_b(st_cur, sn / TN, sn % TN);
+          else fb[sn % FBN] = lds_b(st_nxt, (sn - NSLICE) / TN, (sn - NSLICE) % TN);
         }
         if constexpr (ii == TM - 1) {
           static_for<NLD>([&](auto c) {
@@ -272,13 +290,13 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void qgemm_tile_kernel(
   }
 }
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, int OUT_T, int ACT>
-int launch_tile(const uint8_t* a, uint32_t a_xor, const uint8_t* bp, int M, int K, int N,
-                const EpilogueArgs& e, void* out, hipStream_t st) {
+template <int BM, int BN, int WAVES_M, int WAVES_N, int OUT_T, int ACT, bool FLIP, bool KALIGNED>
+int launch_tile(const uint8_t* a, const uint8_t* bp, int M, int K, int N, const EpilogueArgs& e, void* out,
+                hipStream_t st) {
   const int KT = (K + 63) / 64, NT = (N + kChunkRows - 1) / kChunkRows;
   const int num_m = (M + BM - 1) / BM, num_n = (N + BN - 1) / BN;
   constexpr size_t lds_bytes = 4 * (BM / 16 + BN / 16) * kChunkBytes;
-  auto kern = qgemm_tile_kernel<BM, BN, WAVES_M, WAVES_N, OUT_T, ACT>;
+  auto kern = qgemm_tile_kernel<BM, BN, WAVES_M, WAVES_N, OUT_T, ACT, FLIP, KALIGNED>;
   static bool attr_set = false;  // benign race: the call is idempotent
   if (!attr_set) {
     hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -287,28 +305,40 @@ int launch_tile(const uint8_t* a, uint32_t a_xor, const uint8_t* bp, int M, int 
     attr_set = true;
   }
   kern<<<dim3(static_cast<unsigned>(num_m * num_n)), dim3(64 * WAVES_M * WAVES_N), lds_bytes, st>>>(
-      a, a_xor, bp, M, K, N, KT, NT, num_m, num_n, e, out);
+      a, bp, M, K, N, KT, NT, num_m, num_n, e, out);
   return ITEXHIP_OK;
 }
 
-template <int OUT_T, int ACT>
-int dispatch_tile_shape(const uint8_t* a, uint32_t a_xor, const uint8_t* bp, int M, int K, int N,
-                        const EpilogueArgs& e, void* out, hipStream_t st) {
+template <int OUT_T, int ACT, bool FLIP, bool KALIGNED>
+int dispatch_tile_shape(const uint8_t* a, const uint8_t* bp, int M, int K, int N, const EpilogueArgs& e, void* out,
+                        hipStream_t st) {
   // pick the largest tile that still gives every CU work
   const int64_t tiles_256 = static_cast<int64_t>((M + 255) / 256) * ((N + 255) / 256);
   const int64_t tiles_128 = static_cast<int64_t>((M + 127) / 128) * ((N + 127) / 128);
-  if (tiles_256 >= 256) return launch_tile<256, 256, 2, 2, OUT_T, ACT>(a, a_xor, bp, M, K, N, e, out, st);
-  if (tiles_128 >= 256) return launch_tile<128, 128, 2, 2, OUT_T, ACT>(a, a_xor, bp, M, K, N, e, out, st);
-  return launch_tile<64, 64, 2, 2, OUT_T, ACT>(a, a_xor, bp, M, K, N, e, out, st);
+  if (tiles_256 >= 256) return launch_tile<256, 256, 2, 2, OUT_T, ACT, FLIP, KALIGNED>(a, bp, M, K, N, e, out, st);
+  if (tiles_128 >= 256) return launch_tile<128, 128, 2, 2, OUT_T, ACT, FLIP, KALIGNED>(a, bp, M, K, N, e, out, st);
+  return launch_tile<64, 64, 2, 2, OUT_T, ACT, FLIP, KALIGNED>(a, bp, M, K, N, e, out, st);
 }
 
+// The generic eltwise chain and K not a multiple of 64 are rare: they share the conservative
+// instantiation (run-time eltwise chain, per-lane clamped activation loads) to keep the number of
+// kernels down.
 template <int OUT_T>
 int dispatch_tile(const uint8_t* a, uint32_t a_xor, const uint8_t* bp, int M, int K, int N,
                   const EpilogueArgs& e, void* out, hipStream_t st) {
-  if (e.n_eltwise == 0) return dispatch_tile_shape<OUT_T, 0>(a, a_xor, bp, M, K, N, e, out, st);
-  if (e.n_eltwise == 1 && e.elt[0].alg == ITEXHIP_ELT_RELU && e.elt[0].alpha == 0.0f)
-    return dispatch_tile_shape<OUT_T, 1>(a, a_xor, bp, M, K, N, e, out, st);
-  return dispatch_tile_shape<OUT_T, 2>(a, a_xor, bp, M, K, N, e, out, st);
+  const bool flip = a_xor != 0;
+  const bool kal = (K & 63) == 0;
+  const int act = e.n_eltwise == 0 ? 0
+                  : (e.n_eltwise == 1 && e.elt[0].alg == ITEXHIP_ELT_RELU && e.elt[0].alpha == 0.0f) ? 1 : 2;
+#define ITEXHIP_TILE_CASE(A, F, KA) \
+  if (act == A && flip == F && kal == KA) return dispatch_tile_shape<OUT_T, A, F, KA>(a, bp, M, K, N, e, out, st);
+  ITEXHIP_TILE_CASE(0, true, true)
+  ITEXHIP_TILE_CASE(1, true, true)
+  ITEXHIP_TILE_CASE(0, false, true)
+  ITEXHIP_TILE_CASE(1, false, true)
+#undef ITEXHIP_TILE_CASE
+  if (flip) return dispatch_tile_shape<OUT_T, 2, true, false>(a, bp, M, K, N, e, out, st);
+  return dispatch_tile_shape<OUT_T, 2, false, false>(a, bp, M, K, N, e, out, st);
 }
 
 }  // namespace itexhip
