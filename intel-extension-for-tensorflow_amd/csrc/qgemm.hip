@@ -63,77 +63,77 @@ __global__ __launch_bounds__(256) void prepack_b_kernel(const int8_t* __restrict
 }
 
 // ------------------------------------------------------------------------------------------------
-// Small-M kernel (M <= 16, bandwidth bound on the weight).  One workgroup owns one 32-channel strip
-// of the weight, a contiguous stream of KC chunks (1 KiB each, one fully coalesced wavefront load);
-// its WAVES wavefronts take chunks round-robin (all loads of a batch are issued before the first
-// MFMA), multiply them with the matching activation chunk (rows >= M are zero), and the partial
-// 32x32 tiles are added up in LDS with integer atomics (exact, order free).
+// Small-M kernel (M <= 16, bandwidth bound on the weight).  One workgroup owns a 16-channel strip of
+// the weight (half of each 32-channel chunk), so that even N = 4096 gives every CU a workgroup.  Its
+// WAVES wavefronts take pairs of consecutive k-chunks round-robin; one wavefront load fetches the
+// strip's half of a chunk pair (4 runs of 256 contiguous bytes) in the operand layout of the
+// 16x16x64 MFMA: lane l holds channel (l % 16), k-group (l / 16) of the 64 k of the pair.  A batch of
+// UNROLL loads is issued before the first MFMA of the batch.  The partial 16x16 tiles of the
+// wavefronts are added up in LDS with integer atomics (exact, order free).
 // ------------------------------------------------------------------------------------------------
 template <int WAVES, int OUT_T>
 __global__ __launch_bounds__(64 * WAVES) void qgemv_kernel(const uint8_t* __restrict__ a, uint32_t a_xor,
                                                            const uint8_t* __restrict__ bp, int M, int K,
                                                            int N, int KC, EpilogueArgs e,
                                                            void* __restrict__ out) {
-  constexpr int UNROLL = 4;
-  __shared__ int red[16 * 64];
-  const int nt = blockIdx.x;
+  constexpr int UNROLL = 16;  // weight loads in flight per wavefront
+  __shared__ int red[4 * 64];
+  const int strip = blockIdx.x;  // 16 channels
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const int lrow = lane & 31, lgrp = lane >> 5;
-  const uint8_t* strip = bp + static_cast<int64_t>(nt) * KC * kChunkBytes + lane * 16;
+  const int lrow = lane & 15, lgrp = lane >> 4;  // k-group 0..3 of the chunk pair
+  const int KP = KC >> 1;                         // chunk pairs (K is padded to a multiple of 64)
+  // inside chunk (pair * 2 + lgrp / 2): slot (lgrp % 2) * 32 + (strip % 2) * 16 + lrow
+  const uint8_t* wsrc = bp + (static_cast<int64_t>(strip >> 1) * KC + (lgrp >> 1)) * kChunkBytes +
+                        (((lgrp & 1) * 32 + (strip & 1) * 16 + lrow) << 4);
   const uint8_t* arow = a + static_cast<int64_t>(lrow) * K + lgrp * 16;
   const bool row_ok = lrow < M;
 
-  v16i acc;
-#pragma unroll
-  for (int r = 0; r < 16; ++r) acc[r] = 0;
-  auto act_chunk = [&](int kc) {
+  v4i acc = v4i{0, 0, 0, 0};
+  auto act_piece = [&](int kp) {
     v4i v = v4i{0, 0, 0, 0};
-    if (row_ok && kc * kChunkK + lgrp * 16 < K) {
-      v = *reinterpret_cast<const v4i*>(arow + static_cast<int64_t>(kc) * kChunkK);
+    if (row_ok && kp * 64 + lgrp * 16 < K) {
+      v = *reinterpret_cast<const v4i*>(arow + static_cast<int64_t>(kp) * 64);
       v.x ^= a_xor; v.y ^= a_xor; v.z ^= a_xor; v.w ^= a_xor;
     }
     return v;
   };
-  int kc = wave;
-  for (; kc + (UNROLL - 1) * WAVES < KC; kc += UNROLL * WAVES) {
-    v4i w[UNROLL], x[UNROLL];
+  // batches of up to UNROLL chunk pairs: every weight load of a batch is issued first (the guard is
+  // wavefront uniform), activations are read just before use (they come from L2)
+  for (int kp0 = wave; kp0 < KP; kp0 += UNROLL * WAVES) {
+    v4i w[UNROLL];
 #pragma unroll
-    for (int u = 0; u < UNROLL; ++u)
-      w[u] = __builtin_nontemporal_load(
-          reinterpret_cast<const v4i*>(strip + static_cast<int64_t>(kc + u * WAVES) * kChunkBytes));
+    for (int u = 0; u < UNROLL; ++u) {
+      const int kp = kp0 + u * WAVES;
+      w[u] = v4i{0, 0, 0, 0};
+      if (kp < KP)
+        w[u] = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(wsrc + static_cast<int64_t>(kp) * (2 * kChunkBytes)));
+    }
 #pragma unroll
-    for (int u = 0; u < UNROLL; ++u) x[u] = act_chunk(kc + u * WAVES);
-#pragma unroll
-    for (int u = 0; u < UNROLL; ++u) acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(w[u], x[u], acc, 0, 0, 0);
-  }
-  for (; kc < KC; kc += WAVES) {
-    const v4i w = __builtin_nontemporal_load(
-        reinterpret_cast<const v4i*>(strip + static_cast<int64_t>(kc) * kChunkBytes));
-    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(w, act_chunk(kc), acc, 0, 0, 0);
+    for (int u = 0; u < UNROLL; ++u) {
+      const int kp = kp0 + u * WAVES;
+      if (kp < KP) acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(w[u], act_piece(kp), acc, 0, 0, 0);
+    }
   }
 
   // cross-wavefront reduction: wavefront 0 stores, the others add
   if (wave == 0) {
 #pragma unroll
-    for (int r = 0; r < 16; ++r) red[r * 64 + lane] = acc[r];
+    for (int r = 0; r < 4; ++r) red[r * 64 + lane] = acc[r];
   }
   __syncthreads();
   if (wave != 0) {
 #pragma unroll
-    for (int r = 0; r < 16; ++r) atomicAdd(&red[r * 64 + lane], acc[r]);
+    for (int r = 0; r < 4; ++r) atomicAdd(&red[r * 64 + lane], acc[r]);
   }
   __syncthreads();
   if (wave == 0 && row_ok) {
+    // accumulator layout of the 16x16 MFMA: lane l, register r -> m = l % 16, n = (l / 16) * 4 + r
     const bool vec_ok = (N & 3) == 0 && aligned16(e.scales) && aligned16(e.bias) && aligned16(e.colsum) && aligned16(out);
-#pragma unroll
-    for (int g = 0; g < 4; ++g) {
-      const int n = nt * kChunkRows + g * 8 + lgrp * 4;
-      if (n < N) {
-        const v4i part = v4i{red[(4 * g + 0) * 64 + lane], red[(4 * g + 1) * 64 + lane], red[(4 * g + 2) * 64 + lane],
-                             red[(4 * g + 3) * 64 + lane]};
-        const ChannelParams p = load_channel_params(e, n, N, vec_ok);
-        epilogue_store<OUT_T, 2>(part, p, lrow, n, M, N, e, out, vec_ok);
-      }
+    const int n = strip * 16 + lgrp * 4;
+    if (n < N) {
+      const v4i part = v4i{red[lane], red[64 + lane], red[128 + lane], red[192 + lane]};
+      const ChannelParams p = load_channel_params(e, n, N, vec_ok);
+      epilogue_store<OUT_T, 2>(part, p, lrow, n, M, N, e, out, vec_ok);
     }
   }
 }
@@ -206,13 +206,19 @@ EpilogueArgs make_args(int a_type, const int32_t* colsum, const float* scales, c
 template <int OUT_T>
 int dispatch_gemv(const uint8_t* a, uint32_t a_xor, const uint8_t* bp, int M, int K, int N,
                   const EpilogueArgs& e, void* out, hipStream_t st) {
-  const int KC = 2 * ((K + 63) / 64), NT = (N + kChunkRows - 1) / kChunkRows;
-  if (KC >= 256)
-    qgemv_kernel<16, OUT_T><<<NT, 64 * 16, 0, st>>>(a, a_xor, bp, M, K, N, KC, e, out);
-  else if (KC >= 64)
-    qgemv_kernel<8, OUT_T><<<NT, 64 * 8, 0, st>>>(a, a_xor, bp, M, K, N, KC, e, out);
+  const int KC = 2 * ((K + 63) / 64), strips = (N + 15) / 16;
+  const int KP = KC / 2;
+  // as many wavefronts per strip as it takes for each to own at most ~16 chunk pairs (one batch of
+  // loads), within 16 per workgroup; small problems get fewer
+  const int per16 = (KP + 15) / 16;
+  if (per16 > 8)
+    qgemv_kernel<16, OUT_T><<<strips, 64 * 16, 0, st>>>(a, a_xor, bp, M, K, N, KC, e, out);
+  else if (per16 > 2 || KP >= 64)
+    qgemv_kernel<8, OUT_T><<<strips, 64 * 8, 0, st>>>(a, a_xor, bp, M, K, N, KC, e, out);
+  else if (KP >= 4)
+    qgemv_kernel<4, OUT_T><<<strips, 64 * 4, 0, st>>>(a, a_xor, bp, M, K, N, KC, e, out);
   else
-    qgemv_kernel<2, OUT_T><<<NT, 64 * 2, 0, st>>>(a, a_xor, bp, M, K, N, KC, e, out);
+    qgemv_kernel<1, OUT_T><<<strips, 64, 0, st>>>(a, a_xor, bp, M, K, N, KC, e, out);
   return ITEXHIP_OK;
 }
 
