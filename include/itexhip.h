@@ -46,6 +46,18 @@ const char* itexhip_last_error(void);
 const char* itexhip_build_info(void);
 
 /* ------------------------------------------------------------------------------------------
+ * Stream-ordered host-to-device copy of small parameter vectors (per-channel ranges, per-axis
+ * scales), and a stream wait for the synchronous-execution debug mode.  They stand where the
+ * reference uses the device stream's memcpy().wait() (itex/core/kernels/common/host_data_cache.h:
+ * 84-88) and ITEX_SYNC_EXEC (itex/core/utils/op_kernel.h:869-905).  The host buffer must stay valid
+ * until the copy has executed; pageable memory is staged by the runtime before the call returns.
+ * ---------------------------------------------------------------------------------------- */
+int itexhip_memcpy_h2d_async(void* dst_device, const void* src_host, size_t bytes, void* stream);
+/* device-to-host copy ordered after the work already on `stream`; returns when the data has arrived */
+int itexhip_memcpy_d2h(void* dst_host, const void* src_device, size_t bytes, void* stream);
+int itexhip_stream_synchronize(void* stream);
+
+/* ------------------------------------------------------------------------------------------
  * QuantizeV2.  q[i] = sat_T(rne(fl(x[i] * scale) + addend))
  *   SCALED            : addend = 0            (oneDNN reorder, src scale;
  *                                              itex/core/kernels/common/quantize_op.h:256-275,394)

@@ -1,0 +1,158 @@
+// QuantizeV2 / _ITEXQuantizeV2 op kernel: attribute parsing, host-side range math and output range
+// conventions as in the reference (itex/core/kernels/common/quantize_op.h:68-430), the quantization
+// itself on the GPU through itexhip_quantize / itexhip_quantize_axis.
+#include <cmath>
+#include <string>
+#include <vector>
+
+#include "device_vector_cache.h"
+#include "itexhip.h"
+#include "op_kernel.h"
+#include "qparams.h"
+
+namespace itex_amd {
+namespace {
+
+using qparams::Mode;
+
+class QuantizeV2Op : public OpKernel {
+ public:
+  QuantizeV2Op(OpKernelConstruction* ctx, TF_DataType T) : T_(T) {
+    std::string mode_string;
+    ITEX_REQUIRES_OK(ctx, ctx->GetAttr("mode", &mode_string));
+    if (ctx->HasAttr("classic_asymmetric_algorithm")) {
+      ITEX_REQUIRES_OK(ctx, ctx->GetAttr("classic_asymmetric_algorithm", &classic_));
+    }
+    ITEX_REQUIRES(ctx, (mode_string == "MIN_COMBINED" || mode_string == "MIN_FIRST" || mode_string == "SCALED"),
+                  TF_INVALID_ARGUMENT,
+                  "Mode string must be 'MIN_COMBINED', 'MIN_FIRST', or 'SCALED', is '" + mode_string + "'");
+    mode_ = mode_string == "MIN_COMBINED" ? Mode::MIN_COMBINED : mode_string == "MIN_FIRST" ? Mode::MIN_FIRST : Mode::SCALED;
+    ITEX_REQUIRES(ctx, (mode_string == "SCALED" || mode_string == "MIN_FIRST"), TF_INVALID_ARGUMENT,
+                  "_ITEXQuantizeV2 only supports SCALED and MIN_FIRST MODE");
+    std::string round_mode_string;
+    ITEX_REQUIRES_OK(ctx, ctx->GetAttr("round_mode", &round_mode_string));
+    ITEX_REQUIRES(ctx, (round_mode_string == "HALF_AWAY_FROM_ZERO" || round_mode_string == "HALF_TO_EVEN"),
+                  TF_INVALID_ARGUMENT,
+                  "Round mode string must be 'HALF_AWAY_FROM_ZERO' or 'HALF_TO_EVEN', is '" + round_mode_string + "'");
+    if (round_mode_string == "HALF_TO_EVEN") {
+      ITEX_REQUIRES(ctx, mode_string == "SCALED", TF_INVALID_ARGUMENT,
+                    "Round mode 'HALF_TO_EVEN' only supported for mode 'SCALED', but mode is '" + mode_string + "'.");
+    }
+    // narrow_range is read and, as in the reference, has no effect; rounding is to nearest even in
+    // every mode
+    ITEX_REQUIRES_OK(ctx, ctx->GetAttr("narrow_range", &narrow_range_));
+    ITEX_REQUIRES_OK(ctx, ctx->GetAttr("axis", &axis_));
+    ITEX_REQUIRES_OK(ctx, ctx->GetAttr("ensure_minimum_range", &ensure_minimum_range_));
+    if (ctx->HasAttr("dtype")) {
+      TF_DataType dtype = TF_FLOAT;
+      ITEX_REQUIRES_OK(ctx, ctx->GetAttr("dtype", &dtype));
+      ITEX_REQUIRES(ctx, dtype == TF_FLOAT, TF_UNIMPLEMENTED, "_ITEXQuantizeV2 on this device takes float input only");
+    }
+  }
+
+  void Compute(OpKernelContext* ctx) override {
+    Tensor src = ctx->input(0);
+    Tensor in_min = ctx->input(1);
+    Tensor in_max = ctx->input(2);
+    if (!ctx->ok()) return;
+    ITEX_REQUIRES(ctx, src.dtype() == TF_FLOAT, TF_INVALID_ARGUMENT, "QuantizeV2 input must be float");
+
+    const int64_t num_slices = (axis_ > -1) ? in_min.NumElements() : 1;
+    ITEX_REQUIRES(ctx, in_min.NumElements() >= 1 && in_max.NumElements() >= num_slices, TF_INVALID_ARGUMENT,
+                  "min_range and max_range must hold one value per slice");
+    std::vector<float> mn(num_slices), mx(num_slices), scale(num_slices), addend(num_slices, 0.0f);
+    for (int64_t i = 0; i < num_slices; ++i) {
+      ITEX_REQUIRES(ctx, qparams::AdjustRange(in_min.flat<float>()[i], in_max.flat<float>()[i], ensure_minimum_range_,
+                                              &mn[i], &mx[i]),
+                    TF_INVALID_ARGUMENT, "input_max_range must be larger than input_min_range.");
+    }
+    const bool legacy = mode_ == Mode::MIN_FIRST && !classic_;
+    for (int64_t i = 0; i < num_slices; ++i) {
+      if (!legacy) {
+        int32_t zp = 0;
+        qparams::ScaleZeroPoint(T_, mode_, /*dequantize=*/false, &mn[i], &mx[i], &scale[i], &zp);
+        addend[i] = (mode_ == Mode::MIN_FIRST) ? static_cast<float>(zp) : 0.0f;  // destination zero point
+      } else {
+        scale[i] = qparams::LegacyMinFirstScale(T_, mn[i], mx[i]);
+        const float shift = -mn[i];
+        addend[i] = shift * scale[i];  // second source of the scaled binary add
+      }
+    }
+
+    const std::vector<int64_t> shape = src.shape();
+    int64_t outer = 1, slices = 1, inner = 1;
+    if (num_slices > 1) {
+      ITEX_REQUIRES(ctx, axis_ < static_cast<int>(shape.size()) && shape[axis_] == num_slices, TF_INVALID_ARGUMENT,
+                    "min_range has " + std::to_string(num_slices) + " entries but dimension " + std::to_string(axis_) +
+                        " of the input does not");
+      for (int d = 0; d < axis_; ++d) outer *= shape[d];
+      slices = shape[axis_];
+      for (size_t d = axis_ + 1; d < shape.size(); ++d) inner *= shape[d];
+    }
+
+    Tensor dst = ctx->allocate_output(0, T_, shape);
+    const std::vector<int64_t> mm_shape = (num_slices == 1) ? std::vector<int64_t>{} : in_min.shape();
+    Tensor out_min = ctx->forward_input_or_allocate_output(1, 1, mm_shape, TF_FLOAT);
+    Tensor out_max = ctx->forward_input_or_allocate_output(2, 2, mm_shape, TF_FLOAT);
+    if (!ctx->ok()) return;
+
+    int st;
+    if (num_slices == 1) {
+      st = itexhip_quantize(src.flat<float>(), dst.data(), src.NumElements(), T_, scale[0], addend[0], ctx->stream());
+    } else {
+      std::vector<float> both(scale);
+      both.insert(both.end(), addend.begin(), addend.end());
+      float* dev = params_.Get(ctx, both.data(), both.size(), TF_FLOAT);
+      if (dev == nullptr) return;
+      st = itexhip_quantize_axis(src.flat<float>(), dst.data(), outer, slices, inner, T_, dev, dev + num_slices,
+                                 ctx->stream());
+    }
+    ITEX_REQUIRES(ctx, st == ITEXHIP_OK, st == ITEXHIP_INVALID_ARGUMENT ? TF_INVALID_ARGUMENT : TF_ABORTED,
+                  std::string("Operation received an exception: ") + itexhip_last_error());
+
+    // output ranges; the outputs may alias the inputs, which were consumed above
+    for (int64_t i = 0; i < num_slices; ++i) {
+      if (T_ == TF_QUINT8 && mode_ == Mode::SCALED) {
+        out_min.flat<float>()[i] = 0.0f;
+        out_max.flat<float>()[i] = mx[i];
+      } else {
+        out_min.flat<float>()[i] = mn[i];
+        out_max.flat<float>()[i] = mx[i];
+      }
+    }
+  }
+
+ private:
+  TF_DataType T_;
+  Mode mode_ = Mode::SCALED;
+  bool classic_ = false;
+  bool narrow_range_ = false;
+  int32_t axis_ = -1;
+  float ensure_minimum_range_ = 0.01f;
+  DeviceVectorCache<float> params_;
+};
+
+struct QuantizeQint8 : QuantizeV2Op { explicit QuantizeQint8(OpKernelConstruction* c) : QuantizeV2Op(c, TF_QINT8) {} };
+struct QuantizeQuint8 : QuantizeV2Op { explicit QuantizeQuint8(OpKernelConstruction* c) : QuantizeV2Op(c, TF_QUINT8) {} };
+
+}  // namespace
+
+// names and host-memory arguments as registered by the reference for a device
+// (itex/core/kernels/gpu/quantize_op.cc:24-51)
+void AddQuantizeKernels() {
+  for (const char* op : {"QuantizeV2", "_ITEXQuantizeV2"}) {
+    const bool itex = op[0] == '_';
+    KernelDefBuilder s8(op, "QuantizeV2Op");
+    s8.TypeConstraint("T", TF_QINT8);
+    if (itex) s8.TypeConstraint("dtype", TF_FLOAT);
+    s8.HostMemory("min_range").HostMemory("max_range").HostMemory("output_min").HostMemory("output_max");
+    s8.Register<QuantizeQint8>();
+    KernelDefBuilder u8(op, "QuantizeV2Op");
+    u8.TypeConstraint("T", TF_QUINT8);
+    if (itex) u8.TypeConstraint("dtype", TF_FLOAT);
+    u8.HostMemory("min_range").HostMemory("max_range").HostMemory("output_min").HostMemory("output_max");
+    u8.Register<QuantizeQuint8>();
+  }
+}
+
+}  // namespace itex_amd

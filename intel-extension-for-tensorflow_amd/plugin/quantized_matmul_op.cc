@@ -1,0 +1,307 @@
+// Quantized MatMul op kernels: _QuantizedMatMul / _ITEXQuantizedMatMul (V2),
+// _QuantizedFusedMatMul{,AndRequantize,AndDequantize} (V1) and the legacy
+// QuantizedMatMulWithBias{,AndRelu,AndRequantize,AndReluAndRequantize,AndDequantize}.
+//
+// Mirrors LegacyQuantizedMatMulOpBase and its three subclasses
+// (itex/core/kernels/common/quantized_matmul_common.h:48-736, 1412-1909): attribute parsing, input
+// index conventions, one Compute at a time per node, cached weight preparation, host-memory min/max
+// outputs.  Where the reference builds a oneDNN inner-product primitive, reorders the weight and
+// prepares scales / bias on the host, this kernel prepacks the weight once on the device
+// (itexhip_qgemm_prepack_b, which also yields the column sums the MIN_FIRST compensation needs),
+// lets a small device kernel derive the per-channel scale and bias vectors from the current ranges
+// (itexhip_qmatmul_prepare: no host wait when the activation range changes) and launches
+// itexhip_qgemm.
+#include <algorithm>
+#include <cmath>
+#include <cstring>
+#include <mutex>
+#include <string>
+#include <vector>
+
+#include "device_vector_cache.h"
+#include "itexhip.h"
+#include "op_kernel.h"
+#include "qparams.h"
+
+namespace itex_amd {
+namespace {
+
+enum class Api { V2 = ITEXHIP_API_V2, V1 = ITEXHIP_API_V1, LEGACY = ITEXHIP_API_LEGACY };
+
+struct Variant {
+  Api api;
+  TF_DataType t_in, t_out;
+  bool legacy_relu;  // QuantizedMatMulReluOp
+};
+
+int ActivationFromName(const std::string& n) {
+  if (n == "Relu") return ITEXHIP_ACT_RELU;
+  if (n == "Relu6") return ITEXHIP_ACT_RELU6;
+  if (n == "LeakyRelu") return ITEXHIP_ACT_LEAKYRELU;
+  return -1;
+}
+
+class QuantizedMatMulOp : public OpKernel {
+ public:
+  QuantizedMatMulOp(OpKernelConstruction* ctx, const Variant& v) : v_(v) {
+    ITEX_REQUIRES_OK(ctx, ctx->GetAttr("transpose_a", &transpose_a_));
+    ITEX_REQUIRES_OK(ctx, ctx->GetAttr("transpose_b", &transpose_b_));
+    std::string mode_string;
+    ITEX_REQUIRES_OK(ctx, ctx->GetAttr("input_quant_mode", &mode_string));
+    ITEX_REQUIRES(ctx, mode_string == "MIN_FIRST" || mode_string == "SCALED", TF_INVALID_ARGUMENT,
+                  "Quantization mode must be either MIN_FIRST or SCALED, but received " + mode_string);
+    p_.input_mode = mode_string == "MIN_FIRST" ? ITEXHIP_MIN_FIRST : ITEXHIP_SCALED;
+    p_.api = static_cast<int>(v.api);
+    p_.t_in = v.t_in;
+    p_.t_out = v.t_out;
+    p_.leakyrelu_alpha = 0.2f;
+
+    std::vector<std::string> fused_ops;
+    if (v.api == Api::LEGACY) {  // :1418-1465, :1516-1523
+      if (ctx->HasAttr("is_weight_const")) ITEX_REQUIRES_OK(ctx, ctx->GetAttr("is_weight_const", &is_weight_const_));
+      is_bias_const_ = true;
+      if (v.legacy_relu) p_.activation = ITEXHIP_ACT_RELU;
+      min_a_idx_ = 3;
+      min_out_idx_ = 7;
+    } else if (v.api == Api::V1) {  // :1545-1603
+      ITEX_REQUIRES_OK(ctx, ctx->GetAttr("is_filter_const", &is_weight_const_));
+      ITEX_REQUIRES_OK(ctx, ctx->GetAttr("is_bias_const", &is_bias_const_));
+      ITEX_REQUIRES_OK(ctx, ctx->GetAttr("fused_ops", &fused_ops));
+      ITEX_REQUIRES(ctx, fused_ops.size() <= 2, TF_INVALID_ARGUMENT, "_QuantizedFusedMatMul supports maximum 2 post ops");
+      ITEX_REQUIRES(ctx, fused_ops.empty() || fused_ops[0] == "BiasAdd", TF_INVALID_ARGUMENT,
+                    "_QuantizedFusedMatMul first post op must be BiasAdd");
+      p_.n_fused_ops = static_cast<int>(fused_ops.size());
+      for (size_t i = 1; i < fused_ops.size(); ++i) {
+        ITEX_REQUIRES(ctx, fused_ops[i] != "Add", TF_UNIMPLEMENTED, "the Add fusion is not implemented on this device");
+        const int act = ActivationFromName(fused_ops[i]);
+        ITEX_REQUIRES(ctx, act >= 0, TF_INVALID_ARGUMENT, "Found unsupported fusion in _QuantizedFusedMatMul.");
+        p_.activation = act;
+      }
+      min_a_idx_ = 3;
+      min_out_idx_ = 7;
+    } else {  // V2 :1725-1795
+      std::string out_mode;
+      ITEX_REQUIRES_OK(ctx, ctx->GetAttr("output_quant_mode", &out_mode));
+      p_.out_min_first = out_mode == "MIN_FIRST";
+      ITEX_REQUIRES_OK(ctx, ctx->GetAttr("is_weight_const", &is_weight_const_));
+      ITEX_REQUIRES_OK(ctx, ctx->GetAttr("is_bias_const", &is_bias_const_));
+      ITEX_REQUIRES_OK(ctx, ctx->GetAttr("fused_ops", &fused_ops));
+      for (const std::string& f : fused_ops) {
+        if (f == "BiasAdd" || f == "Quantized") continue;
+        if (f == "Requantize") { p_.has_requantize = 1; continue; }
+        if (f == "Dequantize") { p_.has_dequantize = 1; continue; }
+        ITEX_REQUIRES(ctx, f != "Add", TF_UNIMPLEMENTED, "Quantized addend tensor is not implemented yet.");
+        const int act = ActivationFromName(f);
+        ITEX_REQUIRES(ctx, act >= 0, TF_INVALID_ARGUMENT, "Found unsupported fusion in _QuantizedMatMul.");
+        p_.activation = act;
+      }
+      p_.n_fused_ops = static_cast<int>(fused_ops.size());
+      min_a_idx_ = 3;
+      min_out_idx_ = 7;  // fixed, as in the reference (:1784-1785)
+    }
+    if (p_.activation == ITEXHIP_ACT_LEAKYRELU) ITEX_REQUIRES_OK(ctx, ctx->GetAttr("leakyrelu_alpha", &p_.leakyrelu_alpha));
+    if (ctx->HasAttr("Tbias")) {
+      TF_DataType tb = TF_FLOAT;
+      ITEX_REQUIRES_OK(ctx, ctx->GetAttr("Tbias", &tb));
+      ITEX_REQUIRES(ctx, tb == TF_FLOAT, TF_UNIMPLEMENTED, "only a float bias is implemented on this device");
+    }
+  }
+
+  void Compute(OpKernelContext* ctx) override {
+    std::lock_guard<std::mutex> lock(mu_);  // one Compute at a time per node (:62)
+    Tensor a = ctx->input(0);
+    Tensor w = ctx->input(1);
+    Tensor bias = ctx->input(2);
+    Tensor min_a_t = ctx->input(min_a_idx_), max_a_t = ctx->input(min_a_idx_ + 1);
+    Tensor min_b_t = ctx->input(min_a_idx_ + 2), max_b_t = ctx->input(min_a_idx_ + 3);
+    if (!ctx->ok()) return;
+    ITEX_REQUIRES(ctx, !transpose_a_, TF_UNIMPLEMENTED, "transpose_a is not supported by the quantized MatMul");
+    ITEX_REQUIRES(ctx, a.dims() == 2 && w.dims() == 2, TF_INVALID_ARGUMENT, "quantized MatMul operands must be matrices");
+    ITEX_REQUIRES(ctx, a.dtype() == v_.t_in && w.dtype() == TF_QINT8 && bias.dtype() == TF_FLOAT, TF_INVALID_ARGUMENT,
+                  "quantized MatMul operand types do not match the kernel");
+    const int64_t M = a.dim_size(0), K = a.dim_size(1);
+    const int64_t N = transpose_b_ ? w.dim_size(0) : w.dim_size(1);
+    ITEX_REQUIRES(ctx, (transpose_b_ ? w.dim_size(1) : w.dim_size(0)) == K, TF_INVALID_ARGUMENT,
+                  "Matrix size-incompatible: In[0] inner dimension " + std::to_string(K) + " vs In[1]");
+    ITEX_REQUIRES(ctx, bias.NumElements() == N, TF_INVALID_ARGUMENT, "bias must have one entry per output channel");
+    // the reference's zero-point compensation indexes the weight as [K, N] whatever transpose_b says
+    // (:569-573); that combination is refused instead of reproduced
+    ITEX_REQUIRES(ctx, !(transpose_b_ && p_.input_mode == ITEXHIP_MIN_FIRST), TF_UNIMPLEMENTED,
+                  "transpose_b with MIN_FIRST input quantization is not supported");
+    const int64_t nb = min_b_t.NumElements();
+    ITEX_REQUIRES(ctx, max_b_t.NumElements() == nb && (nb == 1 || nb == N), TF_INVALID_ARGUMENT,
+                  "min_b / max_b must be scalars or hold one entry per output channel");
+    ITEX_REQUIRES(ctx, v_.api != Api::LEGACY || nb == 1, TF_INVALID_ARGUMENT,
+                  "QuantizedMatMulWithBias takes per-tensor weight ranges");
+
+    itexhip_matmul_params p = p_;
+    p.min_a = min_a_t.flat<float>()[0];
+    p.max_a = max_a_t.flat<float>()[0];
+    const bool out_q8 = v_.t_out == TF_QINT8 || v_.t_out == TF_QUINT8;
+    const bool needs_freezed = out_q8 || (v_.api == Api::LEGACY && v_.t_out == TF_FLOAT);
+    if (needs_freezed) {
+      ITEX_REQUIRES(ctx, ctx->num_inputs() > min_out_idx_ + 1, TF_INVALID_ARGUMENT,
+                    "min_freezed_output / max_freezed_output inputs are missing");
+      Tensor mo = ctx->input(min_out_idx_), xo = ctx->input(min_out_idx_ + 1);
+      if (!ctx->ok()) return;
+      p.min_out = mo.flat<float>()[0];
+      p.max_out = xo.flat<float>()[0];
+    }
+    itexhip_epilogue ep;
+    int st = itexhip_qmatmul_epilogue_desc(&p, nb, &ep);
+    ITEX_REQUIRES(ctx, st == ITEXHIP_OK, static_cast<TF_Code>(st), itexhip_last_error());
+
+    void* stream = ctx->stream();
+    // ---- weight: prepacked once when constant, else every call (:238-275)
+    const bool repack = !packed_.valid() || !is_weight_const_ || packed_src_ != w.data() || packed_k_ != K || packed_n_ != N;
+    if (repack) {
+      const int64_t bytes = itexhip_qgemm_packed_bytes(K, N);
+      packed_ = ctx->allocate_temp(TF_QINT8, {std::max<int64_t>(bytes, 16)});
+      colsum_ = ctx->allocate_temp(TF_INT32, {std::max<int64_t>(N, 1)});
+      if (!ctx->ok()) return;
+      st = itexhip_qgemm_prepack_b(w.flat<int8_t>(), transpose_b_ ? 1 : 0, K, N, packed_.flat<int8_t>(),
+                                   colsum_.flat<int32_t>(), stream);
+      ITEX_REQUIRES(ctx, st == ITEXHIP_OK, TF_ABORTED, std::string("Operation received an exception: ") + itexhip_last_error());
+      packed_src_ = w.data();
+      packed_k_ = K;
+      packed_n_ = N;
+      prepared_ = false;
+    }
+    // ---- per-channel scale and bias vectors on the device
+    float* min_b_dev = min_b_cache_.Get(ctx, min_b_t.flat<float>(), nb, TF_FLOAT);
+    float* max_b_dev = max_b_cache_.Get(ctx, max_b_t.flat<float>(), nb, TF_FLOAT);
+    if (min_b_dev == nullptr || max_b_dev == nullptr) return;
+    if (!scales_.valid() || scales_.NumElements() < std::max<int64_t>(N, 1)) {
+      scales_ = ctx->allocate_temp(TF_FLOAT, {std::max<int64_t>(N, 1)});
+      sbias_ = ctx->allocate_temp(TF_FLOAT, {std::max<int64_t>(N, 1)});
+      if (!ctx->ok()) return;
+      prepared_ = false;
+    }
+    // the prepared vectors are reused while nothing they depend on changed (cf. IsCachedBiasValid
+    // :458-464, which tolerates 1e-5; here the comparison is exact)
+    const bool same = prepared_ && is_bias_const_ && is_weight_const_ && bias.data() == prepared_bias_ &&
+                      std::memcmp(&p, &prepared_p_, sizeof(p)) == 0 && !min_b_cache_.changed() && !max_b_cache_.changed();
+    if (!same) {
+      st = itexhip_qmatmul_prepare(&p, min_b_dev, max_b_dev, nb, bias.flat<float>(), colsum_.flat<int32_t>(), N,
+                                   scales_.flat<float>(), sbias_.flat<float>(), stream);
+      ITEX_REQUIRES(ctx, st == ITEXHIP_OK, st == ITEXHIP_INVALID_ARGUMENT ? TF_INVALID_ARGUMENT : TF_ABORTED,
+                    std::string("Operation received an exception: ") + itexhip_last_error());
+      prepared_ = true;
+      prepared_p_ = p;
+      prepared_bias_ = bias.data();
+    }
+
+    // ---- product
+    Tensor out = ctx->allocate_output(0, v_.t_out, {M, N});
+    if (!ctx->ok()) return;
+    if (K % 16 == 0 && K > 0) {
+      st = itexhip_qgemm(a.data(), v_.t_in, packed_.flat<int8_t>(), colsum_.flat<int32_t>(), M, K, N,
+                         scales_.flat<float>(), sbias_.flat<float>(), &ep, v_.t_out, out.data(), stream);
+    } else {
+      st = itexhip_qgemm_naive(a.data(), v_.t_in, w.flat<int8_t>(), transpose_b_ ? 1 : 0, M, K, N, scales_.flat<float>(),
+                               sbias_.flat<float>(), &ep, v_.t_out, out.data(), stream);
+    }
+    ITEX_REQUIRES(ctx, st == ITEXHIP_OK, st == ITEXHIP_INVALID_ARGUMENT ? TF_INVALID_ARGUMENT : TF_ABORTED,
+                  std::string("Operation received an exception: ") + itexhip_last_error());
+
+    // ---- output ranges in host memory (AllocateNativeOutputMinMax,
+    // itex/core/kernels/onednn/block/quantized_ops.h:142-203)
+    if (out_q8) {
+      Tensor omin = ctx->allocate_output(1, TF_FLOAT, {});
+      Tensor omax = ctx->allocate_output(2, TF_FLOAT, {});
+      if (!ctx->ok()) return;
+      omin.flat<float>()[0] = p.min_out;
+      omax.flat<float>()[0] = p.max_out;
+    } else if (v_.t_out == TF_QINT32) {
+      const bool scalar = min_b_t.dims() == 0;
+      const std::vector<int64_t> shp = scalar ? std::vector<int64_t>{} : std::vector<int64_t>{nb};
+      Tensor omin = ctx->allocate_output(1, TF_FLOAT, shp);
+      Tensor omax = ctx->allocate_output(2, TF_FLOAT, shp);
+      if (!ctx->ok()) return;
+      for (int64_t i = 0; i < (scalar ? 1 : nb); ++i)
+        qparams::RangeForMultiplication(v_.t_in, TF_QINT8, p.min_a, p.max_a, min_b_t.flat<float>()[i],
+                                        max_b_t.flat<float>()[i], &omin.flat<float>()[i], &omax.flat<float>()[i]);
+    }
+  }
+
+ private:
+  Variant v_;
+  itexhip_matmul_params p_{};
+  bool transpose_a_ = false, transpose_b_ = false;
+  bool is_weight_const_ = true, is_bias_const_ = true;
+  int min_a_idx_ = 3, min_out_idx_ = 7;
+  std::mutex mu_;
+  // persistent device state of the node
+  Tensor packed_, colsum_, scales_, sbias_;
+  const void* packed_src_ = nullptr;
+  int64_t packed_k_ = -1, packed_n_ = -1;
+  DeviceVectorCache<float> min_b_cache_, max_b_cache_;
+  bool prepared_ = false;
+  itexhip_matmul_params prepared_p_{};
+  const void* prepared_bias_ = nullptr;
+};
+
+template <int API, int TIN, int TOUT, bool RELU>
+struct MatMulKernel : QuantizedMatMulOp {
+  explicit MatMulKernel(OpKernelConstruction* c)
+      : QuantizedMatMulOp(c, Variant{static_cast<Api>(API), static_cast<TF_DataType>(TIN), static_cast<TF_DataType>(TOUT), RELU}) {}
+};
+
+template <int API, int TIN, int TOUT, bool RELU>
+void Reg(const char* op, const char* out_attr, const char* bias_attr, std::initializer_list<const char*> host_args) {
+  KernelDefBuilder b(op, "QuantizedMatMulOp");
+  b.TypeConstraint("T1", static_cast<TF_DataType>(TIN)).TypeConstraint("T2", TF_QINT8);
+  if (bias_attr) b.TypeConstraint(bias_attr, TF_FLOAT);
+  b.TypeConstraint(out_attr, static_cast<TF_DataType>(TOUT));
+  for (const char* h : host_args) b.HostMemory(h);
+  b.Register<MatMulKernel<API, TIN, TOUT, RELU>>();
+}
+
+template <int API, int TOUT>
+void RegBothInputs(const char* op, const char* out_attr, const char* bias_attr, std::initializer_list<const char*> host_args) {
+  Reg<API, TF_QUINT8, TOUT, false>(op, out_attr, bias_attr, host_args);
+  Reg<API, TF_QINT8, TOUT, false>(op, out_attr, bias_attr, host_args);
+}
+
+}  // namespace
+
+// Names, type constraints and host-memory arguments as registered by the reference for a device
+// (itex/core/kernels/gpu/quantized_matmul.cc:35-201); the _ITEX names are the CPU-side renames
+// (itex/core/kernels/cpu/quantized_matmul.cc:97-163), registered as well.
+void AddQuantizedMatMulKernels() {
+  constexpr int V2 = ITEXHIP_API_V2, V1 = ITEXHIP_API_V1, LG = ITEXHIP_API_LEGACY;
+  // legacy ops: quint8 x qint8
+  Reg<LG, TF_QUINT8, TF_QINT32, true>("QuantizedMatMulWithBiasAndRelu", "Toutput", nullptr,
+                                      {"min_a", "max_a", "min_b", "max_b", "min_out", "max_out"});
+  Reg<LG, TF_QUINT8, TF_QINT32, false>("QuantizedMatMulWithBias", "Toutput", "Tbias",
+                                       {"min_a", "max_a", "min_b", "max_b", "min_out", "max_out"});
+  Reg<LG, TF_QUINT8, TF_QUINT8, true>("QuantizedMatMulWithBiasAndReluAndRequantize", "Toutput", "Tbias",
+                                      {"min_a", "max_a", "min_b", "max_b", "min_freezed_output", "max_freezed_output",
+                                       "min_out", "max_out"});
+  Reg<LG, TF_QUINT8, TF_QUINT8, false>("QuantizedMatMulWithBiasAndRequantize", "Toutput", "Tbias",
+                                       {"min_a", "max_a", "min_b", "max_b", "min_freezed_output", "max_freezed_output",
+                                        "min_out", "max_out"});
+  for (const char* op : {"QuantizedMatMulWithBiasAndDequantize", "_ITEXQuantizedMatMulWithBiasAndDequantize"})
+    Reg<LG, TF_QUINT8, TF_FLOAT, false>(op, "Toutput", "Tbias",
+                                        {"min_a", "max_a", "min_b", "max_b", "min_freezed_output", "max_freezed_output"});
+  // V1
+  for (const char* op : {"_QuantizedFusedMatMul", "_ITEXQuantizedFusedMatMul"})
+    RegBothInputs<V1, TF_QINT32>(op, "Toutput", "Targs", {"min_a", "max_a", "min_b", "max_b", "min_product", "max_product"});
+  for (const char* op : {"_QuantizedFusedMatMulAndDequantize", "_ITEXQuantizedFusedMatMulAndDequantize"})
+    RegBothInputs<V1, TF_FLOAT>(op, "Toutput", "Targs", {"min_a", "max_a", "min_b", "max_b"});
+  for (const char* op : {"_QuantizedFusedMatMulAndRequantize", "_ITEXQuantizedFusedMatMulAndRequantize"}) {
+    RegBothInputs<V1, TF_QUINT8>(op, "Toutput", "Targs", {"min_a", "max_a", "min_b", "max_b", "min_freezed_output",
+                                                          "max_freezed_output", "min_product", "max_product"});
+    RegBothInputs<V1, TF_QINT8>(op, "Toutput", "Targs", {"min_a", "max_a", "min_b", "max_b", "min_freezed_output",
+                                                         "max_freezed_output", "min_product", "max_product"});
+  }
+  // V2
+  for (const char* op : {"_QuantizedMatMul", "_ITEXQuantizedMatMul"}) {
+    RegBothInputs<V2, TF_QINT32>(op, "Tout", "Tbias", {"host_inputs", "host_outputs"});
+    RegBothInputs<V2, TF_FLOAT>(op, "Tout", "Tbias", {"host_inputs", "host_outputs"});
+    RegBothInputs<V2, TF_QINT8>(op, "Tout", "Tbias", {"host_inputs", "host_outputs"});
+    RegBothInputs<V2, TF_QUINT8>(op, "Tout", "Tbias", {"host_inputs", "host_outputs"});
+  }
+}
+
+}  // namespace itex_amd

@@ -1,0 +1,590 @@
+// A stand-in for the TensorFlow runtime, for tests: implements the C API subset declared in
+// include/tf_c_api_subset.h over plain memory, records kernel and op registrations, and drives
+// create / compute / delete of a kernel the way TensorFlow's C kernel wrapper does.  Test
+// infrastructure only; it allocates device memory through a callback supplied by the test (PyTorch)
+// or, without one, from the host heap.
+#include <dlfcn.h>
+
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <map>
+#include <memory>
+#include <sstream>
+#include <string>
+#include <vector>
+
+#include "tf_c_api_subset.h"
+
+// ------------------------------------------------------------------------------------------------
+// object definitions
+// ------------------------------------------------------------------------------------------------
+struct TF_Status {
+  TF_Code code = TF_OK;
+  std::string msg;
+};
+
+namespace {
+typedef void* (*AllocFn)(size_t bytes, int on_host);
+typedef void (*FreeFn)(void* p, int on_host);
+AllocFn g_alloc = nullptr;
+FreeFn g_free = nullptr;
+
+struct Buffer {
+  void* data = nullptr;
+  size_t bytes = 0;
+  bool owned = false;
+  bool on_host = true;
+  int refs = 0;
+  ~Buffer() {
+    if (owned && data) {
+      if (!on_host && g_free) g_free(data, 0);
+      else std::free(data);
+    }
+  }
+};
+size_t DtypeSize(TF_DataType t) {
+  switch (t) {
+    case TF_FLOAT: case TF_INT32: case TF_QINT32: return 4;
+    case TF_QINT8: case TF_QUINT8: case TF_INT8: case TF_UINT8: case TF_BOOL: return 1;
+    case TF_BFLOAT16: case TF_HALF: case TF_INT16: return 2;
+    case TF_DOUBLE: case TF_INT64: return 8;
+    default: return 1;
+  }
+}
+}  // namespace
+
+struct TF_Tensor {
+  TF_DataType dtype;
+  std::vector<int64_t> dims;
+  std::shared_ptr<Buffer> buf;
+};
+
+namespace {
+TF_Tensor* NewTensor(TF_DataType dtype, const int64_t* dims, int ndims, bool on_host) {
+  auto* t = new TF_Tensor;
+  t->dtype = dtype;
+  t->dims.assign(dims, dims + ndims);
+  int64_t n = 1;
+  for (int64_t d : t->dims) n *= d;
+  t->buf = std::make_shared<Buffer>();
+  t->buf->bytes = static_cast<size_t>(n) * DtypeSize(dtype);
+  t->buf->owned = true;
+  t->buf->on_host = on_host || g_alloc == nullptr;
+  const size_t bytes = t->buf->bytes ? t->buf->bytes : 1;
+  t->buf->data = t->buf->on_host ? std::calloc(1, bytes + 64) : g_alloc(bytes, 0);
+  return t;
+}
+
+struct AttrValue {
+  enum Kind { STRING, INT, FLOAT, BOOL, TYPE, STRING_LIST, TYPE_LIST } kind;
+  std::string s;
+  int64_t i = 0;
+  float f = 0;
+  bool b = false;
+  TF_DataType t = TF_FLOAT;
+  std::vector<std::string> sl;
+  std::vector<TF_DataType> tl;
+};
+}  // namespace
+
+struct TF_KernelBuilder {
+  std::string op, device, label;
+  void* (*create)(TF_OpKernelConstruction*);
+  void (*compute)(void*, TF_OpKernelContext*);
+  void (*del)(void*);
+  std::vector<std::pair<std::string, TF_DataType>> constraints;
+  std::vector<std::string> host_memory;
+  int priority = 0;
+};
+
+struct TF_OpKernelConstruction {
+  std::string name;
+  std::map<std::string, AttrValue> attrs;
+  TF_Status status;
+};
+
+struct TF_OpKernelContext {
+  struct In { TF_Tensor* t; bool allow_forward; };
+  std::vector<In> inputs;
+  std::vector<TF_Tensor*> outputs;
+  std::vector<int> forwarded_from;
+  std::vector<TF_DataType> out_dtypes;
+  std::vector<char> out_on_host;
+  SP_Stream_st stream{nullptr};
+  TF_Status status;
+  int temp_allocs = 0;
+};
+
+struct TF_OpDefinitionBuilder {
+  std::string name;
+  std::vector<std::string> inputs, outputs, attrs;
+  bool has_shape_fn = false;
+};
+struct TF_ShapeInferenceContext {
+  bool unknown = false;
+};
+
+namespace {
+std::vector<std::unique_ptr<TF_KernelBuilder>> g_kernels;
+std::vector<std::unique_ptr<TF_OpDefinitionBuilder>> g_ops;
+std::vector<std::string> g_stock_ops;
+std::string g_json;
+int g_delete_calls = 0;
+
+struct Node {
+  std::string op, device;
+  TF_OpKernelConstruction construction;
+  TF_OpKernelContext context;
+  TF_KernelBuilder* kernel = nullptr;
+  void* object = nullptr;
+};
+}  // namespace
+
+// ------------------------------------------------------------------------------------------------
+// the C API
+// ------------------------------------------------------------------------------------------------
+extern "C" {
+
+TF_Status* TF_NewStatus(void) { return new TF_Status; }
+void TF_DeleteStatus(TF_Status* s) { delete s; }
+void TF_SetStatus(TF_Status* s, TF_Code code, const char* msg) { s->code = code; s->msg = msg ? msg : ""; }
+TF_Code TF_GetCode(const TF_Status* s) { return s->code; }
+const char* TF_Message(const TF_Status* s) { return s->msg.c_str(); }
+
+void* TF_TensorData(const TF_Tensor* t) { return t->buf->data; }
+int TF_NumDims(const TF_Tensor* t) { return static_cast<int>(t->dims.size()); }
+int64_t TF_Dim(const TF_Tensor* t, int i) { return t->dims[i]; }
+TF_DataType TF_TensorType(const TF_Tensor* t) { return t->dtype; }
+size_t TF_TensorByteSize(const TF_Tensor* t) { return t->buf->bytes; }
+int64_t TF_TensorElementCount(const TF_Tensor* t) {
+  int64_t n = 1;
+  for (int64_t d : t->dims) n *= d;
+  return n;
+}
+void TF_DeleteTensor(TF_Tensor* t) { delete t; }
+
+void TF_DeleteBuffer(TF_Buffer* b) {
+  if (b == nullptr) return;
+  if (b->data_deallocator) b->data_deallocator(const_cast<void*>(b->data), b->length);
+  delete b;
+}
+static void PutVarint(std::string* s, uint64_t v) {
+  while (v >= 0x80) { s->push_back(static_cast<char>(v | 0x80)); v >>= 7; }
+  s->push_back(static_cast<char>(v));
+}
+TF_Buffer* TF_GetAllOpList(void) {
+  std::string list;
+  auto add = [&](const std::string& name) {
+    std::string op;
+    op.push_back(0x0a);  // OpDef.name
+    PutVarint(&op, name.size());
+    op += name;
+    op.push_back(0x1a);  // OpDef.output_arg (an unrelated field the reader must skip)
+    PutVarint(&op, 2);
+    op += "\x0a\x00";
+    list.push_back(0x0a);  // OpList.op
+    PutVarint(&list, op.size());
+    list += op;
+  };
+  for (const auto& n : g_stock_ops) add(n);
+  for (const auto& o : g_ops) add(o->name);
+  auto* b = new TF_Buffer;
+  char* data = static_cast<char*>(std::malloc(list.size() + 1));
+  std::memcpy(data, list.data(), list.size());
+  b->data = data;
+  b->length = list.size();
+  b->data_deallocator = [](void* d, size_t) { std::free(d); };
+  return b;
+}
+
+TF_KernelBuilder* TF_NewKernelBuilder(const char* op_name, const char* device_name,
+                                      void* (*create_func)(TF_OpKernelConstruction*),
+                                      void (*compute_func)(void*, TF_OpKernelContext*), void (*delete_func)(void*)) {
+  auto* b = new TF_KernelBuilder;
+  b->op = op_name;
+  b->device = device_name;
+  b->create = create_func;
+  b->compute = compute_func;
+  b->del = delete_func;
+  return b;
+}
+void TF_KernelBuilder_TypeConstraint(TF_KernelBuilder* b, const char* attr_name, const TF_DataType type, TF_Status* status) {
+  b->constraints.emplace_back(attr_name, type);
+  TF_SetStatus(status, TF_OK, "");
+}
+void TF_KernelBuilder_HostMemory(TF_KernelBuilder* b, const char* arg_name) { b->host_memory.emplace_back(arg_name); }
+void TF_KernelBuilder_Priority(TF_KernelBuilder* b, int32_t p) { b->priority = p; }
+void TF_RegisterKernelBuilder(const char* kernel_name, TF_KernelBuilder* builder, TF_Status* status) {
+  builder->label = kernel_name;
+  // a second registration with the same op, device and constraints is an error in TensorFlow
+  for (const auto& k : g_kernels) {
+    if (k->op == builder->op && k->device == builder->device && k->constraints == builder->constraints) {
+      TF_SetStatus(status, TF_ALREADY_EXISTS, ("duplicate kernel registration for " + builder->op).c_str());
+      delete builder;
+      return;
+    }
+  }
+  g_kernels.emplace_back(builder);
+  TF_SetStatus(status, TF_OK, "");
+}
+
+static const AttrValue* FindAttr(TF_OpKernelConstruction* ctx, const char* name, AttrValue::Kind kind, TF_Status* st) {
+  auto it = ctx->attrs.find(name);
+  if (it == ctx->attrs.end()) {
+    TF_SetStatus(st, TF_INVALID_ARGUMENT, (std::string("No attr named '") + name + "' in NodeDef").c_str());
+    return nullptr;
+  }
+  if (it->second.kind != kind) {
+    TF_SetStatus(st, TF_INVALID_ARGUMENT, (std::string("Attr '") + name + "' has a different type").c_str());
+    return nullptr;
+  }
+  TF_SetStatus(st, TF_OK, "");
+  return &it->second;
+}
+unsigned char TF_OpKernelConstruction_HasAttr(TF_OpKernelConstruction* ctx, const char* attr_name, TF_Status* status) {
+  TF_SetStatus(status, TF_OK, "");
+  return ctx->attrs.count(attr_name) ? 1 : 0;
+}
+void TF_OpKernelConstruction_GetAttrSize(TF_OpKernelConstruction* ctx, const char* attr_name, int32_t* list_size,
+                                         int32_t* total_size, TF_Status* status) {
+  auto it = ctx->attrs.find(attr_name);
+  if (it == ctx->attrs.end()) {
+    TF_SetStatus(status, TF_INVALID_ARGUMENT, (std::string("No attr named '") + attr_name + "' in NodeDef").c_str());
+    return;
+  }
+  TF_SetStatus(status, TF_OK, "");
+  const AttrValue& a = it->second;
+  switch (a.kind) {
+    case AttrValue::STRING: *list_size = -1; *total_size = static_cast<int32_t>(a.s.size()); break;
+    case AttrValue::STRING_LIST: {
+      *list_size = static_cast<int32_t>(a.sl.size());
+      int32_t t = 0;
+      for (const auto& s : a.sl) t += static_cast<int32_t>(s.size());
+      *total_size = t;
+      break;
+    }
+    case AttrValue::TYPE_LIST: *list_size = static_cast<int32_t>(a.tl.size()); *total_size = -1; break;
+    default: *list_size = -1; *total_size = -1; break;
+  }
+}
+void TF_OpKernelConstruction_GetAttrType(TF_OpKernelConstruction* ctx, const char* n, TF_DataType* val, TF_Status* st) {
+  if (const AttrValue* a = FindAttr(ctx, n, AttrValue::TYPE, st)) *val = a->t;
+}
+void TF_OpKernelConstruction_GetAttrInt32(TF_OpKernelConstruction* ctx, const char* n, int32_t* val, TF_Status* st) {
+  if (const AttrValue* a = FindAttr(ctx, n, AttrValue::INT, st)) *val = static_cast<int32_t>(a->i);
+}
+void TF_OpKernelConstruction_GetAttrInt64(TF_OpKernelConstruction* ctx, const char* n, int64_t* val, TF_Status* st) {
+  if (const AttrValue* a = FindAttr(ctx, n, AttrValue::INT, st)) *val = a->i;
+}
+void TF_OpKernelConstruction_GetAttrFloat(TF_OpKernelConstruction* ctx, const char* n, float* val, TF_Status* st) {
+  if (const AttrValue* a = FindAttr(ctx, n, AttrValue::FLOAT, st)) *val = a->f;
+}
+void TF_OpKernelConstruction_GetAttrBool(TF_OpKernelConstruction* ctx, const char* n, unsigned char* val, TF_Status* st) {
+  if (const AttrValue* a = FindAttr(ctx, n, AttrValue::BOOL, st)) *val = a->b ? 1 : 0;
+}
+void TF_OpKernelConstruction_GetAttrString(TF_OpKernelConstruction* ctx, const char* n, char* val, size_t max_length,
+                                           TF_Status* st) {
+  if (const AttrValue* a = FindAttr(ctx, n, AttrValue::STRING, st)) std::memcpy(val, a->s.data(), std::min(max_length, a->s.size()));
+}
+void TF_OpKernelConstruction_GetAttrStringList(TF_OpKernelConstruction* ctx, const char* n, char** values, size_t* lengths,
+                                               int max_values, void* storage, size_t storage_size, TF_Status* st) {
+  const AttrValue* a = FindAttr(ctx, n, AttrValue::STRING_LIST, st);
+  if (!a) return;
+  char* p = static_cast<char*>(storage);
+  size_t used = 0;
+  for (int i = 0; i < max_values && i < static_cast<int>(a->sl.size()); ++i) {
+    const std::string& s = a->sl[i];
+    if (used + s.size() > storage_size) { TF_SetStatus(st, TF_INVALID_ARGUMENT, "storage too small"); return; }
+    std::memcpy(p + used, s.data(), s.size());
+    values[i] = p + used;
+    lengths[i] = s.size();
+    used += s.size();
+  }
+}
+void TF_OpKernelConstruction_GetAttrTypeList(TF_OpKernelConstruction* ctx, const char* n, TF_DataType* vals, int max_vals,
+                                             TF_Status* st) {
+  const AttrValue* a = FindAttr(ctx, n, AttrValue::TYPE_LIST, st);
+  if (!a) return;
+  for (int i = 0; i < max_vals && i < static_cast<int>(a->tl.size()); ++i) vals[i] = a->tl[i];
+}
+TF_StringView TF_OpKernelConstruction_GetName(TF_OpKernelConstruction* ctx) { return TF_StringView{ctx->name.data(), ctx->name.size()}; }
+void TF_OpKernelConstruction_Failure(TF_OpKernelConstruction* ctx, TF_Status* status) {
+  if (ctx->status.code == TF_OK) ctx->status = *status;  // the first failure sticks
+}
+
+int TF_NumInputs(TF_OpKernelContext* ctx) { return static_cast<int>(ctx->inputs.size()); }
+int TF_NumOutputs(TF_OpKernelContext* ctx) { return static_cast<int>(ctx->outputs.size()); }
+void TF_GetInput(TF_OpKernelContext* ctx, int i, TF_Tensor** tensor, TF_Status* status) {
+  if (i < 0 || i >= static_cast<int>(ctx->inputs.size())) {
+    TF_SetStatus(status, TF_OUT_OF_RANGE, "input index out of range");
+    *tensor = nullptr;
+    return;
+  }
+  *tensor = new TF_Tensor(*ctx->inputs[i].t);  // a new handle on the same buffer; the caller deletes it
+  TF_SetStatus(status, TF_OK, "");
+}
+void TF_SetOutput(TF_OpKernelContext* ctx, int i, const TF_Tensor* tensor, TF_Status* status) {
+  if (i < 0 || i >= static_cast<int>(ctx->outputs.size())) { TF_SetStatus(status, TF_OUT_OF_RANGE, "output index out of range"); return; }
+  delete ctx->outputs[i];
+  ctx->outputs[i] = new TF_Tensor(*tensor);
+  TF_SetStatus(status, TF_OK, "");
+}
+TF_DataType TF_ExpectedOutputDataType(TF_OpKernelContext* ctx, int i) { return ctx->out_dtypes[i]; }
+TF_Tensor* TF_AllocateOutput(TF_OpKernelContext* ctx, int index, TF_DataType dtype, const int64_t* dims, int num_dims,
+                             size_t len, TF_Status* status) {
+  if (index < 0 || index >= static_cast<int>(ctx->outputs.size())) { TF_SetStatus(status, TF_OUT_OF_RANGE, "output index out of range"); return nullptr; }
+  if (dtype != ctx->out_dtypes[index]) { TF_SetStatus(status, TF_INVALID_ARGUMENT, "output dtype does not match the node"); return nullptr; }
+  TF_Tensor* t = NewTensor(dtype, dims, num_dims, ctx->out_on_host[index] != 0);
+  if (len != t->buf->bytes) { TF_SetStatus(status, TF_INVALID_ARGUMENT, "byte length does not match shape and dtype"); delete t; return nullptr; }
+  delete ctx->outputs[index];
+  ctx->outputs[index] = new TF_Tensor(*t);
+  TF_SetStatus(status, TF_OK, "");
+  return t;
+}
+TF_Tensor* TF_ForwardInputOrAllocateOutput(TF_OpKernelContext* ctx, const int* cand, int ncand, int output_index,
+                                           const int64_t* output_dims, int output_num_dims, int* forwarded_input,
+                                           TF_Status* status) {
+  if (forwarded_input) *forwarded_input = -1;
+  for (int c = 0; c < ncand; ++c) {
+    const int i = cand[c];
+    if (i < 0 || i >= static_cast<int>(ctx->inputs.size()) || !ctx->inputs[i].allow_forward) continue;
+    TF_Tensor* in = ctx->inputs[i].t;
+    int64_t n_out = 1;
+    for (int d = 0; d < output_num_dims; ++d) n_out *= output_dims[d];
+    if (TF_TensorElementCount(in) != n_out || in->dtype != ctx->out_dtypes[output_index]) continue;
+    auto* t = new TF_Tensor(*in);
+    t->dims.assign(output_dims, output_dims + output_num_dims);
+    delete ctx->outputs[output_index];
+    ctx->outputs[output_index] = new TF_Tensor(*t);
+    ctx->forwarded_from[output_index] = i;
+    if (forwarded_input) *forwarded_input = i;
+    TF_SetStatus(status, TF_OK, "");
+    return t;
+  }
+  int64_t n = 1;
+  for (int d = 0; d < output_num_dims; ++d) n *= output_dims[d];
+  return TF_AllocateOutput(ctx, output_index, ctx->out_dtypes[output_index], output_dims, output_num_dims,
+                           static_cast<size_t>(n) * DtypeSize(ctx->out_dtypes[output_index]), status);
+}
+TF_Tensor* TF_AllocateTemp(TF_OpKernelContext* ctx, TF_DataType dtype, const int64_t* dims, int num_dims,
+                           TF_AllocatorAttributes* attrs, TF_Status* status) {
+  ctx->temp_allocs++;
+  TF_SetStatus(status, TF_OK, "");
+  return NewTensor(dtype, dims, num_dims, attrs && attrs->on_host);
+}
+void TF_OpKernelContext_Failure(TF_OpKernelContext* ctx, TF_Status* status) {
+  if (ctx->status.code == TF_OK) ctx->status = *status;
+}
+SP_Stream TF_GetStream(TF_OpKernelContext* ctx, TF_Status* status) {
+  TF_SetStatus(status, TF_OK, "");
+  return &ctx->stream;
+}
+int64_t TF_StepId(TF_OpKernelContext*) { return 1; }
+
+TF_OpDefinitionBuilder* TF_NewOpDefinitionBuilder(const char* op_name) {
+  auto* b = new TF_OpDefinitionBuilder;
+  b->name = op_name;
+  return b;
+}
+void TF_OpDefinitionBuilderAddInput(TF_OpDefinitionBuilder* b, const char* s) { b->inputs.emplace_back(s); }
+void TF_OpDefinitionBuilderAddOutput(TF_OpDefinitionBuilder* b, const char* s) { b->outputs.emplace_back(s); }
+void TF_OpDefinitionBuilderAddAttr(TF_OpDefinitionBuilder* b, const char* s) { b->attrs.emplace_back(s); }
+void TF_OpDefinitionBuilderSetShapeInferenceFunction(TF_OpDefinitionBuilder* b,
+                                                     void (*fn)(TF_ShapeInferenceContext*, TF_Status*)) {
+  b->has_shape_fn = fn != nullptr;
+  if (fn) {  // exercise it once
+    TF_ShapeInferenceContext c;
+    TF_Status st;
+    fn(&c, &st);
+  }
+}
+void TF_RegisterOpDefinition(TF_OpDefinitionBuilder* b, TF_Status* status) {
+  for (const auto& n : g_stock_ops)
+    if (n == b->name) { TF_SetStatus(status, TF_ALREADY_EXISTS, ("Op with name " + b->name).c_str()); delete b; return; }
+  for (const auto& o : g_ops)
+    if (o->name == b->name) { TF_SetStatus(status, TF_ALREADY_EXISTS, ("Op with name " + b->name).c_str()); delete b; return; }
+  g_ops.emplace_back(b);
+  TF_SetStatus(status, TF_OK, "");
+}
+void TF_ShapeInferenceContextSetUnknownShape(TF_ShapeInferenceContext* ctx, TF_Status* status) {
+  ctx->unknown = true;
+  TF_SetStatus(status, TF_OK, "");
+}
+
+// ------------------------------------------------------------------------------------------------
+// test driver
+// ------------------------------------------------------------------------------------------------
+void mock_set_allocator(AllocFn a, FreeFn f) { g_alloc = a; g_free = f; }
+void mock_add_stock_op(const char* name) { g_stock_ops.emplace_back(name); }
+int mock_delete_calls(void) { return g_delete_calls; }
+
+// dlopen the plugin and call its TF_InitKernel, as TensorFlow does
+int mock_load_plugin(const char* path) {
+  void* h = dlopen(path, RTLD_NOW | RTLD_GLOBAL);
+  if (!h) { std::fprintf(stderr, "mock_tf: dlopen failed: %s\n", dlerror()); return 1; }
+  auto init = reinterpret_cast<void (*)(void)>(dlsym(h, "TF_InitKernel"));
+  if (!init) { std::fprintf(stderr, "mock_tf: TF_InitKernel not exported\n"); return 2; }
+  init();
+  return 0;
+}
+
+static std::string Quote(const std::string& s) {
+  std::string o = "\"";
+  for (char c : s) { if (c == '"' || c == '\\') o.push_back('\\'); o.push_back(c); }
+  return o + "\"";
+}
+const char* mock_dump_registry(void) {
+  std::ostringstream os;
+  os << "{\"kernels\":[";
+  for (size_t i = 0; i < g_kernels.size(); ++i) {
+    const auto& k = g_kernels[i];
+    os << (i ? "," : "") << "{\"op\":" << Quote(k->op) << ",\"device\":" << Quote(k->device) << ",\"label\":" << Quote(k->label)
+       << ",\"constraints\":{";
+    for (size_t c = 0; c < k->constraints.size(); ++c)
+      os << (c ? "," : "") << Quote(k->constraints[c].first) << ":" << static_cast<int>(k->constraints[c].second);
+    os << "},\"host_memory\":[";
+    for (size_t h = 0; h < k->host_memory.size(); ++h) os << (h ? "," : "") << Quote(k->host_memory[h]);
+    os << "]}";
+  }
+  os << "],\"ops\":[";
+  for (size_t i = 0; i < g_ops.size(); ++i) {
+    const auto& o = g_ops[i];
+    auto list = [&](const std::vector<std::string>& v) {
+      os << "[";
+      for (size_t j = 0; j < v.size(); ++j) os << (j ? "," : "") << Quote(v[j]);
+      os << "]";
+    };
+    os << (i ? "," : "") << "{\"name\":" << Quote(o->name) << ",\"inputs\":";
+    list(o->inputs);
+    os << ",\"outputs\":";
+    list(o->outputs);
+    os << ",\"attrs\":";
+    list(o->attrs);
+    os << ",\"shape_fn\":" << (o->has_shape_fn ? "true" : "false") << "}";
+  }
+  os << "]}";
+  g_json = os.str();
+  return g_json.c_str();
+}
+
+void* mock_node_new(const char* op, const char* device) {
+  auto* n = new Node;
+  n->op = op;
+  n->device = device;
+  n->construction.name = std::string("test/") + op;
+  return n;
+}
+static AttrValue& Attr(void* h, const char* name, AttrValue::Kind k) {
+  AttrValue& a = static_cast<Node*>(h)->construction.attrs[name];
+  a.kind = k;
+  return a;
+}
+void mock_node_attr_string(void* h, const char* name, const char* v) { Attr(h, name, AttrValue::STRING).s = v; }
+void mock_node_attr_int(void* h, const char* name, int64_t v) { Attr(h, name, AttrValue::INT).i = v; }
+void mock_node_attr_float(void* h, const char* name, float v) { Attr(h, name, AttrValue::FLOAT).f = v; }
+void mock_node_attr_bool(void* h, const char* name, int v) { Attr(h, name, AttrValue::BOOL).b = v != 0; }
+void mock_node_attr_type(void* h, const char* name, int v) { Attr(h, name, AttrValue::TYPE).t = static_cast<TF_DataType>(v); }
+void mock_node_attr_string_list(void* h, const char* name, const char** v, int n) {
+  AttrValue& a = Attr(h, name, AttrValue::STRING_LIST);
+  a.sl.assign(v, v + n);
+}
+void mock_node_attr_type_list(void* h, const char* name, const int* v, int n) {
+  AttrValue& a = Attr(h, name, AttrValue::TYPE_LIST);
+  a.tl.clear();
+  for (int i = 0; i < n; ++i) a.tl.push_back(static_cast<TF_DataType>(v[i]));
+}
+
+// kernel lookup by op, device and type constraints, then create().  Returns the TF_Code of construction
+// (TF_NOT_FOUND when no kernel matches).
+int mock_node_instantiate(void* h) {
+  Node* n = static_cast<Node*>(h);
+  n->kernel = nullptr;
+  for (const auto& k : g_kernels) {
+    if (k->op != n->op || k->device != n->device) continue;
+    bool match = true;
+    for (const auto& c : k->constraints) {
+      auto it = n->construction.attrs.find(c.first);
+      if (it == n->construction.attrs.end() || it->second.kind != AttrValue::TYPE || it->second.t != c.second) { match = false; break; }
+    }
+    if (match) { n->kernel = k.get(); break; }
+  }
+  if (!n->kernel) {
+    n->construction.status.code = TF_NOT_FOUND;
+    n->construction.status.msg = "No registered kernel for " + n->op + " on " + n->device;
+    return TF_NOT_FOUND;
+  }
+  n->construction.status = TF_Status();
+  n->object = n->kernel->create(&n->construction);
+  if (n->construction.status.code != TF_OK && n->object) {  // TensorFlow deletes a kernel whose construction failed
+    n->kernel->del(n->object);
+    ++g_delete_calls;
+    n->object = nullptr;
+  }
+  return n->construction.status.code;
+}
+const char* mock_node_construction_message(void* h) { return static_cast<Node*>(h)->construction.status.msg.c_str(); }
+
+void mock_node_clear_io(void* h) {
+  Node* n = static_cast<Node*>(h);
+  for (auto& in : n->context.inputs) delete in.t;
+  for (auto* o : n->context.outputs) delete o;
+  n->context.inputs.clear();
+  n->context.outputs.clear();
+  n->context.forwarded_from.clear();
+  n->context.out_dtypes.clear();
+  n->context.out_on_host.clear();
+  n->context.status = TF_Status();
+}
+// the tensor wraps caller-owned memory
+void mock_node_add_input(void* h, int dtype, const int64_t* dims, int ndims, void* data, int on_host, int allow_forward) {
+  Node* n = static_cast<Node*>(h);
+  auto* t = new TF_Tensor;
+  t->dtype = static_cast<TF_DataType>(dtype);
+  t->dims.assign(dims, dims + ndims);
+  t->buf = std::make_shared<Buffer>();
+  int64_t cnt = 1;
+  for (int64_t d : t->dims) cnt *= d;
+  t->buf->bytes = static_cast<size_t>(cnt) * DtypeSize(t->dtype);
+  t->buf->data = data;
+  t->buf->owned = false;
+  t->buf->on_host = on_host != 0;
+  n->context.inputs.push_back({t, allow_forward != 0});
+}
+void mock_node_add_output(void* h, int dtype, int on_host) {
+  Node* n = static_cast<Node*>(h);
+  n->context.outputs.push_back(nullptr);
+  n->context.forwarded_from.push_back(-1);
+  n->context.out_dtypes.push_back(static_cast<TF_DataType>(dtype));
+  n->context.out_on_host.push_back(static_cast<char>(on_host));
+}
+void mock_node_set_stream(void* h, void* stream) { static_cast<Node*>(h)->context.stream.stream_handle = stream; }
+int mock_node_compute(void* h) {
+  Node* n = static_cast<Node*>(h);
+  if (!n->object) return TF_FAILED_PRECONDITION;
+  n->context.status = TF_Status();
+  n->kernel->compute(n->object, &n->context);
+  return n->context.status.code;
+}
+const char* mock_node_compute_message(void* h) { return static_cast<Node*>(h)->context.status.msg.c_str(); }
+int mock_node_temp_allocs(void* h) { return static_cast<Node*>(h)->context.temp_allocs; }
+// returns 0 if the output was produced
+int mock_node_output(void* h, int i, int* dtype, int64_t* dims, int* ndims, void** data, int* forwarded_from) {
+  Node* n = static_cast<Node*>(h);
+  if (i < 0 || i >= static_cast<int>(n->context.outputs.size()) || !n->context.outputs[i]) return 1;
+  TF_Tensor* t = n->context.outputs[i];
+  *dtype = t->dtype;
+  *ndims = static_cast<int>(t->dims.size());
+  for (int d = 0; d < *ndims && d < 8; ++d) dims[d] = t->dims[d];
+  *data = t->buf->data;
+  *forwarded_from = n->context.forwarded_from[i];
+  return 0;
+}
+void mock_node_delete(void* h) {
+  Node* n = static_cast<Node*>(h);
+  mock_node_clear_io(h);
+  if (n->object) { n->kernel->del(n->object); ++g_delete_calls; }
+  delete n;
+}
+
+}  // extern "C"

@@ -1,0 +1,302 @@
+"""GPU tests of the kernel plugin through the mock TensorFlow host: the ops are created from node
+attributes and run with device tensors and host-memory min/max tensors, exactly as TensorFlow would
+call them; results are compared bit for bit with the CPU oracle."""
+import numpy as np
+import pytest
+
+from oracle import pyoracle as orc
+from tests.mock_tf import host as tf
+
+pytestmark = pytest.mark.gpu
+DT = tf.DType
+
+
+@pytest.fixture(scope="module")
+def rt(dev):
+    import torch
+    tf.load()
+    tf.use_torch_allocator(dev)
+    return torch
+
+
+def dev_in(torch, dev, a):
+    t = torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+    return t
+
+
+def fetch(torch, out, np_dtype):
+    """Copies an output tensor of the mock (device or host memory) into numpy."""
+    dtype, shape, addr, _ = out
+    n = int(np.prod(shape, dtype=np.int64)) if len(shape) else 1
+    import ctypes as C
+    torch.cuda.synchronize()
+    host = np.empty(n, np_dtype)
+    # device memory handed out by the torch allocator: wrap it through a uint8 view
+    live = tf._state["alloc_cb"][2]
+    if addr in live:
+        nbytes = n * np.dtype(np_dtype).itemsize
+        host = live[addr][:nbytes].cpu().numpy().view(np_dtype).copy()
+    else:
+        host = tf.read_host(addr, dtype, shape).ravel()
+    return host.reshape(shape)
+
+
+def run_quantize(torch, dev, x, mn, mx, T, mode, axis=-1, classic=None, forward=False, op="QuantizeV2"):
+    attrs = dict(T=DT(T), mode=mode, round_mode="HALF_TO_EVEN" if mode == "SCALED" else "HALF_AWAY_FROM_ZERO",
+                 narrow_range=False, axis=axis, ensure_minimum_range=0.01)
+    if op == "_ITEXQuantizeV2":
+        attrs["dtype"] = DT(tf.FLOAT)
+        if classic is not None:
+            attrs["classic_asymmetric_algorithm"] = bool(classic)
+    node = tf.Node(op, attrs)
+    assert node.code == tf.OK, node.message
+    x_d = dev_in(torch, dev, x)
+    mn_h = np.atleast_1d(np.float32(mn)).copy() if axis >= 0 else np.array(mn, np.float32)
+    mx_h = np.atleast_1d(np.float32(mx)).copy() if axis >= 0 else np.array(mx, np.float32)
+    code, msg, outs = node.run(
+        [(tf.FLOAT, x.shape, x_d.data_ptr(), False), (tf.FLOAT, mn_h.shape, tf.host_array(mn_h), True, forward),
+         (tf.FLOAT, mx_h.shape, tf.host_array(mx_h), True, forward)],
+        [(T, False), (tf.FLOAT, True), (tf.FLOAT, True)], stream=torch.cuda.current_stream().cuda_stream)
+    assert code == tf.OK, msg
+    q = fetch(torch, outs[0], tf.NP_OF[T])
+    omn = fetch(torch, outs[1], np.float32)
+    omx = fetch(torch, outs[2], np.float32)
+    fwd = (outs[1][3], outs[2][3])
+    node.close()
+    return q, omn, omx, fwd, (mn_h, mx_h)
+
+
+def test_quantize_golden_through_plugin(rt, dev, golden):
+    torch = rt
+    T = {"quint8": tf.QUINT8, "qint8": tf.QINT8}
+    for case in golden["quantize_v2"]:
+        x = np.array(case["x"], np.float32).reshape(case["shape"])
+        op = "_ITEXQuantizeV2" if case["classic_asymmetric_algorithm"] else "QuantizeV2"
+        q, omn, omx, _, _ = run_quantize(torch, dev, x, case["min_range"], case["max_range"], T[case["T"]], case["mode"],
+                                         classic=case["classic_asymmetric_algorithm"] or None, op=op)
+        assert q.ravel().tolist() == case["expected"], case["source"]
+
+
+def test_quantize_axis_golden_through_plugin(rt, dev, golden):
+    torch = rt
+    g = golden["quantize_v2_axis"]
+    shape = np.array(g["shape"])
+    values = np.array(g["values"], np.float32)
+    quant = np.array(g["quant_values"], np.int32)
+    expected = np.take(quant, np.remainder(np.arange(np.prod(shape)), len(quant))).reshape(shape)
+    for axis in (1, 2, 3):
+        x = np.take(values, np.remainder(np.arange(np.prod(shape)), len(values))).reshape(shape)
+        sc = [1] * 4
+        sc[axis] = shape[axis]
+        x = (x * np.arange(1, shape[axis] + 1).reshape(sc)).astype(np.float32)
+        mn = [g["min_unit"] * (s + 1) for s in range(shape[axis])]
+        mx = [g["max_unit"] * (s + 1) for s in range(shape[axis])]
+        q, omn, omx, _, _ = run_quantize(torch, dev, x, mn, mx, tf.QINT8, "SCALED", axis=axis)
+        np.testing.assert_array_equal(q.astype(np.int32), expected)
+        np.testing.assert_array_equal(omx, np.abs(np.float32(mn)))
+        np.testing.assert_array_equal(omn, -omx)
+
+
+@pytest.mark.parametrize("forward", [False, True])
+def test_quantize_outputs_and_forwarding(rt, dev, forward):
+    """output_min/max: adjusted range; with forwarding the kernel overwrites the caller's min/max
+    tensors in place (forward_input_or_allocate_output in the reference)."""
+    torch = rt
+    x = np.random.default_rng(0).standard_normal(4099).astype(np.float32)
+    q, omn, omx, fwd, (mn_h, mx_h) = run_quantize(torch, dev, x, 0.5, 2.0, tf.QUINT8, "SCALED", forward=forward)
+    _, q_ref, omn_ref, omx_ref = orc.quantize_v2(x, 0.5, 2.0, orc.QUINT8, orc.SCALED)
+    np.testing.assert_array_equal(q, q_ref)
+    assert omn == omn_ref[0] == 0.0 and omx == omx_ref[0] == 2.0
+    if forward:
+        assert fwd == (1, 2) and mn_h == 0.0 and mx_h == 2.0  # input buffers were reused and rewritten
+    else:
+        assert fwd == (-1, -1) and mn_h == np.float32(0.5)
+
+
+def test_dequantize_through_plugin(rt, dev):
+    torch = rt
+    rng = np.random.default_rng(1)
+    for T, mode in ((tf.QINT8, "SCALED"), (tf.QUINT8, "MIN_FIRST")):
+        q = rng.integers(np.iinfo(tf.NP_OF[T]).min, np.iinfo(tf.NP_OF[T]).max + 1, 5003).astype(tf.NP_OF[T])
+        node = tf.Node("Dequantize", dict(T=DT(T), mode=mode, narrow_range=False, axis=-1, dtype=DT(tf.FLOAT)))
+        assert node.code == tf.OK, node.message
+        mn, mx = np.array(-2.5, np.float32), np.array(3.25, np.float32)
+        q_d = dev_in(torch, dev, q)
+        code, msg, outs = node.run([(T, q.shape, q_d.data_ptr(), False), (tf.FLOAT, (), tf.host_array(mn), True),
+                                    (tf.FLOAT, (), tf.host_array(mx), True)], [(tf.FLOAT, False)],
+                                   stream=torch.cuda.current_stream().cuda_stream)
+        assert code == tf.OK, msg
+        y = fetch(torch, outs[0], np.float32)
+        _, y_ref = orc.dequantize(q, mn, mx, T, orc.SCALED if mode == "SCALED" else orc.MIN_FIRST)
+        np.testing.assert_array_equal(y, y_ref)
+        node.close()
+
+
+def make_problem(M, K, N, seed, per_channel=True):
+    rng = np.random.default_rng(seed)
+    x = rng.standard_normal((M, K)).astype(np.float32)
+    w = (rng.standard_normal((K, N)) * 0.02).astype(np.float32)
+    bias = (rng.standard_normal(N) * 0.01).astype(np.float32)
+    _, xq, xmn, xmx = orc.quantize_v2(x, x.min(), x.max(), orc.QUINT8, orc.MIN_FIRST)
+    if per_channel:
+        r = np.abs(w).max(0).astype(np.float32)
+        _, wq, wmn, wmx = orc.quantize_v2(w, -r, r, orc.QINT8, orc.SCALED, axis=1)
+    else:
+        _, wq, wmn, wmx = orc.quantize_v2(w, w.min(), w.max(), orc.QINT8, orc.SCALED)
+        wmn, wmx = np.array(wmn[0], np.float32), np.array(wmx[0], np.float32)
+    return x, w, bias, xq, np.array(xmn[0], np.float32), np.array(xmx[0], np.float32), wq, wmn, wmx
+
+
+def matmul_inputs(torch, dev, xq, wq, bias, scalars):
+    keep = [dev_in(torch, dev, xq), dev_in(torch, dev, wq), dev_in(torch, dev, bias)]
+    ins = [(tf.QUINT8 if xq.dtype == np.uint8 else tf.QINT8, xq.shape, keep[0].data_ptr(), False),
+           (tf.QINT8, wq.shape, keep[1].data_ptr(), False), (tf.FLOAT, bias.shape, keep[2].data_ptr(), False)]
+    for s in scalars:
+        ins.append((tf.FLOAT, s.shape, tf.host_array(s), True))
+    return ins, keep
+
+
+V2 = dict(T1=DT(tf.QUINT8), T2=DT(tf.QINT8), Tbias=DT(tf.FLOAT), transpose_a=False, transpose_b=False,
+          is_weight_const=True, is_bias_const=True, input_quant_mode="MIN_FIRST", output_quant_mode="SCALED",
+          leakyrelu_alpha=0.2)
+
+
+@pytest.mark.parametrize("M,K,N", [(4, 64, 32), (100, 256, 200), (16, 1024, 512), (2, 3, 4)])
+def test_quantized_matmul_v2_dequantize(rt, dev, M, K, N):
+    torch = rt
+    x, w, bias, xq, xmn, xmx, wq, wmn, wmx = make_problem(M, K, N, seed=M + K)
+    node = tf.Node("_QuantizedMatMul", dict(V2, Tout=DT(tf.FLOAT), fused_ops=["BiasAdd", "Relu", "Dequantize"]))
+    assert node.code == tf.OK, node.message
+    at = orc.matmul_attrs(api=orc.API_V2, t_in=orc.QUINT8, t_out=orc.FLOAT, input_mode=orc.MIN_FIRST,
+                          activation=orc.ACT_RELU, has_dequantize=True)
+    ins, keep = matmul_inputs(torch, dev, xq, wq, bias, [xmn, xmx, wmn, wmx])
+    stream = torch.cuda.current_stream().cuda_stream
+    for it in range(2):  # second run exercises the cached weight / parameter state
+        code, msg, outs = node.run(ins, [(tf.FLOAT, False)], stream=stream)
+        assert code == tf.OK, msg
+        y = fetch(torch, outs[0], np.float32)
+        _, y_ref = orc.qmatmul(at, xq, wq, bias, xmn, xmx, wmn, wmx)
+        np.testing.assert_array_equal(y, y_ref)
+    first = node.temp_allocs()
+    # a new activation range must be picked up without re-preparing the weight
+    xmn2, xmx2 = np.array(xmn * 1.5, np.float32), np.array(xmx * 0.75, np.float32)
+    ins2, keep2 = matmul_inputs(torch, dev, xq, wq, bias, [xmn2, xmx2, wmn, wmx])
+    ins2[1] = ins[1]  # same weight tensor
+    code, msg, outs = node.run(ins2, [(tf.FLOAT, False)], stream=stream)
+    assert code == tf.OK, msg
+    _, y_ref2 = orc.qmatmul(at, xq, wq, bias, xmn2, xmx2, wmn, wmx)
+    np.testing.assert_array_equal(fetch(torch, outs[0], np.float32), y_ref2)
+    assert node.temp_allocs() == first  # no new device allocation
+    node.close()
+
+
+def test_quantized_matmul_requantize_and_minmax_outputs(rt, dev):
+    torch = rt
+    M, K, N = 64, 512, 96
+    x, w, bias, xq, xmn, xmx, wq, wmn, wmx = make_problem(M, K, N, seed=9)
+    r_out = np.float32(np.abs(x @ w + bias).max())
+    mo, xo = np.array(-r_out, np.float32), np.array(r_out, np.float32)
+    stream = torch.cuda.current_stream().cuda_stream
+    # V2 spelling
+    node = tf.Node("_QuantizedMatMul", dict(V2, Tout=DT(tf.QINT8), fused_ops=["BiasAdd", "Requantize"]))
+    ins, keep = matmul_inputs(torch, dev, xq, wq, bias, [xmn, xmx, wmn, wmx, mo, xo])
+    code, msg, outs = node.run(ins, [(tf.QINT8, False), (tf.FLOAT, True), (tf.FLOAT, True)], stream=stream)
+    assert code == tf.OK, msg
+    at = orc.matmul_attrs(api=orc.API_V2, t_in=orc.QUINT8, t_out=orc.QINT8, input_mode=orc.MIN_FIRST, has_requantize=True)
+    _, q_ref = orc.qmatmul(at, xq, wq, bias, xmn, xmx, wmn, wmx, -r_out, r_out)
+    np.testing.assert_array_equal(fetch(torch, outs[0], np.int8), q_ref)
+    assert fetch(torch, outs[1], np.float32) == -r_out and fetch(torch, outs[2], np.float32) == r_out
+    node.close()
+    # V1 spelling, qint32 product with per-channel ranges out
+    v1 = dict(T1=DT(tf.QUINT8), T2=DT(tf.QINT8), Targs=DT(tf.FLOAT), Toutput=DT(tf.QINT32), num_args=1, transpose_a=False,
+              transpose_b=False, fused_ops=["BiasAdd"], is_filter_const=True, is_bias_const=True,
+              input_quant_mode="MIN_FIRST", leakyrelu_alpha=0.2)
+    node = tf.Node("_QuantizedFusedMatMul", v1)
+    assert node.code == tf.OK, node.message
+    ins, keep = matmul_inputs(torch, dev, xq, wq, bias, [xmn, xmx, wmn, wmx])
+    code, msg, outs = node.run(ins, [(tf.QINT32, False), (tf.FLOAT, True), (tf.FLOAT, True)], stream=stream)
+    assert code == tf.OK, msg
+    at = orc.matmul_attrs(api=orc.API_V1, t_in=orc.QUINT8, t_out=orc.QINT32, input_mode=orc.MIN_FIRST, n_fused_ops=1)
+    _, acc_ref = orc.qmatmul(at, xq, wq, bias, xmn, xmx, wmn, wmx)
+    np.testing.assert_array_equal(fetch(torch, outs[0], np.int32), acc_ref)
+    _, omn_ref, omx_ref = orc.qmatmul_output_minmax(at, xmn, xmx, wmn, wmx, 1, 0, 0)
+    np.testing.assert_array_equal(fetch(torch, outs[1], np.float32), omn_ref)
+    np.testing.assert_array_equal(fetch(torch, outs[2], np.float32), omx_ref)
+    node.close()
+
+
+def test_legacy_matmul_with_bias_and_relu_and_requantize(rt, dev):
+    torch = rt
+    M, K, N = 32, 256, 64
+    x, w, bias, xq, xmn, xmx, wq, wmn, wmx = make_problem(M, K, N, seed=5, per_channel=False)
+    r_out = np.float32(np.maximum(x @ w + bias, 0).max())
+    mo, xo = np.array(0.0, np.float32), np.array(r_out, np.float32)
+    node = tf.Node("QuantizedMatMulWithBiasAndReluAndRequantize",
+                   dict(T1=DT(tf.QUINT8), T2=DT(tf.QINT8), Tbias=DT(tf.FLOAT), Toutput=DT(tf.QUINT8), transpose_a=False,
+                        transpose_b=False, input_quant_mode="MIN_FIRST"))
+    assert node.code == tf.OK, node.message
+    ins, keep = matmul_inputs(torch, dev, xq, wq, bias, [xmn, xmx, wmn, wmx, mo, xo])
+    code, msg, outs = node.run(ins, [(tf.QUINT8, False), (tf.FLOAT, True), (tf.FLOAT, True)],
+                               stream=torch.cuda.current_stream().cuda_stream)
+    assert code == tf.OK, msg
+    at = orc.matmul_attrs(api=orc.API_LEGACY, t_in=orc.QUINT8, t_out=orc.QUINT8, input_mode=orc.MIN_FIRST,
+                          activation=orc.ACT_RELU)
+    _, q_ref = orc.qmatmul(at, xq, wq, bias, xmn, xmx, wmn, wmx, 0.0, r_out)
+    np.testing.assert_array_equal(fetch(torch, outs[0], np.uint8), q_ref)
+    node.close()
+
+
+def test_full_chain_config1_shape(rt, dev):
+    """QuantizeV2 -> _QuantizedMatMul [BiasAdd, Relu, Dequantize] -> compared with the fp32 graph at the
+    reference tests' own tolerance, and with the oracle exactly."""
+    torch = rt
+    M, K, N = 128, 1024, 1024
+    rng = np.random.default_rng(0)
+    x = rng.standard_normal((M, K)).astype(np.float32)
+    w = (rng.standard_normal((K, N)) * 0.02).astype(np.float32)
+    bias = (rng.standard_normal(N) * 0.01).astype(np.float32)
+    r = np.abs(w).max(0).astype(np.float32)
+    _, wq, wmn, wmx = orc.quantize_v2(w, -r, r, orc.QINT8, orc.SCALED, axis=1)
+    xq, xmn, xmx, _, _ = run_quantize(torch, dev, x, x.min(), x.max(), tf.QUINT8, "MIN_FIRST")
+    node = tf.Node("_QuantizedMatMul", dict(V2, Tout=DT(tf.FLOAT), fused_ops=["BiasAdd", "Relu", "Dequantize"]))
+    ins, keep = matmul_inputs(torch, dev, xq, wq, bias, [np.array(xmn, np.float32), np.array(xmx, np.float32), wmn, wmx])
+    code, msg, outs = node.run(ins, [(tf.FLOAT, False)], stream=torch.cuda.current_stream().cuda_stream)
+    assert code == tf.OK, msg
+    y = fetch(torch, outs[0], np.float32)
+    np.testing.assert_allclose(y, np.maximum(x @ w + bias, 0), rtol=0.2, atol=0.2)
+    at = orc.matmul_attrs(api=orc.API_V2, t_in=orc.QUINT8, t_out=orc.FLOAT, input_mode=orc.MIN_FIRST,
+                          activation=orc.ACT_RELU, has_dequantize=True)
+    _, y_ref = orc.qmatmul(at, xq, wq, bias, xmn, xmx, wmn, wmx)
+    np.testing.assert_array_equal(y, y_ref)
+    node.close()
+
+
+def test_requantize_per_channel_ops(rt, dev):
+    torch = rt
+    rng = np.random.default_rng(3)
+    x = np.rint(rng.standard_normal((2, 4, 8, 64)) * (1 << 20)).astype(np.int32)
+    in_min = -(rng.random(64).astype(np.float32) + 0.5)
+    in_max = rng.random(64).astype(np.float32) + 0.5
+    x_d = dev_in(torch, dev, x)
+    stream = torch.cuda.current_stream().cuda_stream
+    rng_node = tf.Node("RequantizationRangePerChannel", dict(T=DT(tf.QINT32), clip_value_max=6.0))
+    assert rng_node.code == tf.OK, rng_node.message
+    code, msg, outs = rng_node.run([(tf.QINT32, x.shape, x_d.data_ptr(), False), (tf.FLOAT, (64,), tf.host_array(in_min), True),
+                                    (tf.FLOAT, (64,), tf.host_array(in_max), True)], [(tf.FLOAT, True), (tf.FLOAT, True)],
+                                   stream=stream)
+    assert code == tf.OK, msg
+    _, omn_ref, omx_ref = orc.requantization_range_per_channel(x, in_min, in_max, 6.0)
+    omn, omx = fetch(torch, outs[0], np.float32), fetch(torch, outs[1], np.float32)
+    assert omn == omn_ref and omx == omx_ref
+    rng_node.close()
+    node = tf.Node("RequantizePerChannel", dict(T=DT(tf.QINT32), out_type=DT(tf.QINT8)))
+    assert node.code == tf.OK, node.message
+    rmin, rmax = np.array(omn, np.float32), np.array(omx, np.float32)
+    code, msg, outs = node.run([(tf.QINT32, x.shape, x_d.data_ptr(), False), (tf.FLOAT, (64,), tf.host_array(in_min), True),
+                                (tf.FLOAT, (64,), tf.host_array(in_max), True), (tf.FLOAT, (), tf.host_array(rmin), True),
+                                (tf.FLOAT, (), tf.host_array(rmax), True)],
+                               [(tf.QINT8, False), (tf.FLOAT, True), (tf.FLOAT, True)], stream=stream)
+    assert code == tf.OK, msg
+    _, q_ref, _, _ = orc.requantize_per_channel(x, in_min, in_max, float(rmin), float(rmax), orc.QINT8)
+    np.testing.assert_array_equal(fetch(torch, outs[0], np.int8), q_ref)
+    node.close()
