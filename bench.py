@@ -217,7 +217,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--only", type=str, default="", help="comma list of: headline, prefill, bert, gemv, elementwise")
+    ap.add_argument("--only", type=str, default="", help="comma list of: headline, prefill, bert, gemv, elementwise, copy")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-rows", type=int, default=2048, help="rows of the headline workload the CPU oracle runs")
     args = ap.parse_args()
@@ -280,6 +280,16 @@ def main():
                 r.update(name="decode_gemv", bound="hbm", frac=r["gbs_kernel"] / PEAK_HBM_GBS,
                          note="8 weight copies cycled (470 MB > last-level cache)")
                 others.append(r)
+    if "copy" in only:
+        # device copy of 1 GiB: the kernel of known traffic that calibrates the memory counters
+        nb = 1 << 30
+        src = torch.empty(nb, dtype=torch.uint8, device=dev).random_(0, 256)
+        dst = torch.empty_like(src)
+        st = _stream(torch)
+        ms = timer.run(lambda i: hip.memcpy_d2d_async(dst, src, nb, st), max(10, K_steps // 2), max(3, W // 2))
+        others.append(dict(name="copy_d2d", n=nb, us_kernel=ms * 1e3, bytes=2 * nb, gbs=2 * nb / (ms * 1e-3) / 1e9,
+                           frac=2 * nb / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS, bound="hbm"))
+        del src, dst
     if "elementwise" in only:
         for r in bench_elementwise(torch, hip, timer, 1 << 28, max(10, K_steps // 2), max(3, W // 2), dev):
             r.update(bound="hbm")

@@ -56,6 +56,10 @@ int itexhip_memcpy_h2d_async(void* dst_device, const void* src_host, size_t byte
 /* device-to-host copy ordered after the work already on `stream`; returns when the data has arrived */
 int itexhip_memcpy_d2h(void* dst_host, const void* src_device, size_t bytes, void* stream);
 int itexhip_stream_synchronize(void* stream);
+/* device-to-device copy as a kernel on `stream` (16 B per lane, any alignment and size); it stands
+ * where the reference's stream copies device buffers (itex/core/devices/gpu/gpu_device_plugin.cc,
+ * memcpy_dtod) and is the kernel of known traffic that calibrates the HBM counters */
+int itexhip_memcpy_d2d_async(void* dst_device, const void* src_device, size_t bytes, void* stream);
 
 /* ------------------------------------------------------------------------------------------
  * QuantizeV2.  q[i] = sat_T(rne(fl(x[i] * scale) + addend))

@@ -25,7 +25,7 @@ INCLUDE = os.path.join(ROOT, "include")
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 HIP_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off",
-    "-fno-fast-math", "-fgpu-flush-denormals-to-zero=0" if False else "-fno-gpu-flush-denormals-to-zero",
+    "-fno-fast-math", "-fno-gpu-flush-denormals-to-zero",
     # no packed-fp32 instructions in device code
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wall", "-Wno-unused-function", "-I", INCLUDE, "-I", CSRC,

@@ -304,6 +304,32 @@ inline unsigned blocks_for(int64_t n, int64_t per_block) {
   return static_cast<unsigned>((n + per_block - 1) / per_block);
 }
 
+// ------------------------------------------------------------------------------------------------
+// Plain device-to-device copy (16 B per lane): the kernel of known traffic against which the memory
+// counters are calibrated, and the stream's device copy.
+// ------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(kThreads) void copy_vec_kernel(const i4* __restrict__ src, i4* __restrict__ dst,
+                                                            int64_t n16) {
+  const int64_t base = static_cast<int64_t>(blockIdx.x) * (kThreads * kUnroll) + threadIdx.x;
+  i4 v[kUnroll];
+#pragma unroll
+  for (int j = 0; j < kUnroll; ++j) {
+    const int64_t i = base + j * kThreads;
+    if (i < n16) v[j] = __builtin_nontemporal_load(&src[i]);
+  }
+#pragma unroll
+  for (int j = 0; j < kUnroll; ++j) {
+    const int64_t i = base + j * kThreads;
+    if (i < n16) __builtin_nontemporal_store(v[j], &dst[i]);
+  }
+}
+
+__global__ __launch_bounds__(kThreads) void copy_byte_kernel(const uint8_t* __restrict__ src,
+                                                             uint8_t* __restrict__ dst, int64_t begin, int64_t n) {
+  const int64_t i = begin + static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+  if (i < n) dst[i] = src[i];
+}
+
 }  // namespace
 }  // namespace itexhip
 
@@ -528,5 +554,24 @@ extern "C" int itexhip_minmax_f32(const float* x, int64_t n, float* minmax_out, 
   }
   finish_minmax_f32_kernel<<<1, 1, 0, st>>>(keys);
   ITEXHIP_CHECK_LAUNCH("itexhip_minmax_f32");
+  return ITEXHIP_OK;
+}
+
+extern "C" int itexhip_memcpy_d2d_async(void* dst, const void* src, size_t bytes, void* stream) {
+  if (bytes == 0) return ITEXHIP_OK;
+  ITEXHIP_REQUIRE(dst && src, "itexhip_memcpy_d2d_async: null buffer");
+  hipStream_t st = as_stream(stream);
+  int64_t done = 0;
+  const int64_t n = static_cast<int64_t>(bytes);
+  if (aligned(src, 16) && aligned(dst, 16) && n >= 16) {
+    const int64_t n16 = n / 16;
+    copy_vec_kernel<<<blocks_for(n16, kThreads * kUnroll), kThreads, 0, st>>>(
+        reinterpret_cast<const i4*>(src), reinterpret_cast<i4*>(dst), n16);
+    done = n16 * 16;
+  }
+  if (done < n)
+    copy_byte_kernel<<<blocks_for(n - done, kThreads), kThreads, 0, st>>>(
+        reinterpret_cast<const uint8_t*>(src), reinterpret_cast<uint8_t*>(dst), done, n);
+  ITEXHIP_CHECK_LAUNCH("itexhip_memcpy_d2d_async");
   return ITEXHIP_OK;
 }

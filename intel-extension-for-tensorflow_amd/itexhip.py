@@ -18,7 +18,7 @@ ACT_NONE, ACT_RELU, ACT_RELU6, ACT_LEAKYRELU = 0, 1, 2, 3
 ELT_RELU, ELT_CLIP, ELT_LINEAR = 1, 2, 3
 
 EXPORTS = [
-    "itexhip_last_error", "itexhip_build_info", "itexhip_memcpy_h2d_async", "itexhip_memcpy_d2h", "itexhip_stream_synchronize", "itexhip_quantize", "itexhip_quantize_axis",
+    "itexhip_last_error", "itexhip_build_info", "itexhip_memcpy_h2d_async", "itexhip_memcpy_d2h", "itexhip_memcpy_d2d_async", "itexhip_stream_synchronize", "itexhip_quantize", "itexhip_quantize_axis",
     "itexhip_dequantize", "itexhip_dequantize_axis", "itexhip_requantize_per_channel",
     "itexhip_requantize", "itexhip_minmax_i32_per_channel", "itexhip_minmax_f32",
     "itexhip_qmatmul_epilogue_desc", "itexhip_qmatmul_prepare", "itexhip_qgemm_packed_bytes",
@@ -92,6 +92,10 @@ def _i64(v):
 
 def build_info():
     return _lib.itexhip_build_info().decode()
+
+
+def memcpy_d2d_async(dst, src, nbytes, stream=0):
+    _check(_lib.itexhip_memcpy_d2d_async(_ptr(dst), _ptr(src), C.c_size_t(int(nbytes)), _ptr(stream)))
 
 
 def quantize(x, q, n, dst_type, scale, addend=0.0, stream=0):

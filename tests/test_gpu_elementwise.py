@@ -300,3 +300,16 @@ def test_full_size_quantize_properties(hip, dev):
         err = float((y_d - x_d.clamp(float(omn[0]), float(omx[0]))).abs().max())
         assert err <= step * (0.5 if mode == orc.SCALED else 1.0) * 1.001 + 1e-6
         del q_d, y_d
+
+
+@pytest.mark.parametrize("nbytes,offset", [(1 << 20, 0), (4099, 0), (70001, 3), (15, 1), (0, 0)])
+def test_device_copy_kernel(hip, dev, nbytes, offset):
+    import torch
+    src = torch.randint(0, 256, (nbytes + 64,), dtype=torch.uint8, device=dev)
+    dst = torch.zeros(nbytes + 64, dtype=torch.uint8, device=dev)
+    hip.memcpy_d2d_async(dst.data_ptr() + offset, src.data_ptr() + offset, nbytes,
+                         torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    expect = torch.zeros_like(dst)
+    expect[offset:offset + nbytes] = src[offset:offset + nbytes]
+    assert torch.equal(dst, expect)
