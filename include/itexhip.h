@@ -57,8 +57,8 @@ int itexhip_memcpy_h2d_async(void* dst_device, const void* src_host, size_t byte
 int itexhip_memcpy_d2h(void* dst_host, const void* src_device, size_t bytes, void* stream);
 int itexhip_stream_synchronize(void* stream);
 /* device-to-device copy as a kernel on `stream` (16 B per lane, any alignment and size); it stands
- * where the reference's stream copies device buffers (itex/core/devices/gpu/gpu_device_plugin.cc,
- * memcpy_dtod) and is the kernel of known traffic that calibrates the HBM counters */
+ * where the reference's stream copies device buffers (itex/core/devices/gpu/gpu_device_plugin.cc:
+ * 251-281, gpu_memcpy_dtod) and is the kernel of known traffic that calibrates the HBM counters */
 int itexhip_memcpy_d2d_async(void* dst_device, const void* src_device, size_t bytes, void* stream);
 
 /* ------------------------------------------------------------------------------------------
@@ -172,7 +172,8 @@ int itexhip_qmatmul_prepare(const itexhip_matmul_params* p, const float* min_b, 
                             float* scales_out, float* bias_out, void* stream);
 
 /* Weight prepack: the s8 weight (TF layout [K,N] row-major, or [N,K] when transpose_b) is
- * rearranged into MFMA operand tiles (16 output channels x 64 k per 1 KiB tile, k zero-padded) and
+ * rearranged into MFMA operand chunks (32 output channels x 32 k per 1 KiB chunk, ordered
+ * [N/32][K/32], K zero-padded to a multiple of 64) and
  * its column sums over k are written to colsum[N].  This replaces the reference's cached weight
  * reorder (quantized_matmul_common.h:238-275) and its host-side column-sum loop (:569-573).
  * `packed` must hold itexhip_qgemm_packed_bytes(K, N) bytes. */
