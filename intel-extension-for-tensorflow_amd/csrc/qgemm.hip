@@ -16,6 +16,8 @@
 // Unsigned activations: the MFMA is signed x signed, so u8 values are fed as (a ^ 0x80) = a - 128 and
 // the epilogue adds 128 * colsum[n] back (exact: |acc| <= 255 * 127 * K stays far below 2^31 for the
 // K this library accepts).
+#include <algorithm>
+
 #include "qgemm_common.hpp"
 
 namespace itexhip {
@@ -63,77 +65,103 @@ __global__ __launch_bounds__(256) void prepack_b_kernel(const int8_t* __restrict
 }
 
 // ------------------------------------------------------------------------------------------------
-// Small-M kernel (M <= 16, bandwidth bound on the weight).  One workgroup owns a 16-channel strip of
-// the weight (half of each 32-channel chunk), so that even N = 4096 gives every CU a workgroup.  Its
-// WAVES wavefronts take pairs of consecutive k-chunks round-robin; one wavefront load fetches the
-// strip's half of a chunk pair (4 runs of 256 contiguous bytes) in the operand layout of the
-// 16x16x64 MFMA: lane l holds channel (l % 16), k-group (l / 16) of the 64 k of the pair.  A batch of
-// UNROLL loads is issued before the first MFMA of the batch.  The partial 16x16 tiles of the
-// wavefronts are added up in LDS with integer atomics (exact, order free).
+// Small-M kernel (M <= 16, bandwidth bound on the weight).  One workgroup owns a strip of SW output
+// channels (32 = whole chunks, or 16 = one half of each chunk when N alone would not give every CU a
+// workgroup); its wavefronts split K into contiguous runs of chunk pairs.  Per chunk pair (64 k) a
+// wavefront issues one activation load (lane l: row l % 16, 16 bytes at k-piece l / 16, i.e. 64
+// contiguous bytes per row) and SW / 16 weight loads in the operand layout of the 16x16x64 MFMA
+// (lane l: channel l % 16, k-group l / 16; 4 runs of 256 contiguous bytes).  A batch of U pairs is
+// issued at once, activations first: loads return in order, so each MFMA waits only for its own
+// operands while the rest of the batch is still in flight.  The partial 16x16 tiles of the wavefronts
+// meet in LDS (one slot per wavefront, one barrier) and wavefront t finishes tile t.
+// Rows >= M of the activation operand repeat row M - 1; their results are never stored.
 // ------------------------------------------------------------------------------------------------
-template <int WAVES, int OUT_T>
-__global__ __launch_bounds__(64 * WAVES) void qgemv_kernel(const uint8_t* __restrict__ a, uint32_t a_xor,
-                                                           const uint8_t* __restrict__ bp, int M, int K,
-                                                           int N, int KC, EpilogueArgs e,
-                                                           void* __restrict__ out) {
-  constexpr int UNROLL = 16;  // weight loads in flight per wavefront
-  __shared__ int red[4 * 64];
-  const int strip = blockIdx.x;  // 16 channels
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+template <int SW, int OUT_T>
+__global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(4, 4))) void qgemv_kernel(const uint8_t* __restrict__ a, uint32_t a_xor,
+                                                     const uint8_t* __restrict__ bp, int M, int K, int N,
+                                                     int KC, int cnt, EpilogueArgs e,
+                                                     void* __restrict__ out) {
+  constexpr int U = 8;         // chunk pairs per batch
+  constexpr int NT = SW / 16;  // 16-channel tiles per strip
+  extern __shared__ int red[];  // [waves][NT][4][64]
+  const int strip = blockIdx.x;
+  const int waves = blockDim.x >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const int lrow = lane & 15, lgrp = lane >> 4;  // k-group 0..3 of the chunk pair
   const int KP = KC >> 1;                         // chunk pairs (K is padded to a multiple of 64)
-  // inside chunk (pair * 2 + lgrp / 2): slot (lgrp % 2) * 32 + (strip % 2) * 16 + lrow
-  const uint8_t* wsrc = bp + (static_cast<int64_t>(strip >> 1) * KC + (lgrp >> 1)) * kChunkBytes +
-                        (((lgrp & 1) * 32 + (strip & 1) * 16 + lrow) << 4);
-  const uint8_t* arow = a + static_cast<int64_t>(lrow) * K + lgrp * 16;
-  const bool row_ok = lrow < M;
+  const int p0 = wave * cnt, p1 = min(KP, p0 + cnt);
+  // inside chunk (pair * 2 + lgrp / 2): slot (lgrp % 2) * 32 + half * 16 + lrow
+  const int chunk_row = (SW == 32) ? strip : (strip >> 1);
+  const int half0 = (SW == 32) ? 0 : (strip & 1);
+  const uint8_t* wsrc = bp + (static_cast<int64_t>(chunk_row) * KC + (lgrp >> 1)) * kChunkBytes +
+                        (((lgrp & 1) * 32 + half0 * 16 + lrow) << 4);
+  const uint8_t* arow = a + static_cast<int64_t>(min(lrow, M - 1)) * K;
+  const int kpiece = lgrp * 16, klast = K - 16;  // k beyond K meets zero weights: any in-bounds data will do
 
-  v4i acc = v4i{0, 0, 0, 0};
-  auto act_piece = [&](int kp) {
-    v4i v = v4i{0, 0, 0, 0};
-    if (row_ok && kp * 64 + lgrp * 16 < K) {
-      v = *reinterpret_cast<const v4i*>(arow + static_cast<int64_t>(kp) * 64);
-      v.x ^= a_xor; v.y ^= a_xor; v.z ^= a_xor; v.w ^= a_xor;
-    }
-    return v;
+  v4i acc[NT];
+#pragma unroll
+  for (int t = 0; t < NT; ++t) acc[t] = v4i{0, 0, 0, 0};
+
+  auto load_act = [&](int p) { return *reinterpret_cast<const v4i*>(arow + min(p * 64 + kpiece, klast)); };
+  auto load_act_inside = [&](int p) { return *reinterpret_cast<const v4i*>(arow + (p * 64 + kpiece)); };
+  auto load_w = [&](int p, int t) {
+    return __builtin_nontemporal_load(
+        reinterpret_cast<const v4i*>(wsrc + static_cast<int64_t>(p) * (2 * kChunkBytes) + t * 256));
   };
-  // batches of up to UNROLL chunk pairs: every weight load of a batch is issued first (the guard is
-  // wavefront uniform), activations are read just before use (they come from L2)
-  for (int kp0 = wave; kp0 < KP; kp0 += UNROLL * WAVES) {
-    v4i w[UNROLL];
+  auto mac = [&](const v4i w, v4i x, int t) {
+    x.x ^= a_xor; x.y ^= a_xor; x.z ^= a_xor; x.w ^= a_xor;
+    acc[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w, x, acc[t], 0, 0, 0);
+  };
+
+  int p = p0;
+  const int p_full = min(p1, K >> 6);  // pairs below this index lie entirely inside K
+  for (; p + U <= p_full; p += U) {  // full batches: straight-line code
+    v4i x[U], w[U][NT];
 #pragma unroll
-    for (int u = 0; u < UNROLL; ++u) {
-      const int kp = kp0 + u * WAVES;
-      w[u] = v4i{0, 0, 0, 0};
-      if (kp < KP)
-        w[u] = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(wsrc + static_cast<int64_t>(kp) * (2 * kChunkBytes)));
-    }
+    for (int u = 0; u < U; ++u) x[u] = load_act_inside(p + u);
 #pragma unroll
-    for (int u = 0; u < UNROLL; ++u) {
-      const int kp = kp0 + u * WAVES;
-      if (kp < KP) acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(w[u], act_piece(kp), acc, 0, 0, 0);
-    }
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int t = 0; t < NT; ++t) w[u][t] = load_w(p + u, t);
+    __builtin_amdgcn_sched_barrier(0);  // keep the whole batch of loads ahead of the first MFMA
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int t = 0; t < NT; ++t) mac(w[u][t], x[u], t);
+  }
+  if (p < p1) {  // last, partial batch: the guards are wavefront uniform
+    v4i x[U], w[U][NT];
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+      if (p + u < p1) x[u] = load_act(p + u);
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+      if (p + u < p1) {
+#pragma unroll
+        for (int t = 0; t < NT; ++t) w[u][t] = load_w(p + u, t);
+      }
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+      if (p + u < p1) {
+#pragma unroll
+        for (int t = 0; t < NT; ++t) mac(w[u][t], x[u], t);
+      }
   }
 
-  // cross-wavefront reduction: wavefront 0 stores, the others add
-  if (wave == 0) {
+  // cross-wavefront reduction
 #pragma unroll
-    for (int r = 0; r < 4; ++r) red[r * 64 + lane] = acc[r];
-  }
+  for (int t = 0; t < NT; ++t)
+    *reinterpret_cast<v4i*>(&red[((wave * NT + t) * 64 + lane) * 4]) = acc[t];
   __syncthreads();
-  if (wave != 0) {
-#pragma unroll
-    for (int r = 0; r < 4; ++r) atomicAdd(&red[r * 64 + lane], acc[r]);
-  }
-  __syncthreads();
-  if (wave == 0 && row_ok) {
+  if (wave < NT) {
+    v4i part = v4i{0, 0, 0, 0};
+    for (int w = 0; w < waves; ++w) part += *reinterpret_cast<const v4i*>(&red[((w * NT + wave) * 64 + lane) * 4]);
     // accumulator layout of the 16x16 MFMA: lane l, register r -> m = l % 16, n = (l / 16) * 4 + r
     const bool vec_ok = (N & 3) == 0 && aligned16(e.scales) && aligned16(e.bias) && aligned16(e.colsum) && aligned16(out);
-    const int n = strip * 16 + lgrp * 4;
-    if (n < N) {
-      const v4i part = v4i{red[lane], red[64 + lane], red[128 + lane], red[192 + lane]};
-      const ChannelParams p = load_channel_params(e, n, N, vec_ok);
-      epilogue_store<OUT_T, 2>(part, p, lrow, n, M, N, e, out, vec_ok);
+    const int n = strip * SW + wave * 16 + lgrp * 4;
+    if (lrow < M && n < N) {
+      const ChannelParams cp = load_channel_params(e, n, N, vec_ok);
+      epilogue_store<OUT_T, 2>(part, cp, lrow, n, M, N, e, out, vec_ok);
     }
   }
 }
@@ -206,19 +234,21 @@ EpilogueArgs make_args(int a_type, const int32_t* colsum, const float* scales, c
 template <int OUT_T>
 int dispatch_gemv(const uint8_t* a, uint32_t a_xor, const uint8_t* bp, int M, int K, int N,
                   const EpilogueArgs& e, void* out, hipStream_t st) {
-  const int KC = 2 * ((K + 63) / 64), strips = (N + 15) / 16;
-  const int KP = KC / 2;
-  // as many wavefronts per strip as it takes for each to own at most ~16 chunk pairs (one batch of
-  // loads), within 16 per workgroup; small problems get fewer
-  const int per16 = (KP + 15) / 16;
-  if (per16 > 8)
-    qgemv_kernel<16, OUT_T><<<strips, 64 * 16, 0, st>>>(a, a_xor, bp, M, K, N, KC, e, out);
-  else if (per16 > 2 || KP >= 64)
-    qgemv_kernel<8, OUT_T><<<strips, 64 * 8, 0, st>>>(a, a_xor, bp, M, K, N, KC, e, out);
-  else if (KP >= 4)
-    qgemv_kernel<4, OUT_T><<<strips, 64 * 4, 0, st>>>(a, a_xor, bp, M, K, N, KC, e, out);
-  else
-    qgemv_kernel<1, OUT_T><<<strips, 64, 0, st>>>(a, a_xor, bp, M, K, N, KC, e, out);
+  const int KC = 2 * ((K + 63) / 64), KP = KC / 2;
+  // wavefronts per strip: about one batch of 8 chunk pairs each, at most 16; prefer a count that
+  // divides K into whole batches
+  int waves = std::min(16, (KP + 7) / 8);
+  for (int w = waves; w >= std::max(1, waves / 2); --w)
+    if (KP % (8 * w) == 0) { waves = w; break; }
+  const int cnt = (KP + waves - 1) / waves;
+  const int strips32 = (N + 31) / 32;
+  if (strips32 >= 256) {
+    const size_t lds = static_cast<size_t>(waves) * 2 * 1024;
+    qgemv_kernel<32, OUT_T><<<strips32, 64 * waves, lds, st>>>(a, a_xor, bp, M, K, N, KC, cnt, e, out);
+  } else {
+    const size_t lds = static_cast<size_t>(waves) * 1024;
+    qgemv_kernel<16, OUT_T><<<(N + 15) / 16, 64 * waves, lds, st>>>(a, a_xor, bp, M, K, N, KC, cnt, e, out);
+  }
   return ITEXHIP_OK;
 }
 
