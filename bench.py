@@ -55,6 +55,28 @@ class Timer:
         torch.cuda.synchronize()
         return start.elapsed_time(stop) / steps  # ms per step
 
+    def run_graph(self, make_fn, steps, warmup):
+        """The same `steps` launches captured once into a HIP graph and replayed: host launch cost
+        leaves the measurement.  `make_fn(stream_handle)` returns fn(i) that launches on that stream."""
+        torch = self.torch
+        graph = torch.cuda.CUDAGraph()
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.graph(graph, stream=side):
+            fn = make_fn(torch.cuda.current_stream().cuda_stream)
+            for i in range(steps):
+                fn(warmup + i)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        start = torch.cuda.Event(enable_timing=True)
+        stop = torch.cuda.Event(enable_timing=True)
+        start.record()
+        graph.replay()
+        stop.record()
+        torch.cuda.synchronize()
+        return start.elapsed_time(stop) / steps
+
 
 def _stream(torch):
     return torch.cuda.current_stream().cuda_stream
@@ -102,7 +124,7 @@ def make_acts(torch, hip, M, K, seed, dev, outlier_frac=0.0, outlier_mult=1.0):
 # ------------------------------------------------------------------------------------------------
 # workloads
 # ------------------------------------------------------------------------------------------------
-def bench_linear(torch, hip, timer, M, K, N, kind, steps, warmup, dev, seed, rotate=1):
+def bench_linear(torch, hip, timer, M, K, N, kind, steps, warmup, dev, seed, rotate=1, graph=False):
     """kind: 'requant_s8' ([BiasAdd, Requantize] -> qint8), 'deq' / 'deq_relu' ([.., Dequantize] -> fp32).
     rotate > 1 cycles through that many distinct weight copies so that the weight stream comes from
     HBM, not from the 256 MiB last-level cache."""
@@ -136,13 +158,23 @@ def bench_linear(torch, hip, timer, M, K, N, kind, steps, warmup, dev, seed, rot
         L = layers[i % rotate]
         hip.qgemm(xq, hip.QUINT8, L["packed"], L["colsum"], M, K, N, L["scales"], L["sbias"], ep, t_out, out, st)
 
+    def make_graph_fn(stream):
+        def fn(i):
+            L = layers[i % rotate]
+            hip.qgemm(xq, hip.QUINT8, L["packed"], L["colsum"], M, K, N, L["scales"], L["sbias"], ep, t_out, out, stream)
+        return fn
+
     ms_step = timer.run(step, steps, warmup)
     ms_kernel = timer.run(gemm_only, steps, warmup)
+    ms_graph = timer.run_graph(make_graph_fn, steps, warmup) if graph else None
     ops = 2.0 * M * N * K
     nbytes = M * K + K * N + out_bytes * M * N + 8 * N
     res = dict(M=M, K=K, N=N, kind=kind, ms_per_step=ms_step, us_kernel=ms_kernel * 1e3,
                tops=ops / (ms_step * 1e-3) / 1e12, tops_kernel=ops / (ms_kernel * 1e-3) / 1e12,
                gbs_kernel=nbytes / (ms_kernel * 1e-3) / 1e9, ops=ops, bytes=nbytes)
+    if ms_graph is not None:
+        res.update(us_kernel_graph=ms_graph * 1e3, gbs_kernel_graph=nbytes / (ms_graph * 1e-3) / 1e9,
+                   tops_kernel_graph=ops / (ms_graph * 1e-3) / 1e12)
     res["_ctx"] = dict(layers=layers, xq=xq, p=p, min_a=min_a, max_a=max_a)
     return res
 
@@ -266,7 +298,7 @@ def main():
     if "bert" in only:
         for (k, n, kind, seed) in ((768, 2304, "deq", 1), (768, 768, "deq", 2), (768, 3072, "deq_relu", 3),
                                    (3072, 768, "deq", 4)):
-            r = bench_linear(torch, hip, timer, 4096, k, n, kind, K_steps, W, dev, seed)
+            r = bench_linear(torch, hip, timer, 4096, k, n, kind, K_steps, W, dev, seed, graph=True)
             r.pop("_ctx")
             t_roof = max(r["ops"] / (PEAK_INT8_TOPS * 1e12), r["bytes"] / (PEAK_HBM_GBS * 1e9))
             r.update(name="bert_linear", bound="max(mfma,hbm)", frac=t_roof / (r["us_kernel"] * 1e-6),
@@ -275,9 +307,10 @@ def main():
     if "gemv" in only:
         for (k, n) in ((4096, 14336), (14336, 4096)):
             for m in (1, 4, 16):
-                r = bench_linear(torch, hip, timer, m, k, n, "deq", K_steps, W, dev, seed=10, rotate=8)
+                r = bench_linear(torch, hip, timer, m, k, n, "deq", K_steps, W, dev, seed=10, rotate=8, graph=True)
                 r.pop("_ctx")
                 r.update(name="decode_gemv", bound="hbm", frac=r["gbs_kernel"] / PEAK_HBM_GBS,
+                         frac_graph=r["gbs_kernel_graph"] / PEAK_HBM_GBS,
                          note="8 weight copies cycled (470 MB > last-level cache)")
                 others.append(r)
     if "copy" in only:

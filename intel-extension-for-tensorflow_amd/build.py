@@ -28,7 +28,7 @@ HIP_FLAGS = [
     "-fno-fast-math", "-fno-gpu-flush-denormals-to-zero",
     # no packed-fp32 instructions in device code
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-    "-Wall", "-Wno-unused-function", "-I", INCLUDE, "-I", CSRC,
+    "-Wall", "-Wno-unused-function", "-Wno-inline-asm", "-I", INCLUDE, "-I", CSRC,
 ]
 CXX = os.environ.get("CXX", "g++")
 CXX_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-ffp-contract=off", "-fno-fast-math", "-Wall", "-I", INCLUDE,

@@ -90,13 +90,13 @@ __device__ __forceinline__ ChannelParams load_channel_params(const EpilogueArgs&
 // rounds to nearest even and leaves the integer in the low mantissa bits (two's complement for
 // negatives), so the low byte of the sum is the result: one add instead of round + convert.
 template <int OUT_T, int ACT>
-__device__ __forceinline__ v4i epilogue_convert(const v4i acc, const ChannelParams& p, const EpilogueArgs& e) {
+__device__ __forceinline__ v4i epilogue_convert(const v4i acc, const f4 scale, const f4 bias, const EpilogueArgs& e) {
   float y[4];
 #pragma unroll
   for (int r = 0; r < 4; ++r) {
-    float v = static_cast<float>(acc[r] + p.comp[r]);
-    v = v * p.scale[r];
-    if (e.bias) v = v + p.bias[r];
+    float v = static_cast<float>(acc[r]);  // the zero-point compensation is already part of acc
+    v = v * scale[r];
+    v = v + bias[r];
     if (ACT == 1) {
       v = fmaxf(v, 0.0f);
     } else if (ACT == 2) {
@@ -113,7 +113,7 @@ __device__ __forceinline__ v4i epilogue_convert(const v4i acc, const ChannelPara
     uint32_t b[4];
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
-      float v = fminf(fmaxf(y[r], Sat<OUT_T>::lo), Sat<OUT_T>::hi);
+      const float v = __builtin_amdgcn_fmed3f(y[r], Sat<OUT_T>::lo, Sat<OUT_T>::hi);  // clamp in one instruction
       b[r] = static_cast<uint32_t>(__float_as_int(v + 12582912.0f));
     }
     // bytes: result = {b0.byte0, b1.byte0, b2.byte0, b3.byte0}; v_perm selects from {hi operand bytes 4..7, lo 0..3}

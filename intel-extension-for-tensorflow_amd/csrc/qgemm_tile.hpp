@@ -73,6 +73,12 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void qgemm_tile_kernel(
   static_assert(NSLICE % 2 == 0, "slices come in two halves");
   constexpr int STAGE_BYTES = (A_LOADS + B_LOADS) * kChunkBytes;
   constexpr int B_REGION = A_LOADS * kChunkBytes;
+  // behind the ring: the per-channel epilogue parameters of this block's BN channels
+  constexpr int PANEL_OFF = NSTAGE * STAGE_BYTES;
+  // the element-wise (any alignment, any N, optional bias) epilogue is only compiled into the
+  // conservative instantiation; the host sends such calls there
+  constexpr bool GENERAL = (ACT == 2) && !KALIGNED;
+  static_assert(BN <= 64 * NW, "one thread per channel fills the parameter panel");
 
   extern __shared__ __align__(16) uint8_t lds[];
   const uint32_t lds_base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(
@@ -91,10 +97,9 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void qgemm_tile_kernel(
   const int lrow = lane & 31, lgrp = lane >> 5;
 
   v16i acc[TN * TM];
-  static_for<TN * TM>([&](auto t) {
-#pragma unroll
-    for (int r = 0; r < 16; ++r) acc[t][r] = 0;
-  });
+  int* const panel_comp = reinterpret_cast<int*>(lds + PANEL_OFF);
+  float* const panel_scale = reinterpret_cast<float*>(lds + PANEL_OFF + BN * 4);
+  float* const panel_bias = reinterpret_cast<float*>(lds + PANEL_OFF + BN * 8);
 
   // ---- staging sources of this wavefront
   // activation load `ld` covers rows [16*h, 16*h+16) of 32-row tile rt: lane -> (row q, piece p)
@@ -149,8 +154,27 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void qgemm_tile_kernel(
   static_for<NLD>([&](auto c) { issue_load(c, 0, 0); });
   static_for<NLD>([&](auto c) { issue_load(c, min(1, KT - 1), 1); });
   static_for<NLD>([&](auto c) { issue_load(c, min(2, KT - 1), 2); });
+  // parameter panel: thread t resolves channel n_base + t once (the flags are uniform), so the
+  // epilogue is free of global loads and of branches on them
+  if (threadIdx.x < BN) {
+    const int n = min(n_base + static_cast<int>(threadIdx.x), N - 1);
+    panel_comp[threadIdx.x] = e.comp_mul ? e.comp_mul * e.colsum[n] : 0;
+    panel_scale[threadIdx.x] = e.n_scales > 1 ? e.scales[n] : (e.n_scales == 1 ? e.scales[0] : 1.0f);
+    panel_bias[threadIdx.x] = e.bias ? e.bias[n] : 0.0f;
+  }
   wait_vmcnt<NLD>();
   __syncthreads();
+  // the accumulators start from the zero-point compensation of their channel (exact in int32)
+  static_for<TN>([&](auto j) {
+    static_for<4>([&](auto g) {
+      const v4i c = *reinterpret_cast<const v4i*>(panel_comp + (wn * TN + decltype(j)::value) * 32 + decltype(g)::value * 8 + lgrp * 4);
+      static_for<TM>([&](auto i) {
+        constexpr int t = decltype(j)::value * TM + decltype(i)::value;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) acc[t][decltype(g)::value * 4 + r] = c[r];
+      });
+    });
+  });
 
   // weight fragments rotate through FBN registers sets and are read FBD slices ahead of their use
   constexpr int FBD = (NSLICE >= 4) ? 2 : 1;
@@ -237,8 +261,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void qgemm_tile_kernel(
   constexpr int LPR = ROWB / 16;             // lanes per row when flushing
   constexpr int RPP = 64 / LPR;              // rows per flush instruction
   static_assert(NW * WM * PITCH <= NSTAGE * STAGE_BYTES, "epilogue buffer must fit in the ring");
-  const bool vec_ok = (N & 3) == 0 && aligned16(e.scales) && aligned16(e.bias) && aligned16(e.colsum) && aligned16(out);
-  const bool fast = vec_ok && ((static_cast<int64_t>(N) * ESZ) & 15) == 0;
+  const bool fast = !GENERAL || (e.bias != nullptr && aligned16(out) && ((static_cast<int64_t>(N) * ESZ) & 15) == 0);
   if (fast) {
     uint8_t* ebuf = lds + wave * (WM * PITCH);
     const int f_row = lane / LPR, f_piece = lane % LPR;
@@ -246,13 +269,14 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void qgemm_tile_kernel(
       static_for<JB>([&](auto jj) {
         constexpr int j = decltype(jb)::value * JB + decltype(jj)::value;
         static_for<4>([&](auto g) {
-          const int n = n_base + (wn * TN + j) * 32 + decltype(g)::value * 8 + lgrp * 4;
-          const ChannelParams p = load_channel_params(e, min(n, N - 4), N, true);
+          const int col = (wn * TN + j) * 32 + decltype(g)::value * 8 + lgrp * 4;
+          const f4 sc = *reinterpret_cast<const f4*>(panel_scale + col);
+          const f4 bi = *reinterpret_cast<const f4*>(panel_bias + col);
           static_for<TM>([&](auto i) {
             constexpr int t = j * TM + decltype(i)::value;
             constexpr int r0 = decltype(g)::value * 4;
             const v4i part = v4i{acc[t][r0], acc[t][r0 + 1], acc[t][r0 + 2], acc[t][r0 + 3]};
-            const v4i o = epilogue_convert<OUT_T, ACT>(part, p, e);
+            const v4i o = epilogue_convert<OUT_T, ACT>(part, sc, bi, e);
             uint8_t* dst = ebuf + (decltype(i)::value * 32 + lrow) * PITCH +
                            (decltype(jj)::value * 32 + decltype(g)::value * 8 + lgrp * 4) * ESZ;
             if constexpr (ESZ == 1) *reinterpret_cast<int*>(dst) = o.x;
@@ -271,18 +295,33 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void qgemm_tile_kernel(
           *reinterpret_cast<v4i*>(reinterpret_cast<uint8_t*>(out) + (static_cast<int64_t>(m) * N + n_col) * ESZ) = v;
       }
     });
-  } else {
+  } else if constexpr (GENERAL) {
+    const bool has_bias = e.bias != nullptr;
     static_for<TN>([&](auto j) {
       static_for<4>([&](auto g) {
-        const int n = n_base + (wn * TN + j) * 32 + decltype(g)::value * 8 + lgrp * 4;
+        const int col = (wn * TN + j) * 32 + decltype(g)::value * 8 + lgrp * 4;
+        const int n = n_base + col;
         if (n < N) {
-          const ChannelParams p = load_channel_params(e, n, N, vec_ok);
+          const f4 sc = *reinterpret_cast<const f4*>(panel_scale + col);
+          const f4 bi = *reinterpret_cast<const f4*>(panel_bias + col);
           static_for<TM>([&](auto i) {
             constexpr int t = decltype(j)::value * TM + decltype(i)::value;
             constexpr int r0 = decltype(g)::value * 4;
             const int m = m_base + (wm * TM + i) * 32 + lrow;
-            const v4i part = v4i{acc[t][r0], acc[t][r0 + 1], acc[t][r0 + 2], acc[t][r0 + 3]};
-            epilogue_store<OUT_T, ACT>(part, p, m, n, M, N, e, out, vec_ok);
+            if (m < M) {
+#pragma unroll
+              for (int r = 0; r < 4; ++r) {
+                if (n + r < N) {
+                  float v = static_cast<float>(acc[t][r0 + r]) * sc[r];
+                  if (has_bias) v = v + bi[r];
+                  for (int k = 0; k < e.n_eltwise; ++k) v = apply_eltwise(e.elt[k], v);
+                  const int64_t o = static_cast<int64_t>(m) * N + n + r;
+                  if constexpr (OUT_T == ITEXHIP_FLOAT) reinterpret_cast<float*>(out)[o] = v;
+                  else if constexpr (OUT_T == ITEXHIP_QINT32) reinterpret_cast<int32_t*>(out)[o] = sat_rne<ITEXHIP_QINT32>(v);
+                  else reinterpret_cast<uint8_t*>(out)[o] = static_cast<uint8_t>(sat_rne<OUT_T>(v));
+                }
+              }
+            }
           });
         }
       });
@@ -295,7 +334,7 @@ int launch_tile(const uint8_t* a, const uint8_t* bp, int M, int K, int N, const 
                 hipStream_t st) {
   const int KT = (K + 63) / 64, NT = (N + kChunkRows - 1) / kChunkRows;
   const int num_m = (M + BM - 1) / BM, num_n = (N + BN - 1) / BN;
-  constexpr size_t lds_bytes = 4 * (BM / 16 + BN / 16) * kChunkBytes;
+  constexpr size_t lds_bytes = 4 * (BM / 16 + BN / 16) * kChunkBytes + 12 * BN;
   auto kern = qgemm_tile_kernel<BM, BN, WAVES_M, WAVES_N, OUT_T, ACT, FLIP, KALIGNED>;
   static bool attr_set = false;  // benign race: the call is idempotent
   if (!attr_set) {
@@ -327,7 +366,11 @@ template <int OUT_T>
 int dispatch_tile(const uint8_t* a, uint32_t a_xor, const uint8_t* bp, int M, int K, int N,
                   const EpilogueArgs& e, void* out, hipStream_t st) {
   const bool flip = a_xor != 0;
-  const bool kal = (K & 63) == 0;
+  constexpr int esz = (OUT_T == ITEXHIP_QINT8 || OUT_T == ITEXHIP_QUINT8) ? 1 : 4;
+  // the specialised kernels only carry the vectorised epilogue: bias present, output rows 16-byte aligned
+  const bool plain = e.bias != nullptr && (reinterpret_cast<uintptr_t>(out) & 15) == 0 &&
+                     ((static_cast<int64_t>(N) * esz) & 15) == 0;
+  const bool kal = (K & 63) == 0 && plain;
   const int act = e.n_eltwise == 0 ? 0
                   : (e.n_eltwise == 1 && e.elt[0].alg == ITEXHIP_ELT_RELU && e.elt[0].alpha == 0.0f) ? 1 : 2;
 #define ITEXHIP_TILE_CASE(A, F, KA) \
