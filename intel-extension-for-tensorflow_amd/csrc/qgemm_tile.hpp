@@ -3,6 +3,9 @@
 #ifndef ITEXHIP_QGEMM_TILE_HPP_
 #define ITEXHIP_QGEMM_TILE_HPP_
 
+#include <cmath>
+#include <cstdlib>
+
 #include "qgemm_common.hpp"
 
 namespace itexhip {
@@ -53,11 +56,13 @@ __device__ __forceinline__ void wait_vmcnt() {
   __builtin_amdgcn_s_waitcnt((N & 15) | (7 << 4) | (15 << 8) | ((N >> 4) << 14));
 }
 
-// FLIP: activations are unsigned (fed as x ^ 0x80).  KALIGNED: K is a multiple of 64, so activation
-// loads never need a per-lane clamp and use a uniform base that advances by 64 bytes per step.
-template <int BM, int BN, int WAVES_M, int WAVES_N, int OUT_T, int ACT, bool FLIP, bool KALIGNED>
+// amask: 0x80808080 when the activations are unsigned (they are fed as x ^ 0x80), else 0; a scalar
+// register operand, so the sign flip costs a 4-byte instruction per dword.  KALIGNED: K is a multiple
+// of 64, so activation loads never need a per-lane clamp and use a uniform base that advances by 64
+// bytes per step.
+template <int BM, int BN, int WAVES_M, int WAVES_N, int OUT_T, int ACT, bool KALIGNED>
 __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void qgemm_tile_kernel(
-    const uint8_t* __restrict__ a, const uint8_t* __restrict__ bp, int M, int K, int N,
+    const uint8_t* __restrict__ a, uint32_t amask, const uint8_t* __restrict__ bp, int M, int K, int N,
     int KT, int NT, int num_m, int num_n, EpilogueArgs e, void* __restrict__ out) {
   constexpr int NW = WAVES_M * WAVES_N;
   constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
@@ -143,7 +148,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void qgemm_tile_kernel(
     return *reinterpret_cast<const v4i*>(lds + stage * STAGE_BYTES + (wm * TM + i) * (2 * kChunkBytes) + frag_a_lane[kc]);
   };
   auto flip = [&](v4i v) {  // u8 -> s8 (x - 128) for unsigned activations, identity for signed ones
-    if constexpr (FLIP) { v.x ^= 0x80808080; v.y ^= 0x80808080; v.z ^= 0x80808080; v.w ^= 0x80808080; }
+    v.x ^= amask; v.y ^= amask; v.z ^= amask; v.w ^= amask;
     return v;
   };
   auto lds_b = [&](int stage, int kc, int j) {
@@ -177,8 +182,8 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void qgemm_tile_kernel(
   });
 
   // weight fragments rotate through FBN registers sets and are read FBD slices ahead of their use
-  constexpr int FBD = (NSLICE >= 4) ? 2 : 1;
-  constexpr int FBN = (NSLICE >= 4) ? 4 : 2;
+  constexpr int FBD = (NSLICE % 4 == 0) ? 2 : 1;
+  constexpr int FBN = (NSLICE % 4 == 0) ? 4 : 2;
   static_assert(NSLICE % FBN == 0, "the weight fragment rotation must close over a step");
   v4i fa0[2 * TM], fa1[2 * TM], fb[FBN];
   static_for<2 * TM>([&](auto x) { fa0[x] = lds_a_raw(0, decltype(x)::value / TM, decltype(x)::value % TM); });
@@ -196,8 +201,6 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void qgemm_tile_kernel(
   // activation fragments of the next step, the last slot issues one global->LDS load.
   // The two activation fragment sets swap roles from step to step (loop unrolled by two).
   constexpr int FA = 2 * TM;                       // activation fragments per step
-  constexpr int FA_PER_SLICE = (FA + NSLICE / 2 - 1) / (NSLICE / 2);
-  static_assert(FA_PER_SLICE + 2 <= TM || TM < 4, "slots per slice");
   auto step = [&](int kt, const v4i (&fa_cur)[FA], v4i (&fa_nxt)[FA]) {
     const int st_cur = kt & 3, st_nxt = (kt + 1) & 3, st_fill = (kt + 3) & 3;
     const int kt_load = min(kt + 3, KT - 1);
@@ -219,16 +222,23 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void qgemm_tile_kernel(
             if constexpr (decltype(c)::value * NSLICE / NLD == s) issue_load(c, kt_load, st_fill);
           });
         }
-        if constexpr ((TM < 3) ? (ii == 0) : (ii >= 1 && ii <= FA_PER_SLICE)) {
-          constexpr int slot = (TM < 3) ? 0 : ii - 1;
-          constexpr int per = (TM < 3) ? FA_PER_SLICE : 1;
-          static_for<per>([&](auto u) {
-            constexpr int x = (s % (NSLICE / 2)) * FA_PER_SLICE + slot * per + decltype(u)::value;
-            if constexpr (x < FA) {
-              if constexpr (s < NSLICE / 2) fa_nxt[x] = lds_a_raw(st_nxt, x / TM, x % TM);
-              else fa_nxt[x] = flip(fa_nxt[x]);
-            }
-          });
+        // activation fragments of the next step: read during the first half of the slices, sign
+        // flipped (dword by dword) during the second half, spread evenly over the MFMA slots
+        {
+          constexpr int HALF = NSLICE / 2, Q = HALF * TM;  // slots per half
+          constexpr int q = (s % HALF) * TM + ii;          // this slot's index inside its half
+          constexpr int shift = (Q >= 2 * FA) ? 1 : 0;     // keep clear of the weight-fragment slot when there is room
+          if constexpr (s < HALF) {
+            static_for<FA>([&](auto x) {
+              if constexpr (decltype(x)::value * Q / FA + shift == q)
+                fa_nxt[decltype(x)::value] = lds_a_raw(st_nxt, decltype(x)::value / TM, decltype(x)::value % TM);
+            });
+          } else {
+            static_for<4 * FA>([&](auto d) {
+              if constexpr (decltype(d)::value * Q / (4 * FA) == q)
+                fa_nxt[decltype(d)::value / 4][decltype(d)::value % 4] ^= amask;
+            });
+          }
         }
         __builtin_amdgcn_sched_barrier(0);
       });
@@ -259,7 +269,8 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void qgemm_tile_kernel(
   constexpr int ROWB = JB * 32 * ESZ;        // row bytes in the buffer
   constexpr int PITCH = ROWB + 16;
   constexpr int LPR = ROWB / 16;             // lanes per row when flushing
-  constexpr int RPP = 64 / LPR;              // rows per flush instruction
+  constexpr int RPP = 64 / LPR;              // rows per flush instruction (lanes >= RPP * LPR idle)
+  constexpr int PASSES = (WM + RPP - 1) / RPP;
   static_assert(NW * WM * PITCH <= NSTAGE * STAGE_BYTES, "epilogue buffer must fit in the ring");
   const bool fast = !GENERAL || (e.bias != nullptr && aligned16(out) && ((static_cast<int64_t>(N) * ESZ) & 15) == 0);
   if (fast) {
@@ -287,11 +298,12 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void qgemm_tile_kernel(
       // flush: lane -> (row, 16-byte piece); LDS operations of one wavefront complete in order
       const int n_col = n_base + (wn * TN + decltype(jb)::value * JB) * 32 + f_piece * (16 / ESZ);
 #pragma unroll
-      for (int pass = 0; pass < WM / RPP; ++pass) {
-        const int row = pass * RPP + f_row;
+      for (int pass = 0; pass < PASSES; ++pass) {
+        const int row = min(pass * RPP + f_row, WM - 1);
         const v4i v = *reinterpret_cast<const v4i*>(ebuf + row * PITCH + f_piece * 16);
         const int m = m_base + wm * WM + row;
-        if (m < M && n_col < N)  // N * ESZ is a multiple of 16, so a piece is entirely inside or outside
+        const bool mine = (64 % LPR == 0 || f_row < RPP) && (WM % RPP == 0 || pass * RPP + f_row < WM);
+        if (mine && m < M && n_col < N)  // N * ESZ is a multiple of 16, so a piece is entirely inside or outside
           *reinterpret_cast<v4i*>(reinterpret_cast<uint8_t*>(out) + (static_cast<int64_t>(m) * N + n_col) * ESZ) = v;
       }
     });
@@ -329,13 +341,13 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void qgemm_tile_kernel(
   }
 }
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, int OUT_T, int ACT, bool FLIP, bool KALIGNED>
-int launch_tile(const uint8_t* a, const uint8_t* bp, int M, int K, int N, const EpilogueArgs& e, void* out,
-                hipStream_t st) {
+template <int BM, int BN, int WAVES_M, int WAVES_N, int OUT_T, int ACT, bool KALIGNED>
+int launch_tile(const uint8_t* a, uint32_t amask, const uint8_t* bp, int M, int K, int N, const EpilogueArgs& e,
+                void* out, hipStream_t st) {
   const int KT = (K + 63) / 64, NT = (N + kChunkRows - 1) / kChunkRows;
   const int num_m = (M + BM - 1) / BM, num_n = (N + BN - 1) / BN;
   constexpr size_t lds_bytes = 4 * (BM / 16 + BN / 16) * kChunkBytes + 12 * BN;
-  auto kern = qgemm_tile_kernel<BM, BN, WAVES_M, WAVES_N, OUT_T, ACT, FLIP, KALIGNED>;
+  auto kern = qgemm_tile_kernel<BM, BN, WAVES_M, WAVES_N, OUT_T, ACT, KALIGNED>;
   static bool attr_set = false;  // benign race: the call is idempotent
   if (!attr_set) {
     hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -344,44 +356,59 @@ int launch_tile(const uint8_t* a, const uint8_t* bp, int M, int K, int N, const 
     attr_set = true;
   }
   kern<<<dim3(static_cast<unsigned>(num_m * num_n)), dim3(64 * WAVES_M * WAVES_N), lds_bytes, st>>>(
-      a, bp, M, K, N, KT, NT, num_m, num_n, e, out);
+      a, amask, bp, M, K, N, KT, NT, num_m, num_n, e, out);
   return ITEXHIP_OK;
 }
 
-template <int OUT_T, int ACT, bool FLIP, bool KALIGNED>
-int dispatch_tile_shape(const uint8_t* a, const uint8_t* bp, int M, int K, int N, const EpilogueArgs& e, void* out,
-                        hipStream_t st) {
-  // pick the largest tile that still gives every CU work
-  const int64_t tiles_256 = static_cast<int64_t>((M + 255) / 256) * ((N + 255) / 256);
-  const int64_t tiles_128 = static_cast<int64_t>((M + 127) / 128) * ((N + 127) / 128);
-  if (tiles_256 >= 256) return launch_tile<256, 256, 2, 2, OUT_T, ACT, FLIP, KALIGNED>(a, bp, M, K, N, e, out, st);
-  if (tiles_128 >= 256) return launch_tile<128, 128, 2, 2, OUT_T, ACT, FLIP, KALIGNED>(a, bp, M, K, N, e, out, st);
-  return launch_tile<64, 64, 2, 2, OUT_T, ACT, FLIP, KALIGNED>(a, bp, M, K, N, e, out, st);
+// Tile shape: the one with the smallest estimated time = rounds of workgroups over the 256 CUs x
+// tile area x a penalty for the operand traffic per MFMA of smaller tiles.
+inline int pick_tile_shape(int M, int N, bool wide_only) {
+  struct Shape { int bm, bn; double penalty; };
+  static const Shape shapes[5] = {{256, 256, 1.0}, {256, 192, 1.03}, {256, 128, 1.08}, {128, 128, 1.2}, {64, 64, 1.8}};
+  // ITEXHIP_TILE_SHAPE=0..4 forces a shape (tests exercise every shape on ragged problems with it)
+  if (const char* forced = std::getenv("ITEXHIP_TILE_SHAPE")) {
+    const int f = std::atoi(forced);
+    if (f >= (wide_only ? 3 : 0) && f < 5) return f;
+  }
+  int best = 3;
+  double best_cost = 1e300;
+  for (int i = wide_only ? 3 : 0; i < 5; ++i) {
+    const double tiles = static_cast<double>((M + shapes[i].bm - 1) / shapes[i].bm) * ((N + shapes[i].bn - 1) / shapes[i].bn);
+    const double rounds = std::ceil(tiles / 256.0);
+    const double cost = rounds * shapes[i].bm * shapes[i].bn * shapes[i].penalty;
+    if (cost < best_cost) { best_cost = cost; best = i; }
+  }
+  return best;
 }
 
-// The generic eltwise chain and K not a multiple of 64 are rare: they share the conservative
-// instantiation (run-time eltwise chain, per-lane clamped activation loads) to keep the number of
-// kernels down.
+template <int OUT_T, int ACT>
+int dispatch_tile_shape(const uint8_t* a, uint32_t amask, const uint8_t* bp, int M, int K, int N,
+                        const EpilogueArgs& e, void* out, hipStream_t st) {
+  switch (pick_tile_shape(M, N, false)) {
+    case 0: return launch_tile<256, 256, 2, 2, OUT_T, ACT, true>(a, amask, bp, M, K, N, e, out, st);
+    case 1: return launch_tile<256, 192, 2, 2, OUT_T, ACT, true>(a, amask, bp, M, K, N, e, out, st);
+    case 2: return launch_tile<256, 128, 2, 2, OUT_T, ACT, true>(a, amask, bp, M, K, N, e, out, st);
+    case 3: return launch_tile<128, 128, 2, 2, OUT_T, ACT, true>(a, amask, bp, M, K, N, e, out, st);
+    default: return launch_tile<64, 64, 2, 2, OUT_T, ACT, true>(a, amask, bp, M, K, N, e, out, st);
+  }
+}
+
+// The generic eltwise chain, K not a multiple of 64, a missing bias and unaligned outputs are rare:
+// they share the conservative instantiation (run-time eltwise chain, per-lane clamped activation
+// loads, element-wise stores when needed), in two tile shapes only, to keep the number of kernels down.
 template <int OUT_T>
 int dispatch_tile(const uint8_t* a, uint32_t a_xor, const uint8_t* bp, int M, int K, int N,
                   const EpilogueArgs& e, void* out, hipStream_t st) {
-  const bool flip = a_xor != 0;
   constexpr int esz = (OUT_T == ITEXHIP_QINT8 || OUT_T == ITEXHIP_QUINT8) ? 1 : 4;
   // the specialised kernels only carry the vectorised epilogue: bias present, output rows 16-byte aligned
   const bool plain = e.bias != nullptr && (reinterpret_cast<uintptr_t>(out) & 15) == 0 &&
-                     ((static_cast<int64_t>(N) * esz) & 15) == 0;
-  const bool kal = (K & 63) == 0 && plain;
+                     ((static_cast<int64_t>(N) * esz) & 15) == 0 && (K & 63) == 0;
   const int act = e.n_eltwise == 0 ? 0
                   : (e.n_eltwise == 1 && e.elt[0].alg == ITEXHIP_ELT_RELU && e.elt[0].alpha == 0.0f) ? 1 : 2;
-#define ITEXHIP_TILE_CASE(A, F, KA) \
-  if (act == A && flip == F && kal == KA) return dispatch_tile_shape<OUT_T, A, F, KA>(a, bp, M, K, N, e, out, st);
-  ITEXHIP_TILE_CASE(0, true, true)
-  ITEXHIP_TILE_CASE(1, true, true)
-  ITEXHIP_TILE_CASE(0, false, true)
-  ITEXHIP_TILE_CASE(1, false, true)
-#undef ITEXHIP_TILE_CASE
-  if (flip) return dispatch_tile_shape<OUT_T, 2, true, false>(a, bp, M, K, N, e, out, st);
-  return dispatch_tile_shape<OUT_T, 2, false, false>(a, bp, M, K, N, e, out, st);
+  if (plain && act == 0) return dispatch_tile_shape<OUT_T, 0>(a, a_xor, bp, M, K, N, e, out, st);
+  if (plain && act == 1) return dispatch_tile_shape<OUT_T, 1>(a, a_xor, bp, M, K, N, e, out, st);
+  if (pick_tile_shape(M, N, true) == 3) return launch_tile<128, 128, 2, 2, OUT_T, 2, false>(a, a_xor, bp, M, K, N, e, out, st);
+  return launch_tile<64, 64, 2, 2, OUT_T, 2, false>(a, a_xor, bp, M, K, N, e, out, st);
 }
 
 }  // namespace itexhip

@@ -185,6 +185,25 @@ def test_tile_kernel_vs_oracle(hip, dev, M, K, N, kw):
     np.testing.assert_array_equal(got, ref)
 
 
+@pytest.mark.parametrize("shape", [0, 1, 2, 3, 4])
+@pytest.mark.parametrize("M,K,N,kw", [(300, 448, 528, V2_REQ_S8), (513, 192, 400, V2_DEQ_RELU), (257, 64, 208, V1_S32),
+                                      (40, 1024, 96, V2_REQ_U8_RELU), (256, 320, 200, V2_REQ_S8)])
+def test_every_tile_shape_on_ragged_problems(hip, dev, monkeypatch, shape, M, K, N, kw):
+    """The tile shape is normally chosen from the problem size; ITEXHIP_TILE_SHAPE forces one, so that
+    every shape (256x256, 256x192, 256x128, 128x128, 64x64) meets partial tiles in M and N, odd step
+    counts, K not a multiple of 64 and the element-wise store path (N * element size not a multiple of 16)."""
+    import os
+    monkeypatch.setenv("ITEXHIP_TILE_SHAPE", str(shape))
+    assert os.environ["ITEXHIP_TILE_SHAPE"] == str(shape)
+    layer, w, bias = make_layer(hip, dev, K, N, seed=K + N + shape)
+    x, xq, mn, mx = make_acts(M, K, seed=M)
+    r_out = float(np.abs(np.maximum(x @ w + bias, 0) if kw.get("activation") else x @ w + bias).max())
+    lo = 0.0 if kw["t_out"] == orc.QUINT8 else -r_out
+    ref = layer.oracle(xq, kw, mn, mx, lo, r_out)
+    got = layer.run(xq, kw, mn, mx, lo, r_out, path="tile")
+    np.testing.assert_array_equal(got, ref)
+
+
 @pytest.mark.parametrize("M", [1, 2, 4, 7, 16])
 @pytest.mark.parametrize("K,N", [(64, 16), (256, 100), (4096, 512), (1024, 4096), (8192, 48)])
 @pytest.mark.parametrize("kw", [V2_DEQ, V2_REQ_S8])
