@@ -197,6 +197,15 @@ int itexhip_qgemv(const void* a, int a_type, const int8_t* packed_b, const int32
                   int64_t M, int64_t K, int64_t N, const float* scales, const float* bias,
                   const itexhip_epilogue* ep, int out_type, void* out, void* stream);
 
+/* The whole op in one launch: as itexhip_qmatmul_prepare followed by itexhip_qgemm, but the MatMul
+ * kernel derives each channel's output scale and bias itself from the op's ranges (the same fp32
+ * operation sequence), so no parameter vectors and no second kernel are needed.  This is what the
+ * op kernel calls per Compute (quantized_matmul_common.h:62-460: Init + primitive execute);
+ * a changed min_a / max_a costs nothing extra.  `bias` is the op's raw fp32 bias (may be null). */
+int itexhip_qmatmul(const itexhip_matmul_params* p, const void* a, const int8_t* packed_b,
+                    const int32_t* colsum, int64_t M, int64_t K, int64_t N, const float* min_b,
+                    const float* max_b, int64_t nb, const float* bias, void* out, void* stream);
+
 /* Same contract on the unpacked TF-layout weight, any shape (no alignment requirements): one
  * thread per output element.  Used for shapes the tile kernels do not cover (K not a multiple of
  * 16) and as an on-device cross-check. */

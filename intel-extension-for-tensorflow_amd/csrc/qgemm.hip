@@ -260,19 +260,15 @@ int dispatch_gemv(const uint8_t* a, uint32_t a_xor, const uint8_t* bp, int M, in
     default: st__ = CALL(ITEXHIP_QUINT8); break;                              \
   }
 
-int packed_path(bool gemv, const void* a, int a_type, const int8_t* packed_b, const int32_t* colsum,
-                int64_t M, int64_t K, int64_t N, const float* scales, const float* bias,
-                const itexhip_epilogue* ep, int out_type, void* out, void* stream, const char* who) {
-  if (int st = check_common(a, a_type, packed_b, M, K, N, scales, ep, out_type, out, who)) return st;
-  if (M == 0 || N == 0) return ITEXHIP_OK;
+int launch_packed(bool gemv, const void* a, int a_type, const int8_t* packed_b, int64_t M, int64_t K, int64_t N,
+                  const EpilogueArgs& e, int out_type, void* out, void* stream, const char* who) {
   ITEXHIP_REQUIRE(K % 16 == 0, "%s: K must be a multiple of 16 (got %lld); use itexhip_qgemm_naive", who,
                   static_cast<long long>(K));
   ITEXHIP_REQUIRE(aligned(a, 16) && aligned(packed_b, 16), "%s: operands must be 16-byte aligned", who);
-  ITEXHIP_REQUIRE(a_type != ITEXHIP_QUINT8 || colsum, "%s: quint8 activations need colsum", who);
+  ITEXHIP_REQUIRE(a_type != ITEXHIP_QUINT8 || e.colsum, "%s: quint8 activations need colsum", who);
   ITEXHIP_REQUIRE(!gemv || M <= 16, "%s: M must be <= 16", who);
   ITEXHIP_REQUIRE(M * K < (1LL << 31), "%s: activation matrix too large (M * K must be < 2^31)", who);
   const uint32_t a_xor = (a_type == ITEXHIP_QUINT8) ? 0x80808080u : 0u;
-  const EpilogueArgs e = make_args(a_type, colsum, scales, bias, ep);
   const uint8_t* ap = reinterpret_cast<const uint8_t*>(a);
   const uint8_t* bp = reinterpret_cast<const uint8_t*>(packed_b);
   hipStream_t hs = as_stream(stream);
@@ -290,6 +286,15 @@ int packed_path(bool gemv, const void* a, int a_type, const int8_t* packed_b, co
   if (st__ != ITEXHIP_OK) return st__;
   ITEXHIP_CHECK_LAUNCH(who);
   return ITEXHIP_OK;
+}
+
+int packed_path(bool gemv, const void* a, int a_type, const int8_t* packed_b, const int32_t* colsum,
+                int64_t M, int64_t K, int64_t N, const float* scales, const float* bias,
+                const itexhip_epilogue* ep, int out_type, void* out, void* stream, const char* who) {
+  if (int st = check_common(a, a_type, packed_b, M, K, N, scales, ep, out_type, out, who)) return st;
+  if (M == 0 || N == 0) return ITEXHIP_OK;
+  return launch_packed(gemv, a, a_type, packed_b, M, K, N, make_args(a_type, colsum, scales, bias, ep), out_type, out,
+                       stream, who);
 }
 
 }  // namespace
@@ -370,4 +375,28 @@ extern "C" int itexhip_qgemm_naive(const void* a, int a_type, const int8_t* w, i
   }
   ITEXHIP_CHECK_LAUNCH("itexhip_qgemm_naive");
   return ITEXHIP_OK;
+}
+
+extern "C" int itexhip_qmatmul(const itexhip_matmul_params* p, const void* a, const int8_t* packed_b,
+                               const int32_t* colsum, int64_t M, int64_t K, int64_t N, const float* min_b,
+                               const float* max_b, int64_t nb, const float* bias, void* out, void* stream) {
+  const char* who = "itexhip_qmatmul";
+  itexhip_epilogue ep;
+  if (int st = itexhip_qmatmul_epilogue_desc(p, nb, &ep)) return st;
+  ITEXHIP_REQUIRE(nb == 1 || nb == N, "%s: %lld weight ranges for %lld channels", who, static_cast<long long>(nb),
+                  static_cast<long long>(N));
+  ITEXHIP_REQUIRE(M >= 0 && K >= 0 && N >= 0, "%s: negative dimension", who);
+  ITEXHIP_REQUIRE(M < (1LL << 31) && N < (1LL << 31) && K <= kMaxK, "%s: dimension too large (K <= %lld)", who,
+                  static_cast<long long>(kMaxK));
+  if (M == 0 || N == 0) return ITEXHIP_OK;
+  ITEXHIP_REQUIRE(out != nullptr && min_b != nullptr && max_b != nullptr, "%s: null buffer", who);
+  ITEXHIP_REQUIRE(K == 0 || (a && packed_b), "%s: null operand", who);
+  ITEXHIP_REQUIRE(colsum != nullptr, "%s: null colsum", who);
+  EpilogueArgs e = make_args(p->t_in, colsum, nullptr, bias, &ep);
+  e.fused = 1;
+  e.nb = static_cast<int>(nb);
+  e.min_b = min_b;
+  e.max_b = max_b;
+  e.prep = make_prep_args(p, ep);
+  return launch_packed(M <= 16, a, p->t_in, packed_b, M, K, N, e, p->t_out, out, stream, who);
 }

@@ -6,7 +6,7 @@
 #include <type_traits>
 #include <utility>
 
-#include "common.hpp"
+#include "qmatmul_params.hpp"
 
 namespace itexhip {
 
@@ -21,14 +21,33 @@ constexpr int kChunkBytes = 1024;  // 32 rows x 32 k
 constexpr int64_t kMaxK = 1 << 16; // 255 * 128 * 65536 < 2^31
 
 struct EpilogueArgs {
-  const float* scales;
-  const float* bias;
+  const float* scales;   // prepared per-channel scales (n_scales of them), unused when `fused`
+  const float* bias;     // prepared bias, or the op's raw fp32 bias when `fused`
   const int32_t* colsum;
   int n_scales;
   int comp_mul;  // 128 for u8 activations, 0 for s8
   int n_eltwise;
   itexhip_eltwise elt[2];
+  // fused != 0: the kernel derives scale and bias of a channel itself from the op's ranges
+  int fused;
+  int nb;  // weight ranges (1 or N)
+  const float* min_b;
+  const float* max_b;
+  PrepArgs prep;
 };
+
+// scale, bias and zero-point compensation of channel n (n < N), however the call supplied them
+__device__ __forceinline__ void resolve_channel(const EpilogueArgs& e, int n, int N, int* comp, float* scale, float* bias) {
+  *comp = e.comp_mul ? e.comp_mul * e.colsum[n] : 0;
+  if (e.fused) {
+    const ChannelScaleBias c = channel_scale_bias(e.prep, e.min_b, e.max_b, e.nb, e.bias, e.colsum, N, n);
+    *scale = e.n_scales > 0 ? c.scale : 1.0f;
+    *bias = c.bias;
+  } else {
+    *scale = e.n_scales > 1 ? e.scales[n] : (e.n_scales == 1 ? e.scales[0] : 1.0f);
+    *bias = e.bias ? e.bias[n] : 0.0f;
+  }
+}
 
 // ------------------------------------------------------------------------------------------------
 // Fused epilogue.  A 32x32 accumulator tile is held in MFMA layout: lane l, register r (0..15) ->
@@ -46,6 +65,11 @@ struct ChannelParams {
 
 __device__ __forceinline__ ChannelParams load_channel_params(const EpilogueArgs& e, int n, int N, bool vec_ok) {
   ChannelParams p;
+  if (e.fused) {
+#pragma unroll
+    for (int r = 0; r < 4; ++r) resolve_channel(e, min(n + r, N - 1), N, &p.comp[r], &p.scale[r], &p.bias[r]);
+    return p;
+  }
   if (vec_ok && n + 3 < N) {
     if (e.comp_mul) {
       const v4i c = *reinterpret_cast<const v4i*>(e.colsum + n);
@@ -132,7 +156,7 @@ __device__ __forceinline__ void epilogue_store(const v4i acc, const ChannelParam
   for (int r = 0; r < 4; ++r) {
     float v = static_cast<float>(acc[r] + p.comp[r]);
     v = v * p.scale[r];  // scale 1.0f when the node has no output scale (exact)
-    if (e.bias) v = v + p.bias[r];
+    if (e.bias || e.fused) v = v + p.bias[r];
     if (ACT == 1) {
       v = fmaxf(v, 0.0f);
     } else if (ACT == 2) {

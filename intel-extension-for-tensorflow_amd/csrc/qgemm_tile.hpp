@@ -163,9 +163,12 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void qgemm_tile_kernel(
   // epilogue is free of global loads and of branches on them
   if (threadIdx.x < BN) {
     const int n = min(n_base + static_cast<int>(threadIdx.x), N - 1);
-    panel_comp[threadIdx.x] = e.comp_mul ? e.comp_mul * e.colsum[n] : 0;
-    panel_scale[threadIdx.x] = e.n_scales > 1 ? e.scales[n] : (e.n_scales == 1 ? e.scales[0] : 1.0f);
-    panel_bias[threadIdx.x] = e.bias ? e.bias[n] : 0.0f;
+    int comp;
+    float scale, bias;
+    resolve_channel(e, n, N, &comp, &scale, &bias);
+    panel_comp[threadIdx.x] = comp;
+    panel_scale[threadIdx.x] = scale;
+    panel_bias[threadIdx.x] = bias;
   }
   wait_vmcnt<NLD>();
   __syncthreads();
@@ -272,7 +275,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void qgemm_tile_kernel(
   constexpr int RPP = 64 / LPR;              // rows per flush instruction (lanes >= RPP * LPR idle)
   constexpr int PASSES = (WM + RPP - 1) / RPP;
   static_assert(NW * WM * PITCH <= NSTAGE * STAGE_BYTES, "epilogue buffer must fit in the ring");
-  const bool fast = !GENERAL || (e.bias != nullptr && aligned16(out) && ((static_cast<int64_t>(N) * ESZ) & 15) == 0);
+  const bool fast = !GENERAL || ((e.bias != nullptr || e.fused) && aligned16(out) && ((static_cast<int64_t>(N) * ESZ) & 15) == 0);
   if (fast) {
     uint8_t* ebuf = lds + wave * (WM * PITCH);
     const int f_row = lane / LPR, f_piece = lane % LPR;
@@ -308,7 +311,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void qgemm_tile_kernel(
       }
     });
   } else if constexpr (GENERAL) {
-    const bool has_bias = e.bias != nullptr;
+    const bool has_bias = e.bias != nullptr || e.fused;
     static_for<TN>([&](auto j) {
       static_for<4>([&](auto g) {
         const int col = (wn * TN + j) * 32 + decltype(g)::value * 8 + lgrp * 4;
@@ -401,7 +404,7 @@ int dispatch_tile(const uint8_t* a, uint32_t a_xor, const uint8_t* bp, int M, in
                   const EpilogueArgs& e, void* out, hipStream_t st) {
   constexpr int esz = (OUT_T == ITEXHIP_QINT8 || OUT_T == ITEXHIP_QUINT8) ? 1 : 4;
   // the specialised kernels only carry the vectorised epilogue: bias present, output rows 16-byte aligned
-  const bool plain = e.bias != nullptr && (reinterpret_cast<uintptr_t>(out) & 15) == 0 &&
+  const bool plain = (e.bias != nullptr || e.fused) && (reinterpret_cast<uintptr_t>(out) & 15) == 0 &&
                      ((static_cast<int64_t>(N) * esz) & 15) == 0 && (K & 63) == 0;
   const int act = e.n_eltwise == 0 ? 0
                   : (e.n_eltwise == 1 && e.elt[0].alg == ITEXHIP_ELT_RELU && e.elt[0].alpha == 0.0f) ? 1 : 2;

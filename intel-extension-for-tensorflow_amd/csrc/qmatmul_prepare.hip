@@ -7,20 +7,10 @@
 //                      :1610-1702 (V1), :1809-1908 (V2)
 //   GetScaledBias      quantized_matmul_common.h:466-660 (fp32 bias)
 //   PostOpUtil         itex/core/utils/onednn/onednn_post_op_util.cc:73-128, 237-273
-#include "common.hpp"
+#include "qmatmul_params.hpp"
 
 namespace itexhip {
 namespace {
-
-struct PrepArgs {
-  int api, t_in, t_out, input_mode;
-  int n_scales;        // from the epilogue descriptor
-  int mul_requant;     // multiply the output scale by (max_int8_output / range_output)
-  int legacy_kind;     // 1: u8 out, 2: s8 out, 3: fp32 out (legacy api only)
-  float min_a, max_a, min_out, max_out;
-};
-
-__device__ __forceinline__ float absmax(float a, float b) { return fmaxf(fabsf(a), fabsf(b)); }
 
 __global__ void qmatmul_prepare_kernel(PrepArgs p, const float* __restrict__ min_b,
                                        const float* __restrict__ max_b, int64_t nb,
@@ -29,60 +19,10 @@ __global__ void qmatmul_prepare_kernel(PrepArgs p, const float* __restrict__ min
                                        float* __restrict__ bias_out) {
   const int64_t j = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
   if (j >= N) return;
-  const float max_int8_input = (p.t_in == ITEXHIP_QUINT8) ? 255.0f : 127.0f;
-  const float max_int8_weight = 127.0f;
-  const float max_int8_output = (p.t_out == ITEXHIP_QUINT8) ? 255.0f : 127.0f;
-  const float range_input =
-      (p.input_mode == ITEXHIP_MIN_FIRST) ? p.max_a - p.min_a : absmax(p.min_a, p.max_a);
-  const int64_t jb = (nb == N) ? j : 0;
-  const float range_weight = absmax(min_b[jb], max_b[jb]);
-
-  // ---- output scale of channel j (or the single per-tensor scale) ------------------------------
-  float os = 1.0f;
-  if (p.api == ITEXHIP_API_LEGACY) {
-    if (p.legacy_kind != 0) {
-      const float a_level = (p.max_a - p.min_a) / 255.0f;
-      const float b_level = (max_b[0] - min_b[0]) / 254.0f;
-      const float c_level = a_level * b_level;
-      const float scale_int32 = absmax(c_level * -2147483648.0f, c_level * 2147483648.0f);
-      const float scale_eightbit = absmax(p.min_out, p.max_out);
-      if (p.legacy_kind == 1) os = scale_int32 / scale_eightbit / 8388608.0f;
-      else if (p.legacy_kind == 2) os = scale_int32 / scale_eightbit / 16777216.0f;
-      else os = scale_int32 / 2147483648.0f;
-    }
-  } else if (p.api == ITEXHIP_API_V1 && p.t_out == ITEXHIP_QINT32) {
-    os = 1.0f;
-  } else if (p.n_scales > 0) {
-    os = (range_input * range_weight) / (max_int8_input * max_int8_weight);
-    if (p.mul_requant) {
-      const float range_output = absmax(p.min_out, p.max_out);
-      os = os * (max_int8_output / range_output);
-    }
-  }
-  if (p.n_scales > 1) scales_out[j] = os;
-  else if (p.n_scales == 1 && j == 0) scales_out[0] = os;
-
-  // ---- bias -----------------------------------------------------------------------------------
-  const float bias_scale = (max_int8_input * max_int8_weight) / (range_input * range_weight);
-  const float b = bias ? bias[j] : 0.0f;
-  float out;
-  if (p.input_mode == ITEXHIP_MIN_FIRST) {
-    const float q_min_input = max_int8_input * p.min_a / range_input;
-    const float sum = static_cast<float>(colsum[j]);
-    if (p.t_out == ITEXHIP_FLOAT) {
-      out = b + (sum * q_min_input / bias_scale);
-    } else if (p.t_out == ITEXHIP_QINT8 || p.t_out == ITEXHIP_QUINT8) {
-      // os is this channel's output scale, or the single scale when n_scales == 1
-      out = b * bias_scale * os + (sum * q_min_input * os);
-    } else {
-      out = b * bias_scale + (sum * q_min_input);
-    }
-  } else {
-    // SCALED input: the bias is scaled by the FIRST weight's bias scale for every channel
-    const float bs0 = (max_int8_input * max_int8_weight) / (range_input * absmax(min_b[0], max_b[0]));
-    out = b * bs0;
-  }
-  bias_out[j] = out;
+  const ChannelScaleBias c = channel_scale_bias(p, min_b, max_b, nb, bias, colsum, N, j);
+  if (p.n_scales > 1) scales_out[j] = c.scale;
+  else if (p.n_scales == 1 && j == 0) scales_out[0] = c.scale;
+  bias_out[j] = c.bias;
 }
 
 int eltwise_from_activation(int act, itexhip_eltwise* e) {
@@ -169,20 +109,7 @@ extern "C" int itexhip_qmatmul_prepare(const itexhip_matmul_params* p, const flo
   ITEXHIP_REQUIRE(ep.n_scales == 0 || scales_out, "qmatmul_prepare: null scales_out");
   ITEXHIP_REQUIRE(p->input_mode != ITEXHIP_MIN_FIRST || colsum, "qmatmul_prepare: MIN_FIRST needs colsum");
 
-  PrepArgs a{};
-  a.api = p->api; a.t_in = p->t_in; a.t_out = p->t_out; a.input_mode = p->input_mode;
-  a.n_scales = ep.n_scales;
-  a.min_a = p->min_a; a.max_a = p->max_a; a.min_out = p->min_out; a.max_out = p->max_out;
-  const bool out_q8 = p->t_out == ITEXHIP_QINT8 || p->t_out == ITEXHIP_QUINT8;
-  if (p->api == ITEXHIP_API_V2) {
-    // requantize factor folded into the output scale only without any eltwise post-op
-    a.mul_requant = p->has_requantize && ep.n_eltwise == 0;
-  } else if (p->api == ITEXHIP_API_V1) {
-    a.mul_requant = out_q8 && p->n_fused_ops == 1;
-  } else {
-    a.legacy_kind = p->t_out == ITEXHIP_QUINT8 ? 1 : p->t_out == ITEXHIP_QINT8 ? 2
-                    : p->t_out == ITEXHIP_FLOAT ? 3 : 0;
-  }
+  const PrepArgs a = make_prep_args(p, ep);
   const unsigned grid = static_cast<unsigned>((N + 255) / 256);
   qmatmul_prepare_kernel<<<grid, 256, 0, as_stream(stream)>>>(a, min_b, max_b, nb, bias, colsum, N,
                                                               scales_out, bias_out);

@@ -165,41 +165,30 @@ class QuantizedMatMulOp : public OpKernel {
       packed_src_ = w.data();
       packed_k_ = K;
       packed_n_ = N;
-      prepared_ = false;
     }
     // ---- per-channel scale and bias vectors on the device
     float* min_b_dev = min_b_cache_.Get(ctx, min_b_t.flat<float>(), nb, TF_FLOAT);
     float* max_b_dev = max_b_cache_.Get(ctx, max_b_t.flat<float>(), nb, TF_FLOAT);
     if (min_b_dev == nullptr || max_b_dev == nullptr) return;
-    if (!scales_.valid() || scales_.NumElements() < std::max<int64_t>(N, 1)) {
-      scales_ = ctx->allocate_temp(TF_FLOAT, {std::max<int64_t>(N, 1)});
-      sbias_ = ctx->allocate_temp(TF_FLOAT, {std::max<int64_t>(N, 1)});
-      if (!ctx->ok()) return;
-      prepared_ = false;
-    }
-    // the prepared vectors are reused while nothing they depend on changed (cf. IsCachedBiasValid
-    // :458-464, which tolerates 1e-5; here the comparison is exact)
-    const bool same = prepared_ && is_bias_const_ && is_weight_const_ && bias.data() == prepared_bias_ &&
-                      std::memcmp(&p, &prepared_p_, sizeof(p)) == 0 && !min_b_cache_.changed() && !max_b_cache_.changed();
-    if (!same) {
-      st = itexhip_qmatmul_prepare(&p, min_b_dev, max_b_dev, nb, bias.flat<float>(), colsum_.flat<int32_t>(), N,
-                                   scales_.flat<float>(), sbias_.flat<float>(), stream);
-      ITEX_REQUIRES(ctx, st == ITEXHIP_OK, st == ITEXHIP_INVALID_ARGUMENT ? TF_INVALID_ARGUMENT : TF_ABORTED,
-                    std::string("Operation received an exception: ") + itexhip_last_error());
-      prepared_ = true;
-      prepared_p_ = p;
-      prepared_bias_ = bias.data();
-    }
-
-    // ---- product
+    // ---- product.  K a multiple of 16: one launch, the MatMul kernel derives each channel's output
+    // scale and compensated bias itself, so a new activation range costs nothing extra.  Other K: the
+    // parameter vectors are prepared by a small kernel and the reference-shaped kernel runs.
     Tensor out = ctx->allocate_output(0, v_.t_out, {M, N});
     if (!ctx->ok()) return;
     if (K % 16 == 0 && K > 0) {
-      st = itexhip_qgemm(a.data(), v_.t_in, packed_.flat<int8_t>(), colsum_.flat<int32_t>(), M, K, N,
-                         scales_.flat<float>(), sbias_.flat<float>(), &ep, v_.t_out, out.data(), stream);
+      st = itexhip_qmatmul(&p, a.data(), packed_.flat<int8_t>(), colsum_.flat<int32_t>(), M, K, N, min_b_dev, max_b_dev,
+                           nb, bias.flat<float>(), out.data(), stream);
     } else {
-      st = itexhip_qgemm_naive(a.data(), v_.t_in, w.flat<int8_t>(), transpose_b_ ? 1 : 0, M, K, N, scales_.flat<float>(),
-                               sbias_.flat<float>(), &ep, v_.t_out, out.data(), stream);
+      if (!scales_.valid() || scales_.NumElements() < std::max<int64_t>(N, 1)) {
+        scales_ = ctx->allocate_temp(TF_FLOAT, {std::max<int64_t>(N, 1)});
+        sbias_ = ctx->allocate_temp(TF_FLOAT, {std::max<int64_t>(N, 1)});
+        if (!ctx->ok()) return;
+      }
+      st = itexhip_qmatmul_prepare(&p, min_b_dev, max_b_dev, nb, bias.flat<float>(), colsum_.flat<int32_t>(), N,
+                                   scales_.flat<float>(), sbias_.flat<float>(), stream);
+      if (st == ITEXHIP_OK)
+        st = itexhip_qgemm_naive(a.data(), v_.t_in, w.flat<int8_t>(), transpose_b_ ? 1 : 0, M, K, N, scales_.flat<float>(),
+                                 sbias_.flat<float>(), &ep, v_.t_out, out.data(), stream);
     }
     ITEX_REQUIRES(ctx, st == ITEXHIP_OK, st == ITEXHIP_INVALID_ARGUMENT ? TF_INVALID_ARGUMENT : TF_ABORTED,
                   std::string("Operation received an exception: ") + itexhip_last_error());
@@ -236,9 +225,6 @@ class QuantizedMatMulOp : public OpKernel {
   const void* packed_src_ = nullptr;
   int64_t packed_k_ = -1, packed_n_ = -1;
   DeviceVectorCache<float> min_b_cache_, max_b_cache_;
-  bool prepared_ = false;
-  itexhip_matmul_params prepared_p_{};
-  const void* prepared_bias_ = nullptr;
 };
 
 template <int API, int TIN, int TOUT, bool RELU>

@@ -47,7 +47,10 @@ class Linear:
         x_d = torch.from_numpy(xq).to(self.dev)
         out = torch.empty((M, self.N), dtype=tdt(kw["t_out"]), device=self.dev)
         fn = {"auto": hip.qgemm, "tile": hip.qgemm_tile, "gemv": hip.qgemv}.get(path)
-        if path == "naive":
+        if path == "fused":
+            hip.qmatmul(p, x_d, self.packed, self.colsum, M, self.K, self.N, self.min_b_d, self.max_b_d, nb,
+                        self.bias_d, out)
+        elif path == "naive":
             hip.qgemm_naive(x_d, t_in, self.w_d, False, M, self.K, self.N, self.scales_d, self.sbias_d, ep,
                             kw["t_out"], out)
         else:
@@ -183,6 +186,29 @@ def test_tile_kernel_vs_oracle(hip, dev, M, K, N, kw):
     ref = layer.oracle(xq, kw, mn, mx, -r_out, r_out)
     got = layer.run(xq, kw, mn, mx, -r_out, r_out, path="tile")
     np.testing.assert_array_equal(got, ref)
+    np.testing.assert_array_equal(layer.run(xq, kw, mn, mx, -r_out, r_out, path="fused"), ref)
+
+
+@pytest.mark.parametrize("kw", [V2_DEQ, V2_DEQ_RELU, V2_REQ_S8, V2_REQ_U8_RELU, V1_S32,
+                                dict(api=orc.API_V1, t_out=orc.QINT8, input_mode=orc.MIN_FIRST, n_fused_ops=1),
+                                dict(api=orc.API_LEGACY, t_out=orc.QUINT8, input_mode=orc.MIN_FIRST, activation=orc.ACT_RELU),
+                                dict(api=orc.API_LEGACY, t_out=orc.FLOAT, input_mode=orc.MIN_FIRST),
+                                dict(api=orc.API_V2, t_out=orc.FLOAT, input_mode=orc.SCALED, has_dequantize=True)])
+@pytest.mark.parametrize("per_channel", [True, False])
+@pytest.mark.parametrize("M", [5, 200])
+def test_single_launch_op_vs_oracle(hip, dev, kw, per_channel, M):
+    """itexhip_qmatmul derives the per-channel parameters inside the MatMul kernel (GEMV and tile paths)."""
+    if kw["api"] == orc.API_LEGACY and per_channel:
+        pytest.skip("the legacy ops take per-tensor weight ranges")
+    K, N = 320, 272
+    layer, w, bias = make_layer(hip, dev, K, N, seed=77, per_channel=per_channel)
+    mode = kw["input_mode"]
+    x, xq, mn, mx = make_acts(M, K, seed=M, mode=mode)
+    full = x @ w + bias
+    r_out = float(np.abs(np.maximum(full, 0) if kw.get("activation") else full).max())
+    lo = 0.0 if kw["t_out"] == orc.QUINT8 else -r_out
+    ref = layer.oracle(xq, kw, mn, mx, lo, r_out)
+    np.testing.assert_array_equal(layer.run(xq, kw, mn, mx, lo, r_out, path="fused"), ref)
 
 
 @pytest.mark.parametrize("shape", [0, 1, 2, 3, 4])
@@ -215,6 +241,7 @@ def test_gemv_kernel_vs_oracle(hip, dev, M, K, N, kw):
     np.testing.assert_array_equal(layer.run(xq, kw, mn, mx, -r_out, r_out, path="gemv"), ref)
     np.testing.assert_array_equal(layer.run(xq, kw, mn, mx, -r_out, r_out, path="auto"), ref)
     np.testing.assert_array_equal(layer.run(xq, kw, mn, mx, -r_out, r_out, path="tile"), ref)
+    np.testing.assert_array_equal(layer.run(xq, kw, mn, mx, -r_out, r_out, path="fused"), ref)
 
 
 def test_signed_activations_and_extremes(hip, dev):
