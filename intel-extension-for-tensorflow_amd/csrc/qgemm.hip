@@ -83,7 +83,7 @@ __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(4, 4))) vo
                                                      void* __restrict__ out) {
   constexpr int U = 8;         // chunk pairs per batch
   constexpr int NT = SW / 16;  // 16-channel tiles per strip
-  extern __shared__ int red[];  // [waves][NT][4][64]
+  extern __shared__ int red[];  // [waves][NT][4][64], then the parameter panel [3][SW]
   const int strip = blockIdx.x;
   const int waves = blockDim.x >> 6;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
@@ -101,6 +101,13 @@ __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(4, 4))) vo
   v4i acc[NT];
 #pragma unroll
   for (int t = 0; t < NT; ++t) acc[t] = v4i{0, 0, 0, 0};
+
+  // The last wavefront also resolves the strip's channel parameters, one channel per lane: the loads
+  // go out now, the arithmetic waits until its share of the weight stream is done.
+  int* const panel = red + waves * NT * 256;
+  const bool param_lane = (wave == waves - 1) && lane < SW;
+  RawChannel raw{};
+  if (param_lane) raw = load_raw_channel(e, min(strip * SW + lane, N - 1), N);
 
   auto load_act = [&](int p) { return *reinterpret_cast<const v4i*>(arow + min(p * 64 + kpiece, klast)); };
   auto load_act_inside = [&](int p) { return *reinterpret_cast<const v4i*>(arow + (p * 64 + kpiece)); };
@@ -148,6 +155,14 @@ __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(4, 4))) vo
       }
   }
 
+  if (param_lane) {
+    int comp;
+    float scale, bias;
+    finish_channel(e, raw, &comp, &scale, &bias);
+    panel[lane] = comp;
+    panel[SW + lane] = __float_as_int(scale);
+    panel[2 * SW + lane] = __float_as_int(bias);
+  }
   // cross-wavefront reduction
 #pragma unroll
   for (int t = 0; t < NT; ++t)
@@ -157,10 +172,16 @@ __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(4, 4))) vo
     v4i part = v4i{0, 0, 0, 0};
     for (int w = 0; w < waves; ++w) part += *reinterpret_cast<const v4i*>(&red[((w * NT + wave) * 64 + lane) * 4]);
     // accumulator layout of the 16x16 MFMA: lane l, register r -> m = l % 16, n = (l / 16) * 4 + r
-    const bool vec_ok = (N & 3) == 0 && aligned16(e.scales) && aligned16(e.bias) && aligned16(e.colsum) && aligned16(out);
-    const int n = strip * SW + wave * 16 + lgrp * 4;
+    const bool vec_ok = (N & 3) == 0 && aligned16(out);
+    const int col = wave * 16 + lgrp * 4, n = strip * SW + col;
     if (lrow < M && n < N) {
-      const ChannelParams cp = load_channel_params(e, n, N, vec_ok);
+      ChannelParams cp;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        cp.comp[r] = panel[col + r];
+        cp.scale[r] = __int_as_float(panel[SW + col + r]);
+        cp.bias[r] = __int_as_float(panel[2 * SW + col + r]);
+      }
       epilogue_store<OUT_T, 2>(part, cp, lrow, n, M, N, e, out, vec_ok);
     }
   }
@@ -243,10 +264,10 @@ int dispatch_gemv(const uint8_t* a, uint32_t a_xor, const uint8_t* bp, int M, in
   const int cnt = (KP + waves - 1) / waves;
   const int strips32 = (N + 31) / 32;
   if (strips32 >= 256) {
-    const size_t lds = static_cast<size_t>(waves) * 2 * 1024;
+    const size_t lds = static_cast<size_t>(waves) * 2 * 1024 + 3 * 32 * 4;
     qgemv_kernel<32, OUT_T><<<strips32, 64 * waves, lds, st>>>(a, a_xor, bp, M, K, N, KC, cnt, e, out);
   } else {
-    const size_t lds = static_cast<size_t>(waves) * 1024;
+    const size_t lds = static_cast<size_t>(waves) * 1024 + 3 * 16 * 4;
     qgemv_kernel<16, OUT_T><<<(N + 15) / 16, 64 * waves, lds, st>>>(a, a_xor, bp, M, K, N, KC, cnt, e, out);
   }
   return ITEXHIP_OK;

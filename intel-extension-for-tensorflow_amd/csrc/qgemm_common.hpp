@@ -36,24 +36,53 @@ struct EpilogueArgs {
   PrepArgs prep;
 };
 
-// scale, bias and zero-point compensation of channel n (n < N), however the call supplied them
-__device__ __forceinline__ void resolve_channel(const EpilogueArgs& e, int n, int N, int* comp, float* scale, float* bias) {
-  *comp = e.comp_mul ? e.comp_mul * e.colsum[n] : 0;
+// Scale, bias and zero-point compensation of channel n (n < N), however the call supplied them, in two
+// stages so that a kernel can issue the loads early and do the arithmetic late.
+struct RawChannel {
+  float min_bj, max_bj, min_b0, max_b0;  // fused: weight ranges;  else min_bj holds the prepared scale
+  float bias;
+  int colsum;
+};
+
+__device__ __forceinline__ RawChannel load_raw_channel(const EpilogueArgs& e, int n, int N) {
+  RawChannel r{};
+  r.colsum = e.colsum ? e.colsum[n] : 0;
+  r.bias = e.bias ? e.bias[n] : 0.0f;
   if (e.fused) {
-    const ChannelScaleBias c = channel_scale_bias(e.prep, e.min_b, e.max_b, e.nb, e.bias, e.colsum, N, n);
+    const int jb = (e.nb == N) ? n : 0;
+    r.min_bj = e.min_b[jb];
+    r.max_bj = e.max_b[jb];
+    r.min_b0 = e.min_b[0];
+    r.max_b0 = e.max_b[0];
+  } else {
+    r.min_bj = e.n_scales > 1 ? e.scales[n] : (e.n_scales == 1 ? e.scales[0] : 1.0f);
+  }
+  return r;
+}
+
+__device__ __forceinline__ void finish_channel(const EpilogueArgs& e, const RawChannel& r, int* comp, float* scale,
+                                               float* bias) {
+  *comp = e.comp_mul * r.colsum;
+  if (e.fused) {
+    const ChannelScaleBias c = channel_scale_bias(e.prep, r.min_bj, r.max_bj, r.min_b0, r.max_b0, r.bias, r.colsum);
     *scale = e.n_scales > 0 ? c.scale : 1.0f;
     *bias = c.bias;
   } else {
-    *scale = e.n_scales > 1 ? e.scales[n] : (e.n_scales == 1 ? e.scales[0] : 1.0f);
-    *bias = e.bias ? e.bias[n] : 0.0f;
+    *scale = r.min_bj;
+    *bias = r.bias;
   }
+}
+
+__device__ __forceinline__ void resolve_channel(const EpilogueArgs& e, int n, int N, int* comp, float* scale, float* bias) {
+  const RawChannel r = load_raw_channel(e, n, N);
+  finish_channel(e, r, comp, scale, bias);
 }
 
 // ------------------------------------------------------------------------------------------------
 // Fused epilogue.  A 32x32 accumulator tile is held in MFMA layout: lane l, register r (0..15) ->
 //   m = m0 + (l % 32), n = n0 + (r / 4) * 8 + (l / 32) * 4 + (r % 4),
 // so a lane owns 4 groups of 4 consecutive output channels of one row; epilogue_store handles one group.  The per-channel parameters of those 4
-// channels are loaded once (ChannelParams) and reused for every row tile of the same channel tile.
+// channels are resolved once (ChannelParams) and reused for every row of the same channel group.
 //   y = fl(fl((float)(acc + comp[n]) * scale[n]) + bias[n]);  eltwise chain;  convert.
 // ACT selects the eltwise chain at compile time: 0 = none, 1 = relu (alpha 0), 2 = generic chain.
 // ------------------------------------------------------------------------------------------------
@@ -62,51 +91,6 @@ struct ChannelParams {
   float scale[4];
   float bias[4];
 };
-
-__device__ __forceinline__ ChannelParams load_channel_params(const EpilogueArgs& e, int n, int N, bool vec_ok) {
-  ChannelParams p;
-  if (e.fused) {
-#pragma unroll
-    for (int r = 0; r < 4; ++r) resolve_channel(e, min(n + r, N - 1), N, &p.comp[r], &p.scale[r], &p.bias[r]);
-    return p;
-  }
-  if (vec_ok && n + 3 < N) {
-    if (e.comp_mul) {
-      const v4i c = *reinterpret_cast<const v4i*>(e.colsum + n);
-#pragma unroll
-      for (int r = 0; r < 4; ++r) p.comp[r] = e.comp_mul * c[r];
-    } else {
-#pragma unroll
-      for (int r = 0; r < 4; ++r) p.comp[r] = 0;
-    }
-    if (e.n_scales > 1) {
-      const f4 s = *reinterpret_cast<const f4*>(e.scales + n);
-#pragma unroll
-      for (int r = 0; r < 4; ++r) p.scale[r] = s[r];
-    } else {
-      const float s = e.n_scales == 1 ? e.scales[0] : 1.0f;
-#pragma unroll
-      for (int r = 0; r < 4; ++r) p.scale[r] = s;
-    }
-    if (e.bias) {
-      const f4 b = *reinterpret_cast<const f4*>(e.bias + n);
-#pragma unroll
-      for (int r = 0; r < 4; ++r) p.bias[r] = b[r];
-    } else {
-#pragma unroll
-      for (int r = 0; r < 4; ++r) p.bias[r] = 0.0f;
-    }
-  } else {
-#pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      const int nn = min(n + r, N - 1);  // clamped: out-of-range channels are computed but never stored
-      p.comp[r] = e.comp_mul ? e.comp_mul * e.colsum[nn] : 0;
-      p.scale[r] = e.n_scales > 1 ? e.scales[nn] : (e.n_scales == 1 ? e.scales[0] : 1.0f);
-      p.bias[r] = e.bias ? e.bias[nn] : 0.0f;
-    }
-  }
-  return p;
-}
 
 // The 4 outputs of one channel group in registers: epilogue arithmetic + conversion, no store.
 // 8-bit outputs come back packed in .x; 32-bit outputs as 4 lanes of raw bits.

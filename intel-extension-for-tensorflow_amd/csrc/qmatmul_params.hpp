@@ -27,26 +27,24 @@ struct ChannelScaleBias {
 
 __device__ __forceinline__ float absmax(float a, float b) { return fmaxf(fabsf(a), fabsf(b)); }
 
-// channel j of N; nb = number of weight ranges (1 or N)
-__device__ __forceinline__ ChannelScaleBias channel_scale_bias(const PrepArgs& p, const float* __restrict__ min_b,
-                                                               const float* __restrict__ max_b, int64_t nb,
-                                                               const float* __restrict__ bias,
-                                                               const int32_t* __restrict__ colsum, int64_t N,
-                                                               int64_t j) {
+// Value form: the weight range of the channel (min_bj, max_bj), the first weight range (min_b0, max_b0;
+// the legacy ops and the SCALED-input bias use it for every channel), the channel's raw bias and
+// weight column sum.
+__device__ __forceinline__ ChannelScaleBias channel_scale_bias(const PrepArgs& p, float min_bj, float max_bj,
+                                                               float min_b0, float max_b0, float b, int colsum_j) {
   const float max_int8_input = (p.t_in == ITEXHIP_QUINT8) ? 255.0f : 127.0f;
   const float max_int8_weight = 127.0f;
   const float max_int8_output = (p.t_out == ITEXHIP_QUINT8) ? 255.0f : 127.0f;
   const float range_input =
       (p.input_mode == ITEXHIP_MIN_FIRST) ? p.max_a - p.min_a : absmax(p.min_a, p.max_a);
-  const int64_t jb = (nb == N) ? j : 0;
-  const float range_weight = absmax(min_b[jb], max_b[jb]);
+  const float range_weight = absmax(min_bj, max_bj);
 
-  // ---- output scale of channel j (or the single per-tensor scale) ------------------------------
+  // ---- output scale of the channel (or the single per-tensor scale) ----------------------------
   float os = 1.0f;
   if (p.api == ITEXHIP_API_LEGACY) {
     if (p.legacy_kind != 0) {
       const float a_level = (p.max_a - p.min_a) / 255.0f;
-      const float b_level = (max_b[0] - min_b[0]) / 254.0f;
+      const float b_level = (max_b0 - min_b0) / 254.0f;
       const float c_level = a_level * b_level;
       const float scale_int32 = absmax(c_level * -2147483648.0f, c_level * 2147483648.0f);
       const float scale_eightbit = absmax(p.min_out, p.max_out);
@@ -66,11 +64,10 @@ __device__ __forceinline__ ChannelScaleBias channel_scale_bias(const PrepArgs& p
 
   // ---- bias -----------------------------------------------------------------------------------
   const float bias_scale = (max_int8_input * max_int8_weight) / (range_input * range_weight);
-  const float b = bias ? bias[j] : 0.0f;
   float out;
   if (p.input_mode == ITEXHIP_MIN_FIRST) {
     const float q_min_input = max_int8_input * p.min_a / range_input;
-    const float sum = static_cast<float>(colsum[j]);
+    const float sum = static_cast<float>(colsum_j);
     if (p.t_out == ITEXHIP_FLOAT) {
       out = b + (sum * q_min_input / bias_scale);
     } else if (p.t_out == ITEXHIP_QINT8 || p.t_out == ITEXHIP_QUINT8) {
@@ -81,10 +78,22 @@ __device__ __forceinline__ ChannelScaleBias channel_scale_bias(const PrepArgs& p
     }
   } else {
     // SCALED input: the bias is scaled by the FIRST weight's bias scale for every channel
-    const float bs0 = (max_int8_input * max_int8_weight) / (range_input * absmax(min_b[0], max_b[0]));
+    const float bs0 = (max_int8_input * max_int8_weight) / (range_input * absmax(min_b0, max_b0));
     out = b * bs0;
   }
   return ChannelScaleBias{os, out};
+}
+
+// Pointer form: channel j of N; nb = number of weight ranges (1 or N); colsum is only read for
+// MIN_FIRST input.
+__device__ __forceinline__ ChannelScaleBias channel_scale_bias(const PrepArgs& p, const float* __restrict__ min_b,
+                                                               const float* __restrict__ max_b, int64_t nb,
+                                                               const float* __restrict__ bias,
+                                                               const int32_t* __restrict__ colsum, int64_t N,
+                                                               int64_t j) {
+  const int64_t jb = (nb == N) ? j : 0;
+  return channel_scale_bias(p, min_b[jb], max_b[jb], min_b[0], max_b[0], bias ? bias[j] : 0.0f,
+                            p.input_mode == ITEXHIP_MIN_FIRST ? colsum[j] : 0);
 }
 
 // host: fills PrepArgs from the op parameters and its epilogue descriptor
