@@ -189,27 +189,52 @@ __device__ __forceinline__ int wave_max(int v) {
   return v;
 }
 
-// Whole-tensor (depth == 1) reduction: grid-stride over i4, wavefront reduction, one atomic pair
-// per wavefront.
+// Whole-tensor reductions.  At most kReduceBlocks workgroups walk the tensor; per round a workgroup
+// takes kReduceUnroll consecutive 4 KiB pieces (all loads issued before the first compare).  The
+// wavefronts of a workgroup meet in LDS and one thread issues the workgroup's single atomic pair:
+// atomics on one address are serialised by the memory system (~10 ns each), so their number, not the
+// data, would otherwise set the run time.
+constexpr int kReduceUnroll = 8;
+constexpr int kReduceBlocks = 512;
+
+template <class V, class Less, class Commit>
+__device__ __forceinline__ void block_minmax_commit(V mn, V mx, Less less, Commit commit) {
+  __shared__ V smn[kThreads / 64], smx[kThreads / 64];
+  if ((threadIdx.x & 63) == 0) {
+    smn[threadIdx.x >> 6] = mn;
+    smx[threadIdx.x >> 6] = mx;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+#pragma unroll
+    for (int w = 1; w < kThreads / 64; ++w) {
+      if (less(smn[w], mn)) mn = smn[w];
+      if (less(mx, smx[w])) mx = smx[w];
+    }
+    commit(mn, mx);
+  }
+}
+
 __global__ __launch_bounds__(kThreads) void minmax_i32_flat_kernel(const i4* __restrict__ x, int64_t n4,
                                                                    const int32_t* __restrict__ tail,
                                                                    int ntail, int32_t* mn_out,
                                                                    int32_t* mx_out) {
   int mn = INT32_MAX, mx = INT32_MIN;
-  const int64_t stride = static_cast<int64_t>(gridDim.x) * kThreads;
-  int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
-  for (; i + 3 * stride < n4; i += 4 * stride) {
-    i4 v[4];
+  const int64_t round = static_cast<int64_t>(gridDim.x) * (kThreads * kReduceUnroll);
+  int64_t i = static_cast<int64_t>(blockIdx.x) * (kThreads * kReduceUnroll) + threadIdx.x;
+  for (; i + (kReduceUnroll - 1) * kThreads < n4; i += round) {
+    i4 v[kReduceUnroll];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) v[j] = __builtin_nontemporal_load(&x[i + j * stride]);
+    for (int j = 0; j < kReduceUnroll; ++j) v[j] = __builtin_nontemporal_load(&x[i + j * kThreads]);
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
+    for (int j = 0; j < kReduceUnroll; ++j) {
       mn = min(min(mn, v[j].x), min(v[j].y, min(v[j].z, v[j].w)));
       mx = max(max(mx, v[j].x), max(v[j].y, max(v[j].z, v[j].w)));
     }
   }
-  for (; i < n4; i += stride) {
-    const i4 v = x[i];
+  // the tensor's last, partial group of pieces (it belongs to one workgroup only)
+  for (int j = 0; j < kReduceUnroll && i + j * kThreads < n4; ++j) {
+    const i4 v = x[i + j * kThreads];
     mn = min(min(mn, v.x), min(v.y, min(v.z, v.w)));
     mx = max(max(mx, v.x), max(v.y, max(v.z, v.w)));
   }
@@ -219,10 +244,12 @@ __global__ __launch_bounds__(kThreads) void minmax_i32_flat_kernel(const i4* __r
   }
   mn = wave_min(mn);
   mx = wave_max(mx);
-  if ((threadIdx.x & 63) == 0) {
-    atomicMin(mn_out, mn);
-    atomicMax(mx_out, mx);
-  }
+  block_minmax_commit(
+      mn, mx, [](int p, int q) { return p < q; },
+      [&](int lo, int hi) {
+        atomicMin(mn_out, lo);
+        atomicMax(mx_out, hi);
+      });
 }
 
 // Per-channel reduction, channel = last dim: thread owns one channel of its block's column group
@@ -268,20 +295,21 @@ __global__ __launch_bounds__(kThreads) void minmax_f32_kernel(const f4* __restri
                                                               const float* __restrict__ tail, int ntail,
                                                               int* keys) {
   float mn = __builtin_inff(), mx = -__builtin_inff();
-  const int64_t stride = static_cast<int64_t>(gridDim.x) * kThreads;
-  int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
-  for (; i + 3 * stride < n4; i += 4 * stride) {
-    f4 v[4];
+  const int64_t round = static_cast<int64_t>(gridDim.x) * (kThreads * kReduceUnroll);
+  int64_t i = static_cast<int64_t>(blockIdx.x) * (kThreads * kReduceUnroll) + threadIdx.x;
+  for (; i + (kReduceUnroll - 1) * kThreads < n4; i += round) {
+    f4 v[kReduceUnroll];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) v[j] = __builtin_nontemporal_load(&x[i + j * stride]);
+    for (int j = 0; j < kReduceUnroll; ++j) v[j] = __builtin_nontemporal_load(&x[i + j * kThreads]);
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
+    for (int j = 0; j < kReduceUnroll; ++j) {
       mn = fminf(fminf(mn, v[j].x), fminf(v[j].y, fminf(v[j].z, v[j].w)));
       mx = fmaxf(fmaxf(mx, v[j].x), fmaxf(v[j].y, fmaxf(v[j].z, v[j].w)));
     }
   }
-  for (; i < n4; i += stride) {
-    const f4 v = x[i];
+  // the tensor's last, partial group of pieces (it belongs to one workgroup only)
+  for (int j = 0; j < kReduceUnroll && i + j * kThreads < n4; ++j) {
+    const f4 v = x[i + j * kThreads];
     mn = fminf(fminf(mn, v.x), fminf(v.y, fminf(v.z, v.w)));
     mx = fmaxf(fmaxf(mx, v.x), fmaxf(v.y, fmaxf(v.z, v.w)));
   }
@@ -294,10 +322,12 @@ __global__ __launch_bounds__(kThreads) void minmax_f32_kernel(const f4* __restri
     mn = fminf(mn, __shfl_xor(mn, o, 64));
     mx = fmaxf(mx, __shfl_xor(mx, o, 64));
   }
-  if ((threadIdx.x & 63) == 0) {
-    atomicMin(&keys[0], f2key(mn));
-    atomicMax(&keys[1], f2key(mx));
-  }
+  block_minmax_commit(
+      mn, mx, [](float p, float q) { return p < q; },
+      [&](float lo, float hi) {
+        atomicMin(&keys[0], f2key(lo));
+        atomicMax(&keys[1], f2key(hi));
+      });
 }
 
 inline unsigned blocks_for(int64_t n, int64_t per_block) {
@@ -507,8 +537,8 @@ extern "C" int itexhip_minmax_i32_per_channel(const int32_t* x, int64_t rows, in
       const int64_t n4 = vec ? rows / 4 : 0;
       const int ntail = static_cast<int>(rows - n4 * 4);
       if (vec) {
-        const unsigned grid = static_cast<unsigned>(
-            std::min<int64_t>(2048, std::max<int64_t>(1, (n4 + kThreads - 1) / kThreads)));
+        const unsigned grid = static_cast<unsigned>(std::min<int64_t>(
+            kReduceBlocks, std::max<int64_t>(1, (n4 + kThreads * kReduceUnroll - 1) / (kThreads * kReduceUnroll))));
         minmax_i32_flat_kernel<<<grid, kThreads, 0, st>>>(reinterpret_cast<const i4*>(x), n4,
                                                           x + n4 * 4, ntail, min_out, max_out);
       } else {
@@ -545,8 +575,8 @@ extern "C" int itexhip_minmax_f32(const float* x, int64_t n, float* minmax_out, 
     if (head > n) head = n;
     const int64_t n4 = (n - head) / 4;
     const int64_t ntail = n - head - n4 * 4;
-    const unsigned grid = static_cast<unsigned>(
-        std::min<int64_t>(2048, std::max<int64_t>(1, (n4 + kThreads - 1) / kThreads)));
+    const unsigned grid = static_cast<unsigned>(std::min<int64_t>(
+        kReduceBlocks, std::max<int64_t>(1, (n4 + kThreads * kReduceUnroll - 1) / (kThreads * kReduceUnroll))));
     minmax_f32_kernel<<<grid, kThreads, 0, st>>>(reinterpret_cast<const f4*>(x + head), n4,
                                                  x + head + n4 * 4, static_cast<int>(ntail), keys);
     if (head > 0)
