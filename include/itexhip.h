@@ -213,6 +213,13 @@ int itexhip_qgemm_naive(const void* a, int a_type, const int8_t* w, int transpos
                         int64_t K, int64_t N, const float* scales, const float* bias,
                         const itexhip_epilogue* ep, int out_type, void* out, void* stream);
 
+/* Diagnostic, no counterpart in the reference: `workgroups` x 4 wavefronts each issue iters x 8
+ * independent 32x32x32 i8 MFMAs (2 * 32768 ops each) on the 8 KiB of operand fragments at `operands`
+ * (device memory, 16-byte aligned) and nothing else.  Timed by the caller, it gives the rate the matrix
+ * cores sustain for that operand data on this device, the practical ceiling next to the published
+ * peak.  `sink` takes 256 ints that are practically never written. */
+int itexhip_mfma_probe(int workgroups, int iters, const void* operands, int32_t* sink, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -188,6 +188,38 @@ __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(4, 4))) vo
 }
 
 // ------------------------------------------------------------------------------------------------
+// Matrix-pipe probe: every wavefront issues `iters` x 8 independent 32x32x32 i8 MFMAs back to back on
+// operands taken from `operands` (8 KiB: 4 A and 4 B fragments per lane), no other instruction in the
+// loop.  Timing it gives the rate the matrix cores sustain for that operand data: the clock under
+// MFMA load depends on how much the operand bits toggle, so the ceiling for quantized data sits well
+// below the rate for constant operands.
+// ------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void mfma_probe_kernel(int iters, const v4i* __restrict__ operands, int* __restrict__ sink) {
+  v16i acc[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+#pragma unroll
+    for (int j = 0; j < 16; ++j) acc[i][j] = 0;
+  v4i a[4], b[4];
+  const int lane = threadIdx.x & 63;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    a[i] = operands[i * 64 + lane];
+    b[i] = operands[(4 + i) * 64 + lane];
+  }
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[i & 3], b[(i >> 1) & 3], acc[i], 0, 0, 0);
+  }
+  int s = 0;
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+#pragma unroll
+    for (int j = 0; j < 16; ++j) s += acc[i][j];
+  if (s == 0x7fffffff) sink[threadIdx.x] = s;  // keeps the accumulators alive; practically never taken
+}
+
+// ------------------------------------------------------------------------------------------------
 // Reference-shaped kernel on the unpacked weight: one thread per output element.
 // ------------------------------------------------------------------------------------------------
 template <int OUT_T>
@@ -420,4 +452,12 @@ extern "C" int itexhip_qmatmul(const itexhip_matmul_params* p, const void* a, co
   e.max_b = max_b;
   e.prep = make_prep_args(p, ep);
   return launch_packed(M <= 16, a, p->t_in, packed_b, M, K, N, e, p->t_out, out, stream, who);
+}
+
+extern "C" int itexhip_mfma_probe(int workgroups, int iters, const void* operands, int32_t* sink, void* stream) {
+  ITEXHIP_REQUIRE(workgroups > 0 && workgroups <= 65536 && iters > 0 && iters <= (1 << 22), "itexhip_mfma_probe: bad launch size");
+  ITEXHIP_REQUIRE(operands && sink && aligned(operands, 16), "itexhip_mfma_probe: null or unaligned buffer");
+  mfma_probe_kernel<<<workgroups, 256, 0, as_stream(stream)>>>(iters, reinterpret_cast<const v4i*>(operands), sink);
+  ITEXHIP_CHECK_LAUNCH("itexhip_mfma_probe");
+  return ITEXHIP_OK;
 }
