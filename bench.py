@@ -140,7 +140,7 @@ def make_acts(torch, hip, M, K, seed, dev, outlier_frac=0.0, outlier_mult=1.0):
 # ------------------------------------------------------------------------------------------------
 # workloads
 # ------------------------------------------------------------------------------------------------
-def bench_linear(torch, hip, timer, M, K, N, kind, steps, warmup, dev, seed, rotate=1, graph=False):
+def bench_linear(torch, hip, timer, M, K, N, kind, steps, warmup, dev, seed, rotate=1, graph=False, per_row=False):
     """kind: 'requant_s8' ([BiasAdd, Requantize] -> qint8), 'deq' / 'deq_relu' ([.., Dequantize] -> fp32).
     rotate > 1 cycles through that many distinct weight copies so that the weight stream comes from
     HBM, not from the 256 MiB last-level cache."""
@@ -165,10 +165,18 @@ def bench_linear(torch, hip, timer, M, K, N, kind, steps, warmup, dev, seed, rot
     out = torch.empty(M, N, dtype=out_dtype, device=dev)
     st = _stream(torch)
 
+    if per_row:  # per-token ranges (here: the tensor's range widened a little more for each row)
+        row_min = torch.tensor([min_a * (1.0 + 0.01 * m) for m in range(M)], dtype=torch.float32, device=dev)
+        row_max = torch.tensor([max_a * (1.0 + 0.01 * m) for m in range(M)], dtype=torch.float32, device=dev)
+
     def step(i):
         # what the op kernel runs per Compute: one launch, channel parameters derived inside the kernel
         L = layers[i % rotate]
-        hip.qmatmul(p, xq, L["packed"], L["colsum"], M, K, N, L["min_b"], L["max_b"], N, L["bias"], out, st)
+        if per_row:
+            hip.qmatmul_per_row(p, xq, L["packed"], L["colsum"], M, K, N, row_min, row_max, L["min_b"], L["max_b"], N,
+                                L["bias"], out, st)
+        else:
+            hip.qmatmul(p, xq, L["packed"], L["colsum"], M, K, N, L["min_b"], L["max_b"], N, L["bias"], out, st)
 
     for L in layers:  # parameter vectors for the two-launch form below
         hip.qmatmul_prepare(p, L["min_b"], L["max_b"], N, L["bias"], L["colsum"], N, L["scales"], L["sbias"], st)
@@ -352,6 +360,13 @@ def main():
                          frac_graph=r["gbs_kernel_graph"] / PEAK_HBM_GBS,
                          note="8 weight copies cycled (470 MB > last-level cache)")
                 others.append(r)
+            r = bench_linear(torch, hip, timer, 16, k, n, "deq", K_steps, W, dev, seed=10, rotate=8, per_row=True)
+            r.pop("_ctx")
+            r.update(name="decode_gemv_per_token_ranges", bound="hbm", us_kernel=r["ms_per_step"] * 1e3,
+                     gbs_kernel=r["bytes"] / (r["ms_per_step"] * 1e-3) / 1e9,
+                     frac=r["bytes"] / (r["ms_per_step"] * 1e-3) / 1e9 / PEAK_HBM_GBS,
+                     note="one launch per step, each row with its own activation range")
+            others.append(r)
     if "copy" in only:
         # device copy of 1 GiB: the kernel of known traffic that calibrates the memory counters
         nb = 1 << 30

@@ -206,6 +206,17 @@ int itexhip_qmatmul(const itexhip_matmul_params* p, const void* a, const int8_t*
                     const int32_t* colsum, int64_t M, int64_t K, int64_t N, const float* min_b,
                     const float* max_b, int64_t nb, const float* bias, void* out, void* stream);
 
+/* Decode batches quantized per token: row m of `a` was quantized with its own range
+ * (row_min_a[m], row_max_a[m]; device arrays of M floats, e.g. from QuantizeV2 with axis = 0,
+ * quantize_op.h:166-190) and row m of the result is what itexhip_qmatmul gives for the 1 x K problem
+ * with p->min_a / max_a replaced by that row's range.  The reference's MatMul ops only take a
+ * per-tensor activation range (they read element 0 of min_a / max_a, quantized_matmul_common.h:95-96),
+ * so this entry point is an extension; M <= 16. */
+int itexhip_qmatmul_per_row(const itexhip_matmul_params* p, const void* a, const int8_t* packed_b,
+                            const int32_t* colsum, int64_t M, int64_t K, int64_t N, const float* row_min_a,
+                            const float* row_max_a, const float* min_b, const float* max_b, int64_t nb,
+                            const float* bias, void* out, void* stream);
+
 /* Same contract on the unpacked TF-layout weight, any shape (no alignment requirements): one
  * thread per output element.  Used for shapes the tile kernels do not cover (K not a multiple of
  * 16) and as an on-device cross-check. */

@@ -83,7 +83,7 @@ __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(4, 4))) vo
                                                      void* __restrict__ out) {
   constexpr int U = 8;         // chunk pairs per batch
   constexpr int NT = SW / 16;  // 16-channel tiles per strip
-  extern __shared__ int red[];  // [waves][NT][4][64], then the parameter panel [3][SW]
+  extern __shared__ int red[];  // [waves][NT][4][64], then the parameter panel [3 or 6][SW]
   const int strip = blockIdx.x;
   const int waves = blockDim.x >> 6;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
@@ -156,12 +156,21 @@ __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(4, 4))) vo
   }
 
   if (param_lane) {
-    int comp;
-    float scale, bias;
-    finish_channel(e, raw, &comp, &scale, &bias);
-    panel[lane] = comp;
-    panel[SW + lane] = __float_as_int(scale);
-    panel[2 * SW + lane] = __float_as_int(bias);
+    if (e.row_min_a) {  // per-row ranges: the epilogue lanes finish the arithmetic for their own row
+      panel[lane] = raw.colsum;
+      panel[SW + lane] = __float_as_int(raw.min_bj);
+      panel[2 * SW + lane] = __float_as_int(raw.max_bj);
+      panel[3 * SW + lane] = __float_as_int(raw.min_b0);
+      panel[4 * SW + lane] = __float_as_int(raw.max_b0);
+      panel[5 * SW + lane] = __float_as_int(raw.bias);
+    } else {
+      int comp;
+      float scale, bias;
+      finish_channel(e, raw, &comp, &scale, &bias);
+      panel[lane] = comp;
+      panel[SW + lane] = __float_as_int(scale);
+      panel[2 * SW + lane] = __float_as_int(bias);
+    }
   }
   // cross-wavefront reduction
 #pragma unroll
@@ -176,11 +185,28 @@ __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(4, 4))) vo
     const int col = wave * 16 + lgrp * 4, n = strip * SW + col;
     if (lrow < M && n < N) {
       ChannelParams cp;
+      if (e.row_min_a) {
+        PrepArgs pr = e.prep;
+        pr.min_a = e.row_min_a[lrow];
+        pr.max_a = e.row_max_a[lrow];
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        cp.comp[r] = panel[col + r];
-        cp.scale[r] = __int_as_float(panel[SW + col + r]);
-        cp.bias[r] = __int_as_float(panel[2 * SW + col + r]);
+        for (int r = 0; r < 4; ++r) {
+          const int colsum = panel[col + r];
+          const ChannelScaleBias c = channel_scale_bias(
+              pr, __int_as_float(panel[SW + col + r]), __int_as_float(panel[2 * SW + col + r]),
+              __int_as_float(panel[3 * SW + col + r]), __int_as_float(panel[4 * SW + col + r]),
+              __int_as_float(panel[5 * SW + col + r]), colsum);
+          cp.comp[r] = e.comp_mul * colsum;
+          cp.scale[r] = e.n_scales > 0 ? c.scale : 1.0f;
+          cp.bias[r] = c.bias;
+        }
+      } else {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          cp.comp[r] = panel[col + r];
+          cp.scale[r] = __int_as_float(panel[SW + col + r]);
+          cp.bias[r] = __int_as_float(panel[2 * SW + col + r]);
+        }
       }
       epilogue_store<OUT_T, 2>(part, cp, lrow, n, M, N, e, out, vec_ok);
     }
@@ -296,10 +322,10 @@ int dispatch_gemv(const uint8_t* a, uint32_t a_xor, const uint8_t* bp, int M, in
   const int cnt = (KP + waves - 1) / waves;
   const int strips32 = (N + 31) / 32;
   if (strips32 >= 256) {
-    const size_t lds = static_cast<size_t>(waves) * 2 * 1024 + 3 * 32 * 4;
+    const size_t lds = static_cast<size_t>(waves) * 2 * 1024 + 6 * 32 * 4;
     qgemv_kernel<32, OUT_T><<<strips32, 64 * waves, lds, st>>>(a, a_xor, bp, M, K, N, KC, cnt, e, out);
   } else {
-    const size_t lds = static_cast<size_t>(waves) * 1024 + 3 * 16 * 4;
+    const size_t lds = static_cast<size_t>(waves) * 1024 + 6 * 16 * 4;
     qgemv_kernel<16, OUT_T><<<(N + 15) / 16, 64 * waves, lds, st>>>(a, a_xor, bp, M, K, N, KC, cnt, e, out);
   }
   return ITEXHIP_OK;
@@ -430,10 +456,11 @@ extern "C" int itexhip_qgemm_naive(const void* a, int a_type, const int8_t* w, i
   return ITEXHIP_OK;
 }
 
-extern "C" int itexhip_qmatmul(const itexhip_matmul_params* p, const void* a, const int8_t* packed_b,
-                               const int32_t* colsum, int64_t M, int64_t K, int64_t N, const float* min_b,
-                               const float* max_b, int64_t nb, const float* bias, void* out, void* stream) {
-  const char* who = "itexhip_qmatmul";
+namespace {
+int qmatmul_impl(const char* who, const itexhip_matmul_params* p, const void* a, const int8_t* packed_b,
+                 const int32_t* colsum, int64_t M, int64_t K, int64_t N, const float* row_min_a,
+                 const float* row_max_a, const float* min_b, const float* max_b, int64_t nb, const float* bias,
+                 void* out, void* stream) {
   itexhip_epilogue ep;
   if (int st = itexhip_qmatmul_epilogue_desc(p, nb, &ep)) return st;
   ITEXHIP_REQUIRE(nb == 1 || nb == N, "%s: %lld weight ranges for %lld channels", who, static_cast<long long>(nb),
@@ -451,7 +478,29 @@ extern "C" int itexhip_qmatmul(const itexhip_matmul_params* p, const void* a, co
   e.min_b = min_b;
   e.max_b = max_b;
   e.prep = make_prep_args(p, ep);
+  e.row_min_a = row_min_a;
+  e.row_max_a = row_max_a;
   return launch_packed(M <= 16, a, p->t_in, packed_b, M, K, N, e, p->t_out, out, stream, who);
+}
+}  // namespace
+
+extern "C" int itexhip_qmatmul(const itexhip_matmul_params* p, const void* a, const int8_t* packed_b,
+                               const int32_t* colsum, int64_t M, int64_t K, int64_t N, const float* min_b,
+                               const float* max_b, int64_t nb, const float* bias, void* out, void* stream) {
+  return qmatmul_impl("itexhip_qmatmul", p, a, packed_b, colsum, M, K, N, nullptr, nullptr, min_b, max_b, nb, bias, out,
+                      stream);
+}
+
+extern "C" int itexhip_qmatmul_per_row(const itexhip_matmul_params* p, const void* a, const int8_t* packed_b,
+                                       const int32_t* colsum, int64_t M, int64_t K, int64_t N,
+                                       const float* row_min_a, const float* row_max_a, const float* min_b,
+                                       const float* max_b, int64_t nb, const float* bias, void* out,
+                                       void* stream) {
+  ITEXHIP_REQUIRE(M <= 16, "itexhip_qmatmul_per_row: per-row activation ranges are implemented for M <= 16 (got %lld)",
+                  static_cast<long long>(M));
+  ITEXHIP_REQUIRE(M == 0 || (row_min_a && row_max_a), "itexhip_qmatmul_per_row: null row ranges");
+  return qmatmul_impl("itexhip_qmatmul_per_row", p, a, packed_b, colsum, M, K, N, row_min_a, row_max_a, min_b, max_b, nb,
+                      bias, out, stream);
 }
 
 extern "C" int itexhip_mfma_probe(int workgroups, int iters, const void* operands, int32_t* sink, void* stream) {

@@ -34,6 +34,10 @@ struct EpilogueArgs {
   const float* min_b;
   const float* max_b;
   PrepArgs prep;
+  // per-row activation ranges (decode batches quantized per token): row m uses row_min_a[m], row_max_a[m]
+  // in place of prep.min_a / prep.max_a; null for the reference's per-tensor range
+  const float* row_min_a;
+  const float* row_max_a;
 };
 
 // Scale, bias and zero-point compensation of channel n (n < N), however the call supplied them, in two

@@ -22,7 +22,7 @@ EXPORTS = [
     "itexhip_dequantize", "itexhip_dequantize_axis", "itexhip_requantize_per_channel",
     "itexhip_requantize", "itexhip_minmax_i32_per_channel", "itexhip_minmax_f32",
     "itexhip_qmatmul_epilogue_desc", "itexhip_qmatmul_prepare", "itexhip_qgemm_packed_bytes",
-    "itexhip_qgemm_prepack_b", "itexhip_qgemm", "itexhip_qgemm_tile", "itexhip_qgemv", "itexhip_qmatmul", "itexhip_mfma_probe",
+    "itexhip_qgemm_prepack_b", "itexhip_qgemm", "itexhip_qgemm_tile", "itexhip_qgemv", "itexhip_qmatmul", "itexhip_qmatmul_per_row", "itexhip_mfma_probe",
     "itexhip_qgemm_naive",
 ]
 
@@ -190,6 +190,12 @@ def qmatmul(p, a, packed_b, colsum, M, K, N, min_b, max_b, nb, bias, out, stream
     """The whole op in one launch (parameters derived inside the MatMul kernel)."""
     _check(_lib.itexhip_qmatmul(C.byref(p), _ptr(a), _ptr(packed_b), _ptr(colsum), _i64(M), _i64(K), _i64(N),
                                 _ptr(min_b), _ptr(max_b), _i64(nb), _ptr(bias), _ptr(out), _ptr(stream)))
+
+
+def qmatmul_per_row(p, a, packed_b, colsum, M, K, N, row_min_a, row_max_a, min_b, max_b, nb, bias, out, stream=0):
+    _check(_lib.itexhip_qmatmul_per_row(C.byref(p), _ptr(a), _ptr(packed_b), _ptr(colsum), _i64(M), _i64(K), _i64(N),
+                                        _ptr(row_min_a), _ptr(row_max_a), _ptr(min_b), _ptr(max_b), _i64(nb),
+                                        _ptr(bias), _ptr(out), _ptr(stream)))
 
 
 def mfma_probe(workgroups, iters, operands, sink, stream=0):

@@ -329,3 +329,37 @@ def test_llama_decode_gemv(hip, dev, M, K, N):
     ref = layer_zero_bias.oracle(xq, V2_DEQ, mn, mx)
     np.testing.assert_array_equal(layer_zero_bias.run(xq, V2_DEQ, mn, mx), ref)
     assert np.abs(ref - x @ w).max() < 0.2
+
+
+@pytest.mark.parametrize("M", [1, 3, 16])
+@pytest.mark.parametrize("kw", [V2_DEQ, V2_REQ_S8, V2_DEQ_RELU])
+@pytest.mark.parametrize("K,N", [(512, 272), (4096, 1024)])
+def test_per_token_activation_ranges(hip, dev, M, kw, K, N):
+    """Rows quantized with their own range: row m of the GPU result equals the oracle's 1 x K problem
+    with that row's (min, max).  The reference's MatMul ops have no per-row range; this is the decode
+    configuration's per-token quantization."""
+    import torch
+    layer, w, bias = make_layer(hip, dev, K, N, seed=K + N + 5)
+    rng = np.random.default_rng(M + K)
+    x = (rng.standard_normal((M, K)) * rng.uniform(0.3, 3.0, (M, 1))).astype(np.float32)
+    rows_q, mins, maxs = [], [], []
+    for m in range(M):
+        _, q, mn, mx = orc.quantize_v2(x[m:m + 1], x[m].min(), x[m].max(), orc.QUINT8, orc.MIN_FIRST)
+        rows_q.append(q)
+        mins.append(mn[0])
+        maxs.append(mx[0])
+    xq = np.concatenate(rows_q, 0)
+    full = x @ w + bias
+    r_out = float(np.abs(full).max())
+    ref = np.concatenate([layer.oracle(xq[m:m + 1], kw, mins[m], maxs[m], -r_out, r_out) for m in range(M)], 0)
+    p = hip.matmul_params(t_in=orc.QUINT8, min_a=0.0, max_a=0.0, min_out=-r_out, max_out=r_out, **kw)
+    out = torch.empty((M, N), dtype=tdt(kw["t_out"]), device=dev)
+    mins_d = torch.tensor(mins, dtype=torch.float32, device=dev)
+    maxs_d = torch.tensor(maxs, dtype=torch.float32, device=dev)
+    hip.qmatmul_per_row(p, torch.from_numpy(xq).to(dev), layer.packed, layer.colsum, M, K, N, mins_d, maxs_d,
+                        layer.min_b_d, layer.max_b_d, layer.min_b.size, layer.bias_d, out)
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(out.cpu().numpy(), ref)
+    with pytest.raises(hip.ItexHipError):
+        hip.qmatmul_per_row(p, torch.from_numpy(xq).to(dev), layer.packed, layer.colsum, 17, K, N, mins_d, maxs_d,
+                            layer.min_b_d, layer.max_b_d, layer.min_b.size, layer.bias_d, out)
