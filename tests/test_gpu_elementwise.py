@@ -313,3 +313,50 @@ def test_device_copy_kernel(hip, dev, nbytes, offset):
     expect = torch.zeros_like(dst)
     expect[offset:offset + nbytes] = src[offset:offset + nbytes]
     assert torch.equal(dst, expect)
+
+
+def test_more_than_2_31_elements(hip, dev):
+    """64-bit indexing: QuantizeV2, the range pass and Dequantize over 2^31 + 4099 elements.  Checked through
+    properties (no host copy of 8 GiB): the quantized tensor equals torch's own evaluation of the same
+    formula on slices at the start, across the 2^31 boundary and at the ragged end, and its checksum
+    over the whole tensor equals the sum of the checksums of the slices computed independently."""
+    import torch
+    n = (1 << 31) + 4099
+    free, _ = torch.cuda.mem_get_info()
+    if free < 14 * (1 << 30):
+        pytest.skip("needs ~14 GiB of free device memory")
+    x = torch.empty(n, dtype=torch.float32, device=dev)
+    piece = torch.randn(1 << 24, device=dev)
+    for off in range(0, n, 1 << 24):
+        m = min(1 << 24, n - off)
+        x[off:off + m] = piece[:m] * (1.0 + (off >> 24) * 0.01)
+    x[n - 1] = -77.0   # extreme values behind the 2^31 boundary
+    x[(1 << 31) + 5] = 91.0
+    mm = torch.zeros(2, dtype=torch.float32, device=dev)
+    hip.minmax_f32(x, n, mm)
+    torch.cuda.synchronize()
+    assert mm.cpu().tolist() == [-77.0, 91.0]
+    scale = np.float32(127.0) / np.float32(91.0)
+    q = torch.empty(n, dtype=torch.int8, device=dev)
+    hip.quantize(x, q, n, hip.QINT8, float(scale), 0.0)
+    torch.cuda.synchronize()
+    total = 0
+    for lo, hi in ((0, 1 << 20), ((1 << 31) - 4096, (1 << 31) + 4096), (n - 5000, n)):
+        ref = torch.clamp(torch.round(x[lo:hi] * float(scale)), -128, 127).to(torch.int8)
+        assert torch.equal(q[lo:hi], ref), (lo, hi)
+    for off in range(0, n, 1 << 28):
+        m = min(1 << 28, n - off)
+        ref = torch.clamp(torch.round(x[off:off + m] * float(scale)), -128, 127)
+        total += int(ref.sum(dtype=torch.float64).item())
+    got = 0
+    for off in range(0, n, 1 << 28):
+        m = min(1 << 28, n - off)
+        got += int(q[off:off + m].sum(dtype=torch.int64).item())
+    assert got == total
+    # Dequantize back into the same fp32 buffer (in place of x) and compare the ragged end
+    inv = np.float32(91.0) / np.float32(127.0)
+    q_tail = q[n - 5000:].clone()
+    hip.dequantize(q, x, n, hip.QINT8, float(inv), 0)
+    torch.cuda.synchronize()
+    assert torch.equal(x[n - 5000:], q_tail.to(torch.float32) * float(inv))
+    assert torch.equal(x[(1 << 31) - 8:(1 << 31) + 8], q[(1 << 31) - 8:(1 << 31) + 8].to(torch.float32) * float(inv))

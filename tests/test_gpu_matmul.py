@@ -363,3 +363,52 @@ def test_per_token_activation_ranges(hip, dev, M, kw, K, N):
     with pytest.raises(hip.ItexHipError):
         hip.qmatmul_per_row(p, torch.from_numpy(xq).to(dev), layer.packed, layer.colsum, 17, K, N, mins_d, maxs_d,
                             layer.min_b_d, layer.max_b_d, layer.min_b.size, layer.bias_d, out)
+
+
+def test_hip_graph_replays_match_eager(hip, dev):
+    """The op chain range pass -> QuantizeV2 -> single-launch MatMul captured once into a HIP graph and
+    replayed with new input contents: every replay must equal the eager result on the same input (eager
+    work and synchronisations sit between the replays)."""
+    import torch
+    M, K, N = 64, 512, 384
+    layer, w, bias = make_layer(hip, dev, K, N, seed=3)
+    kw = V2_DEQ_RELU
+    x_static = torch.zeros((M, K), dtype=torch.float32, device=dev)
+    xq = torch.empty((M, K), dtype=torch.uint8, device=dev)
+    mm = torch.zeros(2, dtype=torch.float32, device=dev)
+    out = torch.empty((M, N), dtype=torch.float32, device=dev)
+    # the activation range is fixed at capture time (the host-memory min/max of the ops are call arguments)
+    mn, mx = -4.0, 4.5
+    _, amn, amx = orc.adjust_input_range(mn, mx)
+    scale = orc.legacy_min_first_scale(orc.QUINT8, amn, amx)
+    addend = float(np.float32(-amn) * scale)
+    _, omn, omx, _, _ = orc.scale_zeropoint_align(orc.QUINT8, orc.MIN_FIRST, False, np.float32([amn]), np.float32([amx]))
+    p = hip.matmul_params(t_in=orc.QUINT8, min_a=float(amn), max_a=float(amx), **kw)
+
+    def chain(stream):
+        hip.minmax_f32(x_static, M * K, mm, stream)
+        hip.quantize(x_static, xq, M * K, hip.QUINT8, float(scale), addend, stream)
+        hip.qmatmul(p, xq, layer.packed, layer.colsum, M, K, N, layer.min_b_d, layer.max_b_d, layer.min_b.size,
+                    layer.bias_d, out, stream)
+
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.graph(graph, stream=side):
+        chain(torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    rng = np.random.default_rng(11)
+    for rep in range(4):
+        x = np.clip(rng.standard_normal((M, K)) * (1.0 + 0.3 * rep), -3.9, 4.4).astype(np.float32)
+        x_static.copy_(torch.from_numpy(x).to(dev))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        got, got_mm = out.cpu().numpy().copy(), mm.cpu().numpy().copy()
+        out.zero_()
+        chain(torch.cuda.current_stream().cuda_stream)  # eager, same buffers
+        torch.cuda.synchronize()
+        np.testing.assert_array_equal(got, out.cpu().numpy())
+        np.testing.assert_array_equal(got_mm, np.float32([x.min(), x.max()]))
+        _, xq_ref, _, _ = orc.quantize_v2(x, mn, mx, orc.QUINT8, orc.MIN_FIRST)
+        np.testing.assert_array_equal(got, layer.oracle(xq_ref, kw, amn, amx))
