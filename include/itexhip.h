@@ -62,6 +62,37 @@ int itexhip_stream_synchronize(void* stream);
 int itexhip_memcpy_d2d_async(void* dst_device, const void* src_device, size_t bytes, void* stream);
 
 /* ------------------------------------------------------------------------------------------
+ * Device runtime: what a StreamExecutor device plugin needs from HIP.  They stand where the reference
+ * calls its SYCL runtime wrappers ITEX_GPU* (itex/core/devices/gpu/gpu_device_plugin.cc:27-376:
+ * device count / handles :27-42, raw allocation under its BFC allocator :57-83, pinned host memory
+ * :85-97, streams :121-150, events :159-207, copies :233-297, synchronisation :299-316, fills :318-342,
+ * host callbacks :344-360).  Streams are created at the default priority.  Fills are kernels, so they
+ * can be captured into HIP graphs.
+ * ---------------------------------------------------------------------------------------- */
+int itexhip_device_count(int* count);
+int itexhip_device_info(int device, char* name, size_t name_len, char* pci_bus_id, size_t pci_len,
+                        int64_t* total_memory, int* compute_units);
+int itexhip_mem_info(int device, int64_t* free_bytes, int64_t* total_bytes);
+int itexhip_malloc(int device, size_t bytes, void** ptr);
+int itexhip_free(int device, void* ptr);
+int itexhip_host_malloc(size_t bytes, void** ptr); /* pinned */
+int itexhip_host_free(void* ptr);
+int itexhip_stream_create(int device, void** stream);
+int itexhip_stream_destroy(void* stream);
+int itexhip_stream_query(void* stream, int* done);
+int itexhip_event_create(int device, void** event);
+int itexhip_event_destroy(void* event);
+int itexhip_event_record(void* event, void* stream);
+int itexhip_event_query(void* event, int* done);
+int itexhip_event_synchronize(void* event);
+int itexhip_stream_wait_event(void* stream, void* event);
+int itexhip_device_synchronize(int device);
+int itexhip_memcpy_d2h_async(void* dst_host, const void* src_device, size_t bytes, void* stream);
+int itexhip_memset8_async(void* dst, uint8_t pattern, size_t bytes, void* stream);
+int itexhip_memset32_async(void* dst, uint32_t pattern, size_t bytes, void* stream);
+int itexhip_launch_host_func(void* stream, void (*fn)(void*), void* arg);
+
+/* ------------------------------------------------------------------------------------------
  * QuantizeV2.  q[i] = sat_T(rne(fl(x[i] * scale) + addend))
  *   SCALED            : addend = 0            (oneDNN reorder, src scale;
  *                                              itex/core/kernels/common/quantize_op.h:256-275,394)

@@ -18,6 +18,11 @@ ACT_NONE, ACT_RELU, ACT_RELU6, ACT_LEAKYRELU = 0, 1, 2, 3
 ELT_RELU, ELT_CLIP, ELT_LINEAR = 1, 2, 3
 
 EXPORTS = [
+    "itexhip_device_count", "itexhip_device_info", "itexhip_mem_info", "itexhip_malloc", "itexhip_free",
+    "itexhip_host_malloc", "itexhip_host_free", "itexhip_stream_create", "itexhip_stream_destroy",
+    "itexhip_stream_query", "itexhip_event_create", "itexhip_event_destroy", "itexhip_event_record",
+    "itexhip_event_query", "itexhip_event_synchronize", "itexhip_stream_wait_event", "itexhip_device_synchronize",
+    "itexhip_memcpy_d2h_async", "itexhip_memset8_async", "itexhip_memset32_async", "itexhip_launch_host_func",
     "itexhip_last_error", "itexhip_build_info", "itexhip_memcpy_h2d_async", "itexhip_memcpy_d2h", "itexhip_memcpy_d2d_async", "itexhip_stream_synchronize", "itexhip_quantize", "itexhip_quantize_axis",
     "itexhip_dequantize", "itexhip_dequantize_axis", "itexhip_requantize_per_channel",
     "itexhip_requantize", "itexhip_minmax_i32_per_channel", "itexhip_minmax_f32",

@@ -10,6 +10,10 @@ def build():
     out = os.path.join(HERE, "libmock_tf.so")
     subprocess.run(["g++", "-O1", "-g", "-std=c++17", "-fPIC", "-shared", "-Wall", "-I", os.path.join(ROOT, "include"),
                     os.path.join(HERE, "mock_tf.cc"), "-o", out, "-ldl"], check=True)
+    arena = os.path.join(HERE, "libarena_test.so")
+    subprocess.run(["g++", "-O1", "-g", "-std=c++17", "-fPIC", "-shared", "-Wall",
+                    "-I", os.path.join(ROOT, "intel-extension-for-tensorflow_amd", "plugin"),
+                    os.path.join(HERE, "arena_test_lib.cc"), "-o", arena], check=True)
     return out
 
 

@@ -152,3 +152,94 @@ def read_host(addr, dtype, shape):
     n = int(np.prod(shape, dtype=np.int64)) if len(shape) else 1
     buf = (C.c_char * (n * np.dtype(NP_OF[dtype]).itemsize)).from_address(addr)
     return np.frombuffer(buf, dtype=NP_OF[dtype]).reshape(shape).copy()
+
+
+# ------------------------------------------------------------------------------------------------
+# the StreamExecutor side of the plugin (SE_InitPlugin), driven like TensorFlow's PluggableDevice code
+# ------------------------------------------------------------------------------------------------
+class DevicePlugin:
+    """Device 0 of the plugin: its allocator, stream, copies and fills, through the function tables
+    SE_InitPlugin filled.  load_device() returns the process-wide instance."""
+
+    def __init__(self, lib):
+        self.lib = lib
+        lib.mock_device_error.restype = C.c_char_p
+        lib.mock_device_describe.restype = C.c_char_p
+        lib.mock_device_stream.restype = C.c_void_p
+        lib.mock_device_alloc.restype = C.c_void_p
+        lib.mock_device_alloc.argtypes = [C.c_uint64]
+        lib.mock_device_free.argtypes = [C.c_void_p]
+        lib.mock_device_host_alloc.restype = C.c_void_p
+        lib.mock_device_host_alloc.argtypes = [C.c_uint64]
+        lib.mock_device_host_free.argtypes = [C.c_void_p]
+        for f in (lib.mock_device_h2d, lib.mock_device_d2h, lib.mock_device_d2d):
+            f.argtypes = [C.c_void_p, C.c_void_p, C.c_uint64, C.c_int]
+        lib.mock_device_memset.argtypes = [C.c_void_p, C.c_int, C.c_uint32, C.c_uint64]
+        lib.mock_device_stats.argtypes = [C.POINTER(C.c_int64)]
+        lib.mock_device_stream_event_test.argtypes = [C.c_void_p, C.c_void_p, C.c_uint64, C.c_void_p]
+
+    def error(self):
+        return self.lib.mock_device_error().decode()
+
+    def describe(self):
+        return json.loads(self.lib.mock_device_describe().decode())
+
+    @property
+    def stream(self):
+        return self.lib.mock_device_stream() or 0
+
+    def alloc(self, nbytes):
+        p = self.lib.mock_device_alloc(int(nbytes))
+        if not p:
+            raise MemoryError("device allocation of %d bytes failed" % nbytes)
+        return p
+
+    def free(self, ptr):
+        self.lib.mock_device_free(ptr)
+
+    def upload(self, array, sync=False):
+        """Allocates device memory for `array` and copies it there; returns the device address."""
+        a = np.ascontiguousarray(array)
+        p = self.alloc(max(a.nbytes, 1))
+        rc = self.lib.mock_device_h2d(p, a.ctypes.data, a.nbytes, int(sync))
+        assert rc == 0, self.error()
+        if not sync:
+            self.sync()  # `a` may be a temporary
+        return p
+
+    def download(self, ptr, dtype, shape, sync=False):
+        out = np.empty(shape, dtype)
+        rc = self.lib.mock_device_d2h(out.ctypes.data, ptr, out.nbytes, int(sync))
+        assert rc == 0, self.error()
+        if not sync:
+            self.sync()
+        return out
+
+    def copy(self, dst, src, nbytes, sync=False):
+        assert self.lib.mock_device_d2d(dst, src, int(nbytes), int(sync)) == 0, self.error()
+
+    def memset(self, ptr, kind, pattern, nbytes):
+        assert self.lib.mock_device_memset(ptr, kind, pattern, int(nbytes)) == 0, self.error()
+
+    def sync(self, everything=False):
+        assert self.lib.mock_device_sync(int(everything)) == 0, self.error()
+
+    def stats(self):
+        out = (C.c_int64 * 8)()
+        assert self.lib.mock_device_stats(out) == 0
+        return dict(zip(("num_allocs", "bytes_in_use", "peak_bytes_in_use", "largest_alloc_size", "bytes_reserved",
+                         "largest_free_block_bytes", "device_free", "device_total"), out))
+
+    def use_for_tensors(self):
+        """Outputs, temporaries and host-pinned tensors of the mock now come from the plugin's allocators."""
+        self.lib.mock_device_use_allocator()
+
+
+def load_device(ordinal=0):
+    """SE_InitPlugin + device / stream executor / stream creation; returns (rc, DevicePlugin).  rc 4 means
+    the plugin initialised but reports no device with that ordinal (no GPU in this process)."""
+    lib = load()
+    if "devplug" not in _state:
+        _state["devplug"] = DevicePlugin(lib)
+        _state["devplug_rc"] = lib.mock_device_load(PLUGIN_LIB.encode(), ordinal)
+    return _state["devplug_rc"], _state["devplug"]

@@ -2,12 +2,13 @@
 // include/tf_c_api_subset.h over plain memory, records kernel and op registrations, and drives
 // create / compute / delete of a kernel the way TensorFlow's C kernel wrapper does.  Test
 // infrastructure only; it allocates device memory through a callback supplied by the test (PyTorch)
-// or, without one, from the host heap.
+// or from the device plugin's own allocator (mock_device_*), or, without either, from the host heap.
 #include <dlfcn.h>
 
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <ctime>
 #include <map>
 #include <memory>
 #include <sstream>
@@ -15,6 +16,7 @@
 #include <vector>
 
 #include "tf_c_api_subset.h"
+#include "tf_stream_executor_subset.h"
 
 // ------------------------------------------------------------------------------------------------
 // object definitions
@@ -418,6 +420,209 @@ void TF_ShapeInferenceContextSetUnknownShape(TF_ShapeInferenceContext* ctx, TF_S
 void mock_set_allocator(AllocFn a, FreeFn f) { g_alloc = a; g_free = f; }
 void mock_add_stock_op(const char* name) { g_stock_ops.emplace_back(name); }
 int mock_delete_calls(void) { return g_delete_calls; }
+
+// ---- the StreamExecutor side: what TensorFlow does with a PluggableDevice plugin after dlopen -----
+namespace {
+struct DevicePlugin {
+  bool loaded = false;
+  SE_PlatformRegistrationParams params{};
+  SP_Platform platform{};
+  SP_PlatformFns fns{};
+  SP_Device device{};
+  SP_DeviceFns device_fns{};
+  SP_StreamExecutor se{};
+  SP_TimerFns timer_fns{};
+  SP_Stream stream = nullptr;
+  std::string last_error;
+} g_dev;
+
+void* DeviceAlloc(size_t bytes, int on_host) {
+  if (on_host) return g_dev.se.host_memory_allocate(&g_dev.device, bytes);
+  SP_DeviceMemoryBase m{};
+  g_dev.se.allocate(&g_dev.device, bytes, 0, &m);
+  return m.opaque;
+}
+void DeviceFree(void* p, int on_host) {
+  if (on_host) { g_dev.se.host_memory_deallocate(&g_dev.device, p); return; }
+  SP_DeviceMemoryBase m{};
+  m.struct_size = SP_DEVICE_MEMORY_BASE_STRUCT_SIZE;
+  m.opaque = p;
+  g_dev.se.deallocate(&g_dev.device, &m);
+}
+int Check(TF_Status& st, const char* what) {
+  if (st.code == TF_OK) return 0;
+  g_dev.last_error = std::string(what) + ": " + st.msg;
+  return static_cast<int>(st.code);
+}
+}  // namespace
+
+// dlopen the plugin, call SE_InitPlugin, create device `ordinal`, its stream executor and one stream.
+// 0 on success; the struct sizes the plugin reports must be the ones of the API header.
+int mock_device_load(const char* path, int ordinal) {
+  void* h = dlopen(path, RTLD_NOW | RTLD_GLOBAL);
+  if (!h) { g_dev.last_error = std::string("dlopen failed: ") + dlerror(); return 1; }
+  auto init = reinterpret_cast<void (*)(SE_PlatformRegistrationParams*, TF_Status*)>(dlsym(h, "SE_InitPlugin"));
+  if (!init) { g_dev.last_error = "SE_InitPlugin not exported"; return 2; }
+  g_dev.params = SE_PlatformRegistrationParams{};
+  g_dev.params.struct_size = SE_PLATFORM_REGISTRATION_PARAMS_STRUCT_SIZE;
+  g_dev.platform.struct_size = SP_PLATFORM_STRUCT_SIZE;
+  g_dev.fns.struct_size = SP_PLATFORM_FNS_STRUCT_SIZE;
+  g_dev.params.platform = &g_dev.platform;
+  g_dev.params.platform_fns = &g_dev.fns;
+  TF_Status st;
+  init(&g_dev.params, &st);
+  if (int rc = Check(st, "SE_InitPlugin")) return rc;
+  if (g_dev.platform.struct_size != SP_PLATFORM_STRUCT_SIZE || g_dev.fns.struct_size != SP_PLATFORM_FNS_STRUCT_SIZE ||
+      !g_dev.platform.name || !g_dev.platform.type || !g_dev.fns.create_device || !g_dev.fns.create_stream_executor) {
+    g_dev.last_error = "SE_InitPlugin left the platform tables incomplete";
+    return 3;
+  }
+  int count = 0;
+  g_dev.fns.get_device_count(&g_dev.platform, &count, &st);
+  if (int rc = Check(st, "get_device_count")) return rc;
+  if (ordinal >= count) { g_dev.last_error = "no such device"; return 4; }
+  SE_CreateDeviceParams dp{};
+  dp.struct_size = SE_CREATE_DEVICE_PARAMS_STRUCT_SIZE;
+  dp.ordinal = ordinal;
+  dp.device = &g_dev.device;
+  g_dev.device.struct_size = SP_DEVICE_STRUCT_SIZE;
+  g_dev.fns.create_device(&g_dev.platform, &dp, &st);
+  if (int rc = Check(st, "create_device")) return rc;
+  SE_CreateDeviceFnsParams fp{};
+  fp.struct_size = SE_CREATE_DEVICE_FNS_PARAMS_STRUCT_SIZE;
+  fp.device_fns = &g_dev.device_fns;
+  g_dev.fns.create_device_fns(&g_dev.platform, &fp, &st);
+  if (int rc = Check(st, "create_device_fns")) return rc;
+  SE_CreateStreamExecutorParams sp{};
+  sp.struct_size = SE_CREATE_STREAM_EXECUTOR_PARAMS_STRUCT_SIZE;
+  sp.stream_executor = &g_dev.se;
+  g_dev.fns.create_stream_executor(&g_dev.platform, &sp, &st);
+  if (int rc = Check(st, "create_stream_executor")) return rc;
+  if (g_dev.se.struct_size != SP_STREAMEXECUTOR_STRUCT_SIZE) { g_dev.last_error = "stream executor struct size"; return 5; }
+  g_dev.fns.create_timer_fns(&g_dev.platform, &g_dev.timer_fns, &st);
+  if (int rc = Check(st, "create_timer_fns")) return rc;
+  g_dev.se.create_stream(&g_dev.device, &g_dev.stream, &st);
+  if (int rc = Check(st, "create_stream")) return rc;
+  g_dev.loaded = true;
+  return 0;
+}
+const char* mock_device_error(void) { return g_dev.last_error.c_str(); }
+const char* mock_device_describe(void) {
+  static std::string s;
+  std::ostringstream os;
+  os << "{\"platform_name\":\"" << g_dev.platform.name << "\",\"platform_type\":\"" << g_dev.platform.type
+     << "\",\"use_bfc_allocator\":" << int(g_dev.platform.use_bfc_allocator) << ",\"ordinal\":" << g_dev.device.ordinal
+     << ",\"hardware_name\":\"" << (g_dev.device.hardware_name ? g_dev.device.hardware_name : "") << "\",\"vendor\":\""
+     << (g_dev.device.device_vendor ? g_dev.device.device_vendor : "") << "\",\"pci_bus_id\":\""
+     << (g_dev.device.pci_bus_id ? g_dev.device.pci_bus_id : "") << "\",\"memory_bandwidth\":"
+     << (g_dev.device_fns.get_memory_bandwidth ? g_dev.device_fns.get_memory_bandwidth(&g_dev.device) : -1) << "}";
+  s = os.str();
+  return s.c_str();
+}
+// from now on the mock's device and host-pinned tensors come from the plugin's allocators and kernels
+// get the plugin's stream
+void mock_device_use_allocator(void) { g_alloc = DeviceAlloc; g_free = DeviceFree; }
+void* mock_device_stream(void) { return g_dev.stream ? g_dev.stream->stream_handle : nullptr; }
+void* mock_device_alloc(uint64_t bytes) { return DeviceAlloc(bytes, 0); }
+void mock_device_free(void* p) { DeviceFree(p, 0); }
+void* mock_device_host_alloc(uint64_t bytes) { return DeviceAlloc(bytes, 1); }
+void mock_device_host_free(void* p) { DeviceFree(p, 1); }
+static SP_DeviceMemoryBase Mem(void* p, uint64_t n) {
+  SP_DeviceMemoryBase m{};
+  m.struct_size = SP_DEVICE_MEMORY_BASE_STRUCT_SIZE;
+  m.opaque = p;
+  m.size = n;
+  return m;
+}
+int mock_device_h2d(void* dst, const void* src, uint64_t n, int sync) {
+  TF_Status st;
+  SP_DeviceMemoryBase m = Mem(dst, n);
+  if (sync) g_dev.se.sync_memcpy_htod(&g_dev.device, &m, src, n, &st);
+  else g_dev.se.memcpy_htod(&g_dev.device, g_dev.stream, &m, src, n, &st);
+  return Check(st, "memcpy_htod");
+}
+int mock_device_d2h(void* dst, const void* src, uint64_t n, int sync) {
+  TF_Status st;
+  SP_DeviceMemoryBase m = Mem(const_cast<void*>(src), n);
+  if (sync) g_dev.se.sync_memcpy_dtoh(&g_dev.device, dst, &m, n, &st);
+  else g_dev.se.memcpy_dtoh(&g_dev.device, g_dev.stream, dst, &m, n, &st);
+  return Check(st, "memcpy_dtoh");
+}
+int mock_device_d2d(void* dst, const void* src, uint64_t n, int sync) {
+  TF_Status st;
+  SP_DeviceMemoryBase d = Mem(dst, n), s = Mem(const_cast<void*>(src), n);
+  if (sync) g_dev.se.sync_memcpy_dtod(&g_dev.device, &d, &s, n, &st);
+  else g_dev.se.memcpy_dtod(&g_dev.device, g_dev.stream, &d, &s, n, &st);
+  return Check(st, "memcpy_dtod");
+}
+int mock_device_memset(void* dst, int kind, uint32_t pattern, uint64_t n) {  // kind 0: zero, 8: byte, 32: word
+  TF_Status st;
+  SP_DeviceMemoryBase m = Mem(dst, n);
+  if (kind == 0) g_dev.se.mem_zero(&g_dev.device, g_dev.stream, &m, n, &st);
+  else if (kind == 8) g_dev.se.memset(&g_dev.device, g_dev.stream, &m, static_cast<uint8_t>(pattern), n, &st);
+  else g_dev.se.memset32(&g_dev.device, g_dev.stream, &m, pattern, n, &st);
+  return Check(st, "memset");
+}
+int mock_device_sync(int all) {
+  TF_Status st;
+  if (all) g_dev.se.synchronize_all_activity(&g_dev.device, &st);
+  else g_dev.se.block_host_until_done(&g_dev.device, g_dev.stream, &st);
+  return Check(st, "synchronize");
+}
+int mock_device_stats(int64_t* out /* 8 values */) {
+  SP_AllocatorStats s{};
+  if (!g_dev.se.get_allocator_stats(&g_dev.device, &s)) return 1;
+  out[0] = s.num_allocs; out[1] = s.bytes_in_use; out[2] = s.peak_bytes_in_use; out[3] = s.largest_alloc_size;
+  out[4] = s.bytes_reserved; out[5] = s.largest_free_block_bytes;
+  int64_t f = 0, t = 0;
+  if (!g_dev.se.device_memory_usage(&g_dev.device, &f, &t)) return 2;
+  out[6] = f; out[7] = t;
+  return 0;
+}
+// A second stream that must wait for the first (create_stream_dependency), an event recorded behind the
+// work, a host callback behind the event: returns 0 when the callback ran after the event completed and
+// the data written on the first stream was visible to the copy on the second.
+namespace { volatile int g_callback_ran = 0; void Callback(void* arg, TF_Status* st) { g_callback_ran = *static_cast<int*>(arg); TF_SetStatus(st, TF_OK, ""); } }
+int mock_device_stream_event_test(void* dev_buf, void* dev_buf2, uint64_t n, void* host_out) {
+  TF_Status st;
+  SP_Stream second = nullptr;
+  g_dev.se.create_stream(&g_dev.device, &second, &st);
+  if (int rc = Check(st, "create_stream")) return rc;
+  SP_Event ev = nullptr;
+  g_dev.se.create_event(&g_dev.device, &ev, &st);
+  if (int rc = Check(st, "create_event")) return rc;
+  SP_DeviceMemoryBase a = Mem(dev_buf, n), b = Mem(dev_buf2, n);
+  g_dev.se.memset(&g_dev.device, g_dev.stream, &a, 0x5a, n, &st);                  // stream 1: fill a
+  g_dev.se.create_stream_dependency(&g_dev.device, second, g_dev.stream, &st);     // stream 2 waits for stream 1
+  if (int rc = Check(st, "create_stream_dependency")) return rc;
+  g_dev.se.memcpy_dtod(&g_dev.device, second, &b, &a, n, &st);                     // stream 2: b = a
+  g_dev.se.record_event(&g_dev.device, second, ev, &st);
+  if (int rc = Check(st, "record_event")) return rc;
+  g_dev.se.wait_for_event(&g_dev.device, g_dev.stream, ev, &st);                   // stream 1 waits for the copy
+  if (int rc = Check(st, "wait_for_event")) return rc;
+  g_dev.se.memcpy_dtoh(&g_dev.device, g_dev.stream, host_out, &b, n, &st);         // stream 1: read b back
+  static int token = 7;
+  g_callback_ran = 0;
+  if (!g_dev.se.host_callback(&g_dev.device, g_dev.stream, Callback, &token)) return 100;
+  g_dev.se.block_host_for_event(&g_dev.device, ev, &st);
+  if (int rc = Check(st, "block_host_for_event")) return rc;
+  if (g_dev.se.get_event_status(&g_dev.device, ev) != SE_EVENT_COMPLETE) return 101;
+  g_dev.se.block_host_until_done(&g_dev.device, g_dev.stream, &st);
+  if (int rc = Check(st, "block_host_until_done")) return rc;
+  g_dev.se.get_stream_status(&g_dev.device, g_dev.stream, &st);
+  if (int rc = Check(st, "get_stream_status")) return rc;
+  for (int spin = 0; spin < 2000 && g_callback_ran != 7; ++spin) {  // the callback runs on a runtime thread
+    struct timespec ts = {0, 1000000};
+    nanosleep(&ts, nullptr);
+  }
+  SP_Timer timer = nullptr;
+  g_dev.se.create_timer(&g_dev.device, &timer, &st);  // documented as unimplemented
+  const bool timer_unimplemented = st.code == TF_UNIMPLEMENTED && g_dev.timer_fns.nanoseconds(timer) == 0;
+  g_dev.se.destroy_event(&g_dev.device, ev);
+  g_dev.se.destroy_stream(&g_dev.device, second);
+  if (g_callback_ran != 7) return 102;
+  return timer_unimplemented ? 0 : 103;
+}
 
 // dlopen the plugin and call its TF_InitKernel, as TensorFlow does
 int mock_load_plugin(const char* path) {

@@ -157,3 +157,14 @@ def test_matmul_shape_validation_before_device_work():
     code, msg, _ = n.run(ins, [(tf.FLOAT, False)])
     assert code == tf.INVALID_ARGUMENT and "Matrix size-incompatible" in msg
     n.close()
+
+
+def test_se_init_plugin_without_a_gpu():
+    """SE_InitPlugin is exported and fills the platform tables; with no GPU in the process the device
+    count is 0 and device creation is refused cleanly (rc 4 = no such ordinal)."""
+    import torch
+    rc, plug = tf.load_device()
+    if torch.cuda.is_available():
+        assert rc == 0, plug.error()
+    else:
+        assert rc == 4, (rc, plug.error())
