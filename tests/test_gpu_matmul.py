@@ -268,7 +268,7 @@ def test_signed_activations_and_extremes(hip, dev):
 
 
 def test_config1_literal(hip, dev):
-    """BASELINE config 1: SCALED qint8 activations, per-channel weights, fp32 bias,
+    """The single quantized linear of the reference's CPU-runnable case: SCALED qint8 activations, per-channel weights, fp32 bias,
     [BiasAdd, Relu, Requantize] -> quint8, V1 and V2 spellings agree with the oracle (including the
     reference's as-written bias scaling and dropped requantize factor)."""
     M, K, N = 128, 1024, 1024
@@ -284,7 +284,7 @@ def test_config1_literal(hip, dev):
 
 @pytest.mark.parametrize("K,N,relu", [(768, 2304, False), (768, 768, False), (768, 3072, True), (3072, 768, False)])
 def test_bert_linears_rows_sampled(hip, dev, K, N, relu):
-    """BASELINE config 2 at full size (M = 4096); the oracle checks 96 sampled rows exactly."""
+    """BERT-base encoder linears at full size (M = 4096); the oracle checks 96 sampled rows exactly."""
     M = 4096
     layer, w, bias = make_layer(hip, dev, K, N, seed=K * 3 + N)
     x, xq, mn, mx = make_acts(M, K, seed=1)
@@ -299,7 +299,7 @@ def test_bert_linears_rows_sampled(hip, dev, K, N, relu):
 
 @pytest.mark.parametrize("K,N", [(4096, 4096), (4096, 6144), (4096, 14336), (14336, 4096)])
 def test_llama_prefill_rows_sampled(hip, dev, K, N):
-    """BASELINE config 4 at full size (M = 2048): int8 output bit-exact on 64 sampled rows, and the
+    """Llama-3-8B prefill linears at full size (M = 2048): int8 output bit-exact on 64 sampled rows, and the
     size-independent property sum_n acc[m, n] = a[m, :] . rowsum(w) on the s32 output of all rows."""
     import torch
     M = 2048
@@ -322,7 +322,7 @@ def test_llama_prefill_rows_sampled(hip, dev, K, N):
 @pytest.mark.parametrize("M", [1, 4, 16])
 @pytest.mark.parametrize("K,N", [(4096, 14336), (14336, 4096)])
 def test_llama_decode_gemv(hip, dev, M, K, N):
-    """BASELINE config 3 at full size, every output checked against the oracle."""
+    """Llama-3-8B decode shapes at full size, every output checked against the oracle."""
     layer, w, bias = make_layer(hip, dev, K, N, seed=10 + M)
     layer_zero_bias = Linear(hip, dev, layer.wq, layer.min_b, layer.max_b, np.zeros(N, np.float32))
     x, xq, mn, mx = make_acts(M, K, seed=11 + M)
