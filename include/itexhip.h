@@ -154,8 +154,12 @@ enum {
   ITEXHIP_API_V1 = 1,     /* QuantizedFusedMatMulOp   (:1539-1708) */
   ITEXHIP_API_LEGACY = 2  /* QuantizedMatMulOp / QuantizedMatMulReluOp (:1412-1531) */
 };
-enum { ITEXHIP_ACT_NONE = 0, ITEXHIP_ACT_RELU = 1, ITEXHIP_ACT_RELU6 = 2, ITEXHIP_ACT_LEAKYRELU = 3 };
-enum { ITEXHIP_ELT_RELU = 1, ITEXHIP_ELT_CLIP = 2, ITEXHIP_ELT_LINEAR = 3 };
+enum { ITEXHIP_ACT_NONE = 0, ITEXHIP_ACT_RELU = 1, ITEXHIP_ACT_RELU6 = 2, ITEXHIP_ACT_LEAKYRELU = 3,
+       ITEXHIP_ACT_GELU_APPROX = 4, ITEXHIP_ACT_GELU_EXACT = 5 };
+/* post-ops of the epilogue chain (itex/core/utils/onednn/onednn_post_op_util.cc:34-68); SUM is the
+ * "Add" fusion: y += alpha * addend[m, n] */
+enum { ITEXHIP_ELT_RELU = 1, ITEXHIP_ELT_CLIP = 2, ITEXHIP_ELT_LINEAR = 3, ITEXHIP_ELT_GELU_TANH = 4,
+       ITEXHIP_ELT_GELU_ERF = 5, ITEXHIP_ELT_SUM = 6 };
 
 typedef struct {
   int alg;      /* ITEXHIP_ELT_* */
@@ -167,8 +171,8 @@ typedef struct {
  *   y = fl(fl((float)acc * scale[n]) + bias[n]); eltwise chain; convert to the output type. */
 typedef struct {
   int n_scales;   /* 0: no scale, 1: scales[0] for all channels, N: per output channel */
-  int n_eltwise;  /* 0..2 */
-  itexhip_eltwise elt[2];
+  int n_eltwise;  /* 0..3, in fused_ops order */
+  itexhip_eltwise elt[3];
 } itexhip_epilogue;
 
 /* Attributes and host-memory scalars of one quantized MatMul node. */
@@ -185,6 +189,8 @@ typedef struct {
   float leakyrelu_alpha;
   float min_a, max_a;      /* host scalars */
   float min_out, max_out;  /* min/max_freezed_output (requantize) */
+  int add_position;        /* "Add" in fused_ops: 0 absent, 1 before the activation, 2 after it (fp32 output only) */
+  int t_bias;              /* Tbias: 0 or ITEXHIP_FLOAT = fp32, ITEXHIP_QINT32 = qint32 (:1153-1334) */
 } itexhip_matmul_params;
 
 /* Host-only: the epilogue descriptor (scale count, eltwise chain with the reference's alpha/beta
@@ -195,11 +201,11 @@ int itexhip_qmatmul_epilogue_desc(const itexhip_matmul_params* p, int64_t nb, it
 
 /* Device: per-channel output scales and the scaled / zero-point-compensated bias
  * (ExtendInt8PostOps as above; GetScaledBias, quantized_matmul_common.h:466-660), computed by one
- * small kernel from device copies of min_b / max_b (nb floats each), the fp32 bias (N floats) and
+ * small kernel from device copies of min_b / max_b (nb floats each), the bias (N floats, or N int32 when p->t_bias is QINT32) and
  * the weight column sums (N int32, from itexhip_qgemm_prepack_b).  Writes `scales_out`
  * (max(ep.n_scales,1) floats) and `bias_out` (N floats).  No host synchronisation. */
 int itexhip_qmatmul_prepare(const itexhip_matmul_params* p, const float* min_b, const float* max_b,
-                            int64_t nb, const float* bias, const int32_t* colsum, int64_t N,
+                            int64_t nb, const void* bias, const int32_t* colsum, int64_t N,
                             float* scales_out, float* bias_out, void* stream);
 
 /* Weight prepack: the s8 weight (TF layout [K,N] row-major, or [N,K] when transpose_b) is
@@ -232,10 +238,13 @@ int itexhip_qgemv(const void* a, int a_type, const int8_t* packed_b, const int32
  * kernel derives each channel's output scale and bias itself from the op's ranges (the same fp32
  * operation sequence), so no parameter vectors and no second kernel are needed.  This is what the
  * op kernel calls per Compute (quantized_matmul_common.h:62-460: Init + primitive execute);
- * a changed min_a / max_a costs nothing extra.  `bias` is the op's raw fp32 bias (may be null). */
+ * a changed min_a / max_a costs nothing extra.  `bias` is the op's raw bias (fp32, or int32 when
+ * p->t_bias is QINT32; may be null).  `addend` is the [M, N] fp32 tensor of the "Add" fusion
+ * (p->add_position != 0; the reference adds it in place into the output buffer, :352-389), else null. */
 int itexhip_qmatmul(const itexhip_matmul_params* p, const void* a, const int8_t* packed_b,
                     const int32_t* colsum, int64_t M, int64_t K, int64_t N, const float* min_b,
-                    const float* max_b, int64_t nb, const float* bias, void* out, void* stream);
+                    const float* max_b, int64_t nb, const void* bias, const float* addend, void* out,
+                    void* stream);
 
 /* Decode batches quantized per token: row m of `a` was quantized with its own range
  * (row_min_a[m], row_max_a[m]; device arrays of M floats, e.g. from QuantizeV2 with axis = 0,
@@ -246,7 +255,14 @@ int itexhip_qmatmul(const itexhip_matmul_params* p, const void* a, const int8_t*
 int itexhip_qmatmul_per_row(const itexhip_matmul_params* p, const void* a, const int8_t* packed_b,
                             const int32_t* colsum, int64_t M, int64_t K, int64_t N, const float* row_min_a,
                             const float* row_max_a, const float* min_b, const float* max_b, int64_t nb,
-                            const float* bias, void* out, void* stream);
+                            const void* bias, const float* addend, void* out, void* stream);
+
+/* itexhip_qmatmul on the unpacked TF-layout weight ([K, N], or [N, K] with transpose_b), any K, no
+ * prepack and no column-sum buffer: one thread per output element.  For the shapes the MFMA kernels
+ * do not take (K not a multiple of 16). */
+int itexhip_qmatmul_unpacked(const itexhip_matmul_params* p, const void* a, const int8_t* w, int transpose_b,
+                             int64_t M, int64_t K, int64_t N, const float* min_b, const float* max_b,
+                             int64_t nb, const void* bias, const float* addend, void* out, void* stream);
 
 /* Same contract on the unpacked TF-layout weight, any shape (no alignment requirements): one
  * thread per output element.  Used for shapes the tile kernels do not cover (K not a multiple of

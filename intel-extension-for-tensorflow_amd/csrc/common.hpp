@@ -71,6 +71,12 @@ __device__ __forceinline__ float apply_eltwise(const itexhip_eltwise& e, float x
       return fminf(fmaxf(x, e.alpha), e.beta);
     case ITEXHIP_ELT_LINEAR:
       return e.alpha * x + e.beta;
+    case ITEXHIP_ELT_GELU_TANH: {  // 0.5 x (1 + tanh(sqrt(2/pi) x (1 + 0.044715 x^2)))
+      const float v = tanhf(0.79788458347320556640625f * x * (1.0f + 0.044715f * x * x));
+      return 0.5f * x * (1.0f + v);
+    }
+    case ITEXHIP_ELT_GELU_ERF:  // 0.5 x (1 + erf(x / sqrt(2)))
+      return 0.5f * x * (1.0f + erff(x * 0.707106769084930419921875f));
     default:
       return x;
   }

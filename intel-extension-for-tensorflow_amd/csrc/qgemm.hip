@@ -266,8 +266,41 @@ __global__ __launch_bounds__(256) void qgemm_naive_kernel(const uint8_t* __restr
   float v = static_cast<float>(acc);
   if (e.n_scales == 1) v = v * e.scales[0];
   else if (e.n_scales > 1) v = v * e.scales[n];
-  if (e.bias) v = v + e.bias[n];
-  for (int k = 0; k < e.n_eltwise; ++k) v = apply_eltwise(e.elt[k], v);
+  if (e.bias) v = v + static_cast<const float*>(e.bias)[n];
+  for (int k = 0; k < e.n_eltwise; ++k) v = apply_eltwise(e.elt[k], v);  // no sum post-op on this path
+  if constexpr (OUT_T == ITEXHIP_FLOAT) reinterpret_cast<float*>(out)[idx] = v;
+  else if constexpr (OUT_T == ITEXHIP_QINT32) reinterpret_cast<int32_t*>(out)[idx] = sat_rne<ITEXHIP_QINT32>(v);
+  else reinterpret_cast<uint8_t*>(out)[idx] = static_cast<uint8_t>(sat_rne<OUT_T>(v));
+}
+
+// The whole op on the unpacked weight, any K: the thread also sums its weight column (the zero-point
+// compensation needs it) and derives the channel's scale and bias like the packed kernels do.
+template <int OUT_T>
+__global__ __launch_bounds__(256) void qmatmul_unpacked_kernel(const uint8_t* __restrict__ a, int a_is_u8,
+                                                                const int8_t* __restrict__ w, int transpose_b,
+                                                                int M, int K, int N, EpilogueArgs e,
+                                                                void* __restrict__ out) {
+  const int64_t idx = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (idx >= static_cast<int64_t>(M) * N) return;
+  const int m = static_cast<int>(idx / N), n = static_cast<int>(idx % N);
+  int acc = 0, wsum = 0;
+  for (int k = 0; k < K; ++k) {
+    const int av = a_is_u8 ? static_cast<int>(a[static_cast<int64_t>(m) * K + k])
+                           : static_cast<int>(reinterpret_cast<const int8_t*>(a)[static_cast<int64_t>(m) * K + k]);
+    const int wv = transpose_b ? w[static_cast<int64_t>(n) * K + k] : w[static_cast<int64_t>(k) * N + n];
+    acc += av * wv;
+    wsum += wv;
+  }
+  const int jb = (e.nb == N) ? n : 0;
+  const ChannelScaleBias c = channel_scale_bias(e.prep, e.min_b[jb], e.max_b[jb], e.min_b[0], e.max_b[0],
+                                                bias_entry(e.prep, e.bias, n), wsum);
+  float v = static_cast<float>(acc);
+  if (e.n_scales > 0) v = v * c.scale;
+  v = v + c.bias;
+  for (int k = 0; k < e.n_eltwise; ++k) {
+    if (e.elt[k].alg == ITEXHIP_ELT_SUM) v = v + e.elt[k].alpha * e.addend[idx];
+    else v = apply_eltwise(e.elt[k], v);
+  }
   if constexpr (OUT_T == ITEXHIP_FLOAT) reinterpret_cast<float*>(out)[idx] = v;
   else if constexpr (OUT_T == ITEXHIP_QINT32) reinterpret_cast<int32_t*>(out)[idx] = sat_rne<ITEXHIP_QINT32>(v);
   else reinterpret_cast<uint8_t*>(out)[idx] = static_cast<uint8_t>(sat_rne<OUT_T>(v));
@@ -286,7 +319,9 @@ int check_common(const void* a, int a_type, const void* b, int64_t M, int64_t K,
   ITEXHIP_REQUIRE(M < (1LL << 31) && N < (1LL << 31) && K <= kMaxK, "%s: dimension too large (K <= %lld)", who,
                   static_cast<long long>(kMaxK));
   ITEXHIP_REQUIRE(ep != nullptr, "%s: null epilogue", who);
-  ITEXHIP_REQUIRE(ep->n_eltwise >= 0 && ep->n_eltwise <= 2, "%s: bad eltwise count", who);
+  ITEXHIP_REQUIRE(ep->n_eltwise >= 0 && ep->n_eltwise <= 3, "%s: bad eltwise count", who);
+  for (int k = 0; k < ep->n_eltwise; ++k)
+    ITEXHIP_REQUIRE(ep->elt[k].alg != ITEXHIP_ELT_SUM, "%s: the Add fusion needs itexhip_qmatmul (it takes the addend)", who);
   ITEXHIP_REQUIRE(ep->n_scales == 0 || ep->n_scales == 1 || ep->n_scales == N,
                   "%s: %d scales for %lld channels", who, ep->n_scales, static_cast<long long>(N));
   if (M == 0 || N == 0) return ITEXHIP_OK;
@@ -296,7 +331,7 @@ int check_common(const void* a, int a_type, const void* b, int64_t M, int64_t K,
   return ITEXHIP_OK;
 }
 
-EpilogueArgs make_args(int a_type, const int32_t* colsum, const float* scales, const float* bias,
+EpilogueArgs make_args(int a_type, const int32_t* colsum, const float* scales, const void* bias,
                        const itexhip_epilogue* ep) {
   EpilogueArgs e{};
   e.scales = scales;
@@ -307,6 +342,7 @@ EpilogueArgs make_args(int a_type, const int32_t* colsum, const float* scales, c
   e.n_eltwise = ep->n_eltwise;
   e.elt[0] = ep->elt[0];
   e.elt[1] = ep->elt[1];
+  e.elt[2] = ep->elt[2];
   return e;
 }
 
@@ -459,8 +495,8 @@ extern "C" int itexhip_qgemm_naive(const void* a, int a_type, const int8_t* w, i
 namespace {
 int qmatmul_impl(const char* who, const itexhip_matmul_params* p, const void* a, const int8_t* packed_b,
                  const int32_t* colsum, int64_t M, int64_t K, int64_t N, const float* row_min_a,
-                 const float* row_max_a, const float* min_b, const float* max_b, int64_t nb, const float* bias,
-                 void* out, void* stream) {
+                 const float* row_max_a, const float* min_b, const float* max_b, int64_t nb, const void* bias,
+                 const float* addend, void* out, void* stream) {
   itexhip_epilogue ep;
   if (int st = itexhip_qmatmul_epilogue_desc(p, nb, &ep)) return st;
   ITEXHIP_REQUIRE(nb == 1 || nb == N, "%s: %lld weight ranges for %lld channels", who, static_cast<long long>(nb),
@@ -472,6 +508,7 @@ int qmatmul_impl(const char* who, const itexhip_matmul_params* p, const void* a,
   ITEXHIP_REQUIRE(out != nullptr && min_b != nullptr && max_b != nullptr, "%s: null buffer", who);
   ITEXHIP_REQUIRE(K == 0 || (a && packed_b), "%s: null operand", who);
   ITEXHIP_REQUIRE(colsum != nullptr, "%s: null colsum", who);
+  ITEXHIP_REQUIRE((p->add_position != 0) == (addend != nullptr), "%s: the addend goes with \"Add\" in fused_ops", who);
   EpilogueArgs e = make_args(p->t_in, colsum, nullptr, bias, &ep);
   e.fused = 1;
   e.nb = static_cast<int>(nb);
@@ -480,27 +517,29 @@ int qmatmul_impl(const char* who, const itexhip_matmul_params* p, const void* a,
   e.prep = make_prep_args(p, ep);
   e.row_min_a = row_min_a;
   e.row_max_a = row_max_a;
+  e.addend = addend;
   return launch_packed(M <= 16, a, p->t_in, packed_b, M, K, N, e, p->t_out, out, stream, who);
 }
 }  // namespace
 
 extern "C" int itexhip_qmatmul(const itexhip_matmul_params* p, const void* a, const int8_t* packed_b,
                                const int32_t* colsum, int64_t M, int64_t K, int64_t N, const float* min_b,
-                               const float* max_b, int64_t nb, const float* bias, void* out, void* stream) {
-  return qmatmul_impl("itexhip_qmatmul", p, a, packed_b, colsum, M, K, N, nullptr, nullptr, min_b, max_b, nb, bias, out,
-                      stream);
+                               const float* max_b, int64_t nb, const void* bias, const float* addend, void* out,
+                               void* stream) {
+  return qmatmul_impl("itexhip_qmatmul", p, a, packed_b, colsum, M, K, N, nullptr, nullptr, min_b, max_b, nb, bias,
+                      addend, out, stream);
 }
 
 extern "C" int itexhip_qmatmul_per_row(const itexhip_matmul_params* p, const void* a, const int8_t* packed_b,
                                        const int32_t* colsum, int64_t M, int64_t K, int64_t N,
                                        const float* row_min_a, const float* row_max_a, const float* min_b,
-                                       const float* max_b, int64_t nb, const float* bias, void* out,
-                                       void* stream) {
+                                       const float* max_b, int64_t nb, const void* bias, const float* addend,
+                                       void* out, void* stream) {
   ITEXHIP_REQUIRE(M <= 16, "itexhip_qmatmul_per_row: per-row activation ranges are implemented for M <= 16 (got %lld)",
                   static_cast<long long>(M));
   ITEXHIP_REQUIRE(M == 0 || (row_min_a && row_max_a), "itexhip_qmatmul_per_row: null row ranges");
   return qmatmul_impl("itexhip_qmatmul_per_row", p, a, packed_b, colsum, M, K, N, row_min_a, row_max_a, min_b, max_b, nb,
-                      bias, out, stream);
+                      bias, addend, out, stream);
 }
 
 extern "C" int itexhip_mfma_probe(int workgroups, int iters, const void* operands, int32_t* sink, void* stream) {
@@ -508,5 +547,43 @@ extern "C" int itexhip_mfma_probe(int workgroups, int iters, const void* operand
   ITEXHIP_REQUIRE(operands && sink && aligned(operands, 16), "itexhip_mfma_probe: null or unaligned buffer");
   mfma_probe_kernel<<<workgroups, 256, 0, as_stream(stream)>>>(iters, reinterpret_cast<const v4i*>(operands), sink);
   ITEXHIP_CHECK_LAUNCH("itexhip_mfma_probe");
+  return ITEXHIP_OK;
+}
+
+extern "C" int itexhip_qmatmul_unpacked(const itexhip_matmul_params* p, const void* a, const int8_t* w, int transpose_b,
+                                        int64_t M, int64_t K, int64_t N, const float* min_b, const float* max_b,
+                                        int64_t nb, const void* bias, const float* addend, void* out, void* stream) {
+  const char* who = "itexhip_qmatmul_unpacked";
+  itexhip_epilogue ep;
+  if (int st = itexhip_qmatmul_epilogue_desc(p, nb, &ep)) return st;
+  ITEXHIP_REQUIRE(nb == 1 || nb == N, "%s: %lld weight ranges for %lld channels", who, static_cast<long long>(nb),
+                  static_cast<long long>(N));
+  ITEXHIP_REQUIRE(M >= 0 && K >= 0 && N >= 0 && M < (1LL << 31) && N < (1LL << 31) && K <= kMaxK, "%s: bad dimensions", who);
+  // the reference's compensation indexes the weight as [K, N] whatever transpose_b says; that combination is refused
+  ITEXHIP_REQUIRE(!(transpose_b && p->input_mode == ITEXHIP_MIN_FIRST), "%s: transpose_b with MIN_FIRST input is not supported", who);
+  if (M == 0 || N == 0) return ITEXHIP_OK;
+  ITEXHIP_REQUIRE(out != nullptr && min_b != nullptr && max_b != nullptr, "%s: null buffer", who);
+  ITEXHIP_REQUIRE(K == 0 || (a && w), "%s: null operand", who);
+  ITEXHIP_REQUIRE((p->add_position != 0) == (addend != nullptr), "%s: the addend goes with \"Add\" in fused_ops", who);
+  EpilogueArgs e = make_args(p->t_in, nullptr, nullptr, bias, &ep);
+  e.comp_mul = 0;  // unsigned activations are multiplied directly
+  e.fused = 1;
+  e.nb = static_cast<int>(nb);
+  e.min_b = min_b;
+  e.max_b = max_b;
+  e.prep = make_prep_args(p, ep);
+  e.addend = addend;
+  const int a_is_u8 = p->t_in == ITEXHIP_QUINT8;
+  const uint8_t* ap = reinterpret_cast<const uint8_t*>(a);
+  const unsigned grid = static_cast<unsigned>((M * N + 255) / 256);
+  hipStream_t hs = as_stream(stream);
+  const int Mi = static_cast<int>(M), Ki = static_cast<int>(K), Ni = static_cast<int>(N);
+  switch (p->t_out) {
+    case ITEXHIP_FLOAT: qmatmul_unpacked_kernel<ITEXHIP_FLOAT><<<grid, 256, 0, hs>>>(ap, a_is_u8, w, transpose_b, Mi, Ki, Ni, e, out); break;
+    case ITEXHIP_QINT32: qmatmul_unpacked_kernel<ITEXHIP_QINT32><<<grid, 256, 0, hs>>>(ap, a_is_u8, w, transpose_b, Mi, Ki, Ni, e, out); break;
+    case ITEXHIP_QINT8: qmatmul_unpacked_kernel<ITEXHIP_QINT8><<<grid, 256, 0, hs>>>(ap, a_is_u8, w, transpose_b, Mi, Ki, Ni, e, out); break;
+    default: qmatmul_unpacked_kernel<ITEXHIP_QUINT8><<<grid, 256, 0, hs>>>(ap, a_is_u8, w, transpose_b, Mi, Ki, Ni, e, out); break;
+  }
+  ITEXHIP_CHECK_LAUNCH(who);
   return ITEXHIP_OK;
 }

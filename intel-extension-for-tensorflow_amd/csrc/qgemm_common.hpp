@@ -22,12 +22,13 @@ constexpr int64_t kMaxK = 1 << 16; // 255 * 128 * 65536 < 2^31
 
 struct EpilogueArgs {
   const float* scales;   // prepared per-channel scales (n_scales of them), unused when `fused`
-  const float* bias;     // prepared bias, or the op's raw fp32 bias when `fused`
+  const void* bias;      // prepared fp32 bias, or the op's raw bias (fp32 / int32) when `fused`
   const int32_t* colsum;
   int n_scales;
   int comp_mul;  // 128 for u8 activations, 0 for s8
   int n_eltwise;
-  itexhip_eltwise elt[2];
+  itexhip_eltwise elt[3];
+  const float* addend;   // [M, N] fp32 tensor of the "Add" fusion (ITEXHIP_ELT_SUM in the chain), else null
   // fused != 0: the kernel derives scale and bias of a channel itself from the op's ranges
   int fused;
   int nb;  // weight ranges (1 or N)
@@ -51,7 +52,7 @@ struct RawChannel {
 __device__ __forceinline__ RawChannel load_raw_channel(const EpilogueArgs& e, int n, int N) {
   RawChannel r{};
   r.colsum = e.colsum ? e.colsum[n] : 0;
-  r.bias = e.bias ? e.bias[n] : 0.0f;
+  r.bias = e.fused ? bias_entry(e.prep, e.bias, n) : (e.bias ? static_cast<const float*>(e.bias)[n] : 0.0f);
   if (e.fused) {
     const int jb = (e.nb == N) ? n : 0;
     r.min_bj = e.min_b[jb];
@@ -148,7 +149,10 @@ __device__ __forceinline__ void epilogue_store(const v4i acc, const ChannelParam
     if (ACT == 1) {
       v = fmaxf(v, 0.0f);
     } else if (ACT == 2) {
-      for (int k = 0; k < e.n_eltwise; ++k) v = apply_eltwise(e.elt[k], v);
+      for (int k = 0; k < e.n_eltwise; ++k) {
+        if (e.elt[k].alg == ITEXHIP_ELT_SUM) v = v + e.elt[k].alpha * e.addend[static_cast<int64_t>(m) * N + min(n + r, N - 1)];
+        else v = apply_eltwise(e.elt[k], v);
+      }
     }
     y[r] = v;
   }

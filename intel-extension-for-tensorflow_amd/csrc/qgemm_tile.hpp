@@ -275,7 +275,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void qgemm_tile_kernel(
   constexpr int RPP = 64 / LPR;              // rows per flush instruction (lanes >= RPP * LPR idle)
   constexpr int PASSES = (WM + RPP - 1) / RPP;
   static_assert(NW * WM * PITCH <= NSTAGE * STAGE_BYTES, "epilogue buffer must fit in the ring");
-  const bool fast = !GENERAL || ((e.bias != nullptr || e.fused) && aligned16(out) && ((static_cast<int64_t>(N) * ESZ) & 15) == 0);
+  const bool fast = !GENERAL || (e.addend == nullptr && (e.bias != nullptr || e.fused) && aligned16(out) && ((static_cast<int64_t>(N) * ESZ) & 15) == 0);
   if (fast) {
     uint8_t* ebuf = lds + wave * (WM * PITCH);
     const int f_row = lane / LPR, f_piece = lane % LPR;
@@ -329,8 +329,11 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void qgemm_tile_kernel(
                 if (n + r < N) {
                   float v = static_cast<float>(acc[t][r0 + r]) * sc[r];
                   if (has_bias) v = v + bi[r];
-                  for (int k = 0; k < e.n_eltwise; ++k) v = apply_eltwise(e.elt[k], v);
                   const int64_t o = static_cast<int64_t>(m) * N + n + r;
+                  for (int k = 0; k < e.n_eltwise; ++k) {
+                    if (e.elt[k].alg == ITEXHIP_ELT_SUM) v = v + e.elt[k].alpha * e.addend[o];
+                    else v = apply_eltwise(e.elt[k], v);
+                  }
                   if constexpr (OUT_T == ITEXHIP_FLOAT) reinterpret_cast<float*>(out)[o] = v;
                   else if constexpr (OUT_T == ITEXHIP_QINT32) reinterpret_cast<int32_t*>(out)[o] = sat_rne<ITEXHIP_QINT32>(v);
                   else reinterpret_cast<uint8_t*>(out)[o] = static_cast<uint8_t>(sat_rne<OUT_T>(v));
@@ -404,7 +407,7 @@ int dispatch_tile(const uint8_t* a, uint32_t a_xor, const uint8_t* bp, int M, in
                   const EpilogueArgs& e, void* out, hipStream_t st) {
   constexpr int esz = (OUT_T == ITEXHIP_QINT8 || OUT_T == ITEXHIP_QUINT8) ? 1 : 4;
   // the specialised kernels only carry the vectorised epilogue: bias present, output rows 16-byte aligned
-  const bool plain = (e.bias != nullptr || e.fused) && (reinterpret_cast<uintptr_t>(out) & 15) == 0 &&
+  const bool plain = e.addend == nullptr && (e.bias != nullptr || e.fused) && (reinterpret_cast<uintptr_t>(out) & 15) == 0 &&
                      ((static_cast<int64_t>(N) * esz) & 15) == 0 && (K & 63) == 0;
   const int act = e.n_eltwise == 0 ? 0
                   : (e.n_eltwise == 1 && e.elt[0].alg == ITEXHIP_ELT_RELU && e.elt[0].alpha == 0.0f) ? 1 : 2;

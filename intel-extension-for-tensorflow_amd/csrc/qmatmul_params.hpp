@@ -17,8 +17,15 @@ struct PrepArgs {
   int n_scales;        // from the epilogue descriptor
   int mul_requant;     // multiply the output scale by (max_int8_output / range_output)
   int legacy_kind;     // 1: u8 out, 2: s8 out, 3: fp32 out (legacy api only)
+  int bias_s32;        // Tbias = qint32: the bias vector holds int32 (quantized_matmul_common.h:1153-1334)
   float min_a, max_a, min_out, max_out;
 };
+
+// entry j of the op's bias vector as fp32 (the qint32 bias is cast, :1165-1167); 0 without a bias
+__device__ __forceinline__ float bias_entry(const PrepArgs& p, const void* bias, int64_t j) {
+  if (bias == nullptr) return 0.0f;
+  return p.bias_s32 ? static_cast<float>(static_cast<const int32_t*>(bias)[j]) : static_cast<const float*>(bias)[j];
+}
 
 struct ChannelScaleBias {
   float scale;  // output scale of the channel (the single scale when the node has one; 1 when none)
@@ -63,6 +70,15 @@ __device__ __forceinline__ ChannelScaleBias channel_scale_bias(const PrepArgs& p
   }
 
   // ---- bias -----------------------------------------------------------------------------------
+  if (p.bias_s32) {
+    // qint32 bias: scaled by the inverse of the fp32 path's factor, no zero-point compensation (:1204-1271)
+    const float sj = (range_input * range_weight) / (max_int8_input * max_int8_weight);
+    float out;
+    if (p.input_mode != ITEXHIP_MIN_FIRST || p.t_out == ITEXHIP_FLOAT) out = b * sj;
+    else if (p.t_out == ITEXHIP_QINT8 || p.t_out == ITEXHIP_QUINT8) out = b * os;
+    else out = b;
+    return ChannelScaleBias{os, out};
+  }
   const float bias_scale = (max_int8_input * max_int8_weight) / (range_input * range_weight);
   float out;
   if (p.input_mode == ITEXHIP_MIN_FIRST) {
@@ -88,11 +104,11 @@ __device__ __forceinline__ ChannelScaleBias channel_scale_bias(const PrepArgs& p
 // MIN_FIRST input.
 __device__ __forceinline__ ChannelScaleBias channel_scale_bias(const PrepArgs& p, const float* __restrict__ min_b,
                                                                const float* __restrict__ max_b, int64_t nb,
-                                                               const float* __restrict__ bias,
+                                                               const void* __restrict__ bias,
                                                                const int32_t* __restrict__ colsum, int64_t N,
                                                                int64_t j) {
   const int64_t jb = (nb == N) ? j : 0;
-  return channel_scale_bias(p, min_b[jb], max_b[jb], min_b[0], max_b[0], bias ? bias[j] : 0.0f,
+  return channel_scale_bias(p, min_b[jb], max_b[jb], min_b[0], max_b[0], bias_entry(p, bias, j),
                             p.input_mode == ITEXHIP_MIN_FIRST ? colsum[j] : 0);
 }
 
@@ -101,11 +117,14 @@ inline PrepArgs make_prep_args(const itexhip_matmul_params* p, const itexhip_epi
   PrepArgs a{};
   a.api = p->api; a.t_in = p->t_in; a.t_out = p->t_out; a.input_mode = p->input_mode;
   a.n_scales = ep.n_scales;
+  a.bias_s32 = p->t_bias == ITEXHIP_QINT32;
   a.min_a = p->min_a; a.max_a = p->max_a; a.min_out = p->min_out; a.max_out = p->max_out;
   const bool out_q8 = p->t_out == ITEXHIP_QINT8 || p->t_out == ITEXHIP_QUINT8;
   if (p->api == ITEXHIP_API_V2) {
     // requantize factor folded into the output scale only without any eltwise post-op
-    a.mul_requant = p->has_requantize && ep.n_eltwise == 0;
+    int n_act = 0;
+    for (int k = 0; k < ep.n_eltwise; ++k) n_act += ep.elt[k].alg != ITEXHIP_ELT_SUM;
+    a.mul_requant = p->has_requantize && n_act == 0;
   } else if (p->api == ITEXHIP_API_V1) {
     a.mul_requant = out_q8 && p->n_fused_ops == 1;
   } else {

@@ -14,7 +14,7 @@ namespace {
 
 __global__ void qmatmul_prepare_kernel(PrepArgs p, const float* __restrict__ min_b,
                                        const float* __restrict__ max_b, int64_t nb,
-                                       const float* __restrict__ bias, const int32_t* __restrict__ colsum,
+                                       const void* __restrict__ bias, const int32_t* __restrict__ colsum,
                                        int64_t N, float* __restrict__ scales_out,
                                        float* __restrict__ bias_out) {
   const int64_t j = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
@@ -30,6 +30,8 @@ int eltwise_from_activation(int act, itexhip_eltwise* e) {
     case ITEXHIP_ACT_RELU: *e = {ITEXHIP_ELT_RELU, 0.0f, 0.0f}; return 1;
     case ITEXHIP_ACT_RELU6: *e = {ITEXHIP_ELT_CLIP, 0.0f, 6.0f}; return 1;
     case ITEXHIP_ACT_LEAKYRELU: *e = {ITEXHIP_ELT_RELU, 0.0f, 0.0f}; return 1;
+    case ITEXHIP_ACT_GELU_APPROX: *e = {ITEXHIP_ELT_GELU_TANH, 0.0f, 0.0f}; return 1;
+    case ITEXHIP_ACT_GELU_EXACT: *e = {ITEXHIP_ELT_GELU_ERF, 0.0f, 0.0f}; return 1;
     default: return 0;
   }
 }
@@ -45,6 +47,13 @@ int validate(const itexhip_matmul_params* p, int64_t nb) {
   ITEXHIP_REQUIRE(p->input_mode == ITEXHIP_MIN_FIRST || p->input_mode == ITEXHIP_SCALED,
                   "Quantization mode must be either MIN_FIRST or SCALED");
   ITEXHIP_REQUIRE(nb >= 1, "qmatmul: empty weight range");
+  ITEXHIP_REQUIRE(p->t_bias == 0 || p->t_bias == ITEXHIP_FLOAT || p->t_bias == ITEXHIP_QINT32,
+                  "qmatmul: Tbias must be float or qint32");
+  ITEXHIP_REQUIRE(p->add_position >= 0 && p->add_position <= 2, "qmatmul: bad add_position");
+  if (p->add_position != 0 && p->t_out != ITEXHIP_FLOAT) {
+    set_error("Quantized addend tensor is not implemented yet.");
+    return ITEXHIP_UNIMPLEMENTED;
+  }
   return ITEXHIP_OK;
 }
 
@@ -63,7 +72,10 @@ extern "C" int itexhip_qmatmul_epilogue_desc(const itexhip_matmul_params* p, int
 
   bool has_linear = false;
   const bool has_leaky = p->activation == ITEXHIP_ACT_LEAKYRELU;
+  // post-ops in fused_ops order; "Add" is a sum post-op with scale 1 and no activation
+  if (p->add_position == 1) ep->elt[ep->n_eltwise++] = {ITEXHIP_ELT_SUM, 1.0f, 0.0f};
   if (eltwise_from_activation(p->activation, &ep->elt[ep->n_eltwise])) ep->n_eltwise++;
+  if (p->add_position == 2) ep->elt[ep->n_eltwise++] = {ITEXHIP_ELT_SUM, 1.0f, 0.0f};
   if (p->api == ITEXHIP_API_V2 && p->has_requantize && p->out_min_first) {
     ep->elt[ep->n_eltwise++] = {ITEXHIP_ELT_LINEAR, 1.0f, 0.0f};
     has_linear = true;
@@ -82,6 +94,7 @@ extern "C" int itexhip_qmatmul_epilogue_desc(const itexhip_matmul_params* p, int
     ep->n_scales = (p->t_out == ITEXHIP_QINT32) ? 0 : 1;
   }
   for (int e = 0; e < ep->n_eltwise; ++e) {
+    if (ep->elt[e].alg == ITEXHIP_ELT_SUM) continue;
     if (has_leaky) ep->elt[e].alpha = p->leakyrelu_alpha;
     if (has_linear) {
       ep->elt[e].alpha = linear_alpha;
@@ -96,7 +109,7 @@ extern "C" int itexhip_qmatmul_epilogue_desc(const itexhip_matmul_params* p, int
 }
 
 extern "C" int itexhip_qmatmul_prepare(const itexhip_matmul_params* p, const float* min_b,
-                                       const float* max_b, int64_t nb, const float* bias,
+                                       const float* max_b, int64_t nb, const void* bias,
                                        const int32_t* colsum, int64_t N, float* scales_out,
                                        float* bias_out, void* stream) {
   itexhip_epilogue ep;

@@ -14,8 +14,8 @@ OK, INVALID_ARGUMENT, UNIMPLEMENTED, INTERNAL = 0, 3, 12, 13
 FLOAT, INT32, QINT8, QUINT8, QINT32 = 1, 3, 11, 12, 13
 MIN_COMBINED, MIN_FIRST, SCALED = 0, 1, 2
 API_V2, API_V1, API_LEGACY = 0, 1, 2
-ACT_NONE, ACT_RELU, ACT_RELU6, ACT_LEAKYRELU = 0, 1, 2, 3
-ELT_RELU, ELT_CLIP, ELT_LINEAR = 1, 2, 3
+ACT_NONE, ACT_RELU, ACT_RELU6, ACT_LEAKYRELU, ACT_GELU_APPROX, ACT_GELU_EXACT = 0, 1, 2, 3, 4, 5
+ELT_RELU, ELT_CLIP, ELT_LINEAR, ELT_GELU_TANH, ELT_GELU_ERF, ELT_SUM = 1, 2, 3, 4, 5, 6
 
 EXPORTS = [
     "itexhip_device_count", "itexhip_device_info", "itexhip_mem_info", "itexhip_malloc", "itexhip_free",
@@ -27,7 +27,7 @@ EXPORTS = [
     "itexhip_dequantize", "itexhip_dequantize_axis", "itexhip_requantize_per_channel",
     "itexhip_requantize", "itexhip_minmax_i32_per_channel", "itexhip_minmax_f32",
     "itexhip_qmatmul_epilogue_desc", "itexhip_qmatmul_prepare", "itexhip_qgemm_packed_bytes",
-    "itexhip_qgemm_prepack_b", "itexhip_qgemm", "itexhip_qgemm_tile", "itexhip_qgemv", "itexhip_qmatmul", "itexhip_qmatmul_per_row", "itexhip_mfma_probe",
+    "itexhip_qgemm_prepack_b", "itexhip_qgemm", "itexhip_qgemm_tile", "itexhip_qgemv", "itexhip_qmatmul", "itexhip_qmatmul_per_row", "itexhip_qmatmul_unpacked", "itexhip_mfma_probe",
     "itexhip_qgemm_naive",
 ]
 
@@ -43,7 +43,7 @@ class Eltwise(C.Structure):
 
 
 class Epilogue(C.Structure):
-    _fields_ = [("n_scales", C.c_int), ("n_eltwise", C.c_int), ("elt", Eltwise * 2)]
+    _fields_ = [("n_scales", C.c_int), ("n_eltwise", C.c_int), ("elt", Eltwise * 3)]
 
 
 class MatmulParams(C.Structure):
@@ -51,7 +51,7 @@ class MatmulParams(C.Structure):
                 ("out_min_first", C.c_int), ("activation", C.c_int), ("has_requantize", C.c_int),
                 ("has_dequantize", C.c_int), ("n_fused_ops", C.c_int), ("leakyrelu_alpha", C.c_float),
                 ("min_a", C.c_float), ("max_a", C.c_float), ("min_out", C.c_float),
-                ("max_out", C.c_float)]
+                ("max_out", C.c_float), ("add_position", C.c_int), ("t_bias", C.c_int)]
 
 
 # One HIP runtime per process: PyTorch ships its own libamdhip64.so.7 and loads it by path.  If this
@@ -144,10 +144,10 @@ def minmax_f32(x, n, minmax_out, stream=0):
 
 def matmul_params(api=API_V2, t_in=QUINT8, t_out=FLOAT, input_mode=MIN_FIRST, out_min_first=False,
                   activation=ACT_NONE, has_requantize=False, has_dequantize=False, n_fused_ops=1,
-                  leakyrelu_alpha=0.2, min_a=0.0, max_a=0.0, min_out=0.0, max_out=0.0):
+                  leakyrelu_alpha=0.2, min_a=0.0, max_a=0.0, min_out=0.0, max_out=0.0, add_position=0, t_bias=0):
     return MatmulParams(api, t_in, t_out, input_mode, int(out_min_first), activation,
                         int(has_requantize), int(has_dequantize), n_fused_ops, leakyrelu_alpha,
-                        min_a, max_a, min_out, max_out)
+                        min_a, max_a, min_out, max_out, int(add_position), int(t_bias))
 
 
 def qmatmul_epilogue_desc(params, nb):
@@ -191,16 +191,24 @@ def qgemv(a, a_type, packed_b, colsum, M, K, N, scales, bias, ep, out_type, out,
                out, stream)
 
 
-def qmatmul(p, a, packed_b, colsum, M, K, N, min_b, max_b, nb, bias, out, stream=0):
+def qmatmul(p, a, packed_b, colsum, M, K, N, min_b, max_b, nb, bias, out, stream=0, addend=None):
     """The whole op in one launch (parameters derived inside the MatMul kernel)."""
     _check(_lib.itexhip_qmatmul(C.byref(p), _ptr(a), _ptr(packed_b), _ptr(colsum), _i64(M), _i64(K), _i64(N),
-                                _ptr(min_b), _ptr(max_b), _i64(nb), _ptr(bias), _ptr(out), _ptr(stream)))
+                                _ptr(min_b), _ptr(max_b), _i64(nb), _ptr(bias), _ptr(addend), _ptr(out),
+                                _ptr(stream)))
 
 
-def qmatmul_per_row(p, a, packed_b, colsum, M, K, N, row_min_a, row_max_a, min_b, max_b, nb, bias, out, stream=0):
+def qmatmul_per_row(p, a, packed_b, colsum, M, K, N, row_min_a, row_max_a, min_b, max_b, nb, bias, out, stream=0,
+                    addend=None):
     _check(_lib.itexhip_qmatmul_per_row(C.byref(p), _ptr(a), _ptr(packed_b), _ptr(colsum), _i64(M), _i64(K), _i64(N),
                                         _ptr(row_min_a), _ptr(row_max_a), _ptr(min_b), _ptr(max_b), _i64(nb),
-                                        _ptr(bias), _ptr(out), _ptr(stream)))
+                                        _ptr(bias), _ptr(addend), _ptr(out), _ptr(stream)))
+
+
+def qmatmul_unpacked(p, a, w, transpose_b, M, K, N, min_b, max_b, nb, bias, out, stream=0, addend=None):
+    _check(_lib.itexhip_qmatmul_unpacked(C.byref(p), _ptr(a), _ptr(w), int(bool(transpose_b)), _i64(M), _i64(K), _i64(N),
+                                         _ptr(min_b), _ptr(max_b), _i64(nb), _ptr(bias), _ptr(addend), _ptr(out),
+                                         _ptr(stream)))
 
 
 def mfma_probe(workgroups, iters, operands, sink, stream=0):

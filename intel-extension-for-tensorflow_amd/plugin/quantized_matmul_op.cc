@@ -38,6 +38,8 @@ int ActivationFromName(const std::string& n) {
   if (n == "Relu") return ITEXHIP_ACT_RELU;
   if (n == "Relu6") return ITEXHIP_ACT_RELU6;
   if (n == "LeakyRelu") return ITEXHIP_ACT_LEAKYRELU;
+  if (n == "GeluApproximate") return ITEXHIP_ACT_GELU_APPROX;
+  if (n == "GeluExact") return ITEXHIP_ACT_GELU_EXACT;
   return -1;
 }
 
@@ -72,13 +74,16 @@ class QuantizedMatMulOp : public OpKernel {
                     "_QuantizedFusedMatMul first post op must be BiasAdd");
       p_.n_fused_ops = static_cast<int>(fused_ops.size());
       for (size_t i = 1; i < fused_ops.size(); ++i) {
-        ITEX_REQUIRES(ctx, fused_ops[i] != "Add", TF_UNIMPLEMENTED, "the Add fusion is not implemented on this device");
+        if (fused_ops[i] == "Add") {  // the addend follows the bias in `args` and shifts every min/max input (:1593-1602)
+          p_.add_position = p_.activation == ITEXHIP_ACT_NONE ? 1 : 2;
+          continue;
+        }
         const int act = ActivationFromName(fused_ops[i]);
         ITEX_REQUIRES(ctx, act >= 0, TF_INVALID_ARGUMENT, "Found unsupported fusion in _QuantizedFusedMatMul.");
         p_.activation = act;
       }
-      min_a_idx_ = 3;
-      min_out_idx_ = 7;
+      min_a_idx_ = 3 + (p_.add_position != 0);
+      min_out_idx_ = 7 + (p_.add_position != 0);
     } else {  // V2 :1725-1795
       std::string out_mode;
       ITEX_REQUIRES_OK(ctx, ctx->GetAttr("output_quant_mode", &out_mode));
@@ -90,21 +95,29 @@ class QuantizedMatMulOp : public OpKernel {
         if (f == "BiasAdd" || f == "Quantized") continue;
         if (f == "Requantize") { p_.has_requantize = 1; continue; }
         if (f == "Dequantize") { p_.has_dequantize = 1; continue; }
-        ITEX_REQUIRES(ctx, f != "Add", TF_UNIMPLEMENTED, "Quantized addend tensor is not implemented yet.");
+        if (f == "Add") {
+          ITEX_REQUIRES(ctx, v.t_out == TF_FLOAT, TF_UNIMPLEMENTED, "Quantized addend tensor is not implemented yet.");
+          p_.add_position = p_.activation == ITEXHIP_ACT_NONE ? 1 : 2;
+          continue;
+        }
         const int act = ActivationFromName(f);
         ITEX_REQUIRES(ctx, act >= 0, TF_INVALID_ARGUMENT, "Found unsupported fusion in _QuantizedMatMul.");
         p_.activation = act;
       }
       p_.n_fused_ops = static_cast<int>(fused_ops.size());
-      min_a_idx_ = 3;
+      min_a_idx_ = 3 + (p_.add_position != 0);  // the addend precedes all min/max tensors (:1775-1780)
       min_out_idx_ = 7;  // fixed, as in the reference (:1784-1785)
     }
     if (p_.activation == ITEXHIP_ACT_LEAKYRELU) ITEX_REQUIRES_OK(ctx, ctx->GetAttr("leakyrelu_alpha", &p_.leakyrelu_alpha));
     if (ctx->HasAttr("Tbias")) {
       TF_DataType tb = TF_FLOAT;
       ITEX_REQUIRES_OK(ctx, ctx->GetAttr("Tbias", &tb));
-      ITEX_REQUIRES(ctx, tb == TF_FLOAT, TF_UNIMPLEMENTED, "only a float bias is implemented on this device");
+      ITEX_REQUIRES(ctx, tb == TF_FLOAT || tb == TF_QINT32, TF_UNIMPLEMENTED,
+                    "only float and qint32 biases are implemented on this device");
+      p_.t_bias = tb;
     }
+    if (p_.add_position != 0)
+      ITEX_REQUIRES(ctx, v.t_out == TF_FLOAT, TF_UNIMPLEMENTED, "Quantized addend tensor is not implemented yet.");
   }
 
   void Compute(OpKernelContext* ctx) override {
@@ -117,7 +130,8 @@ class QuantizedMatMulOp : public OpKernel {
     if (!ctx->ok()) return;
     ITEX_REQUIRES(ctx, !transpose_a_, TF_UNIMPLEMENTED, "transpose_a is not supported by the quantized MatMul");
     ITEX_REQUIRES(ctx, a.dims() == 2 && w.dims() == 2, TF_INVALID_ARGUMENT, "quantized MatMul operands must be matrices");
-    ITEX_REQUIRES(ctx, a.dtype() == v_.t_in && w.dtype() == TF_QINT8 && bias.dtype() == TF_FLOAT, TF_INVALID_ARGUMENT,
+    const TF_DataType bias_type = p_.t_bias == ITEXHIP_QINT32 ? TF_QINT32 : TF_FLOAT;
+    ITEX_REQUIRES(ctx, a.dtype() == v_.t_in && w.dtype() == TF_QINT8 && bias.dtype() == bias_type, TF_INVALID_ARGUMENT,
                   "quantized MatMul operand types do not match the kernel");
     const int64_t M = a.dim_size(0), K = a.dim_size(1);
     const int64_t N = transpose_b_ ? w.dim_size(0) : w.dim_size(1);
@@ -153,8 +167,9 @@ class QuantizedMatMulOp : public OpKernel {
 
     void* stream = ctx->stream();
     // ---- weight: prepacked once when constant, else every call (:238-275)
+    const bool packed_path = K % 16 == 0 && K > 0;
     const bool repack = !packed_.valid() || !is_weight_const_ || packed_src_ != w.data() || packed_k_ != K || packed_n_ != N;
-    if (repack) {
+    if (packed_path && repack) {
       const int64_t bytes = itexhip_qgemm_packed_bytes(K, N);
       packed_ = ctx->allocate_temp(TF_QINT8, {std::max<int64_t>(bytes, 16)});
       colsum_ = ctx->allocate_temp(TF_INT32, {std::max<int64_t>(N, 1)});
@@ -166,29 +181,33 @@ class QuantizedMatMulOp : public OpKernel {
       packed_k_ = K;
       packed_n_ = N;
     }
-    // ---- per-channel scale and bias vectors on the device
+    // ---- the weight ranges on the device (uploaded when they change)
     float* min_b_dev = min_b_cache_.Get(ctx, min_b_t.flat<float>(), nb, TF_FLOAT);
     float* max_b_dev = max_b_cache_.Get(ctx, max_b_t.flat<float>(), nb, TF_FLOAT);
     if (min_b_dev == nullptr || max_b_dev == nullptr) return;
-    // ---- product.  K a multiple of 16: one launch, the MatMul kernel derives each channel's output
-    // scale and compensated bias itself, so a new activation range costs nothing extra.  Other K: the
-    // parameter vectors are prepared by a small kernel and the reference-shaped kernel runs.
+    // ---- product: one launch, the MatMul kernel derives each channel's output scale and compensated
+    // bias itself, so a new activation range costs nothing extra.  K a multiple of 16: MFMA kernels on
+    // the prepacked weight; other K: the reference-shaped kernel on the unpacked weight.
+    // "Add": the fp32 addend is input 3 (:352-389 adds it in place into the forwarded output buffer; here the
+    // kernel reads it and writes a fresh output, same values)
+    const float* addend = nullptr;
+    Tensor addend_t;
+    if (p_.add_position != 0) {
+      addend_t = ctx->input(3);
+      if (!ctx->ok()) return;
+      ITEX_REQUIRES(ctx, addend_t.dtype() == TF_FLOAT && addend_t.dims() == 2 && addend_t.dim_size(0) == M &&
+                             addend_t.dim_size(1) == N,
+                    TF_INVALID_ARGUMENT, "the addend must be a float tensor of the output's shape");
+      addend = addend_t.flat<float>();
+    }
     Tensor out = ctx->allocate_output(0, v_.t_out, {M, N});
     if (!ctx->ok()) return;
-    if (K % 16 == 0 && K > 0) {
+    if (packed_path) {
       st = itexhip_qmatmul(&p, a.data(), packed_.flat<int8_t>(), colsum_.flat<int32_t>(), M, K, N, min_b_dev, max_b_dev,
-                           nb, bias.flat<float>(), out.data(), stream);
+                           nb, bias.data(), addend, out.data(), stream);
     } else {
-      if (!scales_.valid() || scales_.NumElements() < std::max<int64_t>(N, 1)) {
-        scales_ = ctx->allocate_temp(TF_FLOAT, {std::max<int64_t>(N, 1)});
-        sbias_ = ctx->allocate_temp(TF_FLOAT, {std::max<int64_t>(N, 1)});
-        if (!ctx->ok()) return;
-      }
-      st = itexhip_qmatmul_prepare(&p, min_b_dev, max_b_dev, nb, bias.flat<float>(), colsum_.flat<int32_t>(), N,
-                                   scales_.flat<float>(), sbias_.flat<float>(), stream);
-      if (st == ITEXHIP_OK)
-        st = itexhip_qgemm_naive(a.data(), v_.t_in, w.flat<int8_t>(), transpose_b_ ? 1 : 0, M, K, N, scales_.flat<float>(),
-                                 sbias_.flat<float>(), &ep, v_.t_out, out.data(), stream);
+      st = itexhip_qmatmul_unpacked(&p, a.data(), w.flat<int8_t>(), transpose_b_ ? 1 : 0, M, K, N, min_b_dev, max_b_dev, nb,
+                                    bias.data(), addend, out.data(), stream);
     }
     ITEX_REQUIRES(ctx, st == ITEXHIP_OK, st == ITEXHIP_INVALID_ARGUMENT ? TF_INVALID_ARGUMENT : TF_ABORTED,
                   std::string("Operation received an exception: ") + itexhip_last_error());
@@ -221,7 +240,7 @@ class QuantizedMatMulOp : public OpKernel {
   int min_a_idx_ = 3, min_out_idx_ = 7;
   std::mutex mu_;
   // persistent device state of the node
-  Tensor packed_, colsum_, scales_, sbias_;
+  Tensor packed_, colsum_;
   const void* packed_src_ = nullptr;
   int64_t packed_k_ = -1, packed_n_ = -1;
   DeviceVectorCache<float> min_b_cache_, max_b_cache_;
@@ -241,6 +260,13 @@ void Reg(const char* op, const char* out_attr, const char* bias_attr, std::initi
   b.TypeConstraint(out_attr, static_cast<TF_DataType>(TOUT));
   for (const char* h : host_args) b.HostMemory(h);
   b.Register<MatMulKernel<API, TIN, TOUT, RELU>>();
+  if (bias_attr && std::string(bias_attr) == "Tbias") {  // the same kernel with Tbias = qint32
+    KernelDefBuilder q(op, "QuantizedMatMulOp");
+    q.TypeConstraint("T1", static_cast<TF_DataType>(TIN)).TypeConstraint("T2", TF_QINT8);
+    q.TypeConstraint(bias_attr, TF_QINT32).TypeConstraint(out_attr, static_cast<TF_DataType>(TOUT));
+    for (const char* h : host_args) q.HostMemory(h);
+    q.Register<MatMulKernel<API, TIN, TOUT, RELU>>();
+  }
 }
 
 template <int API, int TOUT>

@@ -288,6 +288,8 @@ static int eltwise_from_activation(int act, orc_eltwise* e) {
     case ORC_ACT_RELU: e->alg = ORC_ELT_RELU; e->alpha = 0.0f; e->beta = 0.0f; return 1;
     case ORC_ACT_RELU6: e->alg = ORC_ELT_CLIP; e->alpha = 0.0f; e->beta = 6.0f; return 1;
     case ORC_ACT_LEAKYRELU: e->alg = ORC_ELT_RELU; e->alpha = 0.0f; e->beta = 0.0f; return 1;
+    case ORC_ACT_GELU_APPROX: e->alg = ORC_ELT_GELU_TANH; e->alpha = 0.0f; e->beta = 0.0f; return 1;
+    case ORC_ACT_GELU_EXACT: e->alg = ORC_ELT_GELU_ERF; e->alpha = 0.0f; e->beta = 0.0f; return 1;
     default: return 0;
   }
 }
@@ -303,8 +305,11 @@ static int eltwise_from_activation(int act, orc_eltwise* e) {
  */
 int orc_qmatmul_prepare(const orc_matmul_attrs* at, int64_t N, const int32_t* colsum, float min_a,
                         float max_a, const float* min_b, const float* max_b, int64_t nb,
-                        float min_out, float max_out, const float* bias, float* scales,
+                        float min_out, float max_out, const void* bias_v, float* scales,
                         float* bias_out, orc_epilogue_desc* ep) {
+  const int bias_s32 = (at->t_bias == ORC_QINT32);
+  const float* bias = (const float*)bias_v;
+  const int32_t* bias_i32 = (const int32_t*)bias_v;
   const int out_q8 = (at->t_out == ORC_QINT8 || at->t_out == ORC_QUINT8);
   const int out_f32 = (at->t_out == ORC_FLOAT);
   const int out_s32 = (at->t_out == ORC_QINT32);
@@ -324,7 +329,20 @@ int orc_qmatmul_prepare(const orc_matmul_attrs* at, int64_t N, const int32_t* co
   /* ---- post-op chain -------------------------------------------------------------------- */
   int has_linear = 0, has_leaky = 0;
   float linear_alpha = 0.0f, linear_beta = 0.0f;
-  if (eltwise_from_activation(at->activation, &ep->elt[ep->n_eltwise])) ep->n_eltwise++;
+  /* post-ops are appended in fused_ops order (onednn_post_op_util.cc:73-128, 237-266); "Add" is a sum
+   * post-op with scale 1 (:1694-1699, 1902-1906) and does not count as an activation */
+  int n_act = 0;
+  if (at->add_position == 1) {
+    ep->elt[ep->n_eltwise].alg = ORC_ELT_SUM; ep->elt[ep->n_eltwise].alpha = 1.0f; ep->elt[ep->n_eltwise].beta = 0.0f;
+    ep->n_eltwise++;
+  }
+  if (eltwise_from_activation(at->activation, &ep->elt[ep->n_eltwise])) { ep->n_eltwise++; n_act++; }
+  if (at->add_position == 2) {
+    ep->elt[ep->n_eltwise].alg = ORC_ELT_SUM; ep->elt[ep->n_eltwise].alpha = 1.0f; ep->elt[ep->n_eltwise].beta = 0.0f;
+    ep->n_eltwise++;
+  }
+  /* a quantized addend is not implemented upstream either (:1768-1773) */
+  if (at->add_position != 0 && !out_f32) return ORC_UNIMPLEMENTED;
   if (at->activation == ORC_ACT_LEAKYRELU) has_leaky = 1;
   if (at->api == ORC_API_V2 && at->has_requantize && at->out_min_first) {
     /* :1753-1757: "Linear" is appended to fused_ops */
@@ -332,9 +350,10 @@ int orc_qmatmul_prepare(const orc_matmul_attrs* at, int64_t N, const int32_t* co
     ep->elt[ep->n_eltwise].alpha = 1.0f;
     ep->elt[ep->n_eltwise].beta = 0.0f;
     ep->n_eltwise++;
+    n_act++;
     has_linear = 1;
   }
-  const int has_activation = ep->n_eltwise > 0; /* has_activation_ is set by every eltwise */
+  const int has_activation = n_act > 0; /* has_activation_ is set by every eltwise post-op */
 
   /* ---- output scales ---------------------------------------------------------------------- */
   if (at->api == ORC_API_V2) {
@@ -398,6 +417,7 @@ int orc_qmatmul_prepare(const orc_matmul_attrs* at, int64_t N, const int32_t* co
 
   /* alpha / beta overrides applied to EVERY eltwise of the chain, onednn_post_op_util.cc:251-262 */
   for (int e = 0; e < ep->n_eltwise; ++e) {
+    if (ep->elt[e].alg == ORC_ELT_SUM) continue;
     if (has_leaky) ep->elt[e].alpha = at->leakyrelu_alpha;
     if (has_linear) { ep->elt[e].alpha = linear_alpha; ep->elt[e].beta = linear_beta; }
   }
@@ -410,6 +430,28 @@ int orc_qmatmul_prepare(const orc_matmul_attrs* at, int64_t N, const int32_t* co
     bias_scales[i] = (max_int8_input * max_int8_weight) / (range_input * range_weight);
   }
   int st = ORC_OK;
+  if (bias_s32) {
+    /* Tbias = qint32, :1153-1334: the bias is cast to float (:1165-1167) and scaled by
+     * (range_input * range_weight) / (A * 127) (:1204-1211), the inverse of the fp32 path's factor;
+     * no zero-point compensation (the column-sum loop is commented out, :1250-1253) */
+    for (int64_t j = 0; j < N; ++j) {
+      const int64_t jb = (nb != N) ? 0 : j;
+      const float range_weight = fmaxf(fabsf(min_b[jb]), fabsf(max_b[jb]));
+      const float sj = (range_input * range_weight) / (max_int8_input * max_int8_weight);
+      const float bf = (float)bias_i32[j];
+      if (at->input_mode == ORC_MIN_FIRST) { /* :1254-1271 */
+        if (out_f32) bias_out[j] = bf * sj;
+        else if (out_q8) {
+          if (ep->n_scales == 0) { st = ORC_INVALID_ARGUMENT; break; }
+          bias_out[j] = bf * ((ep->n_scales == 1) ? scales[0] : scales[j]);
+        } else bias_out[j] = bf;
+      } else { /* :1273-1305: reorder of the 1-D bias with per-entry source scales */
+        bias_out[j] = bf * sj;
+      }
+    }
+    free(bias_scales);
+    return st;
+  }
   if (at->input_mode == ORC_MIN_FIRST) { /* :520-601 */
     const float q_min_input = max_int8_input * min_a / range_input; /* :557 */
     for (int64_t j = 0; j < N; ++j) {
@@ -443,6 +485,12 @@ static inline float apply_eltwise(const orc_eltwise* e, float x) {
       return fminf(fmaxf(x, e->alpha), e->beta);
     case ORC_ELT_LINEAR: /* alpha * x + beta */
       return e->alpha * x + e->beta;
+    case ORC_ELT_GELU_TANH: { /* eltwise_gelu_tanh: 0.5 x (1 + tanh(sqrt(2/pi) x (1 + 0.044715 x^2))) */
+      const float v = tanhf(0.79788458347320556640625f * x * (1.0f + 0.044715f * x * x));
+      return 0.5f * x * (1.0f + v);
+    }
+    case ORC_ELT_GELU_ERF: /* eltwise_gelu_erf: 0.5 x (1 + erf(x / sqrt(2))) */
+      return 0.5f * x * (1.0f + erff(x * 0.707106769084930419921875f));
     default: return x;
   }
 }
@@ -450,7 +498,8 @@ static inline float apply_eltwise(const orc_eltwise* e, float x) {
 /* oneDNN int8 inner-product epilogue (execute at quantized_matmul_common.h:92):
  * y = fl(fl((float)acc * scale[n]) + bias[n]) -> eltwise chain -> destination conversion. */
 void orc_qmatmul_epilogue(const int32_t* acc, int64_t M, int64_t N, const orc_epilogue_desc* ep,
-                          const float* scales, const float* bias, int t_out, void* out) {
+                          const float* scales, const float* bias, const float* addend, int t_out,
+                          void* out) {
   float lo = 0, hi = 0;
   if (t_out != ORC_FLOAT) sat_bounds(t_out, &lo, &hi);
 #pragma omp parallel for schedule(static)
@@ -460,7 +509,10 @@ void orc_qmatmul_epilogue(const int32_t* acc, int64_t M, int64_t N, const orc_ep
       if (ep->n_scales == 1) y = y * scales[0];
       else if (ep->n_scales > 1) y = y * scales[n];
       y = y + bias[n];
-      for (int e = 0; e < ep->n_eltwise; ++e) y = apply_eltwise(&ep->elt[e], y);
+      for (int e = 0; e < ep->n_eltwise; ++e) {
+        if (ep->elt[e].alg == ORC_ELT_SUM) y = y + ep->elt[e].alpha * addend[m * N + n]; /* dst = v + scale * dst */
+        else y = apply_eltwise(&ep->elt[e], y);
+      }
       if (t_out == ORC_FLOAT) ((float*)out)[m * N + n] = y;
       else store_q(out, m * N + n, t_out, sat_rne(y, lo, hi));
     }
@@ -504,9 +556,10 @@ int orc_qmatmul_output_minmax(const orc_matmul_attrs* at, float min_a, float max
 
 /* LegacyQuantizedMatMulOpBase::Compute, quantized_matmul_common.h:61-102 — whole op. */
 int orc_qmatmul(const orc_matmul_attrs* at, const void* a, const int8_t* w, int transpose_b,
-                int64_t M, int64_t K, int64_t N, const float* bias, float min_a, float max_a,
-                const float* min_b, const float* max_b, int64_t nb, float min_out, float max_out,
-                void* out) {
+                int64_t M, int64_t K, int64_t N, const void* bias, const float* addend, float min_a,
+                float max_a, const float* min_b, const float* max_b, int64_t nb, float min_out,
+                float max_out, void* out) {
+  if (at->add_position != 0 && addend == NULL) return ORC_INVALID_ARGUMENT;
   /* the compensation loop indexes the weight as [K,N] regardless of transpose_b (:569-573) */
   if (transpose_b && at->input_mode == ORC_MIN_FIRST) return ORC_UNIMPLEMENTED;
   int32_t* acc = (int32_t*)malloc(sizeof(int32_t) * (size_t)(M * N));
@@ -520,7 +573,7 @@ int orc_qmatmul(const orc_matmul_attrs* at, const void* a, const int8_t* w, int 
                                bias, scales, sb, &ep);
   if (st == ORC_OK) {
     orc_int_gemm(a, at->t_in, w, transpose_b, M, K, N, acc);
-    orc_qmatmul_epilogue(acc, M, N, &ep, scales, sb, at->t_out, out);
+    orc_qmatmul_epilogue(acc, M, N, &ep, scales, sb, addend, at->t_out, out);
   }
   free(acc); free(colsum); free(scales); free(sb);
   return st;

@@ -23,7 +23,10 @@
  * Parity unpinned (no reference-held vector and no way to execute oneDNN@242d4d9 here):
  *   NaN / Inf inputs to the quantizers; the result of the size-mismatched bias reorder in
  *   orc_qmatmul_prepare (SCALED input, per-channel weights; see the comment there);
- *   abs(INT32_MIN) in orc_requantization_range_per_channel (undefined behaviour upstream).
+ *   abs(INT32_MIN) in orc_requantization_range_per_channel (undefined behaviour upstream);
+ *   the last bits of the GELU post-ops (oneDNN evaluates tanh / erf with its own polynomial
+ *   kernels; here libm's tanhf / erff): pinned only against a float64 evaluation and at the
+ *   reference tests' own tolerance.
  */
 #ifndef ITEX_ORACLE_H_
 #define ITEX_ORACLE_H_
@@ -49,9 +52,11 @@ enum {
 };
 
 /* eltwise post-op algorithms (subset of onednn_post_op_util.cc:34-68) */
-enum { ORC_ELT_RELU = 1, ORC_ELT_CLIP = 2, ORC_ELT_LINEAR = 3 };
+enum { ORC_ELT_RELU = 1, ORC_ELT_CLIP = 2, ORC_ELT_LINEAR = 3, ORC_ELT_GELU_TANH = 4, ORC_ELT_GELU_ERF = 5,
+       ORC_ELT_SUM = 6 /* the "Add" post-op: y += alpha * addend[m,n] (append_sum, :256) */ };
 /* activation names accepted in fused_ops */
-enum { ORC_ACT_NONE = 0, ORC_ACT_RELU = 1, ORC_ACT_RELU6 = 2, ORC_ACT_LEAKYRELU = 3 };
+enum { ORC_ACT_NONE = 0, ORC_ACT_RELU = 1, ORC_ACT_RELU6 = 2, ORC_ACT_LEAKYRELU = 3, ORC_ACT_GELU_APPROX = 4,
+       ORC_ACT_GELU_EXACT = 5 };
 
 typedef struct {
   int alg;
@@ -70,12 +75,14 @@ typedef struct {
   int has_dequantize;    /* V2: "Dequantize" in fused_ops */
   int n_fused_ops;       /* V1: fused_ops.size() (1 = BiasAdd only, 2 = BiasAdd + activation) */
   float leakyrelu_alpha;
+  int add_position;      /* "Add" in fused_ops: 0 absent, 1 before the activation, 2 after it */
+  int t_bias;            /* 0 or ORC_FLOAT: fp32 bias;  ORC_QINT32: Tbias = qint32 (:1153-1334) */
 } orc_matmul_attrs;
 
 typedef struct {
   int n_scales;          /* 0 (no output scale), 1 (per tensor) or N (per output channel) */
-  int n_eltwise;         /* 0..2 */
-  orc_eltwise elt[2];
+  int n_eltwise;         /* 0..3, post-ops in fused_ops order */
+  orc_eltwise elt[3];
 } orc_epilogue_desc;
 
 int orc_adjust_input_range(float in_min, float in_max, float ensure_minimum_range,
@@ -103,18 +110,19 @@ void orc_weight_colsum(const int8_t* w, int64_t K, int64_t N, int32_t* colsum);
 
 int orc_qmatmul_prepare(const orc_matmul_attrs* at, int64_t N, const int32_t* colsum, float min_a,
                         float max_a, const float* min_b, const float* max_b, int64_t nb,
-                        float min_out, float max_out, const float* bias, float* scales,
+                        float min_out, float max_out, const void* bias, float* scales,
                         float* bias_out, orc_epilogue_desc* ep);
 void orc_qmatmul_epilogue(const int32_t* acc, int64_t M, int64_t N, const orc_epilogue_desc* ep,
-                          const float* scales, const float* bias, int t_out, void* out);
+                          const float* scales, const float* bias, const float* addend, int t_out,
+                          void* out);
 int orc_qmatmul_output_minmax(const orc_matmul_attrs* at, float min_a, float max_a,
                               const float* min_b, const float* max_b, int64_t nb, int b_rank,
                               float min_out, float max_out, float* out_min, float* out_max,
                               int64_t* n_out);
 int orc_qmatmul(const orc_matmul_attrs* at, const void* a, const int8_t* w, int transpose_b,
-                int64_t M, int64_t K, int64_t N, const float* bias, float min_a, float max_a,
-                const float* min_b, const float* max_b, int64_t nb, float min_out, float max_out,
-                void* out);
+                int64_t M, int64_t K, int64_t N, const void* bias, const float* addend, float min_a,
+                float max_a, const float* min_b, const float* max_b, int64_t nb, float min_out,
+                float max_out, void* out);
 
 #ifdef __cplusplus
 }

@@ -15,7 +15,7 @@ _LIB_PATH = os.path.join(_HERE, "libitex_oracle.so")
 FLOAT, INT32, QINT8, QUINT8, QINT32 = 1, 3, 11, 12, 13
 MIN_COMBINED, MIN_FIRST, SCALED = 0, 1, 2
 API_V2, API_V1, API_LEGACY = 0, 1, 2
-ACT_NONE, ACT_RELU, ACT_RELU6, ACT_LEAKYRELU = 0, 1, 2, 3
+ACT_NONE, ACT_RELU, ACT_RELU6, ACT_LEAKYRELU, ACT_GELU_APPROX, ACT_GELU_EXACT = 0, 1, 2, 3, 4, 5
 OK, INVALID_ARGUMENT, UNIMPLEMENTED = 0, 3, 12
 
 NP_OF = {QINT8: np.int8, QUINT8: np.uint8, QINT32: np.int32, FLOAT: np.float32}
@@ -35,11 +35,11 @@ class MatmulAttrs(C.Structure):
     _fields_ = [("api", C.c_int), ("t_in", C.c_int), ("t_out", C.c_int), ("input_mode", C.c_int),
                 ("out_min_first", C.c_int), ("activation", C.c_int), ("has_requantize", C.c_int),
                 ("has_dequantize", C.c_int), ("n_fused_ops", C.c_int),
-                ("leakyrelu_alpha", C.c_float)]
+                ("leakyrelu_alpha", C.c_float), ("add_position", C.c_int), ("t_bias", C.c_int)]
 
 
 class EpilogueDesc(C.Structure):
-    _fields_ = [("n_scales", C.c_int), ("n_eltwise", C.c_int), ("elt", Eltwise * 2)]
+    _fields_ = [("n_scales", C.c_int), ("n_eltwise", C.c_int), ("elt", Eltwise * 3)]
 
 
 _lib = None
@@ -167,16 +167,21 @@ def weight_colsum(w):
 
 def matmul_attrs(api=API_V2, t_in=QUINT8, t_out=FLOAT, input_mode=MIN_FIRST, out_min_first=False,
                  activation=ACT_NONE, has_requantize=False, has_dequantize=False, n_fused_ops=1,
-                 leakyrelu_alpha=0.2):
+                 leakyrelu_alpha=0.2, add_position=0, t_bias=0):
     return MatmulAttrs(api, t_in, t_out, input_mode, int(out_min_first), activation,
-                       int(has_requantize), int(has_dequantize), n_fused_ops, leakyrelu_alpha)
+                       int(has_requantize), int(has_dequantize), n_fused_ops, leakyrelu_alpha,
+                       int(add_position), int(t_bias))
+
+
+def _bias(at, bias):
+    return np.ascontiguousarray(bias, dtype=np.int32) if at.t_bias == QINT32 else _f32(bias)
 
 
 def qmatmul_prepare(at, N, colsum, min_a, max_a, min_b, max_b, min_out, max_out, bias):
     """Returns (status, scales[n_scales], scaled_bias[N], EpilogueDesc)."""
     min_b, max_b = _f32(min_b), _f32(max_b)
     nb = min_b.size
-    bias = _f32(bias)
+    bias = _bias(at, bias)
     colsum = np.ascontiguousarray(colsum, dtype=np.int32)
     scales = np.zeros(max(nb, 1), np.float32)
     sb = np.zeros(N, np.float32)
@@ -188,14 +193,15 @@ def qmatmul_prepare(at, N, colsum, min_a, max_a, min_b, max_b, min_out, max_out,
     return st, scales[:ep.n_scales].copy(), sb, ep
 
 
-def qmatmul_epilogue(acc, ep, scales, bias, t_out):
+def qmatmul_epilogue(acc, ep, scales, bias, t_out, addend=None):
     acc = np.ascontiguousarray(acc, dtype=np.int32)
     M, N = acc.shape
     scales = _f32(scales) if ep.n_scales else np.zeros(1, np.float32)
     bias = _f32(bias)
     out = np.zeros((M, N), NP_OF[t_out])
+    addend = None if addend is None else _f32(addend)
     lib().orc_qmatmul_epilogue(_p(acc), C.c_int64(M), C.c_int64(N), C.byref(ep), _p(scales),
-                               _p(bias), t_out, _p(out))
+                               _p(bias), _p(addend) if addend is not None else None, t_out, _p(out))
     return out
 
 
@@ -211,17 +217,19 @@ def qmatmul_output_minmax(at, min_a, max_a, min_b, max_b, b_rank, min_out, max_o
 
 
 def qmatmul(at, a, w, bias, min_a, max_a, min_b, max_b, min_out=0.0, max_out=0.0,
-            transpose_b=False):
+            transpose_b=False, addend=None):
     """Whole op.  Returns (status, out[M,N])."""
     a = np.ascontiguousarray(a)
     w = np.ascontiguousarray(w, dtype=np.int8)
     M, K = a.shape
     N = w.shape[0] if transpose_b else w.shape[1]
     min_b, max_b = _f32(min_b), _f32(max_b)
-    bias = _f32(bias)
+    bias = _bias(at, bias)
+    addend = None if addend is None else _f32(addend)
     out = np.zeros((M, N), NP_OF[at.t_out])
     st = lib().orc_qmatmul(C.byref(at), _p(a), _p(w), int(transpose_b), C.c_int64(M), C.c_int64(K),
-                           C.c_int64(N), _p(bias), C.c_float(min_a), C.c_float(max_a), _p(min_b),
+                           C.c_int64(N), _p(bias), _p(addend) if addend is not None else None,
+                           C.c_float(min_a), C.c_float(max_a), _p(min_b),
                            _p(max_b), C.c_int64(min_b.size), C.c_float(min_out), C.c_float(max_out),
                            _p(out))
     return st, out

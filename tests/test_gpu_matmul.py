@@ -412,3 +412,86 @@ def test_hip_graph_replays_match_eager(hip, dev):
         np.testing.assert_array_equal(got_mm, np.float32([x.min(), x.max()]))
         _, xq_ref, _, _ = orc.quantize_v2(x, mn, mx, orc.QUINT8, orc.MIN_FIRST)
         np.testing.assert_array_equal(got, layer.oracle(xq_ref, kw, amn, amx))
+
+
+def _run_single_launch(hip, dev, layer, kw, xq, mn, mx, bias_host, addend=None, lo=0.0, hi=0.0):
+    import torch
+    M = xq.shape[0]
+    p = hip.matmul_params(t_in=orc.QUINT8 if xq.dtype == np.uint8 else orc.QINT8, min_a=float(mn), max_a=float(mx),
+                          min_out=float(lo), max_out=float(hi), **kw)
+    out = torch.empty((M, layer.N), dtype=tdt(kw["t_out"]), device=dev)
+    bias_d = torch.from_numpy(np.ascontiguousarray(bias_host)).to(dev)
+    add_d = None if addend is None else torch.from_numpy(np.ascontiguousarray(addend)).to(dev)
+    hip.qmatmul(p, torch.from_numpy(xq).to(dev), layer.packed, layer.colsum, M, layer.K, layer.N, layer.min_b_d,
+                layer.max_b_d, layer.min_b.size, bias_d, out, addend=add_d)
+    torch.cuda.synchronize()
+    return out.cpu().numpy()
+
+
+@pytest.mark.parametrize("M", [3, 150])
+@pytest.mark.parametrize("pos,act", [(1, orc.ACT_NONE), (1, orc.ACT_RELU), (2, orc.ACT_RELU), (2, orc.ACT_LEAKYRELU)])
+def test_add_fusion_vs_oracle(hip, dev, M, pos, act):
+    """[BiasAdd, Add, (act), Dequantize] and [BiasAdd, act, Add, Dequantize]: the addend is added in fp32 at its
+    place in the post-op chain; GEMV (M = 3) and tile (M = 150) paths, N not a multiple of 4."""
+    K, N = 256, 203
+    layer, w, bias = make_layer(hip, dev, K, N, seed=31)
+    x, xq, mn, mx = make_acts(M, K, seed=M)
+    z = (np.random.default_rng(4).standard_normal((M, N)) * 2).astype(np.float32)
+    kw = dict(api=orc.API_V2, t_out=orc.FLOAT, input_mode=orc.MIN_FIRST, has_dequantize=True, activation=act,
+              add_position=pos, leakyrelu_alpha=0.3)
+    st, ref = orc.qmatmul(orc.matmul_attrs(t_in=orc.QUINT8, **kw), xq, layer.wq, bias, mn, mx, layer.min_b, layer.max_b,
+                          addend=z)
+    assert st == orc.OK
+    np.testing.assert_array_equal(_run_single_launch(hip, dev, layer, kw, xq, mn, mx, bias, z), ref)
+    with pytest.raises(hip.ItexHipError):   # the addend and "Add" go together
+        _run_single_launch(hip, dev, layer, kw, xq, mn, mx, bias, None)
+    with pytest.raises(hip.ItexHipError):   # a quantized addend does not exist
+        _run_single_launch(hip, dev, layer, dict(kw, t_out=orc.QINT8, has_requantize=True, has_dequantize=False), xq, mn, mx,
+                           bias, z, -1, 1)
+
+
+@pytest.mark.parametrize("M", [4, 130])
+@pytest.mark.parametrize("act", [orc.ACT_GELU_APPROX, orc.ACT_GELU_EXACT])
+def test_gelu_fusion_close_to_oracle(hip, dev, M, act):
+    """GELU post-ops: the device's tanhf / erff need not round like the host's (nor like oneDNN's own
+    kernels), so this is a tolerance check (2e-6 relative, 1e-6 absolute) - parity unpinned at bit level."""
+    K, N = 512, 256
+    layer, w, bias = make_layer(hip, dev, K, N, seed=32)
+    x, xq, mn, mx = make_acts(M, K, seed=M + 9)
+    kw = dict(api=orc.API_V2, t_out=orc.FLOAT, input_mode=orc.MIN_FIRST, has_dequantize=True, activation=act)
+    ref = layer.oracle(xq, kw, mn, mx)
+    got = _run_single_launch(hip, dev, layer, kw, xq, mn, mx, bias)
+    np.testing.assert_allclose(got, ref, rtol=2e-6, atol=1e-6)
+    gelu = x @ w + bias
+    gelu = 0.5 * gelu * (1 + np.tanh(np.sqrt(2 / np.pi) * (gelu + 0.044715 * gelu ** 3)))
+    if act == orc.ACT_GELU_APPROX:
+        np.testing.assert_allclose(got, gelu, rtol=0.2, atol=0.2)   # the reference test's own bar
+
+
+@pytest.mark.parametrize("M", [2, 140])
+@pytest.mark.parametrize("t_out,mode", [(orc.FLOAT, orc.MIN_FIRST), (orc.QINT8, orc.MIN_FIRST), (orc.QINT32, orc.MIN_FIRST),
+                                        (orc.FLOAT, orc.SCALED)])
+def test_qint32_bias_vs_oracle(hip, dev, M, t_out, mode):
+    K, N = 320, 144
+    layer, w, _ = make_layer(hip, dev, K, N, seed=33)
+    x, xq, mn, mx = make_acts(M, K, seed=M + 3, mode=mode)
+    b32 = np.random.default_rng(6).integers(-3000, 3000, N).astype(np.int32)
+    kw = dict(api=orc.API_V2 if t_out != orc.QINT32 else orc.API_V1, t_out=t_out, input_mode=mode,
+              has_dequantize=t_out == orc.FLOAT, has_requantize=t_out == orc.QINT8, t_bias=orc.QINT32)
+    st, ref = orc.qmatmul(orc.matmul_attrs(t_in=orc.QUINT8 if mode == orc.MIN_FIRST else orc.QINT8, **kw), xq, layer.wq, b32,
+                          mn, mx, layer.min_b, layer.max_b, -40.0, 40.0)
+    assert st == orc.OK
+    got = _run_single_launch(hip, dev, layer, kw, xq, mn, mx, b32, lo=-40.0, hi=40.0)
+    np.testing.assert_array_equal(got, ref)
+    # the two-launch form prepares the same vectors
+    import torch
+    p = hip.matmul_params(t_in=orc.QUINT8 if mode == orc.MIN_FIRST else orc.QINT8, min_a=float(mn), max_a=float(mx),
+                          min_out=-40.0, max_out=40.0, **kw)
+    ep = hip.qmatmul_epilogue_desc(p, layer.min_b.size)
+    hip.qmatmul_prepare(p, layer.min_b_d, layer.max_b_d, layer.min_b.size, torch.from_numpy(b32).to(dev), layer.colsum, N,
+                        layer.scales_d, layer.sbias_d)
+    out = torch.empty((M, N), dtype=tdt(t_out), device=dev)
+    hip.qgemm(torch.from_numpy(xq).to(dev), p.t_in, layer.packed, layer.colsum, M, K, N, layer.scales_d, layer.sbias_d, ep,
+              t_out, out)
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(out.cpu().numpy(), ref)

@@ -300,3 +300,88 @@ def test_requantize_per_channel_ops(rt, dev):
     _, q_ref, _, _ = orc.requantize_per_channel(x, in_min, in_max, float(rmin), float(rmax), orc.QINT8)
     np.testing.assert_array_equal(fetch(torch, outs[0], np.int8), q_ref)
     node.close()
+
+
+def _ref_constants(golden):
+    g = golden["fused_matmul"]
+    x, w, b = (np.array(g[k], np.float32) for k in ("x", "w", "bias"))
+    z = np.array(golden["fused_matmul_addend"], np.float32) * 2
+    _, xq, xmn, xmx = orc.quantize_v2(x, x.min(), x.max(), orc.QUINT8, orc.MIN_FIRST)
+    _, wq, wmn, wmx = orc.quantize_v2(w, w.min(), w.max(), orc.QINT8, orc.SCALED)
+    f = lambda v: np.array(v[0], np.float32)
+    return g, x, w, b, z, xq, f(xmn), f(xmx), wq, f(wmn), f(wmx)
+
+
+@pytest.mark.parametrize("api", ["V1", "V2"])
+def test_reference_add_post_op_case_through_plugin(rt, dev, golden, api):
+    """_testAddPostop of the reference's native_quantized_fused_matmul_test.py (K = 3: the unpacked-weight
+    path): [BiasAdd, Add] with the addend as an extra device input that shifts the min/max inputs."""
+    torch = rt
+    g, x, w, b, z, xq, xmn, xmx, wq, wmn, wmx = _ref_constants(golden)
+    if api == "V1":
+        node = tf.Node("_QuantizedFusedMatMulAndDequantize",
+                       dict(T1=DT(tf.QUINT8), T2=DT(tf.QINT8), Targs=DT(tf.FLOAT), Toutput=DT(tf.FLOAT), num_args=2,
+                            transpose_a=False, transpose_b=False, fused_ops=["BiasAdd", "Add"], is_filter_const=True,
+                            is_bias_const=True, input_quant_mode="MIN_FIRST", leakyrelu_alpha=0.2))
+        at = orc.matmul_attrs(api=orc.API_V1, t_out=orc.FLOAT, add_position=1, n_fused_ops=2)
+    else:
+        node = tf.Node("_QuantizedMatMul", dict(V2, Tout=DT(tf.FLOAT), fused_ops=["BiasAdd", "Add", "Dequantize"]))
+        at = orc.matmul_attrs(api=orc.API_V2, t_out=orc.FLOAT, has_dequantize=True, add_position=1)
+    assert node.code == tf.OK, node.message
+    ins, keep = matmul_inputs(torch, dev, xq, wq, b, [])
+    z_d = dev_in(torch, dev, z)
+    ins.append((tf.FLOAT, z.shape, z_d.data_ptr(), False))
+    for s in (xmn, xmx, wmn, wmx):
+        ins.append((tf.FLOAT, s.shape, tf.host_array(s), True))
+    for _ in range(2):   # the reference runs it twice "to check the functionality of object cache"
+        code, msg, outs = node.run(ins, [(tf.FLOAT, False)], stream=torch.cuda.current_stream().cuda_stream)
+        assert code == tf.OK, msg
+        y = fetch(torch, outs[0], np.float32)
+        np.testing.assert_allclose(y, x @ w + b + z, rtol=g["tolerance"], atol=g["tolerance"])
+        _, y_ref = orc.qmatmul(at, xq, wq, b, xmn, xmx, wmn, wmx, addend=z)
+        np.testing.assert_array_equal(y, y_ref)
+    node.close()
+
+
+@pytest.mark.parametrize("per_channel", [False, True])
+def test_reference_gelu_case_through_plugin(rt, dev, golden, per_channel):
+    """_testGeluPerTensorPostop / _testGeluPerchannelPostop: [BiasAdd, GeluApproximate, Dequantize] within the
+    reference's tolerance of the fp32 graph; close to the oracle (the transcendental is unpinned at bit level)."""
+    torch = rt
+    g, x, w, b, z, xq, xmn, xmx, wq, wmn, wmx = _ref_constants(golden)
+    if per_channel:
+        _, wq, wmn, wmx = orc.quantize_v2(w, w.min(0), w.max(0), orc.QINT8, orc.SCALED, axis=1)
+    node = tf.Node("_QuantizedMatMul", dict(V2, Tout=DT(tf.FLOAT), fused_ops=["BiasAdd", "GeluApproximate", "Dequantize"]))
+    assert node.code == tf.OK, node.message
+    ins, keep = matmul_inputs(torch, dev, xq, wq, b, [xmn, xmx, wmn, wmx])
+    code, msg, outs = node.run(ins, [(tf.FLOAT, False)], stream=torch.cuda.current_stream().cuda_stream)
+    assert code == tf.OK, msg
+    y = fetch(torch, outs[0], np.float32)
+    pre = (x @ w + b).astype(np.float64)
+    gelu = 0.5 * pre * (1 + np.tanh(np.sqrt(2 / np.pi) * (pre + 0.044715 * pre ** 3)))
+    np.testing.assert_allclose(y, gelu, rtol=g["tolerance"], atol=g["tolerance"])
+    at = orc.matmul_attrs(api=orc.API_V2, t_out=orc.FLOAT, has_dequantize=True, activation=orc.ACT_GELU_APPROX)
+    _, y_ref = orc.qmatmul(at, xq, wq, b, xmn, xmx, wmn, wmx)
+    np.testing.assert_allclose(y, y_ref, rtol=2e-6, atol=1e-6)
+    node.close()
+
+
+def test_reference_qint32_bias_case_through_plugin(rt, dev, golden):
+    """The qint32-bias variant of _testAddPostop (run there without an assertion): Tbias = qint32 selects the
+    second kernel registration; result bit-equal to the oracle's as-written semantics."""
+    torch = rt
+    g, x, w, b, z, xq, xmn, xmx, wq, wmn, wmx = _ref_constants(golden)
+    b32 = np.array(golden["fused_matmul_bias_qint32"], np.int32)
+    node = tf.Node("_QuantizedMatMul", dict(V2, Tbias=DT(tf.QINT32), Tout=DT(tf.FLOAT), fused_ops=["BiasAdd", "Add", "Dequantize"]))
+    assert node.code == tf.OK, node.message
+    keep = [dev_in(torch, dev, v) for v in (xq, wq, b32, z)]
+    ins = [(tf.QUINT8, xq.shape, keep[0].data_ptr(), False), (tf.QINT8, wq.shape, keep[1].data_ptr(), False),
+           (tf.QINT32, b32.shape, keep[2].data_ptr(), False), (tf.FLOAT, z.shape, keep[3].data_ptr(), False)]
+    for s in (xmn, xmx, wmn, wmx):
+        ins.append((tf.FLOAT, s.shape, tf.host_array(s), True))
+    code, msg, outs = node.run(ins, [(tf.FLOAT, False)], stream=torch.cuda.current_stream().cuda_stream)
+    assert code == tf.OK, msg
+    at = orc.matmul_attrs(api=orc.API_V2, t_out=orc.FLOAT, has_dequantize=True, add_position=1, t_bias=orc.QINT32)
+    _, y_ref = orc.qmatmul(at, xq, wq, b32, xmn, xmx, wmn, wmx, addend=z)
+    np.testing.assert_array_equal(fetch(torch, outs[0], np.float32), y_ref)
+    node.close()

@@ -249,3 +249,112 @@ def test_epilogue_against_torch_onednn():
     ep.elt[0].alg, ep.elt[0].alpha, ep.elt[0].beta = 1, 0.0, 0.0
     np.testing.assert_array_equal(outs[("relu", torch.float32)].numpy(),
                                   orc.qmatmul_epilogue(acc, ep, sw, b, orc.FLOAT))
+
+
+# ------------------------------------------------------------------------------------------------
+# "Add" (sum post-op), GELU post-ops and the qint32 bias
+# ------------------------------------------------------------------------------------------------
+def _toy(seed=0, M=7, K=48, N=12):
+    rng = np.random.default_rng(seed)
+    x = rng.standard_normal((M, K)).astype(np.float32)
+    w = (rng.standard_normal((K, N)) * 0.05).astype(np.float32)
+    _, xq, mn, mx = orc.quantize_v2(x, x.min(), x.max(), orc.QUINT8, orc.MIN_FIRST)
+    r = np.abs(w).max(0).astype(np.float32)
+    _, wq, wmn, wmx = orc.quantize_v2(w, -r, r, orc.QINT8, orc.SCALED, axis=1)
+    return x, w, xq, float(mn[0]), float(mx[0]), wq, wmn, wmx
+
+
+def test_add_post_op_is_a_separately_rounded_fp32_add_in_fused_ops_order():
+    x, w, xq, mn, mx, wq, wmn, wmx = _toy()
+    M, N = x.shape[0], w.shape[1]
+    rng = np.random.default_rng(1)
+    bias = rng.standard_normal(N).astype(np.float32)
+    z = (rng.standard_normal((M, N)) * 3).astype(np.float32)
+    base = orc.matmul_attrs(t_out=orc.FLOAT, has_dequantize=True)
+    _, y0 = orc.qmatmul(base, xq, wq, bias, mn, mx, wmn, wmx)
+    for pos, act in ((1, orc.ACT_NONE), (1, orc.ACT_RELU), (2, orc.ACT_RELU)):
+        at = orc.matmul_attrs(t_out=orc.FLOAT, has_dequantize=True, activation=act, add_position=pos)
+        st, y = orc.qmatmul(at, xq, wq, bias, mn, mx, wmn, wmx, addend=z)
+        assert st == orc.OK
+        if act == orc.ACT_NONE:
+            expect = y0 + z                              # one fp32 add on the rounded pre-add value
+        elif pos == 1:
+            expect = np.maximum(y0 + z, np.float32(0))   # [BiasAdd, Add, Relu]
+        else:
+            expect = np.maximum(y0, np.float32(0)) + z   # [BiasAdd, Relu, Add]
+        np.testing.assert_array_equal(y, expect.astype(np.float32))
+    # the two orders differ wherever relu clips
+    # a quantized addend does not exist upstream: refused, like a missing addend
+    at = orc.matmul_attrs(t_out=orc.QINT8, has_requantize=True, add_position=1)
+    assert orc.qmatmul(at, xq, wq, bias, mn, mx, wmn, wmx, -1.0, 1.0, addend=z)[0] == orc.UNIMPLEMENTED
+    at = orc.matmul_attrs(t_out=orc.FLOAT, has_dequantize=True, add_position=1)
+    assert orc.qmatmul(at, xq, wq, bias, mn, mx, wmn, wmx)[0] == orc.INVALID_ARGUMENT
+
+
+def test_reference_add_post_op_constants(golden):
+    """The constants of the reference's _testAddPostop (native_quantized_fused_matmul_test.py:141-193):
+    [BiasAdd, Add, Dequantize] within its own tolerance of the fp32 graph."""
+    g = golden["fused_matmul"]
+    x, w, b = (np.array(g[k], np.float32) for k in ("x", "w", "bias"))
+    z = np.array(golden["fused_matmul_addend"], np.float32) * 2     # the test doubles it (z + z)
+    _, xq, mn, mx = orc.quantize_v2(x, x.min(), x.max(), orc.QUINT8, orc.MIN_FIRST)
+    _, wq, wmn, wmx = orc.quantize_v2(w, w.min(), w.max(), orc.QINT8, orc.SCALED)
+    for api in (orc.API_V1, orc.API_V2):
+        at = orc.matmul_attrs(api=api, t_out=orc.FLOAT, has_dequantize=True, add_position=1, n_fused_ops=2)
+        st, y = orc.qmatmul(at, xq, wq, b, mn[0], mx[0], wmn, wmx, addend=z)
+        assert st == orc.OK
+        np.testing.assert_allclose(y, x @ w + b + z, rtol=g["tolerance"], atol=g["tolerance"])
+
+
+@pytest.mark.parametrize("act,fn", [
+    (orc.ACT_GELU_APPROX, lambda v: 0.5 * v * (1 + np.tanh(np.sqrt(2 / np.pi) * (v + 0.044715 * v ** 3)))),
+    (orc.ACT_GELU_EXACT, lambda v: 0.5 * v * (1 + np.vectorize(__import__("math").erf)(v / np.sqrt(2))))])
+def test_gelu_post_ops_against_float64(act, fn):
+    """Bit-level parity with oneDNN's own tanh / erf kernels is unpinned; the formula is pinned against a
+    float64 evaluation, at 0 and in both tails."""
+    x, w, xq, mn, mx, wq, wmn, wmx = _toy(seed=2, M=40, K=64, N=24)
+    bias = np.linspace(-3, 3, 24).astype(np.float32)
+    base = orc.matmul_attrs(t_out=orc.FLOAT, has_dequantize=True)
+    _, y0 = orc.qmatmul(base, xq, wq, bias, mn, mx, wmn, wmx)
+    at = orc.matmul_attrs(t_out=orc.FLOAT, has_dequantize=True, activation=act)
+    st, y = orc.qmatmul(at, xq, wq, bias, mn, mx, wmn, wmx)
+    assert st == orc.OK
+    np.testing.assert_allclose(y, fn(y0.astype(np.float64)), rtol=2e-6, atol=2e-7)
+    ep = orc.EpilogueDesc()
+    ep.n_eltwise = 1
+    ep.elt[0].alg = 4 if act == orc.ACT_GELU_APPROX else 5
+    acc = np.array([[0, 1 << 20, -(1 << 20), 3, -3]], np.int32)
+    out = orc.qmatmul_epilogue(acc, ep, np.zeros(1, np.float32), np.zeros(5, np.float32), orc.FLOAT)
+    assert out[0, 0] == 0 and out[0, 1] == np.float32(1 << 20) and abs(out[0, 2]) == 0
+    assert 2.99 < out[0, 3] < 3 and -0.01 < out[0, 4] < 0
+
+
+@pytest.mark.parametrize("mode", [orc.MIN_FIRST, orc.SCALED])
+@pytest.mark.parametrize("t_out", [orc.FLOAT, orc.QINT8, orc.QINT32])
+@pytest.mark.parametrize("per_channel", [True, False])
+def test_qint32_bias_closed_forms(mode, t_out, per_channel):
+    """Tbias = qint32: the bias is cast to fp32 and multiplied by the inverse of the fp32 path's factor;
+    no zero-point compensation (quantized_matmul_common.h:1204-1271)."""
+    N = 9
+    rng = np.random.default_rng(3)
+    b = rng.integers(-5000, 5000, N).astype(np.int32)
+    wmn = -(rng.random(N if per_channel else 1).astype(np.float32) + 0.5)
+    wmx = -wmn * np.float32(0.9)
+    colsum = rng.integers(-999, 999, N).astype(np.int32)
+    min_a, max_a = np.float32(-1.25), np.float32(2.5)
+    at = orc.matmul_attrs(t_in=orc.QUINT8 if mode == orc.MIN_FIRST else orc.QINT8, t_out=t_out, input_mode=mode,
+                          has_dequantize=t_out == orc.FLOAT, has_requantize=t_out == orc.QINT8, t_bias=orc.QINT32)
+    st, scales, sb, ep = orc.qmatmul_prepare(at, N, colsum, min_a, max_a, wmn, wmx, -3.0, 3.0, b)
+    assert st == orc.OK
+    A = np.float32(255 if mode == orc.MIN_FIRST else 127)
+    r_in = (max_a - min_a) if mode == orc.MIN_FIRST else np.float32(2.5)
+    r_w = np.maximum(np.abs(wmn), np.abs(wmx))
+    bs = np.broadcast_to(((r_in * r_w) / (A * np.float32(127))).astype(np.float32), (N,))
+    bf = b.astype(np.float32)
+    if mode == orc.SCALED or t_out == orc.FLOAT:
+        expect = bf * bs
+    elif t_out == orc.QINT8:
+        expect = bf * np.broadcast_to(scales, (N,))
+    else:
+        expect = bf
+    np.testing.assert_array_equal(sb, expect.astype(np.float32))

@@ -58,7 +58,10 @@ def test_host_memory_and_constraints(reg):
     deq = kernels_of(reg, "_QuantizedFusedMatMulAndDequantize")
     assert all(k["host_memory"] == ["min_a", "max_a", "min_b", "max_b"] for k in deq)
     legacy = kernels_of(reg, "QuantizedMatMulWithBiasAndReluAndRequantize")
-    assert len(legacy) == 1 and legacy[0]["constraints"] == {"T1": tf.QUINT8, "T2": tf.QINT8, "Tbias": tf.FLOAT, "Toutput": tf.QUINT8}
+    assert len(legacy) == 2 and {k["constraints"]["Tbias"] for k in legacy} == {tf.FLOAT, tf.QINT32}
+    assert all({**k["constraints"], "Tbias": 0} == {"T1": tf.QUINT8, "T2": tf.QINT8, "Tbias": 0, "Toutput": tf.QUINT8}
+               for k in legacy)
+    assert {k["constraints"]["Tbias"] for k in v2} == {tf.FLOAT, tf.QINT32}
 
 
 def test_op_definitions_only_for_missing_ops(reg):
