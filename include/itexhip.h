@@ -35,7 +35,9 @@ enum {
   ITEXHIP_INT32 = 3,
   ITEXHIP_QINT8 = 11,
   ITEXHIP_QUINT8 = 12,
-  ITEXHIP_QINT32 = 13
+  ITEXHIP_QINT32 = 13,
+  ITEXHIP_BFLOAT16 = 14,
+  ITEXHIP_HALF = 19
 };
 
 /* QuantizeMode, numbered like itex/core/utils/quantization_util.h:29-33 */
@@ -117,6 +119,20 @@ int itexhip_dequantize(const void* q, float* y, int64_t n, int src_type, float s
 int itexhip_dequantize_axis(const void* q, float* y, int64_t outer, int64_t slices, int64_t inner,
                             int src_type, const float* scales, const int32_t* zero_points,
                             void* stream);
+
+/* 16-bit floating point ends of the two ops: QuantizeV2 from a bfloat16 tensor (_ITEXQuantizeV2 with
+ * dtype = bfloat16, itex/core/kernels/gpu/quantize_op.cc:38-51) and Dequantize to bfloat16 or half
+ * (itex/core/kernels/gpu/dequantize_op.cc:24-48).  Same arithmetic in fp32: the bfloat16 source is
+ * widened exactly, the 16-bit result is the fp32 value rounded to nearest even. */
+int itexhip_quantize_bf16(const void* x, void* q, int64_t n, int dst_type, float scale, float addend,
+                          void* stream);
+int itexhip_quantize_axis_bf16(const void* x, void* q, int64_t outer, int64_t slices, int64_t inner,
+                               int dst_type, const float* scales, const float* addends, void* stream);
+int itexhip_dequantize16(const void* q, void* y, int64_t n, int src_type, int y_type, float scale,
+                         int32_t zero_point, void* stream);
+int itexhip_dequantize_axis16(const void* q, void* y, int64_t outer, int64_t slices, int64_t inner,
+                              int src_type, int y_type, const float* scales, const int32_t* zero_points,
+                              void* stream);
 
 /* ------------------------------------------------------------------------------------------
  * RequantizePerChannel.  q[r, c] = sat_T(rne((float)x[r, c] * scale[c])), channel = last dim

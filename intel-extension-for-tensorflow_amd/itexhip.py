@@ -11,7 +11,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "lib", "libitexhip.so")
 
 OK, INVALID_ARGUMENT, UNIMPLEMENTED, INTERNAL = 0, 3, 12, 13
-FLOAT, INT32, QINT8, QUINT8, QINT32 = 1, 3, 11, 12, 13
+FLOAT, INT32, QINT8, QUINT8, QINT32, BFLOAT16, HALF = 1, 3, 11, 12, 13, 14, 19
 MIN_COMBINED, MIN_FIRST, SCALED = 0, 1, 2
 API_V2, API_V1, API_LEGACY = 0, 1, 2
 ACT_NONE, ACT_RELU, ACT_RELU6, ACT_LEAKYRELU, ACT_GELU_APPROX, ACT_GELU_EXACT = 0, 1, 2, 3, 4, 5
@@ -24,7 +24,8 @@ EXPORTS = [
     "itexhip_event_query", "itexhip_event_synchronize", "itexhip_stream_wait_event", "itexhip_device_synchronize",
     "itexhip_memcpy_d2h_async", "itexhip_memset8_async", "itexhip_memset32_async", "itexhip_launch_host_func",
     "itexhip_last_error", "itexhip_build_info", "itexhip_memcpy_h2d_async", "itexhip_memcpy_d2h", "itexhip_memcpy_d2d_async", "itexhip_stream_synchronize", "itexhip_quantize", "itexhip_quantize_axis",
-    "itexhip_dequantize", "itexhip_dequantize_axis", "itexhip_requantize_per_channel",
+    "itexhip_dequantize", "itexhip_dequantize_axis", "itexhip_quantize_bf16", "itexhip_quantize_axis_bf16",
+    "itexhip_dequantize16", "itexhip_dequantize_axis16", "itexhip_requantize_per_channel",
     "itexhip_requantize", "itexhip_minmax_i32_per_channel", "itexhip_minmax_f32",
     "itexhip_qmatmul_epilogue_desc", "itexhip_qmatmul_prepare", "itexhip_qgemm_packed_bytes",
     "itexhip_qgemm_prepack_b", "itexhip_qgemm", "itexhip_qgemm_tile", "itexhip_qgemv", "itexhip_qmatmul", "itexhip_qmatmul_per_row", "itexhip_qmatmul_unpacked", "itexhip_mfma_probe",
@@ -111,6 +112,26 @@ def quantize(x, q, n, dst_type, scale, addend=0.0, stream=0):
 def quantize_axis(x, q, outer, slices, inner, dst_type, scales, addends=None, stream=0):
     _check(_lib.itexhip_quantize_axis(_ptr(x), _ptr(q), _i64(outer), _i64(slices), _i64(inner),
                                       dst_type, _ptr(scales), _ptr(addends), _ptr(stream)))
+
+
+def quantize_bf16(x, q, n, dst_type, scale, addend=0.0, stream=0):
+    _check(_lib.itexhip_quantize_bf16(_ptr(x), _ptr(q), _i64(n), dst_type, C.c_float(scale), C.c_float(addend),
+                                      _ptr(stream)))
+
+
+def quantize_axis_bf16(x, q, outer, slices, inner, dst_type, scales, addends=None, stream=0):
+    _check(_lib.itexhip_quantize_axis_bf16(_ptr(x), _ptr(q), _i64(outer), _i64(slices), _i64(inner), dst_type,
+                                           _ptr(scales), _ptr(addends), _ptr(stream)))
+
+
+def dequantize16(q, y, n, src_type, y_type, scale, zero_point=0, stream=0):
+    _check(_lib.itexhip_dequantize16(_ptr(q), _ptr(y), _i64(n), src_type, y_type, C.c_float(scale),
+                                     C.c_int32(int(zero_point)), _ptr(stream)))
+
+
+def dequantize_axis16(q, y, outer, slices, inner, src_type, y_type, scales, zero_points=None, stream=0):
+    _check(_lib.itexhip_dequantize_axis16(_ptr(q), _ptr(y), _i64(outer), _i64(slices), _i64(inner), src_type, y_type,
+                                          _ptr(scales), _ptr(zero_points), _ptr(stream)))
 
 
 def dequantize(q, y, n, src_type, scale, zero_point=0, stream=0):

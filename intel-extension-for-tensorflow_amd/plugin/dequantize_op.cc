@@ -30,7 +30,9 @@ class DequantizeOp : public OpKernel {
     if (ctx->HasAttr("dtype")) {
       TF_DataType dtype = TF_FLOAT;
       ITEX_REQUIRES_OK(ctx, ctx->GetAttr("dtype", &dtype));
-      ITEX_REQUIRES(ctx, dtype == TF_FLOAT, TF_UNIMPLEMENTED, "Dequantize on this device produces float only");
+      ITEX_REQUIRES(ctx, dtype == TF_FLOAT || dtype == TF_BFLOAT16 || dtype == TF_HALF, TF_INVALID_ARGUMENT,
+                    "Dequantize produces float, bfloat16 or half");
+      dst_type_ = dtype;
     }
   }
 
@@ -50,11 +52,13 @@ class DequantizeOp : public OpKernel {
       if (mode_ != Mode::MIN_FIRST) zp[i] = 0;
     }
     const std::vector<int64_t> shape = src.shape();
-    Tensor dst = ctx->allocate_output(0, TF_FLOAT, shape);
+    Tensor dst = ctx->allocate_output(0, dst_type_, shape);
     if (!ctx->ok()) return;
     int st;
     if (num_slices == 1) {
-      st = itexhip_dequantize(src.data(), dst.flat<float>(), src.NumElements(), T_, scale[0], zp[0], ctx->stream());
+      st = dst_type_ == TF_FLOAT
+               ? itexhip_dequantize(src.data(), dst.flat<float>(), src.NumElements(), T_, scale[0], zp[0], ctx->stream())
+               : itexhip_dequantize16(src.data(), dst.data(), src.NumElements(), T_, dst_type_, scale[0], zp[0], ctx->stream());
     } else {
       ITEX_REQUIRES(ctx, axis_ < static_cast<int>(shape.size()) && shape[axis_] == num_slices, TF_INVALID_ARGUMENT,
                     "min_range has " + std::to_string(num_slices) + " entries but dimension " + std::to_string(axis_) +
@@ -65,8 +69,11 @@ class DequantizeOp : public OpKernel {
       float* sc_dev = scales_.Get(ctx, scale.data(), scale.size(), TF_FLOAT);
       int32_t* zp_dev = zps_.Get(ctx, zp.data(), zp.size(), TF_INT32);
       if (sc_dev == nullptr || zp_dev == nullptr) return;
-      st = itexhip_dequantize_axis(src.data(), dst.flat<float>(), outer, num_slices, inner, T_, sc_dev, zp_dev,
-                                   ctx->stream());
+      st = dst_type_ == TF_FLOAT
+               ? itexhip_dequantize_axis(src.data(), dst.flat<float>(), outer, num_slices, inner, T_, sc_dev, zp_dev,
+                                         ctx->stream())
+               : itexhip_dequantize_axis16(src.data(), dst.data(), outer, num_slices, inner, T_, dst_type_, sc_dev, zp_dev,
+                                           ctx->stream());
     }
     ITEX_REQUIRES(ctx, st == ITEXHIP_OK, st == ITEXHIP_INVALID_ARGUMENT ? TF_INVALID_ARGUMENT : TF_ABORTED,
                   std::string("Operation received an exception: ") + itexhip_last_error());
@@ -74,6 +81,7 @@ class DequantizeOp : public OpKernel {
 
  private:
   TF_DataType T_;
+  TF_DataType dst_type_ = TF_FLOAT;
   Mode mode_ = Mode::SCALED;
   bool narrow_range_ = false;
   int32_t axis_ = -1;
@@ -91,12 +99,14 @@ struct DequantizeQuint8 : DequantizeOp { explicit DequantizeQuint8(OpKernelConst
 // such graphs stay placeable.
 void AddDequantizeKernels() {
   for (const char* op : {"Dequantize", "_ITEXDequantize"}) {
-    KernelDefBuilder s(op, "DequantizeOp");
-    s.TypeConstraint("T", TF_QINT8).TypeConstraint("dtype", TF_FLOAT).HostMemory("min_range").HostMemory("max_range");
-    s.Register<DequantizeQint8>();
-    KernelDefBuilder u(op, "DequantizeOp");
-    u.TypeConstraint("T", TF_QUINT8).TypeConstraint("dtype", TF_FLOAT).HostMemory("min_range").HostMemory("max_range");
-    u.Register<DequantizeQuint8>();
+    for (TF_DataType dtype : {TF_FLOAT, TF_BFLOAT16, TF_HALF}) {
+      KernelDefBuilder s(op, "DequantizeOp");
+      s.TypeConstraint("T", TF_QINT8).TypeConstraint("dtype", dtype).HostMemory("min_range").HostMemory("max_range");
+      s.Register<DequantizeQint8>();
+      KernelDefBuilder u(op, "DequantizeOp");
+      u.TypeConstraint("T", TF_QUINT8).TypeConstraint("dtype", dtype).HostMemory("min_range").HostMemory("max_range");
+      u.Register<DequantizeQuint8>();
+    }
   }
 }
 

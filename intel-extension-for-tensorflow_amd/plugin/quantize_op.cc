@@ -46,7 +46,9 @@ class QuantizeV2Op : public OpKernel {
     if (ctx->HasAttr("dtype")) {
       TF_DataType dtype = TF_FLOAT;
       ITEX_REQUIRES_OK(ctx, ctx->GetAttr("dtype", &dtype));
-      ITEX_REQUIRES(ctx, dtype == TF_FLOAT, TF_UNIMPLEMENTED, "_ITEXQuantizeV2 on this device takes float input only");
+      ITEX_REQUIRES(ctx, dtype == TF_FLOAT || dtype == TF_BFLOAT16, TF_UNIMPLEMENTED,
+                    "_ITEXQuantizeV2 on this device takes float or bfloat16 input");
+      src_type_ = dtype;
     }
   }
 
@@ -55,7 +57,7 @@ class QuantizeV2Op : public OpKernel {
     Tensor in_min = ctx->input(1);
     Tensor in_max = ctx->input(2);
     if (!ctx->ok()) return;
-    ITEX_REQUIRES(ctx, src.dtype() == TF_FLOAT, TF_INVALID_ARGUMENT, "QuantizeV2 input must be float");
+    ITEX_REQUIRES(ctx, src.dtype() == src_type_, TF_INVALID_ARGUMENT, "QuantizeV2 input type does not match the kernel");
 
     const int64_t num_slices = (axis_ > -1) ? in_min.NumElements() : 1;
     ITEX_REQUIRES(ctx, in_min.NumElements() >= 1 && in_max.NumElements() >= num_slices, TF_INVALID_ARGUMENT,
@@ -98,14 +100,19 @@ class QuantizeV2Op : public OpKernel {
 
     int st;
     if (num_slices == 1) {
-      st = itexhip_quantize(src.flat<float>(), dst.data(), src.NumElements(), T_, scale[0], addend[0], ctx->stream());
+      st = src_type_ == TF_BFLOAT16
+               ? itexhip_quantize_bf16(src.data(), dst.data(), src.NumElements(), T_, scale[0], addend[0], ctx->stream())
+               : itexhip_quantize(src.flat<float>(), dst.data(), src.NumElements(), T_, scale[0], addend[0], ctx->stream());
     } else {
       std::vector<float> both(scale);
       both.insert(both.end(), addend.begin(), addend.end());
       float* dev = params_.Get(ctx, both.data(), both.size(), TF_FLOAT);
       if (dev == nullptr) return;
-      st = itexhip_quantize_axis(src.flat<float>(), dst.data(), outer, slices, inner, T_, dev, dev + num_slices,
-                                 ctx->stream());
+      st = src_type_ == TF_BFLOAT16
+               ? itexhip_quantize_axis_bf16(src.data(), dst.data(), outer, slices, inner, T_, dev, dev + num_slices,
+                                            ctx->stream())
+               : itexhip_quantize_axis(src.flat<float>(), dst.data(), outer, slices, inner, T_, dev, dev + num_slices,
+                                       ctx->stream());
     }
     ITEX_REQUIRES(ctx, st == ITEXHIP_OK, st == ITEXHIP_INVALID_ARGUMENT ? TF_INVALID_ARGUMENT : TF_ABORTED,
                   std::string("Operation received an exception: ") + itexhip_last_error());
@@ -124,6 +131,7 @@ class QuantizeV2Op : public OpKernel {
 
  private:
   TF_DataType T_;
+  TF_DataType src_type_ = TF_FLOAT;
   Mode mode_ = Mode::SCALED;
   bool classic_ = false;
   bool narrow_range_ = false;
@@ -153,6 +161,15 @@ void AddQuantizeKernels() {
     u8.HostMemory("min_range").HostMemory("max_range").HostMemory("output_min").HostMemory("output_max");
     u8.Register<QuantizeQuint8>();
   }
+  // _ITEXQuantizeV2 from a bfloat16 tensor (:38-51)
+  KernelDefBuilder bs8("_ITEXQuantizeV2", "QuantizeV2Op");
+  bs8.TypeConstraint("T", TF_QINT8).TypeConstraint("dtype", TF_BFLOAT16);
+  bs8.HostMemory("min_range").HostMemory("max_range").HostMemory("output_min").HostMemory("output_max");
+  bs8.Register<QuantizeQint8>();
+  KernelDefBuilder bu8("_ITEXQuantizeV2", "QuantizeV2Op");
+  bu8.TypeConstraint("T", TF_QUINT8).TypeConstraint("dtype", TF_BFLOAT16);
+  bu8.HostMemory("min_range").HostMemory("max_range").HostMemory("output_min").HostMemory("output_max");
+  bu8.Register<QuantizeQuint8>();
 }
 
 }  // namespace itex_amd

@@ -360,3 +360,97 @@ def test_more_than_2_31_elements(hip, dev):
     torch.cuda.synchronize()
     assert torch.equal(x[n - 5000:], q_tail.to(torch.float32) * float(inv))
     assert torch.equal(x[(1 << 31) - 8:(1 << 31) + 8], q[(1 << 31) - 8:(1 << 31) + 8].to(torch.float32) * float(inv))
+
+
+# ------------------------------------------------------------------------------------------------
+# 16-bit floating point ends: QuantizeV2 from bfloat16, Dequantize to bfloat16 / half
+# ------------------------------------------------------------------------------------------------
+def f32_to_bf16_bits(a):
+    """fp32 -> bfloat16 bit patterns, round to nearest even (NaN kept quiet)."""
+    u = np.ascontiguousarray(a, np.float32).view(np.uint32).astype(np.uint64)
+    rounded = ((u + 0x7fff + ((u >> 16) & 1)) >> 16).astype(np.uint16)
+    nan = (u & 0x7fffffff) > 0x7f800000
+    return np.where(nan, ((u >> 16) | 0x40).astype(np.uint16), rounded)
+
+
+def bf16_bits_to_f32(b):
+    return (np.ascontiguousarray(b, np.uint16).astype(np.uint32) << 16).view(np.float32)
+
+
+@pytest.mark.parametrize("T,mode", [(orc.QINT8, orc.SCALED), (orc.QUINT8, orc.MIN_FIRST)])
+@pytest.mark.parametrize("n,offset", [(1 << 16, 0), (4099, 0), (1001, 3), (5, 0)])
+def test_quantize_from_bfloat16(hip, dev, T, mode, n, offset):
+    """A bfloat16 source widens exactly to fp32; from there on it is the fp32 op (oracle on the widened values)."""
+    import torch
+    rng = np.random.default_rng(n + offset)
+    bits = f32_to_bf16_bits(rng.standard_normal(n + offset) * 3)
+    x = bf16_bits_to_f32(bits[offset:])
+    mn, mx = float(x.min()), float(x.max())
+    scale, addend, omn, omx = host_quant_params(T, mode, False, mn, mx)
+    _, q_ref, _, _ = orc.quantize_v2(x, mn, mx, T, mode)
+    x_d = torch.from_numpy(bits.view(np.int16)).to(dev)
+    q_d = torch.zeros(n + 8, dtype=tdtype(T), device=dev)
+    hip.quantize_bf16(x_d.data_ptr() + 2 * offset, q_d, n, T, float(scale[0]), float(addend[0]))
+    torch.cuda.synchronize()
+    got = q_d.cpu().numpy()
+    np.testing.assert_array_equal(got[:n], q_ref)
+    assert (got[n:] == 0).all()
+
+
+def test_quantize_axis_from_bfloat16(hip, dev):
+    import torch
+    rng = np.random.default_rng(8)
+    shape = (3, 5, 17)
+    bits = f32_to_bf16_bits(rng.standard_normal(shape) * np.arange(1, 6).reshape(1, 5, 1))
+    x = bf16_bits_to_f32(bits)
+    mn, mx = x.min((0, 2)), x.max((0, 2))
+    scale, addend, omn, omx = host_quant_params(orc.QINT8, orc.SCALED, False, mn, mx)
+    _, q_ref, _, _ = orc.quantize_v2(x, mn, mx, orc.QINT8, orc.SCALED, axis=1)
+    q_d = torch.zeros(shape, dtype=torch.int8, device=dev)
+    hip.quantize_axis_bf16(torch.from_numpy(bits.view(np.int16)).to(dev), q_d, 3, 5, 17, orc.QINT8,
+                           torch.from_numpy(scale).to(dev), torch.from_numpy(addend).to(dev))
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(q_d.cpu().numpy(), q_ref)
+
+
+@pytest.mark.parametrize("T,mode", [(orc.QINT8, orc.SCALED), (orc.QUINT8, orc.MIN_FIRST)])
+@pytest.mark.parametrize("y_type", ["bf16", "f16"])
+@pytest.mark.parametrize("n,offset", [(1 << 16, 0), (4099, 0), (1001, 1), (7, 0)])
+def test_dequantize_to_16_bit(hip, dev, T, mode, y_type, n, offset):
+    """The fp32 result of Dequantize rounded to nearest even into bfloat16 / half; the range is chosen so that
+    half overflows to infinity for the largest codes."""
+    import torch
+    rng = np.random.default_rng(n)
+    info = np.iinfo(orc.NP_OF[T])
+    q = rng.integers(info.min, info.max + 1, n + offset).astype(orc.NP_OF[T])
+    mn, mx = (-70000.0, 70000.0) if y_type == "f16" and T == orc.QINT8 else (-2.5, 3.25)
+    _, y32 = orc.dequantize(q[offset:], mn, mx, T, mode)
+    _, _, _, sc, zp = orc.scale_zeropoint_align(T, mode, True, np.float32([mn]), np.float32([mx]))
+    y_d = torch.zeros(n + 8, dtype=torch.int16, device=dev)
+    hip.dequantize16(torch.from_numpy(q).to(dev).data_ptr() + offset, y_d, n, T, hip.BFLOAT16 if y_type == "bf16" else hip.HALF,
+                     float(sc[0]), int(zp[0]) if mode == orc.MIN_FIRST else 0)
+    torch.cuda.synchronize()
+    got = y_d.cpu().numpy().view(np.uint16)
+    with np.errstate(over="ignore"):
+        expect = f32_to_bf16_bits(y32) if y_type == "bf16" else y32.astype(np.float16).view(np.uint16)
+    np.testing.assert_array_equal(got[:n], expect)
+    assert (got[n:] == 0).all()
+    if y_type == "f16" and T == orc.QINT8 and n >= 4099:
+        assert np.isinf(expect.view(np.float16)).any()
+
+
+def test_dequantize_axis_to_16_bit(hip, dev):
+    import torch
+    rng = np.random.default_rng(9)
+    shape = (4, 6, 9)
+    q = rng.integers(0, 256, shape).astype(np.uint8)
+    mn = -np.arange(1, 7, dtype=np.float32)
+    mx = np.arange(1, 7, dtype=np.float32) * 1.5
+    _, y32 = orc.dequantize(q, mn, mx, orc.QUINT8, orc.MIN_FIRST, axis=1)
+    _, _, _, sc, zp = orc.scale_zeropoint_align(orc.QUINT8, orc.MIN_FIRST, True, mn.copy(), mx.copy())
+    for y_type, conv in ((hip.BFLOAT16, f32_to_bf16_bits), (hip.HALF, lambda v: v.astype(np.float16).view(np.uint16))):
+        y_d = torch.zeros(shape, dtype=torch.int16, device=dev)
+        hip.dequantize_axis16(torch.from_numpy(q).to(dev), y_d, 4, 6, 9, orc.QUINT8, y_type, torch.from_numpy(sc).to(dev),
+                              torch.from_numpy(zp).to(dev))
+        torch.cuda.synchronize()
+        np.testing.assert_array_equal(y_d.cpu().numpy().view(np.uint16), conv(y32))

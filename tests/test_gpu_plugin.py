@@ -385,3 +385,40 @@ def test_reference_qint32_bias_case_through_plugin(rt, dev, golden):
     _, y_ref = orc.qmatmul(at, xq, wq, b32, xmn, xmx, wmn, wmx, addend=z)
     np.testing.assert_array_equal(fetch(torch, outs[0], np.float32), y_ref)
     node.close()
+
+
+def test_bfloat16_quantize_and_16_bit_dequantize_through_plugin(rt, dev):
+    """_ITEXQuantizeV2 with dtype = bfloat16 and Dequantize with dtype = bfloat16 / half
+    (itex/core/kernels/gpu/quantize_op.cc:38-51, dequantize_op.cc:24-48)."""
+    torch = rt
+    BF16, HALF = 14, 19
+    rng = np.random.default_rng(12)
+    x32 = (rng.standard_normal(3001) * 2).astype(np.float32)
+    xb = torch.from_numpy(x32).to(dev).to(torch.bfloat16)
+    xw = xb.to(torch.float32).cpu().numpy()          # the exactly widened values
+    node = tf.Node("_ITEXQuantizeV2", dict(T=DT(tf.QINT8), dtype=DT(BF16), mode="SCALED", round_mode="HALF_TO_EVEN",
+                                            narrow_range=False, axis=-1, ensure_minimum_range=0.01))
+    assert node.code == tf.OK, node.message
+    mn, mx = np.array(xw.min(), np.float32), np.array(xw.max(), np.float32)
+    code, msg, outs = node.run([(BF16, xw.shape, xb.data_ptr(), False), (tf.FLOAT, (), tf.host_array(mn), True),
+                                (tf.FLOAT, (), tf.host_array(mx), True)],
+                               [(tf.QINT8, False), (tf.FLOAT, True), (tf.FLOAT, True)], stream=torch.cuda.current_stream().cuda_stream)
+    assert code == tf.OK, msg
+    q = fetch(torch, outs[0], np.int8)
+    _, q_ref, omn, omx = orc.quantize_v2(xw, mn, mx, orc.QINT8, orc.SCALED)
+    np.testing.assert_array_equal(q, q_ref)
+    node.close()
+    q_d = dev_in(torch, dev, q_ref)
+    _, y32 = orc.dequantize(q_ref, omn[0], omx[0], orc.QINT8, orc.SCALED)
+    for dtype, tdt_ in ((BF16, torch.bfloat16), (HALF, torch.float16)):
+        dn = tf.Node("Dequantize", dict(T=DT(tf.QINT8), mode="SCALED", narrow_range=False, axis=-1, dtype=DT(dtype)))
+        assert dn.code == tf.OK, dn.message
+        dmn, dmx = np.array(omn[0], np.float32), np.array(omx[0], np.float32)
+        code, msg, outs = dn.run([(tf.QINT8, q_ref.shape, q_d.data_ptr(), False), (tf.FLOAT, (), tf.host_array(dmn), True),
+                                  (tf.FLOAT, (), tf.host_array(dmx), True)], [(dtype, False)],
+                                 stream=torch.cuda.current_stream().cuda_stream)
+        assert code == tf.OK, msg
+        bits = fetch(torch, outs[0], np.int16)
+        expect = torch.from_numpy(y32).to(tdt_).view(torch.int16).numpy()   # torch rounds to nearest even as well
+        np.testing.assert_array_equal(bits, expect)
+        dn.close()
