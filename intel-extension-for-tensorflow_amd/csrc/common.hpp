@@ -57,6 +57,24 @@ __device__ __forceinline__ int sat_rne(float y) {
   return static_cast<int>(__builtin_rintf(y));
 }
 
+// fp32 <-> bfloat16 bit patterns (round to nearest even, NaN kept quiet)
+__device__ __forceinline__ float bf16_bits_to_f32(uint32_t h) { return __uint_as_float(h << 16); }
+__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x40u;
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return u >> 16;
+}
+
+// one output element of a quantized MatMul: fp32 kept, bfloat16 rounded, integers saturated + rounded
+template <int OUT_T>
+__device__ __forceinline__ void store_output(void* __restrict__ out, int64_t idx, float v) {
+  if constexpr (OUT_T == ITEXHIP_FLOAT) static_cast<float*>(out)[idx] = v;
+  else if constexpr (OUT_T == ITEXHIP_BFLOAT16) static_cast<uint16_t*>(out)[idx] = static_cast<uint16_t>(f32_to_bf16_bits(v));
+  else if constexpr (OUT_T == ITEXHIP_QINT32) static_cast<int32_t*>(out)[idx] = sat_rne<ITEXHIP_QINT32>(v);
+  else static_cast<uint8_t*>(out)[idx] = static_cast<uint8_t>(sat_rne<OUT_T>(v));
+}
+
 __device__ __forceinline__ uint32_t pack4(int a, int b, int c, int d) {
   return (static_cast<uint32_t>(a) & 0xffu) | ((static_cast<uint32_t>(b) & 0xffu) << 8) |
          ((static_cast<uint32_t>(c) & 0xffu) << 16) | ((static_cast<uint32_t>(d) & 0xffu) << 24);

@@ -14,13 +14,8 @@ constexpr int kUnroll = 4;
 typedef unsigned int u2 __attribute__((ext_vector_type(2)));
 typedef unsigned int u4 __attribute__((ext_vector_type(4)));
 
-__device__ __forceinline__ float bf16_to_f32(uint32_t h) { return __uint_as_float(h << 16); }
-__device__ __forceinline__ uint32_t f32_to_bf16(float f) {
-  uint32_t u = __float_as_uint(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x40u;  // NaN stays NaN (quiet)
-  u += 0x7fffu + ((u >> 16) & 1u);                                 // round to nearest even
-  return u >> 16;
-}
+__device__ __forceinline__ float bf16_to_f32(uint32_t h) { return bf16_bits_to_f32(h); }
+__device__ __forceinline__ uint32_t f32_to_bf16(float f) { return f32_to_bf16_bits(f); }
 __device__ __forceinline__ uint32_t f32_to_f16(float f) {
   const _Float16 h = static_cast<_Float16>(f);  // v_cvt_f16_f32, round to nearest even
   unsigned short bits;

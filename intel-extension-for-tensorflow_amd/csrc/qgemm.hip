@@ -268,9 +268,7 @@ __global__ __launch_bounds__(256) void qgemm_naive_kernel(const uint8_t* __restr
   else if (e.n_scales > 1) v = v * e.scales[n];
   if (e.bias) v = v + static_cast<const float*>(e.bias)[n];
   for (int k = 0; k < e.n_eltwise; ++k) v = apply_eltwise(e.elt[k], v);  // no sum post-op on this path
-  if constexpr (OUT_T == ITEXHIP_FLOAT) reinterpret_cast<float*>(out)[idx] = v;
-  else if constexpr (OUT_T == ITEXHIP_QINT32) reinterpret_cast<int32_t*>(out)[idx] = sat_rne<ITEXHIP_QINT32>(v);
-  else reinterpret_cast<uint8_t*>(out)[idx] = static_cast<uint8_t>(sat_rne<OUT_T>(v));
+  store_output<OUT_T>(out, idx, v);
 }
 
 // The whole op on the unpacked weight, any K: the thread also sums its weight column (the zero-point
@@ -301,9 +299,7 @@ __global__ __launch_bounds__(256) void qmatmul_unpacked_kernel(const uint8_t* __
     if (e.elt[k].alg == ITEXHIP_ELT_SUM) v = v + e.elt[k].alpha * e.addend[idx];
     else v = apply_eltwise(e.elt[k], v);
   }
-  if constexpr (OUT_T == ITEXHIP_FLOAT) reinterpret_cast<float*>(out)[idx] = v;
-  else if constexpr (OUT_T == ITEXHIP_QINT32) reinterpret_cast<int32_t*>(out)[idx] = sat_rne<ITEXHIP_QINT32>(v);
-  else reinterpret_cast<uint8_t*>(out)[idx] = static_cast<uint8_t>(sat_rne<OUT_T>(v));
+  store_output<OUT_T>(out, idx, v);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -314,7 +310,7 @@ int check_common(const void* a, int a_type, const void* b, int64_t M, int64_t K,
                  const char* who) {
   ITEXHIP_REQUIRE(a_type == ITEXHIP_QUINT8 || a_type == ITEXHIP_QINT8, "%s: activation type must be quint8 or qint8", who);
   ITEXHIP_REQUIRE(out_type == ITEXHIP_QINT32 || out_type == ITEXHIP_QINT8 || out_type == ITEXHIP_QUINT8 ||
-                      out_type == ITEXHIP_FLOAT, "%s: unsupported output type %d", who, out_type);
+                      out_type == ITEXHIP_FLOAT || out_type == ITEXHIP_BFLOAT16, "%s: unsupported output type %d", who, out_type);
   ITEXHIP_REQUIRE(M >= 0 && K >= 0 && N >= 0, "%s: negative dimension", who);
   ITEXHIP_REQUIRE(M < (1LL << 31) && N < (1LL << 31) && K <= kMaxK, "%s: dimension too large (K <= %lld)", who,
                   static_cast<long long>(kMaxK));
@@ -370,6 +366,7 @@ int dispatch_gemv(const uint8_t* a, uint32_t a_xor, const uint8_t* bp, int M, in
 #define ITEXHIP_DISPATCH_OUT(out_type, CALL)                                  \
   switch (out_type) {                                                         \
     case ITEXHIP_FLOAT: st__ = CALL(ITEXHIP_FLOAT); break;                    \
+    case ITEXHIP_BFLOAT16: st__ = CALL(ITEXHIP_BFLOAT16); break;              \
     case ITEXHIP_QINT32: st__ = CALL(ITEXHIP_QINT32); break;                  \
     case ITEXHIP_QINT8: st__ = CALL(ITEXHIP_QINT8); break;                    \
     default: st__ = CALL(ITEXHIP_QUINT8); break;                              \
@@ -475,6 +472,9 @@ extern "C" int itexhip_qgemm_naive(const void* a, int a_type, const int8_t* w, i
   hipStream_t hs = as_stream(stream);
   const int Mi = static_cast<int>(M), Ki = static_cast<int>(K), Ni = static_cast<int>(N);
   switch (out_type) {
+    case ITEXHIP_BFLOAT16:
+      qgemm_naive_kernel<ITEXHIP_BFLOAT16><<<grid, 256, 0, hs>>>(ap, a_is_u8, w, transpose_b, Mi, Ki, Ni, e, out);
+      break;
     case ITEXHIP_FLOAT:
       qgemm_naive_kernel<ITEXHIP_FLOAT><<<grid, 256, 0, hs>>>(ap, a_is_u8, w, transpose_b, Mi, Ki, Ni, e, out);
       break;
@@ -580,6 +580,7 @@ extern "C" int itexhip_qmatmul_unpacked(const itexhip_matmul_params* p, const vo
   const int Mi = static_cast<int>(M), Ki = static_cast<int>(K), Ni = static_cast<int>(N);
   switch (p->t_out) {
     case ITEXHIP_FLOAT: qmatmul_unpacked_kernel<ITEXHIP_FLOAT><<<grid, 256, 0, hs>>>(ap, a_is_u8, w, transpose_b, Mi, Ki, Ni, e, out); break;
+    case ITEXHIP_BFLOAT16: qmatmul_unpacked_kernel<ITEXHIP_BFLOAT16><<<grid, 256, 0, hs>>>(ap, a_is_u8, w, transpose_b, Mi, Ki, Ni, e, out); break;
     case ITEXHIP_QINT32: qmatmul_unpacked_kernel<ITEXHIP_QINT32><<<grid, 256, 0, hs>>>(ap, a_is_u8, w, transpose_b, Mi, Ki, Ni, e, out); break;
     case ITEXHIP_QINT8: qmatmul_unpacked_kernel<ITEXHIP_QINT8><<<grid, 256, 0, hs>>>(ap, a_is_u8, w, transpose_b, Mi, Ki, Ni, e, out); break;
     default: qmatmul_unpacked_kernel<ITEXHIP_QUINT8><<<grid, 256, 0, hs>>>(ap, a_is_u8, w, transpose_b, Mi, Ki, Ni, e, out); break;

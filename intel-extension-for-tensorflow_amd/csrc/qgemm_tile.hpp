@@ -267,8 +267,8 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void qgemm_tile_kernel(
   // the MFMA layout owns one row and scattered 4-channel groups, which would make every store a
   // 64-address scatter.  The buffer holds [WM rows][ROWB bytes] with a 16-byte pad per row: for 8-bit
   // outputs all TN channel tiles at once, for 32-bit outputs one channel tile per pass.
-  constexpr int ESZ = (OUT_T == ITEXHIP_QINT8 || OUT_T == ITEXHIP_QUINT8) ? 1 : 4;
-  constexpr int JB = (ESZ == 1) ? TN : 1;    // channel tiles per pass
+  constexpr int ESZ = (OUT_T == ITEXHIP_QINT8 || OUT_T == ITEXHIP_QUINT8) ? 1 : (OUT_T == ITEXHIP_BFLOAT16) ? 2 : 4;
+  constexpr int JB = (ESZ == 1) ? TN : (ESZ == 2) ? ((TN % 2 == 0) ? 2 : TN) : 1;  // channel tiles per pass
   constexpr int ROWB = JB * 32 * ESZ;        // row bytes in the buffer
   constexpr int PITCH = ROWB + 16;
   constexpr int LPR = ROWB / 16;             // lanes per row when flushing
@@ -294,6 +294,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void qgemm_tile_kernel(
             uint8_t* dst = ebuf + (decltype(i)::value * 32 + lrow) * PITCH +
                            (decltype(jj)::value * 32 + decltype(g)::value * 8 + lgrp * 4) * ESZ;
             if constexpr (ESZ == 1) *reinterpret_cast<int*>(dst) = o.x;
+            else if constexpr (ESZ == 2) *reinterpret_cast<int2*>(dst) = make_int2(o.x, o.y);
             else *reinterpret_cast<v4i*>(dst) = o;
           });
         });
@@ -334,9 +335,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void qgemm_tile_kernel(
                     if (e.elt[k].alg == ITEXHIP_ELT_SUM) v = v + e.elt[k].alpha * e.addend[o];
                     else v = apply_eltwise(e.elt[k], v);
                   }
-                  if constexpr (OUT_T == ITEXHIP_FLOAT) reinterpret_cast<float*>(out)[o] = v;
-                  else if constexpr (OUT_T == ITEXHIP_QINT32) reinterpret_cast<int32_t*>(out)[o] = sat_rne<ITEXHIP_QINT32>(v);
-                  else reinterpret_cast<uint8_t*>(out)[o] = static_cast<uint8_t>(sat_rne<OUT_T>(v));
+                  store_output<OUT_T>(out, o, v);
                 }
               }
             }
@@ -405,7 +404,7 @@ int dispatch_tile_shape(const uint8_t* a, uint32_t amask, const uint8_t* bp, int
 template <int OUT_T>
 int dispatch_tile(const uint8_t* a, uint32_t a_xor, const uint8_t* bp, int M, int K, int N,
                   const EpilogueArgs& e, void* out, hipStream_t st) {
-  constexpr int esz = (OUT_T == ITEXHIP_QINT8 || OUT_T == ITEXHIP_QUINT8) ? 1 : 4;
+  constexpr int esz = (OUT_T == ITEXHIP_QINT8 || OUT_T == ITEXHIP_QUINT8) ? 1 : (OUT_T == ITEXHIP_BFLOAT16) ? 2 : 4;
   // the specialised kernels only carry the vectorised epilogue: bias present, output rows 16-byte aligned
   const bool plain = e.addend == nullptr && (e.bias != nullptr || e.fused) && (reinterpret_cast<uintptr_t>(out) & 15) == 0 &&
                      ((static_cast<int64_t>(N) * esz) & 15) == 0 && (K & 63) == 0;

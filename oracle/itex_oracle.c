@@ -294,6 +294,23 @@ static int eltwise_from_activation(int act, orc_eltwise* e) {
   }
 }
 
+/* fp32 -> bfloat16, round to nearest even (the destination conversion of a bf16 memory descriptor and
+ * the float -> Eigen::bfloat16 cast) */
+static inline uint16_t f32_to_bf16_bits(float f) {
+  uint32_t u;
+  memcpy(&u, &f, 4);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40u);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (uint16_t)(u >> 16);
+}
+
+static inline float bf16_bits_to_f32(uint16_t h) {
+  const uint32_t u = (uint32_t)h << 16;
+  float f;
+  memcpy(&f, &u, 4);
+  return f;
+}
+
 /*
  * Host-side parameter preparation of the quantized MatMul kernels:
  *   output scales  - ExtendInt8PostOps: V2 quantized_matmul_common.h:1809-1908,
@@ -308,10 +325,14 @@ int orc_qmatmul_prepare(const orc_matmul_attrs* at, int64_t N, const int32_t* co
                         float min_out, float max_out, const void* bias_v, float* scales,
                         float* bias_out, orc_epilogue_desc* ep) {
   const int bias_s32 = (at->t_bias == ORC_QINT32);
-  const float* bias = (const float*)bias_v;
+  /* Tbias = bfloat16: GetScaledBias is generic in Tbias; every entry is widened with
+   * static_cast<float>, the arithmetic is fp32, and the result is stored as Tbias again (:578-599 cast,
+   * :609-617 the reorder's bf16 destination), i.e. rounded to bfloat16 before the primitive reads it */
+  const int bias_bf16 = (at->t_bias == ORC_BFLOAT16);
   const int32_t* bias_i32 = (const int32_t*)bias_v;
   const int out_q8 = (at->t_out == ORC_QINT8 || at->t_out == ORC_QUINT8);
-  const int out_f32 = (at->t_out == ORC_FLOAT);
+  /* the float-output branches upstream test Toutput against float, bfloat16 and half alike (:577, 1255-1257) */
+  const int out_f32 = (at->t_out == ORC_FLOAT || at->t_out == ORC_BFLOAT16);
   const int out_s32 = (at->t_out == ORC_QINT32);
   if (!out_q8 && !out_f32 && !out_s32) return ORC_INVALID_ARGUMENT;
   if (at->input_mode != ORC_MIN_FIRST && at->input_mode != ORC_SCALED) return ORC_INVALID_ARGUMENT;
@@ -342,7 +363,7 @@ int orc_qmatmul_prepare(const orc_matmul_attrs* at, int64_t N, const int32_t* co
     ep->n_eltwise++;
   }
   /* a quantized addend is not implemented upstream either (:1768-1773) */
-  if (at->add_position != 0 && !out_f32) return ORC_UNIMPLEMENTED;
+  if (at->add_position != 0 && at->t_out != ORC_FLOAT) return ORC_UNIMPLEMENTED;
   if (at->activation == ORC_ACT_LEAKYRELU) has_leaky = 1;
   if (at->api == ORC_API_V2 && at->has_requantize && at->out_min_first) {
     /* :1753-1757: "Linear" is appended to fused_ops */
@@ -407,7 +428,7 @@ int orc_qmatmul_prepare(const orc_matmul_attrs* at, int64_t N, const int32_t* co
       float scale;
       if (at->t_out == ORC_QUINT8) scale = scale_int32 / scale_eightbit / 8388608.0f;
       else if (at->t_out == ORC_QINT8) scale = scale_int32 / scale_eightbit / 16777216.0f;
-      else scale = scale_int32 / 2147483648.0f;
+      else scale = scale_int32 / 2147483648.0f; /* float / bfloat16 output */
       scales[0] = scale;
       ep->n_scales = 1;
     }
@@ -430,6 +451,12 @@ int orc_qmatmul_prepare(const orc_matmul_attrs* at, int64_t N, const int32_t* co
     bias_scales[i] = (max_int8_input * max_int8_weight) / (range_input * range_weight);
   }
   int st = ORC_OK;
+  float* bias_wide = NULL;
+  if (bias_bf16) {
+    bias_wide = (float*)malloc(sizeof(float) * (size_t)(N > 0 ? N : 1));
+    for (int64_t j = 0; j < N; ++j) bias_wide[j] = bf16_bits_to_f32(((const uint16_t*)bias_v)[j]);
+  }
+  const float* bias = bias_bf16 ? bias_wide : (const float*)bias_v;
   if (bias_s32) {
     /* Tbias = qint32, :1153-1334: the bias is cast to float (:1165-1167) and scaled by
      * (range_input * range_weight) / (A * 127) (:1204-1211), the inverse of the fp32 path's factor;
@@ -472,6 +499,10 @@ int orc_qmatmul_prepare(const orc_matmul_attrs* at, int64_t N, const int32_t* co
      * single scale (the first) applies to all N entries.  Parity unpinned for nb > 1. */
     for (int64_t j = 0; j < N; ++j) bias_out[j] = bias[j] * bias_scales[0];
   }
+  if (bias_bf16) {
+    for (int64_t j = 0; j < N; ++j) bias_out[j] = bf16_bits_to_f32(f32_to_bf16_bits(bias_out[j]));
+    free(bias_wide);
+  }
   free(bias_scales);
   return st;
 }
@@ -501,7 +532,7 @@ void orc_qmatmul_epilogue(const int32_t* acc, int64_t M, int64_t N, const orc_ep
                           const float* scales, const float* bias, const float* addend, int t_out,
                           void* out) {
   float lo = 0, hi = 0;
-  if (t_out != ORC_FLOAT) sat_bounds(t_out, &lo, &hi);
+  if (t_out != ORC_FLOAT && t_out != ORC_BFLOAT16) sat_bounds(t_out, &lo, &hi);
 #pragma omp parallel for schedule(static)
   for (int64_t m = 0; m < M; ++m) {
     for (int64_t n = 0; n < N; ++n) {
@@ -514,6 +545,7 @@ void orc_qmatmul_epilogue(const int32_t* acc, int64_t M, int64_t N, const orc_ep
         else y = apply_eltwise(&ep->elt[e], y);
       }
       if (t_out == ORC_FLOAT) ((float*)out)[m * N + n] = y;
+      else if (t_out == ORC_BFLOAT16) ((uint16_t*)out)[m * N + n] = f32_to_bf16_bits(y);
       else store_q(out, m * N + n, t_out, sat_rne(y, lo, hi));
     }
   }
@@ -546,7 +578,7 @@ int orc_qmatmul_output_minmax(const orc_matmul_attrs* at, float min_a, float max
       out_max[n] = c_level * (float)q_highest(ORC_QINT32);
     }
     *n_out = cnt;
-  } else if (at->t_out == ORC_FLOAT) {
+  } else if (at->t_out == ORC_FLOAT || at->t_out == ORC_BFLOAT16) {
     *n_out = 0;
   } else {
     return ORC_INVALID_ARGUMENT;

@@ -11,7 +11,7 @@ ROOT = os.path.dirname(os.path.dirname(HERE))
 MOCK_LIB = os.path.join(HERE, "libmock_tf.so")
 PLUGIN_LIB = os.path.join(ROOT, "intel-extension-for-tensorflow_amd", "lib", "libitex_amd.so")
 
-FLOAT, INT32, QINT8, QUINT8, QINT32 = 1, 3, 11, 12, 13
+FLOAT, INT32, QINT8, QUINT8, QINT32, BFLOAT16, HALF = 1, 3, 11, 12, 13, 14, 19
 NP_OF = {FLOAT: np.float32, INT32: np.int32, QINT8: np.int8, QUINT8: np.uint8, QINT32: np.int32}
 OK, INVALID_ARGUMENT, NOT_FOUND, ABORTED, UNIMPLEMENTED = 0, 3, 5, 10, 12
 

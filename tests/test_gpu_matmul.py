@@ -12,7 +12,12 @@ pytestmark = pytest.mark.gpu
 
 def tdt(T):
     import torch
-    return {orc.QINT8: torch.int8, orc.QUINT8: torch.uint8, orc.QINT32: torch.int32, orc.FLOAT: torch.float32}[T]
+    return {orc.QINT8: torch.int8, orc.QUINT8: torch.uint8, orc.QINT32: torch.int32, orc.FLOAT: torch.float32,
+            orc.BFLOAT16: torch.int16}[T]   # bfloat16 travels as bit patterns
+
+
+def bits16(a):
+    return a.view(np.uint16) if a.dtype == np.int16 else a
 
 
 class Linear:
@@ -495,3 +500,81 @@ def test_qint32_bias_vs_oracle(hip, dev, M, t_out, mode):
               t_out, out)
     torch.cuda.synchronize()
     np.testing.assert_array_equal(out.cpu().numpy(), ref)
+
+
+V2_DEQ_BF16 = dict(V2_DEQ, t_out=orc.BFLOAT16)
+
+
+@pytest.mark.parametrize("path", ["gemv", "tile", "auto", "fused", "naive"])
+@pytest.mark.parametrize("M,K,N", [(3, 512, 272), (150, 256, 203), (16, 64, 8), (300, 448, 528)])
+def test_bfloat16_output_vs_oracle(hip, dev, path, M, K, N):
+    """Tout = bfloat16 (_QuantizedMatMul, ...AndDequantize): bit patterns equal the oracle's on every kernel, with
+    N odd / not a multiple of the 8-element vector store."""
+    if path == "gemv" and M > 16:
+        pytest.skip("the small-M kernel takes M <= 16")
+    layer, w, bias = make_layer(hip, dev, K, N, seed=K + N)
+    x, xq, mn, mx = make_acts(M, K, seed=M + 1)
+    for kw in (V2_DEQ_BF16, dict(V2_DEQ_BF16, activation=orc.ACT_RELU)):
+        ref = layer.oracle(xq, kw, mn, mx)
+        assert ref.dtype == np.uint16
+        np.testing.assert_array_equal(bits16(layer.run(xq, kw, mn, mx, path=path)), ref)
+
+
+@pytest.mark.parametrize("shape", [0, 1, 2, 3, 4])
+def test_bfloat16_output_every_tile_shape(hip, dev, monkeypatch, shape):
+    monkeypatch.setenv("ITEXHIP_TILE_SHAPE", str(shape))
+    for M, K, N in [(513, 192, 400), (260, 320, 203)]:
+        layer, w, bias = make_layer(hip, dev, K, N, seed=N + shape)
+        x, xq, mn, mx = make_acts(M, K, seed=M)
+        ref = layer.oracle(xq, V2_DEQ_BF16, mn, mx)
+        np.testing.assert_array_equal(bits16(layer.run(xq, V2_DEQ_BF16, mn, mx, path="tile")), ref)
+        np.testing.assert_array_equal(bits16(layer.run(xq, V2_DEQ_BF16, mn, mx, path="fused")), ref)
+
+
+def test_bfloat16_output_unpacked_weight_odd_k(hip, dev):
+    import torch
+    M, K, N = 37, 75, 61
+    layer, w, bias = make_layer(hip, dev, K, N, seed=5)
+    x, xq, mn, mx = make_acts(M, K, seed=2)
+    ref = layer.oracle(xq, V2_DEQ_BF16, mn, mx)
+    p = hip.matmul_params(t_in=orc.QUINT8, min_a=mn, max_a=mx, **V2_DEQ_BF16)
+    out = torch.empty((M, N), dtype=torch.int16, device=dev)
+    hip.qmatmul_unpacked(p, torch.from_numpy(xq).to(dev), layer.w_d, False, M, K, N, layer.min_b_d, layer.max_b_d,
+                         layer.min_b.size, layer.bias_d, out)
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(bits16(out.cpu().numpy()), ref)
+
+
+@pytest.mark.parametrize("M", [2, 140])
+@pytest.mark.parametrize("t_out,mode", [(orc.FLOAT, orc.MIN_FIRST), (orc.BFLOAT16, orc.MIN_FIRST), (orc.QINT8, orc.MIN_FIRST),
+                                        (orc.QINT32, orc.MIN_FIRST), (orc.FLOAT, orc.SCALED)])
+def test_bfloat16_bias_vs_oracle(hip, dev, M, t_out, mode):
+    """Tbias = bfloat16: the adjusted bias is rounded to bfloat16 before the epilogue adds it."""
+    import torch
+    K, N = 320, 144
+    layer, w, _ = make_layer(hip, dev, K, N, seed=34)
+    x, xq, mn, mx = make_acts(M, K, seed=M + 5, mode=mode)
+    b16 = torch.from_numpy((np.random.default_rng(7).standard_normal(N) * 0.3).astype(np.float32)).to(torch.bfloat16) \
+        .view(torch.int16).numpy().view(np.uint16)
+    isf = t_out in (orc.FLOAT, orc.BFLOAT16)
+    kw = dict(api=orc.API_V2 if t_out != orc.QINT32 else orc.API_V1, t_out=t_out, input_mode=mode,
+              has_dequantize=isf, has_requantize=t_out == orc.QINT8, t_bias=orc.BFLOAT16)
+    t_in = orc.QUINT8 if mode == orc.MIN_FIRST else orc.QINT8
+    st, ref = orc.qmatmul(orc.matmul_attrs(t_in=t_in, **kw), xq, layer.wq, b16, mn, mx, layer.min_b, layer.max_b, -40.0, 40.0)
+    assert st == orc.OK
+    got = _run_single_launch(hip, dev, layer, kw, xq, mn, mx, b16.view(np.int16), lo=-40.0, hi=40.0)
+    np.testing.assert_array_equal(bits16(got), ref)
+    # the widened bias through the fp32 path differs (no rounding of the adjusted bias)
+    st, ref32 = orc.qmatmul(orc.matmul_attrs(t_in=t_in, **dict(kw, t_bias=orc.FLOAT)), xq, layer.wq,
+                            (b16.astype(np.uint32) << 16).view(np.float32), mn, mx, layer.min_b, layer.max_b, -40.0, 40.0)
+    assert st == orc.OK and (t_out != orc.FLOAT or not np.array_equal(ref, ref32))
+    # the two-launch form prepares the same vectors
+    p = hip.matmul_params(t_in=t_in, min_a=float(mn), max_a=float(mx), min_out=-40.0, max_out=40.0, **kw)
+    ep = hip.qmatmul_epilogue_desc(p, layer.min_b.size)
+    hip.qmatmul_prepare(p, layer.min_b_d, layer.max_b_d, layer.min_b.size, torch.from_numpy(b16.view(np.int16)).to(dev),
+                        layer.colsum, N, layer.scales_d, layer.sbias_d)
+    out = torch.empty((M, N), dtype=tdt(t_out), device=dev)
+    hip.qgemm(torch.from_numpy(xq).to(dev), p.t_in, layer.packed, layer.colsum, M, K, N, layer.scales_d, layer.sbias_d, ep,
+              t_out, out)
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(bits16(out.cpu().numpy()), ref)

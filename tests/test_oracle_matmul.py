@@ -358,3 +358,62 @@ def test_qint32_bias_closed_forms(mode, t_out, per_channel):
     else:
         expect = bf
     np.testing.assert_array_equal(sb, expect.astype(np.float32))
+
+
+def _bf16_rne(x):
+    """fp32 -> bfloat16 bit patterns by PyTorch's conversion (round to nearest even), independent of the oracle's."""
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(x, np.float32)).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+
+
+@pytest.mark.parametrize("api,kw", [(orc.API_V2, dict(has_dequantize=True)), (orc.API_V2, dict(has_dequantize=True, activation=orc.ACT_RELU)),
+                                    (orc.API_V1, dict(n_fused_ops=1)), (orc.API_LEGACY, {})])
+def test_bfloat16_output_is_the_rounded_float_output(api, kw):
+    """Tout = bfloat16 follows the float branches of the parameter preparation (:577, 1478-1479) and differs from
+    Tout = float only in the destination conversion: nearest-even bfloat16 of the same fp32 value."""
+    rng = np.random.default_rng(12)
+    M, K, N = 33, 96, 50
+    a = rng.integers(0, 256, (M, K)).astype(np.uint8)
+    w = rng.integers(-127, 128, (K, N)).astype(np.int8)
+    bias = rng.standard_normal(N).astype(np.float32)
+    args = (a, w, bias, -1.5, 2.5, np.float32([-0.7]), np.float32([0.7]), -30.0, 30.0)
+    st, y32 = orc.qmatmul(orc.matmul_attrs(api=api, t_in=orc.QUINT8, t_out=orc.FLOAT, input_mode=orc.MIN_FIRST, **kw), *args)
+    assert st == orc.OK
+    st, y16 = orc.qmatmul(orc.matmul_attrs(api=api, t_in=orc.QUINT8, t_out=orc.BFLOAT16, input_mode=orc.MIN_FIRST, **kw), *args)
+    assert st == orc.OK and y16.dtype == np.uint16
+    np.testing.assert_array_equal(y16, _bf16_rne(y32))
+    assert (y16.astype(np.uint32) << 16).view(np.float32).tolist() != y32.tolist()  # the rounding is not a no-op here
+
+
+def test_bfloat16_output_ties_round_to_even():
+    """Epilogue alone on accumulators whose fp32 results sit exactly between two bfloat16 values."""
+    acc = np.int32([[257, 259, 65536 + 128, 65536 + 384, -257, -259]])   # 1 + 2^-8 -> tie, 1 + 3*2^-8 -> tie, ...
+    ep = orc.EpilogueDesc(1, 0)
+    out = orc.qmatmul_epilogue(acc, ep, np.float32([1.0 / 256]), np.zeros(6, np.float32), orc.BFLOAT16)
+    np.testing.assert_array_equal(out, _bf16_rne(acc.astype(np.float32) / 256))
+    f = (out.astype(np.uint32) << 16).view(np.float32)[0]
+    assert f[0] == 1.0 and f[1] == 1.015625 and f[4] == -1.0 and f[5] == -1.015625
+
+
+@pytest.mark.parametrize("mode", [orc.MIN_FIRST, orc.SCALED])
+@pytest.mark.parametrize("t_out", [orc.FLOAT, orc.QINT8, orc.QINT32])
+def test_bfloat16_bias_is_adjusted_in_fp32_and_stored_as_bfloat16(mode, t_out):
+    """Tbias = bfloat16: GetScaledBias widens each entry, computes as for fp32 and stores the adjusted bias in
+    Tbias again (quantized_matmul_common.h:578-599, 609-617) - so it equals the nearest-even bfloat16 of what the
+    fp32 path gives for the widened bias."""
+    N = 40
+    rng = np.random.default_rng(8)
+    b16 = _bf16_rne(rng.standard_normal(N).astype(np.float32))
+    b32 = (b16.astype(np.uint32) << 16).view(np.float32)
+    wmn = -(rng.random(N).astype(np.float32) + 0.5)
+    wmx = -wmn
+    colsum = rng.integers(-999, 999, N).astype(np.int32)
+    kw = dict(t_in=orc.QUINT8 if mode == orc.MIN_FIRST else orc.QINT8, t_out=t_out, input_mode=mode,
+              api=orc.API_V2 if t_out != orc.QINT32 else orc.API_V1, n_fused_ops=1,
+              has_dequantize=t_out == orc.FLOAT, has_requantize=t_out == orc.QINT8)
+    st, _, sb32, _ = orc.qmatmul_prepare(orc.matmul_attrs(**kw), N, colsum, -1.25, 2.5, wmn, wmx, -3.0, 3.0, b32)
+    assert st == orc.OK
+    st, _, sb16, _ = orc.qmatmul_prepare(orc.matmul_attrs(t_bias=orc.BFLOAT16, **kw), N, colsum, -1.25, 2.5, wmn, wmx, -3.0, 3.0, b16)
+    assert st == orc.OK
+    np.testing.assert_array_equal(sb16, (_bf16_rne(sb32).astype(np.uint32) << 16).view(np.float32))
+    assert not np.array_equal(sb16, sb32)
