@@ -195,7 +195,7 @@ typedef struct {
 typedef struct {
   int api;             /* ITEXHIP_API_* */
   int t_in;            /* T1: QUINT8 | QINT8 */
-  int t_out;           /* QINT32 | QINT8 | QUINT8 | FLOAT | BFLOAT16 (the fp32 result rounded to nearest even) */
+  int t_out;           /* QINT32 | QINT8 | QUINT8 | FLOAT | BFLOAT16 | HALF (the fp32 result rounded to nearest even) */
   int input_mode;      /* input_quant_mode: MIN_FIRST | SCALED */
   int out_min_first;   /* V2: output_quant_mode == "MIN_FIRST" */
   int activation;      /* ITEXHIP_ACT_* */
@@ -207,8 +207,8 @@ typedef struct {
   float min_out, max_out;  /* min/max_freezed_output (requantize) */
   int add_position;        /* "Add" in fused_ops: 0 absent, 1 before the activation, 2 after it (fp32 output only) */
   int t_bias;              /* Tbias: 0 or ITEXHIP_FLOAT = fp32, ITEXHIP_QINT32 = qint32 (:1153-1334),
-                            * ITEXHIP_BFLOAT16 = bfloat16 bit patterns; the adjusted bias is rounded to bfloat16
-                            * again, as GetScaledBias stores it in Tbias (:578-599, 609-617) */
+                            * ITEXHIP_BFLOAT16 / ITEXHIP_HALF = 16-bit patterns; the adjusted bias is rounded to
+                            * that type again, as GetScaledBias stores it in Tbias (:578-599, 609-617) */
 } itexhip_matmul_params;
 
 /* Host-only: the epilogue descriptor (scale count, eltwise chain with the reference's alpha/beta
@@ -219,7 +219,7 @@ int itexhip_qmatmul_epilogue_desc(const itexhip_matmul_params* p, int64_t nb, it
 
 /* Device: per-channel output scales and the scaled / zero-point-compensated bias
  * (ExtendInt8PostOps as above; GetScaledBias, quantized_matmul_common.h:466-660), computed by one
- * small kernel from device copies of min_b / max_b (nb floats each), the bias (N floats; N int32 when p->t_bias is QINT32, N uint16 when BFLOAT16) and
+ * small kernel from device copies of min_b / max_b (nb floats each), the bias (N floats; N int32 when p->t_bias is QINT32, N uint16 when BFLOAT16 / HALF) and
  * the weight column sums (N int32, from itexhip_qgemm_prepack_b).  Writes `scales_out`
  * (max(ep.n_scales,1) floats) and `bias_out` (N floats).  No host synchronisation. */
 int itexhip_qmatmul_prepare(const itexhip_matmul_params* p, const float* min_b, const float* max_b,
@@ -237,7 +237,7 @@ int itexhip_qgemm_prepack_b(const int8_t* w, int transpose_b, int64_t K, int64_t
                             int32_t* colsum, void* stream);
 
 /* out[M,N] = epilogue( a[M,K] (u8 or s8, row-major) x packed weight ), exact int32 accumulation.
- * a_type QUINT8 | QINT8; out_type QINT32 | QINT8 | QUINT8 | FLOAT | BFLOAT16.  `colsum` is needed for QUINT8
+ * a_type QUINT8 | QINT8; out_type QINT32 | QINT8 | QUINT8 | FLOAT | BFLOAT16 | HALF.  `colsum` is needed for QUINT8
  * activations (they are fed to the signed MFMA as a-128 and corrected by 128*colsum[n]).
  * `scales` has ep->n_scales floats (may be NULL when 0), `bias` N floats (NULL = no bias add).
  * Dispatches to the bandwidth-bound small-M kernel for M <= 16 and to the MFMA tile kernel
@@ -257,7 +257,7 @@ int itexhip_qgemv(const void* a, int a_type, const int8_t* packed_b, const int32
  * operation sequence), so no parameter vectors and no second kernel are needed.  This is what the
  * op kernel calls per Compute (quantized_matmul_common.h:62-460: Init + primitive execute);
  * a changed min_a / max_a costs nothing extra.  `bias` is the op's raw bias (fp32; int32 when
- * p->t_bias is QINT32, bfloat16 bits when BFLOAT16; may be null).  `addend` is the [M, N] fp32 tensor of the "Add" fusion
+ * p->t_bias is QINT32, 16-bit patterns when BFLOAT16 / HALF; may be null).  `addend` is the [M, N] fp32 tensor of the "Add" fusion
  * (p->add_position != 0; the reference adds it in place into the output buffer, :352-389), else null. */
 int itexhip_qmatmul(const itexhip_matmul_params* p, const void* a, const int8_t* packed_b,
                     const int32_t* colsum, int64_t M, int64_t K, int64_t N, const float* min_b,

@@ -66,11 +66,35 @@ __device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
   return u >> 16;
 }
 
-// one output element of a quantized MatMul: fp32 kept, bfloat16 rounded, integers saturated + rounded
+// fp32 <-> half bit patterns (v_cvt_f16_f32 / v_cvt_f32_f16: round to nearest even, denormals kept)
+__device__ __forceinline__ uint32_t f32_to_f16_bits(float f) {
+  const _Float16 h = static_cast<_Float16>(f);
+  unsigned short bits;
+  __builtin_memcpy(&bits, &h, 2);
+  return bits;
+}
+__device__ __forceinline__ float f16_bits_to_f32(uint32_t b) {
+  const unsigned short bits = static_cast<unsigned short>(b);
+  _Float16 h;
+  __builtin_memcpy(&h, &bits, 2);
+  return static_cast<float>(h);
+}
+
+// the 16-bit float types travel as bit patterns
+__host__ __device__ constexpr bool is_float16_type(int t) { return t == ITEXHIP_BFLOAT16 || t == ITEXHIP_HALF; }
+// float-like output types: the parameter preparation treats them alike (fp32 epilogue, converted in the store)
+__host__ __device__ constexpr bool is_float_out(int t) { return t == ITEXHIP_FLOAT || is_float16_type(t); }
+template <int T16>
+__device__ __forceinline__ uint32_t f32_to_bits16(float f) {
+  if constexpr (T16 == ITEXHIP_BFLOAT16) return f32_to_bf16_bits(f);
+  else return f32_to_f16_bits(f);
+}
+
+// one output element of a quantized MatMul: fp32 kept, bfloat16 / half rounded, integers saturated + rounded
 template <int OUT_T>
 __device__ __forceinline__ void store_output(void* __restrict__ out, int64_t idx, float v) {
   if constexpr (OUT_T == ITEXHIP_FLOAT) static_cast<float*>(out)[idx] = v;
-  else if constexpr (OUT_T == ITEXHIP_BFLOAT16) static_cast<uint16_t*>(out)[idx] = static_cast<uint16_t>(f32_to_bf16_bits(v));
+  else if constexpr (is_float16_type(OUT_T)) static_cast<uint16_t*>(out)[idx] = static_cast<uint16_t>(f32_to_bits16<OUT_T>(v));
   else if constexpr (OUT_T == ITEXHIP_QINT32) static_cast<int32_t*>(out)[idx] = sat_rne<ITEXHIP_QINT32>(v);
   else static_cast<uint8_t*>(out)[idx] = static_cast<uint8_t>(sat_rne<OUT_T>(v));
 }

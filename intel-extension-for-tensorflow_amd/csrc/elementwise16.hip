@@ -16,12 +16,7 @@ typedef unsigned int u4 __attribute__((ext_vector_type(4)));
 
 __device__ __forceinline__ float bf16_to_f32(uint32_t h) { return bf16_bits_to_f32(h); }
 __device__ __forceinline__ uint32_t f32_to_bf16(float f) { return f32_to_bf16_bits(f); }
-__device__ __forceinline__ uint32_t f32_to_f16(float f) {
-  const _Float16 h = static_cast<_Float16>(f);  // v_cvt_f16_f32, round to nearest even
-  unsigned short bits;
-  __builtin_memcpy(&bits, &h, 2);
-  return bits;
-}
+__device__ __forceinline__ uint32_t f32_to_f16(float f) { return f32_to_f16_bits(f); }
 template <int YT>
 __device__ __forceinline__ uint32_t narrow(float f) {
   return YT == ITEXHIP_BFLOAT16 ? f32_to_bf16(f) : f32_to_f16(f);

@@ -310,7 +310,7 @@ int check_common(const void* a, int a_type, const void* b, int64_t M, int64_t K,
                  const char* who) {
   ITEXHIP_REQUIRE(a_type == ITEXHIP_QUINT8 || a_type == ITEXHIP_QINT8, "%s: activation type must be quint8 or qint8", who);
   ITEXHIP_REQUIRE(out_type == ITEXHIP_QINT32 || out_type == ITEXHIP_QINT8 || out_type == ITEXHIP_QUINT8 ||
-                      out_type == ITEXHIP_FLOAT || out_type == ITEXHIP_BFLOAT16, "%s: unsupported output type %d", who, out_type);
+                      is_float_out(out_type), "%s: unsupported output type %d", who, out_type);
   ITEXHIP_REQUIRE(M >= 0 && K >= 0 && N >= 0, "%s: negative dimension", who);
   ITEXHIP_REQUIRE(M < (1LL << 31) && N < (1LL << 31) && K <= kMaxK, "%s: dimension too large (K <= %lld)", who,
                   static_cast<long long>(kMaxK));
@@ -367,6 +367,7 @@ int dispatch_gemv(const uint8_t* a, uint32_t a_xor, const uint8_t* bp, int M, in
   switch (out_type) {                                                         \
     case ITEXHIP_FLOAT: st__ = CALL(ITEXHIP_FLOAT); break;                    \
     case ITEXHIP_BFLOAT16: st__ = CALL(ITEXHIP_BFLOAT16); break;              \
+    case ITEXHIP_HALF: st__ = CALL(ITEXHIP_HALF); break;                      \
     case ITEXHIP_QINT32: st__ = CALL(ITEXHIP_QINT32); break;                  \
     case ITEXHIP_QINT8: st__ = CALL(ITEXHIP_QINT8); break;                    \
     default: st__ = CALL(ITEXHIP_QUINT8); break;                              \
@@ -475,6 +476,9 @@ extern "C" int itexhip_qgemm_naive(const void* a, int a_type, const int8_t* w, i
     case ITEXHIP_BFLOAT16:
       qgemm_naive_kernel<ITEXHIP_BFLOAT16><<<grid, 256, 0, hs>>>(ap, a_is_u8, w, transpose_b, Mi, Ki, Ni, e, out);
       break;
+    case ITEXHIP_HALF:
+      qgemm_naive_kernel<ITEXHIP_HALF><<<grid, 256, 0, hs>>>(ap, a_is_u8, w, transpose_b, Mi, Ki, Ni, e, out);
+      break;
     case ITEXHIP_FLOAT:
       qgemm_naive_kernel<ITEXHIP_FLOAT><<<grid, 256, 0, hs>>>(ap, a_is_u8, w, transpose_b, Mi, Ki, Ni, e, out);
       break;
@@ -581,6 +585,7 @@ extern "C" int itexhip_qmatmul_unpacked(const itexhip_matmul_params* p, const vo
   switch (p->t_out) {
     case ITEXHIP_FLOAT: qmatmul_unpacked_kernel<ITEXHIP_FLOAT><<<grid, 256, 0, hs>>>(ap, a_is_u8, w, transpose_b, Mi, Ki, Ni, e, out); break;
     case ITEXHIP_BFLOAT16: qmatmul_unpacked_kernel<ITEXHIP_BFLOAT16><<<grid, 256, 0, hs>>>(ap, a_is_u8, w, transpose_b, Mi, Ki, Ni, e, out); break;
+    case ITEXHIP_HALF: qmatmul_unpacked_kernel<ITEXHIP_HALF><<<grid, 256, 0, hs>>>(ap, a_is_u8, w, transpose_b, Mi, Ki, Ni, e, out); break;
     case ITEXHIP_QINT32: qmatmul_unpacked_kernel<ITEXHIP_QINT32><<<grid, 256, 0, hs>>>(ap, a_is_u8, w, transpose_b, Mi, Ki, Ni, e, out); break;
     case ITEXHIP_QINT8: qmatmul_unpacked_kernel<ITEXHIP_QINT8><<<grid, 256, 0, hs>>>(ap, a_is_u8, w, transpose_b, Mi, Ki, Ni, e, out); break;
     default: qmatmul_unpacked_kernel<ITEXHIP_QUINT8><<<grid, 256, 0, hs>>>(ap, a_is_u8, w, transpose_b, Mi, Ki, Ni, e, out); break;

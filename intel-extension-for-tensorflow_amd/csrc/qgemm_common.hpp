@@ -119,9 +119,9 @@ __device__ __forceinline__ v4i epilogue_convert(const v4i acc, const f4 scale, c
   }
   if constexpr (OUT_T == ITEXHIP_FLOAT) {
     return v4i{__float_as_int(y[0]), __float_as_int(y[1]), __float_as_int(y[2]), __float_as_int(y[3])};
-  } else if constexpr (OUT_T == ITEXHIP_BFLOAT16) {  // 4 x 16 bits in .x, .y
-    return v4i{static_cast<int>(f32_to_bf16_bits(y[0]) | (f32_to_bf16_bits(y[1]) << 16)),
-               static_cast<int>(f32_to_bf16_bits(y[2]) | (f32_to_bf16_bits(y[3]) << 16)), 0, 0};
+  } else if constexpr (is_float16_type(OUT_T)) {  // 4 x 16 bits in .x, .y
+    return v4i{static_cast<int>(f32_to_bits16<OUT_T>(y[0]) | (f32_to_bits16<OUT_T>(y[1]) << 16)),
+               static_cast<int>(f32_to_bits16<OUT_T>(y[2]) | (f32_to_bits16<OUT_T>(y[3]) << 16)), 0, 0};
   } else if constexpr (OUT_T == ITEXHIP_QINT32) {
     return v4i{sat_rne<ITEXHIP_QINT32>(y[0]), sat_rne<ITEXHIP_QINT32>(y[1]), sat_rne<ITEXHIP_QINT32>(y[2]),
                sat_rne<ITEXHIP_QINT32>(y[3])};
@@ -168,14 +168,14 @@ __device__ __forceinline__ void epilogue_store(const v4i acc, const ChannelParam
     } else {
       for (int r = 0; r < 4 && n + r < N; ++r) dst[r] = y[r];
     }
-  } else if constexpr (OUT_T == ITEXHIP_BFLOAT16) {
+  } else if constexpr (is_float16_type(OUT_T)) {
     uint16_t* dst = reinterpret_cast<uint16_t*>(out) + o;
     if (full) {
       typedef unsigned int u2 __attribute__((ext_vector_type(2)));
-      *reinterpret_cast<u2*>(dst) = u2{f32_to_bf16_bits(y[0]) | (f32_to_bf16_bits(y[1]) << 16),
-                                       f32_to_bf16_bits(y[2]) | (f32_to_bf16_bits(y[3]) << 16)};
+      *reinterpret_cast<u2*>(dst) = u2{f32_to_bits16<OUT_T>(y[0]) | (f32_to_bits16<OUT_T>(y[1]) << 16),
+                                       f32_to_bits16<OUT_T>(y[2]) | (f32_to_bits16<OUT_T>(y[3]) << 16)};
     } else {
-      for (int r = 0; r < 4 && n + r < N; ++r) dst[r] = static_cast<uint16_t>(f32_to_bf16_bits(y[r]));
+      for (int r = 0; r < 4 && n + r < N; ++r) dst[r] = static_cast<uint16_t>(f32_to_bits16<OUT_T>(y[r]));
     }
   } else if constexpr (OUT_T == ITEXHIP_QINT32) {
     int32_t* dst = reinterpret_cast<int32_t*>(out) + o;

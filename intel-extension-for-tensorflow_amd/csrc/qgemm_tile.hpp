@@ -267,7 +267,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void qgemm_tile_kernel(
   // the MFMA layout owns one row and scattered 4-channel groups, which would make every store a
   // 64-address scatter.  The buffer holds [WM rows][ROWB bytes] with a 16-byte pad per row: for 8-bit
   // outputs all TN channel tiles at once, for 32-bit outputs one channel tile per pass.
-  constexpr int ESZ = (OUT_T == ITEXHIP_QINT8 || OUT_T == ITEXHIP_QUINT8) ? 1 : (OUT_T == ITEXHIP_BFLOAT16) ? 2 : 4;
+  constexpr int ESZ = (OUT_T == ITEXHIP_QINT8 || OUT_T == ITEXHIP_QUINT8) ? 1 : is_float16_type(OUT_T) ? 2 : 4;
   constexpr int JB = (ESZ == 1) ? TN : (ESZ == 2) ? ((TN % 2 == 0) ? 2 : TN) : 1;  // channel tiles per pass
   constexpr int ROWB = JB * 32 * ESZ;        // row bytes in the buffer
   constexpr int PITCH = ROWB + 16;
@@ -404,7 +404,7 @@ int dispatch_tile_shape(const uint8_t* a, uint32_t amask, const uint8_t* bp, int
 template <int OUT_T>
 int dispatch_tile(const uint8_t* a, uint32_t a_xor, const uint8_t* bp, int M, int K, int N,
                   const EpilogueArgs& e, void* out, hipStream_t st) {
-  constexpr int esz = (OUT_T == ITEXHIP_QINT8 || OUT_T == ITEXHIP_QUINT8) ? 1 : (OUT_T == ITEXHIP_BFLOAT16) ? 2 : 4;
+  constexpr int esz = (OUT_T == ITEXHIP_QINT8 || OUT_T == ITEXHIP_QUINT8) ? 1 : is_float16_type(OUT_T) ? 2 : 4;
   // the specialised kernels only carry the vectorised epilogue: bias present, output rows 16-byte aligned
   const bool plain = e.addend == nullptr && (e.bias != nullptr || e.fused) && (reinterpret_cast<uintptr_t>(out) & 15) == 0 &&
                      ((static_cast<int64_t>(N) * esz) & 15) == 0 && (K & 63) == 0;

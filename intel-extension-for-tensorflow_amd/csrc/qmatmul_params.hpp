@@ -18,8 +18,8 @@ struct PrepArgs {
   int mul_requant;     // multiply the output scale by (max_int8_output / range_output)
   int legacy_kind;     // 1: u8 out, 2: s8 out, 3: fp32 out (legacy api only)
   int bias_s32;        // Tbias = qint32: the bias vector holds int32 (quantized_matmul_common.h:1153-1334)
-  int bias_bf16;       // Tbias = bfloat16: widened to fp32, the fp32 arithmetic, and the adjusted bias rounded
-                       // to bfloat16 again, as the generic-in-Tbias code stores it (:578-599, 609-617)
+  int bias_16;         // Tbias = bfloat16 / half (the type, else 0): widened to fp32, the fp32 arithmetic, and the
+                       // adjusted bias rounded to Tbias again, as the generic-in-Tbias code stores it (:578-599, 609-617)
   float min_a, max_a, min_out, max_out;
 };
 
@@ -27,7 +27,8 @@ struct PrepArgs {
 __device__ __forceinline__ float bias_entry(const PrepArgs& p, const void* bias, int64_t j) {
   if (bias == nullptr) return 0.0f;
   if (p.bias_s32) return static_cast<float>(static_cast<const int32_t*>(bias)[j]);
-  if (p.bias_bf16) return bf16_bits_to_f32(static_cast<const uint16_t*>(bias)[j]);
+  if (p.bias_16 == ITEXHIP_BFLOAT16) return bf16_bits_to_f32(static_cast<const uint16_t*>(bias)[j]);
+  if (p.bias_16 == ITEXHIP_HALF) return f16_bits_to_f32(static_cast<const uint16_t*>(bias)[j]);
   return static_cast<const float*>(bias)[j];
 }
 
@@ -78,7 +79,7 @@ __device__ __forceinline__ ChannelScaleBias channel_scale_bias(const PrepArgs& p
     // qint32 bias: scaled by the inverse of the fp32 path's factor, no zero-point compensation (:1204-1271)
     const float sj = (range_input * range_weight) / (max_int8_input * max_int8_weight);
     float out;
-    if (p.input_mode != ITEXHIP_MIN_FIRST || p.t_out == ITEXHIP_FLOAT || p.t_out == ITEXHIP_BFLOAT16) out = b * sj;
+    if (p.input_mode != ITEXHIP_MIN_FIRST || is_float_out(p.t_out)) out = b * sj;
     else if (p.t_out == ITEXHIP_QINT8 || p.t_out == ITEXHIP_QUINT8) out = b * os;
     else out = b;
     return ChannelScaleBias{os, out};
@@ -88,7 +89,7 @@ __device__ __forceinline__ ChannelScaleBias channel_scale_bias(const PrepArgs& p
   if (p.input_mode == ITEXHIP_MIN_FIRST) {
     const float q_min_input = max_int8_input * p.min_a / range_input;
     const float sum = static_cast<float>(colsum_j);
-    if (p.t_out == ITEXHIP_FLOAT || p.t_out == ITEXHIP_BFLOAT16) {
+    if (is_float_out(p.t_out)) {
       out = b + (sum * q_min_input / bias_scale);
     } else if (p.t_out == ITEXHIP_QINT8 || p.t_out == ITEXHIP_QUINT8) {
       // os is this channel's output scale, or the single scale when n_scales == 1
@@ -101,7 +102,8 @@ __device__ __forceinline__ ChannelScaleBias channel_scale_bias(const PrepArgs& p
     const float bs0 = (max_int8_input * max_int8_weight) / (range_input * absmax(min_b0, max_b0));
     out = b * bs0;
   }
-  if (p.bias_bf16) out = bf16_bits_to_f32(f32_to_bf16_bits(out));
+  if (p.bias_16 == ITEXHIP_BFLOAT16) out = bf16_bits_to_f32(f32_to_bf16_bits(out));
+  if (p.bias_16 == ITEXHIP_HALF) out = f16_bits_to_f32(f32_to_f16_bits(out));
   return ChannelScaleBias{os, out};
 }
 
@@ -123,7 +125,7 @@ inline PrepArgs make_prep_args(const itexhip_matmul_params* p, const itexhip_epi
   a.api = p->api; a.t_in = p->t_in; a.t_out = p->t_out; a.input_mode = p->input_mode;
   a.n_scales = ep.n_scales;
   a.bias_s32 = p->t_bias == ITEXHIP_QINT32;
-  a.bias_bf16 = p->t_bias == ITEXHIP_BFLOAT16;
+  a.bias_16 = is_float16_type(p->t_bias) ? p->t_bias : 0;
   a.min_a = p->min_a; a.max_a = p->max_a; a.min_out = p->min_out; a.max_out = p->max_out;
   const bool out_q8 = p->t_out == ITEXHIP_QINT8 || p->t_out == ITEXHIP_QUINT8;
   if (p->api == ITEXHIP_API_V2) {
@@ -135,7 +137,7 @@ inline PrepArgs make_prep_args(const itexhip_matmul_params* p, const itexhip_epi
     a.mul_requant = out_q8 && p->n_fused_ops == 1;
   } else {
     a.legacy_kind = p->t_out == ITEXHIP_QUINT8 ? 1 : p->t_out == ITEXHIP_QINT8 ? 2
-                    : (p->t_out == ITEXHIP_FLOAT || p->t_out == ITEXHIP_BFLOAT16) ? 3 : 0;
+                    : is_float_out(p->t_out) ? 3 : 0;
   }
   return a;
 }

@@ -42,15 +42,15 @@ int validate(const itexhip_matmul_params* p, int64_t nb) {
                   "qmatmul: unknown api %d", p->api);
   ITEXHIP_REQUIRE(p->t_in == ITEXHIP_QUINT8 || p->t_in == ITEXHIP_QINT8, "qmatmul: T1 must be quint8 or qint8");
   ITEXHIP_REQUIRE(p->t_out == ITEXHIP_QINT32 || p->t_out == ITEXHIP_QINT8 || p->t_out == ITEXHIP_QUINT8 ||
-                      p->t_out == ITEXHIP_FLOAT || p->t_out == ITEXHIP_BFLOAT16,
+                      is_float_out(p->t_out),
                   "qmatmul: unsupported output type %d", p->t_out);
   ITEXHIP_REQUIRE(p->input_mode == ITEXHIP_MIN_FIRST || p->input_mode == ITEXHIP_SCALED,
                   "Quantization mode must be either MIN_FIRST or SCALED");
   ITEXHIP_REQUIRE(nb >= 1, "qmatmul: empty weight range");
-  ITEXHIP_REQUIRE(p->t_bias == 0 || p->t_bias == ITEXHIP_FLOAT || p->t_bias == ITEXHIP_QINT32 || p->t_bias == ITEXHIP_BFLOAT16,
-                  "qmatmul: Tbias must be float, bfloat16 or qint32");
+  ITEXHIP_REQUIRE(p->t_bias == 0 || p->t_bias == ITEXHIP_FLOAT || p->t_bias == ITEXHIP_QINT32 || is_float16_type(p->t_bias),
+                  "qmatmul: Tbias must be float, bfloat16, half or qint32");
   ITEXHIP_REQUIRE(p->add_position >= 0 && p->add_position <= 2, "qmatmul: bad add_position");
-  if (p->add_position != 0 && p->t_out != ITEXHIP_FLOAT) {  // (a bfloat16 addend is not implemented here)
+  if (p->add_position != 0 && p->t_out != ITEXHIP_FLOAT) {  // (a bfloat16 / half addend is not implemented here)
     set_error("Quantized addend tensor is not implemented yet.");
     return ITEXHIP_UNIMPLEMENTED;
   }

@@ -114,8 +114,8 @@ class QuantizedMatMulOp : public OpKernel {
     if (ctx->HasAttr(bias_attr)) {
       TF_DataType tb = TF_FLOAT;
       ITEX_REQUIRES_OK(ctx, ctx->GetAttr(bias_attr, &tb));
-      ITEX_REQUIRES(ctx, tb == TF_FLOAT || tb == TF_QINT32 || tb == TF_BFLOAT16, TF_UNIMPLEMENTED,
-                    "only float, bfloat16 and qint32 biases are implemented on this device");
+      ITEX_REQUIRES(ctx, tb == TF_FLOAT || tb == TF_QINT32 || tb == TF_BFLOAT16 || tb == TF_HALF, TF_UNIMPLEMENTED,
+                    "only float, bfloat16, half and qint32 biases are implemented on this device");
       p_.t_bias = tb;
     }
     if (p_.add_position != 0) {
@@ -136,7 +136,7 @@ class QuantizedMatMulOp : public OpKernel {
     if (!ctx->ok()) return;
     ITEX_REQUIRES(ctx, !transpose_a_, TF_UNIMPLEMENTED, "transpose_a is not supported by the quantized MatMul");
     ITEX_REQUIRES(ctx, a.dims() == 2 && w.dims() == 2, TF_INVALID_ARGUMENT, "quantized MatMul operands must be matrices");
-    const TF_DataType bias_type = p_.t_bias == ITEXHIP_QINT32 ? TF_QINT32 : p_.t_bias == ITEXHIP_BFLOAT16 ? TF_BFLOAT16 : TF_FLOAT;
+    const TF_DataType bias_type = p_.t_bias == 0 ? TF_FLOAT : static_cast<TF_DataType>(p_.t_bias);
     ITEX_REQUIRES(ctx, a.dtype() == v_.t_in && w.dtype() == TF_QINT8 && bias.dtype() == bias_type, TF_INVALID_ARGUMENT,
                   "quantized MatMul operand types do not match the kernel");
     const int64_t M = a.dim_size(0), K = a.dim_size(1);
@@ -158,7 +158,8 @@ class QuantizedMatMulOp : public OpKernel {
     p.min_a = min_a_t.flat<float>()[0];
     p.max_a = max_a_t.flat<float>()[0];
     const bool out_q8 = v_.t_out == TF_QINT8 || v_.t_out == TF_QUINT8;
-    const bool needs_freezed = out_q8 || (v_.api == Api::LEGACY && (v_.t_out == TF_FLOAT || v_.t_out == TF_BFLOAT16));
+    const bool needs_freezed =
+        out_q8 || (v_.api == Api::LEGACY && (v_.t_out == TF_FLOAT || v_.t_out == TF_BFLOAT16 || v_.t_out == TF_HALF));
     if (needs_freezed) {
       ITEX_REQUIRES(ctx, ctx->num_inputs() > min_out_idx_ + 1, TF_INVALID_ARGUMENT,
                     "min_freezed_output / max_freezed_output inputs are missing");
@@ -266,9 +267,9 @@ void Reg(const char* op, const char* out_attr, const char* bias_attr, std::initi
   b.TypeConstraint(out_attr, static_cast<TF_DataType>(TOUT));
   for (const char* h : host_args) b.HostMemory(h);
   b.Register<MatMulKernel<API, TIN, TOUT, RELU>>();
-  if (bias_attr) {  // the same kernel with a qint32 bias and, for the V1 / V2 ops, a bfloat16 bias
-    for (TF_DataType tb : {TF_QINT32, TF_BFLOAT16}) {
-      if (tb == TF_BFLOAT16 && API == ITEXHIP_API_LEGACY) continue;
+  if (bias_attr) {  // the same kernel with a qint32 bias and, for the V1 / V2 ops, a bfloat16 / half bias
+    for (TF_DataType tb : {TF_QINT32, TF_BFLOAT16, TF_HALF}) {
+      if (tb != TF_QINT32 && API == ITEXHIP_API_LEGACY) continue;
       KernelDefBuilder q(op, "QuantizedMatMulOp");
       q.TypeConstraint("T1", static_cast<TF_DataType>(TIN)).TypeConstraint("T2", TF_QINT8);
       q.TypeConstraint(bias_attr, tb).TypeConstraint(out_attr, static_cast<TF_DataType>(TOUT));
@@ -305,16 +306,21 @@ void AddQuantizedMatMulKernels() {
   for (const char* op : {"QuantizedMatMulWithBiasAndDequantize", "_ITEXQuantizedMatMulWithBiasAndDequantize"})
     Reg<LG, TF_QUINT8, TF_FLOAT, false>(op, "Toutput", "Tbias",
                                         {"min_a", "max_a", "min_b", "max_b", "min_freezed_output", "max_freezed_output"});
-  for (const char* op : {"QuantizedMatMulWithBiasAndDequantize", "_ITEXQuantizedMatMulWithBiasAndDequantize"})
+  for (const char* op : {"QuantizedMatMulWithBiasAndDequantize", "_ITEXQuantizedMatMulWithBiasAndDequantize"}) {
     Reg<LG, TF_QUINT8, TF_BFLOAT16, false>(op, "Toutput", "Tbias",
                                            {"min_a", "max_a", "min_b", "max_b", "min_freezed_output", "max_freezed_output"});
+    Reg<LG, TF_QUINT8, TF_HALF, false>(op, "Toutput", "Tbias",
+                                       {"min_a", "max_a", "min_b", "max_b", "min_freezed_output", "max_freezed_output"});
+  }
   // V1
   for (const char* op : {"_QuantizedFusedMatMul", "_ITEXQuantizedFusedMatMul"})
     RegBothInputs<V1, TF_QINT32>(op, "Toutput", "Targs", {"min_a", "max_a", "min_b", "max_b", "min_product", "max_product"});
   for (const char* op : {"_QuantizedFusedMatMulAndDequantize", "_ITEXQuantizedFusedMatMulAndDequantize"})
     RegBothInputs<V1, TF_FLOAT>(op, "Toutput", "Targs", {"min_a", "max_a", "min_b", "max_b"});
-  for (const char* op : {"_QuantizedFusedMatMulAndDequantize", "_ITEXQuantizedFusedMatMulAndDequantize"})
+  for (const char* op : {"_QuantizedFusedMatMulAndDequantize", "_ITEXQuantizedFusedMatMulAndDequantize"}) {
     RegBothInputs<V1, TF_BFLOAT16>(op, "Toutput", "Targs", {"min_a", "max_a", "min_b", "max_b"});
+    RegBothInputs<V1, TF_HALF>(op, "Toutput", "Targs", {"min_a", "max_a", "min_b", "max_b"});
+  }
   for (const char* op : {"_QuantizedFusedMatMulAndRequantize", "_ITEXQuantizedFusedMatMulAndRequantize"}) {
     RegBothInputs<V1, TF_QUINT8>(op, "Toutput", "Targs", {"min_a", "max_a", "min_b", "max_b", "min_freezed_output",
                                                           "max_freezed_output", "min_product", "max_product"});

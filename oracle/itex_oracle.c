@@ -304,12 +304,55 @@ static inline uint16_t f32_to_bf16_bits(float f) {
   return (uint16_t)(u >> 16);
 }
 
+/* fp32 -> IEEE half, round to nearest even, overflow to infinity, denormals kept */
+static inline uint16_t f32_to_f16_bits(float f) {
+  uint32_t u;
+  memcpy(&u, &f, 4);
+  const uint16_t sign = (uint16_t)((u >> 16) & 0x8000u);
+  const uint32_t a = u & 0x7fffffffu;
+  if (a > 0x7f800000u) return (uint16_t)(sign | 0x7e00u);          /* NaN */
+  if (a >= 0x477ff000u) return (uint16_t)(sign | 0x7c00u);         /* >= 65520 rounds to infinity */
+  if (a < 0x33000001u) return sign;                                /* <= 2^-25 rounds to zero */
+  const int e = (int)(a >> 23) - 127;
+  uint32_t m = (a & 0x7fffffu) | 0x800000u;                        /* 24-bit significand */
+  int shift;                                                       /* bits dropped from m */
+  uint32_t base;
+  if (e < -14) { shift = 13 + (-14 - e); base = 0; }               /* half denormal: value = m * 2^(e-23) / 2^-24 */
+  else { shift = 13; base = (uint32_t)(e + 15) << 10; m &= 0x7fffffu; }
+  const uint32_t q = m >> shift, rem = m & ((1u << shift) - 1u), halfway = 1u << (shift - 1);
+  uint32_t r = base + q;
+  if (rem > halfway || (rem == halfway && (r & 1u))) r += 1u;      /* carries into the exponent correctly */
+  return (uint16_t)(sign | r);
+}
+
+static inline float f16_bits_to_f32(uint16_t h) {
+  const uint32_t sign = (uint32_t)(h & 0x8000u) << 16;
+  const uint32_t e = (h >> 10) & 0x1fu, m = h & 0x3ffu;
+  uint32_t u;
+  if (e == 0x1fu) u = sign | 0x7f800000u | (m << 13);
+  else if (e != 0) u = sign | ((e + 112u) << 23) | (m << 13);
+  else if (m == 0) u = sign;
+  else {
+    float f = (float)m * 5.9604644775390625e-08f; /* m * 2^-24, exact */
+    memcpy(&u, &f, 4);
+    u |= sign;
+  }
+  float f;
+  memcpy(&f, &u, 4);
+  return f;
+}
+
+static inline uint16_t f32_to_bits16(int t, float f) { return t == ORC_HALF ? f32_to_f16_bits(f) : f32_to_bf16_bits(f); }
+static inline float bits16_to_f32(int t, uint16_t h);
+
 static inline float bf16_bits_to_f32(uint16_t h) {
   const uint32_t u = (uint32_t)h << 16;
   float f;
   memcpy(&f, &u, 4);
   return f;
 }
+
+static inline float bits16_to_f32(int t, uint16_t h) { return t == ORC_HALF ? f16_bits_to_f32(h) : bf16_bits_to_f32(h); }
 
 /*
  * Host-side parameter preparation of the quantized MatMul kernels:
@@ -328,11 +371,11 @@ int orc_qmatmul_prepare(const orc_matmul_attrs* at, int64_t N, const int32_t* co
   /* Tbias = bfloat16: GetScaledBias is generic in Tbias; every entry is widened with
    * static_cast<float>, the arithmetic is fp32, and the result is stored as Tbias again (:578-599 cast,
    * :609-617 the reorder's bf16 destination), i.e. rounded to bfloat16 before the primitive reads it */
-  const int bias_bf16 = (at->t_bias == ORC_BFLOAT16);
+  const int bias_bf16 = (at->t_bias == ORC_BFLOAT16 || at->t_bias == ORC_HALF); /* either 16-bit float type */
   const int32_t* bias_i32 = (const int32_t*)bias_v;
   const int out_q8 = (at->t_out == ORC_QINT8 || at->t_out == ORC_QUINT8);
   /* the float-output branches upstream test Toutput against float, bfloat16 and half alike (:577, 1255-1257) */
-  const int out_f32 = (at->t_out == ORC_FLOAT || at->t_out == ORC_BFLOAT16);
+  const int out_f32 = (at->t_out == ORC_FLOAT || at->t_out == ORC_BFLOAT16 || at->t_out == ORC_HALF);
   const int out_s32 = (at->t_out == ORC_QINT32);
   if (!out_q8 && !out_f32 && !out_s32) return ORC_INVALID_ARGUMENT;
   if (at->input_mode != ORC_MIN_FIRST && at->input_mode != ORC_SCALED) return ORC_INVALID_ARGUMENT;
@@ -454,7 +497,7 @@ int orc_qmatmul_prepare(const orc_matmul_attrs* at, int64_t N, const int32_t* co
   float* bias_wide = NULL;
   if (bias_bf16) {
     bias_wide = (float*)malloc(sizeof(float) * (size_t)(N > 0 ? N : 1));
-    for (int64_t j = 0; j < N; ++j) bias_wide[j] = bf16_bits_to_f32(((const uint16_t*)bias_v)[j]);
+    for (int64_t j = 0; j < N; ++j) bias_wide[j] = bits16_to_f32(at->t_bias, ((const uint16_t*)bias_v)[j]);
   }
   const float* bias = bias_bf16 ? bias_wide : (const float*)bias_v;
   if (bias_s32) {
@@ -500,7 +543,7 @@ int orc_qmatmul_prepare(const orc_matmul_attrs* at, int64_t N, const int32_t* co
     for (int64_t j = 0; j < N; ++j) bias_out[j] = bias[j] * bias_scales[0];
   }
   if (bias_bf16) {
-    for (int64_t j = 0; j < N; ++j) bias_out[j] = bf16_bits_to_f32(f32_to_bf16_bits(bias_out[j]));
+    for (int64_t j = 0; j < N; ++j) bias_out[j] = bits16_to_f32(at->t_bias, f32_to_bits16(at->t_bias, bias_out[j]));
     free(bias_wide);
   }
   free(bias_scales);
@@ -532,7 +575,7 @@ void orc_qmatmul_epilogue(const int32_t* acc, int64_t M, int64_t N, const orc_ep
                           const float* scales, const float* bias, const float* addend, int t_out,
                           void* out) {
   float lo = 0, hi = 0;
-  if (t_out != ORC_FLOAT && t_out != ORC_BFLOAT16) sat_bounds(t_out, &lo, &hi);
+  if (t_out != ORC_FLOAT && t_out != ORC_BFLOAT16 && t_out != ORC_HALF) sat_bounds(t_out, &lo, &hi);
 #pragma omp parallel for schedule(static)
   for (int64_t m = 0; m < M; ++m) {
     for (int64_t n = 0; n < N; ++n) {
@@ -545,7 +588,7 @@ void orc_qmatmul_epilogue(const int32_t* acc, int64_t M, int64_t N, const orc_ep
         else y = apply_eltwise(&ep->elt[e], y);
       }
       if (t_out == ORC_FLOAT) ((float*)out)[m * N + n] = y;
-      else if (t_out == ORC_BFLOAT16) ((uint16_t*)out)[m * N + n] = f32_to_bf16_bits(y);
+      else if (t_out == ORC_BFLOAT16 || t_out == ORC_HALF) ((uint16_t*)out)[m * N + n] = f32_to_bits16(t_out, y);
       else store_q(out, m * N + n, t_out, sat_rne(y, lo, hi));
     }
   }
@@ -578,7 +621,7 @@ int orc_qmatmul_output_minmax(const orc_matmul_attrs* at, float min_a, float max
       out_max[n] = c_level * (float)q_highest(ORC_QINT32);
     }
     *n_out = cnt;
-  } else if (at->t_out == ORC_FLOAT || at->t_out == ORC_BFLOAT16) {
+  } else if (at->t_out == ORC_FLOAT || at->t_out == ORC_BFLOAT16 || at->t_out == ORC_HALF) {
     *n_out = 0;
   } else {
     return ORC_INVALID_ARGUMENT;

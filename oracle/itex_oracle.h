@@ -27,10 +27,10 @@
  *   the last bits of the GELU post-ops (oneDNN evaluates tanh / erf with its own polynomial
  *   kernels; here libm's tanhf / erff): pinned only against a float64 evaluation and at the
  *   reference tests' own tolerance;
- *   the bfloat16 bias (Tbias = bfloat16): the adjusted bias is rounded to bfloat16 as the code is
+ *   the bfloat16 / half bias (Tbias): the adjusted bias is rounded to Tbias as the code is
  *   written (quantized_matmul_common.h:578-599, 609-617); the reference's tests only use float and
- *   qint32 biases.  The bfloat16 OUTPUT is pinned: it must equal the nearest-even bfloat16 of the
- *   float output of the same node, which the tests check.
+ *   qint32 biases.  The bfloat16 / half OUTPUT is pinned: it must equal the nearest-even 16-bit
+ *   value of the float output of the same node, which the tests check against PyTorch's conversion.
  */
 #ifndef ITEX_ORACLE_H_
 #define ITEX_ORACLE_H_
@@ -42,7 +42,7 @@ extern "C" {
 #endif
 
 /* TF_DataType values used at the op boundary (tensorflow/c/tf_datatype.h). */
-enum { ORC_FLOAT = 1, ORC_INT32 = 3, ORC_QINT8 = 11, ORC_QUINT8 = 12, ORC_QINT32 = 13, ORC_BFLOAT16 = 14 };
+enum { ORC_FLOAT = 1, ORC_INT32 = 3, ORC_QINT8 = 11, ORC_QUINT8 = 12, ORC_QINT32 = 13, ORC_BFLOAT16 = 14, ORC_HALF = 19 };
 /* QuantizeMode, same order as itex/core/utils/quantization_util.h:29-33. */
 enum { ORC_MIN_COMBINED = 0, ORC_MIN_FIRST = 1, ORC_SCALED = 2 };
 /* status */
@@ -71,7 +71,7 @@ typedef struct {
 typedef struct {
   int api;               /* ORC_API_* */
   int t_in;              /* ORC_QUINT8 | ORC_QINT8 (T1) */
-  int t_out;             /* ORC_QINT32 | ORC_QINT8 | ORC_QUINT8 | ORC_FLOAT | ORC_BFLOAT16 (fp32 result rounded to nearest even) */
+  int t_out;             /* ORC_QINT32 | ORC_QINT8 | ORC_QUINT8 | ORC_FLOAT | ORC_BFLOAT16 | ORC_HALF (fp32 result rounded to nearest even) */
   int input_mode;        /* ORC_MIN_FIRST | ORC_SCALED */
   int out_min_first;     /* V2 only: output_quant_mode == "MIN_FIRST" */
   int activation;        /* ORC_ACT_* fused after BiasAdd */
@@ -80,7 +80,7 @@ typedef struct {
   int n_fused_ops;       /* V1: fused_ops.size() (1 = BiasAdd only, 2 = BiasAdd + activation) */
   float leakyrelu_alpha;
   int add_position;      /* "Add" in fused_ops: 0 absent, 1 before the activation, 2 after it */
-  int t_bias;            /* 0 or ORC_FLOAT: fp32 bias;  ORC_QINT32: Tbias = qint32 (:1153-1334);  ORC_BFLOAT16: uint16 bit patterns */
+  int t_bias;            /* 0 or ORC_FLOAT: fp32 bias;  ORC_QINT32: Tbias = qint32 (:1153-1334);  ORC_BFLOAT16 / ORC_HALF: uint16 bit patterns */
 } orc_matmul_attrs;
 
 typedef struct {

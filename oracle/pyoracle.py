@@ -12,13 +12,13 @@ import numpy as np
 _HERE = os.path.dirname(os.path.abspath(__file__))
 _LIB_PATH = os.path.join(_HERE, "libitex_oracle.so")
 
-FLOAT, INT32, QINT8, QUINT8, QINT32, BFLOAT16 = 1, 3, 11, 12, 13, 14
+FLOAT, INT32, QINT8, QUINT8, QINT32, BFLOAT16, HALF = 1, 3, 11, 12, 13, 14, 19
 MIN_COMBINED, MIN_FIRST, SCALED = 0, 1, 2
 API_V2, API_V1, API_LEGACY = 0, 1, 2
 ACT_NONE, ACT_RELU, ACT_RELU6, ACT_LEAKYRELU, ACT_GELU_APPROX, ACT_GELU_EXACT = 0, 1, 2, 3, 4, 5
 OK, INVALID_ARGUMENT, UNIMPLEMENTED = 0, 3, 12
 
-NP_OF = {QINT8: np.int8, QUINT8: np.uint8, QINT32: np.int32, FLOAT: np.float32, BFLOAT16: np.uint16}
+NP_OF = {QINT8: np.int8, QUINT8: np.uint8, QINT32: np.int32, FLOAT: np.float32, BFLOAT16: np.uint16, HALF: np.uint16}
 
 
 def build():
@@ -177,7 +177,7 @@ def _bias(at, bias):
     """The bias vector as the C side reads it (a bfloat16 bias is given as uint16 bit patterns)."""
     if at.t_bias == QINT32:
         return np.ascontiguousarray(bias, dtype=np.int32)
-    if at.t_bias == BFLOAT16:
+    if at.t_bias in (BFLOAT16, HALF):
         return np.ascontiguousarray(bias, dtype=np.uint16)
     return _f32(bias)
 

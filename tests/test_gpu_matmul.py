@@ -13,7 +13,7 @@ pytestmark = pytest.mark.gpu
 def tdt(T):
     import torch
     return {orc.QINT8: torch.int8, orc.QUINT8: torch.uint8, orc.QINT32: torch.int32, orc.FLOAT: torch.float32,
-            orc.BFLOAT16: torch.int16}[T]   # bfloat16 travels as bit patterns
+            orc.BFLOAT16: torch.int16, orc.HALF: torch.int16}[T]   # bfloat16 / half travel as bit patterns
 
 
 def bits16(a):
@@ -503,13 +503,16 @@ def test_qint32_bias_vs_oracle(hip, dev, M, t_out, mode):
 
 
 V2_DEQ_BF16 = dict(V2_DEQ, t_out=orc.BFLOAT16)
+V2_DEQ_F16 = dict(V2_DEQ, t_out=orc.HALF)
 
 
+@pytest.mark.parametrize("T16", [orc.BFLOAT16, orc.HALF])
 @pytest.mark.parametrize("path", ["gemv", "tile", "auto", "fused", "naive"])
 @pytest.mark.parametrize("M,K,N", [(3, 512, 272), (150, 256, 203), (16, 64, 8), (300, 448, 528)])
-def test_bfloat16_output_vs_oracle(hip, dev, path, M, K, N):
-    """Tout = bfloat16 (_QuantizedMatMul, ...AndDequantize): bit patterns equal the oracle's on every kernel, with
-    N odd / not a multiple of the 8-element vector store."""
+def test_bfloat16_output_vs_oracle(hip, dev, path, M, K, N, T16):
+    """Tout = bfloat16 / half (_QuantizedMatMul, ...AndDequantize): bit patterns equal the oracle's on every kernel,
+    with N odd / not a multiple of the 8-element vector store."""
+    V2_DEQ_BF16 = dict(V2_DEQ, t_out=T16)
     if path == "gemv" and M > 16:
         pytest.skip("the small-M kernel takes M <= 16")
     layer, w, bias = make_layer(hip, dev, K, N, seed=K + N)
@@ -521,7 +524,8 @@ def test_bfloat16_output_vs_oracle(hip, dev, path, M, K, N):
 
 
 @pytest.mark.parametrize("shape", [0, 1, 2, 3, 4])
-def test_bfloat16_output_every_tile_shape(hip, dev, monkeypatch, shape):
+@pytest.mark.parametrize("V2_DEQ_BF16", [V2_DEQ_BF16, V2_DEQ_F16], ids=["bf16", "f16"])
+def test_bfloat16_output_every_tile_shape(hip, dev, monkeypatch, shape, V2_DEQ_BF16):
     monkeypatch.setenv("ITEXHIP_TILE_SHAPE", str(shape))
     for M, K, N in [(513, 192, 400), (260, 320, 203)]:
         layer, w, bias = make_layer(hip, dev, K, N, seed=N + shape)
@@ -531,7 +535,8 @@ def test_bfloat16_output_every_tile_shape(hip, dev, monkeypatch, shape):
         np.testing.assert_array_equal(bits16(layer.run(xq, V2_DEQ_BF16, mn, mx, path="fused")), ref)
 
 
-def test_bfloat16_output_unpacked_weight_odd_k(hip, dev):
+@pytest.mark.parametrize("V2_DEQ_BF16", [V2_DEQ_BF16, V2_DEQ_F16], ids=["bf16", "f16"])
+def test_bfloat16_output_unpacked_weight_odd_k(hip, dev, V2_DEQ_BF16):
     import torch
     M, K, N = 37, 75, 61
     layer, w, bias = make_layer(hip, dev, K, N, seed=5)
@@ -546,19 +551,21 @@ def test_bfloat16_output_unpacked_weight_odd_k(hip, dev):
 
 
 @pytest.mark.parametrize("M", [2, 140])
-@pytest.mark.parametrize("t_out,mode", [(orc.FLOAT, orc.MIN_FIRST), (orc.BFLOAT16, orc.MIN_FIRST), (orc.QINT8, orc.MIN_FIRST),
+@pytest.mark.parametrize("t_out,mode", [(orc.FLOAT, orc.MIN_FIRST), (orc.BFLOAT16, orc.MIN_FIRST), (orc.HALF, orc.MIN_FIRST),
+                                        (orc.QINT8, orc.MIN_FIRST),
                                         (orc.QINT32, orc.MIN_FIRST), (orc.FLOAT, orc.SCALED)])
-def test_bfloat16_bias_vs_oracle(hip, dev, M, t_out, mode):
-    """Tbias = bfloat16: the adjusted bias is rounded to bfloat16 before the epilogue adds it."""
+@pytest.mark.parametrize("T16", [orc.BFLOAT16, orc.HALF])
+def test_bfloat16_bias_vs_oracle(hip, dev, M, t_out, mode, T16):
+    """Tbias = bfloat16 / half: the adjusted bias is rounded to that type before the epilogue adds it."""
     import torch
     K, N = 320, 144
     layer, w, _ = make_layer(hip, dev, K, N, seed=34)
     x, xq, mn, mx = make_acts(M, K, seed=M + 5, mode=mode)
-    b16 = torch.from_numpy((np.random.default_rng(7).standard_normal(N) * 0.3).astype(np.float32)).to(torch.bfloat16) \
-        .view(torch.int16).numpy().view(np.uint16)
-    isf = t_out in (orc.FLOAT, orc.BFLOAT16)
+    b16 = torch.from_numpy((np.random.default_rng(7).standard_normal(N) * 0.3).astype(np.float32)) \
+        .to(torch.bfloat16 if T16 == orc.BFLOAT16 else torch.float16).view(torch.int16).numpy().view(np.uint16)
+    isf = t_out in (orc.FLOAT, orc.BFLOAT16, orc.HALF)
     kw = dict(api=orc.API_V2 if t_out != orc.QINT32 else orc.API_V1, t_out=t_out, input_mode=mode,
-              has_dequantize=isf, has_requantize=t_out == orc.QINT8, t_bias=orc.BFLOAT16)
+              has_dequantize=isf, has_requantize=t_out == orc.QINT8, t_bias=T16)
     t_in = orc.QUINT8 if mode == orc.MIN_FIRST else orc.QINT8
     st, ref = orc.qmatmul(orc.matmul_attrs(t_in=t_in, **kw), xq, layer.wq, b16, mn, mx, layer.min_b, layer.max_b, -40.0, 40.0)
     assert st == orc.OK
@@ -566,6 +573,7 @@ def test_bfloat16_bias_vs_oracle(hip, dev, M, t_out, mode):
     np.testing.assert_array_equal(bits16(got), ref)
     # the widened bias through the fp32 path differs (no rounding of the adjusted bias)
     st, ref32 = orc.qmatmul(orc.matmul_attrs(t_in=t_in, **dict(kw, t_bias=orc.FLOAT)), xq, layer.wq,
+                            b16.view(np.float16).astype(np.float32) if T16 == orc.HALF else
                             (b16.astype(np.uint32) << 16).view(np.float32), mn, mx, layer.min_b, layer.max_b, -40.0, 40.0)
     assert st == orc.OK and (t_out != orc.FLOAT or not np.array_equal(ref, ref32))
     # the two-launch form prepares the same vectors

@@ -360,15 +360,40 @@ def test_qint32_bias_closed_forms(mode, t_out, per_channel):
     np.testing.assert_array_equal(sb, expect.astype(np.float32))
 
 
-def _bf16_rne(x):
-    """fp32 -> bfloat16 bit patterns by PyTorch's conversion (round to nearest even), independent of the oracle's."""
+def _bf16_rne(x, T=orc.BFLOAT16):
+    """fp32 -> bfloat16 (or half) bit patterns by PyTorch's / numpy's conversion (round to nearest even), independent
+    of the oracle's."""
     import torch
+    if T == orc.HALF:
+        with np.errstate(over="ignore"):
+            return np.ascontiguousarray(x, np.float32).astype(np.float16).view(np.uint16)
     return torch.from_numpy(np.ascontiguousarray(x, np.float32)).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+
+
+def _widen(bits, T=orc.BFLOAT16):
+    if T == orc.HALF:
+        return bits.view(np.float16).astype(np.float32)
+    return (bits.astype(np.uint32) << 16).view(np.float32)
+
+
+def test_half_conversion_of_the_epilogue_over_the_whole_exponent_range():
+    """The oracle's own fp32 -> half rounding (normals, denormals, ties, overflow to infinity) against numpy's."""
+    rng = np.random.default_rng(0)
+    acc = rng.integers(-2**31, 2**31, (64, 512)).astype(np.int32)
+    acc[0, :8] = [65504, 65519, 65520, 65536, -65520, 1, 3, 0]
+    ep = orc.EpilogueDesc(1, 0)
+    for k in range(0, 60, 3):
+        sc = np.float32(2.0 ** -k)
+        out = orc.qmatmul_epilogue(acc, ep, np.float32([sc]), np.zeros(512, np.float32), orc.HALF)
+        with np.errstate(over="ignore"):
+            np.testing.assert_array_equal(out, _bf16_rne(acc.astype(np.float32) * sc, orc.HALF))
+
 
 
 @pytest.mark.parametrize("api,kw", [(orc.API_V2, dict(has_dequantize=True)), (orc.API_V2, dict(has_dequantize=True, activation=orc.ACT_RELU)),
                                     (orc.API_V1, dict(n_fused_ops=1)), (orc.API_LEGACY, {})])
-def test_bfloat16_output_is_the_rounded_float_output(api, kw):
+@pytest.mark.parametrize("T16", [orc.BFLOAT16, orc.HALF])
+def test_bfloat16_output_is_the_rounded_float_output(api, kw, T16):
     """Tout = bfloat16 follows the float branches of the parameter preparation (:577, 1478-1479) and differs from
     Tout = float only in the destination conversion: nearest-even bfloat16 of the same fp32 value."""
     rng = np.random.default_rng(12)
@@ -379,10 +404,10 @@ def test_bfloat16_output_is_the_rounded_float_output(api, kw):
     args = (a, w, bias, -1.5, 2.5, np.float32([-0.7]), np.float32([0.7]), -30.0, 30.0)
     st, y32 = orc.qmatmul(orc.matmul_attrs(api=api, t_in=orc.QUINT8, t_out=orc.FLOAT, input_mode=orc.MIN_FIRST, **kw), *args)
     assert st == orc.OK
-    st, y16 = orc.qmatmul(orc.matmul_attrs(api=api, t_in=orc.QUINT8, t_out=orc.BFLOAT16, input_mode=orc.MIN_FIRST, **kw), *args)
+    st, y16 = orc.qmatmul(orc.matmul_attrs(api=api, t_in=orc.QUINT8, t_out=T16, input_mode=orc.MIN_FIRST, **kw), *args)
     assert st == orc.OK and y16.dtype == np.uint16
-    np.testing.assert_array_equal(y16, _bf16_rne(y32))
-    assert (y16.astype(np.uint32) << 16).view(np.float32).tolist() != y32.tolist()  # the rounding is not a no-op here
+    np.testing.assert_array_equal(y16, _bf16_rne(y32, T16))
+    assert _widen(y16, T16).tolist() != y32.tolist()  # the rounding is not a no-op here
 
 
 def test_bfloat16_output_ties_round_to_even():
@@ -397,14 +422,15 @@ def test_bfloat16_output_ties_round_to_even():
 
 @pytest.mark.parametrize("mode", [orc.MIN_FIRST, orc.SCALED])
 @pytest.mark.parametrize("t_out", [orc.FLOAT, orc.QINT8, orc.QINT32])
-def test_bfloat16_bias_is_adjusted_in_fp32_and_stored_as_bfloat16(mode, t_out):
+@pytest.mark.parametrize("T16", [orc.BFLOAT16, orc.HALF])
+def test_bfloat16_bias_is_adjusted_in_fp32_and_stored_as_bfloat16(mode, t_out, T16):
     """Tbias = bfloat16: GetScaledBias widens each entry, computes as for fp32 and stores the adjusted bias in
     Tbias again (quantized_matmul_common.h:578-599, 609-617) - so it equals the nearest-even bfloat16 of what the
     fp32 path gives for the widened bias."""
     N = 40
     rng = np.random.default_rng(8)
-    b16 = _bf16_rne(rng.standard_normal(N).astype(np.float32))
-    b32 = (b16.astype(np.uint32) << 16).view(np.float32)
+    b16 = _bf16_rne(rng.standard_normal(N).astype(np.float32), T16)
+    b32 = _widen(b16, T16)
     wmn = -(rng.random(N).astype(np.float32) + 0.5)
     wmx = -wmn
     colsum = rng.integers(-999, 999, N).astype(np.int32)
@@ -413,7 +439,7 @@ def test_bfloat16_bias_is_adjusted_in_fp32_and_stored_as_bfloat16(mode, t_out):
               has_dequantize=t_out == orc.FLOAT, has_requantize=t_out == orc.QINT8)
     st, _, sb32, _ = orc.qmatmul_prepare(orc.matmul_attrs(**kw), N, colsum, -1.25, 2.5, wmn, wmx, -3.0, 3.0, b32)
     assert st == orc.OK
-    st, _, sb16, _ = orc.qmatmul_prepare(orc.matmul_attrs(t_bias=orc.BFLOAT16, **kw), N, colsum, -1.25, 2.5, wmn, wmx, -3.0, 3.0, b16)
+    st, _, sb16, _ = orc.qmatmul_prepare(orc.matmul_attrs(t_bias=T16, **kw), N, colsum, -1.25, 2.5, wmn, wmx, -3.0, 3.0, b16)
     assert st == orc.OK
-    np.testing.assert_array_equal(sb16, (_bf16_rne(sb32).astype(np.uint32) << 16).view(np.float32))
+    np.testing.assert_array_equal(sb16, _widen(_bf16_rne(sb32, T16), T16))
     assert not np.array_equal(sb16, sb32)

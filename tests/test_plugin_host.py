@@ -61,12 +61,12 @@ def test_host_memory_and_constraints(reg):
     assert len(legacy) == 2 and {k["constraints"]["Tbias"] for k in legacy} == {tf.FLOAT, tf.QINT32}
     assert all({**k["constraints"], "Tbias": 0} == {"T1": tf.QUINT8, "T2": tf.QINT8, "Tbias": 0, "Toutput": tf.QUINT8}
                for k in legacy)
-    assert {k["constraints"]["Tbias"] for k in v2} == {tf.FLOAT, tf.QINT32, tf.BFLOAT16}
+    assert {k["constraints"]["Tbias"] for k in v2} == {tf.FLOAT, tf.QINT32, tf.BFLOAT16, tf.HALF}
     assert {(k["constraints"]["Targs"], k["constraints"]["Toutput"]) for k in deq} == {
-        (b, o) for b in (tf.FLOAT, tf.QINT32, tf.BFLOAT16) for o in (tf.FLOAT, tf.BFLOAT16)}
+        (b, o) for b in (tf.FLOAT, tf.QINT32, tf.BFLOAT16, tf.HALF) for o in (tf.FLOAT, tf.BFLOAT16, tf.HALF)}
     ldq = kernels_of(reg, "QuantizedMatMulWithBiasAndDequantize")
     assert {(k["constraints"]["Tbias"], k["constraints"]["Toutput"]) for k in ldq} == {
-        (b, o) for b in (tf.FLOAT, tf.QINT32) for o in (tf.FLOAT, tf.BFLOAT16)}
+        (b, o) for b in (tf.FLOAT, tf.QINT32) for o in (tf.FLOAT, tf.BFLOAT16, tf.HALF)}
 
 
 def test_op_definitions_only_for_missing_ops(reg):
