@@ -289,6 +289,45 @@ int itexhip_qgemm_naive(const void* a, int a_type, const int8_t* w, int transpos
                         int64_t K, int64_t N, const float* scales, const float* bias,
                         const itexhip_epilogue* ep, int out_type, void* out, void* stream);
 
+/* ---- quantized BatchMatMul (qint8 x qint8 -> float / bfloat16 / half) --------------------------
+ * The INT8 batch MatMul either side of the linears in attention blocks:
+ *   _QuantizedBatchMatMul, _QuantizedBatchMatMulV2AndDequantize, _QuantizedFusedBatchMatMulV2AndDequantize
+ *   (itex/core/kernels/common/batch_matmul_op.h:36-522, registered for a device in
+ *   itex/core/kernels/gpu/matmul_op.cc:612-655).
+ * out[b, m, n] = convert( binary_1( binary_0( float(sum_k x[b, m, k] * y[b, k, n]) * scale ) ) ):
+ * exact int32 accumulation, one fp32 multiply by the output scale
+ * (range_x * range_y) / (127 * 127)  (:497-515), then each fused "Mul" / "Add" as a separately rounded
+ * fp32 operation with its operand broadcast to the output (oneDNN binary post-ops, :377-413), then the
+ * conversion to the output type (round to nearest even). */
+enum { ITEXHIP_BIN_MUL = 1, ITEXHIP_BIN_ADD = 2 };
+enum { ITEXHIP_BMM_MAX_BATCH_DIMS = 4, ITEXHIP_BMM_MAX_BINARY = 2 };
+
+typedef struct {
+  int alg;                 /* ITEXHIP_BIN_MUL | ITEXHIP_BIN_ADD, applied in array order */
+  const void* data;        /* device memory; elements of the OUTPUT type (:393-394 builds the operand's
+                            * memory descriptor with OneDnnType<Toutput>) */
+  int64_t batch_stride[ITEXHIP_BMM_MAX_BATCH_DIMS]; /* element strides per batch dim; 0 = broadcast */
+  int64_t stride_m, stride_n;                       /* element strides in the matrix; 0 = broadcast */
+} itexhip_bmm_binary;
+
+typedef struct {
+  int n_batch_dims;                                  /* 0..4; the output is [batch_dims..., M, N], row-major */
+  int64_t batch_dims[ITEXHIP_BMM_MAX_BATCH_DIMS];
+  int64_t x_batch_stride[ITEXHIP_BMM_MAX_BATCH_DIMS]; /* element strides of x per batch dim; 0 = broadcast (MatMulBCast, :105-109) */
+  int64_t y_batch_stride[ITEXHIP_BMM_MAX_BATCH_DIMS];
+  int64_t M, K, N;
+  int adj_x, adj_y;        /* x matrices are [M, K] row-major, or [K, M] with adj_x; y [K, N], or [N, K] with adj_y */
+  int out_type;            /* ITEXHIP_FLOAT | ITEXHIP_BFLOAT16 | ITEXHIP_HALF */
+  float scale;             /* the output scale, computed by the caller in fp32 as written above */
+  int n_binary;            /* 0..2 */
+  itexhip_bmm_binary binary[ITEXHIP_BMM_MAX_BINARY];
+} itexhip_bmm_params;
+
+/* x, y, out: device memory.  Any M, K, N >= 0 and any alignment; 16-byte-aligned operands with K (and, for
+ * the transposed layouts, the row length) a multiple of 16 take the vector-load path.  MFMA 32x32x32 i8
+ * tiles of 64 x 64 outputs per workgroup. */
+int itexhip_qbatch_matmul(const itexhip_bmm_params* p, const int8_t* x, const int8_t* y, void* out, void* stream);
+
 /* Diagnostic, no counterpart in the reference: `workgroups` x 4 wavefronts each issue iters x 8
  * independent 32x32x32 i8 MFMAs (2 * 32768 ops each) on the 8 KiB of operand fragments at `operands`
  * (device memory, 16-byte aligned) and nothing else.  Timed by the caller, it gives the rate the matrix

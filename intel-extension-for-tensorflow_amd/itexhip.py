@@ -29,7 +29,7 @@ EXPORTS = [
     "itexhip_requantize", "itexhip_minmax_i32_per_channel", "itexhip_minmax_f32",
     "itexhip_qmatmul_epilogue_desc", "itexhip_qmatmul_prepare", "itexhip_qgemm_packed_bytes",
     "itexhip_qgemm_prepack_b", "itexhip_qgemm", "itexhip_qgemm_tile", "itexhip_qgemv", "itexhip_qmatmul", "itexhip_qmatmul_per_row", "itexhip_qmatmul_unpacked", "itexhip_mfma_probe",
-    "itexhip_qgemm_naive",
+    "itexhip_qgemm_naive", "itexhip_qbatch_matmul",
 ]
 
 
@@ -240,3 +240,75 @@ def qgemm_naive(a, a_type, w, transpose_b, M, K, N, scales, bias, ep, out_type, 
     _check(_lib.itexhip_qgemm_naive(_ptr(a), a_type, _ptr(w), int(bool(transpose_b)), _i64(M),
                                     _i64(K), _i64(N), _ptr(scales), _ptr(bias), C.byref(ep),
                                     out_type, _ptr(out), _ptr(stream)))
+
+
+# ---- quantized BatchMatMul -----------------------------------------------------------------------
+BIN_MUL, BIN_ADD = 1, 2
+
+
+class BmmBinary(C.Structure):
+    _fields_ = [("alg", C.c_int), ("data", C.c_void_p), ("batch_stride", C.c_int64 * 4), ("stride_m", C.c_int64),
+                ("stride_n", C.c_int64)]
+
+
+class BmmParams(C.Structure):
+    _fields_ = [("n_batch_dims", C.c_int), ("batch_dims", C.c_int64 * 4), ("x_batch_stride", C.c_int64 * 4),
+                ("y_batch_stride", C.c_int64 * 4), ("M", C.c_int64), ("K", C.c_int64), ("N", C.c_int64),
+                ("adj_x", C.c_int), ("adj_y", C.c_int), ("out_type", C.c_int), ("scale", C.c_float),
+                ("n_binary", C.c_int), ("binary", BmmBinary * 2)]
+
+
+def _broadcast_strides(shape, out_shape):
+    """Row-major element strides of `shape` (right-aligned against out_shape), 0 where it broadcasts."""
+    shape = (1,) * (len(out_shape) - len(shape)) + tuple(shape)
+    strides, st = [], 1
+    for d, o in zip(reversed(shape), reversed(out_shape)):
+        if d != o and d != 1:
+            raise ValueError("shape %r does not broadcast to %r" % (shape, out_shape))
+        strides.append(0 if d == 1 else st)
+        st *= d
+    return strides[::-1]
+
+
+def bmm_params(x_shape, y_shape, adj_x, adj_y, out_type, scale, binary=()):
+    """Shapes, broadcast strides and post-ops of one quantized BatchMatMul call.
+    binary: sequence of (BIN_MUL | BIN_ADD, device buffer, shape); returns (params, output shape)."""
+    xm = tuple(x_shape[-2:][::-1]) if adj_x else tuple(x_shape[-2:])
+    ym = tuple(y_shape[-2:][::-1]) if adj_y else tuple(y_shape[-2:])
+    if xm[1] != ym[0]:
+        raise ValueError("inner dimensions differ")
+    xb, yb = tuple(x_shape[:-2]), tuple(y_shape[:-2])
+    nb = max(len(xb), len(yb))
+    xb, yb = (1,) * (nb - len(xb)) + xb, (1,) * (nb - len(yb)) + yb
+    batch = tuple(max(a, b) if 0 not in (a, b) else 0 for a, b in zip(xb, yb))
+    if nb > 4:
+        raise ValueError("at most 4 batch dimensions")
+    p = BmmParams()
+    p.n_batch_dims = nb
+    p.M, p.K, p.N = xm[0], xm[1], ym[1]
+    xs = _broadcast_strides(xb + (1,), batch + (1,))[:-1]
+    ys = _broadcast_strides(yb + (1,), batch + (1,))[:-1]
+    for d in range(nb):
+        p.batch_dims[d] = batch[d]
+        p.x_batch_stride[d] = xs[d] * xm[0] * xm[1]
+        p.y_batch_stride[d] = ys[d] * ym[0] * ym[1]
+    p.adj_x, p.adj_y, p.out_type, p.scale = int(bool(adj_x)), int(bool(adj_y)), out_type, scale
+    out_shape = batch + (xm[0], ym[1])
+    p.n_binary = len(binary)
+    for i, (alg, buf, shape) in enumerate(binary):
+        n_el = 1
+        for d in shape:
+            n_el *= d
+        st = [0] * len(out_shape) if n_el == 1 else _broadcast_strides(tuple(shape), out_shape)
+        if n_el != 1 and len(shape) != len(out_shape):
+            raise ValueError("a binary operand has one element or the output's rank")
+        p.binary[i].alg = alg
+        p.binary[i].data = _ptr(buf).value
+        for d in range(nb):
+            p.binary[i].batch_stride[d] = st[d]
+        p.binary[i].stride_m, p.binary[i].stride_n = st[nb], st[nb + 1]
+    return p, out_shape
+
+
+def qbatch_matmul(p, x, y, out, stream=0):
+    _check(_lib.itexhip_qbatch_matmul(C.byref(p), _ptr(x), _ptr(y), _ptr(out), _ptr(stream)))

@@ -653,3 +653,89 @@ int orc_qmatmul(const orc_matmul_attrs* at, const void* a, const int8_t* w, int 
   free(acc); free(colsum); free(scales); free(sb);
   return st;
 }
+
+
+/* ---- quantized BatchMatMul ---------------------------------------------------------------------- */
+int orc_qbatch_matmul(const int8_t* x, int x_rank, const int64_t* x_dims, const int8_t* y, int y_rank,
+                      const int64_t* y_dims, int adj_x, int adj_y, float min_x, float max_x,
+                      float min_y, float max_y, int n_binary, const orc_bmm_binary* bin, int t_out,
+                      void* out, int out_rank, const int64_t* out_dims) {
+  if (x_rank < 2 || y_rank < 2 || x_rank > 8 || y_rank > 8) return ORC_INVALID_ARGUMENT;
+  if (t_out != ORC_FLOAT && t_out != ORC_BFLOAT16 && t_out != ORC_HALF) return ORC_INVALID_ARGUMENT;
+  if (n_binary < 0 || n_binary > 2) return ORC_UNIMPLEMENTED; /* kMaxBinaryNum_, :434 */
+  /* matrix dimensions, :111-125 */
+  int64_t d0 = x_dims[x_rank - 2], d1 = x_dims[x_rank - 1];
+  int64_t d2 = y_dims[y_rank - 2], d3 = y_dims[y_rank - 1];
+  if (adj_x) { int64_t t = d0; d0 = d1; d1 = t; }
+  if (adj_y) { int64_t t = d2; d2 = d3; d3 = t; }
+  if (d1 != d2) return ORC_INVALID_ARGUMENT;
+  const int64_t M = d0, K = d1, N = d3;
+  /* batch broadcast (MatMulBCast, :105-109): right-aligned, equal or 1 */
+  const int nbx = x_rank - 2, nby = y_rank - 2, nbo = nbx > nby ? nbx : nby;
+  if (out_rank != nbo + 2 || out_dims[nbo] != M || out_dims[nbo + 1] != N) return ORC_INVALID_ARGUMENT;
+  int64_t xs[8] = {0}, ys[8] = {0}; /* element strides of the batch dims in x / y, 0 = broadcast */
+  {
+    int64_t sx = d0 * d1, sy = d2 * d3;
+    for (int i = nbo - 1; i >= 0; --i) {
+      const int ix = i - (nbo - nbx), iy = i - (nbo - nby);
+      const int64_t dx = ix >= 0 ? x_dims[ix] : 1, dy = iy >= 0 ? y_dims[iy] : 1;
+      if (dx != dy && dx != 1 && dy != 1) return ORC_INVALID_ARGUMENT;
+      if (out_dims[i] != (dx == 1 ? dy : dx)) return ORC_INVALID_ARGUMENT;
+      xs[i] = dx == 1 ? 0 : sx;
+      ys[i] = dy == 1 ? 0 : sy;
+      sx *= dx; sy *= dy;
+    }
+  }
+  /* binary operands: strides per output dimension */
+  int64_t bs[2][8] = {{0}};
+  for (int b = 0; b < n_binary; ++b) {
+    if (bin[b].alg != ORC_BIN_MUL && bin[b].alg != ORC_BIN_ADD) return ORC_UNIMPLEMENTED;
+    if (bin[b].rank == 0) continue; /* one element */
+    if (bin[b].rank != out_rank) return ORC_INVALID_ARGUMENT;
+    int64_t st = 1;
+    for (int i = out_rank - 1; i >= 0; --i) {
+      if (bin[b].dims[i] != out_dims[i] && bin[b].dims[i] != 1) return ORC_INVALID_ARGUMENT;
+      bs[b][i] = bin[b].dims[i] == 1 ? 0 : st;
+      st *= bin[b].dims[i];
+    }
+  }
+  /* output scale, :507-514 (mul_value starts at 1) */
+  const float range_lhs = fmaxf(fabsf(min_x), fabsf(max_x));
+  const float range_rhs = fmaxf(fabsf(min_y), fabsf(max_y));
+  const float scale_output = range_lhs * range_rhs / (127.0f * 127.0f);
+  const float scale = 1.0f * scale_output;
+
+  int64_t batch = 1;
+  for (int i = 0; i < nbo; ++i) batch *= out_dims[i];
+  if (batch == 0 || M == 0 || N == 0) return ORC_OK;
+#pragma omp parallel for collapse(2) schedule(static)
+  for (int64_t bi = 0; bi < batch; ++bi) {
+    for (int64_t m = 0; m < M; ++m) {
+      int64_t idx[8], rem = bi, xo = 0, yo = 0, bo[2] = {0, 0};
+      for (int i = nbo - 1; i >= 0; --i) { idx[i] = rem % out_dims[i]; rem /= out_dims[i]; }
+      for (int i = 0; i < nbo; ++i) {
+        xo += idx[i] * xs[i]; yo += idx[i] * ys[i];
+        for (int b = 0; b < n_binary; ++b) bo[b] += idx[i] * bs[b][i];
+      }
+      for (int64_t n = 0; n < N; ++n) {
+        int32_t acc = 0;
+        for (int64_t k = 0; k < K; ++k) {
+          const int32_t xv = adj_x ? x[xo + k * M + m] : x[xo + m * K + k];
+          const int32_t yv = adj_y ? y[yo + n * K + k] : y[yo + k * N + n];
+          acc += xv * yv;
+        }
+        float v = (float)acc * scale;
+        for (int b = 0; b < n_binary; ++b) {
+          const int64_t o = bo[b] + m * bs[b][nbo] + n * bs[b][nbo + 1];
+          const float t = t_out == ORC_FLOAT ? ((const float*)bin[b].data)[o]
+                                             : bits16_to_f32(t_out, ((const uint16_t*)bin[b].data)[o]);
+          v = bin[b].alg == ORC_BIN_MUL ? v * t : v + t;
+        }
+        const int64_t oo = (bi * M + m) * N + n;
+        if (t_out == ORC_FLOAT) ((float*)out)[oo] = v;
+        else ((uint16_t*)out)[oo] = f32_to_bits16(t_out, v);
+      }
+    }
+  }
+  return ORC_OK;
+}

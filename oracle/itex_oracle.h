@@ -128,6 +128,29 @@ int orc_qmatmul(const orc_matmul_attrs* at, const void* a, const int8_t* w, int 
                 float max_a, const float* min_b, const float* max_b, int64_t nb, float min_out,
                 float max_out, void* out);
 
+/*
+ * Quantized BatchMatMul, qint8 x qint8 -> float / bfloat16 / half
+ * (itex/core/kernels/common/batch_matmul_op.h: Init :88-273, GetPrimitiveDesc :361-419,
+ *  QuantizedBatchMatMulV2Op::AccumulateMulAndInt8Scale :497-515).
+ * x: [..., M, K] (or [..., K, M] with adj_x), y: [..., K, N] (or [..., N, K] with adj_y); the leading
+ * dimensions broadcast against each other (MatMulBCast).  Each binary operand is a tensor of the
+ * OUTPUT element type with one element, or with the rank of the output and every dimension equal to
+ * the output's or 1 (oneDNN binary post-op broadcast).
+ * Pinned by: brute force in numpy int64 / float32; the three cases of the reference's
+ * quantized_batch_matmul_test.py at its own tolerance; linearity / broadcast identities.
+ */
+enum { ORC_BIN_MUL = 1, ORC_BIN_ADD = 2 };
+typedef struct {
+  int alg;            /* ORC_BIN_MUL | ORC_BIN_ADD */
+  const void* data;   /* elements of the output type */
+  int rank;           /* 0 (one element) or the output's rank */
+  int64_t dims[8];
+} orc_bmm_binary;
+int orc_qbatch_matmul(const int8_t* x, int x_rank, const int64_t* x_dims, const int8_t* y, int y_rank,
+                      const int64_t* y_dims, int adj_x, int adj_y, float min_x, float max_x,
+                      float min_y, float max_y, int n_binary, const orc_bmm_binary* bin, int t_out,
+                      void* out, int out_rank, const int64_t* out_dims);
+
 #ifdef __cplusplus
 }
 #endif

@@ -238,3 +238,42 @@ def qmatmul(at, a, w, bias, min_a, max_a, min_b, max_b, min_out=0.0, max_out=0.0
                            _p(max_b), C.c_int64(min_b.size), C.c_float(min_out), C.c_float(max_out),
                            _p(out))
     return st, out
+
+
+class BmmBinary(C.Structure):
+    _fields_ = [("alg", C.c_int), ("data", C.c_void_p), ("rank", C.c_int), ("dims", C.c_int64 * 8)]
+
+
+BIN_MUL, BIN_ADD = 1, 2
+
+
+def qbatch_matmul(x, y, min_x, max_x, min_y, max_y, adj_x=False, adj_y=False, binary=(), t_out=FLOAT):
+    """binary: sequence of (BIN_MUL | BIN_ADD, array); 16-bit operands are uint16 bit patterns.  Returns (status, out)."""
+    x = np.ascontiguousarray(x, dtype=np.int8)
+    y = np.ascontiguousarray(y, dtype=np.int8)
+    xm = x.shape[-2:][::-1] if adj_x else x.shape[-2:]
+    ym = y.shape[-2:][::-1] if adj_y else y.shape[-2:]
+    try:
+        batch = np.broadcast_shapes(x.shape[:-2], y.shape[:-2])
+    except ValueError:
+        return INVALID_ARGUMENT, None
+    oshape = tuple(batch) + (xm[0], ym[1])
+    out = np.zeros(oshape, NP_OF[t_out])
+    bins = (BmmBinary * max(len(binary), 1))()
+    keep = []
+    for i, (alg, arr) in enumerate(binary):
+        arr = np.ascontiguousarray(arr, dtype=np.float32 if t_out == FLOAT else np.uint16)
+        keep.append(arr)
+        bins[i].alg = alg
+        bins[i].data = arr.ctypes.data
+        bins[i].rank = 0 if arr.size == 1 else arr.ndim
+        for d, v in enumerate(arr.shape if arr.size != 1 else ()):
+            bins[i].dims[d] = v
+    xd = (C.c_int64 * 8)(*x.shape)
+    yd = (C.c_int64 * 8)(*y.shape)
+    od = (C.c_int64 * 8)(*oshape)
+    f = lib().orc_qbatch_matmul
+    f.restype = C.c_int
+    st = f(_p(x), x.ndim, xd, _p(y), y.ndim, yd, int(bool(adj_x)), int(bool(adj_y)), C.c_float(min_x), C.c_float(max_x),
+           C.c_float(min_y), C.c_float(max_y), len(binary), bins, t_out, _p(out), len(oshape), od)
+    return st, out
