@@ -252,6 +252,35 @@ def bench_elementwise(torch, hip, timer, n, steps, warmup, dev):
     return out
 
 
+def bench_bmm(torch, hip, timer, steps, warmup, dev):
+    """The two quantized BatchMatMuls of a BERT-base attention block at the token count of the linears above
+    (32 sequences x 128 tokens, 12 heads of 64): Q.K^T with the 1/sqrt(d) Mul and the mask Add, then P.V.
+    fp32 outputs, so both are bound by the output write; bytes = both int8 operands + the mask + the output."""
+    B, H, S, D = 32, 12, 128, 64
+    g = torch.Generator(device=dev)
+    g.manual_seed(40)
+    rnd = lambda *shape: torch.randint(-128, 128, shape, dtype=torch.int8, device=dev, generator=g)
+    q, k, v, pr = rnd(B, H, S, D), rnd(B, H, S, D), rnd(B, H, S, D), rnd(B, H, S, S)
+    mul = torch.tensor([0.125], dtype=torch.float32, device=dev)
+    mask = torch.zeros(B, 1, 1, S, dtype=torch.float32, device=dev)
+    st = _stream(torch)
+    out = []
+    scale = float(6.0 * 6.0 / (127.0 * 127.0))
+    p1, s1 = hip.bmm_params(q.shape, k.shape, False, True, hip.FLOAT, scale,
+                            [(hip.BIN_MUL, mul, (1,)), (hip.BIN_ADD, mask, tuple(mask.shape))])
+    o1 = torch.empty(s1, dtype=torch.float32, device=dev)
+    p2, s2 = hip.bmm_params(pr.shape, v.shape, False, False, hip.FLOAT, scale)
+    o2 = torch.empty(s2, dtype=torch.float32, device=dev)
+    for name, p, a, b, o, nbytes, ops in (
+            ("bmm_qk_t_mul_add", p1, q, k, o1, q.numel() + k.numel() + 4 * mask.numel() + 4 * o1.numel(), 2 * B * H * S * S * D),
+            ("bmm_p_v", p2, pr, v, o2, pr.numel() + v.numel() + 4 * o2.numel(), 2 * B * H * S * S * D)):
+        ms = timer.run(lambda i: hip.qbatch_matmul(p, a, b, o, st), steps, warmup)
+        out.append(dict(name=name, batch=B * H, M=S, K=D if o is o1 else S, N=S if o is o1 else D, us_kernel=ms * 1e3,
+                        bytes=nbytes, ops=ops, gbs=nbytes / (ms * 1e-3) / 1e9, bound="hbm",
+                        frac=nbytes / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS, frac_mfma=ops / (ms * 1e-3) / 1e12 / PEAK_INT8_TOPS))
+    return out
+
+
 def bench_mfma_ceiling(torch, hip, timer, xq, wq, dev):
     """Matrix-pipe-only rate for operand bits like the workload's (bytes of the quantized activations,
     sign-flipped as the kernel feeds them, and of the weights) and for constant operands."""
@@ -294,14 +323,14 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--only", type=str, default="", help="comma list of: headline, prefill, bert, gemv, elementwise, copy")
+    ap.add_argument("--only", type=str, default="", help="comma list of: headline, prefill, bert, bmm, gemv, elementwise, copy")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-rows", type=int, default=2048, help="rows of the headline workload the CPU oracle runs")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU only: this build has no multi-GPU path (--gpus must be 1)", file=sys.stderr)
         sys.exit(2)
-    only = set(s for s in args.only.split(",") if s) or {"headline", "prefill", "bert", "gemv", "elementwise"}
+    only = set(s for s in args.only.split(",") if s) or {"headline", "prefill", "bert", "bmm", "gemv", "elementwise"}
 
     torch, hip = _setup()
     dev = torch.device("cuda:0")
@@ -351,6 +380,8 @@ def main():
             r.update(name="bert_linear", bound="max(mfma,hbm)", frac=t_roof / (r["us_kernel"] * 1e-6),
                      frac_mfma=r["tops_kernel"] / PEAK_INT8_TOPS, frac_hbm=r["gbs_kernel"] / PEAK_HBM_GBS)
             others.append(r)
+    if "bmm" in only:
+        others.extend(bench_bmm(torch, hip, timer, K_steps, W, dev))
     if "gemv" in only:
         for (k, n) in ((4096, 14336), (14336, 4096)):
             for m in (1, 4, 16):
@@ -397,7 +428,7 @@ def main():
         "dtype": "s8/u8 x s8 -> s32 (fp32 epilogue)", "data": "synthetic",
         "config": {"workload": "Llama-3-8B prefill linear M=2048 K=4096 N=14336: quint8 act (MIN_FIRST, N(0,1) + 0.1% x20 "
                                "outliers) x qint8 per-channel weights, _QuantizedMatMul [BiasAdd, Requantize] -> qint8; "
-                               "step = param-prep kernel + MFMA GEMM kernel"},
+                               "step = one launch of the op (the kernel derives scales and bias itself)"},
         "roofline": {"bound": "mfma", "achieved": head["tops_kernel"], "peak": PEAK_INT8_TOPS, "unit": "TFLOP/s",
                      "frac": head["tops_kernel"] / PEAK_INT8_TOPS, "traffic": traffic,
                      "kernel": "qgemm_tile_kernel", "us_per_launch": head["us_kernel"],

@@ -157,6 +157,7 @@ void RegisterKernels(const char* device_type);
 void AddQuantizeKernels();
 void AddDequantizeKernels();
 void AddQuantizedMatMulKernels();
+void AddQuantizedBatchMatMulKernels();
 void AddRequantizeKernels();
 // op definitions for the ops stock TensorFlow does not have
 void RegisterOps();

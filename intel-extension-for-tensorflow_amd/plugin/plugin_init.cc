@@ -126,7 +126,33 @@ std::vector<OpSpec> OpSpecs() {
     v.push_back(plain);
     v.push_back(req);
     v.push_back(deq);
+    // quantized BatchMatMul, nn_ops.cc:497-560 and :3881-3945
+    const std::vector<const char*> bmm_attrs = {"T1: quantizedtype", "T2: quantizedtype",
+                                                "Toutput: {bfloat16, half, float} = DT_FLOAT", "adj_x: bool = false",
+                                                "adj_y: bool = false", "is_filter_const: bool = false"};
+    OpSpec bmm{nm("QuantizedBatchMatMulV2AndDequantize"),
+               {"x: T1", "y: T2", "min_x: float", "max_x: float", "min_y: float", "max_y: float"},
+               {"output: Toutput"}, bmm_attrs};
+    OpSpec fbmm{nm("QuantizedFusedBatchMatMulV2AndDequantize"),
+                {"x: T1", "y: T2", "args: num_args * T", "min_x: float", "max_x: float", "min_y: float", "max_y: float"},
+                {"output: Toutput"}, bmm_attrs};
+    fbmm.attrs.push_back("T: {bfloat16, half, float} = DT_FLOAT");
+    fbmm.attrs.push_back("num_args: int >= 0");
+    fbmm.attrs.push_back("fused_ops: list(string) = []");
+    v.push_back(bmm);
+    v.push_back(fbmm);
   }
+  // nn_ops.cc:4636-4691
+  for (const char* name : {"_QuantizedBatchMatMul", "_ITEXQuantizedBatchMatMul"})
+    v.push_back({name,
+                 {"device_inputs: Tdevice_inputs", "host_inputs: Thost_inputs"},
+                 {"device_outputs: Tdevice_outputs", "host_outputs: Thost_outputs"},
+                 {"Tdevice_inputs: list(type) >= 0 = []", "Thost_inputs: list(type) >= 0 = []",
+                  "Tdevice_outputs: list(type) >= 0 = []", "Thost_outputs: list(type) >= 0 = []",
+                  "T1: quantizedtype", "T2: quantizedtype", "U: {bfloat16, float, quantizedtype} = DT_FLOAT",
+                  "Tout: {bfloat16, float, quantizedtype} = DT_FLOAT", "adj_x: bool = false", "adj_y: bool = false",
+                  "fused_ops: list(string) = []", "input_quant_mode: {'MIN_FIRST', 'SCALED'} = 'SCALED'",
+                  "output_quant_mode: {'MIN_FIRST', 'SCALED'} = 'SCALED'"}});
   return v;
 }
 
@@ -159,6 +185,7 @@ extern "C" void TF_InitKernel(void) {
     AddQuantizeKernels();
     AddDequantizeKernels();
     AddQuantizedMatMulKernels();
+    AddQuantizedBatchMatMulKernels();
     AddRequantizeKernels();
     // the device type the kernels attach to: ITEX's own PluggableDevice type by default, so that graphs
     // placed by ITEX's passes keep their device strings

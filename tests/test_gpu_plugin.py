@@ -477,3 +477,86 @@ def test_bfloat16_output_and_bias_through_plugin(rt, dev, op, M, K, N, T16):
                        is_bias_const=True, input_quant_mode="MIN_FIRST", leakyrelu_alpha=0.2))
     assert bad.code == tf.UNIMPLEMENTED
     bad.close()
+
+
+@pytest.mark.parametrize("api", ["V1", "V2"])
+@pytest.mark.parametrize("case", ["plain", "mul", "mul_add"])
+def test_reference_batch_matmul_cases_through_plugin(rt, dev, golden, api, case):
+    """_testQuantizeBMM / _testQuantizeBMMMul / _testQuantizeBMMMulAdd of the reference's
+    quantized_batch_matmul_test.py in both spellings: within its tolerance of the fp32 graph, bit-equal to the oracle."""
+    torch = rt
+    g = golden["batch_matmul"]
+    x, y, add = (np.array(g[k], np.float32) for k in ("x", "y", "add"))
+    mul = np.array(g["mul"], np.float32)                       # a scalar tensor, as in the reference test
+    _, xq, xmn, xmx = orc.quantize_v2(x, x.min(), x.max(), orc.QINT8, orc.SCALED)
+    _, yq, ymn, ymx = orc.quantize_v2(y, y.min(), y.max(), orc.QINT8, orc.SCALED)
+    args = {"plain": [], "mul": [mul], "mul_add": [mul, add]}[case]
+    fused = {"plain": [], "mul": ["Mul"], "mul_add": ["Mul", "Add"]}[case]
+    if api == "V1" and not args:
+        node = tf.Node("_QuantizedBatchMatMulV2AndDequantize",
+                       dict(T1=DT(tf.QINT8), T2=DT(tf.QINT8), Toutput=DT(tf.FLOAT), adj_x=False, adj_y=False, is_filter_const=False))
+    elif api == "V1":
+        node = tf.Node("_QuantizedFusedBatchMatMulV2AndDequantize",
+                       dict(T1=DT(tf.QINT8), T2=DT(tf.QINT8), T=DT(tf.FLOAT), Toutput=DT(tf.FLOAT), adj_x=False, adj_y=False,
+                            num_args=len(args), fused_ops=fused, is_filter_const=False))
+    else:
+        node = tf.Node("_QuantizedBatchMatMul",
+                       dict(T1=DT(tf.QINT8), T2=DT(tf.QINT8), U=DT(tf.FLOAT), Tout=DT(tf.FLOAT), adj_x=False, adj_y=False,
+                            fused_ops=fused + ["Dequantize"], input_quant_mode="SCALED", output_quant_mode="SCALED"))
+    assert node.code == tf.OK, node.message
+    keep = [dev_in(torch, dev, v) for v in [xq, yq] + args]
+    ins = [(tf.QINT8, xq.shape, keep[0].data_ptr(), False), (tf.QINT8, yq.shape, keep[1].data_ptr(), False)]
+    for a, k in zip(args, keep[2:]):
+        ins.append((tf.FLOAT, a.shape, k.data_ptr(), False))
+    scal = [np.array(v[0], np.float32) for v in (xmn, xmx, ymn, ymx)]
+    for s in scal:
+        ins.append((tf.FLOAT, (), tf.host_array(s), True))
+    code, msg, outs = node.run(ins, [(tf.FLOAT, False)], stream=torch.cuda.current_stream().cuda_stream)
+    assert code == tf.OK, msg
+    got = fetch(torch, outs[0], np.float32)
+    ref32 = x @ y
+    if args:
+        ref32 = ref32 * mul
+    if len(args) == 2:
+        ref32 = ref32 + add
+    np.testing.assert_allclose(got, ref32, rtol=g["tolerance"], atol=g["tolerance"])
+    binary = [(orc.BIN_MUL, mul.reshape(1)), (orc.BIN_ADD, add)][:len(args)]
+    st, ref = orc.qbatch_matmul(xq, yq, xmn[0], xmx[0], ymn[0], ymx[0], binary=binary)
+    assert st == orc.OK
+    np.testing.assert_array_equal(got, ref)
+    node.close()
+
+
+def test_batch_matmul_attention_through_plugin(rt, dev):
+    """adj_y, broadcast batch dimensions of the mask, bfloat16 output with bfloat16 operands."""
+    torch = rt
+    rng = np.random.default_rng(2)
+    B, H, S, D = 2, 3, 80, 64
+    q = rng.integers(-128, 128, (B, H, S, D)).astype(np.int8)
+    k = rng.integers(-128, 128, (B, H, S, D)).astype(np.int8)
+    mask = torch.from_numpy(np.where(rng.random((B, 1, 1, S)) < 0.3, -10000.0, 0.0).astype(np.float32)).to(torch.bfloat16)
+    mul = torch.tensor([0.125], dtype=torch.bfloat16)
+    node = tf.Node("_QuantizedBatchMatMul",
+                   dict(T1=DT(tf.QINT8), T2=DT(tf.QINT8), U=DT(tf.BFLOAT16), Tout=DT(tf.BFLOAT16), adj_x=False, adj_y=True,
+                        fused_ops=["Mul", "Add", "Dequantize"], input_quant_mode="SCALED", output_quant_mode="SCALED"))
+    assert node.code == tf.OK, node.message
+    keep = [dev_in(torch, dev, q), dev_in(torch, dev, k), mul.to(dev), mask.to(dev)]
+    ins = [(tf.QINT8, q.shape, keep[0].data_ptr(), False), (tf.QINT8, k.shape, keep[1].data_ptr(), False),
+           (tf.BFLOAT16, (1,), keep[2].data_ptr(), False), (tf.BFLOAT16, tuple(mask.shape), keep[3].data_ptr(), False)]
+    scal = [np.array(s, np.float32) for s in (-4.0, 3.5, -2.0, 2.5)]   # kept alive: the node reads their memory
+    for s in scal:
+        ins.append((tf.FLOAT, (), tf.host_array(s), True))
+    code, msg, outs = node.run(ins, [(tf.BFLOAT16, False)], stream=torch.cuda.current_stream().cuda_stream)
+    assert code == tf.OK, msg
+    bits = lambda t: t.view(torch.int16).numpy().view(np.uint16)
+    st, ref = orc.qbatch_matmul(q, k, -4.0, 3.5, -2.0, 2.5, adj_y=True,
+                                binary=((orc.BIN_MUL, bits(mul)), (orc.BIN_ADD, bits(mask))), t_out=orc.BFLOAT16)
+    assert st == orc.OK
+    np.testing.assert_array_equal(fetch(torch, outs[0], np.int16).view(np.uint16), ref)
+    node.close()
+    # an activation is not a fusion this op knows
+    bad = tf.Node("_QuantizedBatchMatMul",
+                  dict(T1=DT(tf.QINT8), T2=DT(tf.QINT8), U=DT(tf.FLOAT), Tout=DT(tf.FLOAT), adj_x=False, adj_y=False,
+                       fused_ops=["Relu", "Dequantize"], input_quant_mode="SCALED", output_quant_mode="SCALED"))
+    assert bad.code == tf.UNIMPLEMENTED and "Fusion is not implemented" in bad.message
+    bad.close()

@@ -176,3 +176,16 @@ def test_se_init_plugin_without_a_gpu():
         assert rc == 0, plug.error()
     else:
         assert rc == 4, (rc, plug.error())
+
+
+def test_batch_matmul_registrations(reg):
+    for op, out_attr, host in (("_QuantizedBatchMatMulV2AndDequantize", "Toutput", ["min_x", "max_x", "min_y", "max_y"]),
+                               ("_QuantizedFusedBatchMatMulV2AndDequantize", "Toutput", ["min_x", "max_x", "min_y", "max_y"]),
+                               ("_QuantizedBatchMatMul", "Tout", ["host_inputs", "host_outputs"])):
+        ks = kernels_of(reg, op)
+        assert {k["constraints"][out_attr] for k in ks} == {tf.FLOAT, tf.BFLOAT16, tf.HALF}
+        assert all(k["constraints"]["T1"] == tf.QINT8 and k["constraints"]["T2"] == tf.QINT8 and k["host_memory"] == host
+                   for k in ks)
+    names = {o["name"] for o in reg["ops"]}
+    assert {"_QuantizedBatchMatMul", "_QuantizedBatchMatMulV2AndDequantize", "_QuantizedFusedBatchMatMulV2AndDequantize",
+            "_ITEXQuantizedBatchMatMulV2AndDequantize"} <= names
