@@ -253,31 +253,38 @@ def bench_elementwise(torch, hip, timer, n, steps, warmup, dev):
 
 
 def bench_bmm(torch, hip, timer, steps, warmup, dev):
-    """The two quantized BatchMatMuls of a BERT-base attention block at the token count of the linears above
-    (32 sequences x 128 tokens, 12 heads of 64): Q.K^T with the 1/sqrt(d) Mul and the mask Add, then P.V.
-    fp32 outputs, so both are bound by the output write; bytes = both int8 operands + the mask + the output."""
-    B, H, S, D = 32, 12, 128, 64
+    """The two quantized BatchMatMuls of a BERT-base attention block (12 heads of 64, 128 tokens): Q.K^T with the
+    1/sqrt(d) Mul and the mask Add, then P.V.  fp32 outputs, so both are bound by the output write;
+    bytes = both int8 operands + the mask + the output.  Two batch sizes: 32 sequences (the token count of the
+    linears above; ~30 MB per launch, where the fixed cost of a launch is about half of the time) and 128 sequences
+    (the sustained rate)."""
+    H, S, D = 12, 128, 64
     g = torch.Generator(device=dev)
     g.manual_seed(40)
     rnd = lambda *shape: torch.randint(-128, 128, shape, dtype=torch.int8, device=dev, generator=g)
-    q, k, v, pr = rnd(B, H, S, D), rnd(B, H, S, D), rnd(B, H, S, D), rnd(B, H, S, S)
-    mul = torch.tensor([0.125], dtype=torch.float32, device=dev)
-    mask = torch.zeros(B, 1, 1, S, dtype=torch.float32, device=dev)
     st = _stream(torch)
     out = []
     scale = float(6.0 * 6.0 / (127.0 * 127.0))
-    p1, s1 = hip.bmm_params(q.shape, k.shape, False, True, hip.FLOAT, scale,
-                            [(hip.BIN_MUL, mul, (1,)), (hip.BIN_ADD, mask, tuple(mask.shape))])
-    o1 = torch.empty(s1, dtype=torch.float32, device=dev)
-    p2, s2 = hip.bmm_params(pr.shape, v.shape, False, False, hip.FLOAT, scale)
-    o2 = torch.empty(s2, dtype=torch.float32, device=dev)
-    for name, p, a, b, o, nbytes, ops in (
-            ("bmm_qk_t_mul_add", p1, q, k, o1, q.numel() + k.numel() + 4 * mask.numel() + 4 * o1.numel(), 2 * B * H * S * S * D),
-            ("bmm_p_v", p2, pr, v, o2, pr.numel() + v.numel() + 4 * o2.numel(), 2 * B * H * S * S * D)):
-        ms = timer.run(lambda i: hip.qbatch_matmul(p, a, b, o, st), steps, warmup)
-        out.append(dict(name=name, batch=B * H, M=S, K=D if o is o1 else S, N=S if o is o1 else D, us_kernel=ms * 1e3,
-                        bytes=nbytes, ops=ops, gbs=nbytes / (ms * 1e-3) / 1e9, bound="hbm",
-                        frac=nbytes / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS, frac_mfma=ops / (ms * 1e-3) / 1e12 / PEAK_INT8_TOPS))
+    for B in (32, 128):
+        q, k, v, pr = rnd(B, H, S, D), rnd(B, H, S, D), rnd(B, H, S, D), rnd(B, H, S, S)
+        mul = torch.tensor([0.125], dtype=torch.float32, device=dev)
+        mask = torch.zeros(B, 1, 1, S, dtype=torch.float32, device=dev)
+        p1, s1 = hip.bmm_params(q.shape, k.shape, False, True, hip.FLOAT, scale,
+                                [(hip.BIN_MUL, mul, (1,)), (hip.BIN_ADD, mask, tuple(mask.shape))])
+        o1 = torch.empty(s1, dtype=torch.float32, device=dev)
+        p2, s2 = hip.bmm_params(pr.shape, v.shape, False, False, hip.FLOAT, scale)
+        o2 = torch.empty(s2, dtype=torch.float32, device=dev)
+        for name, p, a, b, o, nbytes, ops in (
+                ("bmm_qk_t_mul_add", p1, q, k, o1, q.numel() + k.numel() + 4 * mask.numel() + 4 * o1.numel(), 2 * B * H * S * S * D),
+                ("bmm_p_v", p2, pr, v, o2, pr.numel() + v.numel() + 4 * o2.numel(), 2 * B * H * S * S * D)):
+            ms_eager = timer.run(lambda i: hip.qbatch_matmul(p, a, b, o, st), steps, warmup)
+            # launches captured in a HIP graph: the host's launch rate leaves the measurement
+            ms = timer.run_graph(lambda stream: (lambda i: hip.qbatch_matmul(p, a, b, o, stream)), steps, warmup)
+            out.append(dict(name=name, batch=B * H, M=S, K=D if o is o1 else S, N=S if o is o1 else D, us_kernel=ms * 1e3,
+                            us_eager=ms_eager * 1e3, bytes=nbytes, ops=ops, gbs=nbytes / (ms * 1e-3) / 1e9, bound="hbm",
+                            frac=nbytes / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS,
+                            frac_mfma=ops / (ms * 1e-3) / 1e12 / PEAK_INT8_TOPS))
+        del q, k, v, pr, o1, o2
     return out
 
 

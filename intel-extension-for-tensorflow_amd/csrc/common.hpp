@@ -68,6 +68,9 @@ __device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
 
 // fp32 <-> half bit patterns (v_cvt_f16_f32 / v_cvt_f32_f16: round to nearest even, denormals kept)
 __device__ __forceinline__ uint32_t f32_to_f16_bits(float f) {
+  // The value must exist as a rounded fp32 number before it is narrowed: without this the compiler may merge
+  // the producing multiply / add with the conversion into one mixed-precision instruction that rounds once.
+  asm("" : "+v"(f));
   const _Float16 h = static_cast<_Float16>(f);
   unsigned short bits;
   __builtin_memcpy(&bits, &h, 2);

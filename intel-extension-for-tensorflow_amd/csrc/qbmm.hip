@@ -9,6 +9,8 @@
 // adj_y) is transposed on the way into LDS, four bytes at a time.  The output orientation keeps
 // n on the lanes, so every store instruction writes 128 contiguous bytes per half-wavefront: with fp32
 // outputs the op is bound by that write.
+#include <type_traits>
+
 #include "common.hpp"
 
 namespace itexhip {
@@ -27,101 +29,149 @@ struct BmmArgs {
   int vec_x, vec_y;  // operand layouts allow aligned vector loads
 };
 
-// One 64 (rows or columns of the output) x 64 (k) byte tile into LDS, k-contiguous.
-//   KCONT: the operand is stored [R, K] (k fastest);  else [K, R] (r fastest) and is transposed here.
+// One 64 (rows or columns of the output) x 64 (k) byte tile on its way into LDS, k-contiguous there.  The
+// global loads (fetch_tile) and the LDS stores (put_tile) are separate so that the next tile's loads are in
+// flight while the current one is multiplied.
+//   KCONT: the operand is stored [R, K] (k fastest);  else [K, R] (r fastest) and is transposed in put_tile.
 //   VEC:   aligned 16-byte (KCONT) / 4-byte (transposed) global loads are legal and never straddle a bound.
 template <bool KCONT, bool VEC>
-__device__ __forceinline__ void stage_tile(const int8_t* __restrict__ g, int64_t R, int64_t K, int64_t r0, int64_t k0,
-                                           uint8_t* __restrict__ lds, int t) {
-  if constexpr (KCONT) {
-    const int r = t >> 2, seg = t & 3;
-    const int64_t row = r0 + r, k = k0 + seg * 16;
-    v4i v = {0, 0, 0, 0};
-    if (row < R) {
-      const int8_t* src = g + row * K + k;
-      if constexpr (VEC) {
-        if (k < K) v = *reinterpret_cast<const v4i*>(src);
-      } else {
-        uint32_t w[4] = {0, 0, 0, 0};
-#pragma unroll
-        for (int b = 0; b < 16; ++b)
-          if (k + b < K) w[b >> 2] |= static_cast<uint32_t>(static_cast<uint8_t>(src[b])) << (8 * (b & 3));
-        v = v4i{static_cast<int>(w[0]), static_cast<int>(w[1]), static_cast<int>(w[2]), static_cast<int>(w[3])};
+__device__ __forceinline__ void fetch_tile(const int8_t* __restrict__ g, int64_t R, int64_t K, int64_t r0, int64_t k0,
+                                           int t, uint32_t (&w)[4]) {
+  w[0] = w[1] = w[2] = w[3] = 0;
+  if constexpr (KCONT) {  // thread: row t / 4, 16 consecutive k
+    const int64_t row = r0 + (t >> 2), k = k0 + (t & 3) * 16;
+    if (row >= R) return;
+    const int8_t* src = g + row * K + k;
+    if constexpr (VEC) {
+      if (k < K) {
+        const v4i v = *reinterpret_cast<const v4i*>(src);
+        w[0] = v[0]; w[1] = v[1]; w[2] = v[2]; w[3] = v[3];
       }
+    } else {
+#pragma unroll
+      for (int b = 0; b < 16; ++b)
+        if (k + b < K) w[b >> 2] |= static_cast<uint32_t>(static_cast<uint8_t>(src[b])) << (8 * (b & 3));
     }
-    *reinterpret_cast<v4i*>(lds + r * kLdsStride + seg * 16) = v;
-  } else {
-    // 4 (k) x 4 (r) bytes per thread: kb = t / 16 picks the k rows, cb = t % 16 the r columns
+  } else {  // thread: 4 (k) x 4 (r) bytes; kb = t / 16 picks the k rows, cb = t % 16 the r columns; w[i] = k row i
     const int kb = t >> 4, cb = t & 15;
-    uint32_t rows[4];
+    const int64_t r = r0 + cb * 4;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const int64_t k = k0 + kb * 4 + i, r = r0 + cb * 4;
-      uint32_t w = 0;
-      if (k < K) {
-        const int8_t* src = g + k * R + r;
-        if constexpr (VEC) {
-          if (r < R) w = *reinterpret_cast<const uint32_t*>(src);
-        } else {
+      const int64_t k = k0 + kb * 4 + i;
+      if (k >= K) continue;
+      const int8_t* src = g + k * R + r;
+      if constexpr (VEC) {
+        if (r < R) w[i] = *reinterpret_cast<const uint32_t*>(src);
+      } else {
 #pragma unroll
-          for (int b = 0; b < 4; ++b)
-            if (r + b < R) w |= static_cast<uint32_t>(static_cast<uint8_t>(src[b])) << (8 * b);
-        }
+        for (int b = 0; b < 4; ++b)
+          if (r + b < R) w[i] |= static_cast<uint32_t>(static_cast<uint8_t>(src[b])) << (8 * b);
       }
-      rows[i] = w;
     }
+  }
+}
+
+template <bool KCONT>
+__device__ __forceinline__ void put_tile(uint8_t* __restrict__ lds, int t, const uint32_t (&w)[4]) {
+  if constexpr (KCONT) {
+    *reinterpret_cast<v4i*>(lds + (t >> 2) * kLdsStride + (t & 3) * 16) =
+        v4i{static_cast<int>(w[0]), static_cast<int>(w[1]), static_cast<int>(w[2]), static_cast<int>(w[3])};
+  } else {
+    const int kb = t >> 4, cb = t & 15;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {  // byte j of the four k rows -> four consecutive k of column cb * 4 + j
-      const uint32_t w = ((rows[0] >> (8 * j)) & 0xffu) | (((rows[1] >> (8 * j)) & 0xffu) << 8) |
-                         (((rows[2] >> (8 * j)) & 0xffu) << 16) | (((rows[3] >> (8 * j)) & 0xffu) << 24);
-      *reinterpret_cast<uint32_t*>(lds + (cb * 4 + j) * kLdsStride + kb * 4) = w;
+      const uint32_t v = ((w[0] >> (8 * j)) & 0xffu) | (((w[1] >> (8 * j)) & 0xffu) << 8) |
+                         (((w[2] >> (8 * j)) & 0xffu) << 16) | (((w[3] >> (8 * j)) & 0xffu) << 24);
+      *reinterpret_cast<uint32_t*>(lds + (cb * 4 + j) * kLdsStride + kb * 4) = v;
     }
   }
 }
 
-__device__ __forceinline__ float load_operand(const void* __restrict__ data, int64_t off, int out_type) {
-  if (out_type == ITEXHIP_FLOAT) return static_cast<const float*>(data)[off];
-  const uint32_t bits = static_cast<const uint16_t*>(data)[off];
-  return out_type == ITEXHIP_BFLOAT16 ? bf16_bits_to_f32(bits) : f16_bits_to_f32(bits);
+template <int T>
+__device__ __forceinline__ float widen(float v) { return v; }
+template <int T>
+__device__ __forceinline__ float widen(uint16_t bits) {
+  return T == ITEXHIP_BFLOAT16 ? bf16_bits_to_f32(bits) : f16_bits_to_f32(bits);
 }
 
-template <bool ADJ_X, bool ADJ_Y, bool VEC_X, bool VEC_Y>
-__global__ __launch_bounds__(kBmmThreads) void qbmm_kernel(const BmmArgs a, const int8_t* __restrict__ x,
-                                                           const int8_t* __restrict__ y, void* __restrict__ out) {
-  __shared__ __attribute__((aligned(16))) uint8_t xs[kTile * kLdsStride];
-  __shared__ __attribute__((aligned(16))) uint8_t ys[kTile * kLdsStride];
-  const itexhip_bmm_params& p = a.p;
-  const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
-  const int wm = wave >> 1, wn = wave & 1;
+// Where one wavefront's 32 x 32 quadrant goes.  Everything that is the same for the whole wavefront is a
+// 64-bit base address; what differs between lanes and rows is a 32-bit byte offset (the host bounds N and
+// the operand strides so that 64 rows of them fit), which is the addressing form the hardware takes directly.
+struct QuadrantSite {
+  int rows_left, cols_left;   // of the output below / right of the quadrant's first element
+  float scale;
+  int n_binary;
+  int alg[ITEXHIP_BMM_MAX_BINARY];
+  const char* operand[ITEXHIP_BMM_MAX_BINARY];           // address of the quadrant's first operand element
+  uint32_t operand_row[ITEXHIP_BMM_MAX_BINARY], operand_col[ITEXHIP_BMM_MAX_BINARY];  // byte strides
+  char* out;                                             // address of the quadrant's first output element
+  uint32_t out_row;                                      // byte stride between output rows
+};
 
-  // workgroup -> (batch entry, tile); consecutive workgroups walk the tiles of one matrix
-  const int64_t tiles = static_cast<int64_t>(a.tiles_m) * a.tiles_n;
-  const int64_t bi = blockIdx.x / tiles;
-  const int tile = static_cast<int>(blockIdx.x - bi * tiles);
-  const int64_t m0 = static_cast<int64_t>(tile / a.tiles_n) * kTile, n0 = static_cast<int64_t>(tile % a.tiles_n) * kTile;
-
-  int64_t xo = 0, yo = 0, bo[ITEXHIP_BMM_MAX_BINARY] = {0, 0};
-  {
-    int64_t rem = bi;
-    for (int d = p.n_batch_dims - 1; d >= 0; --d) {
-      const int64_t i = rem % p.batch_dims[d];
-      rem /= p.batch_dims[d];
-      xo += i * p.x_batch_stride[d];
-      yo += i * p.y_batch_stride[d];
-      for (int b = 0; b < p.n_binary; ++b) bo[b] += i * p.binary[b].batch_stride[d];
+// Operand values of the lane's 16 results.  Straight-line code: every load is issued whatever the operand's
+// broadcast pattern (rows and columns outside the output read element (0, 0) of the quadrant instead), so that
+// nothing forces a wait before the tiles arrive.
+template <int OUT_T, int NB>
+__device__ __forceinline__ void fetch_operands(const QuadrantSite& s, int lane, float (&o)[ITEXHIP_BMM_MAX_BINARY][16]) {
+  using elem_t = typename std::conditional<OUT_T == ITEXHIP_FLOAT, float, uint16_t>::type;
+  const uint32_t lrow = (lane >> 5) * 4;
+  const uint32_t lcol = static_cast<int>(lane & 31) < s.cols_left ? (lane & 31) : 0;
+#pragma unroll
+  for (int b = 0; b < NB; ++b) {
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const uint32_t row = lrow + (i >> 2) * 8 + (i & 3);
+      const uint32_t off = (static_cast<int>(row) < s.rows_left ? row : 0) * s.operand_row[b] + lcol * s.operand_col[b];
+      o[b][i] = widen<OUT_T>(*reinterpret_cast<const elem_t*>(s.operand[b] + off));
     }
   }
-  const int8_t* xb = x + xo;
-  const int8_t* yb = y + yo;
+}
+
+template <int OUT_T, int NB>
+__device__ __forceinline__ void store_quadrant(const v16i& acc, const QuadrantSite& s, int lane,
+                                               const float (&o)[ITEXHIP_BMM_MAX_BINARY][16]) {
+  using elem_t = typename std::conditional<OUT_T == ITEXHIP_FLOAT, float, uint16_t>::type;
+  const uint32_t lrow = (lane >> 5) * 4, lcol = lane & 31;
+  if (static_cast<int>(lcol) >= s.cols_left) return;
+  const uint32_t obase = lrow * s.out_row + lcol * static_cast<uint32_t>(sizeof(elem_t));
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    const int r = (i >> 2) * 8 + (i & 3);
+    if (static_cast<int>(lrow) + r >= s.rows_left) continue;
+    float v = static_cast<float>(acc[i]) * s.scale;
+    if constexpr (NB > 0) v = s.alg[0] == ITEXHIP_BIN_MUL ? v * o[0][i] : v + o[0][i];
+    if constexpr (NB > 1) v = s.alg[1] == ITEXHIP_BIN_MUL ? v * o[1][i] : v + o[1][i];
+    elem_t* dst = reinterpret_cast<elem_t*>(s.out + (obase + r * s.out_row));
+    if constexpr (OUT_T == ITEXHIP_FLOAT) *dst = v;
+    else *dst = static_cast<uint16_t>(f32_to_bits16<OUT_T>(v));
+  }
+}
+
+// What a workgroup does once it knows where its operands and results are; one straight-line instance per
+// (number of fused operands, output type).
+template <bool ADJ_X, bool ADJ_Y, bool VEC_X, bool VEC_Y, int NB, int OUT_T>
+__device__ __forceinline__ void bmm_body(const itexhip_bmm_params& p, const int8_t* __restrict__ xb,
+                                         const int8_t* __restrict__ yb, int m0, int n0, int wm, int wn, int t, int lane,
+                                         const QuadrantSite& s, uint8_t* __restrict__ xs, uint8_t* __restrict__ ys) {
+  // first tiles and the fused operands: all loads the results depend on are issued before any is needed
+  uint32_t wx[4], wy[4];
+  fetch_tile<!ADJ_X, VEC_X>(xb, p.M, p.K, m0, 0, t, wx);  // x is [M, K] unless adj_x
+  fetch_tile<ADJ_Y, VEC_Y>(yb, p.N, p.K, n0, 0, t, wy);   // y is [N, K] only with adj_y
+  float o[ITEXHIP_BMM_MAX_BINARY][16];
+  fetch_operands<OUT_T, NB>(s, lane, o);
 
   v16i acc;
 #pragma unroll
   for (int i = 0; i < 16; ++i) acc[i] = 0;
 
   for (int64_t k0 = 0; k0 < p.K; k0 += kTile) {
-    stage_tile<!ADJ_X, VEC_X>(xb, p.M, p.K, m0, k0, xs, t);  // x is [M, K] unless adj_x
-    stage_tile<ADJ_Y, VEC_Y>(yb, p.N, p.K, n0, k0, ys, t);   // y is [N, K] only with adj_y
+    put_tile<!ADJ_X>(xs, t, wx);
+    put_tile<ADJ_Y>(ys, t, wy);
     __syncthreads();
+    if (k0 + kTile < p.K) {  // the next tile travels while this one is multiplied
+      fetch_tile<!ADJ_X, VEC_X>(xb, p.M, p.K, m0, k0 + kTile, t, wx);
+      fetch_tile<ADJ_Y, VEC_Y>(yb, p.N, p.K, n0, k0 + kTile, t, wy);
+    }
 #pragma unroll
     for (int kk = 0; kk < 2; ++kk) {
       const int off = kk * 32 + (lane >> 5) * 16;
@@ -131,25 +181,75 @@ __global__ __launch_bounds__(kBmmThreads) void qbmm_kernel(const BmmArgs a, cons
     }
     __syncthreads();
   }
+  store_quadrant<OUT_T, NB>(acc, s, lane, o);
+}
 
-  // accumulator i of a lane: row (i / 4) * 8 + (lane / 32) * 4 + i % 4, column lane % 32 of the quadrant
-  const int64_t n = n0 + wn * 32 + (lane & 31);
-  if (n >= p.N) return;
-  const int64_t ob = bi * p.M * p.N;
-#pragma unroll
-  for (int i = 0; i < 16; ++i) {
-    const int64_t m = m0 + wm * 32 + (i >> 2) * 8 + (lane >> 5) * 4 + (i & 3);
-    if (m >= p.M) continue;
-    float v = static_cast<float>(acc[i]) * p.scale;
-    for (int b = 0; b < p.n_binary; ++b) {
-      const float o = load_operand(p.binary[b].data, bo[b] + m * p.binary[b].stride_m + n * p.binary[b].stride_n, p.out_type);
-      v = p.binary[b].alg == ITEXHIP_BIN_MUL ? v * o : v + o;
+template <bool ADJ_X, bool ADJ_Y, bool VEC_X, bool VEC_Y>
+__global__ __launch_bounds__(kBmmThreads) void qbmm_kernel(const BmmArgs a, const int8_t* __restrict__ x,
+                                                           const int8_t* __restrict__ y, void* __restrict__ out) {
+  __shared__ __attribute__((aligned(16))) uint8_t xs[kTile * kLdsStride];
+  __shared__ __attribute__((aligned(16))) uint8_t ys[kTile * kLdsStride];
+  const itexhip_bmm_params& p = a.p;
+  const int t = threadIdx.x, lane = t & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(t >> 6);  // the same for the whole wavefront: keep it scalar
+  const int wm = wave >> 1, wn = wave & 1;
+
+  // workgroup -> (batch entry, tile); consecutive workgroups walk the tiles of one matrix.  The launch
+  // has fewer than 2^31 workgroups, so 32-bit arithmetic covers the decomposition.
+  const uint32_t tiles = static_cast<uint32_t>(a.tiles_m) * static_cast<uint32_t>(a.tiles_n);
+  const uint32_t bi = blockIdx.x / tiles;
+  const uint32_t tile = blockIdx.x - bi * tiles;
+  const int m0 = static_cast<int>(tile / a.tiles_n) * kTile, n0 = static_cast<int>(tile % a.tiles_n) * kTile;
+
+  int64_t xo = 0, yo = 0, bo[ITEXHIP_BMM_MAX_BINARY] = {0, 0};
+  {
+    uint32_t rem = bi;
+    for (int d = p.n_batch_dims - 1; d >= 0; --d) {
+      const uint32_t dim = static_cast<uint32_t>(p.batch_dims[d]);
+      const uint32_t q = d == 0 ? 0 : rem / dim;   // the outermost index needs no division
+      const int64_t i = rem - q * dim;
+      rem = q;
+      xo += i * p.x_batch_stride[d];
+      yo += i * p.y_batch_stride[d];
+      for (int b = 0; b < p.n_binary; ++b) bo[b] += i * p.binary[b].batch_stride[d];
     }
-    const int64_t oo = ob + m * p.N + n;
-    if (p.out_type == ITEXHIP_FLOAT) static_cast<float*>(out)[oo] = v;
-    else if (p.out_type == ITEXHIP_BFLOAT16) static_cast<uint16_t*>(out)[oo] = static_cast<uint16_t>(f32_to_bf16_bits(v));
-    else static_cast<uint16_t*>(out)[oo] = static_cast<uint16_t>(f32_to_f16_bits(v));
   }
+
+  // the quadrant of this wavefront; accumulator i of a lane is row (i / 4) * 8 + (lane / 32) * 4 + i % 4,
+  // column lane % 32 of it.  A quadrant off the edge of the output stores nothing (its wavefront still
+  // helps staging the tiles) and addresses the tile's first element, which always exists.
+  const bool live = m0 + wm * 32 < p.M && n0 + wn * 32 < p.N;
+  const int64_t qm = live ? m0 + wm * 32 : m0, qn = live ? n0 + wn * 32 : n0;
+  const uint32_t esz = p.out_type == ITEXHIP_FLOAT ? 4 : 2;
+  QuadrantSite s;
+  s.rows_left = live ? static_cast<int>(p.M - qm < 32 ? p.M - qm : 32) : 0;
+  s.cols_left = live ? static_cast<int>(p.N - qn < 32 ? p.N - qn : 32) : 0;
+  s.scale = p.scale;
+  s.n_binary = p.n_binary;
+  for (int b = 0; b < ITEXHIP_BMM_MAX_BINARY; ++b) {
+    s.alg[b] = p.binary[b].alg;
+    s.operand[b] = static_cast<const char*>(p.binary[b].data) +
+                   (bo[b] + qm * p.binary[b].stride_m + qn * p.binary[b].stride_n) * esz;
+    s.operand_row[b] = static_cast<uint32_t>(p.binary[b].stride_m) * esz;
+    s.operand_col[b] = static_cast<uint32_t>(p.binary[b].stride_n) * esz;
+  }
+  s.out = static_cast<char*>(out) + ((static_cast<int64_t>(bi) * p.M + qm) * p.N + qn) * esz;
+  s.out_row = static_cast<uint32_t>(p.N) * esz;
+
+#define ITEXHIP_BMM_BODY(NB, T) bmm_body<ADJ_X, ADJ_Y, VEC_X, VEC_Y, NB, T>(p, x + xo, y + yo, m0, n0, wm, wn, t, lane, s, xs, ys)
+  const int variant = p.n_binary * 3 + (p.out_type == ITEXHIP_FLOAT ? 0 : p.out_type == ITEXHIP_BFLOAT16 ? 1 : 2);
+  switch (variant) {
+    case 0: ITEXHIP_BMM_BODY(0, ITEXHIP_FLOAT); break;
+    case 1: ITEXHIP_BMM_BODY(0, ITEXHIP_BFLOAT16); break;
+    case 2: ITEXHIP_BMM_BODY(0, ITEXHIP_HALF); break;
+    case 3: ITEXHIP_BMM_BODY(1, ITEXHIP_FLOAT); break;
+    case 4: ITEXHIP_BMM_BODY(1, ITEXHIP_BFLOAT16); break;
+    case 5: ITEXHIP_BMM_BODY(1, ITEXHIP_HALF); break;
+    case 6: ITEXHIP_BMM_BODY(2, ITEXHIP_FLOAT); break;
+    case 7: ITEXHIP_BMM_BODY(2, ITEXHIP_BFLOAT16); break;
+    default: ITEXHIP_BMM_BODY(2, ITEXHIP_HALF); break;
+  }
+#undef ITEXHIP_BMM_BODY
 }
 
 template <bool ADJ_X, bool ADJ_Y>
@@ -200,8 +300,35 @@ extern "C" int itexhip_qbatch_matmul(const itexhip_bmm_params* p, const int8_t* 
   ITEXHIP_REQUIRE(out != nullptr && aligned(out, p->out_type == ITEXHIP_FLOAT ? 4 : 2), "%s: null or misaligned output", who);
   ITEXHIP_REQUIRE(p->K == 0 || (x != nullptr && y != nullptr), "%s: null operand", who);
 
+  // lane offsets inside a quadrant are 32-bit byte offsets: 64 rows of N (or of an operand's row stride) must fit
+  ITEXHIP_REQUIRE(p->N < (1LL << 22), "%s: N = %lld is not supported (N < 2^22)", who, static_cast<long long>(p->N));
+  for (int b = 0; b < p->n_binary; ++b)
+    ITEXHIP_REQUIRE(p->binary[b].stride_m < (1LL << 22) && p->binary[b].stride_n < (1LL << 22),
+                    "%s: a binary operand's matrix strides must be below 2^22 elements", who);
+
   BmmArgs a;
   a.p = *p;
+  for (int b = p->n_binary; b < ITEXHIP_BMM_MAX_BINARY; ++b) a.p.binary[b] = itexhip_bmm_binary{};
+  // merge adjacent batch dimensions that every tensor walks with one stride (fewer index divisions per workgroup)
+  for (int d = a.p.n_batch_dims - 2; d >= 0; --d) {
+    const int64_t inner = a.p.batch_dims[d + 1];
+    bool same = a.p.x_batch_stride[d] == a.p.x_batch_stride[d + 1] * inner &&
+                a.p.y_batch_stride[d] == a.p.y_batch_stride[d + 1] * inner;
+    for (int b = 0; b < a.p.n_binary; ++b)
+      same = same && a.p.binary[b].batch_stride[d] == a.p.binary[b].batch_stride[d + 1] * inner;
+    if (!same) continue;
+    a.p.batch_dims[d] *= inner;
+    a.p.x_batch_stride[d] = a.p.x_batch_stride[d + 1];
+    a.p.y_batch_stride[d] = a.p.y_batch_stride[d + 1];
+    for (int b = 0; b < a.p.n_binary; ++b) a.p.binary[b].batch_stride[d] = a.p.binary[b].batch_stride[d + 1];
+    for (int e = d + 1; e + 1 < a.p.n_batch_dims; ++e) {
+      a.p.batch_dims[e] = a.p.batch_dims[e + 1];
+      a.p.x_batch_stride[e] = a.p.x_batch_stride[e + 1];
+      a.p.y_batch_stride[e] = a.p.y_batch_stride[e + 1];
+      for (int b = 0; b < a.p.n_binary; ++b) a.p.binary[b].batch_stride[e] = a.p.binary[b].batch_stride[e + 1];
+    }
+    --a.p.n_batch_dims;
+  }
   a.tiles_m = static_cast<int>((p->M + kTile - 1) / kTile);
   a.tiles_n = static_cast<int>((p->N + kTile - 1) / kTile);
   const int64_t grid = batch * a.tiles_m * a.tiles_n;

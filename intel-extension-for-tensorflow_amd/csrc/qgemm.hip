@@ -351,8 +351,10 @@ int dispatch_gemv(const uint8_t* a, uint32_t a_xor, const uint8_t* bp, int M, in
   int waves = std::min(16, (KP + 7) / 8);
   for (int w = waves; w >= std::max(1, waves / 2); --w)
     if (KP % (8 * w) == 0) { waves = w; break; }
-  const int cnt = (KP + waves - 1) / waves;
   const int strips32 = (N + 31) / 32;
+  // a 32-channel strip is finished by two wavefronts, one per 16-channel tile: never fewer than that
+  if (strips32 >= 256) waves = std::max(waves, 2);
+  const int cnt = (KP + waves - 1) / waves;
   if (strips32 >= 256) {
     const size_t lds = static_cast<size_t>(waves) * 2 * 1024 + 6 * 32 * 4;
     qgemv_kernel<32, OUT_T><<<strips32, 64 * waves, lds, st>>>(a, a_xor, bp, M, K, N, KC, cnt, e, out);

@@ -151,3 +151,23 @@ def test_many_small_matrices(hip, dev):
     x = rng.integers(-128, 128, (3000, 8, 16)).astype(np.int8)
     y = rng.integers(-128, 128, (3000, 16, 8)).astype(np.int8)
     check(hip, dev, x, y)
+
+
+def test_half_output_is_rounded_from_the_fp32_result(hip, dev):
+    """float(acc) * scale is rounded to fp32 and only then to half.  A conversion fused with the multiply would round
+    the exact product once; the two differ on a handful of elements per million, which this problem contains."""
+    rng = np.random.default_rng(11)
+    x = rng.integers(-128, 128, (16, 256, 32)).astype(np.int8)
+    y = rng.integers(-128, 128, (16, 32, 256)).astype(np.int8)
+    rx, ry = 3.0, 1.5
+    acc = np.matmul(x.astype(np.int64), y.astype(np.int64)).astype(np.float64)
+    scale = np.float64(np.float32(np.float32(rx) * np.float32(ry)) / np.float32(127 * 127))
+    with np.errstate(over="ignore"):
+        once = (acc * scale).astype(np.float16)                          # exact product, one rounding
+        twice = (acc * scale).astype(np.float32).astype(np.float16)      # what the op defines
+    differ = once.view(np.uint16) != twice.view(np.uint16)
+    assert differ.sum() >= 3
+    got = run(hip, dev, x, y, rx, ry, t_out=orc.HALF)
+    np.testing.assert_array_equal(got[differ], twice.view(np.uint16)[differ])
+    st, ref = orc.qbatch_matmul(x, y, -rx, rx * 0.5, -ry * 0.25, ry, t_out=orc.HALF)
+    np.testing.assert_array_equal(got, ref)

@@ -236,7 +236,7 @@ def test_every_tile_shape_on_ragged_problems(hip, dev, monkeypatch, shape, M, K,
 
 
 @pytest.mark.parametrize("M", [1, 2, 4, 7, 16])
-@pytest.mark.parametrize("K,N", [(64, 16), (256, 100), (4096, 512), (1024, 4096), (8192, 48)])
+@pytest.mark.parametrize("K,N", [(64, 16), (256, 100), (4096, 512), (1024, 4096), (8192, 48), (64, 8200), (512, 16384)])
 @pytest.mark.parametrize("kw", [V2_DEQ, V2_REQ_S8])
 def test_gemv_kernel_vs_oracle(hip, dev, M, K, N, kw):
     layer, w, bias = make_layer(hip, dev, K, N, seed=K + N + 1)
@@ -586,3 +586,26 @@ def test_bfloat16_bias_vs_oracle(hip, dev, M, t_out, mode, T16):
               t_out, out)
     torch.cuda.synchronize()
     np.testing.assert_array_equal(bits16(out.cpu().numpy()), ref)
+
+
+@pytest.mark.parametrize("path", ["tile", "gemv", "naive"])
+def test_half_output_is_rounded_from_the_fp32_result(hip, dev, path):
+    """The epilogue's fp32 result is rounded to fp32 and only then to half: elements where one rounding of the exact
+    value would differ (a few per million) must follow the two-step definition."""
+    M = 16 if path == "gemv" else 512
+    K, N = 64, 2048 if path != "gemv" else 32768
+    layer, w, bias = make_layer(hip, dev, K, N, seed=3)
+    x, xq, mn, mx = make_acts(M, K, seed=8)
+    ref = layer.oracle(xq, V2_DEQ_F16, mn, mx)
+    ref32 = layer.oracle(xq, V2_DEQ, mn, mx)
+    np.testing.assert_array_equal(ref, ref32.astype(np.float16).view(np.uint16))
+    got = bits16(layer.run(xq, V2_DEQ_F16, mn, mx, path=path))
+    np.testing.assert_array_equal(got, ref)
+    # the sample does contain elements that tell the two roundings apart
+    st, sc, sb, ep = orc.qmatmul_prepare(orc.matmul_attrs(t_in=orc.QUINT8, **V2_DEQ_F16), N, layer.wq.astype(np.int32).sum(0),
+                                         mn, mx, layer.min_b, layer.max_b, 0.0, 0.0, bias)
+    acc = xq.astype(np.int64) @ layer.wq.astype(np.int64)
+    exact = acc.astype(np.float64) * sc.astype(np.float64) + sb.astype(np.float64)
+    with np.errstate(over="ignore"):
+        once = exact.astype(np.float16).view(np.uint16)
+    assert (once != ref).sum() >= 3
