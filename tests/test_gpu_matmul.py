@@ -609,3 +609,24 @@ def test_half_output_is_rounded_from_the_fp32_result(hip, dev, path):
     with np.errstate(over="ignore"):
         once = exact.astype(np.float16).view(np.uint16)
     assert (once != ref).sum() >= 3
+
+
+def test_random_shapes_through_the_single_launch_op(hip, dev):
+    """Seeded sweep over shapes, output types and fusions through itexhip_qmatmul (the dispatcher picks GEMV, tile shape
+    and store path from the shape), every case bit-compared with the oracle."""
+    rng = np.random.default_rng(2024)
+    kinds = [V2_DEQ, V2_DEQ_RELU, V2_REQ_S8, V2_REQ_U8_RELU, V1_S32, V2_DEQ_BF16, V2_DEQ_F16]
+    for case in range(48):
+        M = int(rng.choice([1, 2, 3, 5, 8, 15, 16, 17, 31, 33, 64, 100, 129, 255, 300]))
+        K = 16 * int(rng.integers(1, 96))
+        N = int(rng.choice([1, 7, 16, 31, 32, 33, 100, 255, 256, 1000, 4100, 8200, 9000]))
+        kw = kinds[int(rng.integers(0, len(kinds)))]
+        per_channel = bool(rng.integers(0, 2))
+        layer, w, bias = make_layer(hip, dev, K, N, seed=case, per_channel=per_channel)
+        x, xq, mn, mx = make_acts(M, K, seed=100 + case, mode=kw["input_mode"])
+        full = x @ w + bias
+        r_out = float(np.abs(np.maximum(full, 0) if kw.get("activation") else full).max())
+        lo = 0.0 if kw["t_out"] == orc.QUINT8 else -r_out
+        ref = layer.oracle(xq, kw, mn, mx, lo, r_out)
+        got = bits16(layer.run(xq, kw, mn, mx, lo, r_out, path="fused"))
+        assert np.array_equal(got, ref), (case, M, K, N, kw, per_channel)
