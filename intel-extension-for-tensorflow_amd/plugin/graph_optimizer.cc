@@ -1,0 +1,179 @@
+// TF_InitGraph: the graph-optimizer half of the plugin.  It carries the quantized subset of the reference's
+// native-format pass (itex/core/graph/native_layout/native_layout.cc:113-198, 402-500 and the rewrite rules /
+// attribute copies in itex/core/graph/utils/layout_utils.cc:315-355, 497-545): nodes placed on this plugin's
+// device whose op has an _ITEX twin are renamed to it, with the attributes the twin adds.  For QuantizeV2
+// that rename is not cosmetic: _ITEXQuantizeV2 receives classic_asymmetric_algorithm = "all consumers are
+// Dequantize", which selects the zero-point form of MIN_FIRST instead of the legacy one.
+// ITEX_AMD_NATIVE_FORMAT=0 leaves graphs untouched.
+#include <cstdlib>
+#include <cstring>
+#include <map>
+#include <string>
+#include <vector>
+
+#include "graph_def.h"
+#include "tf_grappler_subset.h"
+
+namespace itex_amd {
+namespace {
+
+constexpr int kDtFloat = 1, kDtQint8 = 11, kDtQuint8 = 12;
+
+enum class Copy { kAll, kQuantize, kQuantizedMatMul };
+enum class Rule { kAlways, kQuantize };
+
+struct Rename {
+  const char* from;
+  const char* to;
+  Copy copy;
+  Rule rule;
+};
+
+// the INT8 rows of the reference's table whose targets this plugin registers kernels for
+const Rename kTable[] = {
+    {"Dequantize", "_ITEXDequantize", Copy::kAll, Rule::kQuantize},
+    {"QuantizeV2", "_ITEXQuantizeV2", Copy::kQuantize, Rule::kQuantize},
+    {"QuantizedMatMulWithBias", "_ITEXQuantizedMatMulWithBias", Copy::kQuantizedMatMul, Rule::kAlways},
+    {"QuantizedMatMulWithBiasAndDequantize", "_ITEXQuantizedMatMulWithBiasAndDequantize", Copy::kQuantizedMatMul, Rule::kAlways},
+    {"QuantizedMatMulWithBiasAndRelu", "_ITEXQuantizedMatMulWithBiasAndRelu", Copy::kQuantizedMatMul, Rule::kAlways},
+    {"QuantizedMatMulWithBiasAndReluAndRequantize", "_ITEXQuantizedMatMulWithBiasAndReluAndRequantize", Copy::kQuantizedMatMul,
+     Rule::kAlways},
+    {"QuantizedMatMulWithBiasAndRequantize", "_ITEXQuantizedMatMulWithBiasAndRequantize", Copy::kQuantizedMatMul, Rule::kAlways},
+    {"_QuantizedBatchMatMul", "_ITEXQuantizedBatchMatMul", Copy::kAll, Rule::kAlways},
+    {"_QuantizedBatchMatMulV2AndDequantize", "_ITEXQuantizedBatchMatMulV2AndDequantize", Copy::kAll, Rule::kAlways},
+    {"_QuantizedFusedBatchMatMulV2AndDequantize", "_ITEXQuantizedFusedBatchMatMulV2AndDequantize", Copy::kAll, Rule::kAlways},
+    {"_QuantizedFusedMatMul", "_ITEXQuantizedFusedMatMul", Copy::kQuantizedMatMul, Rule::kAlways},
+    {"_QuantizedFusedMatMulAndDequantize", "_ITEXQuantizedFusedMatMulAndDequantize", Copy::kQuantizedMatMul, Rule::kAlways},
+    {"_QuantizedFusedMatMulAndRequantize", "_ITEXQuantizedFusedMatMulAndRequantize", Copy::kQuantizedMatMul, Rule::kAlways},
+    {"_QuantizedMatMul", "_ITEXQuantizedMatMul", Copy::kAll, Rule::kAlways},
+};
+
+std::string DeviceType() {
+  const char* dev = std::getenv("ITEX_AMD_DEVICE_TYPE");
+  return dev && dev[0] ? dev : "XPU";
+}
+
+// the producer named by a data input: "name", "name:port"; control inputs ("^name") carry no tensor
+bool SplitInput(const std::string& in, std::string* name, int* port) {
+  if (in.empty() || in[0] == '^') return false;
+  const size_t colon = in.rfind(':');
+  if (colon == std::string::npos) { *name = in; *port = 0; return true; }
+  *name = in.substr(0, colon);
+  *port = std::atoi(in.c_str() + colon + 1);
+  return true;
+}
+
+// layout_utils.cc:661-677: QuantizeV2 / Dequantize are only rewritten for T in {qint8, quint8}
+bool SupportedType(const graph::Node& n) {
+  if (n.op != "QuantizeV2" && n.op != "Dequantize") return true;
+  int t = 0;
+  const std::string* a = n.FindAttr("T");
+  return a && graph::AttrType(*a, &t) && (t == kDtQint8 || t == kDtQuint8);
+}
+
+// layout_utils.cc:315-355.  (Its refusal of MIN_FIRST Dequantize on a GPU does not apply: the kernel
+// this plugin registers implements that mode.)
+bool RewriteQuantize(const graph::Node& n) {
+  std::string mode, round_mode;
+  const std::string* m = n.FindAttr("mode");
+  if (!m || !graph::AttrString(*m, &mode)) return false;
+  if (mode == "MIN_COMBINED") return false;
+  const std::string* r = n.FindAttr("round_mode");
+  if (r && graph::AttrString(*r, &round_mode) && mode == "SCALED" && round_mode != "HALF_TO_EVEN") return false;
+  return true;
+}
+
+struct Optimizer {
+  std::string device_type;
+};
+
+void* Create() { return new Optimizer{DeviceType()}; }
+void Destroy(void* o) { delete static_cast<Optimizer*>(o); }
+
+void FreeBuffer(void* data, size_t) { std::free(data); }
+
+void Optimize(void* opt, const TF_Buffer* in, const TF_GrapplerItem*, TF_Buffer* out, TF_Status* status) {
+  const Optimizer* self = static_cast<const Optimizer*>(opt);
+  graph::Graph g;
+  if (!graph::Parse(in->data, in->length, &g)) {
+    TF_SetStatus(status, TF_INVALID_ARGUMENT, "itex_amd graph optimizer: the GraphDef could not be parsed");
+    return;
+  }
+  const char* sw = std::getenv("ITEX_AMD_NATIVE_FORMAT");
+  const bool enabled = !(sw && std::strcmp(sw, "0") == 0);
+
+  // consumers of output 0 of every node, by op name (for CopyAttrsQuantize)
+  std::map<std::string, std::vector<const graph::Node*>> fanout0;
+  for (const graph::Node& n : g.nodes)
+    for (const std::string& in_name : n.inputs) {
+      std::string producer;
+      int port = 0;
+      if (SplitInput(in_name, &producer, &port) && port == 0) fanout0[producer].push_back(&n);
+    }
+  // decisions first, on the unmodified graph: a QuantizeV2's consumers are looked up by their original op
+  std::vector<const Rename*> plan(g.nodes.size(), nullptr);
+  std::vector<bool> classic(g.nodes.size(), false);
+  for (size_t i = 0; enabled && i < g.nodes.size(); ++i) {
+    const graph::Node& n = g.nodes[i];
+    // NodeIsOnDevice (utils.cc:262-265): the node carries a device string naming this device type
+    if (n.device.empty() || n.device.find(self->device_type) == std::string::npos) continue;
+    if (!SupportedType(n)) continue;
+    for (const Rename& r : kTable) {
+      if (n.op != r.from) continue;
+      if (r.rule == Rule::kQuantize && !RewriteQuantize(n)) break;
+      plan[i] = &r;
+      if (r.copy == Copy::kQuantize) {  // layout_utils.cc:530-541
+        bool all_dequantize = true;
+        for (const graph::Node* c : fanout0[n.name]) all_dequantize = all_dequantize && c->op == "Dequantize";
+        classic[i] = all_dequantize;
+      }
+      break;
+    }
+  }
+  for (size_t i = 0; i < g.nodes.size(); ++i) {
+    if (!plan[i]) continue;
+    graph::Node& n = g.nodes[i];  // name, inputs (control inputs included), device and attributes stay (RewriteNode :411-441)
+    n.op = plan[i]->to;
+    if (plan[i]->copy == Copy::kQuantize) {
+      if (!n.FindAttr("dtype")) n.SetAttr("dtype", graph::MakeAttrType(kDtFloat));
+      n.SetAttr("classic_asymmetric_algorithm", graph::MakeAttrBool(classic[i]));
+    }
+    // CopyAttrsQuantizedMatMul (:497-515) copies every attribute and then Tbias once more: nothing to add
+  }
+
+  const std::string bytes = graph::Serialize(g);
+  void* mem = std::malloc(bytes.size() ? bytes.size() : 1);
+  if (!mem) {
+    TF_SetStatus(status, TF_INTERNAL, "itex_amd graph optimizer: out of memory");
+    return;
+  }
+  std::memcpy(mem, bytes.data(), bytes.size());
+  out->data = mem;
+  out->length = bytes.size();
+  out->data_deallocator = FreeBuffer;
+  TF_SetStatus(status, TF_OK, "");
+}
+
+}  // namespace
+}  // namespace itex_amd
+
+// itex/core/graph/xpu_graph.cc:137-176
+extern "C" void TF_InitGraph(TP_OptimizerRegistrationParams* params, TF_Status* status) {
+  params->struct_size = TP_OPTIMIZER_REGISTRATION_PARAMS_STRUCT_SIZE;
+  params->optimizer_configs->struct_size = TP_OPTIMIZER_CONFIGS_STRUCT_SIZE;
+  params->optimizer->struct_size = TP_OPTIMIZER_STRUCT_SIZE;
+  params->major_version = GO_MAJOR;
+  params->minor_version = GO_MINOR;
+  params->patch_version = GO_PATCH;
+  // TensorFlow's own remapper and layout optimizer stay off while a plugin optimizer is registered, as the
+  // reference sets them (:146-148); this pass does not depend on the others
+  params->optimizer_configs->remapping = TF_TriState_Off;
+  params->optimizer_configs->layout_optimizer = TF_TriState_Off;
+  static std::string device_type;  // must outlive the call
+  device_type = itex_amd::DeviceType();
+  params->device_type = device_type.c_str();
+  params->optimizer->create_func = itex_amd::Create;
+  params->optimizer->optimize_func = itex_amd::Optimize;
+  params->optimizer->destroy_func = itex_amd::Destroy;
+  TF_SetStatus(status, TF_OK, "");
+}

@@ -142,6 +142,34 @@ std::vector<OpSpec> OpSpecs() {
     v.push_back(bmm);
     v.push_back(fbmm);
   }
+  // the _ITEX twins of TensorFlow's QuantizedMatMulWithBias* ops, nn_ops.cc:1600-1770
+  {
+    const std::vector<const char*> in7 = {"a: T1", "b: T2", "bias: Tbias", "min_a: float", "max_a: float", "min_b: float",
+                                          "max_b: float"};
+    std::vector<const char*> in9 = in7;
+    in9.push_back("min_freezed_output: float");
+    in9.push_back("max_freezed_output: float");
+    const std::vector<const char*> out3 = {"out: Toutput", "min_out: float", "max_out: float"};
+    auto attrs = [](const char* tbias, const char* toutput) {
+      std::vector<const char*> a = {"T1: quantizedtype", "T2: quantizedtype"};
+      if (tbias) a.push_back(tbias);
+      a.push_back(toutput);
+      for (const char* x : {"transpose_a: bool = false", "transpose_b: bool = false",
+                            "input_quant_mode: {'MIN_FIRST', 'SCALED'} = 'MIN_FIRST'", "is_weight_const: bool = true"})
+        a.push_back(x);
+      return a;
+    };
+    v.push_back({"_ITEXQuantizedMatMulWithBias", in7, out3, attrs("Tbias: {float, qint32}", "Toutput: quantizedtype = DT_QINT32")});
+    std::vector<const char*> in7f = in7;
+    in7f[2] = "bias: float";
+    v.push_back({"_ITEXQuantizedMatMulWithBiasAndRelu", in7f, out3, attrs(nullptr, "Toutput: quantizedtype = DT_QINT32")});
+    v.push_back({"_ITEXQuantizedMatMulWithBiasAndRequantize", in9, out3,
+                 attrs("Tbias: {float, qint32}", "Toutput: quantizedtype = DT_QUINT8")});
+    v.push_back({"_ITEXQuantizedMatMulWithBiasAndReluAndRequantize", in9, out3,
+                 attrs("Tbias: {float, qint32}", "Toutput: quantizedtype = DT_QUINT8")});
+    v.push_back({"_ITEXQuantizedMatMulWithBiasAndDequantize", in9, {"out: Toutput"},
+                 attrs("Tbias: {float, bfloat16, qint32}", "Toutput: {float, bfloat16}")});
+  }
   // nn_ops.cc:4636-4691
   for (const char* name : {"_QuantizedBatchMatMul", "_ITEXQuantizedBatchMatMul"})
     v.push_back({name,

@@ -293,16 +293,18 @@ void RegBothInputs(const char* op, const char* out_attr, const char* bias_attr, 
 void AddQuantizedMatMulKernels() {
   constexpr int V2 = ITEXHIP_API_V2, V1 = ITEXHIP_API_V1, LG = ITEXHIP_API_LEGACY;
   // legacy ops: quint8 x qint8
-  Reg<LG, TF_QUINT8, TF_QINT32, true>("QuantizedMatMulWithBiasAndRelu", "Toutput", nullptr,
-                                      {"min_a", "max_a", "min_b", "max_b", "min_out", "max_out"});
-  Reg<LG, TF_QUINT8, TF_QINT32, false>("QuantizedMatMulWithBias", "Toutput", "Tbias",
-                                       {"min_a", "max_a", "min_b", "max_b", "min_out", "max_out"});
-  Reg<LG, TF_QUINT8, TF_QUINT8, true>("QuantizedMatMulWithBiasAndReluAndRequantize", "Toutput", "Tbias",
-                                      {"min_a", "max_a", "min_b", "max_b", "min_freezed_output", "max_freezed_output",
-                                       "min_out", "max_out"});
-  Reg<LG, TF_QUINT8, TF_QUINT8, false>("QuantizedMatMulWithBiasAndRequantize", "Toutput", "Tbias",
-                                       {"min_a", "max_a", "min_b", "max_b", "min_freezed_output", "max_freezed_output",
-                                        "min_out", "max_out"});
+  for (const char* op : {"QuantizedMatMulWithBiasAndRelu", "_ITEXQuantizedMatMulWithBiasAndRelu"})
+    Reg<LG, TF_QUINT8, TF_QINT32, true>(op, "Toutput", nullptr, {"min_a", "max_a", "min_b", "max_b", "min_out", "max_out"});
+  for (const char* op : {"QuantizedMatMulWithBias", "_ITEXQuantizedMatMulWithBias"})
+    Reg<LG, TF_QUINT8, TF_QINT32, false>(op, "Toutput", "Tbias", {"min_a", "max_a", "min_b", "max_b", "min_out", "max_out"});
+  for (const char* op : {"QuantizedMatMulWithBiasAndReluAndRequantize", "_ITEXQuantizedMatMulWithBiasAndReluAndRequantize"})
+    Reg<LG, TF_QUINT8, TF_QUINT8, true>(op, "Toutput", "Tbias",
+                                        {"min_a", "max_a", "min_b", "max_b", "min_freezed_output", "max_freezed_output",
+                                         "min_out", "max_out"});
+  for (const char* op : {"QuantizedMatMulWithBiasAndRequantize", "_ITEXQuantizedMatMulWithBiasAndRequantize"})
+    Reg<LG, TF_QUINT8, TF_QUINT8, false>(op, "Toutput", "Tbias",
+                                         {"min_a", "max_a", "min_b", "max_b", "min_freezed_output", "max_freezed_output",
+                                          "min_out", "max_out"});
   for (const char* op : {"QuantizedMatMulWithBiasAndDequantize", "_ITEXQuantizedMatMulWithBiasAndDequantize"})
     Reg<LG, TF_QUINT8, TF_FLOAT, false>(op, "Toutput", "Tbias",
                                         {"min_a", "max_a", "min_b", "max_b", "min_freezed_output", "max_freezed_output"});

@@ -16,6 +16,7 @@
 #include <vector>
 
 #include "tf_c_api_subset.h"
+#include "tf_grappler_subset.h"
 #include "tf_stream_executor_subset.h"
 
 // ------------------------------------------------------------------------------------------------
@@ -633,6 +634,60 @@ int mock_load_plugin(const char* path) {
   init();
   return 0;
 }
+
+// ---- graph optimizer: TF_InitGraph, then create / optimize / destroy as TensorFlow's plugin optimizer wrapper does
+static void* g_plugin_handle = nullptr;
+static TP_Optimizer g_optimizer;
+static TP_OptimizerConfigs g_optimizer_configs;
+static std::string g_optimizer_device;
+static std::string g_optimized;
+
+// returns 0 and fills the registration state, or a nonzero code
+int mock_graph_init(const char* path) {
+  g_plugin_handle = dlopen(path, RTLD_NOW | RTLD_GLOBAL);
+  if (!g_plugin_handle) return 1;
+  auto init = reinterpret_cast<void (*)(TP_OptimizerRegistrationParams*, TF_Status*)>(dlsym(g_plugin_handle, "TF_InitGraph"));
+  if (!init) return 2;
+  std::memset(&g_optimizer, 0, sizeof(g_optimizer));
+  std::memset(&g_optimizer_configs, 0, sizeof(g_optimizer_configs));
+  TP_OptimizerRegistrationParams params;
+  std::memset(&params, 0, sizeof(params));
+  params.struct_size = TP_OPTIMIZER_REGISTRATION_PARAMS_STRUCT_SIZE;
+  params.optimizer = &g_optimizer;
+  params.optimizer_configs = &g_optimizer_configs;
+  TF_Status st;
+  init(&params, &st);
+  if (st.code != TF_OK) return 3;
+  // what TensorFlow validates (c_api_experimental grappler registration): sizes, device type, the three functions
+  if (params.struct_size == 0 || g_optimizer.struct_size == 0 || g_optimizer_configs.struct_size == 0) return 4;
+  if (!params.device_type || !params.device_type[0]) return 5;
+  if (!g_optimizer.optimize_func) return 6;
+  if (params.major_version != GO_MAJOR) return 7;
+  g_optimizer_device = params.device_type;
+  return 0;
+}
+const char* mock_graph_device_type(void) { return g_optimizer_device.c_str(); }
+int mock_graph_config(const char* name) {
+  const std::string n = name;
+  if (n == "remapping") return g_optimizer_configs.remapping;
+  if (n == "layout_optimizer") return g_optimizer_configs.layout_optimizer;
+  if (n == "constant_folding") return g_optimizer_configs.constant_folding;
+  return -1;
+}
+// runs the optimizer on a serialized GraphDef; the result is read with mock_graph_result / _size
+int mock_graph_optimize(const void* graph, size_t len) {
+  void* opt = g_optimizer.create_func ? g_optimizer.create_func() : nullptr;
+  TF_Buffer in{graph, len, nullptr};
+  TF_Buffer out{nullptr, 0, nullptr};
+  TF_Status st;
+  g_optimizer.optimize_func(opt, &in, nullptr, &out, &st);
+  if (g_optimizer.destroy_func) g_optimizer.destroy_func(opt);
+  g_optimized.assign(static_cast<const char*>(out.data), out.length);
+  if (out.data_deallocator) out.data_deallocator(const_cast<void*>(out.data), out.length);
+  return st.code;
+}
+const void* mock_graph_result(void) { return g_optimized.data(); }
+size_t mock_graph_result_size(void) { return g_optimized.size(); }
 
 static std::string Quote(const std::string& s) {
   std::string o = "\"";

@@ -1,0 +1,135 @@
+"""TF_InitGraph through the mock host: registration as TensorFlow checks it, and the quantized subset of the
+reference's native-format rewrite (itex/core/graph/native_layout/native_layout.cc:113-198, layout_utils.cc:315-355,
+497-545) on GraphDefs serialized and parsed by google.protobuf."""
+import ctypes as C
+import os
+
+import pytest
+
+from tests.mock_tf import graphdef as gd
+from tests.mock_tf import host as tf
+
+QINT8, QUINT8, QINT32, FLOAT = 11, 12, 13, 1
+DEV = "/job:localhost/replica:0/task:0/device:XPU:0"
+CPU = "/job:localhost/replica:0/task:0/device:CPU:0"
+
+
+@pytest.fixture(scope="module")
+def opt():
+    lib = tf.load()
+    lib.mock_graph_device_type.restype = C.c_char_p
+    lib.mock_graph_result.restype = C.c_void_p
+    lib.mock_graph_result_size.restype = C.c_size_t
+    assert lib.mock_graph_init(tf.PLUGIN_LIB.encode()) == 0
+    return lib
+
+
+def run(opt, graph):
+    data = graph.SerializeToString()
+    code = opt.mock_graph_optimize(data, C.c_size_t(len(data)))
+    assert code == tf.OK
+    out = gd.GraphDef()
+    out.ParseFromString(C.string_at(opt.mock_graph_result(), opt.mock_graph_result_size()))
+    return out
+
+
+def by_name(g):
+    return {n.name: n for n in g.node}
+
+
+def test_registration(opt):
+    assert opt.mock_graph_device_type() == b"XPU"
+    TF_TriState_Off = 1
+    assert opt.mock_graph_config(b"remapping") == TF_TriState_Off          # xpu_graph.cc:146-148
+    assert opt.mock_graph_config(b"layout_optimizer") == TF_TriState_Off
+    assert opt.mock_graph_config(b"constant_folding") == 0                 # left at TensorFlow's default
+
+
+def qdq_graph():
+    g = gd.GraphDef()
+    g.versions.producer = 1645
+    gd.node(g, "x", "Placeholder", device=DEV, dtype=("type", FLOAT))
+    for c in ("mn", "mx"):
+        gd.node(g, c, "Const", device=CPU, dtype=("type", FLOAT))
+    # q1 feeds only a Dequantize: the classic zero-point algorithm; q2 feeds a matmul: the legacy one
+    gd.node(g, "q1", "QuantizeV2", ["x", "mn", "mx"], DEV, T=("type", QUINT8), mode="MIN_FIRST", round_mode="HALF_AWAY_FROM_ZERO",
+            narrow_range=False, axis=-1, ensure_minimum_range=0.01)
+    gd.node(g, "dq1", "Dequantize", ["q1", "q1:1", "q1:2"], DEV, T=("type", QUINT8), mode="MIN_FIRST", narrow_range=False, axis=-1,
+            dtype=("type", FLOAT))
+    gd.node(g, "q2", "QuantizeV2", ["x", "mn", "mx", "^dq1"], DEV, T=("type", QUINT8), mode="MIN_FIRST",
+            round_mode="HALF_AWAY_FROM_ZERO", narrow_range=False, axis=-1, ensure_minimum_range=0.01)
+    gd.node(g, "mm", "_QuantizedMatMul", ["q2", "w", "b", "q2:1", "q2:2", "wmn", "wmx"], DEV, T1=("type", QUINT8), T2=("type", QINT8),
+            Tbias=("type", FLOAT), Tout=("type", FLOAT), fused_ops=["BiasAdd", "Dequantize"], input_quant_mode="MIN_FIRST")
+    return g
+
+
+def test_quantize_rename_and_classic_algorithm_flag(opt):
+    out = by_name(run(opt, qdq_graph()))
+    assert out["q1"].op == "_ITEXQuantizeV2" and out["q2"].op == "_ITEXQuantizeV2"
+    assert out["dq1"].op == "_ITEXDequantize" and out["mm"].op == "_ITEXQuantizedMatMul"
+    assert out["q1"].attr["classic_asymmetric_algorithm"].b is True
+    assert out["q2"].attr["classic_asymmetric_algorithm"].b is False
+    assert out["q2"].attr["classic_asymmetric_algorithm"].WhichOneof("value") == "b"    # present, not defaulted
+    assert out["q1"].attr["dtype"].type == FLOAT                                         # added for QuantizeV2
+    # everything else is carried over: inputs incl. the control edge, device, the other attributes, other nodes
+    assert list(out["q2"].input) == ["x", "mn", "mx", "^dq1"] and out["q2"].device == DEV
+    assert out["q1"].attr["mode"].s == b"MIN_FIRST" and out["q1"].attr["T"].type == QUINT8
+    assert abs(out["q1"].attr["ensure_minimum_range"].f - 0.01) < 1e-9 and out["q1"].attr["axis"].i == -1
+    assert list(out["mm"].attr["fused_ops"].list.s) == [b"BiasAdd", b"Dequantize"]
+    assert out["x"].op == "Placeholder" and out["mn"].op == "Const"
+    assert run(opt, qdq_graph()).versions.producer == 1645
+
+
+def test_rules_that_block_the_rewrite(opt):
+    g = gd.GraphDef()
+    common = dict(narrow_range=False, axis=-1, ensure_minimum_range=0.01)
+    gd.node(g, "on_cpu", "QuantizeV2", ["x", "a", "b"], CPU, T=("type", QINT8), mode="SCALED", round_mode="HALF_TO_EVEN", **common)
+    gd.node(g, "unplaced", "QuantizeV2", ["x", "a", "b"], "", T=("type", QINT8), mode="SCALED", round_mode="HALF_TO_EVEN", **common)
+    gd.node(g, "min_combined", "QuantizeV2", ["x", "a", "b"], DEV, T=("type", QINT8), mode="MIN_COMBINED",
+            round_mode="HALF_AWAY_FROM_ZERO", **common)
+    gd.node(g, "scaled_away", "QuantizeV2", ["x", "a", "b"], DEV, T=("type", QINT8), mode="SCALED", round_mode="HALF_AWAY_FROM_ZERO",
+            **common)
+    gd.node(g, "qint32", "QuantizeV2", ["x", "a", "b"], DEV, T=("type", QINT32), mode="SCALED", round_mode="HALF_TO_EVEN", **common)
+    gd.node(g, "ok", "QuantizeV2", ["x", "a", "b"], DEV, T=("type", QINT8), mode="SCALED", round_mode="HALF_TO_EVEN", **common)
+    gd.node(g, "relu", "Relu", ["ok"], DEV, T=("type", FLOAT))
+    out = by_name(run(opt, g))
+    for name in ("on_cpu", "unplaced", "min_combined", "scaled_away", "qint32"):
+        assert out[name].op == "QuantizeV2", name
+        assert "classic_asymmetric_algorithm" not in out[name].attr
+    assert out["ok"].op == "_ITEXQuantizeV2" and out["ok"].attr["classic_asymmetric_algorithm"].b is False   # feeds a Relu
+    assert out["relu"].op == "Relu"
+
+
+def test_every_renamed_op_has_a_kernel_and_an_op_definition(opt):
+    reg = tf.registry()
+    kernels = {k["op"] for k in reg["kernels"]}
+    defined = {o["name"] for o in reg["ops"]}
+    ops = ["Dequantize", "QuantizeV2", "QuantizedMatMulWithBias", "QuantizedMatMulWithBiasAndDequantize",
+           "QuantizedMatMulWithBiasAndRelu", "QuantizedMatMulWithBiasAndReluAndRequantize", "QuantizedMatMulWithBiasAndRequantize",
+           "_QuantizedBatchMatMul", "_QuantizedBatchMatMulV2AndDequantize", "_QuantizedFusedBatchMatMulV2AndDequantize",
+           "_QuantizedFusedMatMul", "_QuantizedFusedMatMulAndDequantize", "_QuantizedFusedMatMulAndRequantize", "_QuantizedMatMul"]
+    g = gd.GraphDef()
+    for i, op in enumerate(ops):
+        gd.node(g, "n%d" % i, op, ["x"], DEV, mode="SCALED", T=("type", QINT8))
+    out = run(opt, g)
+    for n, op in zip(out.node, ops):
+        assert n.op == "_ITEX" + op.lstrip("_"), (op, n.op)
+        assert n.op in kernels, n.op
+        assert n.op in defined, n.op
+
+
+def test_switch_and_malformed_input(opt, monkeypatch):
+    monkeypatch.setenv("ITEX_AMD_NATIVE_FORMAT", "0")
+    out = by_name(run(opt, qdq_graph()))
+    assert out["q1"].op == "QuantizeV2" and out["mm"].op == "_QuantizedMatMul"
+    monkeypatch.delenv("ITEX_AMD_NATIVE_FORMAT")
+    bad = b"\x0a\xff\xff\xff\x0f" + b"x" * 8      # a node whose length runs past the buffer
+    assert opt.mock_graph_optimize(bad, C.c_size_t(len(bad))) == tf.INVALID_ARGUMENT
+
+
+def test_unknown_fields_survive(opt):
+    g = qdq_graph()
+    data = g.SerializeToString() + b"\x18\x07"      # GraphDef.version = 3 (varint), unknown to the subset messages
+    assert opt.mock_graph_optimize(data, C.c_size_t(len(data))) == tf.OK
+    raw = C.string_at(opt.mock_graph_result(), opt.mock_graph_result_size())
+    assert raw.endswith(b"\x18\x07")
