@@ -328,6 +328,16 @@ typedef struct {
  * tiles of 64 x 64 outputs per workgroup. */
 int itexhip_qbatch_matmul(const itexhip_bmm_params* p, const int8_t* x, const int8_t* y, void* out, void* stream);
 
+/* ---- quantized Transpose ------------------------------------------------------------------------
+ * y = transpose(x, perm) for a tensor of 1-byte (qint8 / quint8) or 4-byte (qint32) elements: dimension i
+ * of y is dimension perm[i] of x (_QuantizedTranspose, itex/core/kernels/common/transpose_op.h:197-236,
+ * registered for a device in itex/core/kernels/gpu/transpose_op.cc:48-55; its min / max pass through on
+ * the host).  rank <= 8; adjacent dimensions that stay adjacent are merged first; a permutation that keeps
+ * the innermost run of at least 16 bytes moves 16-byte vectors (the [B, S, H, D] <-> [B, H, S, D] moves
+ * of an attention block), any other one moves single elements. */
+int itexhip_transpose(const void* x, void* y, int elem_size, int rank, const int64_t* dims, const int32_t* perm,
+                      void* stream);
+
 /* Diagnostic, no counterpart in the reference: `workgroups` x 4 wavefronts each issue iters x 8
  * independent 32x32x32 i8 MFMAs (2 * 32768 ops each) on the 8 KiB of operand fragments at `operands`
  * (device memory, 16-byte aligned) and nothing else.  Timed by the caller, it gives the rate the matrix

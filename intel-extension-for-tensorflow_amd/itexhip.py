@@ -29,7 +29,7 @@ EXPORTS = [
     "itexhip_requantize", "itexhip_minmax_i32_per_channel", "itexhip_minmax_f32",
     "itexhip_qmatmul_epilogue_desc", "itexhip_qmatmul_prepare", "itexhip_qgemm_packed_bytes",
     "itexhip_qgemm_prepack_b", "itexhip_qgemm", "itexhip_qgemm_tile", "itexhip_qgemv", "itexhip_qmatmul", "itexhip_qmatmul_per_row", "itexhip_qmatmul_unpacked", "itexhip_mfma_probe",
-    "itexhip_qgemm_naive", "itexhip_qbatch_matmul",
+    "itexhip_qgemm_naive", "itexhip_qbatch_matmul", "itexhip_transpose",
 ]
 
 
@@ -312,3 +312,10 @@ def bmm_params(x_shape, y_shape, adj_x, adj_y, out_type, scale, binary=()):
 
 def qbatch_matmul(p, x, y, out, stream=0):
     _check(_lib.itexhip_qbatch_matmul(C.byref(p), _ptr(x), _ptr(y), _ptr(out), _ptr(stream)))
+
+
+def transpose(x, y, elem_size, dims, perm, stream=0):
+    rank = len(dims)
+    d = (C.c_int64 * max(rank, 1))(*dims)
+    pm = (C.c_int32 * max(rank, 1))(*perm)
+    _check(_lib.itexhip_transpose(_ptr(x), _ptr(y), int(elem_size), rank, d, pm, _ptr(stream)))

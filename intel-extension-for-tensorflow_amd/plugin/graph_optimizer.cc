@@ -20,7 +20,7 @@ namespace {
 constexpr int kDtFloat = 1, kDtQint8 = 11, kDtQuint8 = 12;
 
 enum class Copy { kAll, kQuantize, kQuantizedMatMul };
-enum class Rule { kAlways, kQuantize };
+enum class Rule { kAlways, kQuantize, kQint8Only };
 
 struct Rename {
   const char* from;
@@ -46,6 +46,8 @@ const Rename kTable[] = {
     {"_QuantizedFusedMatMulAndDequantize", "_ITEXQuantizedFusedMatMulAndDequantize", Copy::kQuantizedMatMul, Rule::kAlways},
     {"_QuantizedFusedMatMulAndRequantize", "_ITEXQuantizedFusedMatMulAndRequantize", Copy::kQuantizedMatMul, Rule::kAlways},
     {"_QuantizedMatMul", "_ITEXQuantizedMatMul", Copy::kAll, Rule::kAlways},
+    {"QuantizedReshape", "_ITEXQuantizedReshape", Copy::kAll, Rule::kQint8Only},  // RewriteQuantizeReshape, layout_utils.cc:392-400
+    {"_QuantizedTranspose", "_ITEXQuantizedTranspose", Copy::kAll, Rule::kAlways},
 };
 
 std::string DeviceType() {
@@ -121,6 +123,11 @@ void Optimize(void* opt, const TF_Buffer* in, const TF_GrapplerItem*, TF_Buffer*
     for (const Rename& r : kTable) {
       if (n.op != r.from) continue;
       if (r.rule == Rule::kQuantize && !RewriteQuantize(n)) break;
+      if (r.rule == Rule::kQint8Only) {
+        int t = 0;
+        const std::string* a = n.FindAttr("T");
+        if (!a || !graph::AttrType(*a, &t) || t != kDtQint8) break;
+      }
       plan[i] = &r;
       if (r.copy == Copy::kQuantize) {  // layout_utils.cc:530-541
         bool all_dequantize = true;

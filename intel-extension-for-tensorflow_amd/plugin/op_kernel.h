@@ -158,6 +158,7 @@ void AddQuantizeKernels();
 void AddDequantizeKernels();
 void AddQuantizedMatMulKernels();
 void AddQuantizedBatchMatMulKernels();
+void AddQuantizedShapeKernels();
 void AddRequantizeKernels();
 // op definitions for the ops stock TensorFlow does not have
 void RegisterOps();

@@ -170,6 +170,16 @@ std::vector<OpSpec> OpSpecs() {
     v.push_back({"_ITEXQuantizedMatMulWithBiasAndDequantize", in9, {"out: Toutput"},
                  attrs("Tbias: {float, bfloat16, qint32}", "Toutput: {float, bfloat16}")});
   }
+  // nn_ops.cc:562-585 (_QuantizedTranspose), :3266-3290 (_ITEXQuantizedReshape)
+  for (const char* name : {"_QuantizedTranspose", "_ITEXQuantizedTranspose"})
+    v.push_back({name,
+                 {"x: T", "perm: Tperm", "min_x: float", "max_x: float"},
+                 {"y: T", "min_y: float", "max_y: float"},
+                 {"T: quantizedtype", "Tperm: {int32, int64} = DT_INT32"}});
+  v.push_back({"_ITEXQuantizedReshape",
+               {"tensor: T", "shape: Tshape", "input_min: float", "input_max: float"},
+               {"output: T", "output_min: float", "output_max: float"},
+               {"T: type", "Tshape: {int32, int64} = DT_INT32"}});
   // nn_ops.cc:4636-4691
   for (const char* name : {"_QuantizedBatchMatMul", "_ITEXQuantizedBatchMatMul"})
     v.push_back({name,
@@ -214,6 +224,7 @@ extern "C" void TF_InitKernel(void) {
     AddDequantizeKernels();
     AddQuantizedMatMulKernels();
     AddQuantizedBatchMatMulKernels();
+    AddQuantizedShapeKernels();
     AddRequantizeKernels();
     // the device type the kernels attach to: ITEX's own PluggableDevice type by default, so that graphs
     // placed by ITEX's passes keep their device strings

@@ -24,7 +24,7 @@ _state = {}
 def load(device="XPU", stock_ops=("QuantizeV2", "Dequantize", "QuantizedMatMulWithBias", "QuantizedMatMulWithBiasAndRelu",
                                    "QuantizedMatMulWithBiasAndReluAndRequantize", "QuantizedMatMulWithBiasAndRequantize",
                                    "QuantizedMatMulWithBiasAndDequantize", "RequantizePerChannel",
-                                   "RequantizationRangePerChannel", "MatMul", "Relu")):
+                                   "RequantizationRangePerChannel", "QuantizedReshape", "MatMul", "Relu")):
     """Loads the mock host and the plugin once per process; returns the mock's ctypes handle."""
     if "lib" in _state:
         return _state["lib"]

@@ -107,7 +107,8 @@ def test_every_renamed_op_has_a_kernel_and_an_op_definition(opt):
     ops = ["Dequantize", "QuantizeV2", "QuantizedMatMulWithBias", "QuantizedMatMulWithBiasAndDequantize",
            "QuantizedMatMulWithBiasAndRelu", "QuantizedMatMulWithBiasAndReluAndRequantize", "QuantizedMatMulWithBiasAndRequantize",
            "_QuantizedBatchMatMul", "_QuantizedBatchMatMulV2AndDequantize", "_QuantizedFusedBatchMatMulV2AndDequantize",
-           "_QuantizedFusedMatMul", "_QuantizedFusedMatMulAndDequantize", "_QuantizedFusedMatMulAndRequantize", "_QuantizedMatMul"]
+           "_QuantizedFusedMatMul", "_QuantizedFusedMatMulAndDequantize", "_QuantizedFusedMatMulAndRequantize", "_QuantizedMatMul",
+           "QuantizedReshape", "_QuantizedTranspose"]
     g = gd.GraphDef()
     for i, op in enumerate(ops):
         gd.node(g, "n%d" % i, op, ["x"], DEV, mode="SCALED", T=("type", QINT8))
@@ -116,6 +117,14 @@ def test_every_renamed_op_has_a_kernel_and_an_op_definition(opt):
         assert n.op == "_ITEX" + op.lstrip("_"), (op, n.op)
         assert n.op in kernels, n.op
         assert n.op in defined, n.op
+
+
+def test_reshape_is_only_renamed_for_qint8(opt):
+    g = gd.GraphDef()
+    gd.node(g, "a", "QuantizedReshape", ["x", "s", "mn", "mx"], DEV, T=("type", QINT8))
+    gd.node(g, "b", "QuantizedReshape", ["x", "s", "mn", "mx"], DEV, T=("type", QUINT8))   # layout_utils.cc:392-400
+    out = by_name(run(opt, g))
+    assert out["a"].op == "_ITEXQuantizedReshape" and out["b"].op == "QuantizedReshape"
 
 
 def test_switch_and_malformed_input(opt, monkeypatch):

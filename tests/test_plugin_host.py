@@ -189,3 +189,13 @@ def test_batch_matmul_registrations(reg):
     names = {o["name"] for o in reg["ops"]}
     assert {"_QuantizedBatchMatMul", "_QuantizedBatchMatMulV2AndDequantize", "_QuantizedFusedBatchMatMulV2AndDequantize",
             "_ITEXQuantizedBatchMatMulV2AndDequantize"} <= names
+
+
+def test_shape_op_registrations(reg):
+    for op, host in (("_QuantizedTranspose", ["perm", "min_x", "max_x", "min_y", "max_y"]),
+                     ("QuantizedReshape", ["shape", "input_min", "input_max", "output_min", "output_max"])):
+        ks = kernels_of(reg, op)
+        assert {k["constraints"]["T"] for k in ks} == {tf.QINT8, tf.QUINT8, tf.QINT32}
+        assert all(k["host_memory"] == host for k in ks)
+    names = {o["name"] for o in reg["ops"]}
+    assert "_QuantizedTranspose" in names and "_ITEXQuantizedReshape" in names and "QuantizedReshape" not in names
