@@ -245,6 +245,7 @@ class BmmBinary(C.Structure):
 
 
 BIN_MUL, BIN_ADD = 1, 2
+ELT_RELU, ELT_CLIP, ELT_LINEAR, ELT_GELU_TANH, ELT_GELU_ERF, ELT_SUM = 1, 2, 3, 4, 5, 6
 
 
 def qbatch_matmul(x, y, min_x, max_x, min_y, max_y, adj_x=False, adj_y=False, binary=(), t_out=FLOAT):

@@ -251,6 +251,36 @@ def test_epilogue_against_torch_onednn():
                                   orc.qmatmul_epilogue(acc, ep, sw, b, orc.FLOAT))
 
 
+@pytest.mark.parametrize("algo,alg", [("tanh", orc.ELT_GELU_TANH), ("none", orc.ELT_GELU_ERF)])
+def test_gelu_post_ops_against_torch_onednn(algo, alg):
+    """The GELU post-ops are the one place where the oracle (libm tanhf / erff) cannot claim oneDNN's bits: oneDNN
+    evaluates them with its own polynomial kernels.  Against the oneDNN bundled with PyTorch (3.x, another build than
+    the reference pins) the oracle agrees on more than 90 % of the elements bit for bit and everywhere to 1e-6
+    absolute - the tolerance the GPU tests use for these two post-ops."""
+    torch = pytest.importorskip("torch")
+    if not hasattr(torch.ops, "onednn") or not hasattr(torch.ops.onednn, "qlinear_pointwise"):
+        pytest.skip("torch.ops.onednn.qlinear_pointwise unavailable")
+    rng = np.random.default_rng(13)
+    M, K, N = 64, 64, 64
+    xq = rng.integers(0, 256, size=(M, K)).astype(np.uint8)
+    wq = rng.integers(-127, 128, size=(K, N)).astype(np.int8)
+    sw = (rng.random(N).astype(np.float32) * 0.0005 + 0.00005)      # pre-activations spread over about [-100, 100]
+    b = (rng.standard_normal(N) * 0.5).astype(np.float32)
+    try:
+        packed = torch.ops.onednn.qlinear_prepack(torch.from_numpy(np.ascontiguousarray(wq.T)), [M, K])
+        y = torch.ops.onednn.qlinear_pointwise(torch.from_numpy(xq), 1.0, 0, packed, torch.from_numpy(sw),
+                                               torch.zeros(N, dtype=torch.int64), torch.from_numpy(b), 1.0, 0, torch.float32,
+                                               "gelu", [], algo).numpy()
+    except Exception as e:
+        pytest.skip("qlinear_pointwise with a gelu post-op not callable here: %r" % (e,))
+    ep = orc.EpilogueDesc()
+    ep.n_scales, ep.n_eltwise = N, 1
+    ep.elt[0].alg, ep.elt[0].alpha, ep.elt[0].beta = alg, 0.0, 0.0
+    ref = orc.qmatmul_epilogue(orc.int_gemm(xq, wq), ep, sw, b, orc.FLOAT)
+    np.testing.assert_allclose(y, ref, rtol=0, atol=1e-6)
+    assert (y.view(np.int32) == ref.view(np.int32)).mean() > 0.9
+
+
 # ------------------------------------------------------------------------------------------------
 # "Add" (sum post-op), GELU post-ops and the qint32 bias
 # ------------------------------------------------------------------------------------------------
