@@ -251,6 +251,32 @@ def test_epilogue_against_torch_onednn():
                                   orc.qmatmul_epilogue(acc, ep, sw, b, orc.FLOAT))
 
 
+@pytest.mark.parametrize("T16", [orc.BFLOAT16, orc.HALF])
+def test_16_bit_outputs_against_torch_onednn(T16):
+    """bfloat16 / half destination of an int8 inner product in the oneDNN bundled with PyTorch: the fp32 epilogue
+    result narrowed with round-to-nearest-even, bit for bit what the oracle stores."""
+    torch = pytest.importorskip("torch")
+    if not hasattr(torch.ops, "onednn") or not hasattr(torch.ops.onednn, "qlinear_pointwise"):
+        pytest.skip("torch.ops.onednn.qlinear_pointwise unavailable")
+    rng = np.random.default_rng(5)
+    M, K, N = 64, 64, 64
+    xq = rng.integers(0, 256, size=(M, K)).astype(np.uint8)
+    wq = rng.integers(-127, 128, size=(K, N)).astype(np.int8)
+    sw = (rng.random(N).astype(np.float32) * 0.01 + 0.001)
+    b = rng.standard_normal(N).astype(np.float32)
+    try:
+        packed = torch.ops.onednn.qlinear_prepack(torch.from_numpy(np.ascontiguousarray(wq.T)), [M, K])
+        y = torch.ops.onednn.qlinear_pointwise(torch.from_numpy(xq), 1.0, 0, packed, torch.from_numpy(sw),
+                                               torch.zeros(N, dtype=torch.int64), torch.from_numpy(b), 1.0, 0,
+                                               torch.bfloat16 if T16 == orc.BFLOAT16 else torch.float16, "none", [], "")
+    except Exception as e:
+        pytest.skip("qlinear_pointwise with a 16-bit output not callable here: %r" % (e,))
+    ep = orc.EpilogueDesc()
+    ep.n_scales = N
+    np.testing.assert_array_equal(y.view(torch.int16).numpy().view(np.uint16),
+                                  orc.qmatmul_epilogue(orc.int_gemm(xq, wq), ep, sw, b, T16))
+
+
 @pytest.mark.parametrize("algo,alg", [("tanh", orc.ELT_GELU_TANH), ("none", orc.ELT_GELU_ERF)])
 def test_gelu_post_ops_against_torch_onednn(algo, alg):
     """The GELU post-ops are the one place where the oracle (libm tanhf / erff) cannot claim oneDNN's bits: oneDNN
