@@ -251,6 +251,33 @@ def test_epilogue_against_torch_onednn():
                                   orc.qmatmul_epilogue(acc, ep, sw, b, orc.FLOAT))
 
 
+@pytest.mark.parametrize("post", ["sum", "add"])
+def test_sum_and_binary_add_post_ops_against_torch_onednn(post):
+    """The "Add" fusion (a sum post-op in the MatMul, a binary add in the BatchMatMul) in the oneDNN bundled with
+    PyTorch: one more separately rounded fp32 addition after scale and bias, bit for bit the oracle's result."""
+    torch = pytest.importorskip("torch")
+    if not hasattr(torch.ops, "onednn") or not hasattr(torch.ops.onednn, "qlinear_pointwise"):
+        pytest.skip("torch.ops.onednn.qlinear_pointwise unavailable")
+    rng = np.random.default_rng(7)
+    M, K, N = 32, 64, 48
+    xq = rng.integers(0, 256, size=(M, K)).astype(np.uint8)
+    wq = rng.integers(-127, 128, size=(K, N)).astype(np.int8)
+    sw = (rng.random(N).astype(np.float32) * 0.01 + 0.001)
+    b = rng.standard_normal(N).astype(np.float32)
+    other = rng.standard_normal((M, N)).astype(np.float32)
+    try:
+        packed = torch.ops.onednn.qlinear_prepack(torch.from_numpy(np.ascontiguousarray(wq.T)), [M, K])
+        y = torch.ops.onednn.qlinear_pointwise.binary(torch.from_numpy(xq), 1.0, 0, packed, torch.from_numpy(sw),
+                                                      torch.zeros(N, dtype=torch.int64), torch.from_numpy(other.copy()),
+                                                      torch.from_numpy(b), 1.0, 0, torch.float32, 1.0, 0, post, 1.0, "none", [], "")
+    except Exception as e:
+        pytest.skip("qlinear_pointwise.binary not callable here: %r" % (e,))
+    ep = orc.EpilogueDesc()
+    ep.n_scales, ep.n_eltwise = N, 1
+    ep.elt[0].alg, ep.elt[0].alpha, ep.elt[0].beta = orc.ELT_SUM, 1.0, 0.0
+    np.testing.assert_array_equal(y.numpy(), orc.qmatmul_epilogue(orc.int_gemm(xq, wq), ep, sw, b, orc.FLOAT, addend=other))
+
+
 @pytest.mark.parametrize("T16", [orc.BFLOAT16, orc.HALF])
 def test_16_bit_outputs_against_torch_onednn(T16):
     """bfloat16 / half destination of an int8 inner product in the oneDNN bundled with PyTorch: the fp32 epilogue
