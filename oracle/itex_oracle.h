@@ -18,8 +18,12 @@
  *      dequantize_op_test.py:102-170).
  *   - integer GEMM: brute force against numpy int64.
  *   - parameter math: closed forms evaluated independently in numpy float32/float64.
- *   - epilogue order (multiply, then add, separately rounded; saturate; RNE) is cross-checked
- *     against the oneDNN build bundled with PyTorch where that is importable.
+ *   - epilogue order (multiply, then add, separately rounded; saturate; RNE), the sum / binary-add
+ *     post-op, and the bfloat16 / half destination conversion are cross-checked bit for bit against
+ *     the oneDNN build bundled with PyTorch where that is importable; the GELU post-ops agree
+ *     with it to 1e-6 absolute (more than 90 % of elements bit for bit).
+ *   - quantized BatchMatMul: numpy int64 matmul on broadcast operands; the three cases of the
+ *     reference's quantized_batch_matmul_test.py.
  * Parity unpinned (no reference-held vector and no way to execute oneDNN@242d4d9 here):
  *   NaN / Inf inputs to the quantizers; the result of the size-mismatched bias reorder in
  *   orc_qmatmul_prepare (SCALED input, per-channel weights; see the comment there);
