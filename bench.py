@@ -325,6 +325,28 @@ def cpu_baseline_gemm(ctx, M_sample, K, N):
     return 2.0 * M_sample * K * N / dt / 1e12, dt, y
 
 
+def cpu_onednn_in_torch(torch, xq_host, wq_host, w_scale, bias):
+    """The closest executable stand-in for the reference's CPU path on this host: the oneDNN int8 inner product
+    bundled with PyTorch (another oneDNN build than the reference pins; not ITEX).  u8 x s8 per channel, fp32 bias,
+    fp32 output.  Returns (TOP/s, threads) or None when that operator is not callable."""
+    try:
+        M, K = xq_host.shape
+        N = wq_host.shape[1]
+        x = torch.from_numpy(xq_host)
+        packed = torch.ops.onednn.qlinear_prepack(torch.from_numpy(wq_host.T.copy()), [M, K])
+        args = (x, 1.0, 0, packed, torch.from_numpy(w_scale), torch.zeros(N, dtype=torch.int64), torch.from_numpy(bias),
+                1.0, 0, torch.float32, "none", [], "")
+        torch.ops.onednn.qlinear_pointwise(*args)
+        best = 1e30
+        for _ in range(3):
+            t0 = time.perf_counter()
+            torch.ops.onednn.qlinear_pointwise(*args)
+            best = min(best, time.perf_counter() - t0)
+        return 2.0 * M * K * N / best / 1e12, torch.get_num_threads()
+    except Exception:
+        return None
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -370,6 +392,14 @@ def main():
         cpu = dict(value=tops_cpu, unit="TOP/s", cores=cores, kind="port",
                    sample="first %d of %d rows of the headline workload (same weights), %.1f s; GPU rows identical: %s"
                           % (rows, M, dt, same))
+        L = ctx["layers"][0]
+        alt = cpu_onednn_in_torch(torch, ctx["xq"][:rows].cpu().numpy(), L["wq"].cpu().numpy(),
+                                  (L["max_b"].cpu().numpy() / 127.0).astype("float32"), L["bias"].cpu().numpy())
+        if alt:
+            cpu["onednn_in_torch"] = dict(value=alt[0], unit="TOP/s", threads=alt[1],
+                                          note="torch.ops.onednn.qlinear_pointwise (oneDNN bundled with PyTorch, fp32 output) "
+                                               "on the same rows and weights: the nearest executable relative of the "
+                                               "reference's CPU path, not ITEX itself")
     del ctx
 
     if "prefill" in only:
