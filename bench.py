@@ -288,6 +288,52 @@ def bench_bmm(torch, hip, timer, steps, warmup, dev):
     return out
 
 
+def bench_conv(torch, hip, timer, steps, warmup, dev):
+    """Quantized Conv2D [BiasAdd, Relu, Requantize] quint8 -> quint8 at two ResNet-50 layer shapes, batch 32: the patch
+    matrix (itexhip_im2col8) plus the quantized GEMM, as the op kernel runs them; the 1x1 layer needs no patches.
+    Algorithmic bytes = input + filter + output (the patch matrix is this implementation's own extra traffic)."""
+    out = []
+    g_ = torch.Generator(device=dev)
+    g_.manual_seed(50)
+    st = _stream(torch)
+    for name, (B, H, W, C), (KH, KW, O), stride in (("conv3x3_56x56x64_to_64", (32, 56, 56, 64), (3, 3, 64), 1),
+                                                    ("conv1x1_56x56x256_to_64", (32, 56, 56, 256), (1, 1, 64), 1)):
+        x = torch.randint(0, 256, (B, H, W, C), dtype=torch.uint8, device=dev, generator=g_)
+        w = torch.randint(-127, 128, (KH * KW * C, O), dtype=torch.int8, device=dev, generator=g_)
+        K = KH * KW * C
+        M = B * H * W
+        packed = torch.empty(hip.qgemm_packed_bytes(K, O), dtype=torch.int8, device=dev)
+        colsum = torch.empty(O, dtype=torch.int32, device=dev)
+        hip.qgemm_prepack_b(w, False, K, O, packed, colsum, st)
+        scales = torch.full((O,), 1e-4, dtype=torch.float32, device=dev)
+        bias = torch.zeros(O, dtype=torch.float32, device=dev)
+        ep = hip.Epilogue()
+        ep.n_scales, ep.n_eltwise = O, 1
+        ep.elt[0].alg, ep.elt[0].alpha, ep.elt[0].beta = hip.ELT_RELU, 0.0, 0.0
+        y = torch.empty((M, O), dtype=torch.uint8, device=dev)
+        pad = (KH - 1) // 2
+        geo = hip.ConvGeometry(B, H, W, C, KH, KW, H, W, stride, stride, 1, 1, pad, pad)
+        cols = torch.empty((M, K), dtype=torch.uint8, device=dev) if KH * KW > 1 else None
+
+        def make(stream):
+            def fn(i):
+                a = x
+                if cols is not None:
+                    hip.im2col8(x, geo, K, cols, stream)
+                    a = cols
+                hip.qgemm(a, hip.QUINT8, packed, colsum, M, K, O, scales, bias, ep, hip.QUINT8, y, stream)
+            return fn
+        ms = timer.run_graph(make, steps, warmup)
+        nbytes = x.numel() + w.numel() + y.numel()
+        ops = 2 * M * K * O
+        t_roof = max(ops / (PEAK_INT8_TOPS * 1e12), nbytes / (PEAK_HBM_GBS * 1e9))
+        out.append(dict(name=name, M=M, K=K, N=O, us_kernel=ms * 1e3, bytes=nbytes, ops=ops, bound="max(mfma,hbm)",
+                        frac=t_roof / (ms * 1e-3), tops=ops / (ms * 1e-3) / 1e12, gbs=nbytes / (ms * 1e-3) / 1e9,
+                        note="im2col + GEMM launches" if cols is not None else "GEMM launch only"))
+        del x, w, packed, y, cols
+    return out
+
+
 def bench_mfma_ceiling(torch, hip, timer, xq, wq, dev):
     """Matrix-pipe-only rate for operand bits like the workload's (bytes of the quantized activations,
     sign-flipped as the kernel feeds them, and of the weights) and for constant operands."""
@@ -352,14 +398,14 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--only", type=str, default="", help="comma list of: headline, prefill, bert, bmm, gemv, elementwise, copy")
+    ap.add_argument("--only", type=str, default="", help="comma list of: headline, prefill, bert, bmm, conv, gemv, elementwise, copy")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-rows", type=int, default=2048, help="rows of the headline workload the CPU oracle runs")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU only: this build has no multi-GPU path (--gpus must be 1)", file=sys.stderr)
         sys.exit(2)
-    only = set(s for s in args.only.split(",") if s) or {"headline", "prefill", "bert", "bmm", "gemv", "elementwise"}
+    only = set(s for s in args.only.split(",") if s) or {"headline", "prefill", "bert", "bmm", "conv", "gemv", "elementwise"}
 
     torch, hip = _setup()
     dev = torch.device("cuda:0")
@@ -419,6 +465,8 @@ def main():
             others.append(r)
     if "bmm" in only:
         others.extend(bench_bmm(torch, hip, timer, K_steps, W, dev))
+    if "conv" in only:
+        others.extend(bench_conv(torch, hip, timer, K_steps, W, dev))
     if "gemv" in only:
         for (k, n) in ((4096, 14336), (14336, 4096)):
             for m in (1, 4, 16):

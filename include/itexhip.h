@@ -338,6 +338,28 @@ int itexhip_qbatch_matmul(const itexhip_bmm_params* p, const int8_t* x, const in
 int itexhip_transpose(const void* x, void* y, int elem_size, int rank, const int64_t* dims, const int32_t* perm,
                       void* stream);
 
+/* ---- quantized Conv2D --------------------------------------------------------------------------
+ * The quantized convolutions (QuantizedConv2D*, _QuantizedConv2D; itex/core/kernels/common/
+ * quantized_conv_ops.h:63-597 over the oneDNN convolution primitive, conv_ops.h:615-1150) run here as
+ * patch matrix x prepacked filter: itexhip_im2col8 lays the receptive field of every output position out as
+ * one row, k = (kh * KW + kw) * C + c, which is the row order of the HWIO filter read as a [KH*KW*C, O] matrix,
+ * so itexhip_qgemm_prepack_b packs the filter as it is and itexhip_qgemm does the rest.  Quantization is
+ * SCALED (zero points are 0): padding positions hold the integer 0. */
+typedef struct {
+  int64_t batch, in_h, in_w, in_c;   /* NHWC input */
+  int64_t k_h, k_w;                  /* filter window */
+  int64_t out_h, out_w;              /* output extent (the caller applies the padding rule) */
+  int stride_h, stride_w, dil_h, dil_w;
+  int64_t pad_top, pad_left;         /* leading padding */
+} itexhip_conv_geometry;
+/* cols: [batch * out_h * out_w, row_bytes] bytes; row_bytes >= k_h * k_w * in_c, a multiple of 16; the tail of
+ * every row is zero-filled.  1-byte elements (qint8 / quint8). */
+int itexhip_im2col8(const void* x, const itexhip_conv_geometry* g, int64_t row_bytes, void* cols, void* stream);
+/* out[j] = float(bias[j]) * factors[n_factors == 1 ? 0 : j], j < n: the reorder with source scales that the
+ * reference applies to the bias (quantized_conv_ops.h:560-590).  bias_type ITEXHIP_FLOAT or ITEXHIP_QINT32. */
+int itexhip_scale_vector(const void* bias, int bias_type, const float* factors, int64_t n_factors, int64_t n,
+                         float* out, void* stream);
+
 /* Diagnostic, no counterpart in the reference: `workgroups` x 4 wavefronts each issue iters x 8
  * independent 32x32x32 i8 MFMAs (2 * 32768 ops each) on the 8 KiB of operand fragments at `operands`
  * (device memory, 16-byte aligned) and nothing else.  Timed by the caller, it gives the rate the matrix

@@ -126,6 +126,8 @@ void TF_OpKernelConstruction_GetAttrStringList(TF_OpKernelConstruction* ctx, con
                                                void* storage, size_t storage_size, TF_Status* status);
 void TF_OpKernelConstruction_GetAttrTypeList(TF_OpKernelConstruction* ctx, const char* attr_name,
                                              TF_DataType* vals, int max_vals, TF_Status* status);
+void TF_OpKernelConstruction_GetAttrInt64List(TF_OpKernelConstruction* ctx, const char* attr_name, int64_t* vals,
+                                              int max_vals, TF_Status* status);
 TF_StringView TF_OpKernelConstruction_GetName(TF_OpKernelConstruction* ctx);
 void TF_OpKernelConstruction_Failure(TF_OpKernelConstruction* ctx, TF_Status* status);
 

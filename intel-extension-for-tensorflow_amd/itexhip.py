@@ -29,7 +29,7 @@ EXPORTS = [
     "itexhip_requantize", "itexhip_minmax_i32_per_channel", "itexhip_minmax_f32",
     "itexhip_qmatmul_epilogue_desc", "itexhip_qmatmul_prepare", "itexhip_qgemm_packed_bytes",
     "itexhip_qgemm_prepack_b", "itexhip_qgemm", "itexhip_qgemm_tile", "itexhip_qgemv", "itexhip_qmatmul", "itexhip_qmatmul_per_row", "itexhip_qmatmul_unpacked", "itexhip_mfma_probe",
-    "itexhip_qgemm_naive", "itexhip_qbatch_matmul", "itexhip_transpose",
+    "itexhip_qgemm_naive", "itexhip_qbatch_matmul", "itexhip_transpose", "itexhip_im2col8", "itexhip_scale_vector",
 ]
 
 
@@ -319,3 +319,16 @@ def transpose(x, y, elem_size, dims, perm, stream=0):
     d = (C.c_int64 * max(rank, 1))(*dims)
     pm = (C.c_int32 * max(rank, 1))(*perm)
     _check(_lib.itexhip_transpose(_ptr(x), _ptr(y), int(elem_size), rank, d, pm, _ptr(stream)))
+
+
+class ConvGeometry(C.Structure):
+    _fields_ = [(n, C.c_int64) for n in ("batch", "in_h", "in_w", "in_c", "k_h", "k_w", "out_h", "out_w")] + \
+               [(n, C.c_int) for n in ("stride_h", "stride_w", "dil_h", "dil_w")] + [("pad_top", C.c_int64), ("pad_left", C.c_int64)]
+
+
+def im2col8(x, geometry, row_bytes, cols, stream=0):
+    _check(_lib.itexhip_im2col8(_ptr(x), C.byref(geometry), _i64(row_bytes), _ptr(cols), _ptr(stream)))
+
+
+def scale_vector(bias, bias_type, factors, n_factors, n, out, stream=0):
+    _check(_lib.itexhip_scale_vector(_ptr(bias), int(bias_type), _ptr(factors), _i64(n_factors), _i64(n), _ptr(out), _ptr(stream)))

@@ -187,6 +187,12 @@ std::string MakeAttrBool(bool b) {
   return v;
 }
 
+std::string MakeAttrString(const std::string& s) {
+  std::string v;
+  PutBytes(&v, 2, s);
+  return v;
+}
+
 std::string MakeAttrType(int t) {
   std::string v;
   PutVarint(&v, (6u << 3) | 0);

@@ -41,6 +41,7 @@ bool AttrString(const std::string& value, std::string* s);
 bool AttrBool(const std::string& value, bool* b);
 bool AttrType(const std::string& value, int* t);
 std::string MakeAttrBool(bool b);
+std::string MakeAttrString(const std::string& s);
 std::string MakeAttrType(int t);
 
 }  // namespace graph

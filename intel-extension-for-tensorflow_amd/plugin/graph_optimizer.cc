@@ -19,7 +19,7 @@ namespace {
 
 constexpr int kDtFloat = 1, kDtQint8 = 11, kDtQuint8 = 12;
 
-enum class Copy { kAll, kQuantize, kQuantizedMatMul };
+enum class Copy { kAll, kQuantize, kQuantizedMatMul, kQuantizedConv2D };
 enum class Rule { kAlways, kQuantize, kQint8Only };
 
 struct Rename {
@@ -33,6 +33,14 @@ struct Rename {
 const Rename kTable[] = {
     {"Dequantize", "_ITEXDequantize", Copy::kAll, Rule::kQuantize},
     {"QuantizeV2", "_ITEXQuantizeV2", Copy::kQuantize, Rule::kQuantize},
+    {"QuantizedConv2D", "_ITEXQuantizedConv2D", Copy::kQuantizedConv2D, Rule::kAlways},
+    {"QuantizedConv2DAndRequantize", "_ITEXQuantizedConv2DAndRequantize", Copy::kQuantizedConv2D, Rule::kAlways},
+    {"QuantizedConv2DPerChannel", "_ITEXQuantizedConv2DPerChannel", Copy::kQuantizedConv2D, Rule::kAlways},
+    {"QuantizedConv2DWithBias", "_ITEXQuantizedConv2DWithBias", Copy::kQuantizedConv2D, Rule::kAlways},
+    {"QuantizedConv2DWithBiasAndRelu", "_ITEXQuantizedConv2DWithBiasAndRelu", Copy::kQuantizedConv2D, Rule::kAlways},
+    {"QuantizedConv2DWithBiasAndReluAndRequantize", "_ITEXQuantizedConv2DWithBiasAndReluAndRequantize", Copy::kQuantizedConv2D, Rule::kAlways},
+    {"QuantizedConv2DWithBiasAndRequantize", "_ITEXQuantizedConv2DWithBiasAndRequantize", Copy::kQuantizedConv2D, Rule::kAlways},
+    {"_QuantizedConv2D", "_ITEXQuantizedConv2DV2", Copy::kAll, Rule::kAlways},
     {"QuantizedMatMulWithBias", "_ITEXQuantizedMatMulWithBias", Copy::kQuantizedMatMul, Rule::kAlways},
     {"QuantizedMatMulWithBiasAndDequantize", "_ITEXQuantizedMatMulWithBiasAndDequantize", Copy::kQuantizedMatMul, Rule::kAlways},
     {"QuantizedMatMulWithBiasAndRelu", "_ITEXQuantizedMatMulWithBiasAndRelu", Copy::kQuantizedMatMul, Rule::kAlways},
@@ -145,6 +153,7 @@ void Optimize(void* opt, const TF_Buffer* in, const TF_GrapplerItem*, TF_Buffer*
       if (!n.FindAttr("dtype")) n.SetAttr("dtype", graph::MakeAttrType(kDtFloat));
       n.SetAttr("classic_asymmetric_algorithm", graph::MakeAttrBool(classic[i]));
     }
+    if (plan[i]->copy == Copy::kQuantizedConv2D) n.SetAttr("data_format", graph::MakeAttrString("NHWC"));  // :471-495
     // CopyAttrsQuantizedMatMul (:497-515) copies every attribute and then Tbias once more: nothing to add
   }
 

@@ -108,6 +108,17 @@ bool OpKernelConstruction::GetAttr(const char* name, std::vector<std::string>* v
   return true;
 }
 
+bool OpKernelConstruction::GetAttr(const char* name, std::vector<int64_t>* v) {
+  StatusPtr st;
+  int32_t list_size = 0, total_size = 0;
+  TF_OpKernelConstruction_GetAttrSize(ctx_, name, &list_size, &total_size, st);
+  if (!Check(st)) return false;
+  v->assign(static_cast<size_t>(list_size > 0 ? list_size : 0), 0);
+  if (list_size <= 0) return true;
+  TF_OpKernelConstruction_GetAttrInt64List(ctx_, name, v->data(), list_size, st);
+  return Check(st);
+}
+
 // ---- compute (op_kernel.cc:108-129, 234-238, 333-340, 437-443, 511-518; op_kernel.h:406) -------
 void OpKernelContext::CtxFailure(TF_Code code, const std::string& msg) {
   StatusPtr st;

@@ -58,6 +58,7 @@ class OpKernelConstruction {
   bool GetAttr(const char* name, float* v);
   bool GetAttr(const char* name, TF_DataType* v);
   bool GetAttr(const char* name, std::vector<std::string>* v);
+  bool GetAttr(const char* name, std::vector<int64_t>* v);
   void CtxFailure(TF_Code code, const std::string& msg);
   bool ok() const { return ok_; }
   std::string name() const;
@@ -159,6 +160,7 @@ void AddDequantizeKernels();
 void AddQuantizedMatMulKernels();
 void AddQuantizedBatchMatMulKernels();
 void AddQuantizedShapeKernels();
+void AddQuantizedConvKernels();
 void AddRequantizeKernels();
 // op definitions for the ops stock TensorFlow does not have
 void RegisterOps();

@@ -170,6 +170,45 @@ std::vector<OpSpec> OpSpecs() {
     v.push_back({"_ITEXQuantizedMatMulWithBiasAndDequantize", in9, {"out: Toutput"},
                  attrs("Tbias: {float, bfloat16, qint32}", "Toutput: {float, bfloat16}")});
   }
+  // quantized Conv2D: the list-attribute form (nn_ops.cc: _QuantizedConv2D, _ITEXQuantizedConv2DV2) and the _ITEX twins
+  // of TensorFlow's QuantizedConv2D* ops
+  for (const char* name : {"_QuantizedConv2D", "_ITEXQuantizedConv2DV2"})
+    v.push_back({name,
+                 {"device_inputs: Tdevice_inputs", "host_inputs: Thost_inputs"},
+                 {"device_outputs: Tdevice_outputs", "host_outputs: Thost_outputs"},
+                 {"Tinput: quantizedtype = DT_QUINT8", "Tfilter: quantizedtype = DT_QINT8", "Tbias: {float, qint32} = DT_QINT32",
+                  "Tsummand: {float, quint8, qint8, qint32, bfloat16}", "out_type: {qint8, quint8, qint32, float, bfloat16}",
+                  "Tdevice_inputs: list(type) >= 0 = []", "Thost_inputs: list(type) >= 0", "Tdevice_outputs: list(type) >= 0 = []",
+                  "Thost_outputs: list(type) >= 0", "data_format: string = 'NHWC'", "strides: list(int)",
+                  "is_filter_const: bool = true", "is_bias_const: bool = true", "padding: {'SAME', 'VALID', 'EXPLICIT'}",
+                  "explicit_paddings: list(int) = []", "dilations: list(int) = [1, 1, 1, 1]", "fused_ops: list(string) = []",
+                  "alpha: float = 0.0"}});
+  {
+    const std::vector<const char*> base_attrs = {"Tinput: quantizedtype", "Tfilter: quantizedtype", "strides: list(int)",
+                                                 "padding: {'SAME', 'VALID'}", "dilations: list(int) = [1, 1, 1, 1]",
+                                                 "padding_list: list(int) = []", "is_filter_const: bool = true"};
+    struct Twin { const char* name; bool bias, req; const char* out_default; };
+    for (const Twin& t : {Twin{"_ITEXQuantizedConv2D", false, false, "out_type: quantizedtype = DT_QINT32"},
+                          Twin{"_ITEXQuantizedConv2DPerChannel", false, false, "out_type: quantizedtype = DT_QINT32"},
+                          Twin{"_ITEXQuantizedConv2DWithBias", true, false, "out_type: quantizedtype = DT_QINT32"},
+                          Twin{"_ITEXQuantizedConv2DWithBiasAndRelu", true, false, "out_type: quantizedtype = DT_QINT32"},
+                          Twin{"_ITEXQuantizedConv2DAndRelu", false, false, "out_type: quantizedtype = DT_QINT32"},
+                          Twin{"_ITEXQuantizedConv2DAndRequantize", false, true, "out_type: quantizedtype = DT_QINT8"},
+                          Twin{"_ITEXQuantizedConv2DAndReluAndRequantize", false, true, "out_type: quantizedtype = DT_QUINT8"},
+                          Twin{"_ITEXQuantizedConv2DWithBiasAndRequantize", true, true, "out_type: quantizedtype = DT_QINT8"},
+                          Twin{"_ITEXQuantizedConv2DWithBiasAndReluAndRequantize", true, true, "out_type: quantizedtype = DT_QUINT8"}}) {
+      OpSpec s{t.name, {"input: Tinput", "filter: Tfilter"}, {"output: out_type", "min_output: float", "max_output: float"}, base_attrs};
+      if (t.bias) s.inputs.push_back(t.req ? "bias: Tbias" : "bias: float");
+      for (const char* in : {"min_input: float", "max_input: float", "min_filter: float", "max_filter: float"}) s.inputs.push_back(in);
+      if (t.req) {
+        s.inputs.push_back("min_freezed_output: float");
+        s.inputs.push_back("max_freezed_output: float");
+        if (t.bias) s.attrs.push_back("Tbias: {float, qint32}");
+      }
+      s.attrs.push_back(t.out_default);
+      v.push_back(s);
+    }
+  }
   // nn_ops.cc:562-585 (_QuantizedTranspose), :3266-3290 (_ITEXQuantizedReshape)
   for (const char* name : {"_QuantizedTranspose", "_ITEXQuantizedTranspose"})
     v.push_back({name,
@@ -225,6 +264,7 @@ extern "C" void TF_InitKernel(void) {
     AddQuantizedMatMulKernels();
     AddQuantizedBatchMatMulKernels();
     AddQuantizedShapeKernels();
+    AddQuantizedConvKernels();
     AddRequantizeKernels();
     // the device type the kernels attach to: ITEX's own PluggableDevice type by default, so that graphs
     // placed by ITEX's passes keep their device strings

@@ -1,0 +1,377 @@
+// Quantized Conv2D op kernels: QuantizedConv2D, ...PerChannel, ...WithBias, ...AndRelu, ...AndRequantize and
+// their combinations, and the list-attribute form _QuantizedConv2D / _ITEXQuantizedConv2DV2
+// (itex/core/kernels/common/quantized_conv_ops.h:63-597 over conv_ops.h:615-1150; device registrations in
+// itex/core/kernels/gpu/quantized_conv_ops.cc).  Host half as in the reference: attribute and fusion
+// parsing, input indices, geometry, output scales and bias factors; the convolution itself runs as
+// itexhip_im2col8 + itexhip_qgemm on the filter prepacked as a [KH*KW*C, O] matrix.
+// Not carried over: Sum / Elu / Swish / HardSwish / Sigmoid fusions, depthwise and 3-D variants, NCHW.
+#include <algorithm>
+#include <cmath>
+#include <cstring>
+#include <string>
+#include <vector>
+
+#include "device_vector_cache.h"
+#include "itexhip.h"
+#include "op_kernel.h"
+#include "qparams.h"
+
+namespace itex_amd {
+namespace {
+
+// fusions of the ops without a fused_ops attribute (quantized_conv_ops.h:44-60)
+std::vector<std::string> LegacyFusions(const std::string& op) {
+  std::string name = op;
+  if (name.rfind("_ITEX", 0) == 0) name = name.substr(5);
+  if (name == "QuantizedConv2D" || name == "QuantizedConv2DPerChannel") return {};
+  if (name == "QuantizedConv2DWithBias") return {"BiasAdd"};
+  if (name == "QuantizedConv2DWithBiasAndRelu") return {"BiasAdd", "Relu"};
+  if (name == "QuantizedConv2DAndRelu") return {"Relu"};
+  if (name == "QuantizedConv2DAndRequantize") return {"Requantize"};
+  if (name == "QuantizedConv2DAndReluAndRequantize") return {"Relu", "Requantize"};
+  if (name == "QuantizedConv2DWithBiasAndRequantize") return {"BiasAdd", "Requantize"};
+  if (name == "QuantizedConv2DWithBiasAndReluAndRequantize") return {"BiasAdd", "Relu", "Requantize"};
+  return {};
+}
+
+// TensorFlow's GetWindowedOutputSizeVerbose
+bool OutDim(int64_t in, int64_t k, int64_t stride, int64_t dil, const std::string& padding, int64_t before, int64_t after,
+            int64_t* out, int64_t* lead) {
+  const int64_t eff = (k - 1) * dil + 1;
+  if (padding == "VALID") {
+    *out = (in - eff + stride) / stride;
+    *lead = 0;
+  } else if (padding == "SAME") {
+    *out = (in + stride - 1) / stride;
+    *lead = std::max<int64_t>((*out - 1) * stride + eff - in, 0) / 2;
+  } else {
+    *out = (in + before + after - eff + stride) / stride;
+    *lead = before;
+  }
+  return *out >= 0;
+}
+
+class QuantizedConv2DOp : public OpKernel {
+ public:
+  QuantizedConv2DOp(OpKernelConstruction* ctx, const std::string& op, bool new_api, TF_DataType t_in, TF_DataType t_out)
+      : t_in_(t_in), t_out_(t_out) {
+    (void)new_api;
+    std::vector<int64_t> strides, dilations;
+    ITEX_REQUIRES_OK(ctx, ctx->GetAttr("dilations", &dilations));
+    ITEX_REQUIRES_OK(ctx, ctx->GetAttr("strides", &strides));
+    ITEX_REQUIRES(ctx, strides.size() == 4, TF_INVALID_ARGUMENT, "Sliding window strides field must specify 4 dimensions");
+    ITEX_REQUIRES(ctx, dilations.size() == 4, TF_INVALID_ARGUMENT, "Sliding window dilations field must specify 4 dimensions");
+    if (ctx->HasAttr("data_format")) {
+      std::string fmt;
+      ITEX_REQUIRES_OK(ctx, ctx->GetAttr("data_format", &fmt));
+      ITEX_REQUIRES(ctx, fmt == "NHWC" || fmt == "NCHW", TF_INVALID_ARGUMENT, "Invalid data format");
+      ITEX_REQUIRES(ctx, fmt == "NHWC", TF_UNIMPLEMENTED, "the quantized Conv2D on this device takes NHWC tensors");
+    }
+    ITEX_REQUIRES(ctx, strides[0] == 1 && strides[3] == 1, TF_UNIMPLEMENTED,
+                  "Current implementation does not yet support strides in the batch and depth dimensions.");
+    ITEX_REQUIRES(ctx, dilations[0] == 1 && dilations[3] == 1, TF_INVALID_ARGUMENT,
+                  "Current implementation does not yet support dilations in the batch and depth dimensions.");
+    ITEX_REQUIRES(ctx, strides[1] > 0 && strides[2] > 0, TF_INVALID_ARGUMENT, "Row and column strides should be larger than 0.");
+    ITEX_REQUIRES(ctx, dilations[1] > 0 && dilations[2] > 0, TF_INVALID_ARGUMENT, "Dilated rates should be larger than 0.");
+    stride_h_ = strides[1]; stride_w_ = strides[2]; dil_h_ = dilations[1]; dil_w_ = dilations[2];
+    ITEX_REQUIRES_OK(ctx, ctx->GetAttr("padding", &padding_));
+    ITEX_REQUIRES(ctx, padding_ == "SAME" || padding_ == "VALID" || padding_ == "EXPLICIT", TF_INVALID_ARGUMENT,
+                  "padding must be SAME, VALID or EXPLICIT");
+    for (const char* attr : {"explicit_paddings", "padding_list"})  // the second is the legacy spelling (:121-124)
+      if (ctx->HasAttr(attr)) {
+        std::vector<int64_t> p;
+        ITEX_REQUIRES_OK(ctx, ctx->GetAttr(attr, &p));
+        if (!p.empty()) explicit_ = p;
+      }
+    if (!explicit_.empty()) {  // conv_ops.h:412-427: explicit paddings win when present
+      ITEX_REQUIRES(ctx, explicit_.size() == 8, TF_INVALID_ARGUMENT, "explicit paddings must hold 8 values for a 2-D convolution");
+      ITEX_REQUIRES(ctx, explicit_[0] == 0 && explicit_[1] == 0 && explicit_[6] == 0 && explicit_[7] == 0, TF_INVALID_ARGUMENT,
+                    "explicit padding of the batch and depth dimensions must be 0");
+      padding_ = "EXPLICIT";
+    }
+    ITEX_REQUIRES(ctx, padding_ != "EXPLICIT" || explicit_.size() == 8, TF_INVALID_ARGUMENT, "EXPLICIT padding without paddings");
+
+    std::vector<std::string> fused;
+    if (ctx->HasAttr("fused_ops")) ITEX_REQUIRES_OK(ctx, ctx->GetAttr("fused_ops", &fused));
+    const std::vector<std::string> legacy = LegacyFusions(op);
+    ITEX_REQUIRES(ctx, !(fused.size() > 0 && legacy.size() > 0), TF_INVALID_ARGUMENT,
+                  "QuantizedConv fused ops should be only availabe through either new API or old API, got both.");
+    if (fused.empty()) fused = legacy;
+    for (const std::string& f : fused) {
+      if (f == "BiasAdd") fuse_bias_ = true;
+      else if (f == "Requantize") fuse_requantize_ = true;
+      else if (f == "Dequantize") fuse_dequantize_ = true;
+      else if (f == "Relu") activation_ = ITEXHIP_ELT_RELU;
+      else if (f == "LeakyRelu") { activation_ = ITEXHIP_ELT_RELU; leaky_ = true; }
+      else
+        ITEX_REQUIRES(ctx, false, TF_UNIMPLEMENTED, "the " + f + " fusion of the quantized Conv2D is not implemented on this device");
+    }
+    if (leaky_) ITEX_REQUIRES_OK(ctx, ctx->GetAttr("alpha", &alpha_));
+    if (fuse_requantize_)
+      ITEX_REQUIRES(ctx, t_out == TF_QINT8 || t_out == TF_QUINT8, TF_INVALID_ARGUMENT,
+                    "QuantizedConv: unsupported output type when Requantize is fused.");
+    if (fuse_dequantize_)
+      ITEX_REQUIRES(ctx, t_out == TF_FLOAT || t_out == TF_BFLOAT16, TF_INVALID_ARGUMENT,
+                    "QuantizedConv: unsupported output type when Dequantize is fused.");
+    if (fuse_bias_ && ctx->HasAttr("Tbias")) {
+      ITEX_REQUIRES_OK(ctx, ctx->GetAttr("Tbias", &t_bias_));
+      ITEX_REQUIRES(ctx, t_bias_ == TF_FLOAT || t_bias_ == TF_QINT32, TF_UNIMPLEMENTED,
+                    "the quantized Conv2D takes a float or qint32 bias on this device");
+    }
+    if (ctx->HasAttr("is_filter_const")) ITEX_REQUIRES_OK(ctx, ctx->GetAttr("is_filter_const", &is_filter_const_));
+
+    // input positions (:246-317)
+    const int bias_off = fuse_bias_ ? 1 : 0;
+    src_min_idx_ = 2 + bias_off;
+    filter_min_idx_ = src_min_idx_ + 2;
+    freezed_idx_ = 6 + bias_off;  // both spellings, without a summand and with a float / qint32 bias
+  }
+
+  void Compute(OpKernelContext* ctx) override {
+    Tensor x = ctx->input(0);
+    Tensor filter = ctx->input(1);
+    if (!ctx->ok()) return;
+    ITEX_REQUIRES(ctx, ctx->num_inputs() >= filter_min_idx_ + 2 && (!fuse_requantize_ || ctx->num_inputs() >= freezed_idx_ + 2),
+                  TF_INVALID_ARGUMENT, "the min / max inputs are missing");
+    Tensor min_in_t = ctx->input(src_min_idx_), max_in_t = ctx->input(src_min_idx_ + 1);
+    Tensor min_f_t = ctx->input(filter_min_idx_), max_f_t = ctx->input(filter_min_idx_ + 1);
+    if (!ctx->ok()) return;
+    ITEX_REQUIRES(ctx, x.dims() == 4 && filter.dims() == 4, TF_INVALID_ARGUMENT, "input and filter must be 4-dimensional");
+    ITEX_REQUIRES(ctx, x.dtype() == t_in_ && filter.dtype() == TF_QINT8, TF_INVALID_ARGUMENT,
+                  "quantized Conv2D operand types do not match the kernel");
+    const int64_t B = x.dim_size(0), H = x.dim_size(1), W = x.dim_size(2), C = x.dim_size(3);
+    const int64_t KH = filter.dim_size(0), KW = filter.dim_size(1), O = filter.dim_size(3);
+    ITEX_REQUIRES(ctx, filter.dim_size(2) == C, TF_INVALID_ARGUMENT,
+                  "input depth " + std::to_string(C) + " vs. filter input depth " + std::to_string(filter.dim_size(2)));
+    ITEX_REQUIRES(ctx, KH > 0 && KW > 0, TF_INVALID_ARGUMENT, "empty filter window");
+    const int64_t depth = min_f_t.NumElements();
+    ITEX_REQUIRES(ctx, max_f_t.NumElements() == depth && (depth == 1 || depth == O), TF_INVALID_ARGUMENT,
+                  "min_filter / max_filter must be scalars or hold one entry per output channel");
+
+    itexhip_conv_geometry g{};
+    g.batch = B; g.in_h = H; g.in_w = W; g.in_c = C; g.k_h = KH; g.k_w = KW;
+    g.stride_h = static_cast<int>(stride_h_); g.stride_w = static_cast<int>(stride_w_);
+    g.dil_h = static_cast<int>(dil_h_); g.dil_w = static_cast<int>(dil_w_);
+    const int64_t pt = explicit_.empty() ? 0 : explicit_[2], pb = explicit_.empty() ? 0 : explicit_[3];
+    const int64_t pl = explicit_.empty() ? 0 : explicit_[4], pr = explicit_.empty() ? 0 : explicit_[5];
+    ITEX_REQUIRES(ctx, OutDim(H, KH, stride_h_, dil_h_, padding_, pt, pb, &g.out_h, &g.pad_top) &&
+                           OutDim(W, KW, stride_w_, dil_w_, padding_, pl, pr, &g.out_w, &g.pad_left),
+                  TF_INVALID_ARGUMENT, "Computed output size would be negative");
+    const int64_t M = B * g.out_h * g.out_w, K = KH * KW * C, Kp = (K + 15) / 16 * 16;
+
+    // ---- output scales and bias factors (ExtendInt8PostOps :329-393, GetBiasHandle :448-597), fp32 on the host
+    const float min_in = min_in_t.flat<float>()[0], max_in = max_in_t.flat<float>()[0];
+    const float* min_f = min_f_t.flat<float>();
+    const float* max_f = max_f_t.flat<float>();
+    const bool out_q8 = t_out_ == TF_QINT8 || t_out_ == TF_QUINT8;
+    const bool out_f = t_out_ == TF_FLOAT || t_out_ == TF_BFLOAT16;
+    float min_out = 0.0f, max_out = 0.0f;
+    if (out_q8) {
+      ITEX_REQUIRES(ctx, fuse_requantize_, TF_INVALID_ARGUMENT, "an 8-bit output needs the Requantize fusion");
+      Tensor mo = ctx->input(freezed_idx_), xo = ctx->input(freezed_idx_ + 1);
+      if (!ctx->ok()) return;
+      min_out = mo.flat<float>()[0];
+      max_out = xo.flat<float>()[0];
+    }
+    std::vector<float> scales(depth, 1.0f), factors(depth, 1.0f);
+    const float in_range = std::max(std::abs(min_in), std::abs(max_in));
+    const float int_const_scale_limit = (t_in_ == TF_QUINT8) ? static_cast<float>(255.0 * 127.0) : static_cast<float>(127.0 * 127.0);
+    if (out_f) {
+      const float int_input_limit = (t_in_ == TF_QUINT8) ? 255.0f : 127.0f;
+      const float src_qscale_f32 = in_range / int_input_limit;
+      for (int64_t i = 0; i < depth; ++i) {
+        const float wei_qscale_f32 = std::max(std::abs(min_f[i]), std::abs(max_f[i])) / 127.0f;
+        scales[i] = src_qscale_f32 * wei_qscale_f32;
+      }
+    } else if (out_q8) {
+      const float int_output_limit = (t_out_ == TF_QUINT8) ? 255.0f : 127.0f;
+      const float float_output_range = std::max(std::abs(min_out), std::abs(max_out));
+      for (int64_t i = 0; i < depth; ++i) {
+        const float float_filter_range = std::max(std::abs(min_f[i]), std::abs(max_f[i]));
+        scales[i] = int_output_limit * in_range * float_filter_range / (int_const_scale_limit * float_output_range);
+      }
+    }
+    if (fuse_bias_) {
+      for (int64_t i = 0; i < depth; ++i) {
+        const float filt_range = std::max(std::abs(max_f[i]), std::abs(min_f[i]));
+        if (t_bias_ == TF_QINT32) {
+          factors[i] = t_out_ == TF_QINT32 ? 1.0f : out_f ? (in_range * filt_range) / int_const_scale_limit : scales[i];
+        } else {
+          const float tmp_scale = int_const_scale_limit / (in_range * filt_range);
+          factors[i] = tmp_scale * scales[i];
+        }
+      }
+    }
+
+    void* stream = ctx->stream();
+    // ---- filter: packed once when constant (the HWIO tensor read as a [K, O] matrix)
+    const bool repack = !packed_.valid() || !is_filter_const_ || packed_src_ != filter.data() || packed_k_ != K || packed_n_ != O;
+    if (repack && O > 0) {
+      packed_ = ctx->allocate_temp(TF_QINT8, {std::max<int64_t>(itexhip_qgemm_packed_bytes(Kp, O), 16)});
+      colsum_ = ctx->allocate_temp(TF_INT32, {O});
+      if (!ctx->ok()) return;
+      const int st = itexhip_qgemm_prepack_b(filter.flat<int8_t>(), 0, K, O, packed_.flat<int8_t>(), colsum_.flat<int32_t>(), stream);
+      ITEX_REQUIRES(ctx, st == ITEXHIP_OK, TF_ABORTED, std::string("Operation received an exception: ") + itexhip_last_error());
+      packed_src_ = filter.data();
+      packed_k_ = K;
+      packed_n_ = O;
+    }
+    std::vector<float> both(scales);
+    both.insert(both.end(), factors.begin(), factors.end());
+    float* params = params_.Get(ctx, both.data(), both.size(), TF_FLOAT);
+    if (params == nullptr) return;
+
+    Tensor out = ctx->allocate_output(0, t_out_, {B, g.out_h, g.out_w, O});
+    if (!ctx->ok()) return;
+    if (M > 0 && O > 0) {
+      // ---- bias in the epilogue's units
+      Tensor sbias;
+      const float* bias_dev = nullptr;
+      if (fuse_bias_) {
+        Tensor bias = ctx->input(2);
+        if (!ctx->ok()) return;
+        ITEX_REQUIRES(ctx, bias.dtype() == t_bias_ && bias.NumElements() == O, TF_INVALID_ARGUMENT,
+                      "bias must have one entry per output channel and the type of Tbias");
+        sbias = ctx->allocate_temp(TF_FLOAT, {O});
+        if (!ctx->ok()) return;
+        const int st = itexhip_scale_vector(bias.data(), t_bias_, params + depth, depth, O, sbias.flat<float>(), stream);
+        ITEX_REQUIRES(ctx, st == ITEXHIP_OK, TF_ABORTED, std::string("Operation received an exception: ") + itexhip_last_error());
+        bias_dev = sbias.flat<float>();
+      } else {
+        sbias = ctx->allocate_temp(TF_FLOAT, {O});   // the MFMA kernels' vector epilogue wants a bias vector: zeros
+        if (!ctx->ok()) return;
+        const int st = itexhip_memset32_async(sbias.data(), 0, static_cast<size_t>(O) * sizeof(float), stream);
+        ITEX_REQUIRES(ctx, st == ITEXHIP_OK, TF_ABORTED, std::string("Operation received an exception: ") + itexhip_last_error());
+        bias_dev = sbias.flat<float>();
+      }
+      // ---- patches, then the quantized GEMM
+      const void* a = x.data();
+      Tensor cols;
+      const bool pointwise = KH == 1 && KW == 1 && stride_h_ == 1 && stride_w_ == 1 && g.pad_top == 0 && g.pad_left == 0 &&
+                             g.out_h == H && g.out_w == W && K == Kp;
+      if (!pointwise) {
+        cols = ctx->allocate_temp(t_in_, {M, Kp});
+        if (!ctx->ok()) return;
+        const int st = itexhip_im2col8(x.data(), &g, Kp, cols.data(), stream);
+        ITEX_REQUIRES(ctx, st == ITEXHIP_OK, TF_ABORTED, std::string("Operation received an exception: ") + itexhip_last_error());
+        a = cols.data();
+      }
+      itexhip_epilogue ep{};
+      ep.n_scales = static_cast<int>(depth);
+      if (activation_ != 0) {
+        ep.n_eltwise = 1;
+        ep.elt[0].alg = activation_;
+        ep.elt[0].alpha = leaky_ ? alpha_ : 0.0f;
+        ep.elt[0].beta = 0.0f;
+      }
+      const int st = itexhip_qgemm(a, t_in_, packed_.flat<int8_t>(), colsum_.flat<int32_t>(), M, Kp, O, params, bias_dev, &ep,
+                                   t_out_, out.data(), stream);
+      ITEX_REQUIRES(ctx, st == ITEXHIP_OK, st == ITEXHIP_INVALID_ARGUMENT ? TF_INVALID_ARGUMENT : TF_ABORTED,
+                    std::string("Operation received an exception: ") + itexhip_last_error());
+    }
+
+    // ---- output ranges in host memory (AllocateNativeOutputMinMax, quantized_ops.h:142-203)
+    if (out_q8) {
+      Tensor omin = ctx->allocate_output(1, TF_FLOAT, {});
+      Tensor omax = ctx->allocate_output(2, TF_FLOAT, {});
+      if (!ctx->ok()) return;
+      omin.flat<float>()[0] = min_out;
+      omax.flat<float>()[0] = max_out;
+    } else if (t_out_ == TF_QINT32) {
+      const bool scalar = min_f_t.dims() == 0;
+      const std::vector<int64_t> shp = scalar ? std::vector<int64_t>{} : std::vector<int64_t>{depth};
+      Tensor omin = ctx->allocate_output(1, TF_FLOAT, shp);
+      Tensor omax = ctx->allocate_output(2, TF_FLOAT, shp);
+      if (!ctx->ok()) return;
+      for (int64_t i = 0; i < (scalar ? 1 : depth); ++i)
+        qparams::RangeForMultiplication(t_in_, TF_QINT8, min_in, max_in, min_f[i], max_f[i], &omin.flat<float>()[i],
+                                        &omax.flat<float>()[i]);
+    }
+  }
+
+ private:
+  TF_DataType t_in_, t_out_, t_bias_ = TF_FLOAT;
+  int64_t stride_h_ = 1, stride_w_ = 1, dil_h_ = 1, dil_w_ = 1;
+  std::string padding_;
+  std::vector<int64_t> explicit_;
+  bool fuse_bias_ = false, fuse_requantize_ = false, fuse_dequantize_ = false, leaky_ = false;
+  int activation_ = 0;
+  float alpha_ = 0.0f;
+  bool is_filter_const_ = true;
+  int src_min_idx_ = 2, filter_min_idx_ = 4, freezed_idx_ = 6;
+  Tensor packed_, colsum_;
+  const void* packed_src_ = nullptr;
+  int64_t packed_k_ = -1, packed_n_ = -1;
+  DeviceVectorCache<float> params_;
+};
+
+// the op name is needed at construction (legacy fusions), so each registration carries it as a template value
+template <int NAME, bool NEW_API, int TIN, int TOUT>
+struct ConvKernel;
+
+const char* const kLegacyNames[] = {"QuantizedConv2D", "QuantizedConv2DPerChannel", "QuantizedConv2DWithBias",
+                                    "QuantizedConv2DWithBiasAndRelu", "QuantizedConv2DAndRelu", "QuantizedConv2DAndRequantize",
+                                    "QuantizedConv2DAndReluAndRequantize", "QuantizedConv2DWithBiasAndRequantize",
+                                    "QuantizedConv2DWithBiasAndReluAndRequantize"};
+
+template <int NAME, bool NEW_API, int TIN, int TOUT>
+struct ConvKernel : QuantizedConv2DOp {
+  explicit ConvKernel(OpKernelConstruction* c)
+      : QuantizedConv2DOp(c, NEW_API ? "_QuantizedConv2D" : kLegacyNames[NAME], NEW_API, static_cast<TF_DataType>(TIN),
+                          static_cast<TF_DataType>(TOUT)) {}
+};
+
+template <int NAME, int TIN, int TOUT>
+void RegLegacy(bool with_bias_types, std::initializer_list<const char*> host_args) {
+  for (const char* prefix : {"", "_ITEX"}) {
+    const std::string op = std::string(prefix) + kLegacyNames[NAME];
+    for (TF_DataType tb : {TF_FLOAT, TF_QINT32}) {
+      if (!with_bias_types && tb != TF_FLOAT) continue;
+      KernelDefBuilder b(op.c_str(), "QuantizedConvOp");
+      b.TypeConstraint("Tinput", static_cast<TF_DataType>(TIN)).TypeConstraint("Tfilter", TF_QINT8);
+      if (with_bias_types) b.TypeConstraint("Tbias", tb);
+      b.TypeConstraint("out_type", static_cast<TF_DataType>(TOUT));
+      for (const char* h : host_args) b.HostMemory(h);
+      b.Register<ConvKernel<NAME, false, TIN, TOUT>>();
+    }
+  }
+}
+
+template <int TIN, int TOUT>
+void RegNewApi() {
+  for (const char* op : {"_QuantizedConv2D", "_ITEXQuantizedConv2DV2"})
+    for (TF_DataType tb : {TF_FLOAT, TF_QINT32}) {
+      KernelDefBuilder b(op, "QuantizedConvOp");
+      b.TypeConstraint("Tinput", static_cast<TF_DataType>(TIN)).TypeConstraint("Tfilter", TF_QINT8).TypeConstraint("Tbias", tb);
+      b.TypeConstraint("out_type", static_cast<TF_DataType>(TOUT));
+      b.HostMemory("host_inputs").HostMemory("host_outputs");
+      b.Register<ConvKernel<0, true, TIN, TOUT>>();
+    }
+}
+
+}  // namespace
+
+// Names, type constraints and host-memory arguments as registered by the reference for a device
+// (itex/core/kernels/gpu/quantized_conv_ops.cc:77-310); the _ITEX names are the CPU-side renames
+// (itex/core/graph/native_layout/native_layout.cc:118-145, 178-179).
+void AddQuantizedConvKernels() {
+  const std::initializer_list<const char*> plain = {"min_input", "max_input", "min_filter", "max_filter", "min_output", "max_output"};
+  const std::initializer_list<const char*> req = {"min_input", "max_input", "min_filter", "max_filter", "min_freezed_output",
+                                                  "max_freezed_output", "min_output", "max_output"};
+  RegLegacy<0, TF_QINT8, TF_QINT32>(false, plain);  RegLegacy<0, TF_QUINT8, TF_QINT32>(false, plain);
+  RegLegacy<1, TF_QINT8, TF_QINT32>(false, plain);  RegLegacy<1, TF_QUINT8, TF_QINT32>(false, plain);
+  RegLegacy<2, TF_QINT8, TF_QINT32>(false, plain);  RegLegacy<2, TF_QUINT8, TF_QINT32>(false, plain);
+  RegLegacy<3, TF_QINT8, TF_QINT32>(false, plain);  RegLegacy<3, TF_QUINT8, TF_QINT32>(false, plain);
+  RegLegacy<4, TF_QUINT8, TF_QINT32>(false, plain);
+  RegLegacy<5, TF_QINT8, TF_QINT8>(false, req);     RegLegacy<5, TF_QUINT8, TF_QINT8>(false, req);
+  RegLegacy<6, TF_QUINT8, TF_QUINT8>(false, req);
+  RegLegacy<7, TF_QINT8, TF_QINT8>(true, req);      RegLegacy<7, TF_QUINT8, TF_QINT8>(true, req);
+  RegLegacy<8, TF_QINT8, TF_QUINT8>(true, req);     RegLegacy<8, TF_QUINT8, TF_QUINT8>(true, req);
+  RegNewApi<TF_QINT8, TF_QINT8>();   RegNewApi<TF_QUINT8, TF_QINT8>();
+  RegNewApi<TF_QINT8, TF_QUINT8>();  RegNewApi<TF_QUINT8, TF_QUINT8>();
+  RegNewApi<TF_QINT8, TF_FLOAT>();   RegNewApi<TF_QUINT8, TF_FLOAT>();
+  RegNewApi<TF_QINT8, TF_BFLOAT16>(); RegNewApi<TF_QUINT8, TF_BFLOAT16>();
+  RegNewApi<TF_QINT8, TF_QINT32>();  RegNewApi<TF_QUINT8, TF_QINT32>();
+}
+
+}  // namespace itex_amd

@@ -739,3 +739,140 @@ int orc_qbatch_matmul(const int8_t* x, int x_rank, const int64_t* x_dims, const 
   }
   return ORC_OK;
 }
+
+
+/* ---- quantized Conv2D ---------------------------------------------------------------------------- */
+/* TensorFlow's GetWindowedOutputSizeVerbose, which conv_ops.h:405-440 reaches through its shape helper */
+int orc_conv_out_dim(int64_t in, int64_t k, int stride, int dil, int padding, int pad_before, int pad_after,
+                     int64_t* out, int64_t* pad_lead) {
+  const int64_t eff = (k - 1) * dil + 1;
+  if (stride <= 0 || dil <= 0) return ORC_INVALID_ARGUMENT;
+  if (padding == ORC_PAD_VALID) {
+    *out = (in - eff + stride) / stride;
+    *pad_lead = 0;
+  } else if (padding == ORC_PAD_SAME) {
+    *out = (in + stride - 1) / stride;
+    int64_t need = (*out - 1) * stride + eff - in;
+    if (need < 0) need = 0;
+    *pad_lead = need / 2;
+  } else {
+    *out = (in + pad_before + pad_after - eff + stride) / stride;
+    *pad_lead = pad_before;
+  }
+  return *out < 0 ? ORC_INVALID_ARGUMENT : ORC_OK;
+}
+
+void orc_int_conv2d(const void* x, int x_type, const int8_t* w, const orc_conv_geom* g, int64_t out_h,
+                    int64_t out_w, int64_t pad_top, int64_t pad_left, int32_t* acc) {
+  const uint8_t* xu = (const uint8_t*)x;
+  const int8_t* xs = (const int8_t*)x;
+#pragma omp parallel for collapse(2) schedule(static)
+  for (int64_t b = 0; b < g->batch; ++b) {
+    for (int64_t oh = 0; oh < out_h; ++oh) {
+      for (int64_t ow = 0; ow < out_w; ++ow) {
+        int32_t* dst = acc + ((b * out_h + oh) * out_w + ow) * g->out_c;
+        for (int64_t o = 0; o < g->out_c; ++o) dst[o] = 0;
+        for (int64_t kh = 0; kh < g->k_h; ++kh) {
+          const int64_t ih = oh * g->stride_h - pad_top + kh * g->dil_h;
+          if (ih < 0 || ih >= g->in_h) continue; /* zero padding */
+          for (int64_t kw = 0; kw < g->k_w; ++kw) {
+            const int64_t iw = ow * g->stride_w - pad_left + kw * g->dil_w;
+            if (iw < 0 || iw >= g->in_w) continue;
+            const int64_t xo = ((b * g->in_h + ih) * g->in_w + iw) * g->in_c;
+            const int8_t* wf = w + (kh * g->k_w + kw) * g->in_c * g->out_c;
+            for (int64_t c = 0; c < g->in_c; ++c) {
+              const int32_t xv = x_type == ORC_QUINT8 ? (int32_t)xu[xo + c] : (int32_t)xs[xo + c];
+              for (int64_t o = 0; o < g->out_c; ++o) dst[o] += xv * (int32_t)wf[c * g->out_c + o];
+            }
+          }
+        }
+      }
+    }
+  }
+}
+
+int orc_qconv_prepare(const orc_conv_attrs* at, int64_t N, float min_in, float max_in, const float* min_f,
+                      const float* max_f, int64_t depth, float min_out, float max_out, const void* bias,
+                      float* scales, float* bias_out, orc_epilogue_desc* ep) {
+  const int out_q8 = at->t_out == ORC_QINT8 || at->t_out == ORC_QUINT8;
+  const int out_f = at->t_out == ORC_FLOAT || at->t_out == ORC_BFLOAT16 || at->t_out == ORC_HALF;
+  if (!out_q8 && !out_f && at->t_out != ORC_QINT32) return ORC_INVALID_ARGUMENT;
+  if (at->t_in != ORC_QUINT8 && at->t_in != ORC_QINT8) return ORC_INVALID_ARGUMENT;
+  if (depth != 1 && depth != N) return ORC_INVALID_ARGUMENT;
+  memset(ep, 0, sizeof(*ep));
+  /* ---- output scales, ExtendInt8PostOps :329-393 ("Quantized" always sets output scales, :76) */
+  for (int64_t i = 0; i < depth; ++i) scales[i] = 1.0f;
+  if (out_f) {
+    const float int_input_limit = (at->t_in == ORC_QUINT8) ? 255.0f : 127.0f;
+    const float int_filter_limit = 127.0f;
+    const float src_qscale_f32 = fmaxf(fabsf(min_in), fabsf(max_in)) / int_input_limit;
+    for (int64_t i = 0; i < depth; ++i) {
+      const float wei_qscale_f32 = fmaxf(fabsf(min_f[i]), fabsf(max_f[i])) / int_filter_limit;
+      scales[i] = src_qscale_f32 * wei_qscale_f32;
+    }
+  } else if (out_q8) {
+    const float int_output_limit = (at->t_out == ORC_QUINT8) ? 255.0f : 127.0f;
+    const float float_input_range = fmaxf(fabsf(min_in), fabsf(max_in));
+    const float float_output_range = fmaxf(fabsf(min_out), fabsf(max_out));
+    const float int_const_scale_limit = (at->t_in == ORC_QUINT8) ? (float)(255.0 * 127.0) : (float)(127.0 * 127.0);
+    for (int64_t i = 0; i < depth; ++i) {
+      const float float_filter_range = fmaxf(fabsf(min_f[i]), fabsf(max_f[i]));
+      scales[i] = int_output_limit * float_input_range * float_filter_range /
+                  (int_const_scale_limit * float_output_range);
+    }
+  }
+  ep->n_scales = (int)depth;
+  /* ---- post-ops: one eltwise at most here; its post-op scale is set to 1 (:436-445) */
+  if (at->activation == ORC_ACT_RELU) {
+    ep->elt[0].alg = ORC_ELT_RELU; ep->elt[0].alpha = 0.0f; ep->elt[0].beta = 0.0f; ep->n_eltwise = 1;
+  } else if (at->activation == ORC_ACT_LEAKYRELU) {
+    ep->elt[0].alg = ORC_ELT_RELU; ep->elt[0].alpha = at->alpha; ep->elt[0].beta = 0.0f; ep->n_eltwise = 1;
+  } else if (at->activation != ORC_ACT_NONE) {
+    return ORC_UNIMPLEMENTED;
+  }
+  /* ---- bias, GetBiasHandle :448-597 */
+  if (at->t_bias == 0) {
+    for (int64_t j = 0; j < N; ++j) bias_out[j] = 0.0f;
+    return ORC_OK;
+  }
+  const float int_const_scale_limit = (at->t_in == ORC_QUINT8) ? (float)(255.0 * 127.0) : (float)(127.0 * 127.0);
+  const float in_range = fmaxf(fabsf(max_in), fabsf(min_in));
+  for (int64_t j = 0; j < N; ++j) {
+    const int64_t i = depth == 1 ? 0 : j; /* reorder of the 1-D bias: one scale, or one per element (:573-577) */
+    const float filt_range = fmaxf(fabsf(max_f[i]), fabsf(min_f[i]));
+    if (at->t_bias == ORC_QINT32) {
+      const float bf = (float)((const int32_t*)bias)[j]; /* cast to float, :462-468 */
+      if (at->t_out == ORC_QINT32) bias_out[j] = bf;     /* used as is, :450-453 */
+      else if (out_f) bias_out[j] = bf * ((in_range * filt_range) / int_const_scale_limit); /* :489-497 */
+      else bias_out[j] = bf * scales[i];                 /* :505-509 */
+    } else if (at->t_bias == ORC_FLOAT) {
+      const float tmp_scale = int_const_scale_limit / (in_range * filt_range); /* :553-557 */
+      bias_out[j] = ((const float*)bias)[j] * (tmp_scale * scales[i]);         /* :560, reorder */
+    } else {
+      return ORC_UNIMPLEMENTED;
+    }
+  }
+  return ORC_OK;
+}
+
+int orc_qconv2d(const orc_conv_attrs* at, const orc_conv_geom* g, const void* x, const int8_t* w,
+                const void* bias, float min_in, float max_in, const float* min_f, const float* max_f,
+                int64_t depth, float min_out, float max_out, void* out, int64_t* out_h, int64_t* out_w) {
+  int64_t pt = 0, pl = 0;
+  if (orc_conv_out_dim(g->in_h, g->k_h, g->stride_h, g->dil_h, g->padding, g->pad_top, g->pad_bottom, out_h, &pt) ||
+      orc_conv_out_dim(g->in_w, g->k_w, g->stride_w, g->dil_w, g->padding, g->pad_left, g->pad_right, out_w, &pl))
+    return ORC_INVALID_ARGUMENT;
+  const int64_t M = g->batch * *out_h * *out_w, N = g->out_c;
+  if (out == NULL || M == 0 || N == 0) return ORC_OK; /* shape query or empty output */
+  int32_t* acc = (int32_t*)malloc(sizeof(int32_t) * (size_t)(M * N));
+  float* scales = (float*)malloc(sizeof(float) * (size_t)(depth > 0 ? depth : 1));
+  float* sb = (float*)malloc(sizeof(float) * (size_t)N);
+  orc_epilogue_desc ep;
+  int st = orc_qconv_prepare(at, N, min_in, max_in, min_f, max_f, depth, min_out, max_out, bias, scales, sb, &ep);
+  if (st == ORC_OK) {
+    orc_int_conv2d(x, at->t_in, w, g, *out_h, *out_w, pt, pl, acc);
+    orc_qmatmul_epilogue(acc, M, N, &ep, scales, sb, NULL, at->t_out, out);
+  }
+  free(acc); free(scales); free(sb);
+  return st;
+}

@@ -155,6 +155,45 @@ int orc_qbatch_matmul(const int8_t* x, int x_rank, const int64_t* x_dims, const 
                       float min_y, float max_y, int n_binary, const orc_bmm_binary* bin, int t_out,
                       void* out, int out_rank, const int64_t* out_dims);
 
+/*
+ * Quantized Conv2D (NHWC input, HWIO qint8 filter, SCALED quantization: zero points are 0, so the
+ * padding value is the integer 0): itex/core/kernels/common/quantized_conv_ops.h
+ * (constructor :63-318, ExtendInt8PostOps :329-446, GetBiasHandle :448-597) over the geometry of
+ * itex/core/kernels/common/conv_ops.h:615-716 / TensorFlow's GetWindowedOutputSizeVerbose.
+ * Fusions restated: BiasAdd, Relu, LeakyRelu, Requantize, Dequantize.  Sum, Elu, Swish, HardSwish,
+ * Sigmoid and the depthwise / 3-D variants are not.
+ * Pinned by: brute force against float64 direct convolution of the integer operands; the fp32
+ * convolution at the reference's own tolerance (native_quantized_conv_test.py: rtol = atol = 0.3) and
+ * at the bound the quantization steps allow; closed forms of the scales; padding identities.
+ * Parity unpinned: none of the reference's conv tests holds fixed vectors (their inputs are unseeded
+ * random numbers), so nothing beyond those properties pins the restatement.
+ */
+enum { ORC_PAD_VALID = 0, ORC_PAD_SAME = 1, ORC_PAD_EXPLICIT = 2 };
+typedef struct {
+  int64_t batch, in_h, in_w, in_c, k_h, k_w, out_c;
+  int stride_h, stride_w, dil_h, dil_w;
+  int padding;                                   /* ORC_PAD_* */
+  int pad_top, pad_bottom, pad_left, pad_right;  /* ORC_PAD_EXPLICIT only */
+} orc_conv_geom;
+typedef struct {
+  int t_in;              /* ORC_QUINT8 | ORC_QINT8 */
+  int t_out;             /* ORC_QINT32 | ORC_QINT8 | ORC_QUINT8 | ORC_FLOAT | ORC_BFLOAT16 */
+  int t_bias;            /* 0: no BiasAdd;  ORC_FLOAT | ORC_QINT32 */
+  int activation;        /* ORC_ACT_NONE | ORC_ACT_RELU | ORC_ACT_LEAKYRELU */
+  float alpha;           /* LeakyRelu */
+} orc_conv_attrs;
+/* output extent and leading padding of one spatial dimension; returns ORC_INVALID_ARGUMENT for a negative extent */
+int orc_conv_out_dim(int64_t in, int64_t k, int stride, int dil, int padding, int pad_before, int pad_after,
+                     int64_t* out, int64_t* pad_lead);
+void orc_int_conv2d(const void* x, int x_type, const int8_t* w, const orc_conv_geom* g, int64_t out_h,
+                    int64_t out_w, int64_t pad_top, int64_t pad_left, int32_t* acc);
+int orc_qconv_prepare(const orc_conv_attrs* at, int64_t N, float min_in, float max_in, const float* min_f,
+                      const float* max_f, int64_t depth, float min_out, float max_out, const void* bias,
+                      float* scales, float* bias_out, orc_epilogue_desc* ep);
+int orc_qconv2d(const orc_conv_attrs* at, const orc_conv_geom* g, const void* x, const int8_t* w,
+                const void* bias, float min_in, float max_in, const float* min_f, const float* max_f,
+                int64_t depth, float min_out, float max_out, void* out, int64_t* out_h, int64_t* out_w);
+
 #ifdef __cplusplus
 }
 #endif

@@ -278,3 +278,58 @@ def qbatch_matmul(x, y, min_x, max_x, min_y, max_y, adj_x=False, adj_y=False, bi
     st = f(_p(x), x.ndim, xd, _p(y), y.ndim, yd, int(bool(adj_x)), int(bool(adj_y)), C.c_float(min_x), C.c_float(max_x),
            C.c_float(min_y), C.c_float(max_y), len(binary), bins, t_out, _p(out), len(oshape), od)
     return st, out
+
+
+# ---- quantized Conv2D ------------------------------------------------------------------------------
+PAD_VALID, PAD_SAME, PAD_EXPLICIT = 0, 1, 2
+
+
+class ConvGeom(C.Structure):
+    _fields_ = [(n, C.c_int64) for n in ("batch", "in_h", "in_w", "in_c", "k_h", "k_w", "out_c")] + \
+               [(n, C.c_int) for n in ("stride_h", "stride_w", "dil_h", "dil_w", "padding", "pad_top", "pad_bottom", "pad_left",
+                                       "pad_right")]
+
+
+class ConvAttrs(C.Structure):
+    _fields_ = [("t_in", C.c_int), ("t_out", C.c_int), ("t_bias", C.c_int), ("activation", C.c_int), ("alpha", C.c_float)]
+
+
+def conv_geom(x_shape, w_shape, strides=(1, 1), dilations=(1, 1), padding=PAD_SAME, explicit=(0, 0, 0, 0)):
+    b, h, w_, c = x_shape
+    kh, kw, ci, co = w_shape
+    assert ci == c
+    return ConvGeom(b, h, w_, c, kh, kw, co, strides[0], strides[1], dilations[0], dilations[1], padding, *explicit)
+
+
+def qconv_prepare(at, N, min_in, max_in, min_f, max_f, min_out, max_out, bias):
+    min_f, max_f = _f32(min_f), _f32(max_f)
+    depth = min_f.size
+    scales = np.zeros(max(depth, 1), np.float32)
+    sb = np.zeros(N, np.float32)
+    ep = EpilogueDesc()
+    b = None if bias is None else (np.ascontiguousarray(bias, np.int32) if at.t_bias == QINT32 else _f32(bias))
+    f = lib().orc_qconv_prepare
+    f.restype = C.c_int
+    st = f(C.byref(at), C.c_int64(N), C.c_float(min_in), C.c_float(max_in), _p(min_f), _p(max_f), C.c_int64(depth),
+           C.c_float(min_out), C.c_float(max_out), _p(b) if b is not None else None, _p(scales), _p(sb), C.byref(ep))
+    return st, scales, sb, ep
+
+
+def qconv2d(at, g, x, w, bias, min_in, max_in, min_f, max_f, min_out=0.0, max_out=0.0):
+    """x: [B, H, W, C] uint8 / int8, w: [KH, KW, C, O] int8.  Returns (status, out [B, OH, OW, O])."""
+    x = np.ascontiguousarray(x, dtype=np.uint8 if at.t_in == QUINT8 else np.int8)
+    w = np.ascontiguousarray(w, dtype=np.int8)
+    min_f, max_f = _f32(min_f), _f32(max_f)
+    b = None if bias is None else (np.ascontiguousarray(bias, np.int32) if at.t_bias == QINT32 else _f32(bias))
+    oh, ow = C.c_int64(), C.c_int64()
+    f = lib().orc_qconv2d
+    f.restype = C.c_int
+    args = lambda out: (C.byref(at), C.byref(g), _p(x), _p(w), _p(b) if b is not None else None, C.c_float(min_in),
+                        C.c_float(max_in), _p(min_f), _p(max_f), C.c_int64(min_f.size), C.c_float(min_out), C.c_float(max_out),
+                        out, C.byref(oh), C.byref(ow))
+    st = f(*args(None))
+    if st != OK:
+        return st, None
+    out = np.zeros((g.batch, oh.value, ow.value, g.out_c), NP_OF[at.t_out])
+    st = f(*args(_p(out)))
+    return st, out

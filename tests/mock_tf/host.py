@@ -24,7 +24,10 @@ _state = {}
 def load(device="XPU", stock_ops=("QuantizeV2", "Dequantize", "QuantizedMatMulWithBias", "QuantizedMatMulWithBiasAndRelu",
                                    "QuantizedMatMulWithBiasAndReluAndRequantize", "QuantizedMatMulWithBiasAndRequantize",
                                    "QuantizedMatMulWithBiasAndDequantize", "RequantizePerChannel",
-                                   "RequantizationRangePerChannel", "QuantizedReshape", "MatMul", "Relu")):
+                                   "RequantizationRangePerChannel", "QuantizedReshape", "MatMul", "Relu", "QuantizedConv2D",
+                                   "QuantizedConv2DPerChannel", "QuantizedConv2DWithBias", "QuantizedConv2DWithBiasAndRelu",
+                                   "QuantizedConv2DAndRelu", "QuantizedConv2DAndRequantize", "QuantizedConv2DAndReluAndRequantize",
+                                   "QuantizedConv2DWithBiasAndRequantize", "QuantizedConv2DWithBiasAndReluAndRequantize")):
     """Loads the mock host and the plugin once per process; returns the mock's ctypes handle."""
     if "lib" in _state:
         return _state["lib"]
@@ -96,6 +99,9 @@ class Node:
             elif isinstance(v, (list, tuple)) and all(isinstance(x, DType) for x in v):
                 arr = (C.c_int * len(v))(*[int(x) for x in v])
                 self.lib.mock_node_attr_type_list(self.h, kb, arr, len(v))
+            elif isinstance(v, (list, tuple)) and len(v) > 0 and all(isinstance(x, int) for x in v):
+                arr = (C.c_int64 * len(v))(*v)
+                self.lib.mock_node_attr_int_list(self.h, kb, arr, len(v))
             elif isinstance(v, (list, tuple)):
                 arr = (C.c_char_p * len(v))(*[x.encode() for x in v])
                 self.lib.mock_node_attr_string_list(self.h, kb, arr, len(v))

@@ -80,7 +80,7 @@ TF_Tensor* NewTensor(TF_DataType dtype, const int64_t* dims, int ndims, bool on_
 }
 
 struct AttrValue {
-  enum Kind { STRING, INT, FLOAT, BOOL, TYPE, STRING_LIST, TYPE_LIST } kind;
+  enum Kind { STRING, INT, FLOAT, BOOL, TYPE, STRING_LIST, TYPE_LIST, INT_LIST } kind;
   std::string s;
   int64_t i = 0;
   float f = 0;
@@ -88,6 +88,7 @@ struct AttrValue {
   TF_DataType t = TF_FLOAT;
   std::vector<std::string> sl;
   std::vector<TF_DataType> tl;
+  std::vector<int64_t> il;
 };
 }  // namespace
 
@@ -268,6 +269,7 @@ void TF_OpKernelConstruction_GetAttrSize(TF_OpKernelConstruction* ctx, const cha
       break;
     }
     case AttrValue::TYPE_LIST: *list_size = static_cast<int32_t>(a.tl.size()); *total_size = -1; break;
+    case AttrValue::INT_LIST: *list_size = static_cast<int32_t>(a.il.size()); *total_size = -1; break;
     default: *list_size = -1; *total_size = -1; break;
   }
 }
@@ -310,6 +312,12 @@ void TF_OpKernelConstruction_GetAttrTypeList(TF_OpKernelConstruction* ctx, const
   const AttrValue* a = FindAttr(ctx, n, AttrValue::TYPE_LIST, st);
   if (!a) return;
   for (int i = 0; i < max_vals && i < static_cast<int>(a->tl.size()); ++i) vals[i] = a->tl[i];
+}
+void TF_OpKernelConstruction_GetAttrInt64List(TF_OpKernelConstruction* ctx, const char* n, int64_t* vals, int max_vals,
+                                              TF_Status* st) {
+  const AttrValue* a = FindAttr(ctx, n, AttrValue::INT_LIST, st);
+  if (!a) return;
+  for (int i = 0; i < max_vals && i < static_cast<int>(a->il.size()); ++i) vals[i] = a->il[i];
 }
 TF_StringView TF_OpKernelConstruction_GetName(TF_OpKernelConstruction* ctx) { return TF_StringView{ctx->name.data(), ctx->name.size()}; }
 void TF_OpKernelConstruction_Failure(TF_OpKernelConstruction* ctx, TF_Status* status) {
@@ -748,6 +756,10 @@ void mock_node_attr_type(void* h, const char* name, int v) { Attr(h, name, AttrV
 void mock_node_attr_string_list(void* h, const char* name, const char** v, int n) {
   AttrValue& a = Attr(h, name, AttrValue::STRING_LIST);
   a.sl.assign(v, v + n);
+}
+void mock_node_attr_int_list(void* h, const char* name, const int64_t* v, int n) {
+  AttrValue& a = Attr(h, name, AttrValue::INT_LIST);
+  a.il.assign(v, v + n);
 }
 void mock_node_attr_type_list(void* h, const char* name, const int* v, int n) {
   AttrValue& a = Attr(h, name, AttrValue::TYPE_LIST);

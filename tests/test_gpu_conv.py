@@ -1,0 +1,222 @@
+"""Quantized Conv2D on the GPU: the patch matrix (itexhip_im2col8) and bias scaling through the C ABI, and the op
+kernels through the plugin, bit-compared with the CPU oracle (int32 / int8 / fp32 outputs alike: the accumulation
+is integer and the epilogue is the same fp32 sequence)."""
+import numpy as np
+import pytest
+
+from oracle import pyoracle as orc
+from tests.mock_tf import host as tf
+
+pytestmark = pytest.mark.gpu
+DT = tf.DType
+
+
+def same_lead(n, k, s, d):
+    eff = (k - 1) * d + 1
+    out = -(-n // s)
+    return out, max((out - 1) * s + eff - n, 0) // 2
+
+
+@pytest.mark.parametrize("shape,kh,kw,strides,dil", [((2, 7, 9, 3), 3, 3, (2, 2), (1, 1)), ((1, 6, 6, 4), 3, 3, (1, 1), (1, 1)),
+                                                     ((2, 9, 9, 8), 3, 2, (1, 2), (2, 1)), ((1, 12, 12, 16), 1, 1, (2, 2), (1, 1)),
+                                                     ((3, 5, 5, 5), 5, 5, (1, 1), (1, 1)),
+                                                     # channel counts that take the 16-byte-vector kernel
+                                                     ((2, 9, 10, 16), 3, 3, (1, 1), (1, 1)), ((1, 8, 7, 32), 3, 2, (2, 1), (1, 2)),
+                                                     ((2, 6, 6, 48), 2, 2, (1, 1), (1, 1)), ((1, 20, 20, 64), 3, 3, (1, 1), (1, 1))])
+def test_im2col_against_numpy(hip, dev, shape, kh, kw, strides, dil):
+    import torch
+    rng = np.random.default_rng(sum(shape) + kh)
+    x = rng.integers(0, 256, shape).astype(np.uint8)
+    B, H, W, C = shape
+    oh, pt = same_lead(H, kh, strides[0], dil[0])
+    ow, pl = same_lead(W, kw, strides[1], dil[1])
+    K = kh * kw * C
+    Kp = (K + 15) // 16 * 16
+    g = hip.ConvGeometry(B, H, W, C, kh, kw, oh, ow, strides[0], strides[1], dil[0], dil[1], pt, pl)
+    for off in (0, 1):        # aligned, and an unaligned input address (byte loads)
+        raw = torch.zeros(x.size + 8, dtype=torch.uint8, device=dev)
+        raw[off:off + x.size] = torch.from_numpy(x.ravel()).to(dev)
+        cols = torch.full((B * oh * ow, Kp), 0xEE, dtype=torch.uint8, device=dev)
+        hip.im2col8(raw.data_ptr() + off, g, Kp, cols)
+        torch.cuda.synchronize()
+        ref = np.zeros((B, oh, ow, Kp), np.uint8)
+        for i in range(kh):
+            for j in range(kw):
+                for a in range(oh):
+                    ih = a * strides[0] - pt + i * dil[0]
+                    if not 0 <= ih < H:
+                        continue
+                    for b_ in range(ow):
+                        iw = b_ * strides[1] - pl + j * dil[1]
+                        if 0 <= iw < W:
+                            ref[:, a, b_, (i * kw + j) * C:(i * kw + j + 1) * C] = x[:, ih, iw, :]
+        np.testing.assert_array_equal(cols.cpu().numpy(), ref.reshape(-1, Kp))
+
+
+def test_scale_vector(hip, dev):
+    import torch
+    rng = np.random.default_rng(1)
+    for n in (1, 7, 300):
+        bf = rng.standard_normal(n).astype(np.float32)
+        bi = rng.integers(-5000, 5000, n).astype(np.int32)
+        f = (rng.random(n).astype(np.float32) + 0.1)
+        out = torch.empty(n, dtype=torch.float32, device=dev)
+        for bias, T in ((bf, hip.FLOAT), (bi, hip.QINT32)):
+            hip.scale_vector(torch.from_numpy(bias).to(dev), T, torch.from_numpy(f).to(dev), n, n, out)
+            np.testing.assert_array_equal(out.cpu().numpy(), bias.astype(np.float32) * f)
+            hip.scale_vector(torch.from_numpy(bias).to(dev), T, torch.from_numpy(f[:1].copy()).to(dev), 1, n, out)
+            np.testing.assert_array_equal(out.cpu().numpy(), bias.astype(np.float32) * f[0])
+
+
+@pytest.fixture(scope="module")
+def rt(dev):
+    import torch
+    tf.load()
+    tf.use_torch_allocator(dev)
+    return torch
+
+
+def fetch(torch, out, np_dtype):
+    dtype, shape, addr, _ = out
+    n = int(np.prod(shape, dtype=np.int64)) if len(shape) else 1
+    torch.cuda.synchronize()
+    live = tf._state["alloc_cb"][2]
+    if addr in live:
+        return live[addr][:n * np.dtype(np_dtype).itemsize].cpu().numpy().view(np_dtype).copy().reshape(shape)
+    return tf.read_host(addr, dtype, shape)
+
+
+def quantize_inputs(x, w, T_in, per_channel=True):
+    _, xq, xmn, xmx = orc.quantize_v2(x, x.min(), x.max(), T_in, orc.SCALED)
+    if per_channel:
+        mn, mx = w.min(axis=(0, 1, 2)).astype(np.float32), w.max(axis=(0, 1, 2)).astype(np.float32)
+        _, wq, fmn, fmx = orc.quantize_v2(w, mn, mx, orc.QINT8, orc.SCALED, axis=3)
+    else:
+        _, wq, fmn, fmx = orc.quantize_v2(w, w.min(), w.max(), orc.QINT8, orc.SCALED)
+        fmn, fmx = np.array(fmn[0], np.float32), np.array(fmx[0], np.float32)
+    return xq, np.array(xmn[0], np.float32), np.array(xmx[0], np.float32), wq, fmn, fmx
+
+
+def run_conv(torch, dev, node, xq, wq, bias, bias_dt, host_scalars, out_dt, np_out, with_minmax):
+    keep = [torch.from_numpy(np.ascontiguousarray(v)).to(dev) for v in ([xq, wq] + ([bias] if bias is not None else []))]
+    ins = [(tf.QUINT8 if xq.dtype == np.uint8 else tf.QINT8, xq.shape, keep[0].data_ptr(), False),
+           (tf.QINT8, wq.shape, keep[1].data_ptr(), False)]
+    if bias is not None:
+        ins.append((bias_dt, bias.shape, keep[2].data_ptr(), False))
+    for s in host_scalars:
+        ins.append((tf.FLOAT, s.shape, tf.host_array(s), True))
+    outs = [(out_dt, False)] + ([(tf.FLOAT, True), (tf.FLOAT, True)] if with_minmax else [])
+    code, msg, res = node.run(ins, outs, stream=torch.cuda.current_stream().cuda_stream)
+    assert code == tf.OK, msg
+    return fetch(torch, res[0], np_out), res
+
+
+LEGACY = [  # op, fusions -> (bias, relu, requantize), input type, output type
+    ("QuantizedConv2D", False, False, False, tf.QUINT8, tf.QINT32),
+    ("QuantizedConv2DPerChannel", False, False, False, tf.QINT8, tf.QINT32),
+    ("QuantizedConv2DWithBias", True, False, False, tf.QUINT8, tf.QINT32),
+    ("QuantizedConv2DWithBiasAndRelu", True, True, False, tf.QINT8, tf.QINT32),
+    ("QuantizedConv2DAndRelu", False, True, False, tf.QUINT8, tf.QINT32),
+    ("QuantizedConv2DAndRequantize", False, False, True, tf.QINT8, tf.QINT8),
+    ("QuantizedConv2DAndReluAndRequantize", False, True, True, tf.QUINT8, tf.QUINT8),
+    ("QuantizedConv2DWithBiasAndRequantize", True, False, True, tf.QINT8, tf.QINT8),
+    ("QuantizedConv2DWithBiasAndReluAndRequantize", True, True, True, tf.QUINT8, tf.QUINT8),
+]
+NP = {tf.QINT32: np.int32, tf.QINT8: np.int8, tf.QUINT8: np.uint8, tf.FLOAT: np.float32}
+
+
+@pytest.mark.parametrize("op,has_bias,relu,req,t_in,t_out", LEGACY)
+def test_legacy_conv_ops_through_plugin(rt, dev, op, has_bias, relu, req, t_in, t_out):
+    """The shapes of the reference's native_quantized_conv_test.py (x [1,6,6,4], w [3,3,4,4], SAME, stride 1) plus a
+    strided, larger case; outputs and min / max outputs equal the oracle's."""
+    torch = rt
+    for shape, wshape, strides, padding in (((1, 6, 6, 4), (3, 3, 4, 4), [1, 1, 1, 1], "SAME"),
+                                            ((2, 15, 13, 20), (3, 3, 20, 24), [1, 2, 2, 1], "VALID")):
+        rng = np.random.default_rng(len(op) + shape[1])
+        signed = t_in == tf.QINT8
+        x = rng.uniform(-5.0 if signed else 0.0, 5.0, shape).astype(np.float32)
+        w = rng.uniform(-2.0, 2.0, wshape).astype(np.float32)
+        b = rng.uniform(-1.0, 1.0, wshape[3]).astype(np.float32) if has_bias else None
+        xq, xmn, xmx, wq, fmn, fmx = quantize_inputs(x, w, t_in, per_channel=op != "QuantizedConv2D")
+        attrs = dict(Tinput=DT(t_in), Tfilter=DT(tf.QINT8), out_type=DT(t_out), strides=strides, padding=padding,
+                     dilations=[1, 1, 1, 1])
+        if has_bias and req:
+            attrs["Tbias"] = DT(tf.FLOAT)
+        node = tf.Node(op, attrs)
+        assert node.code == tf.OK, node.message
+        zmn, zmx = np.array(-37.5 if t_out == tf.QINT8 else 0.0, np.float32), np.array(41.0, np.float32)
+        scalars = [xmn, xmx, fmn, fmx] + ([zmn, zmx] if req else [])
+        got, res = run_conv(torch, dev, node, xq, wq, b, tf.FLOAT, scalars, t_out, NP[t_out], True)
+        at = orc.ConvAttrs(t_in, t_out, orc.FLOAT if has_bias else 0, orc.ACT_RELU if relu else orc.ACT_NONE, 0.0)
+        g = orc.conv_geom(shape, wshape, strides[1:3], (1, 1), orc.PAD_SAME if padding == "SAME" else orc.PAD_VALID)
+        st, ref = orc.qconv2d(at, g, xq, wq, b, float(xmn), float(xmx), fmn, fmx, float(zmn), float(zmx))
+        assert st == orc.OK
+        np.testing.assert_array_equal(got, ref)
+        mat = orc.matmul_attrs(t_in=t_in, t_out=t_out)
+        st, omn, omx = orc.qmatmul_output_minmax(mat, float(xmn), float(xmx), fmn, fmx, fmn.ndim, float(zmn), float(zmx))
+        np.testing.assert_array_equal(np.ravel(fetch(torch, res[1], np.float32)), omn)
+        np.testing.assert_array_equal(np.ravel(fetch(torch, res[2], np.float32)), omx)
+        node.close()
+
+
+@pytest.mark.parametrize("t_in", [tf.QUINT8, tf.QINT8])
+@pytest.mark.parametrize("fused,t_out,t_bias", [(["BiasAdd", "Relu", "Dequantize"], tf.FLOAT, tf.FLOAT),
+                                                (["BiasAdd", "Dequantize"], tf.FLOAT, tf.QINT32),
+                                                (["BiasAdd", "LeakyRelu", "Requantize"], tf.QINT8, tf.FLOAT),
+                                                (["BiasAdd", "Relu", "Requantize"], tf.QUINT8, tf.QINT32),
+                                                (["Dequantize"], tf.FLOAT, tf.FLOAT), ([], tf.QINT32, tf.FLOAT)])
+def test_new_api_conv_through_plugin(rt, dev, t_in, fused, t_out, t_bias):
+    """_QuantizedConv2D with fused_ops, explicit padding, dilation, channel counts that are not multiples of 16 and a
+    pointwise case that skips the patch matrix; against the oracle, and against the fp32 convolution where that applies."""
+    torch = rt
+    cases = [((2, 10, 9, 6), (3, 3, 6, 10), [1, 1, 2, 1], [1, 2, 1, 1], "EXPLICIT", [0, 0, 2, 1, 0, 3, 0, 0]),
+             ((1, 8, 8, 32), (1, 1, 32, 48), [1, 1, 1, 1], [1, 1, 1, 1], "SAME", []),
+             ((1, 14, 14, 3), (7, 7, 3, 8), [1, 2, 2, 1], [1, 1, 1, 1], "SAME", [])]
+    for shape, wshape, strides, dil, padding, explicit in cases:
+        rng = np.random.default_rng(shape[1] * 3 + len(fused))
+        signed = t_in == tf.QINT8
+        x = rng.uniform(-3.0 if signed else 0.0, 3.0, shape).astype(np.float32)
+        w = rng.uniform(-1.0, 1.0, wshape).astype(np.float32)
+        has_bias = "BiasAdd" in fused
+        xq, xmn, xmx, wq, fmn, fmx = quantize_inputs(x, w, t_in)
+        if t_bias == tf.QINT32:
+            b = rng.integers(-4000, 4000, wshape[3]).astype(np.int32) if has_bias else None
+        else:
+            b = rng.uniform(-1.0, 1.0, wshape[3]).astype(np.float32) if has_bias else None
+        attrs = dict(Tinput=DT(t_in), Tfilter=DT(tf.QINT8), Tbias=DT(t_bias), out_type=DT(t_out), strides=strides, padding=padding,
+                     dilations=dil, fused_ops=fused, alpha=0.2, data_format="NHWC", is_filter_const=True, is_bias_const=True)
+        if explicit:
+            attrs["explicit_paddings"] = explicit
+        node = tf.Node("_QuantizedConv2D", attrs)
+        assert node.code == tf.OK, node.message
+        req = "Requantize" in fused
+        zmn, zmx = np.array(-20.0 if t_out == tf.QINT8 else 0.0, np.float32), np.array(25.0, np.float32)
+        scalars = [xmn, xmx, fmn, fmx] + ([zmn, zmx] if req else [])
+        with_mm = t_out != tf.FLOAT
+        act = orc.ACT_RELU if "Relu" in fused else orc.ACT_LEAKYRELU if "LeakyRelu" in fused else orc.ACT_NONE
+        at = orc.ConvAttrs(t_in, t_out, (orc.QINT32 if t_bias == tf.QINT32 else orc.FLOAT) if has_bias else 0, act, 0.2)
+        pad = {"SAME": orc.PAD_SAME, "VALID": orc.PAD_VALID, "EXPLICIT": orc.PAD_EXPLICIT}[padding]
+        g = orc.conv_geom(shape, wshape, strides[1:3], dil[1:3], pad, tuple(explicit[2:6]) if explicit else (0, 0, 0, 0))
+        st, ref = orc.qconv2d(at, g, xq, wq, b, float(xmn), float(xmx), fmn, fmx, float(zmn), float(zmx))
+        assert st == orc.OK
+        for _ in range(2):      # the second run uses the cached packed filter and parameter vectors
+            got, _res = run_conv(torch, dev, node, xq, wq, b, t_bias, scalars, t_out, NP[t_out], with_mm)
+            np.testing.assert_array_equal(got, ref)
+        node.close()
+
+
+def test_unsupported_fusions_and_formats(rt, dev):
+    base = dict(Tinput=DT(tf.QUINT8), Tfilter=DT(tf.QINT8), Tbias=DT(tf.FLOAT), out_type=DT(tf.FLOAT), strides=[1, 1, 1, 1],
+                padding="SAME", dilations=[1, 1, 1, 1], alpha=0.0)
+    n = tf.Node("_QuantizedConv2D", dict(base, fused_ops=["BiasAdd", "Sum", "Relu", "Dequantize"]))
+    assert n.code == tf.UNIMPLEMENTED and "Sum" in n.message
+    n.close()
+    n = tf.Node("_QuantizedConv2D", dict(base, fused_ops=["Dequantize"], data_format="NCHW"))
+    assert n.code == tf.UNIMPLEMENTED
+    n.close()
+    n = tf.Node("_QuantizedConv2D", dict(base, fused_ops=["Requantize"]))
+    assert n.code == tf.INVALID_ARGUMENT and "Requantize" in n.message
+    n.close()
+    n = tf.Node("_QuantizedConv2D", dict(base, fused_ops=["Dequantize"], strides=[1, 1, 1, 2]))
+    assert n.code == tf.UNIMPLEMENTED
+    n.close()

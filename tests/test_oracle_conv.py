@@ -1,0 +1,184 @@
+"""Pins the CPU oracle's quantized Conv2D restatement.  The reference's own conv tests
+(test/tensorflow/python/kernel_tests/native_quantized_conv_test.py) draw unseeded random inputs and compare with the
+fp32 convolution at rtol = atol = 0.3, so they hold no vectors; what pins the oracle here:
+
+  * integer convolution and geometry (SAME / VALID / EXPLICIT, strides, dilations): an independent numpy evaluation
+    on the explicitly padded input (sliding windows + tensordot in int64);
+  * TensorFlow's output-size / padding rule on known cases (the extra SAME padding goes to the end);
+  * scales and bias handling: the reference test's four pipelines on seeded inputs of the same distributions must
+    reproduce the fp32 convolution within its 0.3 tolerance and within what the quantization steps allow -- a dropped
+    factor, a missing bias scale or a wrong limit (255 vs 127) misses that bound by far;
+  * the qint32-bias and qint32-output forms through their closed forms.
+"""
+import numpy as np
+import pytest
+
+from oracle import pyoracle as orc
+
+
+def ref_int_conv(x, w, strides, dilations, pads):
+    """Direct convolution of integer tensors in int64: pad explicitly, gather windows, contract."""
+    (pt, pb), (pl, pr) = pads
+    xp = np.pad(x.astype(np.int64), ((0, 0), (pt, pb), (pl, pr), (0, 0)))
+    kh, kw, ci, co = w.shape
+    eh, ew = (kh - 1) * dilations[0] + 1, (kw - 1) * dilations[1] + 1
+    oh = (xp.shape[1] - eh) // strides[0] + 1
+    ow = (xp.shape[2] - ew) // strides[1] + 1
+    out = np.zeros((x.shape[0], oh, ow, co), np.int64)
+    for i in range(kh):
+        for j in range(kw):
+            win = xp[:, i * dilations[0]: i * dilations[0] + (oh - 1) * strides[0] + 1: strides[0],
+                     j * dilations[1]: j * dilations[1] + (ow - 1) * strides[1] + 1: strides[1], :]
+            out += np.tensordot(win, w[i, j].astype(np.int64), axes=([3], [0]))
+    return out
+
+
+def same_pads(n, k, s, d):
+    eff = (k - 1) * d + 1
+    out = -(-n // s)
+    need = max((out - 1) * s + eff - n, 0)
+    return need // 2, need - need // 2
+
+
+@pytest.mark.parametrize("x_dtype", [np.uint8, np.int8])
+@pytest.mark.parametrize("shape,wshape,strides,dil,padding,explicit", [
+    ((1, 6, 6, 4), (3, 3, 4, 4), (1, 1), (1, 1), orc.PAD_SAME, None),
+    ((2, 7, 9, 3), (3, 3, 3, 5), (2, 2), (1, 1), orc.PAD_SAME, None),
+    ((2, 8, 8, 3), (3, 3, 3, 5), (2, 2), (1, 1), orc.PAD_SAME, None),       # odd total padding: the extra row goes last
+    ((1, 9, 9, 2), (3, 3, 2, 3), (1, 1), (2, 2), orc.PAD_SAME, None),       # dilation
+    ((2, 7, 9, 3), (3, 2, 3, 5), (2, 1), (1, 1), orc.PAD_VALID, None),
+    ((1, 5, 5, 8), (1, 1, 8, 6), (1, 1), (1, 1), orc.PAD_VALID, None),      # pointwise
+    ((1, 10, 10, 3), (7, 7, 3, 4), (2, 2), (1, 1), orc.PAD_EXPLICIT, (3, 2, 1, 4)),
+])
+def test_integer_convolution_against_numpy(x_dtype, shape, wshape, strides, dil, padding, explicit):
+    rng = np.random.default_rng(sum(shape) + sum(wshape))
+    x = rng.integers(0, 256, shape).astype(np.uint8) if x_dtype == np.uint8 else rng.integers(-128, 128, shape).astype(np.int8)
+    w = rng.integers(-128, 128, wshape).astype(np.int8)
+    g = orc.conv_geom(shape, wshape, strides, dil, padding, explicit or (0, 0, 0, 0))
+    at = orc.ConvAttrs(orc.QUINT8 if x_dtype == np.uint8 else orc.QINT8, orc.QINT32, 0, orc.ACT_NONE, 0.0)
+    st, out = orc.qconv2d(at, g, x, w, None, -1.0, 1.0, np.float32([-1]), np.float32([1]))
+    assert st == orc.OK
+    if padding == orc.PAD_SAME:
+        pads = (same_pads(shape[1], wshape[0], strides[0], dil[0]), same_pads(shape[2], wshape[1], strides[1], dil[1]))
+    elif padding == orc.PAD_VALID:
+        pads = ((0, 0), (0, 0))
+    else:
+        pads = ((explicit[0], explicit[1]), (explicit[2], explicit[3]))
+    np.testing.assert_array_equal(out, ref_int_conv(x, w, strides, dil, pads))
+
+
+def test_tensorflow_padding_rule_known_cases():
+    import ctypes as C
+    f = orc.lib().orc_conv_out_dim
+    f.restype = C.c_int
+
+    def dim(n, k, s, d, padding, before=0, after=0):
+        out, lead = C.c_int64(), C.c_int64()
+        st = f(C.c_int64(n), C.c_int64(k), s, d, padding, before, after, C.byref(out), C.byref(lead))
+        return st, out.value, lead.value
+    assert dim(6, 3, 1, 1, orc.PAD_SAME) == (orc.OK, 6, 1)
+    assert dim(7, 3, 2, 1, orc.PAD_SAME) == (orc.OK, 4, 1)
+    assert dim(8, 3, 2, 1, orc.PAD_SAME) == (orc.OK, 4, 0)         # one row of padding in total, placed after
+    assert dim(224, 7, 2, 1, orc.PAD_SAME) == (orc.OK, 112, 2)     # ResNet stem: 2 before, 3 after
+    assert dim(7, 3, 2, 1, orc.PAD_VALID) == (orc.OK, 3, 0)
+    assert dim(5, 3, 1, 2, orc.PAD_VALID) == (orc.OK, 1, 0)
+    assert dim(224, 7, 2, 1, orc.PAD_EXPLICIT, 3, 3) == (orc.OK, 112, 3)
+    assert dim(6, 3, 1, 1, orc.PAD_SAME)[1:] == dim(6, 3, 1, 1, orc.PAD_EXPLICIT, 1, 1)[1:]
+
+
+def quant_in(x, T):
+    _, q, mn, mx = orc.quantize_v2(x, x.min(), x.max(), T, orc.SCALED)
+    return q, float(mn[0]), float(mx[0])
+
+
+def quant_filter(w):
+    mn, mx = w.min(axis=(0, 1, 2)).astype(np.float32), w.max(axis=(0, 1, 2)).astype(np.float32)
+    _, q, fmn, fmx = orc.quantize_v2(w, mn, mx, orc.QINT8, orc.SCALED, axis=3)
+    return q, fmn, fmx
+
+
+def fp32_conv(x, w):
+    pads = (same_pads(x.shape[1], w.shape[0], 1, 1), same_pads(x.shape[2], w.shape[1], 1, 1))
+    xp = np.pad(x.astype(np.float64), ((0, 0), pads[0], pads[1], (0, 0)))
+    out = np.zeros(x.shape[:3] + (w.shape[3],))
+    for i in range(w.shape[0]):
+        for j in range(w.shape[1]):
+            out += np.tensordot(xp[:, i:i + x.shape[1], j:j + x.shape[2], :], w[i, j].astype(np.float64), axes=([3], [0]))
+    return out
+
+
+@pytest.mark.parametrize("case", ["relu_requantize_u8", "bias_requantize_s8", "bias_relu_requantize_u8", "bias_dequantize",
+                                  "bias_relu_dequantize_s8_in"])
+def test_reference_test_pipelines_on_seeded_inputs(case):
+    """testConvRelu / testConvBias / testConvBiasRelu of the reference (x [1,6,6,4] uniform, w [3,3,4,4] uniform(-2, 2),
+    bias uniform(-1, 1), SAME, stride 1) and the Dequantize spellings of the new API."""
+    rng = np.random.default_rng(sum(map(ord, case)))
+    signed_in = case in ("bias_requantize_s8", "bias_relu_dequantize_s8_in")
+    x = rng.uniform(-5.0 if signed_in else 0.0, 5.0, (1, 6, 6, 4)).astype(np.float32)
+    w = rng.uniform(-2.0, 2.0, (3, 3, 4, 4)).astype(np.float32)
+    b = rng.uniform(-1.0, 1.0, 4).astype(np.float32) if "bias" in case else None
+    relu = "relu" in case
+    ref = fp32_conv(x, w) + (b if b is not None else 0)
+    if relu:
+        ref = np.maximum(ref, 0)
+    T_in = orc.QINT8 if signed_in else orc.QUINT8
+    xq, xmn, xmx = quant_in(x, T_in)
+    wq, fmn, fmx = quant_filter(w)
+    g = orc.conv_geom(x.shape, w.shape)
+    deq = "dequantize" in case
+    t_out = orc.FLOAT if deq else (orc.QINT8 if case.endswith("s8") else orc.QUINT8)
+    at = orc.ConvAttrs(T_in, t_out, orc.FLOAT if b is not None else 0, orc.ACT_RELU if relu else orc.ACT_NONE, 0.0)
+    zmn, zmx = float(ref.min()), float(ref.max())
+    st, out = orc.qconv2d(at, g, xq, wq, b, xmn, xmx, fmn, fmx, zmn, zmx)
+    assert st == orc.OK
+    if deq:
+        got = out
+    else:
+        _, got = orc.dequantize(out, zmn, zmx, t_out, orc.SCALED)
+    np.testing.assert_allclose(got, ref, rtol=0.3, atol=0.3)            # the reference test's own bar
+    # tighter: 36 products, each operand off by at most half a quantization step, plus half an output step
+    rx, rw = np.abs(x).max(), np.abs(w).max(axis=(0, 1, 2)).max()
+    sx = rx / (127 if signed_in else 255) / 2
+    sw = rw / 127 / 2
+    bound = 36 * (sx * rw + sw * rx + sx * sw)
+    if not deq:
+        bound += max(abs(zmn), abs(zmx)) / (127 if t_out == orc.QINT8 else 255) / 2
+    assert np.abs(got - ref).max() <= bound * 1.001
+    assert np.abs(got - ref).max() > 0
+
+
+def test_scales_closed_forms_and_qint32_forms():
+    rng = np.random.default_rng(4)
+    N = 6
+    fmn = -(rng.random(N).astype(np.float32) + 0.5)
+    fmx = (-fmn * np.float32(0.8)).astype(np.float32)
+    rf = np.maximum(np.abs(fmn), np.abs(fmx))
+    b32 = rng.integers(-2000, 2000, N).astype(np.int32)
+    bf = rng.standard_normal(N).astype(np.float32)
+    L = np.float32(255 * 127)
+    # float output: scale = (range_in / 255) * (range_filter / 127); a qint32 bias is multiplied by range_in * range_f / L
+    at = orc.ConvAttrs(orc.QUINT8, orc.FLOAT, orc.QINT32, orc.ACT_NONE, 0.0)
+    st, sc, sb, ep = orc.qconv_prepare(at, N, 0.0, 4.0, fmn, fmx, 0.0, 0.0, b32)
+    assert st == orc.OK and ep.n_scales == N and ep.n_eltwise == 0
+    np.testing.assert_array_equal(sc, (np.float32(4.0) / np.float32(255)) * (rf / np.float32(127)))
+    np.testing.assert_array_equal(sb, b32.astype(np.float32) * ((np.float32(4.0) * rf) / L))
+    # qint8 output from qint8 input: scale = 127 * r_in * r_f / (127 * 127 * r_out); float bias lands as b * 127 / r_out (to rounding)
+    at = orc.ConvAttrs(orc.QINT8, orc.QINT8, orc.FLOAT, orc.ACT_RELU, 0.0)
+    st, sc, sb, ep = orc.qconv_prepare(at, N, -3.0, 2.0, fmn, fmx, -8.0, 6.0, bf)
+    assert st == orc.OK and ep.n_eltwise == 1 and ep.elt[0].alg == orc.ELT_RELU
+    np.testing.assert_array_equal(sc, np.float32(127) * np.float32(3.0) * rf / (np.float32(127 * 127) * np.float32(8.0)))
+    np.testing.assert_allclose(sb, bf * np.float32(127 / 8.0), rtol=3e-7)
+    # qint32 output: unit scales, a qint32 bias is used as it is, a float bias is expressed in accumulator units
+    at = orc.ConvAttrs(orc.QUINT8, orc.QINT32, orc.QINT32, orc.ACT_NONE, 0.0)
+    st, sc, sb, _ = orc.qconv_prepare(at, N, 0.0, 4.0, fmn, fmx, 0.0, 0.0, b32)
+    np.testing.assert_array_equal(sc, np.ones(N, np.float32))
+    np.testing.assert_array_equal(sb, b32.astype(np.float32))
+    at = orc.ConvAttrs(orc.QUINT8, orc.QINT32, orc.FLOAT, orc.ACT_NONE, 0.0)
+    st, sc, sb, _ = orc.qconv_prepare(at, N, 0.0, 4.0, fmn, fmx, 0.0, 0.0, bf)
+    np.testing.assert_array_equal(sb, bf * ((L / (np.float32(4.0) * rf)) * np.float32(1.0)))
+    # per-tensor filter range: one scale for all channels
+    at = orc.ConvAttrs(orc.QUINT8, orc.FLOAT, orc.FLOAT, orc.ACT_LEAKYRELU, 0.1)
+    st, sc, sb, ep = orc.qconv_prepare(at, N, 0.0, 4.0, fmn[:1], fmx[:1], 0.0, 0.0, bf)
+    assert st == orc.OK and ep.n_scales == 1 and ep.elt[0].alpha == np.float32(0.1)
+    st, _, _, _ = orc.qconv_prepare(at, N, 0.0, 4.0, fmn[:3], fmx[:3], 0.0, 0.0, bf)
+    assert st == orc.INVALID_ARGUMENT
