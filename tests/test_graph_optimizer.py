@@ -108,7 +108,9 @@ def test_every_renamed_op_has_a_kernel_and_an_op_definition(opt):
            "QuantizedMatMulWithBiasAndRelu", "QuantizedMatMulWithBiasAndReluAndRequantize", "QuantizedMatMulWithBiasAndRequantize",
            "_QuantizedBatchMatMul", "_QuantizedBatchMatMulV2AndDequantize", "_QuantizedFusedBatchMatMulV2AndDequantize",
            "_QuantizedFusedMatMul", "_QuantizedFusedMatMulAndDequantize", "_QuantizedFusedMatMulAndRequantize", "_QuantizedMatMul",
-           "QuantizedReshape", "_QuantizedTranspose"]
+           "QuantizedReshape", "_QuantizedTranspose", "QuantizedConv2D", "QuantizedConv2DAndRequantize",
+           "QuantizedConv2DPerChannel", "QuantizedConv2DWithBias", "QuantizedConv2DWithBiasAndRelu",
+           "QuantizedConv2DWithBiasAndReluAndRequantize", "QuantizedConv2DWithBiasAndRequantize"]
     g = gd.GraphDef()
     for i, op in enumerate(ops):
         gd.node(g, "n%d" % i, op, ["x"], DEV, mode="SCALED", T=("type", QINT8))
@@ -117,6 +119,21 @@ def test_every_renamed_op_has_a_kernel_and_an_op_definition(opt):
         assert n.op == "_ITEX" + op.lstrip("_"), (op, n.op)
         assert n.op in kernels, n.op
         assert n.op in defined, n.op
+
+
+def test_conv_rows(opt):
+    # legacy names get data_format = "NHWC" added (layout_utils.cc:471-495); the new API op becomes ...V2 with its
+    # attributes copied unchanged (native_layout.cc:178-179)
+    g = gd.GraphDef()
+    gd.node(g, "c1", "QuantizedConv2DWithBiasAndRequantize", ["x", "w", "b"], DEV, Tinput=("type", QUINT8), padding="SAME")
+    gd.node(g, "c2", "_QuantizedConv2D", ["x", "w"], DEV, Tinput=("type", QINT8), data_format="NHWC", padding="VALID")
+    gd.node(g, "c3", "QuantizedConv2D", ["x", "w"], CPU, Tinput=("type", QUINT8))
+    out = by_name(run(opt, g))
+    assert out["c1"].op == "_ITEXQuantizedConv2DWithBiasAndRequantize"
+    assert out["c1"].attr["data_format"].s == b"NHWC" and out["c1"].attr["padding"].s == b"SAME"
+    assert out["c1"].attr["Tinput"].type == QUINT8 and list(out["c1"].input) == ["x", "w", "b"]
+    assert out["c2"].op == "_ITEXQuantizedConv2DV2" and out["c2"].attr["padding"].s == b"VALID"
+    assert out["c3"].op == "QuantizedConv2D" and "data_format" not in out["c3"].attr
 
 
 def test_reshape_is_only_renamed_for_qint8(opt):

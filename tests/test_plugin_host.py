@@ -199,3 +199,49 @@ def test_shape_op_registrations(reg):
         assert all(k["host_memory"] == host for k in ks)
     names = {o["name"] for o in reg["ops"]}
     assert "_QuantizedTranspose" in names and "_ITEXQuantizedReshape" in names and "QuantizedReshape" not in names
+
+
+def test_conv_registrations(reg):
+    # itex/core/kernels/gpu/quantized_conv_ops.cc:77-310
+    plain = ["min_input", "max_input", "min_filter", "max_filter", "min_output", "max_output"]
+    req = plain[:4] + ["min_freezed_output", "max_freezed_output", "min_output", "max_output"]
+    table = {"QuantizedConv2D": ({tf.QINT8, tf.QUINT8}, {tf.QINT32}, plain),
+             "QuantizedConv2DPerChannel": ({tf.QINT8, tf.QUINT8}, {tf.QINT32}, plain),
+             "QuantizedConv2DWithBias": ({tf.QINT8, tf.QUINT8}, {tf.QINT32}, plain),
+             "QuantizedConv2DWithBiasAndRelu": ({tf.QINT8, tf.QUINT8}, {tf.QINT32}, plain),
+             "QuantizedConv2DAndRequantize": ({tf.QINT8, tf.QUINT8}, {tf.QINT8}, req),
+             "QuantizedConv2DWithBiasAndRequantize": ({tf.QINT8, tf.QUINT8}, {tf.QINT8}, req),
+             "QuantizedConv2DWithBiasAndReluAndRequantize": ({tf.QINT8, tf.QUINT8}, {tf.QUINT8}, req)}
+    for name, (tin, tout, host) in table.items():
+        for op in (name, "_ITEX" + name):
+            ks = kernels_of(reg, op)
+            assert ks, op
+            assert {k["constraints"]["Tinput"] for k in ks} == tin, op
+            assert {k["constraints"]["out_type"] for k in ks} == tout, op
+            assert all(k["constraints"]["Tfilter"] == tf.QINT8 and k["host_memory"] == host for k in ks), op
+    for op in ("QuantizedConv2DWithBiasAndRequantize", "QuantizedConv2DWithBiasAndReluAndRequantize"):
+        assert {k["constraints"]["Tbias"] for k in kernels_of(reg, op)} == {tf.FLOAT, tf.QINT32}
+    for op in ("_QuantizedConv2D", "_ITEXQuantizedConv2DV2"):
+        ks = kernels_of(reg, op)
+        assert {k["constraints"]["out_type"] for k in ks} == {tf.QINT8, tf.QUINT8, tf.QINT32, tf.FLOAT, tf.BFLOAT16}
+        assert all(k["host_memory"] == ["host_inputs", "host_outputs"] for k in ks)
+    # stock TensorFlow defines the legacy names and _QuantizedConv2D; the plugin must define the renamed ones only
+    names = {o["name"] for o in reg["ops"]}
+    assert "_ITEXQuantizedConv2DV2" in names and "_ITEXQuantizedConv2DWithBiasAndRequantize" in names
+    assert "QuantizedConv2D" not in names
+
+
+def test_conv_attr_validation():
+    base = dict(Tinput=DT(tf.QUINT8), Tfilter=DT(tf.QINT8), out_type=DT(tf.QINT32), strides=[1, 1, 1, 1], dilations=[1, 1, 1, 1],
+                padding="SAME", padding_list=[])
+    assert tf.Node("QuantizedConv2D", base).code == tf.OK
+    for bad, code, msg in ((dict(strides=[1, 1, 1]), tf.INVALID_ARGUMENT, "Sliding window strides field must specify 4 dimensions"),
+                           (dict(dilations=[1, 1]), tf.INVALID_ARGUMENT, "Sliding window dilations field must specify 4 dimensions"),
+                           (dict(strides=[1, 0, 1, 1]), tf.INVALID_ARGUMENT, "Row and column strides should be larger than 0."),
+                           (dict(dilations=[1, 1, 0, 1]), tf.INVALID_ARGUMENT, "Dilated rates should be larger than 0."),
+                           (dict(padding="EXPLICIT", padding_list=[0, 0, 1]), tf.INVALID_ARGUMENT, None),
+                           (dict(strides=[2, 1, 1, 1]), tf.UNIMPLEMENTED, None)):
+        n = tf.Node("QuantizedConv2D", dict(base, **bad))
+        assert n.code == code, (bad, n.code, n.message)
+        if msg:
+            assert n.message == msg
