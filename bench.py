@@ -289,15 +289,19 @@ def bench_bmm(torch, hip, timer, steps, warmup, dev):
 
 
 def bench_conv(torch, hip, timer, steps, warmup, dev):
-    """Quantized Conv2D [BiasAdd, Relu, Requantize] quint8 -> quint8 at two ResNet-50 layer shapes, batch 32: the patch
-    matrix (itexhip_im2col8) plus the quantized GEMM, as the op kernel runs them; the 1x1 layer needs no patches.
-    Algorithmic bytes = input + filter + output (the patch matrix is this implementation's own extra traffic)."""
+    """Quantized Conv2D [BiasAdd, Relu, Requantize] quint8 -> quint8 at ResNet-50 layer shapes, batch 32, as the op kernel
+    runs them: the 3x3 layers as an implicit GEMM (itexhip_qconv2d) and, for comparison, as patch matrix
+    (itexhip_im2col8) + GEMM; the 1x1 layer is a plain GEMM.  Algorithmic bytes = input + filter + output."""
     out = []
     g_ = torch.Generator(device=dev)
     g_.manual_seed(50)
     st = _stream(torch)
-    for name, (B, H, W, C), (KH, KW, O), stride in (("conv3x3_56x56x64_to_64", (32, 56, 56, 64), (3, 3, 64), 1),
-                                                    ("conv1x1_56x56x256_to_64", (32, 56, 56, 256), (1, 1, 64), 1)):
+    for name, (B, H, W, C), (KH, KW, O), stride, patches in (
+            ("conv3x3_56x56x64_to_64", (32, 56, 56, 64), (3, 3, 64), 1, False),
+            ("conv3x3_56x56x64_to_64_patch_matrix", (32, 56, 56, 64), (3, 3, 64), 1, True),
+            ("conv3x3_28x28x128_to_128", (32, 28, 28, 128), (3, 3, 128), 1, False),
+            ("conv3x3_14x14x256_to_256", (32, 14, 14, 256), (3, 3, 256), 1, False),
+            ("conv1x1_56x56x256_to_64", (32, 56, 56, 256), (1, 1, 64), 1, False)):
         x = torch.randint(0, 256, (B, H, W, C), dtype=torch.uint8, device=dev, generator=g_)
         w = torch.randint(-127, 128, (KH * KW * C, O), dtype=torch.int8, device=dev, generator=g_)
         K = KH * KW * C
@@ -313,10 +317,15 @@ def bench_conv(torch, hip, timer, steps, warmup, dev):
         y = torch.empty((M, O), dtype=torch.uint8, device=dev)
         pad = (KH - 1) // 2
         geo = hip.ConvGeometry(B, H, W, C, KH, KW, H, W, stride, stride, 1, 1, pad, pad)
-        cols = torch.empty((M, K), dtype=torch.uint8, device=dev) if KH * KW > 1 else None
+        cols = torch.empty((M, K), dtype=torch.uint8, device=dev) if patches else None
+        implicit = KH * KW > 1 and not patches
+        assert not implicit or hip.qconv2d_implicit_ok(geo, x, O, hip.QUINT8, y)
 
         def make(stream):
             def fn(i):
+                if implicit:
+                    hip.qconv2d(x, hip.QUINT8, geo, packed, colsum, O, scales, bias, ep, hip.QUINT8, y, stream)
+                    return
                 a = x
                 if cols is not None:
                     hip.im2col8(x, geo, K, cols, stream)
@@ -329,7 +338,7 @@ def bench_conv(torch, hip, timer, steps, warmup, dev):
         t_roof = max(ops / (PEAK_INT8_TOPS * 1e12), nbytes / (PEAK_HBM_GBS * 1e9))
         out.append(dict(name=name, M=M, K=K, N=O, us_kernel=ms * 1e3, bytes=nbytes, ops=ops, bound="max(mfma,hbm)",
                         frac=t_roof / (ms * 1e-3), tops=ops / (ms * 1e-3) / 1e12, gbs=nbytes / (ms * 1e-3) / 1e9,
-                        note="im2col + GEMM launches" if cols is not None else "GEMM launch only"))
+                        note="implicit GEMM, one launch" if implicit else "im2col + GEMM launches" if patches else "GEMM launch only"))
         del x, w, packed, y, cols
     return out
 

@@ -360,6 +360,19 @@ int itexhip_im2col8(const void* x, const itexhip_conv_geometry* g, int64_t row_b
 int itexhip_scale_vector(const void* bias, int bias_type, const float* factors, int64_t n_factors, int64_t n,
                          float* out, void* stream);
 
+/* The convolution without the patch matrix: the MatMul tile kernel gathers its activation tiles straight from the
+ * NHWC input (an implicit GEMM; it stands where the reference executes its oneDNN
+ * convolution primitive, conv_ops.h:1021, 1119), same arguments otherwise as itexhip_qgemm with M = batch * out_h * out_w and
+ * K = k_h * k_w * in_c; `packed_filter` / `colsum` from itexhip_qgemm_prepack_b(filter, 0, K, out_channels, ...).
+ * Takes the calls for which itexhip_qconv2d_implicit_ok returns 1 (in_c a multiple of 16, k_h * k_w * in_c <= 16384,
+ * 16-byte aligned input of less than 2 GiB; output qint32 / qint8 / quint8 / float / bfloat16 with 16-byte aligned
+ * rows) and rejects the others, which go through itexhip_im2col8 + itexhip_qgemm.  `bias` must not be null. */
+int itexhip_qconv2d_implicit_ok(const itexhip_conv_geometry* g, const void* x, int64_t out_channels, int out_type,
+                                const void* out);
+int itexhip_qconv2d(const void* x, int x_type, const itexhip_conv_geometry* g, const int8_t* packed_filter,
+                    const int32_t* colsum, int64_t out_channels, const float* scales, const float* bias,
+                    const itexhip_epilogue* ep, int out_type, void* out, void* stream);
+
 /* Diagnostic, no counterpart in the reference: `workgroups` x 4 wavefronts each issue iters x 8
  * independent 32x32x32 i8 MFMAs (2 * 32768 ops each) on the 8 KiB of operand fragments at `operands`
  * (device memory, 16-byte aligned) and nothing else.  Timed by the caller, it gives the rate the matrix

@@ -27,6 +27,10 @@ template <int OUT_T>
 int dispatch_tile(const uint8_t* a, uint32_t a_xor, const uint8_t* bp, int M, int K, int N,
                   const EpilogueArgs& e, void* out, hipStream_t st);
 
+template <int OUT_T>
+int dispatch_tile_conv(const uint8_t* x, uint32_t a_xor, const uint8_t* bp, int M, int K, int N, const EpilogueArgs& e,
+                       void* out, hipStream_t st, const ConvTileArgs& cv);
+
 namespace {
 
 // ------------------------------------------------------------------------------------------------
@@ -460,6 +464,69 @@ extern "C" int itexhip_qgemm(const void* a, int a_type, const int8_t* packed_b, 
                              const itexhip_epilogue* ep, int out_type, void* out, void* stream) {
   return packed_path(M <= 16, a, a_type, packed_b, colsum, M, K, N, scales, bias, ep, out_type, out, stream,
                      "itexhip_qgemm");
+}
+
+// ------------------------------------------------------------------------------------------------
+// Conv2D as an implicit GEMM
+// ------------------------------------------------------------------------------------------------
+namespace {
+bool conv_implicit_ok(const itexhip_conv_geometry* g, const void* x, int64_t out_channels, int out_type, const void* out) {
+  const int esz = (out_type == ITEXHIP_QINT8 || out_type == ITEXHIP_QUINT8) ? 1 : out_type == ITEXHIP_BFLOAT16 ? 2 : 4;
+  if (out_type == ITEXHIP_HALF || out_channels <= 0 || out_channels >= (1LL << 31) || (out_channels * esz) % 16 != 0 || !aligned(out, 16))
+    return false;
+  if (!g || g->batch <= 0 || g->in_h <= 0 || g->in_w <= 0 || g->in_c <= 0 || g->k_h <= 0 || g->k_w <= 0 ||
+      g->out_h <= 0 || g->out_w <= 0 || g->stride_h <= 0 || g->stride_w <= 0 || g->dil_h <= 0 || g->dil_w <= 0)
+    return false;
+  const int64_t K = g->k_h * g->k_w * g->in_c;
+  const int64_t lim = 1LL << 31;
+  return g->in_c % 16 == 0 && K / 16 <= kMaxConvPieces && aligned(x, 16) && g->batch * g->in_h * g->in_w * g->in_c < lim &&
+         g->batch * g->out_h * g->out_w < lim && (g->k_h - 1) * g->dil_h < (1 << 15) && (g->k_w - 1) * g->dil_w < (1 << 15) &&
+         g->pad_top >= 0 && g->pad_left >= 0 && g->pad_top < (1 << 24) && g->pad_left < (1 << 24) &&
+         g->out_h * g->stride_h < (1LL << 30) && g->out_w * g->stride_w < (1LL << 30);
+}
+}  // namespace
+
+extern "C" int itexhip_qconv2d_implicit_ok(const itexhip_conv_geometry* g, const void* x, int64_t out_channels, int out_type,
+                                           const void* out) {
+  return conv_implicit_ok(g, x, out_channels, out_type, out) ? 1 : 0;
+}
+
+extern "C" int itexhip_qconv2d(const void* x, int x_type, const itexhip_conv_geometry* g, const int8_t* packed_filter,
+                               const int32_t* colsum, int64_t out_channels, const float* scales, const float* bias,
+                               const itexhip_epilogue* ep, int out_type, void* out, void* stream) {
+  const char* who = "itexhip_qconv2d";
+  ITEXHIP_REQUIRE(g != nullptr, "%s: null geometry", who);
+  ITEXHIP_REQUIRE(conv_implicit_ok(g, x, out_channels, out_type, out),
+                  "%s: not a shape for the implicit GEMM (in_c %% 16 == 0, window <= 16 KiB, 16-byte aligned input below 2 GiB, "
+                  "16-byte aligned output rows); use itexhip_im2col8 + itexhip_qgemm", who);
+  ITEXHIP_REQUIRE(bias != nullptr, "%s: needs a bias vector (zeros when the op has none)", who);
+  const int64_t M = g->batch * g->out_h * g->out_w, K = g->k_h * g->k_w * g->in_c, N = out_channels;
+  if (int st = check_common(x, x_type, packed_filter, M, K, N, scales, ep, out_type, out, who)) return st;
+  if (N == 0) return ITEXHIP_OK;
+  ITEXHIP_REQUIRE(aligned(packed_filter, 16), "%s: the packed filter must be 16-byte aligned", who);
+  ITEXHIP_REQUIRE(x_type != ITEXHIP_QUINT8 || colsum, "%s: quint8 input needs colsum", who);
+  const EpilogueArgs e = make_args(x_type, colsum, scales, bias, ep);
+  ConvTileArgs cv;
+  cv.in_h = static_cast<int>(g->in_h); cv.in_w = static_cast<int>(g->in_w); cv.in_c = static_cast<int>(g->in_c);
+  cv.k_w = static_cast<int>(g->k_w); cv.out_h = static_cast<int>(g->out_h); cv.out_w = static_cast<int>(g->out_w);
+  cv.stride_h = g->stride_h; cv.stride_w = g->stride_w; cv.dil_h = g->dil_h; cv.dil_w = g->dil_w;
+  cv.pad_top = static_cast<int>(g->pad_top); cv.pad_left = static_cast<int>(g->pad_left);
+  const uint32_t a_xor = (x_type == ITEXHIP_QUINT8) ? 0x80808080u : 0u;
+  const uint8_t* xp = reinterpret_cast<const uint8_t*>(x);
+  const uint8_t* bp = reinterpret_cast<const uint8_t*>(packed_filter);
+  hipStream_t hs = as_stream(stream);
+  const int Mi = static_cast<int>(M), Ki = static_cast<int>(K), Ni = static_cast<int>(N);
+  int st__ = ITEXHIP_OK;
+  switch (out_type) {
+    case ITEXHIP_FLOAT: st__ = dispatch_tile_conv<ITEXHIP_FLOAT>(xp, a_xor, bp, Mi, Ki, Ni, e, out, hs, cv); break;
+    case ITEXHIP_BFLOAT16: st__ = dispatch_tile_conv<ITEXHIP_BFLOAT16>(xp, a_xor, bp, Mi, Ki, Ni, e, out, hs, cv); break;
+    case ITEXHIP_QINT32: st__ = dispatch_tile_conv<ITEXHIP_QINT32>(xp, a_xor, bp, Mi, Ki, Ni, e, out, hs, cv); break;
+    case ITEXHIP_QINT8: st__ = dispatch_tile_conv<ITEXHIP_QINT8>(xp, a_xor, bp, Mi, Ki, Ni, e, out, hs, cv); break;
+    default: st__ = dispatch_tile_conv<ITEXHIP_QUINT8>(xp, a_xor, bp, Mi, Ki, Ni, e, out, hs, cv); break;
+  }
+  if (st__ != ITEXHIP_OK) return st__;
+  ITEXHIP_CHECK_LAUNCH(who);
+  return ITEXHIP_OK;
 }
 
 extern "C" int itexhip_qgemm_naive(const void* a, int a_type, const int8_t* w, int transpose_b, int64_t M,

@@ -20,6 +20,17 @@ constexpr int kChunkK = 32;        // k per operand chunk
 constexpr int kChunkBytes = 1024;  // 32 rows x 32 k
 constexpr int64_t kMaxK = 1 << 16; // 255 * 128 * 65536 < 2^31
 
+// A post-op chain of the form [one activation] [one linear map], either part optional (every chain the MatMul and
+// convolution ops build without an addend): resolved once on the host, so that the tile kernels apply it with a few
+// wavefront-uniform branches per 32x32 tile instead of a loop over the chain per value.
+enum : int { kChainMax0 = 1, kChainLeaky = 2, kChainClip = 4, kChainLinear = 8, kChainGeluTanh = 16, kChainGeluErf = 32 };
+struct CanonChain {
+  int flags;
+  float alpha;         // leaky slope
+  float lo, hi;        // clip bounds
+  float lin_a, lin_b;  // y = lin_a * x + lin_b
+};
+
 struct EpilogueArgs {
   const float* scales;   // prepared per-channel scales (n_scales of them), unused when `fused`
   const void* bias;      // prepared fp32 bias, or the op's raw bias (fp32 / int32) when `fused`
@@ -39,7 +50,36 @@ struct EpilogueArgs {
   // in place of prep.min_a / prep.max_a; null for the reference's per-tensor range
   const float* row_min_a;
   const float* row_max_a;
+  CanonChain canon;  // filled by the tile dispatch for the kernels that take it
 };
+
+// Host: the chain in canonical form.  Returns 0 (no post-op), 1 (ReLU only), 2 (cheap activation and / or linear map),
+// 3 (GELU, optional linear map) or -1 (anything else: an addend, two activations, ...).
+inline int canon_chain(const EpilogueArgs& e, CanonChain* c) {
+  *c = CanonChain{};
+  int k = 0;
+  if (k < e.n_eltwise) {
+    const itexhip_eltwise& a = e.elt[k];
+    if (a.alg == ITEXHIP_ELT_RELU) {
+      if (a.alpha == 0.0f) c->flags |= kChainMax0; else { c->flags |= kChainLeaky; c->alpha = a.alpha; }
+      ++k;
+    } else if (a.alg == ITEXHIP_ELT_CLIP) {
+      c->flags |= kChainClip; c->lo = a.alpha; c->hi = a.beta;
+      ++k;
+    } else if (a.alg == ITEXHIP_ELT_GELU_TANH || a.alg == ITEXHIP_ELT_GELU_ERF) {
+      c->flags |= a.alg == ITEXHIP_ELT_GELU_TANH ? kChainGeluTanh : kChainGeluErf;
+      ++k;
+    }
+  }
+  if (k < e.n_eltwise && e.elt[k].alg == ITEXHIP_ELT_LINEAR) {
+    c->flags |= kChainLinear; c->lin_a = e.elt[k].alpha; c->lin_b = e.elt[k].beta;
+    ++k;
+  }
+  if (k != e.n_eltwise) return -1;
+  if (c->flags == 0) return 0;
+  if (c->flags == kChainMax0) return 1;
+  return (c->flags & (kChainGeluTanh | kChainGeluErf)) ? 3 : 2;
+}
 
 // Scale, bias and zero-point compensation of channel n (n < N), however the call supplied them, in two
 // stages so that a kernel can issue the loads early and do the arithmetic late.
@@ -97,26 +137,14 @@ struct ChannelParams {
   float bias[4];
 };
 
-// The 4 outputs of one channel group in registers: epilogue arithmetic + conversion, no store.
-// 8-bit outputs come back packed in .x; 32-bit outputs as 4 lanes of raw bits.
+// Four final fp32 values (as bit patterns) -> four outputs of type OUT_T in registers, no store.
+// 8-bit outputs come back packed in .x, 16-bit ones in .x and .y; 32-bit outputs as 4 lanes of raw bits.
 // 8-bit conversion: after the clamp to [lo, hi] (integers, |.| <= 255) adding 1.5 * 2^23 in fp32
 // rounds to nearest even and leaves the integer in the low mantissa bits (two's complement for
 // negatives), so the low byte of the sum is the result: one add instead of round + convert.
-template <int OUT_T, int ACT>
-__device__ __forceinline__ v4i epilogue_convert(const v4i acc, const f4 scale, const f4 bias, const EpilogueArgs& e) {
-  float y[4];
-#pragma unroll
-  for (int r = 0; r < 4; ++r) {
-    float v = static_cast<float>(acc[r]);  // the zero-point compensation is already part of acc
-    v = v * scale[r];
-    v = v + bias[r];
-    if (ACT == 1) {
-      v = fmaxf(v, 0.0f);
-    } else if (ACT == 2) {
-      for (int k = 0; k < e.n_eltwise; ++k) v = apply_eltwise(e.elt[k], v);
-    }
-    y[r] = v;
-  }
+template <int OUT_T>
+__device__ __forceinline__ v4i epilogue_pack(const v4i bits) {
+  const float y[4] = {__int_as_float(bits[0]), __int_as_float(bits[1]), __int_as_float(bits[2]), __int_as_float(bits[3])};
   if constexpr (OUT_T == ITEXHIP_FLOAT) {
     return v4i{__float_as_int(y[0]), __float_as_int(y[1]), __float_as_int(y[2]), __float_as_int(y[3])};
   } else if constexpr (is_float16_type(OUT_T)) {  // 4 x 16 bits in .x, .y
@@ -137,6 +165,26 @@ __device__ __forceinline__ v4i epilogue_convert(const v4i acc, const f4 scale, c
     const uint32_t hi23 = __builtin_amdgcn_perm(b[3], b[2], 0x04000c0cu);  // [0, 0, b2.0, b3.0]
     return v4i{static_cast<int>(lo01 | hi23), 0, 0, 0};
   }
+}
+
+// The 4 outputs of one channel group: accumulators (zero-point compensation already included) -> scale, bias,
+// activation -> epilogue_pack.
+template <int OUT_T, int ACT>
+__device__ __forceinline__ v4i epilogue_convert(const v4i acc, const f4 scale, const f4 bias, const EpilogueArgs& e) {
+  v4i y;
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    float v = static_cast<float>(acc[r]);
+    v = v * scale[r];
+    v = v + bias[r];
+    if (ACT == 1) {
+      v = fmaxf(v, 0.0f);
+    } else if (ACT == 2) {
+      for (int k = 0; k < e.n_eltwise; ++k) v = apply_eltwise(e.elt[k], v);
+    }
+    y[r] = __float_as_int(v);
+  }
+  return epilogue_pack<OUT_T>(y);
 }
 
 template <int OUT_T, int ACT>
@@ -206,6 +254,13 @@ template <int N, class F>
 __device__ __forceinline__ void static_for(F&& f) {
   static_for_impl(static_cast<F&&>(f), std::make_integer_sequence<int, N>{});
 }
+
+// Geometry of a Conv2D computed as an implicit GEMM by the tile kernel (32-bit: the host checks the ranges)
+struct ConvTileArgs {
+  int in_h, in_w, in_c, k_w, out_h, out_w;
+  int stride_h, stride_w, dil_h, dil_w, pad_top, pad_left;
+};
+constexpr int kMaxConvPieces = 1024;  // 16-byte pieces per patch row: 16 KiB of receptive field per output position
 
 }  // namespace itexhip
 #endif  // ITEXHIP_QGEMM_COMMON_HPP_

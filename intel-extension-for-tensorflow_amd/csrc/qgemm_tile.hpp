@@ -56,14 +56,27 @@ __device__ __forceinline__ void wait_vmcnt() {
   __builtin_amdgcn_s_waitcnt((N & 15) | (7 << 4) | (15 << 8) | ((N >> 4) << 14));
 }
 
+// Implicit GEMM of a Conv2D (NHWC input, in_c a multiple of 16): the activation "matrix" is the patch matrix
+// [batch * out_h * out_w, k_h * k_w * in_c], never materialised.  A 16-byte piece of a patch row lies inside one
+// input pixel (or in the padding, then it is read from 16 zero bytes), so only the source address of an activation
+// load changes: row -> window origin once per kernel, piece -> offset inside the window from a table in LDS.
+struct NoConvArgs {};
+template <bool CONV> struct conv_args_of { using type = NoConvArgs; };
+template <> struct conv_args_of<true> { using type = ConvTileArgs; };
+static __device__ __align__(16) const uint32_t kZeroPiece[4] = {0u, 0u, 0u, 0u};
+
 // amask: 0x80808080 when the activations are unsigned (they are fed as x ^ 0x80), else 0; a scalar
 // register operand, so the sign flip costs a 4-byte instruction per dword.  KALIGNED: K is a multiple
 // of 64, so activation loads never need a per-lane clamp and use a uniform base that advances by 64
 // bytes per step.
-template <int BM, int BN, int WAVES_M, int WAVES_N, int OUT_T, int ACT, bool KALIGNED>
+template <int BM, int BN, int WAVES_M, int WAVES_N, int OUT_T, int ACT, bool KALIGNED, bool CONV = false, bool ELEMENTWISE = false>
 __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void qgemm_tile_kernel(
     const uint8_t* __restrict__ a, uint32_t amask, const uint8_t* __restrict__ bp, int M, int K, int N,
-    int KT, int NT, int num_m, int num_n, EpilogueArgs e, void* __restrict__ out) {
+    int KT, int NT, int num_m, int num_n, EpilogueArgs e, void* __restrict__ out,
+    typename conv_args_of<CONV>::type cv) {
+  static_assert(!CONV || !KALIGNED, "the implicit GEMM addresses every activation piece per lane");
+  static_assert(!ELEMENTWISE || (ACT == 2 && !KALIGNED && !CONV), "the element-wise epilogue exists in the conservative form only");
+  static_assert(ACT >= 0 && ACT <= 3, "0 none, 1 ReLU, 2 canonical chain (cheap activation), 3 canonical chain (GELU)");
   constexpr int NW = WAVES_M * WAVES_N;
   constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
   constexpr int TM = WM / 32, TN = WN / 32;
@@ -80,10 +93,13 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void qgemm_tile_kernel(
   constexpr int B_REGION = A_LOADS * kChunkBytes;
   // behind the ring: the per-channel epilogue parameters of this block's BN channels
   constexpr int PANEL_OFF = NSTAGE * STAGE_BYTES;
-  // the element-wise (any alignment, any N, optional bias) epilogue is only compiled into the
-  // conservative instantiation; the host sends such calls there
-  constexpr bool GENERAL = (ACT == 2) && !KALIGNED;
+  // the element-wise (any alignment, any N, optional bias, addend) epilogue is a kernel of its own; the host
+  // sends the calls that need it there.  Compiled next to the vector epilogue it slowed that one down by a third.
+  constexpr bool GENERAL = ELEMENTWISE;
   static_assert(BN <= 64 * NW, "one thread per channel fills the parameter panel");
+  // behind the panel (implicit GEMM only): per 16-byte piece of a patch row, {window row << 16 | window column,
+  // byte offset from the window origin}
+  constexpr int CONV_TAB_OFF = PANEL_OFF + 12 * BN;
 
   extern __shared__ __align__(16) uint8_t lds[];
   const uint32_t lds_base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(
@@ -112,23 +128,56 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void qgemm_tile_kernel(
   const int q_piece = (lane & 3) ^ ((q_row >> 1) & 3);  // piece = 2*kc + g
   uint32_t off_a[A_PER_WAVE];       // byte offset of the lane's row (+ piece when KALIGNED) in the activation matrix
   const uint8_t* src_b[B_PER_WAVE];  // wavefront-uniform chunk pointers of step 0
+  int win_h[A_PER_WAVE], win_w[A_PER_WAVE];  // implicit GEMM: window origin of the lane's row (may lie in the padding)
+  const int2* const conv_tab = reinterpret_cast<const int2*>(lds + CONV_TAB_OFF);
   static_for<A_PER_WAVE>([&](auto c) {
     const int ld = wave * A_PER_WAVE + c;  // 0 .. A_LOADS-1 = (rt, h)
     const int m = min(m_base + ld * 16 + q_row, M - 1);
-    off_a[c] = static_cast<uint32_t>(m) * static_cast<uint32_t>(K) +  // M * K < 2^31 checked by the host
-               (KALIGNED ? q_piece * 16 : 0);
+    if constexpr (CONV) {
+      const int t = m / cv.out_w, ow = m - t * cv.out_w;
+      const int b = t / cv.out_h, oh = t - b * cv.out_h;
+      win_h[c] = oh * cv.stride_h - cv.pad_top;
+      win_w[c] = ow * cv.stride_w - cv.pad_left;
+      // input bytes < 2^31 checked by the host; the origin may be negative, origin + an in-bounds piece is not
+      off_a[c] = static_cast<uint32_t>(((b * cv.in_h + win_h[c]) * cv.in_w + win_w[c]) * cv.in_c);
+    } else {
+      off_a[c] = static_cast<uint32_t>(m) * static_cast<uint32_t>(K) +  // M * K < 2^31 checked by the host
+                 (KALIGNED ? q_piece * 16 : 0);
+    }
   });
+  if constexpr (CONV) {
+    for (int p = threadIdx.x; p < (K >> 4); p += 64 * NW) {
+      const int k0 = p * 16;
+      const int kk = k0 / cv.in_c, cc = k0 - kk * cv.in_c;
+      const int kh = kk / cv.k_w, kw = kk - kh * cv.k_w;
+      const int dh = kh * cv.dil_h, dw = kw * cv.dil_w;  // < 2^15 each, checked by the host
+      reinterpret_cast<int2*>(lds + CONV_TAB_OFF)[p] = make_int2((dh << 16) | dw, (dh * cv.in_w + dw) * cv.in_c + cc);
+    }
+    __syncthreads();
+  }
+  // the table entry of the lane's piece in K step kt (the same for all of the lane's loads of that step)
+  auto conv_piece = [&](int kt) {
+    if constexpr (CONV) return conv_tab[min(kt * 4 + q_piece, (K >> 4) - 1)];
+    else return make_int2(0, 0);
+  };
   static_for<B_PER_WAVE>([&](auto c) {
     const int ld = wave * B_PER_WAVE + c;  // 0 .. B_LOADS-1 = (channel tile, k-chunk)
     const int nt = min((n_base >> 5) + (ld >> 1), NT - 1);
     src_b[c] = bp + (static_cast<int64_t>(nt) * (2 * KT) + (ld & 1)) * kChunkBytes;
   });
   const uint32_t lane16 = lane * 16;
-  auto issue_load = [&](auto c, int kt, int stage) {
+  auto issue_load = [&](auto c, int kt, int stage, int2 piece) {
     constexpr int ci = decltype(c)::value;
     const uint32_t stage_addr = lds_base + stage * STAGE_BYTES;
     if constexpr (ci < A_PER_WAVE) {
-      if constexpr (KALIGNED) {
+      if constexpr (CONV) {
+        const int ih = win_h[ci] + (piece.x >> 16), iw = win_w[ci] + (piece.x & 0xffff);
+        const bool inside = static_cast<unsigned>(ih) < static_cast<unsigned>(cv.in_h) &&
+                            static_cast<unsigned>(iw) < static_cast<unsigned>(cv.in_w);
+        const uint8_t* src = inside ? a + static_cast<int>(off_a[ci] + static_cast<uint32_t>(piece.y))
+                                    : reinterpret_cast<const uint8_t*>(kZeroPiece);
+        lds_dma16(src, stage_addr + (wave * A_PER_WAVE + ci) * kChunkBytes);
+      } else if constexpr (KALIGNED) {
         lds_dma16(a + static_cast<int64_t>(kt) * 64, off_a[ci], stage_addr + (wave * A_PER_WAVE + ci) * kChunkBytes);
       } else {
         const uint32_t kofs = static_cast<uint32_t>(min(kt * 64 + q_piece * 16, K - 16));
@@ -156,9 +205,12 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void qgemm_tile_kernel(
   };
 
   // ---- prologue: loads of steps 0, 1, 2 in flight; wait for steps 0 and 1
-  static_for<NLD>([&](auto c) { issue_load(c, 0, 0); });
-  static_for<NLD>([&](auto c) { issue_load(c, min(1, KT - 1), 1); });
-  static_for<NLD>([&](auto c) { issue_load(c, min(2, KT - 1), 2); });
+  {
+    const int2 p0 = conv_piece(0), p1 = conv_piece(min(1, KT - 1)), p2 = conv_piece(min(2, KT - 1));
+    static_for<NLD>([&](auto c) { issue_load(c, 0, 0, p0); });
+    static_for<NLD>([&](auto c) { issue_load(c, min(1, KT - 1), 1, p1); });
+    static_for<NLD>([&](auto c) { issue_load(c, min(2, KT - 1), 2, p2); });
+  }
   // parameter panel: thread t resolves channel n_base + t once (the flags are uniform), so the
   // epilogue is free of global loads and of branches on them
   if (threadIdx.x < BN) {
@@ -207,6 +259,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void qgemm_tile_kernel(
   auto step = [&](int kt, const v4i (&fa_cur)[FA], v4i (&fa_nxt)[FA]) {
     const int st_cur = kt & 3, st_nxt = (kt + 1) & 3, st_fill = (kt + 3) & 3;
     const int kt_load = min(kt + 3, KT - 1);
+    const int2 piece = conv_piece(kt_load);  // read at the top of the step, used by the load slots
     static_for<NSLICE>([&](auto sl) {
       constexpr int s = decltype(sl)::value;
       constexpr int kc = s / TN, j = s % TN;
@@ -222,7 +275,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void qgemm_tile_kernel(
         }
         if constexpr (ii == TM - 1) {
           static_for<NLD>([&](auto c) {
-            if constexpr (decltype(c)::value * NSLICE / NLD == s) issue_load(c, kt_load, st_fill);
+            if constexpr (decltype(c)::value * NSLICE / NLD == s) issue_load(c, kt_load, st_fill, piece);
           });
         }
         // activation fragments of the next step: read during the first half of the slices, sign
@@ -275,29 +328,89 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void qgemm_tile_kernel(
   constexpr int RPP = 64 / LPR;              // rows per flush instruction (lanes >= RPP * LPR idle)
   constexpr int PASSES = (WM + RPP - 1) / RPP;
   static_assert(NW * WM * PITCH <= NSTAGE * STAGE_BYTES, "epilogue buffer must fit in the ring");
-  const bool fast = !GENERAL || (e.addend == nullptr && (e.bias != nullptr || e.fused) && aligned16(out) && ((static_cast<int64_t>(N) * ESZ) & 15) == 0);
-  if (fast) {
+  if constexpr (!GENERAL) {
     uint8_t* ebuf = lds + wave * (WM * PITCH);
     const int f_row = lane / LPR, f_piece = lane % LPR;
+    // Post-op chain in canonical form (ACT == 2: cheap activation, ACT == 3: GELU; then an optional linear map),
+    // applied to the 16 values of one 32x32 tile at a time under wavefront-uniform branches.  A loop over the chain
+    // with a switch per value made the epilogue several times longer than the whole K loop (instruction fetch, not
+    // arithmetic).  Same expressions as apply_eltwise.
+    auto apply_chain = [&](float (&v)[16]) {
+      const CanonChain& c = e.canon;
+      if constexpr (ACT == 3) {
+        if (c.flags & kChainGeluTanh) {
+          const itexhip_eltwise el{ITEXHIP_ELT_GELU_TANH, 0.0f, 0.0f};
+#pragma unroll
+          for (int r = 0; r < 16; ++r) v[r] = apply_eltwise(el, v[r]);
+        } else {
+          const itexhip_eltwise el{ITEXHIP_ELT_GELU_ERF, 0.0f, 0.0f};
+#pragma unroll
+          for (int r = 0; r < 16; ++r) v[r] = apply_eltwise(el, v[r]);
+        }
+      } else {
+        if (c.flags & kChainMax0) {
+#pragma unroll
+          for (int r = 0; r < 16; ++r) v[r] = fmaxf(v[r], 0.0f);
+        }
+        if (c.flags & kChainLeaky) {
+#pragma unroll
+          for (int r = 0; r < 16; ++r) v[r] = v[r] > 0.0f ? v[r] : v[r] * c.alpha;
+        }
+        if (c.flags & kChainClip) {
+#pragma unroll
+          for (int r = 0; r < 16; ++r) v[r] = fminf(fmaxf(v[r], c.lo), c.hi);
+        }
+      }
+      if (c.flags & kChainLinear) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) v[r] = c.lin_a * v[r] + c.lin_b;
+      }
+    };
     static_for<TN / JB>([&](auto jb) {
       static_for<JB>([&](auto jj) {
         constexpr int j = decltype(jb)::value * JB + decltype(jj)::value;
-        static_for<4>([&](auto g) {
-          const int col = (wn * TN + j) * 32 + decltype(g)::value * 8 + lgrp * 4;
-          const f4 sc = *reinterpret_cast<const f4*>(panel_scale + col);
-          const f4 bi = *reinterpret_cast<const f4*>(panel_bias + col);
+        auto put = [&](auto i, auto g, const v4i o) {
+          uint8_t* dst = ebuf + (decltype(i)::value * 32 + lrow) * PITCH +
+                         (decltype(jj)::value * 32 + decltype(g)::value * 8 + lgrp * 4) * ESZ;
+          if constexpr (ESZ == 1) *reinterpret_cast<int*>(dst) = o.x;
+          else if constexpr (ESZ == 2) *reinterpret_cast<int2*>(dst) = make_int2(o.x, o.y);
+          else *reinterpret_cast<v4i*>(dst) = o;
+        };
+        if constexpr (ACT >= 2) {
+          f4 sc[4], bi[4];
+          static_for<4>([&](auto g) {
+            const int col = (wn * TN + j) * 32 + decltype(g)::value * 8 + lgrp * 4;
+            sc[decltype(g)::value] = *reinterpret_cast<const f4*>(panel_scale + col);
+            bi[decltype(g)::value] = *reinterpret_cast<const f4*>(panel_bias + col);
+          });
           static_for<TM>([&](auto i) {
             constexpr int t = j * TM + decltype(i)::value;
-            constexpr int r0 = decltype(g)::value * 4;
-            const v4i part = v4i{acc[t][r0], acc[t][r0 + 1], acc[t][r0 + 2], acc[t][r0 + 3]};
-            const v4i o = epilogue_convert<OUT_T, ACT>(part, sc, bi, e);
-            uint8_t* dst = ebuf + (decltype(i)::value * 32 + lrow) * PITCH +
-                           (decltype(jj)::value * 32 + decltype(g)::value * 8 + lgrp * 4) * ESZ;
-            if constexpr (ESZ == 1) *reinterpret_cast<int*>(dst) = o.x;
-            else if constexpr (ESZ == 2) *reinterpret_cast<int2*>(dst) = make_int2(o.x, o.y);
-            else *reinterpret_cast<v4i*>(dst) = o;
+            float v[16];
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+              v[r] = static_cast<float>(acc[t][r]) * sc[r >> 2][r & 3];
+              v[r] = v[r] + bi[r >> 2][r & 3];
+            }
+            apply_chain(v);
+            static_for<4>([&](auto g) {
+              constexpr int r0 = decltype(g)::value * 4;
+              put(i, g, epilogue_pack<OUT_T>(v4i{__float_as_int(v[r0]), __float_as_int(v[r0 + 1]), __float_as_int(v[r0 + 2]),
+                                                 __float_as_int(v[r0 + 3])}));
+            });
           });
-        });
+        } else {
+          static_for<4>([&](auto g) {
+            const int col = (wn * TN + j) * 32 + decltype(g)::value * 8 + lgrp * 4;
+            const f4 sc = *reinterpret_cast<const f4*>(panel_scale + col);
+            const f4 bi = *reinterpret_cast<const f4*>(panel_bias + col);
+            static_for<TM>([&](auto i) {
+              constexpr int t = j * TM + decltype(i)::value;
+              constexpr int r0 = decltype(g)::value * 4;
+              const v4i part = v4i{acc[t][r0], acc[t][r0 + 1], acc[t][r0 + 2], acc[t][r0 + 3]};
+              put(i, g, epilogue_convert<OUT_T, ACT>(part, sc, bi, e));
+            });
+          });
+        }
       });
       // flush: lane -> (row, 16-byte piece); LDS operations of one wavefront complete in order
       const int n_col = n_base + (wn * TN + decltype(jb)::value * JB) * 32 + f_piece * (16 / ESZ);
@@ -311,7 +424,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void qgemm_tile_kernel(
           *reinterpret_cast<v4i*>(reinterpret_cast<uint8_t*>(out) + (static_cast<int64_t>(m) * N + n_col) * ESZ) = v;
       }
     });
-  } else if constexpr (GENERAL) {
+  } else {
     const bool has_bias = e.bias != nullptr || e.fused;
     static_for<TN>([&](auto j) {
       static_for<4>([&](auto g) {
@@ -346,13 +459,14 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void qgemm_tile_kernel(
   }
 }
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, int OUT_T, int ACT, bool KALIGNED>
+template <int BM, int BN, int WAVES_M, int WAVES_N, int OUT_T, int ACT, bool KALIGNED, bool CONV = false, bool ELEMENTWISE = false>
 int launch_tile(const uint8_t* a, uint32_t amask, const uint8_t* bp, int M, int K, int N, const EpilogueArgs& e,
-                void* out, hipStream_t st) {
+                void* out, hipStream_t st, typename conv_args_of<CONV>::type cv = {}) {
   const int KT = (K + 63) / 64, NT = (N + kChunkRows - 1) / kChunkRows;
   const int num_m = (M + BM - 1) / BM, num_n = (N + BN - 1) / BN;
-  constexpr size_t lds_bytes = 4 * (BM / 16 + BN / 16) * kChunkBytes + 12 * BN;
-  auto kern = qgemm_tile_kernel<BM, BN, WAVES_M, WAVES_N, OUT_T, ACT, KALIGNED>;
+  constexpr size_t lds_bytes = 4 * (BM / 16 + BN / 16) * kChunkBytes + 12 * BN + (CONV ? kMaxConvPieces * 8 : 0);  // the most
+  const size_t lds_now = lds_bytes - (CONV ? (kMaxConvPieces - (K >> 4)) * 8 : 0);
+  auto kern = qgemm_tile_kernel<BM, BN, WAVES_M, WAVES_N, OUT_T, ACT, KALIGNED, CONV, ELEMENTWISE>;
   static bool attr_set = false;  // benign race: the call is idempotent
   if (!attr_set) {
     hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -360,24 +474,24 @@ int launch_tile(const uint8_t* a, uint32_t amask, const uint8_t* bp, int M, int 
     if (err != hipSuccess) return hip_fail(err, "hipFuncSetAttribute(qgemm_tile_kernel)");
     attr_set = true;
   }
-  kern<<<dim3(static_cast<unsigned>(num_m * num_n)), dim3(64 * WAVES_M * WAVES_N), lds_bytes, st>>>(
-      a, amask, bp, M, K, N, KT, NT, num_m, num_n, e, out);
+  kern<<<dim3(static_cast<unsigned>(num_m * num_n)), dim3(64 * WAVES_M * WAVES_N), lds_now, st>>>(
+      a, amask, bp, M, K, N, KT, NT, num_m, num_n, e, out, cv);
   return ITEXHIP_OK;
 }
 
 // Tile shape: the one with the smallest estimated time = rounds of workgroups over the 256 CUs x
 // tile area x a penalty for the operand traffic per MFMA of smaller tiles.
-inline int pick_tile_shape(int M, int N, bool wide_only) {
+inline int pick_tile_shape(int M, int N, bool wide_only, int first = 0) {
   struct Shape { int bm, bn; double penalty; };
   static const Shape shapes[5] = {{256, 256, 1.0}, {256, 192, 1.03}, {256, 128, 1.08}, {128, 128, 1.2}, {64, 64, 1.8}};
   // ITEXHIP_TILE_SHAPE=0..4 forces a shape (tests exercise every shape on ragged problems with it)
   if (const char* forced = std::getenv("ITEXHIP_TILE_SHAPE")) {
     const int f = std::atoi(forced);
-    if (f >= (wide_only ? 3 : 0) && f < 5) return f;
+    if (f >= (wide_only ? 3 : first) && f < 5) return f;
   }
   int best = 3;
   double best_cost = 1e300;
-  for (int i = wide_only ? 3 : 0; i < 5; ++i) {
+  for (int i = wide_only ? 3 : first; i < 5; ++i) {
     const double tiles = static_cast<double>((M + shapes[i].bm - 1) / shapes[i].bm) * ((N + shapes[i].bn - 1) / shapes[i].bn);
     const double rounds = std::ceil(tiles / 256.0);
     const double cost = rounds * shapes[i].bm * shapes[i].bn * shapes[i].penalty;
@@ -398,22 +512,72 @@ int dispatch_tile_shape(const uint8_t* a, uint32_t amask, const uint8_t* bp, int
   }
 }
 
-// The generic eltwise chain, K not a multiple of 64, a missing bias and unaligned outputs are rare:
-// they share the conservative instantiation (run-time eltwise chain, per-lane clamped activation
-// loads, element-wise stores when needed), in two tile shapes only, to keep the number of kernels down.
+// A bias vector, 16-byte aligned output rows and a post-op chain of the canonical form take the vector epilogue:
+// with K a multiple of 64 the specialised kernels (uniform activation addresses) in every tile shape (GELU: its
+// epilogue is long, so without the two largest shapes); other K: per-lane clamped activation loads, two tile shapes.
+// A missing bias, an addend, other chains or unaligned outputs (rare) go to the element-wise epilogue, a kernel of
+// its own in two shapes.
 template <int OUT_T>
 int dispatch_tile(const uint8_t* a, uint32_t a_xor, const uint8_t* bp, int M, int K, int N,
-                  const EpilogueArgs& e, void* out, hipStream_t st) {
+                  const EpilogueArgs& e_in, void* out, hipStream_t st) {
   constexpr int esz = (OUT_T == ITEXHIP_QINT8 || OUT_T == ITEXHIP_QUINT8) ? 1 : is_float16_type(OUT_T) ? 2 : 4;
-  // the specialised kernels only carry the vectorised epilogue: bias present, output rows 16-byte aligned
-  const bool plain = e.addend == nullptr && (e.bias != nullptr || e.fused) && (reinterpret_cast<uintptr_t>(out) & 15) == 0 &&
-                     ((static_cast<int64_t>(N) * esz) & 15) == 0 && (K & 63) == 0;
-  const int act = e.n_eltwise == 0 ? 0
-                  : (e.n_eltwise == 1 && e.elt[0].alg == ITEXHIP_ELT_RELU && e.elt[0].alpha == 0.0f) ? 1 : 2;
-  if (plain && act == 0) return dispatch_tile_shape<OUT_T, 0>(a, a_xor, bp, M, K, N, e, out, st);
-  if (plain && act == 1) return dispatch_tile_shape<OUT_T, 1>(a, a_xor, bp, M, K, N, e, out, st);
-  if (pick_tile_shape(M, N, true) == 3) return launch_tile<128, 128, 2, 2, OUT_T, 2, false>(a, a_xor, bp, M, K, N, e, out, st);
-  return launch_tile<64, 64, 2, 2, OUT_T, 2, false>(a, a_xor, bp, M, K, N, e, out, st);
+  EpilogueArgs e = e_in;
+  const int act = canon_chain(e, &e.canon);
+  const bool vec_epilogue = act >= 0 && e.addend == nullptr && (e.bias != nullptr || e.fused) &&
+                            (reinterpret_cast<uintptr_t>(out) & 15) == 0 && ((static_cast<int64_t>(N) * esz) & 15) == 0;
+  const bool wide = pick_tile_shape(M, N, true) == 3;
+  if (vec_epilogue && (K & 63) == 0) {
+    if (act == 0) return dispatch_tile_shape<OUT_T, 0>(a, a_xor, bp, M, K, N, e, out, st);
+    if (act == 1) return dispatch_tile_shape<OUT_T, 1>(a, a_xor, bp, M, K, N, e, out, st);
+    if (act == 2) return dispatch_tile_shape<OUT_T, 2>(a, a_xor, bp, M, K, N, e, out, st);
+    switch (pick_tile_shape(M, N, false, 2)) {
+      case 2: return launch_tile<256, 128, 2, 2, OUT_T, 3, true>(a, a_xor, bp, M, K, N, e, out, st);
+      case 3: return launch_tile<128, 128, 2, 2, OUT_T, 3, true>(a, a_xor, bp, M, K, N, e, out, st);
+      default: return launch_tile<64, 64, 2, 2, OUT_T, 3, true>(a, a_xor, bp, M, K, N, e, out, st);
+    }
+  }
+  if (vec_epilogue && act == 3) {
+    if (wide) return launch_tile<128, 128, 2, 2, OUT_T, 3, false>(a, a_xor, bp, M, K, N, e, out, st);
+    return launch_tile<64, 64, 2, 2, OUT_T, 3, false>(a, a_xor, bp, M, K, N, e, out, st);
+  }
+  if (vec_epilogue) {  // the canonical chain covers "none" and "ReLU" too
+    if (wide) return launch_tile<128, 128, 2, 2, OUT_T, 2, false>(a, a_xor, bp, M, K, N, e, out, st);
+    return launch_tile<64, 64, 2, 2, OUT_T, 2, false>(a, a_xor, bp, M, K, N, e, out, st);
+  }
+  if (wide) return launch_tile<128, 128, 2, 2, OUT_T, 2, false, false, true>(a, a_xor, bp, M, K, N, e, out, st);
+  return launch_tile<64, 64, 2, 2, OUT_T, 2, false, false, true>(a, a_xor, bp, M, K, N, e, out, st);
+}
+
+// Implicit GEMM of a Conv2D: `x` is the NHWC input, M = batch * out_h * out_w, K = k_h * k_w * in_c.  Run-time post-op
+// chain in canonical form, vector epilogue (the host checks that the output allows it), three tile shapes (a
+// 256 x 64 shape with four wavefronts stacked along M was slower than 64 x 64 tiles for 64 output channels).
+template <int OUT_T>
+int dispatch_tile_conv(const uint8_t* x, uint32_t a_xor, const uint8_t* bp, int M, int K, int N, const EpilogueArgs& e_in,
+                       void* out, hipStream_t st, const ConvTileArgs& cv) {
+  EpilogueArgs e = e_in;
+  const int act = canon_chain(e, &e.canon);
+  if (act < 0 || act == 3) {
+    set_error("itexhip_qconv2d: the post-ops must be one of ReLU / LeakyReLU / clip, optionally followed by a linear map");
+    return ITEXHIP_INVALID_ARGUMENT;
+  }
+  struct Shape { int bm, bn; double penalty; };
+  static const Shape shapes[3] = {{256, 128, 1.08}, {128, 128, 1.2}, {64, 64, 1.8}};
+  int best = 0;
+  double best_cost = 1e300;
+  for (int i = 0; i < 3; ++i) {
+    const double tiles = static_cast<double>((M + shapes[i].bm - 1) / shapes[i].bm) * ((N + shapes[i].bn - 1) / shapes[i].bn);
+    const double cost = std::ceil(tiles / 256.0) * shapes[i].bm * shapes[i].bn * shapes[i].penalty;
+    if (cost < best_cost) { best_cost = cost; best = i; }
+  }
+  if (const char* forced = std::getenv("ITEXHIP_CONV_TILE_SHAPE")) {  // tests exercise every shape with it
+    const int f = std::atoi(forced);
+    if (f >= 0 && f < 3) best = f;
+  }
+  switch (best) {
+    case 0: return launch_tile<256, 128, 2, 2, OUT_T, 2, false, true>(x, a_xor, bp, M, K, N, e, out, st, cv);
+    case 1: return launch_tile<128, 128, 2, 2, OUT_T, 2, false, true>(x, a_xor, bp, M, K, N, e, out, st, cv);
+    default: return launch_tile<64, 64, 2, 2, OUT_T, 2, false, true>(x, a_xor, bp, M, K, N, e, out, st, cv);
+  }
 }
 
 }  // namespace itexhip

@@ -4,4 +4,6 @@
 namespace itexhip {
 template int dispatch_tile<ITEXHIP_QINT32>(const uint8_t*, uint32_t, const uint8_t*, int, int, int, const EpilogueArgs&, void*,
                                hipStream_t);
+template int dispatch_tile_conv<ITEXHIP_QINT32>(const uint8_t*, uint32_t, const uint8_t*, int, int, int, const EpilogueArgs&, void*,
+                                    hipStream_t, const ConvTileArgs&);
 }  // namespace itexhip

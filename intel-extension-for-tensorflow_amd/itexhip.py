@@ -30,6 +30,7 @@ EXPORTS = [
     "itexhip_qmatmul_epilogue_desc", "itexhip_qmatmul_prepare", "itexhip_qgemm_packed_bytes",
     "itexhip_qgemm_prepack_b", "itexhip_qgemm", "itexhip_qgemm_tile", "itexhip_qgemv", "itexhip_qmatmul", "itexhip_qmatmul_per_row", "itexhip_qmatmul_unpacked", "itexhip_mfma_probe",
     "itexhip_qgemm_naive", "itexhip_qbatch_matmul", "itexhip_transpose", "itexhip_im2col8", "itexhip_scale_vector",
+    "itexhip_qconv2d_implicit_ok", "itexhip_qconv2d",
 ]
 
 
@@ -328,6 +329,15 @@ class ConvGeometry(C.Structure):
 
 def im2col8(x, geometry, row_bytes, cols, stream=0):
     _check(_lib.itexhip_im2col8(_ptr(x), C.byref(geometry), _i64(row_bytes), _ptr(cols), _ptr(stream)))
+
+
+def qconv2d_implicit_ok(geometry, x, out_channels, out_type, out):
+    return bool(_lib.itexhip_qconv2d_implicit_ok(C.byref(geometry), _ptr(x), _i64(out_channels), int(out_type), _ptr(out)))
+
+
+def qconv2d(x, x_type, geometry, packed_filter, colsum, out_channels, scales, bias, ep, out_type, out, stream=0):
+    _check(_lib.itexhip_qconv2d(_ptr(x), int(x_type), C.byref(geometry), _ptr(packed_filter), _ptr(colsum), _i64(out_channels),
+                                _ptr(scales), _ptr(bias), C.byref(ep), int(out_type), _ptr(out), _ptr(stream)))
 
 
 def scale_vector(bias, bias_type, factors, n_factors, n, out, stream=0):

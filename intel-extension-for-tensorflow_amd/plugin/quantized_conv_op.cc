@@ -249,7 +249,9 @@ class QuantizedConv2DOp : public OpKernel {
       Tensor cols;
       const bool pointwise = KH == 1 && KW == 1 && stride_h_ == 1 && stride_w_ == 1 && g.pad_top == 0 && g.pad_left == 0 &&
                              g.out_h == H && g.out_w == W && K == Kp;
-      if (!pointwise) {
+      // windows the tile kernel can gather by itself (input channels a multiple of 16, ...) need no patch matrix
+      const bool implicit = !pointwise && itexhip_qconv2d_implicit_ok(&g, x.data(), O, t_out_, out.data()) != 0;
+      if (!pointwise && !implicit) {
         cols = ctx->allocate_temp(t_in_, {M, Kp});
         if (!ctx->ok()) return;
         const int st = itexhip_im2col8(x.data(), &g, Kp, cols.data(), stream);
@@ -264,8 +266,10 @@ class QuantizedConv2DOp : public OpKernel {
         ep.elt[0].alpha = leaky_ ? alpha_ : 0.0f;
         ep.elt[0].beta = 0.0f;
       }
-      const int st = itexhip_qgemm(a, t_in_, packed_.flat<int8_t>(), colsum_.flat<int32_t>(), M, Kp, O, params, bias_dev, &ep,
-                                   t_out_, out.data(), stream);
+      const int st = implicit ? itexhip_qconv2d(x.data(), t_in_, &g, packed_.flat<int8_t>(), colsum_.flat<int32_t>(), O, params,
+                                                bias_dev, &ep, t_out_, out.data(), stream)
+                              : itexhip_qgemm(a, t_in_, packed_.flat<int8_t>(), colsum_.flat<int32_t>(), M, Kp, O, params,
+                                              bias_dev, &ep, t_out_, out.data(), stream);
       ITEX_REQUIRES(ctx, st == ITEXHIP_OK, st == ITEXHIP_INVALID_ARGUMENT ? TF_INVALID_ARGUMENT : TF_ABORTED,
                     std::string("Operation received an exception: ") + itexhip_last_error());
     }

@@ -68,6 +68,93 @@ def test_scale_vector(hip, dev):
             np.testing.assert_array_equal(out.cpu().numpy(), bias.astype(np.float32) * f[0])
 
 
+IMPLICIT_CASES = [  # input NHWC, filter HWIO, strides, dilations, leading pads (top, left) or None for SAME
+    ((2, 9, 10, 16), (3, 3, 16, 48), (1, 1), (1, 1), None),      # K = 144: a ragged last K step
+    ((1, 8, 7, 32), (3, 2, 32, 64), (2, 1), (1, 2), None),       # strides + dilation
+    ((2, 6, 6, 48), (2, 2, 48, 112), (1, 1), (1, 1), None),      # 48 channels: pieces of one K step span two pixels
+    ((1, 20, 20, 64), (3, 3, 64, 64), (1, 1), (1, 1), None),     # ResNet-like block
+    ((3, 13, 11, 16), (5, 5, 16, 80), (2, 2), (1, 1), (3, 1)),   # explicit asymmetric padding, 400-byte patch rows
+    ((1, 12, 12, 128), (1, 1, 128, 160), (2, 2), (1, 1), None),  # strided pointwise, 128x128 tiles
+    ((1, 3, 3, 16), (3, 3, 16, 16), (1, 1), (1, 1), None),        # fewer output positions than one tile has rows
+]
+
+
+@pytest.mark.parametrize("shape,wshape,strides,dil,lead", IMPLICIT_CASES)
+@pytest.mark.parametrize("signed_in,tile_shape", [(False, None), (True, None), (False, 0), (True, 1), (False, 2)])
+def test_implicit_gemm_conv(hip, dev, monkeypatch, shape, wshape, strides, dil, lead, signed_in, tile_shape):
+    """itexhip_qconv2d (activation tiles gathered from the NHWC input) against a numpy convolution for the int32
+    accumulators, and bit for bit against the patch-matrix path (itexhip_im2col8 + itexhip_qgemm) for every output
+    type with per-channel scales, bias and ReLU."""
+    import torch
+    from tests.test_oracle_conv import ref_int_conv
+    if tile_shape is not None:   # every tile shape of the kernel on every case, ragged edges included
+        monkeypatch.setenv("ITEXHIP_CONV_TILE_SHAPE", str(tile_shape))
+    rng = np.random.default_rng(sum(shape) + sum(wshape) + signed_in)
+    B, H, W, Cin = shape
+    kh, kw, _, O = wshape
+    x = rng.integers(-128, 128, shape).astype(np.int8) if signed_in else rng.integers(0, 256, shape).astype(np.uint8)
+    w = rng.integers(-127, 128, wshape).astype(np.int8)
+    if lead is None:
+        oh, pt = same_lead(H, kh, strides[0], dil[0])
+        ow, pl = same_lead(W, kw, strides[1], dil[1])
+    else:
+        pt, pl = lead
+        oh = (H + 2 * pt - ((kh - 1) * dil[0] + 1)) // strides[0] + 1
+        ow = (W + 2 * pl - ((kw - 1) * dil[1] + 1)) // strides[1] + 1
+    # trailing pads: whatever the output extent needs
+    pb = max((oh - 1) * strides[0] + (kh - 1) * dil[0] + 1 - H - pt, 0)
+    pr = max((ow - 1) * strides[1] + (kw - 1) * dil[1] + 1 - W - pl, 0)
+    ref = ref_int_conv(x, w, strides, dil, ((pt, pb), (pl, pr)))[:, :oh, :ow, :]
+    K, M = kh * kw * Cin, B * oh * ow
+    g = hip.ConvGeometry(B, H, W, Cin, kh, kw, oh, ow, strides[0], strides[1], dil[0], dil[1], pt, pl)
+    T_in = hip.QINT8 if signed_in else hip.QUINT8
+    xd = torch.from_numpy(x).to(dev)
+    acc = torch.full((M, O), 77, dtype=torch.int32, device=dev)
+    assert hip.qconv2d_implicit_ok(g, xd, O, hip.QINT32, acc)
+    packed = torch.empty(hip.qgemm_packed_bytes(K, O), dtype=torch.int8, device=dev)
+    colsum = torch.empty(O, dtype=torch.int32, device=dev)
+    hip.qgemm_prepack_b(torch.from_numpy(w.reshape(K, O)).to(dev), False, K, O, packed, colsum)
+    one = torch.ones(1, dtype=torch.float32, device=dev)
+    zero_bias = torch.zeros(O, dtype=torch.float32, device=dev)
+    ep = hip.Epilogue()
+    ep.n_scales, ep.n_eltwise = 1, 0
+    hip.qconv2d(xd, T_in, g, packed, colsum, O, one, zero_bias, ep, hip.QINT32, acc)
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(acc.cpu().numpy().reshape(B, oh, ow, O), ref)
+
+    cols = torch.empty((M, K), dtype=torch.uint8, device=dev)
+    hip.im2col8(xd, g, K, cols)
+    scales = torch.from_numpy((rng.random(O).astype(np.float32) + 0.5) * np.float32(2e-4)).to(dev)
+    bias = torch.from_numpy(rng.standard_normal(O).astype(np.float32)).to(dev)
+    ep.n_scales, ep.n_eltwise = O, 1
+    ep.elt[0].alg, ep.elt[0].alpha, ep.elt[0].beta = hip.ELT_RELU, 0.0, 0.0
+    for T, dt in ((hip.QINT8, torch.int8), (hip.QUINT8, torch.uint8), (hip.FLOAT, torch.float32), (hip.BFLOAT16, torch.bfloat16),
+                  (hip.QINT32, torch.int32)):
+        a = torch.zeros((M, O), dtype=dt, device=dev)
+        b_ = torch.zeros((M, O), dtype=dt, device=dev)
+        hip.qconv2d(xd, T_in, g, packed, colsum, O, scales, bias, ep, T, a)
+        hip.qgemm(cols, T_in, packed, colsum, M, K, O, scales, bias, ep, T, b_)
+        torch.cuda.synchronize()
+        assert torch.equal(a.view(torch.uint8), b_.view(torch.uint8)), T
+
+
+def test_implicit_gemm_conv_rejects_other_shapes(hip, dev):
+    import torch
+    x = torch.zeros(4 * 4 * 24 + 16, dtype=torch.uint8, device=dev)
+    y = torch.zeros(16 * 16 * 4 + 16, dtype=torch.uint8, device=dev)
+    ok = lambda g, xp=x, O=16, T=hip.QINT32, out=y: hip.qconv2d_implicit_ok(g, xp, O, T, out)
+    assert not ok(hip.ConvGeometry(1, 4, 4, 24, 3, 3, 4, 4, 1, 1, 1, 1, 1, 1))   # 24 channels
+    g16 = hip.ConvGeometry(1, 4, 4, 16, 3, 3, 4, 4, 1, 1, 1, 1, 1, 1)
+    assert ok(g16) and not ok(g16, xp=x.data_ptr() + 4)                         # misaligned input
+    assert not ok(hip.ConvGeometry(1, 40, 40, 1024, 5, 5, 40, 40, 1, 1, 1, 1, 2, 2))  # 25 KiB window
+    assert not ok(g16, O=24, T=hip.QINT8) and ok(g16, O=32, T=hip.QINT8)        # output rows of 24 bytes
+    assert not ok(g16, out=y.data_ptr() + 4) and not ok(g16, T=hip.HALF)
+    ep = hip.Epilogue()
+    with pytest.raises(hip.ItexHipError) as e:
+        hip.qconv2d(x.data_ptr() + 4, hip.QUINT8, g16, x, x, 16, x, x, ep, hip.QINT32, y)
+    assert e.value.code == hip.INVALID_ARGUMENT
+
+
 @pytest.fixture(scope="module")
 def rt(dev):
     import torch

@@ -235,6 +235,45 @@ def test_every_tile_shape_on_ragged_problems(hip, dev, monkeypatch, shape, M, K,
     np.testing.assert_array_equal(got, ref)
 
 
+CHAINS = {   # post-op chains of the form [activation] [linear map] that the vector epilogue resolves on the host
+    "leaky_f32": dict(V2_DEQ, activation=orc.ACT_LEAKYRELU, leakyrelu_alpha=0.2),
+    "relu6_f32": dict(V2_DEQ, activation=orc.ACT_RELU6),
+    "leaky_req_s8": dict(V2_REQ_S8, activation=orc.ACT_LEAKYRELU, leakyrelu_alpha=0.1),
+    "relu6_req_u8": dict(V2_REQ_U8_RELU, activation=orc.ACT_RELU6),
+    "relu_req_minfirst_u8": dict(V2_REQ_U8_RELU, out_min_first=True),       # ReLU, then the linear map of a MIN_FIRST output
+    "leaky_req_minfirst_s8": dict(V2_REQ_S8, activation=orc.ACT_LEAKYRELU, leakyrelu_alpha=0.3, out_min_first=True),
+    "req_minfirst_s8": dict(V2_REQ_S8, out_min_first=True),                 # the linear map alone
+    "gelu_tanh_f32": dict(V2_DEQ, activation=orc.ACT_GELU_APPROX),
+    "gelu_erf_bf16": dict(V2_DEQ, activation=orc.ACT_GELU_EXACT, t_out=orc.BFLOAT16),
+}
+
+
+@pytest.mark.parametrize("shape", [0, 1, 2, 3, 4])
+@pytest.mark.parametrize("chain", sorted(CHAINS))
+def test_canonical_chains_every_tile_shape(hip, dev, monkeypatch, shape, chain):
+    """Every tile shape with every kind of run-time post-op chain, K a multiple of 64 (uniform activation addresses)
+    and not (per-lane clamped addresses), ragged M and N: bit-equal to the oracle except for the GELU chains, where
+    the device's tanhf / erff need not round like the host's (2e-6 relative, 1e-6 absolute; one unit of the
+    output type where that is coarser)."""
+    monkeypatch.setenv("ITEXHIP_TILE_SHAPE", str(shape))
+    kw = CHAINS[chain]
+    for M, K, N in [(300, 448, 528), (257, 208, 400)]:
+        layer, w, bias = make_layer(hip, dev, K, N, seed=K + N + shape)
+        x, xq, mn, mx = make_acts(M, K, seed=M + 1)
+        r_out = float(np.abs(x @ w + bias).max())
+        lo = 0.0 if kw["t_out"] == orc.QUINT8 else -r_out
+        ref = layer.oracle(xq, kw, mn, mx, lo, r_out)
+        for path in ("tile", "fused"):
+            got = layer.run(xq, kw, mn, mx, lo, r_out, path=path)
+            if "gelu" not in chain:
+                np.testing.assert_array_equal(got, ref)
+            elif kw["t_out"] == orc.FLOAT:
+                np.testing.assert_allclose(got, ref, rtol=2e-6, atol=1e-6)
+            else:   # bfloat16 bit patterns: equal, or neighbours where the fp32 values straddle a rounding boundary
+                d = np.abs(bits16(got).astype(np.int64) - bits16(ref).astype(np.int64))
+                assert d.max() <= 1 and (d > 0).mean() < 1e-3
+
+
 @pytest.mark.parametrize("M", [1, 2, 4, 7, 16])
 @pytest.mark.parametrize("K,N", [(64, 16), (256, 100), (4096, 512), (1024, 4096), (8192, 48), (64, 8200), (512, 16384)])
 @pytest.mark.parametrize("kw", [V2_DEQ, V2_REQ_S8])
