@@ -141,7 +141,8 @@ def make_acts(torch, hip, M, K, seed, dev, outlier_frac=0.0, outlier_mult=1.0):
 # workloads
 # ------------------------------------------------------------------------------------------------
 def bench_linear(torch, hip, timer, M, K, N, kind, steps, warmup, dev, seed, rotate=1, graph=False, per_row=False):
-    """kind: 'requant_s8' ([BiasAdd, Requantize] -> qint8), 'deq' / 'deq_relu' ([.., Dequantize] -> fp32).
+    """kind: 'requant_s8' ([BiasAdd, Requantize] -> qint8), 'deq' / 'deq_relu' / 'deq_gelu' ([.., Dequantize] -> fp32;
+    GeluApproximate is what BERT's first feed-forward linear fuses).
     rotate > 1 cycles through that many distinct weight copies so that the weight stream comes from
     HBM, not from the 256 MiB last-level cache."""
     layers = [make_weights(torch, hip, K, N, seed + i, dev) for i in range(rotate)]
@@ -157,7 +158,7 @@ def bench_linear(torch, hip, timer, M, K, N, kind, steps, warmup, dev, seed, rot
         t_out, out_dtype = hip.FLOAT, torch.float32
         p = hip.matmul_params(api=hip.API_V2, t_in=hip.QUINT8, t_out=t_out, input_mode=hip.MIN_FIRST,
                               has_dequantize=True,
-                              activation=hip.ACT_RELU if kind == "deq_relu" else hip.ACT_NONE,
+                              activation={"deq_relu": hip.ACT_RELU, "deq_gelu": hip.ACT_GELU_APPROX}.get(kind, hip.ACT_NONE),
                               min_a=min_a, max_a=max_a)
         out_bytes = 4
     del x
@@ -465,7 +466,7 @@ def main():
             others.append(r)
     if "bert" in only:
         for (k, n, kind, seed) in ((768, 2304, "deq", 1), (768, 768, "deq", 2), (768, 3072, "deq_relu", 3),
-                                   (3072, 768, "deq", 4)):
+                                   (768, 3072, "deq_gelu", 3), (3072, 768, "deq", 4)):
             r = bench_linear(torch, hip, timer, 4096, k, n, kind, K_steps, W, dev, seed, graph=True)
             r.pop("_ctx")
             t_roof = max(r["ops"] / (PEAK_INT8_TOPS * 1e12), r["bytes"] / (PEAK_HBM_GBS * 1e9))
