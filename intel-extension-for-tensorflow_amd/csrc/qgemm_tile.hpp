@@ -513,8 +513,8 @@ int dispatch_tile_shape(const uint8_t* a, uint32_t amask, const uint8_t* bp, int
 }
 
 // A bias vector, 16-byte aligned output rows and a post-op chain of the canonical form take the vector epilogue:
-// with K a multiple of 64 the specialised kernels (uniform activation addresses) in every tile shape (GELU: its
-// epilogue is long, so without the two largest shapes); other K: per-lane clamped activation loads, two tile shapes.
+// with K a multiple of 64 the specialised kernels (uniform activation addresses) in every tile shape; other K:
+// per-lane clamped activation loads, two tile shapes.
 // A missing bias, an addend, other chains or unaligned outputs (rare) go to the element-wise epilogue, a kernel of
 // its own in two shapes.
 template <int OUT_T>
@@ -530,11 +530,7 @@ int dispatch_tile(const uint8_t* a, uint32_t a_xor, const uint8_t* bp, int M, in
     if (act == 0) return dispatch_tile_shape<OUT_T, 0>(a, a_xor, bp, M, K, N, e, out, st);
     if (act == 1) return dispatch_tile_shape<OUT_T, 1>(a, a_xor, bp, M, K, N, e, out, st);
     if (act == 2) return dispatch_tile_shape<OUT_T, 2>(a, a_xor, bp, M, K, N, e, out, st);
-    switch (pick_tile_shape(M, N, false, 2)) {
-      case 2: return launch_tile<256, 128, 2, 2, OUT_T, 3, true>(a, a_xor, bp, M, K, N, e, out, st);
-      case 3: return launch_tile<128, 128, 2, 2, OUT_T, 3, true>(a, a_xor, bp, M, K, N, e, out, st);
-      default: return launch_tile<64, 64, 2, 2, OUT_T, 3, true>(a, a_xor, bp, M, K, N, e, out, st);
-    }
+    return dispatch_tile_shape<OUT_T, 3>(a, a_xor, bp, M, K, N, e, out, st);
   }
   if (vec_epilogue && act == 3) {
     if (wide) return launch_tile<128, 128, 2, 2, OUT_T, 3, false>(a, a_xor, bp, M, K, N, e, out, st);
