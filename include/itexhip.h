@@ -252,6 +252,17 @@ int itexhip_qgemv(const void* a, int a_type, const int8_t* packed_b, const int32
                   int64_t M, int64_t K, int64_t N, const float* scales, const float* bias,
                   const itexhip_epilogue* ep, int out_type, void* out, void* stream);
 
+/* itexhip_qgemm with one ITEXHIP_ELT_SUM in ep->elt: y = y + elt.alpha * addend[m, n] at that place of the chain.
+ * `addend` is an [M, N] tensor of addend_type ITEXHIP_FLOAT, ITEXHIP_QINT8 or ITEXHIP_QUINT8 (the 8-bit values are
+ * converted to fp32 exactly): the sum post-op of oneDNN that the reference uses for the "Add" fusion of the MatMul
+ * (quantized_matmul_common.h:352-389) and the "Sum" fusions of the convolution (quantized_conv_ops.h:398-433,
+ * 604-640, where the summand buffer doubles as the output).  `out` may be the addend buffer itself when both have
+ * the same element size (every element is read before it is written); any other overlap is not allowed. */
+int itexhip_qgemm_sum(const void* a, int a_type, const int8_t* packed_b, const int32_t* colsum,
+                      int64_t M, int64_t K, int64_t N, const float* scales, const float* bias,
+                      const itexhip_epilogue* ep, const void* addend, int addend_type, int out_type, void* out,
+                      void* stream);
+
 /* The whole op in one launch: as itexhip_qmatmul_prepare followed by itexhip_qgemm, but the MatMul
  * kernel derives each channel's output scale and bias itself from the op's ranges (the same fp32
  * operation sequence), so no parameter vectors and no second kernel are needed.  This is what the
@@ -372,6 +383,13 @@ int itexhip_qconv2d_implicit_ok(const itexhip_conv_geometry* g, const void* x, i
 int itexhip_qconv2d(const void* x, int x_type, const itexhip_conv_geometry* g, const int8_t* packed_filter,
                     const int32_t* colsum, int64_t out_channels, const float* scales, const float* bias,
                     const itexhip_epilogue* ep, int out_type, void* out, void* stream);
+/* itexhip_qconv2d with one ITEXHIP_ELT_SUM in ep->elt, as itexhip_qgemm_sum: `addend` is the summand in the output's
+ * layout [batch, out_h, out_w, out_channels], 4-byte (8-bit types) or 16-byte (float) aligned, out_channels a
+ * multiple of 4. */
+int itexhip_qconv2d_sum(const void* x, int x_type, const itexhip_conv_geometry* g, const int8_t* packed_filter,
+                        const int32_t* colsum, int64_t out_channels, const float* scales, const float* bias,
+                        const itexhip_epilogue* ep, const void* addend, int addend_type, int out_type, void* out,
+                        void* stream);
 
 /* Diagnostic, no counterpart in the reference: `workgroups` x 4 wavefronts each issue iters x 8
  * independent 32x32x32 i8 MFMAs (2 * 32768 ops each) on the 8 KiB of operand fragments at `operands`

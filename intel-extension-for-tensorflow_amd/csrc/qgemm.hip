@@ -300,7 +300,7 @@ __global__ __launch_bounds__(256) void qmatmul_unpacked_kernel(const uint8_t* __
   if (e.n_scales > 0) v = v * c.scale;
   v = v + c.bias;
   for (int k = 0; k < e.n_eltwise; ++k) {
-    if (e.elt[k].alg == ITEXHIP_ELT_SUM) v = v + e.elt[k].alpha * e.addend[idx];
+    if (e.elt[k].alg == ITEXHIP_ELT_SUM) v = v + e.elt[k].alpha * load_addend(e, idx);
     else v = apply_eltwise(e.elt[k], v);
   }
   store_output<OUT_T>(out, idx, v);
@@ -311,7 +311,7 @@ __global__ __launch_bounds__(256) void qmatmul_unpacked_kernel(const uint8_t* __
 // ------------------------------------------------------------------------------------------------
 int check_common(const void* a, int a_type, const void* b, int64_t M, int64_t K, int64_t N,
                  const float* scales, const itexhip_epilogue* ep, int out_type, const void* out,
-                 const char* who) {
+                 const char* who, const void* addend = nullptr, int addend_type = 0) {
   ITEXHIP_REQUIRE(a_type == ITEXHIP_QUINT8 || a_type == ITEXHIP_QINT8, "%s: activation type must be quint8 or qint8", who);
   ITEXHIP_REQUIRE(out_type == ITEXHIP_QINT32 || out_type == ITEXHIP_QINT8 || out_type == ITEXHIP_QUINT8 ||
                       is_float_out(out_type), "%s: unsupported output type %d", who, out_type);
@@ -320,8 +320,12 @@ int check_common(const void* a, int a_type, const void* b, int64_t M, int64_t K,
                   static_cast<long long>(kMaxK));
   ITEXHIP_REQUIRE(ep != nullptr, "%s: null epilogue", who);
   ITEXHIP_REQUIRE(ep->n_eltwise >= 0 && ep->n_eltwise <= 3, "%s: bad eltwise count", who);
-  for (int k = 0; k < ep->n_eltwise; ++k)
-    ITEXHIP_REQUIRE(ep->elt[k].alg != ITEXHIP_ELT_SUM, "%s: the Add fusion needs itexhip_qmatmul (it takes the addend)", who);
+  int n_sum = 0;
+  for (int k = 0; k < ep->n_eltwise; ++k) n_sum += ep->elt[k].alg == ITEXHIP_ELT_SUM;
+  ITEXHIP_REQUIRE(n_sum == (addend != nullptr ? 1 : 0),
+                  "%s: one sum post-op goes with an addend (itexhip_qgemm_sum / itexhip_qconv2d_sum / itexhip_qmatmul), none without", who);
+  ITEXHIP_REQUIRE(addend == nullptr || addend_type == ITEXHIP_FLOAT || addend_type == ITEXHIP_QINT8 || addend_type == ITEXHIP_QUINT8,
+                  "%s: the addend must be float, qint8 or quint8", who);
   ITEXHIP_REQUIRE(ep->n_scales == 0 || ep->n_scales == 1 || ep->n_scales == N,
                   "%s: %d scales for %lld channels", who, ep->n_scales, static_cast<long long>(N));
   if (M == 0 || N == 0) return ITEXHIP_OK;
@@ -332,8 +336,10 @@ int check_common(const void* a, int a_type, const void* b, int64_t M, int64_t K,
 }
 
 EpilogueArgs make_args(int a_type, const int32_t* colsum, const float* scales, const void* bias,
-                       const itexhip_epilogue* ep) {
+                       const itexhip_epilogue* ep, const void* addend = nullptr, int addend_type = 0) {
   EpilogueArgs e{};
+  e.addend = addend;
+  e.addend_type = addend_type;
   e.scales = scales;
   e.bias = bias;
   e.colsum = colsum;
@@ -409,11 +415,12 @@ int launch_packed(bool gemv, const void* a, int a_type, const int8_t* packed_b, 
 
 int packed_path(bool gemv, const void* a, int a_type, const int8_t* packed_b, const int32_t* colsum,
                 int64_t M, int64_t K, int64_t N, const float* scales, const float* bias,
-                const itexhip_epilogue* ep, int out_type, void* out, void* stream, const char* who) {
-  if (int st = check_common(a, a_type, packed_b, M, K, N, scales, ep, out_type, out, who)) return st;
+                const itexhip_epilogue* ep, int out_type, void* out, void* stream, const char* who,
+                const void* addend = nullptr, int addend_type = 0) {
+  if (int st = check_common(a, a_type, packed_b, M, K, N, scales, ep, out_type, out, who, addend, addend_type)) return st;
   if (M == 0 || N == 0) return ITEXHIP_OK;
-  return launch_packed(gemv, a, a_type, packed_b, M, K, N, make_args(a_type, colsum, scales, bias, ep), out_type, out,
-                       stream, who);
+  return launch_packed(gemv, a, a_type, packed_b, M, K, N, make_args(a_type, colsum, scales, bias, ep, addend, addend_type),
+                       out_type, out, stream, who);
 }
 
 }  // namespace
@@ -466,6 +473,15 @@ extern "C" int itexhip_qgemm(const void* a, int a_type, const int8_t* packed_b, 
                      "itexhip_qgemm");
 }
 
+extern "C" int itexhip_qgemm_sum(const void* a, int a_type, const int8_t* packed_b, const int32_t* colsum,
+                                 int64_t M, int64_t K, int64_t N, const float* scales, const float* bias,
+                                 const itexhip_epilogue* ep, const void* addend, int addend_type, int out_type, void* out,
+                                 void* stream) {
+  ITEXHIP_REQUIRE(addend != nullptr || M == 0 || N == 0, "itexhip_qgemm_sum: null addend");
+  return packed_path(M <= 16, a, a_type, packed_b, colsum, M, K, N, scales, bias, ep, out_type, out, stream,
+                     "itexhip_qgemm_sum", addend, addend_type);
+}
+
 // ------------------------------------------------------------------------------------------------
 // Conv2D as an implicit GEMM
 // ------------------------------------------------------------------------------------------------
@@ -491,21 +507,21 @@ extern "C" int itexhip_qconv2d_implicit_ok(const itexhip_conv_geometry* g, const
   return conv_implicit_ok(g, x, out_channels, out_type, out) ? 1 : 0;
 }
 
-extern "C" int itexhip_qconv2d(const void* x, int x_type, const itexhip_conv_geometry* g, const int8_t* packed_filter,
-                               const int32_t* colsum, int64_t out_channels, const float* scales, const float* bias,
-                               const itexhip_epilogue* ep, int out_type, void* out, void* stream) {
-  const char* who = "itexhip_qconv2d";
+namespace {
+int qconv2d_impl(const char* who, const void* x, int x_type, const itexhip_conv_geometry* g, const int8_t* packed_filter,
+                 const int32_t* colsum, int64_t out_channels, const float* scales, const float* bias,
+                 const itexhip_epilogue* ep, const void* addend, int addend_type, int out_type, void* out, void* stream) {
   ITEXHIP_REQUIRE(g != nullptr, "%s: null geometry", who);
   ITEXHIP_REQUIRE(conv_implicit_ok(g, x, out_channels, out_type, out),
                   "%s: not a shape for the implicit GEMM (in_c %% 16 == 0, window <= 16 KiB, 16-byte aligned input below 2 GiB, "
                   "16-byte aligned output rows); use itexhip_im2col8 + itexhip_qgemm", who);
   ITEXHIP_REQUIRE(bias != nullptr, "%s: needs a bias vector (zeros when the op has none)", who);
   const int64_t M = g->batch * g->out_h * g->out_w, K = g->k_h * g->k_w * g->in_c, N = out_channels;
-  if (int st = check_common(x, x_type, packed_filter, M, K, N, scales, ep, out_type, out, who)) return st;
+  if (int st = check_common(x, x_type, packed_filter, M, K, N, scales, ep, out_type, out, who, addend, addend_type)) return st;
   if (N == 0) return ITEXHIP_OK;
   ITEXHIP_REQUIRE(aligned(packed_filter, 16), "%s: the packed filter must be 16-byte aligned", who);
   ITEXHIP_REQUIRE(x_type != ITEXHIP_QUINT8 || colsum, "%s: quint8 input needs colsum", who);
-  const EpilogueArgs e = make_args(x_type, colsum, scales, bias, ep);
+  const EpilogueArgs e = make_args(x_type, colsum, scales, bias, ep, addend, addend_type);
   ConvTileArgs cv;
   cv.in_h = static_cast<int>(g->in_h); cv.in_w = static_cast<int>(g->in_w); cv.in_c = static_cast<int>(g->in_c);
   cv.k_w = static_cast<int>(g->k_w); cv.out_h = static_cast<int>(g->out_h); cv.out_w = static_cast<int>(g->out_w);
@@ -527,6 +543,23 @@ extern "C" int itexhip_qconv2d(const void* x, int x_type, const itexhip_conv_geo
   if (st__ != ITEXHIP_OK) return st__;
   ITEXHIP_CHECK_LAUNCH(who);
   return ITEXHIP_OK;
+}
+}  // namespace
+
+extern "C" int itexhip_qconv2d(const void* x, int x_type, const itexhip_conv_geometry* g, const int8_t* packed_filter,
+                               const int32_t* colsum, int64_t out_channels, const float* scales, const float* bias,
+                               const itexhip_epilogue* ep, int out_type, void* out, void* stream) {
+  return qconv2d_impl("itexhip_qconv2d", x, x_type, g, packed_filter, colsum, out_channels, scales, bias, ep, nullptr, 0,
+                      out_type, out, stream);
+}
+
+extern "C" int itexhip_qconv2d_sum(const void* x, int x_type, const itexhip_conv_geometry* g, const int8_t* packed_filter,
+                                   const int32_t* colsum, int64_t out_channels, const float* scales, const float* bias,
+                                   const itexhip_epilogue* ep, const void* addend, int addend_type, int out_type, void* out,
+                                   void* stream) {
+  ITEXHIP_REQUIRE(addend != nullptr, "itexhip_qconv2d_sum: null addend");
+  return qconv2d_impl("itexhip_qconv2d_sum", x, x_type, g, packed_filter, colsum, out_channels, scales, bias, ep, addend,
+                      addend_type, out_type, out, stream);
 }
 
 extern "C" int itexhip_qgemm_naive(const void* a, int a_type, const int8_t* w, int transpose_b, int64_t M,
@@ -591,6 +624,7 @@ int qmatmul_impl(const char* who, const itexhip_matmul_params* p, const void* a,
   e.row_min_a = row_min_a;
   e.row_max_a = row_max_a;
   e.addend = addend;
+  e.addend_type = ITEXHIP_FLOAT;
   return launch_packed(M <= 16, a, p->t_in, packed_b, M, K, N, e, p->t_out, out, stream, who);
 }
 }  // namespace
@@ -646,6 +680,7 @@ extern "C" int itexhip_qmatmul_unpacked(const itexhip_matmul_params* p, const vo
   e.max_b = max_b;
   e.prep = make_prep_args(p, ep);
   e.addend = addend;
+  e.addend_type = ITEXHIP_FLOAT;
   const int a_is_u8 = p->t_in == ITEXHIP_QUINT8;
   const uint8_t* ap = reinterpret_cast<const uint8_t*>(a);
   const unsigned grid = static_cast<unsigned>((M * N + 255) / 256);

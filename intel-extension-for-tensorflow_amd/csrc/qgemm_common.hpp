@@ -20,15 +20,17 @@ constexpr int kChunkK = 32;        // k per operand chunk
 constexpr int kChunkBytes = 1024;  // 32 rows x 32 k
 constexpr int64_t kMaxK = 1 << 16; // 255 * 128 * 65536 < 2^31
 
-// A post-op chain of the form [one activation] [one linear map], either part optional (every chain the MatMul and
-// convolution ops build without an addend): resolved once on the host, so that the tile kernels apply it with a few
+// A post-op chain of the form [sum] [one activation] [sum] [one linear map], every part optional and at most one sum
+// (every chain the MatMul and convolution ops build): resolved once on the host, so that the tile kernels apply it with a few
 // wavefront-uniform branches per 32x32 tile instead of a loop over the chain per value.
-enum : int { kChainMax0 = 1, kChainLeaky = 2, kChainClip = 4, kChainLinear = 8, kChainGeluTanh = 16, kChainGeluErf = 32 };
+enum : int { kChainMax0 = 1, kChainLeaky = 2, kChainClip = 4, kChainLinear = 8, kChainGeluTanh = 16, kChainGeluErf = 32,
+             kChainSumFirst = 64, kChainSumLast = 128 };  // y += sum_scale * addend before / after the activation
 struct CanonChain {
   int flags;
   float alpha;         // leaky slope
   float lo, hi;        // clip bounds
   float lin_a, lin_b;  // y = lin_a * x + lin_b
+  float sum_scale;
 };
 
 struct EpilogueArgs {
@@ -39,7 +41,8 @@ struct EpilogueArgs {
   int comp_mul;  // 128 for u8 activations, 0 for s8
   int n_eltwise;
   itexhip_eltwise elt[3];
-  const float* addend;   // [M, N] fp32 tensor of the "Add" fusion (ITEXHIP_ELT_SUM in the chain), else null
+  const void* addend;    // [M, N] tensor of the "Add" / "Sum" fusion (ITEXHIP_ELT_SUM in the chain), else null
+  int addend_type;       // ITEXHIP_FLOAT, or ITEXHIP_QINT8 / ITEXHIP_QUINT8 (the summand of a quantized convolution)
   // fused != 0: the kernel derives scale and bias of a channel itself from the op's ranges
   int fused;
   int nb;  // weight ranges (1 or N)
@@ -53,11 +56,22 @@ struct EpilogueArgs {
   CanonChain canon;  // filled by the tile dispatch for the kernels that take it
 };
 
-// Host: the chain in canonical form.  Returns 0 (no post-op), 1 (ReLU only), 2 (cheap activation and / or linear map),
-// 3 (GELU, optional linear map) or -1 (anything else: an addend, two activations, ...).
+// one element of the addend as fp32 (exact for the 8-bit types)
+__device__ __forceinline__ float load_addend(const EpilogueArgs& e, int64_t i) {
+  if (e.addend_type == ITEXHIP_QINT8) return static_cast<float>(static_cast<const int8_t*>(e.addend)[i]);
+  if (e.addend_type == ITEXHIP_QUINT8) return static_cast<float>(static_cast<const uint8_t*>(e.addend)[i]);
+  return static_cast<const float*>(e.addend)[i];
+}
+
+// Host: the chain in canonical form.  Returns 0 (no post-op), 1 (ReLU only), 2 (sum, cheap activation and / or linear
+// map), 3 (the same with GELU as the activation) or -1 (anything else: two activations, two sums, ...).
 inline int canon_chain(const EpilogueArgs& e, CanonChain* c) {
   *c = CanonChain{};
   int k = 0;
+  if (k < e.n_eltwise && e.elt[k].alg == ITEXHIP_ELT_SUM) {
+    c->flags |= kChainSumFirst; c->sum_scale = e.elt[k].alpha;
+    ++k;
+  }
   if (k < e.n_eltwise) {
     const itexhip_eltwise& a = e.elt[k];
     if (a.alg == ITEXHIP_ELT_RELU) {
@@ -70,6 +84,10 @@ inline int canon_chain(const EpilogueArgs& e, CanonChain* c) {
       c->flags |= a.alg == ITEXHIP_ELT_GELU_TANH ? kChainGeluTanh : kChainGeluErf;
       ++k;
     }
+  }
+  if (k < e.n_eltwise && e.elt[k].alg == ITEXHIP_ELT_SUM && !(c->flags & kChainSumFirst)) {
+    c->flags |= kChainSumLast; c->sum_scale = e.elt[k].alpha;
+    ++k;
   }
   if (k < e.n_eltwise && e.elt[k].alg == ITEXHIP_ELT_LINEAR) {
     c->flags |= kChainLinear; c->lin_a = e.elt[k].alpha; c->lin_b = e.elt[k].beta;
@@ -201,7 +219,7 @@ __device__ __forceinline__ void epilogue_store(const v4i acc, const ChannelParam
       v = fmaxf(v, 0.0f);
     } else if (ACT == 2) {
       for (int k = 0; k < e.n_eltwise; ++k) {
-        if (e.elt[k].alg == ITEXHIP_ELT_SUM) v = v + e.elt[k].alpha * e.addend[static_cast<int64_t>(m) * N + min(n + r, N - 1)];
+        if (e.elt[k].alg == ITEXHIP_ELT_SUM) v = v + e.elt[k].alpha * load_addend(e, static_cast<int64_t>(m) * N + min(n + r, N - 1));
         else v = apply_eltwise(e.elt[k], v);
       }
     }

@@ -335,8 +335,38 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void qgemm_tile_kernel(
     // applied to the 16 values of one 32x32 tile at a time under wavefront-uniform branches.  A loop over the chain
     // with a switch per value made the epilogue several times longer than the whole K loop (instruction fetch, not
     // arithmetic).  Same expressions as apply_eltwise.
-    auto apply_chain = [&](float (&v)[16]) {
+    // the addend of the 16 values of a tile: row m, channels n0 + 8 g + r (g, r < 4); 4 consecutive channels are
+    // one 16-byte (fp32) or 4-byte (8-bit types) load, aligned because N is a multiple of 4 and the host checked the base
+    auto add_sum = [&](float (&v)[16], int m, int n0) {
       const CanonChain& c = e.canon;
+      if (m >= M) return;
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int n = n0 + g * 8;
+        if (n < N) {
+          const int64_t o = static_cast<int64_t>(m) * N + n;
+          float a[4];
+          if (e.addend_type == ITEXHIP_FLOAT) {
+            const f4 t = *reinterpret_cast<const f4*>(static_cast<const float*>(e.addend) + o);
+            a[0] = t[0]; a[1] = t[1]; a[2] = t[2]; a[3] = t[3];
+          } else {
+            const uint32_t w = *reinterpret_cast<const uint32_t*>(static_cast<const uint8_t*>(e.addend) + o);
+            if (e.addend_type == ITEXHIP_QUINT8) {
+#pragma unroll
+              for (int r = 0; r < 4; ++r) a[r] = static_cast<float>((w >> (8 * r)) & 0xffu);
+            } else {
+#pragma unroll
+              for (int r = 0; r < 4; ++r) a[r] = static_cast<float>(static_cast<int>(w << (24 - 8 * r)) >> 24);
+            }
+          }
+#pragma unroll
+          for (int r = 0; r < 4; ++r) v[g * 4 + r] = v[g * 4 + r] + c.sum_scale * a[r];
+        }
+      }
+    };
+    auto apply_chain = [&](float (&v)[16], int m, int n0) {
+      const CanonChain& c = e.canon;
+      if (c.flags & kChainSumFirst) add_sum(v, m, n0);
       if constexpr (ACT == 3) {
         if (c.flags & kChainGeluTanh) {
           const itexhip_eltwise el{ITEXHIP_ELT_GELU_TANH, 0.0f, 0.0f};
@@ -361,6 +391,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void qgemm_tile_kernel(
           for (int r = 0; r < 16; ++r) v[r] = fminf(fmaxf(v[r], c.lo), c.hi);
         }
       }
+      if (c.flags & kChainSumLast) add_sum(v, m, n0);
       if (c.flags & kChainLinear) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) v[r] = c.lin_a * v[r] + c.lin_b;
@@ -391,7 +422,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void qgemm_tile_kernel(
               v[r] = static_cast<float>(acc[t][r]) * sc[r >> 2][r & 3];
               v[r] = v[r] + bi[r >> 2][r & 3];
             }
-            apply_chain(v);
+            apply_chain(v, m_base + (wm * TM + decltype(i)::value) * 32 + lrow, n_base + (wn * TN + j) * 32 + lgrp * 4);
             static_for<4>([&](auto g) {
               constexpr int r0 = decltype(g)::value * 4;
               put(i, g, epilogue_pack<OUT_T>(v4i{__float_as_int(v[r0]), __float_as_int(v[r0 + 1]), __float_as_int(v[r0 + 2]),
@@ -445,7 +476,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void qgemm_tile_kernel(
                   if (has_bias) v = v + bi[r];
                   const int64_t o = static_cast<int64_t>(m) * N + n + r;
                   for (int k = 0; k < e.n_eltwise; ++k) {
-                    if (e.elt[k].alg == ITEXHIP_ELT_SUM) v = v + e.elt[k].alpha * e.addend[o];
+                    if (e.elt[k].alg == ITEXHIP_ELT_SUM) v = v + e.elt[k].alpha * load_addend(e, o);
                     else v = apply_eltwise(e.elt[k], v);
                   }
                   store_output<OUT_T>(out, o, v);
@@ -523,7 +554,10 @@ int dispatch_tile(const uint8_t* a, uint32_t a_xor, const uint8_t* bp, int M, in
   constexpr int esz = (OUT_T == ITEXHIP_QINT8 || OUT_T == ITEXHIP_QUINT8) ? 1 : is_float16_type(OUT_T) ? 2 : 4;
   EpilogueArgs e = e_in;
   const int act = canon_chain(e, &e.canon);
-  const bool vec_epilogue = act >= 0 && e.addend == nullptr && (e.bias != nullptr || e.fused) &&
+  const bool has_sum = (e.canon.flags & (kChainSumFirst | kChainSumLast)) != 0;
+  const bool sum_ok = !has_sum || (e.addend != nullptr && (N & 3) == 0 &&
+                                   (reinterpret_cast<uintptr_t>(e.addend) & (e.addend_type == ITEXHIP_FLOAT ? 15 : 3)) == 0);
+  const bool vec_epilogue = act >= 0 && sum_ok && (e.bias != nullptr || e.fused) &&
                             (reinterpret_cast<uintptr_t>(out) & 15) == 0 && ((static_cast<int64_t>(N) * esz) & 15) == 0;
   const bool wide = pick_tile_shape(M, N, true) == 3;
   if (vec_epilogue && (K & 63) == 0) {
@@ -553,7 +587,12 @@ int dispatch_tile_conv(const uint8_t* x, uint32_t a_xor, const uint8_t* bp, int 
   EpilogueArgs e = e_in;
   const int act = canon_chain(e, &e.canon);
   if (act < 0 || act == 3) {
-    set_error("itexhip_qconv2d: the post-ops must be one of ReLU / LeakyReLU / clip, optionally followed by a linear map");
+    set_error("itexhip_qconv2d: the post-ops must be [sum] [ReLU / LeakyReLU / clip] [sum] [linear map], at most one sum");
+    return ITEXHIP_INVALID_ARGUMENT;
+  }
+  if ((e.canon.flags & (kChainSumFirst | kChainSumLast)) &&
+      (e.addend == nullptr || (N & 3) != 0 || (reinterpret_cast<uintptr_t>(e.addend) & (e.addend_type == ITEXHIP_FLOAT ? 15 : 3)) != 0)) {
+    set_error("itexhip_qconv2d_sum: the summand must be 4-byte (8-bit types) or 16-byte (float) aligned and out_channels a multiple of 4");
     return ITEXHIP_INVALID_ARGUMENT;
   }
   struct Shape { int bm, bn; double penalty; };

@@ -858,7 +858,21 @@ int orc_qconv_prepare(const orc_conv_attrs* at, int64_t N, float min_in, float m
 int orc_qconv2d(const orc_conv_attrs* at, const orc_conv_geom* g, const void* x, const int8_t* w,
                 const void* bias, float min_in, float max_in, const float* min_f, const float* max_f,
                 int64_t depth, float min_out, float max_out, void* out, int64_t* out_h, int64_t* out_w) {
+  return orc_qconv2d_sum(at, g, x, w, bias, min_in, max_in, min_f, max_f, depth, min_out, max_out, NULL, NULL, out, out_h,
+                         out_w);
+}
+
+int orc_qconv2d_sum(const orc_conv_attrs* at, const orc_conv_geom* g, const void* x, const int8_t* w,
+                    const void* bias, float min_in, float max_in, const float* min_f, const float* max_f,
+                    int64_t depth, float min_out, float max_out, const orc_conv_sum* sum, const void* summand,
+                    void* out, int64_t* out_h, int64_t* out_w) {
   int64_t pt = 0, pl = 0;
+  if (sum != NULL && sum->position != 0) {
+    if (at->t_out != ORC_QINT8 && at->t_out != ORC_QUINT8) return ORC_UNIMPLEMENTED; /* qint32 + float summand: not restated */
+    if (sum->t_summand != ORC_QINT8 && sum->t_summand != ORC_QUINT8) return ORC_INVALID_ARGUMENT;
+    if (sum->t_summand == ORC_QUINT8 && at->t_out == ORC_QINT8) return ORC_INVALID_ARGUMENT; /* :213-218 */
+    if (sum->position != 1 && sum->position != 2) return ORC_INVALID_ARGUMENT;
+  }
   if (orc_conv_out_dim(g->in_h, g->k_h, g->stride_h, g->dil_h, g->padding, g->pad_top, g->pad_bottom, out_h, &pt) ||
       orc_conv_out_dim(g->in_w, g->k_w, g->stride_w, g->dil_w, g->padding, g->pad_left, g->pad_right, out_w, &pl))
     return ORC_INVALID_ARGUMENT;
@@ -869,10 +883,29 @@ int orc_qconv2d(const orc_conv_attrs* at, const orc_conv_geom* g, const void* x,
   float* sb = (float*)malloc(sizeof(float) * (size_t)N);
   orc_epilogue_desc ep;
   int st = orc_qconv_prepare(at, N, min_in, max_in, min_f, max_f, depth, min_out, max_out, bias, scales, sb, &ep);
+  float* addend = NULL;
+  if (st == ORC_OK && sum != NULL && sum->position != 0) {
+    /* :398-433 */
+    const float scale_output = fmaxf(fabsf(min_out), fabsf(max_out));
+    const float scale_summand = fmaxf(fabsf(sum->min_summand), fabsf(sum->max_summand));
+    float sum_post_op_scale;
+    if (at->t_out == ORC_QUINT8 && sum->t_summand == ORC_QINT8) sum_post_op_scale = 255.0f * scale_summand / (scale_output * 127.0f);
+    else sum_post_op_scale = scale_summand / scale_output;
+    /* the destination's previous contents as the output type reads them (:622-626: bytes of a qint8 summand are
+     * taken as quint8 when the output is quint8) */
+    addend = (float*)malloc(sizeof(float) * (size_t)(M * N));
+    for (int64_t i = 0; i < M * N; ++i)
+      addend[i] = (at->t_out == ORC_QUINT8) ? (float)((const uint8_t*)summand)[i] : (float)((const int8_t*)summand)[i];
+    /* place the sum in the chain: before or after the activation */
+    orc_eltwise s_elt;
+    s_elt.alg = ORC_ELT_SUM; s_elt.alpha = sum_post_op_scale; s_elt.beta = 0.0f;
+    if (sum->position == 1 && ep.n_eltwise == 1) { ep.elt[1] = ep.elt[0]; ep.elt[0] = s_elt; ep.n_eltwise = 2; }
+    else { ep.elt[ep.n_eltwise++] = s_elt; }
+  }
   if (st == ORC_OK) {
     orc_int_conv2d(x, at->t_in, w, g, *out_h, *out_w, pt, pl, acc);
-    orc_qmatmul_epilogue(acc, M, N, &ep, scales, sb, NULL, at->t_out, out);
+    orc_qmatmul_epilogue(acc, M, N, &ep, scales, sb, addend, at->t_out, out);
   }
-  free(acc); free(scales); free(sb);
+  free(acc); free(scales); free(sb); free(addend);
   return st;
 }

@@ -193,6 +193,21 @@ int orc_qconv_prepare(const orc_conv_attrs* at, int64_t N, float min_in, float m
 int orc_qconv2d(const orc_conv_attrs* at, const orc_conv_geom* g, const void* x, const int8_t* w,
                 const void* bias, float min_in, float max_in, const float* min_f, const float* max_f,
                 int64_t depth, float min_out, float max_out, void* out, int64_t* out_h, int64_t* out_w);
+/* The "Sum" fusions (QuantizedConv2DWithBias[Signed]SumAndReluAndRequantize, "Sum" in fused_ops of _QuantizedConv2D)
+ * with an 8-bit output, quantized_conv_ops.h:202-218 (type rule), :398-433 (scale of the sum post-op from the frozen
+ * output range and the summand's range), :604-640 (the summand buffer becomes the destination; a qint8 summand under
+ * a quint8 output is bit-cast to quint8, i.e. its bytes are read as unsigned, as written there).
+ * position: 1 = before the activation ([BiasAdd, Sum, Relu]), 2 = after it ([BiasAdd, Relu, Sum]).
+ * `summand` has the output's shape.  parity unpinned: no vectors of the reference cover these ops. */
+typedef struct {
+  int position;
+  int t_summand;                  /* ORC_QINT8 | ORC_QUINT8 */
+  float min_summand, max_summand;
+} orc_conv_sum;
+int orc_qconv2d_sum(const orc_conv_attrs* at, const orc_conv_geom* g, const void* x, const int8_t* w,
+                    const void* bias, float min_in, float max_in, const float* min_f, const float* max_f,
+                    int64_t depth, float min_out, float max_out, const orc_conv_sum* sum, const void* summand,
+                    void* out, int64_t* out_h, int64_t* out_w);
 
 #ifdef __cplusplus
 }

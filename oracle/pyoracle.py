@@ -315,17 +315,25 @@ def qconv_prepare(at, N, min_in, max_in, min_f, max_f, min_out, max_out, bias):
     return st, scales, sb, ep
 
 
-def qconv2d(at, g, x, w, bias, min_in, max_in, min_f, max_f, min_out=0.0, max_out=0.0):
-    """x: [B, H, W, C] uint8 / int8, w: [KH, KW, C, O] int8.  Returns (status, out [B, OH, OW, O])."""
+class ConvSum(C.Structure):
+    _fields_ = [("position", C.c_int), ("t_summand", C.c_int), ("min_summand", C.c_float), ("max_summand", C.c_float)]
+
+
+def qconv2d(at, g, x, w, bias, min_in, max_in, min_f, max_f, min_out=0.0, max_out=0.0, sum=None, summand=None):
+    """x: [B, H, W, C] uint8 / int8, w: [KH, KW, C, O] int8.  Returns (status, out [B, OH, OW, O]).
+    sum: ConvSum(position, t_summand, min, max) with `summand` an array of the output's shape (int8 / uint8)."""
     x = np.ascontiguousarray(x, dtype=np.uint8 if at.t_in == QUINT8 else np.int8)
     w = np.ascontiguousarray(w, dtype=np.int8)
     min_f, max_f = _f32(min_f), _f32(max_f)
     b = None if bias is None else (np.ascontiguousarray(bias, np.int32) if at.t_bias == QINT32 else _f32(bias))
     oh, ow = C.c_int64(), C.c_int64()
-    f = lib().orc_qconv2d
+    f = lib().orc_qconv2d_sum
     f.restype = C.c_int
+    if sum is not None:
+        summand = np.ascontiguousarray(summand, dtype=np.uint8 if sum.t_summand == QUINT8 else np.int8)
     args = lambda out: (C.byref(at), C.byref(g), _p(x), _p(w), _p(b) if b is not None else None, C.c_float(min_in),
                         C.c_float(max_in), _p(min_f), _p(max_f), C.c_int64(min_f.size), C.c_float(min_out), C.c_float(max_out),
+                        C.byref(sum) if sum is not None else None, _p(summand) if sum is not None else None,
                         out, C.byref(oh), C.byref(ow))
     st = f(*args(None))
     if st != OK:

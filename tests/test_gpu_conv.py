@@ -138,6 +138,69 @@ def test_implicit_gemm_conv(hip, dev, monkeypatch, shape, wshape, strides, dil, 
         assert torch.equal(a.view(torch.uint8), b_.view(torch.uint8)), T
 
 
+@pytest.mark.parametrize("t_add", ["u8", "s8", "f32"])
+@pytest.mark.parametrize("position,alpha", [(1, 0.0), (2, 0.0), (1, 0.2), (2, None)])
+def test_sum_post_op_in_conv_and_gemm(hip, dev, t_add, position, alpha):
+    """One sum post-op (y += scale * addend, the addend float / qint8 / quint8) before or after the activation, through
+    itexhip_qconv2d_sum (implicit GEMM), itexhip_qgemm_sum on the patch matrix (tile kernel), on 16 rows of it
+    (the M <= 16 kernel) and in place (output buffer = addend buffer): all equal to the oracle's epilogue on the
+    int32 convolution."""
+    import torch
+    from tests.test_oracle_conv import ref_int_conv
+    rng = np.random.default_rng(position * 10 + len(t_add))
+    shape, wshape = (2, 10, 9, 32), (3, 3, 32, 48)
+    B, H, W, Cin = shape
+    O = wshape[3]
+    x = rng.integers(0, 256, shape).astype(np.uint8)
+    w = rng.integers(-127, 128, wshape).astype(np.int8)
+    acc = ref_int_conv(x, w, (1, 1), (1, 1), ((1, 1), (1, 1))).reshape(-1, O).astype(np.int32)
+    M, K = acc.shape[0], 9 * Cin
+    g = hip.ConvGeometry(B, H, W, Cin, 3, 3, H, W, 1, 1, 1, 1, 1, 1)
+    add_np = {"u8": rng.integers(0, 256, (M, O)).astype(np.uint8), "s8": rng.integers(-128, 128, (M, O)).astype(np.int8),
+              "f32": (rng.standard_normal((M, O)) * 20).astype(np.float32)}[t_add]
+    T_add = {"u8": hip.QUINT8, "s8": hip.QINT8, "f32": hip.FLOAT}[t_add]
+    scales = (rng.random(O).astype(np.float32) + 0.5) * np.float32(3e-4)
+    bias = rng.standard_normal(O).astype(np.float32)
+    chain = [(orc.ELT_SUM, 0.37, 0.0)]
+    if alpha is not None:
+        act = (orc.ELT_RELU, alpha, 0.0)
+        chain = [chain[0], act] if position == 1 else [act, chain[0]]
+    oep, ep = orc.EpilogueDesc(), hip.Epilogue()
+    oep.n_scales = ep.n_scales = O
+    oep.n_eltwise = ep.n_eltwise = len(chain)
+    for k, (alg, a_, b_) in enumerate(chain):
+        oep.elt[k].alg, oep.elt[k].alpha, oep.elt[k].beta = alg, a_, b_
+        ep.elt[k].alg, ep.elt[k].alpha, ep.elt[k].beta = alg, a_, b_
+    xd, add_d = torch.from_numpy(x).to(dev), torch.from_numpy(add_np).to(dev)
+    packed = torch.empty(hip.qgemm_packed_bytes(K, O), dtype=torch.int8, device=dev)
+    colsum = torch.empty(O, dtype=torch.int32, device=dev)
+    hip.qgemm_prepack_b(torch.from_numpy(w.reshape(K, O)).to(dev), False, K, O, packed, colsum)
+    sc_d, bi_d = torch.from_numpy(scales).to(dev), torch.from_numpy(bias).to(dev)
+    cols = torch.empty((M, K), dtype=torch.uint8, device=dev)
+    hip.im2col8(xd, g, K, cols)
+    for T, dt, npdt in ((hip.QUINT8, torch.uint8, np.uint8), (hip.QINT8, torch.int8, np.int8), (hip.FLOAT, torch.float32, np.float32)):
+        ref = orc.qmatmul_epilogue(acc, oep, scales, bias, T, addend=add_np.astype(np.float32))
+        out = torch.zeros((M, O), dtype=dt, device=dev)
+        hip.qconv2d_sum(xd, hip.QUINT8, g, packed, colsum, O, sc_d, bi_d, ep, add_d, T_add, T, out)
+        torch.cuda.synchronize()
+        np.testing.assert_array_equal(out.cpu().numpy(), ref)
+        out.zero_()
+        hip.qgemm_sum(cols, hip.QUINT8, packed, colsum, M, K, O, sc_d, bi_d, ep, add_d, T_add, T, out)
+        torch.cuda.synchronize()
+        np.testing.assert_array_equal(out.cpu().numpy(), ref)
+        out16 = torch.zeros((16, O), dtype=dt, device=dev)
+        hip.qgemm_sum(cols, hip.QUINT8, packed, colsum, 16, K, O, sc_d, bi_d, ep, add_d, T_add, T, out16)
+        torch.cuda.synchronize()
+        np.testing.assert_array_equal(out16.cpu().numpy(), ref[:16])
+        if add_np.dtype.itemsize == np.dtype(npdt).itemsize:     # in place: the addend buffer is the output buffer
+            both = add_d.clone()
+            hip.qconv2d_sum(xd, hip.QUINT8, g, packed, colsum, O, sc_d, bi_d, ep, both, T_add, T, both)
+            torch.cuda.synchronize()
+            np.testing.assert_array_equal(both.cpu().numpy().view(npdt), ref)
+    with pytest.raises(hip.ItexHipError):     # a sum in the chain without an addend
+        hip.qgemm(cols, hip.QUINT8, packed, colsum, M, K, O, sc_d, bi_d, ep, hip.FLOAT, torch.zeros((M, O), device=dev))
+
+
 def test_implicit_gemm_conv_rejects_other_shapes(hip, dev):
     import torch
     x = torch.zeros(4 * 4 * 24 + 16, dtype=torch.uint8, device=dev)

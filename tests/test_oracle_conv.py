@@ -182,3 +182,57 @@ def test_scales_closed_forms_and_qint32_forms():
     assert st == orc.OK and ep.n_scales == 1 and ep.elt[0].alpha == np.float32(0.1)
     st, _, _, _ = orc.qconv_prepare(at, N, 0.0, 4.0, fmn[:3], fmx[:3], 0.0, 0.0, bf)
     assert st == orc.INVALID_ARGUMENT
+
+
+@pytest.mark.parametrize("t_out,t_sum,position", [(orc.QUINT8, orc.QUINT8, 1), (orc.QUINT8, orc.QINT8, 1), (orc.QINT8, orc.QINT8, 1),
+                                                  (orc.QUINT8, orc.QUINT8, 2), (orc.QINT8, orc.QINT8, 2)])
+def test_sum_fusion_against_an_independent_evaluation(t_out, t_sum, position):
+    """[BiasAdd, Sum, Relu, Requantize] and [BiasAdd, Relu, Sum, Requantize]: the fused result equals the unfused int32
+    convolution taken through the same fp32 steps in numpy (scale, bias, sum scale x summand, ReLU, saturate + round
+    half to even), with the sum scale of quantized_conv_ops.h:398-433 written out here from the ranges."""
+    rng = np.random.default_rng(7 + t_out + t_sum + position)
+    x = rng.integers(0, 256, (2, 7, 6, 8)).astype(np.uint8)
+    w = rng.integers(-127, 128, (3, 3, 8, 16)).astype(np.int8)
+    bias = rng.uniform(-1, 1, 16).astype(np.float32)
+    g = orc.conv_geom(x.shape, w.shape)
+    min_in, max_in, min_f, max_f = 0.0, 4.0, np.float32(-0.5), np.float32(0.5)
+    min_out, max_out = (0.0, 30.0) if t_out == orc.QUINT8 else (-30.0, 30.0)
+    summand = (rng.integers(0, 256, (2, 7, 6, 16)).astype(np.uint8) if t_sum == orc.QUINT8
+               else rng.integers(-128, 128, (2, 7, 6, 16)).astype(np.int8))
+    min_s, max_s = (0.0, 12.0) if t_sum == orc.QUINT8 else (-9.0, 12.0)
+    at = orc.ConvAttrs(orc.QUINT8, t_out, orc.FLOAT, orc.ACT_RELU, 0.0)
+    st, got = orc.qconv2d(at, g, x, w, bias, min_in, max_in, min_f, max_f, min_out, max_out,
+                          sum=orc.ConvSum(position, t_sum, min_s, max_s), summand=summand)
+    assert st == orc.OK
+    # independent evaluation
+    st, acc = orc.qconv2d(orc.ConvAttrs(orc.QUINT8, orc.QINT32, 0, orc.ACT_NONE, 0.0), g, x, w, None, min_in, max_in, min_f, max_f)
+    assert st == orc.OK
+    f32 = np.float32
+    lim_out = f32(255.0 if t_out == orc.QUINT8 else 127.0)
+    scale = lim_out * f32(4.0) * f32(0.5) / (f32(255.0 * 127.0) * f32(30.0))
+    bias_scaled = bias * (f32(255.0 * 127.0) / (f32(4.0) * f32(0.5)) * scale)
+    s_out, s_sum = f32(30.0), f32(12.0)
+    sum_scale = f32(255.0) * s_sum / (s_out * f32(127.0)) if (t_out == orc.QUINT8 and t_sum == orc.QINT8) else s_sum / s_out
+    prev = summand.view(np.uint8 if t_out == orc.QUINT8 else np.int8).astype(np.float32)   # read as the output type
+    y = acc.astype(np.float32) * scale + bias_scaled
+    if position == 1:
+        y = np.maximum(y + sum_scale * prev, f32(0))
+    else:
+        y = np.maximum(y, f32(0)) + sum_scale * prev
+    lo, hi = (0, 255) if t_out == orc.QUINT8 else (-128, 127)
+    ref = np.clip(np.rint(y), lo, hi).astype(got.dtype)
+    np.testing.assert_array_equal(got, ref)
+    assert len(np.unique(got)) > 20          # not saturated away
+
+
+def test_sum_fusion_type_rules():
+    x = np.zeros((1, 4, 4, 4), np.uint8)
+    w = np.zeros((1, 1, 4, 4), np.int8)
+    g = orc.conv_geom(x.shape, w.shape)
+    s = np.zeros((1, 4, 4, 4), np.uint8)
+    run = lambda t_out, t_sum: orc.qconv2d(orc.ConvAttrs(orc.QUINT8, t_out, 0, orc.ACT_RELU, 0.0), g, x, w, None, 0.0, 1.0,
+                                           np.float32(-1), np.float32(1), -1.0, 1.0, sum=orc.ConvSum(1, t_sum, 0.0, 1.0),
+                                           summand=s)[0]
+    assert run(orc.QINT8, orc.QUINT8) == orc.INVALID_ARGUMENT      # quantized_conv_ops.h:213-218
+    assert run(orc.QINT32, orc.QUINT8) == orc.UNIMPLEMENTED        # the qint32 form takes a float summand: not restated
+    assert run(orc.QUINT8, orc.QINT8) == orc.OK
