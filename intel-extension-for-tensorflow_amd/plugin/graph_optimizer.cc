@@ -40,6 +40,8 @@ const Rename kTable[] = {
     {"QuantizedConv2DWithBiasAndRelu", "_ITEXQuantizedConv2DWithBiasAndRelu", Copy::kQuantizedConv2D, Rule::kAlways},
     {"QuantizedConv2DWithBiasAndReluAndRequantize", "_ITEXQuantizedConv2DWithBiasAndReluAndRequantize", Copy::kQuantizedConv2D, Rule::kAlways},
     {"QuantizedConv2DWithBiasAndRequantize", "_ITEXQuantizedConv2DWithBiasAndRequantize", Copy::kQuantizedConv2D, Rule::kAlways},
+    {"QuantizedConv2DWithBiasSumAndReluAndRequantize", "_ITEXQuantizedConv2DWithBiasSumAndReluAndRequantize", Copy::kQuantizedConv2D, Rule::kAlways},
+    {"QuantizedConv2DWithBiasSignedSumAndReluAndRequantize", "_ITEXQuantizedConv2DWithBiasSignedSumAndReluAndRequantize", Copy::kQuantizedConv2D, Rule::kAlways},
     {"_QuantizedConv2D", "_ITEXQuantizedConv2DV2", Copy::kAll, Rule::kAlways},
     {"QuantizedMatMulWithBias", "_ITEXQuantizedMatMulWithBias", Copy::kQuantizedMatMul, Rule::kAlways},
     {"QuantizedMatMulWithBiasAndDequantize", "_ITEXQuantizedMatMulWithBiasAndDequantize", Copy::kQuantizedMatMul, Rule::kAlways},

@@ -187,7 +187,7 @@ std::vector<OpSpec> OpSpecs() {
     const std::vector<const char*> base_attrs = {"Tinput: quantizedtype", "Tfilter: quantizedtype", "strides: list(int)",
                                                  "padding: {'SAME', 'VALID'}", "dilations: list(int) = [1, 1, 1, 1]",
                                                  "padding_list: list(int) = []", "is_filter_const: bool = true"};
-    struct Twin { const char* name; bool bias, req; const char* out_default; };
+    struct Twin { const char* name; bool bias, req; const char* out_default; bool sum = false; };
     for (const Twin& t : {Twin{"_ITEXQuantizedConv2D", false, false, "out_type: quantizedtype = DT_QINT32"},
                           Twin{"_ITEXQuantizedConv2DPerChannel", false, false, "out_type: quantizedtype = DT_QINT32"},
                           Twin{"_ITEXQuantizedConv2DWithBias", true, false, "out_type: quantizedtype = DT_QINT32"},
@@ -196,7 +196,10 @@ std::vector<OpSpec> OpSpecs() {
                           Twin{"_ITEXQuantizedConv2DAndRequantize", false, true, "out_type: quantizedtype = DT_QINT8"},
                           Twin{"_ITEXQuantizedConv2DAndReluAndRequantize", false, true, "out_type: quantizedtype = DT_QUINT8"},
                           Twin{"_ITEXQuantizedConv2DWithBiasAndRequantize", true, true, "out_type: quantizedtype = DT_QINT8"},
-                          Twin{"_ITEXQuantizedConv2DWithBiasAndReluAndRequantize", true, true, "out_type: quantizedtype = DT_QUINT8"}}) {
+                          Twin{"_ITEXQuantizedConv2DWithBiasAndReluAndRequantize", true, true, "out_type: quantizedtype = DT_QUINT8"},
+                          Twin{"_ITEXQuantizedConv2DWithBiasSumAndReluAndRequantize", true, true, "out_type: quantizedtype = DT_QUINT8", true},
+                          Twin{"_ITEXQuantizedConv2DWithBiasSignedSumAndReluAndRequantize", true, true,
+                               "out_type: quantizedtype = DT_QUINT8", true}}) {
       OpSpec s{t.name, {"input: Tinput", "filter: Tfilter"}, {"output: out_type", "min_output: float", "max_output: float"}, base_attrs};
       if (t.bias) s.inputs.push_back(t.req ? "bias: Tbias" : "bias: float");
       for (const char* in : {"min_input: float", "max_input: float", "min_filter: float", "max_filter: float"}) s.inputs.push_back(in);
@@ -204,6 +207,10 @@ std::vector<OpSpec> OpSpecs() {
         s.inputs.push_back("min_freezed_output: float");
         s.inputs.push_back("max_freezed_output: float");
         if (t.bias) s.attrs.push_back("Tbias: {float, qint32}");
+      }
+      if (t.sum) {  // nn_ops.cc of TensorFlow: ..., summand, min_summand, max_summand
+        for (const char* in : {"summand: Tsummand", "min_summand: float", "max_summand: float"}) s.inputs.push_back(in);
+        s.attrs.push_back("Tsummand: quantizedtype");
       }
       s.attrs.push_back(t.out_default);
       v.push_back(s);

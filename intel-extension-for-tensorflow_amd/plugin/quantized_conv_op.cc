@@ -31,6 +31,8 @@ std::vector<std::string> LegacyFusions(const std::string& op) {
   if (name == "QuantizedConv2DAndReluAndRequantize") return {"Relu", "Requantize"};
   if (name == "QuantizedConv2DWithBiasAndRequantize") return {"BiasAdd", "Requantize"};
   if (name == "QuantizedConv2DWithBiasAndReluAndRequantize") return {"BiasAdd", "Relu", "Requantize"};
+  if (name == "QuantizedConv2DWithBiasSumAndReluAndRequantize" || name == "QuantizedConv2DWithBiasSignedSumAndReluAndRequantize")
+    return {"BiasAdd", "Sum", "Relu", "Requantize"};
   return {};
 }
 
@@ -55,7 +57,6 @@ class QuantizedConv2DOp : public OpKernel {
  public:
   QuantizedConv2DOp(OpKernelConstruction* ctx, const std::string& op, bool new_api, TF_DataType t_in, TF_DataType t_out)
       : t_in_(t_in), t_out_(t_out) {
-    (void)new_api;
     std::vector<int64_t> strides, dilations;
     ITEX_REQUIRES_OK(ctx, ctx->GetAttr("dilations", &dilations));
     ITEX_REQUIRES_OK(ctx, ctx->GetAttr("strides", &strides));
@@ -101,12 +102,25 @@ class QuantizedConv2DOp : public OpKernel {
       if (f == "BiasAdd") fuse_bias_ = true;
       else if (f == "Requantize") fuse_requantize_ = true;
       else if (f == "Dequantize") fuse_dequantize_ = true;
-      else if (f == "Relu") activation_ = ITEXHIP_ELT_RELU;
-      else if (f == "LeakyRelu") { activation_ = ITEXHIP_ELT_RELU; leaky_ = true; }
+      else if (f == "Relu") { activation_ = ITEXHIP_ELT_RELU; if (sum_position_ == 0) sum_position_ = -1; }
+      else if (f == "LeakyRelu") { activation_ = ITEXHIP_ELT_RELU; leaky_ = true; if (sum_position_ == 0) sum_position_ = -1; }
+      else if (f == "Sum") sum_position_ = sum_position_ == -1 ? 2 : 1;  // after / before the activation
       else
         ITEX_REQUIRES(ctx, false, TF_UNIMPLEMENTED, "the " + f + " fusion of the quantized Conv2D is not implemented on this device");
     }
+    if (sum_position_ < 0) sum_position_ = 0;
     if (leaky_) ITEX_REQUIRES_OK(ctx, ctx->GetAttr("alpha", &alpha_));
+    if (sum_position_ != 0) {
+      // quantized_conv_ops.h:202-218, 398-433: an 8-bit summand under an 8-bit output; the qint32 output with a float
+      // summand (the graph before Requantize is fused) is not built
+      ITEX_REQUIRES(ctx, fuse_requantize_, TF_UNIMPLEMENTED,
+                    "the Sum fusion of the quantized Conv2D is implemented together with Requantize only");
+      ITEX_REQUIRES_OK(ctx, ctx->GetAttr("Tsummand", &t_summand_));
+      ITEX_REQUIRES(ctx, t_summand_ == TF_QINT8 || t_summand_ == TF_QUINT8, TF_UNIMPLEMENTED,
+                    "the Sum fusion of the quantized Conv2D takes a qint8 or quint8 summand on this device");
+      ITEX_REQUIRES(ctx, !(t_summand_ == TF_QUINT8 && t_out == TF_QINT8), TF_INVALID_ARGUMENT,
+                    "Current fusion requires summand has same dtype as output if output is qint8");
+    }
     if (fuse_requantize_)
       ITEX_REQUIRES(ctx, t_out == TF_QINT8 || t_out == TF_QUINT8, TF_INVALID_ARGUMENT,
                     "QuantizedConv: unsupported output type when Requantize is fused.");
@@ -125,13 +139,26 @@ class QuantizedConv2DOp : public OpKernel {
     src_min_idx_ = 2 + bias_off;
     filter_min_idx_ = src_min_idx_ + 2;
     freezed_idx_ = 6 + bias_off;  // both spellings, without a summand and with a float / qint32 bias
+    if (sum_position_ != 0) {
+      if (new_api) {  // input, filter, {bias}, summand, min/max input, min/max filter, min/max summand, min/max freezed output
+        summand_idx_ = 2 + bias_off;
+        src_min_idx_ = 3 + bias_off;
+        filter_min_idx_ = src_min_idx_ + 2;
+        summand_min_idx_ = 6 + bias_off + 1;
+        freezed_idx_ = summand_min_idx_ + 2;
+      } else {        // ..., min/max freezed output, summand, min/max summand
+        summand_idx_ = 8 + bias_off;
+        summand_min_idx_ = 9 + bias_off;
+      }
+    }
   }
 
   void Compute(OpKernelContext* ctx) override {
     Tensor x = ctx->input(0);
     Tensor filter = ctx->input(1);
     if (!ctx->ok()) return;
-    ITEX_REQUIRES(ctx, ctx->num_inputs() >= filter_min_idx_ + 2 && (!fuse_requantize_ || ctx->num_inputs() >= freezed_idx_ + 2),
+    ITEX_REQUIRES(ctx, ctx->num_inputs() >= filter_min_idx_ + 2 && (!fuse_requantize_ || ctx->num_inputs() >= freezed_idx_ + 2) &&
+                           (sum_position_ == 0 || ctx->num_inputs() >= summand_min_idx_ + 2),
                   TF_INVALID_ARGUMENT, "the min / max inputs are missing");
     Tensor min_in_t = ctx->input(src_min_idx_), max_in_t = ctx->input(src_min_idx_ + 1);
     Tensor min_f_t = ctx->input(filter_min_idx_), max_f_t = ctx->input(filter_min_idx_ + 1);
@@ -244,13 +271,32 @@ class QuantizedConv2DOp : public OpKernel {
         ITEX_REQUIRES(ctx, st == ITEXHIP_OK, TF_ABORTED, std::string("Operation received an exception: ") + itexhip_last_error());
         bias_dev = sbias.flat<float>();
       }
+      // ---- summand of the Sum fusion
+      const void* summand_dev = nullptr;
+      int summand_type = 0;
+      float sum_scale = 0.0f;
+      if (sum_position_ != 0) {
+        Tensor summand = ctx->input(summand_idx_);
+        Tensor min_s = ctx->input(summand_min_idx_), max_s = ctx->input(summand_min_idx_ + 1);
+        if (!ctx->ok()) return;
+        ITEX_REQUIRES(ctx, (summand.dtype() == TF_QINT8 || summand.dtype() == TF_QUINT8) && summand.NumElements() == M * O,
+                      TF_INVALID_ARGUMENT, "the summand must be a qint8 / quint8 tensor of the output's shape");
+        // :398-433; the destination's previous contents are read as the output type (:622-626 bit-casts a qint8 summand)
+        const float scale_output = std::max(std::abs(min_out), std::abs(max_out));
+        const float scale_summand = std::max(std::abs(min_s.flat<float>()[0]), std::abs(max_s.flat<float>()[0]));
+        if (t_out_ == TF_QUINT8 && summand.dtype() == TF_QINT8) sum_scale = 255.0f * scale_summand / (scale_output * 127.0f);
+        else sum_scale = scale_summand / scale_output;
+        summand_dev = summand.data();
+        summand_type = t_out_;
+      }
       // ---- patches, then the quantized GEMM
       const void* a = x.data();
       Tensor cols;
       const bool pointwise = KH == 1 && KW == 1 && stride_h_ == 1 && stride_w_ == 1 && g.pad_top == 0 && g.pad_left == 0 &&
                              g.out_h == H && g.out_w == W && K == Kp;
       // windows the tile kernel can gather by itself (input channels a multiple of 16, ...) need no patch matrix
-      const bool implicit = !pointwise && itexhip_qconv2d_implicit_ok(&g, x.data(), O, t_out_, out.data()) != 0;
+      const bool implicit = !pointwise && itexhip_qconv2d_implicit_ok(&g, x.data(), O, t_out_, out.data()) != 0 &&
+                            (reinterpret_cast<uintptr_t>(summand_dev) & 3) == 0;
       if (!pointwise && !implicit) {
         cols = ctx->allocate_temp(t_in_, {M, Kp});
         if (!ctx->ok()) return;
@@ -260,16 +306,21 @@ class QuantizedConv2DOp : public OpKernel {
       }
       itexhip_epilogue ep{};
       ep.n_scales = static_cast<int>(depth);
-      if (activation_ != 0) {
-        ep.n_eltwise = 1;
-        ep.elt[0].alg = activation_;
-        ep.elt[0].alpha = leaky_ ? alpha_ : 0.0f;
-        ep.elt[0].beta = 0.0f;
+      if (sum_position_ == 1) ep.elt[ep.n_eltwise++] = {ITEXHIP_ELT_SUM, sum_scale, 0.0f};
+      if (activation_ != 0) ep.elt[ep.n_eltwise++] = {activation_, leaky_ ? alpha_ : 0.0f, 0.0f};
+      if (sum_position_ == 2) ep.elt[ep.n_eltwise++] = {ITEXHIP_ELT_SUM, sum_scale, 0.0f};
+      int st;
+      if (summand_dev != nullptr) {
+        st = implicit ? itexhip_qconv2d_sum(x.data(), t_in_, &g, packed_.flat<int8_t>(), colsum_.flat<int32_t>(), O, params,
+                                            bias_dev, &ep, summand_dev, summand_type, t_out_, out.data(), stream)
+                      : itexhip_qgemm_sum(a, t_in_, packed_.flat<int8_t>(), colsum_.flat<int32_t>(), M, Kp, O, params, bias_dev,
+                                          &ep, summand_dev, summand_type, t_out_, out.data(), stream);
+      } else {
+        st = implicit ? itexhip_qconv2d(x.data(), t_in_, &g, packed_.flat<int8_t>(), colsum_.flat<int32_t>(), O, params,
+                                        bias_dev, &ep, t_out_, out.data(), stream)
+                      : itexhip_qgemm(a, t_in_, packed_.flat<int8_t>(), colsum_.flat<int32_t>(), M, Kp, O, params, bias_dev,
+                                      &ep, t_out_, out.data(), stream);
       }
-      const int st = implicit ? itexhip_qconv2d(x.data(), t_in_, &g, packed_.flat<int8_t>(), colsum_.flat<int32_t>(), O, params,
-                                                bias_dev, &ep, t_out_, out.data(), stream)
-                              : itexhip_qgemm(a, t_in_, packed_.flat<int8_t>(), colsum_.flat<int32_t>(), M, Kp, O, params,
-                                              bias_dev, &ep, t_out_, out.data(), stream);
       ITEX_REQUIRES(ctx, st == ITEXHIP_OK, st == ITEXHIP_INVALID_ARGUMENT ? TF_INVALID_ARGUMENT : TF_ABORTED,
                     std::string("Operation received an exception: ") + itexhip_last_error());
     }
@@ -295,6 +346,9 @@ class QuantizedConv2DOp : public OpKernel {
 
  private:
   TF_DataType t_in_, t_out_, t_bias_ = TF_FLOAT;
+  TF_DataType t_summand_ = TF_QUINT8;
+  int sum_position_ = 0;  // 0 none, 1 before the activation, 2 after it
+  int summand_idx_ = -1, summand_min_idx_ = -1;
   int64_t stride_h_ = 1, stride_w_ = 1, dil_h_ = 1, dil_w_ = 1;
   std::string padding_;
   std::vector<int64_t> explicit_;
@@ -316,7 +370,9 @@ struct ConvKernel;
 const char* const kLegacyNames[] = {"QuantizedConv2D", "QuantizedConv2DPerChannel", "QuantizedConv2DWithBias",
                                     "QuantizedConv2DWithBiasAndRelu", "QuantizedConv2DAndRelu", "QuantizedConv2DAndRequantize",
                                     "QuantizedConv2DAndReluAndRequantize", "QuantizedConv2DWithBiasAndRequantize",
-                                    "QuantizedConv2DWithBiasAndReluAndRequantize"};
+                                    "QuantizedConv2DWithBiasAndReluAndRequantize",
+                                    "QuantizedConv2DWithBiasSumAndReluAndRequantize",
+                                    "QuantizedConv2DWithBiasSignedSumAndReluAndRequantize"};
 
 template <int NAME, bool NEW_API, int TIN, int TOUT>
 struct ConvKernel : QuantizedConv2DOp {
@@ -326,7 +382,7 @@ struct ConvKernel : QuantizedConv2DOp {
 };
 
 template <int NAME, int TIN, int TOUT>
-void RegLegacy(bool with_bias_types, std::initializer_list<const char*> host_args) {
+void RegLegacy(bool with_bias_types, std::initializer_list<const char*> host_args, int t_summand = 0) {
   for (const char* prefix : {"", "_ITEX"}) {
     const std::string op = std::string(prefix) + kLegacyNames[NAME];
     for (TF_DataType tb : {TF_FLOAT, TF_QINT32}) {
@@ -334,6 +390,7 @@ void RegLegacy(bool with_bias_types, std::initializer_list<const char*> host_arg
       KernelDefBuilder b(op.c_str(), "QuantizedConvOp");
       b.TypeConstraint("Tinput", static_cast<TF_DataType>(TIN)).TypeConstraint("Tfilter", TF_QINT8);
       if (with_bias_types) b.TypeConstraint("Tbias", tb);
+      if (t_summand != 0) b.TypeConstraint("Tsummand", static_cast<TF_DataType>(t_summand));
       b.TypeConstraint("out_type", static_cast<TF_DataType>(TOUT));
       for (const char* h : host_args) b.HostMemory(h);
       b.Register<ConvKernel<NAME, false, TIN, TOUT>>();
@@ -371,6 +428,10 @@ void AddQuantizedConvKernels() {
   RegLegacy<6, TF_QUINT8, TF_QUINT8>(false, req);
   RegLegacy<7, TF_QINT8, TF_QINT8>(true, req);      RegLegacy<7, TF_QUINT8, TF_QINT8>(true, req);
   RegLegacy<8, TF_QINT8, TF_QUINT8>(true, req);     RegLegacy<8, TF_QUINT8, TF_QUINT8>(true, req);
+  const std::initializer_list<const char*> sum = {"min_input", "max_input", "min_filter", "max_filter", "min_freezed_output",
+                                                  "max_freezed_output", "min_summand", "max_summand", "min_output", "max_output"};
+  RegLegacy<9, TF_QUINT8, TF_QUINT8>(true, sum, TF_QUINT8);
+  RegLegacy<10, TF_QUINT8, TF_QUINT8>(true, sum, TF_QINT8);
   RegNewApi<TF_QINT8, TF_QINT8>();   RegNewApi<TF_QUINT8, TF_QINT8>();
   RegNewApi<TF_QINT8, TF_QUINT8>();  RegNewApi<TF_QUINT8, TF_QUINT8>();
   RegNewApi<TF_QINT8, TF_FLOAT>();   RegNewApi<TF_QUINT8, TF_FLOAT>();

@@ -33,7 +33,10 @@
  *   reference tests' own tolerance;
  *   the bfloat16 / half bias (Tbias): the adjusted bias is rounded to Tbias as the code is
  *   written (quantized_matmul_common.h:578-599, 609-617); the reference's tests only use float and
- *   qint32 biases.  The bfloat16 / half OUTPUT is pinned: it must equal the nearest-even 16-bit
+ *   qint32 biases;
+ *   the quantized convolution's host arithmetic at the last bit and its Sum fusions (orc_qconv2d_sum): the
+ *   reference's conv tests hold no vectors, see the comments at those functions.
+ *   The bfloat16 / half OUTPUT is pinned: it must equal the nearest-even 16-bit
  *   value of the float output of the same node, which the tests check against PyTorch's conversion.
  */
 #ifndef ITEX_ORACLE_H_

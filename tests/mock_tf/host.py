@@ -27,7 +27,9 @@ def load(device="XPU", stock_ops=("QuantizeV2", "Dequantize", "QuantizedMatMulWi
                                    "RequantizationRangePerChannel", "QuantizedReshape", "MatMul", "Relu", "QuantizedConv2D",
                                    "QuantizedConv2DPerChannel", "QuantizedConv2DWithBias", "QuantizedConv2DWithBiasAndRelu",
                                    "QuantizedConv2DAndRelu", "QuantizedConv2DAndRequantize", "QuantizedConv2DAndReluAndRequantize",
-                                   "QuantizedConv2DWithBiasAndRequantize", "QuantizedConv2DWithBiasAndReluAndRequantize")):
+                                   "QuantizedConv2DWithBiasAndRequantize", "QuantizedConv2DWithBiasAndReluAndRequantize",
+                                   "QuantizedConv2DWithBiasSumAndReluAndRequantize",
+                                   "QuantizedConv2DWithBiasSignedSumAndReluAndRequantize")):
     """Loads the mock host and the plugin once per process; returns the mock's ctypes handle."""
     if "lib" in _state:
         return _state["lib"]

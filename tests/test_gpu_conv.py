@@ -355,6 +355,60 @@ def test_new_api_conv_through_plugin(rt, dev, t_in, fused, t_out, t_bias):
         node.close()
 
 
+@pytest.mark.parametrize("op,t_sum,fused", [
+    ("QuantizedConv2DWithBiasSumAndReluAndRequantize", tf.QUINT8, None),
+    ("QuantizedConv2DWithBiasSignedSumAndReluAndRequantize", tf.QINT8, None),
+    ("_QuantizedConv2D", tf.QUINT8, ["BiasAdd", "Sum", "Relu", "Requantize"]),
+    ("_QuantizedConv2D", tf.QINT8, ["BiasAdd", "Relu", "Sum", "Requantize"]),
+    ("_QuantizedConv2D", tf.QINT8, ["BiasAdd", "Sum", "LeakyRelu", "Requantize"])])
+def test_sum_fusions_through_plugin(rt, dev, op, t_sum, fused):
+    """The residual-add fusions of a ResNet block: conv + bias + sum (8-bit summand with its own range) + ReLU +
+    requantize, legacy spellings and fused_ops of the new API, implicit-GEMM and patch-matrix shapes; equal to the
+    oracle (which restates the reference's scale and type rules for the sum post-op)."""
+    torch = rt
+    new_api = fused is not None
+    t_out = tf.QINT8 if (new_api and "LeakyRelu" in fused) else tf.QUINT8
+    for shape, wshape in (((2, 9, 8, 16), (3, 3, 16, 32)), ((1, 7, 7, 6), (3, 3, 6, 16))):
+        rng = np.random.default_rng(shape[3] + t_sum + (len(fused) if fused else 0))
+        x = rng.uniform(0.0, 4.0, shape).astype(np.float32)
+        w = rng.uniform(-1.0, 1.0, wshape).astype(np.float32)
+        b = rng.uniform(-1.0, 1.0, wshape[3]).astype(np.float32)
+        xq, xmn, xmx, wq, fmn, fmx = quantize_inputs(x, w, tf.QUINT8)
+        oshape = (shape[0], shape[1], shape[2], wshape[3])
+        summand = (rng.integers(0, 256, oshape).astype(np.uint8) if t_sum == tf.QUINT8 else rng.integers(-128, 128, oshape).astype(np.int8))
+        smn, smx = np.array(0.0 if t_sum == tf.QUINT8 else -11.0, np.float32), np.array(14.0, np.float32)
+        zmn, zmx = np.array(-25.0 if t_out == tf.QINT8 else 0.0, np.float32), np.array(30.0, np.float32)
+        attrs = dict(Tinput=DT(tf.QUINT8), Tfilter=DT(tf.QINT8), Tbias=DT(tf.FLOAT), Tsummand=DT(t_sum), out_type=DT(t_out),
+                     strides=[1, 1, 1, 1], padding="SAME", dilations=[1, 1, 1, 1])
+        if new_api:
+            attrs.update(fused_ops=fused, alpha=0.25, data_format="NHWC", is_filter_const=True, is_bias_const=True)
+        node = tf.Node(op, attrs)
+        assert node.code == tf.OK, node.message
+        keep = [torch.from_numpy(np.ascontiguousarray(v)).to(dev) for v in (xq, wq, b, summand)]
+        dev_in = lambda i, dt, arr: (dt, arr.shape, keep[i].data_ptr(), False)
+        host = lambda v: (tf.FLOAT, v.shape, tf.host_array(v), True)
+        ins = [dev_in(0, tf.QUINT8, xq), dev_in(1, tf.QINT8, wq), dev_in(2, tf.FLOAT, b)]
+        if new_api:
+            ins += [dev_in(3, t_sum, summand)] + [host(v) for v in (xmn, xmx, fmn, fmx, smn, smx, zmn, zmx)]
+        else:
+            ins += [host(v) for v in (xmn, xmx, fmn, fmx, zmn, zmx)] + [dev_in(3, t_sum, summand), host(smn), host(smx)]
+        code, msg, res = node.run(ins, [(t_out, False), (tf.FLOAT, True), (tf.FLOAT, True)],
+                                  stream=torch.cuda.current_stream().cuda_stream)
+        assert code == tf.OK, msg
+        got = fetch(torch, res[0], NP[t_out])
+        leaky = new_api and "LeakyRelu" in fused
+        position = 2 if (new_api and fused.index("Sum") > 1 and not leaky and fused[1] == "Relu") else 1
+        at = orc.ConvAttrs(orc.QUINT8, t_out, orc.FLOAT, orc.ACT_LEAKYRELU if leaky else orc.ACT_RELU, 0.25)
+        g = orc.conv_geom(shape, wshape)
+        st, ref = orc.qconv2d(at, g, xq, wq, b, float(xmn), float(xmx), fmn, fmx, float(zmn), float(zmx),
+                              sum=orc.ConvSum(position, t_sum, float(smn), float(smx)), summand=summand)
+        assert st == orc.OK
+        np.testing.assert_array_equal(got, ref)
+        assert float(np.ravel(fetch(torch, res[1], np.float32))[0]) == float(zmn)
+        assert float(np.ravel(fetch(torch, res[2], np.float32))[0]) == float(zmx)
+        node.close()
+
+
 def test_unsupported_fusions_and_formats(rt, dev):
     base = dict(Tinput=DT(tf.QUINT8), Tfilter=DT(tf.QINT8), Tbias=DT(tf.FLOAT), out_type=DT(tf.FLOAT), strides=[1, 1, 1, 1],
                 padding="SAME", dilations=[1, 1, 1, 1], alpha=0.0)

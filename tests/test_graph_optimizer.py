@@ -110,7 +110,8 @@ def test_every_renamed_op_has_a_kernel_and_an_op_definition(opt):
            "_QuantizedFusedMatMul", "_QuantizedFusedMatMulAndDequantize", "_QuantizedFusedMatMulAndRequantize", "_QuantizedMatMul",
            "QuantizedReshape", "_QuantizedTranspose", "QuantizedConv2D", "QuantizedConv2DAndRequantize",
            "QuantizedConv2DPerChannel", "QuantizedConv2DWithBias", "QuantizedConv2DWithBiasAndRelu",
-           "QuantizedConv2DWithBiasAndReluAndRequantize", "QuantizedConv2DWithBiasAndRequantize"]
+           "QuantizedConv2DWithBiasAndReluAndRequantize", "QuantizedConv2DWithBiasAndRequantize",
+           "QuantizedConv2DWithBiasSumAndReluAndRequantize", "QuantizedConv2DWithBiasSignedSumAndReluAndRequantize"]
     g = gd.GraphDef()
     for i, op in enumerate(ops):
         gd.node(g, "n%d" % i, op, ["x"], DEV, mode="SCALED", T=("type", QINT8))

@@ -221,6 +221,14 @@ def test_conv_registrations(reg):
             assert all(k["constraints"]["Tfilter"] == tf.QINT8 and k["host_memory"] == host for k in ks), op
     for op in ("QuantizedConv2DWithBiasAndRequantize", "QuantizedConv2DWithBiasAndReluAndRequantize"):
         assert {k["constraints"]["Tbias"] for k in kernels_of(reg, op)} == {tf.FLOAT, tf.QINT32}
+    sum_host = req[:6] + ["min_summand", "max_summand", "min_output", "max_output"]
+    for name, t_sum in (("QuantizedConv2DWithBiasSumAndReluAndRequantize", tf.QUINT8),
+                        ("QuantizedConv2DWithBiasSignedSumAndReluAndRequantize", tf.QINT8)):
+        for op in (name, "_ITEX" + name):
+            ks = kernels_of(reg, op)
+            assert {k["constraints"]["Tbias"] for k in ks} == {tf.FLOAT, tf.QINT32}, op
+            assert all(k["constraints"]["Tinput"] == tf.QUINT8 and k["constraints"]["out_type"] == tf.QUINT8 and
+                       k["constraints"]["Tsummand"] == t_sum and k["host_memory"] == sum_host for k in ks), op
     for op in ("_QuantizedConv2D", "_ITEXQuantizedConv2DV2"):
         ks = kernels_of(reg, op)
         assert {k["constraints"]["out_type"] for k in ks} == {tf.QINT8, tf.QUINT8, tf.QINT32, tf.FLOAT, tf.BFLOAT16}
