@@ -1,5 +1,7 @@
 #include "graph_def.h"
 
+#include <algorithm>
+
 namespace itex_amd {
 namespace graph {
 namespace {
@@ -178,6 +180,87 @@ bool AttrType(const std::string& value, int* t) {
   if (!FindField(value, 6, 0, &at)) return false;
   *t = static_cast<int>(at.Varint());
   return at.ok;
+}
+
+bool AttrInt(const std::string& value, int* i) {
+  Reader at{nullptr, nullptr};
+  if (!FindField(value, 3, 0, &at)) { *i = 0; return value.empty(); }  // proto3 omits a zero
+  *i = static_cast<int>(static_cast<int64_t>(at.Varint()));
+  return at.ok;
+}
+
+bool AttrIntTensor(const std::string& value, int* rank, std::vector<int64_t>* elements) {
+  Reader at{nullptr, nullptr};
+  if (!FindField(value, 8, 2, &at)) return false;
+  const auto body = at.Bytes();
+  if (!at.ok) return false;
+  Reader r{body.first, body.first + body.second};
+  int dtype = 0;
+  std::vector<int64_t> dims, vals;
+  std::string content;
+  while (!r.done()) {
+    const uint64_t tag = r.Varint();
+    if (!r.ok) return false;
+    const uint32_t field = static_cast<uint32_t>(tag >> 3), wire = static_cast<uint32_t>(tag & 7);
+    if (field == 1 && wire == 0) {
+      dtype = static_cast<int>(r.Varint());
+    } else if (field == 2 && wire == 2) {  // TensorShapeProto: repeated Dim dim = 2 { int64 size = 1 }
+      const auto sb = r.Bytes();
+      Reader sr{sb.first, sb.first + sb.second};
+      while (!sr.done()) {
+        const uint64_t st = sr.Varint();
+        if (!sr.ok) return false;
+        if ((st >> 3) == 2 && (st & 7) == 2) {
+          const auto db = sr.Bytes();
+          Reader dr{db.first, db.first + db.second};
+          int64_t size = 0;
+          while (!dr.done()) {
+            const uint64_t dt = dr.Varint();
+            if (!dr.ok) return false;
+            if ((dt >> 3) == 1 && (dt & 7) == 0) size = static_cast<int64_t>(dr.Varint());
+            else if (!dr.Skip(static_cast<uint32_t>(dt & 7))) return false;
+          }
+          dims.push_back(size);
+        } else if (!sr.Skip(static_cast<uint32_t>(st & 7))) {
+          return false;
+        }
+      }
+    } else if (field == 4 && wire == 2) {
+      content = Str(r.Bytes());
+    } else if ((field == 7 || field == 10) && wire == 0) {
+      vals.push_back(static_cast<int64_t>(r.Varint()));
+    } else if ((field == 7 || field == 10) && wire == 2) {  // packed
+      const auto pb = r.Bytes();
+      Reader pr{pb.first, pb.first + pb.second};
+      while (!pr.done()) vals.push_back(static_cast<int64_t>(pr.Varint()));
+      if (!pr.ok) return false;
+    } else if (!r.Skip(wire)) {
+      return false;
+    }
+  }
+  if (!r.ok || (dtype != 3 && dtype != 9)) return false;  // DT_INT32, DT_INT64
+  int64_t count = 1;
+  for (int64_t d : dims) {
+    if (d < 0 || d > (1 << 20)) return false;
+    count *= d;
+    if (count > (1 << 20)) return false;
+  }
+  elements->clear();
+  if (!content.empty()) {
+    const size_t esz = dtype == 3 ? 4 : 8;
+    if (content.size() != esz * static_cast<size_t>(count)) return false;
+    for (int64_t i = 0; i < count; ++i) {
+      uint64_t raw = 0;
+      for (size_t b = 0; b < esz; ++b) raw |= static_cast<uint64_t>(static_cast<uint8_t>(content[i * esz + b])) << (8 * b);
+      elements->push_back(dtype == 3 ? static_cast<int64_t>(static_cast<int32_t>(raw)) : static_cast<int64_t>(raw));
+    }
+  } else {
+    if (dtype == 3) for (int64_t& v : vals) v = static_cast<int64_t>(static_cast<int32_t>(v));  // negative int32 arrive sign-extended to 64 bits
+    for (int64_t i = 0; i < count; ++i)  // fewer values than elements: the last one repeats (tensor.proto)
+      elements->push_back(vals.empty() ? 0 : vals[std::min<size_t>(i, vals.size() - 1)]);
+  }
+  *rank = static_cast<int>(dims.size());
+  return true;
 }
 
 std::string MakeAttrBool(bool b) {

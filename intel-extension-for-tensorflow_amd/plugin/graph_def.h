@@ -36,10 +36,14 @@ struct Graph {
 bool Parse(const void* data, size_t len, Graph* g);
 std::string Serialize(const Graph& g);
 
-// AttrValue accessors for the kinds the rewrite reads and writes (attr_value.proto: s = 2, b = 5, type = 6)
+// AttrValue accessors for the kinds the rewrite reads and writes (attr_value.proto: s = 2, b = 5, type = 6, tensor = 8)
 bool AttrString(const std::string& value, std::string* s);
 bool AttrBool(const std::string& value, bool* b);
 bool AttrType(const std::string& value, int* t);
+bool AttrInt(const std::string& value, int* i);  // i = 3
+// The integer tensor of a Const node's "value" attribute (AttrValue.tensor = 8; tensor.proto: dtype = 1,
+// tensor_shape = 2, tensor_content = 4, int_val = 7, int64_val = 10), int32 or int64: its rank and elements.
+bool AttrIntTensor(const std::string& value, int* rank, std::vector<int64_t>* elements);
 std::string MakeAttrBool(bool b);
 std::string MakeAttrString(const std::string& s);
 std::string MakeAttrType(int t);

@@ -95,6 +95,71 @@ bool RewriteQuantize(const graph::Node& n) {
   return true;
 }
 
+// "name" and "name:0" name the same tensor
+std::string Canonical(const std::string& in) {
+  std::string name;
+  int port = 0;
+  if (!SplitInput(in, &name, &port)) return in;
+  return name + ":" + std::to_string(port);
+}
+
+std::vector<std::string> DataInputs(const graph::Node& n) {
+  std::vector<std::string> v;
+  for (const std::string& in : n.inputs)
+    if (!in.empty() && in[0] != '^') v.push_back(in);
+  return v;
+}
+
+// QuantizeV2(x, Min(Reshape(x, [-1]), 0), Max(Reshape(x, [-1]), 0)): the per-tensor dynamic-range quantization that
+// TensorFlow's graph quantization tools emit.  Without Min / Max kernels for this device TensorFlow would place the
+// two reductions on the CPU and copy the whole float tensor to the host for them; the fused op computes the range on
+// the device.  The reference has no such fusion for QuantizeV2 (its remapper fuses QuantizeV2 into convolutions only,
+// itex/core/graph/remapper/remapper.cc:2099-2114).  Returns true when node q matches.
+bool MatchDynamicRange(const graph::Node& q, const std::map<std::string, const graph::Node*>& by_name) {
+  int axis = -1;
+  const std::string* a = q.FindAttr("axis");
+  if (a && !a->empty() && !graph::AttrInt(*a, &axis)) return false;
+  if (axis != -1) return false;
+  const std::vector<std::string> in = DataInputs(q);
+  if (in.size() != 3) return false;
+  auto node_of = [&](const std::string& input, int want_port) -> const graph::Node* {
+    std::string name;
+    int port = 0;
+    if (!SplitInput(input, &name, &port) || port != want_port) return nullptr;
+    const auto it = by_name.find(name);
+    return it == by_name.end() ? nullptr : it->second;
+  };
+  auto const_ints = [&](const std::string& input, int* rank, std::vector<int64_t>* vals) {
+    const graph::Node* c = node_of(input, 0);
+    if (!c || c->op != "Const") return false;
+    const std::string* v = c->FindAttr("value");
+    return v && graph::AttrIntTensor(*v, rank, vals);
+  };
+  const graph::Node* mn = node_of(in[1], 0);
+  const graph::Node* mx = node_of(in[2], 0);
+  if (!mn || !mx || mn->op != "Min" || mx->op != "Max") return false;
+  std::string reduced;
+  for (const graph::Node* red : {mn, mx}) {
+    bool keep = false;
+    const std::string* k = red->FindAttr("keep_dims");
+    if (k && (!graph::AttrBool(*k, &keep) || keep)) return false;
+    const std::vector<std::string> rin = DataInputs(*red);
+    if (rin.size() != 2) return false;
+    int rank = 0;
+    std::vector<int64_t> idx;
+    if (!const_ints(rin[1], &rank, &idx) || rank > 1 || idx.size() != 1 || idx[0] != 0) return false;  // reduce dimension 0
+    if (reduced.empty()) reduced = Canonical(rin[0]);
+    else if (reduced != Canonical(rin[0])) return false;
+  }
+  const graph::Node* flat = node_of(reduced, 0);  // of a tensor flattened to one dimension
+  if (!flat || flat->op != "Reshape") return false;
+  const std::vector<std::string> fin = DataInputs(*flat);
+  if (fin.size() != 2 || Canonical(fin[0]) != Canonical(in[0])) return false;
+  int rank = 0;
+  std::vector<int64_t> shape;
+  return const_ints(fin[1], &rank, &shape) && rank == 1 && shape.size() == 1 && shape[0] == -1;
+}
+
 struct Optimizer {
   std::string device_type;
 };
@@ -122,9 +187,13 @@ void Optimize(void* opt, const TF_Buffer* in, const TF_GrapplerItem*, TF_Buffer*
       int port = 0;
       if (SplitInput(in_name, &producer, &port) && port == 0) fanout0[producer].push_back(&n);
     }
+  std::map<std::string, const graph::Node*> by_name;
+  for (const graph::Node& n : g.nodes) by_name[n.name] = &n;
+  const char* dsw = std::getenv("ITEX_AMD_FUSE_DYNAMIC_RANGE");
+  const bool fuse_dynamic = !(dsw && std::strcmp(dsw, "0") == 0);
   // decisions first, on the unmodified graph: a QuantizeV2's consumers are looked up by their original op
   std::vector<const Rename*> plan(g.nodes.size(), nullptr);
-  std::vector<bool> classic(g.nodes.size(), false);
+  std::vector<bool> classic(g.nodes.size(), false), dynamic(g.nodes.size(), false);
   for (size_t i = 0; enabled && i < g.nodes.size(); ++i) {
     const graph::Node& n = g.nodes[i];
     // NodeIsOnDevice (utils.cc:262-265): the node carries a device string naming this device type
@@ -143,6 +212,7 @@ void Optimize(void* opt, const TF_Buffer* in, const TF_GrapplerItem*, TF_Buffer*
         bool all_dequantize = true;
         for (const graph::Node* c : fanout0[n.name]) all_dequantize = all_dequantize && c->op == "Dequantize";
         classic[i] = all_dequantize;
+        dynamic[i] = fuse_dynamic && n.op == "QuantizeV2" && MatchDynamicRange(n, by_name);
       }
       break;
     }
@@ -154,6 +224,14 @@ void Optimize(void* opt, const TF_Buffer* in, const TF_GrapplerItem*, TF_Buffer*
     if (plan[i]->copy == Copy::kQuantize) {
       if (!n.FindAttr("dtype")) n.SetAttr("dtype", graph::MakeAttrType(kDtFloat));
       n.SetAttr("classic_asymmetric_algorithm", graph::MakeAttrBool(classic[i]));
+      if (dynamic[i]) {  // the range inputs go; Min, Max and Reshape stay for whoever else reads them (else they are pruned)
+        n.op = "_ITEXQuantizeV2DynamicRange";
+        std::vector<std::string> kept;
+        int data = 0;
+        for (const std::string& in_name : n.inputs)
+          if ((!in_name.empty() && in_name[0] == '^') || data++ == 0) kept.push_back(in_name);
+        n.inputs = kept;
+      }
     }
     if (plan[i]->copy == Copy::kQuantizedConv2D) n.SetAttr("data_format", graph::MakeAttrString("NHWC"));  // :471-495
     // CopyAttrsQuantizedMatMul (:497-515) copies every attribute and then Tbias once more: nothing to add

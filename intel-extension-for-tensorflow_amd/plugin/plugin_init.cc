@@ -85,6 +85,14 @@ std::vector<OpSpec> OpSpecs() {
                 "round_mode: {'HALF_AWAY_FROM_ZERO', 'HALF_TO_EVEN'} = 'HALF_AWAY_FROM_ZERO'",
                 "narrow_range: bool = false", "axis: int = -1", "ensure_minimum_range: float = 0.01",
                 "dtype: {bfloat16, float} = DT_FLOAT", "classic_asymmetric_algorithm: bool = false"}});
+  // made by this plugin's graph pass from QuantizeV2 fed by Min / Max of its own input: no range inputs
+  v.push_back({"_ITEXQuantizeV2DynamicRange",
+               {"input: dtype"},
+               {"output: T", "output_min: float", "output_max: float"},
+               {"T: quantizedtype", "mode: {'MIN_COMBINED', 'MIN_FIRST', 'SCALED'} = 'SCALED'",
+                "round_mode: {'HALF_AWAY_FROM_ZERO', 'HALF_TO_EVEN'} = 'HALF_AWAY_FROM_ZERO'",
+                "narrow_range: bool = false", "axis: int = -1", "ensure_minimum_range: float = 0.01",
+                "dtype: {float} = DT_FLOAT", "classic_asymmetric_algorithm: bool = false"}});
   v.push_back({"_ITEXDequantize",
                {"input: T", "min_range: float", "max_range: float"},
                {"output: dtype"},

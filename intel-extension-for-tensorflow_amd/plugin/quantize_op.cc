@@ -17,7 +17,10 @@ using qparams::Mode;
 
 class QuantizeV2Op : public OpKernel {
  public:
-  QuantizeV2Op(OpKernelConstruction* ctx, TF_DataType T) : T_(T) {
+  // dynamic: the op has no min_range / max_range inputs and takes the range of its input tensor, computed on the device
+  // (what the graph pass makes of Reshape -> Min / Max -> QuantizeV2; no counterpart in the reference, whose QuantizeV2
+  // always receives the range from other ops)
+  QuantizeV2Op(OpKernelConstruction* ctx, TF_DataType T, bool dynamic = false) : T_(T), dynamic_(dynamic) {
     std::string mode_string;
     ITEX_REQUIRES_OK(ctx, ctx->GetAttr("mode", &mode_string));
     if (ctx->HasAttr("classic_asymmetric_algorithm")) {
@@ -54,10 +57,29 @@ class QuantizeV2Op : public OpKernel {
 
   void Compute(OpKernelContext* ctx) override {
     Tensor src = ctx->input(0);
-    Tensor in_min = ctx->input(1);
-    Tensor in_max = ctx->input(2);
     if (!ctx->ok()) return;
     ITEX_REQUIRES(ctx, src.dtype() == src_type_, TF_INVALID_ARGUMENT, "QuantizeV2 input type does not match the kernel");
+    Tensor in_min, in_max;
+    if (dynamic_) {
+      ITEX_REQUIRES(ctx, axis_ == -1 && src_type_ == TF_FLOAT, TF_INVALID_ARGUMENT,
+                    "the dynamic-range QuantizeV2 quantizes a float tensor per tensor");
+      in_min = ctx->allocate_temp(TF_FLOAT, {}, /*on_host=*/true);
+      in_max = ctx->allocate_temp(TF_FLOAT, {}, /*on_host=*/true);
+      Tensor range = ctx->allocate_temp(TF_FLOAT, {2});
+      if (!ctx->ok()) return;
+      float host_range[2] = {0.0f, 0.0f};  // the range of an empty tensor, as Min / Max give no usable value there
+      if (src.NumElements() > 0) {
+        int st = itexhip_minmax_f32(src.flat<float>(), src.NumElements(), range.flat<float>(), ctx->stream());
+        if (st == ITEXHIP_OK) st = itexhip_memcpy_d2h(host_range, range.data(), sizeof(host_range), ctx->stream());
+        ITEX_REQUIRES(ctx, st == ITEXHIP_OK, TF_ABORTED, std::string("Operation received an exception: ") + itexhip_last_error());
+      }
+      in_min.flat<float>()[0] = host_range[0];
+      in_max.flat<float>()[0] = host_range[1];
+    } else {
+      in_min = ctx->input(1);
+      in_max = ctx->input(2);
+      if (!ctx->ok()) return;
+    }
 
     const int64_t num_slices = (axis_ > -1) ? in_min.NumElements() : 1;
     ITEX_REQUIRES(ctx, in_min.NumElements() >= 1 && in_max.NumElements() >= num_slices, TF_INVALID_ARGUMENT,
@@ -94,8 +116,8 @@ class QuantizeV2Op : public OpKernel {
 
     Tensor dst = ctx->allocate_output(0, T_, shape);
     const std::vector<int64_t> mm_shape = (num_slices == 1) ? std::vector<int64_t>{} : in_min.shape();
-    Tensor out_min = ctx->forward_input_or_allocate_output(1, 1, mm_shape, TF_FLOAT);
-    Tensor out_max = ctx->forward_input_or_allocate_output(2, 2, mm_shape, TF_FLOAT);
+    Tensor out_min = dynamic_ ? ctx->allocate_output(1, TF_FLOAT, mm_shape) : ctx->forward_input_or_allocate_output(1, 1, mm_shape, TF_FLOAT);
+    Tensor out_max = dynamic_ ? ctx->allocate_output(2, TF_FLOAT, mm_shape) : ctx->forward_input_or_allocate_output(2, 2, mm_shape, TF_FLOAT);
     if (!ctx->ok()) return;
 
     int st;
@@ -131,6 +153,7 @@ class QuantizeV2Op : public OpKernel {
 
  private:
   TF_DataType T_;
+  bool dynamic_ = false;
   TF_DataType src_type_ = TF_FLOAT;
   Mode mode_ = Mode::SCALED;
   bool classic_ = false;
@@ -142,6 +165,8 @@ class QuantizeV2Op : public OpKernel {
 
 struct QuantizeQint8 : QuantizeV2Op { explicit QuantizeQint8(OpKernelConstruction* c) : QuantizeV2Op(c, TF_QINT8) {} };
 struct QuantizeQuint8 : QuantizeV2Op { explicit QuantizeQuint8(OpKernelConstruction* c) : QuantizeV2Op(c, TF_QUINT8) {} };
+struct DynQuantizeQint8 : QuantizeV2Op { explicit DynQuantizeQint8(OpKernelConstruction* c) : QuantizeV2Op(c, TF_QINT8, true) {} };
+struct DynQuantizeQuint8 : QuantizeV2Op { explicit DynQuantizeQuint8(OpKernelConstruction* c) : QuantizeV2Op(c, TF_QUINT8, true) {} };
 
 }  // namespace
 
@@ -170,6 +195,13 @@ void AddQuantizeKernels() {
   bu8.TypeConstraint("T", TF_QUINT8).TypeConstraint("dtype", TF_BFLOAT16);
   bu8.HostMemory("min_range").HostMemory("max_range").HostMemory("output_min").HostMemory("output_max");
   bu8.Register<QuantizeQuint8>();
+  // the dynamic-range form made by this plugin's graph pass
+  KernelDefBuilder ds8("_ITEXQuantizeV2DynamicRange", "QuantizeV2Op");
+  ds8.TypeConstraint("T", TF_QINT8).TypeConstraint("dtype", TF_FLOAT).HostMemory("output_min").HostMemory("output_max");
+  ds8.Register<DynQuantizeQint8>();
+  KernelDefBuilder du8("_ITEXQuantizeV2DynamicRange", "QuantizeV2Op");
+  du8.TypeConstraint("T", TF_QUINT8).TypeConstraint("dtype", TF_FLOAT).HostMemory("output_min").HostMemory("output_max");
+  du8.Register<DynQuantizeQuint8>();
 }
 
 }  // namespace itex_amd

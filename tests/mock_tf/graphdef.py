@@ -20,12 +20,34 @@ def _build():
         f = lst.field.add()
         f.name, f.number, f.type, f.label = name, num, typ, _F.LABEL_REPEATED
 
+    # tensor.proto / tensor_shape.proto: what a Const node's "value" needs
+    shp = fd.message_type.add()
+    shp.name = "TensorShapeProto"
+    dim = shp.nested_type.add()
+    dim.name = "Dim"
+    f = dim.field.add()
+    f.name, f.number, f.type, f.label = "size", 1, _F.TYPE_INT64, _F.LABEL_OPTIONAL
+    f = shp.field.add()
+    f.name, f.number, f.type, f.label, f.type_name = "dim", 2, _F.TYPE_MESSAGE, _F.LABEL_REPEATED, ".tensorflow_subset.TensorShapeProto.Dim"
+    tp = fd.message_type.add()
+    tp.name = "TensorProto"
+    for name, num, typ, label, tn in (("dtype", 1, _F.TYPE_INT32, _F.LABEL_OPTIONAL, None),
+                                      ("tensor_shape", 2, _F.TYPE_MESSAGE, _F.LABEL_OPTIONAL, ".tensorflow_subset.TensorShapeProto"),
+                                      ("tensor_content", 4, _F.TYPE_BYTES, _F.LABEL_OPTIONAL, None),
+                                      ("int_val", 7, _F.TYPE_INT32, _F.LABEL_REPEATED, None),
+                                      ("int64_val", 10, _F.TYPE_INT64, _F.LABEL_REPEATED, None)):
+        f = tp.field.add()
+        f.name, f.number, f.type, f.label = name, num, typ, label
+        if tn:
+            f.type_name = tn
+
     av = fd.message_type.add()
     av.name = "AttrValue"
     av.oneof_decl.add().name = "value"
     for name, num, typ, tn in (("s", 2, _F.TYPE_BYTES, None), ("i", 3, _F.TYPE_INT64, None), ("f", 4, _F.TYPE_FLOAT, None),
                                ("b", 5, _F.TYPE_BOOL, None), ("type", 6, _F.TYPE_INT32, None),
-                               ("list", 1, _F.TYPE_MESSAGE, ".tensorflow_subset.ListValue")):
+                               ("list", 1, _F.TYPE_MESSAGE, ".tensorflow_subset.ListValue"),
+                               ("tensor", 8, _F.TYPE_MESSAGE, ".tensorflow_subset.TensorProto")):
         f = av.field.add()
         f.name, f.number, f.type, f.label = name, num, typ, _F.LABEL_OPTIONAL
         f.oneof_index = 0
@@ -78,7 +100,7 @@ GraphDef, NodeDef, AttrValue = _M["GraphDef"], _M["NodeDef"], _M["AttrValue"]
 
 def node(graph, name, op, inputs=(), device="", **attrs):
     """Adds a node; attribute values: str -> s, bool -> b, int -> i, float -> f, ("type", n) -> type,
-    list of str -> list.s"""
+    list of str -> list.s, ("tensor", dtype, shape, values, as_content) -> an int32 (3) / int64 (9) tensor"""
     n = graph.node.add()
     n.name, n.op, n.device = name, op, device
     n.input.extend(inputs)
@@ -96,6 +118,18 @@ def node(graph, name, op, inputs=(), device="", **attrs):
             a.type = v[1]
         elif isinstance(v, list):
             a.list.s.extend(x.encode() for x in v)
+        elif isinstance(v, tuple) and v[0] == "tensor":     # ("tensor", dtype, shape, values, as_content)
+            _, dtype, shape, values, as_content = v
+            a.tensor.dtype = dtype
+            for d in shape:
+                a.tensor.tensor_shape.dim.add().size = d
+            if as_content:
+                import struct
+                a.tensor.tensor_content = b"".join(struct.pack("<i" if dtype == 3 else "<q", x) for x in values)
+            elif dtype == 3:
+                a.tensor.int_val.extend(values)
+            else:
+                a.tensor.int64_val.extend(values)
         else:
             raise TypeError(k)
     return n

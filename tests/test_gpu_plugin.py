@@ -113,6 +113,33 @@ def test_quantize_outputs_and_forwarding(rt, dev, forward):
         assert fwd == (-1, -1) and mn_h == np.float32(0.5)
 
 
+@pytest.mark.parametrize("T,mode,classic", [(tf.QUINT8, "MIN_FIRST", False), (tf.QUINT8, "MIN_FIRST", True), (tf.QINT8, "SCALED", False),
+                                            (tf.QUINT8, "SCALED", False)])
+def test_dynamic_range_quantize_through_plugin(rt, dev, T, mode, classic):
+    """_ITEXQuantizeV2DynamicRange (what the graph pass makes of Min / Max -> QuantizeV2): the range is the tensor's own,
+    found on the device; output and output_min / output_max equal QuantizeV2 fed with numpy's min and max."""
+    torch = rt
+    rng = np.random.default_rng(11)
+    for n, shift in ((70001, 0.3), (5, -2.0), (1, 1.5)):
+        x = (rng.standard_normal(n) * 3 + shift).astype(np.float32)
+        node = tf.Node("_ITEXQuantizeV2DynamicRange",
+                       dict(T=DT(T), mode=mode, round_mode="HALF_TO_EVEN" if mode == "SCALED" else "HALF_AWAY_FROM_ZERO",
+                            narrow_range=False, axis=-1, ensure_minimum_range=0.01, dtype=DT(tf.FLOAT),
+                            classic_asymmetric_algorithm=classic))
+        assert node.code == tf.OK, node.message
+        x_d = dev_in(torch, dev, x)
+        code, msg, outs = node.run([(tf.FLOAT, x.shape, x_d.data_ptr(), False)], [(T, False), (tf.FLOAT, True), (tf.FLOAT, True)],
+                                   stream=torch.cuda.current_stream().cuda_stream)
+        assert code == tf.OK, msg
+        q = fetch(torch, outs[0], tf.NP_OF[T])
+        omode = orc.SCALED if mode == "SCALED" else orc.MIN_FIRST
+        _, q_ref, omn_ref, omx_ref = orc.quantize_v2(x, x.min(), x.max(), T, omode, classic=classic)
+        np.testing.assert_array_equal(q, q_ref)
+        assert float(np.ravel(fetch(torch, outs[1], np.float32))[0]) == omn_ref[0]
+        assert float(np.ravel(fetch(torch, outs[2], np.float32))[0]) == omx_ref[0]
+        node.close()
+
+
 def test_dequantize_through_plugin(rt, dev):
     torch = rt
     rng = np.random.default_rng(1)

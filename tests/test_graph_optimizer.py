@@ -137,6 +137,58 @@ def test_conv_rows(opt):
     assert out["c3"].op == "QuantizedConv2D" and "data_format" not in out["c3"].attr
 
 
+def dynamic_range_graph(shape_vals=(-1,), shape_dims=(1,), axis_vals=(0,), axis_dims=(), keep_dims=False, q_axis=-1,
+                        max_src="flat", as_content=False, dtype=3, q_device=DEV):
+    g = gd.GraphDef()
+    gd.node(g, "x", "Placeholder", [], DEV)
+    gd.node(g, "other", "Placeholder", [], DEV)
+    gd.node(g, "shape", "Const", [], CPU, value=("tensor", dtype, shape_dims, list(shape_vals), as_content))
+    gd.node(g, "axis", "Const", [], CPU, value=("tensor", dtype, axis_dims, list(axis_vals), as_content))
+    gd.node(g, "flat", "Reshape", ["x", "shape"], DEV)
+    gd.node(g, "flat2", "Reshape", ["other", "shape"], DEV)
+    gd.node(g, "mn", "Min", ["flat:0", "axis"], DEV, keep_dims=keep_dims)
+    gd.node(g, "mx", "Max", [max_src, "axis"], DEV, keep_dims=keep_dims)
+    gd.node(g, "q", "QuantizeV2", ["x:0", "mn", "mx", "^flat"], q_device, T=("type", QUINT8), mode="MIN_FIRST",
+            round_mode="HALF_AWAY_FROM_ZERO", axis=q_axis)
+    gd.node(g, "mm", "_QuantizedMatMul", ["q", "w", "q:1", "q:2"], DEV)
+    return g
+
+
+@pytest.mark.parametrize("as_content,dtype", [(False, 3), (True, 3), (False, 9), (True, 9)])
+def test_min_max_feeding_quantize_become_a_dynamic_range_quantize(opt, as_content, dtype):
+    """QuantizeV2(x, Min(Reshape(x, [-1]), 0), Max(same, 0)) -> _ITEXQuantizeV2DynamicRange(x): the range is computed on
+    the device by the op; the range inputs go, control inputs stay, attributes as for _ITEXQuantizeV2."""
+    out = by_name(run(opt, dynamic_range_graph(as_content=as_content, dtype=dtype)))
+    q = out["q"]
+    assert q.op == "_ITEXQuantizeV2DynamicRange" and list(q.input) == ["x:0", "^flat"]
+    assert q.attr["mode"].s == b"MIN_FIRST" and q.attr["dtype"].type == FLOAT and q.attr["T"].type == QUINT8
+    assert q.attr["classic_asymmetric_algorithm"].b is False        # its consumer is a MatMul, not a Dequantize
+    assert out["mn"].op == "Min" and out["mx"].op == "Max" and out["flat"].op == "Reshape"   # left for other readers / pruning
+    reg = tf.registry()
+    assert "_ITEXQuantizeV2DynamicRange" in {k["op"] for k in reg["kernels"]}
+    assert "_ITEXQuantizeV2DynamicRange" in {o["name"] for o in reg["ops"]}
+
+
+@pytest.mark.parametrize("kw", [dict(shape_vals=(2, -1), shape_dims=(2,)),      # not flattened to one dimension
+                                dict(axis_vals=(1,)),                          # another reduction index
+                                dict(axis_vals=(0, 1), axis_dims=(2,)),
+                                dict(keep_dims=True),
+                                dict(q_axis=0),                                # per-channel quantization
+                                dict(max_src="flat2")],                        # Max of another tensor
+                         ids=["shape", "axis", "two_axes", "keep_dims", "per_channel", "other_tensor"])
+def test_dynamic_range_patterns_that_do_not_match(opt, kw):
+    out = by_name(run(opt, dynamic_range_graph(**kw)))
+    assert out["q"].op == "_ITEXQuantizeV2" and list(out["q"].input) == ["x:0", "mn", "mx", "^flat"]
+
+
+def test_dynamic_range_switch_and_placement(opt, monkeypatch):
+    out = by_name(run(opt, dynamic_range_graph(q_device=CPU)))
+    assert out["q"].op == "QuantizeV2"
+    monkeypatch.setenv("ITEX_AMD_FUSE_DYNAMIC_RANGE", "0")
+    out = by_name(run(opt, dynamic_range_graph()))
+    assert out["q"].op == "_ITEXQuantizeV2" and len(out["q"].input) == 4
+
+
 def test_reshape_is_only_renamed_for_qint8(opt):
     g = gd.GraphDef()
     gd.node(g, "a", "QuantizedReshape", ["x", "s", "mn", "mx"], DEV, T=("type", QINT8))
