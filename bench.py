@@ -341,6 +341,26 @@ def bench_conv(torch, hip, timer, steps, warmup, dev):
                         frac=t_roof / (ms * 1e-3), tops=ops / (ms * 1e-3) / 1e12, gbs=nbytes / (ms * 1e-3) / 1e9,
                         note="implicit GEMM, one launch" if implicit else "im2col + GEMM launches" if patches else "GEMM launch only"))
         del x, w, packed, y, cols
+    # depthwise 3x3 (MobileNet shapes): no matrix product, bound by input + output bytes
+    for name, (B, H, W, C) in (("dwconv3x3_112x112x32", (32, 112, 112, 32)), ("dwconv3x3_56x56x128", (32, 56, 56, 128))):
+        x = torch.randint(0, 256, (B, H, W, C), dtype=torch.uint8, device=dev, generator=g_)
+        w = torch.randint(-127, 128, (3, 3, C, 1), dtype=torch.int8, device=dev, generator=g_)
+        scales = torch.full((C,), 2e-3, dtype=torch.float32, device=dev)
+        bias = torch.zeros(C, dtype=torch.float32, device=dev)
+        ep = hip.Epilogue()
+        ep.n_scales, ep.n_eltwise = C, 1
+        ep.elt[0].alg, ep.elt[0].alpha, ep.elt[0].beta = hip.ELT_RELU, 0.0, 0.0
+        y = torch.empty((B * H * W, C), dtype=torch.uint8, device=dev)
+        geo = hip.ConvGeometry(B, H, W, C, 3, 3, H, W, 1, 1, 1, 1, 1, 1)
+
+        def make_dw(stream):
+            return lambda i: hip.qdepthwise_conv2d(x, hip.QUINT8, geo, 1, w, scales, bias, ep, hip.QUINT8, y, stream)
+        ms = timer.run_graph(make_dw, steps, warmup)
+        nbytes = x.numel() + w.numel() + y.numel()
+        out.append(dict(name=name, M=B * H * W, K=9, N=C, us_kernel=ms * 1e3, bytes=nbytes, ops=2 * 9 * y.numel(), bound="hbm",
+                        frac=nbytes / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS, tops=2 * 9 * y.numel() / (ms * 1e-3) / 1e12,
+                        gbs=nbytes / (ms * 1e-3) / 1e9, note="depthwise kernel, one launch"))
+        del x, w, y
     return out
 
 

@@ -371,6 +371,15 @@ int itexhip_im2col8(const void* x, const itexhip_conv_geometry* g, int64_t row_b
 int itexhip_scale_vector(const void* bias, int bias_type, const float* factors, int64_t n_factors, int64_t n,
                          float* out, void* stream);
 
+/* Depthwise Conv2D (QuantizedDepthwiseConv2D*, _QuantizedDepthwiseConv2D; the reference runs them as a grouped oneDNN
+ * convolution with one group per input channel, conv_ops.h:238-246, 395-397): `filter` is TensorFlow's
+ * [k_h, k_w, in_c, multiplier] qint8 tensor as it is, output channel c * multiplier + m reads input channel c; scales
+ * (0, 1 or in_c * multiplier of them), bias (fp32, may be null) and post-ops as in itexhip_qgemm, without a sum.
+ * Zero points are 0 (SCALED quantization): padding contributes nothing. */
+int itexhip_qdepthwise_conv2d(const void* x, int x_type, const itexhip_conv_geometry* g, int64_t multiplier,
+                              const int8_t* filter, const float* scales, const float* bias,
+                              const itexhip_epilogue* ep, int out_type, void* out, void* stream);
+
 /* The convolution without the patch matrix: the MatMul tile kernel gathers its activation tiles straight from the
  * NHWC input (an implicit GEMM; it stands where the reference executes its oneDNN
  * convolution primitive, conv_ops.h:1021, 1119), same arguments otherwise as itexhip_qgemm with M = batch * out_h * out_w and

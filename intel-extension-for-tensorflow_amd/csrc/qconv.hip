@@ -104,10 +104,292 @@ __global__ __launch_bounds__(256) void scale_vector_kernel(const void* __restric
   out[j] = b * factors[n_factors == 1 ? 0 : j];
 }
 
+// ------------------------------------------------------------------------------------------------
+// Depthwise Conv2D: out[b, oh, ow, c * mult + m] = sum over the window of x[b, ih, iw, c] * w[kh, kw, c, m], exact in
+// int32, then the MatMul's fp32 epilogue (scale per output channel, bias, post-ops, saturate + round).  No matrix
+// product in it (each output channel reads one input channel), so it runs on the vector ALU: one thread per output
+// position and group of 4 consecutive output channels; with mult == 1 those are 4 consecutive input channels, i.e.
+// one dword of x and one dword of w per window tap.  Memory bound in principle (input + output bytes).
+// ------------------------------------------------------------------------------------------------
+struct DepthwiseArgs {
+  int in_h, in_w, in_c, k_h, k_w, out_h, out_w, stride_h, stride_w, dil_h, dil_w, pad_top, pad_left;
+  int mult, out_c, groups4;  // groups of 4 output channels per position
+  int x_signed, vec;         // vec: mult == 1, in_c % 4 == 0, x and w 4-byte aligned
+  int n_scales, n_eltwise;
+  itexhip_eltwise elt[3];
+  int64_t total;             // positions * groups4
+  // the post-op chain as [ReLU | LeakyReLU | clip] [linear map] when it has that form (3x3 kernel): applied under
+  // uniform branches; a loop over the chain with a switch per value costs more instruction fetch than arithmetic
+  int chain;                 // bit 0 max(x, 0), 1 leaky, 2 clip, 3 linear
+  float alpha, lo, hi, lin_a, lin_b;
+};
+
+template <int OUT_T>
+__global__ __launch_bounds__(256) void qdwconv_kernel(const DepthwiseArgs a, const uint8_t* __restrict__ x,
+                                                      const int8_t* __restrict__ w, const float* __restrict__ scales,
+                                                      const float* __restrict__ bias, void* __restrict__ out) {
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < a.total; i += stride) {
+    const int64_t pos = i / a.groups4;
+    const int oc0 = static_cast<int>(i - pos * a.groups4) * 4;
+    const int ow = static_cast<int>(pos % a.out_w);
+    const int64_t t = pos / a.out_w;
+    const int oh = static_cast<int>(t % a.out_h);
+    const int64_t b = t / a.out_h;
+    int acc[4] = {0, 0, 0, 0};
+    for (int kh = 0; kh < a.k_h; ++kh) {
+      const int ih = oh * a.stride_h - a.pad_top + kh * a.dil_h;
+      if (ih < 0 || ih >= a.in_h) continue;
+      for (int kw = 0; kw < a.k_w; ++kw) {
+        const int iw = ow * a.stride_w - a.pad_left + kw * a.dil_w;
+        if (iw < 0 || iw >= a.in_w) continue;
+        const uint8_t* xp = x + ((b * a.in_h + ih) * a.in_w + iw) * a.in_c;
+        const int8_t* wp = w + static_cast<int64_t>(kh * a.k_w + kw) * a.out_c;
+        if (a.vec) {
+          const uint32_t xv = *reinterpret_cast<const uint32_t*>(xp + oc0);
+          const uint32_t wv = *reinterpret_cast<const uint32_t*>(wp + oc0);
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const int xs = a.x_signed ? (static_cast<int>(xv << (24 - 8 * r)) >> 24) : static_cast<int>((xv >> (8 * r)) & 0xffu);
+            acc[r] += __mul24(xs, static_cast<int>(wv << (24 - 8 * r)) >> 24);
+          }
+        } else {
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const int oc = oc0 + r;
+            if (oc < a.out_c) {
+              const int c = oc / a.mult;
+              const int xs = a.x_signed ? static_cast<int>(reinterpret_cast<const int8_t*>(xp)[c]) : static_cast<int>(xp[c]);
+              acc[r] += __mul24(xs, static_cast<int>(wp[oc]));
+            }
+          }
+        }
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int n = oc0 + r;
+      if (n >= a.out_c) break;
+      float v = static_cast<float>(acc[r]);
+      if (a.n_scales == 1) v = v * scales[0];
+      else if (a.n_scales > 1) v = v * scales[n];
+      if (bias) v = v + bias[n];
+      for (int k = 0; k < a.n_eltwise; ++k) v = apply_eltwise(a.elt[k], v);
+      store_output<OUT_T>(out, pos * a.out_c + n, v);
+    }
+  }
+}
+
+// The common case - 3x3 window, stride 1, dilation 1, multiplier 1, channels a multiple of 4 - with the window
+// unrolled and 32-bit index arithmetic: a thread owns 4 consecutive channels of a column of R = 4 output rows, so it
+// loads each input dword once for up to 3 of its outputs (18 input + 9 filter dwords for 16 outputs), and a wavefront's
+// loads cover 256 contiguous bytes (consecutive lanes = consecutive channel groups, then consecutive columns).
+template <int OUT_T, bool X_SIGNED>
+__global__ __launch_bounds__(256) void qdwconv3x3_kernel(const DepthwiseArgs a, const uint8_t* __restrict__ x,
+                                                         const int8_t* __restrict__ w, const float* __restrict__ scales,
+                                                         const float* __restrict__ bias, void* __restrict__ out) {
+  constexpr int R = 4;
+  const uint32_t row_items = static_cast<uint32_t>(a.out_w) * a.groups4;  // (column, channel group) pairs of one output row
+  const uint32_t strips = (a.out_h + R - 1) / R;
+  const uint32_t total = static_cast<uint32_t>(a.total);                  // batch * strips * row_items, < 2^31 (host)
+  const uint32_t stride = gridDim.x * blockDim.x;
+  for (uint32_t i = blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
+    const uint32_t t = i / row_items, item = i - t * row_items;
+    const uint32_t b = t / strips, strip = t - b * strips;
+    const int ow = static_cast<int>(item / a.groups4);
+    const int oc0 = static_cast<int>(item - ow * a.groups4) * 4;
+    const int oh0 = static_cast<int>(strip) * R;
+    int acc[R][4];
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+      for (int c = 0; c < 4; ++c) acc[r][c] = 0;
+    const uint8_t* xb = x + static_cast<uint32_t>(b) * static_cast<uint32_t>(a.in_h * a.in_w * a.in_c) + oc0;  // input bytes < 2^31 (host)
+    // All 18 input dwords are loaded unconditionally from clamped (valid) positions and zeroed afterwards where the
+    // position lies in the padding: a branch around each load would make every load wait for the one before it.
+    uint32_t xin[3][R + 2];
+#pragma unroll
+    for (int kw = 0; kw < 3; ++kw) {
+      const int iw = ow - a.pad_left + kw;
+      const int iwc = min(max(iw, 0), a.in_w - 1);
+#pragma unroll
+      for (int rr = 0; rr < R + 2; ++rr) {
+        const int ih = oh0 - a.pad_top + rr;
+        const int ihc = min(max(ih, 0), a.in_h - 1);
+        xin[kw][rr] = *reinterpret_cast<const uint32_t*>(xb + (ihc * a.in_w + iwc) * a.in_c);
+      }
+    }
+#pragma unroll
+    for (int kw = 0; kw < 3; ++kw) {
+      const int iw = ow - a.pad_left + kw;
+      const bool col_ok = iw >= 0 && iw < a.in_w;
+      uint32_t wv[3];
+#pragma unroll
+      for (int kh = 0; kh < 3; ++kh) wv[kh] = *reinterpret_cast<const uint32_t*>(w + (kh * 3 + kw) * a.out_c + oc0);
+#pragma unroll
+      for (int rr = 0; rr < R + 2; ++rr) {  // input rows oh0 - pad_top + rr feed output rows rr - kh
+        const int ih = oh0 - a.pad_top + rr;
+        const uint32_t xv = (col_ok && ih >= 0 && ih < a.in_h) ? xin[kw][rr] : 0u;
+        int xs[4];
+#pragma unroll
+        for (int c = 0; c < 4; ++c)
+          xs[c] = X_SIGNED ? (static_cast<int>(xv << (24 - 8 * c)) >> 24) : static_cast<int>((xv >> (8 * c)) & 0xffu);
+#pragma unroll
+        for (int kh = 0; kh < 3; ++kh) {
+          const int r = rr - kh;
+          if (r < 0 || r >= R) continue;
+#pragma unroll
+          for (int c = 0; c < 4; ++c)  // 8-bit factors: the 24-bit multiply-add is exact and full rate (a 32-bit multiply is not)
+            acc[r][c] = __mul24(xs[c], static_cast<int>(wv[kh] << (24 - 8 * c)) >> 24) + acc[r][c];
+        }
+      }
+    }
+    float sc[4], bi[4];
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      sc[c] = a.n_scales == 0 ? 1.0f : scales[a.n_scales == 1 ? 0 : oc0 + c];
+      bi[c] = bias ? bias[oc0 + c] : 0.0f;
+    }
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const int oh = oh0 + r;
+      if (oh >= a.out_h) break;
+      const int64_t o = ((static_cast<int64_t>(b) * a.out_h + oh) * a.out_w + ow) * a.out_c + oc0;
+      float y[4];
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        float v = static_cast<float>(acc[r][c]);
+        if (a.n_scales != 0) v = v * sc[c];
+        if (bias) v = v + bi[c];
+        y[c] = v;
+      }
+      if (a.chain & 1) {
+#pragma unroll
+        for (int c = 0; c < 4; ++c) y[c] = fmaxf(y[c], 0.0f);
+      }
+      if (a.chain & 2) {
+#pragma unroll
+        for (int c = 0; c < 4; ++c) y[c] = y[c] > 0.0f ? y[c] : y[c] * a.alpha;
+      }
+      if (a.chain & 4) {
+#pragma unroll
+        for (int c = 0; c < 4; ++c) y[c] = fminf(fmaxf(y[c], a.lo), a.hi);
+      }
+      if (a.chain & 8) {
+#pragma unroll
+        for (int c = 0; c < 4; ++c) y[c] = a.lin_a * y[c] + a.lin_b;
+      }
+      // the 4 channels as one store (the host checked the output's alignment)
+      if constexpr (OUT_T == ITEXHIP_FLOAT) {
+        *reinterpret_cast<f4*>(static_cast<float*>(out) + o) = f4{y[0], y[1], y[2], y[3]};
+      } else if constexpr (is_float16_type(OUT_T)) {
+        typedef unsigned int u2 __attribute__((ext_vector_type(2)));
+        *reinterpret_cast<u2*>(static_cast<uint16_t*>(out) + o) = u2{f32_to_bits16<OUT_T>(y[0]) | (f32_to_bits16<OUT_T>(y[1]) << 16),
+                                                                     f32_to_bits16<OUT_T>(y[2]) | (f32_to_bits16<OUT_T>(y[3]) << 16)};
+      } else if constexpr (OUT_T == ITEXHIP_QINT32) {
+        *reinterpret_cast<i4*>(static_cast<int32_t*>(out) + o) = i4{sat_rne<ITEXHIP_QINT32>(y[0]), sat_rne<ITEXHIP_QINT32>(y[1]),
+                                                                    sat_rne<ITEXHIP_QINT32>(y[2]), sat_rne<ITEXHIP_QINT32>(y[3])};
+      } else {
+        *reinterpret_cast<uint32_t*>(static_cast<uint8_t*>(out) + o) =
+            pack4(sat_rne<OUT_T>(y[0]), sat_rne<OUT_T>(y[1]), sat_rne<OUT_T>(y[2]), sat_rne<OUT_T>(y[3]));
+      }
+    }
+  }
+}
+
 }  // namespace
 }  // namespace itexhip
 
 using namespace itexhip;
+
+extern "C" int itexhip_qdepthwise_conv2d(const void* x, int x_type, const itexhip_conv_geometry* g, int64_t multiplier,
+                                         const int8_t* filter, const float* scales, const float* bias,
+                                         const itexhip_epilogue* ep, int out_type, void* out, void* stream) {
+  const char* who = "itexhip_qdepthwise_conv2d";
+  ITEXHIP_REQUIRE(g != nullptr && ep != nullptr, "%s: null geometry or epilogue", who);
+  ITEXHIP_REQUIRE(x_type == ITEXHIP_QUINT8 || x_type == ITEXHIP_QINT8, "%s: input type must be quint8 or qint8", who);
+  ITEXHIP_REQUIRE(out_type == ITEXHIP_QINT32 || out_type == ITEXHIP_QINT8 || out_type == ITEXHIP_QUINT8 ||
+                      out_type == ITEXHIP_FLOAT || out_type == ITEXHIP_BFLOAT16, "%s: unsupported output type %d", who, out_type);
+  ITEXHIP_REQUIRE(g->batch >= 0 && g->in_h >= 0 && g->in_w >= 0 && g->in_c >= 0 && g->k_h > 0 && g->k_w > 0 && g->out_h >= 0 &&
+                      g->out_w >= 0 && multiplier > 0, "%s: bad extents", who);
+  ITEXHIP_REQUIRE(g->stride_h > 0 && g->stride_w > 0 && g->dil_h > 0 && g->dil_w > 0, "%s: strides and dilations must be positive", who);
+  ITEXHIP_REQUIRE(g->pad_top >= 0 && g->pad_left >= 0, "%s: negative padding", who);
+  const int64_t lim = 1LL << 31;
+  const int64_t out_c = g->in_c * multiplier;
+  ITEXHIP_REQUIRE(g->in_h < lim && g->in_w < lim && out_c < lim && g->out_h < lim && g->out_w < lim && g->k_h < (1 << 15) &&
+                      g->k_w < (1 << 15) && g->pad_top < (1 << 24) && g->pad_left < (1 << 24) &&
+                      g->out_h * g->stride_h < (1LL << 30) && g->out_w * g->stride_w < (1LL << 30) &&
+                      (g->k_h - 1) * g->dil_h < (1LL << 30) && (g->k_w - 1) * g->dil_w < (1LL << 30),
+                  "%s: extent too large", who);
+  ITEXHIP_REQUIRE(g->k_h * g->k_w <= 32767 && 255LL * 128 * g->k_h * g->k_w < lim, "%s: window too large for int32 accumulation", who);
+  ITEXHIP_REQUIRE(ep->n_eltwise >= 0 && ep->n_eltwise <= 3, "%s: bad eltwise count", who);
+  for (int k = 0; k < ep->n_eltwise; ++k)
+    ITEXHIP_REQUIRE(ep->elt[k].alg != ITEXHIP_ELT_SUM, "%s: no sum post-op here", who);
+  ITEXHIP_REQUIRE(ep->n_scales == 0 || ep->n_scales == 1 || ep->n_scales == out_c, "%s: %d scales for %lld channels", who,
+                  ep->n_scales, static_cast<long long>(out_c));
+  const int64_t positions = g->batch * g->out_h * g->out_w;
+  if (positions == 0 || out_c == 0) return ITEXHIP_OK;
+  ITEXHIP_REQUIRE(x && filter && out, "%s: null buffer", who);
+  ITEXHIP_REQUIRE(ep->n_scales == 0 || scales, "%s: null scales", who);
+  DepthwiseArgs a{};
+  a.in_h = static_cast<int>(g->in_h); a.in_w = static_cast<int>(g->in_w); a.in_c = static_cast<int>(g->in_c);
+  a.k_h = static_cast<int>(g->k_h); a.k_w = static_cast<int>(g->k_w); a.out_h = static_cast<int>(g->out_h);
+  a.out_w = static_cast<int>(g->out_w); a.stride_h = g->stride_h; a.stride_w = g->stride_w; a.dil_h = g->dil_h; a.dil_w = g->dil_w;
+  a.pad_top = static_cast<int>(g->pad_top); a.pad_left = static_cast<int>(g->pad_left);
+  a.mult = static_cast<int>(multiplier); a.out_c = static_cast<int>(out_c); a.groups4 = static_cast<int>((out_c + 3) / 4);
+  a.x_signed = x_type == ITEXHIP_QINT8;
+  a.vec = multiplier == 1 && g->in_c % 4 == 0 && aligned(x, 4) && aligned(filter, 4);
+  a.n_scales = ep->n_scales; a.n_eltwise = ep->n_eltwise;
+  a.elt[0] = ep->elt[0]; a.elt[1] = ep->elt[1]; a.elt[2] = ep->elt[2];
+  a.total = positions * a.groups4;
+  const uint8_t* xp = static_cast<const uint8_t*>(x);
+  hipStream_t st = as_stream(stream);
+  const int64_t strip_total = g->batch * ((g->out_h + 3) / 4) * g->out_w * a.groups4;
+  bool canonical = true;
+  {
+    int k = 0;
+    if (k < ep->n_eltwise && ep->elt[k].alg == ITEXHIP_ELT_RELU) {
+      if (ep->elt[k].alpha == 0.0f) a.chain |= 1; else { a.chain |= 2; a.alpha = ep->elt[k].alpha; }
+      ++k;
+    } else if (k < ep->n_eltwise && ep->elt[k].alg == ITEXHIP_ELT_CLIP) {
+      a.chain |= 4; a.lo = ep->elt[k].alpha; a.hi = ep->elt[k].beta;
+      ++k;
+    }
+    if (k < ep->n_eltwise && ep->elt[k].alg == ITEXHIP_ELT_LINEAR) {
+      a.chain |= 8; a.lin_a = ep->elt[k].alpha; a.lin_b = ep->elt[k].beta;
+      ++k;
+    }
+    canonical = k == ep->n_eltwise;
+  }
+  if (canonical && a.vec && aligned(out, 16) && g->k_h == 3 && g->k_w == 3 && g->stride_h == 1 && g->stride_w == 1 && g->dil_h == 1 && g->dil_w == 1 &&
+      strip_total < lim && g->batch * g->in_h * g->in_w * g->in_c < lim) {
+    a.total = strip_total;
+    const unsigned sblocks = static_cast<unsigned>(std::min<int64_t>((a.total + 255) / 256, 256 * 64));
+#define DW3(T)                                                                                           \
+  if (a.x_signed) qdwconv3x3_kernel<T, true><<<sblocks, 256, 0, st>>>(a, xp, filter, scales, bias, out); \
+  else qdwconv3x3_kernel<T, false><<<sblocks, 256, 0, st>>>(a, xp, filter, scales, bias, out)
+    switch (out_type) {
+      case ITEXHIP_FLOAT: DW3(ITEXHIP_FLOAT); break;
+      case ITEXHIP_BFLOAT16: DW3(ITEXHIP_BFLOAT16); break;
+      case ITEXHIP_QINT32: DW3(ITEXHIP_QINT32); break;
+      case ITEXHIP_QINT8: DW3(ITEXHIP_QINT8); break;
+      default: DW3(ITEXHIP_QUINT8); break;
+    }
+#undef DW3
+    ITEXHIP_CHECK_LAUNCH(who);
+    return ITEXHIP_OK;
+  }
+  const unsigned blocks = static_cast<unsigned>(std::min<int64_t>((a.total + 255) / 256, 256 * 64));
+  switch (out_type) {
+    case ITEXHIP_FLOAT: qdwconv_kernel<ITEXHIP_FLOAT><<<blocks, 256, 0, st>>>(a, xp, filter, scales, bias, out); break;
+    case ITEXHIP_BFLOAT16: qdwconv_kernel<ITEXHIP_BFLOAT16><<<blocks, 256, 0, st>>>(a, xp, filter, scales, bias, out); break;
+    case ITEXHIP_QINT32: qdwconv_kernel<ITEXHIP_QINT32><<<blocks, 256, 0, st>>>(a, xp, filter, scales, bias, out); break;
+    case ITEXHIP_QINT8: qdwconv_kernel<ITEXHIP_QINT8><<<blocks, 256, 0, st>>>(a, xp, filter, scales, bias, out); break;
+    default: qdwconv_kernel<ITEXHIP_QUINT8><<<blocks, 256, 0, st>>>(a, xp, filter, scales, bias, out); break;
+  }
+  ITEXHIP_CHECK_LAUNCH(who);
+  return ITEXHIP_OK;
+}
 
 extern "C" int itexhip_im2col8(const void* x, const itexhip_conv_geometry* g, int64_t row_bytes, void* cols, void* stream) {
   const char* who = "itexhip_im2col8";

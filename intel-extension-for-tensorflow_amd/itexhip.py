@@ -30,7 +30,7 @@ EXPORTS = [
     "itexhip_qmatmul_epilogue_desc", "itexhip_qmatmul_prepare", "itexhip_qgemm_packed_bytes",
     "itexhip_qgemm_prepack_b", "itexhip_qgemm", "itexhip_qgemm_tile", "itexhip_qgemv", "itexhip_qmatmul", "itexhip_qmatmul_per_row", "itexhip_qmatmul_unpacked", "itexhip_mfma_probe",
     "itexhip_qgemm_naive", "itexhip_qbatch_matmul", "itexhip_transpose", "itexhip_im2col8", "itexhip_scale_vector",
-    "itexhip_qconv2d_implicit_ok", "itexhip_qconv2d", "itexhip_qgemm_sum", "itexhip_qconv2d_sum",
+    "itexhip_qconv2d_implicit_ok", "itexhip_qconv2d", "itexhip_qgemm_sum", "itexhip_qconv2d_sum", "itexhip_qdepthwise_conv2d",
 ]
 
 
@@ -350,6 +350,11 @@ def qconv2d_sum(x, x_type, geometry, packed_filter, colsum, out_channels, scales
 def qgemm_sum(a, a_type, packed_b, colsum, M, K, N, scales, bias, ep, addend, addend_type, out_type, out, stream=0):
     _check(_lib.itexhip_qgemm_sum(_ptr(a), int(a_type), _ptr(packed_b), _ptr(colsum), _i64(M), _i64(K), _i64(N), _ptr(scales),
                                   _ptr(bias), C.byref(ep), _ptr(addend), int(addend_type), int(out_type), _ptr(out), _ptr(stream)))
+
+
+def qdepthwise_conv2d(x, x_type, geometry, multiplier, filt, scales, bias, ep, out_type, out, stream=0):
+    _check(_lib.itexhip_qdepthwise_conv2d(_ptr(x), int(x_type), C.byref(geometry), _i64(multiplier), _ptr(filt), _ptr(scales),
+                                          _ptr(bias), C.byref(ep), int(out_type), _ptr(out), _ptr(stream)))
 
 
 def scale_vector(bias, bias_type, factors, n_factors, n, out, stream=0):

@@ -43,6 +43,11 @@ const Rename kTable[] = {
     {"QuantizedConv2DWithBiasSumAndReluAndRequantize", "_ITEXQuantizedConv2DWithBiasSumAndReluAndRequantize", Copy::kQuantizedConv2D, Rule::kAlways},
     {"QuantizedConv2DWithBiasSignedSumAndReluAndRequantize", "_ITEXQuantizedConv2DWithBiasSignedSumAndReluAndRequantize", Copy::kQuantizedConv2D, Rule::kAlways},
     {"_QuantizedConv2D", "_ITEXQuantizedConv2DV2", Copy::kAll, Rule::kAlways},
+    {"QuantizedDepthwiseConv2D", "_ITEXQuantizedDepthwiseConv2D", Copy::kQuantizedConv2D, Rule::kAlways},
+    {"QuantizedDepthwiseConv2DWithBias", "_ITEXQuantizedDepthwiseConv2DWithBias", Copy::kQuantizedConv2D, Rule::kAlways},
+    {"QuantizedDepthwiseConv2DWithBiasAndRelu", "_ITEXQuantizedDepthwiseConv2DWithBiasAndRelu", Copy::kQuantizedConv2D, Rule::kAlways},
+    {"QuantizedDepthwiseConv2DWithBiasAndReluAndRequantize", "_ITEXQuantizedDepthwiseConv2DWithBiasAndReluAndRequantize", Copy::kQuantizedConv2D, Rule::kAlways},
+    {"_QuantizedDepthwiseConv2D", "_ITEXQuantizedDepthwiseConv2DV2", Copy::kAll, Rule::kAlways},
     {"QuantizedMatMulWithBias", "_ITEXQuantizedMatMulWithBias", Copy::kQuantizedMatMul, Rule::kAlways},
     {"QuantizedMatMulWithBiasAndDequantize", "_ITEXQuantizedMatMulWithBiasAndDequantize", Copy::kQuantizedMatMul, Rule::kAlways},
     {"QuantizedMatMulWithBiasAndRelu", "_ITEXQuantizedMatMulWithBiasAndRelu", Copy::kQuantizedMatMul, Rule::kAlways},

@@ -178,9 +178,9 @@ std::vector<OpSpec> OpSpecs() {
     v.push_back({"_ITEXQuantizedMatMulWithBiasAndDequantize", in9, {"out: Toutput"},
                  attrs("Tbias: {float, bfloat16, qint32}", "Toutput: {float, bfloat16}")});
   }
-  // quantized Conv2D: the list-attribute form (nn_ops.cc: _QuantizedConv2D, _ITEXQuantizedConv2DV2) and the _ITEX twins
-  // of TensorFlow's QuantizedConv2D* ops
-  for (const char* name : {"_QuantizedConv2D", "_ITEXQuantizedConv2DV2"})
+  // quantized Conv2D and depthwise Conv2D: the list-attribute form (nn_ops.cc:585-700, 752-860) and the _ITEX twins of
+  // TensorFlow's QuantizedConv2D* / QuantizedDepthwiseConv2D* ops
+  for (const char* name : {"_QuantizedConv2D", "_ITEXQuantizedConv2DV2", "_QuantizedDepthwiseConv2D", "_ITEXQuantizedDepthwiseConv2DV2"})
     v.push_back({name,
                  {"device_inputs: Tdevice_inputs", "host_inputs: Thost_inputs"},
                  {"device_outputs: Tdevice_outputs", "host_outputs: Thost_outputs"},
@@ -205,6 +205,11 @@ std::vector<OpSpec> OpSpecs() {
                           Twin{"_ITEXQuantizedConv2DAndReluAndRequantize", false, true, "out_type: quantizedtype = DT_QUINT8"},
                           Twin{"_ITEXQuantizedConv2DWithBiasAndRequantize", true, true, "out_type: quantizedtype = DT_QINT8"},
                           Twin{"_ITEXQuantizedConv2DWithBiasAndReluAndRequantize", true, true, "out_type: quantizedtype = DT_QUINT8"},
+                          Twin{"_ITEXQuantizedDepthwiseConv2D", false, false, "out_type: quantizedtype = DT_QINT32"},
+                          Twin{"_ITEXQuantizedDepthwiseConv2DWithBias", true, false, "out_type: quantizedtype = DT_QINT32"},
+                          Twin{"_ITEXQuantizedDepthwiseConv2DWithBiasAndRelu", true, false, "out_type: quantizedtype = DT_QINT32"},
+                          Twin{"_ITEXQuantizedDepthwiseConv2DWithBiasAndReluAndRequantize", true, true,
+                               "out_type: quantizedtype = DT_QUINT8"},
                           Twin{"_ITEXQuantizedConv2DWithBiasSumAndReluAndRequantize", true, true, "out_type: quantizedtype = DT_QUINT8", true},
                           Twin{"_ITEXQuantizedConv2DWithBiasSignedSumAndReluAndRequantize", true, true,
                                "out_type: quantizedtype = DT_QUINT8", true}}) {

@@ -23,7 +23,10 @@ namespace {
 std::vector<std::string> LegacyFusions(const std::string& op) {
   std::string name = op;
   if (name.rfind("_ITEX", 0) == 0) name = name.substr(5);
-  if (name == "QuantizedConv2D" || name == "QuantizedConv2DPerChannel") return {};
+  if (name == "QuantizedConv2D" || name == "QuantizedConv2DPerChannel" || name == "QuantizedDepthwiseConv2D") return {};
+  if (name == "QuantizedDepthwiseConv2DWithBias") return {"BiasAdd"};
+  if (name == "QuantizedDepthwiseConv2DWithBiasAndRelu") return {"BiasAdd", "Relu"};
+  if (name == "QuantizedDepthwiseConv2DWithBiasAndReluAndRequantize") return {"BiasAdd", "Relu", "Requantize"};
   if (name == "QuantizedConv2DWithBias") return {"BiasAdd"};
   if (name == "QuantizedConv2DWithBiasAndRelu") return {"BiasAdd", "Relu"};
   if (name == "QuantizedConv2DAndRelu") return {"Relu"};
@@ -56,7 +59,7 @@ bool OutDim(int64_t in, int64_t k, int64_t stride, int64_t dil, const std::strin
 class QuantizedConv2DOp : public OpKernel {
  public:
   QuantizedConv2DOp(OpKernelConstruction* ctx, const std::string& op, bool new_api, TF_DataType t_in, TF_DataType t_out)
-      : t_in_(t_in), t_out_(t_out) {
+      : t_in_(t_in), t_out_(t_out), depthwise_(op.find("Depthwise") != std::string::npos) {
     std::vector<int64_t> strides, dilations;
     ITEX_REQUIRES_OK(ctx, ctx->GetAttr("dilations", &dilations));
     ITEX_REQUIRES_OK(ctx, ctx->GetAttr("strides", &strides));
@@ -110,6 +113,7 @@ class QuantizedConv2DOp : public OpKernel {
     }
     if (sum_position_ < 0) sum_position_ = 0;
     if (leaky_) ITEX_REQUIRES_OK(ctx, ctx->GetAttr("alpha", &alpha_));
+    ITEX_REQUIRES(ctx, !(depthwise_ && sum_position_ != 0), TF_UNIMPLEMENTED, "the depthwise convolution has no Sum fusion on this device");
     if (sum_position_ != 0) {
       // quantized_conv_ops.h:202-218, 398-433: an 8-bit summand under an 8-bit output; the qint32 output with a float
       // summand (the graph before Requantize is fused) is not built
@@ -167,7 +171,9 @@ class QuantizedConv2DOp : public OpKernel {
     ITEX_REQUIRES(ctx, x.dtype() == t_in_ && filter.dtype() == TF_QINT8, TF_INVALID_ARGUMENT,
                   "quantized Conv2D operand types do not match the kernel");
     const int64_t B = x.dim_size(0), H = x.dim_size(1), W = x.dim_size(2), C = x.dim_size(3);
-    const int64_t KH = filter.dim_size(0), KW = filter.dim_size(1), O = filter.dim_size(3);
+    // depthwise: the filter is [KH, KW, C, multiplier] and the output has C * multiplier channels (conv_ops.h:395-397)
+    const int64_t KH = filter.dim_size(0), KW = filter.dim_size(1);
+    const int64_t O = depthwise_ ? filter.dim_size(2) * filter.dim_size(3) : filter.dim_size(3);
     ITEX_REQUIRES(ctx, filter.dim_size(2) == C, TF_INVALID_ARGUMENT,
                   "input depth " + std::to_string(C) + " vs. filter input depth " + std::to_string(filter.dim_size(2)));
     ITEX_REQUIRES(ctx, KH > 0 && KW > 0, TF_INVALID_ARGUMENT, "empty filter window");
@@ -232,7 +238,8 @@ class QuantizedConv2DOp : public OpKernel {
 
     void* stream = ctx->stream();
     // ---- filter: packed once when constant (the HWIO tensor read as a [K, O] matrix)
-    const bool repack = !packed_.valid() || !is_filter_const_ || packed_src_ != filter.data() || packed_k_ != K || packed_n_ != O;
+    const bool repack = !depthwise_ &&
+                        (!packed_.valid() || !is_filter_const_ || packed_src_ != filter.data() || packed_k_ != K || packed_n_ != O);
     if (repack && O > 0) {
       packed_ = ctx->allocate_temp(TF_QINT8, {std::max<int64_t>(itexhip_qgemm_packed_bytes(Kp, O), 16)});
       colsum_ = ctx->allocate_temp(TF_INT32, {O});
@@ -271,6 +278,16 @@ class QuantizedConv2DOp : public OpKernel {
         ITEX_REQUIRES(ctx, st == ITEXHIP_OK, TF_ABORTED, std::string("Operation received an exception: ") + itexhip_last_error());
         bias_dev = sbias.flat<float>();
       }
+      itexhip_epilogue dep{};
+      if (depthwise_) {  // no matrix product in it: a kernel of its own on the filter as TensorFlow stores it
+        dep.n_scales = static_cast<int>(depth);
+        if (activation_ != 0) dep.elt[dep.n_eltwise++] = {activation_, leaky_ ? alpha_ : 0.0f, 0.0f};
+        const int st = itexhip_qdepthwise_conv2d(x.data(), t_in_, &g, filter.dim_size(3), filter.flat<int8_t>(), params, bias_dev, &dep,
+                                                 t_out_, out.data(), stream);
+        ITEX_REQUIRES(ctx, st == ITEXHIP_OK, st == ITEXHIP_INVALID_ARGUMENT ? TF_INVALID_ARGUMENT : TF_ABORTED,
+                      std::string("Operation received an exception: ") + itexhip_last_error());
+      }
+      if (!depthwise_) {
       // ---- summand of the Sum fusion
       const void* summand_dev = nullptr;
       int summand_type = 0;
@@ -323,6 +340,7 @@ class QuantizedConv2DOp : public OpKernel {
       }
       ITEX_REQUIRES(ctx, st == ITEXHIP_OK, st == ITEXHIP_INVALID_ARGUMENT ? TF_INVALID_ARGUMENT : TF_ABORTED,
                     std::string("Operation received an exception: ") + itexhip_last_error());
+      }  // !depthwise_
     }
 
     // ---- output ranges in host memory (AllocateNativeOutputMinMax, quantized_ops.h:142-203)
@@ -346,6 +364,7 @@ class QuantizedConv2DOp : public OpKernel {
 
  private:
   TF_DataType t_in_, t_out_, t_bias_ = TF_FLOAT;
+  bool depthwise_ = false;
   TF_DataType t_summand_ = TF_QUINT8;
   int sum_position_ = 0;  // 0 none, 1 before the activation, 2 after it
   int summand_idx_ = -1, summand_min_idx_ = -1;
@@ -372,13 +391,17 @@ const char* const kLegacyNames[] = {"QuantizedConv2D", "QuantizedConv2DPerChanne
                                     "QuantizedConv2DAndReluAndRequantize", "QuantizedConv2DWithBiasAndRequantize",
                                     "QuantizedConv2DWithBiasAndReluAndRequantize",
                                     "QuantizedConv2DWithBiasSumAndReluAndRequantize",
-                                    "QuantizedConv2DWithBiasSignedSumAndReluAndRequantize"};
+                                    "QuantizedConv2DWithBiasSignedSumAndReluAndRequantize",
+                                    "QuantizedDepthwiseConv2D", "QuantizedDepthwiseConv2DWithBias",
+                                    "QuantizedDepthwiseConv2DWithBiasAndRelu",
+                                    "QuantizedDepthwiseConv2DWithBiasAndReluAndRequantize"};
 
+// NAME < 0 with NEW_API: the depthwise op
 template <int NAME, bool NEW_API, int TIN, int TOUT>
 struct ConvKernel : QuantizedConv2DOp {
   explicit ConvKernel(OpKernelConstruction* c)
-      : QuantizedConv2DOp(c, NEW_API ? "_QuantizedConv2D" : kLegacyNames[NAME], NEW_API, static_cast<TF_DataType>(TIN),
-                          static_cast<TF_DataType>(TOUT)) {}
+      : QuantizedConv2DOp(c, NEW_API ? (NAME < 0 ? "_QuantizedDepthwiseConv2D" : "_QuantizedConv2D") : kLegacyNames[NAME < 0 ? 0 : NAME],
+                          NEW_API, static_cast<TF_DataType>(TIN), static_cast<TF_DataType>(TOUT)) {}
 };
 
 template <int NAME, int TIN, int TOUT>
@@ -398,16 +421,26 @@ void RegLegacy(bool with_bias_types, std::initializer_list<const char*> host_arg
   }
 }
 
+// Tsummand as the reference constrains it (quantized_conv_ops.cc:168-262): either 8-bit type under an 8-bit output, the
+// output's own type otherwise
 template <int TIN, int TOUT>
 void RegNewApi() {
-  for (const char* op : {"_QuantizedConv2D", "_ITEXQuantizedConv2DV2"})
-    for (TF_DataType tb : {TF_FLOAT, TF_QINT32}) {
-      KernelDefBuilder b(op, "QuantizedConvOp");
-      b.TypeConstraint("Tinput", static_cast<TF_DataType>(TIN)).TypeConstraint("Tfilter", TF_QINT8).TypeConstraint("Tbias", tb);
-      b.TypeConstraint("out_type", static_cast<TF_DataType>(TOUT));
-      b.HostMemory("host_inputs").HostMemory("host_outputs");
-      b.Register<ConvKernel<0, true, TIN, TOUT>>();
-    }
+  const bool out_q8 = TOUT == TF_QINT8 || TOUT == TF_QUINT8;
+  const std::vector<TF_DataType> summands = out_q8 ? std::vector<TF_DataType>{TF_QINT8, TF_QUINT8}
+                                                   : std::vector<TF_DataType>{static_cast<TF_DataType>(TOUT)};
+  static const char* const kNames[2][2] = {{"_QuantizedConv2D", "_ITEXQuantizedConv2DV2"},
+                                           {"_QuantizedDepthwiseConv2D", "_ITEXQuantizedDepthwiseConv2DV2"}};
+  for (const bool depthwise : {false, true})
+    for (const char* op : kNames[depthwise ? 1 : 0])
+      for (TF_DataType tb : {TF_FLOAT, TF_QINT32})
+        for (TF_DataType ts : summands) {
+          KernelDefBuilder b(op, "QuantizedConvOp");
+          b.TypeConstraint("Tinput", static_cast<TF_DataType>(TIN)).TypeConstraint("Tfilter", TF_QINT8).TypeConstraint("Tbias", tb);
+          b.TypeConstraint("Tsummand", ts).TypeConstraint("out_type", static_cast<TF_DataType>(TOUT));
+          b.HostMemory("host_inputs").HostMemory("host_outputs");
+          if (depthwise) b.Register<ConvKernel<-1, true, TIN, TOUT>>();
+          else b.Register<ConvKernel<0, true, TIN, TOUT>>();
+        }
 }
 
 }  // namespace
@@ -432,6 +465,11 @@ void AddQuantizedConvKernels() {
                                                   "max_freezed_output", "min_summand", "max_summand", "min_output", "max_output"};
   RegLegacy<9, TF_QUINT8, TF_QUINT8>(true, sum, TF_QUINT8);
   RegLegacy<10, TF_QUINT8, TF_QUINT8>(true, sum, TF_QINT8);
+  // depthwise, legacy spellings (:92-99, 126-129): quint8 input only
+  RegLegacy<11, TF_QUINT8, TF_QINT32>(false, plain);
+  RegLegacy<12, TF_QUINT8, TF_QINT32>(false, plain);
+  RegLegacy<13, TF_QUINT8, TF_QINT32>(false, plain);
+  RegLegacy<14, TF_QUINT8, TF_QUINT8>(true, req);
   RegNewApi<TF_QINT8, TF_QINT8>();   RegNewApi<TF_QUINT8, TF_QINT8>();
   RegNewApi<TF_QINT8, TF_QUINT8>();  RegNewApi<TF_QUINT8, TF_QUINT8>();
   RegNewApi<TF_QINT8, TF_FLOAT>();   RegNewApi<TF_QUINT8, TF_FLOAT>();

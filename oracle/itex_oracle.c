@@ -791,6 +791,58 @@ void orc_int_conv2d(const void* x, int x_type, const int8_t* w, const orc_conv_g
   }
 }
 
+/* Depthwise: one group per input channel (conv_ops.h:238-246: oneDNN filter dims G = in_c, O = multiplier, I = 1), so
+ * output channel c * mult + m = sum over the window of x[.., c] * w[kh, kw, c, m]; output depth in_c * mult (:395-397). */
+void orc_int_depthwise_conv2d(const void* x, int x_type, const int8_t* w, const orc_conv_geom* g, int64_t mult,
+                              int64_t out_h, int64_t out_w, int64_t pad_top, int64_t pad_left, int32_t* acc) {
+  const uint8_t* xu = (const uint8_t*)x;
+  const int8_t* xs = (const int8_t*)x;
+  const int64_t oc = g->in_c * mult;
+  for (int64_t b = 0; b < g->batch; ++b)
+    for (int64_t oh = 0; oh < out_h; ++oh)
+      for (int64_t ow = 0; ow < out_w; ++ow) {
+        int32_t* dst = acc + ((b * out_h + oh) * out_w + ow) * oc;
+        for (int64_t o = 0; o < oc; ++o) dst[o] = 0;
+        for (int64_t kh = 0; kh < g->k_h; ++kh) {
+          const int64_t ih = oh * g->stride_h - pad_top + kh * g->dil_h;
+          if (ih < 0 || ih >= g->in_h) continue;
+          for (int64_t kw = 0; kw < g->k_w; ++kw) {
+            const int64_t iw = ow * g->stride_w - pad_left + kw * g->dil_w;
+            if (iw < 0 || iw >= g->in_w) continue;
+            const int64_t xo = ((b * g->in_h + ih) * g->in_w + iw) * g->in_c;
+            const int8_t* wf = w + (kh * g->k_w + kw) * oc;
+            for (int64_t c = 0; c < g->in_c; ++c) {
+              const int32_t xv = x_type == ORC_QUINT8 ? (int32_t)xu[xo + c] : (int32_t)xs[xo + c];
+              for (int64_t m = 0; m < mult; ++m) dst[c * mult + m] += xv * (int32_t)wf[c * mult + m];
+            }
+          }
+        }
+      }
+}
+
+int orc_qdepthwise_conv2d(const orc_conv_attrs* at, const orc_conv_geom* g, int64_t mult, const void* x, const int8_t* w,
+                          const void* bias, float min_in, float max_in, const float* min_f, const float* max_f,
+                          int64_t depth, float min_out, float max_out, void* out, int64_t* out_h, int64_t* out_w) {
+  int64_t pt = 0, pl = 0;
+  if (mult <= 0) return ORC_INVALID_ARGUMENT;
+  if (orc_conv_out_dim(g->in_h, g->k_h, g->stride_h, g->dil_h, g->padding, g->pad_top, g->pad_bottom, out_h, &pt) ||
+      orc_conv_out_dim(g->in_w, g->k_w, g->stride_w, g->dil_w, g->padding, g->pad_left, g->pad_right, out_w, &pl))
+    return ORC_INVALID_ARGUMENT;
+  const int64_t M = g->batch * *out_h * *out_w, N = g->in_c * mult;
+  if (out == NULL || M == 0 || N == 0) return ORC_OK;
+  int32_t* acc = (int32_t*)malloc(sizeof(int32_t) * (size_t)(M * N));
+  float* scales = (float*)malloc(sizeof(float) * (size_t)(depth > 0 ? depth : 1));
+  float* sb = (float*)malloc(sizeof(float) * (size_t)N);
+  orc_epilogue_desc ep;
+  int st = orc_qconv_prepare(at, N, min_in, max_in, min_f, max_f, depth, min_out, max_out, bias, scales, sb, &ep);
+  if (st == ORC_OK) {
+    orc_int_depthwise_conv2d(x, at->t_in, w, g, mult, *out_h, *out_w, pt, pl, acc);
+    orc_qmatmul_epilogue(acc, M, N, &ep, scales, sb, NULL, at->t_out, out);
+  }
+  free(acc); free(scales); free(sb);
+  return st;
+}
+
 int orc_qconv_prepare(const orc_conv_attrs* at, int64_t N, float min_in, float max_in, const float* min_f,
                       const float* max_f, int64_t depth, float min_out, float max_out, const void* bias,
                       float* scales, float* bias_out, orc_epilogue_desc* ep) {

@@ -196,6 +196,13 @@ int orc_qconv_prepare(const orc_conv_attrs* at, int64_t N, float min_in, float m
 int orc_qconv2d(const orc_conv_attrs* at, const orc_conv_geom* g, const void* x, const int8_t* w,
                 const void* bias, float min_in, float max_in, const float* min_f, const float* max_f,
                 int64_t depth, float min_out, float max_out, void* out, int64_t* out_h, int64_t* out_w);
+/* Depthwise form (QuantizedDepthwiseConv2D*, _QuantizedDepthwiseConv2D): w is [k_h, k_w, in_c, mult], the output has
+ * in_c * mult channels (g->out_c is ignored), scales / bias / ranges as for orc_qconv2d with that many channels. */
+void orc_int_depthwise_conv2d(const void* x, int x_type, const int8_t* w, const orc_conv_geom* g, int64_t mult,
+                              int64_t out_h, int64_t out_w, int64_t pad_top, int64_t pad_left, int32_t* acc);
+int orc_qdepthwise_conv2d(const orc_conv_attrs* at, const orc_conv_geom* g, int64_t mult, const void* x, const int8_t* w,
+                          const void* bias, float min_in, float max_in, const float* min_f, const float* max_f,
+                          int64_t depth, float min_out, float max_out, void* out, int64_t* out_h, int64_t* out_w);
 /* The "Sum" fusions (QuantizedConv2DWithBias[Signed]SumAndReluAndRequantize, "Sum" in fused_ops of _QuantizedConv2D)
  * with an 8-bit output, quantized_conv_ops.h:202-218 (type rule), :398-433 (scale of the sum post-op from the frozen
  * output range and the summand's range), :604-640 (the summand buffer becomes the destination; a qint8 summand under

@@ -341,3 +341,25 @@ def qconv2d(at, g, x, w, bias, min_in, max_in, min_f, max_f, min_out=0.0, max_ou
     out = np.zeros((g.batch, oh.value, ow.value, g.out_c), NP_OF[at.t_out])
     st = f(*args(_p(out)))
     return st, out
+
+
+def qdepthwise_conv2d(at, g, x, w, bias, min_in, max_in, min_f, max_f, min_out=0.0, max_out=0.0):
+    """x: [B, H, W, C] uint8 / int8, w: [KH, KW, C, mult] int8 (g built with conv_geom(x.shape, (KH, KW, C, mult))).
+    Returns (status, out [B, OH, OW, C * mult])."""
+    x = np.ascontiguousarray(x, dtype=np.uint8 if at.t_in == QUINT8 else np.int8)
+    w = np.ascontiguousarray(w, dtype=np.int8)
+    mult = w.shape[3]
+    min_f, max_f = _f32(min_f), _f32(max_f)
+    b = None if bias is None else (np.ascontiguousarray(bias, np.int32) if at.t_bias == QINT32 else _f32(bias))
+    oh, ow = C.c_int64(), C.c_int64()
+    f = lib().orc_qdepthwise_conv2d
+    f.restype = C.c_int
+    args = lambda out: (C.byref(at), C.byref(g), C.c_int64(mult), _p(x), _p(w), _p(b) if b is not None else None,
+                        C.c_float(min_in), C.c_float(max_in), _p(min_f), _p(max_f), C.c_int64(min_f.size), C.c_float(min_out),
+                        C.c_float(max_out), out, C.byref(oh), C.byref(ow))
+    st = f(*args(None))
+    if st != OK:
+        return st, None
+    out = np.zeros((g.batch, oh.value, ow.value, g.in_c * mult), NP_OF[at.t_out])
+    st = f(*args(_p(out)))
+    return st, out

@@ -29,7 +29,9 @@ def load(device="XPU", stock_ops=("QuantizeV2", "Dequantize", "QuantizedMatMulWi
                                    "QuantizedConv2DAndRelu", "QuantizedConv2DAndRequantize", "QuantizedConv2DAndReluAndRequantize",
                                    "QuantizedConv2DWithBiasAndRequantize", "QuantizedConv2DWithBiasAndReluAndRequantize",
                                    "QuantizedConv2DWithBiasSumAndReluAndRequantize",
-                                   "QuantizedConv2DWithBiasSignedSumAndReluAndRequantize")):
+                                   "QuantizedConv2DWithBiasSignedSumAndReluAndRequantize", "QuantizedDepthwiseConv2D",
+                                   "QuantizedDepthwiseConv2DWithBias", "QuantizedDepthwiseConv2DWithBiasAndRelu",
+                                   "QuantizedDepthwiseConv2DWithBiasAndReluAndRequantize")):
     """Loads the mock host and the plugin once per process; returns the mock's ctypes handle."""
     if "lib" in _state:
         return _state["lib"]

@@ -201,6 +201,54 @@ def test_sum_post_op_in_conv_and_gemm(hip, dev, t_add, position, alpha):
         hip.qgemm(cols, hip.QUINT8, packed, colsum, M, K, O, sc_d, bi_d, ep, hip.FLOAT, torch.zeros((M, O), device=dev))
 
 
+@pytest.mark.parametrize("shape,kshape,strides,dil", [((2, 14, 13, 32), (3, 3, 32, 1), (1, 1), (1, 1)),   # dword path
+                                                      ((1, 9, 9, 5), (3, 3, 5, 2), (2, 2), (1, 1)),       # multiplier 2, odd channels
+                                                      ((2, 8, 8, 6), (5, 3, 6, 1), (1, 2), (2, 1)),       # channels not a multiple of 4
+                                                      ((1, 6, 6, 4), (3, 3, 4, 3), (1, 1), (1, 1))])
+@pytest.mark.parametrize("signed_in", [False, True])
+def test_depthwise_conv_against_oracle(hip, dev, shape, kshape, strides, dil, signed_in):
+    """itexhip_qdepthwise_conv2d for every output type: per-channel scales, bias, ReLU; bit-equal to the oracle's epilogue
+    on the oracle's depthwise accumulators."""
+    import torch
+    rng = np.random.default_rng(sum(shape) + sum(kshape) + signed_in)
+    B, H, W, Cin = shape
+    kh, kw, _, mult = kshape
+    O = Cin * mult
+    x = rng.integers(-128, 128, shape).astype(np.int8) if signed_in else rng.integers(0, 256, shape).astype(np.uint8)
+    w = rng.integers(-127, 128, kshape).astype(np.int8)
+    oh, pt = same_lead(H, kh, strides[0], dil[0])
+    ow, pl = same_lead(W, kw, strides[1], dil[1])
+    og = orc.conv_geom(shape, (kh, kw, Cin, O), strides, dil)
+    T_in = orc.QINT8 if signed_in else orc.QUINT8
+    st, acc = orc.qdepthwise_conv2d(orc.ConvAttrs(T_in, orc.QINT32, 0, orc.ACT_NONE, 0.0), og, x, w, None, -1.0, 1.0,
+                                    np.float32([-1]), np.float32([1]))
+    assert st == orc.OK and acc.shape == (B, oh, ow, O)
+    g = hip.ConvGeometry(B, H, W, Cin, kh, kw, oh, ow, strides[0], strides[1], dil[0], dil[1], pt, pl)
+    scales = (rng.random(O).astype(np.float32) + 0.5) * np.float32(2e-3)
+    bias = rng.standard_normal(O).astype(np.float32)
+    oep, ep = orc.EpilogueDesc(), hip.Epilogue()
+    oep.n_scales = ep.n_scales = O
+    oep.n_eltwise = ep.n_eltwise = 1
+    for e_ in (oep, ep):
+        e_.elt[0].alg, e_.elt[0].alpha, e_.elt[0].beta = orc.ELT_RELU, 0.0, 0.0
+    xd, wd = torch.from_numpy(x).to(dev), torch.from_numpy(w).to(dev)
+    sc_d, bi_d = torch.from_numpy(scales).to(dev), torch.from_numpy(bias).to(dev)
+    for T, dt in ((hip.QINT8, torch.int8), (hip.QUINT8, torch.uint8), (hip.FLOAT, torch.float32), (hip.BFLOAT16, torch.int16),
+                  (hip.QINT32, torch.int32)):
+        ref = orc.qmatmul_epilogue(acc.reshape(-1, O), oep, scales, bias, T)
+        out = torch.zeros((B * oh * ow, O), dtype=dt, device=dev)
+        hip.qdepthwise_conv2d(xd, T_in, g, mult, wd, sc_d, bi_d, ep, T, out)
+        torch.cuda.synchronize()
+        got = out.cpu().numpy()
+        np.testing.assert_array_equal(got.view(ref.dtype) if got.dtype != ref.dtype else got, ref)
+    # int32 accumulators themselves: no scales, no bias, no post-op
+    ep0 = hip.Epilogue()
+    out = torch.zeros((B * oh * ow, O), dtype=torch.int32, device=dev)
+    hip.qdepthwise_conv2d(xd, T_in, g, mult, wd, None, None, ep0, hip.QINT32, out)
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(out.cpu().numpy().reshape(acc.shape), acc)
+
+
 def test_implicit_gemm_conv_rejects_other_shapes(hip, dev):
     import torch
     x = torch.zeros(4 * 4 * 24 + 16, dtype=torch.uint8, device=dev)
@@ -333,8 +381,9 @@ def test_new_api_conv_through_plugin(rt, dev, t_in, fused, t_out, t_bias):
             b = rng.integers(-4000, 4000, wshape[3]).astype(np.int32) if has_bias else None
         else:
             b = rng.uniform(-1.0, 1.0, wshape[3]).astype(np.float32) if has_bias else None
-        attrs = dict(Tinput=DT(t_in), Tfilter=DT(tf.QINT8), Tbias=DT(t_bias), out_type=DT(t_out), strides=strides, padding=padding,
-                     dilations=dil, fused_ops=fused, alpha=0.2, data_format="NHWC", is_filter_const=True, is_bias_const=True)
+        attrs = dict(Tinput=DT(t_in), Tfilter=DT(tf.QINT8), Tbias=DT(t_bias), Tsummand=DT(t_out), out_type=DT(t_out), strides=strides,
+                     padding=padding, dilations=dil, fused_ops=fused, alpha=0.2, data_format="NHWC", is_filter_const=True,
+                     is_bias_const=True)
         if explicit:
             attrs["explicit_paddings"] = explicit
         node = tf.Node("_QuantizedConv2D", attrs)
@@ -409,9 +458,68 @@ def test_sum_fusions_through_plugin(rt, dev, op, t_sum, fused):
         node.close()
 
 
+@pytest.mark.parametrize("op,has_bias,relu,req", [("QuantizedDepthwiseConv2D", False, False, False),
+                                                  ("QuantizedDepthwiseConv2DWithBias", True, False, False),
+                                                  ("QuantizedDepthwiseConv2DWithBiasAndRelu", True, True, False),
+                                                  ("QuantizedDepthwiseConv2DWithBiasAndReluAndRequantize", True, True, True),
+                                                  ("_QuantizedDepthwiseConv2D", True, True, True),
+                                                  ("_QuantizedDepthwiseConv2D", True, False, False)])
+def test_depthwise_ops_through_plugin(rt, dev, op, has_bias, relu, req):
+    """Depthwise spellings (legacy and new API) against the oracle: multiplier 1 and 2, strides, per-channel filter ranges
+    (one per output channel c * multiplier + m)."""
+    torch = rt
+    new_api = op.startswith("_")
+    for shape, kshape, strides in (((2, 12, 11, 16), (3, 3, 16, 1), [1, 1, 1, 1]), ((1, 9, 9, 6), (3, 3, 6, 2), [1, 2, 2, 1])):
+        rng = np.random.default_rng(shape[3] + len(op))
+        x = rng.uniform(0.0, 4.0, shape).astype(np.float32)
+        w = rng.uniform(-1.0, 1.0, kshape).astype(np.float32)
+        O = kshape[2] * kshape[3]
+        b = rng.uniform(-1.0, 1.0, O).astype(np.float32) if has_bias else None
+        _, xq, xmn, xmx = orc.quantize_v2(x, x.min(), x.max(), orc.QUINT8, orc.SCALED)
+        xmn, xmx = np.array(xmn[0], np.float32), np.array(xmx[0], np.float32)
+        wf = w.reshape(kshape[0], kshape[1], O)          # ranges per output channel
+        mn, mx = wf.min(axis=(0, 1)).astype(np.float32), wf.max(axis=(0, 1)).astype(np.float32)
+        _, wq, fmn, fmx = orc.quantize_v2(wf, mn, mx, orc.QINT8, orc.SCALED, axis=2)
+        wq = wq.reshape(kshape)
+        if new_api and not req:
+            t_out = tf.FLOAT
+        else:
+            t_out = tf.QUINT8 if req else tf.QINT32
+        attrs = dict(Tinput=DT(tf.QUINT8), Tfilter=DT(tf.QINT8), out_type=DT(t_out), strides=strides, padding="SAME",
+                     dilations=[1, 1, 1, 1])
+        if new_api:
+            fused = (["BiasAdd"] if has_bias else []) + (["Relu"] if relu else []) + (["Requantize"] if req else ["Dequantize"])
+            attrs.update(Tbias=DT(tf.FLOAT), Tsummand=DT(t_out), fused_ops=fused, alpha=0.0, data_format="NHWC",
+                         is_filter_const=True, is_bias_const=True)
+        elif has_bias and req:
+            attrs["Tbias"] = DT(tf.FLOAT)
+        node = tf.Node(op, attrs)
+        assert node.code == tf.OK, node.message
+        zmn, zmx = np.array(0.0, np.float32), np.array(20.0, np.float32)
+        scalars = [xmn, xmx, fmn, fmx] + ([zmn, zmx] if req else [])
+        got, _res = run_conv(torch, dev, node, xq, wq, b, tf.FLOAT, scalars, t_out, NP[t_out], t_out != tf.FLOAT)
+        at = orc.ConvAttrs(orc.QUINT8, t_out, orc.FLOAT if has_bias else 0, orc.ACT_RELU if relu else orc.ACT_NONE, 0.0)
+        g = orc.conv_geom(shape, (kshape[0], kshape[1], kshape[2], O), strides[1:3])
+        st, ref = orc.qdepthwise_conv2d(at, g, xq, wq, b, float(xmn), float(xmx), fmn, fmx, float(zmn), float(zmx))
+        assert st == orc.OK
+        np.testing.assert_array_equal(got, ref)
+        if t_out == tf.FLOAT:       # and the fp32 depthwise convolution it stands for, within the quantization steps
+            pads = [(1, 1), (1, 1)] if strides[1] == 1 else [(1, 1), (1, 1)]
+            xp = np.pad(x, ((0, 0), pads[0], pads[1], (0, 0)))
+            oh, ow = ref.shape[1], ref.shape[2]
+            f = np.zeros(ref.shape, np.float64)
+            for i in range(3):
+                for j in range(3):
+                    win = xp[:, i:i + (oh - 1) * strides[1] + 1:strides[1], j:j + (ow - 1) * strides[2] + 1:strides[2], :]
+                    f += np.repeat(win, kshape[3], axis=3) * w[i, j].reshape(-1)
+            f += b if has_bias else 0
+            assert np.abs(got - f).max() < 0.3
+        node.close()
+
+
 def test_unsupported_fusions_and_formats(rt, dev):
-    base = dict(Tinput=DT(tf.QUINT8), Tfilter=DT(tf.QINT8), Tbias=DT(tf.FLOAT), out_type=DT(tf.FLOAT), strides=[1, 1, 1, 1],
-                padding="SAME", dilations=[1, 1, 1, 1], alpha=0.0)
+    base = dict(Tinput=DT(tf.QUINT8), Tfilter=DT(tf.QINT8), Tbias=DT(tf.FLOAT), Tsummand=DT(tf.FLOAT), out_type=DT(tf.FLOAT),
+                strides=[1, 1, 1, 1], padding="SAME", dilations=[1, 1, 1, 1], alpha=0.0)
     n = tf.Node("_QuantizedConv2D", dict(base, fused_ops=["BiasAdd", "Sum", "Relu", "Dequantize"]))
     assert n.code == tf.UNIMPLEMENTED and "Sum" in n.message
     n.close()

@@ -111,7 +111,9 @@ def test_every_renamed_op_has_a_kernel_and_an_op_definition(opt):
            "QuantizedReshape", "_QuantizedTranspose", "QuantizedConv2D", "QuantizedConv2DAndRequantize",
            "QuantizedConv2DPerChannel", "QuantizedConv2DWithBias", "QuantizedConv2DWithBiasAndRelu",
            "QuantizedConv2DWithBiasAndReluAndRequantize", "QuantizedConv2DWithBiasAndRequantize",
-           "QuantizedConv2DWithBiasSumAndReluAndRequantize", "QuantizedConv2DWithBiasSignedSumAndReluAndRequantize"]
+           "QuantizedConv2DWithBiasSumAndReluAndRequantize", "QuantizedConv2DWithBiasSignedSumAndReluAndRequantize",
+           "QuantizedDepthwiseConv2D", "QuantizedDepthwiseConv2DWithBias", "QuantizedDepthwiseConv2DWithBiasAndRelu",
+           "QuantizedDepthwiseConv2DWithBiasAndReluAndRequantize"]
     g = gd.GraphDef()
     for i, op in enumerate(ops):
         gd.node(g, "n%d" % i, op, ["x"], DEV, mode="SCALED", T=("type", QINT8))
@@ -135,6 +137,9 @@ def test_conv_rows(opt):
     assert out["c1"].attr["Tinput"].type == QUINT8 and list(out["c1"].input) == ["x", "w", "b"]
     assert out["c2"].op == "_ITEXQuantizedConv2DV2" and out["c2"].attr["padding"].s == b"VALID"
     assert out["c3"].op == "QuantizedConv2D" and "data_format" not in out["c3"].attr
+    g = gd.GraphDef()
+    gd.node(g, "d", "_QuantizedDepthwiseConv2D", ["x", "w"], DEV, Tinput=("type", QUINT8))
+    assert by_name(run(opt, g))["d"].op == "_ITEXQuantizedDepthwiseConv2DV2"
 
 
 def dynamic_range_graph(shape_vals=(-1,), shape_dims=(1,), axis_vals=(0,), axis_dims=(), keep_dims=False, q_axis=-1,

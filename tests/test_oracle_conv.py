@@ -236,3 +236,43 @@ def test_sum_fusion_type_rules():
     assert run(orc.QINT8, orc.QUINT8) == orc.INVALID_ARGUMENT      # quantized_conv_ops.h:213-218
     assert run(orc.QINT32, orc.QUINT8) == orc.UNIMPLEMENTED        # the qint32 form takes a float summand: not restated
     assert run(orc.QUINT8, orc.QINT8) == orc.OK
+
+
+@pytest.mark.parametrize("x_dtype", [np.uint8, np.int8])
+@pytest.mark.parametrize("shape,kshape,strides,dil", [((2, 7, 6, 8), (3, 3, 8, 1), (1, 1), (1, 1)), ((1, 9, 9, 5), (3, 3, 5, 2), (2, 2), (1, 1)),
+                                                      ((1, 8, 8, 4), (5, 3, 4, 3), (1, 2), (2, 1))])
+def test_depthwise_integer_convolution_against_numpy(x_dtype, shape, kshape, strides, dil):
+    """Depthwise: output channel c * mult + m is the plain convolution of input channel c with filter w[:, :, c, m]; checked
+    channel by channel against the independent numpy evaluation used for the full convolution."""
+    rng = np.random.default_rng(sum(shape) + sum(kshape))
+    info = np.iinfo(x_dtype)
+    x = rng.integers(info.min, info.max + 1, shape).astype(x_dtype)
+    w = rng.integers(-127, 128, kshape).astype(np.int8)
+    g = orc.conv_geom(shape, (kshape[0], kshape[1], kshape[2], kshape[2] * kshape[3]), strides, dil)
+    T_in = orc.QUINT8 if x_dtype == np.uint8 else orc.QINT8
+    st, got = orc.qdepthwise_conv2d(orc.ConvAttrs(T_in, orc.QINT32, 0, orc.ACT_NONE, 0.0), g, x, w, None, -1.0, 1.0,
+                                    np.float32([-1]), np.float32([1]))
+    assert st == orc.OK
+    pads = (same_pads(shape[1], kshape[0], strides[0], dil[0]), same_pads(shape[2], kshape[1], strides[1], dil[1]))
+    C_, mult = kshape[2], kshape[3]
+    assert got.shape[3] == C_ * mult
+    for c in range(C_):
+        for m in range(mult):
+            ref = ref_int_conv(x[..., c:c + 1], w[:, :, c:c + 1, m:m + 1], strides, dil, pads)
+            np.testing.assert_array_equal(got[..., c * mult + m], ref[..., 0])
+
+
+def test_depthwise_scales_follow_the_output_channel():
+    """Per-channel filter ranges: entry c * mult + m scales output channel c * mult + m (same prepare as the full
+    convolution with in_c * mult channels)."""
+    rng = np.random.default_rng(3)
+    x = rng.integers(0, 256, (1, 5, 5, 3)).astype(np.uint8)
+    w = rng.integers(-127, 128, (3, 3, 3, 2)).astype(np.int8)
+    g = orc.conv_geom(x.shape, (3, 3, 3, 6))
+    mn, mx = -np.arange(1, 7, dtype=np.float32), np.arange(1, 7, dtype=np.float32)
+    at = orc.ConvAttrs(orc.QUINT8, orc.FLOAT, 0, orc.ACT_NONE, 0.0)
+    st, got = orc.qdepthwise_conv2d(at, g, x, w, None, 0.0, 2.0, mn, mx)
+    st2, acc = orc.qdepthwise_conv2d(orc.ConvAttrs(orc.QUINT8, orc.QINT32, 0, orc.ACT_NONE, 0.0), g, x, w, None, 0.0, 2.0, mn, mx)
+    assert st == orc.OK and st2 == orc.OK
+    scale = (np.float32(2.0) / np.float32(255.0)) * (mx / np.float32(127.0))
+    np.testing.assert_array_equal(got, acc.astype(np.float32) * scale)

@@ -229,10 +229,20 @@ def test_conv_registrations(reg):
             assert {k["constraints"]["Tbias"] for k in ks} == {tf.FLOAT, tf.QINT32}, op
             assert all(k["constraints"]["Tinput"] == tf.QUINT8 and k["constraints"]["out_type"] == tf.QUINT8 and
                        k["constraints"]["Tsummand"] == t_sum and k["host_memory"] == sum_host for k in ks), op
-    for op in ("_QuantizedConv2D", "_ITEXQuantizedConv2DV2"):
+    for op in ("_QuantizedConv2D", "_ITEXQuantizedConv2DV2", "_QuantizedDepthwiseConv2D", "_ITEXQuantizedDepthwiseConv2DV2"):
         ks = kernels_of(reg, op)
         assert {k["constraints"]["out_type"] for k in ks} == {tf.QINT8, tf.QUINT8, tf.QINT32, tf.FLOAT, tf.BFLOAT16}
         assert all(k["host_memory"] == ["host_inputs", "host_outputs"] for k in ks)
+        # Tsummand as the reference constrains it: either 8-bit type under an 8-bit output, else the output's type
+        for k in ks:
+            out_t, sum_t = k["constraints"]["out_type"], k["constraints"]["Tsummand"]
+            assert sum_t in ((tf.QINT8, tf.QUINT8) if out_t in (tf.QINT8, tf.QUINT8) else (out_t,)), op
+    for name, outs in (("QuantizedDepthwiseConv2D", {tf.QINT32}), ("QuantizedDepthwiseConv2DWithBias", {tf.QINT32}),
+                       ("QuantizedDepthwiseConv2DWithBiasAndRelu", {tf.QINT32}),
+                       ("QuantizedDepthwiseConv2DWithBiasAndReluAndRequantize", {tf.QUINT8})):
+        for op in (name, "_ITEX" + name):
+            ks = kernels_of(reg, op)
+            assert ks and {k["constraints"]["out_type"] for k in ks} == outs and all(k["constraints"]["Tinput"] == tf.QUINT8 for k in ks), op
     # stock TensorFlow defines the legacy names and _QuantizedConv2D; the plugin must define the renamed ones only
     names = {o["name"] for o in reg["ops"]}
     assert "_ITEXQuantizedConv2DV2" in names and "_ITEXQuantizedConv2DWithBiasAndRequantize" in names
