@@ -374,7 +374,8 @@ def bench_mfma_ceiling(torch, hip, timer, xq, wq, dev):
     out = {}
     a_bytes = (xq.reshape(-1)[:4096] ^ 0x80).contiguous()
     w_bytes = wq.reshape(-1)[:4096].contiguous().view(torch.uint8)
-    for name, buf in (("workload_data", torch.cat([a_bytes, w_bytes])),
+    # weights in the first operand slot, activations in the second, as the MatMul kernels feed them
+    for name, buf in (("workload_data", torch.cat([w_bytes, a_bytes])),
                       ("constant_operands", torch.ones(8192, dtype=torch.uint8, device=dev))):
         ms = timer.run(lambda i: hip.mfma_probe(wgs, iters, buf, sink, st), 10, 2)
         out[name] = ops / (ms * 1e-3) / 1e12

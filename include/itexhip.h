@@ -400,9 +400,11 @@ int itexhip_qconv2d_sum(const void* x, int x_type, const itexhip_conv_geometry* 
                         const itexhip_epilogue* ep, const void* addend, int addend_type, int out_type, void* out,
                         void* stream);
 
-/* Diagnostic, no counterpart in the reference: `workgroups` x 4 wavefronts each issue iters x 8
+/* Diagnostic, no counterpart in the reference: `workgroups` x 4 wavefronts each issue iters (even) x 8
  * independent 32x32x32 i8 MFMAs (2 * 32768 ops each) on the 8 KiB of operand fragments at `operands`
- * (device memory, 16-byte aligned) and nothing else.  Timed by the caller, it gives the rate the matrix
+ * (device memory, 16-byte aligned: 4 KiB for the first MFMA operand, which the MatMul kernels use for the
+ * weights and keep for 4 consecutive MFMAs, then 4 KiB for the second, the activations, changed with
+ * every MFMA) and nothing else.  Timed by the caller, it gives the rate the matrix
  * cores sustain for that operand data on this device, the practical ceiling next to the published
  * peak.  `sink` takes 256 ints that are practically never written. */
 int itexhip_mfma_probe(int workgroups, int iters, const void* operands, int32_t* sink, void* stream);
