@@ -249,6 +249,46 @@ def test_depthwise_conv_against_oracle(hip, dev, shape, kshape, strides, dil, si
     np.testing.assert_array_equal(out.cpu().numpy().reshape(acc.shape), acc)
 
 
+def test_conv_empty_and_degenerate_extents(hip, dev, rt):
+    """Zero batch / zero output channels launch nothing and succeed; a window larger than the input under VALID gives
+    an empty output through the op (TensorFlow's rule: (in - eff + stride) / stride = 0); a 1x1 output position."""
+    import torch
+    torch_ = rt
+    x = torch.zeros(16 * 16, dtype=torch.uint8, device=dev)
+    ep = hip.Epilogue()
+    ep.n_scales = 1
+    one = torch.ones(16, dtype=torch.float32, device=dev)
+    out = torch.full((64,), 7, dtype=torch.int32, device=dev)
+    g0 = hip.ConvGeometry(0, 4, 4, 16, 3, 3, 4, 4, 1, 1, 1, 1, 1, 1)
+    hip.im2col8(x, g0, 144, out)                                       # no rows
+    hip.qdepthwise_conv2d(x, hip.QUINT8, g0, 1, x, one, one, ep, hip.QINT32, out)
+    torch.cuda.synchronize()
+    assert int(out.min()) == 7                                          # nothing written
+    # one output position: 3x3 window over a 3x3 input, VALID
+    rng = np.random.default_rng(0)
+    xs = rng.integers(0, 256, (1, 3, 3, 16)).astype(np.uint8)
+    ws = rng.integers(-127, 128, (3, 3, 16, 16)).astype(np.int8)
+    g1 = hip.ConvGeometry(1, 3, 3, 16, 3, 3, 1, 1, 1, 1, 1, 1, 0, 0)
+    packed = torch.empty(hip.qgemm_packed_bytes(144, 16), dtype=torch.int8, device=dev)
+    colsum = torch.empty(16, dtype=torch.int32, device=dev)
+    hip.qgemm_prepack_b(torch.from_numpy(ws.reshape(144, 16)).to(dev), False, 144, 16, packed, colsum)
+    acc = torch.zeros((1, 16), dtype=torch.int32, device=dev)
+    hip.qconv2d(torch.from_numpy(xs).to(dev), hip.QUINT8, g1, packed, colsum, 16, one[:1], torch.zeros(16, device=dev), ep,
+                hip.QINT32, acc)
+    torch_.cuda.synchronize()
+    np.testing.assert_array_equal(acc.cpu().numpy()[0], xs.reshape(-1).astype(np.int64) @ ws.reshape(144, 16).astype(np.int64))
+    # through the op: window larger than the input, VALID -> empty output, ranges still produced
+    node = tf.Node("QuantizedConv2D", dict(Tinput=DT(tf.QUINT8), Tfilter=DT(tf.QINT8), out_type=DT(tf.QINT32), strides=[1, 1, 1, 1],
+                                           padding="VALID", dilations=[1, 1, 1, 1]))
+    assert node.code == tf.OK, node.message
+    xq = np.zeros((2, 2, 2, 4), np.uint8)
+    wq = np.zeros((3, 3, 4, 8), np.int8)
+    s = [np.array(v, np.float32) for v in (0.0, 1.0, -1.0, 1.0)]
+    got, res = run_conv(torch_, dev, node, xq, wq, None, tf.FLOAT, s, tf.QINT32, np.int32, True)
+    assert got.shape == (2, 0, 0, 8)
+    node.close()
+
+
 def test_implicit_gemm_conv_rejects_other_shapes(hip, dev):
     import torch
     x = torch.zeros(4 * 4 * 24 + 16, dtype=torch.uint8, device=dev)
