@@ -297,7 +297,9 @@ def bench_conv(torch, hip, timer, steps, warmup, dev):
     g_ = torch.Generator(device=dev)
     g_.manual_seed(50)
     st = _stream(torch)
+    # (the first layer of ResNet-50 has 3 input channels: patch matrix, rows padded from 147 to 160 bytes)
     for name, (B, H, W, C), (KH, KW, O), stride, patches in (
+            ("conv7x7s2_224x224x3_to_64_patch_matrix", (32, 224, 224, 3), (7, 7, 64), 2, True),
             ("conv3x3_56x56x64_to_64", (32, 56, 56, 64), (3, 3, 64), 1, False),
             ("conv3x3_56x56x64_to_64_patch_matrix", (32, 56, 56, 64), (3, 3, 64), 1, True),
             ("conv3x3_28x28x128_to_128", (32, 28, 28, 128), (3, 3, 128), 1, False),
@@ -306,8 +308,10 @@ def bench_conv(torch, hip, timer, steps, warmup, dev):
         x = torch.randint(0, 256, (B, H, W, C), dtype=torch.uint8, device=dev, generator=g_)
         w = torch.randint(-127, 128, (KH * KW * C, O), dtype=torch.int8, device=dev, generator=g_)
         K = KH * KW * C
-        M = B * H * W
-        packed = torch.empty(hip.qgemm_packed_bytes(K, O), dtype=torch.int8, device=dev)
+        Kp = (K + 15) // 16 * 16
+        OH, OW = -(-H // stride), -(-W // stride)
+        M = B * OH * OW
+        packed = torch.empty(hip.qgemm_packed_bytes(Kp, O), dtype=torch.int8, device=dev)
         colsum = torch.empty(O, dtype=torch.int32, device=dev)
         hip.qgemm_prepack_b(w, False, K, O, packed, colsum, st)
         scales = torch.full((O,), 1e-4, dtype=torch.float32, device=dev)
@@ -316,9 +320,9 @@ def bench_conv(torch, hip, timer, steps, warmup, dev):
         ep.n_scales, ep.n_eltwise = O, 1
         ep.elt[0].alg, ep.elt[0].alpha, ep.elt[0].beta = hip.ELT_RELU, 0.0, 0.0
         y = torch.empty((M, O), dtype=torch.uint8, device=dev)
-        pad = (KH - 1) // 2
-        geo = hip.ConvGeometry(B, H, W, C, KH, KW, H, W, stride, stride, 1, 1, pad, pad)
-        cols = torch.empty((M, K), dtype=torch.uint8, device=dev) if patches else None
+        pad = max((OH - 1) * stride + KH - H, 0) // 2       # SAME: the smaller half leads
+        geo = hip.ConvGeometry(B, H, W, C, KH, KW, OH, OW, stride, stride, 1, 1, pad, pad)
+        cols = torch.empty((M, Kp), dtype=torch.uint8, device=dev) if patches else None
         implicit = KH * KW > 1 and not patches
         assert not implicit or hip.qconv2d_implicit_ok(geo, x, O, hip.QUINT8, y)
 
@@ -329,9 +333,9 @@ def bench_conv(torch, hip, timer, steps, warmup, dev):
                     return
                 a = x
                 if cols is not None:
-                    hip.im2col8(x, geo, K, cols, stream)
+                    hip.im2col8(x, geo, Kp, cols, stream)
                     a = cols
-                hip.qgemm(a, hip.QUINT8, packed, colsum, M, K, O, scales, bias, ep, hip.QUINT8, y, stream)
+                hip.qgemm(a, hip.QUINT8, packed, colsum, M, Kp, O, scales, bias, ep, hip.QUINT8, y, stream)
             return fn
         ms = timer.run_graph(make, steps, warmup)
         nbytes = x.numel() + w.numel() + y.numel()

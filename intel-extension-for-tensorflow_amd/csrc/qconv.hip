@@ -52,6 +52,51 @@ __global__ __launch_bounds__(256) void im2col8_kernel(const Im2colArgs a, const 
   }
 }
 
+// Few input channels (the first layer of a network: in_c = 3): every byte of a patch row may come from another pixel,
+// so the window offsets are tabulated per byte of the row once per workgroup (LDS), a thread decomposes only its row
+// index (32-bit), gathers its 4 bytes unconditionally from clamped positions and zeroes those in the padding.
+constexpr int kMaxRowBytesTable = 2048;
+__global__ __launch_bounds__(256) void im2col8_byte_kernel(const Im2colArgs a, const uint8_t* __restrict__ x,
+                                                           uint32_t* __restrict__ cols) {
+  __shared__ int t_dhw[kMaxRowBytesTable], t_off[kMaxRowBytesTable];  // (window row << 16 | window column), input byte offset
+  const itexhip_conv_geometry& g = a.g;
+  const int C = static_cast<int>(g.in_c), KW = static_cast<int>(g.k_w), W = static_cast<int>(g.in_w), H = static_cast<int>(g.in_h);
+  const uint32_t row_dwords = static_cast<uint32_t>(a.row_dwords);
+  for (uint32_t k = threadIdx.x; k < row_dwords * 4; k += blockDim.x) {
+    if (static_cast<int>(k) < a.K) {
+      const int c = k % C, kk = k / C, kw = kk % KW, kh = kk / KW;
+      t_dhw[k] = ((kh * g.dil_h) << 16) | (kw * g.dil_w);
+      t_off[k] = (kh * g.dil_h * W + kw * g.dil_w) * C + c;
+    } else {
+      t_dhw[k] = -1;  // zero tail of the row
+      t_off[k] = 0;
+    }
+  }
+  __syncthreads();
+  const uint32_t total = static_cast<uint32_t>(a.total);  // dwords; the host keeps this and the input below 2^31
+  const uint32_t OW = static_cast<uint32_t>(g.out_w), OH = static_cast<uint32_t>(g.out_h);
+  const uint32_t stride = gridDim.x * blockDim.x;
+  const int last = H * W * C * static_cast<int>(g.batch) - 1;
+  for (uint32_t i = blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
+    const uint32_t row = i / row_dwords, k0 = (i - row * row_dwords) * 4;
+    const uint32_t t = row / OW, ow = row - t * OW;
+    const uint32_t b = t / OH, oh = t - b * OH;
+    const int ih0 = static_cast<int>(oh) * g.stride_h - static_cast<int>(g.pad_top);
+    const int iw0 = static_cast<int>(ow) * g.stride_w - static_cast<int>(g.pad_left);
+    const int base = ((static_cast<int>(b) * H + ih0) * W + iw0) * C;
+    uint32_t v = 0;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const int dhw = t_dhw[k0 + e];
+      const int ih = ih0 + (dhw >> 16), iw = iw0 + (dhw & 0xffff);
+      const bool ok = dhw >= 0 && ih >= 0 && ih < H && iw >= 0 && iw < W;
+      const uint32_t byte = x[min(max(base + t_off[k0 + e], 0), last)];
+      v |= (ok ? byte : 0u) << (8 * e);
+    }
+    cols[i] = v;
+  }
+}
+
 // in_c a multiple of 16: every 16-byte vector of a patch row lies inside one input pixel.  The workgroup first
 // tabulates, per vector of the row, its offset inside the window (rows / columns to add to the window origin,
 // byte offset in the input), so that a thread only decomposes its row index.
@@ -421,6 +466,20 @@ extern "C" int itexhip_im2col8(const void* x, const itexhip_conv_geometry* g, in
     const int64_t vblocks = std::min<int64_t>((vecs + 255) / 256, 256 * 32);
     im2col8_vec_kernel<<<static_cast<unsigned>(vblocks), 256, 0, as_stream(stream)>>>(a, static_cast<const uint8_t*>(x),
                                                                                      static_cast<i4*>(cols));
+    ITEXHIP_CHECK_LAUNCH(who);
+    return ITEXHIP_OK;
+  }
+  // extremes of the 32-bit byte offsets the table kernel forms before clamping (window origins may lie in the padding)
+  const int64_t hi_off = ((g->batch * g->in_h + (g->out_h - 1) * g->stride_h - g->pad_top) * g->in_w + (g->out_w - 1) * g->stride_w -
+                          g->pad_left) * g->in_c + ((g->k_h - 1) * g->dil_h * g->in_w + (g->k_w - 1) * g->dil_w + 1) * g->in_c;
+  const int64_t lo_off = (g->pad_top * g->in_w + g->pad_left) * g->in_c;
+  if (!a.vec && hi_off < (1LL << 31) && lo_off < (1LL << 31) &&
+      row_bytes <= kMaxRowBytesTable && a.total < (1LL << 31) && in_bytes > 0 && in_bytes < (1LL << 31) &&
+      (g->k_h - 1) * g->dil_h < (1 << 15) && (g->k_w - 1) * g->dil_w < (1 << 15) && g->pad_top < (1 << 24) && g->pad_left < (1 << 24) &&
+      g->out_h * g->stride_h < (1LL << 30) && g->out_w * g->stride_w < (1LL << 30)) {
+    const int64_t bblocks = std::min<int64_t>((a.total + 255) / 256, 256 * 32);
+    im2col8_byte_kernel<<<static_cast<unsigned>(bblocks), 256, 0, as_stream(stream)>>>(a, static_cast<const uint8_t*>(x),
+                                                                                      static_cast<uint32_t*>(cols));
     ITEXHIP_CHECK_LAUNCH(who);
     return ITEXHIP_OK;
   }
