@@ -137,6 +137,7 @@ class QuantizedConv2DOp : public OpKernel {
                     "the quantized Conv2D takes a float or qint32 bias on this device");
     }
     if (ctx->HasAttr("is_filter_const")) ITEX_REQUIRES_OK(ctx, ctx->GetAttr("is_filter_const", &is_filter_const_));
+    if (ctx->HasAttr("is_bias_const")) ITEX_REQUIRES_OK(ctx, ctx->GetAttr("is_bias_const", &is_bias_const_));
 
     // input positions (:246-317)
     const int bias_off = fuse_bias_ ? 1 : 0;
@@ -259,25 +260,31 @@ class QuantizedConv2DOp : public OpKernel {
     if (!ctx->ok()) return;
     if (M > 0 && O > 0) {
       // ---- bias in the epilogue's units
-      Tensor sbias;
+      // A constant bias (is_bias_const, quantized_conv_ops.h:168-174, 448-455: the reference caches the scaled bias too) is
+      // scaled once and kept while its buffer and the factors stay the same; likewise the zero vector of a node without
+      // bias (the MFMA kernels' vector epilogue wants a bias vector).
       const float* bias_dev = nullptr;
+      const void* bias_src = nullptr;
       if (fuse_bias_) {
         Tensor bias = ctx->input(2);
         if (!ctx->ok()) return;
         ITEX_REQUIRES(ctx, bias.dtype() == t_bias_ && bias.NumElements() == O, TF_INVALID_ARGUMENT,
                       "bias must have one entry per output channel and the type of Tbias");
-        sbias = ctx->allocate_temp(TF_FLOAT, {O});
-        if (!ctx->ok()) return;
-        const int st = itexhip_scale_vector(bias.data(), t_bias_, params + depth, depth, O, sbias.flat<float>(), stream);
-        ITEX_REQUIRES(ctx, st == ITEXHIP_OK, TF_ABORTED, std::string("Operation received an exception: ") + itexhip_last_error());
-        bias_dev = sbias.flat<float>();
-      } else {
-        sbias = ctx->allocate_temp(TF_FLOAT, {O});   // the MFMA kernels' vector epilogue wants a bias vector: zeros
-        if (!ctx->ok()) return;
-        const int st = itexhip_memset32_async(sbias.data(), 0, static_cast<size_t>(O) * sizeof(float), stream);
-        ITEX_REQUIRES(ctx, st == ITEXHIP_OK, TF_ABORTED, std::string("Operation received an exception: ") + itexhip_last_error());
-        bias_dev = sbias.flat<float>();
+        bias_src = bias.data();
       }
+      const bool reuse = sbias_.valid() && sbias_n_ == O && sbias_src_ == bias_src && sbias_factors_ == factors &&
+                         (!fuse_bias_ || is_bias_const_);
+      if (!reuse) {
+        sbias_ = ctx->allocate_temp(TF_FLOAT, {O});
+        if (!ctx->ok()) return;
+        const int st = fuse_bias_ ? itexhip_scale_vector(bias_src, t_bias_, params + depth, depth, O, sbias_.flat<float>(), stream)
+                                  : itexhip_memset32_async(sbias_.data(), 0, static_cast<size_t>(O) * sizeof(float), stream);
+        ITEX_REQUIRES(ctx, st == ITEXHIP_OK, TF_ABORTED, std::string("Operation received an exception: ") + itexhip_last_error());
+        sbias_n_ = O;
+        sbias_src_ = bias_src;
+        sbias_factors_ = factors;
+      }
+      bias_dev = sbias_.flat<float>();
       itexhip_epilogue dep{};
       if (depthwise_) {  // no matrix product in it: a kernel of its own on the filter as TensorFlow stores it
         dep.n_scales = static_cast<int>(depth);
@@ -375,6 +382,11 @@ class QuantizedConv2DOp : public OpKernel {
   int activation_ = 0;
   float alpha_ = 0.0f;
   bool is_filter_const_ = true;
+  bool is_bias_const_ = true;   // the legacy ops have no such attribute: their bias is taken as constant (:168-174)
+  Tensor sbias_;
+  const void* sbias_src_ = nullptr;
+  int64_t sbias_n_ = -1;
+  std::vector<float> sbias_factors_;
   int src_min_idx_ = 2, filter_min_idx_ = 4, freezed_idx_ = 6;
   Tensor packed_, colsum_;
   const void* packed_src_ = nullptr;

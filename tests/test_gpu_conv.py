@@ -557,6 +557,38 @@ def test_depthwise_ops_through_plugin(rt, dev, op, has_bias, relu, req):
         node.close()
 
 
+def test_conv_cached_bias_follows_its_inputs(rt, dev):
+    """The op keeps the scaled bias of a constant-bias node; a bias at another address or other ranges (other scaling
+    factors) must still give that call's own result."""
+    torch = rt
+    rng = np.random.default_rng(5)
+    shape, wshape = (1, 8, 8, 16), (3, 3, 16, 16)
+    x = rng.uniform(0.0, 3.0, shape).astype(np.float32)
+    w = rng.uniform(-1.0, 1.0, wshape).astype(np.float32)
+    xq, xmn, xmx, wq, fmn, fmx = quantize_inputs(x, w, tf.QUINT8)
+    attrs = dict(Tinput=DT(tf.QUINT8), Tfilter=DT(tf.QINT8), Tbias=DT(tf.FLOAT), Tsummand=DT(tf.FLOAT), out_type=DT(tf.FLOAT),
+                 strides=[1, 1, 1, 1], padding="SAME", dilations=[1, 1, 1, 1], fused_ops=["BiasAdd", "Dequantize"], alpha=0.0,
+                 data_format="NHWC", is_filter_const=True, is_bias_const=True)
+    node = tf.Node("_QuantizedConv2D", attrs)
+    assert node.code == tf.OK, node.message
+    at = orc.ConvAttrs(orc.QUINT8, orc.FLOAT, orc.FLOAT, orc.ACT_NONE, 0.0)
+    g = orc.conv_geom(shape, wshape)
+    hold = []                                  # keep every device buffer alive so that addresses differ between calls
+    for bias, in_max in ((rng.uniform(-1, 1, 16).astype(np.float32), xmx), (rng.uniform(-1, 1, 16).astype(np.float32), xmx),
+                         (np.zeros(16, np.float32) + 0.5, np.array(float(xmx) * 2, np.float32))):
+        keep = [torch.from_numpy(np.ascontiguousarray(v)).to(dev) for v in (xq, wq, bias)]
+        hold.append(keep)
+        ins = [(tf.QUINT8, xq.shape, keep[0].data_ptr(), False), (tf.QINT8, wq.shape, keep[1].data_ptr(), False),
+               (tf.FLOAT, bias.shape, keep[2].data_ptr(), False)]
+        ins += [(tf.FLOAT, v.shape, tf.host_array(v), True) for v in (xmn, in_max, fmn, fmx)]
+        code, msg, res = node.run(ins, [(tf.FLOAT, False)], stream=torch.cuda.current_stream().cuda_stream)
+        assert code == tf.OK, msg
+        st, ref = orc.qconv2d(at, g, xq, wq, bias, float(xmn), float(in_max), fmn, fmx)
+        assert st == orc.OK
+        np.testing.assert_array_equal(fetch(torch, res[0], np.float32), ref)
+    node.close()
+
+
 def test_unsupported_fusions_and_formats(rt, dev):
     base = dict(Tinput=DT(tf.QUINT8), Tfilter=DT(tf.QINT8), Tbias=DT(tf.FLOAT), Tsummand=DT(tf.FLOAT), out_type=DT(tf.FLOAT),
                 strides=[1, 1, 1, 1], padding="SAME", dilations=[1, 1, 1, 1], alpha=0.0)
