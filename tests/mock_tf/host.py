@@ -1,5 +1,6 @@
 """Python driver of the mock TensorFlow host (tests/mock_tf/mock_tf.cc): loads the plugin the way
 TensorFlow does (dlopen + TF_InitKernel), instantiates kernels from node attributes and runs them."""
+import collections
 import ctypes as C
 import json
 import os
@@ -153,8 +154,13 @@ class DType(int):
     """Marks an integer attribute value as a TF_DataType."""
 
 
+_recent_host_arrays = collections.deque(maxlen=512)
+
+
 def host_array(a):
-    """(dtype-agnostic) address of a numpy array that the caller keeps alive."""
+    """(dtype-agnostic) address of a numpy array.  The last few hundred arrays passed here are kept alive, so that a
+    temporary handed over in a call expression cannot be freed (and its memory reused) before the op has read it."""
+    _recent_host_arrays.append(a)
     return a.ctypes.data
 
 

@@ -589,6 +589,64 @@ def test_conv_cached_bias_follows_its_inputs(rt, dev):
     node.close()
 
 
+def test_int8_bottleneck_block_end_to_end(rt, dev):
+    """A ResNet bottleneck block chained through the plugin's ops, every tensor between them quint8 on the device:
+    1x1 conv (plain GEMM) -> 3x3 conv (implicit GEMM) -> 1x1 conv + residual Sum + ReLU, each with bias and requantize;
+    the final tensor equals the same chain through the oracle."""
+    torch = rt
+    rng = np.random.default_rng(77)
+    B, H, W, C, Cm = 2, 14, 14, 64, 16
+    x = rng.uniform(0.0, 4.0, (B, H, W, C)).astype(np.float32)
+    _, xq, xmn, xmx = orc.quantize_v2(x, x.min(), x.max(), orc.QUINT8, orc.SCALED)
+    rng_in = (float(xmn[0]), float(xmx[0]))
+    layers = [((1, 1, C, Cm), 0, 6.0), ((3, 3, Cm, Cm), 0, 9.0), ((1, 1, Cm, C), 1, 12.0)]   # filter, sum position, frozen output max
+    cur_dev = torch.from_numpy(xq).to(dev)
+    cur_ref, cur_rng = xq, rng_in
+    keep = [cur_dev]
+    for wshape, sum_pos, zmax in layers:
+        w = rng.uniform(-0.5, 0.5, wshape).astype(np.float32)
+        b = rng.uniform(-0.5, 0.5, wshape[3]).astype(np.float32)
+        mn, mx = w.min(axis=(0, 1, 2)).astype(np.float32), w.max(axis=(0, 1, 2)).astype(np.float32)
+        _, wq, fmn, fmx = orc.quantize_v2(w, mn, mx, orc.QINT8, orc.SCALED, axis=3)
+        fused = ["BiasAdd"] + (["Sum"] if sum_pos else []) + ["Relu", "Requantize"]
+        attrs = dict(Tinput=DT(tf.QUINT8), Tfilter=DT(tf.QINT8), Tbias=DT(tf.FLOAT), Tsummand=DT(tf.QUINT8), out_type=DT(tf.QUINT8),
+                     strides=[1, 1, 1, 1], padding="SAME", dilations=[1, 1, 1, 1], fused_ops=fused, alpha=0.0, data_format="NHWC",
+                     is_filter_const=True, is_bias_const=True)
+        node = tf.Node("_QuantizedConv2D", attrs)
+        assert node.code == tf.OK, node.message
+        w_d, b_d = torch.from_numpy(wq).to(dev), torch.from_numpy(b).to(dev)
+        keep += [w_d, b_d]
+        def host(v):            # host scalars must outlive the call: keep the arrays
+            arr = np.array(v, np.float32)
+            keep.append(arr)
+            return (tf.FLOAT, (), tf.host_array(arr), True)
+        hostv = lambda v: (tf.FLOAT, v.shape, tf.host_array(v), True)
+        shape_in = tuple(cur_ref.shape)
+        ins = [(tf.QUINT8, shape_in, cur_dev.data_ptr(), False), (tf.QINT8, wq.shape, w_d.data_ptr(), False),
+               (tf.FLOAT, b.shape, b_d.data_ptr(), False)]
+        if sum_pos:
+            ins.append((tf.QUINT8, xq.shape, keep[0].data_ptr(), False))
+        ins += [host(cur_rng[0]), host(cur_rng[1]), hostv(fmn), hostv(fmx)]
+        if sum_pos:
+            ins += [host(rng_in[0]), host(rng_in[1])]
+        ins += [host(0.0), host(zmax)]
+        code, msg, res = node.run(ins, [(tf.QUINT8, False), (tf.FLOAT, True), (tf.FLOAT, True)],
+                                  stream=torch.cuda.current_stream().cuda_stream)
+        assert code == tf.OK, msg
+        got = fetch(torch, res[0], np.uint8)
+        at = orc.ConvAttrs(orc.QUINT8, orc.QUINT8, orc.FLOAT, orc.ACT_RELU, 0.0)
+        g = orc.conv_geom(shape_in, wshape)
+        kw = dict(sum=orc.ConvSum(1, orc.QUINT8, rng_in[0], rng_in[1]), summand=xq) if sum_pos else {}
+        st, ref = orc.qconv2d(at, g, cur_ref, wq, b, cur_rng[0], cur_rng[1], fmn, fmx, 0.0, zmax, **kw)
+        assert st == orc.OK
+        np.testing.assert_array_equal(got, ref, err_msg="layer %s" % (wshape,))
+        assert len(np.unique(got)) > 8
+        cur_ref, cur_rng = ref, (0.0, zmax)
+        cur_dev = torch.from_numpy(got).to(dev)       # the next op reads the device tensor this one produced
+        keep.append(cur_dev)
+        node.close()
+
+
 def test_unsupported_fusions_and_formats(rt, dev):
     base = dict(Tinput=DT(tf.QUINT8), Tfilter=DT(tf.QINT8), Tbias=DT(tf.FLOAT), Tsummand=DT(tf.FLOAT), out_type=DT(tf.FLOAT),
                 strides=[1, 1, 1, 1], padding="SAME", dilations=[1, 1, 1, 1], alpha=0.0)
