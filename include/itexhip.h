@@ -352,10 +352,12 @@ int itexhip_transpose(const void* x, void* y, int elem_size, int rank, const int
 /* ---- quantized Conv2D --------------------------------------------------------------------------
  * The quantized convolutions (QuantizedConv2D*, _QuantizedConv2D; itex/core/kernels/common/
  * quantized_conv_ops.h:63-597 over the oneDNN convolution primitive, conv_ops.h:615-1150) run here as
- * patch matrix x prepacked filter: itexhip_im2col8 lays the receptive field of every output position out as
- * one row, k = (kh * KW + kw) * C + c, which is the row order of the HWIO filter read as a [KH*KW*C, O] matrix,
- * so itexhip_qgemm_prepack_b packs the filter as it is and itexhip_qgemm does the rest.  Quantization is
- * SCALED (zero points are 0): padding positions hold the integer 0. */
+ * patch matrix x prepacked filter.  The receptive field of an output position is one row of the patch matrix,
+ * k = (kh * KW + kw) * C + c, which is the row order of the HWIO filter read as a [KH*KW*C, O] matrix, so
+ * itexhip_qgemm_prepack_b packs the filter as it is.  itexhip_qconv2d (below) never builds the patch matrix: the
+ * MatMul kernel gathers its rows from the input; itexhip_im2col8 writes it out for the shapes that kernel does
+ * not take, and itexhip_qgemm does the rest.  Quantization is SCALED (zero points are 0): padding positions hold
+ * the integer 0. */
 typedef struct {
   int64_t batch, in_h, in_w, in_c;   /* NHWC input */
   int64_t k_h, k_w;                  /* filter window */
