@@ -171,11 +171,16 @@ enum {
   ITEXHIP_API_LEGACY = 2  /* QuantizedMatMulOp / QuantizedMatMulReluOp (:1412-1531) */
 };
 enum { ITEXHIP_ACT_NONE = 0, ITEXHIP_ACT_RELU = 1, ITEXHIP_ACT_RELU6 = 2, ITEXHIP_ACT_LEAKYRELU = 3,
-       ITEXHIP_ACT_GELU_APPROX = 4, ITEXHIP_ACT_GELU_EXACT = 5 };
+       ITEXHIP_ACT_GELU_APPROX = 4, ITEXHIP_ACT_GELU_EXACT = 5,
+       /* "Elu", "Sigmoid", "Tanh", "_ITEXSwish", "_ITEXMish" of the post-op table (onednn_post_op_util.cc:34-68) */
+       ITEXHIP_ACT_ELU = 6, ITEXHIP_ACT_SIGMOID = 7, ITEXHIP_ACT_TANH = 8, ITEXHIP_ACT_SWISH = 9, ITEXHIP_ACT_MISH = 10 };
 /* post-ops of the epilogue chain (itex/core/utils/onednn/onednn_post_op_util.cc:34-68); SUM is the
  * "Add" fusion: y += alpha * addend[m, n] */
 enum { ITEXHIP_ELT_RELU = 1, ITEXHIP_ELT_CLIP = 2, ITEXHIP_ELT_LINEAR = 3, ITEXHIP_ELT_GELU_TANH = 4,
-       ITEXHIP_ELT_GELU_ERF = 5, ITEXHIP_ELT_SUM = 6 };
+       ITEXHIP_ELT_GELU_ERF = 5, ITEXHIP_ELT_SUM = 6,
+       /* oneDNN eltwise_elu (x > 0 ? x : alpha (e^x - 1)), eltwise_logistic (1 / (1 + e^-x)), eltwise_tanh,
+        * eltwise_swish (x / (1 + e^(-alpha x))), eltwise_mish (x tanh(ln(1 + e^x))) */
+       ITEXHIP_ELT_ELU = 7, ITEXHIP_ELT_LOGISTIC = 8, ITEXHIP_ELT_TANH = 9, ITEXHIP_ELT_SWISH = 10, ITEXHIP_ELT_MISH = 11 };
 
 typedef struct {
   int alg;      /* ITEXHIP_ELT_* */

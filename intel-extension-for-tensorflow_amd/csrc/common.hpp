@@ -126,6 +126,22 @@ __device__ __forceinline__ float apply_eltwise(const itexhip_eltwise& e, float x
     }
     case ITEXHIP_ELT_GELU_ERF:  // 0.5 x (1 + erf(x / sqrt(2)))
       return 0.5f * x * (1.0f + erff(x * 0.707106769084930419921875f));
+    // The exponential-based ones go through the hardware exp2 and reciprocal (about 1 ulp each), in forms that neither
+    // overflow nor cancel: a few 1e-7 from the libm evaluation, like the GELU above.
+    case ITEXHIP_ELT_ELU:  // x > 0 ? x : alpha (e^x - 1)
+      return x > 0.0f ? x : e.alpha * expm1f(x);
+    case ITEXHIP_ELT_LOGISTIC:  // 1 / (1 + e^-x)
+      return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(x * -1.44269502162933349609375f));
+    case ITEXHIP_ELT_TANH:  // 1 - 2 / (1 + e^(2x)): e^(2x) = inf gives 1, 0 gives -1
+      return 1.0f - 2.0f * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(x * 2.885390043258667f));
+    case ITEXHIP_ELT_SWISH:  // x / (1 + e^(-alpha x))
+      return x * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(e.alpha * x * -1.44269502162933349609375f));
+    case ITEXHIP_ELT_MISH: {  // x tanh(ln(1 + e^x)) = x t / (t + 2), t = e^x (e^x + 2); x beyond 20: tanh(.) = 1 in fp32
+      if (x > 20.0f) return x;
+      const float n = __builtin_amdgcn_exp2f(x * 1.44269502162933349609375f);
+      const float t = n * (n + 2.0f);
+      return x * t * __builtin_amdgcn_rcpf(t + 2.0f);
+    }
     default:
       return x;
   }

@@ -24,13 +24,15 @@ constexpr int64_t kMaxK = 1 << 16; // 255 * 128 * 65536 < 2^31
 // (every chain the MatMul and convolution ops build): resolved once on the host, so that the tile kernels apply it with a few
 // wavefront-uniform branches per 32x32 tile instead of a loop over the chain per value.
 enum : int { kChainMax0 = 1, kChainLeaky = 2, kChainClip = 4, kChainLinear = 8, kChainGeluTanh = 16, kChainGeluErf = 32,
-             kChainSumFirst = 64, kChainSumLast = 128 };  // y += sum_scale * addend before / after the activation
+             kChainSumFirst = 64, kChainSumLast = 128,  // y += sum_scale * addend before / after the activation
+             kChainOther = 256 };                       // another transcendental activation: `other`
 struct CanonChain {
   int flags;
   float alpha;         // leaky slope
   float lo, hi;        // clip bounds
   float lin_a, lin_b;  // y = lin_a * x + lin_b
   float sum_scale;
+  itexhip_eltwise other;  // kChainOther: ELU, logistic, tanh, swish, mish (with its alpha)
 };
 
 struct EpilogueArgs {
@@ -83,6 +85,9 @@ inline int canon_chain(const EpilogueArgs& e, CanonChain* c) {
     } else if (a.alg == ITEXHIP_ELT_GELU_TANH || a.alg == ITEXHIP_ELT_GELU_ERF) {
       c->flags |= a.alg == ITEXHIP_ELT_GELU_TANH ? kChainGeluTanh : kChainGeluErf;
       ++k;
+    } else if (a.alg >= ITEXHIP_ELT_ELU && a.alg <= ITEXHIP_ELT_MISH) {
+      c->flags |= kChainOther; c->other = a;
+      ++k;
     }
   }
   if (k < e.n_eltwise && e.elt[k].alg == ITEXHIP_ELT_SUM && !(c->flags & kChainSumFirst)) {
@@ -96,7 +101,7 @@ inline int canon_chain(const EpilogueArgs& e, CanonChain* c) {
   if (k != e.n_eltwise) return -1;
   if (c->flags == 0) return 0;
   if (c->flags == kChainMax0) return 1;
-  return (c->flags & (kChainGeluTanh | kChainGeluErf)) ? 3 : 2;
+  return (c->flags & (kChainGeluTanh | kChainGeluErf | kChainOther)) ? 3 : 2;
 }
 
 // Scale, bias and zero-point compensation of channel n (n < N), however the call supplied them, in two

@@ -331,7 +331,8 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void qgemm_tile_kernel(
   if constexpr (!GENERAL) {
     uint8_t* ebuf = lds + wave * (WM * PITCH);
     const int f_row = lane / LPR, f_piece = lane % LPR;
-    // Post-op chain in canonical form (ACT == 2: cheap activation, ACT == 3: GELU; then an optional linear map),
+    // Post-op chain in canonical form (ACT == 2: cheap activation, ACT == 3: GELU or another transcendental one; then
+    // an optional linear map),
     // applied to the 16 values of one 32x32 tile at a time under wavefront-uniform branches.  A loop over the chain
     // with a switch per value made the epilogue several times longer than the whole K loop (instruction fetch, not
     // arithmetic).  Same expressions as apply_eltwise.
@@ -372,10 +373,44 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void qgemm_tile_kernel(
           const itexhip_eltwise el{ITEXHIP_ELT_GELU_TANH, 0.0f, 0.0f};
 #pragma unroll
           for (int r = 0; r < 16; ++r) v[r] = apply_eltwise(el, v[r]);
-        } else {
+        } else if (c.flags & kChainGeluErf) {
           const itexhip_eltwise el{ITEXHIP_ELT_GELU_ERF, 0.0f, 0.0f};
 #pragma unroll
           for (int r = 0; r < 16; ++r) v[r] = apply_eltwise(el, v[r]);
+        } else {  // one of the other transcendental ones: a uniform switch around each 16-value loop
+          const float al = c.other.alpha;
+          switch (c.other.alg) {
+            case ITEXHIP_ELT_ELU: {
+              const itexhip_eltwise el{ITEXHIP_ELT_ELU, al, 0.0f};
+#pragma unroll
+              for (int r = 0; r < 16; ++r) v[r] = apply_eltwise(el, v[r]);
+              break;
+            }
+            case ITEXHIP_ELT_LOGISTIC: {
+              const itexhip_eltwise el{ITEXHIP_ELT_LOGISTIC, al, 0.0f};
+#pragma unroll
+              for (int r = 0; r < 16; ++r) v[r] = apply_eltwise(el, v[r]);
+              break;
+            }
+            case ITEXHIP_ELT_TANH: {
+              const itexhip_eltwise el{ITEXHIP_ELT_TANH, al, 0.0f};
+#pragma unroll
+              for (int r = 0; r < 16; ++r) v[r] = apply_eltwise(el, v[r]);
+              break;
+            }
+            case ITEXHIP_ELT_SWISH: {
+              const itexhip_eltwise el{ITEXHIP_ELT_SWISH, al, 0.0f};
+#pragma unroll
+              for (int r = 0; r < 16; ++r) v[r] = apply_eltwise(el, v[r]);
+              break;
+            }
+            default: {
+              const itexhip_eltwise el{ITEXHIP_ELT_MISH, al, 0.0f};
+#pragma unroll
+              for (int r = 0; r < 16; ++r) v[r] = apply_eltwise(el, v[r]);
+              break;
+            }
+          }
         }
       } else {
         if (c.flags & kChainMax0) {

@@ -32,6 +32,11 @@ int eltwise_from_activation(int act, itexhip_eltwise* e) {
     case ITEXHIP_ACT_LEAKYRELU: *e = {ITEXHIP_ELT_RELU, 0.0f, 0.0f}; return 1;
     case ITEXHIP_ACT_GELU_APPROX: *e = {ITEXHIP_ELT_GELU_TANH, 0.0f, 0.0f}; return 1;
     case ITEXHIP_ACT_GELU_EXACT: *e = {ITEXHIP_ELT_GELU_ERF, 0.0f, 0.0f}; return 1;
+    case ITEXHIP_ACT_ELU: *e = {ITEXHIP_ELT_ELU, 1.0f, 0.0f}; return 1;
+    case ITEXHIP_ACT_SIGMOID: *e = {ITEXHIP_ELT_LOGISTIC, 1.0f, 0.0f}; return 1;
+    case ITEXHIP_ACT_TANH: *e = {ITEXHIP_ELT_TANH, 0.0f, 0.0f}; return 1;
+    case ITEXHIP_ACT_SWISH: *e = {ITEXHIP_ELT_SWISH, 1.0f, 0.0f}; return 1;
+    case ITEXHIP_ACT_MISH: *e = {ITEXHIP_ELT_MISH, 0.0f, 0.0f}; return 1;
     default: return 0;
   }
 }

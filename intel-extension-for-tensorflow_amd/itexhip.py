@@ -15,7 +15,9 @@ FLOAT, INT32, QINT8, QUINT8, QINT32, BFLOAT16, HALF = 1, 3, 11, 12, 13, 14, 19
 MIN_COMBINED, MIN_FIRST, SCALED = 0, 1, 2
 API_V2, API_V1, API_LEGACY = 0, 1, 2
 ACT_NONE, ACT_RELU, ACT_RELU6, ACT_LEAKYRELU, ACT_GELU_APPROX, ACT_GELU_EXACT = 0, 1, 2, 3, 4, 5
+ACT_ELU, ACT_SIGMOID, ACT_TANH, ACT_SWISH, ACT_MISH = 6, 7, 8, 9, 10
 ELT_RELU, ELT_CLIP, ELT_LINEAR, ELT_GELU_TANH, ELT_GELU_ERF, ELT_SUM = 1, 2, 3, 4, 5, 6
+ELT_ELU, ELT_LOGISTIC, ELT_TANH, ELT_SWISH, ELT_MISH = 7, 8, 9, 10, 11
 
 EXPORTS = [
     "itexhip_device_count", "itexhip_device_info", "itexhip_mem_info", "itexhip_malloc", "itexhip_free",

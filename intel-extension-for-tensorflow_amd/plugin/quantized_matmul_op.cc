@@ -40,6 +40,11 @@ int ActivationFromName(const std::string& n) {
   if (n == "LeakyRelu") return ITEXHIP_ACT_LEAKYRELU;
   if (n == "GeluApproximate") return ITEXHIP_ACT_GELU_APPROX;
   if (n == "GeluExact") return ITEXHIP_ACT_GELU_EXACT;
+  if (n == "Elu") return ITEXHIP_ACT_ELU;
+  if (n == "Sigmoid") return ITEXHIP_ACT_SIGMOID;
+  if (n == "Tanh") return ITEXHIP_ACT_TANH;
+  if (n == "_ITEXSwish") return ITEXHIP_ACT_SWISH;
+  if (n == "_ITEXMish") return ITEXHIP_ACT_MISH;
   return -1;
 }
 

@@ -290,6 +290,11 @@ static int eltwise_from_activation(int act, orc_eltwise* e) {
     case ORC_ACT_LEAKYRELU: e->alg = ORC_ELT_RELU; e->alpha = 0.0f; e->beta = 0.0f; return 1;
     case ORC_ACT_GELU_APPROX: e->alg = ORC_ELT_GELU_TANH; e->alpha = 0.0f; e->beta = 0.0f; return 1;
     case ORC_ACT_GELU_EXACT: e->alg = ORC_ELT_GELU_ERF; e->alpha = 0.0f; e->beta = 0.0f; return 1;
+    case ORC_ACT_ELU: e->alg = ORC_ELT_ELU; e->alpha = 1.0f; e->beta = 0.0f; return 1;          /* "Elu", kAlphaOne */
+    case ORC_ACT_SIGMOID: e->alg = ORC_ELT_LOGISTIC; e->alpha = 1.0f; e->beta = 0.0f; return 1; /* "Sigmoid", kAlphaOne */
+    case ORC_ACT_TANH: e->alg = ORC_ELT_TANH; e->alpha = 0.0f; e->beta = 0.0f; return 1;        /* "Tanh" */
+    case ORC_ACT_SWISH: e->alg = ORC_ELT_SWISH; e->alpha = 1.0f; e->beta = 0.0f; return 1;      /* "_ITEXSwish", kAlphaOne */
+    case ORC_ACT_MISH: e->alg = ORC_ELT_MISH; e->alpha = 0.0f; e->beta = 0.0f; return 1;        /* "_ITEXMish" */
     default: return 0;
   }
 }
@@ -565,6 +570,13 @@ static inline float apply_eltwise(const orc_eltwise* e, float x) {
     }
     case ORC_ELT_GELU_ERF: /* eltwise_gelu_erf: 0.5 x (1 + erf(x / sqrt(2))) */
       return 0.5f * x * (1.0f + erff(x * 0.707106769084930419921875f));
+    /* oneDNN's reference forms of the other transcendental post-ops, in fp32 with libm (its own kernels evaluate
+     * them with polynomial approximations: parity unpinned at the last bits, as for the GELUs) */
+    case ORC_ELT_ELU: return x > 0.0f ? x : e->alpha * expm1f(x);
+    case ORC_ELT_LOGISTIC: return 1.0f / (1.0f + expf(-x));
+    case ORC_ELT_TANH: return tanhf(x);
+    case ORC_ELT_SWISH: return x / (1.0f + expf(-e->alpha * x));
+    case ORC_ELT_MISH: return x * tanhf(log1pf(expf(x)));
     default: return x;
   }
 }

@@ -64,10 +64,11 @@ enum {
 
 /* eltwise post-op algorithms (subset of onednn_post_op_util.cc:34-68) */
 enum { ORC_ELT_RELU = 1, ORC_ELT_CLIP = 2, ORC_ELT_LINEAR = 3, ORC_ELT_GELU_TANH = 4, ORC_ELT_GELU_ERF = 5,
-       ORC_ELT_SUM = 6 /* the "Add" post-op: y += alpha * addend[m,n] (append_sum, :256) */ };
+       ORC_ELT_SUM = 6, /* the "Add" post-op: y += alpha * addend[m,n] (append_sum, :256) */
+       ORC_ELT_ELU = 7, ORC_ELT_LOGISTIC = 8, ORC_ELT_TANH = 9, ORC_ELT_SWISH = 10, ORC_ELT_MISH = 11 };
 /* activation names accepted in fused_ops */
 enum { ORC_ACT_NONE = 0, ORC_ACT_RELU = 1, ORC_ACT_RELU6 = 2, ORC_ACT_LEAKYRELU = 3, ORC_ACT_GELU_APPROX = 4,
-       ORC_ACT_GELU_EXACT = 5 };
+       ORC_ACT_GELU_EXACT = 5, ORC_ACT_ELU = 6, ORC_ACT_SIGMOID = 7, ORC_ACT_TANH = 8, ORC_ACT_SWISH = 9, ORC_ACT_MISH = 10 };
 
 typedef struct {
   int alg;

@@ -16,6 +16,7 @@ FLOAT, INT32, QINT8, QUINT8, QINT32, BFLOAT16, HALF = 1, 3, 11, 12, 13, 14, 19
 MIN_COMBINED, MIN_FIRST, SCALED = 0, 1, 2
 API_V2, API_V1, API_LEGACY = 0, 1, 2
 ACT_NONE, ACT_RELU, ACT_RELU6, ACT_LEAKYRELU, ACT_GELU_APPROX, ACT_GELU_EXACT = 0, 1, 2, 3, 4, 5
+ACT_ELU, ACT_SIGMOID, ACT_TANH, ACT_SWISH, ACT_MISH = 6, 7, 8, 9, 10
 OK, INVALID_ARGUMENT, UNIMPLEMENTED = 0, 3, 12
 
 NP_OF = {QINT8: np.int8, QUINT8: np.uint8, QINT32: np.int32, FLOAT: np.float32, BFLOAT16: np.uint16, HALF: np.uint16}
@@ -246,6 +247,7 @@ class BmmBinary(C.Structure):
 
 BIN_MUL, BIN_ADD = 1, 2
 ELT_RELU, ELT_CLIP, ELT_LINEAR, ELT_GELU_TANH, ELT_GELU_ERF, ELT_SUM = 1, 2, 3, 4, 5, 6
+ELT_ELU, ELT_LOGISTIC, ELT_TANH, ELT_SWISH, ELT_MISH = 7, 8, 9, 10, 11
 
 
 def qbatch_matmul(x, y, min_x, max_x, min_y, max_y, adj_x=False, adj_y=False, binary=(), t_out=FLOAT):

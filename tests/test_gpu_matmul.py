@@ -245,6 +245,11 @@ CHAINS = {   # post-op chains of the form [activation] [linear map] that the vec
     "req_minfirst_s8": dict(V2_REQ_S8, out_min_first=True),                 # the linear map alone
     "gelu_tanh_f32": dict(V2_DEQ, activation=orc.ACT_GELU_APPROX),
     "gelu_erf_bf16": dict(V2_DEQ, activation=orc.ACT_GELU_EXACT, t_out=orc.BFLOAT16),
+    "transc_tanh_f32": dict(V2_DEQ, activation=orc.ACT_TANH),
+    "transc_sigmoid_f32": dict(V2_DEQ, activation=orc.ACT_SIGMOID),
+    "transc_swish_f32": dict(V2_DEQ, activation=orc.ACT_SWISH),
+    "transc_elu_f32": dict(V2_DEQ, activation=orc.ACT_ELU),
+    "transc_mish_bf16": dict(V2_DEQ, activation=orc.ACT_MISH, t_out=orc.BFLOAT16),
 }
 
 
@@ -252,8 +257,8 @@ CHAINS = {   # post-op chains of the form [activation] [linear map] that the vec
 @pytest.mark.parametrize("chain", sorted(CHAINS))
 def test_canonical_chains_every_tile_shape(hip, dev, monkeypatch, shape, chain):
     """Every tile shape with every kind of run-time post-op chain, K a multiple of 64 (uniform activation addresses)
-    and not (per-lane clamped addresses), ragged M and N: bit-equal to the oracle except for the GELU chains, where
-    the device's tanhf / erff need not round like the host's (2e-6 relative, 1e-6 absolute; one unit of the
+    and not (per-lane clamped addresses), ragged M and N: bit-equal to the oracle except for the GELU and the other
+    transcendental chains, where the device's exp / erf need not round like the host's (2e-6 relative, 1e-6 absolute; one unit of the
     output type where that is coarser)."""
     monkeypatch.setenv("ITEXHIP_TILE_SHAPE", str(shape))
     kw = CHAINS[chain]
@@ -265,7 +270,7 @@ def test_canonical_chains_every_tile_shape(hip, dev, monkeypatch, shape, chain):
         ref = layer.oracle(xq, kw, mn, mx, lo, r_out)
         for path in ("tile", "fused"):
             got = layer.run(xq, kw, mn, mx, lo, r_out, path=path)
-            if "gelu" not in chain:
+            if "gelu" not in chain and "transc" not in chain:
                 np.testing.assert_array_equal(got, ref)
             elif kw["t_out"] == orc.FLOAT:
                 np.testing.assert_allclose(got, ref, rtol=2e-6, atol=1e-6)

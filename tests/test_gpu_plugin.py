@@ -140,6 +140,26 @@ def test_dynamic_range_quantize_through_plugin(rt, dev, T, mode, classic):
         node.close()
 
 
+@pytest.mark.parametrize("fused,act", [("Tanh", orc.ACT_TANH), ("Sigmoid", orc.ACT_SIGMOID), ("_ITEXSwish", orc.ACT_SWISH)])
+def test_quantized_matmul_transcendental_post_ops(rt, dev, fused, act):
+    """_QuantizedMatMul [BiasAdd, Tanh | Sigmoid | _ITEXSwish, Dequantize] (a BERT pooler, gates): within 2e-6 of the oracle
+    (the device evaluates exp with the hardware instruction)."""
+    torch = rt
+    M, K, N = 50, 256, 96
+    x, w, bias, xq, xmn, xmx, wq, wmn, wmx = make_problem(M, K, N, seed=act)
+    node = tf.Node("_QuantizedMatMul", dict(V2, Tout=DT(tf.FLOAT), fused_ops=["BiasAdd", fused, "Dequantize"]))
+    assert node.code == tf.OK, node.message
+    at = orc.matmul_attrs(api=orc.API_V2, t_in=orc.QUINT8, t_out=orc.FLOAT, input_mode=orc.MIN_FIRST, has_dequantize=True,
+                          activation=act)
+    st, ref = orc.qmatmul(at, xq, wq, bias, xmn, xmx, wmn, wmx)
+    assert st == orc.OK
+    ins, keep = matmul_inputs(torch, dev, xq, wq, bias, [xmn, xmx, wmn, wmx])
+    code, msg, outs = node.run(ins, [(tf.FLOAT, False)], stream=torch.cuda.current_stream().cuda_stream)
+    assert code == tf.OK, msg
+    np.testing.assert_allclose(fetch(torch, outs[0], np.float32), ref, rtol=2e-6, atol=1e-6)
+    node.close()
+
+
 def test_dequantize_through_plugin(rt, dev):
     torch = rt
     rng = np.random.default_rng(1)

@@ -526,3 +526,27 @@ def test_bfloat16_bias_is_adjusted_in_fp32_and_stored_as_bfloat16(mode, t_out, T
     assert st == orc.OK
     np.testing.assert_array_equal(sb16, _widen(_bf16_rne(sb32, T16), T16))
     assert not np.array_equal(sb16, sb32)
+
+
+@pytest.mark.parametrize("act,f", [
+    (orc.ACT_ELU, lambda x: np.where(x > 0, x, np.expm1(x))),
+    (orc.ACT_SIGMOID, lambda x: 1.0 / (1.0 + np.exp(-x))),
+    (orc.ACT_TANH, np.tanh),
+    (orc.ACT_SWISH, lambda x: x / (1.0 + np.exp(-x))),
+    (orc.ACT_MISH, lambda x: x * np.tanh(np.log1p(np.exp(x))))])
+def test_transcendental_post_ops_against_float64(act, f):
+    """Elu / Sigmoid / Tanh / _ITEXSwish / _ITEXMish of the post-op table (onednn_post_op_util.cc:34-68, alpha 1 where the
+    table says kAlphaOne): the oracle's fp32 libm evaluation against the textbook formula in float64."""
+    rng = np.random.default_rng(act)
+    M, K, N = 9, 64, 40
+    a = rng.integers(0, 256, (M, K)).astype(np.uint8)
+    w = rng.integers(-127, 128, (K, N)).astype(np.int8)
+    bias = rng.standard_normal(N).astype(np.float32)
+    kw = dict(api=orc.API_V2, t_in=orc.QUINT8, t_out=orc.FLOAT, input_mode=orc.SCALED, has_dequantize=True)
+    st, lin = orc.qmatmul(orc.matmul_attrs(**kw), a, w, bias, 0.0, 6.0, np.float32(-1.5), np.float32(1.5))
+    st2, got = orc.qmatmul(orc.matmul_attrs(activation=act, **kw), a, w, bias, 0.0, 6.0, np.float32(-1.5), np.float32(1.5))
+    assert st == orc.OK and st2 == orc.OK
+    assert lin.min() < -3 and lin.max() > 3          # both tails of every function are exercised
+    with np.errstate(over="ignore"):                  # e^x overflows to inf in the far tails, as the formulas allow
+        want = f(lin.astype(np.float64))
+    np.testing.assert_allclose(got, want, rtol=2e-6, atol=1e-6)
