@@ -119,8 +119,8 @@ def make_weights(torch, hip, K, N, seed, dev):
 
 
 def make_acts(torch, hip, M, K, seed, dev, outlier_frac=0.0, outlier_mult=1.0):
-    """fp32 N(0,1) activations (+ outliers) quantized to quint8 with MIN_FIRST by the HIP kernel."""
-    from oracle import pyoracle as orc
+    """fp32 N(0,1) activations (+ outliers) quantized to quint8 with MIN_FIRST against their own range, all on the
+    device (itexhip_quantize_dynamic); returns the op's output range as the MatMul's min_a / max_a."""
     g = torch.Generator(device=dev)
     g.manual_seed(seed)
     x = torch.randn(M, K, device=dev, generator=g)
@@ -128,12 +128,11 @@ def make_acts(torch, hip, M, K, seed, dev, outlier_frac=0.0, outlier_mult=1.0):
         n_out = max(1, int(M * K * outlier_frac))
         idx = torch.randint(0, M * K, (n_out,), device=dev, generator=g)
         x.view(-1)[idx] *= outlier_mult
-    mn, mx = float(x.min()), float(x.max())
-    _, amn, amx = orc.adjust_input_range(mn, mx)
-    scale = orc.legacy_min_first_scale(orc.QUINT8, amn, amx)
     xq = torch.empty(M, K, dtype=torch.uint8, device=dev)
-    import numpy as np
-    hip.quantize(x, xq, M * K, hip.QUINT8, float(scale), float(np.float32(-amn) * scale), _stream(torch))
+    state = torch.zeros(8, dtype=torch.float32, device=dev)
+    hip.quantize_dynamic(x, xq, M * K, hip.QUINT8, hip.MIN_FIRST, 0.01, state, _stream(torch))
+    torch.cuda.synchronize()
+    amn, amx = [float(v) for v in state[2:4].cpu().numpy()]
     return x, xq, float(amn), float(amx)
 
 
@@ -208,9 +207,47 @@ def bench_linear(torch, hip, timer, M, K, N, kind, steps, warmup, dev, seed, rot
     return res
 
 
+def bench_dynamic_linear(torch, hip, timer, M, K, N, steps, warmup, dev, seed):
+    """A dynamically quantized linear from float activations: range of x, QuantizeV2 (MIN_FIRST quint8), MatMul
+    [BiasAdd, Dequantize].  `device_range`: itexhip_quantize_dynamic + itexhip_qmatmul_device_range, nothing waits on the
+    host (what _ITEXQuantizedMatMulDynamicInput enqueues).  `host_range`: the range is copied to the host between the
+    reduction and the quantization, as the separate ops need for their host-memory min / max tensors."""
+    import numpy as np
+    L = make_weights(torch, hip, K, N, seed, dev)
+    g = torch.Generator(device=dev)
+    g.manual_seed(seed + 100)
+    x = torch.randn(M, K, device=dev, generator=g)
+    xq = torch.empty(M, K, dtype=torch.uint8, device=dev)
+    out = torch.empty(M, N, dtype=torch.float32, device=dev)
+    state = torch.zeros(8, dtype=torch.float32, device=dev)
+    st = _stream(torch)
+    p = hip.matmul_params(api=hip.API_V2, t_in=hip.QUINT8, t_out=hip.FLOAT, input_mode=hip.MIN_FIRST, has_dequantize=True)
+
+    def device_range(i):
+        hip.quantize_dynamic(x, xq, M * K, hip.QUINT8, hip.MIN_FIRST, 0.01, state, st)
+        hip.qmatmul_device_range(p, xq, L["packed"], L["colsum"], M, K, N, state[2:], L["min_b"], L["max_b"], N, L["bias"], out, st)
+
+    host = np.zeros(2, np.float32)
+    f32 = np.float32
+
+    def host_range(i):
+        hip.minmax_f32(x, M * K, state, st)
+        hip.memcpy_d2h(host, state, 8, st)   # waits for the stream
+        amn, amx = min(f32(0.0), host[0]), max(f32(0.0), host[1])
+        scale = f32(255.0 / float(amx - amn))
+        hip.quantize(x, xq, M * K, hip.QUINT8, float(scale), float(f32(-amn) * scale), st)
+        p.min_a, p.max_a = float(amn), float(amx)
+        hip.qmatmul(p, xq, L["packed"], L["colsum"], M, K, N, L["min_b"], L["max_b"], N, L["bias"], out, st)
+
+    ms_dev = timer.run(device_range, steps, warmup)
+    ms_host = timer.run(host_range, steps, warmup)
+    return dict(name="dynamic_linear_from_float", M=M, K=K, N=N, us_device_range=ms_dev * 1e3, us_host_range=ms_host * 1e3,
+                note="range + QuantizeV2 + MatMul[BiasAdd, Dequantize] per step; device_range: no host wait; host_range: "
+                     "the range crosses to the host between reduction and quantization")
+
+
 def bench_elementwise(torch, hip, timer, n, steps, warmup, dev):
     import numpy as np
-    from oracle import pyoracle as orc
     g = torch.Generator(device=dev)
     g.manual_seed(30)
     x = torch.randn(n, device=dev, generator=g)
@@ -228,18 +265,21 @@ def bench_elementwise(torch, hip, timer, n, steps, warmup, dev):
 
     q8 = torch.empty(n, dtype=torch.int8, device=dev)
     qu8 = torch.empty(n, dtype=torch.uint8, device=dev)
-    _, amn, amx = orc.adjust_input_range(mn, mx)
-    _, _, _, sc, _ = orc.scale_zeropoint_align(orc.QINT8, orc.SCALED, False, amn, amx)
-    add("quantize_v2_scaled_qint8", lambda i: hip.quantize(x, q8, n, hip.QINT8, float(sc[0]), 0.0, st), 5 * n)
-    scale = orc.legacy_min_first_scale(orc.QUINT8, amn, amx)
-    addend = float(np.float32(-amn) * scale)
+    # the ops' host parameter math for this range, in fp32 (range widened to hold 0; SCALED: 127 / max|.|; legacy
+    # MIN_FIRST: 255 / (max - min) with the shift folded into an addend; Dequantize: the inverse scales)
+    f32 = np.float32
+    amn, amx = min(f32(0.0), f32(mn)), max(f32(0.0), f32(mx))
+    r = max(abs(amn), abs(amx))
+    add("quantize_v2_scaled_qint8", lambda i: hip.quantize(x, q8, n, hip.QINT8, float(f32(127.0) / r), 0.0, st), 5 * n)
+    scale = f32(255.0 / float(amx - amn))
+    addend = float(f32(-amn) * scale)
     add("quantize_v2_min_first_quint8", lambda i: hip.quantize(x, qu8, n, hip.QUINT8, float(scale), addend, st), 5 * n)
     add("minmax_f32_range_pass", lambda i: hip.minmax_f32(x, n, mm, st), 4 * n)
     y = x  # reuse the fp32 buffer as the dequantize output
-    _, _, _, dsc, dzp = orc.scale_zeropoint_align(orc.QUINT8, orc.MIN_FIRST, True, amn, amx)
-    add("dequantize_min_first_quint8", lambda i: hip.dequantize(qu8, y, n, hip.QUINT8, float(dsc[0]), int(dzp[0]), st), 5 * n)
-    _, _, _, dsc, _ = orc.scale_zeropoint_align(orc.QINT8, orc.SCALED, True, amn, amx)
-    add("dequantize_scaled_qint8", lambda i: hip.dequantize(q8, y, n, hip.QINT8, float(dsc[0]), 0, st), 5 * n)
+    dsc = (amx - amn) / f32(255.0)
+    dzp = int(np.round(f32(255.0) - amx / dsc))
+    add("dequantize_min_first_quint8", lambda i: hip.dequantize(qu8, y, n, hip.QUINT8, float(dsc), dzp, st), 5 * n)
+    add("dequantize_scaled_qint8", lambda i: hip.dequantize(q8, y, n, hip.QINT8, float(r / f32(127.0)), 0, st), 5 * n)
     # Requantize: int32 accumulators ~ N(0, 2^20), range pass then per-tensor requantize to qint8
     acc = (torch.randn(n, device=dev, generator=g) * float(1 << 20)).round_().to(torch.int32)
     imn = torch.zeros(1, dtype=torch.int32, device=dev)
@@ -511,6 +551,7 @@ def main():
                          frac_graph=r["gbs_kernel_graph"] / PEAK_HBM_GBS,
                          note="8 weight copies cycled (470 MB > last-level cache)")
                 others.append(r)
+            others.append(bench_dynamic_linear(torch, hip, timer, 16, k, n, K_steps, W, dev, seed=10))
             r = bench_linear(torch, hip, timer, 16, k, n, "deq", K_steps, W, dev, seed=10, rotate=8, per_row=True)
             r.pop("_ctx")
             r.update(name="decode_gemv_per_token_ranges", bound="hbm", us_kernel=r["ms_per_step"] * 1e3,

@@ -159,6 +159,18 @@ int itexhip_minmax_i32_per_channel(const int32_t* x, int64_t rows, int64_t depth
                                    int32_t* max_out, void* stream);
 int itexhip_minmax_f32(const float* x, int64_t n, float* minmax_out, void* stream);
 
+/* QuantizeV2 of a float tensor with the tensor's own range, nothing crossing to the host: the range reduction, the
+ * op's parameter math (range adjustment quantize_op.h:130-152; SCALED scale quantization_util.h:54-84; legacy
+ * MIN_FIRST scale quantize_op.h:204-214 — per tensor, the same fp32 / fp64 operations as the host code) in a one-thread
+ * kernel, and the quantization reading scale and addend from device memory.  mode: ITEXHIP_SCALED (qint8 / quint8) or
+ * ITEXHIP_MIN_FIRST (quint8, the non-classic algorithm).  `state` is a device array of 8 floats:
+ * [0..1] the tensor's min and max, [2..3] the op's output_min / output_max (what a consuming MatMul takes as
+ * min_a / max_a: pass state + 2 to itexhip_qmatmul_device_range), [4..5] scale and addend.  n > 0.  The reference
+ * has no such op (its QuantizeV2 takes the range from the host); this is the producer half of the
+ * Min/Max -> QuantizeV2 -> MatMul fusion of this plugin's graph pass. */
+int itexhip_quantize_dynamic(const float* x, void* q, int64_t n, int dst_type, int mode, float ensure_minimum_range,
+                             float* state, void* stream);
+
 /* ------------------------------------------------------------------------------------------
  * Quantized MatMul (oneDNN inner_product_forward u8/s8 x s8 -> s32 with fused epilogue;
  * itex/core/kernels/common/quantized_matmul_common.h:223-226 (primitive), :92 (execute)).
@@ -290,6 +302,15 @@ int itexhip_qmatmul_per_row(const itexhip_matmul_params* p, const void* a, const
                             const int32_t* colsum, int64_t M, int64_t K, int64_t N, const float* row_min_a,
                             const float* row_max_a, const float* min_b, const float* max_b, int64_t nb,
                             const void* bias, const float* addend, void* out, void* stream);
+
+/* itexhip_qmatmul with the per-tensor activation range in device memory (range_a[0] = min_a, range_a[1] = max_a, e.g.
+ * state + 2 of itexhip_quantize_dynamic enqueued earlier on the same stream) in place of p->min_a / p->max_a, which are
+ * ignored: the kernels derive scales and bias from it exactly as from the host values.  Not for a qint32 result (its
+ * output range, quantized_ops.h:40-54, is host math on the activation range).  An extension, as itexhip_qmatmul_per_row. */
+int itexhip_qmatmul_device_range(const itexhip_matmul_params* p, const void* a, const int8_t* packed_b,
+                                 const int32_t* colsum, int64_t M, int64_t K, int64_t N, const float* range_a,
+                                 const float* min_b, const float* max_b, int64_t nb, const void* bias,
+                                 const float* addend, void* out, void* stream);
 
 /* itexhip_qmatmul on the unpacked TF-layout weight ([K, N], or [N, K] with transpose_b), any K, no
  * prepack and no column-sum buffer: one thread per output element.  For the shapes the MFMA kernels

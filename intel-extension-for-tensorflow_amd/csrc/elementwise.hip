@@ -23,7 +23,12 @@ __device__ __forceinline__ uint32_t quantize4(f4 v, float scale, float addend) {
 template <int T>
 __global__ __launch_bounds__(kThreads) void quantize_vec_kernel(const f4* __restrict__ x,
                                                                 uint32_t* __restrict__ q, int64_t n4,
-                                                                float scale, float addend) {
+                                                                float scale, float addend,
+                                                                const float* __restrict__ dev_params) {
+  if (dev_params) {  // {scale, addend} left in device memory by quantize_dynamic_params_kernel
+    scale = dev_params[0];
+    addend = dev_params[1];
+  }
   const int64_t base = static_cast<int64_t>(blockIdx.x) * (kThreads * kUnroll) + threadIdx.x;
   f4 v[kUnroll];
 #pragma unroll
@@ -42,7 +47,12 @@ template <int T>
 __global__ __launch_bounds__(kThreads) void quantize_scalar_kernel(const float* __restrict__ x,
                                                                    uint8_t* __restrict__ q,
                                                                    int64_t begin, int64_t n,
-                                                                   float scale, float addend) {
+                                                                   float scale, float addend,
+                                                                   const float* __restrict__ dev_params) {
+  if (dev_params) {
+    scale = dev_params[0];
+    addend = dev_params[1];
+  }
   const int64_t i = begin + static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
   if (i < n) {
     const float t = x[i] * scale;
@@ -330,6 +340,23 @@ __global__ __launch_bounds__(kThreads) void minmax_f32_kernel(const f4* __restri
       });
 }
 
+// fill + reduction of n > 0 floats into the two order-preserving integer keys (finish_minmax_f32_kernel, or a
+// consumer that decodes the keys itself, turns them into floats)
+inline void enqueue_minmax_f32(const float* x, int64_t n, int* keys, hipStream_t st) {
+  fill_minmax_f32_kernel<<<1, 1, 0, st>>>(keys);
+  // the vector body starts at the first 16-byte boundary; head and tail go through `tail` slots
+  const uintptr_t addr = reinterpret_cast<uintptr_t>(x);
+  int64_t head = static_cast<int64_t>(((16 - (addr & 15)) & 15) / 4);
+  if (head > n) head = n;
+  const int64_t n4 = (n - head) / 4;
+  const int64_t ntail = n - head - n4 * 4;
+  const unsigned grid = static_cast<unsigned>(std::min<int64_t>(
+      kReduceBlocks, std::max<int64_t>(1, (n4 + kThreads * kReduceUnroll - 1) / (kThreads * kReduceUnroll))));
+  minmax_f32_kernel<<<grid, kThreads, 0, st>>>(reinterpret_cast<const f4*>(x + head), n4, x + head + n4 * 4,
+                                               static_cast<int>(ntail), keys);
+  if (head > 0) minmax_f32_kernel<<<1, kThreads, 0, st>>>(nullptr, 0, x, static_cast<int>(head), keys);
+}
+
 inline unsigned blocks_for(int64_t n, int64_t per_block) {
   return static_cast<unsigned>((n + per_block - 1) / per_block);
 }
@@ -365,6 +392,75 @@ __global__ __launch_bounds__(kThreads) void copy_byte_kernel(const uint8_t* __re
 
 using namespace itexhip;
 
+namespace itexhip {
+namespace {
+// std::min / std::max as the host code evaluates them (the first argument unless the second is smaller / larger)
+__device__ __forceinline__ float host_min(float a, float b) { return b < a ? b : a; }
+__device__ __forceinline__ float host_max(float a, float b) { return a < b ? b : a; }
+
+// The QuantizeV2 parameter math of a per-tensor range, on the device (quantize_op.h:130-152 range adjustment,
+// quantization_util.h:54-84 SCALED scale, quantize_op.h:204-214 legacy MIN_FIRST scale): state[0..1] = the tensor's
+// min and max -> state[2..3] = the op's output_min / output_max, state[4..5] = scale and addend of the kernel.
+__global__ void quantize_dynamic_params_kernel(float* state, int dst_type, int mode, float ensure_minimum_range) {
+  // state[0..1] arrive as the reduction's integer keys; they leave as floats
+  const float in_min = key2f(reinterpret_cast<const int*>(state)[0]), in_max = key2f(reinterpret_cast<const int*>(state)[1]);
+  state[0] = in_min;
+  state[1] = in_max;
+  const float lo = host_min(0.0f, in_min);
+  const float epsilon = host_max(1.0f, host_max(fabsf(in_min), fabsf(in_max))) * ensure_minimum_range;
+  const float widened = lo + epsilon;
+  float mn = lo, mx = host_max(0.0f, host_max(in_max, widened));
+  float scale, addend;
+  if (mode == ITEXHIP_SCALED) {
+    const float q_high = dst_type == ITEXHIP_QINT8 ? 127.0f : 255.0f;
+    const float r = host_max(fabsf(mn), fabsf(mx));
+    mx = r;
+    mn = -r;
+    scale = q_high / r;
+    addend = 0.0f;
+    if (dst_type == ITEXHIP_QUINT8) mn = 0.0f;  // output_min of an unsigned SCALED result (:402-408)
+  } else {  // the 255 steps are a double, so the division is done in double and rounded once
+    scale = static_cast<float>(255.0 / static_cast<double>(mx - mn));
+    const float shift = -mn;
+    addend = shift * scale;
+  }
+  state[2] = mn;
+  state[3] = mx;
+  state[4] = scale;
+  state[5] = addend;
+}
+
+int launch_quantize(const char* who, const float* x, void* q, int64_t n, int dst_type, float scale, float addend,
+                    const float* dev_params, hipStream_t st) {
+  int64_t done = 0;
+  if (aligned(x, 16) && aligned(q, 4) && n >= 4) {
+    const int64_t n4 = n / 4;
+    const unsigned grid = blocks_for(n4, kThreads * kUnroll);
+    if (dst_type == ITEXHIP_QINT8)
+      quantize_vec_kernel<ITEXHIP_QINT8><<<grid, kThreads, 0, st>>>(
+          reinterpret_cast<const f4*>(x), reinterpret_cast<uint32_t*>(q), n4, scale, addend, dev_params);
+    else
+      quantize_vec_kernel<ITEXHIP_QUINT8><<<grid, kThreads, 0, st>>>(
+          reinterpret_cast<const f4*>(x), reinterpret_cast<uint32_t*>(q), n4, scale, addend, dev_params);
+    done = n4 * 4;
+  }
+  if (done < n) {
+    const unsigned grid = blocks_for(n - done, kThreads);
+    if (dst_type == ITEXHIP_QINT8)
+      quantize_scalar_kernel<ITEXHIP_QINT8><<<grid, kThreads, 0, st>>>(
+          x, reinterpret_cast<uint8_t*>(q), done, n, scale, addend, dev_params);
+    else
+      quantize_scalar_kernel<ITEXHIP_QUINT8><<<grid, kThreads, 0, st>>>(
+          x, reinterpret_cast<uint8_t*>(q), done, n, scale, addend, dev_params);
+  }
+  ITEXHIP_CHECK_LAUNCH(who);
+  return ITEXHIP_OK;
+}
+}  // namespace
+}  // namespace itexhip
+
+using namespace itexhip;
+
 extern "C" int itexhip_quantize(const float* x, void* q, int64_t n, int dst_type, float scale,
                                 float addend, void* stream) {
   ITEXHIP_REQUIRE(dst_type == ITEXHIP_QINT8 || dst_type == ITEXHIP_QUINT8,
@@ -372,30 +468,20 @@ extern "C" int itexhip_quantize(const float* x, void* q, int64_t n, int dst_type
   ITEXHIP_REQUIRE(n >= 0, "itexhip_quantize: negative size");
   if (n == 0) return ITEXHIP_OK;
   ITEXHIP_REQUIRE(x && q, "itexhip_quantize: null buffer");
-  hipStream_t st = as_stream(stream);
-  int64_t done = 0;
-  if (aligned(x, 16) && aligned(q, 4) && n >= 4) {
-    const int64_t n4 = n / 4;
-    const unsigned grid = blocks_for(n4, kThreads * kUnroll);
-    if (dst_type == ITEXHIP_QINT8)
-      quantize_vec_kernel<ITEXHIP_QINT8><<<grid, kThreads, 0, st>>>(
-          reinterpret_cast<const f4*>(x), reinterpret_cast<uint32_t*>(q), n4, scale, addend);
-    else
-      quantize_vec_kernel<ITEXHIP_QUINT8><<<grid, kThreads, 0, st>>>(
-          reinterpret_cast<const f4*>(x), reinterpret_cast<uint32_t*>(q), n4, scale, addend);
-    done = n4 * 4;
-  }
-  if (done < n) {
-    const unsigned grid = blocks_for(n - done, kThreads);
-    if (dst_type == ITEXHIP_QINT8)
-      quantize_scalar_kernel<ITEXHIP_QINT8><<<grid, kThreads, 0, st>>>(
-          x, reinterpret_cast<uint8_t*>(q), done, n, scale, addend);
-    else
-      quantize_scalar_kernel<ITEXHIP_QUINT8><<<grid, kThreads, 0, st>>>(
-          x, reinterpret_cast<uint8_t*>(q), done, n, scale, addend);
-  }
-  ITEXHIP_CHECK_LAUNCH("itexhip_quantize");
-  return ITEXHIP_OK;
+  return launch_quantize("itexhip_quantize", x, q, n, dst_type, scale, addend, nullptr, as_stream(stream));
+}
+
+extern "C" int itexhip_quantize_dynamic(const float* x, void* q, int64_t n, int dst_type, int mode,
+                                        float ensure_minimum_range, float* state, void* stream) {
+  ITEXHIP_REQUIRE(dst_type == ITEXHIP_QINT8 || dst_type == ITEXHIP_QUINT8,
+                  "itexhip_quantize_dynamic: dst_type must be qint8 or quint8, got %d", dst_type);
+  ITEXHIP_REQUIRE(mode == ITEXHIP_SCALED || (mode == ITEXHIP_MIN_FIRST && dst_type == ITEXHIP_QUINT8),
+                  "itexhip_quantize_dynamic: SCALED, or MIN_FIRST to quint8");
+  ITEXHIP_REQUIRE(n > 0, "itexhip_quantize_dynamic: an empty tensor has no range");
+  ITEXHIP_REQUIRE(x && q && state && aligned(state, 8), "itexhip_quantize_dynamic: null or unaligned buffer");
+  enqueue_minmax_f32(x, n, reinterpret_cast<int*>(state), as_stream(stream));
+  quantize_dynamic_params_kernel<<<1, 1, 0, as_stream(stream)>>>(state, dst_type, mode, ensure_minimum_range);
+  return launch_quantize("itexhip_quantize_dynamic", x, q, n, dst_type, 0.0f, 0.0f, state + 4, as_stream(stream));
 }
 
 extern "C" int itexhip_quantize_axis(const float* x, void* q, int64_t outer, int64_t slices,
@@ -566,21 +652,11 @@ extern "C" int itexhip_minmax_f32(const float* x, int64_t n, float* minmax_out, 
   ITEXHIP_REQUIRE(minmax_out, "itexhip_minmax_f32: null output");
   hipStream_t st = as_stream(stream);
   int* keys = reinterpret_cast<int*>(minmax_out);
-  fill_minmax_f32_kernel<<<1, 1, 0, st>>>(keys);
   if (n > 0) {
     ITEXHIP_REQUIRE(x, "itexhip_minmax_f32: null input");
-    // the vector body starts at the first 16-byte boundary; head and tail go through `tail` slots
-    const uintptr_t addr = reinterpret_cast<uintptr_t>(x);
-    int64_t head = static_cast<int64_t>(((16 - (addr & 15)) & 15) / 4);
-    if (head > n) head = n;
-    const int64_t n4 = (n - head) / 4;
-    const int64_t ntail = n - head - n4 * 4;
-    const unsigned grid = static_cast<unsigned>(std::min<int64_t>(
-        kReduceBlocks, std::max<int64_t>(1, (n4 + kThreads * kReduceUnroll - 1) / (kThreads * kReduceUnroll))));
-    minmax_f32_kernel<<<grid, kThreads, 0, st>>>(reinterpret_cast<const f4*>(x + head), n4,
-                                                 x + head + n4 * 4, static_cast<int>(ntail), keys);
-    if (head > 0)
-      minmax_f32_kernel<<<1, kThreads, 0, st>>>(nullptr, 0, x, static_cast<int>(head), keys);
+    enqueue_minmax_f32(x, n, keys, st);
+  } else {
+    fill_minmax_f32_kernel<<<1, 1, 0, st>>>(keys);
   }
   finish_minmax_f32_kernel<<<1, 1, 0, st>>>(keys);
   ITEXHIP_CHECK_LAUNCH("itexhip_minmax_f32");

@@ -606,7 +606,7 @@ namespace {
 int qmatmul_impl(const char* who, const itexhip_matmul_params* p, const void* a, const int8_t* packed_b,
                  const int32_t* colsum, int64_t M, int64_t K, int64_t N, const float* row_min_a,
                  const float* row_max_a, const float* min_b, const float* max_b, int64_t nb, const void* bias,
-                 const float* addend, void* out, void* stream) {
+                 const float* addend, void* out, void* stream, const float* range_a = nullptr) {
   itexhip_epilogue ep;
   if (int st = itexhip_qmatmul_epilogue_desc(p, nb, &ep)) return st;
   ITEXHIP_REQUIRE(nb == 1 || nb == N, "%s: %lld weight ranges for %lld channels", who, static_cast<long long>(nb),
@@ -627,6 +627,7 @@ int qmatmul_impl(const char* who, const itexhip_matmul_params* p, const void* a,
   e.prep = make_prep_args(p, ep);
   e.row_min_a = row_min_a;
   e.row_max_a = row_max_a;
+  e.range_a = range_a;
   e.addend = addend;
   e.addend_type = ITEXHIP_FLOAT;
   return launch_packed(M <= 16, a, p->t_in, packed_b, M, K, N, e, p->t_out, out, stream, who);
@@ -639,6 +640,17 @@ extern "C" int itexhip_qmatmul(const itexhip_matmul_params* p, const void* a, co
                                void* stream) {
   return qmatmul_impl("itexhip_qmatmul", p, a, packed_b, colsum, M, K, N, nullptr, nullptr, min_b, max_b, nb, bias,
                       addend, out, stream);
+}
+
+extern "C" int itexhip_qmatmul_device_range(const itexhip_matmul_params* p, const void* a, const int8_t* packed_b,
+                                           const int32_t* colsum, int64_t M, int64_t K, int64_t N, const float* range_a,
+                                           const float* min_b, const float* max_b, int64_t nb, const void* bias,
+                                           const float* addend, void* out, void* stream) {
+  ITEXHIP_REQUIRE(range_a != nullptr, "itexhip_qmatmul_device_range: null activation range");
+  ITEXHIP_REQUIRE(p->t_out != ITEXHIP_QINT32, "itexhip_qmatmul_device_range: a qint32 result's range is computed on the "
+                                              "host from the activation range; use itexhip_qmatmul");
+  return qmatmul_impl("itexhip_qmatmul_device_range", p, a, packed_b, colsum, M, K, N, nullptr, nullptr, min_b, max_b, nb,
+                      bias, addend, out, stream, range_a);
 }
 
 extern "C" int itexhip_qmatmul_per_row(const itexhip_matmul_params* p, const void* a, const int8_t* packed_b,

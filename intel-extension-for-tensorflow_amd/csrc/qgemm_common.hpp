@@ -55,6 +55,9 @@ struct EpilogueArgs {
   // in place of prep.min_a / prep.max_a; null for the reference's per-tensor range
   const float* row_min_a;
   const float* row_max_a;
+  // per-tensor activation range in device memory ({min_a, max_a}, written by an earlier kernel on the same stream) in
+  // place of prep.min_a / prep.max_a; null when the caller knows the range on the host
+  const float* range_a;
   CanonChain canon;  // filled by the tile dispatch for the kernels that take it
 };
 
@@ -132,7 +135,12 @@ __device__ __forceinline__ void finish_channel(const EpilogueArgs& e, const RawC
                                                float* bias) {
   *comp = e.comp_mul * r.colsum;
   if (e.fused) {
-    const ChannelScaleBias c = channel_scale_bias(e.prep, r.min_bj, r.max_bj, r.min_b0, r.max_b0, r.bias, r.colsum);
+    PrepArgs pr = e.prep;
+    if (e.range_a) {
+      pr.min_a = e.range_a[0];
+      pr.max_a = e.range_a[1];
+    }
+    const ChannelScaleBias c = channel_scale_bias(pr, r.min_bj, r.max_bj, r.min_b0, r.max_b0, r.bias, r.colsum);
     *scale = e.n_scales > 0 ? c.scale : 1.0f;
     *bias = c.bias;
   } else {

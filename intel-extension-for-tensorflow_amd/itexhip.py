@@ -30,7 +30,7 @@ EXPORTS = [
     "itexhip_dequantize16", "itexhip_dequantize_axis16", "itexhip_requantize_per_channel",
     "itexhip_requantize", "itexhip_minmax_i32_per_channel", "itexhip_minmax_f32",
     "itexhip_qmatmul_epilogue_desc", "itexhip_qmatmul_prepare", "itexhip_qgemm_packed_bytes",
-    "itexhip_qgemm_prepack_b", "itexhip_qgemm", "itexhip_qgemm_tile", "itexhip_qgemv", "itexhip_qmatmul", "itexhip_qmatmul_per_row", "itexhip_qmatmul_unpacked", "itexhip_mfma_probe",
+    "itexhip_qgemm_prepack_b", "itexhip_qgemm", "itexhip_qgemm_tile", "itexhip_qgemv", "itexhip_qmatmul", "itexhip_qmatmul_per_row", "itexhip_qmatmul_device_range", "itexhip_quantize_dynamic", "itexhip_qmatmul_unpacked", "itexhip_mfma_probe",
     "itexhip_qgemm_naive", "itexhip_qbatch_matmul", "itexhip_transpose", "itexhip_im2col8", "itexhip_scale_vector",
     "itexhip_qconv2d_implicit_ok", "itexhip_qconv2d", "itexhip_qgemm_sum", "itexhip_qconv2d_sum", "itexhip_qdepthwise_conv2d",
 ]
@@ -101,6 +101,11 @@ def _i64(v):
 
 def build_info():
     return _lib.itexhip_build_info().decode()
+
+
+def memcpy_d2h(host_array, src, nbytes, stream=0):
+    """Device -> host (a numpy array) copy that returns when the bytes have arrived."""
+    _check(_lib.itexhip_memcpy_d2h(C.c_void_p(host_array.ctypes.data), _ptr(src), C.c_size_t(int(nbytes)), _ptr(stream)))
 
 
 def memcpy_d2d_async(dst, src, nbytes, stream=0):
@@ -227,6 +232,17 @@ def qmatmul_per_row(p, a, packed_b, colsum, M, K, N, row_min_a, row_max_a, min_b
     _check(_lib.itexhip_qmatmul_per_row(C.byref(p), _ptr(a), _ptr(packed_b), _ptr(colsum), _i64(M), _i64(K), _i64(N),
                                         _ptr(row_min_a), _ptr(row_max_a), _ptr(min_b), _ptr(max_b), _i64(nb),
                                         _ptr(bias), _ptr(addend), _ptr(out), _ptr(stream)))
+
+
+def qmatmul_device_range(p, a, packed_b, colsum, M, K, N, range_a, min_b, max_b, nb, bias, out, stream=0, addend=None):
+    _check(_lib.itexhip_qmatmul_device_range(C.byref(p), _ptr(a), _ptr(packed_b), _ptr(colsum), _i64(M), _i64(K), _i64(N),
+                                             _ptr(range_a), _ptr(min_b), _ptr(max_b), _i64(nb), _ptr(bias),
+                                             _ptr(addend), _ptr(out), _ptr(stream)))
+
+
+def quantize_dynamic(x, q, n, dst_type, mode, ensure_minimum_range, state, stream=0):
+    _check(_lib.itexhip_quantize_dynamic(_ptr(x), _ptr(q), _i64(n), int(dst_type), int(mode),
+                                         C.c_float(ensure_minimum_range), _ptr(state), _ptr(stream)))
 
 
 def qmatmul_unpacked(p, a, w, transpose_b, M, K, N, min_b, max_b, nb, bias, out, stream=0, addend=None):

@@ -263,6 +263,65 @@ bool AttrIntTensor(const std::string& value, int* rank, std::vector<int64_t>* el
   return true;
 }
 
+// AttrValue.list = 1 (ListValue: s = 2, type = 6; repeated enums arrive packed or one by one)
+bool AttrTypeList(const std::string& value, std::vector<int>* types) {
+  types->clear();
+  if (value.empty()) return true;
+  Reader at{nullptr, nullptr};
+  if (!FindField(value, 1, 2, &at)) return false;
+  const auto body = at.Bytes();
+  if (!at.ok) return false;
+  Reader r{body.first, body.first + body.second};
+  while (!r.done()) {
+    const uint64_t tag = r.Varint();
+    if (!r.ok) return false;
+    if ((tag >> 3) == 6 && (tag & 7) == 2) {
+      const auto packed = r.Bytes();
+      if (!r.ok) return false;
+      Reader e{packed.first, packed.first + packed.second};
+      while (!e.done()) {
+        types->push_back(static_cast<int>(e.Varint()));
+        if (!e.ok) return false;
+      }
+    } else if ((tag >> 3) == 6 && (tag & 7) == 0) {
+      types->push_back(static_cast<int>(r.Varint()));
+      if (!r.ok) return false;
+    } else if (!r.Skip(static_cast<uint32_t>(tag & 7))) {
+      return false;
+    }
+  }
+  return true;
+}
+
+bool AttrStringList(const std::string& value, std::vector<std::string>* strings) {
+  strings->clear();
+  if (value.empty()) return true;
+  Reader at{nullptr, nullptr};
+  if (!FindField(value, 1, 2, &at)) return false;
+  const auto body = at.Bytes();
+  if (!at.ok) return false;
+  Reader r{body.first, body.first + body.second};
+  while (!r.done()) {
+    const uint64_t tag = r.Varint();
+    if (!r.ok) return false;
+    if ((tag >> 3) == 2 && (tag & 7) == 2) {
+      strings->push_back(Str(r.Bytes()));
+      if (!r.ok) return false;
+    } else if (!r.Skip(static_cast<uint32_t>(tag & 7))) {
+      return false;
+    }
+  }
+  return true;
+}
+
+std::string MakeAttrTypeList(const std::vector<int>& types) {
+  std::string packed, list, v;
+  for (int t : types) PutVarint(&packed, static_cast<uint64_t>(t));
+  if (!types.empty()) PutBytes(&list, 6, packed);
+  PutBytes(&v, 1, list);
+  return v;
+}
+
 std::string MakeAttrBool(bool b) {
   std::string v;
   PutVarint(&v, (5u << 3) | 0);

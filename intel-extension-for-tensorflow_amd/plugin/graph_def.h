@@ -44,6 +44,10 @@ bool AttrInt(const std::string& value, int* i);  // i = 3
 // The integer tensor of a Const node's "value" attribute (AttrValue.tensor = 8; tensor.proto: dtype = 1,
 // tensor_shape = 2, tensor_content = 4, int_val = 7, int64_val = 10), int32 or int64: its rank and elements.
 bool AttrIntTensor(const std::string& value, int* rank, std::vector<int64_t>* elements);
+// list(type) and list(string) attributes (AttrValue.list = 1; ListValue: s = 2, type = 6)
+bool AttrTypeList(const std::string& value, std::vector<int>* types);
+bool AttrStringList(const std::string& value, std::vector<std::string>* strings);
+std::string MakeAttrTypeList(const std::vector<int>& types);
 std::string MakeAttrBool(bool b);
 std::string MakeAttrString(const std::string& s);
 std::string MakeAttrType(int t);

@@ -5,6 +5,7 @@
 // that rename is not cosmetic: _ITEXQuantizeV2 receives classic_asymmetric_algorithm = "all consumers are
 // Dequantize", which selects the zero-point form of MIN_FIRST instead of the legacy one.
 // ITEX_AMD_NATIVE_FORMAT=0 leaves graphs untouched.
+#include <algorithm>
 #include <cstdlib>
 #include <cstring>
 #include <map>
@@ -165,6 +166,102 @@ bool MatchDynamicRange(const graph::Node& q, const std::map<std::string, const g
   return const_ints(fin[1], &rank, &shape) && rank == 1 && shape.size() == 1 && shape[0] == -1;
 }
 
+// _ITEXQuantizeV2DynamicRange(x) -> _ITEXQuantizedMatMul becomes one node, _ITEXQuantizedMatMulDynamicInput(x, ...): the
+// range of x, its quantization and the product are enqueued back to back and the range never crosses to the host
+// (as separate nodes, output_min / output_max of the first are host tensors, so every step waits for the reduction).
+// The reference fuses QuantizeV2 into its consumer for convolutions only (remapper.cc:2099-2114).  Conditions: the
+// MatMul is the only reader of all three outputs, both nodes sit on the same device, the quantization parameters
+// agree (T1 / input_quant_mode), the MatMul has no addend and a Requantize or Dequantize output (the range of a
+// qint32 result is host math on the activation range).  Returns the number of fused pairs.
+int FuseDynamicQuantizeIntoMatMul(graph::Graph* g) {
+  std::map<std::string, size_t> index;
+  std::map<std::string, std::vector<size_t>> readers;  // by producer name: every node with a data or control input from it
+  for (size_t i = 0; i < g->nodes.size(); ++i) {
+    index[g->nodes[i].name] = i;
+    for (const std::string& in : g->nodes[i].inputs) {
+      std::string producer;
+      int port = 0;
+      if (!in.empty() && in[0] == '^') producer = in.substr(1);
+      else if (!SplitInput(in, &producer, &port)) continue;
+      readers[producer].push_back(i);
+    }
+  }
+  std::vector<bool> dead(g->nodes.size(), false);
+  int fused = 0;
+  for (size_t mi = 0; mi < g->nodes.size(); ++mi) {
+    graph::Node& m = g->nodes[mi];
+    if (m.op != "_ITEXQuantizedMatMul") continue;
+    const std::vector<std::string> data = DataInputs(m);
+    if (data.size() != 7 && data.size() != 9) continue;  // a, w, bias, min_a, max_a, min_b, max_b [, min_out, max_out]
+    std::string qname;
+    int port = 0;
+    if (!SplitInput(data[0], &qname, &port) || port != 0) continue;
+    const auto qi = index.find(qname);
+    if (qi == index.end() || dead[qi->second]) continue;
+    const graph::Node& q = g->nodes[qi->second];
+    if (q.op != "_ITEXQuantizeV2DynamicRange" || q.device != m.device) continue;
+    if (Canonical(data[3]) != qname + ":1" || Canonical(data[4]) != qname + ":2") continue;
+    bool only_reader = true;
+    for (size_t r : readers[qname]) only_reader = only_reader && r == mi;
+    if (!only_reader) continue;
+    // the MatMul's side
+    std::vector<int> dev_types, host_types;
+    std::vector<std::string> fused_ops;
+    const std::string *tdi = m.FindAttr("Tdevice_inputs"), *thi = m.FindAttr("Thost_inputs"), *fo = m.FindAttr("fused_ops");
+    if (!tdi || !thi || !fo || !graph::AttrTypeList(*tdi, &dev_types) || !graph::AttrTypeList(*thi, &host_types) ||
+        !graph::AttrStringList(*fo, &fused_ops))
+      continue;
+    if (dev_types.size() != 3 || host_types.size() + 3 != data.size()) continue;
+    bool out_given = false, has_add = false;
+    for (const std::string& f : fused_ops) {
+      out_given = out_given || f == "Requantize" || f == "Dequantize";
+      has_add = has_add || f == "Add";
+    }
+    if (!out_given || has_add) continue;
+    bool transpose_a = false;
+    if (const std::string* ta = m.FindAttr("transpose_a")) {
+      if (!graph::AttrBool(*ta, &transpose_a) || transpose_a) continue;
+    }
+    // the quantization's side
+    int t_q = 0, t1 = 0, axis = -1;
+    std::string q_mode, m_mode = "SCALED";
+    const std::string *qt = q.FindAttr("T"), *mt = m.FindAttr("T1"), *qm = q.FindAttr("mode");
+    if (!qt || !mt || !graph::AttrType(*qt, &t_q) || !graph::AttrType(*mt, &t1) || t_q != t1 || dev_types[0] != t1) continue;
+    if (!qm || !graph::AttrString(*qm, &q_mode)) continue;
+    if (const std::string* mm = m.FindAttr("input_quant_mode")) {
+      if (!graph::AttrString(*mm, &m_mode)) continue;
+    }
+    if (q_mode != m_mode || (q_mode != "SCALED" && !(q_mode == "MIN_FIRST" && t_q == kDtQuint8))) continue;
+    if (const std::string* ax = q.FindAttr("axis")) {
+      if (!ax->empty() && (!graph::AttrInt(*ax, &axis) || axis != -1)) continue;
+    }
+    const std::vector<std::string> q_data = DataInputs(q);
+    if (q_data.size() != 1) continue;
+    // ---- rewrite
+    std::vector<std::string> inputs = {q_data[0], data[1], data[2]};
+    for (size_t k = 5; k < data.size(); ++k) inputs.push_back(data[k]);
+    for (const graph::Node* from : {static_cast<const graph::Node*>(&m), &q})
+      for (const std::string& in : from->inputs)
+        if (!in.empty() && in[0] == '^' && std::find(inputs.begin(), inputs.end(), in) == inputs.end()) inputs.push_back(in);
+    dev_types[0] = kDtFloat;
+    host_types.erase(host_types.begin(), host_types.begin() + 2);
+    if (const std::string* emr = q.FindAttr("ensure_minimum_range")) m.SetAttr("ensure_minimum_range", *emr);
+    m.SetAttr("Tdevice_inputs", graph::MakeAttrTypeList(dev_types));
+    m.SetAttr("Thost_inputs", graph::MakeAttrTypeList(host_types));
+    m.inputs = inputs;
+    m.op = "_ITEXQuantizedMatMulDynamicInput";
+    dead[qi->second] = true;
+    ++fused;
+  }
+  if (fused) {
+    std::vector<graph::Node> kept;
+    for (size_t i = 0; i < g->nodes.size(); ++i)
+      if (!dead[i]) kept.push_back(std::move(g->nodes[i]));
+    g->nodes.swap(kept);
+  }
+  return fused;
+}
+
 struct Optimizer {
   std::string device_type;
 };
@@ -241,6 +338,9 @@ void Optimize(void* opt, const TF_Buffer* in, const TF_GrapplerItem*, TF_Buffer*
     if (plan[i]->copy == Copy::kQuantizedConv2D) n.SetAttr("data_format", graph::MakeAttrString("NHWC"));  // :471-495
     // CopyAttrsQuantizedMatMul (:497-515) copies every attribute and then Tbias once more: nothing to add
   }
+
+  const char* msw = std::getenv("ITEX_AMD_FUSE_QUANTIZE_MATMUL");
+  if (enabled && fuse_dynamic && !(msw && std::strcmp(msw, "0") == 0)) FuseDynamicQuantizeIntoMatMul(&g);
 
   const std::string bytes = graph::Serialize(g);
   void* mem = std::malloc(bytes.size() ? bytes.size() : 1);

@@ -98,7 +98,7 @@ std::vector<OpSpec> OpSpecs() {
                {"output: dtype"},
                {"T: quantizedtype", "mode: {'MIN_COMBINED', 'MIN_FIRST', 'SCALED'} = 'SCALED'",
                 "narrow_range: bool = false", "axis: int = -1", "dtype: {bfloat16, float} = DT_FLOAT"}});
-  for (const char* name : {"_QuantizedMatMul", "_ITEXQuantizedMatMul"})
+  for (const char* name : {"_QuantizedMatMul", "_ITEXQuantizedMatMul", "_ITEXQuantizedMatMulDynamicInput"}) {
     v.push_back({name,
                  {"device_inputs: Tdevice_inputs", "host_inputs: Thost_inputs"},
                  {"device_outputs: Tdevice_outputs", "host_outputs: Thost_outputs"},
@@ -110,6 +110,10 @@ std::vector<OpSpec> OpSpecs() {
                   "is_bias_const: bool = true", "fused_ops: list(string) = []",
                   "input_quant_mode: {'MIN_FIRST', 'SCALED'} = 'SCALED'",
                   "output_quant_mode: {'MIN_FIRST', 'SCALED'} = 'SCALED'", "leakyrelu_alpha: float = 0.2"}});
+    // the last name is made by this plugin's graph pass from _ITEXQuantizeV2DynamicRange -> _ITEXQuantizedMatMul:
+    // device_inputs[0] is the float tensor, host_inputs start at min_b, and the quantization's range floor comes along
+    if (std::strcmp(name, "_ITEXQuantizedMatMulDynamicInput") == 0) v.back().attrs.push_back("ensure_minimum_range: float = 0.01");
+  }
   const std::vector<const char*> v1_attrs = {
       "T1: quantizedtype", "T2: quantizedtype", "num_args: int >= 0", "Targs: {float, bfloat16, half, quantizedtype}",
       "transpose_a: bool = false", "transpose_b: bool = false", "fused_ops: list(string) = []",

@@ -32,6 +32,9 @@ struct Variant {
   Api api;
   TF_DataType t_in, t_out;
   bool legacy_relu;  // QuantizedMatMulReluOp
+  // _ITEXQuantizedMatMulDynamicInput (made by this plugin's graph pass; no counterpart in the reference): input 0 is
+  // the float tensor, quantized here against its own range, and the min_a / max_a inputs are gone
+  bool dynamic_input = false;
 };
 
 int ActivationFromName(const std::string& n) {
@@ -112,6 +115,14 @@ class QuantizedMatMulOp : public OpKernel {
       p_.n_fused_ops = static_cast<int>(fused_ops.size());
       min_a_idx_ = 3 + (p_.add_position != 0);  // the addend precedes all min/max tensors (:1775-1780)
       min_out_idx_ = 7;  // fixed, as in the reference (:1784-1785)
+      if (v.dynamic_input) {
+        ITEX_REQUIRES(ctx, p_.add_position == 0 && (p_.has_requantize || p_.has_dequantize), TF_INVALID_ARGUMENT,
+                      "_ITEXQuantizedMatMulDynamicInput takes no addend and needs Requantize or Dequantize in fused_ops");
+        ITEX_REQUIRES(ctx, p_.input_mode == ITEXHIP_SCALED || v.t_in == TF_QUINT8, TF_INVALID_ARGUMENT,
+                      "MIN_FIRST input quantization gives quint8");
+        if (ctx->HasAttr("ensure_minimum_range")) ITEX_REQUIRES_OK(ctx, ctx->GetAttr("ensure_minimum_range", &ensure_minimum_range_));
+        min_out_idx_ = 5;
+      }
     }
     if (p_.activation == ITEXHIP_ACT_LEAKYRELU) ITEX_REQUIRES_OK(ctx, ctx->GetAttr("leakyrelu_alpha", &p_.leakyrelu_alpha));
     // the bias type attribute is "Targs" for the V1 ops (:1533-1537), "Tbias" elsewhere
@@ -136,13 +147,19 @@ class QuantizedMatMulOp : public OpKernel {
     Tensor a = ctx->input(0);
     Tensor w = ctx->input(1);
     Tensor bias = ctx->input(2);
-    Tensor min_a_t = ctx->input(min_a_idx_), max_a_t = ctx->input(min_a_idx_ + 1);
-    Tensor min_b_t = ctx->input(min_a_idx_ + 2), max_b_t = ctx->input(min_a_idx_ + 3);
+    const bool dyn = v_.dynamic_input;
+    const int min_b_idx = dyn ? min_a_idx_ : min_a_idx_ + 2;
+    Tensor min_a_t, max_a_t;
+    if (!dyn) {
+      min_a_t = ctx->input(min_a_idx_);
+      max_a_t = ctx->input(min_a_idx_ + 1);
+    }
+    Tensor min_b_t = ctx->input(min_b_idx), max_b_t = ctx->input(min_b_idx + 1);
     if (!ctx->ok()) return;
     ITEX_REQUIRES(ctx, !transpose_a_, TF_UNIMPLEMENTED, "transpose_a is not supported by the quantized MatMul");
     ITEX_REQUIRES(ctx, a.dims() == 2 && w.dims() == 2, TF_INVALID_ARGUMENT, "quantized MatMul operands must be matrices");
     const TF_DataType bias_type = p_.t_bias == 0 ? TF_FLOAT : static_cast<TF_DataType>(p_.t_bias);
-    ITEX_REQUIRES(ctx, a.dtype() == v_.t_in && w.dtype() == TF_QINT8 && bias.dtype() == bias_type, TF_INVALID_ARGUMENT,
+    ITEX_REQUIRES(ctx, a.dtype() == (dyn ? TF_FLOAT : v_.t_in) && w.dtype() == TF_QINT8 && bias.dtype() == bias_type, TF_INVALID_ARGUMENT,
                   "quantized MatMul operand types do not match the kernel");
     const int64_t M = a.dim_size(0), K = a.dim_size(1);
     const int64_t N = transpose_b_ ? w.dim_size(0) : w.dim_size(1);
@@ -160,8 +177,10 @@ class QuantizedMatMulOp : public OpKernel {
                   "QuantizedMatMulWithBias takes per-tensor weight ranges");
 
     itexhip_matmul_params p = p_;
-    p.min_a = min_a_t.flat<float>()[0];
-    p.max_a = max_a_t.flat<float>()[0];
+    if (!dyn) {
+      p.min_a = min_a_t.flat<float>()[0];
+      p.max_a = max_a_t.flat<float>()[0];
+    }
     const bool out_q8 = v_.t_out == TF_QINT8 || v_.t_out == TF_QUINT8;
     const bool needs_freezed =
         out_q8 || (v_.api == Api::LEGACY && (v_.t_out == TF_FLOAT || v_.t_out == TF_BFLOAT16 || v_.t_out == TF_HALF));
@@ -214,7 +233,41 @@ class QuantizedMatMulOp : public OpKernel {
     }
     Tensor out = ctx->allocate_output(0, v_.t_out, {M, N});
     if (!ctx->ok()) return;
-    if (packed_path) {
+    if (dyn && M * K > 0) {
+      // range reduction, parameter math and quantization of the float tensor, then the product reading the range
+      // from device memory: nothing waits on the host.  K not a multiple of 16 (no MFMA kernel): the range is
+      // fetched once for the reference-shaped kernel.
+      Tensor aq = ctx->allocate_temp(v_.t_in, {M, K});
+      Tensor state = ctx->allocate_temp(TF_FLOAT, {8});
+      if (!ctx->ok()) return;
+      st = itexhip_quantize_dynamic(a.flat<float>(), aq.data(), M * K, v_.t_in, p_.input_mode, ensure_minimum_range_,
+                                    state.flat<float>(), stream);
+      if (st == ITEXHIP_OK && packed_path) {
+        st = itexhip_qmatmul_device_range(&p, aq.data(), packed_.flat<int8_t>(), colsum_.flat<int32_t>(), M, K, N,
+                                          state.flat<float>() + 2, min_b_dev, max_b_dev, nb, bias.data(), nullptr,
+                                          out.data(), stream);
+      } else if (st == ITEXHIP_OK) {
+        float range[2] = {0.0f, 0.0f};
+        st = itexhip_memcpy_d2h(range, state.flat<float>() + 2, sizeof(range), stream);
+        p.min_a = range[0];
+        p.max_a = range[1];
+        if (st == ITEXHIP_OK)
+          st = itexhip_qmatmul_unpacked(&p, aq.data(), w.flat<int8_t>(), transpose_b_ ? 1 : 0, M, K, N, min_b_dev, max_b_dev,
+                                        nb, bias.data(), nullptr, out.data(), stream);
+      }
+    } else if (dyn) {  // no elements to take a range from: the bias (K == 0) or nothing (M == 0)
+      float mn = 0.0f, mx = 0.0f;  // what _ITEXQuantizeV2DynamicRange reports for an empty tensor
+      qparams::AdjustRange(0.0f, 0.0f, ensure_minimum_range_, &mn, &mx);
+      if (p_.input_mode == ITEXHIP_SCALED) {
+        const float r = std::max(std::fabs(mn), std::fabs(mx));
+        mx = r;
+        mn = v_.t_in == TF_QUINT8 ? 0.0f : -r;
+      }
+      p.min_a = mn;
+      p.max_a = mx;
+      st = itexhip_qmatmul_unpacked(&p, a.data(), w.flat<int8_t>(), transpose_b_ ? 1 : 0, M, K, N, min_b_dev, max_b_dev, nb,
+                                    bias.data(), nullptr, out.data(), stream);
+    } else if (packed_path) {
       st = itexhip_qmatmul(&p, a.data(), packed_.flat<int8_t>(), colsum_.flat<int32_t>(), M, K, N, min_b_dev, max_b_dev,
                            nb, bias.data(), addend, out.data(), stream);
     } else {
@@ -250,6 +303,7 @@ class QuantizedMatMulOp : public OpKernel {
   bool transpose_a_ = false, transpose_b_ = false;
   bool is_weight_const_ = true, is_bias_const_ = true;
   int min_a_idx_ = 3, min_out_idx_ = 7;
+  float ensure_minimum_range_ = 0.01f;
   std::mutex mu_;
   // persistent device state of the node
   Tensor packed_, colsum_;
@@ -263,6 +317,23 @@ struct MatMulKernel : QuantizedMatMulOp {
   explicit MatMulKernel(OpKernelConstruction* c)
       : QuantizedMatMulOp(c, Variant{static_cast<Api>(API), static_cast<TF_DataType>(TIN), static_cast<TF_DataType>(TOUT), RELU}) {}
 };
+
+template <int TIN, int TOUT>
+struct DynamicInputMatMulKernel : QuantizedMatMulOp {
+  explicit DynamicInputMatMulKernel(OpKernelConstruction* c)
+      : QuantizedMatMulOp(c, Variant{Api::V2, static_cast<TF_DataType>(TIN), static_cast<TF_DataType>(TOUT), false, true}) {}
+};
+
+template <int TIN, int TOUT>
+void RegDynamicInput() {
+  for (TF_DataType tb : {TF_FLOAT, TF_QINT32, TF_BFLOAT16, TF_HALF}) {
+    KernelDefBuilder b("_ITEXQuantizedMatMulDynamicInput", "QuantizedMatMulOp");
+    b.TypeConstraint("T1", static_cast<TF_DataType>(TIN)).TypeConstraint("T2", TF_QINT8);
+    b.TypeConstraint("Tbias", tb).TypeConstraint("Tout", static_cast<TF_DataType>(TOUT));
+    b.HostMemory("host_inputs").HostMemory("host_outputs");
+    b.Register<DynamicInputMatMulKernel<TIN, TOUT>>();
+  }
+}
 
 template <int API, int TIN, int TOUT, bool RELU>
 void Reg(const char* op, const char* out_attr, const char* bias_attr, std::initializer_list<const char*> host_args) {
@@ -342,6 +413,15 @@ void AddQuantizedMatMulKernels() {
     RegBothInputs<V2, TF_QINT8>(op, "Tout", "Tbias", {"host_inputs", "host_outputs"});
     RegBothInputs<V2, TF_QUINT8>(op, "Tout", "Tbias", {"host_inputs", "host_outputs"});
   }
+  // the fused node of this plugin's graph pass (float activations, quantized here against their own range)
+  RegDynamicInput<TF_QUINT8, TF_FLOAT>();
+  RegDynamicInput<TF_QINT8, TF_FLOAT>();
+  RegDynamicInput<TF_QUINT8, TF_BFLOAT16>();
+  RegDynamicInput<TF_QINT8, TF_BFLOAT16>();
+  RegDynamicInput<TF_QUINT8, TF_QINT8>();
+  RegDynamicInput<TF_QINT8, TF_QINT8>();
+  RegDynamicInput<TF_QUINT8, TF_QUINT8>();
+  RegDynamicInput<TF_QINT8, TF_QUINT8>();
 }
 
 }  // namespace itex_amd

@@ -99,7 +99,7 @@ GraphDef, NodeDef, AttrValue = _M["GraphDef"], _M["NodeDef"], _M["AttrValue"]
 
 
 def node(graph, name, op, inputs=(), device="", **attrs):
-    """Adds a node; attribute values: str -> s, bool -> b, int -> i, float -> f, ("type", n) -> type,
+    """Adds a node; attribute values: str -> s, bool -> b, int -> i, float -> f, ("type", n) -> type, ("types", [n, ...]) -> list.type,
     list of str -> list.s, ("tensor", dtype, shape, values, as_content) -> an int32 (3) / int64 (9) tensor"""
     n = graph.node.add()
     n.name, n.op, n.device = name, op, device
@@ -116,6 +116,9 @@ def node(graph, name, op, inputs=(), device="", **attrs):
             a.f = v
         elif isinstance(v, tuple) and v[0] == "type":
             a.type = v[1]
+        elif isinstance(v, tuple) and v[0] == "types":      # ("types", [n, ...]) -> list.type
+            a.list.SetInParent()
+            a.list.type.extend(v[1])
         elif isinstance(v, list):
             a.list.s.extend(x.encode() for x in v)
         elif isinstance(v, tuple) and v[0] == "tensor":     # ("tensor", dtype, shape, values, as_content)

@@ -279,6 +279,68 @@ def test_canonical_chains_every_tile_shape(hip, dev, monkeypatch, shape, chain):
                 assert d.max() <= 1 and (d > 0).mean() < 1e-3
 
 
+@pytest.mark.parametrize("T,mode", [(orc.QUINT8, orc.MIN_FIRST), (orc.QINT8, orc.SCALED), (orc.QUINT8, orc.SCALED)],
+                         ids=["min_first_u8", "scaled_s8", "scaled_u8"])
+@pytest.mark.parametrize("M,K,N", [(4, 448, 528), (300, 448, 528), (16, 1024, 96), (257, 208, 400), (1, 16, 8), (513, 64, 2051)])
+def test_dynamic_quantize_then_device_range_matmul(hip, dev, T, mode, M, K, N):
+    """itexhip_quantize_dynamic + itexhip_qmatmul_device_range: the range of the float tensor, the op's parameter
+    math, the quantization and the MatMul's scale / bias derivation all on the device.  Bit-equal to QuantizeV2 fed
+    with the tensor's min and max followed by the MatMul fed with its output range (oracle), for the small-M and the
+    tile kernels, unaligned sizes included."""
+    import torch
+    rng = np.random.default_rng(M * 7 + K + N)
+    x = (rng.standard_normal((M, K)) * 2.5 + (0.4 if T == orc.QUINT8 and mode == orc.SCALED else 0.0)).astype(np.float32)
+    if T == orc.QUINT8 and mode == orc.SCALED:
+        x = np.abs(x)
+    layer, w, bias = make_layer(hip, dev, K, N, seed=K + N + 3)
+    _, xq_ref, omn, omx = orc.quantize_v2(x, x.min(), x.max(), T, mode)
+    x_d = torch.from_numpy(x).to(dev)
+    xq_d = torch.empty((M, K), dtype=tdt(T), device=dev)
+    state = torch.full((8,), float("nan"), dtype=torch.float32, device=dev)
+    for emr in (0.01,):
+        hip.quantize_dynamic(x_d, xq_d, M * K, T, mode, emr, state)
+    torch.cuda.synchronize()
+    st = state.cpu().numpy()
+    assert st[0] == x.min() and st[1] == x.max()
+    assert st[2] == omn[0] and st[3] == omx[0]
+    np.testing.assert_array_equal(xq_d.cpu().numpy(), xq_ref)
+    r_out = float(np.abs(x @ w + bias).max())
+    for kw in (dict(V2_DEQ, input_mode=mode), dict(V2_REQ_S8, input_mode=mode),
+               dict(V2_DEQ, input_mode=mode, activation=orc.ACT_GELU_APPROX)):
+        p = hip.matmul_params(t_in=T, min_a=123.0, max_a=-7.0, min_out=-r_out, max_out=r_out, **kw)   # min_a / max_a unused
+        out = torch.empty((M, N), dtype=tdt(kw["t_out"]), device=dev)
+        hip.qmatmul_device_range(p, xq_d, layer.packed, layer.colsum, M, K, N, state[2:], layer.min_b_d, layer.max_b_d,
+                                 layer.min_b.size, layer.bias_d, out)
+        torch.cuda.synchronize()
+        ref = layer.oracle(xq_ref, kw, float(omn[0]), float(omx[0]), -r_out, r_out)
+        if kw.get("activation"):
+            np.testing.assert_allclose(out.cpu().numpy(), ref, rtol=2e-6, atol=1e-6)
+        else:
+            np.testing.assert_array_equal(out.cpu().numpy(), ref)
+
+
+def test_dynamic_quantize_range_floor_and_constant_tensors(hip, dev):
+    """ensure_minimum_range widens a degenerate range exactly as the host code does (quantize_op.h:130-152): all-zero,
+    constant positive, constant negative and tiny tensors, both modes."""
+    import torch
+    for fill, emr in ((0.0, 0.01), (3.0, 0.01), (-2.0, 0.01), (1e-6, 0.5), (0.0, 0.0 + 1e-3)):
+        x = np.full(37, fill, np.float32)
+        for T, mode in ((orc.QUINT8, orc.MIN_FIRST), (orc.QINT8, orc.SCALED)):
+            _, q_ref, omn, omx = orc.quantize_v2(x, x.min(), x.max(), T, mode, ensure_minimum_range=emr)
+            x_d = torch.from_numpy(x).to(dev)
+            q_d = torch.empty(37, dtype=tdt(T), device=dev)
+            state = torch.zeros(8, dtype=torch.float32, device=dev)
+            hip.quantize_dynamic(x_d, q_d, 37, T, mode, emr, state)
+            torch.cuda.synchronize()
+            st = state.cpu().numpy()
+            assert st[2] == omn[0] and st[3] == omx[0], (fill, emr, T, st, omn, omx)
+            np.testing.assert_array_equal(q_d.cpu().numpy(), q_ref)
+    with pytest.raises(hip.ItexHipError):
+        hip.quantize_dynamic(x_d, q_d, 0, orc.QINT8, orc.SCALED, 0.01, state)
+    with pytest.raises(hip.ItexHipError):
+        hip.quantize_dynamic(x_d, q_d, 37, orc.QINT8, orc.MIN_FIRST, 0.01, state)
+
+
 @pytest.mark.parametrize("M", [1, 2, 4, 7, 16])
 @pytest.mark.parametrize("K,N", [(64, 16), (256, 100), (4096, 512), (1024, 4096), (8192, 48), (64, 8200), (512, 16384)])
 @pytest.mark.parametrize("kw", [V2_DEQ, V2_REQ_S8])

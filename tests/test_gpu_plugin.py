@@ -140,6 +140,50 @@ def test_dynamic_range_quantize_through_plugin(rt, dev, T, mode, classic):
         node.close()
 
 
+@pytest.mark.parametrize("T,mode", [(tf.QUINT8, "MIN_FIRST"), (tf.QINT8, "SCALED")])
+@pytest.mark.parametrize("M,K,N", [(100, 256, 200), (8, 1024, 512), (37, 75, 61)])
+def test_dynamic_input_matmul_through_plugin(rt, dev, T, mode, M, K, N):
+    """_ITEXQuantizedMatMulDynamicInput (what the graph pass makes of _ITEXQuantizeV2DynamicRange -> _ITEXQuantizedMatMul):
+    float activations in, the result of the two separate ops out - Dequantize and Requantize outputs, MFMA kernels and
+    (K = 75) the kernel on the unpacked weight; the second run reuses the node's cached weight."""
+    torch = rt
+    x, w, bias, _, _, _, wq, wmn, wmx = make_problem(M, K, N, seed=M + N)
+    omode = orc.SCALED if mode == "SCALED" else orc.MIN_FIRST
+    _, xq, xmn, xmx = orc.quantize_v2(x, x.min(), x.max(), T, omode)
+    r_out = np.float32(np.abs(x @ w + bias).max())
+    keep = [dev_in(torch, dev, x), dev_in(torch, dev, wq), dev_in(torch, dev, bias)]
+    base = [(tf.FLOAT, x.shape, keep[0].data_ptr(), False), (tf.QINT8, wq.shape, keep[1].data_ptr(), False),
+            (tf.FLOAT, bias.shape, keep[2].data_ptr(), False)]
+    stream = torch.cuda.current_stream().cuda_stream
+    for fused, t_out, host in ((["BiasAdd", "Relu", "Dequantize"], tf.FLOAT, [wmn, wmx]),
+                               (["BiasAdd", "Requantize"], tf.QINT8, [wmn, wmx, np.float32(-r_out), np.float32(r_out)])):
+        node = tf.Node("_ITEXQuantizedMatMulDynamicInput",
+                       dict(V2, T1=DT(T), input_quant_mode=mode, Tout=DT(t_out), fused_ops=fused, ensure_minimum_range=0.01))
+        assert node.code == tf.OK, node.message
+        requant = t_out == tf.QINT8
+        at = orc.matmul_attrs(api=orc.API_V2, t_in=T, t_out=t_out, input_mode=omode, has_dequantize=not requant,
+                              has_requantize=requant, activation=orc.ACT_NONE if requant else orc.ACT_RELU)
+        st, ref = orc.qmatmul(at, xq, wq, bias, xmn[0], xmx[0], wmn, wmx, -r_out if requant else 0.0, r_out if requant else 0.0)
+        assert st == orc.OK
+        ins = base + [(tf.FLOAT, np.shape(h), tf.host_array(np.asarray(h, np.float32)), True) for h in host]
+        outs_spec = [(t_out, False)] + ([(tf.FLOAT, True), (tf.FLOAT, True)] if requant else [])
+        for _ in range(2):
+            code, msg, outs = node.run(ins, outs_spec, stream=stream)
+            assert code == tf.OK, msg
+            np.testing.assert_array_equal(fetch(torch, outs[0], tf.NP_OF[t_out]), ref)
+        if requant:
+            assert float(np.ravel(fetch(torch, outs[1], np.float32))[0]) == -r_out
+            assert float(np.ravel(fetch(torch, outs[2], np.float32))[0]) == r_out
+        node.close()
+
+
+def test_dynamic_input_matmul_attr_validation(rt, dev):
+    bad = tf.Node("_ITEXQuantizedMatMulDynamicInput", dict(V2, Tout=DT(tf.FLOAT), fused_ops=["BiasAdd", "Add", "Dequantize"]))
+    assert bad.code == tf.INVALID_ARGUMENT
+    bad = tf.Node("_ITEXQuantizedMatMulDynamicInput", dict(V2, T1=DT(tf.QINT8), Tout=DT(tf.FLOAT), fused_ops=["BiasAdd", "Dequantize"]))
+    assert bad.code == tf.INVALID_ARGUMENT and "quint8" in bad.message     # MIN_FIRST gives quint8
+
+
 @pytest.mark.parametrize("fused,act", [("Tanh", orc.ACT_TANH), ("Sigmoid", orc.ACT_SIGMOID), ("_ITEXSwish", orc.ACT_SWISH)])
 def test_quantized_matmul_transcendental_post_ops(rt, dev, fused, act):
     """_QuantizedMatMul [BiasAdd, Tanh | Sigmoid | _ITEXSwish, Dequantize] (a BERT pooler, gates): within 2e-6 of the oracle

@@ -194,6 +194,72 @@ def test_dynamic_range_switch_and_placement(opt, monkeypatch):
     assert out["q"].op == "_ITEXQuantizeV2" and len(out["q"].input) == 4
 
 
+def dynamic_linear_graph(fused_ops=("BiasAdd", "Dequantize"), q_mode="MIN_FIRST", m_mode="MIN_FIRST", t_q=QUINT8, t1=QUINT8,
+                         extra_reader=False, with_out_range=False, mm_device=DEV, emr=0.02):
+    """x -> Reshape -> Min / Max -> QuantizeV2 -> _QuantizedMatMul, as a dynamically quantized linear arrives"""
+    g = gd.GraphDef()
+    gd.node(g, "x", "Placeholder", [], DEV)
+    gd.node(g, "shape", "Const", [], CPU, value=("tensor", 3, (1,), [-1], False))
+    gd.node(g, "axis", "Const", [], CPU, value=("tensor", 3, (), [0], False))
+    gd.node(g, "flat", "Reshape", ["x", "shape"], DEV)
+    gd.node(g, "mn", "Min", ["flat", "axis"], DEV, keep_dims=False)
+    gd.node(g, "mx", "Max", ["flat", "axis"], DEV, keep_dims=False)
+    gd.node(g, "q", "QuantizeV2", ["x", "mn", "mx", "^ctl_q"], DEV, T=("type", t_q), mode=q_mode,
+            round_mode="HALF_TO_EVEN" if q_mode == "SCALED" else "HALF_AWAY_FROM_ZERO", axis=-1, ensure_minimum_range=emr)
+    host = ["q:1", "q:2", "wmn", "wmx"] + (["omn", "omx"] if with_out_range else [])
+    gd.node(g, "mm", "_QuantizedMatMul", ["q", "w", "b"] + host + ["^ctl_m"], mm_device, T1=("type", t1), T2=("type", QINT8),
+            Tbias=("type", FLOAT), Tout=("type", QINT8 if with_out_range else FLOAT), fused_ops=list(fused_ops),
+            input_quant_mode=m_mode, Tdevice_inputs=("types", [t1, QINT8, FLOAT]), Thost_inputs=("types", [FLOAT] * len(host)),
+            Tdevice_outputs=("types", [QINT8 if with_out_range else FLOAT]),
+            Thost_outputs=("types", [FLOAT, FLOAT] if with_out_range else []))
+    if extra_reader:
+        gd.node(g, "spy", "Identity", ["q:1"], CPU)
+    return g
+
+
+@pytest.mark.parametrize("with_out_range", [False, True])
+def test_dynamic_quantize_and_matmul_become_one_node(opt, with_out_range):
+    """_ITEXQuantizeV2DynamicRange(x) read only by an _ITEXQuantizedMatMul -> _ITEXQuantizedMatMulDynamicInput(x, w, bias,
+    min_b, max_b[, min_out, max_out]): the quantize node goes, its range floor and control inputs move over, the type
+    lists follow the inputs."""
+    fused = ("BiasAdd", "Relu", "Requantize") if with_out_range else ("BiasAdd", "Dequantize")
+    out = by_name(run(opt, dynamic_linear_graph(fused_ops=fused, with_out_range=with_out_range)))
+    assert "q" not in out
+    mm = out["mm"]
+    assert mm.op == "_ITEXQuantizedMatMulDynamicInput"
+    tail = ["omn", "omx"] if with_out_range else []
+    assert list(mm.input) == ["x", "w", "b", "wmn", "wmx"] + tail + ["^ctl_m", "^ctl_q"]
+    assert list(mm.attr["Tdevice_inputs"].list.type) == [FLOAT, QINT8, FLOAT]
+    assert list(mm.attr["Thost_inputs"].list.type) == [FLOAT] * (2 + len(tail))
+    assert mm.attr["T1"].type == QUINT8 and mm.attr["input_quant_mode"].s == b"MIN_FIRST"
+    assert abs(mm.attr["ensure_minimum_range"].f - 0.02) < 1e-9
+    assert [f.decode() for f in mm.attr["fused_ops"].list.s] == list(fused)
+    reg = tf.registry()
+    assert "_ITEXQuantizedMatMulDynamicInput" in {k["op"] for k in reg["kernels"]}
+    assert "_ITEXQuantizedMatMulDynamicInput" in {o["name"] for o in reg["ops"]}
+
+
+@pytest.mark.parametrize("kw", [dict(extra_reader=True),                                  # someone else reads the range
+                                dict(fused_ops=("BiasAdd",)),                             # qint32 result: its range is host math
+                                dict(fused_ops=("BiasAdd", "Add", "Dequantize")),         # an addend shifts the inputs
+                                dict(q_mode="SCALED", t_q=QINT8, t1=QINT8),               # modes disagree
+                                dict(t_q=QUINT8, t1=QINT8),                               # types disagree
+                                dict(mm_device=CPU)],                                     # the MatMul is not ours
+                         ids=["other_reader", "s32_out", "addend", "mode", "type", "placement"])
+def test_dynamic_quantize_matmul_pairs_that_stay_apart(opt, kw):
+    out = by_name(run(opt, dynamic_linear_graph(**kw)))
+    assert out["q"].op == "_ITEXQuantizeV2DynamicRange"
+    assert out["mm"].op in ("_ITEXQuantizedMatMul", "_QuantizedMatMul") and out["mm"].input[0] == "q"
+
+
+def test_dynamic_quantize_matmul_scaled_and_switch(opt, monkeypatch):
+    out = by_name(run(opt, dynamic_linear_graph(q_mode="SCALED", m_mode="SCALED", t_q=QINT8, t1=QINT8)))
+    assert "q" not in out and out["mm"].op == "_ITEXQuantizedMatMulDynamicInput"
+    monkeypatch.setenv("ITEX_AMD_FUSE_QUANTIZE_MATMUL", "0")
+    out = by_name(run(opt, dynamic_linear_graph()))
+    assert out["q"].op == "_ITEXQuantizeV2DynamicRange" and out["mm"].op == "_ITEXQuantizedMatMul"
+
+
 def test_reshape_is_only_renamed_for_qint8(opt):
     g = gd.GraphDef()
     gd.node(g, "a", "QuantizedReshape", ["x", "s", "mn", "mx"], DEV, T=("type", QINT8))
