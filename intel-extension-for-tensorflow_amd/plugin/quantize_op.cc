@@ -63,6 +63,27 @@ class QuantizeV2Op : public OpKernel {
     if (dynamic_) {
       ITEX_REQUIRES(ctx, axis_ == -1 && src_type_ == TF_FLOAT, TF_INVALID_ARGUMENT,
                     "the dynamic-range QuantizeV2 quantizes a float tensor per tensor");
+      // SCALED and the legacy MIN_FIRST algorithm: reduction, parameter math and quantization are enqueued back to
+      // back (itexhip_quantize_dynamic) and the host only waits once, at the end, for the two floats of the output
+      // range.  The classic zero-point algorithm takes the path below (range to the host, then QuantizeV2 as usual).
+      const bool device_params = src.NumElements() > 0 && !classic_ &&
+                                 (mode_ == Mode::SCALED || (mode_ == Mode::MIN_FIRST && T_ == TF_QUINT8));
+      if (device_params) {
+        Tensor dst = ctx->allocate_output(0, T_, src.shape());
+        Tensor out_min = ctx->allocate_output(1, TF_FLOAT, {});
+        Tensor out_max = ctx->allocate_output(2, TF_FLOAT, {});
+        Tensor state = ctx->allocate_temp(TF_FLOAT, {8});
+        if (!ctx->ok()) return;
+        float range[2] = {0.0f, 0.0f};
+        int st = itexhip_quantize_dynamic(src.flat<float>(), dst.data(), src.NumElements(), T_,
+                                          mode_ == Mode::SCALED ? ITEXHIP_SCALED : ITEXHIP_MIN_FIRST, ensure_minimum_range_,
+                                          state.flat<float>(), ctx->stream());
+        if (st == ITEXHIP_OK) st = itexhip_memcpy_d2h(range, state.flat<float>() + 2, sizeof(range), ctx->stream());
+        ITEX_REQUIRES(ctx, st == ITEXHIP_OK, TF_ABORTED, std::string("Operation received an exception: ") + itexhip_last_error());
+        out_min.flat<float>()[0] = range[0];
+        out_max.flat<float>()[0] = range[1];
+        return;
+      }
       in_min = ctx->allocate_temp(TF_FLOAT, {}, /*on_host=*/true);
       in_max = ctx->allocate_temp(TF_FLOAT, {}, /*on_host=*/true);
       Tensor range = ctx->allocate_temp(TF_FLOAT, {2});
