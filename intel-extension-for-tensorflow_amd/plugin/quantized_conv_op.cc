@@ -107,6 +107,9 @@ class QuantizedConv2DOp : public OpKernel {
       else if (f == "Dequantize") fuse_dequantize_ = true;
       else if (f == "Relu") { activation_ = ITEXHIP_ELT_RELU; if (sum_position_ == 0) sum_position_ = -1; }
       else if (f == "LeakyRelu") { activation_ = ITEXHIP_ELT_RELU; leaky_ = true; if (sum_position_ == 0) sum_position_ = -1; }
+      // quantized_conv_ops.h:83, 86, 100, 103 with the table's alpha = 1 (onednn_post_op_util.cc:38, 59-60)
+      else if (f == "Elu") { activation_ = ITEXHIP_ELT_ELU; transcendental_ = true; }
+      else if (f == "Sigmoid") { activation_ = ITEXHIP_ELT_LOGISTIC; transcendental_ = true; }
       else if (f == "Sum") sum_position_ = sum_position_ == -1 ? 2 : 1;  // after / before the activation
       else
         ITEX_REQUIRES(ctx, false, TF_UNIMPLEMENTED, "the " + f + " fusion of the quantized Conv2D is not implemented on this device");
@@ -114,6 +117,8 @@ class QuantizedConv2DOp : public OpKernel {
     if (sum_position_ < 0) sum_position_ = 0;
     if (leaky_) ITEX_REQUIRES_OK(ctx, ctx->GetAttr("alpha", &alpha_));
     ITEX_REQUIRES(ctx, !(depthwise_ && sum_position_ != 0), TF_UNIMPLEMENTED, "the depthwise convolution has no Sum fusion on this device");
+    ITEX_REQUIRES(ctx, !(transcendental_ && (depthwise_ || sum_position_ != 0)), TF_UNIMPLEMENTED,
+                  "Elu / Sigmoid are fused into the plain quantized Conv2D only (no Sum, not depthwise) on this device");
     if (sum_position_ != 0) {
       // quantized_conv_ops.h:202-218, 398-433: an 8-bit summand under an 8-bit output; the qint32 output with a float
       // summand (the graph before Requantize is fused) is not built
@@ -319,7 +324,8 @@ class QuantizedConv2DOp : public OpKernel {
       const bool pointwise = KH == 1 && KW == 1 && stride_h_ == 1 && stride_w_ == 1 && g.pad_top == 0 && g.pad_left == 0 &&
                              g.out_h == H && g.out_w == W && K == Kp;
       // windows the tile kernel can gather by itself (input channels a multiple of 16, ...) need no patch matrix
-      const bool implicit = !pointwise && itexhip_qconv2d_implicit_ok(&g, x.data(), O, t_out_, out.data()) != 0 &&
+      // (the implicit-GEMM kernels carry the cheap post-op chains only: Elu / Sigmoid go through the patch matrix)
+      const bool implicit = !pointwise && !transcendental_ && itexhip_qconv2d_implicit_ok(&g, x.data(), O, t_out_, out.data()) != 0 &&
                             (reinterpret_cast<uintptr_t>(summand_dev) & 3) == 0;
       if (!pointwise && !implicit) {
         cols = ctx->allocate_temp(t_in_, {M, Kp});
@@ -331,7 +337,7 @@ class QuantizedConv2DOp : public OpKernel {
       itexhip_epilogue ep{};
       ep.n_scales = static_cast<int>(depth);
       if (sum_position_ == 1) ep.elt[ep.n_eltwise++] = {ITEXHIP_ELT_SUM, sum_scale, 0.0f};
-      if (activation_ != 0) ep.elt[ep.n_eltwise++] = {activation_, leaky_ ? alpha_ : 0.0f, 0.0f};
+      if (activation_ != 0) ep.elt[ep.n_eltwise++] = {activation_, transcendental_ ? 1.0f : leaky_ ? alpha_ : 0.0f, 0.0f};
       if (sum_position_ == 2) ep.elt[ep.n_eltwise++] = {ITEXHIP_ELT_SUM, sum_scale, 0.0f};
       int st;
       if (summand_dev != nullptr) {
@@ -378,7 +384,7 @@ class QuantizedConv2DOp : public OpKernel {
   int64_t stride_h_ = 1, stride_w_ = 1, dil_h_ = 1, dil_w_ = 1;
   std::string padding_;
   std::vector<int64_t> explicit_;
-  bool fuse_bias_ = false, fuse_requantize_ = false, fuse_dequantize_ = false, leaky_ = false;
+  bool fuse_bias_ = false, fuse_requantize_ = false, fuse_dequantize_ = false, leaky_ = false, transcendental_ = false;
   int activation_ = 0;
   float alpha_ = 0.0f;
   bool is_filter_const_ = true;

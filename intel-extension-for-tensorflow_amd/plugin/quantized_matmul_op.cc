@@ -156,12 +156,14 @@ class QuantizedMatMulOp : public OpKernel {
     }
     Tensor min_b_t = ctx->input(min_b_idx), max_b_t = ctx->input(min_b_idx + 1);
     if (!ctx->ok()) return;
-    ITEX_REQUIRES(ctx, !transpose_a_, TF_UNIMPLEMENTED, "transpose_a is not supported by the quantized MatMul");
     ITEX_REQUIRES(ctx, a.dims() == 2 && w.dims() == 2, TF_INVALID_ARGUMENT, "quantized MatMul operands must be matrices");
     const TF_DataType bias_type = p_.t_bias == 0 ? TF_FLOAT : static_cast<TF_DataType>(p_.t_bias);
     ITEX_REQUIRES(ctx, a.dtype() == (dyn ? TF_FLOAT : v_.t_in) && w.dtype() == TF_QINT8 && bias.dtype() == bias_type, TF_INVALID_ARGUMENT,
                   "quantized MatMul operand types do not match the kernel");
-    const int64_t M = a.dim_size(0), K = a.dim_size(1);
+    // transpose_a: the reference swaps the two dimensions but still describes the buffer as a row-major [batch, k]
+    // matrix (:183-198, format_tag::nc), so nothing is transposed - the [k, batch] tensor is read as [batch, k].
+    // Reproduced as written.
+    const int64_t M = a.dim_size(transpose_a_ ? 1 : 0), K = a.dim_size(transpose_a_ ? 0 : 1);
     const int64_t N = transpose_b_ ? w.dim_size(0) : w.dim_size(1);
     ITEX_REQUIRES(ctx, (transpose_b_ ? w.dim_size(1) : w.dim_size(0)) == K, TF_INVALID_ARGUMENT,
                   "Matrix size-incompatible: In[0] inner dimension " + std::to_string(K) + " vs In[1]");

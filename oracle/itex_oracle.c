@@ -891,7 +891,13 @@ int orc_qconv_prepare(const orc_conv_attrs* at, int64_t N, float min_in, float m
     ep->elt[0].alg = ORC_ELT_RELU; ep->elt[0].alpha = 0.0f; ep->elt[0].beta = 0.0f; ep->n_eltwise = 1;
   } else if (at->activation == ORC_ACT_LEAKYRELU) {
     ep->elt[0].alg = ORC_ELT_RELU; ep->elt[0].alpha = at->alpha; ep->elt[0].beta = 0.0f; ep->n_eltwise = 1;
+  } else if (at->activation == ORC_ACT_ELU) {      /* table entries of onednn_post_op_util.cc:38, 59-60: alpha 1 */
+    ep->elt[0].alg = ORC_ELT_ELU; ep->elt[0].alpha = 1.0f; ep->elt[0].beta = 0.0f; ep->n_eltwise = 1;
+  } else if (at->activation == ORC_ACT_SIGMOID) {
+    ep->elt[0].alg = ORC_ELT_LOGISTIC; ep->elt[0].alpha = 1.0f; ep->elt[0].beta = 0.0f; ep->n_eltwise = 1;
   } else if (at->activation != ORC_ACT_NONE) {
+    /* "_FusedSwish" / "_FusedHardSwish" become "Swish" / "HardSwish" (:135-138); the table has no "Swish", and the
+     * result of AddOps is not checked (:225), so that fusion silently drops the activation: not restated */
     return ORC_UNIMPLEMENTED;
   }
   /* ---- bias, GetBiasHandle :448-597 */

@@ -164,8 +164,8 @@ int orc_qbatch_matmul(const int8_t* x, int x_rank, const int64_t* x_dims, const 
  * padding value is the integer 0): itex/core/kernels/common/quantized_conv_ops.h
  * (constructor :63-318, ExtendInt8PostOps :329-446, GetBiasHandle :448-597) over the geometry of
  * itex/core/kernels/common/conv_ops.h:615-716 / TensorFlow's GetWindowedOutputSizeVerbose.
- * Fusions restated: BiasAdd, Relu, LeakyRelu, Requantize, Dequantize.  Sum, Elu, Swish, HardSwish,
- * Sigmoid and the depthwise / 3-D variants are not.
+ * Fusions restated: BiasAdd, Relu, LeakyRelu, Elu, Sigmoid, Requantize, Dequantize (Sum and the depthwise form: the
+ * functions further down).  Swish, HardSwish and the 3-D variants are not.
  * Pinned by: brute force against float64 direct convolution of the integer operands; the fp32
  * convolution at the reference's own tolerance (native_quantized_conv_test.py: rtol = atol = 0.3) and
  * at the bound the quantization steps allow; closed forms of the scales; padding identities.
@@ -183,7 +183,7 @@ typedef struct {
   int t_in;              /* ORC_QUINT8 | ORC_QINT8 */
   int t_out;             /* ORC_QINT32 | ORC_QINT8 | ORC_QUINT8 | ORC_FLOAT | ORC_BFLOAT16 */
   int t_bias;            /* 0: no BiasAdd;  ORC_FLOAT | ORC_QINT32 */
-  int activation;        /* ORC_ACT_NONE | ORC_ACT_RELU | ORC_ACT_LEAKYRELU */
+  int activation;        /* ORC_ACT_NONE | ORC_ACT_RELU | ORC_ACT_LEAKYRELU | ORC_ACT_ELU | ORC_ACT_SIGMOID */
   float alpha;           /* LeakyRelu */
 } orc_conv_attrs;
 /* output extent and leading padding of one spatial dimension; returns ORC_INVALID_ARGUMENT for a negative extent */

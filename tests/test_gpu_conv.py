@@ -444,6 +444,49 @@ def test_new_api_conv_through_plugin(rt, dev, t_in, fused, t_out, t_bias):
         node.close()
 
 
+@pytest.mark.parametrize("fused,t_out", [(["BiasAdd", "Elu", "Dequantize"], tf.FLOAT), (["BiasAdd", "Sigmoid", "Dequantize"], tf.FLOAT),
+                                         (["BiasAdd", "Elu", "Requantize"], tf.QINT8), (["BiasAdd", "Sigmoid", "Requantize"], tf.QUINT8)])
+def test_elu_and_sigmoid_fusions_through_plugin(rt, dev, fused, t_out):
+    """_QuantizedConv2D [BiasAdd, Elu | Sigmoid, Requantize | Dequantize] (quantized_conv_ops.h:83, 86, 100, 103): the
+    activation works on the already scaled value (the output scale, requantization included, comes first).  Float
+    results within 2e-6 of the oracle (the device evaluates exp with the hardware instruction), 8-bit ones equal or, where
+    the float value sits on a rounding boundary, one unit off.  A 3x3 window on 16 channels (would be the implicit
+    GEMM) and a 1x1 one."""
+    torch = rt
+    for shape, wshape in (((2, 9, 8, 16), (3, 3, 16, 32)), ((1, 6, 6, 32), (1, 1, 32, 16))):
+        rng = np.random.default_rng(shape[1] + len(fused[1]))
+        x = rng.uniform(0.0, 3.0, shape).astype(np.float32)
+        w = rng.uniform(-1.0, 1.0, wshape).astype(np.float32)
+        xq, xmn, xmx, wq, fmn, fmx = quantize_inputs(x, w, tf.QUINT8)
+        b = rng.uniform(-1.0, 1.0, wshape[3]).astype(np.float32)
+        node = tf.Node("_QuantizedConv2D", dict(Tinput=DT(tf.QUINT8), Tfilter=DT(tf.QINT8), Tbias=DT(tf.FLOAT), Tsummand=DT(t_out),
+                                                out_type=DT(t_out), strides=[1, 1, 1, 1], padding="SAME", dilations=[1, 1, 1, 1],
+                                                fused_ops=fused, alpha=0.2, data_format="NHWC", is_filter_const=True,
+                                                is_bias_const=True))
+        assert node.code == tf.OK, node.message
+        req = "Requantize" in fused
+        zmn, zmx = np.array(-4.0 if t_out == tf.QINT8 else 0.0, np.float32), np.array(6.0, np.float32)
+        scalars = [xmn, xmx, fmn, fmx] + ([zmn, zmx] if req else [])
+        at = orc.ConvAttrs(tf.QUINT8, t_out, orc.FLOAT, orc.ACT_ELU if "Elu" in fused else orc.ACT_SIGMOID, 0.2)
+        g = orc.conv_geom(shape, wshape, (1, 1), (1, 1), orc.PAD_SAME, (0, 0, 0, 0))
+        st, ref = orc.qconv2d(at, g, xq, wq, b, float(xmn), float(xmx), fmn, fmx, float(zmn), float(zmx))
+        assert st == orc.OK
+        got, _res = run_conv(torch, dev, node, xq, wq, b, tf.FLOAT, scalars, t_out, NP[t_out], req)
+        if t_out == tf.FLOAT:
+            np.testing.assert_allclose(got, ref, rtol=2e-6, atol=1e-6)
+        else:
+            d = np.abs(got.astype(np.int32) - ref.astype(np.int32))
+            assert d.max() <= 1 and (d > 0).mean() < 1e-3
+        node.close()
+    for bad in (["BiasAdd", "_FusedSwish", "Dequantize"], ["BiasAdd", "_FusedHardSwish", "Requantize"]):
+        bad_out = tf.QINT8 if "Requantize" in bad else tf.FLOAT
+        n = tf.Node("_QuantizedConv2D", dict(Tinput=DT(tf.QUINT8), Tfilter=DT(tf.QINT8), Tbias=DT(tf.FLOAT), Tsummand=DT(bad_out),
+                                             out_type=DT(bad_out), strides=[1, 1, 1, 1],
+                                             padding="SAME", dilations=[1, 1, 1, 1], fused_ops=bad, alpha=0.2, data_format="NHWC",
+                                             is_filter_const=True, is_bias_const=True))
+        assert n.code == tf.UNIMPLEMENTED
+
+
 @pytest.mark.parametrize("op,t_sum,fused", [
     ("QuantizedConv2DWithBiasSumAndReluAndRequantize", tf.QUINT8, None),
     ("QuantizedConv2DWithBiasSignedSumAndReluAndRequantize", tf.QINT8, None),

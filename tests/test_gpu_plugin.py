@@ -177,6 +177,25 @@ def test_dynamic_input_matmul_through_plugin(rt, dev, T, mode, M, K, N):
         node.close()
 
 
+def test_quantized_matmul_transpose_a_as_written(rt, dev):
+    """transpose_a = true: the reference takes batch and k from the swapped dimensions but describes the buffer as a
+    row-major [batch, k] matrix (quantized_matmul_common.h:183-198), i.e. the [k, batch] tensor is reinterpreted, not
+    transposed.  The plugin gives what the reference gives."""
+    torch = rt
+    M, K, N = 24, 64, 48
+    x, w, bias, xq, xmn, xmx, wq, wmn, wmx = make_problem(M, K, N, seed=5)
+    node = tf.Node("_QuantizedMatMul", dict(V2, transpose_a=True, Tout=DT(tf.FLOAT), fused_ops=["BiasAdd", "Dequantize"]))
+    assert node.code == tf.OK, node.message
+    at = orc.matmul_attrs(api=orc.API_V2, t_in=orc.QUINT8, t_out=orc.FLOAT, input_mode=orc.MIN_FIRST, has_dequantize=True)
+    _, ref = orc.qmatmul(at, xq, wq, bias, xmn, xmx, wmn, wmx)
+    as_k_by_m = xq.reshape(K, M)          # the same bytes, declared [k, batch]
+    ins, keep = matmul_inputs(torch, dev, as_k_by_m, wq, bias, [xmn, xmx, wmn, wmx])
+    code, msg, outs = node.run(ins, [(tf.FLOAT, False)], stream=torch.cuda.current_stream().cuda_stream)
+    assert code == tf.OK, msg
+    np.testing.assert_array_equal(fetch(torch, outs[0], np.float32), ref)
+    node.close()
+
+
 def test_dynamic_input_matmul_attr_validation(rt, dev):
     bad = tf.Node("_ITEXQuantizedMatMulDynamicInput", dict(V2, Tout=DT(tf.FLOAT), fused_ops=["BiasAdd", "Add", "Dequantize"]))
     assert bad.code == tf.INVALID_ARGUMENT

@@ -147,6 +147,36 @@ def test_reference_test_pipelines_on_seeded_inputs(case):
     assert np.abs(got - ref).max() > 0
 
 
+@pytest.mark.parametrize("act", ["elu", "sigmoid"])
+def test_elu_and_sigmoid_act_on_the_scaled_value(act):
+    """[BiasAdd, Elu | Sigmoid, Requantize | Dequantize] (quantized_conv_ops.h:83, 86, 100, 103): the output scale -
+    requantization included - is applied first, the activation (table alpha 1, post-op scale 1, :436-445) sees that
+    value.  Checked against the activation-free convolution: float output = act(float output without it) in float64;
+    8-bit output = sat(rne(act(v))) with v rebuilt from the activation-free float output times 127 / range_out."""
+    rng = np.random.default_rng(9)
+    x = rng.integers(0, 256, (1, 6, 5, 8)).astype(np.uint8)
+    w = rng.integers(-127, 128, (3, 3, 8, 4)).astype(np.int8)
+    bias = rng.standard_normal(4).astype(np.float32)
+    fmn, fmx = np.full(4, -0.05, np.float32), np.full(4, 0.05, np.float32)
+    g = orc.conv_geom(x.shape, w.shape, (1, 1), (1, 1), orc.PAD_SAME, (0, 0, 0, 0))
+    code = orc.ACT_ELU if act == "elu" else orc.ACT_SIGMOID
+    f = (lambda v: np.where(v > 0, v, np.expm1(v))) if act == "elu" else (lambda v: 1.0 / (1.0 + np.exp(-v)))
+    _, plain = orc.qconv2d(orc.ConvAttrs(orc.QUINT8, orc.FLOAT, orc.FLOAT, orc.ACT_NONE, 0.0), g, x, w, bias, 0.0, 2.0, fmn, fmx)
+    st, got = orc.qconv2d(orc.ConvAttrs(orc.QUINT8, orc.FLOAT, orc.FLOAT, code, 0.0), g, x, w, bias, 0.0, 2.0, fmn, fmx)
+    assert st == orc.OK
+    np.testing.assert_allclose(got, f(plain.astype(np.float64)), rtol=1e-6, atol=1e-7)
+    r_out = 3.0
+    st, q = orc.qconv2d(orc.ConvAttrs(orc.QUINT8, orc.QINT8, orc.FLOAT, code, 0.0), g, x, w, bias, 0.0, 2.0, fmn, fmx, -r_out, r_out)
+    assert st == orc.OK
+    v = f(plain.astype(np.float64) * (127.0 / r_out))
+    want = np.clip(np.rint(v), -128, 127)
+    near_tie = np.abs(v - np.floor(v) - 0.5) < 1e-3           # the float32 value may fall on the other side
+    assert np.all((q == want) | near_tie) and near_tie.mean() < 0.02
+    # the swish spellings are refused (the reference's table has no entry for the name the op looks up)
+    st, _ = orc.qconv2d(orc.ConvAttrs(orc.QUINT8, orc.FLOAT, orc.FLOAT, orc.ACT_SWISH, 0.0), g, x, w, bias, 0.0, 2.0, fmn, fmx)
+    assert st == orc.UNIMPLEMENTED
+
+
 def test_scales_closed_forms_and_qint32_forms():
     rng = np.random.default_rng(4)
     N = 6
