@@ -196,6 +196,60 @@ def test_quantized_matmul_transpose_a_as_written(rt, dev):
     node.close()
 
 
+def test_graph_pass_output_runs_on_the_kernel(rt, dev):
+    """x -> Reshape -> Min / Max -> QuantizeV2 -> _QuantizedMatMul through TF_InitGraph's optimizer, then the one node it
+    leaves, built from the attributes and the input order of the rewritten NodeDef, on the device: equal to the two ops
+    evaluated by the oracle."""
+    import ctypes as C
+    from tests.mock_tf import graphdef as gd
+    from tests.test_graph_optimizer import dynamic_linear_graph
+    torch = rt
+    lib = tf.load()
+    lib.mock_graph_result.restype = C.c_void_p
+    lib.mock_graph_result_size.restype = C.c_size_t
+    assert lib.mock_graph_init(tf.PLUGIN_LIB.encode()) == 0
+    data = dynamic_linear_graph(emr=0.01).SerializeToString()
+    assert lib.mock_graph_optimize(data, C.c_size_t(len(data))) == tf.OK
+    out = gd.GraphDef()
+    out.ParseFromString(C.string_at(lib.mock_graph_result(), lib.mock_graph_result_size()))
+    mm = {n.name: n for n in out.node}["mm"]
+    assert mm.op == "_ITEXQuantizedMatMulDynamicInput"
+    attrs = {}
+    for k, v in mm.attr.items():
+        kind = v.WhichOneof("value")
+        if kind == "type":
+            attrs[k] = DT(v.type)
+        elif kind == "s":
+            attrs[k] = v.s.decode()
+        elif kind in ("b", "f", "i"):
+            attrs[k] = getattr(v, kind)
+        elif kind == "list" and len(v.list.s):
+            attrs[k] = [x.decode() for x in v.list.s]
+    node = tf.Node(mm.op, dict(V2, **attrs))      # attributes the graph leaves at their defaults come from V2
+    assert node.code == tf.OK, node.message
+    M, K, N = 33, 128, 80
+    x, w, bias, xq, xmn, xmx, wq, wmn, wmx = make_problem(M, K, N, seed=3)
+    tensors = {"x": x, "w": wq, "b": bias, "wmn": wmn, "wmx": wmx}
+    keep, ins = [], []
+    n_dev = len(mm.attr["Tdevice_inputs"].list.type)
+    data_inputs = [i for i in mm.input if not i.startswith("^")]
+    assert len(data_inputs) == n_dev + len(mm.attr["Thost_inputs"].list.type)
+    for pos, name in enumerate(data_inputs):
+        t = tensors[name]
+        dt = {np.float32: tf.FLOAT, np.int8: tf.QINT8}[t.dtype.type]
+        if pos < n_dev:
+            keep.append(dev_in(torch, dev, t))
+            ins.append((dt, t.shape, keep[-1].data_ptr(), False))
+        else:
+            ins.append((dt, t.shape, tf.host_array(t), True))
+    code, msg, outs = node.run(ins, [(tf.FLOAT, False)], stream=torch.cuda.current_stream().cuda_stream)
+    assert code == tf.OK, msg
+    at = orc.matmul_attrs(api=orc.API_V2, t_in=orc.QUINT8, t_out=orc.FLOAT, input_mode=orc.MIN_FIRST, has_dequantize=True)
+    _, ref = orc.qmatmul(at, xq, wq, bias, xmn, xmx, wmn, wmx)
+    np.testing.assert_array_equal(fetch(torch, outs[0], np.float32), ref)
+    node.close()
+
+
 def test_dynamic_input_matmul_attr_validation(rt, dev):
     bad = tf.Node("_ITEXQuantizedMatMulDynamicInput", dict(V2, Tout=DT(tf.FLOAT), fused_ops=["BiasAdd", "Add", "Dequantize"]))
     assert bad.code == tf.INVALID_ARGUMENT
