@@ -166,6 +166,7 @@ int itexhip_minmax_f32(const float* x, int64_t n, float* minmax_out, void* strea
  * ITEXHIP_MIN_FIRST (quint8, the non-classic algorithm).  `state` is a device array of 8 floats:
  * [0..1] the tensor's min and max, [2..3] the op's output_min / output_max (what a consuming MatMul takes as
  * min_a / max_a: pass state + 2 to itexhip_qmatmul_device_range), [4..5] scale and addend.  n > 0.  The reference
+ * (Up to 128 K elements, 16-byte aligned, n a multiple of 4: all three steps in one launch.)  The reference
  * has no such op (its QuantizeV2 takes the range from the host); this is the producer half of the
  * Min/Max -> QuantizeV2 -> MatMul fusion of this plugin's graph pass. */
 int itexhip_quantize_dynamic(const float* x, void* q, int64_t n, int dst_type, int mode, float ensure_minimum_range,

@@ -401,33 +401,110 @@ __device__ __forceinline__ float host_max(float a, float b) { return a < b ? b :
 // The QuantizeV2 parameter math of a per-tensor range, on the device (quantize_op.h:130-152 range adjustment,
 // quantization_util.h:54-84 SCALED scale, quantize_op.h:204-214 legacy MIN_FIRST scale): state[0..1] = the tensor's
 // min and max -> state[2..3] = the op's output_min / output_max, state[4..5] = scale and addend of the kernel.
-__global__ void quantize_dynamic_params_kernel(float* state, int dst_type, int mode, float ensure_minimum_range) {
-  // state[0..1] arrive as the reduction's integer keys; they leave as floats
-  const float in_min = key2f(reinterpret_cast<const int*>(state)[0]), in_max = key2f(reinterpret_cast<const int*>(state)[1]);
-  state[0] = in_min;
-  state[1] = in_max;
+struct DynamicParams {
+  float out_min, out_max, scale, addend;
+};
+
+__device__ __forceinline__ DynamicParams dynamic_params(float in_min, float in_max, int dst_type, int mode,
+                                                        float ensure_minimum_range) {
   const float lo = host_min(0.0f, in_min);
   const float epsilon = host_max(1.0f, host_max(fabsf(in_min), fabsf(in_max))) * ensure_minimum_range;
   const float widened = lo + epsilon;
   float mn = lo, mx = host_max(0.0f, host_max(in_max, widened));
-  float scale, addend;
+  DynamicParams p;
   if (mode == ITEXHIP_SCALED) {
     const float q_high = dst_type == ITEXHIP_QINT8 ? 127.0f : 255.0f;
     const float r = host_max(fabsf(mn), fabsf(mx));
     mx = r;
     mn = -r;
-    scale = q_high / r;
-    addend = 0.0f;
+    p.scale = q_high / r;
+    p.addend = 0.0f;
     if (dst_type == ITEXHIP_QUINT8) mn = 0.0f;  // output_min of an unsigned SCALED result (:402-408)
   } else {  // the 255 steps are a double, so the division is done in double and rounded once
-    scale = static_cast<float>(255.0 / static_cast<double>(mx - mn));
+    p.scale = static_cast<float>(255.0 / static_cast<double>(mx - mn));
     const float shift = -mn;
-    addend = shift * scale;
+    p.addend = shift * p.scale;
   }
-  state[2] = mn;
-  state[3] = mx;
-  state[4] = scale;
-  state[5] = addend;
+  p.out_min = mn;
+  p.out_max = mx;
+  return p;
+}
+
+__global__ void quantize_dynamic_params_kernel(float* state, int dst_type, int mode, float ensure_minimum_range) {
+  // state[0..1] arrive as the reduction's integer keys; they leave as floats
+  const float in_min = key2f(reinterpret_cast<const int*>(state)[0]), in_max = key2f(reinterpret_cast<const int*>(state)[1]);
+  const DynamicParams p = dynamic_params(in_min, in_max, dst_type, mode, ensure_minimum_range);
+  state[0] = in_min;
+  state[1] = in_max;
+  state[2] = p.out_min;
+  state[3] = p.out_max;
+  state[4] = p.scale;
+  state[5] = p.addend;
+}
+
+// Small tensors (a decode batch: a few rows of activations) in ONE launch: every workgroup reduces the whole tensor
+// (it comes from L2 after the first touch), derives the parameters, and quantizes its own slice; workgroup 0 also
+// leaves the state.  Several kernels in a row would cost more in launches than in work at this size.
+constexpr int kSmallThreads = 1024;
+constexpr int kSmallLoads = 8;                                   // 16-byte loads in flight per thread
+constexpr int64_t kSmallMax = 4 * kSmallThreads * kSmallLoads * 4;   // elements: up to 4 rounds of loads per thread
+
+template <int T>
+__global__ __launch_bounds__(kSmallThreads) void quantize_dynamic_small_kernel(const f4* __restrict__ x4,
+                                                                               uint32_t* __restrict__ q4, int n4,
+                                                                               float* __restrict__ state, int mode,
+                                                                               float ensure_minimum_range) {
+  __shared__ float red[2 * (kSmallThreads / 64)];
+  __shared__ float params[2];
+  float mn = __builtin_inff(), mx = -__builtin_inff();
+  for (int base = threadIdx.x; base < n4; base += kSmallThreads * kSmallLoads) {
+    f4 v[kSmallLoads];
+#pragma unroll
+    for (int j = 0; j < kSmallLoads; ++j) {
+      const int i = base + j * kSmallThreads;
+      if (i < n4) v[j] = x4[i];
+    }
+#pragma unroll
+    for (int j = 0; j < kSmallLoads; ++j) {
+      if (base + j * kSmallThreads < n4) {
+        mn = fminf(fminf(mn, v[j].x), fminf(v[j].y, fminf(v[j].z, v[j].w)));
+        mx = fmaxf(fmaxf(mx, v[j].x), fmaxf(v[j].y, fmaxf(v[j].z, v[j].w)));
+      }
+    }
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    mn = fminf(mn, __shfl_xor(mn, o, 64));
+    mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+  }
+  const int wave = threadIdx.x >> 6;
+  if ((threadIdx.x & 63) == 0) {
+    red[2 * wave] = mn;
+    red[2 * wave + 1] = mx;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < kSmallThreads / 64; ++w) {
+      mn = fminf(mn, red[2 * w]);
+      mx = fmaxf(mx, red[2 * w + 1]);
+    }
+    const DynamicParams p = dynamic_params(mn, mx, T, mode, ensure_minimum_range);
+    params[0] = p.scale;
+    params[1] = p.addend;
+    if (blockIdx.x == 0) {
+      state[0] = mn;
+      state[1] = mx;
+      state[2] = p.out_min;
+      state[3] = p.out_max;
+      state[4] = p.scale;
+      state[5] = p.addend;
+    }
+  }
+  __syncthreads();
+  const float scale = params[0], addend = params[1];
+  const int per = (n4 + gridDim.x - 1) / gridDim.x;
+  const int end = min(n4, static_cast<int>(blockIdx.x + 1) * per);
+  for (int i = blockIdx.x * per + threadIdx.x; i < end; i += kSmallThreads) q4[i] = quantize4<T>(x4[i], scale, addend);
 }
 
 int launch_quantize(const char* who, const float* x, void* q, int64_t n, int dst_type, float scale, float addend,
@@ -479,6 +556,18 @@ extern "C" int itexhip_quantize_dynamic(const float* x, void* q, int64_t n, int 
                   "itexhip_quantize_dynamic: SCALED, or MIN_FIRST to quint8");
   ITEXHIP_REQUIRE(n > 0, "itexhip_quantize_dynamic: an empty tensor has no range");
   ITEXHIP_REQUIRE(x && q && state && aligned(state, 8), "itexhip_quantize_dynamic: null or unaligned buffer");
+  if (n <= kSmallMax && n % 4 == 0 && aligned(x, 16) && aligned(q, 4)) {
+    const int n4 = static_cast<int>(n / 4);
+    const unsigned grid = static_cast<unsigned>(std::min<int64_t>(16, (n4 + kSmallThreads - 1) / kSmallThreads));
+    if (dst_type == ITEXHIP_QINT8)
+      quantize_dynamic_small_kernel<ITEXHIP_QINT8><<<grid, kSmallThreads, 0, as_stream(stream)>>>(
+          reinterpret_cast<const f4*>(x), reinterpret_cast<uint32_t*>(q), n4, state, mode, ensure_minimum_range);
+    else
+      quantize_dynamic_small_kernel<ITEXHIP_QUINT8><<<grid, kSmallThreads, 0, as_stream(stream)>>>(
+          reinterpret_cast<const f4*>(x), reinterpret_cast<uint32_t*>(q), n4, state, mode, ensure_minimum_range);
+    ITEXHIP_CHECK_LAUNCH("itexhip_quantize_dynamic");
+    return ITEXHIP_OK;
+  }
   enqueue_minmax_f32(x, n, reinterpret_cast<int*>(state), as_stream(stream));
   quantize_dynamic_params_kernel<<<1, 1, 0, as_stream(stream)>>>(state, dst_type, mode, ensure_minimum_range);
   return launch_quantize("itexhip_quantize_dynamic", x, q, n, dst_type, 0.0f, 0.0f, state + 4, as_stream(stream));
