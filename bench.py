@@ -239,9 +239,18 @@ def bench_dynamic_linear(torch, hip, timer, M, K, N, steps, warmup, dev, seed):
         p.min_a, p.max_a = float(amn), float(amx)
         hip.qmatmul(p, xq, L["packed"], L["colsum"], M, K, N, L["min_b"], L["max_b"], N, L["bias"], out, st)
 
+    rmn = torch.empty(M, dtype=torch.float32, device=dev)
+    rmx = torch.empty(M, dtype=torch.float32, device=dev)
+
+    def per_token(i):   # every row against its own range (M <= 16)
+        hip.quantize_dynamic_rows(x, xq, M, K, hip.QUINT8, hip.MIN_FIRST, 0.01, rmn, rmx, st)
+        hip.qmatmul_per_row(p, xq, L["packed"], L["colsum"], M, K, N, rmn, rmx, L["min_b"], L["max_b"], N, L["bias"], out, st)
+
     ms_dev = timer.run(device_range, steps, warmup)
+    ms_tok = timer.run(per_token, steps, warmup) if M <= 16 else None
     ms_host = timer.run(host_range, steps, warmup)
     return dict(name="dynamic_linear_from_float", M=M, K=K, N=N, us_device_range=ms_dev * 1e3, us_host_range=ms_host * 1e3,
+                us_device_range_per_token=None if ms_tok is None else ms_tok * 1e3,
                 note="range + QuantizeV2 + MatMul[BiasAdd, Dequantize] per step; device_range: no host wait; host_range: "
                      "the range crosses to the host between reduction and quantization")
 

@@ -171,6 +171,12 @@ int itexhip_minmax_f32(const float* x, int64_t n, float* minmax_out, void* strea
  * Min/Max -> QuantizeV2 -> MatMul fusion of this plugin's graph pass. */
 int itexhip_quantize_dynamic(const float* x, void* q, int64_t n, int dst_type, int mode, float ensure_minimum_range,
                              float* state, void* stream);
+/* The per-row (per-token) form: row m of x [rows, cols] is quantized against its own range (QuantizeV2 with axis = 0 and
+ * the rows' min / max as ranges, quantize_op.h:166-190, same parameter math per row), one workgroup per row, one launch;
+ * row_min_out / row_max_out (device arrays of `rows` floats) receive the rows' output_min / output_max, which is what
+ * itexhip_qmatmul_per_row takes.  cols > 0. */
+int itexhip_quantize_dynamic_rows(const float* x, void* q, int64_t rows, int64_t cols, int dst_type, int mode,
+                                  float ensure_minimum_range, float* row_min_out, float* row_max_out, void* stream);
 
 /* ------------------------------------------------------------------------------------------
  * Quantized MatMul (oneDNN inner_product_forward u8/s8 x s8 -> s32 with fused epilogue;

@@ -507,6 +507,69 @@ __global__ __launch_bounds__(kSmallThreads) void quantize_dynamic_small_kernel(c
   for (int i = blockIdx.x * per + threadIdx.x; i < end; i += kSmallThreads) q4[i] = quantize4<T>(x4[i], scale, addend);
 }
 
+// Per-row (per-token) form: workgroup m reduces row m, derives its parameters and quantizes it; the rows' output
+// ranges go to two device arrays (what itexhip_qmatmul_per_row takes).
+constexpr int kRowThreads = 256;
+
+template <int T>
+__global__ __launch_bounds__(kRowThreads) void quantize_dynamic_rows_kernel(const float* __restrict__ x,
+                                                                            uint8_t* __restrict__ q, int cols, int vec,
+                                                                            float* __restrict__ row_min,
+                                                                            float* __restrict__ row_max, int mode,
+                                                                            float ensure_minimum_range) {
+  __shared__ float red[2 * (kRowThreads / 64)];
+  __shared__ float params[2];
+  const float* xr = x + static_cast<int64_t>(blockIdx.x) * cols;
+  uint8_t* qr = q + static_cast<int64_t>(blockIdx.x) * cols;
+  float mn = __builtin_inff(), mx = -__builtin_inff();
+  if (vec) {
+    const f4* x4 = reinterpret_cast<const f4*>(xr);
+    for (int i = threadIdx.x; i < cols / 4; i += kRowThreads) {
+      const f4 v = x4[i];
+      mn = fminf(fminf(mn, v.x), fminf(v.y, fminf(v.z, v.w)));
+      mx = fmaxf(fmaxf(mx, v.x), fmaxf(v.y, fmaxf(v.z, v.w)));
+    }
+  } else {
+    for (int i = threadIdx.x; i < cols; i += kRowThreads) {
+      mn = fminf(mn, xr[i]);
+      mx = fmaxf(mx, xr[i]);
+    }
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    mn = fminf(mn, __shfl_xor(mn, o, 64));
+    mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+  }
+  if ((threadIdx.x & 63) == 0) {
+    red[2 * (threadIdx.x >> 6)] = mn;
+    red[2 * (threadIdx.x >> 6) + 1] = mx;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < kRowThreads / 64; ++w) {
+      mn = fminf(mn, red[2 * w]);
+      mx = fmaxf(mx, red[2 * w + 1]);
+    }
+    const DynamicParams p = dynamic_params(mn, mx, T, mode, ensure_minimum_range);
+    params[0] = p.scale;
+    params[1] = p.addend;
+    row_min[blockIdx.x] = p.out_min;
+    row_max[blockIdx.x] = p.out_max;
+  }
+  __syncthreads();
+  const float scale = params[0], addend = params[1];
+  if (vec) {
+    const f4* x4 = reinterpret_cast<const f4*>(xr);
+    uint32_t* q4 = reinterpret_cast<uint32_t*>(qr);
+    for (int i = threadIdx.x; i < cols / 4; i += kRowThreads) q4[i] = quantize4<T>(x4[i], scale, addend);
+  } else {
+    for (int i = threadIdx.x; i < cols; i += kRowThreads) {
+      const float t = xr[i] * scale;
+      qr[i] = static_cast<uint8_t>(sat_rne<T>(t + addend));
+    }
+  }
+}
+
 int launch_quantize(const char* who, const float* x, void* q, int64_t n, int dst_type, float scale, float addend,
                     const float* dev_params, hipStream_t st) {
   int64_t done = 0;
@@ -571,6 +634,29 @@ extern "C" int itexhip_quantize_dynamic(const float* x, void* q, int64_t n, int 
   enqueue_minmax_f32(x, n, reinterpret_cast<int*>(state), as_stream(stream));
   quantize_dynamic_params_kernel<<<1, 1, 0, as_stream(stream)>>>(state, dst_type, mode, ensure_minimum_range);
   return launch_quantize("itexhip_quantize_dynamic", x, q, n, dst_type, 0.0f, 0.0f, state + 4, as_stream(stream));
+}
+
+extern "C" int itexhip_quantize_dynamic_rows(const float* x, void* q, int64_t rows, int64_t cols, int dst_type, int mode,
+                                             float ensure_minimum_range, float* row_min_out, float* row_max_out,
+                                             void* stream) {
+  ITEXHIP_REQUIRE(dst_type == ITEXHIP_QINT8 || dst_type == ITEXHIP_QUINT8,
+                  "itexhip_quantize_dynamic_rows: dst_type must be qint8 or quint8, got %d", dst_type);
+  ITEXHIP_REQUIRE(mode == ITEXHIP_SCALED || (mode == ITEXHIP_MIN_FIRST && dst_type == ITEXHIP_QUINT8),
+                  "itexhip_quantize_dynamic_rows: SCALED, or MIN_FIRST to quint8");
+  ITEXHIP_REQUIRE(rows >= 0 && rows < (1LL << 31) && cols > 0 && cols < (1LL << 31),
+                  "itexhip_quantize_dynamic_rows: bad shape (an empty row has no range)");
+  if (rows == 0) return ITEXHIP_OK;
+  ITEXHIP_REQUIRE(x && q && row_min_out && row_max_out, "itexhip_quantize_dynamic_rows: null buffer");
+  const int vec = cols % 4 == 0 && aligned(x, 16) && aligned(q, 4);
+  const unsigned grid = static_cast<unsigned>(rows);
+  if (dst_type == ITEXHIP_QINT8)
+    quantize_dynamic_rows_kernel<ITEXHIP_QINT8><<<grid, kRowThreads, 0, as_stream(stream)>>>(
+        x, reinterpret_cast<uint8_t*>(q), static_cast<int>(cols), vec, row_min_out, row_max_out, mode, ensure_minimum_range);
+  else
+    quantize_dynamic_rows_kernel<ITEXHIP_QUINT8><<<grid, kRowThreads, 0, as_stream(stream)>>>(
+        x, reinterpret_cast<uint8_t*>(q), static_cast<int>(cols), vec, row_min_out, row_max_out, mode, ensure_minimum_range);
+  ITEXHIP_CHECK_LAUNCH("itexhip_quantize_dynamic_rows");
+  return ITEXHIP_OK;
 }
 
 extern "C" int itexhip_quantize_axis(const float* x, void* q, int64_t outer, int64_t slices,

@@ -319,6 +319,41 @@ def test_dynamic_quantize_then_device_range_matmul(hip, dev, T, mode, M, K, N):
             np.testing.assert_array_equal(out.cpu().numpy(), ref)
 
 
+@pytest.mark.parametrize("T,mode", [(orc.QUINT8, orc.MIN_FIRST), (orc.QINT8, orc.SCALED)], ids=["min_first_u8", "scaled_s8"])
+@pytest.mark.parametrize("M,K,N", [(16, 1024, 96), (5, 448, 528), (3, 75 * 16, 40), (1, 16, 8)])
+def test_per_token_dynamic_quantize_then_per_row_matmul(hip, dev, T, mode, M, K, N):
+    """itexhip_quantize_dynamic_rows + itexhip_qmatmul_per_row: every row quantized against its own range on the device
+    and multiplied with that range.  Row m equals QuantizeV2 (axis 0, the rows' min / max) and the 1 x K MatMul fed with
+    row m's output range (oracle); also with an unaligned view (scalar path)."""
+    import torch
+    rng = np.random.default_rng(M + K)
+    x = (rng.standard_normal((M, K)) * (1.0 + np.arange(M)[:, None])).astype(np.float32)
+    layer, w, bias = make_layer(hip, dev, K, N, seed=K + N + 9)
+    _, xq_ref, omn, omx = orc.quantize_v2(x, x.min(1), x.max(1), T, mode, axis=0)
+    for shift in (0, 1):     # 1: the tensor starts 4 bytes off a 16-byte boundary
+        buf = torch.zeros(M * K + 4, dtype=torch.float32, device=dev)
+        x_d = buf[shift:shift + M * K].view(M, K)
+        x_d.copy_(torch.from_numpy(x))
+        xq_d = torch.empty((M, K), dtype=tdt(T), device=dev)
+        rmn = torch.empty(M, dtype=torch.float32, device=dev)
+        rmx = torch.empty(M, dtype=torch.float32, device=dev)
+        hip.quantize_dynamic_rows(x_d, xq_d, M, K, T, mode, 0.01, rmn, rmx)
+        torch.cuda.synchronize()
+        np.testing.assert_array_equal(xq_d.cpu().numpy(), xq_ref)
+        np.testing.assert_array_equal(rmn.cpu().numpy(), omn)
+        np.testing.assert_array_equal(rmx.cpu().numpy(), omx)
+    kw = dict(V2_DEQ, input_mode=mode)
+    p = hip.matmul_params(t_in=T, **kw)
+    out = torch.empty((M, N), dtype=torch.float32, device=dev)
+    hip.qmatmul_per_row(p, xq_d, layer.packed, layer.colsum, M, K, N, rmn, rmx, layer.min_b_d, layer.max_b_d, layer.min_b.size,
+                        layer.bias_d, out)
+    torch.cuda.synchronize()
+    got = out.cpu().numpy()
+    for m in range(M):
+        ref = layer.oracle(xq_ref[m:m + 1], kw, float(omn[m]), float(omx[m]))
+        np.testing.assert_array_equal(got[m:m + 1], ref)
+
+
 def test_dynamic_quantize_range_floor_and_constant_tensors(hip, dev):
     """ensure_minimum_range widens a degenerate range exactly as the host code does (quantize_op.h:130-152): all-zero,
     constant positive, constant negative and tiny tensors, both modes."""
