@@ -509,7 +509,7 @@ __global__ __launch_bounds__(kSmallThreads) void quantize_dynamic_small_kernel(c
 
 // Per-row (per-token) form: workgroup m reduces row m, derives its parameters and quantizes it; the rows' output
 // ranges go to two device arrays (what itexhip_qmatmul_per_row takes).
-constexpr int kRowThreads = 256;
+constexpr int kRowThreads = 1024;
 
 template <int T>
 __global__ __launch_bounds__(kRowThreads) void quantize_dynamic_rows_kernel(const float* __restrict__ x,
