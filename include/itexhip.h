@@ -292,11 +292,12 @@ int itexhip_qgemm_sum(const void* a, int a_type, const int8_t* packed_b, const i
  * operation sequence), so no parameter vectors and no second kernel are needed.  This is what the
  * op kernel calls per Compute (quantized_matmul_common.h:62-460: Init + primitive execute);
  * a changed min_a / max_a costs nothing extra.  `bias` is the op's raw bias (fp32; int32 when
- * p->t_bias is QINT32, 16-bit patterns when BFLOAT16 / HALF; may be null).  `addend` is the [M, N] fp32 tensor of the "Add" fusion
- * (p->add_position != 0; the reference adds it in place into the output buffer, :352-389), else null. */
+ * p->t_bias is QINT32, 16-bit patterns when BFLOAT16 / HALF; may be null).  `addend` is the [M, N] tensor of the "Add" fusion
+ * (p->add_position != 0; the reference adds it in place into the output buffer, :341-389, so it has the output's type:
+ * fp32, or 16-bit patterns for a bfloat16 / half result, widened exactly before the addition), else null. */
 int itexhip_qmatmul(const itexhip_matmul_params* p, const void* a, const int8_t* packed_b,
                     const int32_t* colsum, int64_t M, int64_t K, int64_t N, const float* min_b,
-                    const float* max_b, int64_t nb, const void* bias, const float* addend, void* out,
+                    const float* max_b, int64_t nb, const void* bias, const void* addend, void* out,
                     void* stream);
 
 /* Decode batches quantized per token: row m of `a` was quantized with its own range
@@ -308,7 +309,7 @@ int itexhip_qmatmul(const itexhip_matmul_params* p, const void* a, const int8_t*
 int itexhip_qmatmul_per_row(const itexhip_matmul_params* p, const void* a, const int8_t* packed_b,
                             const int32_t* colsum, int64_t M, int64_t K, int64_t N, const float* row_min_a,
                             const float* row_max_a, const float* min_b, const float* max_b, int64_t nb,
-                            const void* bias, const float* addend, void* out, void* stream);
+                            const void* bias, const void* addend, void* out, void* stream);
 
 /* itexhip_qmatmul with the per-tensor activation range in device memory (range_a[0] = min_a, range_a[1] = max_a, e.g.
  * state + 2 of itexhip_quantize_dynamic enqueued earlier on the same stream) in place of p->min_a / p->max_a, which are
@@ -317,14 +318,14 @@ int itexhip_qmatmul_per_row(const itexhip_matmul_params* p, const void* a, const
 int itexhip_qmatmul_device_range(const itexhip_matmul_params* p, const void* a, const int8_t* packed_b,
                                  const int32_t* colsum, int64_t M, int64_t K, int64_t N, const float* range_a,
                                  const float* min_b, const float* max_b, int64_t nb, const void* bias,
-                                 const float* addend, void* out, void* stream);
+                                 const void* addend, void* out, void* stream);
 
 /* itexhip_qmatmul on the unpacked TF-layout weight ([K, N], or [N, K] with transpose_b), any K, no
  * prepack and no column-sum buffer: one thread per output element.  For the shapes the MFMA kernels
  * do not take (K not a multiple of 16). */
 int itexhip_qmatmul_unpacked(const itexhip_matmul_params* p, const void* a, const int8_t* w, int transpose_b,
                              int64_t M, int64_t K, int64_t N, const float* min_b, const float* max_b,
-                             int64_t nb, const void* bias, const float* addend, void* out, void* stream);
+                             int64_t nb, const void* bias, const void* addend, void* out, void* stream);
 
 /* Same contract on the unpacked TF-layout weight, any shape (no alignment requirements): one
  * thread per output element.  Used for shapes the tile kernels do not cover (K not a multiple of

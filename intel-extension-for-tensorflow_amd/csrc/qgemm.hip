@@ -328,8 +328,9 @@ int check_common(const void* a, int a_type, const void* b, int64_t M, int64_t K,
   for (int k = 0; k < ep->n_eltwise; ++k) n_sum += ep->elt[k].alg == ITEXHIP_ELT_SUM;
   ITEXHIP_REQUIRE(n_sum == (addend != nullptr ? 1 : 0),
                   "%s: one sum post-op goes with an addend (itexhip_qgemm_sum / itexhip_qconv2d_sum / itexhip_qmatmul), none without", who);
-  ITEXHIP_REQUIRE(addend == nullptr || addend_type == ITEXHIP_FLOAT || addend_type == ITEXHIP_QINT8 || addend_type == ITEXHIP_QUINT8,
-                  "%s: the addend must be float, qint8 or quint8", who);
+  ITEXHIP_REQUIRE(addend == nullptr || addend_type == ITEXHIP_FLOAT || is_float16_type(addend_type) ||
+                      addend_type == ITEXHIP_QINT8 || addend_type == ITEXHIP_QUINT8,
+                  "%s: the addend must be float, bfloat16, half, qint8 or quint8", who);
   ITEXHIP_REQUIRE(ep->n_scales == 0 || ep->n_scales == 1 || ep->n_scales == N,
                   "%s: %d scales for %lld channels", who, ep->n_scales, static_cast<long long>(N));
   if (M == 0 || N == 0) return ITEXHIP_OK;
@@ -606,7 +607,7 @@ namespace {
 int qmatmul_impl(const char* who, const itexhip_matmul_params* p, const void* a, const int8_t* packed_b,
                  const int32_t* colsum, int64_t M, int64_t K, int64_t N, const float* row_min_a,
                  const float* row_max_a, const float* min_b, const float* max_b, int64_t nb, const void* bias,
-                 const float* addend, void* out, void* stream, const float* range_a = nullptr) {
+                 const void* addend, void* out, void* stream, const float* range_a = nullptr) {
   itexhip_epilogue ep;
   if (int st = itexhip_qmatmul_epilogue_desc(p, nb, &ep)) return st;
   ITEXHIP_REQUIRE(nb == 1 || nb == N, "%s: %lld weight ranges for %lld channels", who, static_cast<long long>(nb),
@@ -629,14 +630,14 @@ int qmatmul_impl(const char* who, const itexhip_matmul_params* p, const void* a,
   e.row_max_a = row_max_a;
   e.range_a = range_a;
   e.addend = addend;
-  e.addend_type = ITEXHIP_FLOAT;
+  e.addend_type = is_float16_type(p->t_out) ? p->t_out : ITEXHIP_FLOAT;  // the addend has the output's type
   return launch_packed(M <= 16, a, p->t_in, packed_b, M, K, N, e, p->t_out, out, stream, who);
 }
 }  // namespace
 
 extern "C" int itexhip_qmatmul(const itexhip_matmul_params* p, const void* a, const int8_t* packed_b,
                                const int32_t* colsum, int64_t M, int64_t K, int64_t N, const float* min_b,
-                               const float* max_b, int64_t nb, const void* bias, const float* addend, void* out,
+                               const float* max_b, int64_t nb, const void* bias, const void* addend, void* out,
                                void* stream) {
   return qmatmul_impl("itexhip_qmatmul", p, a, packed_b, colsum, M, K, N, nullptr, nullptr, min_b, max_b, nb, bias,
                       addend, out, stream);
@@ -645,7 +646,7 @@ extern "C" int itexhip_qmatmul(const itexhip_matmul_params* p, const void* a, co
 extern "C" int itexhip_qmatmul_device_range(const itexhip_matmul_params* p, const void* a, const int8_t* packed_b,
                                            const int32_t* colsum, int64_t M, int64_t K, int64_t N, const float* range_a,
                                            const float* min_b, const float* max_b, int64_t nb, const void* bias,
-                                           const float* addend, void* out, void* stream) {
+                                           const void* addend, void* out, void* stream) {
   ITEXHIP_REQUIRE(range_a != nullptr, "itexhip_qmatmul_device_range: null activation range");
   ITEXHIP_REQUIRE(p->t_out != ITEXHIP_QINT32, "itexhip_qmatmul_device_range: a qint32 result's range is computed on the "
                                               "host from the activation range; use itexhip_qmatmul");
@@ -656,7 +657,7 @@ extern "C" int itexhip_qmatmul_device_range(const itexhip_matmul_params* p, cons
 extern "C" int itexhip_qmatmul_per_row(const itexhip_matmul_params* p, const void* a, const int8_t* packed_b,
                                        const int32_t* colsum, int64_t M, int64_t K, int64_t N,
                                        const float* row_min_a, const float* row_max_a, const float* min_b,
-                                       const float* max_b, int64_t nb, const void* bias, const float* addend,
+                                       const float* max_b, int64_t nb, const void* bias, const void* addend,
                                        void* out, void* stream) {
   ITEXHIP_REQUIRE(M <= 16, "itexhip_qmatmul_per_row: per-row activation ranges are implemented for M <= 16 (got %lld)",
                   static_cast<long long>(M));
@@ -676,7 +677,7 @@ extern "C" int itexhip_mfma_probe(int workgroups, int iters, const void* operand
 
 extern "C" int itexhip_qmatmul_unpacked(const itexhip_matmul_params* p, const void* a, const int8_t* w, int transpose_b,
                                         int64_t M, int64_t K, int64_t N, const float* min_b, const float* max_b,
-                                        int64_t nb, const void* bias, const float* addend, void* out, void* stream) {
+                                        int64_t nb, const void* bias, const void* addend, void* out, void* stream) {
   const char* who = "itexhip_qmatmul_unpacked";
   itexhip_epilogue ep;
   if (int st = itexhip_qmatmul_epilogue_desc(p, nb, &ep)) return st;
@@ -697,7 +698,7 @@ extern "C" int itexhip_qmatmul_unpacked(const itexhip_matmul_params* p, const vo
   e.max_b = max_b;
   e.prep = make_prep_args(p, ep);
   e.addend = addend;
-  e.addend_type = ITEXHIP_FLOAT;
+  e.addend_type = is_float16_type(p->t_out) ? p->t_out : ITEXHIP_FLOAT;  // the addend has the output's type
   const int a_is_u8 = p->t_in == ITEXHIP_QUINT8;
   const uint8_t* ap = reinterpret_cast<const uint8_t*>(a);
   const unsigned grid = static_cast<unsigned>((M * N + 255) / 256);

@@ -44,7 +44,8 @@ struct EpilogueArgs {
   int n_eltwise;
   itexhip_eltwise elt[3];
   const void* addend;    // [M, N] tensor of the "Add" / "Sum" fusion (ITEXHIP_ELT_SUM in the chain), else null
-  int addend_type;       // ITEXHIP_FLOAT, or ITEXHIP_QINT8 / ITEXHIP_QUINT8 (the summand of a quantized convolution)
+  int addend_type;       // ITEXHIP_FLOAT / BFLOAT16 / HALF (the MatMul's "Add": the output's type), or ITEXHIP_QINT8 /
+                         // ITEXHIP_QUINT8 (the summand of a quantized convolution)
   // fused != 0: the kernel derives scale and bias of a channel itself from the op's ranges
   int fused;
   int nb;  // weight ranges (1 or N)
@@ -65,6 +66,8 @@ struct EpilogueArgs {
 __device__ __forceinline__ float load_addend(const EpilogueArgs& e, int64_t i) {
   if (e.addend_type == ITEXHIP_QINT8) return static_cast<float>(static_cast<const int8_t*>(e.addend)[i]);
   if (e.addend_type == ITEXHIP_QUINT8) return static_cast<float>(static_cast<const uint8_t*>(e.addend)[i]);
+  if (e.addend_type == ITEXHIP_BFLOAT16) return bf16_bits_to_f32(static_cast<const uint16_t*>(e.addend)[i]);
+  if (e.addend_type == ITEXHIP_HALF) return f16_bits_to_f32(static_cast<const uint16_t*>(e.addend)[i]);
   return static_cast<const float*>(e.addend)[i];
 }
 

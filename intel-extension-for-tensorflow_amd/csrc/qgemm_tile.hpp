@@ -337,7 +337,8 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void qgemm_tile_kernel(
     // with a switch per value made the epilogue several times longer than the whole K loop (instruction fetch, not
     // arithmetic).  Same expressions as apply_eltwise.
     // the addend of the 16 values of a tile: row m, channels n0 + 8 g + r (g, r < 4); 4 consecutive channels are
-    // one 16-byte (fp32) or 4-byte (8-bit types) load, aligned because N is a multiple of 4 and the host checked the base
+    // one 16-byte (fp32), 8-byte (16-bit types) or 4-byte (8-bit types) load, aligned because N is a multiple of 4 and
+    // the host checked the base
     auto add_sum = [&](float (&v)[16], int m, int n0) {
       const CanonChain& c = e.canon;
       if (m >= M) return;
@@ -350,6 +351,11 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void qgemm_tile_kernel(
           if (e.addend_type == ITEXHIP_FLOAT) {
             const f4 t = *reinterpret_cast<const f4*>(static_cast<const float*>(e.addend) + o);
             a[0] = t[0]; a[1] = t[1]; a[2] = t[2]; a[3] = t[3];
+          } else if (is_float16_type(e.addend_type)) {
+            const uint2 t = *reinterpret_cast<const uint2*>(static_cast<const uint16_t*>(e.addend) + o);
+            const uint32_t h[4] = {t.x & 0xffffu, t.x >> 16, t.y & 0xffffu, t.y >> 16};
+#pragma unroll
+            for (int r = 0; r < 4; ++r) a[r] = e.addend_type == ITEXHIP_BFLOAT16 ? bf16_bits_to_f32(h[r]) : f16_bits_to_f32(h[r]);
           } else {
             const uint32_t w = *reinterpret_cast<const uint32_t*>(static_cast<const uint8_t*>(e.addend) + o);
             if (e.addend_type == ITEXHIP_QUINT8) {
@@ -591,7 +597,8 @@ int dispatch_tile(const uint8_t* a, uint32_t a_xor, const uint8_t* bp, int M, in
   const int act = canon_chain(e, &e.canon);
   const bool has_sum = (e.canon.flags & (kChainSumFirst | kChainSumLast)) != 0;
   const bool sum_ok = !has_sum || (e.addend != nullptr && (N & 3) == 0 &&
-                                   (reinterpret_cast<uintptr_t>(e.addend) & (e.addend_type == ITEXHIP_FLOAT ? 15 : 3)) == 0);
+                                   (reinterpret_cast<uintptr_t>(e.addend) &
+                                    (e.addend_type == ITEXHIP_FLOAT ? 15 : is_float16_type(e.addend_type) ? 7 : 3)) == 0);
   const bool vec_epilogue = act >= 0 && sum_ok && (e.bias != nullptr || e.fused) &&
                             (reinterpret_cast<uintptr_t>(out) & 15) == 0 && ((static_cast<int64_t>(N) * esz) & 15) == 0;
   const bool wide = pick_tile_shape(M, N, true) == 3;

@@ -55,7 +55,9 @@ int validate(const itexhip_matmul_params* p, int64_t nb) {
   ITEXHIP_REQUIRE(p->t_bias == 0 || p->t_bias == ITEXHIP_FLOAT || p->t_bias == ITEXHIP_QINT32 || is_float16_type(p->t_bias),
                   "qmatmul: Tbias must be float, bfloat16, half or qint32");
   ITEXHIP_REQUIRE(p->add_position >= 0 && p->add_position <= 2, "qmatmul: bad add_position");
-  if (p->add_position != 0 && p->t_out != ITEXHIP_FLOAT) {  // (a bfloat16 / half addend is not implemented here)
+  // the addend has the output's type (the sum post-op reads the destination, quantized_matmul_common.h:341-389): float,
+  // bfloat16 or half; a quantized one is refused upstream as well
+  if (p->add_position != 0 && !is_float_out(p->t_out)) {
     set_error("Quantized addend tensor is not implemented yet.");
     return ITEXHIP_UNIMPLEMENTED;
   }

@@ -104,7 +104,8 @@ class QuantizedMatMulOp : public OpKernel {
         if (f == "Requantize") { p_.has_requantize = 1; continue; }
         if (f == "Dequantize") { p_.has_dequantize = 1; continue; }
         if (f == "Add") {
-          ITEX_REQUIRES(ctx, v.t_out == TF_FLOAT, TF_UNIMPLEMENTED, "Quantized addend tensor is not implemented yet.");
+          ITEX_REQUIRES(ctx, v.t_out == TF_FLOAT || v.t_out == TF_BFLOAT16 || v.t_out == TF_HALF, TF_UNIMPLEMENTED,
+                        "Quantized addend tensor is not implemented yet.");
           p_.add_position = p_.activation == ITEXHIP_ACT_NONE ? 1 : 2;
           continue;
         }
@@ -135,10 +136,13 @@ class QuantizedMatMulOp : public OpKernel {
       p_.t_bias = tb;
     }
     if (p_.add_position != 0) {
-      ITEX_REQUIRES(ctx, v.t_out == TF_FLOAT, TF_UNIMPLEMENTED, "Quantized addend tensor is not implemented yet.");
-      // the V1 ops pass bias and addend in one `args` list of type Targs; the addend is taken as fp32
-      ITEX_REQUIRES(ctx, v.api != Api::V1 || p_.t_bias == 0 || p_.t_bias == ITEXHIP_FLOAT, TF_UNIMPLEMENTED,
-                    "the Add fusion of _QuantizedFusedMatMul takes float args on this device");
+      ITEX_REQUIRES(ctx, v.t_out == TF_FLOAT || v.t_out == TF_BFLOAT16 || v.t_out == TF_HALF, TF_UNIMPLEMENTED,
+                    "Quantized addend tensor is not implemented yet.");
+      // the V1 ops pass bias and addend in one `args` list of type Targs, and the addend has the output's type
+      // (:341-389): Targs must be that type
+      const TF_DataType targs = p_.t_bias == 0 ? TF_FLOAT : static_cast<TF_DataType>(p_.t_bias);
+      ITEX_REQUIRES(ctx, v.api != Api::V1 || targs == v.t_out, TF_INVALID_ARGUMENT,
+                    "the Add fusion of _QuantizedFusedMatMul needs args of the output's type");
     }
   }
 
@@ -221,17 +225,17 @@ class QuantizedMatMulOp : public OpKernel {
     // ---- product: one launch, the MatMul kernel derives each channel's output scale and compensated
     // bias itself, so a new activation range costs nothing extra.  K a multiple of 16: MFMA kernels on
     // the prepacked weight; other K: the reference-shaped kernel on the unpacked weight.
-    // "Add": the fp32 addend is input 3 (:352-389 adds it in place into the forwarded output buffer; here the
+    // "Add": the addend (of the output's type: float, bfloat16 or half) is input 3 (:352-389 adds it in place into the forwarded output buffer; here the
     // kernel reads it and writes a fresh output, same values)
-    const float* addend = nullptr;
+    const void* addend = nullptr;
     Tensor addend_t;
     if (p_.add_position != 0) {
       addend_t = ctx->input(3);
       if (!ctx->ok()) return;
-      ITEX_REQUIRES(ctx, addend_t.dtype() == TF_FLOAT && addend_t.dims() == 2 && addend_t.dim_size(0) == M &&
+      ITEX_REQUIRES(ctx, addend_t.dtype() == v_.t_out && addend_t.dims() == 2 && addend_t.dim_size(0) == M &&
                              addend_t.dim_size(1) == N,
-                    TF_INVALID_ARGUMENT, "the addend must be a float tensor of the output's shape");
-      addend = addend_t.flat<float>();
+                    TF_INVALID_ARGUMENT, "the addend must be a tensor of the output's type and shape");
+      addend = addend_t.data();
     }
     Tensor out = ctx->allocate_output(0, v_.t_out, {M, N});
     if (!ctx->ok()) return;

@@ -410,8 +410,11 @@ int orc_qmatmul_prepare(const orc_matmul_attrs* at, int64_t N, const int32_t* co
     ep->elt[ep->n_eltwise].alg = ORC_ELT_SUM; ep->elt[ep->n_eltwise].alpha = 1.0f; ep->elt[ep->n_eltwise].beta = 0.0f;
     ep->n_eltwise++;
   }
-  /* a quantized addend is not implemented upstream either (:1768-1773) */
-  if (at->add_position != 0 && at->t_out != ORC_FLOAT) return ORC_UNIMPLEMENTED;
+  /* a quantized addend is not implemented upstream either (:1768-1773).  The addend has the output's type (the sum
+   * post-op reads the destination buffer, :341-389); for a bfloat16 / half result the caller passes its values widened
+   * to float, which is exact, and the sum is formed in fp32 before the result is rounded to the 16-bit type. */
+  if (at->add_position != 0 && at->t_out != ORC_FLOAT && at->t_out != ORC_BFLOAT16 && at->t_out != ORC_HALF)
+    return ORC_UNIMPLEMENTED;
   if (at->activation == ORC_ACT_LEAKYRELU) has_leaky = 1;
   if (at->api == ORC_API_V2 && at->has_requantize && at->out_min_first) {
     /* :1753-1757: "Linear" is appended to fused_ops */

@@ -596,6 +596,36 @@ def test_add_fusion_vs_oracle(hip, dev, M, pos, act):
                            bias, z, -1, 1)
 
 
+def _widen16(bits, T):
+    """uint16 bit patterns of bfloat16 / half values -> float32 (exact)"""
+    if T == orc.BFLOAT16:
+        return (bits.astype(np.uint32) << 16).view(np.float32)
+    return bits.view(np.float16).astype(np.float32)
+
+
+@pytest.mark.parametrize("T16", [orc.BFLOAT16, orc.HALF], ids=["bf16", "f16"])
+@pytest.mark.parametrize("M,N", [(3, 203), (150, 203), (150, 208), (260, 528)])
+@pytest.mark.parametrize("pos,act", [(1, orc.ACT_RELU), (2, orc.ACT_LEAKYRELU)])
+def test_add_fusion_with_16_bit_output(hip, dev, T16, M, N, pos, act):
+    """[BiasAdd, Add / act, Dequantize] with a bfloat16 / half result: the addend has the output's type (the sum post-op
+    reads the destination, quantized_matmul_common.h:341-389), is widened exactly, added in fp32, and the result is
+    rounded once.  Bit patterns equal the oracle's (fed the widened addend); small-M, element-wise (N = 203) and
+    vector (N = 208, 528) epilogues."""
+    K = 256
+    layer, w, bias = make_layer(hip, dev, K, N, seed=N)
+    x, xq, mn, mx = make_acts(M, K, seed=M)
+    rng = np.random.default_rng(N + M)
+    zf = (rng.standard_normal((M, N)) * 2).astype(np.float32)
+    zbits = ((zf.view(np.uint32) >> 16).astype(np.uint16) if T16 == orc.BFLOAT16 else zf.astype(np.float16).view(np.uint16))
+    kw = dict(api=orc.API_V2, t_out=T16, input_mode=orc.MIN_FIRST, has_dequantize=True, activation=act,
+              add_position=pos, leakyrelu_alpha=0.3)
+    st, ref = orc.qmatmul(orc.matmul_attrs(t_in=orc.QUINT8, **kw), xq, layer.wq, bias, mn, mx, layer.min_b, layer.max_b,
+                          addend=_widen16(zbits, T16))
+    assert st == orc.OK and ref.dtype == np.uint16
+    got = _run_single_launch(hip, dev, layer, kw, xq, mn, mx, bias, zbits.view(np.int16))
+    np.testing.assert_array_equal(bits16(got), ref)
+
+
 @pytest.mark.parametrize("M", [4, 130])
 @pytest.mark.parametrize("act", [orc.ACT_GELU_APPROX, orc.ACT_GELU_EXACT])
 def test_gelu_fusion_close_to_oracle(hip, dev, M, act):

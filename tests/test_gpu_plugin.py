@@ -634,13 +634,51 @@ def test_bfloat16_output_and_bias_through_plugin(rt, dev, op, M, K, N, T16):
         assert st == orc.OK
         np.testing.assert_array_equal(fetch(torch, outs[0], np.int16).view(np.uint16), y_ref)
         node.close()
-    # a bfloat16 / qint32 args list cannot carry the fp32 addend of the Add fusion
+    # the args list of the Add fusion (bias, addend) must have the output's type: the addend is read as the destination
     bad = tf.Node("_QuantizedFusedMatMulAndDequantize",
                   dict(T1=DT(tf.QUINT8), T2=DT(tf.QINT8), Targs=DT(tf.BFLOAT16), Toutput=DT(tf.FLOAT), num_args=2,
                        transpose_a=False, transpose_b=False, fused_ops=["BiasAdd", "Add"], is_filter_const=True,
                        is_bias_const=True, input_quant_mode="MIN_FIRST", leakyrelu_alpha=0.2))
-    assert bad.code == tf.UNIMPLEMENTED
+    assert bad.code == tf.INVALID_ARGUMENT
     bad.close()
+
+
+@pytest.mark.parametrize("api", ["V1", "V2"])
+def test_add_fusion_with_bfloat16_output_through_plugin(rt, dev, api):
+    """[BiasAdd, Add] with a bfloat16 result: the addend is a bfloat16 tensor (it is read as the destination,
+    quantized_matmul_common.h:341-389; V1 passes bias and addend in one bfloat16 args list); bit patterns equal the
+    oracle's, which gets the addend widened to float."""
+    torch = rt
+    M, K, N = 40, 128, 96
+    x, w, bias, xq, xmn, xmx, wq, wmn, wmx = make_problem(M, K, N, seed=21)
+    z = (np.random.default_rng(2).standard_normal((M, N)) * 2).astype(np.float32)
+    zbits = (z.view(np.uint32) >> 16).astype(np.uint16)
+    zwide = (zbits.astype(np.uint32) << 16).view(np.float32)
+    if api == "V1":
+        bbits = (bias.view(np.uint32) >> 16).astype(np.uint16)
+        node = tf.Node("_QuantizedFusedMatMulAndDequantize",
+                       dict(T1=DT(tf.QUINT8), T2=DT(tf.QINT8), Targs=DT(tf.BFLOAT16), Toutput=DT(tf.BFLOAT16), num_args=2,
+                            transpose_a=False, transpose_b=False, fused_ops=["BiasAdd", "Add"], is_filter_const=True,
+                            is_bias_const=True, input_quant_mode="MIN_FIRST", leakyrelu_alpha=0.2))
+        at = orc.matmul_attrs(api=orc.API_V1, t_out=orc.BFLOAT16, add_position=1, n_fused_ops=2, t_bias=orc.BFLOAT16)
+        b_host, b_dt = bbits, tf.BFLOAT16
+    else:
+        node = tf.Node("_QuantizedMatMul", dict(V2, Tout=DT(tf.BFLOAT16), fused_ops=["BiasAdd", "Add", "Dequantize"]))
+        at = orc.matmul_attrs(api=orc.API_V2, t_out=orc.BFLOAT16, has_dequantize=True, add_position=1)
+        b_host, b_dt = bias, tf.FLOAT
+    assert node.code == tf.OK, node.message
+    keep = [dev_in(torch, dev, xq), dev_in(torch, dev, wq), dev_in(torch, dev, b_host.view(np.int16) if b_dt == tf.BFLOAT16 else b_host),
+            dev_in(torch, dev, zbits.view(np.int16))]
+    ins = [(tf.QUINT8, xq.shape, keep[0].data_ptr(), False), (tf.QINT8, wq.shape, keep[1].data_ptr(), False),
+           (b_dt, bias.shape, keep[2].data_ptr(), False), (tf.BFLOAT16, z.shape, keep[3].data_ptr(), False)]
+    for s_ in (xmn, xmx, wmn, wmx):
+        ins.append((tf.FLOAT, s_.shape, tf.host_array(s_), True))
+    code, msg, outs = node.run(ins, [(tf.BFLOAT16, False)], stream=torch.cuda.current_stream().cuda_stream)
+    assert code == tf.OK, msg
+    st, y_ref = orc.qmatmul(at, xq, wq, b_host, xmn, xmx, wmn, wmx, addend=zwide)
+    assert st == orc.OK
+    np.testing.assert_array_equal(fetch(torch, outs[0], np.int16).view(np.uint16), y_ref)
+    node.close()
 
 
 @pytest.mark.parametrize("api", ["V1", "V2"])

@@ -550,3 +550,32 @@ def test_transcendental_post_ops_against_float64(act, f):
     with np.errstate(over="ignore"):                  # e^x overflows to inf in the far tails, as the formulas allow
         want = f(lin.astype(np.float64))
     np.testing.assert_allclose(got, want, rtol=2e-6, atol=1e-6)
+
+
+@pytest.mark.parametrize("T16", [orc.BFLOAT16, orc.HALF])
+def test_add_fusion_with_a_16_bit_result_rounds_the_fp32_sum_once(T16):
+    """The addend of a bfloat16 / half result has that type (quantized_matmul_common.h:341-389); widened to float it
+    enters the same fp32 chain as a float addend, so the 16-bit result is the float result rounded to nearest even."""
+    rng = np.random.default_rng(8)
+    M, K, N = 9, 32, 20
+    xq = rng.integers(0, 256, (M, K)).astype(np.uint8)
+    wq = rng.integers(-127, 128, (K, N)).astype(np.int8)
+    bias = rng.standard_normal(N).astype(np.float32)
+    z = rng.standard_normal((M, N)).astype(np.float32)
+    z = ((z.view(np.uint32) >> 16) << 16).view(np.float32) if T16 == orc.BFLOAT16 else z.astype(np.float16).astype(np.float32)
+    kw = dict(api=orc.API_V2, t_in=orc.QUINT8, input_mode=orc.MIN_FIRST, has_dequantize=True, add_position=2,
+              activation=orc.ACT_RELU)
+    mnb, mxb = np.float32(-0.7), np.float32(0.7)
+    st, y32 = orc.qmatmul(orc.matmul_attrs(t_out=orc.FLOAT, **kw), xq, wq, bias, -1.5, 2.5, mnb, mxb, addend=z)
+    assert st == orc.OK
+    st, y16 = orc.qmatmul(orc.matmul_attrs(t_out=T16, **kw), xq, wq, bias, -1.5, 2.5, mnb, mxb, addend=z)
+    assert st == orc.OK and y16.dtype == np.uint16
+    if T16 == orc.HALF:
+        want = y32.astype(np.float16).view(np.uint16)
+    else:
+        u = y32.view(np.uint32).astype(np.uint64)
+        want = ((u + 0x7fff + ((u >> 16) & 1)) >> 16).astype(np.uint16)
+    np.testing.assert_array_equal(y16, want)
+    st, _ = orc.qmatmul(orc.matmul_attrs(t_out=orc.QINT8, api=orc.API_V2, t_in=orc.QUINT8, has_requantize=True, add_position=1),
+                        xq, wq, bias, -1.5, 2.5, mnb, mxb, -3.0, 3.0, addend=z)
+    assert st == orc.UNIMPLEMENTED
