@@ -533,6 +533,7 @@ def main():
     del ctx
 
     if "prefill" in only:
+        others.append(bench_dynamic_linear(torch, hip, timer, 2048, 4096, 14336, max(10, K_steps // 2), max(3, W // 2), dev, seed=22))
         for (k, n, seed) in ((4096, 4096, 20), (4096, 6144, 21), (14336, 4096, 23)):
             r = bench_linear(torch, hip, timer, 2048, k, n, "requant_s8", K_steps, W, dev, seed)
             r.pop("_ctx")
