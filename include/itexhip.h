@@ -41,7 +41,9 @@ enum {
 };
 
 /* QuantizeMode, numbered like itex/core/utils/quantization_util.h:29-33 */
-enum { ITEXHIP_MIN_COMBINED = 0, ITEXHIP_MIN_FIRST = 1, ITEXHIP_SCALED = 2 };
+enum { ITEXHIP_MIN_COMBINED = 0, ITEXHIP_MIN_FIRST = 1, ITEXHIP_SCALED = 2,
+       /* itexhip_quantize_dynamic{,_rows} only: MIN_FIRST with classic_asymmetric_algorithm (scale and rounded zero point) */
+       ITEXHIP_MIN_FIRST_CLASSIC = 3 };
 
 const char* itexhip_last_error(void);
 /* "gfx950" and the library version; no GPU call. */
@@ -163,7 +165,8 @@ int itexhip_minmax_f32(const float* x, int64_t n, float* minmax_out, void* strea
  * op's parameter math (range adjustment quantize_op.h:130-152; SCALED scale quantization_util.h:54-84; legacy
  * MIN_FIRST scale quantize_op.h:204-214 — per tensor, the same fp32 / fp64 operations as the host code) in a one-thread
  * kernel, and the quantization reading scale and addend from device memory.  mode: ITEXHIP_SCALED (qint8 / quint8) or
- * ITEXHIP_MIN_FIRST (quint8, the non-classic algorithm).  `state` is a device array of 8 floats:
+ * ITEXHIP_MIN_FIRST (quint8, the non-classic algorithm) or ITEXHIP_MIN_FIRST_CLASSIC (the zero-point form,
+ * quantization_util.h:54-84).  `state` is a device array of 8 floats:
  * [0..1] the tensor's min and max, [2..3] the op's output_min / output_max (what a consuming MatMul takes as
  * min_a / max_a: pass state + 2 to itexhip_qmatmul_device_range), [4..5] scale and addend.  n > 0.  The reference
  * (Up to 128 K elements, 16-byte aligned, n a multiple of 4: all three steps in one launch.)  The reference

@@ -420,6 +420,12 @@ __device__ __forceinline__ DynamicParams dynamic_params(float in_min, float in_m
     p.scale = q_high / r;
     p.addend = 0.0f;
     if (dst_type == ITEXHIP_QUINT8) mn = 0.0f;  // output_min of an unsigned SCALED result (:402-408)
+  } else if (mode == ITEXHIP_MIN_FIRST_CLASSIC) {  // scale and zero point, the latter rounded half away from zero
+    const float q_high = dst_type == ITEXHIP_QINT8 ? 127.0f : 255.0f;
+    const float span = mx - mn;
+    p.scale = 255.0f / span;
+    const float scaled_max = mx * p.scale;
+    p.addend = static_cast<float>(static_cast<int>(roundf(q_high - scaled_max)));
   } else {  // the 255 steps are a double, so the division is done in double and rounded once
     p.scale = static_cast<float>(255.0 / static_cast<double>(mx - mn));
     const float shift = -mn;
@@ -615,8 +621,8 @@ extern "C" int itexhip_quantize_dynamic(const float* x, void* q, int64_t n, int 
                                         float ensure_minimum_range, float* state, void* stream) {
   ITEXHIP_REQUIRE(dst_type == ITEXHIP_QINT8 || dst_type == ITEXHIP_QUINT8,
                   "itexhip_quantize_dynamic: dst_type must be qint8 or quint8, got %d", dst_type);
-  ITEXHIP_REQUIRE(mode == ITEXHIP_SCALED || (mode == ITEXHIP_MIN_FIRST && dst_type == ITEXHIP_QUINT8),
-                  "itexhip_quantize_dynamic: SCALED, or MIN_FIRST to quint8");
+  ITEXHIP_REQUIRE(mode == ITEXHIP_SCALED || mode == ITEXHIP_MIN_FIRST_CLASSIC || (mode == ITEXHIP_MIN_FIRST && dst_type == ITEXHIP_QUINT8),
+                  "itexhip_quantize_dynamic: SCALED, MIN_FIRST_CLASSIC, or MIN_FIRST to quint8");
   ITEXHIP_REQUIRE(n > 0, "itexhip_quantize_dynamic: an empty tensor has no range");
   ITEXHIP_REQUIRE(x && q && state && aligned(state, 8), "itexhip_quantize_dynamic: null or unaligned buffer");
   if (n <= kSmallMax && n % 4 == 0 && aligned(x, 16) && aligned(q, 4)) {
@@ -641,8 +647,8 @@ extern "C" int itexhip_quantize_dynamic_rows(const float* x, void* q, int64_t ro
                                              void* stream) {
   ITEXHIP_REQUIRE(dst_type == ITEXHIP_QINT8 || dst_type == ITEXHIP_QUINT8,
                   "itexhip_quantize_dynamic_rows: dst_type must be qint8 or quint8, got %d", dst_type);
-  ITEXHIP_REQUIRE(mode == ITEXHIP_SCALED || (mode == ITEXHIP_MIN_FIRST && dst_type == ITEXHIP_QUINT8),
-                  "itexhip_quantize_dynamic_rows: SCALED, or MIN_FIRST to quint8");
+  ITEXHIP_REQUIRE(mode == ITEXHIP_SCALED || mode == ITEXHIP_MIN_FIRST_CLASSIC || (mode == ITEXHIP_MIN_FIRST && dst_type == ITEXHIP_QUINT8),
+                  "itexhip_quantize_dynamic_rows: SCALED, MIN_FIRST_CLASSIC, or MIN_FIRST to quint8");
   ITEXHIP_REQUIRE(rows >= 0 && rows < (1LL << 31) && cols > 0 && cols < (1LL << 31),
                   "itexhip_quantize_dynamic_rows: bad shape (an empty row has no range)");
   if (rows == 0) return ITEXHIP_OK;

@@ -63,11 +63,11 @@ class QuantizeV2Op : public OpKernel {
     if (dynamic_) {
       ITEX_REQUIRES(ctx, axis_ == -1 && src_type_ == TF_FLOAT, TF_INVALID_ARGUMENT,
                     "the dynamic-range QuantizeV2 quantizes a float tensor per tensor");
-      // SCALED and the legacy MIN_FIRST algorithm: reduction, parameter math and quantization are enqueued back to
-      // back (itexhip_quantize_dynamic) and the host only waits once, at the end, for the two floats of the output
-      // range.  The classic zero-point algorithm takes the path below (range to the host, then QuantizeV2 as usual).
-      const bool device_params = src.NumElements() > 0 && !classic_ &&
-                                 (mode_ == Mode::SCALED || (mode_ == Mode::MIN_FIRST && T_ == TF_QUINT8));
+      // reduction, parameter math and quantization are enqueued back to back (itexhip_quantize_dynamic) and the host
+      // only waits once, at the end, for the two floats of the output range.  (The legacy MIN_FIRST algorithm to
+      // qint8 takes the path below: range to the host, then QuantizeV2 as usual.)
+      const bool device_params = src.NumElements() > 0 &&
+                                 (mode_ == Mode::SCALED || (mode_ == Mode::MIN_FIRST && (classic_ || T_ == TF_QUINT8)));
       if (device_params) {
         Tensor dst = ctx->allocate_output(0, T_, src.shape());
         Tensor out_min = ctx->allocate_output(1, TF_FLOAT, {});
@@ -76,7 +76,8 @@ class QuantizeV2Op : public OpKernel {
         if (!ctx->ok()) return;
         float range[2] = {0.0f, 0.0f};
         int st = itexhip_quantize_dynamic(src.flat<float>(), dst.data(), src.NumElements(), T_,
-                                          mode_ == Mode::SCALED ? ITEXHIP_SCALED : ITEXHIP_MIN_FIRST, ensure_minimum_range_,
+                                          mode_ == Mode::SCALED ? ITEXHIP_SCALED : classic_ ? ITEXHIP_MIN_FIRST_CLASSIC : ITEXHIP_MIN_FIRST,
+                                          ensure_minimum_range_,
                                           state.flat<float>(), ctx->stream());
         if (st == ITEXHIP_OK) st = itexhip_memcpy_d2h(range, state.flat<float>() + 2, sizeof(range), ctx->stream());
         ITEX_REQUIRES(ctx, st == ITEXHIP_OK, TF_ABORTED, std::string("Operation received an exception: ") + itexhip_last_error());

@@ -360,8 +360,10 @@ def test_dynamic_quantize_range_floor_and_constant_tensors(hip, dev):
     import torch
     for fill, emr in ((0.0, 0.01), (3.0, 0.01), (-2.0, 0.01), (1e-6, 0.5), (0.0, 0.0 + 1e-3)):
         x = np.full(37, fill, np.float32)
-        for T, mode in ((orc.QUINT8, orc.MIN_FIRST), (orc.QINT8, orc.SCALED)):
-            _, q_ref, omn, omx = orc.quantize_v2(x, x.min(), x.max(), T, mode, ensure_minimum_range=emr)
+        for T, mode, classic in ((orc.QUINT8, orc.MIN_FIRST, False), (orc.QINT8, orc.SCALED, False),
+                                 (orc.QUINT8, orc.MIN_FIRST, True), (orc.QINT8, orc.MIN_FIRST, True)):
+            _, q_ref, omn, omx = orc.quantize_v2(x, x.min(), x.max(), T, mode, ensure_minimum_range=emr, classic=classic)
+            mode = 3 if classic else mode     # ITEXHIP_MIN_FIRST_CLASSIC
             x_d = torch.from_numpy(x).to(dev)
             q_d = torch.empty(37, dtype=tdt(T), device=dev)
             state = torch.zeros(8, dtype=torch.float32, device=dev)
