@@ -260,6 +260,18 @@ def test_dynamic_quantize_matmul_scaled_and_switch(opt, monkeypatch):
     assert out["q"].op == "_ITEXQuantizeV2DynamicRange" and out["mm"].op == "_ITEXQuantizedMatMul"
 
 
+@pytest.mark.parametrize("make", ["qdq", "dynamic_range", "dynamic_linear", "dynamic_linear_requantize"])
+def test_the_pass_is_idempotent(opt, make):
+    """Grappler may run a custom optimizer more than once: the second run leaves the first run's output as it is."""
+    g = {"qdq": qdq_graph, "dynamic_range": dynamic_range_graph, "dynamic_linear": dynamic_linear_graph,
+         "dynamic_linear_requantize": lambda: dynamic_linear_graph(fused_ops=("BiasAdd", "Requantize"), with_out_range=True)}[make]()
+    once = run(opt, g)
+    twice = run(opt, once)
+    view = lambda gr: [(n.name, n.op, list(n.input), n.device, {k: v.SerializeToString() for k, v in n.attr.items()})
+                       for n in gr.node]       # attribute maps carry no order
+    assert view(twice) == view(once)
+
+
 def test_reshape_is_only_renamed_for_qint8(opt):
     g = gd.GraphDef()
     gd.node(g, "a", "QuantizedReshape", ["x", "s", "mn", "mx"], DEV, T=("type", QINT8))
