@@ -129,7 +129,7 @@ def make_acts(torch, hip, M, K, seed, dev, outlier_frac=0.0, outlier_mult=1.0):
         idx = torch.randint(0, M * K, (n_out,), device=dev, generator=g)
         x.view(-1)[idx] *= outlier_mult
     xq = torch.empty(M, K, dtype=torch.uint8, device=dev)
-    state = torch.zeros(8, dtype=torch.float32, device=dev)
+    state = torch.zeros(hip.DYNAMIC_STATE_FLOATS, dtype=torch.float32, device=dev)
     hip.quantize_dynamic(x, xq, M * K, hip.QUINT8, hip.MIN_FIRST, 0.01, state, _stream(torch))
     torch.cuda.synchronize()
     amn, amx = [float(v) for v in state[2:4].cpu().numpy()]
@@ -219,7 +219,7 @@ def bench_dynamic_linear(torch, hip, timer, M, K, N, steps, warmup, dev, seed):
     x = torch.randn(M, K, device=dev, generator=g)
     xq = torch.empty(M, K, dtype=torch.uint8, device=dev)
     out = torch.empty(M, N, dtype=torch.float32, device=dev)
-    state = torch.zeros(8, dtype=torch.float32, device=dev)
+    state = torch.zeros(hip.DYNAMIC_STATE_FLOATS, dtype=torch.float32, device=dev)
     st = _stream(torch)
     p = hip.matmul_params(api=hip.API_V2, t_in=hip.QUINT8, t_out=hip.FLOAT, input_mode=hip.MIN_FIRST, has_dequantize=True)
 

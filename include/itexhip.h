@@ -166,12 +166,15 @@ int itexhip_minmax_f32(const float* x, int64_t n, float* minmax_out, void* strea
  * MIN_FIRST scale quantize_op.h:204-214 — per tensor, the same fp32 / fp64 operations as the host code) in a one-thread
  * kernel, and the quantization reading scale and addend from device memory.  mode: ITEXHIP_SCALED (qint8 / quint8) or
  * ITEXHIP_MIN_FIRST (quint8, the non-classic algorithm) or ITEXHIP_MIN_FIRST_CLASSIC (the zero-point form,
- * quantization_util.h:54-84).  `state` is a device array of 8 floats:
+ * quantization_util.h:54-84).  `state` is a device array of ITEXHIP_DYNAMIC_STATE_FLOATS floats (the first 8 carry
+ * results, the rest is room for the partial ranges of the reduction's workgroups):
  * [0..1] the tensor's min and max, [2..3] the op's output_min / output_max (what a consuming MatMul takes as
  * min_a / max_a: pass state + 2 to itexhip_qmatmul_device_range), [4..5] scale and addend.  n > 0.  The reference
- * (Up to 128 K elements, 16-byte aligned, n a multiple of 4: all three steps in one launch.)  The reference
+ * (Up to 128 K elements, 16-byte aligned, n a multiple of 4: all three steps in one launch; larger aligned tensors:
+ * two launches.)  The reference
  * has no such op (its QuantizeV2 takes the range from the host); this is the producer half of the
  * Min/Max -> QuantizeV2 -> MatMul fusion of this plugin's graph pass. */
+#define ITEXHIP_DYNAMIC_STATE_FLOATS 1032
 int itexhip_quantize_dynamic(const float* x, void* q, int64_t n, int dst_type, int mode, float ensure_minimum_range,
                              float* state, void* stream);
 /* The per-row (per-token) form: row m of x [rows, cols] is quantized against its own range (QuantizeV2 with axis = 0 and

@@ -301,6 +301,9 @@ __global__ void finish_minmax_f32_kernel(int* keys) {
   reinterpret_cast<float*>(keys)[1] = mx;
 }
 
+// PARTIALS: workgroup b leaves its own minimum and maximum as floats in keys[2b], keys[2b + 1] (no initialisation and
+// no atomics needed; a consumer reduces the gridDim.x pairs); else the two order-preserving keys are updated atomically.
+template <bool PARTIALS>
 __global__ __launch_bounds__(kThreads) void minmax_f32_kernel(const f4* __restrict__ x, int64_t n4,
                                                               const float* __restrict__ tail, int ntail,
                                                               int* keys) {
@@ -335,8 +338,13 @@ __global__ __launch_bounds__(kThreads) void minmax_f32_kernel(const f4* __restri
   block_minmax_commit(
       mn, mx, [](float p, float q) { return p < q; },
       [&](float lo, float hi) {
-        atomicMin(&keys[0], f2key(lo));
-        atomicMax(&keys[1], f2key(hi));
+        if constexpr (PARTIALS) {
+          reinterpret_cast<float*>(keys)[2 * blockIdx.x] = lo;
+          reinterpret_cast<float*>(keys)[2 * blockIdx.x + 1] = hi;
+        } else {
+          atomicMin(&keys[0], f2key(lo));
+          atomicMax(&keys[1], f2key(hi));
+        }
       });
 }
 
@@ -352,9 +360,9 @@ inline void enqueue_minmax_f32(const float* x, int64_t n, int* keys, hipStream_t
   const int64_t ntail = n - head - n4 * 4;
   const unsigned grid = static_cast<unsigned>(std::min<int64_t>(
       kReduceBlocks, std::max<int64_t>(1, (n4 + kThreads * kReduceUnroll - 1) / (kThreads * kReduceUnroll))));
-  minmax_f32_kernel<<<grid, kThreads, 0, st>>>(reinterpret_cast<const f4*>(x + head), n4, x + head + n4 * 4,
-                                               static_cast<int>(ntail), keys);
-  if (head > 0) minmax_f32_kernel<<<1, kThreads, 0, st>>>(nullptr, 0, x, static_cast<int>(head), keys);
+  minmax_f32_kernel<false><<<grid, kThreads, 0, st>>>(reinterpret_cast<const f4*>(x + head), n4, x + head + n4 * 4,
+                                                      static_cast<int>(ntail), keys);
+  if (head > 0) minmax_f32_kernel<false><<<1, kThreads, 0, st>>>(nullptr, 0, x, static_cast<int>(head), keys);
 }
 
 inline unsigned blocks_for(int64_t n, int64_t per_block) {
@@ -576,6 +584,62 @@ __global__ __launch_bounds__(kRowThreads) void quantize_dynamic_rows_kernel(cons
   }
 }
 
+// Second half of the two-launch form for larger tensors: every workgroup reduces the partial ranges the reduction
+// left behind the state (at most kReduceBlocks pairs), derives the parameters, and quantizes its share; workgroup 0
+// also leaves the state and quantizes the last n % 4 elements.
+template <int T>
+__global__ __launch_bounds__(kThreads) void quantize_dynamic_finish_kernel(const f4* __restrict__ x4, uint32_t* __restrict__ q4,
+                                                                           int64_t n4, const float* __restrict__ xtail,
+                                                                           uint8_t* __restrict__ qtail, int ntail,
+                                                                           float* __restrict__ state, int n_partials, int mode,
+                                                                           float ensure_minimum_range) {
+  __shared__ float params[2];
+  const float* partials = state + 8;
+  float mn = __builtin_inff(), mx = -__builtin_inff();
+  for (int i = threadIdx.x; i < n_partials; i += kThreads) {
+    mn = fminf(mn, partials[2 * i]);
+    mx = fmaxf(mx, partials[2 * i + 1]);
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    mn = fminf(mn, __shfl_xor(mn, o, 64));
+    mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+  }
+  block_minmax_commit(
+      mn, mx, [](float p, float q) { return p < q; },
+      [&](float lo, float hi) {
+        const DynamicParams p = dynamic_params(lo, hi, T, mode, ensure_minimum_range);
+        params[0] = p.scale;
+        params[1] = p.addend;
+        if (blockIdx.x == 0) {
+          state[0] = lo;
+          state[1] = hi;
+          state[2] = p.out_min;
+          state[3] = p.out_max;
+          state[4] = p.scale;
+          state[5] = p.addend;
+        }
+      });
+  __syncthreads();
+  const float scale = params[0], addend = params[1];
+  const int64_t base = static_cast<int64_t>(blockIdx.x) * (kThreads * kUnroll) + threadIdx.x;
+  f4 v[kUnroll];
+#pragma unroll
+  for (int j = 0; j < kUnroll; ++j) {
+    const int64_t i = base + j * kThreads;
+    if (i < n4) v[j] = __builtin_nontemporal_load(&x4[i]);
+  }
+#pragma unroll
+  for (int j = 0; j < kUnroll; ++j) {
+    const int64_t i = base + j * kThreads;
+    if (i < n4) __builtin_nontemporal_store(quantize4<T>(v[j], scale, addend), &q4[i]);
+  }
+  if (blockIdx.x == 0 && static_cast<int>(threadIdx.x) < ntail) {
+    const float t = xtail[threadIdx.x] * scale;
+    qtail[threadIdx.x] = static_cast<uint8_t>(sat_rne<T>(t + addend));
+  }
+}
+
 int launch_quantize(const char* who, const float* x, void* q, int64_t n, int dst_type, float scale, float addend,
                     const float* dev_params, hipStream_t st) {
   int64_t done = 0;
@@ -634,6 +698,26 @@ extern "C" int itexhip_quantize_dynamic(const float* x, void* q, int64_t n, int 
     else
       quantize_dynamic_small_kernel<ITEXHIP_QUINT8><<<grid, kSmallThreads, 0, as_stream(stream)>>>(
           reinterpret_cast<const f4*>(x), reinterpret_cast<uint32_t*>(q), n4, state, mode, ensure_minimum_range);
+    ITEXHIP_CHECK_LAUNCH("itexhip_quantize_dynamic");
+    return ITEXHIP_OK;
+  }
+  if (aligned(x, 16) && aligned(q, 4) && n >= 4) {  // two launches: partial ranges, then parameters + quantization
+    hipStream_t st = as_stream(stream);
+    const int64_t n4 = n / 4;
+    const int ntail = static_cast<int>(n - n4 * 4);
+    const unsigned g1 = static_cast<unsigned>(std::min<int64_t>(
+        kReduceBlocks, std::max<int64_t>(1, (n4 + kThreads * kReduceUnroll - 1) / (kThreads * kReduceUnroll))));
+    minmax_f32_kernel<true><<<g1, kThreads, 0, st>>>(reinterpret_cast<const f4*>(x), n4, x + n4 * 4, ntail,
+                                                     reinterpret_cast<int*>(state + 8));
+    const unsigned g2 = blocks_for(n4, kThreads * kUnroll);
+    if (dst_type == ITEXHIP_QINT8)
+      quantize_dynamic_finish_kernel<ITEXHIP_QINT8><<<g2, kThreads, 0, st>>>(
+          reinterpret_cast<const f4*>(x), reinterpret_cast<uint32_t*>(q), n4, x + n4 * 4,
+          reinterpret_cast<uint8_t*>(q) + n4 * 4, ntail, state, static_cast<int>(g1), mode, ensure_minimum_range);
+    else
+      quantize_dynamic_finish_kernel<ITEXHIP_QUINT8><<<g2, kThreads, 0, st>>>(
+          reinterpret_cast<const f4*>(x), reinterpret_cast<uint32_t*>(q), n4, x + n4 * 4,
+          reinterpret_cast<uint8_t*>(q) + n4 * 4, ntail, state, static_cast<int>(g1), mode, ensure_minimum_range);
     ITEXHIP_CHECK_LAUNCH("itexhip_quantize_dynamic");
     return ITEXHIP_OK;
   }

@@ -13,6 +13,7 @@ LIB_PATH = os.path.join(_HERE, "lib", "libitexhip.so")
 OK, INVALID_ARGUMENT, UNIMPLEMENTED, INTERNAL = 0, 3, 12, 13
 FLOAT, INT32, QINT8, QUINT8, QINT32, BFLOAT16, HALF = 1, 3, 11, 12, 13, 14, 19
 MIN_COMBINED, MIN_FIRST, SCALED, MIN_FIRST_CLASSIC = 0, 1, 2, 3
+DYNAMIC_STATE_FLOATS = 1032   # floats of device memory itexhip_quantize_dynamic needs for its state
 API_V2, API_V1, API_LEGACY = 0, 1, 2
 ACT_NONE, ACT_RELU, ACT_RELU6, ACT_LEAKYRELU, ACT_GELU_APPROX, ACT_GELU_EXACT = 0, 1, 2, 3, 4, 5
 ACT_ELU, ACT_SIGMOID, ACT_TANH, ACT_SWISH, ACT_MISH = 6, 7, 8, 9, 10

@@ -72,7 +72,7 @@ class QuantizeV2Op : public OpKernel {
         Tensor dst = ctx->allocate_output(0, T_, src.shape());
         Tensor out_min = ctx->allocate_output(1, TF_FLOAT, {});
         Tensor out_max = ctx->allocate_output(2, TF_FLOAT, {});
-        Tensor state = ctx->allocate_temp(TF_FLOAT, {8});
+        Tensor state = ctx->allocate_temp(TF_FLOAT, {ITEXHIP_DYNAMIC_STATE_FLOATS});
         if (!ctx->ok()) return;
         float range[2] = {0.0f, 0.0f};
         int st = itexhip_quantize_dynamic(src.flat<float>(), dst.data(), src.NumElements(), T_,

@@ -244,7 +244,7 @@ class QuantizedMatMulOp : public OpKernel {
       // from device memory: nothing waits on the host.  K not a multiple of 16 (no MFMA kernel): the range is
       // fetched once for the reference-shaped kernel.
       Tensor aq = ctx->allocate_temp(v_.t_in, {M, K});
-      Tensor state = ctx->allocate_temp(TF_FLOAT, {8});
+      Tensor state = ctx->allocate_temp(TF_FLOAT, {ITEXHIP_DYNAMIC_STATE_FLOATS});
       if (!ctx->ok()) return;
       st = itexhip_quantize_dynamic(a.flat<float>(), aq.data(), M * K, v_.t_in, p_.input_mode, ensure_minimum_range_,
                                     state.flat<float>(), stream);

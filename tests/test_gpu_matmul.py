@@ -296,7 +296,7 @@ def test_dynamic_quantize_then_device_range_matmul(hip, dev, T, mode, M, K, N):
     _, xq_ref, omn, omx = orc.quantize_v2(x, x.min(), x.max(), T, mode)
     x_d = torch.from_numpy(x).to(dev)
     xq_d = torch.empty((M, K), dtype=tdt(T), device=dev)
-    state = torch.full((8,), float("nan"), dtype=torch.float32, device=dev)
+    state = torch.full((hip.DYNAMIC_STATE_FLOATS,), float("nan"), dtype=torch.float32, device=dev)
     for emr in (0.01,):
         hip.quantize_dynamic(x_d, xq_d, M * K, T, mode, emr, state)
     torch.cuda.synchronize()
@@ -366,12 +366,23 @@ def test_dynamic_quantize_range_floor_and_constant_tensors(hip, dev):
             mode = 3 if classic else mode     # ITEXHIP_MIN_FIRST_CLASSIC
             x_d = torch.from_numpy(x).to(dev)
             q_d = torch.empty(37, dtype=tdt(T), device=dev)
-            state = torch.zeros(8, dtype=torch.float32, device=dev)
+            state = torch.zeros(hip.DYNAMIC_STATE_FLOATS, dtype=torch.float32, device=dev)
             hip.quantize_dynamic(x_d, q_d, 37, T, mode, emr, state)
             torch.cuda.synchronize()
             st = state.cpu().numpy()
             assert st[2] == omn[0] and st[3] == omx[0], (fill, emr, T, st, omn, omx)
             np.testing.assert_array_equal(q_d.cpu().numpy(), q_ref)
+    # a tensor that starts 4 bytes off a 16-byte boundary takes the grid-wide reduction with atomics
+    x = np.random.default_rng(1).standard_normal(70003).astype(np.float32)
+    buf = torch.zeros(70004, dtype=torch.float32, device=dev)
+    buf[1:].copy_(torch.from_numpy(x))
+    q_d = torch.empty(70003, dtype=torch.int8, device=dev)
+    hip.quantize_dynamic(buf[1:], q_d, 70003, orc.QINT8, orc.SCALED, 0.01, state)
+    torch.cuda.synchronize()
+    _, q_ref, omn, omx = orc.quantize_v2(x, x.min(), x.max(), orc.QINT8, orc.SCALED)
+    np.testing.assert_array_equal(q_d.cpu().numpy(), q_ref)
+    assert state[2].item() == omn[0] and state[3].item() == omx[0]
+    x_d, q_d = buf[:37], q_d[:37]
     with pytest.raises(hip.ItexHipError):
         hip.quantize_dynamic(x_d, q_d, 0, orc.QINT8, orc.SCALED, 0.01, state)
     with pytest.raises(hip.ItexHipError):
