@@ -69,121 +69,169 @@ __global__ __launch_bounds__(256) void prepack_b_kernel(const int8_t* __restrict
 }
 
 // ------------------------------------------------------------------------------------------------
-// Small-M kernel (M <= 16, bandwidth bound on the weight).  One workgroup owns a strip of SW output
-// channels (32 = whole chunks, or 16 = one half of each chunk when N alone would not give every CU a
-// workgroup); its wavefronts split K into contiguous runs of chunk pairs.  Per chunk pair (64 k) a
-// wavefront issues one activation load (lane l: row l % 16, 16 bytes at k-piece l / 16, i.e. 64
-// contiguous bytes per row) and SW / 16 weight loads in the operand layout of the 16x16x64 MFMA
-// (lane l: channel l % 16, k-group l / 16; 4 runs of 256 contiguous bytes).  A batch of U pairs is
-// issued at once, activations first: loads return in order, so each MFMA waits only for its own
-// operands while the rest of the batch is still in flight.  The partial 16x16 tiles of the wavefronts
-// meet in LDS (one slot per wavefront, one barrier) and wavefront t finishes tile t.
-// Rows >= M of the activation operand repeat row M - 1; their results are never stored.
+// Small-M kernel (M <= 16, bandwidth bound on the weight).  One workgroup owns a strip of 16 * NT output
+// channels (NT = 2: whole chunks; NT = 1: one half of each chunk, when N alone would not give every CU a
+// workgroup); its wavefronts split K into contiguous runs of chunk pairs (64 k each).  Per chunk pair a
+// wavefront needs NT weight fragments in the operand layout of the 16x16x64 MFMA (lane l: channel l % 16,
+// k-group l / 16; 4 runs of 256 contiguous bytes of the packed weight, loaded to registers) and one
+// activation fragment (lane l: row l % 16, the 16 bytes of k-group l / 16).  Loading that fragment straight
+// from the row-major activations would put 64 lanes on 64 different 16-byte pieces of 16 rows, which the
+// texture addresser serves at a quarter of its rate; instead the 16 rows x 64 bytes travel by a direct
+// global -> LDS load whose lanes are contiguous in groups of four (lane 4 q + j: row q, piece
+// j ^ ((q >> 1) & 3)) into a 1 KiB slot of a ring private to the wavefront, and the fragment is read back
+// from LDS (the rotation of the pieces makes that read conflict free).  The loads of a batch of U pairs
+// are issued while the previous batch is multiplied, so 2 U (NT + 1) KiB per wavefront are in flight.
+// The partial 16x16 tiles of the wavefronts meet in LDS (the rings, free by then; one barrier) and
+// wavefront t finishes tile t.  One more wavefront per workgroup streams nothing: it resolves the strip's
+// channel parameters (a chain of dependent kernel-argument and vector loads, then divisions) while the others
+// stream, so that no streaming wavefront starts its loads late or stops for arithmetic.  Rows >= M of the
+// activation operand repeat row M - 1; their results are never stored.  Pairs past the end of a wavefront's
+// run are loaded from clamped addresses and not used.
 // ------------------------------------------------------------------------------------------------
-template <int SW, int OUT_T>
-__global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(4, 4))) void qgemv_kernel(const uint8_t* __restrict__ a, uint32_t a_xor,
+constexpr int kGemvBatch = 4;                 // chunk pairs per batch
+constexpr int kGemvRing = 2 * kGemvBatch;     // activation slots of 1 KiB per wavefront
+
+template <int NT, int OUT_T>
+__global__ __launch_bounds__(576) void qgemv_kernel(const uint8_t* __restrict__ a, uint32_t a_xor,
                                                      const uint8_t* __restrict__ bp, int M, int K, int N,
                                                      int KC, int cnt, EpilogueArgs e,
                                                      void* __restrict__ out) {
-  constexpr int U = 8;         // chunk pairs per batch
-  constexpr int NT = SW / 16;  // 16-channel tiles per strip
-  extern __shared__ int red[];  // [waves][NT][4][64], then the parameter panel [3 or 6][SW]
+  constexpr int SW = 16 * NT;
+  constexpr int U = kGemvBatch, RING = kGemvRing;
+  constexpr int L = U * (NT + 1);  // loads per batch
+  extern __shared__ __align__(16) uint8_t smem[];  // [waves][RING][1 KiB], then the parameter panel [3 or 6][SW]
   const int strip = blockIdx.x;
-  const int waves = blockDim.x >> 6;
+  const int waves = (blockDim.x >> 6) - 1;  // streaming wavefronts; one more resolves the channel parameters
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
-  const int lrow = lane & 15, lgrp = lane >> 4;  // k-group 0..3 of the chunk pair
+  const int lrow = lane & 15, lgrp = lane >> 4;  // fragment lane: row / channel, k-group 0..3 of the chunk pair
   const int KP = KC >> 1;                         // chunk pairs (K is padded to a multiple of 64)
   const int p0 = wave * cnt, p1 = min(KP, p0 + cnt);
   // inside chunk (pair * 2 + lgrp / 2): slot (lgrp % 2) * 32 + half * 16 + lrow
-  const int chunk_row = (SW == 32) ? strip : (strip >> 1);
-  const int half0 = (SW == 32) ? 0 : (strip & 1);
+  const int chunk_row = (NT == 2) ? strip : (strip >> 1);
+  const int half0 = (NT == 2) ? 0 : (strip & 1);
   const uint8_t* wsrc = bp + (static_cast<int64_t>(chunk_row) * KC + (lgrp >> 1)) * kChunkBytes +
                         (((lgrp & 1) * 32 + half0 * 16 + lrow) << 4);
-  const uint8_t* arow = a + static_cast<int64_t>(min(lrow, M - 1)) * K;
-  const int kpiece = lgrp * 16, klast = K - 16;  // k beyond K meets zero weights: any in-bounds data will do
+  // activation staging: lane -> (row q, piece j) of the 16 x 64 byte tile
+  const int q = lane >> 2;
+  const int dpiece = ((lane & 3) ^ ((q >> 1) & 3)) * 16;
+  const uint8_t* arow = a + static_cast<int64_t>(min(q, M - 1)) * K;
+  const int klast = K - 16;  // k beyond K meets zero weights: any in-bounds data will do
+  uint8_t* const ring = smem + wave * (RING * 1024);
+  const uint32_t frag_off = static_cast<uint32_t>((4 * lrow + (lgrp ^ ((lrow >> 1) & 3))) * 16);
 
   v4i acc[NT];
 #pragma unroll
   for (int t = 0; t < NT; ++t) acc[t] = v4i{0, 0, 0, 0};
 
-  // The last wavefront also resolves the strip's channel parameters, one channel per lane: the loads
-  // go out now, the arithmetic waits until its share of the weight stream is done.
-  int* const panel = red + waves * NT * 256;
-  const bool param_lane = (wave == waves - 1) && lane < SW;
-  RawChannel raw{};
-  if (param_lane) raw = load_raw_channel(e, min(strip * SW + lane, N - 1), N);
+  int* const panel = reinterpret_cast<int*>(smem + waves * (RING * 1024));
 
-  auto load_act = [&](int p) { return *reinterpret_cast<const v4i*>(arow + min(p * 64 + kpiece, klast)); };
-  auto load_act_inside = [&](int p) { return *reinterpret_cast<const v4i*>(arow + (p * 64 + kpiece)); };
-  auto load_w = [&](int p, int t) {
-    return __builtin_nontemporal_load(
-        reinterpret_cast<const v4i*>(wsrc + static_cast<int64_t>(p) * (2 * kChunkBytes) + t * 256));
-  };
-  auto mac = [&](const v4i w, v4i x, int t) {
-    x.x ^= a_xor; x.y ^= a_xor; x.z ^= a_xor; x.w ^= a_xor;
-    acc[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w, x, acc[t], 0, 0, 0);
-  };
-
-  int p = p0;
+  // Batches that lie entirely inside the wavefront's run and inside K take their addresses from two running per-lane
+  // pointers plus constants; the last, ragged batch clamps every pair (a pair past the end is loaded from a valid
+  // address and not used).
+  const uint8_t* wptr = wsrc + static_cast<int64_t>(p0) * (2 * kChunkBytes);
+  const uint8_t* aptr = arow + dpiece + static_cast<int64_t>(p0) * 64;
   const int p_full = min(p1, K >> 6);  // pairs below this index lie entirely inside K
-  for (; p + U <= p_full; p += U) {  // full batches: straight-line code
-    v4i x[U], w[U][NT];
+  auto issue = [&](int pb, int slot0, v4i (&w)[U][NT]) {
+    if (pb + U <= p_full) {
 #pragma unroll
-    for (int u = 0; u < U; ++u) x[u] = load_act_inside(p + u);
+      for (int u = 0; u < U; ++u)
+        // the builtin, not inline assembly: the compiler's own vmcnt bookkeeping for the weight loads must see these
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(aptr + u * 64),
+                                         (__attribute__((address_space(3))) void*)(ring + (slot0 + u) * 1024), 16, 0, 0);
 #pragma unroll
-    for (int u = 0; u < U; ++u)
+      for (int u = 0; u < U; ++u)
 #pragma unroll
-      for (int t = 0; t < NT; ++t) w[u][t] = load_w(p + u, t);
-    __builtin_amdgcn_sched_barrier(0);  // keep the whole batch of loads ahead of the first MFMA
-#pragma unroll
-    for (int u = 0; u < U; ++u)
-#pragma unroll
-      for (int t = 0; t < NT; ++t) mac(w[u][t], x[u], t);
-  }
-  if (p < p1) {  // last, partial batch: the guards are wavefront uniform
-    v4i x[U], w[U][NT];
-#pragma unroll
-    for (int u = 0; u < U; ++u)
-      if (p + u < p1) x[u] = load_act(p + u);
-#pragma unroll
-    for (int u = 0; u < U; ++u)
-      if (p + u < p1) {
-#pragma unroll
-        for (int t = 0; t < NT; ++t) w[u][t] = load_w(p + u, t);
-      }
-#pragma unroll
-    for (int u = 0; u < U; ++u)
-      if (p + u < p1) {
-#pragma unroll
-        for (int t = 0; t < NT; ++t) mac(w[u][t], x[u], t);
-      }
-  }
-
-  if (param_lane) {
-    if (e.row_min_a) {  // per-row ranges: the epilogue lanes finish the arithmetic for their own row
-      panel[lane] = raw.colsum;
-      panel[SW + lane] = __float_as_int(raw.min_bj);
-      panel[2 * SW + lane] = __float_as_int(raw.max_bj);
-      panel[3 * SW + lane] = __float_as_int(raw.min_b0);
-      panel[4 * SW + lane] = __float_as_int(raw.max_b0);
-      panel[5 * SW + lane] = __float_as_int(raw.bias);
+        for (int t = 0; t < NT; ++t)
+          w[u][t] = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(wptr + u * (2 * kChunkBytes) + t * 256));
     } else {
-      int comp;
-      float scale, bias;
-      finish_channel(e, raw, &comp, &scale, &bias);
-      panel[lane] = comp;
-      panel[SW + lane] = __float_as_int(scale);
-      panel[2 * SW + lane] = __float_as_int(bias);
-    }
-  }
-  // cross-wavefront reduction
 #pragma unroll
-  for (int t = 0; t < NT; ++t)
-    *reinterpret_cast<v4i*>(&red[((wave * NT + t) * 64 + lane) * 4]) = acc[t];
+      for (int u = 0; u < U; ++u) {
+        const int p = min(pb + u, KP - 1);
+        __builtin_amdgcn_global_load_lds(
+            (const __attribute__((address_space(1))) void*)(arow + min(p * 64 + dpiece, klast)),
+            (__attribute__((address_space(3))) void*)(ring + (slot0 + u) * 1024), 16, 0, 0);
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int p = min(pb + u, KP - 1);
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+          w[u][t] = __builtin_nontemporal_load(
+              reinterpret_cast<const v4i*>(wsrc + static_cast<int64_t>(p) * (2 * kChunkBytes) + t * 256));
+      }
+    }
+    wptr += U * (2 * kChunkBytes);
+    aptr += U * 64;
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  auto compute = [&](int pb, int slot0, const v4i (&w)[U][NT]) {
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      if (pb + u < p1) {  // wavefront uniform
+        v4i x = *reinterpret_cast<const v4i*>(ring + (slot0 + u) * 1024 + frag_off);
+        x.x ^= a_xor; x.y ^= a_xor; x.z ^= a_xor; x.w ^= a_xor;
+#pragma unroll
+        for (int t = 0; t < NT; ++t) acc[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w[u][t], x, acc[t], 0, 0, 0);
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  // wait until at most the next batch's loads of this wavefront are outstanding (they complete in order), then let
+  // the LDS reads of the staged activations go ahead
+  auto landed = [&](bool next_in_flight) {
+    if (next_in_flight) wait_vmcnt<L>(); else wait_vmcnt<0>();
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+  };
+
+  if (wave == waves) {
+    // The extra wavefront resolves the strip's channel parameters, one channel per lane, while the others stream:
+    // fetching pointers and flags from the kernel arguments (a chain of dependent scalar loads), the parameter loads
+    // and the arithmetic (divisions) all stay off the streaming wavefronts' instruction streams.
+    if (lane < SW) {
+      const RawChannel raw = load_raw_channel(e, min(strip * SW + lane, N - 1), N);
+      if (e.row_min_a) {  // per-row ranges: the epilogue lanes finish the arithmetic for their own row
+        panel[lane] = raw.colsum;
+        panel[SW + lane] = __float_as_int(raw.min_bj);
+        panel[2 * SW + lane] = __float_as_int(raw.max_bj);
+        panel[3 * SW + lane] = __float_as_int(raw.min_b0);
+        panel[4 * SW + lane] = __float_as_int(raw.max_b0);
+        panel[5 * SW + lane] = __float_as_int(bias_from_bits(e.prep, raw.bias));
+      } else {
+        int comp;
+        float scale, bias;
+        finish_channel(e, raw, &comp, &scale, &bias);
+        panel[lane] = comp;
+        panel[SW + lane] = __float_as_int(scale);
+        panel[2 * SW + lane] = __float_as_int(bias);
+      }
+    }
+  } else {
+    v4i w0[U][NT], w1[U][NT];
+    int pb = p0;
+    if (pb < p1) issue(pb, 0, w0);
+    while (pb < p1) {
+      const bool more1 = pb + U < p1;
+      if (more1) issue(pb + U, U, w1);
+      landed(more1);
+      compute(pb, 0, w0);
+      pb += U;
+      if (!more1) break;
+      const bool more2 = pb + U < p1;
+      if (more2) issue(pb + U, 0, w0);
+      landed(more2);
+      compute(pb, U, w1);
+      pb += U;
+    }
+    // partial tiles -> the wavefront's own ring (its loads have landed and its reads are done)
+#pragma unroll
+    for (int t = 0; t < NT; ++t) *reinterpret_cast<v4i*>(ring + t * 1024 + lane * 16) = acc[t];
+  }
+  // cross-wavefront reduction through the rings
   __syncthreads();
   if (wave < NT) {
     v4i part = v4i{0, 0, 0, 0};
-    for (int w = 0; w < waves; ++w) part += *reinterpret_cast<const v4i*>(&red[((w * NT + wave) * 64 + lane) * 4]);
+    for (int w = 0; w < waves; ++w) part += *reinterpret_cast<const v4i*>(smem + w * (RING * 1024) + wave * 1024 + lane * 16);
     // accumulator layout of the 16x16 MFMA: lane l, register r -> m = l % 16, n = (l / 16) * 4 + r
     const bool vec_ok = (N & 3) == 0 && aligned16(out);
     const int col = wave * 16 + lgrp * 4, n = strip * SW + col;
@@ -357,27 +405,40 @@ EpilogueArgs make_args(int a_type, const int32_t* colsum, const float* scales, c
   return e;
 }
 
+template <int NT, int OUT_T>
+int launch_gemv(const uint8_t* a, uint32_t a_xor, const uint8_t* bp, int M, int K, int N, int KC, int waves, int cnt,
+                const EpilogueArgs& e, void* out, hipStream_t st) {
+  auto kern = qgemv_kernel<NT, OUT_T>;
+  constexpr size_t lds_max = 8 * kGemvRing * 1024 + 6 * 16 * NT * 4;
+  static bool attr_set = false;  // benign race: the call is idempotent
+  if (!attr_set) {
+    hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                         static_cast<int>(lds_max));
+    if (err != hipSuccess) return hip_fail(err, "hipFuncSetAttribute(qgemv_kernel)");
+    attr_set = true;
+  }
+  const size_t lds = static_cast<size_t>(waves) * kGemvRing * 1024 + 6 * 16 * NT * 4;
+  const int strips = (N + 16 * NT - 1) / (16 * NT);
+  kern<<<strips, 64 * (waves + 1), lds, st>>>(a, a_xor, bp, M, K, N, KC, cnt, e, out);
+  return ITEXHIP_OK;
+}
+
 template <int OUT_T>
 int dispatch_gemv(const uint8_t* a, uint32_t a_xor, const uint8_t* bp, int M, int K, int N,
                   const EpilogueArgs& e, void* out, hipStream_t st) {
   const int KC = 2 * ((K + 63) / 64), KP = KC / 2;
-  // wavefronts per strip: about one batch of 8 chunk pairs each, at most 16; prefer a count that
-  // divides K into whole batches
-  int waves = std::min(16, (KP + 7) / 8);
-  for (int w = waves; w >= std::max(1, waves / 2); --w)
-    if (KP % (8 * w) == 0) { waves = w; break; }
-  const int strips32 = (N + 31) / 32;
-  // a 32-channel strip is finished by two wavefronts, one per 16-channel tile: never fewer than that
-  if (strips32 >= 256) waves = std::max(waves, 2);
+  // 32-channel strips when they alone give every CU a workgroup, else 16-channel strips; a strip is finished by one
+  // wavefront per 16-channel tile, so never fewer wavefronts than that.  Wavefronts per strip: about 16 chunk pairs
+  // (four batches) each, at most 8 (measured on 4096 x 14336 and 14336 x 4096: more, smaller wavefronts start their
+  // streams later and reduce more partial tiles than they gain in loads in flight); prefer a count that divides K
+  // into whole batches.
+  const int nt = (N + 31) / 32 >= 256 ? 2 : 1;
+  int waves = std::max(nt, std::min(8, (KP + 15) / 16));
+  for (int w = waves; w >= std::max(nt, waves / 2 + 1); --w)
+    if (KP % (kGemvBatch * w) == 0) { waves = w; break; }
   const int cnt = (KP + waves - 1) / waves;
-  if (strips32 >= 256) {
-    const size_t lds = static_cast<size_t>(waves) * 2 * 1024 + 6 * 32 * 4;
-    qgemv_kernel<32, OUT_T><<<strips32, 64 * waves, lds, st>>>(a, a_xor, bp, M, K, N, KC, cnt, e, out);
-  } else {
-    const size_t lds = static_cast<size_t>(waves) * 1024 + 6 * 16 * 4;
-    qgemv_kernel<16, OUT_T><<<(N + 15) / 16, 64 * waves, lds, st>>>(a, a_xor, bp, M, K, N, KC, cnt, e, out);
-  }
-  return ITEXHIP_OK;
+  if (nt == 2) return launch_gemv<2, OUT_T>(a, a_xor, bp, M, K, N, KC, waves, cnt, e, out, st);
+  return launch_gemv<1, OUT_T>(a, a_xor, bp, M, K, N, KC, waves, cnt, e, out, st);
 }
 
 #define ITEXHIP_DISPATCH_OUT(out_type, CALL)                                  \

@@ -112,24 +112,35 @@ inline int canon_chain(const EpilogueArgs& e, CanonChain* c) {
 
 // Scale, bias and zero-point compensation of channel n (n < N), however the call supplied them, in two
 // stages so that a kernel can issue the loads early and do the arithmetic late.
+__device__ __forceinline__ int first_lane_zero() {
+  int z = 0;
+  asm volatile("" : "+v"(z));
+  return z;
+}
+
 struct RawChannel {
   float min_bj, max_bj, min_b0, max_b0;  // fused: weight ranges;  else min_bj holds the prepared scale
-  float bias;
+  uint32_t bias;                         // fused: the raw bias entry as loaded;  else the bits of the prepared fp32 bias
   int colsum;
 };
 
+// Only loads, all of them per-lane vector loads that nothing waits for here: a wavefront can issue them ahead of a
+// long stream of other loads and meet the values at the end.  (A load from a wavefront-uniform address would become a
+// scalar load, whose result the compiler wants at once: the lane-dependent zero keeps the first weight range on the
+// vector path.)
 __device__ __forceinline__ RawChannel load_raw_channel(const EpilogueArgs& e, int n, int N) {
-  RawChannel r{};
+  RawChannel r;  // the fields a path does not use stay undefined: assigning them would wait for the loads in flight
   r.colsum = e.colsum ? e.colsum[n] : 0;
-  r.bias = e.fused ? bias_entry(e.prep, e.bias, n) : (e.bias ? static_cast<const float*>(e.bias)[n] : 0.0f);
+  r.bias = e.fused ? bias_bits(e.prep, e.bias, n) : (e.bias ? static_cast<const uint32_t*>(e.bias)[n] : 0u);
   if (e.fused) {
     const int jb = (e.nb == N) ? n : 0;
+    const int first = first_lane_zero();
     r.min_bj = e.min_b[jb];
     r.max_bj = e.max_b[jb];
-    r.min_b0 = e.min_b[0];
-    r.max_b0 = e.max_b[0];
+    r.min_b0 = e.min_b[first];
+    r.max_b0 = e.max_b[first];
   } else {
-    r.min_bj = e.n_scales > 1 ? e.scales[n] : (e.n_scales == 1 ? e.scales[0] : 1.0f);
+    r.min_bj = e.n_scales > 1 ? e.scales[n] : (e.n_scales == 1 ? e.scales[first_lane_zero()] : 1.0f);
   }
   return r;
 }
@@ -143,12 +154,13 @@ __device__ __forceinline__ void finish_channel(const EpilogueArgs& e, const RawC
       pr.min_a = e.range_a[0];
       pr.max_a = e.range_a[1];
     }
-    const ChannelScaleBias c = channel_scale_bias(pr, r.min_bj, r.max_bj, r.min_b0, r.max_b0, r.bias, r.colsum);
+    const ChannelScaleBias c = channel_scale_bias(pr, r.min_bj, r.max_bj, r.min_b0, r.max_b0, bias_from_bits(e.prep, r.bias),
+                                                  r.colsum);
     *scale = e.n_scales > 0 ? c.scale : 1.0f;
     *bias = c.bias;
   } else {
     *scale = r.min_bj;
-    *bias = r.bias;
+    *bias = __uint_as_float(r.bias);
   }
 }
 
@@ -287,6 +299,24 @@ __device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int
 template <int N, class F>
 __device__ __forceinline__ void static_for(F&& f) {
   static_for_impl(static_cast<F&&>(f), std::make_integer_sequence<int, N>{});
+}
+
+// Direct global -> LDS loads (global_load_lds_dwordx4): each lane's 16 bytes land at LDS base + 16 * lane, no VGPRs
+// and no ds_write on the way.  They count in vmcnt like any other vector memory load and return in order with them.
+__device__ __forceinline__ void lds_dma16(const void* gptr, uint32_t lds_addr) {
+  // m0 = LDS byte address of lane 0's destination; the instruction adds 16 * lane
+  asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(gptr), "s"(lds_addr) : "memory", "m0");
+}
+// same with a wavefront-uniform 64-bit base (SGPR pair) and a 32-bit per-lane byte offset: no vector
+// address arithmetic per load
+__device__ __forceinline__ void lds_dma16(const void* sbase, uint32_t lane_off, uint32_t lds_addr) {
+  asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(lane_off), "s"(sbase), "s"(lds_addr) : "memory", "m0");
+}
+
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+  // s_waitcnt with only vmcnt active (gfx9 encoding: vmcnt[3:0] | expcnt 7 << 4 | lgkmcnt 15 << 8 | vmcnt[5:4] << 14)
+  __builtin_amdgcn_s_waitcnt((N & 15) | (7 << 4) | (15 << 8) | ((N >> 4) << 14));
 }
 
 // Geometry of a Conv2D computed as an implicit GEMM by the tile kernel (32-bit: the host checks the ranges)

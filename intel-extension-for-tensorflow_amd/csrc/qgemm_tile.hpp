@@ -40,22 +40,6 @@ namespace itexhip {
 //   Rows >= M and channel tiles >= NT are loaded from clamped (valid) addresses: whatever they
 //   contribute lands in outputs that are never stored.  Columns k >= K multiply zero-padded weights.
 // ------------------------------------------------------------------------------------------------
-__device__ __forceinline__ void lds_dma16(const void* gptr, uint32_t lds_addr) {
-  // m0 = LDS byte address of lane 0's destination; the instruction adds 16 * lane
-  asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(gptr), "s"(lds_addr) : "memory", "m0");
-}
-// same with a wavefront-uniform 64-bit base (SGPR pair) and a 32-bit per-lane byte offset: no vector
-// address arithmetic per load
-__device__ __forceinline__ void lds_dma16(const void* sbase, uint32_t lane_off, uint32_t lds_addr) {
-  asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(lane_off), "s"(sbase), "s"(lds_addr) : "memory", "m0");
-}
-
-template <int N>
-__device__ __forceinline__ void wait_vmcnt() {
-  // s_waitcnt with only vmcnt active (gfx9 encoding: vmcnt[3:0] | expcnt 7 << 4 | lgkmcnt 15 << 8 | vmcnt[5:4] << 14)
-  __builtin_amdgcn_s_waitcnt((N & 15) | (7 << 4) | (15 << 8) | ((N >> 4) << 14));
-}
-
 // Implicit GEMM of a Conv2D (NHWC input, in_c a multiple of 16): the activation "matrix" is the patch matrix
 // [batch * out_h * out_w, k_h * k_w * in_c], never materialised.  A 16-byte piece of a patch row lies inside one
 // input pixel (or in the padding, then it is read from 16 zero bytes), so only the source address of an activation

@@ -23,13 +23,22 @@ struct PrepArgs {
   float min_a, max_a, min_out, max_out;
 };
 
-// entry j of the op's bias vector as fp32 (the qint32 bias is cast, :1165-1167); 0 without a bias
+// entry j of the op's bias vector: the raw bits first (a load that nothing waits for), the fp32 value later
+// (the qint32 bias is cast, :1165-1167); 0 without a bias
+__device__ __forceinline__ uint32_t bias_bits(const PrepArgs& p, const void* bias, int64_t j) {
+  if (bias == nullptr) return 0u;
+  if (p.bias_s32) return static_cast<uint32_t>(static_cast<const int32_t*>(bias)[j]);
+  if (p.bias_16 != 0) return static_cast<const uint16_t*>(bias)[j];
+  return static_cast<const uint32_t*>(bias)[j];
+}
+__device__ __forceinline__ float bias_from_bits(const PrepArgs& p, uint32_t b) {
+  if (p.bias_s32) return static_cast<float>(static_cast<int32_t>(b));
+  if (p.bias_16 == ITEXHIP_BFLOAT16) return bf16_bits_to_f32(b);
+  if (p.bias_16 == ITEXHIP_HALF) return f16_bits_to_f32(b);
+  return __uint_as_float(b);
+}
 __device__ __forceinline__ float bias_entry(const PrepArgs& p, const void* bias, int64_t j) {
-  if (bias == nullptr) return 0.0f;
-  if (p.bias_s32) return static_cast<float>(static_cast<const int32_t*>(bias)[j]);
-  if (p.bias_16 == ITEXHIP_BFLOAT16) return bf16_bits_to_f32(static_cast<const uint16_t*>(bias)[j]);
-  if (p.bias_16 == ITEXHIP_HALF) return f16_bits_to_f32(static_cast<const uint16_t*>(bias)[j]);
-  return static_cast<const float*>(bias)[j];
+  return bias_from_bits(p, bias_bits(p, bias, j));
 }
 
 struct ChannelScaleBias {
