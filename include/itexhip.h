@@ -184,6 +184,19 @@ int itexhip_quantize_dynamic(const float* x, void* q, int64_t n, int dst_type, i
 int itexhip_quantize_dynamic_rows(const float* x, void* q, int64_t rows, int64_t cols, int dst_type, int mode,
                                   float ensure_minimum_range, float* row_min_out, float* row_max_out, void* stream);
 
+/* itexhip_quantize_dynamic without a workspace argument and without any allocation.  It has no counterpart in the
+ * reference; it is for callers that cannot allocate device memory around the call: code under HIP graph capture,
+ * tight serving loops, harnesses that forbid allocation.  The partial ranges of the reduction (one {min, max} pair per
+ * workgroup of the range pass, at most 512 pairs = 4 KiB whatever n) live in a fixed array of the library's own device
+ * memory, one copy per GPU, kept until the process ends; the call itself allocates and frees nothing.  Always two
+ * launches (partial ranges, then parameters + quantization).  range_out: 6 floats of device memory, filled like
+ * state[0..5] of itexhip_quantize_dynamic ([0..1] the tensor's min and max, [2..3] the op's output_min / output_max,
+ * [4..5] scale and addend).  4 <= n <= 2^36; x 16-byte, q 4-byte, range_out 8-byte aligned; anything else is rejected.
+ * Same bytes in q and the same six floats as itexhip_quantize_dynamic.  Calls that overlap in time on one GPU (two
+ * streams, two threads) share the array and race: serialise them. */
+int itexhip_quantize_dynamic_static(const float* x, void* q, int64_t n, int dst_type, int mode, float ensure_minimum_range,
+                                    float* range_out, void* stream);
+
 /* ------------------------------------------------------------------------------------------
  * Quantized MatMul (oneDNN inner_product_forward u8/s8 x s8 -> s32 with fused epilogue;
  * itex/core/kernels/common/quantized_matmul_common.h:223-226 (primitive), :92 (execute)).

@@ -1,6 +1,9 @@
 // HBM-bound elementwise kernels: QuantizeV2, Dequantize, RequantizePerChannel and the min/max
 // reductions.  One wavefront instruction moves 1 KiB (16 B per lane, lanes contiguous); each thread
 // keeps several such loads in flight before it converts and stores.
+#include <algorithm>
+#include <mutex>
+
 #include "common.hpp"
 
 namespace itexhip {
@@ -591,10 +594,10 @@ template <int T>
 __global__ __launch_bounds__(kThreads) void quantize_dynamic_finish_kernel(const f4* __restrict__ x4, uint32_t* __restrict__ q4,
                                                                            int64_t n4, const float* __restrict__ xtail,
                                                                            uint8_t* __restrict__ qtail, int ntail,
-                                                                           float* __restrict__ state, int n_partials, int mode,
-                                                                           float ensure_minimum_range) {
+                                                                           float* __restrict__ state,
+                                                                           const float* __restrict__ partials, int n_partials,
+                                                                           int mode, float ensure_minimum_range) {
   __shared__ float params[2];
-  const float* partials = state + 8;
   float mn = __builtin_inff(), mx = -__builtin_inff();
   for (int i = threadIdx.x; i < n_partials; i += kThreads) {
     mn = fminf(mn, partials[2 * i]);
@@ -713,11 +716,11 @@ extern "C" int itexhip_quantize_dynamic(const float* x, void* q, int64_t n, int 
     if (dst_type == ITEXHIP_QINT8)
       quantize_dynamic_finish_kernel<ITEXHIP_QINT8><<<g2, kThreads, 0, st>>>(
           reinterpret_cast<const f4*>(x), reinterpret_cast<uint32_t*>(q), n4, x + n4 * 4,
-          reinterpret_cast<uint8_t*>(q) + n4 * 4, ntail, state, static_cast<int>(g1), mode, ensure_minimum_range);
+          reinterpret_cast<uint8_t*>(q) + n4 * 4, ntail, state, state + 8, static_cast<int>(g1), mode, ensure_minimum_range);
     else
       quantize_dynamic_finish_kernel<ITEXHIP_QUINT8><<<g2, kThreads, 0, st>>>(
           reinterpret_cast<const f4*>(x), reinterpret_cast<uint32_t*>(q), n4, x + n4 * 4,
-          reinterpret_cast<uint8_t*>(q) + n4 * 4, ntail, state, static_cast<int>(g1), mode, ensure_minimum_range);
+          reinterpret_cast<uint8_t*>(q) + n4 * 4, ntail, state, state + 8, static_cast<int>(g1), mode, ensure_minimum_range);
     ITEXHIP_CHECK_LAUNCH("itexhip_quantize_dynamic");
     return ITEXHIP_OK;
   }
@@ -944,5 +947,74 @@ extern "C" int itexhip_memcpy_d2d_async(void* dst, const void* src, size_t bytes
     copy_byte_kernel<<<blocks_for(n - done, kThreads), kThreads, 0, st>>>(
         reinterpret_cast<const uint8_t*>(src), reinterpret_cast<uint8_t*>(dst), done, n);
   ITEXHIP_CHECK_LAUNCH("itexhip_memcpy_d2d_async");
+  return ITEXHIP_OK;
+}
+
+// ------------------------------------------------------------------------------------------------
+// itexhip_quantize_dynamic for callers that cannot allocate (HIP graph capture, serving loops): the partial
+// ranges of the reduction's workgroups live in a fixed array of the library's own device memory instead of a
+// workspace argument.  Every GPU holds its own copy of the array at its own address, resolved once per device.
+// ------------------------------------------------------------------------------------------------
+namespace itexhip {
+namespace {
+// one {min, max} pair per workgroup of the range pass, kReduceBlocks of them at most whatever the tensor's size
+static __device__ __align__(256) float scratch[2 * kReduceBlocks];
+
+constexpr int kMaxDevices = 64;
+constexpr int64_t kStaticMaxElements = int64_t{1} << 36;  // 256 GiB of fp32: more than a device holds beside its result
+
+// the device address of `scratch` on the current device (the array's name is only a host-side handle)
+int scratch_address(float** out) {
+  static float* ptrs[kMaxDevices] = {};
+  static std::mutex mu;
+  int dev = 0;
+  hipError_t err = hipGetDevice(&dev);
+  if (err != hipSuccess) return hip_fail(err, "hipGetDevice");
+  ITEXHIP_REQUIRE(dev >= 0 && dev < kMaxDevices, "itexhip_quantize_dynamic_static: device ordinal %d out of range", dev);
+  std::lock_guard<std::mutex> lock(mu);
+  if (ptrs[dev] == nullptr) {
+    void* p = nullptr;
+    err = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (err != hipSuccess) return hip_fail(err, "hipGetSymbolAddress(scratch)");
+    ptrs[dev] = static_cast<float*>(p);
+  }
+  *out = ptrs[dev];
+  return ITEXHIP_OK;
+}
+}  // namespace
+}  // namespace itexhip
+
+extern "C" int itexhip_quantize_dynamic_static(const float* x, void* q, int64_t n, int dst_type, int mode,
+                                               float ensure_minimum_range, float* range_out, void* stream) {
+  const char* who = "itexhip_quantize_dynamic_static";
+  ITEXHIP_REQUIRE(dst_type == ITEXHIP_QINT8 || dst_type == ITEXHIP_QUINT8, "%s: dst_type must be qint8 or quint8, got %d", who, dst_type);
+  ITEXHIP_REQUIRE(mode == ITEXHIP_SCALED || mode == ITEXHIP_MIN_FIRST_CLASSIC || (mode == ITEXHIP_MIN_FIRST && dst_type == ITEXHIP_QUINT8),
+                  "%s: SCALED, MIN_FIRST_CLASSIC, or MIN_FIRST to quint8", who);
+  ITEXHIP_REQUIRE(n >= 4, "%s: at least 4 elements (got %lld)", who, static_cast<long long>(n));
+  ITEXHIP_REQUIRE(n <= kStaticMaxElements, "%s: at most 2^36 elements (got %lld)", who, static_cast<long long>(n));
+  ITEXHIP_REQUIRE(x && q && range_out, "%s: null buffer", who);
+  ITEXHIP_REQUIRE(aligned(x, 16) && aligned(q, 4) && aligned(range_out, 8),
+                  "%s: x must be 16-byte, q 4-byte and range_out 8-byte aligned", who);
+  float* partials = nullptr;
+  if (int st = scratch_address(&partials)) return st;
+  hipStream_t st = as_stream(stream);
+  const int64_t n4 = n / 4;
+  const int ntail = static_cast<int>(n - n4 * 4);
+  // every workgroup of the range pass overwrites its own pair, and the second kernel reads exactly those: nothing
+  // in the array has to be cleared between calls
+  const unsigned g1 = static_cast<unsigned>(std::min<int64_t>(
+      kReduceBlocks, std::max<int64_t>(1, (n4 + kThreads * kReduceUnroll - 1) / (kThreads * kReduceUnroll))));
+  minmax_f32_kernel<true><<<g1, kThreads, 0, st>>>(reinterpret_cast<const f4*>(x), n4, x + n4 * 4, ntail,
+                                                   reinterpret_cast<int*>(partials));
+  const unsigned g2 = blocks_for(n4, kThreads * kUnroll);
+  if (dst_type == ITEXHIP_QINT8)
+    quantize_dynamic_finish_kernel<ITEXHIP_QINT8><<<g2, kThreads, 0, st>>>(
+        reinterpret_cast<const f4*>(x), reinterpret_cast<uint32_t*>(q), n4, x + n4 * 4, reinterpret_cast<uint8_t*>(q) + n4 * 4,
+        ntail, range_out, partials, static_cast<int>(g1), mode, ensure_minimum_range);
+  else
+    quantize_dynamic_finish_kernel<ITEXHIP_QUINT8><<<g2, kThreads, 0, st>>>(
+        reinterpret_cast<const f4*>(x), reinterpret_cast<uint32_t*>(q), n4, x + n4 * 4, reinterpret_cast<uint8_t*>(q) + n4 * 4,
+        ntail, range_out, partials, static_cast<int>(g1), mode, ensure_minimum_range);
+  ITEXHIP_CHECK_LAUNCH(who);
   return ITEXHIP_OK;
 }
