@@ -53,6 +53,12 @@ static __device__ __align__(16) const uint32_t kZeroPiece[4] = {0u, 0u, 0u, 0u};
 // register operand, so the sign flip costs a 4-byte instruction per dword.  KALIGNED: K is a multiple
 // of 64, so activation loads never need a per-lane clamp and use a uniform base that advances by 64
 // bytes per step.
+#ifdef ITEXHIP_TILE_TRACE
+__device__ unsigned long long g_tile_trace[2048 * 8];
+#define TILE_T(i) do { if (threadIdx.x == 0 && blockIdx.x < 2048) g_tile_trace[blockIdx.x * 8 + (i)] = wall_clock64(); } while (0)
+#else
+#define TILE_T(i)
+#endif
 template <int BM, int BN, int WAVES_M, int WAVES_N, int OUT_T, int ACT, bool KALIGNED, bool CONV = false, bool ELEMENTWISE = false>
 __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void qgemm_tile_kernel(
     const uint8_t* __restrict__ a, uint32_t amask, const uint8_t* __restrict__ bp, int M, int K, int N,
@@ -85,6 +91,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void qgemm_tile_kernel(
   // byte offset from the window origin}
   constexpr int CONV_TAB_OFF = PANEL_OFF + 12 * BN;
 
+  TILE_T(0);
   extern __shared__ __align__(16) uint8_t lds[];
   const uint32_t lds_base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(
       (__attribute__((address_space(3))) void*)lds));
@@ -208,6 +215,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void qgemm_tile_kernel(
   }
   wait_vmcnt<NLD>();
   __syncthreads();
+  TILE_T(1);
   // the accumulators start from the zero-point compensation of their channel (exact in int32)
   static_for<TN>([&](auto j) {
     static_for<4>([&](auto g) {
@@ -298,6 +306,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void qgemm_tile_kernel(
   }
   wait_vmcnt<0>();  // no load may still be writing LDS when the epilogue reuses it
   __syncthreads();
+  TILE_T(2);
 
   // ---- epilogue.  Fast path: convert in registers, transpose through a private LDS buffer (the ring
   // is free after the last barrier) and store rows of 128 contiguous bytes, 16 B per lane.  A lane of
@@ -477,7 +486,8 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void qgemm_tile_kernel(
         const int m = m_base + wm * WM + row;
         const bool mine = (64 % LPR == 0 || f_row < RPP) && (WM % RPP == 0 || pass * RPP + f_row < WM);
         if (mine && m < M && n_col < N)  // N * ESZ is a multiple of 16, so a piece is entirely inside or outside
-          *reinterpret_cast<v4i*>(reinterpret_cast<uint8_t*>(out) + (static_cast<int64_t>(m) * N + n_col) * ESZ) = v;
+          // streaming stores: written back as they go, not held dirty in L2 until the flush at the end of the kernel
+          __builtin_nontemporal_store(v, reinterpret_cast<v4i*>(reinterpret_cast<uint8_t*>(out) + (static_cast<int64_t>(m) * N + n_col) * ESZ));
       }
     });
   } else {
@@ -513,6 +523,11 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void qgemm_tile_kernel(
       });
     });
   }
+  TILE_T(3);
+#ifdef ITEXHIP_TILE_TRACE
+  wait_vmcnt<0>();
+  TILE_T(4);
+#endif
 }
 
 template <int BM, int BN, int WAVES_M, int WAVES_N, int OUT_T, int ACT, bool KALIGNED, bool CONV = false, bool ELEMENTWISE = false>

@@ -8,7 +8,7 @@ import ctypes as C
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "lib", "libitexhip.so")
+LIB_PATH = os.environ.get("ITEXHIP_LIB") or os.path.join(_HERE, "lib", "libitexhip.so")  # ITEXHIP_LIB: another build, for A/B timing
 
 OK, INVALID_ARGUMENT, UNIMPLEMENTED, INTERNAL = 0, 3, 12, 13
 FLOAT, INT32, QINT8, QUINT8, QINT32, BFLOAT16, HALF = 1, 3, 11, 12, 13, 14, 19
