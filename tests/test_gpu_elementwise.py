@@ -302,6 +302,96 @@ def test_full_size_quantize_properties(hip, dev):
         del q_d, y_d
 
 
+def _windows(n, size=1 << 20):
+    return (0, n // 2 - 12345, n - size)
+
+
+def test_full_size_scaled_quint8_and_dequantize_vs_oracle(hip, dev):
+    """2^28 elements: QuantizeV2 SCALED -> quint8 (negatives clamp to 0, output range (0, r)) and Dequantize of both
+    8-bit types in both modes against the oracle on three windows of 2^20 elements, plus a whole-tensor int64 checksum
+    of the quantized bytes against torch's evaluation of the same formula."""
+    import torch
+    n = 1 << 28
+    g = torch.Generator(device=dev)
+    g.manual_seed(30)
+    x_d = torch.randn(n, device=dev, generator=g)
+    x_d[::9973] *= 50.0
+    mn, mx = float(x_d.min()), float(x_d.max())
+    sc, add, omn, omx = host_quant_params(orc.QUINT8, orc.SCALED, False, mn, mx)
+    assert omn[0] == 0.0
+    q_d = torch.empty(n, dtype=torch.uint8, device=dev)
+    hip.quantize(x_d, q_d, n, orc.QUINT8, float(sc[0]), float(add[0]))
+    torch.cuda.synchronize()
+    for lo in _windows(n):
+        xs = x_d[lo:lo + (1 << 20)].cpu().numpy()
+        st, q_ref, _, _ = orc.quantize_v2(xs, mn, mx, orc.QUINT8, orc.SCALED)
+        np.testing.assert_array_equal(q_d[lo:lo + (1 << 20)].cpu().numpy(), q_ref)
+    expect_sum = 0
+    for lo in range(0, n, 1 << 26):   # the same fp32 multiply, round-half-even and clamp, by torch
+        part = torch.round(x_d[lo:lo + (1 << 26)] * float(sc[0])).clamp_(0, 255)
+        expect_sum += int(part.sum(dtype=torch.float64).item())
+    assert int(q_d.sum(dtype=torch.int64).item()) == expect_sum
+    del x_d
+    # Dequantize at full size: the quint8 bytes above in both modes, and the same bytes read as qint8
+    y_d = torch.empty(n, dtype=torch.float32, device=dev)
+    for T, mode, rmn, rmx in ((orc.QUINT8, orc.SCALED, 0.0, mx), (orc.QUINT8, orc.MIN_FIRST, mn, mx),
+                              (orc.QINT8, orc.SCALED, mn, mx), (orc.QINT8, orc.MIN_FIRST, mn, mx)):
+        st, _, _, dsc, dzp = orc.scale_zeropoint_align(T, mode, True, rmn, rmx)
+        src = q_d if T == orc.QUINT8 else q_d.view(torch.int8)
+        hip.dequantize(src, y_d, n, T, float(dsc[0]), int(dzp[0]) if mode == orc.MIN_FIRST else 0)
+        torch.cuda.synchronize()
+        for lo in _windows(n):
+            st, y_ref = orc.dequantize(src[lo:lo + (1 << 20)].cpu().numpy(), rmn, rmx, T, mode)
+            np.testing.assert_array_equal(y_d[lo:lo + (1 << 20)].cpu().numpy(), y_ref)
+        # whole tensor: y is an exact function of the byte, so the histogram of q fixes the sum of y in float64
+        table = orc.dequantize(np.arange(256, dtype=np.uint8).view(orc.NP_OF[T]), rmn, rmx, T, mode)[1].astype(np.float64)
+        counts = torch.bincount(q_d.to(torch.int32), minlength=256).cpu().numpy()
+        assert abs(float(y_d.sum(dtype=torch.float64).item()) - float((counts * table).sum())) <= 1e-6 * abs(float((counts * table).sum())) + 1e-3
+
+
+def test_full_size_requantize_and_range_vs_oracle(hip, dev):
+    """2^28 int32 accumulators: RequantizationRange (depth 1) is the exact min / max, its float range equals the
+    oracle's on the same extremes, and Requantize int32 -> qint8 / quint8 equals the oracle on three windows; the
+    whole tensor through an int64 checksum against torch's evaluation of the same fp32 multiply, rounding and clamp."""
+    import torch
+    n = 1 << 28
+    g = torch.Generator(device=dev)
+    g.manual_seed(31)
+    acc = (torch.randn(n, device=dev, generator=g) * float(1 << 20)).round_().to(torch.int32)
+    acc[12345] = -(1 << 27)
+    acc[n - 77] = (1 << 27) + 12345
+    imn = torch.zeros(1, dtype=torch.int32, device=dev)
+    imx = torch.zeros(1, dtype=torch.int32, device=dev)
+    hip.minmax_i32_per_channel(acc, n, 1, imn, imx)
+    torch.cuda.synchronize()
+    lo_i, hi_i = int(imn.item()), int(imx.item())
+    assert lo_i == int(acc.min().item()) == -(1 << 27) and hi_i == int(acc.max().item()) == (1 << 27) + 12345
+    # the op's float range is host math on the two integers: the oracle on a tensor holding just the extremes
+    in_min, in_max = np.float32(-1.5), np.float32(2.25)
+    st, omn_ref, omx_ref = orc.requantization_range_per_channel(np.array([[lo_i], [hi_i]], np.int32), [in_min], [in_max], 6.0)
+    amax = np.float32(max(abs(lo_i), abs(hi_i)))
+    rng_f = np.float32(max(abs(in_min), abs(in_max))) * amax / np.float32(2 ** 31)
+    assert np.float32(min(rng_f, np.float32(6.0))) == omx_ref and -omx_ref == omn_ref
+    for out_type, tdt in ((orc.QINT8, torch.int8), (orc.QUINT8, torch.uint8)):
+        factor = np.float32(127.0 if out_type == orc.QINT8 else 255.0)
+        req = np.float32(omx_ref)
+        scale = factor * (np.float32(max(abs(in_min), abs(in_max))) / req / np.float32(2 ** 31))
+        q_d = torch.empty(n, dtype=tdt, device=dev)
+        hip.requantize(acc, q_d, n, out_type, float(scale))
+        torch.cuda.synchronize()
+        for lo in _windows(n):
+            xs = acc[lo:lo + (1 << 20)].cpu().numpy().reshape(1, 1, -1, 1)
+            st, q_ref, _, _ = orc.requantize_per_channel(xs, [in_min], [in_max], -float(req), float(req), out_type)
+            np.testing.assert_array_equal(q_d[lo:lo + (1 << 20)].cpu().numpy(), q_ref.reshape(-1))
+        info = np.iinfo(orc.NP_OF[out_type])
+        expect_sum = 0
+        for lo in range(0, n, 1 << 26):
+            part = torch.round(acc[lo:lo + (1 << 26)].to(torch.float32) * float(scale)).clamp_(float(info.min), float(info.max))
+            expect_sum += int(part.sum(dtype=torch.float64).item())
+        assert int(q_d.sum(dtype=torch.int64).item()) == expect_sum
+        del q_d
+
+
 @pytest.mark.parametrize("nbytes,offset", [(1 << 20, 0), (4099, 0), (70001, 3), (15, 1), (0, 0)])
 def test_device_copy_kernel(hip, dev, nbytes, offset):
     import torch

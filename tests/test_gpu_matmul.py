@@ -473,9 +473,11 @@ def test_llama_prefill_rows_sampled(hip, dev, K, N):
     layer0 = Linear(hip, dev, layer.wq, layer.min_b, layer.max_b, np.zeros(N, np.float32))
     kw = dict(api=orc.API_V1, t_out=orc.QINT32, input_mode=orc.SCALED, n_fused_ops=1)
     acc = layer0.run(xq, kw, mn, mx).astype(np.int64)
-    if np.abs(acc).max() < 2 ** 24:  # exact through the fp32 epilogue only below 2^24
-        rowsum_w = layer.wq.astype(np.int64).sum(1)
-        np.testing.assert_array_equal(acc.sum(1), xq.astype(np.int64) @ rowsum_w)
+    # the qint32 result passes through fp32 (scale 1.0), which is exact below 2^24: true for this data at every K
+    # tested (|acc| stays below ~3e6), and asserted so that the identity below can never be skipped silently
+    assert np.abs(acc).max() < 2 ** 24
+    rowsum_w = layer.wq.astype(np.int64).sum(1)
+    np.testing.assert_array_equal(acc.sum(1), xq.astype(np.int64) @ rowsum_w)
 
 
 @pytest.mark.parametrize("M", [1, 4, 16])
@@ -522,6 +524,64 @@ def test_per_token_activation_ranges(hip, dev, M, kw, K, N):
     with pytest.raises(hip.ItexHipError):
         hip.qmatmul_per_row(p, torch.from_numpy(xq).to(dev), layer.packed, layer.colsum, 17, K, N, mins_d, maxs_d,
                             layer.min_b_d, layer.max_b_d, layer.min_b.size, layer.bias_d, out)
+
+
+@pytest.mark.parametrize("M", [1, 4, 16])
+@pytest.mark.parametrize("K,N", [(4096, 14336), (14336, 4096)])
+def test_llama_decode_per_token_full_size(hip, dev, M, K, N):
+    """The decode shapes at full size with per-token activation ranges, from float activations: the per-row dynamic
+    quantization (itexhip_quantize_dynamic_rows) must equal QuantizeV2 of each row against its own range, and every
+    output of itexhip_qmatmul_per_row the oracle's 1 x K problem with that row's range."""
+    import torch
+    layer, w, bias = make_layer(hip, dev, K, N, seed=30 + M)
+    rng = np.random.default_rng(40 + M + K)
+    x = (rng.standard_normal((M, K)) * rng.uniform(0.5, 2.0, (M, 1))).astype(np.float32)
+    rows_q, mins, maxs = [], [], []
+    for m in range(M):
+        _, q, mn, mx = orc.quantize_v2(x[m:m + 1], x[m].min(), x[m].max(), orc.QUINT8, orc.MIN_FIRST)
+        rows_q.append(q)
+        mins.append(mn[0])
+        maxs.append(mx[0])
+    xq_ref = np.concatenate(rows_q, 0)
+    x_d = torch.from_numpy(x).to(dev)
+    xq_d = torch.empty((M, K), dtype=torch.uint8, device=dev)
+    rmn = torch.empty(M, dtype=torch.float32, device=dev)
+    rmx = torch.empty(M, dtype=torch.float32, device=dev)
+    hip.quantize_dynamic_rows(x_d, xq_d, M, K, orc.QUINT8, orc.MIN_FIRST, 0.01, rmn, rmx)
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(xq_d.cpu().numpy(), xq_ref)
+    np.testing.assert_array_equal(rmn.cpu().numpy(), np.array(mins, np.float32))
+    np.testing.assert_array_equal(rmx.cpu().numpy(), np.array(maxs, np.float32))
+    ref = np.concatenate([layer.oracle(xq_ref[m:m + 1], V2_DEQ, mins[m], maxs[m]) for m in range(M)], 0)
+    p = hip.matmul_params(t_in=orc.QUINT8, min_a=0.0, max_a=0.0, **V2_DEQ)
+    out = torch.empty((M, N), dtype=torch.float32, device=dev)
+    hip.qmatmul_per_row(p, xq_d, layer.packed, layer.colsum, M, K, N, rmn, rmx, layer.min_b_d, layer.max_b_d,
+                        layer.min_b.size, layer.bias_d, out)
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(out.cpu().numpy(), ref)
+    assert np.abs(ref - (x @ w + bias)).max() < 0.35
+
+
+@pytest.mark.parametrize("T,mode", [(orc.QUINT8, orc.MIN_FIRST), (orc.QINT8, orc.SCALED)])
+@pytest.mark.parametrize("n,offset_elems", [((1 << 23) + 8, 0), ((1 << 23) + 6, 0), ((1 << 24) + 1, 0)])
+def test_dynamic_quantize_large_tensors(hip, dev, T, mode, n, offset_elems):
+    """itexhip_quantize_dynamic above 4 M elements: the range pass takes several grid-stride rounds and all 512
+    partial ranges are in use (aligned sizes, sizes with a tail of 1 .. 3 elements); bytes and ranges against
+    QuantizeV2 fed with the tensor's min and max."""
+    import torch
+    rng = np.random.default_rng(n)
+    x = rng.standard_normal(n).astype(np.float32)
+    x[n - 2] = 9.5      # the extremes sit in the last workgroup's share and in the tail
+    x[n // 3] = -7.25
+    _, q_ref, omn, omx = orc.quantize_v2(x, x.min(), x.max(), T, mode)
+    x_d = torch.from_numpy(x).to(dev)
+    q_d = torch.empty(n, dtype=tdt(T), device=dev)
+    state = torch.full((hip.DYNAMIC_STATE_FLOATS,), float("nan"), dtype=torch.float32, device=dev)
+    hip.quantize_dynamic(x_d, q_d, n, T, mode, 0.01, state)
+    torch.cuda.synchronize()
+    st = state.cpu().numpy()
+    assert st[0] == -7.25 and st[1] == 9.5 and st[2] == omn[0] and st[3] == omx[0]
+    np.testing.assert_array_equal(q_d.cpu().numpy(), q_ref)
 
 
 def test_hip_graph_replays_match_eager(hip, dev):

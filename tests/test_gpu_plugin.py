@@ -41,9 +41,9 @@ def fetch(torch, out, np_dtype):
     return host.reshape(shape)
 
 
-def run_quantize(torch, dev, x, mn, mx, T, mode, axis=-1, classic=None, forward=False, op="QuantizeV2"):
+def run_quantize(torch, dev, x, mn, mx, T, mode, axis=-1, classic=None, forward=False, op="QuantizeV2", narrow_range=False):
     attrs = dict(T=DT(T), mode=mode, round_mode="HALF_TO_EVEN" if mode == "SCALED" else "HALF_AWAY_FROM_ZERO",
-                 narrow_range=False, axis=axis, ensure_minimum_range=0.01)
+                 narrow_range=bool(narrow_range), axis=axis, ensure_minimum_range=0.01)
     if op == "_ITEXQuantizeV2":
         attrs["dtype"] = DT(tf.FLOAT)
         if classic is not None:
@@ -294,6 +294,40 @@ def test_dequantize_through_plugin(rt, dev):
         _, y_ref = orc.dequantize(q, mn, mx, T, orc.SCALED if mode == "SCALED" else orc.MIN_FIRST)
         np.testing.assert_array_equal(y, y_ref)
         node.close()
+
+
+def test_narrow_range_attr_changes_nothing_through_plugin(rt, dev):
+    """narrow_range is parsed and never used by the reference (quantize_op.h:118; Dequantize reads it as an attribute of
+    the op definition only): QuantizeV2 and Dequantize nodes built with narrow_range = true give the bytes, ranges and
+    floats of the nodes built with false, -128 included for saturating inputs."""
+    torch = rt
+    rng = np.random.default_rng(5)
+    x = (rng.standard_normal(4099) * 1.5).astype(np.float32)
+    x[:3] = [-50.0, 50.0, -1.0]    # saturate on both sides
+    for T, mode in ((tf.QINT8, "SCALED"), (tf.QUINT8, "SCALED"), (tf.QUINT8, "MIN_FIRST")):
+        a = run_quantize(torch, dev, x, -1.0, 1.0, T, mode, narrow_range=False)
+        b = run_quantize(torch, dev, x, -1.0, 1.0, T, mode, narrow_range=True)
+        np.testing.assert_array_equal(a[0], b[0])
+        assert a[1] == b[1] and a[2] == b[2]
+        if T == tf.QINT8:
+            assert b[0][0] == -128 and b[0][1] == 127   # full range, not -127
+        _, q_ref, omn, omx = orc.quantize_v2(x, -1.0, 1.0, T, orc.SCALED if mode == "SCALED" else orc.MIN_FIRST)
+        np.testing.assert_array_equal(b[0], q_ref)
+        ys = []
+        for nr in (False, True):
+            node = tf.Node("Dequantize", dict(T=DT(T), mode=mode, narrow_range=nr, axis=-1, dtype=DT(tf.FLOAT)))
+            assert node.code == tf.OK, node.message
+            mn, mx = np.array(omn[0], np.float32), np.array(omx[0], np.float32)
+            q_d = dev_in(torch, dev, b[0])
+            code, msg, outs = node.run([(T, b[0].shape, q_d.data_ptr(), False), (tf.FLOAT, (), tf.host_array(mn), True),
+                                        (tf.FLOAT, (), tf.host_array(mx), True)], [(tf.FLOAT, False)],
+                                       stream=torch.cuda.current_stream().cuda_stream)
+            assert code == tf.OK, msg
+            ys.append(fetch(torch, outs[0], np.float32))
+            node.close()
+        np.testing.assert_array_equal(ys[0], ys[1])
+        _, y_ref = orc.dequantize(b[0], omn[0], omx[0], T, orc.SCALED if mode == "SCALED" else orc.MIN_FIRST)
+        np.testing.assert_array_equal(ys[1], y_ref)
 
 
 def make_problem(M, K, N, seed, per_channel=True):
