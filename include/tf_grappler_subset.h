@@ -73,6 +73,16 @@ typedef struct TP_OptimizerRegistrationParams {
 } TP_OptimizerRegistrationParams;
 #define TP_OPTIMIZER_REGISTRATION_PARAMS_STRUCT_SIZE (offsetof(TP_OptimizerRegistrationParams, optimizer) + sizeof(TP_Optimizer*))
 
+/* Provided by TensorFlow: the names a rewrite must keep (the item's fetch nodes and its nodes to preserve).  Called as
+ * the reference does (itex/core/graph/utils/grappler_item.cc:23-68): size query first, then the list into caller-owned
+ * storage; values[i] / lengths[i] are not NUL-terminated. */
+void TF_GetNodesToPreserveListSize(const TF_GrapplerItem* item, int* num_values, size_t* storage_size, TF_Status* status);
+void TF_GetNodesToPreserveList(const TF_GrapplerItem* item, char** values, size_t* lengths, int num_values, void* storage,
+                               size_t storage_size, TF_Status* status);
+void TF_GetFetchNodesListSize(const TF_GrapplerItem* item, int* num_values, size_t* storage_size, TF_Status* status);
+void TF_GetFetchNodesList(const TF_GrapplerItem* item, char** values, size_t* lengths, int num_values, void* storage,
+                          size_t storage_size, TF_Status* status);
+
 /* looked up by TensorFlow after dlopen of the plugin */
 void TF_InitGraph(TP_OptimizerRegistrationParams* params, TF_Status* status);
 

@@ -1,4 +1,5 @@
 // Dequantize / _ITEXDequantize op kernel (itex/core/kernels/common/dequantize_op.h:43-186).
+#include <mutex>
 #include <string>
 #include <vector>
 
@@ -37,6 +38,10 @@ class DequantizeOp : public OpKernel {
   }
 
   void Compute(OpKernelContext* ctx) override {
+    // one Compute at a time per node: the cached device vectors below are reassigned in place, and TensorFlow may run
+    // one node from several threads (the reference serialises its kernels the same way, conv_ops.h:786,
+    // quantized_matmul_common.h:62)
+    std::lock_guard<std::mutex> lock(mu_);
     Tensor src = ctx->input(0);
     Tensor in_min = ctx->input(1);
     Tensor in_max = ctx->input(2);
@@ -85,6 +90,7 @@ class DequantizeOp : public OpKernel {
   Mode mode_ = Mode::SCALED;
   bool narrow_range_ = false;
   int32_t axis_ = -1;
+  std::mutex mu_;
   DeviceVectorCache<float> scales_;
   DeviceVectorCache<int32_t> zps_;
 };

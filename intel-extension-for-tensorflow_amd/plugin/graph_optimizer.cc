@@ -9,6 +9,7 @@
 #include <cstdlib>
 #include <cstring>
 #include <map>
+#include <set>
 #include <string>
 #include <vector>
 
@@ -173,7 +174,7 @@ bool MatchDynamicRange(const graph::Node& q, const std::map<std::string, const g
 // MatMul is the only reader of all three outputs, both nodes sit on the same device, the quantization parameters
 // agree (T1 / input_quant_mode), the MatMul has no addend and a Requantize or Dequantize output (the range of a
 // qint32 result is host math on the activation range).  Returns the number of fused pairs.
-int FuseDynamicQuantizeIntoMatMul(graph::Graph* g) {
+int FuseDynamicQuantizeIntoMatMul(graph::Graph* g, const std::set<std::string>& preserve) {
   std::map<std::string, size_t> index;
   std::map<std::string, std::vector<size_t>> readers;  // by producer name: every node with a data or control input from it
   for (size_t i = 0; i < g->nodes.size(); ++i) {
@@ -200,6 +201,9 @@ int FuseDynamicQuantizeIntoMatMul(graph::Graph* g) {
     if (qi == index.end() || dead[qi->second]) continue;
     const graph::Node& q = g->nodes[qi->second];
     if (q.op != "_ITEXQuantizeV2DynamicRange" || q.device != m.device) continue;
+    // a fetched or preserved quantize node has readers outside the graph (its tensor or its range is a session
+    // result): it stays, as the reference keeps preserved nodes out of every fusion (remapper.cc:6373-6390)
+    if (preserve.count(qname)) continue;
     if (Canonical(data[3]) != qname + ":1" || Canonical(data[4]) != qname + ":2") continue;
     bool only_reader = true;
     for (size_t r : readers[qname]) only_reader = only_reader && r == mi;
@@ -271,7 +275,38 @@ void Destroy(void* o) { delete static_cast<Optimizer*>(o); }
 
 void FreeBuffer(void* data, size_t) { std::free(data); }
 
-void Optimize(void* opt, const TF_Buffer* in, const TF_GrapplerItem*, TF_Buffer* out, TF_Status* status) {
+// names the session fetches or asked to keep (itex/core/graph/utils/grappler_item.cc:23-68); a fetch may name a port
+std::set<std::string> NamesToKeep(const TF_GrapplerItem* item) {
+  std::set<std::string> keep;
+  if (item == nullptr) return keep;
+  using SizeFn = void (*)(const TF_GrapplerItem*, int*, size_t*, TF_Status*);
+  using ListFn = void (*)(const TF_GrapplerItem*, char**, size_t*, int, void*, size_t, TF_Status*);
+  const std::pair<SizeFn, ListFn> lists[2] = {{TF_GetNodesToPreserveListSize, TF_GetNodesToPreserveList},
+                                              {TF_GetFetchNodesListSize, TF_GetFetchNodesList}};
+  TF_Status* st = TF_NewStatus();
+  for (const auto& fn : lists) {
+    int count = 0;
+    size_t storage_size = 0;
+    fn.first(item, &count, &storage_size, st);
+    if (TF_GetCode(st) != TF_OK || count <= 0) continue;
+    std::vector<char*> values(count);
+    std::vector<size_t> lengths(count);
+    std::vector<char> storage(storage_size + 1);
+    fn.second(item, values.data(), lengths.data(), count, storage.data(), storage_size, st);
+    if (TF_GetCode(st) != TF_OK) continue;
+    for (int i = 0; i < count; ++i) {
+      std::string name(values[i], lengths[i]);
+      const size_t colon = name.find(':');
+      if (colon != std::string::npos) name.resize(colon);
+      if (!name.empty() && name[0] == '^') name.erase(0, 1);
+      keep.insert(name);
+    }
+  }
+  TF_DeleteStatus(st);
+  return keep;
+}
+
+void Optimize(void* opt, const TF_Buffer* in, const TF_GrapplerItem* item, TF_Buffer* out, TF_Status* status) {
   const Optimizer* self = static_cast<const Optimizer*>(opt);
   graph::Graph g;
   if (!graph::Parse(in->data, in->length, &g)) {
@@ -340,7 +375,7 @@ void Optimize(void* opt, const TF_Buffer* in, const TF_GrapplerItem*, TF_Buffer*
   }
 
   const char* msw = std::getenv("ITEX_AMD_FUSE_QUANTIZE_MATMUL");
-  if (enabled && fuse_dynamic && !(msw && std::strcmp(msw, "0") == 0)) FuseDynamicQuantizeIntoMatMul(&g);
+  if (enabled && fuse_dynamic && !(msw && std::strcmp(msw, "0") == 0)) FuseDynamicQuantizeIntoMatMul(&g, NamesToKeep(item));
 
   const std::string bytes = graph::Serialize(g);
   void* mem = std::malloc(bytes.size() ? bytes.size() : 1);

@@ -1,6 +1,7 @@
 // QuantizeV2 / _ITEXQuantizeV2 op kernel: attribute parsing, host-side range math and output range
 // conventions as in the reference (itex/core/kernels/common/quantize_op.h:68-430), the quantization
 // itself on the GPU through itexhip_quantize / itexhip_quantize_axis.
+#include <mutex>
 #include <cmath>
 #include <string>
 #include <vector>
@@ -56,6 +57,10 @@ class QuantizeV2Op : public OpKernel {
   }
 
   void Compute(OpKernelContext* ctx) override {
+    // one Compute at a time per node: the cached device vectors below are reassigned in place, and TensorFlow may run
+    // one node from several threads (the reference serialises its kernels the same way, conv_ops.h:786,
+    // quantized_matmul_common.h:62)
+    std::lock_guard<std::mutex> lock(mu_);
     Tensor src = ctx->input(0);
     if (!ctx->ok()) return;
     ITEX_REQUIRES(ctx, src.dtype() == src_type_, TF_INVALID_ARGUMENT, "QuantizeV2 input type does not match the kernel");
@@ -182,6 +187,7 @@ class QuantizeV2Op : public OpKernel {
   bool narrow_range_ = false;
   int32_t axis_ = -1;
   float ensure_minimum_range_ = 0.01f;
+  std::mutex mu_;
   DeviceVectorCache<float> params_;
 };
 

@@ -5,6 +5,7 @@
 // parsing, input indices, geometry, output scales and bias factors; the convolution itself runs as
 // itexhip_im2col8 + itexhip_qgemm on the filter prepacked as a [KH*KW*C, O] matrix.
 // Not carried over: Sum / Elu / Swish / HardSwish / Sigmoid fusions, depthwise and 3-D variants, NCHW.
+#include <mutex>
 #include <algorithm>
 #include <cmath>
 #include <cstring>
@@ -164,6 +165,10 @@ class QuantizedConv2DOp : public OpKernel {
   }
 
   void Compute(OpKernelContext* ctx) override {
+    // one Compute at a time per node: the cached device vectors below are reassigned in place, and TensorFlow may run
+    // one node from several threads (the reference serialises its kernels the same way, conv_ops.h:786,
+    // quantized_matmul_common.h:62)
+    std::lock_guard<std::mutex> lock(mu_);
     Tensor x = ctx->input(0);
     Tensor filter = ctx->input(1);
     if (!ctx->ok()) return;
@@ -397,6 +402,7 @@ class QuantizedConv2DOp : public OpKernel {
   Tensor packed_, colsum_;
   const void* packed_src_ = nullptr;
   int64_t packed_k_ = -1, packed_n_ = -1;
+  std::mutex mu_;
   DeviceVectorCache<float> params_;
 };
 

@@ -4,6 +4,7 @@
 #include <cmath>
 #include <cstdlib>
 #include <limits>
+#include <mutex>
 #include <string>
 #include <vector>
 
@@ -24,6 +25,8 @@ class RequantizePerChannelOp : public OpKernel {
     out_type_ = t;
   }
   void Compute(OpKernelContext* ctx) override {
+    // one Compute at a time per node: the cached scale vector is reassigned in place
+    std::lock_guard<std::mutex> lock(mu_);
     Tensor input = ctx->input(0), in_min = ctx->input(1), in_max = ctx->input(2);
     Tensor req_min = ctx->input(3), req_max = ctx->input(4);
     if (!ctx->ok()) return;
@@ -57,6 +60,7 @@ class RequantizePerChannelOp : public OpKernel {
 
  private:
   TF_DataType out_type_;
+  std::mutex mu_;
   DeviceVectorCache<float> scales_;
 };
 struct RequantizeS8 : RequantizePerChannelOp { explicit RequantizeS8(OpKernelConstruction* c) : RequantizePerChannelOp(c, TF_QINT8) {} };

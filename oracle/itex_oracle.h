@@ -34,6 +34,11 @@
  *   the bfloat16 / half bias (Tbias): the adjusted bias is rounded to Tbias as the code is
  *   written (quantized_matmul_common.h:578-599, 609-617); the reference's tests only use float and
  *   qint32 biases;
+ *   legacy MIN_FIRST QuantizeV2 with an axis (per-slice ranges): the reference describes the shift operand of its
+ *   binary_add as a one-element tensor (quantize_op.h:302-303, dims all 1) while handing it a shift per slice and
+ *   per-axis scale masks that the oneDNN binary primitive does not take; its tests run per-axis quantization in
+ *   SCALED mode only.  orc_quantize_v2 gives every slice its own shift -min'[s] and scale (the evident intent;
+ *   pinned as such by tests/test_oracle_quantize.py::test_min_first_per_axis_uses_each_slices_shift);
  *   the quantized convolution's host arithmetic at the last bit and its Sum fusions (orc_qconv2d_sum): the
  *   reference's conv tests hold no vectors, see the comments at those functions.
  *   The bfloat16 / half OUTPUT is pinned: it must equal the nearest-even 16-bit

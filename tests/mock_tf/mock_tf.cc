@@ -682,18 +682,62 @@ int mock_graph_config(const char* name) {
   if (n == "constant_folding") return g_optimizer_configs.constant_folding;
   return -1;
 }
-// runs the optimizer on a serialized GraphDef; the result is read with mock_graph_result / _size
-int mock_graph_optimize(const void* graph, size_t len) {
+// the grappler item of a run: what the session fetches and what it asked to keep
+struct TF_GrapplerItem {
+  std::vector<std::string> preserve, fetch;
+};
+static void ListSize(const std::vector<std::string>& v, int* num_values, size_t* storage_size, TF_Status* status) {
+  *num_values = static_cast<int>(v.size());
+  *storage_size = 0;
+  for (const std::string& s : v) *storage_size += s.size();
+  status->code = TF_OK;
+}
+static void ListFill(const std::vector<std::string>& v, char** values, size_t* lengths, int num_values, void* storage,
+                     size_t storage_size, TF_Status* status) {
+  char* p = static_cast<char*>(storage);
+  size_t used = 0;
+  for (int i = 0; i < num_values && i < static_cast<int>(v.size()); ++i) {
+    if (used + v[i].size() > storage_size) { status->code = TF_INVALID_ARGUMENT; return; }
+    std::memcpy(p + used, v[i].data(), v[i].size());
+    values[i] = p + used;
+    lengths[i] = v[i].size();
+    used += v[i].size();
+  }
+  status->code = TF_OK;
+}
+void TF_GetNodesToPreserveListSize(const TF_GrapplerItem* item, int* n, size_t* bytes, TF_Status* st) { ListSize(item->preserve, n, bytes, st); }
+void TF_GetNodesToPreserveList(const TF_GrapplerItem* item, char** values, size_t* lengths, int n, void* storage, size_t bytes,
+                               TF_Status* st) { ListFill(item->preserve, values, lengths, n, storage, bytes, st); }
+void TF_GetFetchNodesListSize(const TF_GrapplerItem* item, int* n, size_t* bytes, TF_Status* st) { ListSize(item->fetch, n, bytes, st); }
+void TF_GetFetchNodesList(const TF_GrapplerItem* item, char** values, size_t* lengths, int n, void* storage, size_t bytes,
+                          TF_Status* st) { ListFill(item->fetch, values, lengths, n, storage, bytes, st); }
+
+static std::vector<std::string> SplitCsv(const char* csv) {
+  std::vector<std::string> out;
+  if (!csv) return out;
+  std::string cur;
+  for (const char* c = csv; ; ++c) {
+    if (*c == ',' || *c == 0) { if (!cur.empty()) out.push_back(cur); cur.clear(); if (*c == 0) break; }
+    else cur.push_back(*c);
+  }
+  return out;
+}
+
+// runs the optimizer on a serialized GraphDef; the result is read with mock_graph_result / _size.  `preserve` / `fetch`:
+// comma-separated node names of the grappler item (null: the optimizer gets no item at all)
+int mock_graph_optimize_item(const void* graph, size_t len, const char* preserve, const char* fetch) {
   void* opt = g_optimizer.create_func ? g_optimizer.create_func() : nullptr;
   TF_Buffer in{graph, len, nullptr};
   TF_Buffer out{nullptr, 0, nullptr};
   TF_Status st;
-  g_optimizer.optimize_func(opt, &in, nullptr, &out, &st);
+  TF_GrapplerItem item{SplitCsv(preserve), SplitCsv(fetch)};
+  g_optimizer.optimize_func(opt, &in, (preserve || fetch) ? &item : nullptr, &out, &st);
   if (g_optimizer.destroy_func) g_optimizer.destroy_func(opt);
   g_optimized.assign(static_cast<const char*>(out.data), out.length);
   if (out.data_deallocator) out.data_deallocator(const_cast<void*>(out.data), out.length);
   return st.code;
 }
+int mock_graph_optimize(const void* graph, size_t len) { return mock_graph_optimize_item(graph, len, nullptr, nullptr); }
 const void* mock_graph_result(void) { return g_optimized.data(); }
 size_t mock_graph_result_size(void) { return g_optimized.size(); }
 

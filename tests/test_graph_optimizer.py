@@ -33,6 +33,16 @@ def run(opt, graph):
     return out
 
 
+def run_with_item(opt, graph, preserve="", fetch=""):
+    """The same with a grappler item: comma-separated names the session asked to preserve / fetches."""
+    data = graph.SerializeToString()
+    code = opt.mock_graph_optimize_item(data, C.c_size_t(len(data)), preserve.encode(), fetch.encode())
+    assert code == tf.OK
+    out = gd.GraphDef()
+    out.ParseFromString(C.string_at(opt.mock_graph_result(), opt.mock_graph_result_size()))
+    return out
+
+
 def by_name(g):
     return {n.name: n for n in g.node}
 
@@ -250,6 +260,18 @@ def test_dynamic_quantize_matmul_pairs_that_stay_apart(opt, kw):
     out = by_name(run(opt, dynamic_linear_graph(**kw)))
     assert out["q"].op == "_ITEXQuantizeV2DynamicRange"
     assert out["mm"].op in ("_ITEXQuantizedMatMul", "_QuantizedMatMul") and out["mm"].input[0] == "q"
+
+
+@pytest.mark.parametrize("item", [dict(preserve="q"), dict(fetch="q:1"), dict(fetch="q"), dict(preserve="w,q,b")])
+def test_preserved_or_fetched_quantize_node_is_not_fused_away(opt, item):
+    """A quantize node whose tensor or range the session fetches (or asked to preserve) has no reader inside the graph
+    besides the MatMul, yet it must survive: the fusion reads the grappler item and leaves such a pair alone."""
+    out = by_name(run_with_item(opt, dynamic_linear_graph(), **item))
+    assert out["q"].op == "_ITEXQuantizeV2DynamicRange"
+    assert out["mm"].op in ("_ITEXQuantizedMatMul", "_QuantizedMatMul") and out["mm"].input[0] == "q"
+    # an item that names other nodes only does not stand in the way
+    out = by_name(run_with_item(opt, dynamic_linear_graph(), preserve="w", fetch="mm"))
+    assert "q" not in out and out["mm"].op == "_ITEXQuantizedMatMulDynamicInput"
 
 
 def test_dynamic_quantize_matmul_scaled_and_switch(opt, monkeypatch):

@@ -245,6 +245,26 @@ def test_requantization_range_per_channel():
     assert omx == np.finfo(np.float32).tiny and omn == 0.0
 
 
+def test_min_first_per_axis_uses_each_slices_shift():
+    """Legacy MIN_FIRST with an axis: slice s is quantized with its own scale 255 / (max'[s] - min'[s]) and its own
+    shift -min'[s] (parity unpinned against the reference, whose text describes a one-element shift tensor,
+    quantize_op.h:302-303; this pins the behaviour chosen here).  Each slice must equal the per-tensor op run on
+    that slice alone, and a slice whose minimum differs from slice 0's must differ from what slice 0's shift would
+    give."""
+    x = np.array([[-1.0, 0.0, 0.5, 3.0], [-4.0, -2.0, 1.0, 2.0]], np.float32)
+    mn, mx = np.array([-1.0, -4.0], np.float32), np.array([3.0, 2.0], np.float32)
+    st, q, omn, omx = orc.quantize_v2(x, mn, mx, orc.QUINT8, orc.MIN_FIRST, axis=0)
+    assert st == orc.OK
+    for s in range(2):
+        _, q1, mn1, mx1 = orc.quantize_v2(x[s], mn[s], mx[s], orc.QUINT8, orc.MIN_FIRST)
+        np.testing.assert_array_equal(q[s], q1)
+        assert omn[s] == mn1[0] and omx[s] == mx1[0]
+    # closed form, slice 1: scale 255 / 6 = 42.5, shift 4 -> round(x * 42.5 + 170)
+    assert q[1].tolist() == [0, 85, 212, 255]
+    # with slice 0's shift (1 -> 42.5) the same slice would read [0, 0, 85, 128]
+    assert q[1].tolist() != [0, 0, 85, 128]
+
+
 def test_narrow_range_has_no_effect_documented():
     # the reference reads narrow_range and never uses it (quantize_op.h:118): the oracle has no such
     # parameter at all; out-of-range negatives saturate to -128

@@ -61,9 +61,11 @@ def test_host_memory_and_constraints(reg):
     assert len(legacy) == 2 and {k["constraints"]["Tbias"] for k in legacy} == {tf.FLOAT, tf.QINT32}
     assert all({**k["constraints"], "Tbias": 0} == {"T1": tf.QUINT8, "T2": tf.QINT8, "Tbias": 0, "Toutput": tf.QUINT8}
                for k in legacy)
-    assert {k["constraints"]["Tbias"] for k in v2} == {tf.FLOAT, tf.QINT32, tf.BFLOAT16, tf.HALF}
+    # every bias / args type the reference registers for a device (kernels/gpu/quantized_matmul.cc:118-133)
+    all_bias = {tf.FLOAT, tf.QINT32, tf.BFLOAT16, tf.HALF, tf.QINT8, tf.QUINT8}
+    assert {k["constraints"]["Tbias"] for k in v2} == all_bias
     assert {(k["constraints"]["Targs"], k["constraints"]["Toutput"]) for k in deq} == {
-        (b, o) for b in (tf.FLOAT, tf.QINT32, tf.BFLOAT16, tf.HALF) for o in (tf.FLOAT, tf.BFLOAT16, tf.HALF)}
+        (b, o) for b in all_bias for o in (tf.FLOAT, tf.BFLOAT16, tf.HALF)}
     ldq = kernels_of(reg, "QuantizedMatMulWithBiasAndDequantize")
     assert {(k["constraints"]["Tbias"], k["constraints"]["Toutput"]) for k in ldq} == {
         (b, o) for b in (tf.FLOAT, tf.QINT32) for o in (tf.FLOAT, tf.BFLOAT16, tf.HALF)}
@@ -149,6 +151,27 @@ def test_matmul_attr_validation():
     n = tf.Node("_QuantizedFusedMatMulAndRequantize", dict(v1, fused_ops=["BiasAdd", "Relu", "Relu6"]))
     assert n.code == tf.INVALID_ARGUMENT and n.message == "_QuantizedFusedMatMul supports maximum 2 post ops"
     assert tf.Node("_QuantizedFusedMatMulAndRequantize", dict(v1, fused_ops=["BiasAdd", "Relu"])).code == tf.OK
+
+
+def test_eight_bit_bias_is_placed_and_refused_at_compute():
+    """Tbias = qint8 / quint8 is registered (a graph naming it finds a kernel, as on the reference's device) and the
+    node is constructed; Compute refuses it with TF_UNIMPLEMENTED before any device work."""
+    for tb in (tf.QINT8, tf.QUINT8):
+        base = dict(T1=DT(tf.QUINT8), T2=DT(tf.QINT8), Tbias=DT(tb), Tout=DT(tf.FLOAT), transpose_a=False,
+                    transpose_b=False, is_weight_const=True, is_bias_const=True, fused_ops=["BiasAdd", "Dequantize"],
+                    input_quant_mode="MIN_FIRST", output_quant_mode="SCALED", leakyrelu_alpha=0.2)
+        n = tf.Node("_QuantizedMatMul", base)
+        assert n.code == tf.OK, n.message
+        a = np.zeros((4, 32), np.uint8)
+        w = np.zeros((32, 8), np.int8)
+        b = np.zeros(8, tf.NP_OF[tb])
+        s = [np.array(v, np.float32) for v in (0.0, 1.0)]
+        wr = [np.full(8, v, np.float32) for v in (-1.0, 1.0)]
+        code, msg, _ = n.run([(tf.QUINT8, a.shape, tf.host_array(a), False), (tf.QINT8, w.shape, tf.host_array(w), False),
+                              (tb, b.shape, tf.host_array(b), False)] +
+                             [(tf.FLOAT, v.shape, tf.host_array(v), True) for v in s + wr], [(tf.FLOAT, False)])
+        assert code == tf.UNIMPLEMENTED and "qint8 or quint8" in msg
+        n.close()
 
 
 def test_matmul_shape_validation_before_device_work():
