@@ -26,6 +26,15 @@ PEAK_HBM_GBS = 8000.0      # MI355X HBM3E, published
 PEAK_INT8_TOPS = 5000.0    # MI355X dense int8 MFMA, published (tera-ops/s)
 
 
+def kernel_source_sha(root):
+    """sha256 over the sources of the headline kernel: ties a counter measurement to the code it was taken on."""
+    import hashlib
+    h = hashlib.sha256()
+    for f in ("qgemm_tile.hpp", "qgemm_common.hpp", "qmatmul_params.hpp"):
+        h.update(open(os.path.join(root, "intel-extension-for-tensorflow_amd", "csrc", f), "rb").read())
+    return h.hexdigest()
+
+
 def _setup():
     import torch
     import __graft_entry__ as entry
@@ -417,6 +426,139 @@ def bench_conv(torch, hip, timer, steps, warmup, dev):
     return out
 
 
+
+def bench_config1_chain(torch, hip, timer, steps, warmup, dev):
+    """BASELINE config 1 as a chain of three ops on one stream, 128 x 1024 x 1024: QuantizeV2 (given range) ->
+    quantized MatMul [BiasAdd, Relu, Requantize] -> quint8 -> Dequantize (SCALED).  Latency-bound: reported in us per
+    chain, launched eagerly and replayed from a HIP graph.  `literal`: SCALED qint8 activations as the configuration
+    states it, V1 (_QuantizedFusedMatMulAndRequantize, fused_ops [BiasAdd, Relu]) and V2 (_QuantizedMatMul, fused_ops
+    [BiasAdd, Relu, Requantize]) spellings, with the reference's as-written bias scaling and dropped requantize factor;
+    `min_first`: the same chain with MIN_FIRST quint8 activations (the V2 spelling), where those two quirks do not
+    apply."""
+    import numpy as np
+    M, K, N = 128, 1024, 1024
+    L = make_weights(torch, hip, K, N, 0, dev)
+    g = torch.Generator(device=dev)
+    g.manual_seed(0)
+    x = torch.randn(M, K, device=dev, generator=g)
+    mn, mx = float(x.min()), float(x.max())
+    r_out = float(torch.relu(x @ (L["wq"].float() * (L["max_b"] / 127.0)) + L["bias"]).max())
+    f32 = np.float32
+    y = torch.empty(M, N, dtype=torch.float32, device=dev)
+    out = []
+    for name, t_in, mode, api in (("literal_v1", hip.QINT8, hip.SCALED, hip.API_V1), ("literal_v2", hip.QINT8, hip.SCALED, hip.API_V2),
+                                  ("min_first_v2", hip.QUINT8, hip.MIN_FIRST, hip.API_V2)):
+        amn, amx = min(f32(0.0), f32(mn)), max(f32(0.0), f32(mx))
+        if mode == hip.SCALED:
+            r = max(abs(amn), abs(amx))
+            q_scale, q_add, min_a, max_a = float(f32(127.0) / r), 0.0, float(-r), float(r)
+        else:
+            sc = f32(255.0 / float(amx - amn))
+            q_scale, q_add, min_a, max_a = float(sc), float(f32(-amn) * sc), float(amn), float(amx)
+        xq = torch.empty(M, K, dtype=torch.int8 if t_in == hip.QINT8 else torch.uint8, device=dev)
+        q8 = torch.empty(M, N, dtype=torch.uint8, device=dev)
+        kw = dict(api=api, t_in=t_in, t_out=hip.QUINT8, input_mode=mode, activation=hip.ACT_RELU, min_a=min_a, max_a=max_a,
+                  min_out=0.0, max_out=r_out)
+        if api == hip.API_V1:
+            kw["n_fused_ops"] = 2
+        else:
+            kw["has_requantize"] = True
+        p = hip.matmul_params(**kw)
+        dq_scale = float(f32(r_out) / f32(255.0))   # Dequantize SCALED of a quint8 tensor with range (0, r_out)
+
+        def make(stream):
+            def chain(i):
+                hip.quantize(x, xq, M * K, t_in, q_scale, q_add, stream)
+                hip.qmatmul(p, xq, L["packed"], L["colsum"], M, K, N, L["min_b"], L["max_b"], N, L["bias"], q8, stream)
+                hip.dequantize(q8, y, M * N, hip.QUINT8, dq_scale, 0, stream)
+            return chain
+        ms_eager = timer.run(make(_stream(torch)), steps, warmup)
+        ms_graph = timer.run_graph(make, steps, warmup)
+        out.append(dict(name="config1_chain_" + name, M=M, K=K, N=N, us_per_chain=ms_graph * 1e3, us_per_chain_eager=ms_eager * 1e3,
+                        launches=3, ops=2.0 * M * K * N, bound="latency",
+                        note="QuantizeV2 -> MatMul [BiasAdd, Relu, Requantize] -> Dequantize, three launches; graph replay / eager"))
+    return out
+
+
+def bench_read_floor(torch, hip, timer, nbytes, steps, warmup, dev, copies=8):
+    """What one launch that only reads `nbytes` from HBM costs on this box (`copies` distinct buffers cycled): the floor
+    under the decode MatMul, which has to stream as many weight bytes per launch."""
+    bufs = [torch.randint(0, 256, (nbytes,), dtype=torch.uint8, device=dev) for _ in range(copies)]
+    sink = torch.zeros(256, dtype=torch.int32, device=dev)
+    st = _stream(torch)
+    ms = timer.run(lambda i: hip.read_probe(bufs[i % copies], nbytes, sink, st), steps, warmup)
+    ms_g = timer.run_graph(lambda stream: (lambda i: hip.read_probe(bufs[i % copies], nbytes, sink, stream)), steps, warmup)
+    best = min(ms, ms_g)
+    return dict(name="hbm_read_floor", bytes=nbytes, us_kernel=best * 1e3, us_eager=ms * 1e3, us_graph=ms_g * 1e3,
+                gbs=nbytes / (best * 1e-3) / 1e9, frac=nbytes / (best * 1e-3) / 1e9 / PEAK_HBM_GBS, bound="hbm",
+                note="itexhip_read_probe: one launch that only reads the decode weight's byte count (8 buffers cycled)")
+
+
+class PowerSampler:
+    """Socket power and shader clock from the amdgpu sysfs files, sampled while `fn` is launched back to back for
+    `seconds`: the evidence for (or against) a power-limited kernel.  Returns None where the files are not readable."""
+
+    def __init__(self):
+        import glob
+        self.power = (glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*/power1_input") +
+                      glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*/power1_average") + [None])[0]
+        self.cap = (glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*/power1_cap") + [None])[0]
+        self.sclk = (glob.glob("/sys/class/drm/card*/device/pp_dpm_sclk") + [None])[0]
+
+    @staticmethod
+    def _read(path):
+        try:
+            return open(path).read()
+        except Exception:
+            return None
+
+    def _sample(self):
+        pw = self._read(self.power) if self.power else None
+        ck = self._read(self.sclk) if self.sclk else None
+        mhz = None
+        if ck:
+            cur = [l for l in ck.splitlines() if "*" in l]
+            if cur:
+                digits = "".join(c for c in cur[0].split(":")[1] if c.isdigit())
+                mhz = float(digits) if digits else None
+        return (float(pw) / 1e6 if pw else None), mhz
+
+    def run(self, torch, fn, seconds=1.5):
+        import threading
+        if not self.power:
+            return None
+        stop = [False]
+        count = [0]
+
+        def worker():
+            torch.cuda.set_device(0)
+            while not stop[0]:
+                for _ in range(100):
+                    fn()
+                torch.cuda.synchronize()
+                count[0] += 100
+        th = threading.Thread(target=worker)
+        t0 = time.perf_counter()
+        th.start()
+        watts, mhz = [], []
+        while time.perf_counter() - t0 < seconds:
+            time.sleep(0.05)
+            if time.perf_counter() - t0 < 0.4:   # let the governor settle
+                continue
+            w, c = self._sample()
+            if w is not None:
+                watts.append(w)
+            if c is not None:
+                mhz.append(c)
+        stop[0] = True
+        th.join()
+        dt = time.perf_counter() - t0
+        cap = self._read(self.cap)
+        return dict(power_w=sum(watts) / len(watts) if watts else None, sclk_mhz=sum(mhz) / len(mhz) if mhz else None,
+                    power_cap_w=float(cap) / 1e6 if cap else None, us_per_launch_sustained=dt / max(count[0], 1) * 1e6,
+                    samples=len(watts))
+
+
 def bench_mfma_ceiling(torch, hip, timer, xq, wq, dev):
     """Matrix-pipe-only rate for operand bits like the workload's (bytes of the quantized activations,
     sign-flipped as the kernel feeds them, and of the weights) and for constant operands."""
@@ -482,14 +624,14 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--only", type=str, default="", help="comma list of: headline, prefill, bert, bmm, conv, gemv, elementwise, copy")
+    ap.add_argument("--only", type=str, default="", help="comma list of: headline, c1, prefill, bert, bmm, conv, gemv, elementwise, copy, power")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-rows", type=int, default=2048, help="rows of the headline workload the CPU oracle runs")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU only: this build has no multi-GPU path (--gpus must be 1)", file=sys.stderr)
         sys.exit(2)
-    only = set(s for s in args.only.split(",") if s) or {"headline", "prefill", "bert", "bmm", "conv", "gemv", "elementwise"}
+    only = set(s for s in args.only.split(",") if s) or {"headline", "c1", "prefill", "bert", "bmm", "conv", "gemv", "elementwise", "power"}
 
     torch, hip = _setup()
     dev = torch.device("cuda:0")
@@ -503,6 +645,28 @@ def main():
     ctx = head.pop("_ctx")
 
     ceiling = bench_mfma_ceiling(torch, hip, timer, ctx["xq"], ctx["layers"][0]["wq"], dev)
+
+    power = None
+    if "power" in only:
+        # socket power and shader clock under the headline kernel, under the matrix-pipe probe on the workload's
+        # operand bytes and on constant operands, and at idle: a kernel whose clock drops while the power sits at the
+        # board's limit is limited by energy per operation, not by issue slots
+        sampler = PowerSampler()
+        L0, p0, xq0 = ctx["layers"][0], ctx["p"], ctx["xq"]
+        out0 = torch.empty(M, N, dtype=torch.int8, device=dev)
+        st0 = _stream(torch)
+        sink = torch.zeros(256, dtype=torch.int32, device=dev)
+        wl = torch.cat([L0["wq"].reshape(-1)[:4096].contiguous().view(torch.uint8), (xq0.reshape(-1)[:4096] ^ 0x80).contiguous()])
+        ones = torch.ones(8192, dtype=torch.uint8, device=dev)
+        time.sleep(0.5)
+        idle = sampler._sample()
+        power = dict(
+            idle_w=idle[0],
+            headline_gemm=sampler.run(torch, lambda: hip.qmatmul(p0, xq0, L0["packed"], L0["colsum"], M, K, N, L0["min_b"], L0["max_b"], N,
+                                                                 L0["bias"], out0, st0)),
+            mfma_probe_workload_data=sampler.run(torch, lambda: hip.mfma_probe(256, 200, wl, sink, st0)),
+            mfma_probe_constant_operands=sampler.run(torch, lambda: hip.mfma_probe(256, 200, ones, sink, st0)),
+            note="amdgpu sysfs (power1_input, pp_dpm_sclk) sampled every 50 ms over 1.5 s of back-to-back launches")
 
     cpu = None
     if not args.no_cpu:
@@ -532,6 +696,8 @@ def main():
                                                "reference's CPU path, not ITEX itself")
     del ctx
 
+    if "c1" in only:
+        others.extend(bench_config1_chain(torch, hip, timer, K_steps, W, dev))
     if "prefill" in only:
         others.append(bench_dynamic_linear(torch, hip, timer, 2048, 4096, 14336, max(10, K_steps // 2), max(3, W // 2), dev, seed=22))
         for (k, n, seed) in ((4096, 4096, 20), (4096, 6144, 21), (14336, 4096, 23)):
@@ -553,12 +719,15 @@ def main():
     if "conv" in only:
         others.extend(bench_conv(torch, hip, timer, K_steps, W, dev))
     if "gemv" in only:
+        floor = bench_read_floor(torch, hip, timer, 4096 * 14336, K_steps, W, dev)
+        others.append(floor)
         for (k, n) in ((4096, 14336), (14336, 4096)):
             for m in (1, 4, 16):
                 r = bench_linear(torch, hip, timer, m, k, n, "deq", K_steps, W, dev, seed=10, rotate=8, graph=True)
                 r.pop("_ctx")
                 r.update(name="decode_gemv", bound="hbm", frac=r["gbs_kernel"] / PEAK_HBM_GBS,
                          frac_graph=r["gbs_kernel_graph"] / PEAK_HBM_GBS,
+                         read_floor_us=floor["us_kernel"], frac_of_read_floor=floor["us_kernel"] / r["us_kernel"],
                          note="8 weight copies cycled (470 MB > last-level cache)")
                 others.append(r)
             others.append(bench_dynamic_linear(torch, hip, timer, 16, k, n, K_steps, W, dev, seed=10))
@@ -584,11 +753,16 @@ def main():
             r.update(bound="hbm")
             others.append(r)
 
-    traffic = None
+    # HBM bytes per launch of the headline kernel as the memory counters measured them (rocprofv3 --pmc FETCH_SIZE /
+    # WRITE_SIZE, see profiles/): only reported when the kernel's source is still the one that was profiled
+    traffic, traffic_note = None, "not measured for this version of the kernel source"
     tpath = os.path.join(ROOT, "profiles", "traffic.json")
     if os.path.exists(tpath):
         try:
-            traffic = json.load(open(tpath)).get("qgemm_tile_prefill_2048x4096x14336")
+            rec = json.load(open(tpath))
+            if rec.get("_detail", {}).get("kernel_source_sha256") == kernel_source_sha(ROOT):
+                traffic = rec.get("qgemm_tile_prefill_2048x4096x14336")
+                traffic_note = "bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, see profiles/"
         except Exception:
             traffic = None
 
@@ -600,8 +774,9 @@ def main():
         "config": {"workload": "Llama-3-8B prefill linear M=2048 K=4096 N=14336: quint8 act (MIN_FIRST, N(0,1) + 0.1% x20 "
                                "outliers) x qint8 per-channel weights, _QuantizedMatMul [BiasAdd, Requantize] -> qint8; "
                                "step = one launch of the op (the kernel derives scales and bias itself)"},
-        "roofline": {"bound": "mfma", "achieved": head["tops_kernel"], "peak": PEAK_INT8_TOPS, "unit": "TFLOP/s",
-                     "frac": head["tops_kernel"] / PEAK_INT8_TOPS, "traffic": traffic,
+        "roofline": {"bound": "mfma", "achieved": head["tops_kernel"], "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
+                     "frac": head["tops_kernel"] / PEAK_INT8_TOPS, "traffic": traffic, "traffic_note": traffic_note,
+                     "power": power,
                      "kernel": "qgemm_tile_kernel", "us_per_launch": head["us_kernel"],
                      "note": "ops are int8 multiply-accumulates (2*M*N*K per launch); achieved and peak are tera-ops/s",
                      "mfma_only_rate_measured": ceiling,

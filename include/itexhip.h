@@ -464,6 +464,12 @@ int itexhip_qconv2d_sum(const void* x, int x_type, const itexhip_conv_geometry* 
  * peak.  `sink` takes 256 ints that are practically never written. */
 int itexhip_mfma_probe(int workgroups, int iters, const void* operands, int32_t* sink, void* stream);
 
+/* Diagnostic, no counterpart in the reference: one launch that reads `bytes` (a multiple of 16 KiB is read in full;
+ * 16-byte aligned) from `src` and keeps nothing (`sink`: 256 ints, practically never written).  Timed by the caller,
+ * it gives what a single launch that only streams that many bytes from HBM costs on this device: the floor next to
+ * which the bandwidth-bound kernels (the decode MatMul above all) are to be read. */
+int itexhip_read_probe(const void* src, size_t bytes, int32_t* sink, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -391,6 +391,23 @@ __global__ __launch_bounds__(kThreads) void copy_vec_kernel(const i4* __restrict
   }
 }
 
+// Read-only sweep: every workgroup walks the buffer a whole grid apart with four 16-byte loads in flight per lane and
+// keeps nothing.  Timed by the caller, it gives what one launch that only reads that many bytes costs on a device:
+// the floor under any kernel that has to stream the same bytes once.
+__global__ __launch_bounds__(kThreads) void read_probe_kernel(const i4* __restrict__ src, int64_t n16, int* __restrict__ sink) {
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * (kThreads * kUnroll);
+  i4 acc = i4{0, 0, 0, 0};
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * (kThreads * kUnroll) + threadIdx.x; i + (kUnroll - 1) * kThreads < n16; i += stride) {
+    i4 v[kUnroll];
+#pragma unroll
+    for (int j = 0; j < kUnroll; ++j) v[j] = __builtin_nontemporal_load(&src[i + j * kThreads]);
+#pragma unroll
+    for (int j = 0; j < kUnroll; ++j) acc ^= v[j];
+  }
+  const int s = acc.x ^ acc.y ^ acc.z ^ acc.w;
+  if (s == 0x5a17c0de) sink[threadIdx.x] = s;  // keeps the loads alive; practically never taken
+}
+
 __global__ __launch_bounds__(kThreads) void copy_byte_kernel(const uint8_t* __restrict__ src,
                                                              uint8_t* __restrict__ dst, int64_t begin, int64_t n) {
   const int64_t i = begin + static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
@@ -946,6 +963,15 @@ extern "C" int itexhip_memcpy_d2d_async(void* dst, const void* src, size_t bytes
     copy_byte_kernel<<<blocks_for(n - done, kThreads), kThreads, 0, st>>>(
         reinterpret_cast<const uint8_t*>(src), reinterpret_cast<uint8_t*>(dst), done, n);
   ITEXHIP_CHECK_LAUNCH("itexhip_memcpy_d2d_async");
+  return ITEXHIP_OK;
+}
+
+extern "C" int itexhip_read_probe(const void* src, size_t bytes, int32_t* sink, void* stream) {
+  ITEXHIP_REQUIRE(src && sink && aligned(src, 16) && bytes >= 16384, "itexhip_read_probe: 16-byte aligned buffer of at least 16 KiB");
+  const int64_t n16 = static_cast<int64_t>(bytes / 16);
+  const unsigned grid = static_cast<unsigned>(std::min<int64_t>(1024, n16 / (kThreads * kUnroll)));
+  read_probe_kernel<<<grid, kThreads, 0, as_stream(stream)>>>(reinterpret_cast<const i4*>(src), n16, sink);
+  ITEXHIP_CHECK_LAUNCH("itexhip_read_probe");
   return ITEXHIP_OK;
 }
 

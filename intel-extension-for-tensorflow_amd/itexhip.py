@@ -31,7 +31,7 @@ EXPORTS = [
     "itexhip_dequantize16", "itexhip_dequantize_axis16", "itexhip_requantize_per_channel",
     "itexhip_requantize", "itexhip_minmax_i32_per_channel", "itexhip_minmax_f32",
     "itexhip_qmatmul_epilogue_desc", "itexhip_qmatmul_prepare", "itexhip_qgemm_packed_bytes",
-    "itexhip_qgemm_prepack_b", "itexhip_qgemm", "itexhip_qgemm_tile", "itexhip_qgemv", "itexhip_qmatmul", "itexhip_qmatmul_per_row", "itexhip_qmatmul_device_range", "itexhip_quantize_dynamic", "itexhip_quantize_dynamic_static", "itexhip_quantize_dynamic_rows", "itexhip_qmatmul_unpacked", "itexhip_mfma_probe",
+    "itexhip_qgemm_prepack_b", "itexhip_qgemm", "itexhip_qgemm_tile", "itexhip_qgemv", "itexhip_qmatmul", "itexhip_qmatmul_per_row", "itexhip_qmatmul_device_range", "itexhip_quantize_dynamic", "itexhip_quantize_dynamic_static", "itexhip_quantize_dynamic_rows", "itexhip_qmatmul_unpacked", "itexhip_mfma_probe", "itexhip_read_probe",
     "itexhip_qgemm_naive", "itexhip_qbatch_matmul", "itexhip_transpose", "itexhip_im2col8", "itexhip_scale_vector",
     "itexhip_qconv2d_implicit_ok", "itexhip_qconv2d", "itexhip_qgemm_sum", "itexhip_qconv2d_sum", "itexhip_qdepthwise_conv2d",
 ]
@@ -244,6 +244,10 @@ def qmatmul_device_range(p, a, packed_b, colsum, M, K, N, range_a, min_b, max_b,
 def quantize_dynamic(x, q, n, dst_type, mode, ensure_minimum_range, state, stream=0):
     _check(_lib.itexhip_quantize_dynamic(_ptr(x), _ptr(q), _i64(n), int(dst_type), int(mode),
                                          C.c_float(ensure_minimum_range), _ptr(state), _ptr(stream)))
+
+
+def read_probe(src, nbytes, sink, stream=0):
+    _check(_lib.itexhip_read_probe(_ptr(src), C.c_size_t(nbytes), _ptr(sink), _ptr(stream)))
 
 
 def quantize_dynamic_static(x, q, n, dst_type, mode, ensure_minimum_range, range_out, stream=0):
