@@ -53,12 +53,6 @@ static __device__ __align__(16) const uint32_t kZeroPiece[4] = {0u, 0u, 0u, 0u};
 // register operand, so the sign flip costs a 4-byte instruction per dword.  KALIGNED: K is a multiple
 // of 64, so activation loads never need a per-lane clamp and use a uniform base that advances by 64
 // bytes per step.
-#ifdef ITEXHIP_TILE_TRACE
-__device__ unsigned long long g_tile_trace[2048 * 8];
-#define TILE_T(i) do { if (threadIdx.x == 0 && blockIdx.x < 2048) g_tile_trace[blockIdx.x * 8 + (i)] = wall_clock64(); } while (0)
-#else
-#define TILE_T(i)
-#endif
 template <int BM, int BN, int WAVES_M, int WAVES_N, int OUT_T, int ACT, bool KALIGNED, bool CONV = false, bool ELEMENTWISE = false>
 __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void qgemm_tile_kernel(
     const uint8_t* __restrict__ a, uint32_t amask, const uint8_t* __restrict__ bp, int M, int K, int N,
@@ -91,7 +85,6 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void qgemm_tile_kernel(
   // byte offset from the window origin}
   constexpr int CONV_TAB_OFF = PANEL_OFF + 12 * BN;
 
-  TILE_T(0);
   extern __shared__ __align__(16) uint8_t lds[];
   const uint32_t lds_base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(
       (__attribute__((address_space(3))) void*)lds));
@@ -215,7 +208,6 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void qgemm_tile_kernel(
   }
   wait_vmcnt<NLD>();
   __syncthreads();
-  TILE_T(1);
   // the accumulators start from the zero-point compensation of their channel (exact in int32)
   static_for<TN>([&](auto j) {
     static_for<4>([&](auto g) {
@@ -306,7 +298,6 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void qgemm_tile_kernel(
   }
   wait_vmcnt<0>();  // no load may still be writing LDS when the epilogue reuses it
   __syncthreads();
-  TILE_T(2);
 
   // ---- epilogue.  Fast path: convert in registers, transpose through a private LDS buffer (the ring
   // is free after the last barrier) and store rows of 128 contiguous bytes, 16 B per lane.  A lane of
@@ -523,11 +514,6 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void qgemm_tile_kernel(
       });
     });
   }
-  TILE_T(3);
-#ifdef ITEXHIP_TILE_TRACE
-  wait_vmcnt<0>();
-  TILE_T(4);
-#endif
 }
 
 template <int BM, int BN, int WAVES_M, int WAVES_N, int OUT_T, int ACT, bool KALIGNED, bool CONV = false, bool ELEMENTWISE = false>

@@ -7,8 +7,3 @@ template int dispatch_tile<ITEXHIP_FLOAT>(const uint8_t*, uint32_t, const uint8_
 template int dispatch_tile_conv<ITEXHIP_FLOAT>(const uint8_t*, uint32_t, const uint8_t*, int, int, int, const EpilogueArgs&, void*,
                                     hipStream_t, const ConvTileArgs&);
 }  // namespace itexhip
-#ifdef ITEXHIP_TILE_TRACE
-extern "C" int itexhip_debug_tile_trace(void* host) {
-  return hipMemcpyFromSymbol(host, HIP_SYMBOL(itexhip::g_tile_trace), sizeof(itexhip::g_tile_trace)) == hipSuccess ? 0 : 13;
-}
-#endif
