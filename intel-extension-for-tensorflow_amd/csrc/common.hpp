@@ -120,8 +120,8 @@ __device__ __forceinline__ float apply_eltwise(const itexhip_eltwise& e, float x
       // 0.5 x (1 + tanh(u)), u = sqrt(2/pi) x (1 + 0.044715 x^2), evaluated as x / (1 + exp(-2u)): the same function
       // (1 + tanh(u) = 2 / (1 + exp(-2u))) at a fifth of the instructions of tanhf, within 4e-7 relative of it
       // (hardware exp2 and reciprocal, about 1 ulp each); exp overflows to inf only where the result is -0.
-      const float u = 0.79788458347320556640625f * x * (1.0f + 0.044715f * x * x);
-      const float e = __builtin_amdgcn_exp2f(u * -2.885390043258667f);  // exp(-2u) = 2^(-2u log2 e)
+      // exp(-2u) = 2^(x (c1 + c2 x^2)) with c1 = -2 sqrt(2/pi) log2(e), c2 = 0.044715 c1.
+      const float e = __builtin_amdgcn_exp2f(x * fmaf(x * x, -0.10294324159622192f, -2.3022081851959229f));
       return x * __builtin_amdgcn_rcpf(1.0f + e);
     }
     case ITEXHIP_ELT_GELU_ERF:  // 0.5 x (1 + erf(x / sqrt(2)))
