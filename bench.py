@@ -308,6 +308,20 @@ def bench_elementwise(torch, hip, timer, n, steps, warmup, dev):
     req = np.float32(1.0) * np.float32(amax) / np.float32(2.0 ** 31)
     rscale = float(np.float32(127.0) * (np.float32(1.0) / req / np.float32(2.0 ** 31)))
     add("requantize_int32_to_qint8", lambda i: hip.requantize(acc, q8, n, hip.QINT8, rscale, st), 5 * n)
+    # per-channel (per-axis) forms on a [4096, 14336] fp32 weight: the weight-quantization path; channels innermost
+    # (axis 1) and outermost (axis 0 of the transposed layout)
+    K, N = 4096, 14336
+    nw = K * N
+    if nw <= n:
+        w, wq = x[:nw], q8[:nw]
+        sc_n = torch.rand(N, device=dev, generator=g) * 50.0 + 10.0
+        sc_k = torch.rand(K, device=dev, generator=g) * 50.0 + 10.0
+        for name, fn in (("quantize_per_channel_axis1_4096x14336", lambda i: hip.quantize_axis(w, wq, K, N, 1, hip.QINT8, sc_n, None, st)),
+                         ("quantize_per_channel_axis0_4096x14336", lambda i: hip.quantize_axis(w, wq, 1, K, N, hip.QINT8, sc_k, None, st)),
+                         ("dequantize_per_channel_axis1_4096x14336", lambda i: hip.dequantize_axis(wq, w, K, N, 1, hip.QINT8, sc_n, None, st))):
+            ms = timer.run(fn, steps, warmup)
+            out.append(dict(name=name, n=nw, us_kernel=ms * 1e3, gbs=5 * nw / (ms * 1e-3) / 1e9, bytes=5 * nw,
+                            frac=5 * nw / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS))
     return out
 
 

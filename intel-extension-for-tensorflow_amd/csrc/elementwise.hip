@@ -84,6 +84,34 @@ __global__ __launch_bounds__(kThreads) void quantize_axis_kernel(const float* __
   }
 }
 
+// The same, 4 elements per lane, 32-bit index arithmetic (the host sends tensors of 2^32 groups or more, odd shapes
+// and unaligned buffers to the kernel above).  LAST: the quantized axis is the innermost one (inner == 1, slices a
+// multiple of 4): a lane's 4 elements are 4 consecutive slices, their parameters one 16-byte load each.  Otherwise
+// inner is a multiple of 4 and the 4 elements share a slice.  Same expression per element as above.
+template <int T, bool LAST>
+__global__ __launch_bounds__(kThreads) void quantize_axis_vec_kernel(const f4* __restrict__ x, uint32_t* __restrict__ q,
+                                                                     uint32_t n4, uint32_t slices, uint32_t inner4,
+                                                                     const float* __restrict__ scales,
+                                                                     const float* __restrict__ addends) {
+  const uint32_t i = blockIdx.x * kThreads + threadIdx.x;
+  if (i >= n4) return;
+  const f4 v = __builtin_nontemporal_load(&x[i]);
+  f4 sc, ad = {0.0f, 0.0f, 0.0f, 0.0f};
+  if constexpr (LAST) {
+    const uint32_t s4 = i % (slices >> 2);
+    sc = reinterpret_cast<const f4*>(scales)[s4];
+    if (addends) ad = reinterpret_cast<const f4*>(addends)[s4];
+  } else {
+    const uint32_t sl = (i / inner4) % slices;
+    const float c = scales[sl], a = addends ? addends[sl] : 0.0f;
+    sc = f4{c, c, c, c};
+    ad = f4{a, a, a, a};
+  }
+  const float a = v.x * sc.x, b = v.y * sc.y, c = v.z * sc.z, d = v.w * sc.w;
+  __builtin_nontemporal_store(pack4(sat_rne<T>(a + ad.x), sat_rne<T>(b + ad.y), sat_rne<T>(c + ad.z), sat_rne<T>(d + ad.w)),
+                              &q[i]);
+}
+
 // ------------------------------------------------------------------------------------------------
 // Dequantize: y = ((float)q - zp) * scale
 // ------------------------------------------------------------------------------------------------
@@ -139,6 +167,37 @@ __global__ __launch_bounds__(kThreads) void dequantize_axis_kernel(const uint8_t
                                          : static_cast<float>(q[i]);
     y[i] = (v - zp) * sc;
   }
+}
+
+// Per-slice dequantization, 4 elements per lane; LAST and the index arithmetic as in quantize_axis_vec_kernel.
+template <int T, bool LAST>
+__global__ __launch_bounds__(kThreads) void dequantize_axis_vec_kernel(const uint32_t* __restrict__ q, f4* __restrict__ y,
+                                                                       uint32_t n4, uint32_t slices, uint32_t inner4,
+                                                                       const float* __restrict__ scales,
+                                                                       const int32_t* __restrict__ zps) {
+  const uint32_t i = blockIdx.x * kThreads + threadIdx.x;
+  if (i >= n4) return;
+  const uint32_t w = __builtin_nontemporal_load(&q[i]);
+  f4 sc, zp = {0.0f, 0.0f, 0.0f, 0.0f};
+  if constexpr (LAST) {
+    const uint32_t s4 = i % (slices >> 2);
+    sc = reinterpret_cast<const f4*>(scales)[s4];
+    if (zps) {
+      const i4 z = reinterpret_cast<const i4*>(zps)[s4];
+      zp = f4{static_cast<float>(z.x), static_cast<float>(z.y), static_cast<float>(z.z), static_cast<float>(z.w)};
+    }
+  } else {
+    const uint32_t sl = (i / inner4) % slices;
+    const float c = scales[sl], z = zps ? static_cast<float>(zps[sl]) : 0.0f;
+    sc = f4{c, c, c, c};
+    zp = f4{z, z, z, z};
+  }
+  f4 r;
+  r.x = (widen<T>(w, 0) - zp.x) * sc.x;
+  r.y = (widen<T>(w, 1) - zp.y) * sc.y;
+  r.z = (widen<T>(w, 2) - zp.z) * sc.z;
+  r.w = (widen<T>(w, 3) - zp.w) * sc.w;
+  __builtin_nontemporal_store(r, &y[i]);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -777,6 +836,24 @@ extern "C" int itexhip_quantize_axis(const float* x, void* q, int64_t outer, int
   const int64_t n = outer * slices * inner;
   if (n == 0) return ITEXHIP_OK;
   ITEXHIP_REQUIRE(x && q && scales, "itexhip_quantize_axis: null buffer");
+  // 4 elements per lane when a group of 4 never straddles two slices in a way one 16-byte parameter load cannot follow
+  const bool last = inner == 1 && slices % 4 == 0 && aligned(scales, 16) && (!addends || aligned(addends, 16));
+  if ((last || inner % 4 == 0) && aligned(x, 16) && aligned(q, 4) && n / 4 < (1LL << 31) && slices < (1LL << 31)) {
+    const uint32_t n4 = static_cast<uint32_t>(n / 4), sl = static_cast<uint32_t>(slices), in4 = static_cast<uint32_t>(inner / 4);
+    const unsigned vgrid = blocks_for(n4, kThreads);
+    const f4* xv = reinterpret_cast<const f4*>(x);
+    uint32_t* qv = reinterpret_cast<uint32_t*>(q);
+    hipStream_t st = as_stream(stream);
+    if (dst_type == ITEXHIP_QINT8) {
+      if (last) quantize_axis_vec_kernel<ITEXHIP_QINT8, true><<<vgrid, kThreads, 0, st>>>(xv, qv, n4, sl, in4, scales, addends);
+      else quantize_axis_vec_kernel<ITEXHIP_QINT8, false><<<vgrid, kThreads, 0, st>>>(xv, qv, n4, sl, in4, scales, addends);
+    } else {
+      if (last) quantize_axis_vec_kernel<ITEXHIP_QUINT8, true><<<vgrid, kThreads, 0, st>>>(xv, qv, n4, sl, in4, scales, addends);
+      else quantize_axis_vec_kernel<ITEXHIP_QUINT8, false><<<vgrid, kThreads, 0, st>>>(xv, qv, n4, sl, in4, scales, addends);
+    }
+    ITEXHIP_CHECK_LAUNCH("itexhip_quantize_axis");
+    return ITEXHIP_OK;
+  }
   const unsigned grid = blocks_for(n, kThreads);
   if (dst_type == ITEXHIP_QINT8)
     quantize_axis_kernel<ITEXHIP_QINT8><<<grid, kThreads, 0, as_stream(stream)>>>(
@@ -831,6 +908,23 @@ extern "C" int itexhip_dequantize_axis(const void* q, float* y, int64_t outer, i
   const int64_t n = outer * slices * inner;
   if (n == 0) return ITEXHIP_OK;
   ITEXHIP_REQUIRE(q && y && scales, "itexhip_dequantize_axis: null buffer");
+  const bool last = inner == 1 && slices % 4 == 0 && aligned(scales, 16) && (!zero_points || aligned(zero_points, 16));
+  if ((last || inner % 4 == 0) && aligned(q, 4) && aligned(y, 16) && n / 4 < (1LL << 31) && slices < (1LL << 31)) {
+    const uint32_t n4 = static_cast<uint32_t>(n / 4), sl = static_cast<uint32_t>(slices), in4 = static_cast<uint32_t>(inner / 4);
+    const unsigned vgrid = blocks_for(n4, kThreads);
+    const uint32_t* qv = reinterpret_cast<const uint32_t*>(q);
+    f4* yv = reinterpret_cast<f4*>(y);
+    hipStream_t st = as_stream(stream);
+    if (src_type == ITEXHIP_QINT8) {
+      if (last) dequantize_axis_vec_kernel<ITEXHIP_QINT8, true><<<vgrid, kThreads, 0, st>>>(qv, yv, n4, sl, in4, scales, zero_points);
+      else dequantize_axis_vec_kernel<ITEXHIP_QINT8, false><<<vgrid, kThreads, 0, st>>>(qv, yv, n4, sl, in4, scales, zero_points);
+    } else {
+      if (last) dequantize_axis_vec_kernel<ITEXHIP_QUINT8, true><<<vgrid, kThreads, 0, st>>>(qv, yv, n4, sl, in4, scales, zero_points);
+      else dequantize_axis_vec_kernel<ITEXHIP_QUINT8, false><<<vgrid, kThreads, 0, st>>>(qv, yv, n4, sl, in4, scales, zero_points);
+    }
+    ITEXHIP_CHECK_LAUNCH("itexhip_dequantize_axis");
+    return ITEXHIP_OK;
+  }
   const unsigned grid = blocks_for(n, kThreads);
   if (src_type == ITEXHIP_QINT8)
     dequantize_axis_kernel<ITEXHIP_QINT8><<<grid, kThreads, 0, as_stream(stream)>>>(

@@ -198,6 +198,57 @@ def test_dequantize_golden(hip, dev, golden):
         np.testing.assert_array_equal(y, y_ref)
 
 
+# Shapes for the per-axis kernels: the axis innermost with a multiple of 4 slices (one 16-byte parameter load per
+# lane), inner a multiple of 4 (the lane's 4 elements share a slice), and shapes neither rule takes (element kernel).
+AXIS_CASES = [((768, 3072), 1), ((3, 5, 64), 2), ((3072, 768), 0), ((6, 5, 12), 1), ((7, 16, 4), 1), ((3, 3, 16, 8), 3),
+              ((5, 6), 1), ((4, 7, 3), 1), ((1, 4), 1), ((2, 1, 8), 1)]
+
+
+@pytest.mark.parametrize("T,mode,classic", [(orc.QINT8, orc.SCALED, False), (orc.QUINT8, orc.MIN_FIRST, True),
+                                            (orc.QUINT8, orc.MIN_FIRST, False)])
+@pytest.mark.parametrize("shape,axis", AXIS_CASES)
+def test_quantize_axis_vector_paths_vs_oracle(hip, dev, shape, axis, T, mode, classic):
+    rng = np.random.default_rng(sum(shape) * 7 + axis)
+    ns = shape[axis]
+    bshape = [1] * len(shape)
+    bshape[axis] = ns
+    spread = (0.05 + rng.random(ns) * 3).astype(np.float32)
+    x = (rng.standard_normal(shape) * spread.reshape(bshape)).astype(np.float32)
+    x.flat[::97] *= 40.0  # saturating values
+    x.flat[1::53] = np.rint(x.flat[1::53]) + np.float32(0.5)  # ties after scaling by powers of two
+    red = tuple(d for d in range(len(shape)) if d != axis)
+    mn = np.minimum(x.min(axis=red), 0).astype(np.float32) * np.float32(0.5)
+    mx = np.maximum(x.max(axis=red), 0).astype(np.float32) * np.float32(0.5)
+    st, q_ref, mn_ref, mx_ref = orc.quantize_v2(x, mn, mx, T, mode, axis=axis, classic=classic)
+    assert st == orc.OK
+    q, omn, omx = gpu_quantize(hip, dev, x, T, mode, mn, mx, axis=axis, classic=classic)
+    np.testing.assert_array_equal(q.view(np.uint8), np.asarray(q_ref).view(np.uint8).reshape(shape))
+    np.testing.assert_array_equal(omn, mn_ref)
+    np.testing.assert_array_equal(omx, mx_ref)
+
+
+@pytest.mark.parametrize("T,mode", [(orc.QINT8, orc.SCALED), (orc.QUINT8, orc.MIN_FIRST)])
+@pytest.mark.parametrize("shape,axis", AXIS_CASES)
+def test_dequantize_axis_vector_paths_vs_oracle(hip, dev, shape, axis, T, mode):
+    import torch
+    rng = np.random.default_rng(sum(shape) * 11 + axis)
+    ns = shape[axis]
+    q = rng.integers(0, 256, size=shape, dtype=np.uint8).view(np.int8 if T == orc.QINT8 else np.uint8)
+    mn = -(0.1 + rng.random(ns) * 5).astype(np.float32)
+    mx = (0.1 + rng.random(ns) * 7).astype(np.float32)
+    st, y_ref = orc.dequantize(q, mn, mx, T, mode, axis)
+    assert st == orc.OK
+    st, _, _, sc, zp = orc.scale_zeropoint_align(T, mode, True, mn, mx)
+    assert st == orc.OK
+    outer = int(np.prod(shape[:axis], dtype=np.int64))
+    inner = int(np.prod(shape[axis + 1:], dtype=np.int64))
+    y_d = torch.empty(shape, dtype=torch.float32, device=dev)
+    zp_d = torch.from_numpy(np.ascontiguousarray(zp, np.int32)).to(dev) if mode == orc.MIN_FIRST else None
+    hip.dequantize_axis(torch.from_numpy(q).to(dev), y_d, outer, ns, inner, T, torch.from_numpy(sc).to(dev), zp_d)
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(y_d.cpu().numpy(), np.asarray(y_ref).reshape(shape))
+
+
 @pytest.mark.parametrize("out_type", [orc.QINT8, orc.QUINT8])
 @pytest.mark.parametrize("shape", [(1, 1, 1, 1), (2, 3, 5, 7), (2, 4, 8, 64), (1, 1, 4096, 1), (1, 1, 1000, 3), (4, 8, 16, 256)])
 def test_requantize_per_channel_vs_oracle(hip, dev, out_type, shape):
