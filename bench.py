@@ -681,6 +681,15 @@ def main():
             mfma_probe_workload_data=sampler.run(torch, lambda: hip.mfma_probe(256, 200, wl, sink, st0)),
             mfma_probe_constant_operands=sampler.run(torch, lambda: hip.mfma_probe(256, 200, ones, sink, st0)),
             note="amdgpu sysfs (power1_input, pp_dpm_sclk) sampled every 50 ms over 1.5 s of back-to-back launches")
+        # the vendor library on the same int8 problem (hipBLASLt behind torch._int_mm, int32 output, no epilogue), as a
+        # point of comparison for rate and power: a measurement only, nothing of the product calls it
+        try:
+            a8 = (xq0 ^ 0x80).view(torch.int8).contiguous()
+            b8 = L0["wq"].contiguous()
+            torch._int_mm(a8, b8)
+            power["vendor_int8_gemm_torch_int_mm"] = sampler.run(torch, lambda: torch._int_mm(a8, b8))
+        except Exception as exc:  # not available in this PyTorch build
+            power["vendor_int8_gemm_torch_int_mm"] = dict(error=str(exc)[:200])
 
     cpu = None
     if not args.no_cpu:
