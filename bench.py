@@ -753,6 +753,13 @@ def main():
                          read_floor_us=floor["us_kernel"], frac_of_read_floor=floor["us_kernel"] / r["us_kernel"],
                          note="8 weight copies cycled (470 MB > last-level cache)")
                 others.append(r)
+            # a batched decode step of 32 rows: the small-M kernel in two blocks of 16 rows (the workgroups of a strip share
+            # its weights through one L2); the tile kernel would run 64 x 64 tiles over a fraction of the CUs here
+            r = bench_linear(torch, hip, timer, 32, k, n, "deq", K_steps, W, dev, seed=10, rotate=8, graph=True)
+            r.pop("_ctx")
+            r.update(name="decode_gemv_32_rows", bound="hbm", frac=r["gbs_kernel"] / PEAK_HBM_GBS,
+                     note="8 weight copies cycled; rows in blocks of 16")
+            others.append(r)
             others.append(bench_dynamic_linear(torch, hip, timer, 16, k, n, K_steps, W, dev, seed=10))
             r = bench_linear(torch, hip, timer, 16, k, n, "deq", K_steps, W, dev, seed=10, rotate=8, per_row=True)
             r.pop("_ctx")

@@ -283,8 +283,9 @@ int itexhip_qgemm_prepack_b(const int8_t* w, int transpose_b, int64_t K, int64_t
  * a_type QUINT8 | QINT8; out_type QINT32 | QINT8 | QUINT8 | FLOAT | BFLOAT16 | HALF.  `colsum` is needed for QUINT8
  * activations (they are fed to the signed MFMA as a-128 and corrected by 128*colsum[n]).
  * `scales` has ep->n_scales floats (may be NULL when 0), `bias` N floats (NULL = no bias add).
- * Dispatches to the bandwidth-bound small-M kernel for M <= 16 and to the MFMA tile kernel
- * otherwise; the two explicit entry points below force one path. */
+ * Dispatches to the bandwidth-bound small-M kernel (M <= 32; up to 128 rows when the weight is small or the tile
+ * kernel would leave most CUs idle) and to the MFMA tile kernel otherwise; both give the same bytes.  The two
+ * explicit entry points below force one path (itexhip_qgemv: M <= 128). */
 int itexhip_qgemm(const void* a, int a_type, const int8_t* packed_b, const int32_t* colsum,
                   int64_t M, int64_t K, int64_t N, const float* scales, const float* bias,
                   const itexhip_epilogue* ep, int out_type, void* out, void* stream);

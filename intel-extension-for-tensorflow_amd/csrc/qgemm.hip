@@ -69,8 +69,9 @@ __global__ __launch_bounds__(256) void prepack_b_kernel(const int8_t* __restrict
 }
 
 // ------------------------------------------------------------------------------------------------
-// Small-M kernel (M <= 16, bandwidth bound on the weight).  One workgroup owns a strip of 16 * NT output
-// channels (NT = 2: whole chunks; NT = 1: one half of each chunk, when N alone would not give every CU a
+// Small-M kernel (bandwidth bound on the weight).  One workgroup owns a strip of 16 * NT output channels and a block
+// of 16 rows (M <= 16: the whole problem's rows; up to 128 rows in 8 blocks, whose workgroups share the strip's
+// weights through one L2) (NT = 2: whole chunks; NT = 1: one half of each chunk, when N alone would not give every CU a
 // workgroup); its wavefronts split K into contiguous runs of chunk pairs (64 k each).  Per chunk pair a
 // wavefront needs NT weight fragments in the operand layout of the 16x16x64 MFMA (lane l: channel l % 16,
 // k-group l / 16; 4 runs of 256 contiguous bytes of the packed weight, loaded to registers) and one
@@ -91,7 +92,7 @@ __global__ __launch_bounds__(256) void prepack_b_kernel(const int8_t* __restrict
 constexpr int kGemvBatch = 4;                 // chunk pairs per batch
 constexpr int kGemvRing = 2 * kGemvBatch;     // activation slots of 1 KiB per wavefront
 
-template <int NT, int OUT_T>
+template <int NT, int OUT_T, bool ROW_BLOCKS>
 __global__ __launch_bounds__(576) void qgemv_kernel(const uint8_t* __restrict__ a, uint32_t a_xor,
                                                      const uint8_t* __restrict__ bp, int M, int K, int N,
                                                      int KC, int cnt, EpilogueArgs e,
@@ -100,7 +101,13 @@ __global__ __launch_bounds__(576) void qgemv_kernel(const uint8_t* __restrict__ 
   constexpr int U = kGemvBatch, RING = kGemvRing;
   constexpr int L = U * (NT + 1);  // loads per batch
   extern __shared__ __align__(16) uint8_t smem[];  // [waves][RING][1 KiB], then the parameter panel [3 or 6][SW]
-  const int strip = blockIdx.x;
+  // Workgroup -> (strip, block of 16 rows).  Consecutive workgroup ids go round robin to the 8 XCDs: the row blocks of
+  // a strip get ids 8 apart, so they run at the same time on the same XCD and its L2 fetches the strip's weights once.
+  // Grid with ROW_BLOCKS (M > 16): x = 8 * row blocks, y = groups of 8 strips (x runs fastest in launch order); the
+  // grid is padded to whole groups of 8 strips.  Without: one workgroup per strip.
+  const int strip = ROW_BLOCKS ? blockIdx.y * 8 + (blockIdx.x & 7) : blockIdx.x;
+  const int m_base = ROW_BLOCKS ? (blockIdx.x >> 3) * 16 : 0;
+  if (ROW_BLOCKS && strip * SW >= N) return;
   const int waves = (blockDim.x >> 6) - 1;  // streaming wavefronts; one more resolves the channel parameters
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const int lrow = lane & 15, lgrp = lane >> 4;  // fragment lane: row / channel, k-group 0..3 of the chunk pair
@@ -114,7 +121,7 @@ __global__ __launch_bounds__(576) void qgemv_kernel(const uint8_t* __restrict__ 
   // activation staging: lane -> (row q, piece j) of the 16 x 64 byte tile
   const int q = lane >> 2;
   const int dpiece = ((lane & 3) ^ ((q >> 1) & 3)) * 16;
-  const uint8_t* arow = a + static_cast<int64_t>(min(q, M - 1)) * K;
+  const uint8_t* arow = a + static_cast<int64_t>(min(m_base + q, M - 1)) * K;
   const int klast = K - 16;  // k beyond K meets zero weights: any in-bounds data will do
   uint8_t* const ring = smem + wave * (RING * 1024);
   const uint32_t frag_off = static_cast<uint32_t>((4 * lrow + (lgrp ^ ((lrow >> 1) & 3))) * 16);
@@ -235,12 +242,13 @@ __global__ __launch_bounds__(576) void qgemv_kernel(const uint8_t* __restrict__ 
     // accumulator layout of the 16x16 MFMA: lane l, register r -> m = l % 16, n = (l / 16) * 4 + r
     const bool vec_ok = (N & 3) == 0 && aligned16(out);
     const int col = wave * 16 + lgrp * 4, n = strip * SW + col;
-    if (lrow < M && n < N) {
+    const int m = m_base + lrow;
+    if (m < M && n < N) {
       ChannelParams cp;
       if (e.row_min_a) {
         PrepArgs pr = e.prep;
-        pr.min_a = e.row_min_a[lrow];
-        pr.max_a = e.row_max_a[lrow];
+        pr.min_a = e.row_min_a[m];
+        pr.max_a = e.row_max_a[m];
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
           const int colsum = panel[col + r];
@@ -260,7 +268,7 @@ __global__ __launch_bounds__(576) void qgemv_kernel(const uint8_t* __restrict__ 
           cp.bias[r] = __int_as_float(panel[2 * SW + col + r]);
         }
       }
-      epilogue_store<OUT_T, 2>(part, cp, lrow, n, M, N, e, out, vec_ok);
+      epilogue_store<OUT_T, 2>(part, cp, m, n, M, N, e, out, vec_ok);
     }
   }
 }
@@ -408,18 +416,20 @@ EpilogueArgs make_args(int a_type, const int32_t* colsum, const float* scales, c
 template <int NT, int OUT_T>
 int launch_gemv(const uint8_t* a, uint32_t a_xor, const uint8_t* bp, int M, int K, int N, int KC, int waves, int cnt,
                 const EpilogueArgs& e, void* out, hipStream_t st) {
-  auto kern = qgemv_kernel<NT, OUT_T>;
+  auto kern = M > 16 ? qgemv_kernel<NT, OUT_T, true> : qgemv_kernel<NT, OUT_T, false>;
   constexpr size_t lds_max = 8 * kGemvRing * 1024 + 6 * 16 * NT * 4;
-  static bool attr_set = false;  // benign race: the call is idempotent
-  if (!attr_set) {
+  static bool attr_set[2] = {false, false};  // benign race: the call is idempotent
+  if (!attr_set[M > 16]) {
     hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                                          static_cast<int>(lds_max));
     if (err != hipSuccess) return hip_fail(err, "hipFuncSetAttribute(qgemv_kernel)");
-    attr_set = true;
+    attr_set[M > 16] = true;
   }
   const size_t lds = static_cast<size_t>(waves) * kGemvRing * 1024 + 6 * 16 * NT * 4;
   const int strips = (N + 16 * NT - 1) / (16 * NT);
-  kern<<<strips, 64 * (waves + 1), lds, st>>>(a, a_xor, bp, M, K, N, KC, cnt, e, out);
+  const int rbs = (M + 15) / 16;
+  const dim3 grid = M > 16 ? dim3(8 * rbs, (strips + 7) / 8) : dim3(strips);
+  kern<<<grid, 64 * (waves + 1), lds, st>>>(a, a_xor, bp, M, K, N, KC, cnt, e, out);
   return ITEXHIP_OK;
 }
 
@@ -451,13 +461,26 @@ int dispatch_gemv(const uint8_t* a, uint32_t a_xor, const uint8_t* bp, int M, in
     default: st__ = CALL(ITEXHIP_QUINT8); break;                              \
   }
 
+// Which packed kernel takes a call.  The small-M kernel (a strip of channels x 16 rows x all of K per workgroup)
+// streams the weight once per block of 16 rows; the tile kernel needs enough 64 x 64 tiles to fill the device.
+// Measured on 4096 x 14336 / 14336 x 4096 weights (us, small-M against tile kernel): M = 32: 18 / 21 against 23 / 67;
+// M = 64: 29 / 34 against 23 / 68; M = 128: 49 / 57 against 28 / 67; on a 1024 x 1024 weight the small-M kernel takes
+// 3.5 against 4.8 up to M = 128.  Both kernels accumulate exactly and share the epilogue: the same bytes either way.
+constexpr int kSmallMaxRows = 128;
+static bool small_m(int64_t M, int64_t K, int64_t N) {
+  if (M <= 32) return true;
+  if (M > kSmallMaxRows) return false;
+  if (K * N <= (8LL << 20)) return true;                       // the weight stays in L2: launch-bound either way
+  return ((M + 63) / 64) * ((N + 63) / 64) <= 128;             // the tile kernel would leave half of the CUs idle
+}
+
 int launch_packed(bool gemv, const void* a, int a_type, const int8_t* packed_b, int64_t M, int64_t K, int64_t N,
                   const EpilogueArgs& e, int out_type, void* out, void* stream, const char* who) {
   ITEXHIP_REQUIRE(K % 16 == 0, "%s: K must be a multiple of 16 (got %lld); use itexhip_qgemm_naive", who,
                   static_cast<long long>(K));
   ITEXHIP_REQUIRE(aligned(a, 16) && aligned(packed_b, 16), "%s: operands must be 16-byte aligned", who);
   ITEXHIP_REQUIRE(a_type != ITEXHIP_QUINT8 || e.colsum, "%s: quint8 activations need colsum", who);
-  ITEXHIP_REQUIRE(!gemv || M <= 16, "%s: M must be <= 16", who);
+  ITEXHIP_REQUIRE(!gemv || M <= kSmallMaxRows, "%s: M must be <= %d", who, kSmallMaxRows);
   ITEXHIP_REQUIRE(M * K < (1LL << 31), "%s: activation matrix too large (M * K must be < 2^31)", who);
   const uint32_t a_xor = (a_type == ITEXHIP_QUINT8) ? 0x80808080u : 0u;
   const uint8_t* ap = reinterpret_cast<const uint8_t*>(a);
@@ -535,7 +558,7 @@ extern "C" int itexhip_qgemv(const void* a, int a_type, const int8_t* packed_b, 
 extern "C" int itexhip_qgemm(const void* a, int a_type, const int8_t* packed_b, const int32_t* colsum,
                              int64_t M, int64_t K, int64_t N, const float* scales, const float* bias,
                              const itexhip_epilogue* ep, int out_type, void* out, void* stream) {
-  return packed_path(M <= 16, a, a_type, packed_b, colsum, M, K, N, scales, bias, ep, out_type, out, stream,
+  return packed_path(small_m(M, K, N), a, a_type, packed_b, colsum, M, K, N, scales, bias, ep, out_type, out, stream,
                      "itexhip_qgemm");
 }
 
@@ -544,7 +567,7 @@ extern "C" int itexhip_qgemm_sum(const void* a, int a_type, const int8_t* packed
                                  const itexhip_epilogue* ep, const void* addend, int addend_type, int out_type, void* out,
                                  void* stream) {
   ITEXHIP_REQUIRE(addend != nullptr || M == 0 || N == 0, "itexhip_qgemm_sum: null addend");
-  return packed_path(M <= 16, a, a_type, packed_b, colsum, M, K, N, scales, bias, ep, out_type, out, stream,
+  return packed_path(small_m(M, K, N), a, a_type, packed_b, colsum, M, K, N, scales, bias, ep, out_type, out, stream,
                      "itexhip_qgemm_sum", addend, addend_type);
 }
 
@@ -692,7 +715,7 @@ int qmatmul_impl(const char* who, const itexhip_matmul_params* p, const void* a,
   e.range_a = range_a;
   e.addend = addend;
   e.addend_type = is_float16_type(p->t_out) ? p->t_out : ITEXHIP_FLOAT;  // the addend has the output's type
-  return launch_packed(M <= 16, a, p->t_in, packed_b, M, K, N, e, p->t_out, out, stream, who);
+  return launch_packed(small_m(M, K, N), a, p->t_in, packed_b, M, K, N, e, p->t_out, out, stream, who);
 }
 }  // namespace
 

@@ -47,7 +47,7 @@ def test_argument_validation_needs_no_gpu(hip):
         hip.qgemm(16, hip.QUINT8, 16, 16, 32, 3, 16, None, None, ep, hip.FLOAT, 16)
     assert "multiple of 16" in str(e.value)
     with pytest.raises(hip.ItexHipError):
-        hip.qgemv(16, hip.QUINT8, 16, 16, 17, 64, 16, None, None, ep, hip.FLOAT, 16)
+        hip.qgemv(16, hip.QUINT8, 16, 16, 129, 64, 16, None, None, ep, hip.FLOAT, 16)
     assert hip.qgemm_packed_bytes(4096, 14336) == 4096 * 14336
     assert hip.qgemm_packed_bytes(3, 4) == 2048
 

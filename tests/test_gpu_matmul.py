@@ -194,6 +194,22 @@ def test_tile_kernel_vs_oracle(hip, dev, M, K, N, kw):
     np.testing.assert_array_equal(layer.run(xq, kw, mn, mx, -r_out, r_out, path="fused"), ref)
 
 
+@pytest.mark.parametrize("M,K,N", [(17, 64, 16), (32, 4096, 1000), (33, 448, 528), (64, 1024, 100), (100, 256, 200),
+                                   (128, 1024, 1024), (127, 2048, 24), (48, 80, 2051)])
+@pytest.mark.parametrize("kw", [V2_DEQ_RELU, V2_REQ_S8, V2_REQ_U8_RELU, V1_S32])
+def test_small_m_kernel_in_row_blocks_vs_oracle(hip, dev, M, K, N, kw):
+    """17 .. 128 rows go through the small-M kernel in blocks of 16 rows (ragged last block, strips that do not fill a
+    group of 8, K not a multiple of 64): forced, through the dispatching entry point and as the single-launch op."""
+    layer, w, bias = make_layer(hip, dev, K, N, seed=K + N + 1)
+    x, xq, mn, mx = make_acts(M, K, seed=M + 3)
+    full = x @ w + bias
+    r_out = float(np.abs(np.maximum(full, 0) if kw.get("activation") else full).max())
+    lo = 0.0 if kw["t_out"] == orc.QUINT8 else -r_out
+    ref = layer.oracle(xq, kw, mn, mx, lo, r_out)
+    for path in ("gemv", "auto", "fused"):
+        np.testing.assert_array_equal(layer.run(xq, kw, mn, mx, lo, r_out, path=path), ref, err_msg=path)
+
+
 @pytest.mark.parametrize("kw", [V2_DEQ, V2_DEQ_RELU, V2_REQ_S8, V2_REQ_U8_RELU, V1_S32,
                                 dict(api=orc.API_V1, t_out=orc.QINT8, input_mode=orc.MIN_FIRST, n_fused_ops=1),
                                 dict(api=orc.API_LEGACY, t_out=orc.QUINT8, input_mode=orc.MIN_FIRST, activation=orc.ACT_RELU),
@@ -757,8 +773,8 @@ def test_bfloat16_output_vs_oracle(hip, dev, path, M, K, N, T16):
     """Tout = bfloat16 / half (_QuantizedMatMul, ...AndDequantize): bit patterns equal the oracle's on every kernel,
     with N odd / not a multiple of the 8-element vector store."""
     V2_DEQ_BF16 = dict(V2_DEQ, t_out=T16)
-    if path == "gemv" and M > 16:
-        pytest.skip("the small-M kernel takes M <= 16")
+    if path == "gemv" and M > 128:
+        pytest.skip("the small-M kernel takes M <= 128")
     layer, w, bias = make_layer(hip, dev, K, N, seed=K + N)
     x, xq, mn, mx = make_acts(M, K, seed=M + 1)
     for kw in (V2_DEQ_BF16, dict(V2_DEQ_BF16, activation=orc.ACT_RELU)):
