@@ -70,8 +70,8 @@ __global__ __launch_bounds__(256) void prepack_b_kernel(const int8_t* __restrict
 
 // ------------------------------------------------------------------------------------------------
 // Small-M kernel (bandwidth bound on the weight).  One workgroup owns a strip of 16 * NT output channels and a block
-// of 16 rows (M <= 16: the whole problem's rows; up to 128 rows in 8 blocks, whose workgroups share the strip's
-// weights through one L2) (NT = 2: whole chunks; NT = 1: one half of each chunk, when N alone would not give every CU a
+// of 16 R rows (M <= 16: R = 1, the whole problem's rows; up to 128 rows in blocks of 32, R = 2, whose workgroups
+// share the strip's weights through one L2) (NT = 2: whole chunks; NT = 1: one half of each chunk, when N alone would not give every CU a
 // workgroup); its wavefronts split K into contiguous runs of chunk pairs (64 k each).  Per chunk pair a
 // wavefront needs NT weight fragments in the operand layout of the 16x16x64 MFMA (lane l: channel l % 16,
 // k-group l / 16; 4 runs of 256 contiguous bytes of the packed weight, loaded to registers) and one
@@ -92,22 +92,24 @@ __global__ __launch_bounds__(256) void prepack_b_kernel(const int8_t* __restrict
 constexpr int kGemvBatch = 4;                 // chunk pairs per batch
 constexpr int kGemvRing = 2 * kGemvBatch;     // activation slots of 1 KiB per wavefront
 
-template <int NT, int OUT_T, bool ROW_BLOCKS>
+template <int NT, int OUT_T, int R>
 __global__ __launch_bounds__(576) void qgemv_kernel(const uint8_t* __restrict__ a, uint32_t a_xor,
                                                      const uint8_t* __restrict__ bp, int M, int K, int N,
                                                      int KC, int cnt, EpilogueArgs e,
                                                      void* __restrict__ out) {
   constexpr int SW = 16 * NT;
   constexpr int U = kGemvBatch, RING = kGemvRing;
-  constexpr int L = U * (NT + 1);  // loads per batch
-  extern __shared__ __align__(16) uint8_t smem[];  // [waves][RING][1 KiB], then the parameter panel [3 or 6][SW]
-  // Workgroup -> (strip, block of 16 rows).  Consecutive workgroup ids go round robin to the 8 XCDs: the row blocks of
-  // a strip get ids 8 apart, so they run at the same time on the same XCD and its L2 fetches the strip's weights once.
-  // Grid with ROW_BLOCKS (M > 16): x = 8 * row blocks, y = groups of 8 strips (x runs fastest in launch order); the
-  // grid is padded to whole groups of 8 strips.  Without: one workgroup per strip.
-  const int strip = ROW_BLOCKS ? blockIdx.y * 8 + (blockIdx.x & 7) : blockIdx.x;
-  const int m_base = ROW_BLOCKS ? (blockIdx.x >> 3) * 16 : 0;
-  if (ROW_BLOCKS && strip * SW >= N) return;
+  constexpr int L = U * (NT + R);  // loads per batch
+  constexpr int ROWS = 16 * R;     // activation rows per workgroup
+  extern __shared__ __align__(16) uint8_t smem[];  // [waves][RING][R][1 KiB], then the parameter panel [3 or 6][SW]
+  // R = 1 (M <= 16): one workgroup per strip.  R = 2 (M > 16): a workgroup takes 32 rows of a strip - every weight
+  // fragment meets two activation fragments - and the grid is x = 8 * row blocks, y = groups of 8 strips (x runs
+  // fastest in launch order, consecutive workgroup ids go round robin to the 8 XCDs): the row blocks of a strip get
+  // ids 8 apart, so they run at the same time on the same XCD and its L2 fetches the strip's weights once.  The grid
+  // is padded to whole groups of 8 strips.
+  const int strip = R > 1 ? blockIdx.y * 8 + (blockIdx.x & 7) : blockIdx.x;
+  const int m_base = R > 1 ? (blockIdx.x >> 3) * ROWS : 0;
+  if (R > 1 && strip * SW >= N) return;
   const int waves = (blockDim.x >> 6) - 1;  // streaming wavefronts; one more resolves the channel parameters
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const int lrow = lane & 15, lgrp = lane >> 4;  // fragment lane: row / channel, k-group 0..3 of the chunk pair
@@ -121,30 +123,38 @@ __global__ __launch_bounds__(576) void qgemv_kernel(const uint8_t* __restrict__ 
   // activation staging: lane -> (row q, piece j) of the 16 x 64 byte tile
   const int q = lane >> 2;
   const int dpiece = ((lane & 3) ^ ((q >> 1) & 3)) * 16;
-  const uint8_t* arow = a + static_cast<int64_t>(min(m_base + q, M - 1)) * K;
+  const uint8_t* arow[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) arow[r] = a + static_cast<int64_t>(min(m_base + 16 * r + q, M - 1)) * K;
   const int klast = K - 16;  // k beyond K meets zero weights: any in-bounds data will do
-  uint8_t* const ring = smem + wave * (RING * 1024);
+  uint8_t* const ring = smem + wave * (RING * R * 1024);
   const uint32_t frag_off = static_cast<uint32_t>((4 * lrow + (lgrp ^ ((lrow >> 1) & 3))) * 16);
 
-  v4i acc[NT];
+  v4i acc[R][NT];
 #pragma unroll
-  for (int t = 0; t < NT; ++t) acc[t] = v4i{0, 0, 0, 0};
+  for (int r = 0; r < R; ++r)
+#pragma unroll
+    for (int t = 0; t < NT; ++t) acc[r][t] = v4i{0, 0, 0, 0};
 
-  int* const panel = reinterpret_cast<int*>(smem + waves * (RING * 1024));
+  int* const panel = reinterpret_cast<int*>(smem + waves * (RING * R * 1024));
 
   // Batches that lie entirely inside the wavefront's run and inside K take their addresses from two running per-lane
   // pointers plus constants; the last, ragged batch clamps every pair (a pair past the end is loaded from a valid
   // address and not used).
   const uint8_t* wptr = wsrc + static_cast<int64_t>(p0) * (2 * kChunkBytes);
-  const uint8_t* aptr = arow + dpiece + static_cast<int64_t>(p0) * 64;
+  const uint8_t* aptr[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) aptr[r] = arow[r] + dpiece + static_cast<int64_t>(p0) * 64;
   const int p_full = min(p1, K >> 6);  // pairs below this index lie entirely inside K
   auto issue = [&](int pb, int slot0, v4i (&w)[U][NT]) {
     if (pb + U <= p_full) {
 #pragma unroll
       for (int u = 0; u < U; ++u)
-        // the builtin, not inline assembly: the compiler's own vmcnt bookkeeping for the weight loads must see these
-        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(aptr + u * 64),
-                                         (__attribute__((address_space(3))) void*)(ring + (slot0 + u) * 1024), 16, 0, 0);
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+          // the builtin, not inline assembly: the compiler's own vmcnt bookkeeping for the weight loads must see these
+          __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(aptr[r] + u * 64),
+                                           (__attribute__((address_space(3))) void*)(ring + ((slot0 + u) * R + r) * 1024), 16, 0, 0);
 #pragma unroll
       for (int u = 0; u < U; ++u)
 #pragma unroll
@@ -154,9 +164,11 @@ __global__ __launch_bounds__(576) void qgemv_kernel(const uint8_t* __restrict__ 
 #pragma unroll
       for (int u = 0; u < U; ++u) {
         const int p = min(pb + u, KP - 1);
-        __builtin_amdgcn_global_load_lds(
-            (const __attribute__((address_space(1))) void*)(arow + min(p * 64 + dpiece, klast)),
-            (__attribute__((address_space(3))) void*)(ring + (slot0 + u) * 1024), 16, 0, 0);
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+          __builtin_amdgcn_global_load_lds(
+              (const __attribute__((address_space(1))) void*)(arow[r] + min(p * 64 + dpiece, klast)),
+              (__attribute__((address_space(3))) void*)(ring + ((slot0 + u) * R + r) * 1024), 16, 0, 0);
       }
 #pragma unroll
       for (int u = 0; u < U; ++u) {
@@ -168,17 +180,21 @@ __global__ __launch_bounds__(576) void qgemv_kernel(const uint8_t* __restrict__ 
       }
     }
     wptr += U * (2 * kChunkBytes);
-    aptr += U * 64;
+#pragma unroll
+    for (int r = 0; r < R; ++r) aptr[r] += U * 64;
     __builtin_amdgcn_sched_barrier(0);
   };
   auto compute = [&](int pb, int slot0, const v4i (&w)[U][NT]) {
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       if (pb + u < p1) {  // wavefront uniform
-        v4i x = *reinterpret_cast<const v4i*>(ring + (slot0 + u) * 1024 + frag_off);
-        x.x ^= a_xor; x.y ^= a_xor; x.z ^= a_xor; x.w ^= a_xor;
 #pragma unroll
-        for (int t = 0; t < NT; ++t) acc[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w[u][t], x, acc[t], 0, 0, 0);
+        for (int r = 0; r < R; ++r) {
+          v4i x = *reinterpret_cast<const v4i*>(ring + ((slot0 + u) * R + r) * 1024 + frag_off);
+          x.x ^= a_xor; x.y ^= a_xor; x.z ^= a_xor; x.w ^= a_xor;
+#pragma unroll
+          for (int t = 0; t < NT; ++t) acc[r][t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w[u][t], x, acc[r][t], 0, 0, 0);
+        }
       }
     }
     __builtin_amdgcn_sched_barrier(0);
@@ -232,17 +248,21 @@ __global__ __launch_bounds__(576) void qgemv_kernel(const uint8_t* __restrict__ 
     }
     // partial tiles -> the wavefront's own ring (its loads have landed and its reads are done)
 #pragma unroll
-    for (int t = 0; t < NT; ++t) *reinterpret_cast<v4i*>(ring + t * 1024 + lane * 16) = acc[t];
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+      for (int t = 0; t < NT; ++t) *reinterpret_cast<v4i*>(ring + (r * NT + t) * 1024 + lane * 16) = acc[r][t];
   }
   // cross-wavefront reduction through the rings
   __syncthreads();
-  if (wave < NT) {
+  // the R * NT tiles of 16 x 16 go round the wavefronts (R = 1: wavefront t finishes tile t)
+  for (int tile = wave; tile < R * NT; tile += waves + 1) {
+    const int tr = tile / NT, tc = tile - tr * NT;
     v4i part = v4i{0, 0, 0, 0};
-    for (int w = 0; w < waves; ++w) part += *reinterpret_cast<const v4i*>(smem + w * (RING * 1024) + wave * 1024 + lane * 16);
+    for (int w = 0; w < waves; ++w) part += *reinterpret_cast<const v4i*>(smem + w * (RING * R * 1024) + tile * 1024 + lane * 16);
     // accumulator layout of the 16x16 MFMA: lane l, register r -> m = l % 16, n = (l / 16) * 4 + r
     const bool vec_ok = (N & 3) == 0 && aligned16(out);
-    const int col = wave * 16 + lgrp * 4, n = strip * SW + col;
-    const int m = m_base + lrow;
+    const int col = tc * 16 + lgrp * 4, n = strip * SW + col;
+    const int m = m_base + 16 * tr + lrow;
     if (m < M && n < N) {
       ChannelParams cp;
       if (e.row_min_a) {
@@ -416,8 +436,9 @@ EpilogueArgs make_args(int a_type, const int32_t* colsum, const float* scales, c
 template <int NT, int OUT_T>
 int launch_gemv(const uint8_t* a, uint32_t a_xor, const uint8_t* bp, int M, int K, int N, int KC, int waves, int cnt,
                 const EpilogueArgs& e, void* out, hipStream_t st) {
-  auto kern = M > 16 ? qgemv_kernel<NT, OUT_T, true> : qgemv_kernel<NT, OUT_T, false>;
-  constexpr size_t lds_max = 8 * kGemvRing * 1024 + 6 * 16 * NT * 4;
+  auto kern = M > 16 ? qgemv_kernel<NT, OUT_T, 2> : qgemv_kernel<NT, OUT_T, 1>;
+  const int R = M > 16 ? 2 : 1;
+  const size_t lds_max = static_cast<size_t>(8 * kGemvRing * 1024) * R + 6 * 16 * NT * 4;
   static bool attr_set[2] = {false, false};  // benign race: the call is idempotent
   if (!attr_set[M > 16]) {
     hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -425,9 +446,9 @@ int launch_gemv(const uint8_t* a, uint32_t a_xor, const uint8_t* bp, int M, int 
     if (err != hipSuccess) return hip_fail(err, "hipFuncSetAttribute(qgemv_kernel)");
     attr_set[M > 16] = true;
   }
-  const size_t lds = static_cast<size_t>(waves) * kGemvRing * 1024 + 6 * 16 * NT * 4;
+  const size_t lds = static_cast<size_t>(waves) * kGemvRing * 1024 * R + 6 * 16 * NT * 4;
   const int strips = (N + 16 * NT - 1) / (16 * NT);
-  const int rbs = (M + 15) / 16;
+  const int rbs = (M + 31) / 32;  // row blocks of the R = 2 kernel
   const dim3 grid = M > 16 ? dim3(8 * rbs, (strips + 7) / 8) : dim3(strips);
   kern<<<grid, 64 * (waves + 1), lds, st>>>(a, a_xor, bp, M, K, N, KC, cnt, e, out);
   return ITEXHIP_OK;
@@ -463,9 +484,9 @@ int dispatch_gemv(const uint8_t* a, uint32_t a_xor, const uint8_t* bp, int M, in
 
 // Which packed kernel takes a call.  The small-M kernel (a strip of channels x 16 rows x all of K per workgroup)
 // streams the weight once per block of 16 rows; the tile kernel needs enough 64 x 64 tiles to fill the device.
-// Measured on 4096 x 14336 / 14336 x 4096 weights (us, small-M against tile kernel): M = 32: 18 / 21 against 23 / 67;
-// M = 64: 29 / 34 against 23 / 68; M = 128: 49 / 57 against 28 / 67; on a 1024 x 1024 weight the small-M kernel takes
-// 3.5 against 4.8 up to M = 128.  Both kernels accumulate exactly and share the epilogue: the same bytes either way.
+// Measured on 4096 x 14336 / 14336 x 4096 weights (us, small-M against tile kernel): M = 32: 15 / 17 against 23 / 67;
+// M = 64: 23 / 29 against 23 / 68; M = 128: 40 / 50 against 28 / 67; on a 1024 x 1024 weight the small-M kernel takes
+// 3.6 against 4.8 up to M = 128.  Both kernels accumulate exactly and share the epilogue: the same bytes either way.
 constexpr int kSmallMaxRows = 128;
 static bool small_m(int64_t M, int64_t K, int64_t N) {
   if (M <= 32) return true;
