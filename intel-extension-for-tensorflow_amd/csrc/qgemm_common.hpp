@@ -145,6 +145,48 @@ __device__ __forceinline__ RawChannel load_raw_channel(const EpilogueArgs& e, in
   return r;
 }
 
+// The same loads as load_raw_channel, written as assembly so that the compiler neither sees them nor waits for them:
+// a kernel issues them, then a long run of global -> LDS loads (assembly as well), waits itself until only those are
+// outstanding (vector memory loads return in the order issued) and calls settle_raw_channel before it touches a value.
+__device__ __forceinline__ uint32_t early_load32(const void* p) {
+  uint32_t v;
+  asm volatile("global_load_dword %0, %1, off" : "=&v"(v) : "v"(p) : "memory");
+  return v;
+}
+__device__ __forceinline__ uint32_t early_load16(const void* p) {
+  uint32_t v;
+  asm volatile("global_load_ushort %0, %1, off" : "=&v"(v) : "v"(p) : "memory");
+  return v;
+}
+constexpr int kEarlyChannelLoads = 6;  // at most: colsum, bias, four weight-range entries
+__device__ __forceinline__ RawChannel load_raw_channel_early(const EpilogueArgs& e, int n, int N) {
+  RawChannel r;
+  r.colsum = 0;
+  r.bias = 0u;
+  r.min_bj = 1.0f;
+  r.max_bj = r.min_b0 = r.max_b0 = 0.0f;
+  uint32_t t;
+  if (e.colsum) r.colsum = static_cast<int>(early_load32(e.colsum + n));
+  if (e.bias) {
+    if (e.fused && e.prep.bias_16 != 0) r.bias = early_load16(static_cast<const uint16_t*>(e.bias) + n);
+    else r.bias = early_load32(static_cast<const uint32_t*>(e.bias) + n);
+  }
+  if (e.fused) {
+    const int jb = (e.nb == N) ? n : 0;
+    t = early_load32(e.min_b + jb); r.min_bj = __uint_as_float(t);
+    t = early_load32(e.max_b + jb); r.max_bj = __uint_as_float(t);
+    t = early_load32(e.min_b); r.min_b0 = __uint_as_float(t);
+    t = early_load32(e.max_b); r.max_b0 = __uint_as_float(t);
+  } else if (e.n_scales >= 1) {
+    t = early_load32(e.scales + (e.n_scales > 1 ? n : 0)); r.min_bj = __uint_as_float(t);
+  }
+  return r;
+}
+// after the kernel's own wait: ties every later use of the values to this point of the instruction stream
+__device__ __forceinline__ void settle_raw_channel(RawChannel& r) {
+  asm volatile("" : "+v"(r.min_bj), "+v"(r.max_bj), "+v"(r.min_b0), "+v"(r.max_b0), "+v"(r.bias), "+v"(r.colsum));
+}
+
 __device__ __forceinline__ void finish_channel(const EpilogueArgs& e, const RawChannel& r, int* comp, float* scale,
                                                float* bias) {
   *comp = e.comp_mul * r.colsum;

@@ -219,20 +219,26 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void qgemm_tile_kernel(
     return *reinterpret_cast<const v4i*>(lds + stage * STAGE_BYTES + B_REGION + ((wn * TN + j) * 2 + kc) * kChunkBytes + lane * 16);
   };
 
-  // ---- prologue: loads of steps 0, 1, 2 in flight; wait for steps 0 and 1
+  // ---- prologue.  First the few loads of the channel parameters (thread t resolves channel n_base + t once, so the
+  // epilogue is free of global loads and of branches on them), then the operand loads of steps 0, 1, 2.  Loads return
+  // in the order issued: the parameters are there when only the operand loads are outstanding, and their arithmetic
+  // runs while those travel.
+  static_assert(kEarlyChannelLoads + 3 * NLD < 64, "vmcnt budget of the prologue");
+  const bool panel_thread = threadIdx.x < BN;
+  RawChannel raw;
+  if (panel_thread) raw = load_raw_channel_early(e, min(n_base + static_cast<int>(threadIdx.x), N - 1), N);
   {
     const int2 p0 = conv_piece(0), p1 = conv_piece(min(1, KT - 1)), p2 = conv_piece(min(2, KT - 1));
     static_for<NLD>([&](auto c) { issue_load(c, 0, 0, p0); });
     static_for<NLD>([&](auto c) { issue_load(c, min(1, KT - 1), 1, p1); });
     static_for<NLD>([&](auto c) { issue_load(c, min(2, KT - 1), 2, p2); });
   }
-  // parameter panel: thread t resolves channel n_base + t once (the flags are uniform), so the
-  // epilogue is free of global loads and of branches on them
-  if (threadIdx.x < BN) {
-    const int n = min(n_base + static_cast<int>(threadIdx.x), N - 1);
+  wait_vmcnt<3 * NLD>();
+  if (panel_thread) {
+    settle_raw_channel(raw);
     int comp;
     float scale, bias;
-    resolve_channel(e, n, N, &comp, &scale, &bias);
+    finish_channel(e, raw, &comp, &scale, &bias);
     panel_comp[threadIdx.x] = comp;
     panel_scale[threadIdx.x] = scale;
     panel_bias[threadIdx.x] = bias;
