@@ -122,6 +122,7 @@ struct RawChannel {
   float min_bj, max_bj, min_b0, max_b0;  // fused: weight ranges;  else min_bj holds the prepared scale
   uint32_t bias;                         // fused: the raw bias entry as loaded;  else the bits of the prepared fp32 bias
   int colsum;
+  float min_a, max_a;                    // load_raw_channel_early only: the activation range the call runs with
 };
 
 // Only loads, all of them per-lane vector loads that nothing waits for here: a wavefront can issue them ahead of a
@@ -158,13 +159,13 @@ __device__ __forceinline__ uint32_t early_load16(const void* p) {
   asm volatile("global_load_ushort %0, %1, off" : "=&v"(v) : "v"(p) : "memory");
   return v;
 }
-constexpr int kEarlyChannelLoads = 6;  // at most: colsum, bias, four weight-range entries
+constexpr int kEarlyChannelLoads = 8;  // at most: colsum, bias, four weight-range entries, the activation range
 __device__ __forceinline__ RawChannel load_raw_channel_early(const EpilogueArgs& e, int n, int N) {
   RawChannel r;
   r.colsum = 0;
   r.bias = 0u;
   r.min_bj = 1.0f;
-  r.max_bj = r.min_b0 = r.max_b0 = 0.0f;
+  r.max_bj = r.min_b0 = r.max_b0 = r.min_a = r.max_a = 0.0f;
   uint32_t t;
   if (e.colsum) r.colsum = static_cast<int>(early_load32(e.colsum + n));
   if (e.bias) {
@@ -177,6 +178,12 @@ __device__ __forceinline__ RawChannel load_raw_channel_early(const EpilogueArgs&
     t = early_load32(e.max_b + jb); r.max_bj = __uint_as_float(t);
     t = early_load32(e.min_b); r.min_b0 = __uint_as_float(t);
     t = early_load32(e.max_b); r.max_b0 = __uint_as_float(t);
+    r.min_a = e.prep.min_a;
+    r.max_a = e.prep.max_a;
+    if (e.range_a) {  // the range left in device memory by a dynamic quantization
+      t = early_load32(e.range_a); r.min_a = __uint_as_float(t);
+      t = early_load32(e.range_a + 1); r.max_a = __uint_as_float(t);
+    }
   } else if (e.n_scales >= 1) {
     t = early_load32(e.scales + (e.n_scales > 1 ? n : 0)); r.min_bj = __uint_as_float(t);
   }
@@ -184,7 +191,25 @@ __device__ __forceinline__ RawChannel load_raw_channel_early(const EpilogueArgs&
 }
 // after the kernel's own wait: ties every later use of the values to this point of the instruction stream
 __device__ __forceinline__ void settle_raw_channel(RawChannel& r) {
-  asm volatile("" : "+v"(r.min_bj), "+v"(r.max_bj), "+v"(r.min_b0), "+v"(r.max_b0), "+v"(r.bias), "+v"(r.colsum));
+  asm volatile("" : "+v"(r.min_bj), "+v"(r.max_bj), "+v"(r.min_b0), "+v"(r.max_b0), "+v"(r.bias), "+v"(r.colsum), "+v"(r.min_a),
+               "+v"(r.max_a));
+}
+// finish_channel for values that load_raw_channel_early brought: no load of its own
+__device__ __forceinline__ void finish_channel_early(const EpilogueArgs& e, const RawChannel& r, int* comp, float* scale,
+                                                     float* bias) {
+  *comp = e.comp_mul * r.colsum;
+  if (e.fused) {
+    PrepArgs pr = e.prep;
+    pr.min_a = r.min_a;
+    pr.max_a = r.max_a;
+    const ChannelScaleBias c = channel_scale_bias(pr, r.min_bj, r.max_bj, r.min_b0, r.max_b0, bias_from_bits(e.prep, r.bias),
+                                                  r.colsum);
+    *scale = e.n_scales > 0 ? c.scale : 1.0f;
+    *bias = c.bias;
+  } else {
+    *scale = r.min_bj;
+    *bias = __uint_as_float(r.bias);
+  }
 }
 
 __device__ __forceinline__ void finish_channel(const EpilogueArgs& e, const RawChannel& r, int* comp, float* scale,

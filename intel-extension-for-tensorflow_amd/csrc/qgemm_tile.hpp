@@ -238,7 +238,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void qgemm_tile_kernel(
     settle_raw_channel(raw);
     int comp;
     float scale, bias;
-    finish_channel(e, raw, &comp, &scale, &bias);
+    finish_channel_early(e, raw, &comp, &scale, &bias);
     panel_comp[threadIdx.x] = comp;
     panel_scale[threadIdx.x] = scale;
     panel_bias[threadIdx.x] = bias;
