@@ -44,7 +44,7 @@ namespace itexhip {
 // How the tile grid is dealt to the 8 XCDs (each with an L2 of its own).  0: every XCD takes a contiguous range of
 // tiles, m fastest.  When the grid fits the device in one round and such a range would pull more operand bytes
 // through one L2 than it keeps (3 of its 4 MB), the grid is cut into gm x (8 / gm) rectangles of tiles instead, one
-// per XCD, as square in bytes as the divisors of the grid allow; the result is gm.  Below that size the contiguous
+// per XCD, as square in bytes as the divisors of the grid allow; the result describes the rectangles (see below).  Below that size the contiguous
 // range measured faster (BERT-base 768 -> 768 at 4096 tokens: 7.2 against 7.9 us), above it the rectangles
 // (3072 -> 768: 15.4 against 18.7 us).
 inline int xcd_rectangles(int num_m, int num_n, int BM, int BN, int K) {
@@ -59,7 +59,13 @@ inline int xcd_rectangles(int num_m, int num_n, int BM, int BN, int K) {
     const int cost = (num_m / g) * BM + (num_n / gn) * BN;
     if (cost < best) { best = cost; gm = g; }
   }
-  return gm;
+  if (gm == 0) return 0;
+  // what the kernel needs, packed: log2(gm) + 1, the rectangle's extent in tiles (sm x sn, each <= 32 because the grid
+  // has at most 256 tiles) and ceil(2^12 / sm) for its division by sm
+  const int sm = num_m / gm, sn = num_n / (8 / gm);
+  int lg = 0;
+  while ((1 << lg) < gm) ++lg;
+  return (lg + 1) | (sm << 3) | (sn << 9) | (((4096 + sm - 1) / sm) << 15);
 }
 
 // Implicit GEMM of a Conv2D (NHWC input, in_c a multiple of 16): the activation "matrix" is the patch matrix
@@ -116,10 +122,12 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void qgemm_tile_kernel(
   // xcd_gm != 0 (see xcd_rectangles) the tile grid is cut into xcd_gm x (8 / xcd_gm) rectangles, one per XCD.
   int pid = blockIdx.x;
   int tile_m, tile_n;
-  if (xcd_gm != 0) {
-    const int sm = num_m / xcd_gm, sn = num_n / (8 / xcd_gm), xcd = pid & 7, local = pid >> 3;
-    tile_m = (xcd % xcd_gm) * sm + local % sm;
-    tile_n = (xcd / xcd_gm) * sn + local / sm;
+  if (xcd_gm != 0) {  // packed by xcd_rectangles: no division here, the first operand loads wait for this arithmetic
+    const int lg = (xcd_gm & 7) - 1, sm = (xcd_gm >> 3) & 63, sn = (xcd_gm >> 9) & 63, inv = xcd_gm >> 15;
+    const int xcd = pid & 7, local = pid >> 3;
+    const int ln = (local * inv) >> 12;  // local / sm, exact for local, sm <= 32
+    tile_m = (xcd & ((1 << lg) - 1)) * sm + (local - ln * sm);
+    tile_n = (xcd >> lg) * sn + ln;
   } else {
     const int total = num_m * num_n;
     if ((total & 7) == 0) pid = (pid & 7) * (total >> 3) + (pid >> 3);
