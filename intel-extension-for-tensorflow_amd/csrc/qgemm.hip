@@ -91,6 +91,7 @@ __global__ __launch_bounds__(256) void prepack_b_kernel(const int8_t* __restrict
 // ------------------------------------------------------------------------------------------------
 constexpr int kGemvBatch = 4;                 // chunk pairs per batch
 constexpr int kGemvRing = 2 * kGemvBatch;     // activation slots of 1 KiB per wavefront
+constexpr int kGemvPanelWords = 6 + 32;       // per channel of the strip: 6 parameter words + {scale, bias} of 16 rows
 
 template <int NT, int OUT_T, int R>
 __global__ __launch_bounds__(576) void qgemv_kernel(const uint8_t* __restrict__ a, uint32_t a_xor,
@@ -101,6 +102,11 @@ __global__ __launch_bounds__(576) void qgemv_kernel(const uint8_t* __restrict__ 
   constexpr int U = kGemvBatch, RING = kGemvRing;
   constexpr int L = U * (NT + R);  // loads per batch
   constexpr int ROWS = 16 * R;     // activation rows per workgroup
+  // Per-row activation ranges (M <= 16): with 16-channel strips the parameter wavefront works out scale and bias of
+  // every (row, channel) while the others stream and the epilogue reads a table (14336 -> 4096, M = 16: 14.9 -> 13.9 us);
+  // with 32-channel strips (4 streaming wavefronts, shorter streams, twice the pairs) that wavefront finished last
+  // (13.9 -> 14.9 us), so there the two finishing wavefronts do the arithmetic in the epilogue.
+  constexpr bool ROW_TABLE = (NT == 1);
   extern __shared__ __align__(16) uint8_t smem[];  // [waves][RING][R][1 KiB], then the parameter panel [3 or 6][SW]
   // R = 1 (M <= 16): one workgroup per strip.  R = 2 (M > 16): a workgroup takes 32 rows of a strip - every weight
   // fragment meets two activation fragments - and the grid is x = 8 * row blocks, y = groups of 8 strips (x runs
@@ -229,6 +235,25 @@ __global__ __launch_bounds__(576) void qgemv_kernel(const uint8_t* __restrict__ 
         panel[2 * SW + lane] = __float_as_int(bias);
       }
     }
+    if (ROW_TABLE && e.row_min_a) {
+      // Per-row ranges: scale and bias of every (row, channel) of the strip, 16 * SW pairs over the 64 lanes, worked
+      // out here while the other wavefronts stream (the raw channel values come back from the panel: LDS operations
+      // of one wavefront complete in order).  The epilogue then only reads the table.
+      float* const rowtab = reinterpret_cast<float*>(panel + 6 * SW);  // [16][SW]{scale, bias}
+      for (int idx = lane; idx < 16 * SW; idx += 64) {
+        const int mm = idx / SW, c = idx - mm * SW;
+        if (m_base + mm < M) {
+          PrepArgs pr = e.prep;
+          pr.min_a = e.row_min_a[m_base + mm];
+          pr.max_a = e.row_max_a[m_base + mm];
+          const ChannelScaleBias cs = channel_scale_bias(
+              pr, __int_as_float(panel[SW + c]), __int_as_float(panel[2 * SW + c]), __int_as_float(panel[3 * SW + c]),
+              __int_as_float(panel[4 * SW + c]), __int_as_float(panel[5 * SW + c]), panel[c]);
+          rowtab[2 * idx] = e.n_scales > 0 ? cs.scale : 1.0f;
+          rowtab[2 * idx + 1] = cs.bias;
+        }
+      }
+    }
   } else {
     v4i w0[U][NT], w1[U][NT];
     int pb = p0;
@@ -266,19 +291,29 @@ __global__ __launch_bounds__(576) void qgemv_kernel(const uint8_t* __restrict__ 
     if (m < M && n < N) {
       ChannelParams cp;
       if (e.row_min_a) {
-        PrepArgs pr = e.prep;
-        pr.min_a = e.row_min_a[m];
-        pr.max_a = e.row_max_a[m];
+        if constexpr (ROW_TABLE) {
+          const float* const rowtab = reinterpret_cast<const float*>(panel + 6 * SW) + 2 * ((m - m_base) * SW + col);
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          const int colsum = panel[col + r];
-          const ChannelScaleBias c = channel_scale_bias(
-              pr, __int_as_float(panel[SW + col + r]), __int_as_float(panel[2 * SW + col + r]),
-              __int_as_float(panel[3 * SW + col + r]), __int_as_float(panel[4 * SW + col + r]),
-              __int_as_float(panel[5 * SW + col + r]), colsum);
-          cp.comp[r] = e.comp_mul * colsum;
-          cp.scale[r] = e.n_scales > 0 ? c.scale : 1.0f;
-          cp.bias[r] = c.bias;
+          for (int r = 0; r < 4; ++r) {
+            cp.comp[r] = e.comp_mul * panel[col + r];
+            cp.scale[r] = rowtab[2 * r];
+            cp.bias[r] = rowtab[2 * r + 1];
+          }
+        } else {
+          PrepArgs pr = e.prep;
+          pr.min_a = e.row_min_a[m];
+          pr.max_a = e.row_max_a[m];
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const int colsum = panel[col + r];
+            const ChannelScaleBias c = channel_scale_bias(
+                pr, __int_as_float(panel[SW + col + r]), __int_as_float(panel[2 * SW + col + r]),
+                __int_as_float(panel[3 * SW + col + r]), __int_as_float(panel[4 * SW + col + r]),
+                __int_as_float(panel[5 * SW + col + r]), colsum);
+            cp.comp[r] = e.comp_mul * colsum;
+            cp.scale[r] = e.n_scales > 0 ? c.scale : 1.0f;
+            cp.bias[r] = c.bias;
+          }
         }
       } else {
 #pragma unroll
@@ -438,7 +473,7 @@ int launch_gemv(const uint8_t* a, uint32_t a_xor, const uint8_t* bp, int M, int 
                 const EpilogueArgs& e, void* out, hipStream_t st) {
   auto kern = M > 16 ? qgemv_kernel<NT, OUT_T, 2> : qgemv_kernel<NT, OUT_T, 1>;
   const int R = M > 16 ? 2 : 1;
-  const size_t lds_max = static_cast<size_t>(8 * kGemvRing * 1024) * R + 6 * 16 * NT * 4;
+  const size_t lds_max = static_cast<size_t>(8 * kGemvRing * 1024) * R + kGemvPanelWords * 16 * NT * 4;
   static bool attr_set[2] = {false, false};  // benign race: the call is idempotent
   if (!attr_set[M > 16]) {
     hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -446,7 +481,7 @@ int launch_gemv(const uint8_t* a, uint32_t a_xor, const uint8_t* bp, int M, int 
     if (err != hipSuccess) return hip_fail(err, "hipFuncSetAttribute(qgemv_kernel)");
     attr_set[M > 16] = true;
   }
-  const size_t lds = static_cast<size_t>(waves) * kGemvRing * 1024 * R + 6 * 16 * NT * 4;
+  const size_t lds = static_cast<size_t>(waves) * kGemvRing * 1024 * R + kGemvPanelWords * 16 * NT * 4;
   const int strips = (N + 16 * NT - 1) / (16 * NT);
   const int rbs = (M + 31) / 32;  // row blocks of the R = 2 kernel
   const dim3 grid = M > 16 ? dim3(8 * rbs, (strips + 7) / 8) : dim3(strips);
