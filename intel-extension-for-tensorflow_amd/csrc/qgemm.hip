@@ -279,6 +279,30 @@ __global__ __launch_bounds__(576) void qgemv_kernel(const uint8_t* __restrict__ 
   }
   // cross-wavefront reduction through the rings
   __syncthreads();
+  if (!ROW_TABLE && e.row_min_a != nullptr) {
+    // Per-row ranges with 32-channel strips: every output has its own scale and bias to work out (three divisions
+    // each), so the 4 channels of a lane's group go to different wavefronts - all of them, the parameter wavefront
+    // included - instead of one wavefront per tile doing four in a row.
+    for (int unit = wave; unit < 4 * R * NT; unit += waves + 1) {
+      const int tile = unit >> 2, r = unit & 3;
+      const int tr = tile / NT, tc = tile - tr * NT;
+      int part = 0;
+      for (int w = 0; w < waves; ++w) part += reinterpret_cast<const int*>(smem + w * (RING * R * 1024) + tile * 1024 + lane * 16)[r];
+      const int col = tc * 16 + lgrp * 4 + r, n = strip * SW + col;
+      const int m = m_base + 16 * tr + lrow;
+      if (m < M && n < N) {
+        PrepArgs pr = e.prep;
+        pr.min_a = e.row_min_a[m];
+        pr.max_a = e.row_max_a[m];
+        const int colsum = panel[col];
+        const ChannelScaleBias c = channel_scale_bias(pr, __int_as_float(panel[SW + col]), __int_as_float(panel[2 * SW + col]),
+                                                      __int_as_float(panel[3 * SW + col]), __int_as_float(panel[4 * SW + col]),
+                                                      __int_as_float(panel[5 * SW + col]), colsum);
+        epilogue_store_one<OUT_T>(part, e.comp_mul * colsum, e.n_scales > 0 ? c.scale : 1.0f, c.bias, m, n, N, e, out);
+      }
+    }
+    return;
+  }
   // the R * NT tiles of 16 x 16 go round the wavefronts (R = 1: wavefront t finishes tile t)
   for (int tile = wave; tile < R * NT; tile += waves + 1) {
     const int tr = tile / NT, tc = tile - tr * NT;
