@@ -30,6 +30,13 @@ __device__ __forceinline__ uint32_t quantize4(f4 v, float scale, float addend) {
                sat_rne<T>(d + addend));
 }
 
+// The 4-byte stores of the narrowing kernels (4 or 16 bytes read per byte written) go out as system-scope stores (sc0 sc1:
+// written through instead of held in L2): next to streaming loads that measured 6 % faster than streaming (nt) stores
+// (QuantizeV2 over 2^28 elements: 199 -> 188 us).  The widening kernels are the other way round (nt stores 182 us, sc1 205 us).
+__device__ __forceinline__ void store_through(uint32_t* p, uint32_t v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+
 // n4 = number of complete groups of 4 elements; the caller handles the tail.
 template <int T>
 __global__ __launch_bounds__(kThreads) void quantize_vec_kernel(const f4* __restrict__ x,
@@ -46,7 +53,7 @@ __global__ __launch_bounds__(kThreads) void quantize_vec_kernel(const f4* __rest
   for (int step = 0; step < kNarrowSteps; ++step, i += stride) {
     if (i < n4) {
       const f4 v = __builtin_nontemporal_load(&x[i]);
-      __builtin_nontemporal_store(quantize4<T>(v, scale, addend), &q[i]);
+      store_through(&q[i], quantize4<T>(v, scale, addend));
     }
   }
 }
@@ -108,8 +115,7 @@ __global__ __launch_bounds__(kThreads) void quantize_axis_vec_kernel(const f4* _
     ad = f4{a, a, a, a};
   }
   const float a = v.x * sc.x, b = v.y * sc.y, c = v.z * sc.z, d = v.w * sc.w;
-  __builtin_nontemporal_store(pack4(sat_rne<T>(a + ad.x), sat_rne<T>(b + ad.y), sat_rne<T>(c + ad.z), sat_rne<T>(d + ad.w)),
-                              &q[i]);
+  store_through(&q[i], pack4(sat_rne<T>(a + ad.x), sat_rne<T>(b + ad.y), sat_rne<T>(c + ad.z), sat_rne<T>(d + ad.w)));
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -222,7 +228,7 @@ __global__ __launch_bounds__(kThreads) void requantize_vec_kernel(const i4* __re
       if (kMode == 1) s = reinterpret_cast<const f4*>(scales)[i % depth4];
       const float a = static_cast<float>(v.x) * s.x, b = static_cast<float>(v.y) * s.y;
       const float c = static_cast<float>(v.z) * s.z, d = static_cast<float>(v.w) * s.w;
-      __builtin_nontemporal_store(pack4(sat_rne<T>(a), sat_rne<T>(b), sat_rne<T>(c), sat_rne<T>(d)), &q[i]);
+      store_through(&q[i], pack4(sat_rne<T>(a), sat_rne<T>(b), sat_rne<T>(c), sat_rne<T>(d)));
     }
   }
 }
@@ -712,7 +718,7 @@ __global__ __launch_bounds__(kThreads) void quantize_dynamic_finish_kernel(const
 #pragma unroll
   for (int j = 0; j < kUnroll; ++j) {
     const int64_t i = base + j * kThreads;
-    if (i < n4) __builtin_nontemporal_store(quantize4<T>(v[j], scale, addend), &q4[i]);
+    if (i < n4) store_through(&q4[i], quantize4<T>(v[j], scale, addend));
   }
   if (blockIdx.x == 0 && static_cast<int>(threadIdx.x) < ntail) {
     const float t = xtail[threadIdx.x] * scale;
