@@ -48,7 +48,11 @@ __global__ __launch_bounds__(kThreads) void quantize_bf16_vec_kernel(const u4* _
         const uint32_t h = (v[j][e >> 1] >> (16 * (e & 1))) & 0xffffu;
         o[e >> 2] |= quantize1<T>(bf16_to_f32(h), scale, addend) << (8 * (e & 3));
       }
-      __builtin_nontemporal_store(u2{o[0], o[1]}, &q[i]);
+      {  // written through (system scope), like the stores of the other narrowing kernels
+        u2* const dst = &q[i];
+        const u2 val = u2{o[0], o[1]};
+        asm volatile("global_store_dwordx2 %0, %1, off sc1" : : "v"(dst), "v"(val) : "memory");
+      }
     }
   }
 }
@@ -87,7 +91,7 @@ __global__ __launch_bounds__(kThreads) void dequantize16_vec_kernel(const u2* __
 #pragma unroll
   for (int j = 0; j < kUnroll; ++j) {
     const int64_t i = base + j * kThreads;
-    if (i < n8) w[j] = __builtin_nontemporal_load(&q[i]);
+    if (i < n8) w[j] = q[i];  // ordinary load, as in the fp32 Dequantize
   }
 #pragma unroll
   for (int j = 0; j < kUnroll; ++j) {
