@@ -100,22 +100,26 @@ __global__ __launch_bounds__(kThreads) void quantize_axis_vec_kernel(const f4* _
                                                                      uint32_t n4, uint32_t slices, uint32_t inner4,
                                                                      const float* __restrict__ scales,
                                                                      const float* __restrict__ addends) {
-  const uint32_t i = blockIdx.x * kThreads + threadIdx.x;
-  if (i >= n4) return;
-  const f4 v = __builtin_nontemporal_load(&x[i]);
-  f4 sc, ad = {0.0f, 0.0f, 0.0f, 0.0f};
-  if constexpr (LAST) {
-    const uint32_t s4 = i % (slices >> 2);
-    sc = reinterpret_cast<const f4*>(scales)[s4];
-    if (addends) ad = reinterpret_cast<const f4*>(addends)[s4];
-  } else {
-    const uint32_t sl = (i / inner4) % slices;
-    const float c = scales[sl], a = addends ? addends[sl] : 0.0f;
-    sc = f4{c, c, c, c};
-    ad = f4{a, a, a, a};
+  const uint32_t stride = gridDim.x * kThreads;  // two steps a whole grid apart, as in quantize_vec_kernel
+  uint32_t i = blockIdx.x * kThreads + threadIdx.x;
+#pragma unroll 1
+  for (int step = 0; step < kNarrowSteps; ++step, i += stride) {
+    if (i >= n4) return;
+    const f4 v = __builtin_nontemporal_load(&x[i]);
+    f4 sc, ad = {0.0f, 0.0f, 0.0f, 0.0f};
+    if constexpr (LAST) {
+      const uint32_t s4 = i % (slices >> 2);
+      sc = reinterpret_cast<const f4*>(scales)[s4];
+      if (addends) ad = reinterpret_cast<const f4*>(addends)[s4];
+    } else {
+      const uint32_t sl = (i / inner4) % slices;
+      const float c = scales[sl], a = addends ? addends[sl] : 0.0f;
+      sc = f4{c, c, c, c};
+      ad = f4{a, a, a, a};
+    }
+    const float a = v.x * sc.x, b = v.y * sc.y, c = v.z * sc.z, d = v.w * sc.w;
+    store_through(&q[i], pack4(sat_rne<T>(a + ad.x), sat_rne<T>(b + ad.y), sat_rne<T>(c + ad.z), sat_rne<T>(d + ad.w)));
   }
-  const float a = v.x * sc.x, b = v.y * sc.y, c = v.z * sc.z, d = v.w * sc.w;
-  store_through(&q[i], pack4(sat_rne<T>(a + ad.x), sat_rne<T>(b + ad.y), sat_rne<T>(c + ad.z), sat_rne<T>(d + ad.w)));
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -848,7 +852,7 @@ extern "C" int itexhip_quantize_axis(const float* x, void* q, int64_t outer, int
   const bool last = inner == 1 && slices % 4 == 0 && aligned(scales, 16) && (!addends || aligned(addends, 16));
   if ((last || inner % 4 == 0) && aligned(x, 16) && aligned(q, 4) && n / 4 < (1LL << 31) && slices < (1LL << 31)) {
     const uint32_t n4 = static_cast<uint32_t>(n / 4), sl = static_cast<uint32_t>(slices), in4 = static_cast<uint32_t>(inner / 4);
-    const unsigned vgrid = blocks_for(n4, kThreads);
+    const unsigned vgrid = blocks_for(n4, kThreads * kNarrowSteps);
     const f4* xv = reinterpret_cast<const f4*>(x);
     uint32_t* qv = reinterpret_cast<uint32_t*>(q);
     hipStream_t st = as_stream(stream);
