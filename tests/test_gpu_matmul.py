@@ -510,7 +510,7 @@ def test_llama_decode_gemv(hip, dev, M, K, N):
 
 @pytest.mark.parametrize("M", [1, 3, 16])
 @pytest.mark.parametrize("kw", [V2_DEQ, V2_REQ_S8, V2_DEQ_RELU])
-@pytest.mark.parametrize("K,N", [(512, 272), (4096, 1024)])
+@pytest.mark.parametrize("K,N", [(512, 272), (4096, 1024), (128, 8200)])  # the last one: 32-channel strips, ragged N
 def test_per_token_activation_ranges(hip, dev, M, kw, K, N):
     """Rows quantized with their own range: row m of the GPU result equals the oracle's 1 x K problem
     with that row's (min, max).  The reference's MatMul ops have no per-row range; this is the decode
