@@ -48,11 +48,10 @@ __global__ __launch_bounds__(kThreads) void quantize_bf16_vec_kernel(const u4* _
         const uint32_t h = (v[j][e >> 1] >> (16 * (e & 1))) & 0xffffu;
         o[e >> 2] |= quantize1<T>(bf16_to_f32(h), scale, addend) << (8 * (e & 3));
       }
-      {  // written through (system scope), like the stores of the other narrowing kernels
-        u2* const dst = &q[i];
-        const u2 val = u2{o[0], o[1]};
-        asm volatile("global_store_dwordx2 %0, %1, off sc1" : : "v"(dst), "v"(val) : "memory");
-      }
+      // written through (system scope), like the stores of the other narrowing kernels
+      __hip_atomic_store(reinterpret_cast<unsigned long long*>(&q[i]),
+                         static_cast<unsigned long long>(o[0]) | (static_cast<unsigned long long>(o[1]) << 32), __ATOMIC_RELAXED,
+                         __HIP_MEMORY_SCOPE_SYSTEM);
     }
   }
 }

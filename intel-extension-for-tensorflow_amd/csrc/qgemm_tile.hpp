@@ -527,7 +527,9 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void qgemm_tile_kernel(
           // through; 8- and 16-bit outputs, and the GELU epilogue whose stores trickle out between long runs of
           // arithmetic, measured 1-8 % faster as streaming (nontemporal) stores.
           uint8_t* const dst = reinterpret_cast<uint8_t*>(out) + (static_cast<int64_t>(m) * N + n_col) * ESZ;
-          if constexpr (ESZ == 4 && ACT != 3) asm volatile("global_store_dwordx4 %0, %1, off sc1" : : "v"(dst), "v"(v) : "memory");
+          // (the s_nop: a store of more than 8 bytes reads its data registers for a cycle or two after it issues, and the
+          // compiler, which cannot see a store inside the assembly, may let the next vector instruction overwrite them)
+          if constexpr (ESZ == 4 && ACT != 3) asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 1" : : "v"(dst), "v"(v) : "memory");
           else __builtin_nontemporal_store(v, reinterpret_cast<v4i*>(dst));
         }
       }

@@ -194,6 +194,18 @@ def test_tile_kernel_vs_oracle(hip, dev, M, K, N, kw):
     np.testing.assert_array_equal(layer.run(xq, kw, mn, mx, -r_out, r_out, path="fused"), ref)
 
 
+@pytest.mark.parametrize("M,K,N", [(127, 240, 8316), (100, 144, 8340)])
+def test_tile_kernel_repeated_launches_equal_the_oracle(hip, dev, M, K, N):
+    """fp32 outputs of the tile kernel, many workgroups, K not a multiple of 64, launched several times: every launch
+    must equal the oracle (an epilogue store whose data registers were overwritten too early showed as a few wrong
+    elements in some launches only)."""
+    layer, w, bias = make_layer(hip, dev, K, N, seed=K + N)
+    x, xq, mn, mx = make_acts(M, K, seed=M)
+    ref = layer.oracle(xq, V2_DEQ_RELU, mn, mx)
+    for launch in range(8):
+        np.testing.assert_array_equal(layer.run(xq, V2_DEQ_RELU, mn, mx, path="tile"), ref, err_msg="launch %d" % launch)
+
+
 @pytest.mark.parametrize("M,K,N", [(17, 64, 16), (32, 4096, 1000), (33, 448, 528), (64, 1024, 100), (100, 256, 200),
                                    (128, 1024, 1024), (127, 2048, 24), (48, 80, 2051)])
 @pytest.mark.parametrize("kw", [V2_DEQ_RELU, V2_REQ_S8, V2_REQ_U8_RELU, V1_S32])
