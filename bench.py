@@ -681,6 +681,19 @@ def main():
             mfma_probe_workload_data=sampler.run(torch, lambda: hip.mfma_probe(256, 200, wl, sink, st0)),
             mfma_probe_constant_operands=sampler.run(torch, lambda: hip.mfma_probe(256, 200, ones, sink, st0)),
             note="amdgpu sysfs (power1_input, pp_dpm_sclk) sampled every 50 ms over 1.5 s of back-to-back launches")
+        # the headline kernel itself on constant operands (every activation byte 0x81, every weight 1): the same
+        # instructions and memory traffic with almost no bit toggling in the matrix pipe and on the data paths, i.e. what
+        # the kernel's schedule delivers when the clock is not held down by the energy of the data
+        try:
+            w1 = torch.ones(K, N, dtype=torch.int8, device=dev)
+            packed1, colsum1 = torch.empty_like(L0["packed"]), torch.empty_like(L0["colsum"])
+            hip.qgemm_prepack_b(w1, False, K, N, packed1, colsum1, st0)
+            x1 = torch.full_like(xq0, 0x81)
+            power["headline_gemm_constant_operands"] = sampler.run(
+                torch, lambda: hip.qmatmul(p0, x1, packed1, colsum1, M, K, N, L0["min_b"], L0["max_b"], N, L0["bias"], out0, st0))
+            del w1, packed1, colsum1, x1
+        except Exception as exc:
+            power["headline_gemm_constant_operands"] = dict(error=str(exc)[:200])
         # the vendor library on the same int8 problem (hipBLASLt behind torch._int_mm, int32 output, no epilogue), as a
         # point of comparison for rate and power: a measurement only, nothing of the product calls it
         try:

@@ -125,6 +125,34 @@ def test_binary_operand_broadcast_forms(hip, dev):
         check(hip, dev, x, y, binary=((orc.BIN_MUL, t), (orc.BIN_ADD, t)))
 
 
+@pytest.mark.parametrize("seed", range(4))
+def test_random_shapes_layouts_and_operands(hip, dev, seed):
+    """Seeded random batch shapes, matrix sizes, layouts, operand base offsets, output types and fused operands in every
+    broadcast form, each case launched twice."""
+    import torch
+    rng = np.random.default_rng(3000 + seed)
+    for case in range(25):
+        B = [(), (1,), (3,), (2, 2), (2, 1, 3)][int(rng.integers(0, 5))]
+        M = int(rng.choice([1, 5, 16, 31, 32, 33, 64, 70, 100, 128, 130]))
+        K = int(rng.choice([1, 4, 16, 17, 32, 48, 64, 100, 128, 200]))
+        N = int(rng.choice([1, 4, 8, 21, 32, 36, 64, 96, 128, 130]))
+        adj_x, adj_y = bool(rng.random() < 0.3), bool(rng.random() < 0.5)
+        t_out = [orc.FLOAT, orc.FLOAT, orc.BFLOAT16, orc.HALF][int(rng.integers(0, 4))]
+        x = rng.integers(-128, 128, B + ((K, M) if adj_x else (M, K))).astype(np.int8)
+        y = rng.integers(-128, 128, B + ((N, K) if adj_y else (K, N))).astype(np.int8)
+        ones = (1,) * len(B)
+        binary = []
+        for _ in range(int(rng.choice([0, 0, 1, 2]))):
+            shape = [(1,), B + (M, N), ones + (1, N), ones + (M, 1), ones + (M, N)][int(rng.integers(0, 5))]
+            t = rng.standard_normal(shape).astype(np.float32)
+            if t_out != orc.FLOAT:
+                t = to16(torch, t, t_out)
+            binary.append((orc.BIN_MUL if rng.random() < 0.5 else orc.BIN_ADD, t))
+        x_off, y_off = [(0, 0), (16, 16), (1, 0), (4, 3)][int(rng.integers(0, 4))]
+        for launch in range(2):
+            check(hip, dev, x, y, adj_x, adj_y, tuple(binary), t_out, x_off, y_off)
+
+
 def test_empty_and_invalid(hip, dev):
     import torch
     z = np.zeros((2, 0, 8), np.int8)

@@ -85,11 +85,40 @@ def test_implicit_gemm_conv(hip, dev, monkeypatch, shape, wshape, strides, dil, 
     """itexhip_qconv2d (activation tiles gathered from the NHWC input) against a numpy convolution for the int32
     accumulators, and bit for bit against the patch-matrix path (itexhip_im2col8 + itexhip_qgemm) for every output
     type with per-channel scales, bias and ReLU."""
-    import torch
-    from tests.test_oracle_conv import ref_int_conv
     if tile_shape is not None:   # every tile shape of the kernel on every case, ragged edges included
         monkeypatch.setenv("ITEXHIP_CONV_TILE_SHAPE", str(tile_shape))
-    rng = np.random.default_rng(sum(shape) + sum(wshape) + signed_in)
+    check_implicit_conv(hip, dev, shape, wshape, strides, dil, lead, signed_in, np.random.default_rng(sum(shape) + sum(wshape) + signed_in))
+
+
+@pytest.mark.parametrize("seed", range(4))
+def test_implicit_gemm_conv_random_geometries(hip, dev, monkeypatch, seed):
+    """Seeded random geometries (window, strides, dilation, SAME and explicit leading pads, channel counts, batch) on
+    random tile shapes, checked like the fixed cases above."""
+    rng = np.random.default_rng(2000 + seed)
+    done = 0
+    while done < 10:
+        B, H, W = int(rng.integers(1, 4)), int(rng.integers(3, 24)), int(rng.integers(3, 24))
+        C = 16 * int(rng.choice([1, 1, 2, 3, 4, 6]))
+        kh, kw = [(1, 1), (3, 3), (2, 2), (5, 5), (1, 3), (3, 1), (7, 7)][int(rng.integers(0, 7))]
+        strides = [(1, 1), (2, 2), (2, 1), (3, 3)][int(rng.integers(0, 4))]
+        dil = [(1, 1), (1, 1), (2, 2), (1, 2)][int(rng.integers(0, 4))]
+        O = int(rng.choice([16, 32, 48, 64, 80, 128, 144, 272]))
+        lead = None if rng.random() < 0.6 else (int(rng.integers(0, kh + 1)), int(rng.integers(0, kw + 1)))
+        if lead is not None and ((H + 2 * lead[0] - ((kh - 1) * dil[0] + 1)) // strides[0] + 1 <= 0 or
+                                 (W + 2 * lead[1] - ((kw - 1) * dil[1] + 1)) // strides[1] + 1 <= 0):
+            continue
+        tile_shape = int(rng.integers(-1, 3))
+        if tile_shape >= 0:
+            monkeypatch.setenv("ITEXHIP_CONV_TILE_SHAPE", str(tile_shape))
+        else:
+            monkeypatch.delenv("ITEXHIP_CONV_TILE_SHAPE", raising=False)
+        check_implicit_conv(hip, dev, (B, H, W, C), (kh, kw, C, O), strides, dil, lead, bool(rng.integers(0, 2)), rng)
+        done += 1
+
+
+def check_implicit_conv(hip, dev, shape, wshape, strides, dil, lead, signed_in, rng):
+    import torch
+    from tests.test_oracle_conv import ref_int_conv
     B, H, W, Cin = shape
     kh, kw, _, O = wshape
     x = rng.integers(-128, 128, shape).astype(np.int8) if signed_in else rng.integers(0, 256, shape).astype(np.uint8)
@@ -130,8 +159,10 @@ def test_implicit_gemm_conv(hip, dev, monkeypatch, shape, wshape, strides, dil, 
     ep.elt[0].alg, ep.elt[0].alpha, ep.elt[0].beta = hip.ELT_RELU, 0.0, 0.0
     for T, dt in ((hip.QINT8, torch.int8), (hip.QUINT8, torch.uint8), (hip.FLOAT, torch.float32), (hip.BFLOAT16, torch.bfloat16),
                   (hip.QINT32, torch.int32)):
-        a = torch.zeros((M, O), dtype=dt, device=dev)
-        b_ = torch.zeros((M, O), dtype=dt, device=dev)
+        a = torch.empty((M, O), dtype=dt, device=dev)
+        b_ = torch.empty((M, O), dtype=dt, device=dev)
+        a.view(torch.uint8).fill_(0x55)          # different fillers: an element neither path writes shows up
+        b_.view(torch.uint8).fill_(0xAA)
         hip.qconv2d(xd, T_in, g, packed, colsum, O, scales, bias, ep, T, a)
         hip.qgemm(cols, T_in, packed, colsum, M, K, O, scales, bias, ep, T, b_)
         torch.cuda.synchronize()

@@ -51,6 +51,7 @@ class Linear:
                             self.scales_d, self.sbias_d)
         x_d = torch.from_numpy(xq).to(self.dev)
         out = torch.empty((M, self.N), dtype=tdt(kw["t_out"]), device=self.dev)
+        out.view(torch.uint8).fill_(0x55)        # an element the kernel does not write cannot pass by luck
         fn = {"auto": hip.qgemm, "tile": hip.qgemm_tile, "gemv": hip.qgemv}.get(path)
         if path == "fused":
             hip.qmatmul(p, x_d, self.packed, self.colsum, M, self.K, self.N, self.min_b_d, self.max_b_d, nb,
@@ -204,6 +205,34 @@ def test_tile_kernel_repeated_launches_equal_the_oracle(hip, dev, M, K, N):
     ref = layer.oracle(xq, V2_DEQ_RELU, mn, mx)
     for launch in range(8):
         np.testing.assert_array_equal(layer.run(xq, V2_DEQ_RELU, mn, mx, path="tile"), ref, err_msg="launch %d" % launch)
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_random_shapes_on_every_path_vs_oracle(hip, dev, monkeypatch, seed):
+    """Seeded random problem sizes (ragged in M, N and K), output types and forced tile shapes; the tile kernel, the
+    small-M kernel where it takes the row count, the dispatching entry point and the single-launch op against the
+    oracle, each launched twice into pre-filled outputs."""
+    rng = np.random.default_rng(1000 + seed)
+    for case in range(8):
+        M = int(rng.choice([1, 3, 16, 17, 33, 64, 100, 127, 128, 129, 200, 257, 300]))
+        K = 16 * int(rng.integers(1, 48))
+        N = 4 * int(rng.integers(1, 500)) if case % 2 else 16 * int(rng.integers(1, 130))
+        kw = [V2_DEQ, V2_DEQ_RELU, V2_REQ_S8, V2_REQ_U8_RELU, V1_S32][int(rng.integers(0, 5))]
+        shape = int(rng.integers(-1, 5))
+        if shape >= 0:
+            monkeypatch.setenv("ITEXHIP_TILE_SHAPE", str(shape))
+        else:
+            monkeypatch.delenv("ITEXHIP_TILE_SHAPE", raising=False)
+        layer, w, bias = make_layer(hip, dev, K, N, seed=seed * 100 + case)
+        x, xq, mn, mx = make_acts(M, K, seed=seed * 100 + case + 50)
+        full = x @ w + bias
+        r_out = float(np.abs(np.maximum(full, 0) if kw.get("activation") else full).max())
+        lo = 0.0 if kw["t_out"] == orc.QUINT8 else -r_out
+        ref = layer.oracle(xq, kw, mn, mx, lo, r_out)
+        for path in ("tile", "auto", "fused") + (("gemv",) if M <= 128 else ()):
+            for launch in range(2):
+                np.testing.assert_array_equal(layer.run(xq, kw, mn, mx, lo, r_out, path=path), ref,
+                                              err_msg="case %d: M %d K %d N %d shape %d %s launch %d" % (case, M, K, N, shape, path, launch))
 
 
 @pytest.mark.parametrize("M,K,N", [(17, 64, 16), (32, 4096, 1000), (33, 448, 528), (64, 1024, 100), (100, 256, 200),
