@@ -143,6 +143,45 @@ def test_quantize_unaligned_pointers(hip, dev):
     assert got[0] == 0 and np.all(got[1003:] == 0)
 
 
+@pytest.mark.parametrize("seed", range(3))
+def test_random_sizes_and_offsets_vs_oracle(hip, dev, seed):
+    """Seeded random element counts (1 .. 3 million: vector body, grid-strided second group, scalar head and tail) and
+    random element offsets of input and output inside larger buffers; QuantizeV2 in every mode, Dequantize and
+    Requantize against the oracle, with guard bytes around each output that must stay untouched."""
+    import torch
+    rng = np.random.default_rng(4000 + seed)
+    modes = [(orc.QINT8, orc.SCALED, False), (orc.QUINT8, orc.SCALED, False), (orc.QUINT8, orc.MIN_FIRST, False),
+             (orc.QINT8, orc.MIN_FIRST, False), (orc.QUINT8, orc.MIN_FIRST, True)]
+    for case in range(12):
+        n = int(rng.choice([rng.integers(1, 300), rng.integers(300, 70000), rng.integers(70000, 3000000)]))
+        xo, qo = int(rng.integers(0, 8)), int(rng.integers(0, 16))
+        T, mode, classic = modes[int(rng.integers(0, 5))]
+        x = outlier_normal(rng, n, 1e-4, 50.0)
+        mn, mx = float(x.min()), float(x.max())
+        st, q_ref, _, _ = orc.quantize_v2(x, mn, mx, T, mode, None, classic)
+        sc, add, _, _ = host_quant_params(T, mode, classic, mn, mx)
+        xb = torch.zeros(n + 8, dtype=torch.float32, device=dev)
+        xb[xo:xo + n] = torch.from_numpy(x).to(dev)
+        qb = torch.full((n + 32,), 0x55, dtype=torch.uint8, device=dev)
+        hip.quantize(xb.data_ptr() + 4 * xo, qb.data_ptr() + qo, n, T, float(sc[0]), float(add[0]))
+        torch.cuda.synchronize()
+        got = qb.cpu().numpy()
+        msg = "quantize n %d offsets %d %d type %d mode %d classic %d" % (n, xo, qo, T, mode, classic)
+        np.testing.assert_array_equal(got[qo:qo + n].view(orc.NP_OF[T]), q_ref, err_msg=msg)
+        assert np.all(got[:qo] == 0x55) and np.all(got[qo + n:] == 0x55), msg
+        # Dequantize of those bytes
+        dmode = orc.SCALED if mode == orc.SCALED else orc.MIN_FIRST
+        st, y_ref = orc.dequantize(q_ref, np.float32(-3.7), np.float32(5.2), T, dmode)
+        st, _, _, dsc, dzp = orc.scale_zeropoint_align(T, dmode, True, np.float32(-3.7), np.float32(5.2))
+        yo = int(rng.integers(0, 8))
+        yb = torch.full((n + 16,), -7.0, dtype=torch.float32, device=dev)
+        hip.dequantize(qb.data_ptr() + qo, yb.data_ptr() + 4 * yo, n, T, float(dsc[0]), int(dzp[0]) if dmode == orc.MIN_FIRST else 0)
+        torch.cuda.synchronize()
+        goty = yb.cpu().numpy()
+        np.testing.assert_array_equal(goty[yo:yo + n], y_ref, err_msg="de" + msg)
+        assert np.all(goty[:yo] == -7.0) and np.all(goty[yo + n:] == -7.0), "de" + msg
+
+
 def test_narrow_range_flag_is_inert(hip, dev):
     # the reference reads narrow_range and ignores it: there is no such argument at this level;
     # saturation is full-range (-128) in both cases
