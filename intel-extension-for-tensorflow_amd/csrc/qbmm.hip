@@ -27,6 +27,7 @@ struct BmmArgs {
   itexhip_bmm_params p;
   int tiles_m, tiles_n;
   int vec_x, vec_y;  // operand layouts allow aligned vector loads
+  int grid3;         // launched as (tiles, innermost batch dimension, the other batch dimensions): no division finds them
 };
 
 // One 64 (rows or columns of the output) x 64 (k) byte tile on its way into LDS, k-contiguous there.  The
@@ -78,12 +79,16 @@ __device__ __forceinline__ void put_tile(uint8_t* __restrict__ lds, int t, const
         v4i{static_cast<int>(w[0]), static_cast<int>(w[1]), static_cast<int>(w[2]), static_cast<int>(w[3])};
   } else {
     const int kb = t >> 4, cb = t & 15;
+    // 4 x 4 byte transpose in two rounds of byte permutes: byte j of the four k rows -> four consecutive k of column
+    // cb * 4 + j  (v_perm_b32 numbers the bytes of its second operand 0..3 and of its first 4..7)
+    const uint32_t lo01 = __builtin_amdgcn_perm(w[1], w[0], 0x05010400u);  // w0.b0 w1.b0 w0.b1 w1.b1
+    const uint32_t hi01 = __builtin_amdgcn_perm(w[1], w[0], 0x07030602u);  // w0.b2 w1.b2 w0.b3 w1.b3
+    const uint32_t lo23 = __builtin_amdgcn_perm(w[3], w[2], 0x05010400u);
+    const uint32_t hi23 = __builtin_amdgcn_perm(w[3], w[2], 0x07030602u);
+    const uint32_t v[4] = {__builtin_amdgcn_perm(lo23, lo01, 0x05040100u), __builtin_amdgcn_perm(lo23, lo01, 0x07060302u),
+                           __builtin_amdgcn_perm(hi23, hi01, 0x05040100u), __builtin_amdgcn_perm(hi23, hi01, 0x07060302u)};
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {  // byte j of the four k rows -> four consecutive k of column cb * 4 + j
-      const uint32_t v = ((w[0] >> (8 * j)) & 0xffu) | (((w[1] >> (8 * j)) & 0xffu) << 8) |
-                         (((w[2] >> (8 * j)) & 0xffu) << 16) | (((w[3] >> (8 * j)) & 0xffu) << 24);
-      *reinterpret_cast<uint32_t*>(lds + (cb * 4 + j) * kLdsStride + kb * 4) = v;
-    }
+    for (int j = 0; j < 4; ++j) *reinterpret_cast<uint32_t*>(lds + (cb * 4 + j) * kLdsStride + kb * 4) = v[j];
   }
 }
 
@@ -111,15 +116,21 @@ struct QuadrantSite {
 // Operand values of the lane's 16 results.  Straight-line code: every load is issued whatever the operand's
 // broadcast pattern (rows and columns outside the output read element (0, 0) of the quadrant instead), so that
 // nothing forces a wait before the tiles arrive.
-template <int OUT_T, int NB>
-__device__ __forceinline__ void fetch_operands(const QuadrantSite& s, int lane, float (&o)[ITEXHIP_BMM_MAX_BINARY][16]) {
+// ROWB: no operand depends on the row (a scalar, or a mask broadcast over the rows): one value per lane and operand
+// instead of 16, which is what lets twice as many wavefronts share a SIMD.
+template <int OUT_T, int NB, bool ROWB>
+__device__ __forceinline__ void fetch_operands(const QuadrantSite& s, int lane, float (&o)[ITEXHIP_BMM_MAX_BINARY][ROWB ? 1 : 16]) {
   using elem_t = typename std::conditional<OUT_T == ITEXHIP_FLOAT, float, uint16_t>::type;
   const uint32_t lrow = (lane >> 5) * 4;
   const uint32_t lcol = static_cast<int>(lane & 31) < s.cols_left ? (lane & 31) : 0;
 #pragma unroll
   for (int b = 0; b < NB; ++b) {
+    if constexpr (ROWB) {
+      o[b][0] = widen<OUT_T>(*reinterpret_cast<const elem_t*>(s.operand[b] + lcol * s.operand_col[b]));
+      continue;
+    }
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
+    for (int i = 0; i < (ROWB ? 1 : 16); ++i) {
       const uint32_t row = lrow + (i >> 2) * 8 + (i & 3);
       const uint32_t off = (static_cast<int>(row) < s.rows_left ? row : 0) * s.operand_row[b] + lcol * s.operand_col[b];
       o[b][i] = widen<OUT_T>(*reinterpret_cast<const elem_t*>(s.operand[b] + off));
@@ -127,33 +138,66 @@ __device__ __forceinline__ void fetch_operands(const QuadrantSite& s, int lane, 
   }
 }
 
-template <int OUT_T, int NB>
-__device__ __forceinline__ void store_quadrant(const v16i& acc, const QuadrantSite& s, int lane,
-                                               const float (&o)[ITEXHIP_BMM_MAX_BINARY][16]) {
+// One result on its way out: scale, fused operands in order (each separately rounded), narrowing, store.
+template <int OUT_T, int NB, bool ROWB, int ALG0, int ALG1>
+__device__ __forceinline__ void store_one(int acc, const QuadrantSite& s, int i, uint32_t off,
+                                          const float (&o)[ITEXHIP_BMM_MAX_BINARY][ROWB ? 1 : 16]) {
+  using elem_t = typename std::conditional<OUT_T == ITEXHIP_FLOAT, float, uint16_t>::type;
+  float v = static_cast<float>(acc) * s.scale;
+  if constexpr (NB > 0) v = ALG0 == ITEXHIP_BIN_MUL ? v * o[0][ROWB ? 0 : i] : v + o[0][ROWB ? 0 : i];
+  if constexpr (NB > 1) v = ALG1 == ITEXHIP_BIN_MUL ? v * o[1][ROWB ? 0 : i] : v + o[1][ROWB ? 0 : i];
+  elem_t* dst = reinterpret_cast<elem_t*>(s.out + off);
+  // the output is written back as it goes instead of staying dirty in L2 until the kernel ends: as system-scope
+  // (write-through) stores without fused operands (P.V over 128 sequences: 21.3 -> 18.8 us), as streaming stores
+  // with them (Q.K^T + Mul + Add measured 3 % slower written through)
+  if constexpr (OUT_T == ITEXHIP_FLOAT && NB == 0) __hip_atomic_store(dst, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+  else if constexpr (OUT_T == ITEXHIP_FLOAT) __builtin_nontemporal_store(v, dst);
+  else __builtin_nontemporal_store(static_cast<uint16_t>(f32_to_bits16<OUT_T>(v)), dst);
+}
+
+template <int OUT_T, int NB, bool ROWB, int ALG0, int ALG1>
+__device__ __forceinline__ void store_rows(const v16i& acc, const QuadrantSite& s, int lane,
+                                           const float (&o)[ITEXHIP_BMM_MAX_BINARY][ROWB ? 1 : 16]) {
   using elem_t = typename std::conditional<OUT_T == ITEXHIP_FLOAT, float, uint16_t>::type;
   const uint32_t lrow = (lane >> 5) * 4, lcol = lane & 31;
-  if (static_cast<int>(lcol) >= s.cols_left) return;
   const uint32_t obase = lrow * s.out_row + lcol * static_cast<uint32_t>(sizeof(elem_t));
+  if (s.rows_left == 32 && s.cols_left == 32) {  // a whole quadrant (the same answer for the wavefront): nothing to test
+#pragma unroll
+    for (int i = 0; i < 16; ++i)
+      store_one<OUT_T, NB, ROWB, ALG0, ALG1>(acc[i], s, i, obase + static_cast<uint32_t>((i >> 2) * 8 + (i & 3)) * s.out_row, o);
+    return;
+  }
+  if (static_cast<int>(lcol) >= s.cols_left) return;
 #pragma unroll
   for (int i = 0; i < 16; ++i) {
     const int r = (i >> 2) * 8 + (i & 3);
     if (static_cast<int>(lrow) + r >= s.rows_left) continue;
-    float v = static_cast<float>(acc[i]) * s.scale;
-    if constexpr (NB > 0) v = s.alg[0] == ITEXHIP_BIN_MUL ? v * o[0][i] : v + o[0][i];
-    if constexpr (NB > 1) v = s.alg[1] == ITEXHIP_BIN_MUL ? v * o[1][i] : v + o[1][i];
-    elem_t* dst = reinterpret_cast<elem_t*>(s.out + (obase + r * s.out_row));
-    // the output is written back as it goes instead of staying dirty in L2 until the kernel ends: as system-scope
-    // (write-through) stores without fused operands (P.V over 128 sequences: 21.3 -> 18.8 us), as streaming stores
-    // with them (Q.K^T + Mul + Add measured 3 % slower written through)
-    if constexpr (OUT_T == ITEXHIP_FLOAT && NB == 0) __hip_atomic_store(dst, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-    else if constexpr (OUT_T == ITEXHIP_FLOAT) __builtin_nontemporal_store(v, dst);
-    else __builtin_nontemporal_store(static_cast<uint16_t>(f32_to_bits16<OUT_T>(v)), dst);
+    store_one<OUT_T, NB, ROWB, ALG0, ALG1>(acc[i], s, i, obase + r * s.out_row, o);
+  }
+}
+
+// The operands' algorithms are the same for the whole launch: one copy of the store loop per combination, chosen by
+// a branch, instead of computing product and sum of every element and selecting.
+template <int OUT_T, int NB, bool ROWB>
+__device__ __forceinline__ void store_quadrant(const v16i& acc, const QuadrantSite& s, int lane,
+                                               const float (&o)[ITEXHIP_BMM_MAX_BINARY][ROWB ? 1 : 16]) {
+  constexpr int MUL = ITEXHIP_BIN_MUL, ADD = ITEXHIP_BIN_ADD;
+  if constexpr (NB == 0) {
+    store_rows<OUT_T, NB, ROWB, ADD, ADD>(acc, s, lane, o);
+  } else if constexpr (NB == 1) {
+    if (s.alg[0] == MUL) store_rows<OUT_T, NB, ROWB, MUL, ADD>(acc, s, lane, o);
+    else store_rows<OUT_T, NB, ROWB, ADD, ADD>(acc, s, lane, o);
+  } else {
+    if (s.alg[0] == MUL && s.alg[1] == MUL) store_rows<OUT_T, NB, ROWB, MUL, MUL>(acc, s, lane, o);
+    else if (s.alg[0] == MUL) store_rows<OUT_T, NB, ROWB, MUL, ADD>(acc, s, lane, o);
+    else if (s.alg[1] == MUL) store_rows<OUT_T, NB, ROWB, ADD, MUL>(acc, s, lane, o);
+    else store_rows<OUT_T, NB, ROWB, ADD, ADD>(acc, s, lane, o);
   }
 }
 
 // What a workgroup does once it knows where its operands and results are; one straight-line instance per
 // (number of fused operands, output type).
-template <bool ADJ_X, bool ADJ_Y, bool VEC_X, bool VEC_Y, int NB, int OUT_T>
+template <bool ADJ_X, bool ADJ_Y, bool VEC_X, bool VEC_Y, int NB, int OUT_T, bool ROWB>
 __device__ __forceinline__ void bmm_body(const itexhip_bmm_params& p, const int8_t* __restrict__ xb,
                                          const int8_t* __restrict__ yb, int m0, int n0, int wm, int wn, int t, int lane,
                                          const QuadrantSite& s, uint8_t* __restrict__ xs, uint8_t* __restrict__ ys) {
@@ -161,8 +205,8 @@ __device__ __forceinline__ void bmm_body(const itexhip_bmm_params& p, const int8
   uint32_t wx[4], wy[4];
   fetch_tile<!ADJ_X, VEC_X>(xb, p.M, p.K, m0, 0, t, wx);  // x is [M, K] unless adj_x
   fetch_tile<ADJ_Y, VEC_Y>(yb, p.N, p.K, n0, 0, t, wy);   // y is [N, K] only with adj_y
-  float o[ITEXHIP_BMM_MAX_BINARY][16];
-  fetch_operands<OUT_T, NB>(s, lane, o);
+  float o[ITEXHIP_BMM_MAX_BINARY][ROWB ? 1 : 16];
+  fetch_operands<OUT_T, NB, ROWB>(s, lane, o);
 
   v16i acc;
 #pragma unroll
@@ -185,10 +229,13 @@ __device__ __forceinline__ void bmm_body(const itexhip_bmm_params& p, const int8
     }
     __syncthreads();
   }
-  store_quadrant<OUT_T, NB>(acc, s, lane, o);
+  store_quadrant<OUT_T, NB, ROWB>(acc, s, lane, o);
 }
 
-template <bool ADJ_X, bool ADJ_Y, bool VEC_X, bool VEC_Y>
+// One kernel per (layouts, number of fused operands, output type, operands independent of the row): compiled as one
+// kernel with a switch over these, every variant took the registers of the largest (112 - 140, three or four
+// wavefronts per SIMD; P.V over 128 sequences 18.7 -> 16.4 us as a kernel of its own).
+template <bool ADJ_X, bool ADJ_Y, bool VEC_X, bool VEC_Y, int NB, int OUT_T, bool ROWB>
 __global__ __launch_bounds__(kBmmThreads) void qbmm_kernel(const BmmArgs a, const int8_t* __restrict__ x,
                                                            const int8_t* __restrict__ y, void* __restrict__ out) {
   __shared__ __attribute__((aligned(16))) uint8_t xs[kTile * kLdsStride];
@@ -198,24 +245,43 @@ __global__ __launch_bounds__(kBmmThreads) void qbmm_kernel(const BmmArgs a, cons
   const int wave = __builtin_amdgcn_readfirstlane(t >> 6);  // the same for the whole wavefront: keep it scalar
   const int wm = wave >> 1, wn = wave & 1;
 
-  // workgroup -> (batch entry, tile); consecutive workgroups walk the tiles of one matrix.  The launch
-  // has fewer than 2^31 workgroups, so 32-bit arithmetic covers the decomposition.
-  const uint32_t tiles = static_cast<uint32_t>(a.tiles_m) * static_cast<uint32_t>(a.tiles_n);
-  const uint32_t bi = blockIdx.x / tiles;
-  const uint32_t tile = blockIdx.x - bi * tiles;
-  const int m0 = static_cast<int>(tile / a.tiles_n) * kTile, n0 = static_cast<int>(tile % a.tiles_n) * kTile;
+  // workgroup -> (batch entry, tile); consecutive workgroups walk the tiles of one matrix.  Launched as a 3-d grid
+  // (whenever its extents allow) the innermost batch index and the product of the others come from the workgroup id;
+  // otherwise, and for more than two batch dimensions, divisions find them.  The launch has fewer than 2^31
+  // workgroups, so 32-bit arithmetic covers the decomposition.
+  const uint32_t tile = a.grid3 ? blockIdx.x : blockIdx.x % (static_cast<uint32_t>(a.tiles_m) * static_cast<uint32_t>(a.tiles_n));
+  const int tm = a.tiles_n == 1 ? static_cast<int>(tile) : static_cast<int>(tile / a.tiles_n);
+  const int m0 = tm * kTile, n0 = static_cast<int>(tile - tm * a.tiles_n) * kTile;
 
   int64_t xo = 0, yo = 0, bo[ITEXHIP_BMM_MAX_BINARY] = {0, 0};
+  uint32_t bi;  // index of the output matrix
   {
-    uint32_t rem = bi;
-    for (int d = p.n_batch_dims - 1; d >= 0; --d) {
+    int d = p.n_batch_dims - 1;
+    uint32_t rem;
+    if (a.grid3) {
+      if (d >= 0) {  // the innermost batch dimension: blockIdx.y
+        const int64_t i = blockIdx.y;
+        xo = i * p.x_batch_stride[d];
+        yo = i * p.y_batch_stride[d];
+#pragma unroll
+        for (int b = 0; b < NB; ++b) bo[b] = i * p.binary[b].batch_stride[d];
+        --d;
+      }
+      rem = blockIdx.z;
+      bi = blockIdx.z * gridDim.y + blockIdx.y;
+    } else {
+      bi = blockIdx.x / (static_cast<uint32_t>(a.tiles_m) * static_cast<uint32_t>(a.tiles_n));
+      rem = bi;
+    }
+    for (; d >= 0; --d) {
       const uint32_t dim = static_cast<uint32_t>(p.batch_dims[d]);
       const uint32_t q = d == 0 ? 0 : rem / dim;   // the outermost index needs no division
       const int64_t i = rem - q * dim;
       rem = q;
       xo += i * p.x_batch_stride[d];
       yo += i * p.y_batch_stride[d];
-      for (int b = 0; b < p.n_binary; ++b) bo[b] += i * p.binary[b].batch_stride[d];
+#pragma unroll
+      for (int b = 0; b < NB; ++b) bo[b] += i * p.binary[b].batch_stride[d];
     }
   }
 
@@ -230,7 +296,8 @@ __global__ __launch_bounds__(kBmmThreads) void qbmm_kernel(const BmmArgs a, cons
   s.cols_left = live ? static_cast<int>(p.N - qn < 32 ? p.N - qn : 32) : 0;
   s.scale = p.scale;
   s.n_binary = p.n_binary;
-  for (int b = 0; b < ITEXHIP_BMM_MAX_BINARY; ++b) {
+#pragma unroll
+  for (int b = 0; b < NB; ++b) {
     s.alg[b] = p.binary[b].alg;
     s.operand[b] = static_cast<const char*>(p.binary[b].data) +
                    (bo[b] + qm * p.binary[b].stride_m + qn * p.binary[b].stride_n) * esz;
@@ -240,28 +307,35 @@ __global__ __launch_bounds__(kBmmThreads) void qbmm_kernel(const BmmArgs a, cons
   s.out = static_cast<char*>(out) + ((static_cast<int64_t>(bi) * p.M + qm) * p.N + qn) * esz;
   s.out_row = static_cast<uint32_t>(p.N) * esz;
 
-#define ITEXHIP_BMM_BODY(NB, T) bmm_body<ADJ_X, ADJ_Y, VEC_X, VEC_Y, NB, T>(p, x + xo, y + yo, m0, n0, wm, wn, t, lane, s, xs, ys)
-  const int variant = p.n_binary * 3 + (p.out_type == ITEXHIP_FLOAT ? 0 : p.out_type == ITEXHIP_BFLOAT16 ? 1 : 2);
-  switch (variant) {
-    case 0: ITEXHIP_BMM_BODY(0, ITEXHIP_FLOAT); break;
-    case 1: ITEXHIP_BMM_BODY(0, ITEXHIP_BFLOAT16); break;
-    case 2: ITEXHIP_BMM_BODY(0, ITEXHIP_HALF); break;
-    case 3: ITEXHIP_BMM_BODY(1, ITEXHIP_FLOAT); break;
-    case 4: ITEXHIP_BMM_BODY(1, ITEXHIP_BFLOAT16); break;
-    case 5: ITEXHIP_BMM_BODY(1, ITEXHIP_HALF); break;
-    case 6: ITEXHIP_BMM_BODY(2, ITEXHIP_FLOAT); break;
-    case 7: ITEXHIP_BMM_BODY(2, ITEXHIP_BFLOAT16); break;
-    default: ITEXHIP_BMM_BODY(2, ITEXHIP_HALF); break;
+  bmm_body<ADJ_X, ADJ_Y, VEC_X, VEC_Y, NB, OUT_T, ROWB>(p, x + xo, y + yo, m0, n0, wm, wn, t, lane, s, xs, ys);
+}
+
+template <bool ADJ_X, bool ADJ_Y, int NB, int OUT_T, bool ROWB>
+void launch_vec(const BmmArgs& a, const int8_t* x, const int8_t* y, void* out, dim3 grid, hipStream_t st) {
+  if (a.vec_x && a.vec_y) qbmm_kernel<ADJ_X, ADJ_Y, true, true, NB, OUT_T, ROWB><<<grid, kBmmThreads, 0, st>>>(a, x, y, out);
+  else if (a.vec_x) qbmm_kernel<ADJ_X, ADJ_Y, true, false, NB, OUT_T, ROWB><<<grid, kBmmThreads, 0, st>>>(a, x, y, out);
+  else if (a.vec_y) qbmm_kernel<ADJ_X, ADJ_Y, false, true, NB, OUT_T, ROWB><<<grid, kBmmThreads, 0, st>>>(a, x, y, out);
+  else qbmm_kernel<ADJ_X, ADJ_Y, false, false, NB, OUT_T, ROWB><<<grid, kBmmThreads, 0, st>>>(a, x, y, out);
+}
+
+template <bool ADJ_X, bool ADJ_Y, int OUT_T>
+void launch_operands(const BmmArgs& a, const int8_t* x, const int8_t* y, void* out, dim3 grid, hipStream_t st) {
+  bool rowb = true;  // no fused operand depends on the row
+  for (int b = 0; b < a.p.n_binary; ++b) rowb = rowb && a.p.binary[b].stride_m == 0;
+  switch (a.p.n_binary * 2 + (rowb ? 1 : 0)) {
+    case 2: launch_vec<ADJ_X, ADJ_Y, 1, OUT_T, false>(a, x, y, out, grid, st); break;
+    case 3: launch_vec<ADJ_X, ADJ_Y, 1, OUT_T, true>(a, x, y, out, grid, st); break;
+    case 4: launch_vec<ADJ_X, ADJ_Y, 2, OUT_T, false>(a, x, y, out, grid, st); break;
+    case 5: launch_vec<ADJ_X, ADJ_Y, 2, OUT_T, true>(a, x, y, out, grid, st); break;
+    default: launch_vec<ADJ_X, ADJ_Y, 0, OUT_T, false>(a, x, y, out, grid, st); break;
   }
-#undef ITEXHIP_BMM_BODY
 }
 
 template <bool ADJ_X, bool ADJ_Y>
-void launch_layout(const BmmArgs& a, const int8_t* x, const int8_t* y, void* out, unsigned grid, hipStream_t st) {
-  if (a.vec_x && a.vec_y) qbmm_kernel<ADJ_X, ADJ_Y, true, true><<<grid, kBmmThreads, 0, st>>>(a, x, y, out);
-  else if (a.vec_x) qbmm_kernel<ADJ_X, ADJ_Y, true, false><<<grid, kBmmThreads, 0, st>>>(a, x, y, out);
-  else if (a.vec_y) qbmm_kernel<ADJ_X, ADJ_Y, false, true><<<grid, kBmmThreads, 0, st>>>(a, x, y, out);
-  else qbmm_kernel<ADJ_X, ADJ_Y, false, false><<<grid, kBmmThreads, 0, st>>>(a, x, y, out);
+void launch_layout(const BmmArgs& a, const int8_t* x, const int8_t* y, void* out, dim3 grid, hipStream_t st) {
+  if (a.p.out_type == ITEXHIP_FLOAT) launch_operands<ADJ_X, ADJ_Y, ITEXHIP_FLOAT>(a, x, y, out, grid, st);
+  else if (a.p.out_type == ITEXHIP_BFLOAT16) launch_operands<ADJ_X, ADJ_Y, ITEXHIP_BFLOAT16>(a, x, y, out, grid, st);
+  else launch_operands<ADJ_X, ADJ_Y, ITEXHIP_HALF>(a, x, y, out, grid, st);
 }
 
 // An operand's matrices may be read with aligned vector loads when every matrix starts on the vector
@@ -341,7 +415,12 @@ extern "C" int itexhip_qbatch_matmul(const itexhip_bmm_params* p, const int8_t* 
   a.vec_x = p->adj_x ? vector_layout(x, p->x_batch_stride, p->n_batch_dims, p->M, 4) : vector_layout(x, p->x_batch_stride, p->n_batch_dims, p->K, 16);
   a.vec_y = p->adj_y ? vector_layout(y, p->y_batch_stride, p->n_batch_dims, p->K, 16) : vector_layout(y, p->y_batch_stride, p->n_batch_dims, p->N, 4);
   hipStream_t st = as_stream(stream);
-  const unsigned g = static_cast<unsigned>(grid);
+  // (tiles of a matrix, innermost batch dimension, product of the other batch dimensions) when the extents fit a grid
+  const int64_t tiles = static_cast<int64_t>(a.tiles_m) * a.tiles_n;
+  const int64_t inner = a.p.n_batch_dims > 0 ? a.p.batch_dims[a.p.n_batch_dims - 1] : 1;
+  a.grid3 = inner <= 65535 && batch / inner <= 65535 ? 1 : 0;
+  const dim3 g = a.grid3 ? dim3(static_cast<unsigned>(tiles), static_cast<unsigned>(inner), static_cast<unsigned>(batch / inner))
+                         : dim3(static_cast<unsigned>(grid));
   if (p->adj_x && p->adj_y) launch_layout<true, true>(a, x, y, out, g, st);
   else if (p->adj_x) launch_layout<true, false>(a, x, y, out, g, st);
   else if (p->adj_y) launch_layout<false, true>(a, x, y, out, g, st);
