@@ -369,8 +369,10 @@ def bench_conv(torch, hip, timer, steps, warmup, dev):
     g_ = torch.Generator(device=dev)
     g_.manual_seed(50)
     st = _stream(torch)
-    # (the first layer of ResNet-50 has 3 input channels: patch matrix, rows padded from 147 to 160 bytes)
+    # (the first layer of ResNet-50 has 3 input channels: the op kernel copies the input to 4 channels with the spatial
+    # padding in place and gathers pixel runs from the copy; before, the patch matrix with rows padded from 147 to 160 bytes)
     for name, (B, H, W, C), (KH, KW, O), stride, patches in (
+            ("conv7x7s2_224x224x3_to_64", (32, 224, 224, 3), (7, 7, 64), 2, "narrow"),
             ("conv7x7s2_224x224x3_to_64_patch_matrix", (32, 224, 224, 3), (7, 7, 64), 2, True),
             ("conv3x3_56x56x64_to_64", (32, 56, 56, 64), (3, 3, 64), 1, False),
             ("conv3x3_56x56x64_to_64_patch_matrix", (32, 56, 56, 64), (3, 3, 64), 1, True),
@@ -394,12 +396,27 @@ def bench_conv(torch, hip, timer, steps, warmup, dev):
         y = torch.empty((M, O), dtype=torch.uint8, device=dev)
         pad = max((OH - 1) * stride + KH - H, 0) // 2       # SAME: the smaller half leads
         geo = hip.ConvGeometry(B, H, W, C, KH, KW, OH, OW, stride, stride, 1, 1, pad, pad)
-        cols = torch.empty((M, Kp), dtype=torch.uint8, device=dev) if patches else None
+        cols = torch.empty((M, Kp), dtype=torch.uint8, device=dev) if patches is True else None
         implicit = KH * KW > 1 and not patches
         assert not implicit or hip.qconv2d_implicit_ok(geo, x, O, hip.QUINT8, y)
+        if patches == "narrow":   # 4 channels, window rows of 8 pixels = 32 bytes, padding written into the copy
+            Cn, KWn = 4, 8
+            Hn, Wn = max(pad + H, (OH - 1) * stride + KH), max(pad + W, (OW - 1) * stride + KWn)
+            xn = torch.empty((B, Hn, Wn, Cn), dtype=torch.uint8, device=dev)
+            wn = torch.empty((KH, KWn, Cn, O), dtype=torch.int8, device=dev)
+            hip.pad_nhwc8(w, KH, KW, C, O, 0, 0, KWn, Cn, O, wn, st)
+            Kn = KH * KWn * Cn
+            packed_n = torch.empty(hip.qgemm_packed_bytes(Kn, O), dtype=torch.int8, device=dev)
+            hip.qgemm_prepack_b(wn, False, Kn, O, packed_n, colsum, st)
+            geo_n = hip.ConvGeometry(B, Hn, Wn, Cn, KH, KWn, OH, OW, stride, stride, 1, 1, 0, 0)
+            assert hip.qconv2d_implicit_ok(geo_n, xn, O, hip.QUINT8, y)
 
         def make(stream):
             def fn(i):
+                if patches == "narrow":
+                    hip.pad_nhwc8(x, B, H, W, C, pad, pad, Hn, Wn, Cn, xn, stream)
+                    hip.qconv2d(xn, hip.QUINT8, geo_n, packed_n, colsum, O, scales, bias, ep, hip.QUINT8, y, stream)
+                    return
                 if implicit:
                     hip.qconv2d(x, hip.QUINT8, geo, packed, colsum, O, scales, bias, ep, hip.QUINT8, y, stream)
                     return
@@ -415,7 +432,8 @@ def bench_conv(torch, hip, timer, steps, warmup, dev):
         t_roof = max(ops / (PEAK_INT8_TOPS * 1e12), nbytes / (PEAK_HBM_GBS * 1e9))
         out.append(dict(name=name, M=M, K=K, N=O, us_kernel=ms * 1e3, bytes=nbytes, ops=ops, bound="max(mfma,hbm)",
                         frac=t_roof / (ms * 1e-3), tops=ops / (ms * 1e-3) / 1e12, gbs=nbytes / (ms * 1e-3) / 1e9,
-                        note="implicit GEMM, one launch" if implicit else "im2col + GEMM launches" if patches else "GEMM launch only"))
+                        note="channel- and window-padded copy + implicit GEMM, two launches" if patches == "narrow" else
+                        "implicit GEMM, one launch" if implicit else "im2col + GEMM launches" if patches else "GEMM launch only"))
         del x, w, packed, y, cols
     # depthwise 3x3 (MobileNet shapes): no matrix product, bound by input + output bytes
     for name, (B, H, W, C) in (("dwconv3x3_112x112x32", (32, 112, 112, 32)), ("dwconv3x3_56x56x128", (32, 56, 56, 128))):

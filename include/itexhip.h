@@ -422,6 +422,16 @@ typedef struct {
 /* cols: [batch * out_h * out_w, row_bytes] bytes; row_bytes >= k_h * k_w * in_c, a multiple of 16; the tail of
  * every row is zero-filled.  1-byte elements (qint8 / quint8). */
 int itexhip_im2col8(const void* x, const itexhip_conv_geometry* g, int64_t row_bytes, void* cols, void* stream);
+/* Zero-padded copy of a 4-d tensor of 1-byte elements: out[n][oh][ow][oc] = x[n][oh - lead_h][ow - lead_w][oc] where
+ * that element exists, else 0; out is [n, out_h, out_w, out_c] with out_h >= lead_h + h, out_w >= lead_w + w,
+ * out_c >= c a multiple of 4.  What a convolution with fewer than 16 input channels (the first layer of a vision
+ * network: in_c = 3) needs to run as an implicit GEMM: the NHWC input padded to 4 (or 8) channels together with the
+ * window's spatial padding, and the HWIO filter (as the 4-d tensor [k_h, k_w, in_c, out_c]: n = k_h, h = k_w, w = in_c)
+ * padded to the same channel count and to a window row of a multiple of 16 bytes; the padding bytes are zero on both
+ * sides, so the integer sums are those of the reference's convolution (conv_ops.h:615-1150 over the oneDNN primitive,
+ * which pads implicitly). */
+int itexhip_pad_nhwc8(const void* x, int64_t n, int64_t h, int64_t w, int64_t c, int64_t lead_h, int64_t lead_w,
+                      int64_t out_h, int64_t out_w, int64_t out_c, void* out, void* stream);
 /* out[j] = float(bias[j]) * factors[n_factors == 1 ? 0 : j], j < n: the reorder with source scales that the
  * reference applies to the bias (quantized_conv_ops.h:560-590).  bias_type ITEXHIP_FLOAT or ITEXHIP_QINT32. */
 int itexhip_scale_vector(const void* bias, int bias_type, const float* factors, int64_t n_factors, int64_t n,
@@ -440,7 +450,8 @@ int itexhip_qdepthwise_conv2d(const void* x, int x_type, const itexhip_conv_geom
  * NHWC input (an implicit GEMM; it stands where the reference executes its oneDNN
  * convolution primitive, conv_ops.h:1021, 1119), same arguments otherwise as itexhip_qgemm with M = batch * out_h * out_w and
  * K = k_h * k_w * in_c; `packed_filter` / `colsum` from itexhip_qgemm_prepack_b(filter, 0, K, out_channels, ...).
- * Takes the calls for which itexhip_qconv2d_implicit_ok returns 1 (in_c a multiple of 16, k_h * k_w * in_c <= 16384,
+ * Takes the calls for which itexhip_qconv2d_implicit_ok returns 1 (in_c a multiple of 16, or in_c 4 / 8 with no window
+ * in the padding, no dilation along the row and k_w * in_c a multiple of 16; k_h * k_w * in_c <= 16384,
  * 16-byte aligned input of less than 2 GiB; output qint32 / qint8 / quint8 / float / bfloat16 with 16-byte aligned
  * rows) and rejects the others, which go through itexhip_im2col8 + itexhip_qgemm.  `bias` must not be null. */
 int itexhip_qconv2d_implicit_ok(const itexhip_conv_geometry* g, const void* x, int64_t out_channels, int out_type,

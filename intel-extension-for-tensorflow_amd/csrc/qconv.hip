@@ -52,6 +52,30 @@ __global__ __launch_bounds__(256) void im2col8_kernel(const Im2colArgs a, const 
   }
 }
 
+// Zero-padded copy of a 4-d tensor of bytes: out[n][h][w][c] = x[n][h - lead_h][w - lead_w][c] where that exists, else 0.
+// One thread per 4 output bytes (out_c is a multiple of 4, so they belong to one pixel).
+struct Pad4dArgs {
+  int n, h, w, c, lead_h, lead_w, out_h, out_w, out_c;
+  uint32_t total;  // output dwords
+};
+__global__ __launch_bounds__(256) void pad_nhwc8_kernel(const Pad4dArgs a, const uint8_t* __restrict__ x, uint32_t* __restrict__ out) {
+  const uint32_t i = blockIdx.x * 256u + threadIdx.x;
+  if (i >= a.total) return;
+  const uint32_t per_pixel = static_cast<uint32_t>(a.out_c) >> 2;
+  const uint32_t pixel = i / per_pixel, c0 = (i - pixel * per_pixel) * 4;
+  const uint32_t row = pixel / static_cast<uint32_t>(a.out_w), ow = pixel - row * static_cast<uint32_t>(a.out_w);
+  const uint32_t n = row / static_cast<uint32_t>(a.out_h), oh = row - n * static_cast<uint32_t>(a.out_h);
+  const int ih = static_cast<int>(oh) - a.lead_h, iw = static_cast<int>(ow) - a.lead_w;
+  uint32_t v = 0;
+  if (ih >= 0 && ih < a.h && iw >= 0 && iw < a.w) {
+    const uint8_t* src = x + ((static_cast<int64_t>(n) * a.h + ih) * a.w + iw) * a.c;
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+      if (static_cast<int>(c0) + e < a.c) v |= static_cast<uint32_t>(src[c0 + e]) << (8 * e);
+  }
+  out[i] = v;
+}
+
 // Few input channels (the first layer of a network: in_c = 3): every byte of a patch row may come from another pixel,
 // so the window offsets are tabulated per byte of the row once per workgroup (LDS), a thread decomposes only its row
 // index (32-bit), gathers its 4 bytes unconditionally from clamped positions and zeroes those in the padding.
@@ -486,6 +510,31 @@ extern "C" int itexhip_im2col8(const void* x, const itexhip_conv_geometry* g, in
   const int64_t blocks = std::min<int64_t>((a.total + 255) / 256, 256 * 32);
   im2col8_kernel<<<static_cast<unsigned>(blocks), 256, 0, as_stream(stream)>>>(a, static_cast<const uint8_t*>(x),
                                                                                 static_cast<uint32_t*>(cols));
+  ITEXHIP_CHECK_LAUNCH(who);
+  return ITEXHIP_OK;
+}
+
+extern "C" int itexhip_pad_nhwc8(const void* x, int64_t n, int64_t h, int64_t w, int64_t c, int64_t lead_h, int64_t lead_w,
+                                 int64_t out_h, int64_t out_w, int64_t out_c, void* out, void* stream) {
+  const char* who = "itexhip_pad_nhwc8";
+  ITEXHIP_REQUIRE(n >= 0 && h >= 0 && w >= 0 && c >= 0 && lead_h >= 0 && lead_w >= 0, "%s: negative extent", who);
+  ITEXHIP_REQUIRE(out_h >= lead_h + h && out_w >= lead_w + w && out_c >= c, "%s: the output must hold the input behind its leading padding", who);
+  ITEXHIP_REQUIRE(out_c % 4 == 0, "%s: out_c must be a multiple of 4", who);
+  const int64_t lim = 1LL << 31;
+  ITEXHIP_REQUIRE(n < lim && h < lim && w < lim && c < lim && out_h < lim && out_w < lim && out_c < lim, "%s: extent too large", who);
+  const int64_t total = n * out_h * out_w * out_c / 4;  // factors below 2^31 each; the product is checked next
+  ITEXHIP_REQUIRE(n == 0 || out_h == 0 || out_w == 0 || out_c == 0 || (n * out_h < lim && n * out_h * out_w < lim && total < lim),
+                  "%s: the padded tensor must stay below 2^31 dwords", who);
+  if (total == 0) return ITEXHIP_OK;
+  ITEXHIP_REQUIRE(out != nullptr && aligned(out, 4), "%s: null or misaligned output", who);
+  ITEXHIP_REQUIRE(x != nullptr || n * h * w * c == 0, "%s: null input", who);
+  Pad4dArgs a;
+  a.n = static_cast<int>(n); a.h = static_cast<int>(h); a.w = static_cast<int>(w); a.c = static_cast<int>(c);
+  a.lead_h = static_cast<int>(lead_h); a.lead_w = static_cast<int>(lead_w);
+  a.out_h = static_cast<int>(out_h); a.out_w = static_cast<int>(out_w); a.out_c = static_cast<int>(out_c);
+  a.total = static_cast<uint32_t>(total);
+  pad_nhwc8_kernel<<<static_cast<unsigned>((total + 255) / 256), 256, 0, as_stream(stream)>>>(a, static_cast<const uint8_t*>(x),
+                                                                                              static_cast<uint32_t*>(out));
   ITEXHIP_CHECK_LAUNCH(who);
   return ITEXHIP_OK;
 }

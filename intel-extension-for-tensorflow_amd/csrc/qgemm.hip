@@ -669,7 +669,16 @@ bool conv_implicit_ok(const itexhip_conv_geometry* g, const void* x, int64_t out
     return false;
   const int64_t K = g->k_h * g->k_w * g->in_c;
   const int64_t lim = 1LL << 31;
-  return g->in_c % 16 == 0 && K / 16 <= kMaxConvPieces && aligned(x, 16) && g->batch * g->in_h * g->in_w * g->in_c < lim &&
+  // A 16-byte piece of a patch row must be 16 contiguous input bytes that exist (or lie in the padding) as a whole.
+  // With in_c a multiple of 16 a piece is part of one pixel.  With 4 or 8 channels it is a run of 4 or 2 pixels of one
+  // window row: contiguous without dilation along the row, whole runs when the window row is a multiple of 16 bytes, and
+  // never cut by the edge of the input when no window needs padding (the caller pads the input itself: itexhip_pad_nhwc8).
+  const bool pixel_pieces = g->in_c % 16 == 0;
+  const bool run_pieces = (g->in_c == 4 || g->in_c == 8) && (g->k_w * g->in_c) % 16 == 0 && g->dil_w == 1 &&
+                          g->pad_top == 0 && g->pad_left == 0 &&
+                          (g->out_h - 1) * g->stride_h + (g->k_h - 1) * g->dil_h + 1 <= g->in_h &&
+                          (g->out_w - 1) * g->stride_w + g->k_w <= g->in_w;
+  return (pixel_pieces || run_pieces) && K / 16 <= kMaxConvPieces && aligned(x, 16) && g->batch * g->in_h * g->in_w * g->in_c < lim &&
          g->batch * g->out_h * g->out_w < lim && (g->k_h - 1) * g->dil_h < (1 << 15) && (g->k_w - 1) * g->dil_w < (1 << 15) &&
          g->pad_top >= 0 && g->pad_left >= 0 && g->pad_top < (1 << 24) && g->pad_left < (1 << 24) &&
          g->out_h * g->stride_h < (1LL << 30) && g->out_w * g->stride_w < (1LL << 30);
@@ -687,8 +696,9 @@ int qconv2d_impl(const char* who, const void* x, int x_type, const itexhip_conv_
                  const itexhip_epilogue* ep, const void* addend, int addend_type, int out_type, void* out, void* stream) {
   ITEXHIP_REQUIRE(g != nullptr, "%s: null geometry", who);
   ITEXHIP_REQUIRE(conv_implicit_ok(g, x, out_channels, out_type, out),
-                  "%s: not a shape for the implicit GEMM (in_c %% 16 == 0, window <= 16 KiB, 16-byte aligned input below 2 GiB, "
-                  "16-byte aligned output rows); use itexhip_im2col8 + itexhip_qgemm", who);
+                  "%s: not a shape for the implicit GEMM (in_c %% 16 == 0, or 4 / 8 channels with unpadded windows whose rows are "
+                  "a multiple of 16 bytes; window <= 16 KiB, 16-byte aligned input below 2 GiB, 16-byte aligned output rows); "
+                  "use itexhip_im2col8 + itexhip_qgemm", who);
   ITEXHIP_REQUIRE(bias != nullptr, "%s: needs a bias vector (zeros when the op has none)", who);
   const int64_t M = g->batch * g->out_h * g->out_w, K = g->k_h * g->k_w * g->in_c, N = out_channels;
   if (int st = check_common(x, x_type, packed_filter, M, K, N, scales, ep, out_type, out, who, addend, addend_type)) return st;

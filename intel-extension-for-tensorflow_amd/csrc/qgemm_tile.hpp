@@ -68,10 +68,12 @@ inline int xcd_rectangles(int num_m, int num_n, int BM, int BN, int K) {
   return (lg + 1) | (sm << 3) | (sn << 9) | (((4096 + sm - 1) / sm) << 15);
 }
 
-// Implicit GEMM of a Conv2D (NHWC input, in_c a multiple of 16): the activation "matrix" is the patch matrix
-// [batch * out_h * out_w, k_h * k_w * in_c], never materialised.  A 16-byte piece of a patch row lies inside one
-// input pixel (or in the padding, then it is read from 16 zero bytes), so only the source address of an activation
-// load changes: row -> window origin once per kernel, piece -> offset inside the window from a table in LDS.
+// Implicit GEMM of a Conv2D (NHWC input): the activation "matrix" is the patch matrix
+// [batch * out_h * out_w, k_h * k_w * in_c], never materialised.  With in_c a multiple of 16 a 16-byte piece of a patch
+// row lies inside one input pixel (or in the padding, then it is read from 16 zero bytes); with 4 or 8 channels it is a
+// run of 4 or 2 pixels of one window row, which the host admits only where no window touches the padding.  Either way
+// only the source address of an activation load changes: row -> window origin once per kernel, piece -> offset inside
+// the window from a table in LDS.
 struct NoConvArgs {};
 template <bool CONV> struct conv_args_of { using type = NoConvArgs; };
 template <> struct conv_args_of<true> { using type = ConvTileArgs; };

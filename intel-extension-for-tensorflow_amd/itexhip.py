@@ -32,7 +32,7 @@ EXPORTS = [
     "itexhip_requantize", "itexhip_minmax_i32_per_channel", "itexhip_minmax_f32",
     "itexhip_qmatmul_epilogue_desc", "itexhip_qmatmul_prepare", "itexhip_qgemm_packed_bytes",
     "itexhip_qgemm_prepack_b", "itexhip_qgemm", "itexhip_qgemm_tile", "itexhip_qgemv", "itexhip_qmatmul", "itexhip_qmatmul_per_row", "itexhip_qmatmul_device_range", "itexhip_quantize_dynamic", "itexhip_quantize_dynamic_static", "itexhip_quantize_dynamic_rows", "itexhip_qmatmul_unpacked", "itexhip_mfma_probe", "itexhip_read_probe",
-    "itexhip_qgemm_naive", "itexhip_qbatch_matmul", "itexhip_transpose", "itexhip_im2col8", "itexhip_scale_vector",
+    "itexhip_qgemm_naive", "itexhip_qbatch_matmul", "itexhip_transpose", "itexhip_im2col8", "itexhip_pad_nhwc8", "itexhip_scale_vector",
     "itexhip_qconv2d_implicit_ok", "itexhip_qconv2d", "itexhip_qgemm_sum", "itexhip_qconv2d_sum", "itexhip_qdepthwise_conv2d",
 ]
 
@@ -363,6 +363,11 @@ class ConvGeometry(C.Structure):
 
 def im2col8(x, geometry, row_bytes, cols, stream=0):
     _check(_lib.itexhip_im2col8(_ptr(x), C.byref(geometry), _i64(row_bytes), _ptr(cols), _ptr(stream)))
+
+
+def pad_nhwc8(x, n, h, w, c, lead_h, lead_w, out_h, out_w, out_c, out, stream=0):
+    _check(_lib.itexhip_pad_nhwc8(_ptr(x), _i64(n), _i64(h), _i64(w), _i64(c), _i64(lead_h), _i64(lead_w), _i64(out_h),
+                                  _i64(out_w), _i64(out_c), _ptr(out), _ptr(stream)))
 
 
 def qconv2d_implicit_ok(geometry, x, out_channels, out_type, out):

@@ -248,17 +248,46 @@ class QuantizedConv2DOp : public OpKernel {
     }
 
     void* stream = ctx->stream();
+    // ---- fewer than 16 input channels (the first layer of a vision network): the patch rows have no 16-byte piece that
+    // lies inside one pixel.  Instead of writing the patch matrix out, the input is copied once with 4 or 8 channels and
+    // with the windows' spatial padding in place, the filter is padded to the same channel count and to a window row of
+    // a multiple of 16 bytes, and the tile kernel gathers runs of whole pixels from that copy.  All padding bytes are
+    // zero on both sides: the integer sums are unchanged.
+    itexhip_conv_geometry gn = g;
+    bool narrow = false;
+    const int64_t Cn = C <= 4 ? 4 : 8, KWn = (KW * Cn + 15) / 16 * 16 / Cn;
+    if (!depthwise_ && C > 0 && C <= 8 && dil_w_ == 1 && !transcendental_ && sum_position_ == 0 && M > 0 && O > 0 && O % 4 == 0) {
+      gn.in_c = Cn;
+      gn.k_w = KWn;
+      gn.in_h = std::max<int64_t>(g.pad_top + H, (g.out_h - 1) * stride_h_ + (KH - 1) * dil_h_ + 1);
+      gn.in_w = std::max<int64_t>(g.pad_left + W, (g.out_w - 1) * stride_w_ + KWn);
+      gn.pad_top = gn.pad_left = 0;
+      // legality without the buffers (they come 16-byte aligned from the allocator)
+      const void* aligned16 = reinterpret_cast<const void*>(static_cast<uintptr_t>(64));
+      narrow = itexhip_qconv2d_implicit_ok(&gn, aligned16, O, t_out_, aligned16) != 0;
+    }
+    const int64_t Kn = KH * KWn * Cn;
     // ---- filter: packed once when constant (the HWIO tensor read as a [K, O] matrix)
+    const int64_t pack_k = narrow ? Kn : K;
     const bool repack = !depthwise_ &&
-                        (!packed_.valid() || !is_filter_const_ || packed_src_ != filter.data() || packed_k_ != K || packed_n_ != O);
+                        (!packed_.valid() || !is_filter_const_ || packed_src_ != filter.data() || packed_k_ != pack_k || packed_n_ != O);
     if (repack && O > 0) {
-      packed_ = ctx->allocate_temp(TF_QINT8, {std::max<int64_t>(itexhip_qgemm_packed_bytes(Kp, O), 16)});
+      packed_ = ctx->allocate_temp(TF_QINT8, {std::max<int64_t>(itexhip_qgemm_packed_bytes(narrow ? Kn : Kp, O), 16)});
       colsum_ = ctx->allocate_temp(TF_INT32, {O});
       if (!ctx->ok()) return;
-      const int st = itexhip_qgemm_prepack_b(filter.flat<int8_t>(), 0, K, O, packed_.flat<int8_t>(), colsum_.flat<int32_t>(), stream);
+      const int8_t* w = filter.flat<int8_t>();
+      Tensor padded_filter;
+      if (narrow) {  // [KH, KW, C, O] -> [KH, KWn, Cn, O]
+        padded_filter = ctx->allocate_temp(TF_QINT8, {KH, KWn, Cn, O});
+        if (!ctx->ok()) return;
+        const int st = itexhip_pad_nhwc8(w, KH, KW, C, O, 0, 0, KWn, Cn, O, padded_filter.data(), stream);
+        ITEX_REQUIRES(ctx, st == ITEXHIP_OK, TF_ABORTED, std::string("Operation received an exception: ") + itexhip_last_error());
+        w = padded_filter.flat<int8_t>();
+      }
+      const int st = itexhip_qgemm_prepack_b(w, 0, pack_k, O, packed_.flat<int8_t>(), colsum_.flat<int32_t>(), stream);
       ITEX_REQUIRES(ctx, st == ITEXHIP_OK, TF_ABORTED, std::string("Operation received an exception: ") + itexhip_last_error());
       packed_src_ = filter.data();
-      packed_k_ = K;
+      packed_k_ = pack_k;
       packed_n_ = O;
     }
     std::vector<float> both(scales);
@@ -325,7 +354,23 @@ class QuantizedConv2DOp : public OpKernel {
       }
       // ---- patches, then the quantized GEMM
       const void* a = x.data();
-      Tensor cols;
+      Tensor cols, x_narrow;
+      if (narrow) {
+        x_narrow = ctx->allocate_temp(t_in_, {B, gn.in_h, gn.in_w, Cn});
+        if (!ctx->ok()) return;
+        int st = itexhip_pad_nhwc8(x.data(), B, H, W, C, g.pad_top, g.pad_left, gn.in_h, gn.in_w, Cn, x_narrow.data(), stream);
+        ITEX_REQUIRES(ctx, st == ITEXHIP_OK, TF_ABORTED, std::string("Operation received an exception: ") + itexhip_last_error());
+        ITEX_REQUIRES(ctx, itexhip_qconv2d_implicit_ok(&gn, x_narrow.data(), O, t_out_, out.data()) != 0, TF_INTERNAL,
+                      "the padded input or the output is not 16-byte aligned");
+        itexhip_epilogue epn{};
+        epn.n_scales = static_cast<int>(depth);
+        if (activation_ != 0) epn.elt[epn.n_eltwise++] = {activation_, leaky_ ? alpha_ : 0.0f, 0.0f};
+        st = itexhip_qconv2d(x_narrow.data(), t_in_, &gn, packed_.flat<int8_t>(), colsum_.flat<int32_t>(), O, params, bias_dev, &epn,
+                             t_out_, out.data(), stream);
+        ITEX_REQUIRES(ctx, st == ITEXHIP_OK, st == ITEXHIP_INVALID_ARGUMENT ? TF_INVALID_ARGUMENT : TF_ABORTED,
+                      std::string("Operation received an exception: ") + itexhip_last_error());
+      }
+      if (!narrow) {
       const bool pointwise = KH == 1 && KW == 1 && stride_h_ == 1 && stride_w_ == 1 && g.pad_top == 0 && g.pad_left == 0 &&
                              g.out_h == H && g.out_w == W && K == Kp;
       // windows the tile kernel can gather by itself (input channels a multiple of 16, ...) need no patch matrix
@@ -358,6 +403,7 @@ class QuantizedConv2DOp : public OpKernel {
       }
       ITEX_REQUIRES(ctx, st == ITEXHIP_OK, st == ITEXHIP_INVALID_ARGUMENT ? TF_INVALID_ARGUMENT : TF_ABORTED,
                     std::string("Operation received an exception: ") + itexhip_last_error());
+      }  // !narrow
       }  // !depthwise_
     }
 

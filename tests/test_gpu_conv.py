@@ -68,6 +68,102 @@ def test_scale_vector(hip, dev):
             np.testing.assert_array_equal(out.cpu().numpy(), bias.astype(np.float32) * f[0])
 
 
+@pytest.mark.parametrize("shape,lead,out_hw,out_c", [((2, 5, 7, 3), (2, 3), (9, 12), 4), ((7, 7, 3, 64), (0, 0), (8, 4), 64),
+                                                     ((1, 1, 1, 1), (0, 0), (1, 1), 4), ((3, 4, 4, 8), (1, 0), (5, 4), 8),
+                                                     ((2, 0, 3, 2), (1, 1), (2, 5), 4)])
+def test_pad_nhwc8_against_numpy(hip, dev, shape, lead, out_hw, out_c):
+    import torch
+    rng = np.random.default_rng(sum(shape))
+    x = rng.integers(1, 256, shape).astype(np.uint8)
+    n, h, w, c = shape
+    ref = np.zeros((n, out_hw[0], out_hw[1], out_c), np.uint8)
+    ref[:, lead[0]:lead[0] + h, lead[1]:lead[1] + w, :c] = x
+    xd = torch.from_numpy(x).to(dev) if x.size else torch.zeros(1, dtype=torch.uint8, device=dev)
+    out = torch.full(ref.shape, 0x55, dtype=torch.uint8, device=dev)
+    hip.pad_nhwc8(xd, n, h, w, c, lead[0], lead[1], out_hw[0], out_hw[1], out_c, out)
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(out.cpu().numpy(), ref)
+    with pytest.raises(hip.ItexHipError):
+        hip.pad_nhwc8(xd, n, h, w, c, lead[0], lead[1], out_hw[0], out_hw[1], out_c + 2, out)   # out_c % 4
+    with pytest.raises(hip.ItexHipError):
+        hip.pad_nhwc8(xd, n, h + 1, w, c, out_hw[0], lead[1], out_hw[0], out_hw[1], out_c, out)  # does not fit
+
+
+@pytest.mark.parametrize("shape,wshape,strides,dil_h,signed_in", [((2, 30, 26, 3), (7, 7, 3, 64), (2, 2), 1, False),
+                                                                  ((1, 12, 9, 4), (3, 3, 4, 32), (1, 1), 2, True),
+                                                                  ((2, 9, 9, 7), (3, 2, 7, 48), (1, 2), 1, False),
+                                                                  ((1, 6, 5, 1), (5, 5, 1, 16), (1, 1), 1, True)])
+def test_implicit_gemm_conv_few_input_channels(hip, dev, shape, wshape, strides, dil_h, signed_in):
+    """A SAME convolution with fewer than 16 input channels as the op kernel runs it: input and filter zero-padded
+    (itexhip_pad_nhwc8) to 4 / 8 channels, to the windows' spatial padding and to window rows of a multiple of 16 bytes,
+    then itexhip_qconv2d on the padded geometry; int32 accumulators against a numpy convolution of the original
+    tensors, 8-bit outputs with scales, bias and ReLU against the patch-matrix path on the original tensors."""
+    import torch
+    from tests.test_oracle_conv import ref_int_conv
+    rng = np.random.default_rng(sum(shape) + sum(wshape))
+    B, H, W, C = shape
+    kh, kw, _, O = wshape
+    x = rng.integers(-128, 128, shape).astype(np.int8) if signed_in else rng.integers(0, 256, shape).astype(np.uint8)
+    w = rng.integers(-127, 128, wshape).astype(np.int8)
+    oh, pt = same_lead(H, kh, strides[0], dil_h)
+    ow, pl = same_lead(W, kw, strides[1], 1)
+    pb = max((oh - 1) * strides[0] + (kh - 1) * dil_h + 1 - H - pt, 0)
+    pr = max((ow - 1) * strides[1] + kw - W - pl, 0)
+    ref = ref_int_conv(x, w, strides, (dil_h, 1), ((pt, pb), (pl, pr)))[:, :oh, :ow, :]
+    T_in = hip.QINT8 if signed_in else hip.QUINT8
+    cn = 4 if C <= 4 else 8
+    kwn = (kw * cn + 15) // 16 * 16 // cn
+    hp = max(pt + H, (oh - 1) * strides[0] + (kh - 1) * dil_h + 1)
+    wp = max(pl + W, (ow - 1) * strides[1] + kwn)
+    xd = torch.from_numpy(x).to(dev)
+    xp = torch.empty((B, hp, wp, cn), dtype=xd.dtype, device=dev)
+    hip.pad_nhwc8(xd, B, H, W, C, pt, pl, hp, wp, cn, xp)
+    wpad = torch.empty((kh, kwn, cn, O), dtype=torch.int8, device=dev)
+    hip.pad_nhwc8(torch.from_numpy(w).to(dev), kh, kw, C, O, 0, 0, kwn, cn, O, wpad)
+    Kn, M = kh * kwn * cn, B * oh * ow
+    gn = hip.ConvGeometry(B, hp, wp, cn, kh, kwn, oh, ow, strides[0], strides[1], dil_h, 1, 0, 0)
+    acc = torch.full((M, O), 77, dtype=torch.int32, device=dev)
+    assert hip.qconv2d_implicit_ok(gn, xp, O, hip.QINT32, acc)
+    packed = torch.empty(hip.qgemm_packed_bytes(Kn, O), dtype=torch.int8, device=dev)
+    colsum = torch.empty(O, dtype=torch.int32, device=dev)
+    hip.qgemm_prepack_b(wpad, False, Kn, O, packed, colsum)
+    one = torch.ones(1, dtype=torch.float32, device=dev)
+    zero_bias = torch.zeros(O, dtype=torch.float32, device=dev)
+    ep = hip.Epilogue()
+    ep.n_scales, ep.n_eltwise = 1, 0
+    hip.qconv2d(xp, T_in, gn, packed, colsum, O, one, zero_bias, ep, hip.QINT32, acc)
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(acc.cpu().numpy().reshape(B, oh, ow, O), ref)
+    # the patch-matrix path on the original tensors
+    K = kh * kw * C
+    Kp = (K + 15) // 16 * 16
+    g = hip.ConvGeometry(B, H, W, C, kh, kw, oh, ow, strides[0], strides[1], dil_h, 1, pt, pl)
+    cols = torch.empty((M, Kp), dtype=torch.uint8, device=dev)
+    hip.im2col8(xd, g, Kp, cols)
+    packed0 = torch.empty(hip.qgemm_packed_bytes(Kp, O), dtype=torch.int8, device=dev)
+    colsum0 = torch.empty(O, dtype=torch.int32, device=dev)
+    hip.qgemm_prepack_b(torch.from_numpy(w.reshape(K, O)).to(dev), False, K, O, packed0, colsum0)
+    scales = torch.from_numpy((rng.random(O).astype(np.float32) + 0.5) * np.float32(2e-3)).to(dev)
+    bias = torch.from_numpy(rng.standard_normal(O).astype(np.float32)).to(dev)
+    ep.n_scales, ep.n_eltwise = O, 1
+    ep.elt[0].alg, ep.elt[0].alpha, ep.elt[0].beta = hip.ELT_RELU, 0.0, 0.0
+    for T, dt in ((hip.QUINT8, torch.uint8), (hip.QINT8, torch.int8), (hip.FLOAT, torch.float32)):
+        a = torch.empty((M, O), dtype=dt, device=dev)
+        b_ = torch.empty((M, O), dtype=dt, device=dev)
+        a.view(torch.uint8).fill_(0x55)
+        b_.view(torch.uint8).fill_(0xAA)
+        hip.qconv2d(xp, T_in, gn, packed, colsum, O, scales, bias, ep, T, a)
+        hip.qgemm(cols, T_in, packed0, colsum0, M, Kp, O, scales, bias, ep, T, b_)
+        torch.cuda.synchronize()
+        assert torch.equal(a.view(torch.uint8), b_.view(torch.uint8)), T
+    # a window that needs padding, a dilated row or a window row that is not a multiple of 16 bytes is refused
+    assert not hip.qconv2d_implicit_ok(hip.ConvGeometry(B, hp, wp, cn, kh, kwn, oh, ow, strides[0], strides[1], dil_h, 1, 1, 0), xp, O, hip.QINT32, acc)
+    assert not hip.qconv2d_implicit_ok(hip.ConvGeometry(B, hp, wp, cn, kh, kwn, oh, ow, strides[0], strides[1], dil_h, 2, 0, 0), xp, O, hip.QINT32, acc)
+    assert not hip.qconv2d_implicit_ok(hip.ConvGeometry(B, hp, wp + 1, cn, kh, kwn + 1, oh, ow, strides[0], strides[1], dil_h, 1, 0, 0), xp, O, hip.QINT32, acc)
+    assert not hip.qconv2d_implicit_ok(hip.ConvGeometry(B, hp, (ow - 1) * strides[1] + kwn - 1, cn, kh, kwn, oh, ow, strides[0], strides[1], dil_h, 1, 0, 0),
+                                       xp, O, hip.QINT32, acc)
+
+
 IMPLICIT_CASES = [  # input NHWC, filter HWIO, strides, dilations, leading pads (top, left) or None for SAME
     ((2, 9, 10, 16), (3, 3, 16, 48), (1, 1), (1, 1), None),      # K = 144: a ragged last K step
     ((1, 8, 7, 32), (3, 2, 32, 64), (2, 1), (1, 2), None),       # strides + dilation
@@ -440,7 +536,12 @@ def test_new_api_conv_through_plugin(rt, dev, t_in, fused, t_out, t_bias):
     torch = rt
     cases = [((2, 10, 9, 6), (3, 3, 6, 10), [1, 1, 2, 1], [1, 2, 1, 1], "EXPLICIT", [0, 0, 2, 1, 0, 3, 0, 0]),
              ((1, 8, 8, 32), (1, 1, 32, 48), [1, 1, 1, 1], [1, 1, 1, 1], "SAME", []),
-             ((1, 14, 14, 3), (7, 7, 3, 8), [1, 2, 2, 1], [1, 1, 1, 1], "SAME", [])]
+             ((1, 14, 14, 3), (7, 7, 3, 8), [1, 2, 2, 1], [1, 1, 1, 1], "SAME", []),
+             # fewer than 16 input channels with 16-byte output rows: input and filter are padded to 4 / 8 channels and the
+             # tile kernel gathers pixel runs (first layer of ResNet-50 in small; explicit pads; dilation down the rows)
+             ((2, 23, 21, 3), (7, 7, 3, 64), [1, 2, 2, 1], [1, 1, 1, 1], "SAME", []),
+             ((1, 9, 11, 8), (3, 3, 8, 16), [1, 1, 1, 1], [1, 2, 1, 1], "EXPLICIT", [0, 0, 1, 2, 3, 0, 0, 0]),
+             ((1, 7, 7, 5), (1, 1, 5, 32), [1, 1, 1, 1], [1, 1, 1, 1], "VALID", [])]
     for shape, wshape, strides, dil, padding, explicit in cases:
         rng = np.random.default_rng(shape[1] * 3 + len(fused))
         signed = t_in == tf.QINT8
