@@ -401,7 +401,7 @@ def bench_conv(torch, hip, timer, steps, warmup, dev):
         assert not implicit or hip.qconv2d_implicit_ok(geo, x, O, hip.QUINT8, y)
         if patches == "narrow":   # 4 channels, window rows of 8 pixels = 32 bytes, padding written into the copy
             Cn, KWn = 4, 8
-            Hn, Wn = max(pad + H, (OH - 1) * stride + KH), max(pad + W, (OW - 1) * stride + KWn)
+            Hn, Wn = max(pad + H, (OH - 1) * stride + KH), (max(pad + W, (OW - 1) * stride + KWn) + 3) // 4 * 4
             xn = torch.empty((B, Hn, Wn, Cn), dtype=torch.uint8, device=dev)
             wn = torch.empty((KH, KWn, Cn, O), dtype=torch.int8, device=dev)
             hip.pad_nhwc8(w, KH, KW, C, O, 0, 0, KWn, Cn, O, wn, st)

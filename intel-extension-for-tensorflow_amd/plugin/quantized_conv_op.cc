@@ -261,6 +261,7 @@ class QuantizedConv2DOp : public OpKernel {
       gn.k_w = KWn;
       gn.in_h = std::max<int64_t>(g.pad_top + H, (g.out_h - 1) * stride_h_ + (KH - 1) * dil_h_ + 1);
       gn.in_w = std::max<int64_t>(g.pad_left + W, (g.out_w - 1) * stride_w_ + KWn);
+      gn.in_w = (gn.in_w + 16 / Cn - 1) / (16 / Cn) * (16 / Cn);  // rows of whole 16-byte vectors: the copy writes one per thread
       gn.pad_top = gn.pad_left = 0;
       // legality without the buffers (they come 16-byte aligned from the allocator)
       const void* aligned16 = reinterpret_cast<const void*>(static_cast<uintptr_t>(64));
