@@ -10,6 +10,7 @@
 // n on the lanes, so every store instruction writes 128 contiguous bytes per half-wavefront: with fp32
 // outputs the op is bound by that write.
 #include <type_traits>
+#include <utility>
 
 #include "common.hpp"
 
@@ -28,6 +29,7 @@ struct BmmArgs {
   int tiles_m, tiles_n;
   int vec_x, vec_y;  // operand layouts allow aligned vector loads
   int grid3;         // launched as (tiles, innermost batch dimension, the other batch dimensions): no division finds them
+  int rm, rn;        // the tile is (64 rm) x (64 rn)
 };
 
 // One 64 (rows or columns of the output) x 64 (k) byte tile on its way into LDS, k-contiguous there.  The
@@ -195,51 +197,117 @@ __device__ __forceinline__ void store_quadrant(const v16i& acc, const QuadrantSi
   }
 }
 
-// What a workgroup does once it knows where its operands and results are; one straight-line instance per
-// (number of fused operands, output type).
-template <bool ADJ_X, bool ADJ_Y, bool VEC_X, bool VEC_Y, int NB, int OUT_T, bool ROWB>
-__device__ __forceinline__ void bmm_body(const itexhip_bmm_params& p, const int8_t* __restrict__ xb,
-                                         const int8_t* __restrict__ yb, int m0, int n0, int wm, int wn, int t, int lane,
-                                         const QuadrantSite& s, uint8_t* __restrict__ xs, uint8_t* __restrict__ ys) {
-  // first tiles and the fused operands: all loads the results depend on are issued before any is needed
-  uint32_t wx[4], wy[4];
-  fetch_tile<!ADJ_X, VEC_X>(xb, p.M, p.K, m0, 0, t, wx);  // x is [M, K] unless adj_x
-  fetch_tile<ADJ_Y, VEC_Y>(yb, p.N, p.K, n0, 0, t, wy);   // y is [N, K] only with adj_y
-  float o[ITEXHIP_BMM_MAX_BINARY][ROWB ? 1 : 16];
-  fetch_operands<OUT_T, NB, ROWB>(s, lane, o);
+// f(integral_constant<int, 0>) ... f(integral_constant<int, N - 1>)
+template <class F, int... I>
+__device__ __forceinline__ void quadrants_impl(F&& f, std::integer_sequence<int, I...>) {
+  (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, class F>
+__device__ __forceinline__ void quadrants(F&& f) {
+  quadrants_impl(static_cast<F&&>(f), std::make_integer_sequence<int, N>{});
+}
 
-  v16i acc;
+// Where quadrant (qm, qn) of the output matrix bi goes and what its fused operands are.  A quadrant off the edge of the
+// output stores nothing (its wavefront still helps staging the tiles) and addresses the tile's first element, which
+// always exists.
+template <int NB>
+__device__ __forceinline__ QuadrantSite quadrant_site(const itexhip_bmm_params& p, const int64_t (&bo)[ITEXHIP_BMM_MAX_BINARY],
+                                                      uint32_t bi, int m0, int n0, int qm_, int qn_, void* __restrict__ out) {
+  const bool live = qm_ < p.M && qn_ < p.N;
+  const int64_t qm = live ? qm_ : m0, qn = live ? qn_ : n0;
+  const uint32_t esz = p.out_type == ITEXHIP_FLOAT ? 4 : 2;
+  QuadrantSite s;
+  s.rows_left = live ? static_cast<int>(p.M - qm < 32 ? p.M - qm : 32) : 0;
+  s.cols_left = live ? static_cast<int>(p.N - qn < 32 ? p.N - qn : 32) : 0;
+  s.scale = p.scale;
+  s.n_binary = p.n_binary;
 #pragma unroll
-  for (int i = 0; i < 16; ++i) acc[i] = 0;
+  for (int b = 0; b < NB; ++b) {
+    s.alg[b] = p.binary[b].alg;
+    s.operand[b] = static_cast<const char*>(p.binary[b].data) +
+                   (bo[b] + qm * p.binary[b].stride_m + qn * p.binary[b].stride_n) * esz;
+    s.operand_row[b] = static_cast<uint32_t>(p.binary[b].stride_m) * esz;
+    s.operand_col[b] = static_cast<uint32_t>(p.binary[b].stride_n) * esz;
+  }
+  s.out = static_cast<char*>(out) + ((static_cast<int64_t>(bi) * p.M + qm) * p.N + qn) * esz;
+  s.out_row = static_cast<uint32_t>(p.N) * esz;
+  return s;
+}
+
+// What a workgroup does once it knows where its operands are: a (64 RM) x (64 RN) output tile, each of the four
+// wavefronts RM x RN quadrants of 32 x 32.  One straight-line instance per (number of fused operands, output type).
+// The larger tiles amortise what a wavefront spends around its MFMAs (a 64 x 64 tile of K = 64 is two MFMAs and some
+// 450 other instructions per wavefront) and read each operand half as often; they exist for the calls whose fused
+// operands take one register per lane and quadrant column (none, or ROWB).
+template <bool ADJ_X, bool ADJ_Y, bool VEC_X, bool VEC_Y, int NB, int OUT_T, bool ROWB, int RM, int RN>
+__device__ __forceinline__ void bmm_body(const itexhip_bmm_params& p, const int8_t* __restrict__ xb,
+                                         const int8_t* __restrict__ yb, const int64_t (&bo)[ITEXHIP_BMM_MAX_BINARY], uint32_t bi,
+                                         int m0, int n0, int wm, int wn, int t, int lane, void* __restrict__ out,
+                                         uint8_t* __restrict__ xs, uint8_t* __restrict__ ys) {
+  static_assert(RM * RN == 1 || NB == 0 || ROWB, "larger tiles keep the operands of all their quadrants in registers");
+  // first tiles and the fused operands: all loads the results depend on are issued before any is needed
+  uint32_t wx[RM][4], wy[RN][4];
+#pragma unroll
+  for (int h = 0; h < RM; ++h) fetch_tile<!ADJ_X, VEC_X>(xb, p.M, p.K, m0 + 64 * h, 0, t, wx[h]);  // x is [M, K] unless adj_x
+#pragma unroll
+  for (int h = 0; h < RN; ++h) fetch_tile<ADJ_Y, VEC_Y>(yb, p.N, p.K, n0 + 64 * h, 0, t, wy[h]);   // y is [N, K] only with adj_y
+  // (the quadrants are walked with compile-time indices: what describes a quadrant is the same for the whole
+  // wavefront and must stay in scalar registers, which an indexed array of descriptors does not)
+  float o[RM * RN][ITEXHIP_BMM_MAX_BINARY][ROWB ? 1 : 16];
+  quadrants<RM * RN>([&](auto q) {
+    constexpr int i = decltype(q)::value / RN, j = decltype(q)::value % RN;
+    const QuadrantSite s = quadrant_site<NB>(p, bo, bi, m0, n0, m0 + (wm * RM + i) * 32, n0 + (wn * RN + j) * 32, out);
+    fetch_operands<OUT_T, NB, ROWB>(s, lane, o[decltype(q)::value]);
+  });
+
+  v16i acc[RM * RN];
+  quadrants<RM * RN>([&](auto q) {
+#pragma unroll
+    for (int e = 0; e < 16; ++e) acc[decltype(q)::value][e] = 0;
+  });
 
   for (int64_t k0 = 0; k0 < p.K; k0 += kTile) {
-    put_tile<!ADJ_X>(xs, t, wx);
-    put_tile<ADJ_Y>(ys, t, wy);
+#pragma unroll
+    for (int h = 0; h < RM; ++h) put_tile<!ADJ_X>(xs + h * 64 * kLdsStride, t, wx[h]);
+#pragma unroll
+    for (int h = 0; h < RN; ++h) put_tile<ADJ_Y>(ys + h * 64 * kLdsStride, t, wy[h]);
     __syncthreads();
     if (k0 + kTile < p.K) {  // the next tile travels while this one is multiplied
-      fetch_tile<!ADJ_X, VEC_X>(xb, p.M, p.K, m0, k0 + kTile, t, wx);
-      fetch_tile<ADJ_Y, VEC_Y>(yb, p.N, p.K, n0, k0 + kTile, t, wy);
+#pragma unroll
+      for (int h = 0; h < RM; ++h) fetch_tile<!ADJ_X, VEC_X>(xb, p.M, p.K, m0 + 64 * h, k0 + kTile, t, wx[h]);
+#pragma unroll
+      for (int h = 0; h < RN; ++h) fetch_tile<ADJ_Y, VEC_Y>(yb, p.N, p.K, n0 + 64 * h, k0 + kTile, t, wy[h]);
     }
 #pragma unroll
     for (int kk = 0; kk < 2; ++kk) {
       const int off = kk * 32 + (lane >> 5) * 16;
-      const v4i fx = *reinterpret_cast<const v4i*>(xs + (wm * 32 + (lane & 31)) * kLdsStride + off);
-      const v4i fy = *reinterpret_cast<const v4i*>(ys + (wn * 32 + (lane & 31)) * kLdsStride + off);
-      acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(fx, fy, acc, 0, 0, 0);
+      v4i fx[RM], fy[RN];
+#pragma unroll
+      for (int i = 0; i < RM; ++i) fx[i] = *reinterpret_cast<const v4i*>(xs + ((wm * RM + i) * 32 + (lane & 31)) * kLdsStride + off);
+#pragma unroll
+      for (int j = 0; j < RN; ++j) fy[j] = *reinterpret_cast<const v4i*>(ys + ((wn * RN + j) * 32 + (lane & 31)) * kLdsStride + off);
+      quadrants<RM * RN>([&](auto q) {
+        constexpr int i = decltype(q)::value / RN, j = decltype(q)::value % RN;
+        acc[decltype(q)::value] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fx[i], fy[j], acc[decltype(q)::value], 0, 0, 0);
+      });
     }
     __syncthreads();
   }
-  store_quadrant<OUT_T, NB, ROWB>(acc, s, lane, o);
+  quadrants<RM * RN>([&](auto q) {
+    constexpr int i = decltype(q)::value / RN, j = decltype(q)::value % RN;
+    const QuadrantSite s = quadrant_site<NB>(p, bo, bi, m0, n0, m0 + (wm * RM + i) * 32, n0 + (wn * RN + j) * 32, out);
+    store_quadrant<OUT_T, NB, ROWB>(acc[decltype(q)::value], s, lane, o[decltype(q)::value]);
+  });
 }
 
 // One kernel per (layouts, number of fused operands, output type, operands independent of the row): compiled as one
 // kernel with a switch over these, every variant took the registers of the largest (112 - 140, three or four
 // wavefronts per SIMD; P.V over 128 sequences 18.7 -> 16.4 us as a kernel of its own).
-template <bool ADJ_X, bool ADJ_Y, bool VEC_X, bool VEC_Y, int NB, int OUT_T, bool ROWB>
+template <bool ADJ_X, bool ADJ_Y, bool VEC_X, bool VEC_Y, int NB, int OUT_T, bool ROWB, int RM = 1, int RN = 1>
 __global__ __launch_bounds__(kBmmThreads) void qbmm_kernel(const BmmArgs a, const int8_t* __restrict__ x,
                                                            const int8_t* __restrict__ y, void* __restrict__ out) {
-  __shared__ __attribute__((aligned(16))) uint8_t xs[kTile * kLdsStride];
-  __shared__ __attribute__((aligned(16))) uint8_t ys[kTile * kLdsStride];
+  __shared__ __attribute__((aligned(16))) uint8_t xs[RM * kTile * kLdsStride];
+  __shared__ __attribute__((aligned(16))) uint8_t ys[RN * kTile * kLdsStride];
   const itexhip_bmm_params& p = a.p;
   const int t = threadIdx.x, lane = t & 63;
   const int wave = __builtin_amdgcn_readfirstlane(t >> 6);  // the same for the whole wavefront: keep it scalar
@@ -251,7 +319,7 @@ __global__ __launch_bounds__(kBmmThreads) void qbmm_kernel(const BmmArgs a, cons
   // workgroups, so 32-bit arithmetic covers the decomposition.
   const uint32_t tile = a.grid3 ? blockIdx.x : blockIdx.x % (static_cast<uint32_t>(a.tiles_m) * static_cast<uint32_t>(a.tiles_n));
   const int tm = a.tiles_n == 1 ? static_cast<int>(tile) : static_cast<int>(tile / a.tiles_n);
-  const int m0 = tm * kTile, n0 = static_cast<int>(tile - tm * a.tiles_n) * kTile;
+  const int m0 = tm * (RM * kTile), n0 = static_cast<int>(tile - tm * a.tiles_n) * (RN * kTile);
 
   int64_t xo = 0, yo = 0, bo[ITEXHIP_BMM_MAX_BINARY] = {0, 0};
   uint32_t bi;  // index of the output matrix
@@ -284,34 +352,22 @@ __global__ __launch_bounds__(kBmmThreads) void qbmm_kernel(const BmmArgs a, cons
       for (int b = 0; b < NB; ++b) bo[b] += i * p.binary[b].batch_stride[d];
     }
   }
-
-  // the quadrant of this wavefront; accumulator i of a lane is row (i / 4) * 8 + (lane / 32) * 4 + i % 4,
-  // column lane % 32 of it.  A quadrant off the edge of the output stores nothing (its wavefront still
-  // helps staging the tiles) and addresses the tile's first element, which always exists.
-  const bool live = m0 + wm * 32 < p.M && n0 + wn * 32 < p.N;
-  const int64_t qm = live ? m0 + wm * 32 : m0, qn = live ? n0 + wn * 32 : n0;
-  const uint32_t esz = p.out_type == ITEXHIP_FLOAT ? 4 : 2;
-  QuadrantSite s;
-  s.rows_left = live ? static_cast<int>(p.M - qm < 32 ? p.M - qm : 32) : 0;
-  s.cols_left = live ? static_cast<int>(p.N - qn < 32 ? p.N - qn : 32) : 0;
-  s.scale = p.scale;
-  s.n_binary = p.n_binary;
-#pragma unroll
-  for (int b = 0; b < NB; ++b) {
-    s.alg[b] = p.binary[b].alg;
-    s.operand[b] = static_cast<const char*>(p.binary[b].data) +
-                   (bo[b] + qm * p.binary[b].stride_m + qn * p.binary[b].stride_n) * esz;
-    s.operand_row[b] = static_cast<uint32_t>(p.binary[b].stride_m) * esz;
-    s.operand_col[b] = static_cast<uint32_t>(p.binary[b].stride_n) * esz;
-  }
-  s.out = static_cast<char*>(out) + ((static_cast<int64_t>(bi) * p.M + qm) * p.N + qn) * esz;
-  s.out_row = static_cast<uint32_t>(p.N) * esz;
-
-  bmm_body<ADJ_X, ADJ_Y, VEC_X, VEC_Y, NB, OUT_T, ROWB>(p, x + xo, y + yo, m0, n0, wm, wn, t, lane, s, xs, ys);
+  // accumulator e of a lane is row (e / 4) * 8 + (lane / 32) * 4 + e % 4, column lane % 32 of its quadrant
+  bmm_body<ADJ_X, ADJ_Y, VEC_X, VEC_Y, NB, OUT_T, ROWB, RM, RN>(p, x + xo, y + yo, bo, bi, m0, n0, wm, wn, t, lane, out, xs, ys);
 }
 
 template <bool ADJ_X, bool ADJ_Y, int NB, int OUT_T, bool ROWB>
 void launch_vec(const BmmArgs& a, const int8_t* x, const int8_t* y, void* out, dim3 grid, hipStream_t st) {
+  if constexpr (NB == 0 || ROWB) {  // the larger tiles (chosen by the host for aligned operands only)
+    if (a.rm == 2 && a.rn == 2) {
+      qbmm_kernel<ADJ_X, ADJ_Y, true, true, NB, OUT_T, ROWB, 2, 2><<<grid, kBmmThreads, 0, st>>>(a, x, y, out);
+      return;
+    }
+    if (a.rm == 2 && a.rn == 1) {
+      qbmm_kernel<ADJ_X, ADJ_Y, true, true, NB, OUT_T, ROWB, 2, 1><<<grid, kBmmThreads, 0, st>>>(a, x, y, out);
+      return;
+    }
+  }
   if (a.vec_x && a.vec_y) qbmm_kernel<ADJ_X, ADJ_Y, true, true, NB, OUT_T, ROWB><<<grid, kBmmThreads, 0, st>>>(a, x, y, out);
   else if (a.vec_x) qbmm_kernel<ADJ_X, ADJ_Y, true, false, NB, OUT_T, ROWB><<<grid, kBmmThreads, 0, st>>>(a, x, y, out);
   else if (a.vec_y) qbmm_kernel<ADJ_X, ADJ_Y, false, true, NB, OUT_T, ROWB><<<grid, kBmmThreads, 0, st>>>(a, x, y, out);
@@ -407,13 +463,27 @@ extern "C" int itexhip_qbatch_matmul(const itexhip_bmm_params* p, const int8_t* 
     }
     --a.p.n_batch_dims;
   }
-  a.tiles_m = static_cast<int>((p->M + kTile - 1) / kTile);
-  a.tiles_n = static_cast<int>((p->N + kTile - 1) / kTile);
-  const int64_t grid = batch * a.tiles_m * a.tiles_n;
-  ITEXHIP_REQUIRE(grid < (1LL << 31), "%s: %lld output tiles exceed one launch", who, static_cast<long long>(grid));
   // [R, K] layouts load 16 bytes along k, [K, R] layouts 4 bytes along r
   a.vec_x = p->adj_x ? vector_layout(x, p->x_batch_stride, p->n_batch_dims, p->M, 4) : vector_layout(x, p->x_batch_stride, p->n_batch_dims, p->K, 16);
   a.vec_y = p->adj_y ? vector_layout(y, p->y_batch_stride, p->n_batch_dims, p->K, 16) : vector_layout(y, p->y_batch_stride, p->n_batch_dims, p->N, 4);
+  // Tiles of 128 rows (and 128 columns) where more than 64 exist, the operands are aligned, the fused operands do not
+  // depend on the row, and at least 1024 tiles remain (four per CU); else 64 x 64.  BERT-base attention over 128
+  // sequences, 1536 tiles: Q.K^T + Mul + Add 24.6 -> 20.0 us, P.V 16.9 -> 14.2 us; over 32 sequences the 384 larger
+  // tiles measured slower than the 1536 small ones (7.4 against 6.5 us).
+  bool rowb = true;
+  for (int b = 0; b < p->n_binary; ++b) rowb = rowb && p->binary[b].stride_m == 0;
+  a.rm = a.rn = 1;
+  if (a.vec_x && a.vec_y && rowb && p->M > kTile) {
+    const int rn = p->N > kTile ? 2 : 1;
+    if (batch * ((p->M + 2 * kTile - 1) / (2 * kTile)) * ((p->N + rn * kTile - 1) / (rn * kTile)) >= 1024) {
+      a.rm = 2;
+      a.rn = rn;
+    }
+  }
+  a.tiles_m = static_cast<int>((p->M + a.rm * kTile - 1) / (a.rm * kTile));
+  a.tiles_n = static_cast<int>((p->N + a.rn * kTile - 1) / (a.rn * kTile));
+  const int64_t grid = batch * a.tiles_m * a.tiles_n;
+  ITEXHIP_REQUIRE(grid < (1LL << 31), "%s: %lld output tiles exceed one launch", who, static_cast<long long>(grid));
   hipStream_t st = as_stream(stream);
   // (tiles of a matrix, innermost batch dimension, product of the other batch dimensions) when the extents fit a grid
   const int64_t tiles = static_cast<int64_t>(a.tiles_m) * a.tiles_n;

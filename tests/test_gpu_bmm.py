@@ -153,6 +153,26 @@ def test_random_shapes_layouts_and_operands(hip, dev, seed):
             check(hip, dev, x, y, adj_x, adj_y, tuple(binary), t_out, x_off, y_off)
 
 
+@pytest.mark.parametrize("adj_x,adj_y", [(False, False), (False, True), (True, False), (True, True)])
+@pytest.mark.parametrize("M,K,N", [(72, 48, 132), (128, 64, 128), (100, 80, 36), (68, 16, 64)])
+def test_tiles_of_128_rows(hip, dev, adj_x, adj_y, M, K, N):
+    """Calls with at least 1024 tiles of 128 rows, aligned operands and fused operands that do not depend on the row run
+    tiles of 128 x 128 (N > 64) or 128 x 64 outputs, ragged at both edges here; every layout, fp32 without operands,
+    bfloat16 with a scalar Mul and a mask broadcast over the rows, and with a per-row operand the 64 x 64 tiles again."""
+    import torch
+    rng = np.random.default_rng(M + K + N + adj_x * 2 + adj_y)
+    B = (1030,)
+    x = rng.integers(-128, 128, B + ((K, M) if adj_x else (M, K))).astype(np.int8)
+    y = rng.integers(-128, 128, B + ((N, K) if adj_y else (K, N))).astype(np.int8)
+    check(hip, dev, x, y, adj_x, adj_y)
+    mul = to16(torch, np.float32([0.125]), orc.BFLOAT16)
+    mask = to16(torch, np.where(rng.random((1, 1, N)) < 0.3, np.float32(-100.0), np.float32(0.0)).astype(np.float32), orc.BFLOAT16)
+    check(hip, dev, x, y, adj_x, adj_y, binary=((orc.BIN_MUL, mul), (orc.BIN_ADD, mask)), t_out=orc.BFLOAT16)
+    if (adj_x, adj_y) == (False, True):
+        per_row = rng.standard_normal((1, M, 1)).astype(np.float32)
+        check(hip, dev, x, y, adj_x, adj_y, binary=((orc.BIN_ADD, per_row),))
+
+
 def test_empty_and_invalid(hip, dev):
     import torch
     z = np.zeros((2, 0, 8), np.int8)
