@@ -308,6 +308,11 @@ def bench_elementwise(torch, hip, timer, n, steps, warmup, dev):
     req = np.float32(1.0) * np.float32(amax) / np.float32(2.0 ** 31)
     rscale = float(np.float32(127.0) * (np.float32(1.0) / req / np.float32(2.0 ** 31)))
     add("requantize_int32_to_qint8", lambda i: hip.requantize(acc, q8, n, hip.QINT8, rscale, st), 5 * n)
+    # the same tensor as [2^20, 256] with one scale per channel (RequantizePerChannel on an NHWC tensor of 256 channels)
+    depth = 256
+    rsc = torch.full((depth,), rscale, dtype=torch.float32, device=dev) * (torch.rand(depth, device=dev, generator=g) * 0.5 + 0.75)
+    add("requantize_per_channel_int32_to_qint8_256_channels",
+        lambda i: hip.requantize_per_channel(acc, q8, n // depth, depth, hip.QINT8, rsc, st), 5 * n)
     # per-channel (per-axis) forms on a [4096, 14336] fp32 weight: the weight-quantization path; channels innermost
     # (axis 1) and outermost (axis 0 of the transposed layout)
     K, N = 4096, 14336
