@@ -389,8 +389,9 @@ typedef struct {
 } itexhip_bmm_params;
 
 /* x, y, out: device memory.  Any M, K, N >= 0 and any alignment; 16-byte-aligned operands with K (and, for
- * the transposed layouts, the row length) a multiple of 16 take the vector-load path.  MFMA 32x32x32 i8
- * tiles of 64 x 64 outputs per workgroup. */
+ * the transposed layouts, the row length) a multiple of 16 take the vector-load path.  MFMA 32x32x32 i8,
+ * tiles of 64 x 64 outputs per workgroup, 128 x 128 / 128 x 64 for calls with at least 1024 such tiles, aligned
+ * operands and fused operands that do not depend on the row. */
 int itexhip_qbatch_matmul(const itexhip_bmm_params* p, const int8_t* x, const int8_t* y, void* out, void* stream);
 
 /* ---- quantized Transpose ------------------------------------------------------------------------

@@ -5,7 +5,8 @@
 // Both operands are activations (the Q.K^T and P.V products of an attention block), so nothing can be
 // prepacked: every workgroup stages a 64 x 64 byte tile of each operand in LDS, k-contiguous per output row /
 // column, and its four wavefronts each own one 32 x 32 quadrant of the 64 x 64 output tile
-// (v_mfma_i32_32x32x32_i8).  An operand stored with k as the slow dimension (x with adj_x, y without
+// (v_mfma_i32_32x32x32_i8); large calls run tiles of 128 rows (and columns) with two (four) quadrants per
+// wavefront.  An operand stored with k as the slow dimension (x with adj_x, y without
 // adj_y) is transposed on the way into LDS, four bytes at a time.  The output orientation keeps
 // n on the lanes, so every store instruction writes 128 contiguous bytes per half-wavefront: with fp32
 // outputs the op is bound by that write.
