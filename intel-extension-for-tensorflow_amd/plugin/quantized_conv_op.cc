@@ -2,9 +2,11 @@
 // their combinations, and the list-attribute form _QuantizedConv2D / _ITEXQuantizedConv2DV2
 // (itex/core/kernels/common/quantized_conv_ops.h:63-597 over conv_ops.h:615-1150; device registrations in
 // itex/core/kernels/gpu/quantized_conv_ops.cc).  Host half as in the reference: attribute and fusion
-// parsing, input indices, geometry, output scales and bias factors; the convolution itself runs as
-// itexhip_im2col8 + itexhip_qgemm on the filter prepacked as a [KH*KW*C, O] matrix.
-// Not carried over: Sum / Elu / Swish / HardSwish / Sigmoid fusions, depthwise and 3-D variants, NCHW.
+// parsing, input indices, geometry, output scales and bias factors; the convolution itself runs on the filter
+// prepacked as a [KH*KW*C, O] matrix: as an implicit GEMM (itexhip_qconv2d) where the input channels are a multiple
+// of 16, on a channel- and window-padded copy (itexhip_pad_nhwc8) where they are at most 8, as a plain GEMM for 1x1
+// windows, else as itexhip_im2col8 + itexhip_qgemm; depthwise windows have a kernel of their own.
+// Not carried over: Swish / HardSwish fusions, 3-D variants, NCHW.
 #include <mutex>
 #include <algorithm>
 #include <cmath>
