@@ -79,8 +79,9 @@ __global__ __launch_bounds__(256) void prepack_b_kernel(const int8_t* __restrict
 // from the row-major activations would put 64 lanes on 64 different 16-byte pieces of 16 rows, which the
 // texture addresser serves at a quarter of its rate; instead the 16 rows x 64 bytes travel by a direct
 // global -> LDS load whose lanes are contiguous in groups of four (lane 4 q + j: row q, piece
-// j ^ ((q >> 1) & 3)) into a 1 KiB slot of a ring private to the wavefront, and the fragment is read back
-// from LDS (the rotation of the pieces makes that read conflict free).  The loads of a batch of U pairs
+// j ^ ((q >> 2) & 3)) into a 1 KiB slot of a ring private to the wavefront, and the fragment is read back
+// from LDS (the rotation of the pieces makes that read conflict free: the 16 lanes served per LDS cycle read 16
+// rows, whose slots 4 q + (j ^ (q >> 2)) fall into 16 different bank groups).  The loads of a batch of U pairs
 // are issued while the previous batch is multiplied, so 2 U (NT + 1) KiB per wavefront are in flight.
 // The partial 16x16 tiles of the wavefronts meet in LDS (the rings, free by then; one barrier) and
 // wavefront t finishes tile t.  One more wavefront per workgroup streams nothing: it resolves the strip's
@@ -128,13 +129,13 @@ __global__ __launch_bounds__(576) void qgemv_kernel(const uint8_t* __restrict__ 
                         (((lgrp & 1) * 32 + half0 * 16 + lrow) << 4);
   // activation staging: lane -> (row q, piece j) of the 16 x 64 byte tile
   const int q = lane >> 2;
-  const int dpiece = ((lane & 3) ^ ((q >> 1) & 3)) * 16;
+  const int dpiece = ((lane & 3) ^ ((q >> 2) & 3)) * 16;
   const uint8_t* arow[R];
 #pragma unroll
   for (int r = 0; r < R; ++r) arow[r] = a + static_cast<int64_t>(min(m_base + 16 * r + q, M - 1)) * K;
   const int klast = K - 16;  // k beyond K meets zero weights: any in-bounds data will do
   uint8_t* const ring = smem + wave * (RING * R * 1024);
-  const uint32_t frag_off = static_cast<uint32_t>((4 * lrow + (lgrp ^ ((lrow >> 1) & 3))) * 16);
+  const uint32_t frag_off = static_cast<uint32_t>((4 * lrow + (lgrp ^ ((lrow >> 2) & 3))) * 16);
 
   v4i acc[R][NT];
 #pragma unroll

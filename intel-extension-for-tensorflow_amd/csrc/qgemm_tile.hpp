@@ -33,8 +33,11 @@ namespace itexhip {
 //   Activation staging.  One wavefront load covers 16 rows x 64 B, 4 consecutive lanes per row (the
 //   texture addresser serves a quad of lanes per cycle only when the quad is contiguous).  Quad q of a
 //   load holds row q; inside the quad, piece p (= 2*kc + g, 16 bytes of k) sits at lane
-//   p ^ ((q >> 1) & 3).  That rotation makes the fragment reads conflict free: the 8 lanes an LDS cycle
-//   serves read 8 consecutive rows, whose 16-byte slots then fall into 8 different bank groups.
+//   p ^ ((q >> 2) & 3).  That rotation makes the fragment reads conflict free: the 16 lanes an LDS cycle
+//   serves (256 B per cycle on this device) read 16 consecutive rows, whose 16-byte slots then fall into 16
+//   different bank groups (slot 4 q + (p ^ (q >> 2)): q & 3 picks a group of four, the rotation one of them).
+//   Rotating by (q >> 1), which spreads 8 lanes over 8 bank groups, left a two-way conflict on every
+//   activation fragment read (SQ_LDS_BANK_CONFLICT: a third of the K loop's LDS cycles).
 //   Weight chunks are already in fragment lane order in memory and are copied linearly.
 //   Unsigned activations are turned into signed ones (x ^ 0x80) after the fragment read.
 //
@@ -150,7 +153,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void qgemm_tile_kernel(
   // ---- staging sources of this wavefront
   // activation load `ld` covers rows [16*h, 16*h+16) of 32-row tile rt: lane -> (row q, piece p)
   const int q_row = lane >> 2;
-  const int q_piece = (lane & 3) ^ ((q_row >> 1) & 3);  // piece = 2*kc + g
+  const int q_piece = (lane & 3) ^ ((q_row >> 2) & 3);  // piece = 2*kc + g
   uint32_t off_a[A_PER_WAVE];       // byte offset of the lane's row (+ piece when KALIGNED) in the activation matrix
   const uint8_t* src_b[B_PER_WAVE];  // wavefront-uniform chunk pointers of step 0
   int win_h[A_PER_WAVE], win_w[A_PER_WAVE];  // implicit GEMM: window origin of the lane's row (may lie in the padding)
@@ -216,8 +219,8 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void qgemm_tile_kernel(
   // fragment reads: activation fragment (k-chunk kc, row tile i of this wavefront), weight fragment (kc, j)
   const int fq = lrow & 15, fh = lrow >> 4;
   const uint32_t frag_a_lane[2] = {
-      static_cast<uint32_t>(fh * kChunkBytes + ((4 * fq + ((0 + lgrp) ^ ((fq >> 1) & 3))) << 4)),
-      static_cast<uint32_t>(fh * kChunkBytes + ((4 * fq + ((2 + lgrp) ^ ((fq >> 1) & 3))) << 4))};
+      static_cast<uint32_t>(fh * kChunkBytes + ((4 * fq + ((0 + lgrp) ^ ((fq >> 2) & 3))) << 4)),
+      static_cast<uint32_t>(fh * kChunkBytes + ((4 * fq + ((2 + lgrp) ^ ((fq >> 2) & 3))) << 4))};
   auto lds_a_raw = [&](int stage, int kc, int i) {
     return *reinterpret_cast<const v4i*>(lds + stage * STAGE_BYTES + (wm * TM + i) * (2 * kChunkBytes) + frag_a_lane[kc]);
   };
