@@ -150,7 +150,7 @@ def make_acts(torch, hip, M, K, seed, dev, outlier_frac=0.0, outlier_mult=1.0):
 # ------------------------------------------------------------------------------------------------
 def bench_linear(torch, hip, timer, M, K, N, kind, steps, warmup, dev, seed, rotate=1, graph=False, per_row=False):
     """kind: 'requant_s8' ([BiasAdd, Requantize] -> qint8), 'deq' / 'deq_relu' / 'deq_gelu' ([.., Dequantize] -> fp32;
-    GeluApproximate is what BERT's first feed-forward linear fuses).
+    GeluApproximate is what BERT's first feed-forward linear fuses), the same with '_bf16' appended -> bfloat16.
     rotate > 1 cycles through that many distinct weight copies so that the weight stream comes from
     HBM, not from the 256 MiB last-level cache."""
     layers = [make_weights(torch, hip, K, N, seed + i, dev) for i in range(rotate)]
@@ -163,12 +163,14 @@ def bench_linear(torch, hip, timer, M, K, N, kind, steps, warmup, dev, seed, rot
                               has_requantize=True, min_a=min_a, max_a=max_a, min_out=-r_out, max_out=r_out)
         out_bytes = 1
     else:
-        t_out, out_dtype = hip.FLOAT, torch.float32
+        bf16 = kind.endswith("_bf16")  # Dequantize to bfloat16: half the output bytes of the fp32 rows
+        t_out, out_dtype = (hip.BFLOAT16, torch.bfloat16) if bf16 else (hip.FLOAT, torch.float32)
+        act = kind[:-5] if bf16 else kind
         p = hip.matmul_params(api=hip.API_V2, t_in=hip.QUINT8, t_out=t_out, input_mode=hip.MIN_FIRST,
                               has_dequantize=True,
-                              activation={"deq_relu": hip.ACT_RELU, "deq_gelu": hip.ACT_GELU_APPROX}.get(kind, hip.ACT_NONE),
+                              activation={"deq_relu": hip.ACT_RELU, "deq_gelu": hip.ACT_GELU_APPROX}.get(act, hip.ACT_NONE),
                               min_a=min_a, max_a=max_a)
-        out_bytes = 4
+        out_bytes = 2 if bf16 else 4
     del x
     ep = hip.qmatmul_epilogue_desc(p, N)
     out = torch.empty(M, N, dtype=out_dtype, device=dev)
@@ -766,7 +768,8 @@ def main():
             others.append(r)
     if "bert" in only:
         for (k, n, kind, seed) in ((768, 2304, "deq", 1), (768, 768, "deq", 2), (768, 3072, "deq_relu", 3),
-                                   (768, 3072, "deq_gelu", 3), (3072, 768, "deq", 4)):
+                                   (768, 3072, "deq_gelu", 3), (3072, 768, "deq", 4),
+                                   (768, 2304, "deq_bf16", 1), (768, 3072, "deq_gelu_bf16", 3)):
             r = bench_linear(torch, hip, timer, 4096, k, n, kind, K_steps, W, dev, seed, graph=True)
             r.pop("_ctx")
             t_roof = max(r["ops"] / (PEAK_INT8_TOPS * 1e12), r["bytes"] / (PEAK_HBM_GBS * 1e9))

@@ -380,8 +380,7 @@ __global__ __launch_bounds__(256) void qdwconv3x3_kernel(const DepthwiseArgs a, 
         *reinterpret_cast<f4*>(static_cast<float*>(out) + o) = f4{y[0], y[1], y[2], y[3]};
       } else if constexpr (is_float16_type(OUT_T)) {
         typedef unsigned int u2 __attribute__((ext_vector_type(2)));
-        *reinterpret_cast<u2*>(static_cast<uint16_t*>(out) + o) = u2{f32_to_bits16<OUT_T>(y[0]) | (f32_to_bits16<OUT_T>(y[1]) << 16),
-                                                                     f32_to_bits16<OUT_T>(y[2]) | (f32_to_bits16<OUT_T>(y[3]) << 16)};
+        *reinterpret_cast<u2*>(static_cast<uint16_t*>(out) + o) = u2{f32x2_to_bits16<OUT_T>(y[0], y[1]), f32x2_to_bits16<OUT_T>(y[2], y[3])};
       } else if constexpr (OUT_T == ITEXHIP_QINT32) {
         *reinterpret_cast<i4*>(static_cast<int32_t*>(out) + o) = i4{sat_rne<ITEXHIP_QINT32>(y[0]), sat_rne<ITEXHIP_QINT32>(y[1]),
                                                                     sat_rne<ITEXHIP_QINT32>(y[2]), sat_rne<ITEXHIP_QINT32>(y[3])};

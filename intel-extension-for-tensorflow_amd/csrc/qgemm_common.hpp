@@ -261,8 +261,7 @@ __device__ __forceinline__ v4i epilogue_pack(const v4i bits) {
   if constexpr (OUT_T == ITEXHIP_FLOAT) {
     return v4i{__float_as_int(y[0]), __float_as_int(y[1]), __float_as_int(y[2]), __float_as_int(y[3])};
   } else if constexpr (is_float16_type(OUT_T)) {  // 4 x 16 bits in .x, .y
-    return v4i{static_cast<int>(f32_to_bits16<OUT_T>(y[0]) | (f32_to_bits16<OUT_T>(y[1]) << 16)),
-               static_cast<int>(f32_to_bits16<OUT_T>(y[2]) | (f32_to_bits16<OUT_T>(y[3]) << 16)), 0, 0};
+    return v4i{static_cast<int>(f32x2_to_bits16<OUT_T>(y[0], y[1])), static_cast<int>(f32x2_to_bits16<OUT_T>(y[2], y[3])), 0, 0};
   } else if constexpr (OUT_T == ITEXHIP_QINT32) {
     return v4i{sat_rne<ITEXHIP_QINT32>(y[0]), sat_rne<ITEXHIP_QINT32>(y[1]), sat_rne<ITEXHIP_QINT32>(y[2]),
                sat_rne<ITEXHIP_QINT32>(y[3])};
@@ -333,8 +332,7 @@ __device__ __forceinline__ void epilogue_store(const v4i acc, const ChannelParam
     uint16_t* dst = reinterpret_cast<uint16_t*>(out) + o;
     if (full) {
       typedef unsigned int u2 __attribute__((ext_vector_type(2)));
-      *reinterpret_cast<u2*>(dst) = u2{f32_to_bits16<OUT_T>(y[0]) | (f32_to_bits16<OUT_T>(y[1]) << 16),
-                                       f32_to_bits16<OUT_T>(y[2]) | (f32_to_bits16<OUT_T>(y[3]) << 16)};
+      *reinterpret_cast<u2*>(dst) = u2{f32x2_to_bits16<OUT_T>(y[0], y[1]), f32x2_to_bits16<OUT_T>(y[2], y[3])};
     } else {
       for (int r = 0; r < 4 && n + r < N; ++r) dst[r] = static_cast<uint16_t>(f32_to_bits16<OUT_T>(y[r]));
     }
