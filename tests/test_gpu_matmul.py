@@ -824,6 +824,44 @@ def test_bfloat16_output_vs_oracle(hip, dev, path, M, K, N, T16):
         np.testing.assert_array_equal(bits16(layer.run(xq, kw, mn, mx, path=path)), ref)
 
 
+@pytest.mark.parametrize("path", ["gemv", "tile", "naive"])
+def test_bfloat16_rounding_of_special_values(hip, dev, path):
+    """The bfloat16 store rounds with the GPU's conversion instruction; the oracle with the integer formula.  All-zero
+    weight columns make the fp32 result of a column equal its bias exactly, so any fp32 bit pattern can be sent through the
+    epilogue's conversion: ties to even in both directions, carries into the exponent, the largest finite values
+    (rounding to infinity), denormals (fp32 denormals that stay bfloat16 denormals or round up to the smallest normal),
+    infinities and NaNs.  Bit patterns must equal the oracle's, except that a NaN only has to be a NaN."""
+    M, K, N = 40, 256, 96
+    rng = np.random.default_rng(5)
+    w = (rng.standard_normal((K, N)) * 0.02).astype(np.float32)
+    r = np.abs(w).max(0).astype(np.float32)
+    _, wq, mn_b, mx_b = orc.quantize_v2(w, -r, r, orc.QINT8, orc.SCALED, axis=1)
+    special = np.array([0x3f808000, 0x3f818000, 0x3f807fff, 0x3f808001, 0x3fffffff, 0x3fff8000, 0x7f7fffff, 0x7f7f8000,
+                        0x7f7f7fff, 0xff7fffff, 0x00000001, 0x00008000, 0x00008001, 0x00018000, 0x007fffff, 0x007f8000,
+                        0x807fffff, 0x00800000, 0x80000000, 0x00000000, 0x7f800000, 0xff800000, 0x7fc00000, 0xffc00000,
+                        0x33333333, 0xb3333333, 0x4b7fffff, 0xcb7f8000, 0x0000ffff, 0x80010000, 0x7f000000, 0x3effffff],
+                       dtype=np.uint32)
+    cols = np.arange(special.size) * 3  # spread over the 32-channel tiles and their 4-channel groups
+    wq[:, cols] = 0
+    bias = (rng.standard_normal(N) * 0.01).astype(np.float32)
+    bias[cols] = special.view(np.float32)
+    layer = Linear(hip, dev, wq, mn_b, mx_b, bias)
+    x, xq, mn, mx = make_acts(M, K, seed=9)
+    kw = dict(V2_DEQ, t_out=orc.BFLOAT16)
+    ref = layer.oracle(xq, kw, mn, mx)
+    got = bits16(layer.run(xq, kw, mn, mx, path=path))
+    nan = (ref & 0x7fff) > 0x7f80
+    assert nan[:, cols[22]].all() and nan[:, cols[23]].all() and nan.sum() == 2 * M
+    np.testing.assert_array_equal((got & 0x7fff) > 0x7f80, nan)
+    np.testing.assert_array_equal(got[~nan], ref[~nan])
+    # the special columns really carry the rounded bias (the fixture does what it says)
+    f = special.astype(np.uint64)
+    want = ((f + 0x7fff + ((f >> 16) & 1)) >> 16).astype(np.uint16)
+    want[18] = 0  # a bias of -0 is added to the accumulator's +0
+    finite = np.array([i for i in range(special.size) if i not in (22, 23)])
+    np.testing.assert_array_equal(ref[0, cols[finite]], want[finite])
+
+
 @pytest.mark.parametrize("shape", [0, 1, 2, 3, 4])
 @pytest.mark.parametrize("V2_DEQ_BF16", [V2_DEQ_BF16, V2_DEQ_F16], ids=["bf16", "f16"])
 def test_bfloat16_output_every_tile_shape(hip, dev, monkeypatch, shape, V2_DEQ_BF16):
