@@ -774,6 +774,32 @@ def test_gelu_fusion_close_to_oracle(hip, dev, M, act):
         np.testing.assert_allclose(got, gelu, rtol=0.2, atol=0.2)   # the reference test's own bar
 
 
+@pytest.mark.parametrize("act", [orc.ACT_GELU_APPROX, orc.ACT_GELU_EXACT, orc.ACT_ELU, orc.ACT_SIGMOID, orc.ACT_TANH,
+                                 orc.ACT_SWISH, orc.ACT_MISH])
+@pytest.mark.parametrize("path", ["tile", "gemv"])
+def test_transcendental_activations_over_a_dense_range(hip, dev, act, path):
+    """The device evaluates these activations with the hardware's exp2 / reciprocal and its own polynomial forms.  With
+    an all-zero weight the fp32 value entering the activation is the bias itself, so the whole input range is swept, not
+    only what a matrix product happens to produce: 16 K points over [-30, 30] (dense around 0), the break points of the
+    device's forms and the large magnitudes where exp overflows.  Same tolerance as the other GELU tests."""
+    M, K = 3, 64
+    xs = np.concatenate([np.linspace(-30, 30, 8192), np.linspace(-1, 1, 4096), np.linspace(-12, -2, 4000),
+                         [-0.35, -0.3500001, -0.3499999, 20.0, 20.00001, 19.99999, 0.0, -0.0, 1e-8, -1e-8, 1e-30, -1e-30,
+                          88.0, -88.0, 104.0, -104.0, 1e4, -1e4, 3e38, -3e38]]).astype(np.float32)
+    N = ((xs.size + 31) // 32) * 32
+    bias = np.zeros(N, np.float32)
+    bias[:xs.size] = xs
+    wq = np.zeros((K, N), np.int8)
+    one = np.ones(N, np.float32)
+    layer = Linear(hip, dev, wq, -one, one, bias)
+    x, xq, mn, mx = make_acts(M, K, seed=3)
+    kw = dict(V2_DEQ, activation=act)
+    ref = layer.oracle(xq, kw, mn, mx)
+    got = layer.run(xq, kw, mn, mx, path=path)
+    assert np.isfinite(ref[:, :xs.size - 2]).all()
+    np.testing.assert_allclose(got, ref, rtol=2e-6, atol=1e-6)
+
+
 @pytest.mark.parametrize("M", [2, 140])
 @pytest.mark.parametrize("t_out,mode", [(orc.FLOAT, orc.MIN_FIRST), (orc.QINT8, orc.MIN_FIRST), (orc.QINT32, orc.MIN_FIRST),
                                         (orc.FLOAT, orc.SCALED)])
