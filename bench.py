@@ -169,12 +169,14 @@ def bench_linear(torch, hip, timer, M, K, N, kind, steps, warmup, dev, seed, rot
         p = hip.matmul_params(api=hip.API_V2, t_in=hip.QUINT8, t_out=t_out, input_mode=hip.MIN_FIRST,
                               has_dequantize=True,
                               activation={"deq_relu": hip.ACT_RELU, "deq_gelu": hip.ACT_GELU_APPROX}.get(act, hip.ACT_NONE),
-                              min_a=min_a, max_a=max_a)
+                              min_a=min_a, max_a=max_a, add_position=1 if act == "deq_add" else 0)
         out_bytes = 2 if bf16 else 4
     del x
     ep = hip.qmatmul_epilogue_desc(p, N)
     out = torch.empty(M, N, dtype=out_dtype, device=dev)
     st = _stream(torch)
+    # [BiasAdd, Add, Dequantize]: the residual connection fused as the "Add" post-op, an fp32 tensor of the output's shape
+    addend = torch.randn(M, N, dtype=out_dtype, device=dev) if kind == "deq_add" else None
 
     if per_row:  # per-token ranges (here: the tensor's range widened a little more for each row)
         row_min = torch.tensor([min_a * (1.0 + 0.01 * m) for m in range(M)], dtype=torch.float32, device=dev)
@@ -187,7 +189,7 @@ def bench_linear(torch, hip, timer, M, K, N, kind, steps, warmup, dev, seed, rot
             hip.qmatmul_per_row(p, xq, L["packed"], L["colsum"], M, K, N, row_min, row_max, L["min_b"], L["max_b"], N,
                                 L["bias"], out, st)
         else:
-            hip.qmatmul(p, xq, L["packed"], L["colsum"], M, K, N, L["min_b"], L["max_b"], N, L["bias"], out, st)
+            hip.qmatmul(p, xq, L["packed"], L["colsum"], M, K, N, L["min_b"], L["max_b"], N, L["bias"], out, st, addend=addend)
 
     for L in layers:  # parameter vectors for the two-launch form below
         hip.qmatmul_prepare(p, L["min_b"], L["max_b"], N, L["bias"], L["colsum"], N, L["scales"], L["sbias"], st)
@@ -195,19 +197,22 @@ def bench_linear(torch, hip, timer, M, K, N, kind, steps, warmup, dev, seed, rot
     def gemm_only(i):
         # the MatMul kernel alone, parameters prepared beforehand
         L = layers[i % rotate]
-        hip.qgemm(xq, hip.QUINT8, L["packed"], L["colsum"], M, K, N, L["scales"], L["sbias"], ep, t_out, out, st)
+        if addend is not None:
+            hip.qgemm_sum(xq, hip.QUINT8, L["packed"], L["colsum"], M, K, N, L["scales"], L["sbias"], ep, addend, t_out, t_out, out, st)
+        else:
+            hip.qgemm(xq, hip.QUINT8, L["packed"], L["colsum"], M, K, N, L["scales"], L["sbias"], ep, t_out, out, st)
 
     def make_graph_fn(stream):
         def fn(i):
             L = layers[i % rotate]
-            hip.qmatmul(p, xq, L["packed"], L["colsum"], M, K, N, L["min_b"], L["max_b"], N, L["bias"], out, stream)
+            hip.qmatmul(p, xq, L["packed"], L["colsum"], M, K, N, L["min_b"], L["max_b"], N, L["bias"], out, stream, addend=addend)
         return fn
 
     ms_step = timer.run(step, steps, warmup)
     ms_kernel = timer.run(gemm_only, steps, warmup)
     ms_graph = timer.run_graph(make_graph_fn, steps, warmup) if graph else None
     ops = 2.0 * M * N * K
-    nbytes = M * K + K * N + out_bytes * M * N + 8 * N
+    nbytes = M * K + K * N + out_bytes * M * N * (2 if addend is not None else 1) + 8 * N
     res = dict(M=M, K=K, N=N, kind=kind, ms_per_step=ms_step, us_kernel=ms_kernel * 1e3,
                tops=ops / (ms_step * 1e-3) / 1e12, tops_kernel=ops / (ms_kernel * 1e-3) / 1e12,
                gbs_kernel=nbytes / (ms_kernel * 1e-3) / 1e9, ops=ops, bytes=nbytes)
@@ -769,7 +774,7 @@ def main():
     if "bert" in only:
         for (k, n, kind, seed) in ((768, 2304, "deq", 1), (768, 768, "deq", 2), (768, 3072, "deq_relu", 3),
                                    (768, 3072, "deq_gelu", 3), (3072, 768, "deq", 4),
-                                   (768, 2304, "deq_bf16", 1), (768, 3072, "deq_gelu_bf16", 3)):
+                                   (768, 2304, "deq_bf16", 1), (768, 3072, "deq_gelu_bf16", 3), (3072, 768, "deq_add", 4)):
             r = bench_linear(torch, hip, timer, 4096, k, n, kind, K_steps, W, dev, seed, graph=True)
             r.pop("_ctx")
             t_roof = max(r["ops"] / (PEAK_INT8_TOPS * 1e12), r["bytes"] / (PEAK_HBM_GBS * 1e9))
