@@ -447,6 +447,38 @@ def bench_conv(torch, hip, timer, steps, warmup, dev):
                         note="channel- and window-padded copy + implicit GEMM, two launches" if patches == "narrow" else
                         "implicit GEMM, one launch" if implicit else "im2col + GEMM launches" if patches else "GEMM launch only"))
         del x, w, packed, y, cols
+    # the last 1x1 convolution of a ResNet-50 bottleneck block (56x56x64 -> 256) with the block's residual fused as the Sum
+    # post-op: [BiasAdd, Sum, Relu, Requantize], quint8 addend of the output's shape; a plain GEMM with one more operand
+    M, K, O = 32 * 56 * 56, 64, 256
+    x = torch.randint(0, 256, (M, K), dtype=torch.uint8, device=dev, generator=g_)
+    w = torch.randint(-127, 128, (K, O), dtype=torch.int8, device=dev, generator=g_)
+    z = torch.randint(0, 256, (M, O), dtype=torch.uint8, device=dev, generator=g_)
+    packed = torch.empty(hip.qgemm_packed_bytes(K, O), dtype=torch.int8, device=dev)
+    colsum = torch.empty(O, dtype=torch.int32, device=dev)
+    hip.qgemm_prepack_b(w, False, K, O, packed, colsum, st)
+    scales = torch.full((O,), 1e-4, dtype=torch.float32, device=dev)
+    bias = torch.zeros(O, dtype=torch.float32, device=dev)
+    y = torch.empty((M, O), dtype=torch.uint8, device=dev)
+    for with_sum in (False, True):
+        ep = hip.Epilogue()
+        ep.n_scales, ep.n_eltwise = O, 2 if with_sum else 1
+        k = 0
+        if with_sum:
+            ep.elt[0].alg, ep.elt[0].alpha, ep.elt[0].beta = hip.ELT_SUM, 0.5, 0.0
+            k = 1
+        ep.elt[k].alg, ep.elt[k].alpha, ep.elt[k].beta = hip.ELT_RELU, 0.0, 0.0
+
+        def make_sum(stream):
+            if with_sum:
+                return lambda i: hip.qgemm_sum(x, hip.QUINT8, packed, colsum, M, K, O, scales, bias, ep, z, hip.QUINT8, hip.QUINT8, y, stream)
+            return lambda i: hip.qgemm(x, hip.QUINT8, packed, colsum, M, K, O, scales, bias, ep, hip.QUINT8, y, stream)
+        ms = timer.run_graph(make_sum, steps, warmup)
+        nbytes = x.numel() + w.numel() + y.numel() * (2 if with_sum else 1)
+        ops = 2 * M * K * O
+        out.append(dict(name="conv1x1_56x56x64_to_256" + ("_sum_relu" if with_sum else "_relu"), M=M, K=K, N=O, us_kernel=ms * 1e3,
+                        bytes=nbytes, ops=ops, bound="hbm", frac=nbytes / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS,
+                        tops=ops / (ms * 1e-3) / 1e12, gbs=nbytes / (ms * 1e-3) / 1e9, note="GEMM launch only"))
+    del x, w, z, packed, y
     # depthwise 3x3 (MobileNet shapes): no matrix product, bound by input + output bytes
     for name, (B, H, W, C) in (("dwconv3x3_112x112x32", (32, 112, 112, 32)), ("dwconv3x3_56x56x128", (32, 56, 56, 128))):
         x = torch.randint(0, 256, (B, H, W, C), dtype=torch.uint8, device=dev, generator=g_)
