@@ -380,7 +380,8 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void qgemm_tile_kernel(
       // 6 + lgrp of the 32 bytes its row has in this tile.  Read as four single dwords a wavefront load fetched 8 bytes
       // of each of 32 rows (56x56x64 -> 256 with a quint8 addend: 18.9 us without the Sum, 49.3 us with it); the whole
       // row segment in two 16-byte loads (4-byte aligned: N % 4 == 0) brings that to 39.3 us.  Fetching the segments a
-      // column of tiles ahead measured slower (43.1 us): the cost is 32-byte pieces of memory lines, not latency.
+      // column of tiles ahead measured slower (43.1 us), and staging the addend through LDS in rows of contiguous bytes
+      // gained only 1 us more: the rest of the Sum's cost is the arithmetic of the general chain epilogue, not memory.
       const bool addend8 = e.addend_type == ITEXHIP_QUINT8 || e.addend_type == ITEXHIP_QINT8;
       const int seg = n0 - lgrp * 4;  // first channel of the tile
       if (addend8 && seg + 32 <= N) {
