@@ -148,7 +148,8 @@ def make_acts(torch, hip, M, K, seed, dev, outlier_frac=0.0, outlier_mult=1.0):
 # ------------------------------------------------------------------------------------------------
 # workloads
 # ------------------------------------------------------------------------------------------------
-def bench_linear(torch, hip, timer, M, K, N, kind, steps, warmup, dev, seed, rotate=1, graph=False, per_row=False):
+def bench_linear(torch, hip, timer, M, K, N, kind, steps, warmup, dev, seed, rotate=1, graph=False, per_row=False,
+                 keep_out=False):
     """kind: 'requant_s8' ([BiasAdd, Requantize] -> qint8), 'deq' / 'deq_relu' / 'deq_gelu' ([.., Dequantize] -> fp32;
     GeluApproximate is what BERT's first feed-forward linear fuses), the same with '_bf16' appended -> bfloat16.
     rotate > 1 cycles through that many distinct weight copies so that the weight stream comes from
@@ -209,6 +210,8 @@ def bench_linear(torch, hip, timer, M, K, N, kind, steps, warmup, dev, seed, rot
         return fn
 
     ms_step = timer.run(step, steps, warmup)
+    # what the last of the timed single-launch calls left in the output buffer (it ran on layer (warmup+steps-1) % rotate)
+    out_timed = out.clone() if keep_out else None
     ms_kernel = timer.run(gemm_only, steps, warmup)
     ms_graph = timer.run_graph(make_graph_fn, steps, warmup) if graph else None
     ops = 2.0 * M * N * K
@@ -219,7 +222,7 @@ def bench_linear(torch, hip, timer, M, K, N, kind, steps, warmup, dev, seed, rot
     if ms_graph is not None:
         res.update(us_kernel_graph=ms_graph * 1e3, gbs_kernel_graph=nbytes / (ms_graph * 1e-3) / 1e9,
                    tops_kernel_graph=ops / (ms_graph * 1e-3) / 1e12)
-    res["_ctx"] = dict(layers=layers, xq=xq, p=p, min_a=min_a, max_a=max_a)
+    res["_ctx"] = dict(layers=layers, xq=xq, p=p, min_a=min_a, max_a=max_a, out_timed=out_timed)
     return res
 
 
@@ -695,6 +698,47 @@ def cpu_onednn_in_torch(torch, xq_host, wq_host, w_scale, bias):
         return None
 
 
+MAX_LINE_BYTES = 4096  # the final stdout line must stay a short record; everything else goes on an earlier line
+
+
+def _best(rows, name, pred=lambda r: True, key="frac", fn=min):
+    vals = [r[key] for r in rows if r.get("name") == name and pred(r) and r.get(key) is not None]
+    return round(fn(vals), 4) if vals else None
+
+
+def summary_line(head, steps, warmup, traffic, cpu, others):
+    """The one-line record: the headline workload with its roofline and CPU baseline, plus the roofline fractions of
+    the other workloads the metric names (worst row of each family)."""
+    targets = {
+        "prefill_gemm_other_shapes_frac_mfma_min": _best(others, "prefill_gemm"),
+        "bert_linear_fp32_frac_min": _best(others, "bert_linear", lambda r: r.get("kind") in ("deq", "deq_relu")),
+        "decode_gemv_m1_m4_frac_hbm_min": _best(others, "decode_gemv", lambda r: r.get("M", 99) <= 4),
+        "decode_gemv_m16_frac_hbm_min": _best(others, "decode_gemv", lambda r: r.get("M") == 16),
+        "quantize_v2_frac_hbm_min": _best([dict(r, name="q") for r in others
+                                           if str(r.get("name", "")).startswith("quantize_v2_")], "q"),
+        "dequantize_frac_hbm_min": _best([dict(r, name="d") for r in others
+                                          if str(r.get("name", "")).startswith("dequantize_") and "per_channel" not in r["name"]], "d"),
+        "requantize_frac_hbm": _best(others, "requantize_int32_to_qint8"),
+    }
+    line = {
+        "metric": "int8 GEMM TOPS (% MFMA peak); quantize/GEMV GB/s (% HBM peak), 1 MI355X",
+        "value": head["tops"], "unit": "TOP/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
+        "ms_per_step": head["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "s8", "data": "synthetic",
+        "config": {"workload": "Llama-3-8B prefill linear M=2048 K=4096 N=14336, quint8 act x qint8 per-channel weights, "
+                               "_QuantizedMatMul [BiasAdd, Requantize] -> qint8, one launch per step"},
+        "roofline": {"bound": "mfma", "achieved": head["tops_kernel"], "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
+                     "frac": head["tops_kernel"] / PEAK_INT8_TOPS, "traffic": traffic,
+                     "kernel": "qgemm_tile_kernel", "us_per_launch": head["us_kernel"]},
+        "cpu_baseline": cpu,
+        "targets": {k: v for k, v in targets.items() if v is not None},
+    }
+    text = json.dumps(line)
+    if len(text) >= MAX_LINE_BYTES:   # never let an optional part push the record over the limit
+        line.pop("targets")
+    return line
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -717,7 +761,7 @@ def main():
     others = []
 
     M, K, N = 2048, 4096, 14336
-    head = bench_linear(torch, hip, timer, M, K, N, "requant_s8", K_steps, W, dev, seed=22)
+    head = bench_linear(torch, hip, timer, M, K, N, "requant_s8", K_steps, W, dev, seed=22, keep_out=True)
     ctx = head.pop("_ctx")
 
     ceiling = bench_mfma_ceiling(torch, hip, timer, ctx["xq"], ctx["layers"][0]["wq"], dev)
@@ -766,32 +810,24 @@ def main():
         except Exception as exc:  # not available in this PyTorch build
             power["vendor_int8_gemm_torch_int_mm"] = dict(error=str(exc)[:200])
 
-    cpu = None
+    cpu, cpu_detail = None, None
     if not args.no_cpu:
         rows = min(args.cpu_rows, M)
         tops_cpu, dt, y_cpu = cpu_baseline_gemm(ctx, rows, K, N)
-        # the same rows from the GPU must be identical
-        L = ctx["layers"][0]
-        ep = hip.qmatmul_epilogue_desc(ctx["p"], N)
-        out = torch.empty(M, N, dtype=torch.int8, device=dev)
-        hip.qmatmul_prepare(ctx["p"], L["min_b"], L["max_b"], N, L["bias"], L["colsum"], N, L["scales"], L["sbias"],
-                            _stream(torch))
-        hip.qgemm(ctx["xq"], hip.QUINT8, L["packed"], L["colsum"], M, K, N, L["scales"], L["sbias"], ep, hip.QINT8,
-                  out, _stream(torch))
-        torch.cuda.synchronize()
-        same = bool((out[:rows].cpu().numpy() == y_cpu).all())
+        # the same rows as the timed launches of itexhip_qmatmul left them in the output buffer must be identical
+        same = bool((ctx["out_timed"][:rows].cpu().numpy() == y_cpu).all())
         cores = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
         cpu = dict(value=tops_cpu, unit="TOP/s", cores=cores, kind="port",
-                   sample="first %d of %d rows of the headline workload (same weights), %.1f s; GPU rows identical: %s"
-                          % (rows, M, dt, same))
+                   sample="first %d of %d rows of the headline workload (same weights), %.1f s; output of the timed GPU "
+                          "launches identical: %s" % (rows, M, dt, same))
         L = ctx["layers"][0]
         alt = cpu_onednn_in_torch(torch, ctx["xq"][:rows].cpu().numpy(), L["wq"].cpu().numpy(),
                                   (L["max_b"].cpu().numpy() / 127.0).astype("float32"), L["bias"].cpu().numpy())
         if alt:
-            cpu["onednn_in_torch"] = dict(value=alt[0], unit="TOP/s", threads=alt[1],
+            cpu_detail = dict(onednn_in_torch=dict(value=alt[0], unit="TOP/s", threads=alt[1],
                                           note="torch.ops.onednn.qlinear_pointwise (oneDNN bundled with PyTorch, fp32 output) "
                                                "on the same rows and weights: the nearest executable relative of the "
-                                               "reference's CPU path, not ITEX itself")
+                                               "reference's CPU path, not ITEX itself"))
     del ctx
 
     if "c1" in only:
@@ -872,26 +908,31 @@ def main():
         except Exception:
             traffic = None
 
-    line = {
-        "metric": "int8 GEMM TOPS (% MFMA peak); quantize/GEMV GB/s (% HBM peak), 1 MI355X",
-        "value": head["tops"], "unit": "TOP/s", "n_gpus": 1, "steps": K_steps, "warmup": W,
-        "ms_per_step": head["ms_per_step"], "clock_ramp_ms": RAMP_MS, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "s8/u8 x s8 -> s32 (fp32 epilogue)", "data": "synthetic",
-        "config": {"workload": "Llama-3-8B prefill linear M=2048 K=4096 N=14336: quint8 act (MIN_FIRST, N(0,1) + 0.1% x20 "
-                               "outliers) x qint8 per-channel weights, _QuantizedMatMul [BiasAdd, Requantize] -> qint8; "
-                               "step = one launch of the op (the kernel derives scales and bias itself)"},
-        "roofline": {"bound": "mfma", "achieved": head["tops_kernel"], "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
-                     "frac": head["tops_kernel"] / PEAK_INT8_TOPS, "traffic": traffic, "traffic_note": traffic_note,
-                     "power": power,
-                     "kernel": "qgemm_tile_kernel", "us_per_launch": head["us_kernel"],
-                     "note": "ops are int8 multiply-accumulates (2*M*N*K per launch); achieved and peak are tera-ops/s",
-                     "mfma_only_rate_measured": ceiling,
-                     "mfma_only_note": "TOP/s of back-to-back 32x32x32 i8 MFMAs on all CUs with no other instruction, "
-                                       "measured in this run: the matrix cores' sustained rate depends on operand bit "
-                                       "toggling (clock under load), so 'workload_data' is the practical ceiling"},
-        "cpu_baseline": cpu,
+    detail = {
+        "clock_ramp_ms": RAMP_MS,
+        "roofline_detail": {
+            "traffic_note": traffic_note, "power": power,
+            "note": "ops are int8 multiply-accumulates (2*M*N*K per launch); achieved and peak are tera-ops/s",
+            "mfma_only_rate_measured": ceiling,
+            "mfma_only_note": "TOP/s of back-to-back 32x32x32 i8 MFMAs on all CUs with no other instruction, "
+                              "measured in this run: the matrix cores' sustained rate depends on operand bit "
+                              "toggling (clock under load), so 'workload_data' is the practical ceiling"},
+        "cpu_baseline_detail": cpu_detail,
         "others": others,
     }
+    line = summary_line(head, K_steps, W, traffic, cpu, others)
+    # every other workload and the long notes: on an earlier line (and in a file next to the other run outputs), so
+    # that the last line of stdout stays a short record
+    full = dict(line)
+    full.update(detail)
+    print("BENCH_DETAIL " + json.dumps(full))
+    try:
+        os.makedirs(os.path.join(ROOT, "gpurun_out"), exist_ok=True)
+        with open(os.path.join(ROOT, "gpurun_out", "bench_full.json"), "w") as f:
+            json.dump(full, f)
+    except OSError:
+        pass
+    sys.stdout.flush()
     print(json.dumps(line))
 
 

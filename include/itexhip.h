@@ -48,6 +48,10 @@ enum { ITEXHIP_MIN_COMBINED = 0, ITEXHIP_MIN_FIRST = 1, ITEXHIP_SCALED = 2,
 const char* itexhip_last_error(void);
 /* "gfx950" and the library version; no GPU call. */
 const char* itexhip_build_info(void);
+/* Test hook (no counterpart in the reference): forces the tile shape of the MatMul tile kernel (0..4 = 256x256,
+ * 256x192, 256x128, 128x128, 64x64) and of the implicit-GEMM Conv2D (0..2 = 256x128, 128x128, 64x64) for every later
+ * call of the process; -1 gives the choice back to the library.  Results do not depend on the shape. */
+void itexhip_test_force_tile_shape(int matmul_shape, int conv_shape);
 
 /* ------------------------------------------------------------------------------------------
  * Stream-ordered host-to-device copy of small parameter vectors (per-channel ranges, per-axis
@@ -193,7 +197,11 @@ int itexhip_quantize_dynamic_rows(const float* x, void* q, int64_t rows, int64_t
  * state[0..5] of itexhip_quantize_dynamic ([0..1] the tensor's min and max, [2..3] the op's output_min / output_max,
  * [4..5] scale and addend).  4 <= n <= 2^36; x 16-byte, q 4-byte, range_out 8-byte aligned; anything else is rejected.
  * Same bytes in q and the same six floats as itexhip_quantize_dynamic.  Calls that overlap in time on one GPU (two
- * streams, two threads) share the array and race: serialise them. */
+ * streams, two threads) share the array and race: serialise them.
+ * The first call on each device looks the array's address up (hipGetDevice + hipGetSymbolAddress, which may load the
+ * code object); every later call on that device only launches the two kernels.  A caller that captures the call into a
+ * HIP graph therefore makes one ordinary call on that device before the capture starts.  `stream` must belong to the
+ * current device, as for any kernel launch. */
 int itexhip_quantize_dynamic_static(const float* x, void* q, int64_t n, int dst_type, int mode, float ensure_minimum_range,
                                     float* range_out, void* stream);
 

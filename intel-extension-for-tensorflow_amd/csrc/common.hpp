@@ -19,6 +19,9 @@ typedef int i4 __attribute__((ext_vector_type(4)));
 
 void set_error(const char* fmt, ...);
 
+// Tile shape forced by itexhip_test_force_tile_shape (-1: chosen from the problem size); [0] MatMul, [1] Conv2D.
+extern int g_forced_tile_shape[2];
+
 inline int hip_fail(hipError_t e, const char* what) {
   set_error("%s: %s", what, hipGetErrorString(e));
   return ITEXHIP_INTERNAL;

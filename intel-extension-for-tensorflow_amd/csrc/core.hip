@@ -8,6 +8,8 @@ namespace {
 thread_local char g_error[512] = "";
 }
 
+int g_forced_tile_shape[2] = {-1, -1};
+
 void set_error(const char* fmt, ...) {
   va_list ap;
   va_start(ap, fmt);
@@ -17,6 +19,11 @@ void set_error(const char* fmt, ...) {
 }  // namespace itexhip
 
 extern "C" const char* itexhip_last_error(void) { return itexhip::g_error; }
+
+extern "C" void itexhip_test_force_tile_shape(int matmul_shape, int conv_shape) {
+  __atomic_store_n(&itexhip::g_forced_tile_shape[0], matmul_shape, __ATOMIC_RELAXED);
+  __atomic_store_n(&itexhip::g_forced_tile_shape[1], conv_shape, __ATOMIC_RELAXED);
+}
 
 extern "C" const char* itexhip_build_info(void) { return "itexhip 0.1 gfx950"; }
 

@@ -625,11 +625,9 @@ int launch_tile(const uint8_t* a, uint32_t amask, const uint8_t* bp, int M, int 
 inline int pick_tile_shape(int M, int N, bool wide_only, int first = 0) {
   struct Shape { int bm, bn; double penalty; };
   static const Shape shapes[5] = {{256, 256, 1.0}, {256, 192, 1.03}, {256, 128, 1.08}, {128, 128, 1.2}, {64, 64, 1.8}};
-  // ITEXHIP_TILE_SHAPE=0..4 forces a shape (tests exercise every shape on ragged problems with it)
-  if (const char* forced = std::getenv("ITEXHIP_TILE_SHAPE")) {
-    const int f = std::atoi(forced);
-    if (f >= (wide_only ? 3 : first) && f < 5) return f;
-  }
+  // itexhip_test_force_tile_shape forces a shape (tests exercise every shape on ragged problems with it)
+  const int f = __atomic_load_n(&g_forced_tile_shape[0], __ATOMIC_RELAXED);
+  if (f >= (wide_only ? 3 : first) && f < 5) return f;
   int best = 3;
   double best_cost = 1e300;
   for (int i = wide_only ? 3 : first; i < 5; ++i) {
@@ -715,10 +713,8 @@ int dispatch_tile_conv(const uint8_t* x, uint32_t a_xor, const uint8_t* bp, int 
     const double cost = std::ceil(tiles / 256.0) * shapes[i].bm * shapes[i].bn * shapes[i].penalty;
     if (cost < best_cost) { best_cost = cost; best = i; }
   }
-  if (const char* forced = std::getenv("ITEXHIP_CONV_TILE_SHAPE")) {  // tests exercise every shape with it
-    const int f = std::atoi(forced);
-    if (f >= 0 && f < 3) best = f;
-  }
+  const int f = __atomic_load_n(&g_forced_tile_shape[1], __ATOMIC_RELAXED);  // tests exercise every shape with it
+  if (f >= 0 && f < 3) best = f;
   switch (best) {
     case 0: return launch_tile<256, 128, 2, 2, OUT_T, 2, false, true>(x, a_xor, bp, M, K, N, e, out, st, cv);
     case 1: return launch_tile<128, 128, 2, 2, OUT_T, 2, false, true>(x, a_xor, bp, M, K, N, e, out, st, cv);

@@ -26,7 +26,7 @@ EXPORTS = [
     "itexhip_stream_query", "itexhip_event_create", "itexhip_event_destroy", "itexhip_event_record",
     "itexhip_event_query", "itexhip_event_synchronize", "itexhip_stream_wait_event", "itexhip_device_synchronize",
     "itexhip_memcpy_d2h_async", "itexhip_memset8_async", "itexhip_memset32_async", "itexhip_launch_host_func",
-    "itexhip_last_error", "itexhip_build_info", "itexhip_memcpy_h2d_async", "itexhip_memcpy_d2h", "itexhip_memcpy_d2d_async", "itexhip_stream_synchronize", "itexhip_quantize", "itexhip_quantize_axis",
+    "itexhip_last_error", "itexhip_build_info", "itexhip_test_force_tile_shape", "itexhip_memcpy_h2d_async", "itexhip_memcpy_d2h", "itexhip_memcpy_d2d_async", "itexhip_stream_synchronize", "itexhip_quantize", "itexhip_quantize_axis",
     "itexhip_dequantize", "itexhip_dequantize_axis", "itexhip_quantize_bf16", "itexhip_quantize_axis_bf16",
     "itexhip_dequantize16", "itexhip_dequantize_axis16", "itexhip_requantize_per_channel",
     "itexhip_requantize", "itexhip_minmax_i32_per_channel", "itexhip_minmax_f32",
@@ -102,6 +102,13 @@ def _i64(v):
 
 def build_info():
     return _lib.itexhip_build_info().decode()
+
+
+def force_tile_shape(matmul=-1, conv=-1):
+    """Test hook: forces the tile shape of the MatMul tile kernel / the implicit-GEMM Conv2D for every later call (-1: the
+    library chooses)."""
+    _lib.itexhip_test_force_tile_shape.restype = None
+    _lib.itexhip_test_force_tile_shape(C.c_int(int(matmul)), C.c_int(int(conv)))
 
 
 def memcpy_d2h(host_array, src, nbytes, stream=0):

@@ -34,6 +34,11 @@
  *   the bfloat16 / half bias (Tbias): the adjusted bias is rounded to Tbias as the code is
  *   written (quantized_matmul_common.h:578-599, 609-617); the reference's tests only use float and
  *   qint32 biases;
+ *   classic MIN_FIRST QuantizeV2 (classic_asymmetric_algorithm): orc_quantize_v2 adds the zero point in fp32 BEFORE
+ *   rounding, sat(rne(fl(x * scale) + zp)), which is how a oneDNN reorder applies a destination zero point; the
+ *   other reading, rne(x * scale) + zp, differs when x * scale lies just under a half and the sum rounds up to one
+ *   (1.4999999 + 64 -> 65.5 -> 66 against 65).  The reference's vector [0,144,176,223,239,255] holds no such
+ *   element, so it does not separate the two;
  *   legacy MIN_FIRST QuantizeV2 with an axis (per-slice ranges): the reference describes the shift operand of its
  *   binary_add as a one-element tensor (quantize_op.h:302-303, dims all 1) while handing it a shift per slice and
  *   per-axis scale masks that the oneDNN binary primitive does not take; its tests run per-axis quantization in

@@ -31,3 +31,12 @@ def dev():
     import torch
     assert torch.cuda.is_available(), "GPU tests need a GPU"
     return torch.device("cuda:0")
+
+
+@pytest.fixture(autouse=True)
+def _tile_shape_choice_restored():
+    """A test that forced a tile shape (hip.force_tile_shape) does not leave it forced for the next one."""
+    yield
+    pkg = sys.modules.get("itex_amd")
+    if pkg is not None and hasattr(pkg, "itexhip"):
+        pkg.itexhip.force_tile_shape(-1, -1)

@@ -182,7 +182,7 @@ def test_implicit_gemm_conv(hip, dev, monkeypatch, shape, wshape, strides, dil, 
     accumulators, and bit for bit against the patch-matrix path (itexhip_im2col8 + itexhip_qgemm) for every output
     type with per-channel scales, bias and ReLU."""
     if tile_shape is not None:   # every tile shape of the kernel on every case, ragged edges included
-        monkeypatch.setenv("ITEXHIP_CONV_TILE_SHAPE", str(tile_shape))
+        hip.force_tile_shape(conv=tile_shape)
     check_implicit_conv(hip, dev, shape, wshape, strides, dil, lead, signed_in, np.random.default_rng(sum(shape) + sum(wshape) + signed_in))
 
 
@@ -205,9 +205,9 @@ def test_implicit_gemm_conv_random_geometries(hip, dev, monkeypatch, seed):
             continue
         tile_shape = int(rng.integers(-1, 3))
         if tile_shape >= 0:
-            monkeypatch.setenv("ITEXHIP_CONV_TILE_SHAPE", str(tile_shape))
+            hip.force_tile_shape(conv=tile_shape)
         else:
-            monkeypatch.delenv("ITEXHIP_CONV_TILE_SHAPE", raising=False)
+            hip.force_tile_shape(conv=-1)
         check_implicit_conv(hip, dev, (B, H, W, C), (kh, kw, C, O), strides, dil, lead, bool(rng.integers(0, 2)), rng)
         done += 1
 

@@ -220,9 +220,9 @@ def test_random_shapes_on_every_path_vs_oracle(hip, dev, monkeypatch, seed):
         kw = [V2_DEQ, V2_DEQ_RELU, V2_REQ_S8, V2_REQ_U8_RELU, V1_S32][int(rng.integers(0, 5))]
         shape = int(rng.integers(-1, 5))
         if shape >= 0:
-            monkeypatch.setenv("ITEXHIP_TILE_SHAPE", str(shape))
+            hip.force_tile_shape(matmul=shape)
         else:
-            monkeypatch.delenv("ITEXHIP_TILE_SHAPE", raising=False)
+            hip.force_tile_shape(matmul=-1)
         layer, w, bias = make_layer(hip, dev, K, N, seed=seed * 100 + case)
         x, xq, mn, mx = make_acts(M, K, seed=seed * 100 + case + 50)
         full = x @ w + bias
@@ -277,12 +277,10 @@ def test_single_launch_op_vs_oracle(hip, dev, kw, per_channel, M):
 @pytest.mark.parametrize("M,K,N,kw", [(300, 448, 528, V2_REQ_S8), (513, 192, 400, V2_DEQ_RELU), (257, 64, 208, V1_S32),
                                       (40, 1024, 96, V2_REQ_U8_RELU), (256, 320, 200, V2_REQ_S8)])
 def test_every_tile_shape_on_ragged_problems(hip, dev, monkeypatch, shape, M, K, N, kw):
-    """The tile shape is normally chosen from the problem size; ITEXHIP_TILE_SHAPE forces one, so that
+    """The tile shape is normally chosen from the problem size; itexhip_test_force_tile_shape forces one, so that
     every shape (256x256, 256x192, 256x128, 128x128, 64x64) meets partial tiles in M and N, odd step
     counts, K not a multiple of 64 and the element-wise store path (N * element size not a multiple of 16)."""
-    import os
-    monkeypatch.setenv("ITEXHIP_TILE_SHAPE", str(shape))
-    assert os.environ["ITEXHIP_TILE_SHAPE"] == str(shape)
+    hip.force_tile_shape(matmul=shape)
     layer, w, bias = make_layer(hip, dev, K, N, seed=K + N + shape)
     x, xq, mn, mx = make_acts(M, K, seed=M)
     r_out = float(np.abs(np.maximum(x @ w + bias, 0) if kw.get("activation") else x @ w + bias).max())
@@ -317,7 +315,7 @@ def test_canonical_chains_every_tile_shape(hip, dev, monkeypatch, shape, chain):
     and not (per-lane clamped addresses), ragged M and N: bit-equal to the oracle except for the GELU and the other
     transcendental chains, where the device's exp / erf need not round like the host's (2e-6 relative, 1e-6 absolute; one unit of the
     output type where that is coarser)."""
-    monkeypatch.setenv("ITEXHIP_TILE_SHAPE", str(shape))
+    hip.force_tile_shape(matmul=shape)
     kw = CHAINS[chain]
     for M, K, N in [(300, 448, 528), (257, 208, 400)]:
         layer, w, bias = make_layer(hip, dev, K, N, seed=K + N + shape)
@@ -498,14 +496,17 @@ def test_config1_literal(hip, dev):
         np.testing.assert_array_equal(layer.run(xq, kw, mn, mx, 0.0, r_out), ref)
 
 
+@pytest.mark.parametrize("path", ["auto", "fused"])
 @pytest.mark.parametrize("K,N,relu", [(768, 2304, False), (768, 768, False), (768, 3072, True), (3072, 768, False)])
-def test_bert_linears_rows_sampled(hip, dev, K, N, relu):
-    """BERT-base encoder linears at full size (M = 4096); the oracle checks 96 sampled rows exactly."""
+def test_bert_linears_rows_sampled(hip, dev, K, N, relu, path):
+    """BERT-base encoder linears at full size (M = 4096); the oracle checks 96 sampled rows exactly.  Both forms of
+    the op: parameter vectors prepared by a launch of their own ("auto") and the single launch the op kernel and
+    the benchmark use, which derives them inside the MatMul kernel ("fused")."""
     M = 4096
     layer, w, bias = make_layer(hip, dev, K, N, seed=K * 3 + N)
     x, xq, mn, mx = make_acts(M, K, seed=1)
     kw = V2_DEQ_RELU if relu else V2_DEQ
-    got = layer.run(xq, kw, mn, mx)
+    got = layer.run(xq, kw, mn, mx, path=path)
     rows = np.random.default_rng(2).choice(M, 96, replace=False)
     ref = layer.oracle(xq[rows], kw, mn, mx)
     np.testing.assert_array_equal(got[rows], ref)
@@ -516,13 +517,17 @@ def test_bert_linears_rows_sampled(hip, dev, K, N, relu):
 @pytest.mark.parametrize("K,N", [(4096, 4096), (4096, 6144), (4096, 14336), (14336, 4096)])
 def test_llama_prefill_rows_sampled(hip, dev, K, N):
     """Llama-3-8B prefill linears at full size (M = 2048): int8 output bit-exact on 64 sampled rows, and the
-    size-independent property sum_n acc[m, n] = a[m, :] . rowsum(w) on the s32 output of all rows."""
+    size-independent property sum_n acc[m, n] = a[m, :] . rowsum(w) on the s32 output of all rows.  The single-launch
+    form of the op (what the op kernel and the benchmark time) must give the same bytes as the two-step form
+    everywhere, not only on the sampled rows."""
     import torch
     M = 2048
     layer, w, bias = make_layer(hip, dev, K, N, seed=20 + K % 7 + N % 11)
     x, xq, mn, mx = make_acts(M, K, seed=21, outlier=1e-3)
     r_out = float(np.abs(x[:64] @ w + bias).max()) * 1.5
     got = layer.run(xq, V2_REQ_S8, mn, mx, -r_out, r_out)
+    got_single = layer.run(xq, V2_REQ_S8, mn, mx, -r_out, r_out, path="fused")
+    np.testing.assert_array_equal(got_single, got)
     rows = np.random.default_rng(3).choice(M, 64, replace=False)
     ref = layer.oracle(xq[rows], V2_REQ_S8, mn, mx, -r_out, r_out)
     np.testing.assert_array_equal(got[rows], ref)
@@ -537,15 +542,20 @@ def test_llama_prefill_rows_sampled(hip, dev, K, N):
     np.testing.assert_array_equal(acc.sum(1), xq.astype(np.int64) @ rowsum_w)
 
 
+@pytest.mark.parametrize("mode", [orc.MIN_FIRST, orc.SCALED])
 @pytest.mark.parametrize("M", [1, 4, 16])
 @pytest.mark.parametrize("K,N", [(4096, 14336), (14336, 4096)])
-def test_llama_decode_gemv(hip, dev, M, K, N):
-    """Llama-3-8B decode shapes at full size, every output checked against the oracle."""
+def test_llama_decode_gemv(hip, dev, M, K, N, mode):
+    """Llama-3-8B decode shapes at full size, every output checked against the oracle: MIN_FIRST quint8 and SCALED
+    qint8 activations (zero bias, which also keeps the reference's as-written bias scaling of the SCALED form out of
+    the result), two-step and single-launch form."""
     layer, w, bias = make_layer(hip, dev, K, N, seed=10 + M)
     layer_zero_bias = Linear(hip, dev, layer.wq, layer.min_b, layer.max_b, np.zeros(N, np.float32))
-    x, xq, mn, mx = make_acts(M, K, seed=11 + M)
-    ref = layer_zero_bias.oracle(xq, V2_DEQ, mn, mx)
-    np.testing.assert_array_equal(layer_zero_bias.run(xq, V2_DEQ, mn, mx), ref)
+    x, xq, mn, mx = make_acts(M, K, seed=11 + M, mode=mode)
+    kw = dict(V2_DEQ, input_mode=mode)
+    ref = layer_zero_bias.oracle(xq, kw, mn, mx)
+    np.testing.assert_array_equal(layer_zero_bias.run(xq, kw, mn, mx), ref)
+    np.testing.assert_array_equal(layer_zero_bias.run(xq, kw, mn, mx, path="fused"), ref)
     assert np.abs(ref - x @ w).max() < 0.2
 
 
@@ -583,34 +593,37 @@ def test_per_token_activation_ranges(hip, dev, M, kw, K, N):
                             layer.min_b_d, layer.max_b_d, layer.min_b.size, layer.bias_d, out)
 
 
+@pytest.mark.parametrize("T,mode", [(orc.QUINT8, orc.MIN_FIRST), (orc.QINT8, orc.SCALED)])
 @pytest.mark.parametrize("M", [1, 4, 16])
 @pytest.mark.parametrize("K,N", [(4096, 14336), (14336, 4096)])
-def test_llama_decode_per_token_full_size(hip, dev, M, K, N):
+def test_llama_decode_per_token_full_size(hip, dev, M, K, N, T, mode):
     """The decode shapes at full size with per-token activation ranges, from float activations: the per-row dynamic
     quantization (itexhip_quantize_dynamic_rows) must equal QuantizeV2 of each row against its own range, and every
-    output of itexhip_qmatmul_per_row the oracle's 1 x K problem with that row's range."""
+    output of itexhip_qmatmul_per_row the oracle's 1 x K problem with that row's range.  MIN_FIRST quint8 and SCALED qint8
+    activations."""
     import torch
     layer, w, bias = make_layer(hip, dev, K, N, seed=30 + M)
     rng = np.random.default_rng(40 + M + K)
     x = (rng.standard_normal((M, K)) * rng.uniform(0.5, 2.0, (M, 1))).astype(np.float32)
     rows_q, mins, maxs = [], [], []
     for m in range(M):
-        _, q, mn, mx = orc.quantize_v2(x[m:m + 1], x[m].min(), x[m].max(), orc.QUINT8, orc.MIN_FIRST)
+        _, q, mn, mx = orc.quantize_v2(x[m:m + 1], x[m].min(), x[m].max(), T, mode)
         rows_q.append(q)
         mins.append(mn[0])
         maxs.append(mx[0])
     xq_ref = np.concatenate(rows_q, 0)
     x_d = torch.from_numpy(x).to(dev)
-    xq_d = torch.empty((M, K), dtype=torch.uint8, device=dev)
+    xq_d = torch.empty((M, K), dtype=tdt(T), device=dev)
     rmn = torch.empty(M, dtype=torch.float32, device=dev)
     rmx = torch.empty(M, dtype=torch.float32, device=dev)
-    hip.quantize_dynamic_rows(x_d, xq_d, M, K, orc.QUINT8, orc.MIN_FIRST, 0.01, rmn, rmx)
+    hip.quantize_dynamic_rows(x_d, xq_d, M, K, T, mode, 0.01, rmn, rmx)
     torch.cuda.synchronize()
     np.testing.assert_array_equal(xq_d.cpu().numpy(), xq_ref)
     np.testing.assert_array_equal(rmn.cpu().numpy(), np.array(mins, np.float32))
     np.testing.assert_array_equal(rmx.cpu().numpy(), np.array(maxs, np.float32))
-    ref = np.concatenate([layer.oracle(xq_ref[m:m + 1], V2_DEQ, mins[m], maxs[m]) for m in range(M)], 0)
-    p = hip.matmul_params(t_in=orc.QUINT8, min_a=0.0, max_a=0.0, **V2_DEQ)
+    kw = dict(V2_DEQ, input_mode=mode)
+    ref = np.concatenate([layer.oracle(xq_ref[m:m + 1], kw, mins[m], maxs[m]) for m in range(M)], 0)
+    p = hip.matmul_params(t_in=T, min_a=0.0, max_a=0.0, **kw)
     out = torch.empty((M, N), dtype=torch.float32, device=dev)
     hip.qmatmul_per_row(p, xq_d, layer.packed, layer.colsum, M, K, N, rmn, rmx, layer.min_b_d, layer.max_b_d,
                         layer.min_b.size, layer.bias_d, out)
@@ -891,7 +904,7 @@ def test_bfloat16_rounding_of_special_values(hip, dev, path):
 @pytest.mark.parametrize("shape", [0, 1, 2, 3, 4])
 @pytest.mark.parametrize("V2_DEQ_BF16", [V2_DEQ_BF16, V2_DEQ_F16], ids=["bf16", "f16"])
 def test_bfloat16_output_every_tile_shape(hip, dev, monkeypatch, shape, V2_DEQ_BF16):
-    monkeypatch.setenv("ITEXHIP_TILE_SHAPE", str(shape))
+    hip.force_tile_shape(matmul=shape)
     for M, K, N in [(513, 192, 400), (260, 320, 203)]:
         layer, w, bias = make_layer(hip, dev, K, N, seed=N + shape)
         x, xq, mn, mx = make_acts(M, K, seed=M)

@@ -70,3 +70,39 @@ def test_static_scratch_entry_rejects_what_it_cannot_take(hip, dev):
         hip.quantize_dynamic_static(x[1:], q, 32, orc.QINT8, orc.SCALED, 0.01, r)
     with pytest.raises(hip.ItexHipError):
         hip.quantize_dynamic_static(x, q, 64, orc.QINT8, orc.MIN_FIRST, 0.01, r)   # MIN_FIRST quantizes to quint8
+
+
+def test_static_scratch_entry_in_a_hip_graph(hip, dev):
+    """After one ordinary call on the device the entry point only launches kernels, so it can be captured into a HIP
+    graph.  The graph is replayed on new input contents with eager work and synchronisations between the replays,
+    and every replay must leave the bytes itexhip_quantize_dynamic leaves for the same input."""
+    import torch
+    T, mode = orc.QUINT8, orc.MIN_FIRST
+    n = (1 << 20) + 8
+    x_static = torch.zeros(n, dtype=torch.float32, device=dev)
+    q_graph = torch.zeros(n, dtype=torch.uint8, device=dev)
+    r_graph = torch.zeros(8, dtype=torch.float32, device=dev)
+    q_eager = torch.zeros(n, dtype=torch.uint8, device=dev)
+    state = torch.zeros(hip.DYNAMIC_STATE_FLOATS, dtype=torch.float32, device=dev)
+    hip.quantize_dynamic_static(x_static, q_graph, n, T, mode, 0.01, r_graph)   # resolves the array's address: not capturable
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.graph(graph, stream=side):
+        hip.quantize_dynamic_static(x_static, q_graph, n, T, mode, 0.01, r_graph, torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    rng = np.random.default_rng(5)
+    for rep in range(4):
+        x = (rng.standard_normal(n) * (0.5 + rep)).astype(np.float32)
+        x_static.copy_(torch.from_numpy(x).to(dev))
+        q_graph.fill_(7)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        hip.quantize_dynamic(x_static, q_eager, n, T, mode, 0.01, state)
+        torch.cuda.synchronize()
+        np.testing.assert_array_equal(q_graph.cpu().numpy(), q_eager.cpu().numpy())
+        np.testing.assert_array_equal(r_graph[:6].cpu().numpy().view(np.uint32), state[:6].cpu().numpy().view(np.uint32))
+        _, q_orc, _, _ = orc.quantize_v2(x, x.min(), x.max(), T, mode)
+        np.testing.assert_array_equal(q_graph.cpu().numpy(), q_orc)
