@@ -1,14 +1,19 @@
 #!/usr/bin/env python3
 """Benchmark of the INT8 quantized-inference hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only NAME[,NAME...]] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only NAME[,NAME...]] [--no-cpu] [--tile-shape S]
 
 Headline ("value"): the Llama-3-8B-shaped INT8 prefill linear, M=2048 K=4096 N=14336, quint8
 activations x per-channel qint8 weights, fused bias + requantize to qint8 (`_QuantizedMatMul`
-fused_ops=[BiasAdd, Requantize]).  One step = the device-side parameter preparation kernel plus the
-MFMA GEMM kernel, inputs resident in HBM.  The same JSON line carries, under "others", the other
-benchmark workloads (standalone quantization ops at 2^28 elements, decode GEMV, BERT linears, the
-remaining prefill shapes), each with its own roofline fraction.
+fused_ops=[BiasAdd, Requantize]).  One step = one launch of the op (the kernel derives the channels'
+scales and biases itself), inputs resident in HBM.
+
+Output.  The LAST line of stdout is one short JSON record (under 4 KB): the headline workload with its
+`roofline` and `cpu_baseline`, plus `targets`, the worst roofline fraction of each other workload family.
+The line before it, prefixed "BENCH_DETAIL ", is the same record with everything else: under "others" every
+other workload (standalone quantization ops at 2^28 elements, decode GEMV, BERT linears, the remaining
+prefill shapes, ...) with its own roofline fraction, and under "roofline" the power samples and notes; the
+same JSON is written to gpurun_out/bench_<sections>.json.
 
 Timing uses HIP events on the stream the kernels are launched on (PyTorch's current stream, whose
 raw handle is passed through the C ABI).
@@ -746,6 +751,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--only", type=str, default="", help="comma list of: headline, c1, prefill, bert, bmm, conv, gemv, elementwise, copy, power")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--tile-shape", type=int, default=-1,
+                    help="force the tile shape of the MatMul tile kernel (0..4) for this run; results do not depend on it")
     ap.add_argument("--cpu-rows", type=int, default=2048, help="rows of the headline workload the CPU oracle runs")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -756,8 +763,13 @@ def main():
     torch, hip = _setup()
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    if args.tile_shape >= 0:
+        hip.force_tile_shape(matmul=args.tile_shape)
     timer = Timer(torch)
     K_steps, W = args.steps, args.warmup
+    # launches of 4 - 25 us (every workload below except the prefill shapes and the 2^28-element ops): the start of a
+    # timed region costs a fixed 10 - 20 us, which 20 such launches do not amortise, so these rows time at least 100
+    S_steps = max(K_steps, 100)
     others = []
 
     M, K, N = 2048, 4096, 14336
@@ -831,7 +843,7 @@ def main():
     del ctx
 
     if "c1" in only:
-        others.extend(bench_config1_chain(torch, hip, timer, K_steps, W, dev))
+        others.extend(bench_config1_chain(torch, hip, timer, S_steps, W, dev))
     if "prefill" in only:
         others.append(bench_dynamic_linear(torch, hip, timer, 2048, 4096, 14336, max(10, K_steps // 2), max(3, W // 2), dev, seed=22))
         for (k, n, seed) in ((4096, 4096, 20), (4096, 6144, 21), (14336, 4096, 23)):
@@ -843,22 +855,22 @@ def main():
         for (k, n, kind, seed) in ((768, 2304, "deq", 1), (768, 768, "deq", 2), (768, 3072, "deq_relu", 3),
                                    (768, 3072, "deq_gelu", 3), (3072, 768, "deq", 4),
                                    (768, 2304, "deq_bf16", 1), (768, 3072, "deq_gelu_bf16", 3), (3072, 768, "deq_add", 4)):
-            r = bench_linear(torch, hip, timer, 4096, k, n, kind, K_steps, W, dev, seed, graph=True)
+            r = bench_linear(torch, hip, timer, 4096, k, n, kind, S_steps, W, dev, seed, graph=True)
             r.pop("_ctx")
             t_roof = max(r["ops"] / (PEAK_INT8_TOPS * 1e12), r["bytes"] / (PEAK_HBM_GBS * 1e9))
             r.update(name="bert_linear", bound="max(mfma,hbm)", frac=t_roof / (r["us_kernel"] * 1e-6),
                      frac_mfma=r["tops_kernel"] / PEAK_INT8_TOPS, frac_hbm=r["gbs_kernel"] / PEAK_HBM_GBS)
             others.append(r)
     if "bmm" in only:
-        others.extend(bench_bmm(torch, hip, timer, K_steps, W, dev))
+        others.extend(bench_bmm(torch, hip, timer, S_steps, W, dev))
     if "conv" in only:
-        others.extend(bench_conv(torch, hip, timer, K_steps, W, dev))
+        others.extend(bench_conv(torch, hip, timer, S_steps, W, dev))
     if "gemv" in only:
-        floor = bench_read_floor(torch, hip, timer, 4096 * 14336, K_steps, W, dev)
+        floor = bench_read_floor(torch, hip, timer, 4096 * 14336, S_steps, W, dev)
         others.append(floor)
         for (k, n) in ((4096, 14336), (14336, 4096)):
             for m in (1, 4, 16):
-                r = bench_linear(torch, hip, timer, m, k, n, "deq", K_steps, W, dev, seed=10, rotate=8, graph=True)
+                r = bench_linear(torch, hip, timer, m, k, n, "deq", S_steps, W, dev, seed=10, rotate=8, graph=True)
                 r.pop("_ctx")
                 r.update(name="decode_gemv", bound="hbm", frac=r["gbs_kernel"] / PEAK_HBM_GBS,
                          frac_graph=r["gbs_kernel_graph"] / PEAK_HBM_GBS,
@@ -867,13 +879,13 @@ def main():
                 others.append(r)
             # a batched decode step of 32 rows: the small-M kernel in two blocks of 16 rows (the workgroups of a strip share
             # its weights through one L2); the tile kernel would run 64 x 64 tiles over a fraction of the CUs here
-            r = bench_linear(torch, hip, timer, 32, k, n, "deq", K_steps, W, dev, seed=10, rotate=8, graph=True)
+            r = bench_linear(torch, hip, timer, 32, k, n, "deq", S_steps, W, dev, seed=10, rotate=8, graph=True)
             r.pop("_ctx")
             r.update(name="decode_gemv_32_rows", bound="hbm", frac=r["gbs_kernel"] / PEAK_HBM_GBS,
                      note="8 weight copies cycled; rows in blocks of 16")
             others.append(r)
-            others.append(bench_dynamic_linear(torch, hip, timer, 16, k, n, K_steps, W, dev, seed=10))
-            r = bench_linear(torch, hip, timer, 16, k, n, "deq", K_steps, W, dev, seed=10, rotate=8, per_row=True)
+            others.append(bench_dynamic_linear(torch, hip, timer, 16, k, n, S_steps, W, dev, seed=10))
+            r = bench_linear(torch, hip, timer, 16, k, n, "deq", S_steps, W, dev, seed=10, rotate=8, per_row=True)
             r.pop("_ctx")
             r.update(name="decode_gemv_per_token_ranges", bound="hbm", us_kernel=r["ms_per_step"] * 1e3,
                      gbs_kernel=r["bytes"] / (r["ms_per_step"] * 1e-3) / 1e9,
@@ -908,27 +920,25 @@ def main():
         except Exception:
             traffic = None
 
-    detail = {
-        "clock_ramp_ms": RAMP_MS,
-        "roofline_detail": {
-            "traffic_note": traffic_note, "power": power,
-            "note": "ops are int8 multiply-accumulates (2*M*N*K per launch); achieved and peak are tera-ops/s",
-            "mfma_only_rate_measured": ceiling,
-            "mfma_only_note": "TOP/s of back-to-back 32x32x32 i8 MFMAs on all CUs with no other instruction, "
-                              "measured in this run: the matrix cores' sustained rate depends on operand bit "
-                              "toggling (clock under load), so 'workload_data' is the practical ceiling"},
-        "cpu_baseline_detail": cpu_detail,
-        "others": others,
-    }
     line = summary_line(head, K_steps, W, traffic, cpu, others)
     # every other workload and the long notes: on an earlier line (and in a file next to the other run outputs), so
     # that the last line of stdout stays a short record
     full = dict(line)
-    full.update(detail)
+    full["clock_ramp_ms"] = RAMP_MS
+    full["roofline"] = dict(line["roofline"], traffic_note=traffic_note, power=power,
+                            note="ops are int8 multiply-accumulates (2*M*N*K per launch); achieved and peak are tera-ops/s",
+                            mfma_only_rate_measured=ceiling,
+                            mfma_only_note="TOP/s of back-to-back 32x32x32 i8 MFMAs on all CUs with no other instruction, "
+                                           "measured in this run: the matrix cores' sustained rate depends on operand bit "
+                                           "toggling (clock under load), so 'workload_data' is the practical ceiling")
+    if cpu is not None and cpu_detail:
+        full["cpu_baseline"] = dict(cpu, **cpu_detail)
+    full["others"] = others
     print("BENCH_DETAIL " + json.dumps(full))
     try:
         os.makedirs(os.path.join(ROOT, "gpurun_out"), exist_ok=True)
-        with open(os.path.join(ROOT, "gpurun_out", "bench_full.json"), "w") as f:
+        tag = "full" if not args.only else args.only.replace(",", "_")
+        with open(os.path.join(ROOT, "gpurun_out", "bench_%s.json" % tag), "w") as f:
             json.dump(full, f)
     except OSError:
         pass
