@@ -43,6 +43,18 @@ inline int hip_fail(hipError_t e, const char* what) {
 
 inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s); }
 
+// One bit per device ordinal (64 of them) for state that is per device, not per process, such as the dynamic
+// shared memory limit of a kernel: device_bit(mask, false) tells whether the current device's bit is set,
+// device_bit(mask, true) sets it (and returns whether it was set before).  Callers test, do their idempotent set-up,
+// then set the bit; two threads that arrive together both do the set-up.
+inline bool device_bit(unsigned long long* mask, bool set) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) dev = 0;
+  const unsigned long long bit = 1ull << (dev & 63);
+  if (set) return (__atomic_fetch_or(mask, bit, __ATOMIC_ACQ_REL) & bit) != 0;
+  return (__atomic_load_n(mask, __ATOMIC_ACQUIRE) & bit) != 0;
+}
+
 inline bool aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
 
 // Saturation bounds of the destination type, in fp32 (the s32 upper bound is the largest float

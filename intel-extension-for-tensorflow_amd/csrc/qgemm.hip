@@ -522,12 +522,12 @@ int launch_gemv(const uint8_t* a, uint32_t a_xor, const uint8_t* bp, int M, int 
   // the kernel's table of per-row parameters holds 16 rows
   ITEXHIP_REQUIRE(e.row_min_a == nullptr || M <= 16, "the small-M kernel takes per-row activation ranges for M <= 16 only");
   const size_t lds_max = static_cast<size_t>(8 * kGemvRing * 1024) * R + kGemvPanelWords * 16 * NT * 4;
-  static bool attr_set[3] = {false, false, false};  // benign race: the call is idempotent
-  if (!attr_set[variant]) {
+  static unsigned long long attr_done[3] = {0, 0, 0};  // per variant: devices on which the attribute is set
+  if (!device_bit(&attr_done[variant], false)) {
     hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                                          static_cast<int>(lds_max));
     if (err != hipSuccess) return hip_fail(err, "hipFuncSetAttribute(qgemv_kernel)");
-    attr_set[variant] = true;
+    device_bit(&attr_done[variant], true);
   }
   const size_t lds = static_cast<size_t>(waves) * kGemvRing * 1024 * R + kGemvPanelWords * 16 * NT * 4;
   const int strips = (N + 16 * NT - 1) / (16 * NT);

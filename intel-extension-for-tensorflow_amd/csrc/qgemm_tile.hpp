@@ -662,12 +662,12 @@ int launch_tile(const uint8_t* a, uint32_t amask, const uint8_t* bp, int M, int 
   constexpr size_t lds_bytes = 4 * (BM / 16 + BN / 16) * kChunkBytes + 12 * BN + (CONV ? kMaxConvPieces * 8 : 0);  // the most
   const size_t lds_now = lds_bytes - (CONV ? (kMaxConvPieces - (K >> 4)) * 8 : 0);
   auto kern = qgemm_tile_kernel<BM, BN, WAVES_M, WAVES_N, OUT_T, ACT, KALIGNED, CONV, ELEMENTWISE>;
-  static bool attr_set = false;  // benign race: the call is idempotent
-  if (!attr_set) {
+  static unsigned long long attr_done = 0;  // devices on which this instantiation's attribute is set
+  if (!device_bit(&attr_done, false)) {
     hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                          hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes));
     if (err != hipSuccess) return hip_fail(err, "hipFuncSetAttribute(qgemm_tile_kernel)");
-    attr_set = true;
+    device_bit(&attr_done, true);
   }
   kern<<<dim3(static_cast<unsigned>(num_m * num_n)), dim3(64 * WAVES_M * WAVES_N), lds_now, st>>>(
       a, amask, bp, M, K, N, KT, NT, num_m, num_n, xcd_rectangles(num_m, num_n, BM, BN, K), e, out, cv);
