@@ -858,8 +858,11 @@ def main():
             r = bench_linear(torch, hip, timer, 4096, k, n, kind, S_steps, W, dev, seed, graph=True)
             r.pop("_ctx")
             t_roof = max(r["ops"] / (PEAK_INT8_TOPS * 1e12), r["bytes"] / (PEAK_HBM_GBS * 1e9))
-            r.update(name="bert_linear", bound="max(mfma,hbm)", frac=t_roof / (r["us_kernel"] * 1e-6),
-                     frac_mfma=r["tops_kernel"] / PEAK_INT8_TOPS, frac_hbm=r["gbs_kernel"] / PEAK_HBM_GBS)
+            # launches of ~15 us: the better of back-to-back launches from the host and replays of the same launches
+            # from a HIP graph (a host hiccup in a region of 100 launches shows in the first, never in the second)
+            best = min(r["us_kernel"], r["us_kernel_graph"])
+            r.update(name="bert_linear", bound="max(mfma,hbm)", us_best=best, frac=t_roof / (best * 1e-6),
+                     frac_mfma=r["ops"] / (best * 1e-6) / 1e12 / PEAK_INT8_TOPS, frac_hbm=r["bytes"] / (best * 1e-6) / 1e9 / PEAK_HBM_GBS)
             others.append(r)
     if "bmm" in only:
         others.extend(bench_bmm(torch, hip, timer, S_steps, W, dev))
@@ -872,9 +875,10 @@ def main():
             for m in (1, 4, 16):
                 r = bench_linear(torch, hip, timer, m, k, n, "deq", S_steps, W, dev, seed=10, rotate=8, graph=True)
                 r.pop("_ctx")
-                r.update(name="decode_gemv", bound="hbm", frac=r["gbs_kernel"] / PEAK_HBM_GBS,
-                         frac_graph=r["gbs_kernel_graph"] / PEAK_HBM_GBS,
-                         read_floor_us=floor["us_kernel"], frac_of_read_floor=floor["us_kernel"] / r["us_kernel"],
+                best = min(r["us_kernel"], r["us_kernel_graph"])   # as for the read floor: eager or graph replay
+                r.update(name="decode_gemv", bound="hbm", us_best=best, frac=r["bytes"] / (best * 1e-6) / 1e9 / PEAK_HBM_GBS,
+                         frac_eager=r["gbs_kernel"] / PEAK_HBM_GBS, frac_graph=r["gbs_kernel_graph"] / PEAK_HBM_GBS,
+                         read_floor_us=floor["us_kernel"], frac_of_read_floor=floor["us_kernel"] / best,
                          note="8 weight copies cycled (470 MB > last-level cache)")
                 others.append(r)
             # a batched decode step of 32 rows: the small-M kernel in two blocks of 16 rows (the workgroups of a strip share

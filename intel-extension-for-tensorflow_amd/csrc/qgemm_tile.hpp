@@ -9,6 +9,15 @@
 
 #include "qgemm_common.hpp"
 
+// Measurement builds only (ablate.py): a bit mask of parts of the kernel that are compiled out, so that time, power
+// and energy of a launch can be attributed to them.  Such a build computes wrong results; the library is built with 0.
+//   1: no activation-fragment reads from LDS      2: no weight-fragment reads from LDS
+//   4: no operand loads inside the K loop (global -> LDS)      8: no MFMAs
+//  16: no epilogue (conversion, transposition, stores)        32: no sign flips of the activation fragments
+#ifndef ITEXHIP_ABLATE
+#define ITEXHIP_ABLATE 0
+#endif
+
 namespace itexhip {
 
 // ------------------------------------------------------------------------------------------------
@@ -300,16 +309,18 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void qgemm_tile_kernel(
       static_for<TM>([&](auto i) {
         constexpr int ii = decltype(i)::value;
         constexpr int t = j * TM + ii;
-        acc[t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fb[s % FBN], fa_cur[kc * TM + ii], acc[t], 0, 0, 0);
+        if constexpr ((ITEXHIP_ABLATE & 8) == 0) acc[t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fb[s % FBN], fa_cur[kc * TM + ii], acc[t], 0, 0, 0);
+        else asm volatile("" : : "v"(fb[s % FBN]), "v"(fa_cur[kc * TM + ii]));  // the fragments stay live
         // ---- the slot behind this MFMA
         if constexpr (ii == 0) {
           constexpr int sn = s + FBD;  // the slice whose weight fragment is read now
-          if constexpr (sn < NSLICE) fb[sn % FBN] = lds_b(st_cur, sn / TN, sn % TN);
+          if constexpr ((ITEXHIP_ABLATE & 2) != 0) asm volatile("" : "+v"(fb[sn % FBN]));
+          else if constexpr (sn < NSLICE) fb[sn % FBN] = lds_b(st_cur, sn / TN, sn % TN);
           else fb[sn % FBN] = lds_b(st_nxt, (sn - NSLICE) / TN, (sn - NSLICE) % TN);
         }
         if constexpr (ii == TM - 1) {
           static_for<NLD>([&](auto c) {
-            if constexpr (decltype(c)::value * NSLICE / NLD == s) issue_load(c, kt_load, st_fill, piece);
+            if constexpr ((ITEXHIP_ABLATE & 4) == 0 && decltype(c)::value * NSLICE / NLD == s) issue_load(c, kt_load, st_fill, piece);
           });
         }
         // activation fragments of the next step: read during the first half of the slices, sign
@@ -320,12 +331,12 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void qgemm_tile_kernel(
           constexpr int shift = (Q >= 2 * FA) ? 1 : 0;     // keep clear of the weight-fragment slot when there is room
           if constexpr (s < HALF) {
             static_for<FA>([&](auto x) {
-              if constexpr (decltype(x)::value * Q / FA + shift == q)
+              if constexpr ((ITEXHIP_ABLATE & 1) == 0 && decltype(x)::value * Q / FA + shift == q)
                 fa_nxt[decltype(x)::value] = lds_a_raw(st_nxt, decltype(x)::value / TM, decltype(x)::value % TM);
             });
           } else {
             static_for<4 * FA>([&](auto d) {
-              if constexpr (decltype(d)::value * Q / (4 * FA) == q)
+              if constexpr ((ITEXHIP_ABLATE & 32) == 0 && decltype(d)::value * Q / (4 * FA) == q)
                 fa_nxt[decltype(d)::value / 4][decltype(d)::value % 4] ^= amask;
             });
           }
@@ -348,6 +359,15 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void qgemm_tile_kernel(
   }
   wait_vmcnt<0>();  // no load may still be writing LDS when the epilogue reuses it
   __syncthreads();
+  if constexpr ((ITEXHIP_ABLATE & 16) != 0) {  // every accumulator stays live, nothing is stored
+    int all = 0;
+#pragma unroll
+    for (int t = 0; t < TN * TM; ++t)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) all ^= acc[t][r];
+    if (all == 0x12345678) reinterpret_cast<int*>(out)[threadIdx.x] = all;
+    return;
+  }
 
   // ---- epilogue.  Fast path: convert in registers, transpose through a private LDS buffer (the ring
   // is free after the last barrier) and store rows of 128 contiguous bytes, 16 B per lane.  A lane of

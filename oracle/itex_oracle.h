@@ -30,7 +30,9 @@
  *   abs(INT32_MIN) in orc_requantization_range_per_channel (undefined behaviour upstream);
  *   the last bits of the GELU post-ops (oneDNN evaluates tanh / erf with its own polynomial
  *   kernels; here libm's tanhf / erff): pinned only against a float64 evaluation and at the
- *   reference tests' own tolerance;
+ *   reference tests' own tolerance.  The device evaluates the exact GELU's erf with a five-term
+ *   rational-exponential form good to 1.5e-7 absolute, so it is compared with this oracle to 1e-6
+ *   absolute (2e-6 relative), which near zero is many last-place units;
  *   the bfloat16 / half bias (Tbias): the adjusted bias is rounded to Tbias as the code is
  *   written (quantized_matmul_common.h:578-599, 609-617); the reference's tests only use float and
  *   qint32 biases;
