@@ -735,6 +735,8 @@ int qconv2d_impl(const char* who, const void* x, int x_type, const itexhip_conv_
   cv.k_w = static_cast<int>(g->k_w); cv.out_h = static_cast<int>(g->out_h); cv.out_w = static_cast<int>(g->out_w);
   cv.stride_h = g->stride_h; cv.stride_w = g->stride_w; cv.dil_h = g->dil_h; cv.dil_w = g->dil_w;
   cv.pad_top = static_cast<int>(g->pad_top); cv.pad_left = static_cast<int>(g->pad_left);
+  cv.by_out_w = make_fast_div(g->out_w); cv.by_out_h = make_fast_div(g->out_h);
+  cv.by_in_c = make_fast_div(g->in_c); cv.by_k_w = make_fast_div(g->k_w);
   const uint32_t a_xor = (x_type == ITEXHIP_QUINT8) ? 0x80808080u : 0u;
   const uint8_t* xp = reinterpret_cast<const uint8_t*>(x);
   const uint8_t* bp = reinterpret_cast<const uint8_t*>(packed_filter);

@@ -400,10 +400,26 @@ __device__ __forceinline__ void wait_vmcnt() {
   __builtin_amdgcn_s_waitcnt((N & 15) | (7 << 4) | (15 << 8) | ((N >> 4) << 14));
 }
 
+// Division of a dividend below 2^31 by a divisor that is fixed per launch: n / d = (n * mul) >> sh with
+// sh = 31 + ceil(log2 d) and mul = ceil(2^sh / d) < 2^32, exact for every 0 <= n < 2^31 because
+// 2^sh <= mul * d <= 2^sh + 2^(sh - 31) (Granlund and Montgomery, division by invariant integers).  One 32 x 32 -> 64 bit
+// multiply and a shift where the division of two registers is a sequence of some thirty instructions.
+struct FastDiv { uint32_t mul, sh; };
+inline FastDiv make_fast_div(int64_t d) {  // host; 1 <= d < 2^31
+  uint32_t s = 0;
+  while ((1ull << s) < static_cast<uint64_t>(d)) ++s;
+  const uint32_t sh = 31 + s;
+  return FastDiv{static_cast<uint32_t>(((1ull << sh) + static_cast<uint64_t>(d) - 1) / static_cast<uint64_t>(d)), sh};
+}
+__device__ __forceinline__ int fast_div(int n, FastDiv f) {
+  return static_cast<int>((static_cast<uint64_t>(static_cast<uint32_t>(n)) * f.mul) >> f.sh);
+}
+
 // Geometry of a Conv2D computed as an implicit GEMM by the tile kernel (32-bit: the host checks the ranges)
 struct ConvTileArgs {
   int in_h, in_w, in_c, k_w, out_h, out_w;
   int stride_h, stride_w, dil_h, dil_w, pad_top, pad_left;
+  FastDiv by_out_w, by_out_h, by_in_c, by_k_w;  // the kernel's row and window decompositions divide by these
 };
 constexpr int kMaxConvPieces = 1024;  // 16-byte pieces per patch row: 16 KiB of receptive field per output position
 

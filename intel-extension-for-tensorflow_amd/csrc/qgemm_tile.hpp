@@ -171,8 +171,8 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void qgemm_tile_kernel(
     const int ld = wave * A_PER_WAVE + c;  // 0 .. A_LOADS-1 = (rt, h)
     const int m = min(m_base + ld * 16 + q_row, M - 1);
     if constexpr (CONV) {
-      const int t = m / cv.out_w, ow = m - t * cv.out_w;
-      const int b = t / cv.out_h, oh = t - b * cv.out_h;
+      const int t = fast_div(m, cv.by_out_w), ow = m - t * cv.out_w;
+      const int b = fast_div(t, cv.by_out_h), oh = t - b * cv.out_h;
       win_h[c] = oh * cv.stride_h - cv.pad_top;
       win_w[c] = ow * cv.stride_w - cv.pad_left;
       // input bytes < 2^31 checked by the host; the origin may be negative, origin + an in-bounds piece is not
@@ -185,8 +185,8 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void qgemm_tile_kernel(
   if constexpr (CONV) {
     for (int p = threadIdx.x; p < (K >> 4); p += 64 * NW) {
       const int k0 = p * 16;
-      const int kk = k0 / cv.in_c, cc = k0 - kk * cv.in_c;
-      const int kh = kk / cv.k_w, kw = kk - kh * cv.k_w;
+      const int kk = fast_div(k0, cv.by_in_c), cc = k0 - kk * cv.in_c;
+      const int kh = fast_div(kk, cv.by_k_w), kw = kk - kh * cv.k_w;
       const int dh = kh * cv.dil_h, dw = kw * cv.dil_w;  // < 2^15 each, checked by the host
       reinterpret_cast<int2*>(lds + CONV_TAB_OFF)[p] = make_int2((dh << 16) | dw, (dh * cv.in_w + dw) * cv.in_c + cc);
     }
