@@ -90,22 +90,22 @@ __global__ __launch_bounds__(256) void prepack_b_kernel(const int8_t* __restrict
 // activation operand repeat row M - 1; their results are never stored.  Pairs past the end of a wavefront's
 // run are loaded from clamped addresses and not used.
 // ------------------------------------------------------------------------------------------------
-constexpr int kGemvBatch = 4;                 // chunk pairs per batch
-constexpr int kGemvRing = 2 * kGemvBatch;     // activation slots of 1 KiB per wavefront
+constexpr int kGemvBatch = 4;                 // chunk pairs per batch (2 for up to 4 rows, see UB below)
 constexpr int kGemvPanelWords = 6 + 32;       // per channel of the strip: 6 parameter words + {scale, bias} of 16 rows
 
-// WIDE (M <= 4, R = 1): the activations of a whole batch of chunk pairs travel in one global -> LDS load of 4 rows x
-// 256 bytes (rows past M repeat row M - 1) instead of one load of 16 rows x 64 bytes per pair: a quarter of the
-// activation load instructions (with 16-channel strips every second load instruction of the kernel was one of them).
-template <int NT, int OUT_T, int R, bool WIDE = false>
+// UB: chunk pairs per batch; two batches of a wavefront are in flight.  4, except for up to 4 rows, where 2 measured
+// faster (4096 -> 14336 and 14336 -> 4096 at M = 4: 11.6 -> 11.3 and 11.3 -> 11.0 us, M = 1 unchanged; a form that
+// fetched the 4 rows of a whole batch of 4 pairs in one load of 4 x 256 bytes was no faster than that and is gone),
+// while 16 and more rows lose with it on long K (14336 -> 4096 at M = 16: 13.0 -> 15.2 us) and 1 is slower everywhere.
+template <int NT, int OUT_T, int R, int UB = kGemvBatch>
 __global__ __launch_bounds__(576) void qgemv_kernel(const uint8_t* __restrict__ a, uint32_t a_xor,
                                                      const uint8_t* __restrict__ bp, int M, int K, int N,
                                                      int KC, int cnt, EpilogueArgs e,
                                                      void* __restrict__ out) {
   constexpr int SW = 16 * NT;
-  constexpr int U = kGemvBatch, RING = kGemvRing;
-  constexpr int L = WIDE ? U * NT + 1 : U * (NT + R);  // loads per batch
-  static_assert(!WIDE || (R == 1 && U == 4), "the wide activation tile holds the 4 pairs of a batch for up to 4 rows");
+  constexpr int U = UB, RING = 2 * UB;  // RING: activation slots of 1 KiB per wavefront and row block
+  constexpr int L = U * (NT + R);       // loads per batch
+  static_assert(RING >= NT, "the partial tiles of a wavefront are handed over in its own ring");
   constexpr int ROWS = 16 * R;     // activation rows per workgroup
   // Per-row activation ranges (M <= 16): with 16-channel strips the parameter wavefront works out scale and bias of
   // every (row, channel) while the others stream and the epilogue reads a table (14336 -> 4096, M = 16: 14.9 -> 13.9 us);
@@ -132,18 +132,14 @@ __global__ __launch_bounds__(576) void qgemv_kernel(const uint8_t* __restrict__ 
   const uint8_t* wsrc = bp + (static_cast<int64_t>(chunk_row) * KC + (lgrp >> 1)) * kChunkBytes +
                         (((lgrp & 1) * 32 + half0 * 16 + lrow) << 4);
   // activation staging: lane -> (row q, piece j) of the 16 x 64 byte tile
-  // (WIDE: lane 16 q + s: row q, slot s of the row's 16 pieces, which holds piece s ^ q - the four rows' copies of a
-  // piece sit in four different bank groups)
-  const int q = WIDE ? (lane >> 4) : (lane >> 2);
-  const int dpiece = WIDE ? (((lane & 15) ^ q) * 16) : (((lane & 3) ^ ((q >> 2) & 3)) * 16);
+  const int q = lane >> 2;
+  const int dpiece = ((lane & 3) ^ ((q >> 2) & 3)) * 16;
   const uint8_t* arow[R];
 #pragma unroll
   for (int r = 0; r < R; ++r) arow[r] = a + static_cast<int64_t>(min(m_base + 16 * r + q, M - 1)) * K;
   const int klast = K - 16;  // k beyond K meets zero weights: any in-bounds data will do
   uint8_t* const ring = smem + wave * (RING * R * 1024);
   const uint32_t frag_off = static_cast<uint32_t>((4 * lrow + (lgrp ^ ((lrow >> 2) & 3))) * 16);
-  const int wrow = min(lrow, 3);  // WIDE: fragment row (rows from M on are copies of row M - 1 and never stored)
-  auto wide_off = [&](int u) { return static_cast<uint32_t>((wrow * 16 + ((u * 4 + lgrp) ^ wrow)) * 16); };
 
   v4i acc[R][NT];
 #pragma unroll
@@ -163,38 +159,27 @@ __global__ __launch_bounds__(576) void qgemv_kernel(const uint8_t* __restrict__ 
   const int p_full = min(p1, K >> 6);  // pairs below this index lie entirely inside K
   auto issue = [&](int pb, int slot0, v4i (&w)[U][NT]) {
     if (pb + U <= p_full) {
-      if constexpr (WIDE) {
-        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(aptr[0]),
-                                         (__attribute__((address_space(3))) void*)(ring + slot0 * 1024), 16, 0, 0);
-      } else {
 #pragma unroll
-        for (int u = 0; u < U; ++u)
+      for (int u = 0; u < U; ++u)
 #pragma unroll
-          for (int r = 0; r < R; ++r)
-            // the builtin, not inline assembly: the compiler's own vmcnt bookkeeping for the weight loads must see these
-            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(aptr[r] + u * 64),
-                                             (__attribute__((address_space(3))) void*)(ring + ((slot0 + u) * R + r) * 1024), 16, 0, 0);
-      }
+        for (int r = 0; r < R; ++r)
+          // the builtin, not inline assembly: the compiler's own vmcnt bookkeeping for the weight loads must see these
+          __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(aptr[r] + u * 64),
+                                           (__attribute__((address_space(3))) void*)(ring + ((slot0 + u) * R + r) * 1024), 16, 0, 0);
 #pragma unroll
       for (int u = 0; u < U; ++u)
 #pragma unroll
         for (int t = 0; t < NT; ++t)
           w[u][t] = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(wptr + u * (2 * kChunkBytes) + t * 256));
     } else {
-      if constexpr (WIDE) {
-        __builtin_amdgcn_global_load_lds(
-            (const __attribute__((address_space(1))) void*)(arow[0] + min(min(pb, KP - 1) * 64 + dpiece, klast)),
-            (__attribute__((address_space(3))) void*)(ring + slot0 * 1024), 16, 0, 0);
-      } else {
 #pragma unroll
-        for (int u = 0; u < U; ++u) {
-          const int p = min(pb + u, KP - 1);
+      for (int u = 0; u < U; ++u) {
+        const int p = min(pb + u, KP - 1);
 #pragma unroll
-          for (int r = 0; r < R; ++r)
-            __builtin_amdgcn_global_load_lds(
-                (const __attribute__((address_space(1))) void*)(arow[r] + min(p * 64 + dpiece, klast)),
-                (__attribute__((address_space(3))) void*)(ring + ((slot0 + u) * R + r) * 1024), 16, 0, 0);
-        }
+        for (int r = 0; r < R; ++r)
+          __builtin_amdgcn_global_load_lds(
+              (const __attribute__((address_space(1))) void*)(arow[r] + min(p * 64 + dpiece, klast)),
+              (__attribute__((address_space(3))) void*)(ring + ((slot0 + u) * R + r) * 1024), 16, 0, 0);
       }
 #pragma unroll
       for (int u = 0; u < U; ++u) {
@@ -216,7 +201,7 @@ __global__ __launch_bounds__(576) void qgemv_kernel(const uint8_t* __restrict__ 
       if (pb + u < p1) {  // wavefront uniform
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-          v4i x = *reinterpret_cast<const v4i*>(WIDE ? ring + slot0 * 1024 + wide_off(u) : ring + ((slot0 + u) * R + r) * 1024 + frag_off);
+          v4i x = *reinterpret_cast<const v4i*>(ring + ((slot0 + u) * R + r) * 1024 + frag_off);
           x.x ^= a_xor; x.y ^= a_xor; x.z ^= a_xor; x.w ^= a_xor;
 #pragma unroll
           for (int t = 0; t < NT; ++t) acc[r][t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w[u][t], x, acc[r][t], 0, 0, 0);
@@ -512,16 +497,19 @@ EpilogueArgs make_args(int a_type, const int32_t* colsum, const float* scales, c
   return e;
 }
 
+inline int gemv_batch(int M) { return M <= 4 ? 2 : kGemvBatch; }  // chunk pairs per batch of the variant that takes M rows
+
 template <int NT, int OUT_T>
 int launch_gemv(const uint8_t* a, uint32_t a_xor, const uint8_t* bp, int M, int K, int N, int KC, int waves, int cnt,
                 const EpilogueArgs& e, void* out, hipStream_t st) {
-  // up to 4 rows: the wide activation tile; up to 16: one tile of 16 rows per chunk pair; more: blocks of 32 rows
+  // up to 4 rows: batches of 2 chunk pairs; up to 16: batches of 4; more: blocks of 32 rows, batches of 4
   const int variant = M > 16 ? 2 : (M <= 4 ? 1 : 0);
-  auto kern = variant == 2 ? qgemv_kernel<NT, OUT_T, 2> : variant == 1 ? qgemv_kernel<NT, OUT_T, 1, true> : qgemv_kernel<NT, OUT_T, 1>;
+  auto kern = variant == 2 ? qgemv_kernel<NT, OUT_T, 2, 4> : variant == 1 ? qgemv_kernel<NT, OUT_T, 1, 2> : qgemv_kernel<NT, OUT_T, 1, 4>;
   const int R = M > 16 ? 2 : 1;
+  const int ring = 2 * gemv_batch(M);  // KiB per wavefront and row block
   // the kernel's table of per-row parameters holds 16 rows
   ITEXHIP_REQUIRE(e.row_min_a == nullptr || M <= 16, "the small-M kernel takes per-row activation ranges for M <= 16 only");
-  const size_t lds_max = static_cast<size_t>(8 * kGemvRing * 1024) * R + kGemvPanelWords * 16 * NT * 4;
+  const size_t lds_max = static_cast<size_t>(8 * ring * 1024) * R + kGemvPanelWords * 16 * NT * 4;
   static unsigned long long attr_done[3] = {0, 0, 0};  // per variant: devices on which the attribute is set
   if (!device_bit(&attr_done[variant], false)) {
     hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -529,7 +517,7 @@ int launch_gemv(const uint8_t* a, uint32_t a_xor, const uint8_t* bp, int M, int 
     if (err != hipSuccess) return hip_fail(err, "hipFuncSetAttribute(qgemv_kernel)");
     device_bit(&attr_done[variant], true);
   }
-  const size_t lds = static_cast<size_t>(waves) * kGemvRing * 1024 * R + kGemvPanelWords * 16 * NT * 4;
+  const size_t lds = static_cast<size_t>(waves) * ring * 1024 * R + kGemvPanelWords * 16 * NT * 4;
   const int strips = (N + 16 * NT - 1) / (16 * NT);
   const int rbs = (M + 31) / 32;  // row blocks of the R = 2 kernel
   const dim3 grid = M > 16 ? dim3(8 * rbs, (strips + 7) / 8) : dim3(strips);
@@ -549,7 +537,7 @@ int dispatch_gemv(const uint8_t* a, uint32_t a_xor, const uint8_t* bp, int M, in
   const int nt = (N + 31) / 32 >= 256 ? 2 : 1;
   int waves = std::max(nt, std::min(8, (KP + 15) / 16));
   for (int w = waves; w >= std::max(nt, waves / 2 + 1); --w)
-    if (KP % (kGemvBatch * w) == 0) { waves = w; break; }
+    if (KP % (gemv_batch(M) * w) == 0) { waves = w; break; }
   // From 16 rows on, half as many wavefronts with runs twice as long: fewer partial tiles to reduce and fewer rings
   // (4096 -> 14336 at M = 16: 12.45 -> 11.8 us with 2 instead of 4; 14336 -> 4096: 13.4 -> 13.0 us with 4 instead of 8);
   // below that the longer ramp of fewer wavefronts costs more than it saves (14336 -> 4096 at M = 1: 11.2 -> 12.5 us).
