@@ -90,13 +90,14 @@ __global__ __launch_bounds__(256) void prepack_b_kernel(const int8_t* __restrict
 // activation operand repeat row M - 1; their results are never stored.  Pairs past the end of a wavefront's
 // run are loaded from clamped addresses and not used.
 // ------------------------------------------------------------------------------------------------
-constexpr int kGemvBatch = 4;                 // chunk pairs per batch (2 for up to 4 rows, see UB below)
+constexpr int kGemvBatch = 4;                 // chunk pairs per batch of the 32-row kernel (2 for up to 16 rows, see UB below)
 constexpr int kGemvPanelWords = 6 + 32;       // per channel of the strip: 6 parameter words + {scale, bias} of 16 rows
 
-// UB: chunk pairs per batch; two batches of a wavefront are in flight.  4, except for up to 4 rows, where 2 measured
-// faster (4096 -> 14336 and 14336 -> 4096 at M = 4: 11.6 -> 11.3 and 11.3 -> 11.0 us, M = 1 unchanged; a form that
-// fetched the 4 rows of a whole batch of 4 pairs in one load of 4 x 256 bytes was no faster than that and is gone),
-// while 16 and more rows lose with it on long K (14336 -> 4096 at M = 16: 13.0 -> 15.2 us) and 1 is slower everywhere.
+// UB: chunk pairs per batch; two batches of a wavefront are in flight.  2 for up to 16 rows, 4 for the blocks of 32
+// rows.  Measured on 4096 -> 14336 / 14336 -> 4096 with the wavefront counts the host picks for each: M = 4 11.6 -> 10.95
+// and 11.3 -> 11.0 us, M = 1 11.3 -> 10.95 us and unchanged, M = 16 unchanged and 13.0 -> 12.7 us against batches of 4
+// (a form that fetched the 4 rows of a whole batch of 4 pairs in one load of 4 x 256 bytes was no faster and is gone);
+// batches of 1 or 3 are slower everywhere, and with 32 rows batches of 2 lose on long K.
 template <int NT, int OUT_T, int R, int UB = kGemvBatch>
 __global__ __launch_bounds__(576) void qgemv_kernel(const uint8_t* __restrict__ a, uint32_t a_xor,
                                                      const uint8_t* __restrict__ bp, int M, int K, int N,
@@ -497,20 +498,20 @@ EpilogueArgs make_args(int a_type, const int32_t* colsum, const float* scales, c
   return e;
 }
 
-inline int gemv_batch(int M) { return M <= 4 ? 2 : kGemvBatch; }  // chunk pairs per batch of the variant that takes M rows
+inline int gemv_batch(int M) { return M <= 16 ? 2 : kGemvBatch; }  // chunk pairs per batch of the variant that takes M rows
 
 template <int NT, int OUT_T>
 int launch_gemv(const uint8_t* a, uint32_t a_xor, const uint8_t* bp, int M, int K, int N, int KC, int waves, int cnt,
                 const EpilogueArgs& e, void* out, hipStream_t st) {
-  // up to 4 rows: batches of 2 chunk pairs; up to 16: batches of 4; more: blocks of 32 rows, batches of 4
-  const int variant = M > 16 ? 2 : (M <= 4 ? 1 : 0);
-  auto kern = variant == 2 ? qgemv_kernel<NT, OUT_T, 2, 4> : variant == 1 ? qgemv_kernel<NT, OUT_T, 1, 2> : qgemv_kernel<NT, OUT_T, 1, 4>;
+  // up to 16 rows: batches of 2 chunk pairs; more: blocks of 32 rows, batches of 4
+  const int variant = M > 16 ? 1 : 0;
+  auto kern = variant == 1 ? qgemv_kernel<NT, OUT_T, 2, 4> : qgemv_kernel<NT, OUT_T, 1, 2>;
   const int R = M > 16 ? 2 : 1;
   const int ring = 2 * gemv_batch(M);  // KiB per wavefront and row block
   // the kernel's table of per-row parameters holds 16 rows
   ITEXHIP_REQUIRE(e.row_min_a == nullptr || M <= 16, "the small-M kernel takes per-row activation ranges for M <= 16 only");
   const size_t lds_max = static_cast<size_t>(8 * ring * 1024) * R + kGemvPanelWords * 16 * NT * 4;
-  static unsigned long long attr_done[3] = {0, 0, 0};  // per variant: devices on which the attribute is set
+  static unsigned long long attr_done[2] = {0, 0};  // per variant: devices on which the attribute is set
   if (!device_bit(&attr_done[variant], false)) {
     hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                                          static_cast<int>(lds_max));
@@ -530,19 +531,19 @@ int dispatch_gemv(const uint8_t* a, uint32_t a_xor, const uint8_t* bp, int M, in
                   const EpilogueArgs& e, void* out, hipStream_t st) {
   const int KC = 2 * ((K + 63) / 64), KP = KC / 2;
   // 32-channel strips when they alone give every CU a workgroup, else 16-channel strips; a strip is finished by one
-  // wavefront per 16-channel tile, so never fewer wavefronts than that.  Wavefronts per strip: about 16 chunk pairs
-  // (four batches) each, at most 8 (measured on 4096 x 14336 and 14336 x 4096: more, smaller wavefronts start their
-  // streams later and reduce more partial tiles than they gain in loads in flight); prefer a count that divides K
-  // into whole batches.
+  // wavefront per 16-channel tile, so never fewer wavefronts than that.  Wavefronts per strip, at most 8, measured on
+  // 4096 x 14336 and 14336 x 4096 with every count from 2 to 8, both strip widths and both batch sizes: up to 4 rows
+  // about 8 chunk pairs (four batches of 2) each (4096 -> 14336 at M = 1 / 4: 11.3 -> 10.95 us with 8 instead of 4);
+  // 5 to 16 rows about 16 pairs each (4096 -> 14336 at M = 16: 4 wavefronts 11.7 us, 8 over 11.8 us; 14336 -> 4096: 8
+  // wavefronts 12.7 us, 4 wavefronts 15.2 us); prefer a count that divides K into whole batches.
   const int nt = (N + 31) / 32 >= 256 ? 2 : 1;
-  int waves = std::max(nt, std::min(8, (KP + 15) / 16));
+  const int per_wave = M <= 4 ? 8 : 16;
+  int waves = std::max(nt, std::min(8, (KP + per_wave - 1) / per_wave));
   for (int w = waves; w >= std::max(nt, waves / 2 + 1); --w)
     if (KP % (gemv_batch(M) * w) == 0) { waves = w; break; }
-  // From 16 rows on, half as many wavefronts with runs twice as long: fewer partial tiles to reduce and fewer rings
-  // (4096 -> 14336 at M = 16: 12.45 -> 11.8 us with 2 instead of 4; 14336 -> 4096: 13.4 -> 13.0 us with 4 instead of 8);
-  // below that the longer ramp of fewer wavefronts costs more than it saves (14336 -> 4096 at M = 1: 11.2 -> 12.5 us).
-  // (not with per-row ranges on 32-channel strips, whose epilogue is spread over all the wavefronts)
-  if (M >= 16 && !(e.row_min_a != nullptr && nt == 2)) waves = std::max(nt, waves / 2);
+  // Blocks of 32 rows (batches of 4): half as many wavefronts with runs twice as long, fewer partial tiles to reduce
+  // and fewer rings.
+  if (M > 16) waves = std::max(nt, waves / 2);
   const int cnt = (KP + waves - 1) / waves;
   if (nt == 2) return launch_gemv<2, OUT_T>(a, a_xor, bp, M, K, N, KC, waves, cnt, e, out, st);
   return launch_gemv<1, OUT_T>(a, a_xor, bp, M, K, N, KC, waves, cnt, e, out, st);
