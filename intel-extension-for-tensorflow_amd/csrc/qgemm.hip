@@ -108,11 +108,10 @@ __global__ __launch_bounds__(576) void qgemv_kernel(const uint8_t* __restrict__ 
   constexpr int L = U * (NT + R);       // loads per batch
   static_assert(RING >= NT, "the partial tiles of a wavefront are handed over in its own ring");
   constexpr int ROWS = 16 * R;     // activation rows per workgroup
-  // Per-row activation ranges (M <= 16): with 16-channel strips the parameter wavefront works out scale and bias of
-  // every (row, channel) while the others stream and the epilogue reads a table (14336 -> 4096, M = 16: 14.9 -> 13.9 us);
-  // with 32-channel strips (4 streaming wavefronts, shorter streams, twice the pairs) that wavefront finished last
-  // (13.9 -> 14.9 us), so there the two finishing wavefronts do the arithmetic in the epilogue.
-  constexpr bool ROW_TABLE = (NT == 1);
+  // Per-row activation ranges (M <= 16): the parameter wavefront works out scale and bias of every (row, channel) of
+  // the strip while the others stream, and the epilogue reads a table (14336 -> 4096, M = 16: 14.9 -> 13.9 us; 32-channel
+  // strips, 4096 -> 14336: 13.0 -> 12.1 us once that wavefront fetched the 16 rows' ranges in one round trip instead of
+  // one per table entry - before that it finished last there).
   extern __shared__ __align__(16) uint8_t smem[];  // [waves][RING][R][1 KiB], then the parameter panel [3 or 6][SW]
   // R = 1 (M <= 16): one workgroup per strip.  R = 2 (M > 16): a workgroup takes 32 rows of a strip - every weight
   // fragment meets two activation fragments - and the grid is x = 8 * row blocks, y = groups of 8 strips (x runs
@@ -241,17 +240,24 @@ __global__ __launch_bounds__(576) void qgemv_kernel(const uint8_t* __restrict__ 
         panel[2 * SW + lane] = __float_as_int(bias);
       }
     }
-    if (ROW_TABLE && e.row_min_a) {
+    if (e.row_min_a) {
       // Per-row ranges: scale and bias of every (row, channel) of the strip, 16 * SW pairs over the 64 lanes, worked
       // out here while the other wavefronts stream (the raw channel values come back from the panel: LDS operations
       // of one wavefront complete in order).  The epilogue then only reads the table.
       float* const rowtab = reinterpret_cast<float*>(panel + 6 * SW);  // [16][SW]{scale, bias}
+      // the 16 rows' ranges: one round trip to memory for all of them (lane r holds row r), handed round by lane index
+      float rmin = 0.0f, rmax = 0.0f;
+      if (lane < 16 && m_base + lane < M) {
+        rmin = e.row_min_a[m_base + lane];
+        rmax = e.row_max_a[m_base + lane];
+      }
       for (int idx = lane; idx < 16 * SW; idx += 64) {
         const int mm = idx / SW, c = idx - mm * SW;
+        const float lo = __shfl(rmin, mm, 64), hi = __shfl(rmax, mm, 64);
         if (m_base + mm < M) {
           PrepArgs pr = e.prep;
-          pr.min_a = e.row_min_a[m_base + mm];
-          pr.max_a = e.row_max_a[m_base + mm];
+          pr.min_a = lo;
+          pr.max_a = hi;
           const ChannelScaleBias cs = channel_scale_bias(
               pr, __int_as_float(panel[SW + c]), __int_as_float(panel[2 * SW + c]), __int_as_float(panel[3 * SW + c]),
               __int_as_float(panel[4 * SW + c]), __int_as_float(panel[5 * SW + c]), panel[c]);
@@ -285,30 +291,6 @@ __global__ __launch_bounds__(576) void qgemv_kernel(const uint8_t* __restrict__ 
   }
   // cross-wavefront reduction through the rings
   __syncthreads();
-  if (!ROW_TABLE && e.row_min_a != nullptr) {
-    // Per-row ranges with 32-channel strips: every output has its own scale and bias to work out (three divisions
-    // each), so the 4 channels of a lane's group go to different wavefronts - all of them, the parameter wavefront
-    // included - instead of one wavefront per tile doing four in a row.
-    for (int unit = wave; unit < 4 * R * NT; unit += waves + 1) {
-      const int tile = unit >> 2, r = unit & 3;
-      const int tr = tile / NT, tc = tile - tr * NT;
-      int part = 0;
-      for (int w = 0; w < waves; ++w) part += reinterpret_cast<const int*>(smem + w * (RING * R * 1024) + tile * 1024 + lane * 16)[r];
-      const int col = tc * 16 + lgrp * 4 + r, n = strip * SW + col;
-      const int m = m_base + 16 * tr + lrow;
-      if (m < M && n < N) {
-        PrepArgs pr = e.prep;
-        pr.min_a = e.row_min_a[m];
-        pr.max_a = e.row_max_a[m];
-        const int colsum = panel[col];
-        const ChannelScaleBias c = channel_scale_bias(pr, __int_as_float(panel[SW + col]), __int_as_float(panel[2 * SW + col]),
-                                                      __int_as_float(panel[3 * SW + col]), __int_as_float(panel[4 * SW + col]),
-                                                      __int_as_float(panel[5 * SW + col]), colsum);
-        epilogue_store_one<OUT_T>(part, e.comp_mul * colsum, e.n_scales > 0 ? c.scale : 1.0f, c.bias, m, n, N, e, out);
-      }
-    }
-    return;
-  }
   // the R * NT tiles of 16 x 16 go round the wavefronts (R = 1: wavefront t finishes tile t)
   for (int tile = wave; tile < R * NT; tile += waves + 1) {
     const int tr = tile / NT, tc = tile - tr * NT;
@@ -321,29 +303,12 @@ __global__ __launch_bounds__(576) void qgemv_kernel(const uint8_t* __restrict__ 
     if (m < M && n < N) {
       ChannelParams cp;
       if (e.row_min_a) {
-        if constexpr (ROW_TABLE) {
-          const float* const rowtab = reinterpret_cast<const float*>(panel + 6 * SW) + 2 * ((m - m_base) * SW + col);
+        const float* const rowtab = reinterpret_cast<const float*>(panel + 6 * SW) + 2 * ((m - m_base) * SW + col);
 #pragma unroll
-          for (int r = 0; r < 4; ++r) {
-            cp.comp[r] = e.comp_mul * panel[col + r];
-            cp.scale[r] = rowtab[2 * r];
-            cp.bias[r] = rowtab[2 * r + 1];
-          }
-        } else {
-          PrepArgs pr = e.prep;
-          pr.min_a = e.row_min_a[m];
-          pr.max_a = e.row_max_a[m];
-#pragma unroll
-          for (int r = 0; r < 4; ++r) {
-            const int colsum = panel[col + r];
-            const ChannelScaleBias c = channel_scale_bias(
-                pr, __int_as_float(panel[SW + col + r]), __int_as_float(panel[2 * SW + col + r]),
-                __int_as_float(panel[3 * SW + col + r]), __int_as_float(panel[4 * SW + col + r]),
-                __int_as_float(panel[5 * SW + col + r]), colsum);
-            cp.comp[r] = e.comp_mul * colsum;
-            cp.scale[r] = e.n_scales > 0 ? c.scale : 1.0f;
-            cp.bias[r] = c.bias;
-          }
+        for (int r = 0; r < 4; ++r) {
+          cp.comp[r] = e.comp_mul * panel[col + r];
+          cp.scale[r] = rowtab[2 * r];
+          cp.bias[r] = rowtab[2 * r + 1];
         }
       } else {
 #pragma unroll

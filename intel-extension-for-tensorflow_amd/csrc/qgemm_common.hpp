@@ -355,22 +355,6 @@ __device__ __forceinline__ void epilogue_store(const v4i acc, const ChannelParam
   }
 }
 
-// One output element, same arithmetic as epilogue_store with the generic chain (for callers that spread the
-// channels of a group over several wavefronts).
-template <int OUT_T>
-__device__ __forceinline__ void epilogue_store_one(int acc, int comp, float scale, float bias, int m, int n, int N,
-                                                   const EpilogueArgs& e, void* __restrict__ out) {
-  float v = static_cast<float>(acc + comp);
-  v = v * scale;
-  if (e.bias || e.fused) v = v + bias;
-  const int64_t o = static_cast<int64_t>(m) * N + n;
-  for (int k = 0; k < e.n_eltwise; ++k) {
-    if (e.elt[k].alg == ITEXHIP_ELT_SUM) v = v + e.elt[k].alpha * load_addend(e, o);
-    else v = apply_eltwise(e.elt[k], v);
-  }
-  store_output<OUT_T>(out, o, v);
-}
-
 // Compile-time loop: f(std::integral_constant<int, 0>{}), ..., f(<N-1>).  Indices into register arrays
 // are constants from the start, so the arrays are split into registers without relying on loop unrolling.
 template <class F, int... I>
