@@ -495,13 +495,16 @@ template <int OUT_T>
 int dispatch_gemv(const uint8_t* a, uint32_t a_xor, const uint8_t* bp, int M, int K, int N,
                   const EpilogueArgs& e, void* out, hipStream_t st) {
   const int KC = 2 * ((K + 63) / 64), KP = KC / 2;
-  // 32-channel strips when they alone give every CU a workgroup, else 16-channel strips; a strip is finished by one
+  // 32-channel strips when they give every CU a workgroup, else 16-channel strips; a strip is finished by one
   // wavefront per 16-channel tile, so never fewer wavefronts than that.  Wavefronts per strip, at most 8, measured on
   // 4096 x 14336 and 14336 x 4096 with every count from 2 to 8, both strip widths and both batch sizes: up to 4 rows
   // about 8 chunk pairs (four batches of 2) each (4096 -> 14336 at M = 1 / 4: 11.3 -> 10.95 us with 8 instead of 4);
   // 5 to 16 rows about 16 pairs each (4096 -> 14336 at M = 16: 4 wavefronts 11.7 us, 8 over 11.8 us; 14336 -> 4096: 8
   // wavefronts 12.7 us, 4 wavefronts 15.2 us); prefer a count that divides K into whole batches.
-  const int nt = (N + 31) / 32 >= 256 ? 2 : 1;
+  // (blocks of 32 rows count as workgroups of their own: 14336 -> 4096 at M = 64 28.1 -> 20.0 us with 32-channel strips,
+  // 256 workgroups instead of 512 that read the activations twice as often)
+  const int row_blocks = M > 16 ? (M + 31) / 32 : 1;
+  const int nt = ((N + 31) / 32) * row_blocks >= 256 ? 2 : 1;
   const int per_wave = M <= 4 ? 8 : 16;
   int waves = std::max(nt, std::min(8, (KP + per_wave - 1) / per_wave));
   for (int w = waves; w >= std::max(nt, waves / 2 + 1); --w)
@@ -527,7 +530,7 @@ int dispatch_gemv(const uint8_t* a, uint32_t a_xor, const uint8_t* bp, int M, in
 // Which packed kernel takes a call.  The small-M kernel (a strip of channels x 16 rows x all of K per workgroup)
 // streams the weight once per block of 16 rows; the tile kernel needs enough 64 x 64 tiles to fill the device.
 // Measured on 4096 x 14336 / 14336 x 4096 weights (us, small-M against tile kernel): M = 32: 15 / 17 against 23 / 67;
-// M = 64: 23 / 29 against 23 / 68; M = 128: 40 / 50 against 28 / 67; on a 1024 x 1024 weight the small-M kernel takes
+// M = 64: 23 / 21 against 23 / 68; M = 128: 28 / 34 against 28 / 67; on a 1024 x 1024 weight the small-M kernel takes
 // 3.6 against 4.8 up to M = 128.  Both kernels accumulate exactly and share the epilogue: the same bytes either way.
 constexpr int kSmallMaxRows = 128;
 static bool small_m(int64_t M, int64_t K, int64_t N) {
