@@ -696,12 +696,25 @@ int launch_tile(const uint8_t* a, uint32_t amask, const uint8_t* bp, int M, int 
 
 // Tile shape: the one with the smallest estimated time = rounds of workgroups over the 256 CUs x
 // tile area x a penalty for the operand traffic per MFMA of smaller tiles.
-inline int pick_tile_shape(int M, int N, bool wide_only, int first = 0) {
+//
+// long_epilogue_short_k: a transcendental activation (GELU ...) on a short K.  The epilogue is then a large part of the
+// launch, and 128 x 128 tiles, two or three workgroups per CU, run one tile's epilogue under another's K loop: BERT-base
+// 768 -> 3072 + GeluApproximate at 4096 tokens 22.4 -> 20.0 us (fp32), 20.8 -> 17.2 us (bfloat16); measured on 4096 x 3072,
+// 2048 x 4096 and 4096 x 4096 outputs the small tiles win up to K = 1536 - 2048 and lose beyond (the K loop's operand
+// traffic), and lose at any K when there are fewer than two tiles per CU (512 x 3072).  With any epilogue the same holds
+// up to K = 256, where a launch is little more than its epilogue (100352 x 256 outputs, the last 1 x 1 convolution of a
+// ResNet-50 block, K = 64: 18.7 -> 12.4 us, with the residual Sum 39.5 -> 20.5 us; 4096 x 3072, 16384 x 1024 and
+// 2048 x 14336 outputs, 8-bit and fp32: 5 - 30 % faster at K = 64 - 256, mixed at 384, slower from 512 on).
+inline int pick_tile_shape(int M, int N, bool wide_only, int first = 0, bool long_epilogue_short_k = false) {
   struct Shape { int bm, bn; double penalty; };
   static const Shape shapes[5] = {{256, 256, 1.0}, {256, 192, 1.03}, {256, 128, 1.08}, {128, 128, 1.2}, {64, 64, 1.8}};
   // itexhip_test_force_tile_shape forces a shape (tests exercise every shape on ragged problems with it)
   const int f = __atomic_load_n(&g_forced_tile_shape[0], __ATOMIC_RELAXED);
   if (f >= (wide_only ? 3 : first) && f < 5) return f;
+  if (long_epilogue_short_k) {  // at least two 128 x 128 tiles per CU, at most 15 % of their area outside the output
+    const int64_t t128 = static_cast<int64_t>((M + 127) / 128) * ((N + 127) / 128);
+    if (t128 >= 512 && t128 * (128 * 128) * 100 <= static_cast<int64_t>(M) * N * 115) return 3;
+  }
   int best = 3;
   double best_cost = 1e300;
   for (int i = wide_only ? 3 : first; i < 5; ++i) {
@@ -716,7 +729,7 @@ inline int pick_tile_shape(int M, int N, bool wide_only, int first = 0) {
 template <int OUT_T, int ACT>
 int dispatch_tile_shape(const uint8_t* a, uint32_t amask, const uint8_t* bp, int M, int K, int N,
                         const EpilogueArgs& e, void* out, hipStream_t st) {
-  switch (pick_tile_shape(M, N, false)) {
+  switch (pick_tile_shape(M, N, false, 0, (ACT == 3 && K <= 1536) || K <= 256)) {
     case 0: return launch_tile<256, 256, 2, 2, OUT_T, ACT, true>(a, amask, bp, M, K, N, e, out, st);
     case 1: return launch_tile<256, 192, 2, 2, OUT_T, ACT, true>(a, amask, bp, M, K, N, e, out, st);
     case 2: return launch_tile<256, 128, 2, 2, OUT_T, ACT, true>(a, amask, bp, M, K, N, e, out, st);
